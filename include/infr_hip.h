@@ -1,0 +1,240 @@
+/*
+ * infr_hip.h — C ABI of the MI355X (gfx950) backend for the routed-expert MoE FFN path.
+ *
+ * The entry points mirror, one for one, the object-safe trait `infr_core::backend::Backend`
+ * of the reference engine (crates/infr-core/src/backend.rs:630-1088) together with its
+ * `Buffer` (:423-452), `Plan` (:468-482), `Bindings` (:522-620) and the slice of the graph IR
+ * (`Graph`/`Op`, crates/infr-core/src/graph.rs) that the MoE FFN path uses.  A Rust crate
+ * implementing `Backend` binds exactly these symbols through `extern "C"`.
+ *
+ * Conventions
+ *   - every fallible call returns an infr_status; the message is read with
+ *     infr_hip_last_error() (thread-local, UTF-8, valid until the next failing call on
+ *     that thread).  No exception, abort or panic crosses this boundary
+ *     (reference: `Result<T, infr_core::Error>`, crates/infr-core/src/error.rs:11-31).
+ *   - handles are opaque; a handle from another backend instance is an INVALID error, never
+ *     undefined behaviour (reference: `as_any().downcast_ref`, backend.rs:433-436).
+ *   - all entry points are thread-safe (`Backend: Send + Sync`).
+ *   - work is stream-ordered on one internal HIP stream: execute() enqueues and returns;
+ *     download() and sync() wait.
+ */
+#ifndef INFR_HIP_H
+#define INFR_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* infr_core::Error variants that can occur on this path (error.rs:11-31). */
+typedef enum infr_status {
+    INFR_OK = 0,
+    INFR_ERR_BACKEND = 1,     /* Error::Backend: HIP failure, bad binding, size mismatch */
+    INFR_ERR_UNSUPPORTED = 2, /* Error::Unsupported: op / dtype / option not implemented */
+    INFR_ERR_ABORTED = 3,     /* Error::Aborted: shutdown latch set */
+    INFR_ERR_INVALID = 4      /* null / foreign handle, malformed graph */
+} infr_status;
+
+/* infr_core::DType, same ordinal order (crates/infr-core/src/tensor.rs:7-57). */
+typedef enum infr_dtype {
+    INFR_F32 = 0, INFR_F16 = 1, INFR_BF16 = 2, INFR_I32 = 3, INFR_U32 = 4,
+    INFR_Q4_0 = 5, INFR_Q4_1 = 6, INFR_Q5_0 = 7, INFR_Q5_1 = 8, INFR_Q8_0 = 9,
+    INFR_Q2K = 10, INFR_Q3K = 11, INFR_Q4K = 12, INFR_Q5K = 13, INFR_Q6K = 14
+    /* ordinals 15.. (i-quants, ternary, fp4, turbo) are accepted in declarations and
+     * rejected with INFR_ERR_UNSUPPORTED by any op that would decode them */
+} infr_dtype;
+
+/* infr_core::backend::BufferUsage (backend.rs:384-406). */
+typedef enum infr_buffer_usage {
+    INFR_USAGE_WEIGHTS = 0, INFR_USAGE_ACTIVATIONS = 1, INFR_USAGE_KV_CACHE = 2,
+    INFR_USAGE_STAGING = 3, INFR_USAGE_READBACK = 4, INFR_USAGE_HOST_WEIGHTS = 5
+} infr_buffer_usage;
+
+/* infr_core::graph::TensorKind (graph.rs:119-131). */
+typedef enum infr_tensor_kind {
+    INFR_KIND_INPUT = 0, INFR_KIND_WEIGHT = 1, INFR_KIND_INTERNAL = 2, INFR_KIND_OUTPUT = 3
+} infr_tensor_kind;
+
+/* infr_core::graph::Activation (graph.rs:47-54), MoeGating (graph.rs:73-85). */
+typedef enum infr_activation { INFR_ACT_SILU = 0, INFR_ACT_GELU = 1, INFR_ACT_SIGMOID = 2 } infr_activation;
+typedef enum infr_moe_gating {
+    INFR_GATING_SOFTMAX = 0, INFR_GATING_SIGMOID = 1, INFR_GATING_SQRT_SOFTPLUS = 2
+} infr_moe_gating;
+
+#define INFR_NO_TENSOR 0xFFFFFFFFu /* Option<TensorId>::None */
+
+/* TensorDecl { desc: TensorDesc { shape, dtype }, kind } (graph.rs:133-140, tensor.rs:258-261). */
+typedef struct infr_tensor_decl {
+    uint32_t rank;      /* 0..4 */
+    uint64_t shape[4];
+    int32_t dtype;      /* infr_dtype */
+    int32_t kind;       /* infr_tensor_kind */
+} infr_tensor_decl;
+
+/* Op variants on the MoE FFN path.  Every other Op of the reference IR has no encoding here:
+ * a front end that meets one reports Unsupported itself, as the reference's GPU adapter does
+ * for combinations it cannot lower (crates/infr-vulkan/src/adapter.rs:8936-8985). */
+typedef enum infr_op_kind {
+    INFR_OP_MOE_FFN = 0,               /* Op::MoeFfn              graph.rs:1259-1352 */
+    INFR_OP_LINEAR = 1,                /* Op::Linear              graph.rs:200-212   */
+    INFR_OP_GATED_ACT = 2,             /* Op::GatedAct            graph.rs:935-975   */
+    INFR_OP_ADD = 3,                   /* Op::Add                                   */
+    INFR_OP_MOE_SHARED_EXPERT_ADD = 4  /* Op::MoeSharedExpertAdd  graph.rs:1449-1463 */
+} infr_op_kind;
+
+/* Field-for-field Op::MoeFfn.  Option<TensorId> = INFR_NO_TENSOR; Option<f32> and
+ * Option<(u32,u32)> carry a has_* flag. */
+typedef struct infr_op_moe_ffn {
+    uint32_t x, router_x, router, gate_exps, up_exps, down_exps;
+    uint32_t down_scale;           /* optional */
+    uint32_t fused_gate_up;        /* bool */
+    uint32_t dst;
+    uint32_t ne, n_expert, n_used, n_ff_exp;
+    float scale;
+    int32_t act;                   /* infr_activation */
+    uint32_t has_swiglu_clamp; float swiglu_clamp;
+    int32_t gating;                /* infr_moe_gating */
+    uint32_t norm_w;               /* bool */
+    uint32_t weight_before;        /* bool */
+    uint32_t has_ep_band; uint32_t ep_base, ep_n_local;
+    uint32_t exp_probs_b;          /* optional */
+    uint32_t n_expert_groups, n_expert_groups_used;
+    uint32_t expert_ids;           /* optional */
+} infr_op_moe_ffn;
+
+typedef struct infr_op_linear {
+    uint32_t x, weight, dst;
+    uint32_t m, in_f, out_f, w_off;
+} infr_op_linear;
+
+typedef struct infr_op_gated_act {
+    uint32_t gate, up, dst;
+    uint32_t rows, nff;
+    int32_t act;
+    uint32_t up_off, up_stride, gate_stride, gate_block_width;
+    uint32_t has_swiglu_clamp; float swiglu_clamp;
+} infr_op_gated_act;
+
+typedef struct infr_op_add { uint32_t a, b, dst, n; } infr_op_add;
+
+typedef struct infr_op_moe_shared_expert_add {
+    uint32_t moe, shexp, gate, dst;
+    uint32_t rows, n;
+} infr_op_moe_shared_expert_add;
+
+typedef struct infr_op {
+    int32_t kind; /* infr_op_kind */
+    union {
+        infr_op_moe_ffn moe_ffn;
+        infr_op_linear linear;
+        infr_op_gated_act gated_act;
+        infr_op_add add;
+        infr_op_moe_shared_expert_add moe_shared_expert_add;
+    } u;
+} infr_op;
+
+/* Graph { tensors, ops } (graph.rs:2056-2123); the inputs/weights/outputs lists are implied by
+ * each declaration's kind. */
+typedef struct infr_graph {
+    const infr_tensor_decl *tensors; uint32_t n_tensors;
+    const infr_op *ops;              uint32_t n_ops;
+} infr_graph;
+
+typedef struct infr_hip_backend infr_hip_backend;
+typedef struct infr_hip_buffer infr_hip_buffer;
+typedef struct infr_hip_plan infr_hip_plan;
+
+/* One Bindings::bind(id, buf) (backend.rs:582-590). */
+typedef struct infr_binding { uint32_t tensor; const infr_hip_buffer *buffer; } infr_binding;
+
+/* Subset of Capabilities (backend.rs:45-236) a caller of this path consults. */
+typedef struct infr_hip_capabilities {
+    char name[64];
+    uint32_t f16, bf16, i8, i8_dot;
+    uint32_t subgroup_min, subgroup_max;
+    uint32_t integrated, compute_units;
+    uint32_t buffer_device_address;
+    uint32_t max_shared_memory_bytes;
+    uint32_t unified_memory, decode_replay, combined_gu, graph_input_inplace;
+    uint64_t device_memory_bytes;
+} infr_hip_capabilities;
+
+typedef struct infr_hip_config {
+    /* 0: let execute() replay a captured HIP graph when a plan is re-run with identical
+     *    bindings; 1: always launch kernels directly. */
+    uint32_t disable_graph_replay;
+    /* rows above which Op::MoeFfn takes the bucketed grouped-GEMM path instead of the
+     * per-token GEMV path; 0 selects the built-in default. */
+    uint32_t moe_batched_min_rows;
+    uint32_t reserved[6];
+} infr_hip_config;
+
+/* Construction of the backend object (reference: VulkanBackend::new / CpuBackend::new,
+ * crates/infr-cpu/src/lib.rs:868).  cfg may be NULL.  Fails with INFR_ERR_BACKEND when no
+ * gfx950 device is visible: there is no CPU fallback. */
+infr_status infr_hip_create(int device_ordinal, const infr_hip_config *cfg, infr_hip_backend **out);
+void infr_hip_destroy(infr_hip_backend *be);
+
+/* Backend::name (backend.rs:631), Backend::capabilities (:632). */
+const char *infr_hip_name(const infr_hip_backend *be);
+infr_status infr_hip_capabilities_get(const infr_hip_backend *be, infr_hip_capabilities *out);
+
+/* Backend::alloc — zero-initialised, max(bytes,4) (backend.rs:651-656; CPU impl
+ * crates/infr-cpu/src/lib.rs:930-932).  Backend::alloc_uninit (:657-666): contents unspecified. */
+infr_status infr_hip_alloc(infr_hip_backend *be, size_t bytes, int32_t usage, infr_hip_buffer **out);
+infr_status infr_hip_alloc_uninit(infr_hip_backend *be, size_t bytes, int32_t usage, infr_hip_buffer **out);
+/* Buffer::len_bytes (backend.rs:424-433), Buffer::device_addr (:437-451), drop. */
+size_t infr_hip_buffer_len(const infr_hip_buffer *buf);
+uint64_t infr_hip_buffer_device_addr(const infr_hip_buffer *buf);
+void infr_hip_buffer_free(infr_hip_buffer *buf);
+
+/* Backend::upload / download (backend.rs:759-760): copy a prefix of n bytes. */
+infr_status infr_hip_upload(infr_hip_backend *be, infr_hip_buffer *dst, const void *src, size_t n);
+infr_status infr_hip_download(infr_hip_backend *be, const infr_hip_buffer *src, void *dst, size_t n);
+/* Backend::upload_range / download_range (backend.rs:700-748). */
+infr_status infr_hip_upload_range(infr_hip_backend *be, infr_hip_buffer *dst, size_t offset, const void *src, size_t n);
+infr_status infr_hip_download_range(infr_hip_backend *be, const infr_hip_buffer *src, size_t offset, void *dst, size_t n);
+/* Backend::copy_buffer (backend.rs:827-837): device-to-device prefix copy. */
+infr_status infr_hip_copy_buffer(infr_hip_backend *be, const infr_hip_buffer *src, infr_hip_buffer *dst, size_t n);
+
+/* Backend::compile (backend.rs:907): validates the graph, sizes internal scratch. */
+infr_status infr_hip_compile(infr_hip_backend *be, const infr_graph *graph, infr_hip_plan **out);
+void infr_hip_plan_free(infr_hip_plan *plan);
+/* Backend::execute (backend.rs:908): binds Input/Weight/Output handles for this call only. */
+infr_status infr_hip_execute(infr_hip_backend *be, infr_hip_plan *plan, const infr_binding *bindings, uint32_t n_bindings);
+/* Backend::sync (backend.rs:1006). */
+infr_status infr_hip_sync(infr_hip_backend *be);
+
+/* Thread-local message of the last failing call on this thread ("" if none). */
+const char *infr_hip_last_error(void);
+
+/* Per-kernel timing, the counterpart of the reference's per-op profiler seam
+ * (crates/infr-core/src/prof.rs:54-120, enabled by `prof.ops`): while enabled every kernel
+ * launch is bracketed by HIP events on the backend's stream.  Reading drains and resets. */
+typedef struct infr_hip_prof_entry {
+    char kernel[64];
+    uint64_t launches;
+    double total_ms;
+    double min_ms, max_ms;
+} infr_hip_prof_entry;
+infr_status infr_hip_prof_enable(infr_hip_backend *be, int on);
+infr_status infr_hip_prof_read(infr_hip_backend *be, infr_hip_prof_entry *out, uint32_t cap, uint32_t *n_out);
+
+/* Debug taps used by the parity tests: Op::MoeFfn's routing decision and bucketing of the
+ * LAST executed MoeFfn op of `plan` (the reference exposes the same facts through
+ * `debug.moe_counts`, crates/infr-cpu/src/lib.rs:3919-3980).  ids/weights are
+ * [rows, n_used] in rank order; any pointer may be NULL. */
+infr_status infr_hip_plan_moe_routing(infr_hip_backend *be, const infr_hip_plan *plan, uint32_t op_index,
+                                      int32_t *ids, float *weights, float *logits, float *probs);
+
+/* Standalone weight decode (reference: infr_gguf::dequant::dequant_block,
+ * crates/infr-gguf/src/dequant.rs:11-55): dst f32 buffer receives the decoded prefix of
+ * `numel` elements of `src` interpreted as `dtype`. */
+infr_status infr_hip_dequant(infr_hip_backend *be, const infr_hip_buffer *src, int32_t dtype, uint64_t numel, infr_hip_buffer *dst);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* INFR_HIP_H */

@@ -1,0 +1,831 @@
+// Host side of the gfx950 backend: the object behind the C ABI in include/infr_hip.h.
+//
+// Mirrors the reference's `Backend` contract (crates/infr-core/src/backend.rs:630-1088):
+// buffers are opaque device allocations, a plan is a validated copy of the graph plus its
+// internal scratch, execute() resolves the caller's bindings and walks the op list in
+// order, launching kernels on one HIP stream.  Nothing here computes on the CPU: when no
+// gfx950 device is present, creation fails.
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "../../include/infr_hip.h"
+#include "kernels.h"
+
+namespace {
+
+thread_local std::string g_last_error;
+
+infr_status fail(infr_status st, const char* fmt, ...) {
+    char buf[1024];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    g_last_error = buf;
+    return st;
+}
+
+#define HIP_TRY(expr)                                                                                        \
+    do {                                                                                                     \
+        hipError_t e_ = (expr);                                                                              \
+        if (e_ != hipSuccess) return fail(INFR_ERR_BACKEND, "hip: %s failed: %s", #expr, hipGetErrorString(e_)); \
+    } while (0)
+
+constexpr uint64_t kBackendMagic = 0x494e465242454e44ull;  // "INFRBEND"
+constexpr uint64_t kBufferMagic = 0x494e465242554646ull;   // "INFRBUFF"
+constexpr uint64_t kPlanMagic = 0x494e4652504c414eull;     // "INFRPLAN"
+
+bool geometry(int dtype, int* elems, int* bytes) {
+    switch (dtype) {
+        case INFR_F32: case INFR_I32: case INFR_U32: *elems = 1; *bytes = 4; return true;
+        case INFR_F16: case INFR_BF16: *elems = 1; *bytes = 2; return true;
+        case INFR_Q8_0: *elems = 32; *bytes = 34; return true;
+        case INFR_Q4K: *elems = 256; *bytes = 144; return true;
+        case INFR_Q6K: *elems = 256; *bytes = 210; return true;
+        default: return false;
+    }
+}
+
+const char* dtype_name(int dt) {
+    static const char* names[] = {"F32", "F16", "Bf16", "I32", "U32", "Q4_0", "Q4_1", "Q5_0", "Q5_1", "Q8_0",
+                                  "Q2K", "Q3K", "Q4K", "Q5K", "Q6K"};
+    if (dt >= 0 && dt < (int)(sizeof names / sizeof names[0])) return names[dt];
+    return "dtype?";
+}
+
+struct ProfSlot {
+    uint64_t launches = 0;
+    double total_ms = 0, min_ms = 1e30, max_ms = 0;
+};
+
+}  // namespace
+
+struct infr_hip_buffer {
+    uint64_t magic = kBufferMagic;
+    infr_hip_backend* be = nullptr;
+    void* dptr = nullptr;
+    size_t len = 0;  // logical length the caller asked for (>= 4)
+    size_t cap = 0;  // allocated bytes
+    int usage = 0;
+};
+
+struct MoeScratch {
+    float* logits = nullptr;  // [rows, n_expert]
+    float* probs = nullptr;   // [rows, n_expert]
+    int32_t* ids = nullptr;   // [rows, n_used]
+    float* weights = nullptr; // [rows, n_used]
+    float* h = nullptr;       // [rows, n_used, nff]
+    int rows = 0;
+};
+
+struct infr_hip_plan {
+    uint64_t magic = kPlanMagic;
+    infr_hip_backend* be = nullptr;
+    std::vector<infr_tensor_decl> tensors;
+    std::vector<infr_op> ops;
+    std::vector<uint64_t> numel;       // per tensor
+    std::vector<size_t> internal_off;  // per tensor: offset into arena (Internal only)
+    void* arena = nullptr;             // Internal tensors + per-op scratch
+    size_t arena_bytes = 0;
+    std::vector<MoeScratch> moe;       // per op (valid for MoeFfn ops)
+    int last_moe_op = -1;
+};
+
+struct infr_hip_backend {
+    uint64_t magic = kBackendMagic;
+    int device = 0;
+    hipStream_t stream = nullptr;
+    hipDeviceProp_t prop{};
+    infr_hip_config cfg{};
+    std::mutex mu;  // serialises stream submission and profiling state
+    std::atomic<int> prof_on{0};
+    std::map<std::string, ProfSlot> prof;
+    struct Pending { std::string name; hipEvent_t a, b; };
+    std::vector<Pending> pending;
+    std::vector<hipEvent_t> event_pool;
+};
+
+namespace {
+
+bool ok_backend(const infr_hip_backend* be) { return be && be->magic == kBackendMagic; }
+bool ok_buffer(const infr_hip_buffer* b) { return b && b->magic == kBufferMagic; }
+bool ok_plan(const infr_hip_plan* p) { return p && p->magic == kPlanMagic; }
+
+// Brackets one kernel launch with events when profiling is on.
+struct Timed {
+    infr_hip_backend* be;
+    const char* name;
+    hipEvent_t a = nullptr, b = nullptr;
+    Timed(infr_hip_backend* be_, const char* n) : be(be_), name(n) {
+        if (!be->prof_on.load(std::memory_order_relaxed)) return;
+        auto get = [&]() {
+            hipEvent_t e = nullptr;
+            if (!be->event_pool.empty()) { e = be->event_pool.back(); be->event_pool.pop_back(); }
+            else if (hipEventCreate(&e) != hipSuccess) e = nullptr;
+            return e;
+        };
+        a = get();
+        b = get();
+        if (a) (void)hipEventRecord(a, be->stream);
+    }
+    ~Timed() {
+        if (!a || !b) return;
+        (void)hipEventRecord(b, be->stream);
+        be->pending.push_back({name, a, b});
+    }
+};
+
+void drain_prof(infr_hip_backend* be) {
+    for (auto& p : be->pending) {
+        float ms = 0;
+        if (hipEventSynchronize(p.b) == hipSuccess && hipEventElapsedTime(&ms, p.a, p.b) == hipSuccess) {
+            ProfSlot& s = be->prof[p.name];
+            s.launches++;
+            s.total_ms += ms;
+            if (ms < s.min_ms) s.min_ms = ms;
+            if (ms > s.max_ms) s.max_ms = ms;
+        }
+        be->event_pool.push_back(p.a);
+        be->event_pool.push_back(p.b);
+    }
+    be->pending.clear();
+}
+
+size_t round_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+}  // namespace
+
+// ============================================================================ lifecycle
+extern "C" const char* infr_hip_last_error(void) { return g_last_error.c_str(); }
+
+extern "C" infr_status infr_hip_create(int device_ordinal, const infr_hip_config* cfg, infr_hip_backend** out) {
+    if (!out) return fail(INFR_ERR_INVALID, "infr_hip_create: out is null");
+    *out = nullptr;
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n <= 0)
+        return fail(INFR_ERR_BACKEND, "hip backend: no HIP device visible (%s); this backend has no CPU fallback",
+                    e == hipSuccess ? "device count 0" : hipGetErrorString(e));
+    if (device_ordinal < 0 || device_ordinal >= n)
+        return fail(INFR_ERR_INVALID, "hip backend: device ordinal %d out of range (0..%d)", device_ordinal, n - 1);
+    HIP_TRY(hipSetDevice(device_ordinal));
+    auto* be = new infr_hip_backend();
+    be->device = device_ordinal;
+    if (cfg) be->cfg = *cfg;
+    e = hipGetDeviceProperties(&be->prop, device_ordinal);
+    if (e != hipSuccess) {
+        delete be;
+        return fail(INFR_ERR_BACKEND, "hip: hipGetDeviceProperties failed: %s", hipGetErrorString(e));
+    }
+    if (strncmp(be->prop.gcnArchName, "gfx950", 6) != 0) {
+        std::string arch = be->prop.gcnArchName;
+        delete be;
+        return fail(INFR_ERR_UNSUPPORTED, "hip backend: kernels are built for gfx950 only, device %d is %s",
+                    device_ordinal, arch.c_str());
+    }
+    e = hipStreamCreateWithFlags(&be->stream, hipStreamNonBlocking);
+    if (e != hipSuccess) {
+        delete be;
+        return fail(INFR_ERR_BACKEND, "hip: hipStreamCreate failed: %s", hipGetErrorString(e));
+    }
+    *out = be;
+    return INFR_OK;
+}
+
+extern "C" void infr_hip_destroy(infr_hip_backend* be) {
+    if (!ok_backend(be)) return;
+    (void)hipSetDevice(be->device);
+    (void)hipStreamSynchronize(be->stream);
+    for (auto& p : be->pending) { (void)hipEventDestroy(p.a); (void)hipEventDestroy(p.b); }
+    for (auto e : be->event_pool) (void)hipEventDestroy(e);
+    (void)hipStreamDestroy(be->stream);
+    be->magic = 0;
+    delete be;
+}
+
+extern "C" const char* infr_hip_name(const infr_hip_backend* be) { return ok_backend(be) ? "hip-gfx950" : ""; }
+
+extern "C" infr_status infr_hip_capabilities_get(const infr_hip_backend* be, infr_hip_capabilities* out) {
+    if (!ok_backend(be) || !out) return fail(INFR_ERR_INVALID, "capabilities: bad handle");
+    memset(out, 0, sizeof *out);
+    snprintf(out->name, sizeof out->name, "hip-gfx950 (%s)", be->prop.name);
+    out->f16 = 1; out->bf16 = 1; out->i8 = 1; out->i8_dot = 1;
+    out->subgroup_min = 64; out->subgroup_max = 64;
+    out->integrated = 0;
+    out->compute_units = (uint32_t)be->prop.multiProcessorCount;
+    out->buffer_device_address = 1;
+    out->max_shared_memory_bytes = (uint32_t)be->prop.sharedMemPerBlock;
+    out->unified_memory = 0;
+    out->decode_replay = 0;
+    out->combined_gu = 0;
+    out->graph_input_inplace = 1;
+    out->device_memory_bytes = (uint64_t)be->prop.totalGlobalMem;
+    return INFR_OK;
+}
+
+// ============================================================================ memory
+static infr_status alloc_impl(infr_hip_backend* be, size_t bytes, int32_t usage, bool zero, infr_hip_buffer** out) {
+    if (!ok_backend(be) || !out) return fail(INFR_ERR_INVALID, "alloc: bad handle");
+    *out = nullptr;
+    if (usage < INFR_USAGE_WEIGHTS || usage > INFR_USAGE_HOST_WEIGHTS)
+        return fail(INFR_ERR_INVALID, "alloc: unknown buffer usage %d", usage);
+    size_t len = bytes < 4 ? 4 : bytes;  // reference: vec![0u8; bytes.max(4)]
+    size_t cap = round_up(len, 256);
+    std::lock_guard<std::mutex> lk(be->mu);
+    HIP_TRY(hipSetDevice(be->device));
+    void* p = nullptr;
+    hipError_t e = hipMalloc(&p, cap);
+    if (e != hipSuccess)
+        return fail(INFR_ERR_BACKEND, "alloc: hipMalloc(%zu) failed: %s", cap, hipGetErrorString(e));
+    if (zero) infr::launch_fill_zero(be->stream, p, cap);
+    auto* b = new infr_hip_buffer();
+    b->be = be; b->dptr = p; b->len = len; b->cap = cap; b->usage = usage;
+    *out = b;
+    return INFR_OK;
+}
+
+extern "C" infr_status infr_hip_alloc(infr_hip_backend* be, size_t bytes, int32_t usage, infr_hip_buffer** out) {
+    return alloc_impl(be, bytes, usage, true, out);
+}
+extern "C" infr_status infr_hip_alloc_uninit(infr_hip_backend* be, size_t bytes, int32_t usage, infr_hip_buffer** out) {
+    return alloc_impl(be, bytes, usage, false, out);
+}
+extern "C" size_t infr_hip_buffer_len(const infr_hip_buffer* buf) { return ok_buffer(buf) ? buf->len : 0; }
+extern "C" uint64_t infr_hip_buffer_device_addr(const infr_hip_buffer* buf) {
+    return ok_buffer(buf) ? (uint64_t)(uintptr_t)buf->dptr : 0;
+}
+extern "C" void infr_hip_buffer_free(infr_hip_buffer* buf) {
+    if (!ok_buffer(buf)) return;
+    infr_hip_backend* be = buf->be;
+    if (ok_backend(be)) {
+        std::lock_guard<std::mutex> lk(be->mu);
+        (void)hipSetDevice(be->device);
+        (void)hipStreamSynchronize(be->stream);  // work that still reads it must drain first
+        (void)hipFree(buf->dptr);
+    }
+    buf->magic = 0;
+    delete buf;
+}
+
+static infr_status check_owned(infr_hip_backend* be, const infr_hip_buffer* b, const char* what) {
+    if (!ok_backend(be)) return fail(INFR_ERR_INVALID, "%s: backend handle is not a hip backend", what);
+    if (!ok_buffer(b)) return fail(INFR_ERR_INVALID, "%s: buffer is not a hip buffer", what);
+    if (b->be != be) return fail(INFR_ERR_INVALID, "%s: buffer belongs to another backend instance", what);
+    return INFR_OK;
+}
+
+extern "C" infr_status infr_hip_upload_range(infr_hip_backend* be, infr_hip_buffer* dst, size_t offset,
+                                             const void* src, size_t n) {
+    if (infr_status st = check_owned(be, dst, "upload")) return st;
+    if (n && !src) return fail(INFR_ERR_INVALID, "upload: src is null");
+    if (offset > dst->len || n > dst->len - offset)
+        return fail(INFR_ERR_BACKEND, "upload: byte range %zu..%zu exceeds buffer size %zu", offset, offset + n, dst->len);
+    if (n == 0) return INFR_OK;
+    std::lock_guard<std::mutex> lk(be->mu);
+    HIP_TRY(hipSetDevice(be->device));
+    HIP_TRY(hipMemcpyAsync((char*)dst->dptr + offset, src, n, hipMemcpyHostToDevice, be->stream));
+    HIP_TRY(hipStreamSynchronize(be->stream));  // src may be freed by the caller on return
+    return INFR_OK;
+}
+extern "C" infr_status infr_hip_upload(infr_hip_backend* be, infr_hip_buffer* dst, const void* src, size_t n) {
+    return infr_hip_upload_range(be, dst, 0, src, n);
+}
+extern "C" infr_status infr_hip_download_range(infr_hip_backend* be, const infr_hip_buffer* src, size_t offset,
+                                               void* dst, size_t n) {
+    if (infr_status st = check_owned(be, src, "download")) return st;
+    if (n && !dst) return fail(INFR_ERR_INVALID, "download: dst is null");
+    if (offset > src->len || n > src->len - offset)
+        return fail(INFR_ERR_BACKEND, "download_range: byte range %zu..%zu exceeds committed buffer size %zu", offset,
+                    offset + n, src->len);
+    std::lock_guard<std::mutex> lk(be->mu);
+    HIP_TRY(hipSetDevice(be->device));
+    if (n) HIP_TRY(hipMemcpyAsync(dst, (const char*)src->dptr + offset, n, hipMemcpyDeviceToHost, be->stream));
+    HIP_TRY(hipStreamSynchronize(be->stream));
+    return INFR_OK;
+}
+extern "C" infr_status infr_hip_download(infr_hip_backend* be, const infr_hip_buffer* src, void* dst, size_t n) {
+    return infr_hip_download_range(be, src, 0, dst, n);
+}
+extern "C" infr_status infr_hip_copy_buffer(infr_hip_backend* be, const infr_hip_buffer* src, infr_hip_buffer* dst,
+                                            size_t n) {
+    if (infr_status st = check_owned(be, src, "copy_buffer")) return st;
+    if (infr_status st = check_owned(be, dst, "copy_buffer")) return st;
+    if (n > src->len || n > dst->len)
+        return fail(INFR_ERR_BACKEND, "copy_buffer: %zu bytes exceed src (%zu) or dst (%zu)", n, src->len, dst->len);
+    if (n == 0) return INFR_OK;
+    std::lock_guard<std::mutex> lk(be->mu);
+    HIP_TRY(hipSetDevice(be->device));
+    HIP_TRY(hipMemcpyAsync(dst->dptr, src->dptr, n, hipMemcpyDeviceToDevice, be->stream));
+    return INFR_OK;
+}
+
+extern "C" infr_status infr_hip_sync(infr_hip_backend* be) {
+    if (!ok_backend(be)) return fail(INFR_ERR_INVALID, "sync: bad handle");
+    std::lock_guard<std::mutex> lk(be->mu);
+    HIP_TRY(hipSetDevice(be->device));
+    HIP_TRY(hipStreamSynchronize(be->stream));
+    HIP_TRY(hipGetLastError());
+    return INFR_OK;
+}
+
+// ============================================================================ compile
+namespace {
+
+struct Check {
+    const infr_hip_plan& p;
+    std::string err;
+    infr_status st = INFR_OK;
+    bool tensor(uint32_t id, const char* role, bool optional = false) {
+        if (id == INFR_NO_TENSOR && optional) return true;
+        if (id >= p.tensors.size()) {
+            set(INFR_ERR_INVALID, std::string(role) + ": tensor id out of range");
+            return false;
+        }
+        return true;
+    }
+    void set(infr_status s, const std::string& m) {
+        if (st == INFR_OK) { st = s; err = m; }
+    }
+    int dt(uint32_t id) const { return p.tensors[id].dtype; }
+    uint64_t n(uint32_t id) const { return p.numel[id]; }
+    int kind(uint32_t id) const { return p.tensors[id].kind; }
+    void want_f32(uint32_t id, const char* role) {
+        if (dt(id) != INFR_F32) set(INFR_ERR_UNSUPPORTED, std::string(role) + " must be F32, got " + dtype_name(dt(id)));
+    }
+    void want_numel(uint32_t id, uint64_t expect, const char* role) {
+        if (n(id) != expect)
+            set(INFR_ERR_INVALID, std::string(role) + ": declared " + std::to_string(n(id)) + " elements, op needs " +
+                                      std::to_string(expect));
+    }
+    void want_weight_dtype(uint32_t id, uint64_t in_f, const char* role) {
+        int be = 0, bb = 0;
+        if (!geometry(dt(id), &be, &bb) || dt(id) == INFR_I32 || dt(id) == INFR_U32) {
+            set(INFR_ERR_UNSUPPORTED, std::string(role) + ": weight dtype " + dtype_name(dt(id)) +
+                                          " has no decode on this backend (F32/F16/Bf16/Q8_0/Q4K/Q6K)");
+            return;
+        }
+        if (in_f % (uint64_t)be != 0)
+            set(INFR_ERR_INVALID, std::string(role) + ": row length " + std::to_string(in_f) +
+                                      " is not a whole number of " + dtype_name(dt(id)) + " blocks");
+    }
+    void want_writable(uint32_t id, const char* role) {
+        if (kind(id) == INFR_KIND_WEIGHT) set(INFR_ERR_INVALID, std::string(role) + ": destination is a Weight");
+    }
+};
+
+size_t tensor_bytes(const infr_tensor_decl& t, uint64_t numel) {
+    int be = 1, bb = 4;
+    if (!geometry(t.dtype, &be, &bb)) return 0;
+    return (size_t)((numel + (uint64_t)be - 1) / (uint64_t)be) * (size_t)bb;
+}
+
+}  // namespace
+
+extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* g, infr_hip_plan** out) {
+    if (!ok_backend(be) || !g || !out) return fail(INFR_ERR_INVALID, "compile: bad handle");
+    *out = nullptr;
+    if ((g->n_tensors && !g->tensors) || (g->n_ops && !g->ops)) return fail(INFR_ERR_INVALID, "compile: null arrays");
+    auto plan = new infr_hip_plan();
+    plan->be = be;
+    plan->tensors.assign(g->tensors, g->tensors + g->n_tensors);
+    plan->ops.assign(g->ops, g->ops + g->n_ops);
+    plan->numel.resize(g->n_tensors);
+    plan->internal_off.assign(g->n_tensors, (size_t)-1);
+    plan->moe.resize(g->n_ops);
+    auto bail = [&](infr_status st, const std::string& m) {
+        delete plan;
+        return fail(st, "%s", m.c_str());
+    };
+    size_t arena = 0;
+    for (uint32_t i = 0; i < g->n_tensors; i++) {
+        const infr_tensor_decl& t = plan->tensors[i];
+        if (t.rank > 4) return bail(INFR_ERR_INVALID, "compile: tensor rank > 4");
+        if (t.kind < INFR_KIND_INPUT || t.kind > INFR_KIND_OUTPUT) return bail(INFR_ERR_INVALID, "compile: bad tensor kind");
+        uint64_t n = 1;
+        for (uint32_t d = 0; d < t.rank; d++) n *= t.shape[d];
+        plan->numel[i] = n;
+        if (t.kind == INFR_KIND_INTERNAL) {
+            if (t.dtype != INFR_F32) return bail(INFR_ERR_UNSUPPORTED, "compile: Internal tensors must be F32");
+            plan->internal_off[i] = arena;
+            arena += round_up((size_t)n * 4 + 4, 256);
+        }
+    }
+    Check c{*plan};
+    std::vector<size_t> moe_off(g->n_ops, 0);
+    for (uint32_t oi = 0; oi < g->n_ops && c.st == INFR_OK; oi++) {
+        const infr_op& op = plan->ops[oi];
+        switch (op.kind) {
+            case INFR_OP_MOE_FFN: {
+                const infr_op_moe_ffn& m = op.u.moe_ffn;
+                bool ok = c.tensor(m.x, "MoeFfn.x") && c.tensor(m.router_x, "MoeFfn.router_x") &&
+                          c.tensor(m.router, "MoeFfn.router") && c.tensor(m.gate_exps, "MoeFfn.gate_exps") &&
+                          c.tensor(m.down_exps, "MoeFfn.down_exps") && c.tensor(m.dst, "MoeFfn.dst") &&
+                          c.tensor(m.down_scale, "MoeFfn.down_scale", true) &&
+                          c.tensor(m.exp_probs_b, "MoeFfn.exp_probs_b", true) &&
+                          c.tensor(m.expert_ids, "MoeFfn.expert_ids", true) &&
+                          (m.fused_gate_up || c.tensor(m.up_exps, "MoeFfn.up_exps"));
+                if (!ok) break;
+                if (!m.ne || !m.n_expert || !m.n_used || !m.n_ff_exp || m.n_used > m.n_expert) {
+                    c.set(INFR_ERR_INVALID, "MoeFfn: ne/n_expert/n_used/n_ff_exp must be positive and n_used <= n_expert");
+                    break;
+                }
+                if (m.n_expert > 2048) { c.set(INFR_ERR_UNSUPPORTED, "MoeFfn: n_expert > 2048"); break; }
+                if (m.has_ep_band) {
+                    c.set(INFR_ERR_UNSUPPORTED, "MoeFfn: ep_band (expert-parallel shard) is a multi-device lowering; "
+                                                "this backend runs all experts on one device");
+                    break;
+                }
+                // Same refusals as the reference (crates/infr-cpu/src/lib.rs:3613-3629).
+                if (m.has_swiglu_clamp && (m.act == INFR_ACT_SIGMOID || m.weight_before)) {
+                    c.set(INFR_ERR_INVALID, "MoeFfn: swiglu_clamp is defined for the gated SiLU/GELU forms with "
+                                            "output-side weighting only");
+                    break;
+                }
+                if (m.expert_ids != INFR_NO_TENSOR && (m.exp_probs_b != INFR_NO_TENSOR || m.n_expert_groups > 1)) {
+                    c.set(INFR_ERR_INVALID, "MoeFfn: expert_ids (hash routing) supplies the selection, so exp_probs_b "
+                                            "and group routing must be absent");
+                    break;
+                }
+                if (m.act < INFR_ACT_SILU || m.act > INFR_ACT_SIGMOID || m.gating < INFR_GATING_SOFTMAX ||
+                    m.gating > INFR_GATING_SQRT_SOFTPLUS) {
+                    c.set(INFR_ERR_INVALID, "MoeFfn: unknown activation or gating");
+                    break;
+                }
+                if (m.n_expert_groups > 1 && m.n_expert % m.n_expert_groups != 0) {
+                    c.set(INFR_ERR_INVALID, "MoeFfn: n_expert is not a multiple of n_expert_groups");
+                    break;
+                }
+                c.want_f32(m.x, "MoeFfn.x");
+                c.want_f32(m.router_x, "MoeFfn.router_x");
+                c.want_f32(m.dst, "MoeFfn.dst");
+                c.want_writable(m.dst, "MoeFfn.dst");
+                if (c.n(m.x) % m.ne != 0) { c.set(INFR_ERR_INVALID, "MoeFfn.x: element count is not a multiple of ne"); break; }
+                uint64_t rows = c.n(m.x) / m.ne;  // reference: rows = xs.len() / ne (lib.rs:3644)
+                c.want_numel(m.router_x, rows * m.ne, "MoeFfn.router_x");
+                c.want_numel(m.dst, rows * m.ne, "MoeFfn.dst");
+                c.want_numel(m.router, (uint64_t)m.n_expert * m.ne, "MoeFfn.router");
+                uint64_t gu_rows = m.fused_gate_up ? 2ull * m.n_ff_exp : m.n_ff_exp;
+                c.want_numel(m.gate_exps, (uint64_t)m.n_expert * gu_rows * m.ne, "MoeFfn.gate_exps");
+                if (!m.fused_gate_up) c.want_numel(m.up_exps, (uint64_t)m.n_expert * m.n_ff_exp * m.ne, "MoeFfn.up_exps");
+                c.want_numel(m.down_exps, (uint64_t)m.n_expert * m.ne * m.n_ff_exp, "MoeFfn.down_exps");
+                c.want_weight_dtype(m.router, m.ne, "MoeFfn.router");
+                c.want_weight_dtype(m.gate_exps, m.ne, "MoeFfn.gate_exps");
+                if (!m.fused_gate_up) c.want_weight_dtype(m.up_exps, m.ne, "MoeFfn.up_exps");
+                c.want_weight_dtype(m.down_exps, m.n_ff_exp, "MoeFfn.down_exps");
+                if (m.down_scale != INFR_NO_TENSOR) { c.want_f32(m.down_scale, "MoeFfn.down_scale"); c.want_numel(m.down_scale, m.n_expert, "MoeFfn.down_scale"); }
+                if (m.exp_probs_b != INFR_NO_TENSOR) { c.want_f32(m.exp_probs_b, "MoeFfn.exp_probs_b"); c.want_numel(m.exp_probs_b, m.n_expert, "MoeFfn.exp_probs_b"); }
+                if (m.expert_ids != INFR_NO_TENSOR) {
+                    if (c.dt(m.expert_ids) != INFR_I32) c.set(INFR_ERR_UNSUPPORTED, "MoeFfn.expert_ids must be I32");
+                    if (c.n(m.expert_ids) < rows * m.n_used) c.set(INFR_ERR_INVALID, "MoeFfn.expert_ids holds fewer than rows*n_used slots");
+                }
+                if (rows > 0x7fffffffull / (m.n_used * (uint64_t)m.n_ff_exp + 1)) { c.set(INFR_ERR_UNSUPPORTED, "MoeFfn: rows too large"); break; }
+                // scratch: logits, probs, ids, weights, h
+                moe_off[oi] = arena;
+                arena += round_up((size_t)rows * m.n_expert * 4 + 4, 256) * 2;
+                arena += round_up((size_t)rows * m.n_used * 4 + 4, 256) * 2;
+                arena += round_up((size_t)rows * m.n_used * m.n_ff_exp * 4 + 4, 256);
+                plan->moe[oi].rows = (int)rows;
+                break;
+            }
+            case INFR_OP_LINEAR: {
+                const infr_op_linear& l = op.u.linear;
+                if (!(c.tensor(l.x, "Linear.x") && c.tensor(l.weight, "Linear.weight") && c.tensor(l.dst, "Linear.dst"))) break;
+                if (!l.in_f || !l.out_f) { c.set(INFR_ERR_INVALID, "Linear: in_f/out_f must be positive"); break; }
+                c.want_f32(l.x, "Linear.x");
+                c.want_f32(l.dst, "Linear.dst");
+                c.want_writable(l.dst, "Linear.dst");
+                c.want_numel(l.x, (uint64_t)l.m * l.in_f, "Linear.x");
+                c.want_numel(l.dst, (uint64_t)l.m * l.out_f, "Linear.dst");
+                c.want_weight_dtype(l.weight, l.in_f, "Linear.weight");
+                if (c.n(l.weight) % l.in_f != 0 || l.w_off % l.in_f != 0 ||
+                    (uint64_t)l.w_off / l.in_f + l.out_f > c.n(l.weight) / l.in_f)
+                    c.set(INFR_ERR_INVALID, "Linear: w_off/out_f select rows outside the weight tensor");
+                break;
+            }
+            case INFR_OP_GATED_ACT: {
+                const infr_op_gated_act& a = op.u.gated_act;
+                if (!(c.tensor(a.gate, "GatedAct.gate") && c.tensor(a.up, "GatedAct.up") && c.tensor(a.dst, "GatedAct.dst"))) break;
+                c.want_f32(a.gate, "GatedAct.gate");
+                c.want_f32(a.up, "GatedAct.up");
+                c.want_f32(a.dst, "GatedAct.dst");
+                c.want_writable(a.dst, "GatedAct.dst");
+                c.want_numel(a.dst, (uint64_t)a.rows * a.nff, "GatedAct.dst");
+                if (a.has_swiglu_clamp && a.act == INFR_ACT_SIGMOID)
+                    c.set(INFR_ERR_INVALID, "GatedAct: swiglu_clamp is defined for the gated SiLU/GELU forms only");
+                if (a.act < INFR_ACT_SILU || a.act > INFR_ACT_SIGMOID) c.set(INFR_ERR_INVALID, "GatedAct: unknown activation");
+                {
+                    // highest element each operand is read at must exist
+                    uint64_t rows = a.rows, nff = a.nff;
+                    if (rows && nff) {
+                        uint64_t umax = (a.up_stride == 0 ? (rows - 1) * nff : (rows - 1) * (uint64_t)a.up_stride) + a.up_off + nff;
+                        uint64_t gmax;
+                        if (a.gate_block_width > 0) {
+                            uint64_t headw = a.gate_block_width / 2;
+                            if (headw == 0) { c.set(INFR_ERR_INVALID, "GatedAct: gate_block_width < 2"); break; }
+                            uint64_t head = (nff - 1) / headw, off = (nff - 1) % headw;
+                            gmax = (rows - 1) * (uint64_t)a.gate_stride + head * a.gate_block_width + headw + off + 1;
+                        } else {
+                            gmax = (a.gate_stride > 0 ? (rows - 1) * (uint64_t)a.gate_stride : (rows - 1) * nff) + nff;
+                        }
+                        if (umax > c.n(a.up)) c.set(INFR_ERR_INVALID, "GatedAct.up: strides read past the tensor");
+                        if (gmax > c.n(a.gate)) c.set(INFR_ERR_INVALID, "GatedAct.gate: strides read past the tensor");
+                    }
+                }
+                break;
+            }
+            case INFR_OP_ADD: {
+                const infr_op_add& a = op.u.add;
+                if (!(c.tensor(a.a, "Add.a") && c.tensor(a.b, "Add.b") && c.tensor(a.dst, "Add.dst"))) break;
+                c.want_f32(a.a, "Add.a"); c.want_f32(a.b, "Add.b"); c.want_f32(a.dst, "Add.dst");
+                c.want_writable(a.dst, "Add.dst");
+                if (c.n(a.a) < a.n || c.n(a.b) < a.n || c.n(a.dst) < a.n) c.set(INFR_ERR_INVALID, "Add: n exceeds an operand");
+                break;
+            }
+            case INFR_OP_MOE_SHARED_EXPERT_ADD: {
+                const infr_op_moe_shared_expert_add& a = op.u.moe_shared_expert_add;
+                if (!(c.tensor(a.moe, "MoeSharedExpertAdd.moe") && c.tensor(a.shexp, "MoeSharedExpertAdd.shexp") &&
+                      c.tensor(a.gate, "MoeSharedExpertAdd.gate") && c.tensor(a.dst, "MoeSharedExpertAdd.dst"))) break;
+                c.want_f32(a.moe, "MoeSharedExpertAdd.moe"); c.want_f32(a.shexp, "MoeSharedExpertAdd.shexp");
+                c.want_f32(a.gate, "MoeSharedExpertAdd.gate"); c.want_f32(a.dst, "MoeSharedExpertAdd.dst");
+                c.want_writable(a.dst, "MoeSharedExpertAdd.dst");
+                uint64_t tot = (uint64_t)a.rows * a.n;
+                if (c.n(a.moe) < tot || c.n(a.shexp) < tot || c.n(a.dst) < tot || c.n(a.gate) < a.rows)
+                    c.set(INFR_ERR_INVALID, "MoeSharedExpertAdd: rows*n exceeds an operand");
+                break;
+            }
+            default:
+                c.set(INFR_ERR_UNSUPPORTED, "compile: op kind " + std::to_string(op.kind) +
+                                                " is not on the routed-expert FFN path this backend implements");
+        }
+        if (c.st != INFR_OK) c.err = "op " + std::to_string(oi) + ": " + c.err;
+    }
+    if (c.st != INFR_OK) return bail(c.st, c.err);
+
+    std::lock_guard<std::mutex> lk(be->mu);
+    hipError_t e = hipSetDevice(be->device);
+    if (e == hipSuccess && arena) e = hipMalloc(&plan->arena, arena);
+    if (e != hipSuccess) return bail(INFR_ERR_BACKEND, std::string("compile: scratch hipMalloc failed: ") + hipGetErrorString(e));
+    plan->arena_bytes = arena;
+    for (uint32_t oi = 0; oi < g->n_ops; oi++) {
+        if (plan->ops[oi].kind != INFR_OP_MOE_FFN) continue;
+        const infr_op_moe_ffn& m = plan->ops[oi].u.moe_ffn;
+        MoeScratch& s = plan->moe[oi];
+        char* p = (char*)plan->arena + moe_off[oi];
+        size_t rows = (size_t)s.rows;
+        s.logits = (float*)p; p += round_up(rows * m.n_expert * 4 + 4, 256);
+        s.probs = (float*)p;  p += round_up(rows * m.n_expert * 4 + 4, 256);
+        s.ids = (int32_t*)p;  p += round_up(rows * m.n_used * 4 + 4, 256);
+        s.weights = (float*)p; p += round_up(rows * m.n_used * 4 + 4, 256);
+        s.h = (float*)p;
+    }
+    *out = plan;
+    return INFR_OK;
+}
+
+extern "C" void infr_hip_plan_free(infr_hip_plan* plan) {
+    if (!ok_plan(plan)) return;
+    infr_hip_backend* be = plan->be;
+    if (ok_backend(be)) {
+        std::lock_guard<std::mutex> lk(be->mu);
+        (void)hipSetDevice(be->device);
+        (void)hipStreamSynchronize(be->stream);
+        if (plan->arena) (void)hipFree(plan->arena);
+    }
+    plan->magic = 0;
+    delete plan;
+}
+
+// ============================================================================ execute
+extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* plan, const infr_binding* bindings,
+                                        uint32_t n_bindings) {
+    if (!ok_backend(be)) return fail(INFR_ERR_INVALID, "execute: backend handle is not a hip backend");
+    if (!ok_plan(plan) || plan->be != be) return fail(INFR_ERR_BACKEND, "hip backend: incompatible plan");
+    if (n_bindings && !bindings) return fail(INFR_ERR_INVALID, "execute: bindings is null");
+    const size_t nt = plan->tensors.size();
+    std::vector<const infr_hip_buffer*> bound(nt, nullptr);
+    for (uint32_t i = 0; i < n_bindings; i++) {
+        if (bindings[i].tensor >= nt) return fail(INFR_ERR_INVALID, "execute: binding for tensor %u, graph has %zu", bindings[i].tensor, nt);
+        if (infr_status st = check_owned(be, bindings[i].buffer, "execute")) return st;
+        bound[bindings[i].tensor] = bindings[i].buffer;  // re-binding an id overwrites (backend.rs:582-590)
+    }
+    // Resolve every tensor the ops touch to a device pointer, checking extents.
+    std::vector<void*> ptr(nt, nullptr);
+    for (size_t i = 0; i < nt; i++) {
+        const infr_tensor_decl& t = plan->tensors[i];
+        if (t.kind == INFR_KIND_INTERNAL) {
+            ptr[i] = (char*)plan->arena + plan->internal_off[i];
+        } else if (bound[i]) {
+            size_t need = tensor_bytes(t, plan->numel[i]);
+            if (bound[i]->len < need)
+                return fail(INFR_ERR_BACKEND, "execute: tensor %zu needs %zu bytes, bound buffer holds %zu", i, need, bound[i]->len);
+            ptr[i] = bound[i]->dptr;
+        }
+    }
+    auto need = [&](uint32_t id, const char* role) -> bool {
+        if (id == INFR_NO_TENSOR) return true;
+        if (!ptr[id]) {
+            const char* k = plan->tensors[id].kind == INFR_KIND_WEIGHT ? "Weight" : plan->tensors[id].kind == INFR_KIND_INPUT ? "Input" : "Output";
+            fail(INFR_ERR_BACKEND, "hip backend: unbound %s (%s, tensor %u)", k, role, id);
+            return false;
+        }
+        return true;
+    };
+    std::lock_guard<std::mutex> lk(be->mu);
+    HIP_TRY(hipSetDevice(be->device));
+    hipStream_t s = be->stream;
+    const int n_cu = be->prop.multiProcessorCount;
+    for (size_t oi = 0; oi < plan->ops.size(); oi++) {
+        const infr_op& op = plan->ops[oi];
+        switch (op.kind) {
+            case INFR_OP_MOE_FFN: {
+                const infr_op_moe_ffn& m = op.u.moe_ffn;
+                if (!(need(m.x, "MoeFfn.x") && need(m.router_x, "MoeFfn.router_x") && need(m.router, "MoeFfn.router") &&
+                      need(m.gate_exps, "MoeFfn.gate_exps") && (m.fused_gate_up || need(m.up_exps, "MoeFfn.up_exps")) &&
+                      need(m.down_exps, "MoeFfn.down_exps") && need(m.dst, "MoeFfn.dst") &&
+                      need(m.down_scale, "MoeFfn.down_scale") && need(m.exp_probs_b, "MoeFfn.exp_probs_b") &&
+                      need(m.expert_ids, "MoeFfn.expert_ids")))
+                    return INFR_ERR_BACKEND;
+                MoeScratch& sc = plan->moe[oi];
+                const int rows = sc.rows;
+                plan->last_moe_op = (int)oi;
+                if (rows == 0) break;
+                int re = 1, rb = 4;
+                geometry(plan->tensors[m.router].dtype, &re, &rb);
+                size_t router_row_bytes = (size_t)(m.ne / re) * rb;
+                {
+                    Timed t(be, "router_logits");
+                    if (!infr::launch_router_logits(s, (const uint8_t*)ptr[m.router], plan->tensors[m.router].dtype,
+                                                    router_row_bytes, (const float*)ptr[m.router_x], (int)m.ne,
+                                                    (int)m.n_expert, rows, sc.logits))
+                        return fail(INFR_ERR_UNSUPPORTED, "MoeFfn: ne=%u does not fit the router kernel's LDS budget", m.ne);
+                }
+                {
+                    infr::RouteParams rp{};
+                    rp.logits = sc.logits; rp.n_expert = (int)m.n_expert; rp.n_used = (int)m.n_used; rp.rows = rows;
+                    rp.gating = m.gating; rp.norm_w = (int)m.norm_w; rp.scale = m.scale;
+                    rp.exp_probs_b = m.exp_probs_b == INFR_NO_TENSOR ? nullptr : (const float*)ptr[m.exp_probs_b];
+                    rp.n_groups = (int)m.n_expert_groups; rp.n_groups_used = (int)m.n_expert_groups_used;
+                    rp.expert_ids = m.expert_ids == INFR_NO_TENSOR ? nullptr : (const int32_t*)ptr[m.expert_ids];
+                    rp.ids = sc.ids; rp.weights = sc.weights; rp.probs = sc.probs;
+                    Timed t(be, "route_topk");
+                    infr::launch_route(s, rp);
+                }
+                infr::MoeGemvParams gp{};
+                gp.ids = sc.ids; gp.weights = sc.weights;
+                gp.gate_dt = plan->tensors[m.gate_exps].dtype;
+                gp.down_dt = plan->tensors[m.down_exps].dtype;
+                size_t gbytes = tensor_bytes(plan->tensors[m.gate_exps], plan->numel[m.gate_exps]);
+                size_t dbytes = tensor_bytes(plan->tensors[m.down_exps], plan->numel[m.down_exps]);
+                gp.gate = (const uint8_t*)ptr[m.gate_exps];
+                gp.gate_stride = gbytes / m.n_expert;  // reference: gst = gb.len() / n_expert (lib.rs:3666)
+                if (m.fused_gate_up) {
+                    // gate rows first, up rows second inside each expert slice
+                    gp.up = gp.gate + gp.gate_stride / 2;
+                    gp.up_stride = gp.gate_stride;
+                    gp.up_dt = gp.gate_dt;
+                } else {
+                    size_t ubytes = tensor_bytes(plan->tensors[m.up_exps], plan->numel[m.up_exps]);
+                    gp.up = (const uint8_t*)ptr[m.up_exps];
+                    gp.up_stride = ubytes / m.n_expert;
+                    gp.up_dt = plan->tensors[m.up_exps].dtype;
+                }
+                gp.down = (const uint8_t*)ptr[m.down_exps];
+                gp.down_stride = dbytes / m.n_expert;
+                gp.down_scale = m.down_scale == INFR_NO_TENSOR ? nullptr : (const float*)ptr[m.down_scale];
+                gp.rows = rows; gp.ne = (int)m.ne; gp.nff = (int)m.n_ff_exp; gp.n_used = (int)m.n_used; gp.n_expert = (int)m.n_expert;
+                gp.act = m.act; gp.has_clamp = (int)m.has_swiglu_clamp; gp.clamp = m.swiglu_clamp;
+                gp.weight_before = (int)m.weight_before; gp.fused_gate_up = (int)m.fused_gate_up;
+                gp.h = sc.h; gp.dst = (float*)ptr[m.dst]; gp.n_cu = n_cu;
+                gp.x = (const float*)ptr[m.x];
+                {
+                    Timed t(be, "moe_gate_up");
+                    infr::launch_moe_gate_up(s, gp);
+                }
+                gp.x = nullptr;
+                {
+                    Timed t(be, "moe_down_combine");
+                    infr::launch_moe_down_combine(s, gp);
+                }
+                break;
+            }
+            case INFR_OP_LINEAR: {
+                const infr_op_linear& l = op.u.linear;
+                if (!(need(l.x, "Linear.x") && need(l.weight, "Linear.weight") && need(l.dst, "Linear.dst"))) return INFR_ERR_BACKEND;
+                if (l.m == 0) break;
+                int we = 1, wb = 4;
+                geometry(plan->tensors[l.weight].dtype, &we, &wb);
+                size_t row_bytes = (size_t)(l.in_f / we) * wb;
+                const uint8_t* w = (const uint8_t*)ptr[l.weight] + (size_t)(l.w_off / l.in_f) * row_bytes;
+                Timed t(be, "linear");
+                infr::launch_linear(s, (const float*)ptr[l.x], w, plan->tensors[l.weight].dtype, row_bytes, (int)l.m,
+                                    (int)l.in_f, (int)l.out_f, (float*)ptr[l.dst], n_cu);
+                break;
+            }
+            case INFR_OP_GATED_ACT: {
+                const infr_op_gated_act& a = op.u.gated_act;
+                if (!(need(a.gate, "GatedAct.gate") && need(a.up, "GatedAct.up") && need(a.dst, "GatedAct.dst"))) return INFR_ERR_BACKEND;
+                Timed t(be, "gated_act");
+                infr::launch_gated_act(s, (const float*)ptr[a.gate], (const float*)ptr[a.up], (float*)ptr[a.dst], (int)a.rows,
+                                       (int)a.nff, a.act, (int)a.up_off, (int)a.up_stride, (int)a.gate_stride,
+                                       (int)a.gate_block_width, (int)a.has_swiglu_clamp, a.swiglu_clamp);
+                break;
+            }
+            case INFR_OP_ADD: {
+                const infr_op_add& a = op.u.add;
+                if (!(need(a.a, "Add.a") && need(a.b, "Add.b") && need(a.dst, "Add.dst"))) return INFR_ERR_BACKEND;
+                Timed t(be, "add");
+                infr::launch_add(s, (const float*)ptr[a.a], (const float*)ptr[a.b], (float*)ptr[a.dst], a.n);
+                break;
+            }
+            case INFR_OP_MOE_SHARED_EXPERT_ADD: {
+                const infr_op_moe_shared_expert_add& a = op.u.moe_shared_expert_add;
+                if (!(need(a.moe, "MoeSharedExpertAdd.moe") && need(a.shexp, "MoeSharedExpertAdd.shexp") &&
+                      need(a.gate, "MoeSharedExpertAdd.gate") && need(a.dst, "MoeSharedExpertAdd.dst")))
+                    return INFR_ERR_BACKEND;
+                Timed t(be, "moe_shared_expert_add");
+                infr::launch_moe_shared_expert_add(s, (const float*)ptr[a.moe], (const float*)ptr[a.shexp],
+                                                   (const float*)ptr[a.gate], (float*)ptr[a.dst], (int)a.rows, (int)a.n);
+                break;
+            }
+            default:
+                return fail(INFR_ERR_UNSUPPORTED, "execute: op kind %d", op.kind);
+        }
+    }
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(INFR_ERR_BACKEND, "execute: kernel launch failed: %s", hipGetErrorString(e));
+    return INFR_OK;
+}
+
+// ============================================================================ taps
+extern "C" infr_status infr_hip_prof_enable(infr_hip_backend* be, int on) {
+    if (!ok_backend(be)) return fail(INFR_ERR_INVALID, "prof: bad handle");
+    std::lock_guard<std::mutex> lk(be->mu);
+    be->prof_on.store(on ? 1 : 0);
+    return INFR_OK;
+}
+
+extern "C" infr_status infr_hip_prof_read(infr_hip_backend* be, infr_hip_prof_entry* out, uint32_t cap, uint32_t* n_out) {
+    if (!ok_backend(be) || !n_out) return fail(INFR_ERR_INVALID, "prof: bad handle");
+    std::lock_guard<std::mutex> lk(be->mu);
+    HIP_TRY(hipSetDevice(be->device));
+    drain_prof(be);
+    uint32_t n = 0;
+    for (auto& kv : be->prof) {
+        if (out && n < cap) {
+            memset(&out[n], 0, sizeof out[n]);
+            snprintf(out[n].kernel, sizeof out[n].kernel, "%s", kv.first.c_str());
+            out[n].launches = kv.second.launches;
+            out[n].total_ms = kv.second.total_ms;
+            out[n].min_ms = kv.second.min_ms;
+            out[n].max_ms = kv.second.max_ms;
+        }
+        n++;
+    }
+    *n_out = n;
+    if (out) be->prof.clear();
+    return INFR_OK;
+}
+
+extern "C" infr_status infr_hip_plan_moe_routing(infr_hip_backend* be, const infr_hip_plan* plan, uint32_t op_index,
+                                                 int32_t* ids, float* weights, float* logits, float* probs) {
+    if (!ok_backend(be) || !ok_plan(plan) || plan->be != be) return fail(INFR_ERR_INVALID, "moe_routing: bad handle");
+    if (op_index >= plan->ops.size() || plan->ops[op_index].kind != INFR_OP_MOE_FFN)
+        return fail(INFR_ERR_INVALID, "moe_routing: op %u is not a MoeFfn", op_index);
+    const infr_op_moe_ffn& m = plan->ops[op_index].u.moe_ffn;
+    const MoeScratch& sc = plan->moe[op_index];
+    std::lock_guard<std::mutex> lk(be->mu);
+    HIP_TRY(hipSetDevice(be->device));
+    HIP_TRY(hipStreamSynchronize(be->stream));
+    size_t rows = (size_t)sc.rows;
+    if (rows == 0) return INFR_OK;
+    if (ids) HIP_TRY(hipMemcpy(ids, sc.ids, rows * m.n_used * 4, hipMemcpyDeviceToHost));
+    if (weights) HIP_TRY(hipMemcpy(weights, sc.weights, rows * m.n_used * 4, hipMemcpyDeviceToHost));
+    if (logits) HIP_TRY(hipMemcpy(logits, sc.logits, rows * m.n_expert * 4, hipMemcpyDeviceToHost));
+    if (probs) HIP_TRY(hipMemcpy(probs, sc.probs, rows * m.n_expert * 4, hipMemcpyDeviceToHost));
+    return INFR_OK;
+}
+
+extern "C" infr_status infr_hip_dequant(infr_hip_backend* be, const infr_hip_buffer* src, int32_t dtype, uint64_t numel,
+                                        infr_hip_buffer* dst) {
+    if (infr_status st = check_owned(be, src, "dequant")) return st;
+    if (infr_status st = check_owned(be, dst, "dequant")) return st;
+    int e = 1, b = 4;
+    if (!geometry(dtype, &e, &b)) return fail(INFR_ERR_UNSUPPORTED, "dequant: dtype %s has no decode on this backend", dtype_name(dtype));
+    if (numel % (uint64_t)e != 0) return fail(INFR_ERR_INVALID, "dequant: %llu elements is not a whole number of blocks", (unsigned long long)numel);
+    size_t need_src = (size_t)(numel / (uint64_t)e) * (size_t)b;
+    if (src->len < need_src) return fail(INFR_ERR_BACKEND, "dequant: source holds %zu bytes, %zu needed", src->len, need_src);
+    if (dst->len < numel * 4) return fail(INFR_ERR_BACKEND, "dequant: destination holds %zu bytes, %llu needed", dst->len, (unsigned long long)numel * 4);
+    std::lock_guard<std::mutex> lk(be->mu);
+    HIP_TRY(hipSetDevice(be->device));
+    Timed t(be, "dequant");
+    infr::launch_dequant(be->stream, (const uint8_t*)src->dptr, dtype, numel, (float*)dst->dptr);
+    return INFR_OK;
+}

@@ -1,0 +1,197 @@
+// Device-side helpers shared by the gfx950 kernels: exact scalar decode of GGUF blocks,
+// wave64 reductions, and an expf whose results equal the host libm's bit for bit.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/infr_hip.h"
+
+namespace infr {
+
+constexpr int kWave = 64;
+
+// Unaligned load.  gfx950 code objects run with unaligned global access enabled, so this is
+// one global_load of sizeof(T) bytes even at a 2-byte-aligned address (Q6_K blocks are 210 B,
+// Q8_0 blocks 34 B).
+template <class T>
+__device__ __forceinline__ T ldu(const void* p) {
+    T v;
+    __builtin_memcpy(&v, p, sizeof(T));
+    return v;
+}
+
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t bits) {
+    _Float16 h;
+    uint16_t b = (uint16_t)bits;
+    __builtin_memcpy(&h, &b, 2);
+    return (float)h;  // exact, subnormals included
+}
+
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits) {
+    return __uint_as_float((bits & 0xFFFFu) << 16);
+}
+
+// ---------------------------------------------------------------------------------------------
+// expf with the same results as glibc's expf on an FMA-capable x86-64 host (the function the
+// reference's f32::exp resolves to): table of 2^(i/32) in double, degree-3 polynomial, every
+// multiply-add fused, including the range reduction r = x*N/ln2 - k.  Checked against the
+// host expf over every float with |x| <= 104 (zero differences).
+__device__ __forceinline__ float expf_libm(float x) {
+    constexpr uint64_t T[32] = {
+        0x3ff0000000000000ull, 0x3fefd9b0d3158574ull, 0x3fefb5586cf9890full, 0x3fef9301d0125b51ull,
+        0x3fef72b83c7d517bull, 0x3fef54873168b9aaull, 0x3fef387a6e756238ull, 0x3fef1e9df51fdee1ull,
+        0x3fef06fe0a31b715ull, 0x3feef1a7373aa9cbull, 0x3feedea64c123422ull, 0x3feece086061892dull,
+        0x3feebfdad5362a27ull, 0x3feeb42b569d4f82ull, 0x3feeab07dd485429ull, 0x3feea47eb03a5585ull,
+        0x3feea09e667f3bcdull, 0x3fee9f75e8ec5f74ull, 0x3feea11473eb0187ull, 0x3feea589994cce13ull,
+        0x3feeace5422aa0dbull, 0x3feeb737b0cdc5e5ull, 0x3feec49182a3f090ull, 0x3feed503b23e255dull,
+        0x3feee89f995ad3adull, 0x3feeff76f2fb5e47ull, 0x3fef199bdd85529cull, 0x3fef3720dcef9069ull,
+        0x3fef5818dcfba487ull, 0x3fef7c97337b9b5full, 0x3fefa4afa2a490daull, 0x3fefd0765b6e4540ull};
+    // Out-of-range and non-finite inputs: same special cases as libm.
+    if (!(x == x)) return x + x;
+    if (x > 0x1.62e42ep6f) return __builtin_huge_valf();
+    if (x < -0x1.9fe368p6f) return 0.0f;
+    const double InvLn2N = 0x1.71547652b82fep+0 * 32.0;
+    const double Shift = 0x1.8p+52;
+    const double C0 = 0x1.c6af84b912394p-5 / 32.0 / 32.0 / 32.0;
+    const double C1 = 0x1.ebfce50fac4f3p-3 / 32.0 / 32.0;
+    const double C2 = 0x1.62e42ff0c52d6p-1 / 32.0;
+    double xd = (double)x;
+    double z = __dmul_rn(InvLn2N, xd);
+    double kd = __dadd_rn(z, Shift);
+    uint64_t ki = (uint64_t)__double_as_longlong(kd);
+    kd = __dsub_rn(kd, Shift);
+    double r = __fma_rn(InvLn2N, xd, -kd);
+    uint64_t t = T[ki & 31u] + (ki << 47);
+    double s = __longlong_as_double((long long)t);
+    double p = __fma_rn(C0, r, C1);
+    double r2 = __dmul_rn(r, r);
+    double y = __fma_rn(C2, r, 1.0);
+    y = __fma_rn(p, r2, y);
+    y = __dmul_rn(y, s);
+    return (float)y;
+}
+
+// act_fn of the reference (crates/infr-cpu/src/kernels.rs:6664-6672), same operation order.
+__device__ __forceinline__ float act_fn(int act, float g) {
+    if (act == INFR_ACT_SILU) return __fdiv_rn(g, __fadd_rn(1.0f, expf_libm(-g)));
+    if (act == INFR_ACT_GELU) {
+        float g3 = __fmul_rn(__fmul_rn(__fmul_rn(0.044715f, g), g), g);
+        float inner = __fmul_rn(0.7978846f, __fadd_rn(g, g3));
+        float t = __fadd_rn(1.0f, tanhf(inner));
+        return __fmul_rn(__fmul_rn(0.5f, g), t);
+    }
+    return __fdiv_rn(1.0f, __fadd_rn(1.0f, expf_libm(-g)));
+}
+
+// gated_act_fn (kernels.rs:6678-6683).
+__device__ __forceinline__ float gated_act_fn(int act, bool has_clamp, float clamp, float gate, float up) {
+    if (!has_clamp) return __fmul_rn(act_fn(act, gate), up);
+    float gm = gate < clamp ? gate : clamp;
+    float uc = up;
+    if (uc < -clamp) uc = -clamp;
+    if (uc > clamp) uc = clamp;
+    return __fmul_rn(act_fn(act, gm), uc);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Block geometry, host and device.
+__host__ __device__ inline bool block_geometry(int dtype, int* elems, int* bytes) {
+    switch (dtype) {
+        case INFR_F32: case INFR_I32: case INFR_U32: *elems = 1; *bytes = 4; return true;
+        case INFR_F16: case INFR_BF16: *elems = 1; *bytes = 2; return true;
+        case INFR_Q8_0: *elems = 32; *bytes = 34; return true;
+        case INFR_Q4K: *elems = 256; *bytes = 144; return true;
+        case INFR_Q6K: *elems = 256; *bytes = 210; return true;
+        default: return false;
+    }
+}
+
+// get_scale_min_k4 (crates/infr-gguf/src/dequant.rs:77-87).
+__device__ __forceinline__ void k4(int j, const uint8_t* q, uint32_t& sc, uint32_t& m) {
+    if (j < 4) {
+        sc = q[j] & 63u;
+        m = q[j + 4] & 63u;
+    } else {
+        sc = (uint32_t)((q[j + 4] & 0x0F) | ((q[j - 4] >> 6) << 4));
+        m = (uint32_t)((q[j + 4] >> 4) | ((q[j] >> 6) << 4));
+    }
+}
+
+// Exact decode of element k of a row of `dtype`, with the reference's operation order
+// (crates/infr-gguf/src/dequant.rs:35-51: sc = d*f32(sc_i); mn = dmin*f32(m_i);
+// out = sc*f32(code) + mn, separate multiply and add).  Slow path: used by the standalone
+// decode kernel and by the shape-generic GEMV.
+__device__ inline float decode_elem(int dtype, const uint8_t* row, uint32_t k) {
+    switch (dtype) {
+        case INFR_F32: return ldu<float>(row + 4u * k);
+        case INFR_F16: return f16_bits_to_f32(ldu<uint16_t>(row + 2u * k));
+        case INFR_BF16: return bf16_bits_to_f32(ldu<uint16_t>(row + 2u * k));
+        case INFR_I32: return (float)ldu<int32_t>(row + 4u * k);
+        case INFR_U32: return (float)ldu<uint32_t>(row + 4u * k);
+        case INFR_Q8_0: {
+            const uint8_t* blk = row + (size_t)(k >> 5) * 34u;
+            float d = f16_bits_to_f32(ldu<uint16_t>(blk));
+            int code = (int)(int8_t)blk[2 + (k & 31u)] + 128;
+            float sc = __fmul_rn(d, 1.0f);
+            float mn = __fmul_rn(d, -128.0f);
+            return __fadd_rn(__fmul_rn(sc, (float)code), mn);
+        }
+        case INFR_Q4K: {
+            const uint8_t* blk = row + (size_t)(k >> 8) * 144u;
+            uint32_t w = k & 255u;
+            uint32_t j = w >> 6, hi = (w >> 5) & 1u, l = w & 31u;
+            float d = f16_bits_to_f32(ldu<uint16_t>(blk));
+            float dmin = f16_bits_to_f32(ldu<uint16_t>(blk + 2));
+            uint32_t sc, m;
+            k4((int)(2 * j + hi), blk + 4, sc, m);
+            uint8_t v = blk[16 + j * 32 + l];
+            uint32_t code = hi ? (uint32_t)(v >> 4) : (uint32_t)(v & 0xF);
+            float scf = __fmul_rn(d, (float)(int)sc);
+            float mn = __fmul_rn(dmin, (float)(-(int)m));
+            return __fadd_rn(__fmul_rn(scf, (float)code), mn);
+        }
+        case INFR_Q6K: {
+            const uint8_t* blk = row + (size_t)(k >> 8) * 210u;
+            uint32_t w = k & 255u;
+            uint32_t half = w >> 7, g = (w >> 5) & 3u, l = w & 31u;
+            const uint8_t* ql = blk + half * 64;
+            const uint8_t* qh = blk + 128 + half * 32;
+            uint32_t lo = (g & 1u) ? ql[l + 32] : ql[l];
+            lo = (g & 2u) ? (lo >> 4) : (lo & 0xFu);
+            uint32_t hi2 = ((uint32_t)qh[l] >> (2u * g)) & 3u;
+            uint32_t code = lo | (hi2 << 4);
+            int s = (int)(int8_t)blk[192 + (w >> 4)];
+            float d = f16_bits_to_f32(ldu<uint16_t>(blk + 208));
+            float scf = __fmul_rn(d, (float)s);
+            float mn = __fmul_rn(d, (float)(-32 * s));
+            return __fadd_rn(__fmul_rn(scf, (float)code), mn);
+        }
+        default: return 0.0f;
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+// Wave64 helpers.
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+    return v;
+}
+
+// Sum of v over each run of `seg` consecutive lanes (seg need not be a power of two); the
+// total lands in the first lane of the run.  pos = lane's index inside its run.
+__device__ __forceinline__ float segment_sum(float v, int seg, int pos) {
+    for (int off = 1; off < seg; off <<= 1) {
+        float t = __shfl_down(v, off, kWave);
+        if (pos + off < seg) v += t;
+    }
+    return v;
+}
+
+}  // namespace infr

@@ -1,0 +1,108 @@
+// Small kernels around the expert path: standalone block decode, the elementwise ops of
+// the shared-expert branch, and a fill used instead of memset nodes (safe under graph capture).
+#include "device_common.h"
+#include "kernels.h"
+
+namespace infr {
+
+__global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict__ src, int dtype, uint64_t numel,
+                                                      float* __restrict__ out) {
+    uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+    const uint64_t step = (uint64_t)gridDim.x * 256;
+    int be = 1, bb = 4;
+    block_geometry(dtype, &be, &bb);
+    for (; i < numel; i += step) {
+        // decode_elem indexes with 32 bits inside a row; address by block so any tensor size works
+        uint64_t blk = i / (uint64_t)be;
+        uint32_t k = (uint32_t)(i - blk * (uint64_t)be);
+        out[i] = decode_elem(dtype, src + blk * (uint64_t)bb, k);
+    }
+}
+
+void launch_dequant(hipStream_t s, const uint8_t* src, int dtype, uint64_t numel, float* out) {
+    if (numel == 0) return;
+    uint64_t blocks = (numel + 255) / 256;
+    if (blocks > 65535ull * 16) blocks = 65535ull * 16;
+    hipLaunchKernelGGL(dequant_kernel, dim3((uint32_t)blocks), dim3(256), 0, s, src, dtype, numel, out);
+}
+
+// Op::GatedAct (crates/infr-cpu/src/lib.rs:2973-3027), strides and block-interleaved gate included.
+__global__ __launch_bounds__(256) void gated_act_kernel(const float* __restrict__ gate, const float* __restrict__ up,
+                                                        float* __restrict__ dst, int rows, int nff, int act,
+                                                        int up_off, int up_stride, int gate_stride,
+                                                        int gate_block_width, int has_clamp, float clamp) {
+    const int64_t total = (int64_t)rows * nff;
+    for (int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * 256) {
+        int r = (int)(idx / nff), i = (int)(idx - (int64_t)r * nff);
+        int64_t gb = (gate_block_width > 0 || gate_stride > 0) ? (int64_t)r * gate_stride : (int64_t)r * nff;
+        int64_t ub = up_stride == 0 ? (int64_t)r * nff + up_off : (int64_t)r * up_stride + up_off;
+        int64_t gi;
+        if (gate_block_width > 0) {
+            int headw = gate_block_width / 2;
+            int head = i / headw, off = i - head * headw;
+            gi = gb + (int64_t)head * gate_block_width + headw + off;
+        } else {
+            gi = gb + i;
+        }
+        dst[idx] = gated_act_fn(act, has_clamp != 0, clamp, gate[gi], up[ub + i]);
+    }
+}
+
+void launch_gated_act(hipStream_t s, const float* gate, const float* up, float* dst, int rows, int nff, int act,
+                      int up_off, int up_stride, int gate_stride, int gate_block_width, int has_clamp, float clamp) {
+    int64_t total = (int64_t)rows * nff;
+    if (total == 0) return;
+    int64_t blocks = (total + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(gated_act_kernel, dim3((uint32_t)blocks), dim3(256), 0, s, gate, up, dst, rows, nff, act,
+                       up_off, up_stride, gate_stride, gate_block_width, has_clamp, clamp);
+}
+
+__global__ __launch_bounds__(256) void add_kernel(const float* __restrict__ a, const float* __restrict__ b,
+                                                  float* __restrict__ dst, uint32_t n) {
+    for (uint32_t i = blockIdx.x * 256 + threadIdx.x; i < n; i += gridDim.x * 256) dst[i] = __fadd_rn(a[i], b[i]);
+}
+
+void launch_add(hipStream_t s, const float* a, const float* b, float* dst, uint32_t n) {
+    if (n == 0) return;
+    uint32_t blocks = (n + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(add_kernel, dim3(blocks), dim3(256), 0, s, a, b, dst, n);
+}
+
+// Op::MoeSharedExpertAdd (crates/infr-cpu/src/lib.rs:3336-3356):
+// dst = moe + sigmoid(gate[r]) * shexp, multiply and add rounded separately.
+__global__ __launch_bounds__(256) void moe_shared_expert_add_kernel(const float* __restrict__ moe,
+                                                                    const float* __restrict__ shexp,
+                                                                    const float* __restrict__ gate,
+                                                                    float* __restrict__ dst, int rows, int n) {
+    const int r = blockIdx.y;
+    const float g = __fdiv_rn(1.0f, __fadd_rn(1.0f, expf_libm(-gate[r])));
+    for (int c = blockIdx.x * 256 + threadIdx.x; c < n; c += gridDim.x * 256) {
+        size_t i = (size_t)r * n + c;
+        dst[i] = __fadd_rn(moe[i], __fmul_rn(g, shexp[i]));
+    }
+    (void)rows;
+}
+
+void launch_moe_shared_expert_add(hipStream_t s, const float* moe, const float* shexp, const float* gate, float* dst,
+                                  int rows, int n) {
+    if (rows == 0 || n == 0) return;
+    int bx = (n + 255) / 256;
+    if (bx > 64) bx = 64;
+    hipLaunchKernelGGL(moe_shared_expert_add_kernel, dim3(bx, rows), dim3(256), 0, s, moe, shexp, gate, dst, rows, n);
+}
+
+__global__ __launch_bounds__(256) void fill_zero_kernel(uint32_t* p, size_t words) {
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < words; i += (size_t)gridDim.x * 256) p[i] = 0u;
+}
+
+void launch_fill_zero(hipStream_t s, void* p, size_t bytes) {
+    size_t words = (bytes + 3) / 4;
+    if (words == 0) return;
+    size_t blocks = (words + 255) / 256;
+    if (blocks > 8192) blocks = 8192;
+    hipLaunchKernelGGL(fill_zero_kernel, dim3((uint32_t)blocks), dim3(256), 0, s, (uint32_t*)p, words);
+}
+
+}  // namespace infr

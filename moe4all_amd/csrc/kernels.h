@@ -1,0 +1,66 @@
+// Host-callable launchers of the gfx950 kernels.  Every launcher validates nothing: the
+// backend checks shapes, dtypes and buffer extents before it calls one.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace infr {
+
+// Router logits with the reference's dot order (8 FMA lanes, lanes summed 0..7).
+// logits[rows, n_expert]; router rows are `row_bytes` apart, decoded as `rdt`.
+// Returns false when the shape does not fit the kernel's LDS budget.
+bool launch_router_logits(hipStream_t s, const uint8_t* router, int rdt, size_t row_bytes, const float* x,
+                          int ne, int n_expert, int rows, float* logits);
+
+struct RouteParams {
+    const float* logits;      // [rows, n_expert]
+    int n_expert, n_used, rows;
+    int gating, norm_w;
+    float scale;
+    const float* exp_probs_b; // [n_expert] or null
+    int n_groups, n_groups_used;
+    const int32_t* expert_ids;  // [rows, n_used] or null (hash routing)
+    int32_t* ids;             // out [rows, n_used] rank order
+    float* weights;           // out [rows, n_used]
+    float* probs;             // out [rows, n_expert]
+};
+void launch_route(hipStream_t s, const RouteParams& p);
+
+struct MoeGemvParams {
+    const float* x;           // gate/up: [rows, ne]; down: h [rows, n_used, nff]
+    const int32_t* ids;       // [rows, n_used]
+    const float* weights;     // [rows, n_used]
+    const uint8_t* gate; size_t gate_stride;   // per-expert byte stride
+    const uint8_t* up;   size_t up_stride;
+    const uint8_t* down; size_t down_stride;
+    const float* down_scale;  // [n_expert] or null
+    int gate_dt, up_dt, down_dt;
+    int rows, ne, nff, n_used, n_expert;
+    int act; int has_clamp; float clamp;
+    int weight_before;
+    int fused_gate_up;
+    float* h;                 // [rows, n_used, nff]
+    float* dst;               // [rows, ne]
+    int n_cu;
+};
+// h = act(gate.x) * (up.x) for every (row, slot).
+void launch_moe_gate_up(hipStream_t s, const MoeGemvParams& p);
+// dst[row] = sum over slots (rank order) of w * (down . h).
+void launch_moe_down_combine(hipStream_t s, const MoeGemvParams& p);
+
+// Standalone decode: out[i] = value of element i (exact reference arithmetic).
+void launch_dequant(hipStream_t s, const uint8_t* src, int dtype, uint64_t numel, float* out);
+
+// dst[m, out_f] = x[m, in_f] . W^T (W rows start at `w`, `row_bytes` apart).
+void launch_linear(hipStream_t s, const float* x, const uint8_t* w, int dt, size_t row_bytes, int m, int in_f,
+                   int out_f, float* dst, int n_cu);
+void launch_gated_act(hipStream_t s, const float* gate, const float* up, float* dst, int rows, int nff, int act,
+                      int up_off, int up_stride, int gate_stride, int gate_block_width, int has_clamp, float clamp);
+void launch_add(hipStream_t s, const float* a, const float* b, float* dst, uint32_t n);
+void launch_moe_shared_expert_add(hipStream_t s, const float* moe, const float* shexp, const float* gate, float* dst,
+                                  int rows, int n);
+void launch_fill_zero(hipStream_t s, void* p, size_t bytes);
+
+}  // namespace infr

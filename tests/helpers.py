@@ -1,0 +1,281 @@
+"""Shared test utilities: deterministic generators shaped like the reference's test helpers,
+and an INDEPENDENT numpy/f64 restatement of the GGUF block decoders (written from ggml's
+published dequantize_row_* loops, not from the oracle) used to pin the oracle."""
+from __future__ import annotations
+
+import numpy as np
+
+F32, F16, BF16 = 0, 1, 2
+Q8_0, Q4K, Q6K = 9, 12, 14
+BLOCK = {Q8_0: (32, 34), Q4K: (256, 144), Q6K: (256, 210), F32: (1, 4), F16: (1, 2), BF16: (1, 2)}
+
+
+# ---- generators of the reference's tests ------------------------------------------------
+def lcg_bytes_blocks(seed: int, nblk: int, nbytes: int) -> np.ndarray:
+    """lcg_bytes(seed ^ block_index, nbytes) for every block
+    (crates/infr-testkit/src/lib.rs:49-56, :106-123), vectorised over blocks."""
+    s = (np.uint32(seed) ^ np.arange(nblk, dtype=np.uint32)).astype(np.uint64)
+    out = np.empty((nblk, nbytes), np.uint8)
+    for i in range(nbytes):
+        s = (s * np.uint64(1664525) + np.uint64(1013904223)) & np.uint64(0xFFFFFFFF)
+        out[:, i] = (s >> np.uint64(16)).astype(np.uint8)
+    return out
+
+
+def f16_bytes(v: float) -> np.ndarray:
+    return np.array([v], np.float16).view(np.uint8)
+
+
+def synth_weight(dtype: int, n_elem: int, seed: int) -> np.ndarray:
+    """Valid blocks with LCG payload and sane f16 scales (testkit synth_weight + synth_scales;
+    same bytes as crates/infr-metal/tests/parity.rs:426-451 for Q4_K / Q6_K)."""
+    be, bb = BLOCK[dtype]
+    assert n_elem % be == 0
+    nblk = n_elem // be
+    if dtype == Q4K:
+        blk = np.empty((nblk, 144), np.uint8)
+        blk[:, 4:] = lcg_bytes_blocks(seed, nblk, 140)
+        blk[:, 0:2] = f16_bytes(0.05)
+        blk[:, 2:4] = f16_bytes(0.10)
+    elif dtype == Q6K:
+        blk = np.empty((nblk, 210), np.uint8)
+        blk[:, :208] = lcg_bytes_blocks(seed, nblk, 208)
+        blk[:, 208:210] = f16_bytes(0.03)
+    elif dtype == Q8_0:
+        blk = lcg_bytes_blocks(seed, nblk, 34)
+        blk[:, 0:2] = f16_bytes(0.01)
+    else:
+        raise ValueError(dtype)
+    return blk.reshape(-1)
+
+
+def rand_f32(n: int, seed: int) -> np.ndarray:
+    """crates/infr-metal/tests/parity.rs:15-25: 64-bit LCG, top 24 bits -> [-1, 1)."""
+    out = np.empty(n, np.float32)
+    s = seed & 0xFFFFFFFFFFFFFFFF
+    for i in range(n):
+        s = (s * 6364136223846793005 + 1442695040888963407) & 0xFFFFFFFFFFFFFFFF
+        out[i] = np.float32(np.float32(s >> 40) / np.float32(1 << 24)) * np.float32(2.0) - np.float32(1.0)
+    return out
+
+
+def gen(n: int, salt: int) -> np.ndarray:
+    """crates/infr-llama/tests/seam_op_parity.rs:257-261."""
+    i = np.arange(n, dtype=np.int64)
+    return (((i * 13 + salt) % 29).astype(np.float32) - np.float32(14.0)) * np.float32(0.05)
+
+
+def quantize_q8_0(w: np.ndarray) -> np.ndarray:
+    """The reference's test-local Q8_0 quantiser (crates/infr-metal/tests/parity.rs:271-287)."""
+    w = np.asarray(w, np.float32).reshape(-1, 32)
+    amax = np.abs(w).max(axis=1)
+    d = np.where(amax > 0, amax / np.float32(127.0), np.float32(0)).astype(np.float32)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        q = np.where(d[:, None] > 0, w / d[:, None], 0).astype(np.float32)
+    q = np.clip(np.sign(q) * np.floor(np.abs(q) + np.float32(0.5)), -127, 127).astype(np.int8)  # round half away
+    out = np.empty((w.shape[0], 34), np.uint8)
+    out[:, 0:2] = d.astype(np.float16).view(np.uint8).reshape(-1, 2)
+    out[:, 2:] = q.view(np.uint8)
+    return out.reshape(-1)
+
+
+# ---- independent decoders (ggml's dequantize_row_q8_0 / q4_K / q6_K), exact in f64 --------
+def _f16(b: np.ndarray) -> np.ndarray:
+    # x87 extended precision (64-bit significand): d*sc*q - dmin*m needs up to ~61 bits when the
+    # two f16 scales sit at opposite ends of the f16 exponent range, so f64 could round it twice.
+    return np.ascontiguousarray(b).view(np.float16).astype(np.longdouble).reshape(-1)
+
+
+def ggml_dequant(dtype: int, data: np.ndarray) -> np.ndarray:
+    """Returns the EXACT decoded values (x87 extended); one cast to f32 is the single rounding
+    the reference's f32 expression `sc*code + mn` performs (both products are exact there)."""
+    data = np.ascontiguousarray(data).view(np.uint8).reshape(-1)
+    if dtype == F32:
+        return data.view(np.float32).astype(np.float64)
+    if dtype == F16:
+        return data.view(np.float16).astype(np.float64)
+    if dtype == BF16:
+        return (data.view(np.uint16).astype(np.uint32) << 16).view(np.float32).astype(np.float64)
+    be, bb = BLOCK[dtype]
+    blk = data.reshape(-1, bb)
+    nb = blk.shape[0]
+    if dtype == Q8_0:
+        d = _f16(blk[:, 0:2])
+        q = blk[:, 2:].view(np.int8).astype(np.longdouble)
+        # the reference's affine form d*(q+128) + d*(-128): a cancelling sum is +0.0, never -0.0
+        return ((q + 128) * d[:, None] + (d * -128)[:, None]).reshape(-1)
+    if dtype == Q4K:
+        d = _f16(blk[:, 0:2])
+        dmin = _f16(blk[:, 2:4])
+        sc_b = blk[:, 4:16].astype(np.int64)
+        qs = blk[:, 16:144].astype(np.int64)
+        y = np.empty((nb, 256), np.longdouble)
+        for is_ in range(8):  # ggml: for j in 0..QK_K step 64 { is, is+1 } with q += 32 per step
+            if is_ < 4:
+                sc = sc_b[:, is_] & 63
+                m = sc_b[:, is_ + 4] & 63
+            else:
+                sc = (sc_b[:, is_ + 4] & 0xF) | ((sc_b[:, is_ - 4] >> 6) << 4)
+                m = (sc_b[:, is_ + 4] >> 4) | ((sc_b[:, is_] >> 6) << 4)
+            q = qs[:, (is_ // 2) * 32:(is_ // 2) * 32 + 32]
+            nib = (q & 0xF) if is_ % 2 == 0 else (q >> 4)
+            y[:, is_ * 32:(is_ + 1) * 32] = (d * sc)[:, None] * nib - (dmin * m)[:, None]
+        return y.reshape(-1)
+    if dtype == Q6K:
+        ql = blk[:, 0:128].astype(np.int64)
+        qh = blk[:, 128:192].astype(np.int64)
+        sc = blk[:, 192:208].view(np.int8).astype(np.int64)
+        d = _f16(blk[:, 208:210])
+        y = np.empty((nb, 256), np.longdouble)
+        for n in range(2):  # ggml: for n in 0..QK_K step 128
+            l = np.arange(32)
+            is_ = l // 16
+            qln, qhn, scn = ql[:, 64 * n:64 * n + 64], qh[:, 32 * n:32 * n + 32], sc[:, 8 * n:8 * n + 8]
+            q1 = ((qln[:, l] & 0xF) | (((qhn[:, l] >> 0) & 3) << 4))
+            q2 = ((qln[:, l + 32] & 0xF) | (((qhn[:, l] >> 2) & 3) << 4))
+            q3 = ((qln[:, l] >> 4) | (((qhn[:, l] >> 4) & 3) << 4))
+            q4 = ((qln[:, l + 32] >> 4) | (((qhn[:, l] >> 6) & 3) << 4))
+            base = 128 * n
+            # affine form of the reference, d*sc*q + d*(-32*sc) (ggml writes d*sc*(q-32)): same
+            # value, but an exact cancellation is +0.0 here and would be -0.0 there
+            y[:, base + l] = d[:, None] * scn[:, is_ + 0] * q1 + d[:, None] * (-32 * scn[:, is_ + 0])
+            y[:, base + l + 32] = d[:, None] * scn[:, is_ + 2] * q2 + d[:, None] * (-32 * scn[:, is_ + 2])
+            y[:, base + l + 64] = d[:, None] * scn[:, is_ + 4] * q3 + d[:, None] * (-32 * scn[:, is_ + 4])
+            y[:, base + l + 96] = d[:, None] * scn[:, is_ + 6] * q4 + d[:, None] * (-32 * scn[:, is_ + 6])
+        return y.reshape(-1)
+    raise ValueError(dtype)
+
+
+# ---- independent f64 model of Op::MoeFfn (shape of moe_ref / moe_v4_ref) -----------------
+def moe_ffn_f64(x, router_w, gate_w, up_w, down_w, *, ne, n_expert, n_used, n_ff, scale=1.0, gating="softmax",
+                norm_w=True, bias=None, n_groups=0, n_groups_used=0, weight_before=False, down_scale=None,
+                clamp=None, act="silu", hash_ids=None):
+    """x [rows, ne]; weights already decoded to float arrays (router [E,ne], gate/up [E,nff,ne],
+    down [E,ne,nff]).  Plain f64 everywhere; follows the f32/f64 references in
+    crates/infr-llama/tests/seam_op_parity.rs:2245-2343 and :5635-5696."""
+    x = np.asarray(x, np.float64).reshape(-1, ne)
+    R = np.asarray(router_w, np.float64).reshape(n_expert, ne)
+    G = np.asarray(gate_w, np.float64).reshape(n_expert, n_ff, ne)
+    U = np.asarray(up_w, np.float64).reshape(n_expert, n_ff, ne)
+    D = np.asarray(down_w, np.float64).reshape(n_expert, ne, n_ff)
+    out = np.zeros_like(x)
+    sel_idx = []
+    for r in range(x.shape[0]):
+        logits = R @ x[r]
+        if gating == "softmax":
+            p = np.exp(logits - logits.max())
+            p /= p.sum()
+        elif gating == "sigmoid":
+            p = 1.0 / (1.0 + np.exp(-logits))
+        else:
+            sp = np.where(logits > 20.0, logits, np.log1p(np.exp(np.minimum(logits, 700))))
+            p = np.sqrt(sp)
+        if hash_ids is not None:
+            idx = [int(v) for v in np.asarray(hash_ids).reshape(-1, n_used)[r]]
+        else:
+            sel = p + (np.asarray(bias, np.float64) if bias is not None else 0.0)
+            if n_groups > 1 and n_groups_used > 0:
+                per = n_expert // n_groups
+                gs = [np.sort(sel[g * per:(g + 1) * per])[-2:].sum() for g in range(n_groups)]
+                keep = sorted(range(n_groups), key=lambda g: (-gs[g], g))[:n_groups_used]
+                for g in range(n_groups):
+                    if g not in keep:
+                        sel[g * per:(g + 1) * per] = -np.inf
+            idx = sorted(range(n_expert), key=lambda e: (-sel[e], e))[:n_used]
+        w = p[idx] / max(p[idx].sum(), 1e-20) * scale if norm_w else p[idx] * scale
+        sel_idx.append(idx)
+        for k, e in enumerate(idx):
+            wp = w[k] if weight_before else 1.0
+            g = wp * (G[e] @ x[r])
+            u = wp * (U[e] @ x[r])
+            if clamp is not None:
+                g = np.minimum(g, clamp)
+                u = np.clip(u, -clamp, clamp)
+            if act == "silu":
+                a = g / (1.0 + np.exp(-g))
+            elif act == "gelu":
+                a = 0.5 * g * (1.0 + np.tanh(0.7978846 * (g + 0.044715 * g ** 3)))
+            else:
+                a = 1.0 / (1.0 + np.exp(-g))
+            y = D[e] @ (a * u)
+            if down_scale is not None:
+                y = y * down_scale[e]
+            out[r] += (1.0 if weight_before else w[k]) * y
+    return out, np.array(sel_idx, np.int32)
+
+
+def rel_l2(a, b) -> float:
+    a, b = np.asarray(a, np.float64).ravel(), np.asarray(b, np.float64).ravel()
+    return float(np.linalg.norm(a - b) / max(np.linalg.norm(b), 1e-30))
+
+
+def elem_rel_err(got, want) -> float:
+    """The per-element measure of the reference's device parity tests:
+    |c - m| / max(|c|, 1)  (crates/infr-metal/tests/parity.rs:158-163)."""
+    got, want = np.asarray(got, np.float64).ravel(), np.asarray(want, np.float64).ravel()
+    return float(np.max(np.abs(got - want) / np.maximum(np.abs(want), 1.0))) if got.size else 0.0
+
+
+def max_abs(a, b) -> float:
+    return float(np.max(np.abs(np.asarray(a, np.float64) - np.asarray(b, np.float64)))) if np.size(a) else 0.0
+
+
+# ---- the reference-specified cases behind tests/golden/*.npz --------------------------------
+def pattern(n, mul, add):
+    return ((np.arange(n, dtype=np.int64) * mul + add) & 0xFF).astype(np.uint8)
+
+
+def dequant_cases():
+    out = {}
+    b = pattern(288, 37, 11)
+    for blk in range(2):
+        b[blk * 144:blk * 144 + 2] = f16_bytes(0.375)
+        b[blk * 144 + 2:blk * 144 + 4] = f16_bytes(-0.125)
+    out["q4k_ref_pattern"] = (Q4K, b)
+    b = pattern(420, 53, 7)
+    for blk in range(2):
+        b[blk * 210 + 208:blk * 210 + 210] = f16_bytes(0.05)
+    out["q6k_ref_pattern"] = (Q6K, b)
+    for name, dt, bb in (("q8_0", Q8_0, 34), ("q4k", Q4K, 144), ("q6k", Q6K, 210)):
+        out[f"{name}_all_formats_pattern"] = (dt, pattern(2 * bb, 29, 3))
+    out["q8_0_lcg"] = (Q8_0, synth_weight(Q8_0, 32 * 24, 5))
+    out["q4k_lcg"] = (Q4K, synth_weight(Q4K, 256 * 6, 80))
+    out["q6k_lcg"] = (Q6K, synth_weight(Q6K, 256 * 6, 90))
+    return out
+
+
+def moe_cases():
+    cases = {}
+    # seam_op_parity.rs moe_sqrt_softplus_parity
+    ne, E, K, nff = 32, 6, 2, 32
+    lead = np.array([24.0, 1.0, 0.75, 0.5, -1.5, -1.0], np.float32)
+    router = np.zeros((E, ne), np.float32)
+    router[:, 0] = lead
+    cases["sqrt_softplus"] = dict(ne=ne, n_expert=E, n_used=K, n_ff=nff, gating=2, x=np.ones(ne, np.float32),
+                                  router=router.reshape(-1), gate=gen(E * nff * ne, 12), up=gen(E * nff * ne, 13),
+                                  down=gen(E * ne * nff, 14), dtype=F32, expect_idx=[0, 1])
+    # seam_op_parity.rs moe_groups_bias_parity
+    E = 8
+    lead = np.array([3.0, 2.5, 2.0, 1.5, 1.0, 0.9, 0.8, 0.7], np.float32)
+    router = np.zeros((E, ne), np.float32)
+    router[:, 0] = lead
+    cases["groups_bias"] = dict(ne=ne, n_expert=E, n_used=K, n_ff=nff, gating=1, x=np.ones(ne, np.float32),
+                                router=router.reshape(-1), gate=gen(E * nff * ne, 15), up=gen(E * nff * ne, 16),
+                                down=gen(E * ne * nff, 17), dtype=F32,
+                                bias=np.array([0, 0, 0, 0, .6, .6, .6, .6], np.float32), n_groups=2, n_groups_used=1,
+                                expect_idx=[4, 5])
+    # metal parity.rs moe_ffn_parity (f32, softmax)
+    ne, E, K, nff = 64, 8, 2, 128
+    cases["metal_f32"] = dict(ne=ne, n_expert=E, n_used=K, n_ff=nff, gating=0, x=rand_f32(ne, 60),
+                              router=rand_f32(E * ne, 61), gate=rand_f32(E * nff * ne, 62),
+                              up=rand_f32(E * nff * ne, 63), down=rand_f32(E * ne * nff, 64), dtype=F32)
+    # metal parity.rs moe_quant_test (Q4_K seed 80, Q6_K seed 90)
+    ne, E, K, nff = 256, 8, 3, 256
+    for name, dt, seed in (("metal_q4k", Q4K, 80), ("metal_q6k", Q6K, 90)):
+        cases[name] = dict(ne=ne, n_expert=E, n_used=K, n_ff=nff, gating=0, x=rand_f32(ne, seed),
+                           router=rand_f32(E * ne, seed + 1), gate=synth_weight(dt, E * nff * ne, seed + 2),
+                           up=synth_weight(dt, E * nff * ne, seed + 3), down=synth_weight(dt, E * ne * nff, seed + 4),
+                           dtype=dt)
+    return cases
+
+

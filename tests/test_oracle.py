@@ -1,0 +1,392 @@
+"""Pins the CPU oracle (oracle/infr_oracle.c) WITHOUT running the reference (Rust, not
+buildable here): against the committed golden fixtures, against an independent extended-precision
+decoder written from ggml's published loops, against closed forms / brute force, and against the
+facts the reference's own tests state (selected experts, tolerances)."""
+import os
+from fractions import Fraction
+
+import numpy as np
+import pytest
+
+import helpers as H
+import oracle as O
+
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+
+
+# ------------------------------------------------------------------ geometry / f16 / k4
+def test_block_geometry_matches_ggml_formulas():
+    # crates/infr-core/src/decode_spec.rs:455-504 restates ggml: Q8_0 2+32, Q4_K 2+2+12+128, Q6_K 128+64+16+2
+    assert O.block_geometry(O.Q8_0) == (32, 2 + 32)
+    assert O.block_geometry(O.Q4K) == (256, 2 + 2 + 12 + 128)
+    assert O.block_geometry(O.Q6K) == (256, 128 + 64 + 16 + 2)
+    assert O.bytes_for(O.Q4K, 768 * 2048) == 884736
+    assert O.bytes_for(O.Q6K, 2048 * 768) == 1290240
+    assert O.bytes_for(O.Q8_0, 768 * 2048) == 1671168
+    with pytest.raises(ValueError):
+        O.bytes_for(O.Q4K, 100)
+
+
+def test_f16_to_f32_all_65536_values():
+    h = np.arange(65536, dtype=np.uint16)
+    want = h.view(np.float16).astype(np.float32)
+    got = np.array([O.f16_to_f32(int(v)) for v in h], np.float32)
+    assert np.array_equal(got.view(np.uint32)[~np.isnan(want)], want.view(np.uint32)[~np.isnan(want)])
+    assert np.isnan(got[np.isnan(want)]).all()
+
+
+def test_k4_inverts_ggml_scale_packing_exhaustively():
+    """get_scale_min_k4 must invert the packing ggml's quantiser writes
+    (scales[j]=ls, scales[j+4]=lm for j<4; else scales[j+4]=(ls&0xF)|((lm&0xF)<<4),
+    scales[j-4]|=(ls>>4)<<6, scales[j]|=(lm>>4)<<6) for every 6-bit (ls, lm) at every j."""
+    rng = np.random.default_rng(0)
+    for j in range(8):
+        for ls in range(64):
+            for lm in range(0, 64, 3):
+                other = rng.integers(0, 64, size=(8, 2))
+                other[j] = (ls, lm)
+                s = np.zeros(12, np.uint8)
+                for jj in range(8):
+                    a, b = int(other[jj][0]), int(other[jj][1])
+                    if jj < 4:
+                        s[jj] |= a
+                        s[jj + 4] |= b
+                    else:
+                        s[jj + 4] = (a & 0xF) | ((b & 0xF) << 4)
+                        s[jj - 4] |= (a >> 4) << 6
+                        s[jj] |= (b >> 4) << 6
+                for jj in range(8):
+                    assert O.k4(jj, s) == (int(other[jj][0]), int(other[jj][1]))
+
+
+# ------------------------------------------------------------------ dequant
+def test_dequant_matches_golden_fixture_bit_for_bit():
+    g = np.load(os.path.join(GOLD, "dequant.npz"))
+    names = sorted({k.rsplit(".", 1)[0] for k in g.files})
+    assert len(names) == 8
+    for n in names:
+        got = O.dequant(int(g[n + ".dtype"]), g[n + ".bytes"])
+        assert np.array_equal(got.view(np.uint32), g[n + ".bits"]), n
+
+
+def test_dequant_fixture_inputs_are_the_reference_test_patterns():
+    g = np.load(os.path.join(GOLD, "dequant.npz"))
+    for n, (dt, b) in H.dequant_cases().items():
+        assert np.array_equal(g[n + ".bytes"], b) and int(g[n + ".dtype"]) == dt
+
+
+@pytest.mark.parametrize("dt,seed", [(O.Q8_0, 1), (O.Q4K, 2), (O.Q6K, 3)])
+def test_dequant_matches_independent_decoder_on_random_blocks(dt, seed):
+    be, bb = O.block_geometry(dt)
+    b = H.synth_weight(dt, be * 64, seed)
+    want = H.ggml_dequant(dt, b).astype(np.float32)
+    assert np.array_equal(O.dequant(dt, b).view(np.uint32), want.view(np.uint32))
+
+
+def test_dequant_hand_computed_values():
+    # Q8_0: d = 0.5, q = -128..-97: y = d*q exactly
+    blk = np.zeros(34, np.uint8)
+    blk[0:2] = H.f16_bytes(0.5)
+    blk[2:] = np.arange(-128, -96).astype(np.int8).view(np.uint8)
+    assert np.array_equal(O.dequant(O.Q8_0, blk), np.arange(-128, -96, dtype=np.float32) * 0.5)
+    # Q4_K: one block, d=1, dmin=1, sub-block 0: sc=3,m=2 -> y = 3*q - 2; sub-block 5 (j>=4): sc=33, m=50
+    blk = np.zeros(144, np.uint8)
+    blk[0:2] = H.f16_bytes(1.0)
+    blk[2:4] = H.f16_bytes(1.0)
+    s = blk[4:16]
+    s[0] = 3
+    s[4] = 2
+    s[5 + 4] = (33 & 0xF) | ((50 & 0xF) << 4)
+    s[5 - 4] |= (33 >> 4) << 6
+    s[5] |= (50 >> 4) << 6
+    blk[16 + 0] = 0x0F           # element 0 (low nibble of qs[0]) = 15, element 32 (high nibble) = 0
+    blk[16 + 64 + 7] = 0xA0      # qs[71]: j=2 -> elements 128+7 (low)=0 and 160+7 (high, sub-block 5)=10
+    y = O.dequant(O.Q4K, blk)
+    assert y[0] == 3 * 15 - 2 and y[1] == -2.0
+    assert y[160 + 7] == 33 * 10 - 50 and y[160] == -50.0
+    # Q6_K: d=2, scale[9] = -3, element 128+16+3 (half 1, l=19, group 0 -> scale index 8+1): q = ql lo | qh bits0-1
+    blk = np.zeros(210, np.uint8)
+    blk[208:210] = H.f16_bytes(2.0)
+    blk[192 + 9] = np.array([-3], np.int8).view(np.uint8)[0]
+    blk[64 + 19] = 0x05          # ql[64+19] low nibble 5
+    blk[128 + 32 + 19] = 0x02    # qh[32+19] bits 0-1 = 2 -> q = 5 | (2<<4) = 37
+    y = O.dequant(O.Q6K, blk)
+    assert y[128 + 19] == 2.0 * -3 * (37 - 32)
+    assert y[128 + 16] == 2.0 * -3 * (0 - 32)
+
+
+def test_dequant_float_dtypes():
+    v = np.array([1.5, -2.25, 65504.0, 6e-8], np.float32)
+    assert np.array_equal(O.dequant(O.F16, v.astype(np.float16)), v.astype(np.float16).astype(np.float32))
+    bf = (v.view(np.uint32) >> 16).astype(np.uint16)
+    assert np.array_equal(O.dequant(O.BF16, bf), (bf.astype(np.uint32) << 16).view(np.float32))
+    assert np.array_equal(O.dequant(O.F32, v), v)
+    assert np.array_equal(O.dequant(O.I32, np.array([-7, 3], np.int32)), np.array([-7.0, 3.0], np.float32))
+
+
+# ------------------------------------------------------------------ dot
+def _round_f32(fr: Fraction) -> np.float32:
+    """Exact round-to-nearest-even of a rational to f32."""
+    if fr == 0:
+        return np.float32(0.0)
+    f = np.float32(float(fr))  # float(Fraction) is correctly rounded to f64; fix the second rounding
+    cands = {f, np.nextafter(f, np.float32(np.inf)), np.nextafter(f, np.float32(-np.inf))}
+    best = None
+    for c in cands:
+        if not np.isfinite(c):
+            continue
+        err = abs(Fraction(float(c)) - fr)
+        key = (err, int(np.float32(c).view(np.uint32)) & 1)
+        if best is None or key < best[0]:
+            best = (key, c)
+    return np.float32(best[1])
+
+
+def _dot_exact_model(a, b):
+    """kernels.rs:6568-6583 evaluated with exact rational arithmetic and one rounding per FMA / add."""
+    n = len(a)
+    acc = [np.float32(0)] * 8
+    for c in range(n // 8):
+        for j in range(8):
+            i = 8 * c + j
+            acc[j] = _round_f32(Fraction(float(a[i])) * Fraction(float(b[i])) + Fraction(float(acc[j])))
+    s = np.float32(0)
+    for j in range(8):
+        s = _round_f32(Fraction(float(s)) + Fraction(float(acc[j])))
+    for i in range(n // 8 * 8, n):
+        s = _round_f32(Fraction(float(a[i])) * Fraction(float(b[i])) + Fraction(float(s)))
+    return s
+
+
+@pytest.mark.parametrize("n", [0, 1, 7, 8, 9, 15, 16, 17, 63, 64, 65, 200])
+def test_dot_lane_order_and_fma_bit_exact(n):
+    rng = np.random.default_rng(n)
+    # wide dynamic range so a different association or an unfused multiply changes the bits
+    a = (rng.standard_normal(n) * 10.0 ** rng.integers(-3, 4, n)).astype(np.float32)
+    b = (rng.standard_normal(n) * 10.0 ** rng.integers(-3, 4, n)).astype(np.float32)
+    got = O.dot(a, b)
+    want = _dot_exact_model(a, b)
+    assert got.view(np.uint32) == want.view(np.uint32)
+
+
+def test_dot_distinguishes_plausible_wrong_orders():
+    # The 8-lane order must differ from a sequential sum and from a pairwise/tree lane reduction
+    # on this input, otherwise the test above could not catch those mistakes.
+    rng = np.random.default_rng(7)
+    a = (rng.standard_normal(64) * 10.0 ** rng.integers(-4, 5, 64)).astype(np.float32)
+    b = rng.standard_normal(64).astype(np.float32)
+    seq = np.float32(0)
+    for i in range(64):
+        seq = _round_f32(Fraction(float(a[i])) * Fraction(float(b[i])) + Fraction(float(seq)))
+    assert O.dot(a, b).view(np.uint32) != seq.view(np.uint32)
+    assert abs(float(O.dot(a, b)) - float(np.dot(a.astype(np.float64), b.astype(np.float64)))) < 1e-2 * np.abs(a * b).sum()
+
+
+# ------------------------------------------------------------------ activations
+def test_act_fn_closed_forms():
+    for g in (-30.0, -3.0, -0.5, 0.0, 0.5, 3.0, 30.0):
+        silu = g / (1.0 + np.exp(-g))
+        assert abs(float(O.act(O.ACT_SILU, g)) - silu) <= 2e-7 * max(1.0, abs(silu))
+        sig = 1.0 / (1.0 + np.exp(-g))
+        assert abs(float(O.act(O.ACT_SIGMOID, g)) - sig) <= 2e-7
+        gelu = 0.5 * g * (1.0 + np.tanh(0.7978846 * (g + 0.044715 * g ** 3)))
+        assert abs(float(O.act(O.ACT_GELU, g)) - gelu) <= 4e-7 * max(1.0, abs(gelu))
+    assert float(O.act(O.ACT_SILU, 0.0)) == 0.0
+    # clamp: act(min(gate, l)) * clamp(up, -l, l)  (graph.rs:953-971)
+    assert O.gated_act(O.ACT_SILU, 5.0, 9.0, clamp=2.0) == np.float32(O.act(O.ACT_SILU, 2.0) * np.float32(2.0))
+    assert O.gated_act(O.ACT_SILU, -5.0, -9.0, clamp=2.0) == np.float32(O.act(O.ACT_SILU, -5.0) * np.float32(-2.0))
+    assert O.gated_act(O.ACT_SILU, 1.0, 3.0) == np.float32(O.act(O.ACT_SILU, 1.0) * np.float32(3.0))
+
+
+# ------------------------------------------------------------------ routing
+def test_route_softmax_topk_renorm():
+    rng = np.random.default_rng(3)
+    lg = rng.standard_normal(128).astype(np.float32)
+    probs, idx, w = O.route_row(lg, 8)
+    p64 = np.exp(lg.astype(np.float64) - lg.max())
+    p64 /= p64.sum()
+    assert np.allclose(probs, p64, rtol=2e-6, atol=0)
+    assert list(idx) == list(np.argsort(-p64, kind="stable")[:8])
+    assert np.allclose(w, p64[idx] / p64[idx].sum(), rtol=3e-6)
+    assert abs(float(w.sum()) - 1.0) < 1e-6
+    # not renormalised, scaled
+    _, idx2, w2 = O.route_row(lg, 8, norm_w=False, scale=2.5)
+    assert list(idx2) == list(idx) and np.allclose(w2, p64[idx] * 2.5, rtol=3e-6)
+
+
+def test_route_ties_keep_ascending_expert_id():
+    lg = np.zeros(16, np.float32)
+    lg[[11, 3, 7]] = 1.0  # three equal maxima, then all-equal rest
+    _, idx, w = O.route_row(lg, 5)
+    assert list(idx) == [3, 7, 11, 0, 1]
+    assert np.allclose(w[:3], w[0]) and np.allclose(w[3:], w[3])
+
+
+def test_route_groups_bias_selects_what_the_reference_test_states():
+    # seam_op_parity.rs:2495-2504: sigmoid gating, +0.6 bias on group 1 -> group 1 wins, experts 4 and 5,
+    # while the weights come from the UNBIASED probabilities.
+    lg = np.array([3.0, 2.5, 2.0, 1.5, 1.0, 0.9, 0.8, 0.7], np.float32)
+    bias = np.array([0, 0, 0, 0, .6, .6, .6, .6], np.float32)
+    probs, idx, w = O.route_row(lg, 2, gating=O.GATE_SIGMOID, exp_probs_b=bias, n_groups=2, n_groups_used=1)
+    assert list(idx) == [4, 5]
+    sig = 1 / (1 + np.exp(-lg.astype(np.float64)))
+    assert np.allclose(w, sig[[4, 5]] / sig[[4, 5]].sum(), rtol=1e-6)
+    # group scores from the comment: 1.877 vs 1.442 unbiased, 2.642 biased
+    assert abs(np.sort(sig[:4])[-2:].sum() - 1.877) < 1e-3 and abs(np.sort(sig[4:])[-2:].sum() + 1.2 - 2.642) < 1e-3
+    _, idx_nobias, _ = O.route_row(lg, 2, gating=O.GATE_SIGMOID, n_groups=2, n_groups_used=1)
+    assert list(idx_nobias) == [0, 1]
+
+
+def test_route_sqrt_softplus_and_hash_ids():
+    lg = np.array([24.0, 1.0, 0.75, 0.5, -1.5, -1.0], np.float32)  # seam_op_parity.rs:2393-2396
+    probs, idx, w = O.route_row(lg, 2, gating=O.GATE_SQRT_SOFTPLUS)
+    assert list(idx) == [0, 1]
+    assert probs[0] == np.float32(np.sqrt(np.float32(24.0)))  # v > 20 shortcut: sp = v
+    assert abs(float(probs[1]) - np.sqrt(np.log1p(np.exp(1.0)))) < 1e-6
+    # hash routing: ids in table order, weights = renormalised probs at those ids (graph.rs:1318-1351)
+    p2, idx2, w2 = O.route_row(lg, 2, hash_ids=[5, 2])
+    assert list(idx2) == [5, 2] and np.allclose(w2, p2[[5, 2]] / p2[[5, 2]].sum(), rtol=1e-6)
+    with pytest.raises(ValueError):
+        O.route_row(lg, 2, hash_ids=[6, 0])
+
+
+# ------------------------------------------------------------------ Op::MoeFfn
+def _run_case(c, **kw):
+    return O.moe_ffn(c["x"], c["router"], c["gate"], c["up"], c["down"], ne=c["ne"], n_expert=c["n_expert"],
+                     n_used=c["n_used"], n_ff_exp=c["n_ff"], gate_dtype=c["dtype"], gating=c["gating"],
+                     exp_probs_b=c.get("bias"), n_expert_groups=c.get("n_groups", 0),
+                     n_expert_groups_used=c.get("n_groups_used", 0), **kw)
+
+
+def test_moe_ffn_matches_golden_cases_of_the_reference_tests():
+    g = np.load(os.path.join(GOLD, "moe_small.npz"))
+    cases = H.moe_cases()
+    assert sorted(cases) == sorted({k.split(".")[0] for k in g.files})
+    for name, c in cases.items():
+        r = _run_case(c)
+        assert np.array_equal(r["idx"], g[name + ".idx"]), name
+        # seam_op_parity.rs asserts max-abs 1e-4 on its f32 cases; metal parity.rs asserts
+        # |c-m|/max(|c|,1) <= 1e-3 on its (large-magnitude) synthetic quantised cases
+        if name in ("sqrt_softplus", "groups_bias"):
+            assert H.max_abs(r["dst"], g[name + ".want"]) < 1e-4, name
+        assert H.elem_rel_err(r["dst"], g[name + ".want"]) < 1e-3, name
+        assert H.rel_l2(r["dst"], g[name + ".want"]) < 1e-5, name
+
+
+@pytest.mark.parametrize("gdt,ddt", [(O.Q4K, O.Q6K), (O.Q8_0, O.Q8_0), (O.Q6K, O.Q4K)])
+@pytest.mark.parametrize("rows", [1, 5])
+def test_moe_ffn_quantised_multirow_vs_f64_model(gdt, ddt, rows):
+    ne, E, K, nff = 256, 16, 4, 512
+    rng = np.random.default_rng(rows * 100 + gdt)
+    x = rng.standard_normal((rows, ne)).astype(np.float32)
+    router = (rng.standard_normal((E, ne)) * 0.1).astype(np.float32)
+    gate, up = H.synth_weight(gdt, E * nff * ne, 11), H.synth_weight(gdt, E * nff * ne, 12)
+    down = H.synth_weight(ddt, E * ne * nff, 13)
+    r = O.moe_ffn(x, router, gate, up, down, ne=ne, n_expert=E, n_used=K, n_ff_exp=nff, gate_dtype=gdt,
+                  down_dtype=ddt, scale=1.3)
+    want, idx = H.moe_ffn_f64(x, router, H.ggml_dequant(gdt, gate), H.ggml_dequant(gdt, up),
+                              H.ggml_dequant(ddt, down), ne=ne, n_expert=E, n_used=K, n_ff=nff, scale=1.3)
+    assert np.array_equal(r["idx"], idx)
+    assert H.rel_l2(r["dst"], want) < 2e-6
+    # thread count must not change a single bit (every output is owned by one task)
+    r1 = O.moe_ffn(x, router, gate, up, down, ne=ne, n_expert=E, n_used=K, n_ff_exp=nff, gate_dtype=gdt,
+                   down_dtype=ddt, scale=1.3, n_threads=1)
+    assert np.array_equal(r1["dst"].view(np.uint32), r["dst"].view(np.uint32))
+
+
+def test_moe_ffn_variants_vs_f64_model():
+    ne, E, K, nff = 64, 8, 3, 96
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((3, ne)).astype(np.float32)
+    router = rng.standard_normal((E, ne)).astype(np.float32) * 0.3
+    gate = rng.standard_normal((E, nff, ne)).astype(np.float32) * 0.2
+    up = rng.standard_normal((E, nff, ne)).astype(np.float32) * 0.2
+    down = rng.standard_normal((E, ne, nff)).astype(np.float32) * 0.2
+    ds = rng.uniform(0.5, 1.5, E).astype(np.float32)
+    common = dict(ne=ne, n_expert=E, n_used=K, n_ff_exp=nff)
+    # weight_before (llama4), sigmoid gating, no renorm
+    r = O.moe_ffn(x, router, gate, up, down, gating=O.GATE_SIGMOID, norm_w=False, weight_before=True, **common)
+    want, _ = H.moe_ffn_f64(x, router, gate, up, down, ne=ne, n_expert=E, n_used=K, n_ff=nff, gating="sigmoid",
+                            norm_w=False, weight_before=True)
+    assert H.rel_l2(r["dst"], want) < 2e-6
+    # down_scale + clamp + gelu
+    r = O.moe_ffn(x, router, gate, up, down, down_scale=ds, swiglu_clamp=0.7, act=O.ACT_GELU, **common)
+    want, _ = H.moe_ffn_f64(x, router, gate, up, down, ne=ne, n_expert=E, n_used=K, n_ff=nff, down_scale=ds,
+                            clamp=0.7, act="gelu")
+    assert H.rel_l2(r["dst"], want) < 2e-6
+    # fused gate_up: gate rows first, up rows second per expert (graph.rs:1279-1285)
+    fused = np.concatenate([gate, up], axis=1)
+    rf = O.moe_ffn(x, router, fused, None, down, fused_gate_up=True, **common)
+    rs = O.moe_ffn(x, router, gate, up, down, **common)
+    assert np.array_equal(rf["dst"].view(np.uint32), rs["dst"].view(np.uint32))
+    # hash routing
+    ids = np.array([[1, 5, 2], [0, 7, 3], [4, 4, 6]], np.int32)
+    r = O.moe_ffn(x, router, gate, up, down, expert_ids=ids.astype(np.float32), **common)
+    want, _ = H.moe_ffn_f64(x, router, gate, up, down, ne=ne, n_expert=E, n_used=K, n_ff=nff, hash_ids=ids)
+    assert np.array_equal(r["idx"], ids) and H.rel_l2(r["dst"], want) < 2e-6
+    # refused combinations (lib.rs:3613-3629)
+    with pytest.raises(ValueError):
+        O.moe_ffn(x, router, gate, up, down, swiglu_clamp=1.0, weight_before=True, **common)
+    with pytest.raises(ValueError):
+        O.moe_ffn(x, router, gate, up, down, expert_ids=ids.astype(np.float32), exp_probs_b=np.zeros(E), **common)
+
+
+def test_bucketing_order_and_inverse_map():
+    ne, E, K, nff, rows = 32, 12, 3, 32, 40
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((rows, ne)).astype(np.float32)
+    router = rng.standard_normal((E, ne)).astype(np.float32)
+    w = (rng.standard_normal(E * nff * ne) * 0.1).astype(np.float32)
+    r = O.moe_ffn(x, router, w, w, (rng.standard_normal(E * ne * nff) * 0.1).astype(np.float32), ne=ne, n_expert=E,
+                  n_used=K, n_ff_exp=nff)
+    idx = r["idx"]
+    # brute force of lib.rs:3887-3906: experts ascending, rows ascending inside an expert
+    pairs = sorted((int(idx[rr, k]), rr, k) for rr in range(rows) for k in range(K))
+    assert list(r["pair_row"]) == [p[1] for p in pairs]
+    experts = sorted({p[0] for p in pairs})
+    assert list(r["bucket_expert"]) == experts and r["n_buckets"] == len(experts)
+    counts = [sum(1 for p in pairs if p[0] == e) for e in experts]
+    assert list(r["bucket_count"]) == counts and int(np.sum(counts)) == rows * K
+    assert list(r["bucket_p0"]) == list(np.cumsum([0] + counts[:-1]))
+    for flat, (e, rr, k) in enumerate(pairs):
+        assert r["slot_pair"][rr, k] == flat
+    assert sorted(r["slot_pair"].ravel()) == list(range(rows * K))  # a permutation
+
+
+def test_moe_ffn_empty_rows():
+    r = O.moe_ffn(np.zeros((0, 32), np.float32), np.zeros(4 * 32, np.float32), np.zeros(4 * 32 * 32, np.float32),
+                  np.zeros(4 * 32 * 32, np.float32), np.zeros(4 * 32 * 32, np.float32), ne=32, n_expert=4, n_used=2,
+                  n_ff_exp=32)
+    assert r["dst"].shape == (0, 32) and r["n_buckets"] == 0
+
+
+# ------------------------------------------------------------------ neighbours
+@pytest.mark.parametrize("dt", [O.Q4K, O.Q6K, O.Q8_0, O.F32, O.F16])
+def test_linear_reference_mode_vs_f64(dt):
+    in_f, out_f, m = 512, 24, 3
+    rng = np.random.default_rng(dt)
+    x = rng.standard_normal((m, in_f)).astype(np.float32)
+    if dt in (O.F32, O.F16):
+        w = (rng.standard_normal(out_f * in_f) * 0.1).astype(np.float32 if dt == O.F32 else np.float16)
+    else:
+        w = H.synth_weight(dt, out_f * in_f, 21)
+    got = O.linear(x, w, dt, in_f, out_f)
+    W = np.asarray(H.ggml_dequant(dt, w), np.float64).reshape(out_f, in_f)
+    want = x.astype(np.float64) @ W.T
+    # decode_parity.rs:93-102 holds reference mode to 1e-5 of the f64 GEMV
+    assert H.rel_l2(got, want) < 1e-5
+    # w_off selects a row band of a concatenated weight (graph.rs:208-211)
+    got2 = O.linear(x, w, dt, in_f, 8, w_off=8 * in_f)
+    assert np.array_equal(got2.view(np.uint32), np.ascontiguousarray(got[:, 8:16]).view(np.uint32))
+
+
+def test_elementwise_neighbours():
+    rng = np.random.default_rng(2)
+    a, b = rng.standard_normal((3, 40)).astype(np.float32), rng.standard_normal((3, 40)).astype(np.float32)
+    assert np.array_equal(O.add(a, b), a + b)
+    ga = O.gated_act_rows(a, b)
+    assert np.allclose(ga, a / (1 + np.exp(-a.astype(np.float64))) * b, rtol=1e-6, atol=1e-7)
+    gate = np.array([0.3, -1.2, 4.0], np.float32)
+    got = O.moe_shared_expert_add(a, b, gate)
+    want = a + (1 / (1 + np.exp(-gate.astype(np.float64))))[:, None] * b
+    assert np.allclose(got, want, rtol=1e-6, atol=1e-7)
