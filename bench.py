@@ -1,0 +1,212 @@
+#!/usr/bin/env python3
+"""Decode benchmark of the routed-expert MoE FFN path on one MI355X.
+
+A step is one decode token through every MoE layer of the workload (one execute of a graph
+with one Op::MoeFfn per layer, each with its own HBM-resident weights and its own N(0,1)
+activation row).  Default workload: the Qwen3-30B-A3B-shaped stack (48 layers, hidden 2048,
+128 experts, top-8, intermediate 768, Q4_K gate/up + Q6_K down), synthetic seeded weights.
+
+Prints ONE JSON line: whole-job decode tok/s, the roofline of the dominant kernel measured
+live with HIP events on the backend's stream, and a CPU baseline (the oracle, a C restatement
+of the reference's CPU path, timed on this host's cores on a bounded sample).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+import moe4all_amd as M  # noqa: E402
+from moe4all_amd import DType, TensorDesc, synth  # noqa: E402
+
+HBM_PEAK_GBPS = 8000.0
+SEED0 = 20260101
+N_TOKENS = 8  # distinct activation sets rotated through the steps
+
+
+def build_stack(be, shape, n_layer, batch):
+    """One graph with n_layer MoeFfn ops (+ shared-expert ops), weights generated in HBM."""
+    g = M.Graph()
+    layers, ids = [], []
+    for l in range(n_layer):
+        lw = synth.LayerWeights(be, shape, SEED0, l, on_device=True)
+        layers.append(lw)
+        x = g.input(TensorDesc([batch, shape.ne], DType.F32))
+        router = g.weight(TensorDesc([shape.n_expert, shape.ne], DType.F32))
+        gate = g.weight(TensorDesc([shape.n_expert, shape.n_ff, shape.ne], shape.gate_dtype))
+        up = g.weight(TensorDesc([shape.n_expert, shape.n_ff, shape.ne], shape.gate_dtype))
+        down = g.weight(TensorDesc([shape.n_expert, shape.ne, shape.n_ff], shape.down_dtype))
+        dst = g.output(TensorDesc([batch, shape.ne], DType.F32))
+        d = dict(x=x, router=router, gate=gate, up=up, down=down, dst=dst)
+        if shape.shared_ff:
+            moe = g.internal(TensorDesc([batch, shape.ne], DType.F32))
+            g.moe_ffn(x=x, router=router, gate_exps=gate, up_exps=up, down_exps=down, dst=moe, ne=shape.ne,
+                      n_expert=shape.n_expert, n_used=shape.n_used, n_ff_exp=shape.n_ff)
+            sg = g.weight(TensorDesc([shape.shared_ff, shape.ne], shape.gate_dtype))
+            su = g.weight(TensorDesc([shape.shared_ff, shape.ne], shape.gate_dtype))
+            sd = g.weight(TensorDesc([shape.ne, shape.shared_ff], shape.down_dtype))
+            tg, tu = (g.internal(TensorDesc([batch, shape.shared_ff], DType.F32)) for _ in range(2))
+            ta = g.internal(TensorDesc([batch, shape.shared_ff], DType.F32))
+            ts = g.internal(TensorDesc([batch, shape.ne], DType.F32))
+            g.linear(x=x, weight=sg, dst=tg, m=batch, in_f=shape.ne, out_f=shape.shared_ff)
+            g.linear(x=x, weight=su, dst=tu, m=batch, in_f=shape.ne, out_f=shape.shared_ff)
+            g.gated_act(gate=tg, up=tu, dst=ta, rows=batch, nff=shape.shared_ff)
+            g.linear(x=ta, weight=sd, dst=ts, m=batch, in_f=shape.shared_ff, out_f=shape.ne)
+            g.add(a=moe, b=ts, dst=dst, n=batch * shape.ne)
+            d.update(sg=sg, su=su, sd=sd)
+        else:
+            g.moe_ffn(x=x, router=router, gate_exps=gate, up_exps=up, down_exps=down, dst=dst, ne=shape.ne,
+                      n_expert=shape.n_expert, n_used=shape.n_used, n_ff_exp=shape.n_ff)
+        ids.append(d)
+    return g, layers, ids
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c5"])
+    ap.add_argument("--layers", type=int, default=0, help="override the layer count (0 = the config's)")
+    ap.add_argument("--batch", type=int, default=1)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-kernel-timing", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus must be 1 (no multi-GPU path exists in this tree)",
+              file=sys.stderr)
+        sys.exit(2)
+
+    shape = {"c1": synth.CONFIG_1, "c2": synth.CONFIG_2, "c5": synth.CONFIG_5}[args.config]
+    n_layer = args.layers or shape.n_layer
+    batch = args.batch
+    be = M.Backend(0)
+    caps = be.capabilities()
+    t_setup = time.time()
+    g, layers, ids = build_stack(be, shape, n_layer, batch)
+    plan = be.compile(g)
+    # activations: N_TOKENS independent sets of per-layer N(0,1) rows, resident in HBM
+    xbufs = []
+    for t in range(N_TOKENS):
+        row = []
+        for l in range(n_layer):
+            xb = be.alloc(batch * shape.ne * 4)
+            synth.weights_device(be, xb, DType.F32, synth.stream_seed(SEED0 + 1 + t, l, synth.ROLE_X),
+                                 batch * shape.ne, sigma=1.0)
+            row.append(xb)
+        xbufs.append(row)
+    ybufs = [be.alloc(batch * shape.ne * 4) for _ in range(n_layer)]
+    binds = []
+    for t in range(N_TOKENS):
+        b = M.Bindings()
+        for l in range(n_layer):
+            d, lw = ids[l], layers[l]
+            b.bind(d["x"], xbufs[t][l]).bind(d["router"], lw.router).bind(d["gate"], lw.gate)
+            b.bind(d["up"], lw.up).bind(d["down"], lw.down).bind(d["dst"], ybufs[l])
+            if shape.shared_ff:
+                b.bind(d["sg"], lw.shared[0]).bind(d["su"], lw.shared[1]).bind(d["sd"], lw.shared[2])
+        binds.append(b)
+    be.sync()
+    setup_s = time.time() - t_setup
+
+    for i in range(args.warmup):
+        be.execute(plan, binds[i % N_TOKENS])
+    be.sync()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        be.execute(plan, binds[i % N_TOKENS])
+    be.sync()
+    elapsed = time.perf_counter() - t0
+    ms_per_step = elapsed * 1e3 / args.steps
+    tok_s = batch * args.steps / elapsed
+
+    # distinct experts actually selected per layer (batch > 1 shares experts between tokens)
+    r = be.moe_routing(plan, 0)
+    distinct = len(set(r["idx"].ravel().tolist()))
+    layer_bytes = shape.algorithmic_bytes(batch, distinct if batch > 1 else None)
+    layer_gbps = layer_bytes * n_layer / (ms_per_step * 1e-3) / 1e9
+
+    # ---- per-kernel durations, HIP events on the backend's own stream, separate pass
+    roofline = None
+    kernels = {}
+    if not args.no_kernel_timing:
+        be.prof_enable(True)
+        ksteps = max(1, min(args.steps, 50))
+        for i in range(ksteps):
+            be.execute(plan, binds[i % N_TOKENS])
+        be.sync()
+        prof = be.prof_read()
+        be.prof_enable(False)
+        gate_b = M.backend.bytes_for(shape.gate_dtype, shape.n_ff * shape.ne)
+        down_b = M.backend.bytes_for(shape.down_dtype, shape.ne * shape.n_ff)
+        n_sel = distinct if batch > 1 else shape.n_used
+        pairs = batch * shape.n_used
+        alg = {  # algorithmic HBM bytes per launch
+            "router_logits": shape.router_bytes() + batch * shape.ne * 4 + batch * shape.n_expert * 4,
+            "moe_gate_up": n_sel * 2 * gate_b + batch * shape.ne * 4 + pairs * shape.n_ff * 4,
+            "moe_down_combine": n_sel * down_b + pairs * shape.n_ff * 4 + batch * shape.ne * 4,
+        }
+        for name, p in prof.items():
+            avg_us = p["total_ms"] * 1e3 / max(p["launches"], 1)
+            kernels[name] = {"launches": int(p["launches"]), "avg_us": round(avg_us, 3), "min_us": round(p["min_ms"] * 1e3, 3)}
+            if name in alg:
+                kernels[name]["alg_bytes"] = alg[name]
+                kernels[name]["GBps"] = round(alg[name] / (avg_us * 1e-6) / 1e9, 1)
+        dom = max((k for k in kernels if k in alg), key=lambda k: kernels[k]["avg_us"] * kernels[k]["launches"], default=None)
+        if dom:
+            ach = alg[dom] / (kernels[dom]["avg_us"] * 1e-6) / 1e9
+            roofline = {"bound": "hbm", "kernel": dom, "achieved": round(ach, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                        "frac": round(ach / HBM_PEAK_GBPS, 4), "traffic": None,
+                        "alg_bytes_per_launch": alg[dom], "avg_launch_us": kernels[dom]["avg_us"]}
+
+    # ---- CPU baseline: the oracle on this host's cores, layer 0's weights, a bounded sample
+    cpu = None
+    if not args.no_cpu_baseline:
+        import oracle as O
+        lw = layers[0]
+        router = be.download(lw.router, dtype=np.float32)
+        gate, up, down = be.download(lw.gate), be.download(lw.up), be.download(lw.down)
+        threads = O.hw_threads()
+        n_sample, spent, budget_s = 0, 0.0, 12.0
+        while spent < budget_s and n_sample < 4 * n_layer:
+            x = synth.normal(synth.stream_seed(SEED0 + 1, n_sample, synth.ROLE_X), batch * shape.ne, 1.0)
+            t1 = time.perf_counter()
+            O.moe_ffn(x, router, gate, up, down, ne=shape.ne, n_expert=shape.n_expert, n_used=shape.n_used,
+                      n_ff_exp=shape.n_ff, gate_dtype=int(shape.gate_dtype), down_dtype=int(shape.down_dtype),
+                      n_threads=threads)
+            spent += time.perf_counter() - t1
+            n_sample += 1
+        per_layer_s = spent / n_sample
+        cpu = {"value": round(batch / (per_layer_s * n_layer), 3), "unit": "tok/s", "cores": threads, "kind": "port",
+               "sample": f"{n_sample} layer-passes of layer 0 (routed experts only) with distinct seeded tokens, "
+                         f"{per_layer_s * 1e3:.2f} ms per layer-pass, f32 reference numerics, "
+                         f"scaled to {n_layer} layers",
+               "ms_per_layer": round(per_layer_s * 1e3, 3)}
+
+    out = {
+        "metric": "MoE decode tok/s", "value": round(tok_s, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": shape.name if n_layer == shape.n_layer else f"{shape.name}[{n_layer} layers]",
+                   "layers": n_layer, "hidden": shape.ne, "experts": shape.n_expert, "top_k": shape.n_used,
+                   "intermediate": shape.n_ff, "gate_up": shape.gate_dtype.name, "down": shape.down_dtype.name,
+                   "shared_intermediate": shape.shared_ff, "batch": batch, "parallelism": "single-gpu",
+                   "resident_weight_bytes": shape.layer_resident_bytes() * n_layer},
+        "layer": {"us_per_layer": round(ms_per_step * 1e3 / n_layer, 3), "alg_bytes_per_layer": layer_bytes,
+                  "achieved_GBps": round(layer_gbps, 1), "frac_of_hbm_peak": round(layer_gbps / HBM_PEAK_GBPS, 4),
+                  "distinct_experts_layer0": distinct},
+        "roofline": roofline, "kernels": kernels, "cpu_baseline": cpu,
+        "device": caps["name"], "compute_units": caps["compute_units"], "setup_s": round(setup_s, 1),
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -336,6 +336,30 @@ extern "C" infr_status infr_hip_sync(infr_hip_backend* be) {
     return INFR_OK;
 }
 
+// ---- shared with sibling translation units of this library (not part of the public ABI)
+extern "C" infr_status infr_hip_internal_fail(infr_status st, const char* msg) { return fail(st, "%s", msg); }
+
+// Validates [byte_offset, byte_offset+bytes) of buf, makes the device current and returns the
+// device pointer and the backend's stream WITH the submission lock held; the caller enqueues
+// its work and then calls infr_hip_internal_unlock.  On error the lock is not held.
+extern "C" infr_status infr_hip_internal_buffer_span(infr_hip_backend* be, infr_hip_buffer* buf, size_t byte_offset,
+                                                     size_t bytes, void** dptr, hipStream_t* stream) {
+    if (infr_status st = check_owned(be, buf, "buffer_span")) return st;
+    if (byte_offset > buf->len || bytes > buf->len - byte_offset)
+        return fail(INFR_ERR_BACKEND, "byte range %zu..%zu exceeds buffer size %zu", byte_offset, byte_offset + bytes,
+                    buf->len);
+    be->mu.lock();
+    hipError_t e = hipSetDevice(be->device);
+    if (e != hipSuccess) {
+        be->mu.unlock();
+        return fail(INFR_ERR_BACKEND, "hip: hipSetDevice failed: %s", hipGetErrorString(e));
+    }
+    *dptr = (char*)buf->dptr + byte_offset;
+    *stream = be->stream;
+    return INFR_OK;
+}
+extern "C" void infr_hip_internal_unlock(infr_hip_backend* be) { be->mu.unlock(); }
+
 // ============================================================================ compile
 namespace {
 

@@ -217,7 +217,8 @@ def elem_rel_err(got, want) -> float:
 
 
 def max_abs(a, b) -> float:
-    return float(np.max(np.abs(np.asarray(a, np.float64) - np.asarray(b, np.float64)))) if np.size(a) else 0.0
+    a, b = np.asarray(a, np.float64).ravel(), np.asarray(b, np.float64).ravel()
+    return float(np.max(np.abs(a - b))) if a.size else 0.0
 
 
 # ---- the reference-specified cases behind tests/golden/*.npz --------------------------------

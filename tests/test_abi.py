@@ -13,12 +13,13 @@ from moe4all_amd import backend as B
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADER = os.path.join(ROOT, "include", "infr_hip.h")
+SYNTH_HEADER = os.path.join(ROOT, "include", "infr_synth.h")
 
 
-def declared_symbols():
-    src = open(HEADER).read()
+def declared_symbols(path=HEADER, prefix="infr_hip_"):
+    src = open(path).read()
     src = re.sub(r"/\*.*?\*/", "", src, flags=re.S)
-    return sorted(set(re.findall(r"\b(infr_hip_[a-z0-9_]+)\s*\(", src)))
+    return sorted(set(re.findall(r"\b(" + prefix + r"[a-z0-9_]+)\s*\(", src)))
 
 
 def test_header_declares_the_backend_trait_surface():
@@ -37,6 +38,10 @@ def test_library_exports_every_declared_symbol():
         assert hasattr(lib, s), f"{s} declared in include/infr_hip.h but not exported"
     # and the Python mirror binds exactly the declared set
     assert sorted(B._SIGNATURES) == declared_symbols()
+    synth = declared_symbols(SYNTH_HEADER, "infr_synth_")
+    assert len(synth) == 4
+    for s in synth:
+        assert hasattr(lib, s), f"{s} declared in include/infr_synth.h but not exported"
 
 
 def test_struct_layouts_match_the_header(tmp_path):

@@ -377,3 +377,79 @@ def test_shared_expert_branch_matches_oracle(be):
     g2.add(a=a, b=b, dst=d, n=rows * ne)
     got2 = M.run_graph(be, g2, [(a, x), (b, moe)], d, rows * ne)
     assert np.array_equal(got2, O.add(x, moe).ravel())
+
+
+# ------------------------------------------------------------------ synthetic workloads at full size
+from moe4all_amd import synth as S  # noqa: E402
+
+
+@pytest.mark.parametrize("dt", [DType.F32, DType.Q8_0, DType.Q4K, DType.Q6K])
+def test_device_generator_writes_the_host_generator_bytes(be, dt):
+    numel = 256 * 1000
+    seed = S.stream_seed(42, 7, int(dt))
+    buf = be.alloc_uninit(M.backend.bytes_for(dt, numel))
+    S.weights_device(be, buf, dt, seed, numel)
+    dev = be.download(buf)
+    buf.free()
+    host = S.weights_host(dt, seed, numel).view(np.uint8)
+    assert np.array_equal(dev, host), f"{int((dev != host).sum())} differing bytes"
+
+
+@pytest.mark.parametrize("shape,batch", [(S.CONFIG_1, 1), (S.CONFIG_2, 1), (S.CONFIG_1, 4), (S.CONFIG_1, 16),
+                                         (S.CONFIG_2, 8), (S.CONFIG_5, 1), (S.CONFIG_5, 8)])
+def test_benchmark_config_layer_matches_oracle_at_full_size(be, shape, batch):
+    """One full-size layer of each benchmark configuration: N(0,0.02) weights quantised on the
+    device, N(0,1) activations; the oracle runs on the downloaded bytes."""
+    lw = S.LayerWeights(be, shape, seed0=77, layer=3, on_device=True)
+    s = shape
+    x = S.normal(S.stream_seed(78, 3, S.ROLE_X), batch * s.ne, 1.0).reshape(batch, s.ne)
+    g = M.Graph()
+    xi = g.input(TensorDesc([batch, s.ne], DType.F32))
+    ri = g.weight(TensorDesc([s.n_expert, s.ne], DType.F32))
+    gi = g.weight(TensorDesc([s.n_expert, s.n_ff, s.ne], s.gate_dtype))
+    ui = g.weight(TensorDesc([s.n_expert, s.n_ff, s.ne], s.gate_dtype))
+    di = g.weight(TensorDesc([s.n_expert, s.ne, s.n_ff], s.down_dtype))
+    yi = g.output(TensorDesc([batch, s.ne], DType.F32))
+    b = M.Bindings().bind(ri, lw.router).bind(gi, lw.gate).bind(ui, lw.up).bind(di, lw.down)
+    if s.shared_ff:
+        moe = g.internal(TensorDesc([batch, s.ne], DType.F32))
+        g.moe_ffn(x=xi, router=ri, gate_exps=gi, up_exps=ui, down_exps=di, dst=moe, ne=s.ne, n_expert=s.n_expert,
+                  n_used=s.n_used, n_ff_exp=s.n_ff)
+        sg, su = g.weight(TensorDesc([s.shared_ff, s.ne], s.gate_dtype)), g.weight(TensorDesc([s.shared_ff, s.ne], s.gate_dtype))
+        sd = g.weight(TensorDesc([s.ne, s.shared_ff], s.down_dtype))
+        tg, tu, ta = (g.internal(TensorDesc([batch, s.shared_ff], DType.F32)) for _ in range(3))
+        ts = g.internal(TensorDesc([batch, s.ne], DType.F32))
+        g.linear(x=xi, weight=sg, dst=tg, m=batch, in_f=s.ne, out_f=s.shared_ff)
+        g.linear(x=xi, weight=su, dst=tu, m=batch, in_f=s.ne, out_f=s.shared_ff)
+        g.gated_act(gate=tg, up=tu, dst=ta, rows=batch, nff=s.shared_ff)
+        g.linear(x=ta, weight=sd, dst=ts, m=batch, in_f=s.shared_ff, out_f=s.ne)
+        g.add(a=moe, b=ts, dst=yi, n=batch * s.ne)
+        b.bind(sg, lw.shared[0]).bind(su, lw.shared[1]).bind(sd, lw.shared[2])
+    else:
+        g.moe_ffn(x=xi, router=ri, gate_exps=gi, up_exps=ui, down_exps=di, dst=yi, ne=s.ne, n_expert=s.n_expert,
+                  n_used=s.n_used, n_ff_exp=s.n_ff)
+    plan = be.compile(g)
+    xb, yb = be.buffer_from(x, M.BufferUsage.Activations), be.alloc(batch * s.ne * 4, M.BufferUsage.Readback)
+    b.bind(xi, xb).bind(yi, yb)
+    be.execute(plan, b)
+    got = be.download(yb, batch * s.ne * 4, np.float32).reshape(batch, s.ne)
+    r = be.moe_routing(plan, 0)
+    router = be.download(lw.router, dtype=np.float32)
+    gate, up, down = be.download(lw.gate), be.download(lw.up), be.download(lw.down)
+    ref = O.moe_ffn(x, router, gate, up, down, ne=s.ne, n_expert=s.n_expert, n_used=s.n_used, n_ff_exp=s.n_ff,
+                    gate_dtype=int(s.gate_dtype), down_dtype=int(s.down_dtype))
+    want = ref["dst"]
+    if s.shared_ff:
+        sgb, sub, sdb = (be.download(t) for t in lw.shared)
+        a = O.gated_act_rows(O.linear(x, sgb, int(s.gate_dtype), s.ne, s.shared_ff),
+                             O.linear(x, sub, int(s.gate_dtype), s.ne, s.shared_ff))
+        want = O.add(want, O.linear(a, sdb, int(s.down_dtype), s.shared_ff, s.ne))
+    assert np.array_equal(r["idx"], ref["idx"])
+    assert np.array_equal(bits(r["w"]), bits(ref["w"]))
+    assert 0.01 < float(np.sqrt(np.mean(want ** 2))) < 1.0   # magnitudes of the real workload
+    assert H.max_abs(got, want) < MAX_ABS, H.max_abs(got, want)
+    assert H.rel_l2(got, want) < REL_L2, H.rel_l2(got, want)
+    for buf in (xb, yb):
+        buf.free()
+    plan.free()
+    lw.free()

@@ -1,0 +1,109 @@
+"""CPU checks of the synthetic-workload generator and the ggml-compatible quantisers, plus the
+round trip quantise -> oracle decode, which pins the oracle's decoders from the other side:
+a wrong nibble order, scale index or sign in the decode shows up as a reconstruction error far
+above the format's quantisation step."""
+import numpy as np
+import pytest
+
+import helpers as H
+import oracle as O
+from moe4all_amd import DType, synth as S
+
+
+def test_normal_stream_is_counter_based_and_gaussian():
+    a = S.normal(123, 4096)
+    b = S.normal(123, 1024, offset=1000)
+    assert np.array_equal(a[1000:2024], b)            # random access by element index
+    assert not np.array_equal(a[:1024], S.normal(124, 1024))
+    z = S.normal(7, 1 << 18).astype(np.float64)
+    assert abs(z.mean()) < 0.01 and abs(z.std() - 1.0) < 0.01
+    assert abs(np.mean(z ** 3)) < 0.03 and abs(np.mean(z ** 4) - 3.0) < 0.08
+    assert 4.0 < np.abs(z).max() < 6.5                # tails are there (not a sum-of-uniforms)
+    w = S.normal(7, 1 << 16, sigma=0.02)
+    assert abs(w.std() - 0.02) < 4e-4
+
+
+def test_normal_matches_box_muller_on_the_same_uniforms():
+    """Pins the hand-written log / sincos: same SplitMix64 outputs through numpy's libm."""
+    def splitmix(seed, k):
+        z = (seed + (k + 1) * 0x9E3779B97F4A7C15) & 0xFFFFFFFFFFFFFFFF
+        z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & 0xFFFFFFFFFFFFFFFF
+        z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & 0xFFFFFFFFFFFFFFFF
+        return z ^ (z >> 31)
+    seed, n = 99, 2000
+    got = S.normal(seed, n).astype(np.float64)
+    want = np.empty(n)
+    for k in range(n // 2):
+        u1 = ((splitmix(seed, 2 * k) >> 11) + 1) / 9007199254740992.0
+        u2 = (splitmix(seed, 2 * k + 1) >> 11) / 9007199254740992.0
+        r = np.sqrt(-2.0 * np.log(u1))
+        want[2 * k], want[2 * k + 1] = r * np.cos(2 * np.pi * u2), r * np.sin(2 * np.pi * u2)
+    assert np.max(np.abs(got - want)) < 5e-7          # f32 rounding of an f64-accurate value
+
+
+def test_f16_rounding_inside_the_quantisers_is_ieee():
+    # d of a Q8_0 block is f16(amax/127): drive many magnitudes through it, subnormals included
+    rng = np.random.default_rng(0)
+    for scale in (1e-9, 1e-7, 3e-6, 1e-4, 0.02, 1.0, 300.0):
+        w = (rng.standard_normal(32 * 64) * scale).astype(np.float32)
+        q = S.quantize(DType.Q8_0, w).reshape(-1, 34)
+        d = (np.abs(w.reshape(-1, 32)).max(axis=1) / np.float32(127.0)).astype(np.float32)
+        with np.errstate(over="ignore"):
+            assert np.array_equal(q[:, :2].copy().view(np.float16).ravel(), d.astype(np.float16))
+
+
+def test_q8_0_equals_the_reference_test_quantiser():
+    w = S.normal(5, 32 * 200, 0.02)
+    assert np.array_equal(S.quantize(DType.Q8_0, w), H.quantize_q8_0(w))
+
+
+@pytest.mark.parametrize("dt,rel_rmse", [(DType.Q8_0, 0.006), (DType.Q6K, 0.02), (DType.Q4K, 0.085)])
+def test_quantise_then_oracle_decode_reconstructs_the_weights(dt, rel_rmse):
+    w = S.normal(11 + int(dt), 256 * 96, 0.02)
+    back = O.dequant(int(dt), S.quantize(dt, w))
+    err = np.sqrt(np.mean((back - w) ** 2)) / np.sqrt(np.mean(w ** 2))
+    # typical ggml figures for Gaussian data: Q8_0 ~0.4 %, Q6_K ~1.3 %, Q4_K ~6 %
+    assert err < rel_rmse, err
+    assert err > rel_rmse / 20                        # and it really quantised
+    # per-element error bounded by about one quantisation step of the block
+    step = {DType.Q8_0: 1 / 127, DType.Q6K: 1 / 31, DType.Q4K: 1 / 7}[dt]
+    amax = np.abs(w.reshape(-1, 256)).max(axis=1, keepdims=True)
+    assert (np.abs(back - w).reshape(-1, 256) <= step * amax * 1.01 + 1e-9).all()
+
+
+def test_quantisers_accept_degenerate_blocks():
+    z = np.zeros(256, np.float32)
+    for dt in (DType.Q8_0, DType.Q4K, DType.Q6K):
+        assert not O.dequant(int(dt), S.quantize(dt, z)).any()
+    c = np.full(256, 0.5, np.float32)
+    assert np.allclose(O.dequant(int(DType.Q4K), S.quantize(DType.Q4K, c)), 0.5, atol=0.02)
+    assert np.allclose(O.dequant(int(DType.Q6K), S.quantize(DType.Q6K, c)), 0.5, atol=0.02)
+
+
+def test_weights_host_is_stream_quantised_and_thread_independent():
+    seed = S.stream_seed(1, 3, S.ROLE_GATE)
+    a = S.weights_host(DType.Q4K, seed, 256 * 40, n_threads=1)
+    b = S.weights_host(DType.Q4K, seed, 256 * 40, n_threads=5)
+    assert np.array_equal(a, b)
+    assert np.array_equal(a, S.quantize(DType.Q4K, S.normal(seed, 256 * 40, 0.02)))
+    tail = S.weights_host(DType.Q4K, seed, 256 * 8, offset=256 * 32)
+    assert np.array_equal(tail, a[32 * 144:])
+    f = S.weights_host(DType.F32, seed, 512)
+    assert np.array_equal(f, S.normal(seed, 512, 0.02))
+    with pytest.raises(ValueError):
+        S.weights_host(DType.Q4K, seed, 100)
+
+
+def test_config_byte_counts():
+    # per-expert bytes and per-layer-token algorithmic bytes of the benchmark configurations
+    assert S.CONFIG_1.expert_bytes() == 5_013_504 and S.CONFIG_1.algorithmic_bytes(1) == 41_172_992
+    assert S.CONFIG_2.expert_bytes() == 3_059_712 and S.CONFIG_2.algorithmic_bytes(1) == 25_542_656
+    assert S.CONFIG_5.expert_bytes() == 12_238_848
+    assert S.CONFIG_5.algorithmic_bytes(1) == 9 * 12_238_848 + 4_194_304 + 32_768
+    assert S.CONFIG_2.layer_resident_bytes() * 48 == (128 * 3_059_712 + 1_048_576) * 48
+
+
+def test_zipf_bias_is_a_normalised_skewed_popularity():
+    b = S.zipf_bias(128, 1.1, 3)
+    p = np.exp(b.astype(np.float64))
+    assert abs(p.sum() - 1.0) < 1e-5 and sorted(p)[-1] / sorted(p)[0] == pytest.approx(128 ** 1.1, rel=1e-4)
