@@ -461,7 +461,7 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
                     c.set(INFR_ERR_INVALID, "MoeFfn: ne/n_expert/n_used/n_ff_exp must be positive and n_used <= n_expert");
                     break;
                 }
-                if (m.n_expert > 2048) { c.set(INFR_ERR_UNSUPPORTED, "MoeFfn: n_expert > 2048"); break; }
+                if (m.n_expert > 2048 || m.n_used > 64) { c.set(INFR_ERR_UNSUPPORTED, "MoeFfn: n_expert > 2048 or n_used > 64"); break; }
                 if (m.has_ep_band) {
                     c.set(INFR_ERR_UNSUPPORTED, "MoeFfn: ep_band (expert-parallel shard) is a multi-device lowering; "
                                                 "this backend runs all experts on one device");
@@ -610,6 +610,7 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
         s.weights = (float*)p; p += round_up(rows * m.n_used * 4 + 4, 256);
         s.h = (float*)p;
     }
+    if (plan->arena) infr::launch_fill_zero(be->stream, plan->arena, arena);
     *out = plan;
     return INFR_OK;
 }
@@ -684,23 +685,19 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                 int re = 1, rb = 4;
                 geometry(plan->tensors[m.router].dtype, &re, &rb);
                 size_t router_row_bytes = (size_t)(m.ne / re) * rb;
+                infr::RouteParams rp{};
+                rp.logits = sc.logits; rp.n_expert = (int)m.n_expert; rp.n_used = (int)m.n_used; rp.rows = rows;
+                rp.gating = m.gating; rp.norm_w = (int)m.norm_w; rp.scale = m.scale;
+                rp.exp_probs_b = m.exp_probs_b == INFR_NO_TENSOR ? nullptr : (const float*)ptr[m.exp_probs_b];
+                rp.n_groups = (int)m.n_expert_groups; rp.n_groups_used = (int)m.n_expert_groups_used;
+                rp.expert_ids = m.expert_ids == INFR_NO_TENSOR ? nullptr : (const int32_t*)ptr[m.expert_ids];
+                rp.ids = sc.ids; rp.weights = sc.weights; rp.probs = sc.probs;
                 {
                     Timed t(be, "router_logits");
                     if (!infr::launch_router_logits(s, (const uint8_t*)ptr[m.router], plan->tensors[m.router].dtype,
                                                     router_row_bytes, (const float*)ptr[m.router_x], (int)m.ne,
                                                     (int)m.n_expert, rows, sc.logits))
                         return fail(INFR_ERR_UNSUPPORTED, "MoeFfn: ne=%u does not fit the router kernel's LDS budget", m.ne);
-                }
-                {
-                    infr::RouteParams rp{};
-                    rp.logits = sc.logits; rp.n_expert = (int)m.n_expert; rp.n_used = (int)m.n_used; rp.rows = rows;
-                    rp.gating = m.gating; rp.norm_w = (int)m.norm_w; rp.scale = m.scale;
-                    rp.exp_probs_b = m.exp_probs_b == INFR_NO_TENSOR ? nullptr : (const float*)ptr[m.exp_probs_b];
-                    rp.n_groups = (int)m.n_expert_groups; rp.n_groups_used = (int)m.n_expert_groups_used;
-                    rp.expert_ids = m.expert_ids == INFR_NO_TENSOR ? nullptr : (const int32_t*)ptr[m.expert_ids];
-                    rp.ids = sc.ids; rp.weights = sc.weights; rp.probs = sc.probs;
-                    Timed t(be, "route_topk");
-                    infr::launch_route(s, rp);
                 }
                 infr::MoeGemvParams gp{};
                 gp.ids = sc.ids; gp.weights = sc.weights;
@@ -729,8 +726,14 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                 gp.weight_before = (int)m.weight_before; gp.fused_gate_up = (int)m.fused_gate_up;
                 gp.h = sc.h; gp.dst = (float*)ptr[m.dst]; gp.n_cu = n_cu;
                 gp.x = (const float*)ptr[m.x];
+                gp.route = rp;
+                gp.route_inline = infr::moe_gate_up_routes_inline(gp) ? 1 : 0;
+                if (!gp.route_inline) {
+                    Timed t(be, "route_topk");
+                    infr::launch_route(s, rp);
+                }
                 {
-                    Timed t(be, "moe_gate_up");
+                    Timed t(be, gp.route_inline ? "moe_route_gate_up" : "moe_gate_up");
                     infr::launch_moe_gate_up(s, gp);
                 }
                 gp.x = nullptr;

@@ -37,16 +37,19 @@ __device__ __forceinline__ float bf16_bits_to_f32(uint32_t bits) {
 // reference's f32::exp resolves to): table of 2^(i/32) in double, degree-3 polynomial, every
 // multiply-add fused, including the range reduction r = x*N/ln2 - k.  Checked against the
 // host expf over every float with |x| <= 104 (zero differences).
-__device__ __forceinline__ float expf_libm(float x) {
-    constexpr uint64_t T[32] = {
-        0x3ff0000000000000ull, 0x3fefd9b0d3158574ull, 0x3fefb5586cf9890full, 0x3fef9301d0125b51ull,
-        0x3fef72b83c7d517bull, 0x3fef54873168b9aaull, 0x3fef387a6e756238ull, 0x3fef1e9df51fdee1ull,
-        0x3fef06fe0a31b715ull, 0x3feef1a7373aa9cbull, 0x3feedea64c123422ull, 0x3feece086061892dull,
-        0x3feebfdad5362a27ull, 0x3feeb42b569d4f82ull, 0x3feeab07dd485429ull, 0x3feea47eb03a5585ull,
-        0x3feea09e667f3bcdull, 0x3fee9f75e8ec5f74ull, 0x3feea11473eb0187ull, 0x3feea589994cce13ull,
-        0x3feeace5422aa0dbull, 0x3feeb737b0cdc5e5ull, 0x3feec49182a3f090ull, 0x3feed503b23e255dull,
-        0x3feee89f995ad3adull, 0x3feeff76f2fb5e47ull, 0x3fef199bdd85529cull, 0x3fef3720dcef9069ull,
-        0x3fef5818dcfba487ull, 0x3fef7c97337b9b5full, 0x3fefa4afa2a490daull, 0x3fefd0765b6e4540ull};
+__device__ const uint64_t kExp2Table[32] = {
+    0x3ff0000000000000ull, 0x3fefd9b0d3158574ull, 0x3fefb5586cf9890full, 0x3fef9301d0125b51ull,
+    0x3fef72b83c7d517bull, 0x3fef54873168b9aaull, 0x3fef387a6e756238ull, 0x3fef1e9df51fdee1ull,
+    0x3fef06fe0a31b715ull, 0x3feef1a7373aa9cbull, 0x3feedea64c123422ull, 0x3feece086061892dull,
+    0x3feebfdad5362a27ull, 0x3feeb42b569d4f82ull, 0x3feeab07dd485429ull, 0x3feea47eb03a5585ull,
+    0x3feea09e667f3bcdull, 0x3fee9f75e8ec5f74ull, 0x3feea11473eb0187ull, 0x3feea589994cce13ull,
+    0x3feeace5422aa0dbull, 0x3feeb737b0cdc5e5ull, 0x3feec49182a3f090ull, 0x3feed503b23e255dull,
+    0x3feee89f995ad3adull, 0x3feeff76f2fb5e47ull, 0x3fef199bdd85529cull, 0x3fef3720dcef9069ull,
+    0x3fef5818dcfba487ull, 0x3fef7c97337b9b5full, 0x3fefa4afa2a490daull, 0x3fefd0765b6e4540ull};
+
+// T: the 32-entry table above, in global memory or a copy staged in LDS (a kernel on a latency
+// critical path copies it once at start so later lookups do not wait on a global load).
+__device__ __forceinline__ float expf_libm(float x, const uint64_t* T) {
     // Out-of-range and non-finite inputs: same special cases as libm.
     if (!(x == x)) return x + x;
     if (x > 0x1.62e42ep6f) return __builtin_huge_valf();
@@ -71,27 +74,29 @@ __device__ __forceinline__ float expf_libm(float x) {
     y = __dmul_rn(y, s);
     return (float)y;
 }
+__device__ __forceinline__ float expf_libm(float x) { return expf_libm(x, kExp2Table); }
 
 // act_fn of the reference (crates/infr-cpu/src/kernels.rs:6664-6672), same operation order.
-__device__ __forceinline__ float act_fn(int act, float g) {
-    if (act == INFR_ACT_SILU) return __fdiv_rn(g, __fadd_rn(1.0f, expf_libm(-g)));
+__device__ __forceinline__ float act_fn(int act, float g, const uint64_t* T = kExp2Table) {
+    if (act == INFR_ACT_SILU) return __fdiv_rn(g, __fadd_rn(1.0f, expf_libm(-g, T)));
     if (act == INFR_ACT_GELU) {
         float g3 = __fmul_rn(__fmul_rn(__fmul_rn(0.044715f, g), g), g);
         float inner = __fmul_rn(0.7978846f, __fadd_rn(g, g3));
         float t = __fadd_rn(1.0f, tanhf(inner));
         return __fmul_rn(__fmul_rn(0.5f, g), t);
     }
-    return __fdiv_rn(1.0f, __fadd_rn(1.0f, expf_libm(-g)));
+    return __fdiv_rn(1.0f, __fadd_rn(1.0f, expf_libm(-g, T)));
 }
 
 // gated_act_fn (kernels.rs:6678-6683).
-__device__ __forceinline__ float gated_act_fn(int act, bool has_clamp, float clamp, float gate, float up) {
-    if (!has_clamp) return __fmul_rn(act_fn(act, gate), up);
+__device__ __forceinline__ float gated_act_fn(int act, bool has_clamp, float clamp, float gate, float up,
+                                              const uint64_t* T = kExp2Table) {
+    if (!has_clamp) return __fmul_rn(act_fn(act, gate, T), up);
     float gm = gate < clamp ? gate : clamp;
     float uc = up;
     if (uc < -clamp) uc = -clamp;
     if (uc > clamp) uc = clamp;
-    return __fmul_rn(act_fn(act, gm), uc);
+    return __fmul_rn(act_fn(act, gm, T), uc);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -172,16 +177,74 @@ __device__ inline float decode_elem(int dtype, const uint8_t* row, uint32_t k) {
 }
 
 // ---------------------------------------------------------------------------------------------
-// Wave64 helpers.
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off, kWave);
+// Wave64 helpers.  Cross-lane steps inside a row of 16 lanes use DPP (no LDS round trip);
+// the four row results meet through readlane.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+template <int CTRL>
+__device__ __forceinline__ uint32_t dpp_u(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xF, 0xF, true);
+}
+// Rows selected by ROW_MASK read the DPP source, the other rows read 0 (used with
+// row_bcast:15 / row_bcast:31 to carry a row's total into the following rows).
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_rows_f(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xF, false));
+}
+constexpr int kDppXor1 = 0xB1;        // quad_perm [1,0,3,2]
+constexpr int kDppXor2 = 0x4E;        // quad_perm [2,3,0,1]
+constexpr int kDppHalfMirror = 0x141; // lane i <-> 7-i inside each 8
+constexpr int kDppMirror = 0x140;     // lane i <-> 15-i inside each 16
+
+__device__ __forceinline__ float quad_sum(float v) {
+    v += dpp_f<kDppXor1>(v);
+    v += dpp_f<kDppXor2>(v);
     return v;
 }
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, kWave));
+__device__ __forceinline__ float oct_sum(float v) {
+    v = quad_sum(v);
+    return v + dpp_f<kDppHalfMirror>(v);
+}
+__device__ __forceinline__ float row16_sum(float v) {
+    v = quad_sum(v);
+    v += dpp_f<kDppHalfMirror>(v);
+    v += dpp_f<kDppMirror>(v);
     return v;
+}
+__device__ __forceinline__ float readlane_f(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+// Every lane receives the sum over the wavefront.
+__device__ __forceinline__ float wave_sum(float v) {
+    v = row16_sum(v);
+    return (readlane_f(v, 0) + readlane_f(v, 16)) + (readlane_f(v, 32) + readlane_f(v, 48));
+}
+__device__ __forceinline__ float wave_max(float v) {
+    v = fmaxf(v, dpp_f<kDppXor1>(v));
+    v = fmaxf(v, dpp_f<kDppXor2>(v));
+    v = fmaxf(v, dpp_f<kDppHalfMirror>(v));
+    v = fmaxf(v, dpp_f<kDppMirror>(v));
+    return fmaxf(fmaxf(readlane_f(v, 0), readlane_f(v, 16)), fmaxf(readlane_f(v, 32), readlane_f(v, 48)));
+}
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+    v = max(v, dpp_u<kDppXor1>(v));
+    v = max(v, dpp_u<kDppXor2>(v));
+    v = max(v, dpp_u<kDppHalfMirror>(v));
+    v = max(v, dpp_u<kDppMirror>(v));
+    uint32_t a = max((uint32_t)__builtin_amdgcn_readlane((int)v, 0), (uint32_t)__builtin_amdgcn_readlane((int)v, 16));
+    uint32_t b = max((uint32_t)__builtin_amdgcn_readlane((int)v, 32), (uint32_t)__builtin_amdgcn_readlane((int)v, 48));
+    return max(a, b);
+}
+__device__ __forceinline__ uint32_t wave_min_u32(uint32_t v) {
+    v = min(v, dpp_u<kDppXor1>(v));
+    v = min(v, dpp_u<kDppXor2>(v));
+    v = min(v, dpp_u<kDppHalfMirror>(v));
+    v = min(v, dpp_u<kDppMirror>(v));
+    uint32_t a = min((uint32_t)__builtin_amdgcn_readlane((int)v, 0), (uint32_t)__builtin_amdgcn_readlane((int)v, 16));
+    uint32_t b = min((uint32_t)__builtin_amdgcn_readlane((int)v, 32), (uint32_t)__builtin_amdgcn_readlane((int)v, 48));
+    return min(a, b);
 }
 
 // Sum of v over each run of `seg` consecutive lanes (seg need not be a power of two); the

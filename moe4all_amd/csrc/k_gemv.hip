@@ -2,32 +2,172 @@
 // gated activation fused (h = act(gate.x) * (up.x)), and over the down bank with the
 // rank-ordered weighted combine fused into the epilogue.
 //
-// Layout idea: a wavefront owns whole weight rows.  Every lane owns a FIXED slice of the K
-// dimension, so its slice of the activation vector stays in registers for all the rows the
-// wavefront streams; only packed weight blocks move from HBM, in 128-bit loads.  A row of
-// nblk blocks occupies nblk*LPB consecutive lanes (LPB = lanes per block, a property of the
-// format); when that is <= 32 several rows ride in one wavefront side by side.
+// Layout: a wavefront owns whole weight rows.  Every lane owns a FIXED slice of the K
+// dimension (64 elements for the K-quants, 32 for Q8_0), so its slice of the activation
+// vector is prepared once and stays in registers for all rows the wavefront streams; only
+// packed weight blocks move from HBM, in 128-bit loads.  A row of nblk blocks occupies
+// nblk*LPB consecutive lanes (LPB = lanes per block); when that is <= 32 several rows ride in
+// one wavefront side by side.  All weight loads of a round are issued before the first dot.
 //
-// Numerics: f32 everywhere.  A block's contribution is evaluated in factored form,
-//   sum_i (d*sc)*q_i*x_i + (dmin*m)*x_i  =  (d*sc) * (sum q_i x_i) + (dmin*m) * (sum x_i),
-// which is exact-product arithmetic for a one-hot x, so a one-hot activation reads back the
-// reference's decoded weight bit for bit (crates/infr-gguf/src/dequant.rs:35-51).
+// Arithmetic.  The lane's activation slice is held as 23-bit fixed point per group of 16/32
+// elements, x ~ 2^k * X with |X| <= 2^21 (k from the group's largest magnitude; a power of
+// two, so scaling is exact), and X is split into three signed bytes X = 65536*A + 256*B + C.
+// Packed weight codes q (4, 6 or 8 bits) contract with A, B and C in V_DOT4_I32_I8; the three
+// integer sums are exact and are joined in f32, which rounds the group's sum(q*x~) once at
+// 2^-24 relative.  The block scales are applied in f32 in factored form,
+//     (d*sc) * sum(q*x~) + (dmin*m) * sum(x~),
+// so a one-hot x reads back the reference's decoded weight bit for bit
+// (crates/infr-gguf/src/dequant.rs:35-51).  For general x the rounding of x to 2^-22 of its
+// group's largest magnitude is of the order of f32's own 2^-24, so results track the f32
+// reference as closely as a reordered f32 summation does.
 #include "device_common.h"
 #include "kernels.h"
+#include "route.h"
 
 namespace infr {
 
-__device__ __forceinline__ float ub0(uint32_t v) { return (float)(v & 0xFFu); }
-__device__ __forceinline__ float ub1(uint32_t v) { return (float)((v >> 8) & 0xFFu); }
-__device__ __forceinline__ float ub2(uint32_t v) { return (float)((v >> 16) & 0xFFu); }
-__device__ __forceinline__ float ub3(uint32_t v) { return (float)(v >> 24); }
+#ifdef INFR_TRACE
+// Experiment-only stage timestamps (100 MHz wall clock), one record of 8 per wave.
+__device__ unsigned long long g_trace[8 * 8192];
+unsigned long long* trace_ptr() {
+    void* p = nullptr;
+    (void)hipGetSymbolAddress(&p, HIP_SYMBOL(g_trace));
+    return (unsigned long long*)p;
+}
+#define TRACE(slot, dep)                                                               \
+    do {                                                                               \
+        asm volatile("" ::"v"(dep));                                                   \
+        if (lane == 0) g_trace[(size_t)((blockIdx.x * 8 + wave) & 8191) * 8 + (slot)] = wall_clock64(); \
+    } while (0)
+#else
+#define TRACE(slot, dep) do {} while (0)
+#endif
 
-__device__ __forceinline__ float dot4(uint32_t packed, const float* x, float acc) {
-    acc = fmaf(ub0(packed), x[0], acc);
-    acc = fmaf(ub1(packed), x[1], acc);
-    acc = fmaf(ub2(packed), x[2], acc);
-    acc = fmaf(ub3(packed), x[3], acc);
-    return acc;
+__device__ __forceinline__ int dot4i(uint32_t a, uint32_t b, int c) {
+    return __builtin_amdgcn_sdot4((int)a, (int)b, c, false);
+}
+
+// ---- activation staging -------------------------------------------------------------------
+// A wavefront converts the activation vector once, cooperatively, into LDS "cells" of 32
+// elements (28 dwords: byte planes A, B, C of the fixed-point values, then scales and sums),
+// and each lane then fetches the cells of its own K slice.  Element 4k+q of a group sits in
+// byte q of dword k of each plane, the order in which byte-parallel unpacking yields codes.
+//   G == 32: [A 8][B 8][C 8][scale][sum][pad 2]            one group of 32
+//   G == 16: [A0 4][B0 4][C0 4][A1 4][B1 4][C1 4][k0][s0][k1][s1]   two groups of 16
+// SIGNED digits (X = 65536*A + 256*B + C with every digit in [-128,127]) serve signed weight
+// codes; otherwise B and C are the plain unsigned bytes of X's two's complement (A signed),
+// which costs no arithmetic to extract and pairs with the unsigned dot for non-negative codes.
+constexpr int kCellDwords = 28;
+
+__device__ __forceinline__ uint32_t perm(uint32_t hi, uint32_t lo, uint32_t sel) {
+    return __builtin_amdgcn_perm(hi, lo, sel);
+}
+
+// Byte `B` of four dwords -> one dword (x0's byte in byte 0).
+template <int B>
+__device__ __forceinline__ uint32_t gather_byte(uint32_t x0, uint32_t x1, uint32_t x2, uint32_t x3) {
+    // v_perm_b32 selects bytes from {hi,lo}: selector values 0-3 = lo bytes, 4-7 = hi bytes
+    const uint32_t lo = perm(x1, x0, (uint32_t)(B | ((4 + B) << 8)));          // [x0.B, x1.B, -, -]
+    const uint32_t hi = perm(x3, x2, (uint32_t)(B | ((4 + B) << 8)));          // [x2.B, x3.B, -, -]
+    return perm(hi, lo, 0x05040100u);                                          // [lo.0, lo.1, hi.0, hi.1]
+}
+
+template <int N, bool SIGNED>
+__device__ __forceinline__ void quant_to_cell(const float* x, uint32_t* a, uint32_t* b, uint32_t* c, uint32_t* ks) {
+    float amax = 0.f;
+#pragma unroll
+    for (int i = 0; i < N; i++) amax = fmaxf(amax, fabsf(x[i]));
+    const uint32_t eb = (__float_as_uint(amax) >> 23) & 0xFFu;  // amax in [2^(eb-127), 2^(eb-126))
+    const bool live = eb >= 22u && eb < 255u;
+    const float inv = live ? __uint_as_float((274u - eb) << 23) : 0.f;  // 2^(20 - E): |x| * inv < 2^21
+    const float scale = live ? __uint_as_float((eb - 20u) << 23) : 0.f; // 2^(E - 20)
+    int sx = 0;
+#pragma unroll
+    for (int k = 0; k < N / 4; k++) {
+        int X[4];
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            X[q] = __float2int_rn(x[4 * k + q] * inv);  // exact scaling, |X| <= 2^21
+            sx += X[q];
+        }
+        if (SIGNED) {
+            uint32_t aw = 0, bw = 0, cw = 0;
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const int C = (int)(int8_t)(X[q] & 0xFF);
+                const int R = (X[q] - C) >> 8;
+                const int B = (int)(int8_t)(R & 0xFF);
+                const int A = (R - B) >> 8;
+                aw |= (uint32_t)(A & 0xFF) << (8 * q);
+                bw |= (uint32_t)(B & 0xFF) << (8 * q);
+                cw |= (uint32_t)(C & 0xFF) << (8 * q);
+            }
+            a[k] = aw; b[k] = bw; c[k] = cw;
+        } else {
+            a[k] = gather_byte<2>((uint32_t)X[0], (uint32_t)X[1], (uint32_t)X[2], (uint32_t)X[3]);
+            b[k] = gather_byte<1>((uint32_t)X[0], (uint32_t)X[1], (uint32_t)X[2], (uint32_t)X[3]);
+            c[k] = gather_byte<0>((uint32_t)X[0], (uint32_t)X[1], (uint32_t)X[2], (uint32_t)X[3]);
+        }
+    }
+    ks[0] = __float_as_uint(scale);
+    ks[1] = __float_as_uint((float)sx * scale);  // sum(x~); |sx| <= 2^26 rounds at 2^-24 like any f32 sum
+}
+
+// Lane L of the wave converts elements [32L, 32L+32) of x[0..n) (n <= 2048 per pass).  The
+// global loads are split from the conversion so a kernel can request x early and convert it
+// while later loads are in flight.
+struct XLoad { float t[32]; };
+__device__ __forceinline__ XLoad stage_x_load(const float* __restrict__ x, int n, int c0) {
+    XLoad l;
+    const float4* src = reinterpret_cast<const float4*>(x + (size_t)(c0 * 32 < n ? c0 : 0) * 32);
+#pragma unroll
+    for (int k = 0; k < 8; k++) {
+        float4 v = src[k];
+        l.t[4 * k] = v.x; l.t[4 * k + 1] = v.y; l.t[4 * k + 2] = v.z; l.t[4 * k + 3] = v.w;
+    }
+    return l;
+}
+template <int G, bool SIGNED>
+__device__ __forceinline__ void stage_x_convert(const XLoad& l, int n, int c0, uint32_t* cells) {
+    if (c0 * 32 >= n) return;
+    uint32_t cell[kCellDwords];
+    if (G == 32) {
+        quant_to_cell<32, SIGNED>(l.t, cell, cell + 8, cell + 16, cell + 24);
+        cell[26] = cell[27] = 0;
+    } else {
+        quant_to_cell<16, SIGNED>(l.t, cell, cell + 4, cell + 8, cell + 24);
+        quant_to_cell<16, SIGNED>(l.t + 16, cell + 12, cell + 16, cell + 20, cell + 26);
+    }
+    uint4* dst = reinterpret_cast<uint4*>(cells + (size_t)c0 * kCellDwords);
+#pragma unroll
+    for (int k = 0; k < 7; k++) dst[k] = make_uint4(cell[4 * k], cell[4 * k + 1], cell[4 * k + 2], cell[4 * k + 3]);
+}
+// Whole vector, any n: first pass from an early load, further passes loaded here.
+template <int G, bool SIGNED>
+__device__ __forceinline__ void stage_x_finish(const XLoad& first, const float* __restrict__ x, int n, uint32_t* cells,
+                                               int lane) {
+    stage_x_convert<G, SIGNED>(first, n, lane, cells);
+    for (int c0 = lane + kWave; c0 * 32 < n; c0 += kWave) {
+        XLoad l = stage_x_load(x, n, c0);
+        stage_x_convert<G, SIGNED>(l, n, c0, cells);
+    }
+}
+
+__device__ __forceinline__ void fetch_dwords(uint32_t* dst, const uint32_t* src, int n4) {
+    const uint4* s4 = reinterpret_cast<const uint4*>(src);
+    for (int k = 0; k < n4; k++) {
+        uint4 v = s4[k];
+        dst[4 * k] = v.x; dst[4 * k + 1] = v.y; dst[4 * k + 2] = v.z; dst[4 * k + 3] = v.w;
+    }
+}
+
+__device__ __forceinline__ int udot4i(uint32_t a, uint32_t b, int c) {
+    return (int)__builtin_amdgcn_udot4(a, b, (uint32_t)c, false);
+}
+
+// sum(q * X) from the three exact byte-plane sums, rounded once or twice at 2^-24.
+__device__ __forceinline__ float join3(int sa, int sb, int sc) {
+    return fmaf((float)sa, 65536.0f, fmaf((float)sb, 256.0f, (float)sc));
 }
 
 __device__ __forceinline__ void load16(float* dst, const float* src) {
@@ -40,37 +180,48 @@ __device__ __forceinline__ void load16(float* dst, const float* src) {
 }
 
 // ------------------------------------------------------------------------------- Q4_K
-// 144 B: [f16 d][f16 dmin][12 B 6-bit scales/mins][128 B nibbles].  8 lanes per block; lane i
-// owns nibble bytes [16i, 16i+16): low nibbles are elements j*64+l0+t, high nibbles
-// j*64+32+l0+t (j = i/2, l0 = 16*(i&1)), i.e. sub-blocks 2j and 2j+1.
+// 144 B: [f16 d][f16 dmin][12 B 6-bit scales/mins][128 B nibbles].  4 lanes per block; lane j
+// owns nibble bytes [32j, 32j+32): low nibbles are elements j*64+t (sub-block 2j), high
+// nibbles j*64+32+t (sub-block 2j+1), t < 32.
 struct Q4KFmt {
-    static constexpr int kBlockBytes = 144, kBlockElems = 256, kLPB = 8;
-    struct X { float lo[16], hi[16]; float slo, shi; };
-    struct Raw { uint4 hdr, qs; };
-    static __device__ __forceinline__ void load_x(X& x, const float* xb, int i) {
-        const int j = i >> 1, l0 = (i & 1) * 16;
-        load16(x.lo, xb + j * 64 + l0);
-        load16(x.hi, xb + j * 64 + 32 + l0);
-        float a = 0.f, b = 0.f;
+    static constexpr int kBlockBytes = 144, kBlockElems = 256, kLPB = 4;
+    static constexpr int kGroup = 32;
+    static constexpr bool kSigned = false;
+    struct X { uint32_t alo[8], blo[8], clo[8], ahi[8], bhi[8], chi[8]; float klo, khi, slo, shi; };
+    struct Raw { uint4 hdr, qa, qb; };
+    // lane j of block blk: cells 8*blk + 2j (low nibbles) and + 1 (high nibbles)
+    static __device__ __forceinline__ void fetch_x(X& x, const uint32_t* cells, int blk, int j) {
+        const uint32_t* lo = cells + (size_t)(8 * blk + 2 * j) * kCellDwords;
+        const uint32_t* hi = lo + kCellDwords;
+        uint32_t t[28];
 #pragma unroll
-        for (int t = 0; t < 16; t++) { a += x.lo[t]; b += x.hi[t]; }
-        x.slo = a; x.shi = b;
-    }
-    static __device__ __forceinline__ void zero_x(X& x) {
+        for (int k = 0; k < 7; k++) {
+            uint4 v = reinterpret_cast<const uint4*>(lo)[k];
+            t[4 * k] = v.x; t[4 * k + 1] = v.y; t[4 * k + 2] = v.z; t[4 * k + 3] = v.w;
+        }
 #pragma unroll
-        for (int t = 0; t < 16; t++) { x.lo[t] = 0.f; x.hi[t] = 0.f; }
-        x.slo = 0.f; x.shi = 0.f;
+        for (int k = 0; k < 8; k++) { x.alo[k] = t[k]; x.blo[k] = t[8 + k]; x.clo[k] = t[16 + k]; }
+        x.klo = __uint_as_float(t[24]); x.slo = __uint_as_float(t[25]);
+#pragma unroll
+        for (int k = 0; k < 7; k++) {
+            uint4 v = reinterpret_cast<const uint4*>(hi)[k];
+            t[4 * k] = v.x; t[4 * k + 1] = v.y; t[4 * k + 2] = v.z; t[4 * k + 3] = v.w;
+        }
+#pragma unroll
+        for (int k = 0; k < 8; k++) { x.ahi[k] = t[k]; x.bhi[k] = t[8 + k]; x.chi[k] = t[16 + k]; }
+        x.khi = __uint_as_float(t[24]); x.shi = __uint_as_float(t[25]);
     }
-    static __device__ __forceinline__ Raw load(const uint8_t* blk, int i) {
+    static __device__ __forceinline__ Raw load(const uint8_t* blk, int j) {
         Raw r;
         r.hdr = *reinterpret_cast<const uint4*>(blk);
-        r.qs = *reinterpret_cast<const uint4*>(blk + 16 + 16 * i);
+        r.qa = *reinterpret_cast<const uint4*>(blk + 16 + 32 * j);
+        r.qb = *reinterpret_cast<const uint4*>(blk + 32 + 32 * j);
         return r;
     }
-    static __device__ __forceinline__ float dot(const Raw& r, int i, const X& x) {
-        const int j = i >> 1;
+    static __device__ __forceinline__ float dot(const Raw& r, int j, const X& x) {
         const float d = f16_bits_to_f32(r.hdr.x & 0xFFFFu);
         const float dmin = f16_bits_to_f32(r.hdr.x >> 16);
+        // 6-bit (scale, min) of sub-blocks 2j and 2j+1, as adjacent bytes (get_scale_min_k4)
         const uint32_t sh = (uint32_t)(j & 1) * 16u;
         const uint32_t y = r.hdr.y >> sh, z = r.hdr.z >> sh, w = r.hdr.w >> sh;
         uint32_t sc, m;
@@ -81,16 +232,23 @@ struct Q4KFmt {
             sc = (w & 0x0F0Fu) | ((y >> 2) & 0x3030u);
             m = ((w >> 4) & 0x0F0Fu) | ((z >> 2) & 0x3030u);
         }
-        float alo = 0.f, ahi = 0.f;
-        const uint32_t q[4] = {r.qs.x, r.qs.y, r.qs.z, r.qs.w};
+        const uint32_t q[8] = {r.qa.x, r.qa.y, r.qa.z, r.qa.w, r.qb.x, r.qb.y, r.qb.z, r.qb.w};
+        int la = 0, lb = 0, lc = 0, ha = 0, hb = 0, hc = 0;
 #pragma unroll
-        for (int k = 0; k < 4; k++) {
-            alo = dot4(q[k] & 0x0F0F0F0Fu, x.lo + 4 * k, alo);
-            ahi = dot4((q[k] >> 4) & 0x0F0F0F0Fu, x.hi + 4 * k, ahi);
+        for (int k = 0; k < 8; k++) {
+            const uint32_t lo = q[k] & 0x0F0F0F0Fu, hi = (q[k] >> 4) & 0x0F0F0F0Fu;
+            la = dot4i(lo, x.alo[k], la);   // A signed; B, C plain unsigned bytes; codes are 0..15
+            lb = udot4i(lo, x.blo[k], lb);
+            lc = udot4i(lo, x.clo[k], lc);
+            ha = dot4i(hi, x.ahi[k], ha);
+            hb = udot4i(hi, x.bhi[k], hb);
+            hc = udot4i(hi, x.chi[k], hc);
         }
-        const float s0 = d * ub0(sc), s1 = d * ub1(sc);
-        const float m0 = dmin * ub0(m), m1 = dmin * ub1(m);
-        return (s0 * alo - m0 * x.slo) + (s1 * ahi - m1 * x.shi);
+        const float flo = join3(la, lb, lc) * x.klo;
+        const float fhi = join3(ha, hb, hc) * x.khi;
+        const float s0 = d * (float)(sc & 0xFFu), s1 = d * (float)(sc >> 8);
+        const float m0 = dmin * (float)(m & 0xFFu), m1 = dmin * (float)(m >> 8);
+        return (s0 * flo - m0 * x.slo) + (s1 * fhi - m1 * x.shi);
     }
 };
 
@@ -101,25 +259,27 @@ struct Q4KFmt {
 // h*128 + g*32 + l0 (scale byte h*8 + 2g + (i&1)).  Blocks are only 2-byte aligned.
 struct Q6KFmt {
     static constexpr int kBlockBytes = 210, kBlockElems = 256, kLPB = 4;
-    struct X { float v[4][16]; float s32[4]; };
+    static constexpr int kGroup = 16;
+    static constexpr bool kSigned = false;
+    struct X { uint32_t a[4][4], b[4][4], c[4][4]; float k[4], s32[4]; };
     struct Raw { uint4 qla, qlb, qh; uint2 sc; uint32_t d; };
-    static __device__ __forceinline__ void load_x(X& x, const float* xb, int i) {
-        const int h = i >> 1, l0 = (i & 1) * 16;
+    // lane i of block blk: 16-groups 16*blk + 8h + 2g + (i&1), g = 0..3; a cell holds two
+    static __device__ __forceinline__ void fetch_x(X& x, const uint32_t* cells, int blk, int i) {
+        const int h = i >> 1, odd = i & 1;
 #pragma unroll
         for (int g = 0; g < 4; g++) {
-            load16(x.v[g], xb + h * 128 + g * 32 + l0);
-            float a = 0.f;
+            const int t = 16 * blk + 8 * h + 2 * g + odd;
+            const uint32_t* cell = cells + (size_t)(t >> 1) * kCellDwords;
+            const uint32_t* pl = cell + (t & 1) * 12;
 #pragma unroll
-            for (int t = 0; t < 16; t++) a += x.v[g][t];
-            x.s32[g] = 32.0f * a;
-        }
-    }
-    static __device__ __forceinline__ void zero_x(X& x) {
-#pragma unroll
-        for (int g = 0; g < 4; g++) {
-#pragma unroll
-            for (int t = 0; t < 16; t++) x.v[g][t] = 0.f;
-            x.s32[g] = 0.f;
+            for (int q = 0; q < 3; q++) {
+                uint4 v = reinterpret_cast<const uint4*>(pl)[q];
+                uint32_t* dst = q == 0 ? x.a[g] : q == 1 ? x.b[g] : x.c[g];
+                dst[0] = v.x; dst[1] = v.y; dst[2] = v.z; dst[3] = v.w;
+            }
+            const uint2 ks = *reinterpret_cast<const uint2*>(cell + 24 + 2 * (t & 1));
+            x.k[g] = __uint_as_float(ks.x);
+            x.s32[g] = 32.0f * __uint_as_float(ks.y);
         }
     }
     static __device__ __forceinline__ Raw load(const uint8_t* blk, int i) {
@@ -136,49 +296,55 @@ struct Q6KFmt {
         const uint32_t a[4] = {r.qla.x, r.qla.y, r.qla.z, r.qla.w};
         const uint32_t b[4] = {r.qlb.x, r.qlb.y, r.qlb.z, r.qlb.w};
         const uint32_t hq[4] = {r.qh.x, r.qh.y, r.qh.z, r.qh.w};
-        float acc[4] = {0.f, 0.f, 0.f, 0.f};
+        int sa[4] = {0, 0, 0, 0}, sb[4] = {0, 0, 0, 0}, sc[4] = {0, 0, 0, 0};
 #pragma unroll
         for (int k = 0; k < 4; k++) {
-            const uint32_t q0 = (a[k] & 0x0F0F0F0Fu) | ((hq[k] << 4) & 0x30303030u);
-            const uint32_t q1 = (b[k] & 0x0F0F0F0Fu) | ((hq[k] << 2) & 0x30303030u);
-            const uint32_t q2 = ((a[k] >> 4) & 0x0F0F0F0Fu) | (hq[k] & 0x30303030u);
-            const uint32_t q3 = ((b[k] >> 4) & 0x0F0F0F0Fu) | ((hq[k] >> 2) & 0x30303030u);
-            acc[0] = dot4(q0, x.v[0] + 4 * k, acc[0]);
-            acc[1] = dot4(q1, x.v[1] + 4 * k, acc[1]);
-            acc[2] = dot4(q2, x.v[2] + 4 * k, acc[2]);
-            acc[3] = dot4(q3, x.v[3] + 4 * k, acc[3]);
+            uint32_t q[4];
+            q[0] = (a[k] & 0x0F0F0F0Fu) | ((hq[k] << 4) & 0x30303030u);
+            q[1] = (b[k] & 0x0F0F0F0Fu) | ((hq[k] << 2) & 0x30303030u);
+            q[2] = ((a[k] >> 4) & 0x0F0F0F0Fu) | (hq[k] & 0x30303030u);
+            q[3] = ((b[k] >> 4) & 0x0F0F0F0Fu) | ((hq[k] >> 2) & 0x30303030u);
+#pragma unroll
+            for (int g = 0; g < 4; g++) {
+                sa[g] = dot4i(q[g], x.a[g][k], sa[g]);   // codes are 0..63
+                sb[g] = udot4i(q[g], x.b[g][k], sb[g]);
+                sc[g] = udot4i(q[g], x.c[g][k], sc[g]);
+            }
         }
         const float d = f16_bits_to_f32(r.d);
         const uint32_t sx = (i & 1) ? (r.sc.x >> 8) : r.sc.x;
         const uint32_t sy = (i & 1) ? (r.sc.y >> 8) : r.sc.y;
-        const float s0 = (float)(int)(int8_t)(sx & 0xFFu);
-        const float s1 = (float)(int)(int8_t)((sx >> 16) & 0xFFu);
-        const float s2 = (float)(int)(int8_t)(sy & 0xFFu);
-        const float s3 = (float)(int)(int8_t)((sy >> 16) & 0xFFu);
-        return ((d * s0) * (acc[0] - x.s32[0]) + (d * s1) * (acc[1] - x.s32[1])) +
-               ((d * s2) * (acc[2] - x.s32[2]) + (d * s3) * (acc[3] - x.s32[3]));
+        const float s[4] = {(float)(int)(int8_t)(sx & 0xFFu), (float)(int)(int8_t)((sx >> 16) & 0xFFu),
+                            (float)(int)(int8_t)(sy & 0xFFu), (float)(int)(int8_t)((sy >> 16) & 0xFFu)};
+        float acc = 0.f;
+#pragma unroll
+        for (int g = 0; g < 4; g++) {
+            const float f = join3(sa[g], sb[g], sc[g]) * x.k[g];  // sum(q*x~)
+            acc += (d * s[g]) * (f - x.s32[g]);                    // d*s*sum((q-32)*x~)
+        }
+        return acc;
     }
 };
 
 // ------------------------------------------------------------------------------- Q8_0
-// 34 B: [f16 d][32 x i8].  One lane per block.  Signed bytes are biased to unsigned
-// (q+128) for the byte->float conversion and the bias leaves through 128 * sum(x).
+// 34 B: [f16 d][32 x i8].  One lane per block; the signed codes contract directly.
 struct Q80Fmt {
     static constexpr int kBlockBytes = 34, kBlockElems = 32, kLPB = 1;
-    struct X { float v[32]; float s128; };
+    static constexpr int kGroup = 32;
+    static constexpr bool kSigned = true;  // signed weight codes need signed digits throughout
+    struct X { uint32_t a[8], b[8], c[8]; float k; };
     struct Raw { uint4 a, b; uint32_t d; };
-    static __device__ __forceinline__ void load_x(X& x, const float* xb, int) {
-        load16(x.v, xb);
-        load16(x.v + 16, xb + 16);
-        float a = 0.f;
+    static __device__ __forceinline__ void fetch_x(X& x, const uint32_t* cells, int blk, int) {
+        const uint32_t* cell = cells + (size_t)blk * kCellDwords;
+        uint32_t t[28];
 #pragma unroll
-        for (int t = 0; t < 32; t++) a += x.v[t];
-        x.s128 = 128.0f * a;
-    }
-    static __device__ __forceinline__ void zero_x(X& x) {
+        for (int k = 0; k < 7; k++) {
+            uint4 v = reinterpret_cast<const uint4*>(cell)[k];
+            t[4 * k] = v.x; t[4 * k + 1] = v.y; t[4 * k + 2] = v.z; t[4 * k + 3] = v.w;
+        }
 #pragma unroll
-        for (int t = 0; t < 32; t++) x.v[t] = 0.f;
-        x.s128 = 0.f;
+        for (int k = 0; k < 8; k++) { x.a[k] = t[k]; x.b[k] = t[8 + k]; x.c[k] = t[16 + k]; }
+        x.k = __uint_as_float(t[24]);
     }
     static __device__ __forceinline__ Raw load(const uint8_t* blk, int) {
         Raw r;
@@ -189,175 +355,208 @@ struct Q80Fmt {
     }
     static __device__ __forceinline__ float dot(const Raw& r, int, const X& x) {
         const uint32_t q[8] = {r.a.x, r.a.y, r.a.z, r.a.w, r.b.x, r.b.y, r.b.z, r.b.w};
-        float acc = 0.f;
+        int sa = 0, sb = 0, sc = 0;
 #pragma unroll
-        for (int k = 0; k < 8; k++) acc = dot4(q[k] ^ 0x80808080u, x.v + 4 * k, acc);
-        return f16_bits_to_f32(r.d) * (acc - x.s128);
+        for (int k = 0; k < 8; k++) {
+            sa = dot4i(q[k], x.a[k], sa);
+            sb = dot4i(q[k], x.b[k], sb);
+            sc = dot4i(q[k], x.c[k], sc);
+        }
+        const float f = join3(sa, sb, sc) * x.k;
+        return f16_bits_to_f32(r.d) * f;
     }
 };
 
-// Lane placement of a wavefront over weight rows of nblk blocks.
-//   KS == 1: lanes_per_row = nblk*LPB <= 64, rows_per_wave = 64 / lanes_per_row.
-//   KS == 2: 64 < lanes_per_row <= 128, one row per wave, two K slices per lane.
-template <class F, int KS>
+// Lane placement of a wavefront over weight rows of nblk blocks: lanes_per_row = nblk*LPB
+// (<= 64), rows_per_wave = 64 / lanes_per_row.  Left-over lanes of the wave are pointed at the
+// last row and flagged off: they load and compute like everyone else, so the code stays
+// branch-free and every load of a round is issued back to back; their result is dropped.
+template <class F>
 struct Place {
-    int lpr, rw_count, rw, pos;          // lanes per row, rows per wave, my row, my lane in row
-    int blk[KS], sub[KS];                // my block in the row and lane inside the block
-    bool on[KS];
+    int lpr, rw_count, rw, pos;  // lanes per row, rows per wave, my row (clamped), my lane in the row
+    bool row_on;
+    int blk, sub;                // my block in the row and my lane inside the block
+    int wpos;                    // lane-in-row where the row's sum lands
     __device__ __forceinline__ Place(int nblk, int lane) {
         lpr = nblk * F::kLPB;
-        if (KS == 1) {
-            rw_count = kWave / lpr;
-            rw = lane / lpr;
-            pos = lane - rw * lpr;
-        } else {
-            rw_count = 1;
-            rw = 0;
-            pos = lane;
-        }
-#pragma unroll
-        for (int ks = 0; ks < KS; ks++) {
-            int id = pos + kWave * ks;
-            blk[ks] = id / F::kLPB;
-            sub[ks] = id - blk[ks] * F::kLPB;
-            on[ks] = rw < rw_count && blk[ks] < nblk;
-        }
+        rw_count = kWave / lpr;
+        const int rw_raw = lane / lpr;
+        pos = lane - rw_raw * lpr;
+        row_on = rw_raw < rw_count;
+        rw = row_on ? rw_raw : rw_count - 1;
+        blk = pos / F::kLPB;
+        sub = pos - blk * F::kLPB;
+        wpos = (lpr == 64 || lpr == 32 || lpr == 16) ? lpr - 1 : 0;
     }
+    __device__ __forceinline__ bool writer() const { return row_on && pos == wpos; }
 };
 
-template <class F, int KS>
-__device__ __forceinline__ void load_x_all(typename F::X (&xs)[KS], const Place<F, KS>& pl, const float* x) {
-#pragma unroll
-    for (int ks = 0; ks < KS; ks++) {
-        if (pl.on[ks]) F::load_x(xs[ks], x + (size_t)pl.blk[ks] * F::kBlockElems, pl.sub[ks]);
-        else F::zero_x(xs[ks]);
+// LDS bytes one wave needs to stage an activation vector of n elements.
+static inline size_t cells_bytes(int n) { return (size_t)((n + 31) / 32) * kCellDwords * sizeof(uint32_t); }
+template <class F>
+__device__ __forceinline__ typename F::Raw load_row(const Place<F>& pl, const uint8_t* row) {
+    return F::load(row + (size_t)pl.blk * F::kBlockBytes, pl.sub);
+}
+
+// Sum of v over the lanes of each weight row; valid in the row's writer lane.
+template <class F>
+__device__ __forceinline__ float row_sum(float v, const Place<F>& pl, int nblk) {
+    if (pl.lpr >= 16 && (pl.lpr & (pl.lpr - 1)) == 0) {
+        v = row16_sum(v);                                            // every lane: sum of its 16
+        if (pl.lpr >= 32) v += dpp_rows_f<0x142, 0xA>(v);            // rows 1,3 += lane 15 of rows 0,2
+        if (pl.lpr == 64) v += dpp_rows_f<0x143, 0xC>(v);            // rows 2,3 += lane 31
+        return v;
     }
-}
-
-template <class F, int KS>
-__device__ __forceinline__ void load_row(typename F::Raw (&raw)[KS], const Place<F, KS>& pl, const uint8_t* row,
-                                         bool valid) {
-#pragma unroll
-    for (int ks = 0; ks < KS; ks++)
-        if (valid && pl.on[ks]) raw[ks] = F::load(row + (size_t)pl.blk[ks] * F::kBlockBytes, pl.sub[ks]);
-}
-
-template <class F, int KS>
-__device__ __forceinline__ float dot_row(const typename F::Raw (&raw)[KS], const Place<F, KS>& pl,
-                                         const typename F::X (&xs)[KS], bool valid) {
-    float s = 0.f;
-#pragma unroll
-    for (int ks = 0; ks < KS; ks++)
-        if (valid && pl.on[ks]) s += F::dot(raw[ks], pl.sub[ks], xs[ks]);
-    return s;
-}
-
-template <class F, int KS>
-__device__ __forceinline__ float row_sum(float v, const Place<F, KS>& pl) {
-    if (KS == 2 || pl.lpr == kWave) return wave_sum(v);
-    return segment_sum(v, pl.lpr, pl.pos);
+    // lanes of one block first (rows start at multiples of kLPB lanes, so DPP groups line up) ...
+    if (F::kLPB == 4) v = quad_sum(v);
+    // ... then the row's blocks, by doubling; the total lands in the row's first lane
+    for (int ob = 1; ob < nblk; ob <<= 1) {
+        float t = __shfl_down(v, ob * F::kLPB, kWave);
+        if (pl.blk + ob < nblk) v += t;
+    }
+    return v;
 }
 
 // ------------------------------------------------------------------------------- gate/up
 // grid.x = tiles of `ft` features, grid.y = token row.  A block's 4 waves share the items
-// (slot, f) of its tile round-robin; x is identical for every slot of a token.
-template <class F, int KS>
+// (slot, f) of its tile; x is identical for every slot of a token.  U = items a wave has in
+// flight per round.  Results wait in LDS and one lane per item applies the gated activation
+// after the round, so the f64 exp and the divide run once per wave, not once per item.
+template <class F, int U>
 __global__ __launch_bounds__(256) void moe_gate_up_fast(MoeGemvParams p, int ft) {
+    extern __shared__ uint32_t dyn_lds[];
+    __shared__ uint64_t s_tab[32];
+    __shared__ int32_t s_ids[64];
+    __shared__ float s_w[64];
+    __shared__ float s_g[4][64], s_u[4][64];
     const int r = blockIdx.y;
     const int f0 = blockIdx.x * ft;
     const int fcount = min(ft, p.nff - f0);
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int nblk = p.ne / F::kBlockElems;
     const size_t row_bytes = (size_t)nblk * F::kBlockBytes;
-    const Place<F, KS> pl(nblk, lane);
-    typename F::X xs[KS];
-    load_x_all<F, KS>(xs, pl, p.x + (size_t)r * p.ne);
-
-    const int nitems = fcount * p.n_used;
-    const int32_t* ids = p.ids + (size_t)r * p.n_used;
-    const int stride = 4 * pl.rw_count;
-    typename F::Raw graw[KS], uraw[KS];
-    int it = wave * pl.rw_count + pl.rw;
-    auto rows_of = [&](int item, const uint8_t*& grow, const uint8_t*& urow) {
-        int slot = item / fcount, f = f0 + (item - slot * fcount);
-        int e = ids[slot];
-        grow = p.gate + (size_t)e * p.gate_stride + (size_t)f * row_bytes;
-        urow = p.up + (size_t)e * p.up_stride + (size_t)f * row_bytes;
-    };
-    {
-        const uint8_t *g = nullptr, *u = nullptr;
-        bool v = it < nitems;
-        if (v) rows_of(it, g, u);
-        load_row<F, KS>(graw, pl, g, v);
-        load_row<F, KS>(uraw, pl, u, v);
+    const Place<F> pl(nblk, lane);
+    const size_t cell_words = (size_t)((p.ne + 31) / 32) * kCellDwords;
+    uint32_t* cells = dyn_lds + (size_t)wave * cell_words;
+    TRACE(0, lane);
+    // x is requested first; it does not depend on the routing
+    const float* xrow = p.x + (size_t)r * p.ne;
+    const XLoad xl = stage_x_load(xrow, p.ne, lane);
+    if (threadIdx.x < 32) s_tab[threadIdx.x] = kExp2Table[threadIdx.x];
+    if (p.route_inline) {
+        // every block routes its token row itself (one wave, redundantly across blocks)
+        __syncthreads();
+        if (wave == 0)
+            route_row_any(p.route, r, lane, reinterpret_cast<float*>(dyn_lds + 4 * cell_words), s_tab, s_ids, s_w,
+                          blockIdx.x == 0);
+    } else if ((int)threadIdx.x < p.n_used) {  // n_used <= 64
+        s_ids[threadIdx.x] = p.ids[(size_t)r * p.n_used + threadIdx.x];
+        s_w[threadIdx.x] = p.weights[(size_t)r * p.n_used + threadIdx.x];
     }
-    for (int base = wave * pl.rw_count; base < nitems; base += stride, it += stride) {
-        const bool valid = it < nitems;
-        typename F::Raw gn[KS], un[KS];
-        {
-            const uint8_t *g = nullptr, *u = nullptr;
-            bool v = it + stride < nitems;
-            if (v) rows_of(it + stride, g, u);
-            load_row<F, KS>(gn, pl, g, v);
-            load_row<F, KS>(un, pl, u, v);
-        }
-        float gs = dot_row<F, KS>(graw, pl, xs, valid);
-        float us = dot_row<F, KS>(uraw, pl, xs, valid);
-        gs = row_sum<F, KS>(gs, pl);
-        us = row_sum<F, KS>(us, pl);
-        if (valid && pl.pos == 0 && pl.rw < pl.rw_count) {
-            int slot = it / fcount, f = f0 + (it - slot * fcount);
-            if (p.weight_before) {
-                float wp = p.weights[(size_t)r * p.n_used + slot];
-                gs = __fmul_rn(wp, gs);
-                us = __fmul_rn(wp, us);
-            }
-            p.h[((size_t)r * p.n_used + slot) * p.nff + f] = gated_act_fn(p.act, p.has_clamp, p.clamp, gs, us);
-        }
+    __syncthreads();
+    TRACE(1, s_ids[0]);
+    __builtin_amdgcn_wave_barrier();
+    const int nitems = fcount * p.n_used;
+    const int per_round = 4 * pl.rw_count;
+    typename F::X x;
+    bool have_x = false;
+    for (int base = 0; base < nitems; base += per_round * U) {
+        typename F::Raw graw[U], uraw[U];
 #pragma unroll
-        for (int ks = 0; ks < KS; ks++) { graw[ks] = gn[ks]; uraw[ks] = un[ks]; }
+        for (int u = 0; u < U; u++) {
+            const int it = min(base + (u * 4 + wave) * pl.rw_count + pl.rw, nitems - 1);  // past the end: re-read the last
+            const int slot = it / fcount, f = f0 + (it - slot * fcount);
+            const int e = s_ids[slot];
+            graw[u] = load_row<F>(pl, p.gate + (size_t)e * p.gate_stride + (size_t)f * row_bytes);
+            uraw[u] = load_row<F>(pl, p.up + (size_t)e * p.up_stride + (size_t)f * row_bytes);
+        }
+        if (!have_x) {
+            // while the weights are in flight: the wave converts x to fixed point once, together
+            stage_x_finish<F::kGroup, F::kSigned>(xl, xrow, p.ne, cells, lane);
+            __builtin_amdgcn_wave_barrier();
+            F::fetch_x(x, cells, pl.blk, pl.sub);
+            have_x = true;
+        }
+        TRACE(4, *reinterpret_cast<const uint32_t*>(&x));
+        TRACE(2, *reinterpret_cast<const uint32_t*>(&graw[0]));
+        TRACE(3, *reinterpret_cast<const uint32_t*>(&uraw[U - 1]));
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            float gs = row_sum<F>(F::dot(graw[u], pl.sub, x), pl, nblk);
+            float us = row_sum<F>(F::dot(uraw[u], pl.sub, x), pl, nblk);
+            if (pl.writer()) {
+                s_g[wave][u * pl.rw_count + pl.rw] = gs;
+                s_u[wave][u * pl.rw_count + pl.rw] = us;
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+        TRACE(5, s_g[wave][0]);
+        if (lane < U * pl.rw_count) {
+            const int u = lane / pl.rw_count, rw = lane - u * pl.rw_count;
+            const int it = base + (u * 4 + wave) * pl.rw_count + rw;
+            if (it < nitems) {
+                const int slot = it / fcount, f = f0 + (it - slot * fcount);
+                float gs = s_g[wave][lane], us = s_u[wave][lane];
+                if (p.weight_before) {
+                    const float wp = s_w[slot];
+                    gs = __fmul_rn(wp, gs);
+                    us = __fmul_rn(wp, us);
+                }
+                p.h[((size_t)r * p.n_used + slot) * p.nff + f] = gated_act_fn(p.act, p.has_clamp, p.clamp, gs, us, s_tab);
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+        TRACE(6, lane);
     }
 }
 
 // ------------------------------------------------------------------------------- down
-// grid.x = tiles of `ot` output rows, grid.y = token row.  Wave w streams the down rows of
-// slots w, w+4, ... for the block's output rows (that slot's h stays in registers), the
-// per-slot results meet in LDS and are combined in rank order:
-//   out += w_rank * y_rank  as a separate multiply and add (crates/infr-cpu/src/lib.rs:4290-4302).
+// grid.x = tiles of `ot` = S * rows-per-wave output rows, grid.y = token row.  One wave per
+// slot: it holds that slot's h and streams the S row groups of its expert's down matrix, all
+// loads issued up front.  The per-slot results meet in LDS and are combined in rank order:
+// out += w_rank * y_rank as a separate multiply and add
+// (crates/infr-cpu/src/lib.rs:4290-4302).
 constexpr int kMaxUsedFast = 16;
-constexpr int kMaxOt = 32;
+constexpr int kMaxOt = 64;
 
-template <class F, int KS>
-__global__ __launch_bounds__(256) void moe_down_combine_fast(MoeGemvParams p, int ot) {
+template <class F, int S>
+__global__ __launch_bounds__(512) void moe_down_combine_fast(MoeGemvParams p, int ot) {
+    extern __shared__ uint32_t dyn_lds[];
     __shared__ float ypart[kMaxUsedFast][kMaxOt];
     const int r = blockIdx.y;
     const int o0 = blockIdx.x * ot;
     const int ocount = min(ot, p.ne - o0);
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int nwaves = blockDim.x >> 6;
     const int nblk = p.nff / F::kBlockElems;
     const size_t row_bytes = (size_t)nblk * F::kBlockBytes;
-    const Place<F, KS> pl(nblk, lane);
+    const Place<F> pl(nblk, lane);
     const int32_t* ids = p.ids + (size_t)r * p.n_used;
+    uint32_t* cells = dyn_lds + (size_t)wave * ((p.nff + 31) / 32) * kCellDwords;
 
-    for (int slot = wave; slot < p.n_used; slot += 4) {
-        const int e = ids[slot];
+    for (int slot = wave; slot < p.n_used; slot += nwaves) {
+        const int e = ids[slot];  // first: every weight address below waits on it
+        const float* hrow = p.h + ((size_t)r * p.n_used + slot) * p.nff;
+        const XLoad xl = stage_x_load(hrow, p.nff, lane);
         const uint8_t* bank = p.down + (size_t)e * p.down_stride + (size_t)o0 * row_bytes;
-        typename F::X xs[KS];
-        load_x_all<F, KS>(xs, pl, p.h + ((size_t)r * p.n_used + slot) * p.nff);
-        const float ds = p.down_scale ? p.down_scale[e] : 1.0f;
-        typename F::Raw raw[KS];
-        load_row<F, KS>(raw, pl, bank + (size_t)pl.rw * row_bytes, pl.rw < ocount);
-        for (int oo = 0; oo < ocount; oo += pl.rw_count) {
-            const int o = oo + pl.rw;
-            const bool valid = o < ocount;
-            typename F::Raw nx[KS];
-            const int on = o + pl.rw_count;
-            load_row<F, KS>(nx, pl, bank + (size_t)on * row_bytes, on < ocount);
-            float y = dot_row<F, KS>(raw, pl, xs, valid);
-            y = row_sum<F, KS>(y, pl);
-            if (valid && pl.pos == 0 && pl.rw < pl.rw_count) ypart[slot][o] = p.down_scale ? __fmul_rn(y, ds) : y;
+        typename F::Raw raw[S];
 #pragma unroll
-            for (int ks = 0; ks < KS; ks++) raw[ks] = nx[ks];
+        for (int st = 0; st < S; st++) {
+            const int o = min(st * pl.rw_count + pl.rw, ocount - 1);  // rows past the tile re-read its last row
+            raw[st] = load_row<F>(pl, bank + (size_t)o * row_bytes);
+        }
+        // while the weights are in flight: this slot's h to fixed point, once per wave
+        __builtin_amdgcn_wave_barrier();
+        stage_x_finish<F::kGroup, F::kSigned>(xl, hrow, p.nff, cells, lane);
+        __builtin_amdgcn_wave_barrier();
+        typename F::X x;
+        F::fetch_x(x, cells, pl.blk, pl.sub);
+        const float ds = p.down_scale ? p.down_scale[e] : 1.0f;
+#pragma unroll
+        for (int st = 0; st < S; st++) {
+            const int o = st * pl.rw_count + pl.rw;
+            float y = row_sum<F>(F::dot(raw[st], pl.sub, x), pl, nblk);
+            if (o < ocount && pl.writer()) ypart[slot][o] = p.down_scale ? __fmul_rn(y, ds) : y;
         }
     }
     __syncthreads();
@@ -373,13 +572,14 @@ __global__ __launch_bounds__(256) void moe_down_combine_fast(MoeGemvParams p, in
 }
 
 // ------------------------------------------------------------------------------- generic
-// Any dtype decode_elem understands and any shape: one wave per output, lanes stride over K.
+// Any dtype decode_elem understands and any shape: one wave per output, lanes stride over K,
+// plain f32.
 __global__ __launch_bounds__(256) void moe_gate_up_generic(MoeGemvParams p, size_t g_row_bytes, size_t u_row_bytes) {
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int f = blockIdx.x * 4 + wave;
     const int pair = blockIdx.y;
     if (f >= p.nff) return;
-    const int r = pair / p.n_used, slot = pair - r * p.n_used;
+    const int r = pair / p.n_used;
     const int e = p.ids[pair];
     const uint8_t* grow = p.gate + (size_t)e * p.gate_stride + (size_t)f * g_row_bytes;
     const uint8_t* urow = p.up + (size_t)e * p.up_stride + (size_t)f * u_row_bytes;
@@ -400,7 +600,6 @@ __global__ __launch_bounds__(256) void moe_gate_up_generic(MoeGemvParams p, size
         }
         p.h[(size_t)pair * p.nff + f] = gated_act_fn(p.act, p.has_clamp, p.clamp, gs, us);
     }
-    (void)slot;
 }
 
 __global__ __launch_bounds__(256) void moe_down_combine_generic(MoeGemvParams p, size_t row_bytes) {
@@ -430,39 +629,43 @@ static size_t row_bytes_of(int dt, int in_f) {
     return (size_t)(in_f / be) * bb;
 }
 
-// 0: no fast path; 1 or 2: K slices per lane.
+// The fast kernels cover rows of up to 64 lanes (K-quants: in_f <= 4096, Q8_0: in_f <= 2048).
 template <class F>
-static int fast_ks(int in_f) {
-    if (in_f % F::kBlockElems != 0) return 0;
-    int lpr = in_f / F::kBlockElems * F::kLPB;
-    if (lpr <= 64) return 1;
-    if (lpr <= 128) return 2;
-    return 0;
+static bool fast_ok(int in_f) {
+    if (in_f <= 0 || in_f % F::kBlockElems != 0) return false;
+    return in_f / F::kBlockElems * F::kLPB <= 64;
 }
 
-static int tile_for(int total, int n_cu, int granule, int cap) {
-    // about one block per compute unit, a multiple of the rows a wave carries at once
-    int t = (total + n_cu - 1) / n_cu;
-    t = (t + granule - 1) / granule * granule;
-    if (t < granule) t = granule;
-    if (t > cap) t = cap / granule * granule;
-    if (t < 1) t = 1;
-    return t;
-}
+static int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
 template <class F>
 static bool try_gate_up(hipStream_t s, const MoeGemvParams& p) {
-    int ks = fast_ks<F>(p.ne);
-    if (!ks) return false;
-    int lpr = p.ne / F::kBlockElems * F::kLPB;
-    int rw = ks == 1 ? 64 / lpr : 1;
-    // items per block = ft * n_used, spread over 4 waves carrying rw rows each
-    int ft = tile_for(p.nff, p.n_cu, 1, 1 << 20);
-    (void)rw;
-    dim3 grid((p.nff + ft - 1) / ft, p.rows), block(256);
-    if (ks == 1) hipLaunchKernelGGL((moe_gate_up_fast<F, 1>), grid, block, 0, s, p, ft);
-    else hipLaunchKernelGGL((moe_gate_up_fast<F, 2>), grid, block, 0, s, p, ft);
+    if (!fast_ok<F>(p.ne) || p.n_used > 64) return false;
+    const int rw = 64 / (p.ne / F::kBlockElems * F::kLPB);
+    // about one block per compute unit; a block's ft * n_used items go to 4 waves of rw rows each
+    int ft = ceil_div(p.nff, p.n_cu);
+    if (ft < 1) ft = 1;
+    const int per_wave = ceil_div(ft * p.n_used, 4 * rw);
+    dim3 grid(ceil_div(p.nff, ft), p.rows), block(256);
+    // U * rw results per wave must fit the 64-entry staging rows
+    int u = per_wave < 1 ? 1 : per_wave;
+    while (u * rw > 64) u--;
+    const size_t lds = 4 * cells_bytes(p.ne) +
+                       (p.route_inline ? route_scratch_floats(p.route.n_expert, p.route.n_groups) * sizeof(float) : 0);
+    if (u >= 6) hipLaunchKernelGGL((moe_gate_up_fast<F, 6>), grid, block, lds, s, p, ft);
+    else if (u == 5 || u == 4) hipLaunchKernelGGL((moe_gate_up_fast<F, 4>), grid, block, lds, s, p, ft);
+    else if (u == 3) hipLaunchKernelGGL((moe_gate_up_fast<F, 3>), grid, block, lds, s, p, ft);
+    else if (u == 2) hipLaunchKernelGGL((moe_gate_up_fast<F, 2>), grid, block, lds, s, p, ft);
+    else hipLaunchKernelGGL((moe_gate_up_fast<F, 1>), grid, block, lds, s, p, ft);
     return true;
+}
+
+bool moe_gate_up_routes_inline(const MoeGemvParams& p) {
+    if (p.gate_dt != p.up_dt || p.n_used > 64) return false;
+    if (p.gate_dt == INFR_Q4K) return fast_ok<Q4KFmt>(p.ne);
+    if (p.gate_dt == INFR_Q6K) return fast_ok<Q6KFmt>(p.ne);
+    if (p.gate_dt == INFR_Q8_0) return fast_ok<Q80Fmt>(p.ne);
+    return false;
 }
 
 void launch_moe_gate_up(hipStream_t s, const MoeGemvParams& p) {
@@ -480,15 +683,24 @@ void launch_moe_gate_up(hipStream_t s, const MoeGemvParams& p) {
 
 template <class F>
 static bool try_down(hipStream_t s, const MoeGemvParams& p) {
-    int ks = fast_ks<F>(p.nff);
-    if (!ks || p.n_used > kMaxUsedFast) return false;
-    int lpr = p.nff / F::kBlockElems * F::kLPB;
-    int rw = ks == 1 ? 64 / lpr : 1;
-    int ot = tile_for(p.ne, p.n_cu, rw, kMaxOt);
-    if (ot > kMaxOt) ot = kMaxOt;
-    dim3 grid((p.ne + ot - 1) / ot, p.rows), block(256);
-    if (ks == 1) hipLaunchKernelGGL((moe_down_combine_fast<F, 1>), grid, block, 0, s, p, ot);
-    else hipLaunchKernelGGL((moe_down_combine_fast<F, 2>), grid, block, 0, s, p, ot);
+    if (!fast_ok<F>(p.nff) || p.n_used > kMaxUsedFast) return false;
+    const int rw = 64 / (p.nff / F::kBlockElems * F::kLPB);
+    // output rows per block ~ ne / n_cu, as S row groups of rw rows per wave, S in {1,2,4,8}
+    const int want = ceil_div(p.ne, p.n_cu);
+    int steps = 1;
+    while (steps < 8 && steps * rw < want) steps <<= 1;
+    while (steps > 1 && steps * rw > kMaxOt) steps >>= 1;
+    if (steps * rw > kMaxOt) return false;
+    const int ot = steps * rw;
+    const int nwaves = p.n_used < 8 ? p.n_used : 8;
+    dim3 grid(ceil_div(p.ne, ot), p.rows), block(64 * nwaves);
+    const size_t lds = nwaves * cells_bytes(p.nff);
+    switch (steps) {
+        case 1: hipLaunchKernelGGL((moe_down_combine_fast<F, 1>), grid, block, lds, s, p, ot); break;
+        case 2: hipLaunchKernelGGL((moe_down_combine_fast<F, 2>), grid, block, lds, s, p, ot); break;
+        case 4: hipLaunchKernelGGL((moe_down_combine_fast<F, 4>), grid, block, lds, s, p, ot); break;
+        default: hipLaunchKernelGGL((moe_down_combine_fast<F, 8>), grid, block, lds, s, p, ot); break;
+    }
     return true;
 }
 
@@ -504,32 +716,44 @@ void launch_moe_down_combine(hipStream_t s, const MoeGemvParams& p) {
 
 // ------------------------------------------------------------------------------- Op::Linear
 // dst[m, out_f] = x . W^T, the dense neighbour of the expert GEMVs (shared expert).
-template <class F, int KS>
-__global__ __launch_bounds__(256) void linear_fast(const float* __restrict__ x, const uint8_t* __restrict__ w,
+template <class F>
+__global__ __launch_bounds__(256) void linear_fast(const float* __restrict__ xin, const uint8_t* __restrict__ w,
                                                    int in_f, int out_f, float* __restrict__ dst, int ot) {
+    extern __shared__ uint32_t dyn_lds[];
+    constexpr int U = 4;  // rows a wave keeps in flight
     const int r = blockIdx.y;
     const int o0 = blockIdx.x * ot;
     const int ocount = min(ot, out_f - o0);
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int nblk = in_f / F::kBlockElems;
     const size_t row_bytes = (size_t)nblk * F::kBlockBytes;
-    const Place<F, KS> pl(nblk, lane);
-    typename F::X xs[KS];
-    load_x_all<F, KS>(xs, pl, x + (size_t)r * in_f);
+    const Place<F> pl(nblk, lane);
     const uint8_t* bank = w + (size_t)o0 * row_bytes;
-    const int stride = 4 * pl.rw_count;
-    typename F::Raw raw[KS];
-    int o = wave * pl.rw_count + pl.rw;
-    load_row<F, KS>(raw, pl, bank + (size_t)o * row_bytes, o < ocount);
-    for (int base = wave * pl.rw_count; base < ocount; base += stride, o += stride) {
-        const bool valid = o < ocount;
-        typename F::Raw nx[KS];
-        load_row<F, KS>(nx, pl, bank + (size_t)(o + stride) * row_bytes, o + stride < ocount);
-        float y = dot_row<F, KS>(raw, pl, xs, valid);
-        y = row_sum<F, KS>(y, pl);
-        if (valid && pl.pos == 0 && pl.rw < pl.rw_count) dst[(size_t)r * out_f + o0 + o] = y;
+    const int per_round = 4 * pl.rw_count;
+    uint32_t* cells = dyn_lds + (size_t)wave * ((in_f + 31) / 32) * kCellDwords;
+    const float* xrow = xin + (size_t)r * in_f;
+    const XLoad xl = stage_x_load(xrow, in_f, lane);
+    typename F::X x;
+    bool have_x = false;
+    for (int base = 0; base < ocount; base += per_round * U) {
+        typename F::Raw raw[U];
 #pragma unroll
-        for (int ks = 0; ks < KS; ks++) raw[ks] = nx[ks];
+        for (int u = 0; u < U; u++) {
+            const int o = min(base + (u * 4 + wave) * pl.rw_count + pl.rw, ocount - 1);
+            raw[u] = load_row<F>(pl, bank + (size_t)o * row_bytes);
+        }
+        if (!have_x) {
+            stage_x_finish<F::kGroup, F::kSigned>(xl, xrow, in_f, cells, lane);
+            __builtin_amdgcn_wave_barrier();
+            F::fetch_x(x, cells, pl.blk, pl.sub);
+            have_x = true;
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int o = base + (u * 4 + wave) * pl.rw_count + pl.rw;
+            float y = row_sum<F>(F::dot(raw[u], pl.sub, x), pl, nblk);
+            if (o < ocount && pl.writer()) dst[(size_t)r * out_f + o0 + o] = y;
+        }
     }
 }
 
@@ -551,14 +775,12 @@ __global__ __launch_bounds__(256) void linear_generic(const float* __restrict__ 
 template <class F>
 static bool try_linear(hipStream_t s, const float* x, const uint8_t* w, int m, int in_f, int out_f, float* dst,
                        int n_cu) {
-    int ks = fast_ks<F>(in_f);
-    if (!ks) return false;
-    int lpr = in_f / F::kBlockElems * F::kLPB;
-    int rw = ks == 1 ? 64 / lpr : 1;
-    int ot = tile_for(out_f, n_cu, 4 * rw, 1 << 20);
-    dim3 grid((out_f + ot - 1) / ot, m), block(256);
-    if (ks == 1) hipLaunchKernelGGL((linear_fast<F, 1>), grid, block, 0, s, x, w, in_f, out_f, dst, ot);
-    else hipLaunchKernelGGL((linear_fast<F, 2>), grid, block, 0, s, x, w, in_f, out_f, dst, ot);
+    if (!fast_ok<F>(in_f)) return false;
+    const int rw = 64 / (in_f / F::kBlockElems * F::kLPB);
+    int ot = ceil_div(out_f, n_cu);
+    ot = ceil_div(ot, 4 * rw) * 4 * rw;  // whole rounds of the block's 4 waves
+    dim3 grid(ceil_div(out_f, ot), m), block(256);
+    hipLaunchKernelGGL((linear_fast<F>), grid, block, 4 * cells_bytes(in_f), s, x, w, in_f, out_f, dst, ot);
     return true;
 }
 

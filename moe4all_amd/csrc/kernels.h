@@ -44,7 +44,13 @@ struct MoeGemvParams {
     float* h;                 // [rows, n_used, nff]
     float* dst;               // [rows, ne]
     int n_cu;
+    // When set, the gate/up kernel routes each token row itself from route.logits (every block
+    // redundantly; block 0 of a row publishes ids / weights / probs) and no route launch is needed.
+    int route_inline;
+    RouteParams route;
 };
+// True when launch_moe_gate_up will take the kernel that can route inline.
+bool moe_gate_up_routes_inline(const MoeGemvParams& p);
 // h = act(gate.x) * (up.x) for every (row, slot).
 void launch_moe_gate_up(hipStream_t s, const MoeGemvParams& p);
 // dst[row] = sum over slots (rank order) of w * (down . h).

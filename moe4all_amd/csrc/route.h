@@ -1,0 +1,204 @@
+// Routing of one token row by one wavefront: gating -> selection -> routing weights, in the
+// reference's operation order (crates/infr-cpu/src/lib.rs:3741-3863).  Shared by the
+// standalone route kernel and by the decode GEMV kernel, where every block routes its own
+// token row redundantly instead of waiting for a separate launch.
+#pragma once
+
+#include "device_common.h"
+#include "kernels.h"
+
+namespace infr {
+
+// ---------------------------------------------------------------------------------------------
+// Routing of one token row by one wavefront.  lds: 2*n floats (+ n_groups) of scratch, tab: the
+// exp table staged in LDS.  NS = candidates per lane (n <= 64*NS).
+__device__ __forceinline__ uint32_t order_key(float v) {
+    uint32_t u = __float_as_uint(v);
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+
+// Results go to global memory (p.ids / p.weights / p.probs) when store_global is set, and to
+// lds_ids / lds_w when those are non-null.
+template <int NS>
+__device__ __forceinline__ void route_row(const RouteParams& p, int row, int lane, float* lds, const uint64_t* tab,
+                                          int32_t* lds_ids, float* lds_w, bool store_global) {
+    const int n = p.n_expert;
+    float* prob = lds;
+    float* sel = lds + n;
+    float* gscore = sel + n;
+    const float* lg = p.logits + (size_t)row * n;
+    const float ninf = -__builtin_huge_valf();
+
+    float pr[NS];
+#pragma unroll
+    for (int s = 0; s < NS; s++) {
+        int i = s * kWave + lane;
+        pr[s] = i < n ? lg[i] : ninf;
+    }
+    // ---- gating (lib.rs:3746-3774)
+    if (p.gating == INFR_GATING_SOFTMAX) {
+        float m = ninf;
+#pragma unroll
+        for (int s = 0; s < NS; s++) m = fmaxf(m, pr[s]);
+        m = wave_max(m);
+#pragma unroll
+        for (int s = 0; s < NS; s++) pr[s] = (s * kWave + lane < n) ? expf_libm(__fsub_rn(pr[s], m), tab) : 0.0f;
+        // psum = p[0] + p[1] + ... strictly left to right: element s*64+l sits in lane l, slot s
+        // (constant lane numbers: the chain is one readlane + one add per element)
+        float psum = 0.0f;
+#pragma unroll
+        for (int s = 0; s < NS; s++) {
+            const int cnt = n - s * kWave;
+            if (cnt >= kWave) {
+#pragma unroll
+                for (int l = 0; l < kWave; l++) psum = __fadd_rn(psum, readlane_f(pr[s], l));
+            } else {
+                for (int l = 0; l < cnt; l++) psum = __fadd_rn(psum, readlane_f(pr[s], l));
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < NS; s++) pr[s] = __fdiv_rn(pr[s], psum);
+    } else if (p.gating == INFR_GATING_SIGMOID) {
+#pragma unroll
+        for (int s = 0; s < NS; s++) pr[s] = __fdiv_rn(1.0f, __fadd_rn(1.0f, expf_libm(-pr[s], tab)));
+    } else {
+#pragma unroll
+        for (int s = 0; s < NS; s++) {
+            float v = pr[s];
+            float sp = v > 20.0f ? v : logf(__fadd_rn(1.0f, expf_libm(v, tab)));
+            pr[s] = __fsqrt_rn(sp);
+        }
+    }
+#pragma unroll
+    for (int s = 0; s < NS; s++) {
+        int i = s * kWave + lane;
+        if (i < n) prob[i] = pr[s];
+    }
+    __builtin_amdgcn_wave_barrier();
+
+    int32_t* ids_out = p.ids + (size_t)row * p.n_used;
+    float* w_out = p.weights + (size_t)row * p.n_used;
+    int my_id = 0;  // lane k < n_used holds the rank-k expert
+    if (p.expert_ids) {
+        // Hash routing (lib.rs:3776-3793): the supplied ids are the selection, in table order.
+        if (lane < p.n_used) {
+            int e = p.expert_ids[(size_t)row * p.n_used + lane];
+            my_id = e < 0 ? 0 : (e >= n ? n - 1 : e);
+        }
+    } else {
+        float sl[NS];
+        // lib.rs:3797-3806: bias on a selection-only copy.
+#pragma unroll
+        for (int s = 0; s < NS; s++) {
+            int i = s * kWave + lane;
+            sl[s] = (p.exp_probs_b && i < n) ? __fadd_rn(pr[s], p.exp_probs_b[i]) : pr[s];
+        }
+        // lib.rs:3809-3846: group-limited routing.
+        if (p.n_groups > 1 && p.n_groups_used > 0) {
+            const int ng = p.n_groups, per = n / ng;
+#pragma unroll
+            for (int s = 0; s < NS; s++) {
+                int i = s * kWave + lane;
+                if (i < n) sel[i] = sl[s];
+            }
+            __builtin_amdgcn_wave_barrier();
+            for (int g = lane; g < ng; g += kWave) {
+                float b0 = ninf, b1 = ninf;
+                for (int i = g * per; i < (g + 1) * per; i++) {
+                    float sv = sel[i];
+                    if (sv > b0) { b1 = b0; b0 = sv; }
+                    else if (sv > b1) { b1 = sv; }
+                }
+                gscore[g] = __fadd_rn(b0, b1);
+            }
+            __builtin_amdgcn_wave_barrier();
+            // Keep the top n_groups_used groups (stable descending).  chosen: group g -> lane g%64, bit g/64.
+            uint32_t chosen = 0;
+            const int ngu = p.n_groups_used < ng ? p.n_groups_used : ng;
+            for (int k = 0; k < ngu; k++) {
+                uint32_t bk = 0, bi = 0xFFFFFFFFu;
+                for (int g = lane, t = 0; g < ng; g += kWave, t++) {
+                    if (chosen & (1u << t)) continue;
+                    uint32_t key = order_key(gscore[g]);
+                    if (bi == 0xFFFFFFFFu || key > bk) { bk = key; bi = (uint32_t)g; }
+                }
+                uint32_t kmax = wave_max_u32(bi == 0xFFFFFFFFu ? 0u : bk);
+                uint32_t win = wave_min_u32((bi != 0xFFFFFFFFu && bk == kmax) ? bi : 0xFFFFFFFFu);
+                if (win != 0xFFFFFFFFu && (int)(win & 63u) == lane) chosen |= 1u << (win >> 6);
+            }
+            for (int g = lane, t = 0; g < ng; g += kWave, t++) {
+                if (!(chosen & (1u << t)))
+                    for (int i = g * per; i < (g + 1) * per; i++) sel[i] = ninf;
+            }
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int s = 0; s < NS; s++) {
+                int i = s * kWave + lane;
+                if (i < n) sl[s] = sel[i];
+            }
+        }
+        // Top n_used by (sel desc, id asc).
+        uint32_t taken = 0;
+#pragma unroll
+        for (int s = 0; s < NS; s++)
+            if (s * kWave + lane >= n) taken |= 1u << s;
+        for (int k = 0; k < p.n_used; k++) {
+            uint32_t bk = 0, bi = 0xFFFFFFFFu;
+#pragma unroll
+            for (int s = 0; s < NS; s++) {
+                if (taken & (1u << s)) continue;
+                uint32_t key = order_key(sl[s]);
+                if (bi == 0xFFFFFFFFu || key > bk) { bk = key; bi = (uint32_t)(s * kWave + lane); }
+            }
+            uint32_t kmax = wave_max_u32(bi == 0xFFFFFFFFu ? 0u : bk);
+            uint32_t win = wave_min_u32((bi != 0xFFFFFFFFu && bk == kmax) ? bi : 0xFFFFFFFFu);
+            if (win == 0xFFFFFFFFu) win = 0;
+            if ((int)(win & 63u) == lane) taken |= 1u << (win >> 6);
+            if (lane == k) my_id = (int)win;
+        }
+    }
+    // ---- routing weights (lib.rs:3856-3861): lane k owns rank k
+    const bool mine = lane < p.n_used;
+    float pk = mine ? prob[my_id] : 0.0f;
+    float w;
+    if (p.norm_w) {
+        float wsum = 0.0f;
+        for (int k = 0; k < p.n_used; k++) wsum = __fadd_rn(wsum, readlane_f(pk, k));
+        wsum = fmaxf(wsum, 1e-20f);
+        w = __fmul_rn(__fdiv_rn(pk, wsum), p.scale);
+    } else {
+        w = __fmul_rn(pk, p.scale);
+    }
+    if (mine) {
+        if (store_global) {
+            ids_out[lane] = my_id;
+            w_out[lane] = w;
+        }
+        if (lds_ids) lds_ids[lane] = my_id;
+        if (lds_w) lds_w[lane] = w;
+    }
+    if (p.probs && store_global) {
+#pragma unroll
+        for (int s = 0; s < NS; s++) {
+            int i = s * kWave + lane;
+            if (i < n) p.probs[(size_t)row * n + i] = pr[s];
+        }
+    }
+}
+
+__device__ __forceinline__ void route_row_any(const RouteParams& p, int row, int lane, float* lds, const uint64_t* tab,
+                                              int32_t* lds_ids = nullptr, float* lds_w = nullptr,
+                                              bool store_global = true) {
+    const int n = p.n_expert;
+    if (n <= 128) route_row<2>(p, row, lane, lds, tab, lds_ids, lds_w, store_global);
+    else if (n <= 256) route_row<4>(p, row, lane, lds, tab, lds_ids, lds_w, store_global);
+    else if (n <= 512) route_row<8>(p, row, lane, lds, tab, lds_ids, lds_w, store_global);
+    else route_row<32>(p, row, lane, lds, tab, lds_ids, lds_w, store_global);
+}
+
+// LDS floats route_row_any needs behind the 64-float exp table.
+__host__ __device__ inline size_t route_scratch_floats(int n_expert, int n_groups) {
+    return (size_t)2 * n_expert + (size_t)(n_groups > 0 ? n_groups : 0);
+}
+
+}  // namespace infr
