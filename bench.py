@@ -78,6 +78,9 @@ def main():
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-timing", action="store_true")
+    ap.add_argument("--copy-probe-mib", type=int, default=0,
+                    help="also run one plain device-to-device copy of this many MiB (a known-size kernel that "
+                         "calibrates hardware byte counters in a profiler run)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus must be 1 (no multi-GPU path exists in this tree)",
@@ -113,6 +116,13 @@ def main():
             if shape.shared_ff:
                 b.bind(d["sg"], lw.shared[0]).bind(d["su"], lw.shared[1]).bind(d["sd"], lw.shared[2])
         binds.append(b)
+    if args.copy_probe_mib:
+        n = args.copy_probe_mib << 20
+        src, dst = be.alloc(n), be.alloc(n)
+        be.copy_buffer(src, dst, n)
+        be.sync()
+        src.free()
+        dst.free()
     be.sync()
     setup_s = time.time() - t_setup
 
@@ -153,6 +163,8 @@ def main():
             "moe_gate_up": n_sel * 2 * gate_b + batch * shape.ne * 4 + pairs * shape.n_ff * 4,
             "moe_down_combine": n_sel * down_b + pairs * shape.n_ff * 4 + batch * shape.ne * 4,
         }
+        # the decode kernel that routes its own token row also reads that row's logits
+        alg["moe_route_gate_up"] = alg["moe_gate_up"] + batch * shape.n_expert * 4
         for name, p in prof.items():
             avg_us = p["total_ms"] * 1e3 / max(p["launches"], 1)
             kernels[name] = {"launches": int(p["launches"]), "avg_us": round(avg_us, 3), "min_us": round(p["min_ms"] * 1e3, 3)}
@@ -161,9 +173,18 @@ def main():
                 kernels[name]["GBps"] = round(alg[name] / (avg_us * 1e-6) / 1e9, 1)
         dom = max((k for k in kernels if k in alg), key=lambda k: kernels[k]["avg_us"] * kernels[k]["launches"], default=None)
         if dom:
+            # HBM bytes per launch measured with hardware counters in a separate profiler run of this
+            # same command (profiles/), reported only for the workload they were taken on
+            traffic = None
+            try:
+                with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
+                    if n_layer == shape.n_layer:
+                        traffic = json.load(f).get(f"{args.config}/batch{batch}", {}).get(dom)
+            except OSError:
+                pass
             ach = alg[dom] / (kernels[dom]["avg_us"] * 1e-6) / 1e9
             roofline = {"bound": "hbm", "kernel": dom, "achieved": round(ach, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                        "frac": round(ach / HBM_PEAK_GBPS, 4), "traffic": None,
+                        "frac": round(ach / HBM_PEAK_GBPS, 4), "traffic": traffic,
                         "alg_bytes_per_launch": alg[dom], "avg_launch_us": kernels[dom]["avg_us"]}
 
     # ---- CPU baseline: the oracle on this host's cores, layer 0's weights, a bounded sample

@@ -119,11 +119,12 @@ bool ok_backend(const infr_hip_backend* be) { return be && be->magic == kBackend
 bool ok_buffer(const infr_hip_buffer* b) { return b && b->magic == kBufferMagic; }
 bool ok_plan(const infr_hip_plan* p) { return p && p->magic == kPlanMagic; }
 
-// Brackets one kernel launch with events when profiling is on.
+// Times one kernel launch when profiling is on: the events ride on the kernel's own dispatch
+// (begin / end of execution), see INFR_LAUNCH.
 struct Timed {
     infr_hip_backend* be;
     const char* name;
-    hipEvent_t a = nullptr, b = nullptr;
+    infr::LaunchTiming lt{nullptr, nullptr};
     Timed(infr_hip_backend* be_, const char* n) : be(be_), name(n) {
         if (!be->prof_on.load(std::memory_order_relaxed)) return;
         auto get = [&]() {
@@ -132,14 +133,14 @@ struct Timed {
             else if (hipEventCreate(&e) != hipSuccess) e = nullptr;
             return e;
         };
-        a = get();
-        b = get();
-        if (a) (void)hipEventRecord(a, be->stream);
+        lt.start = get();
+        lt.stop = get();
+        if (lt.start && lt.stop) infr::tl_launch_timing = &lt;
     }
     ~Timed() {
-        if (!a || !b) return;
-        (void)hipEventRecord(b, be->stream);
-        be->pending.push_back({name, a, b});
+        if (infr::tl_launch_timing != &lt) return;
+        infr::tl_launch_timing = nullptr;
+        be->pending.push_back({name, lt.start, lt.stop});
     }
 };
 

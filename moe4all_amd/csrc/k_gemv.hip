@@ -652,11 +652,11 @@ static bool try_gate_up(hipStream_t s, const MoeGemvParams& p) {
     while (u * rw > 64) u--;
     const size_t lds = 4 * cells_bytes(p.ne) +
                        (p.route_inline ? route_scratch_floats(p.route.n_expert, p.route.n_groups) * sizeof(float) : 0);
-    if (u >= 6) hipLaunchKernelGGL((moe_gate_up_fast<F, 6>), grid, block, lds, s, p, ft);
-    else if (u == 5 || u == 4) hipLaunchKernelGGL((moe_gate_up_fast<F, 4>), grid, block, lds, s, p, ft);
-    else if (u == 3) hipLaunchKernelGGL((moe_gate_up_fast<F, 3>), grid, block, lds, s, p, ft);
-    else if (u == 2) hipLaunchKernelGGL((moe_gate_up_fast<F, 2>), grid, block, lds, s, p, ft);
-    else hipLaunchKernelGGL((moe_gate_up_fast<F, 1>), grid, block, lds, s, p, ft);
+    if (u >= 6) INFR_LAUNCH((moe_gate_up_fast<F, 6>), grid, block, lds, s, p, ft);
+    else if (u == 5 || u == 4) INFR_LAUNCH((moe_gate_up_fast<F, 4>), grid, block, lds, s, p, ft);
+    else if (u == 3) INFR_LAUNCH((moe_gate_up_fast<F, 3>), grid, block, lds, s, p, ft);
+    else if (u == 2) INFR_LAUNCH((moe_gate_up_fast<F, 2>), grid, block, lds, s, p, ft);
+    else INFR_LAUNCH((moe_gate_up_fast<F, 1>), grid, block, lds, s, p, ft);
     return true;
 }
 
@@ -677,7 +677,7 @@ void launch_moe_gate_up(hipStream_t s, const MoeGemvParams& p) {
         if (done) return;
     }
     dim3 grid((p.nff + 3) / 4, p.rows * p.n_used), block(256);
-    hipLaunchKernelGGL(moe_gate_up_generic, grid, block, 0, s, p, row_bytes_of(p.gate_dt, p.ne),
+    INFR_LAUNCH(moe_gate_up_generic, grid, block, 0, s, p, row_bytes_of(p.gate_dt, p.ne),
                        row_bytes_of(p.up_dt, p.ne));
 }
 
@@ -696,10 +696,10 @@ static bool try_down(hipStream_t s, const MoeGemvParams& p) {
     dim3 grid(ceil_div(p.ne, ot), p.rows), block(64 * nwaves);
     const size_t lds = nwaves * cells_bytes(p.nff);
     switch (steps) {
-        case 1: hipLaunchKernelGGL((moe_down_combine_fast<F, 1>), grid, block, lds, s, p, ot); break;
-        case 2: hipLaunchKernelGGL((moe_down_combine_fast<F, 2>), grid, block, lds, s, p, ot); break;
-        case 4: hipLaunchKernelGGL((moe_down_combine_fast<F, 4>), grid, block, lds, s, p, ot); break;
-        default: hipLaunchKernelGGL((moe_down_combine_fast<F, 8>), grid, block, lds, s, p, ot); break;
+        case 1: INFR_LAUNCH((moe_down_combine_fast<F, 1>), grid, block, lds, s, p, ot); break;
+        case 2: INFR_LAUNCH((moe_down_combine_fast<F, 2>), grid, block, lds, s, p, ot); break;
+        case 4: INFR_LAUNCH((moe_down_combine_fast<F, 4>), grid, block, lds, s, p, ot); break;
+        default: INFR_LAUNCH((moe_down_combine_fast<F, 8>), grid, block, lds, s, p, ot); break;
     }
     return true;
 }
@@ -711,7 +711,7 @@ void launch_moe_down_combine(hipStream_t s, const MoeGemvParams& p) {
     else if (p.down_dt == INFR_Q8_0) done = try_down<Q80Fmt>(s, p);
     if (done) return;
     dim3 grid((p.ne + 3) / 4, p.rows), block(256);
-    hipLaunchKernelGGL(moe_down_combine_generic, grid, block, 0, s, p, row_bytes_of(p.down_dt, p.nff));
+    INFR_LAUNCH(moe_down_combine_generic, grid, block, 0, s, p, row_bytes_of(p.down_dt, p.nff));
 }
 
 // ------------------------------------------------------------------------------- Op::Linear
@@ -780,7 +780,7 @@ static bool try_linear(hipStream_t s, const float* x, const uint8_t* w, int m, i
     int ot = ceil_div(out_f, n_cu);
     ot = ceil_div(ot, 4 * rw) * 4 * rw;  // whole rounds of the block's 4 waves
     dim3 grid(ceil_div(out_f, ot), m), block(256);
-    hipLaunchKernelGGL((linear_fast<F>), grid, block, 4 * cells_bytes(in_f), s, x, w, in_f, out_f, dst, ot);
+    INFR_LAUNCH((linear_fast<F>), grid, block, 4 * cells_bytes(in_f), s, x, w, in_f, out_f, dst, ot);
     return true;
 }
 
@@ -792,7 +792,7 @@ void launch_linear(hipStream_t s, const float* x, const uint8_t* w, int dt, size
     else if (dt == INFR_Q8_0) done = try_linear<Q80Fmt>(s, x, w, m, in_f, out_f, dst, n_cu);
     if (done) return;
     dim3 grid((out_f + 3) / 4, m), block(256);
-    hipLaunchKernelGGL(linear_generic, grid, block, 0, s, x, w, dt, row_bytes, in_f, out_f, dst);
+    INFR_LAUNCH(linear_generic, grid, block, 0, s, x, w, dt, row_bytes, in_f, out_f, dst);
 }
 
 }  // namespace infr

@@ -5,6 +5,8 @@
 
 namespace infr {
 
+thread_local const LaunchTiming* tl_launch_timing = nullptr;
+
 __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict__ src, int dtype, uint64_t numel,
                                                       float* __restrict__ out) {
     uint64_t i = (uint64_t)blockIdx.x * 256 + threadIdx.x;
@@ -23,7 +25,7 @@ void launch_dequant(hipStream_t s, const uint8_t* src, int dtype, uint64_t numel
     if (numel == 0) return;
     uint64_t blocks = (numel + 255) / 256;
     if (blocks > 65535ull * 16) blocks = 65535ull * 16;
-    hipLaunchKernelGGL(dequant_kernel, dim3((uint32_t)blocks), dim3(256), 0, s, src, dtype, numel, out);
+    INFR_LAUNCH(dequant_kernel, dim3((uint32_t)blocks), dim3(256), 0, s, src, dtype, numel, out);
 }
 
 // Op::GatedAct (crates/infr-cpu/src/lib.rs:2973-3027), strides and block-interleaved gate included.
@@ -54,7 +56,7 @@ void launch_gated_act(hipStream_t s, const float* gate, const float* up, float* 
     if (total == 0) return;
     int64_t blocks = (total + 255) / 256;
     if (blocks > 4096) blocks = 4096;
-    hipLaunchKernelGGL(gated_act_kernel, dim3((uint32_t)blocks), dim3(256), 0, s, gate, up, dst, rows, nff, act,
+    INFR_LAUNCH(gated_act_kernel, dim3((uint32_t)blocks), dim3(256), 0, s, gate, up, dst, rows, nff, act,
                        up_off, up_stride, gate_stride, gate_block_width, has_clamp, clamp);
 }
 
@@ -67,7 +69,7 @@ void launch_add(hipStream_t s, const float* a, const float* b, float* dst, uint3
     if (n == 0) return;
     uint32_t blocks = (n + 255) / 256;
     if (blocks > 4096) blocks = 4096;
-    hipLaunchKernelGGL(add_kernel, dim3(blocks), dim3(256), 0, s, a, b, dst, n);
+    INFR_LAUNCH(add_kernel, dim3(blocks), dim3(256), 0, s, a, b, dst, n);
 }
 
 // Op::MoeSharedExpertAdd (crates/infr-cpu/src/lib.rs:3336-3356):
@@ -90,7 +92,7 @@ void launch_moe_shared_expert_add(hipStream_t s, const float* moe, const float* 
     if (rows == 0 || n == 0) return;
     int bx = (n + 255) / 256;
     if (bx > 64) bx = 64;
-    hipLaunchKernelGGL(moe_shared_expert_add_kernel, dim3(bx, rows), dim3(256), 0, s, moe, shexp, gate, dst, rows, n);
+    INFR_LAUNCH(moe_shared_expert_add_kernel, dim3(bx, rows), dim3(256), 0, s, moe, shexp, gate, dst, rows, n);
 }
 
 __global__ __launch_bounds__(256) void fill_zero_kernel(uint32_t* p, size_t words) {
@@ -102,7 +104,7 @@ void launch_fill_zero(hipStream_t s, void* p, size_t bytes) {
     if (words == 0) return;
     size_t blocks = (words + 255) / 256;
     if (blocks > 8192) blocks = 8192;
-    hipLaunchKernelGGL(fill_zero_kernel, dim3((uint32_t)blocks), dim3(256), 0, s, (uint32_t*)p, words);
+    INFR_LAUNCH(fill_zero_kernel, dim3((uint32_t)blocks), dim3(256), 0, s, (uint32_t*)p, words);
 }
 
 }  // namespace infr

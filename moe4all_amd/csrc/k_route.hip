@@ -29,7 +29,7 @@ static size_t route_lds_bytes(const RouteParams& p) {
 }
 
 void launch_route(hipStream_t s, const RouteParams& p) {
-    hipLaunchKernelGGL(route_kernel, dim3(p.rows), dim3(64), route_lds_bytes(p), s, p);
+    INFR_LAUNCH(route_kernel, dim3(p.rows), dim3(64), route_lds_bytes(p), s, p);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -55,8 +55,52 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const uint8_t* __res
     const int tid = threadIdx.x;
     const int e0 = blockIdx.x * EPB;
 
-    if (rdt == INFR_F32 && (ne & 3) == 0) {
-        const int nv = ne >> 2;
+    // Decode-sized launch (one pass over <= 2 token rows, f32 router): every global load of the
+    // block, activations included, is issued before the first LDS store, so the block pays the
+    // memory latency once.
+    const int nv = ne >> 2;
+    const bool one_shot = rdt == INFR_F32 && (ne & 3) == 0 && gridDim.y == 1 && rows <= rpb && EPB * nv <= 8 * 256 &&
+                          rpb * nv <= 4 * 256;
+    if (one_shot) {
+        float4 wr[8], xr[4];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int idx = tid + 256 * i, rr = idx / nv, v = idx - rr * nv;
+            xr[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (rr < rows) xr[i] = reinterpret_cast<const float4*>(x + (size_t)rr * ne)[v];
+        }
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int idx = tid + 256 * i, e = idx / nv, v = idx - e * nv;
+            wr[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (e < EPB && e0 + e < n_expert)
+                wr[i] = reinterpret_cast<const float4*>(router + (size_t)(e0 + e) * row_bytes)[v];
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int idx = tid + 256 * i, rr = idx / nv, v = idx - rr * nv;
+            if (rr >= rpb) continue;
+            const float fv[4] = {xr[i].x, xr[i].y, xr[i].z, xr[i].w};
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                int k = 4 * v + q, c = k >> 3, j = k & 7;
+                if (c < nc) xs[rr * estride + j * jstride + c] = fv[q];
+                else xt[rr * 8 + j] = fv[q];
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const int idx = tid + 256 * i, e = idx / nv, v = idx - e * nv;
+            if (e >= EPB) continue;
+            const float fv[4] = {wr[i].x, wr[i].y, wr[i].z, wr[i].w};
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                int k = 4 * v + q, c = k >> 3, j = k & 7;
+                if (c < nc) w[e * estride + j * jstride + c] = fv[q];
+                else wt[e * 8 + j] = fv[q];
+            }
+        }
+    } else if (rdt == INFR_F32 && (ne & 3) == 0) {
         for (int idx = tid; idx < EPB * nv; idx += 256) {
             int e = idx / nv, v = idx - e * nv;
             float4 f = make_float4(0.f, 0.f, 0.f, 0.f);
@@ -84,8 +128,8 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const uint8_t* __res
     const int j = tid & 7;
     const int lane = tid & 63;
     for (int r0 = blockIdx.y * rpb; r0 < rows; r0 += gridDim.y * rpb) {
-        __syncthreads();
-        for (int rr = 0; rr < rpb; rr++) {
+        if (!one_shot) __syncthreads();
+        for (int rr = 0; rr < (one_shot ? 0 : rpb); rr++) {
             const bool row_ok = r0 + rr < rows;
             const float* xr = x + (size_t)(row_ok ? r0 + rr : 0) * ne;
             for (int k = tid; k < ne; k += 256) {
@@ -151,7 +195,7 @@ bool launch_router_logits(hipStream_t s, const uint8_t* router, int rdt, size_t 
                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)budget);                   \
             attr_set = true;                                                                                       \
         }                                                                                                          \
-        hipLaunchKernelGGL(router_logits_kernel<E>, grid, block, lds, s, router, rdt, row_bytes, x, ne, n_expert,  \
+        INFR_LAUNCH(router_logits_kernel<E>, grid, block, lds, s, router, rdt, row_bytes, x, ne, n_expert,  \
                            rows, rpb, logits);                                                        \
     } while (0)
     switch (epb) {

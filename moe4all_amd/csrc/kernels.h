@@ -6,7 +6,24 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#include <hip/hip_ext.h>
+
 namespace infr {
+
+// Per-kernel timing.  While a thread has tl_launch_timing set, every launch it makes through
+// INFR_LAUNCH attaches the two events to the kernel's own dispatch packet: `start` is stamped
+// when the kernel begins executing and `stop` when its last wave retires, so their difference
+// is the kernel's execution time without the dispatch gap around it.
+struct LaunchTiming {
+    hipEvent_t start, stop;
+};
+extern thread_local const LaunchTiming* tl_launch_timing;
+#define INFR_LAUNCH(kernel, grid, block, lds, stream, ...)                                                       \
+    do {                                                                                                         \
+        const ::infr::LaunchTiming* lt_ = ::infr::tl_launch_timing;                                              \
+        if (lt_) hipExtLaunchKernelGGL(kernel, grid, block, lds, stream, lt_->start, lt_->stop, 0, __VA_ARGS__); \
+        else hipLaunchKernelGGL(kernel, grid, block, lds, stream, __VA_ARGS__);                                  \
+    } while (0)
 
 // Router logits with the reference's dot order (8 FMA lanes, lanes summed 0..7).
 // logits[rows, n_expert]; router rows are `row_bytes` apart, decoded as `rdt`.
