@@ -229,6 +229,15 @@ infr_status infr_hip_prof_read(infr_hip_backend *be, infr_hip_prof_entry *out, u
 infr_status infr_hip_plan_moe_routing(infr_hip_backend *be, const infr_hip_plan *plan, uint32_t op_index,
                                       int32_t *ids, float *weights, float *logits, float *probs);
 
+/* Bucketing of the last execution of MoeFfn op `op_index` when it took the batched path
+ * (reference: crates/infr-cpu/src/lib.rs:3874-3908).  offsets[n_expert + 1]: first bucket
+ * position of each expert (experts ascending); pair_src[rows * n_used]: flat index
+ * row * n_used + rank of the pair at each bucket position (rows ascending inside a bucket);
+ * slot_pair[rows * n_used]: bucket position of pair (row, rank), -1 for an expert id outside
+ * [0, n_expert).  INFR_ERR_INVALID when the op ran the per-token path.  Any pointer may be NULL. */
+infr_status infr_hip_plan_moe_bucketing(infr_hip_backend *be, const infr_hip_plan *plan, uint32_t op_index,
+                                        int32_t *offsets, int32_t *pair_src, int32_t *slot_pair);
+
 /* Standalone weight decode (reference: infr_gguf::dequant::dequant_block,
  * crates/infr-gguf/src/dequant.rs:11-55): dst f32 buffer receives the decoded prefix of
  * `numel` elements of `src` interpreted as `dtype`. */

@@ -183,6 +183,7 @@ _SIGNATURES = {
     "infr_hip_prof_enable": ([_V, C.c_int], C.c_int),
     "infr_hip_prof_read": ([_V, C.POINTER(_ProfEntry), C.c_uint32, C.POINTER(C.c_uint32)], C.c_int),
     "infr_hip_plan_moe_routing": ([_V, _V, C.c_uint32, _V, _V, _V, _V], C.c_int),
+    "infr_hip_plan_moe_bucketing": ([_V, _V, C.c_uint32, _V, _V, _V], C.c_int),
     "infr_hip_dequant": ([_V, _V, C.c_int32, C.c_uint64, _V], C.c_int),
 }
 
@@ -533,6 +534,19 @@ class Backend:
                                                    w.ctypes.data_as(_V), logits.ctypes.data_as(_V),
                                                    probs.ctypes.data_as(_V)))
         return {"idx": ids, "w": w, "logits": logits, "probs": probs}
+
+    def moe_bucketing(self, plan: Plan, op_index: int = 0) -> dict:
+        """Bucketing of the last execution of a MoeFfn op that took the batched path
+        (crates/infr-cpu/src/lib.rs:3874-3908): `offsets` [n_expert+1], `pair_row` / `pair_rank`
+        [rows*n_used] in bucket order, `slot_pair` [rows, n_used] bucket position of each pair."""
+        m = plan.graph.ops[op_index].u.moe_ffn
+        rows = plan.graph.desc(m.x).numel() // m.ne
+        offsets = np.zeros(m.n_expert + 1, np.int32)
+        src = np.zeros(rows * m.n_used, np.int32)
+        slot = np.zeros((rows, m.n_used), np.int32)
+        _check(self._lib.infr_hip_plan_moe_bucketing(self._h, plan._h, op_index, offsets.ctypes.data_as(_V),
+                                                     src.ctypes.data_as(_V), slot.ctypes.data_as(_V)))
+        return {"offsets": offsets, "pair_row": src // m.n_used, "pair_rank": src % m.n_used, "slot_pair": slot}
 
     def dequant(self, src: Buffer, dtype: DType, numel: int) -> np.ndarray:
         dst = self.alloc(numel * 4, BufferUsage.Readback)

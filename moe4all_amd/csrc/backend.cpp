@@ -42,6 +42,9 @@ infr_status fail(infr_status st, const char* fmt, ...) {
 constexpr uint64_t kBackendMagic = 0x494e465242454e44ull;  // "INFRBEND"
 constexpr uint64_t kBufferMagic = 0x494e465242554646ull;   // "INFRBUFF"
 constexpr uint64_t kPlanMagic = 0x494e4652504c414eull;     // "INFRPLAN"
+// Token rows from which Op::MoeFfn buckets tokens by expert and runs grouped GEMMs on the matrix
+// cores (f16 operands, f32 accumulation) instead of one GEMV pass per token row.
+constexpr uint32_t kBatchedMinRows = 32;
 
 bool geometry(int dtype, int* elems, int* bytes) {
     switch (dtype) {
@@ -82,8 +85,18 @@ struct MoeScratch {
     float* probs = nullptr;   // [rows, n_expert]
     int32_t* ids = nullptr;   // [rows, n_used]
     float* weights = nullptr; // [rows, n_used]
-    float* h = nullptr;       // [rows, n_used, nff]
+    float* h = nullptr;       // [rows, n_used, nff] (bucket order on the batched path); shared by all ops of a plan
     int rows = 0;
+    // batched path (bucketing + grouped GEMMs); the large buffers are shared by all ops of a plan
+    bool batched = false;
+    int32_t* offsets = nullptr;   // [n_expert + 1]
+    int32_t* pair_src = nullptr;  // [rows * n_used]
+    int32_t* slot_pair = nullptr; // [rows * n_used]
+    _Float16* xh = nullptr;       // [rows, ne]
+    float* xs = nullptr;          // [rows]
+    _Float16* hh = nullptr;       // [rows * n_used, nff]
+    float* hs = nullptr;          // [rows * n_used]
+    float* y = nullptr;           // [rows * n_used, ne]
 };
 
 struct infr_hip_plan {
@@ -445,6 +458,7 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
     }
     Check c{*plan};
     std::vector<size_t> moe_off(g->n_ops, 0);
+    size_t shared_need = 0;
     for (uint32_t oi = 0; oi < g->n_ops && c.st == INFR_OK; oi++) {
         const infr_op& op = plan->ops[oi];
         switch (op.kind) {
@@ -512,12 +526,27 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
                     if (c.n(m.expert_ids) < rows * m.n_used) c.set(INFR_ERR_INVALID, "MoeFfn.expert_ids holds fewer than rows*n_used slots");
                 }
                 if (rows > 0x7fffffffull / (m.n_used * (uint64_t)m.n_ff_exp + 1)) { c.set(INFR_ERR_UNSUPPORTED, "MoeFfn: rows too large"); break; }
-                // scratch: logits, probs, ids, weights, h
+                // per-op scratch: logits, probs, ids, weights (+ bucketing tables); h and the batched
+                // path's staging buffers live in one region shared by every op of the plan
                 moe_off[oi] = arena;
                 arena += round_up((size_t)rows * m.n_expert * 4 + 4, 256) * 2;
                 arena += round_up((size_t)rows * m.n_used * 4 + 4, 256) * 2;
-                arena += round_up((size_t)rows * m.n_used * m.n_ff_exp * 4 + 4, 256);
+                const size_t pairs = (size_t)rows * m.n_used;
+                size_t shared = round_up(pairs * m.n_ff_exp * 4 + 4, 256);
+                const uint32_t min_rows = be->cfg.moe_batched_min_rows ? be->cfg.moe_batched_min_rows : kBatchedMinRows;
+                const bool batched = rows >= min_rows && m.n_used <= 64 && !m.fused_gate_up &&
+                                     c.dt(m.gate_exps) == c.dt(m.up_exps) &&
+                                     infr::grouped_supported(c.dt(m.gate_exps), (int)m.ne) &&
+                                     infr::grouped_supported(c.dt(m.down_exps), (int)m.n_ff_exp);
+                if (batched) {
+                    arena += round_up(((size_t)m.n_expert + 2) * 4, 256) + 2 * round_up(pairs * 4 + 4, 256);
+                    shared += round_up((size_t)rows * m.ne * 2, 256) + round_up((size_t)rows * 4, 256) +
+                              round_up(pairs * m.n_ff_exp * 2, 256) + round_up(pairs * 4, 256) +
+                              round_up(pairs * m.ne * 4, 256);
+                }
+                if (shared > shared_need) shared_need = shared;
                 plan->moe[oi].rows = (int)rows;
+                plan->moe[oi].batched = batched;
                 break;
             }
             case INFR_OP_LINEAR: {
@@ -593,6 +622,8 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
         if (c.st != INFR_OK) c.err = "op " + std::to_string(oi) + ": " + c.err;
     }
     if (c.st != INFR_OK) return bail(c.st, c.err);
+    const size_t shared_off = arena;
+    arena += shared_need;
 
     std::lock_guard<std::mutex> lk(be->mu);
     hipError_t e = hipSetDevice(be->device);
@@ -609,7 +640,21 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
         s.probs = (float*)p;  p += round_up(rows * m.n_expert * 4 + 4, 256);
         s.ids = (int32_t*)p;  p += round_up(rows * m.n_used * 4 + 4, 256);
         s.weights = (float*)p; p += round_up(rows * m.n_used * 4 + 4, 256);
-        s.h = (float*)p;
+        const size_t pairs = rows * m.n_used;
+        if (s.batched) {
+            s.offsets = (int32_t*)p;   p += round_up(((size_t)m.n_expert + 2) * 4, 256);
+            s.pair_src = (int32_t*)p;  p += round_up(pairs * 4 + 4, 256);
+            s.slot_pair = (int32_t*)p;
+        }
+        p = (char*)plan->arena + shared_off;
+        s.h = (float*)p; p += round_up(pairs * m.n_ff_exp * 4 + 4, 256);
+        if (s.batched) {
+            s.xh = (_Float16*)p; p += round_up(rows * m.ne * 2, 256);
+            s.xs = (float*)p;    p += round_up(rows * 4, 256);
+            s.hh = (_Float16*)p; p += round_up(pairs * m.n_ff_exp * 2, 256);
+            s.hs = (float*)p;    p += round_up(pairs * 4, 256);
+            s.y = (float*)p;
+        }
     }
     if (plan->arena) infr::launch_fill_zero(be->stream, plan->arena, arena);
     *out = plan;
@@ -727,6 +772,48 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                 gp.weight_before = (int)m.weight_before; gp.fused_gate_up = (int)m.fused_gate_up;
                 gp.h = sc.h; gp.dst = (float*)ptr[m.dst]; gp.n_cu = n_cu;
                 gp.x = (const float*)ptr[m.x];
+                if (sc.batched) {
+                    const int pairs = rows * (int)m.n_used;
+                    {
+                        Timed t(be, "route_topk");
+                        infr::launch_route(s, rp);
+                    }
+                    {
+                        Timed t(be, "moe_bucket");
+                        infr::launch_bucket(s, sc.ids, pairs, (int)m.n_expert, sc.offsets, sc.pair_src, sc.slot_pair);
+                    }
+                    {
+                        Timed t(be, "rows_to_f16");
+                        infr::launch_rows_to_f16(s, gp.gate_dt, gp.x, rows, (int)m.ne, sc.xh, sc.xs);
+                    }
+                    infr::GroupedParams q{};
+                    q.a = sc.xh; q.a_scale = sc.xs; q.offsets = sc.offsets; q.pair_src = sc.pair_src;
+                    q.w0 = gp.gate; q.w0_stride = gp.gate_stride; q.w1 = gp.up; q.w1_stride = gp.up_stride;
+                    q.route_w = sc.weights; q.down_scale = nullptr; q.out = sc.h;
+                    q.K = (int)m.ne; q.N = (int)m.n_ff_exp; q.n_expert = (int)m.n_expert; q.n_used = (int)m.n_used;
+                    q.n_pairs = pairs; q.act = m.act; q.has_clamp = (int)m.has_swiglu_clamp; q.clamp = m.swiglu_clamp;
+                    q.weight_before = (int)m.weight_before;
+                    {
+                        Timed t(be, "moe_grouped_gate_up");
+                        infr::launch_grouped_gate_up(s, gp.gate_dt, q);
+                    }
+                    {
+                        Timed t(be, "rows_to_f16");
+                        infr::launch_rows_to_f16(s, gp.down_dt, sc.h, pairs, (int)m.n_ff_exp, sc.hh, sc.hs);
+                    }
+                    q.a = sc.hh; q.a_scale = sc.hs; q.w0 = gp.down; q.w0_stride = gp.down_stride; q.w1 = nullptr; q.w1_stride = 0;
+                    q.down_scale = gp.down_scale; q.out = sc.y; q.K = (int)m.n_ff_exp; q.N = (int)m.ne;
+                    {
+                        Timed t(be, "moe_grouped_down");
+                        infr::launch_grouped_down(s, gp.down_dt, q);
+                    }
+                    {
+                        Timed t(be, "moe_unbucket_combine");
+                        infr::launch_unbucket_combine(s, sc.y, sc.slot_pair, sc.weights, rows, (int)m.ne, (int)m.n_used,
+                                                      (int)m.weight_before, gp.dst);
+                    }
+                    break;
+                }
                 gp.route = rp;
                 gp.route_inline = infr::moe_gate_up_routes_inline(gp) ? 1 : 0;
                 if (!gp.route_inline) {
@@ -838,6 +925,25 @@ extern "C" infr_status infr_hip_plan_moe_routing(infr_hip_backend* be, const inf
     if (weights) HIP_TRY(hipMemcpy(weights, sc.weights, rows * m.n_used * 4, hipMemcpyDeviceToHost));
     if (logits) HIP_TRY(hipMemcpy(logits, sc.logits, rows * m.n_expert * 4, hipMemcpyDeviceToHost));
     if (probs) HIP_TRY(hipMemcpy(probs, sc.probs, rows * m.n_expert * 4, hipMemcpyDeviceToHost));
+    return INFR_OK;
+}
+
+extern "C" infr_status infr_hip_plan_moe_bucketing(infr_hip_backend* be, const infr_hip_plan* plan, uint32_t op_index,
+                                                   int32_t* offsets, int32_t* pair_src, int32_t* slot_pair) {
+    if (!ok_backend(be) || !ok_plan(plan) || plan->be != be) return fail(INFR_ERR_INVALID, "moe_bucketing: bad handle");
+    if (op_index >= plan->ops.size() || plan->ops[op_index].kind != INFR_OP_MOE_FFN)
+        return fail(INFR_ERR_INVALID, "moe_bucketing: op %u is not a MoeFfn", op_index);
+    const infr_op_moe_ffn& m = plan->ops[op_index].u.moe_ffn;
+    const MoeScratch& sc = plan->moe[op_index];
+    if (!sc.batched)
+        return fail(INFR_ERR_INVALID, "moe_bucketing: op %u runs the per-token path (%d rows), which does not bucket", op_index, sc.rows);
+    std::lock_guard<std::mutex> lk(be->mu);
+    HIP_TRY(hipSetDevice(be->device));
+    HIP_TRY(hipStreamSynchronize(be->stream));
+    const size_t pairs = (size_t)sc.rows * m.n_used;
+    if (offsets) HIP_TRY(hipMemcpy(offsets, sc.offsets, ((size_t)m.n_expert + 1) * 4, hipMemcpyDeviceToHost));
+    if (pair_src) HIP_TRY(hipMemcpy(pair_src, sc.pair_src, pairs * 4, hipMemcpyDeviceToHost));
+    if (slot_pair) HIP_TRY(hipMemcpy(slot_pair, sc.slot_pair, pairs * 4, hipMemcpyDeviceToHost));
     return INFR_OK;
 }
 

@@ -1,0 +1,510 @@
+// Batched Op::MoeFfn: token -> expert bucketing and per-expert grouped GEMMs on the matrix cores.
+//
+// The CPU reference groups the (token row, rank) pairs of a batch by expert, experts ascending
+// and rows ascending inside a bucket (crates/infr-cpu/src/lib.rs:3874-3908), and runs one GEMM
+// per bucket (crates/infr-cpu/src/moe.rs:142-173).  Here:
+//
+//   bucket_kernel         offsets[e] = number of pairs whose expert id is below e, and the stable
+//                         scatter of the pairs into that order (one wavefront per expert; order is
+//                         an integer contract and is reproduced exactly).
+//   rows_to_f16_kernel    activation rows -> f16 with one power-of-two scale per row (so any f32
+//                         magnitude fits), laid out in the k order the weight format unpacks to.
+//   grouped_mfma<F,DOWN>  per (expert, 128-token tile, 128/256-feature tile): quantised weight rows
+//                         are unpacked to f16 straight into LDS with packed 16-bit arithmetic, the
+//                         contraction runs on v_mfma_f32_32x32x16_f16 with f32 accumulation;
+//                         epilogue = SwiGLU (gate/up) or plain scaled store (down).
+//   unbucket_combine      dst[row] = sum over ranks (rank order, separate mul and add,
+//                         lib.rs:4290-4302) of w * y[pair of (row, rank)].
+//
+// Unpacking trick: a code c in 0..1023 or'ed into 0x6400 is the f16 number 1024 + c, so a pair of
+// codes sitting in the two halves of a dword becomes a pair of f16 values with one AND/OR, an
+// exact packed subtract and one packed multiply(-add) with the group's scale.  The order in
+// which codes fall out of a dword is not the element order; since a dot product does not care
+// about the order of its terms, the activation rows are stored in that same ("virtual") order.
+#include "device_common.h"
+#include "kernels.h"
+
+namespace infr {
+
+typedef _Float16 half8 __attribute__((ext_vector_type(8)));
+typedef _Float16 half2v __attribute__((ext_vector_type(2)));
+typedef float float16v __attribute__((ext_vector_type(16)));
+
+namespace {
+
+constexpr int kBM = 128;        // token rows per tile
+constexpr int kSlice = 64;      // k elements per LDS stage
+constexpr int kAStride = 129;   // 16-byte chunks per k-group of the activation tile (+1: bank spread)
+
+__device__ __forceinline__ half2v as_h2(uint32_t v) { return __builtin_bit_cast(half2v, v); }
+__device__ __forceinline__ uint32_t as_u32(half2v v) { return __builtin_bit_cast(uint32_t, v); }
+__device__ __forceinline__ half2v splat(float v) {
+    _Float16 h = (_Float16)v;
+    return half2v{h, h};
+}
+// (1024 + code pair) -> code pair - bias, exact
+__device__ __forceinline__ half2v unbias(uint32_t magic_pair, float bias) { return as_h2(magic_pair) - splat(bias); }
+
+// --------------------------------------------------------------------------------------------
+// Weight formats.  load() fetches the 64 k-elements of virtual slice s of one weight row,
+// expand() turns them into 8 operand chunks of 8 f16 (chunk g = virtual k 8g..8g+7 of the slice).
+// chunk_src() gives, for virtual chunk c of a row, the two real offsets whose float4s feed it
+// and whether the 4 elements of each come out in the order 0,2,1,3.
+struct MQ4K {
+    static constexpr int kDt = INFR_Q4K, kBlockElems = 256, kBlockBytes = 144;
+    struct Raw {
+        uint4 hdr, qa, qb;
+    };
+    static __device__ __forceinline__ Raw load(const uint8_t* row, int s) {
+        const uint8_t* blk = row + (size_t)(s >> 2) * 144;
+        const uint4* q = reinterpret_cast<const uint4*>(blk + 16 + (s & 3) * 32);
+        return Raw{*reinterpret_cast<const uint4*>(blk), q[0], q[1]};
+    }
+    static __device__ __forceinline__ uint32_t scale_byte(const uint4& hdr, int i) {  // scales[i], i in 0..11
+        const uint32_t w = i < 4 ? hdr.y : (i < 8 ? hdr.z : hdr.w);
+        return (w >> (8 * (i & 3))) & 0xFFu;
+    }
+    static __device__ __forceinline__ void scale_min(const uint4& hdr, int j, uint32_t& sc, uint32_t& m) {
+        // get_scale_min_k4 (crates/infr-gguf/src/dequant.rs:77-87)
+        if (j < 4) {
+            sc = scale_byte(hdr, j) & 63u;
+            m = scale_byte(hdr, j + 4) & 63u;
+        } else {
+            sc = (scale_byte(hdr, j + 4) & 0x0Fu) | ((scale_byte(hdr, j - 4) >> 6) << 4);
+            m = (scale_byte(hdr, j + 4) >> 4) | ((scale_byte(hdr, j) >> 6) << 4);
+        }
+    }
+    static __device__ __forceinline__ void expand(const Raw& r, int s, uint4 out[8]) {
+        const int j = s & 3;
+        const float d = f16_bits_to_f32(r.hdr.x & 0xFFFFu), dmin = f16_bits_to_f32(r.hdr.x >> 16);
+        uint32_t sc0, m0, sc1, m1;
+        scale_min(r.hdr, 2 * j, sc0, m0);
+        scale_min(r.hdr, 2 * j + 1, sc1, m1);
+        const half2v s_lo = splat(d * (float)sc0), n_lo = splat(-(dmin * (float)m0));
+        const half2v s_hi = splat(d * (float)sc1), n_hi = splat(-(dmin * (float)m1));
+        const uint32_t q[8] = {r.qa.x, r.qa.y, r.qa.z, r.qa.w, r.qb.x, r.qb.y, r.qb.z, r.qb.w};
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const uint32_t v = q[i];
+            const half2v a = unbias((v & 0x000F000Fu) | 0x64006400u, 1024.f);
+            const half2v b = unbias(((v >> 8) & 0x000F000Fu) | 0x64006400u, 1024.f);
+            const half2v c = unbias(((v >> 4) & 0x000F000Fu) | 0x64006400u, 1024.f);
+            const half2v e = unbias(((v >> 12) & 0x000F000Fu) | 0x64006400u, 1024.f);
+            out[i] = uint4{as_u32(__builtin_elementwise_fma(a, s_lo, n_lo)), as_u32(__builtin_elementwise_fma(b, s_lo, n_lo)),
+                           as_u32(__builtin_elementwise_fma(c, s_hi, n_hi)), as_u32(__builtin_elementwise_fma(e, s_hi, n_hi))};
+        }
+    }
+    static __device__ __forceinline__ void chunk_src(int c, int& lo, int& hi, bool& swz) {
+        const int i = c & 7;
+        lo = (c >> 3) * 64 + 4 * i;
+        hi = lo + 32;
+        swz = true;
+    }
+};
+
+struct MQ6K {
+    static constexpr int kDt = INFR_Q6K, kBlockElems = 256, kBlockBytes = 210;
+    struct Raw {
+        uint4 la, lb, ha, hb;
+        uint32_t sc_lo, sc_hi, d;  // two int8 scales each, f16 d
+    };
+    // virtual slice t of a block: t = 2*half + ab; ab picks ql bytes [32ab, 32ab+32) of the half
+    static __device__ __forceinline__ Raw load(const uint8_t* row, int s) {
+        const uint8_t* blk = row + (size_t)(s >> 2) * 210;
+        const int hh = (s >> 1) & 1, ab = s & 1;
+        Raw r;
+        r.la = ldu<uint4>(blk + 64 * hh + 32 * ab);
+        r.lb = ldu<uint4>(blk + 64 * hh + 32 * ab + 16);
+        r.ha = ldu<uint4>(blk + 128 + 32 * hh);
+        r.hb = ldu<uint4>(blk + 128 + 32 * hh + 16);
+        r.sc_lo = ldu<uint16_t>(blk + 192 + 8 * hh + 2 * ab);
+        r.sc_hi = ldu<uint16_t>(blk + 192 + 8 * hh + 2 * ab + 4);
+        r.d = ldu<uint16_t>(blk + 208);
+        return r;
+    }
+    static __device__ __forceinline__ void expand(const Raw& r, int s, uint4 out[8]) {
+        const int sh = 2 * (s & 1);  // qh bit pair of this slice: bits sh..sh+1 (low codes), sh+4.. (high codes)
+        const float d = f16_bits_to_f32(r.d);
+        const half2v sl[2] = {splat(d * (float)(int8_t)(r.sc_lo & 0xFF)), splat(d * (float)(int8_t)(r.sc_lo >> 8))};
+        const half2v sh2[2] = {splat(d * (float)(int8_t)(r.sc_hi & 0xFF)), splat(d * (float)(int8_t)(r.sc_hi >> 8))};
+        const uint32_t ql[8] = {r.la.x, r.la.y, r.la.z, r.la.w, r.lb.x, r.lb.y, r.lb.z, r.lb.w};
+        const uint32_t qh[8] = {r.ha.x, r.ha.y, r.ha.z, r.ha.w, r.hb.x, r.hb.y, r.hb.z, r.hb.w};
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const uint32_t L = ql[i], H = qh[i] >> sh;
+            const uint32_t a = (L & 0x000F000Fu) | ((H & 0x00030003u) << 4) | 0x64006400u;
+            const uint32_t b = ((L >> 8) & 0x000F000Fu) | (((H >> 8) & 0x00030003u) << 4) | 0x64006400u;
+            const uint32_t c = ((L >> 4) & 0x000F000Fu) | (H & 0x00300030u) | 0x64006400u;
+            const uint32_t e = ((L >> 12) & 0x000F000Fu) | ((H >> 8) & 0x00300030u) | 0x64006400u;
+            const half2v s0 = sl[i >> 2], s1 = sh2[i >> 2];
+            out[i] = uint4{as_u32(unbias(a, 1056.f) * s0), as_u32(unbias(b, 1056.f) * s0), as_u32(unbias(c, 1056.f) * s1),
+                           as_u32(unbias(e, 1056.f) * s1)};
+        }
+    }
+    static __device__ __forceinline__ void chunk_src(int c, int& lo, int& hi, bool& swz) {
+        const int blk = c >> 5, t = (c >> 3) & 3, i = c & 7;
+        lo = blk * 256 + 128 * (t >> 1) + 32 * (t & 1) + 4 * i;
+        hi = lo + 64;
+        swz = true;
+    }
+};
+
+struct MQ80 {
+    static constexpr int kDt = INFR_Q8_0, kBlockElems = 32, kBlockBytes = 34;
+    struct Raw {
+        uint32_t q[16];
+        uint32_t d0, d1;
+    };
+    static __device__ __forceinline__ Raw load(const uint8_t* row, int s) {
+        const uint8_t* p = row + (size_t)s * 68;
+        Raw r;
+        r.d0 = ldu<uint16_t>(p);
+        r.d1 = ldu<uint16_t>(p + 34);
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            r.q[i] = ldu<uint32_t>(p + 2 + 4 * i);
+            r.q[8 + i] = ldu<uint32_t>(p + 36 + 4 * i);
+        }
+        return r;
+    }
+    static __device__ __forceinline__ void expand(const Raw& r, int, uint4 out[8]) {
+        const half2v d[2] = {splat(f16_bits_to_f32(r.d0)), splat(f16_bits_to_f32(r.d1))};
+#pragma unroll
+        for (int g = 0; g < 8; g++) {
+            uint32_t o[4];
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const uint32_t v = r.q[2 * g + h];
+                // bytes (b0,b1) and (b2,b3) to the low bytes of the two halves; x ^ 0x80 = x + 128 as unsigned
+                const uint32_t p01 = __builtin_amdgcn_perm(0u, v, 0x0C010C00u) ^ 0x64806480u;
+                const uint32_t p23 = __builtin_amdgcn_perm(0u, v, 0x0C030C02u) ^ 0x64806480u;
+                o[2 * h] = as_u32(unbias(p01, 1152.f) * d[g >> 2]);
+                o[2 * h + 1] = as_u32(unbias(p23, 1152.f) * d[g >> 2]);
+            }
+            out[g] = uint4{o[0], o[1], o[2], o[3]};
+        }
+    }
+    static __device__ __forceinline__ void chunk_src(int c, int& lo, int& hi, bool& swz) {
+        lo = 8 * c;
+        hi = lo + 4;
+        swz = false;
+    }
+};
+
+// --------------------------------------------------------------------------------------------
+// One block per row: amax -> power-of-two scale -> f16 in the virtual k order of format F.
+template <class F>
+__global__ __launch_bounds__(256) void rows_to_f16_kernel(const float* __restrict__ src, int n,
+                                                          _Float16* __restrict__ dst, float* __restrict__ scale) {
+    __shared__ float s_max[4];
+    const size_t row = blockIdx.x;
+    const float* x = src + row * n;
+    float m = 0.0f;
+    for (int k = threadIdx.x * 4; k < n; k += 1024) {
+        const float4 v = *reinterpret_cast<const float4*>(x + k);
+        m = fmaxf(fmaxf(m, fmaxf(fabsf(v.x), fabsf(v.y))), fmaxf(fabsf(v.z), fabsf(v.w)));
+    }
+    m = wave_max(m);
+    if ((threadIdx.x & 63) == 0) s_max[threadIdx.x >> 6] = m;
+    __syncthreads();
+    m = fmaxf(fmaxf(s_max[0], s_max[1]), fmaxf(s_max[2], s_max[3]));
+    int e = 0;
+    if (m > 0.0f && m < __builtin_inff()) (void)frexpf(m, &e);  // m = f * 2^e, f in [0.5, 1)
+    const float inv = ldexpf(1.0f, -e);
+    if (threadIdx.x == 0) scale[row] = ldexpf(1.0f, e);
+    uint4* out = reinterpret_cast<uint4*>(dst + row * n);
+    for (int c = threadIdx.x; c < n / 8; c += 256) {
+        int lo, hi;
+        bool swz;
+        F::chunk_src(c, lo, hi, swz);
+        const float4 a = *reinterpret_cast<const float4*>(x + lo), b = *reinterpret_cast<const float4*>(x + hi);
+        half2v h0, h1, h2, h3;
+        if (swz) {
+            h0 = half2v{(_Float16)(a.x * inv), (_Float16)(a.z * inv)};
+            h1 = half2v{(_Float16)(a.y * inv), (_Float16)(a.w * inv)};
+            h2 = half2v{(_Float16)(b.x * inv), (_Float16)(b.z * inv)};
+            h3 = half2v{(_Float16)(b.y * inv), (_Float16)(b.w * inv)};
+        } else {
+            h0 = half2v{(_Float16)(a.x * inv), (_Float16)(a.y * inv)};
+            h1 = half2v{(_Float16)(a.z * inv), (_Float16)(a.w * inv)};
+            h2 = half2v{(_Float16)(b.x * inv), (_Float16)(b.y * inv)};
+            h3 = half2v{(_Float16)(b.z * inv), (_Float16)(b.w * inv)};
+        }
+        out[c] = uint4{as_u32(h0), as_u32(h1), as_u32(h2), as_u32(h3)};
+    }
+}
+
+// --------------------------------------------------------------------------------------------
+// One wavefront per expert e in 0..n_expert (the extra one writes the total and marks pairs
+// whose id is out of range).  Every wave scans all pair ids; the scan order is the flat
+// (row, rank) order, so buckets come out rows ascending.
+__global__ __launch_bounds__(1024) void bucket_kernel(const int32_t* __restrict__ ids, int n_pairs, int n_expert,
+                                                      int32_t* __restrict__ offsets, int32_t* __restrict__ pair_src,
+                                                      int32_t* __restrict__ slot_pair) {
+    const int lane = threadIdx.x & 63;
+    const int e = blockIdx.x * 16 + (threadIdx.x >> 6);
+    if (e > n_expert) return;
+    uint32_t below = 0;
+    for (int i0 = 0; i0 < n_pairs; i0 += 64) {
+        const int i = i0 + lane;
+        const uint32_t id = i < n_pairs ? (uint32_t)ids[i] : 0xFFFFFFFFu;
+        below += (uint32_t)__popcll(__ballot(id < (uint32_t)e));
+        if (e == n_expert && i < n_pairs && id >= (uint32_t)n_expert) slot_pair[i] = -1;
+    }
+    if (lane == 0) offsets[e] = (int32_t)below;
+    if (e == n_expert) return;
+    uint32_t run = below;
+    for (int i0 = 0; i0 < n_pairs; i0 += 64) {
+        const int i = i0 + lane;
+        const bool hit = i < n_pairs && (uint32_t)ids[i] == (uint32_t)e;
+        const unsigned long long mask = __ballot(hit);
+        if (hit) {
+            const uint32_t p = run + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
+            pair_src[p] = i;
+            slot_pair[i] = (int32_t)p;
+        }
+        run += (uint32_t)__popcll(mask);
+    }
+}
+
+// --------------------------------------------------------------------------------------------
+struct Tile {
+    int e, p0, cnt;
+};
+// Tile number `tile` in the order (expert ascending, 128-row tile ascending).  Uniform per wave.
+__device__ __forceinline__ bool find_tile(const int32_t* __restrict__ offsets, int n_expert, int tile, int lane, Tile& t) {
+    const int epl = (n_expert + 63) >> 6;
+    const int e_lo = lane * epl, e_hi = min(n_expert, e_lo + epl);
+    int mine = 0;
+    for (int e = e_lo; e < e_hi; e++) mine += (offsets[e + 1] - offsets[e] + kBM - 1) / kBM;
+    int incl = mine;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const int o = __shfl_up(incl, d, 64);
+        if (lane >= d) incl += o;
+    }
+    const unsigned long long past = __ballot(incl > tile);
+    if (past == 0) return false;
+    const int owner = __ffsll((long long)past) - 1;
+    int rem = tile - (__shfl(incl, owner, 64) - __shfl(mine, owner, 64));
+    const int o_lo = owner * epl, o_hi = min(n_expert, o_lo + epl);
+    for (int e = o_lo; e < o_hi; e++) {
+        const int cnt = offsets[e + 1] - offsets[e];
+        const int nt = (cnt + kBM - 1) / kBM;
+        if (rem < nt) {
+            t.e = e;
+            t.p0 = offsets[e] + rem * kBM;
+            t.cnt = min(kBM, cnt - rem * kBM);
+            return true;
+        }
+        rem -= nt;
+    }
+    return false;
+}
+
+// --------------------------------------------------------------------------------------------
+// 256 threads = 4 waves.  Thread r stages weight row r of the 256-row B tile (gate rows then up
+// rows, or 256 down rows); wave w owns two 32-feature column tiles (gate w / up w, or down
+// 2w / 2w+1) against up to four 32-token row tiles.
+template <class F, bool DOWN>
+__global__ __launch_bounds__(256, 2) void grouped_mfma(GroupedParams p) {
+    __shared__ uint4 sA[8 * kAStride];
+    __shared__ uint4 sB[8 * 256];
+    __shared__ float s_scale[kBM];
+    __shared__ uint64_t s_tab[32];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int nt = blockIdx.x % p.n_tiles_n;
+    Tile t;
+    if (!find_tile(p.offsets, p.n_expert, blockIdx.x / p.n_tiles_n, lane, t)) return;
+    constexpr int kBN = DOWN ? 256 : 128;
+    const int n0 = nt * kBN;
+    if (tid < 32) s_tab[tid] = kExp2Table[tid];
+
+    const size_t row_bytes = (size_t)(p.K / F::kBlockElems) * F::kBlockBytes;
+    const int feat = min(n0 + (DOWN ? tid : (tid & 127)), p.N - 1);
+    const uint8_t* wrow = ((DOWN || tid < 128) ? p.w0 + (size_t)t.e * p.w0_stride : p.w1 + (size_t)t.e * p.w1_stride) +
+                          (size_t)feat * row_bytes;
+    const uint4* asrc[4];
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const int c = tid + 256 * q, tok = c >> 3, kg = c & 7;
+        const int pr = t.p0 + min(tok, t.cnt - 1);
+        const size_t src_row = DOWN ? (size_t)pr : (size_t)(p.pair_src[pr] / p.n_used);
+        asrc[q] = reinterpret_cast<const uint4*>(p.a + src_row * p.K) + kg;
+    }
+    if (tid < kBM) {
+        const int pr = t.p0 + min(tid, t.cnt - 1);
+        s_scale[tid] = p.a_scale[DOWN ? pr : p.pair_src[pr] / p.n_used];
+    }
+    const int n_msub = (t.cnt + 31) >> 5;
+    float16v acc0[4], acc1[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc0[i][r] = acc1[i][r] = 0.0f;
+
+    const int n_slices = p.K / kSlice;
+    typename F::Raw raw = F::load(wrow, 0);
+    uint4 araw[4];
+#pragma unroll
+    for (int q = 0; q < 4; q++) araw[q] = asrc[q][0];
+    const int bt0 = DOWN ? 2 * wave : wave, bt1 = DOWN ? 2 * wave + 1 : 4 + wave;
+    for (int s = 0; s < n_slices; s++) {
+        {
+            uint4 ch[8];
+            F::expand(raw, s, ch);
+#pragma unroll
+            for (int g = 0; g < 8; g++) sB[g * 256 + tid] = ch[g];
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const int c = tid + 256 * q;
+                sA[(c & 7) * kAStride + (c >> 3)] = araw[q];
+            }
+        }
+        __syncthreads();
+        if (s + 1 < n_slices) {
+            raw = F::load(wrow, s + 1);
+#pragma unroll
+            for (int q = 0; q < 4; q++) araw[q] = asrc[q][(s + 1) * (kSlice / 8)];
+        }
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) {
+            const int kg = 2 * ks + (lane >> 5);
+            const half8 b0 = __builtin_bit_cast(half8, sB[kg * 256 + bt0 * 32 + (lane & 31)]);
+            const half8 b1 = __builtin_bit_cast(half8, sB[kg * 256 + bt1 * 32 + (lane & 31)]);
+#pragma unroll
+            for (int mi = 0; mi < 4; mi++) {
+                if (mi < n_msub) {
+                    const half8 a = __builtin_bit_cast(half8, sA[kg * kAStride + mi * 32 + (lane & 31)]);
+                    acc0[mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b0, acc0[mi], 0, 0, 0);
+                    acc1[mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b1, acc1[mi], 0, 0, 0);
+                }
+            }
+        }
+        __syncthreads();
+    }
+
+    // accumulator register r of a 32x32 tile: row 8*(r/4) + 4*(lane/32) + r%4, column lane%32
+    const float ds = (DOWN && p.down_scale) ? p.down_scale[t.e] : 1.0f;
+#pragma unroll
+    for (int mi = 0; mi < 4; mi++) {
+        if (mi >= n_msub) continue;
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int m = 32 * mi + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+            if (m >= t.cnt) continue;
+            const float sc = s_scale[m];
+            float* orow = p.out + (size_t)(t.p0 + m) * p.N;
+            if (DOWN) {
+                const int f0 = n0 + 64 * wave + (lane & 31), f1 = f0 + 32;
+                float y0 = __fmul_rn(acc0[mi][r], sc), y1 = __fmul_rn(acc1[mi][r], sc);
+                if (p.down_scale) {
+                    y0 = __fmul_rn(y0, ds);
+                    y1 = __fmul_rn(y1, ds);
+                }
+                if (f0 < p.N) orow[f0] = y0;
+                if (f1 < p.N) orow[f1] = y1;
+            } else {
+                const int f = n0 + 32 * wave + (lane & 31);
+                float g = __fmul_rn(acc0[mi][r], sc), u = __fmul_rn(acc1[mi][r], sc);
+                if (p.weight_before) {
+                    const float wp = p.route_w[p.pair_src[t.p0 + m]];
+                    g = __fmul_rn(wp, g);
+                    u = __fmul_rn(wp, u);
+                }
+                if (f < p.N) orow[f] = gated_act_fn(p.act, p.has_clamp, p.clamp, g, u, s_tab);
+            }
+        }
+    }
+}
+
+// dst[row, :] = sum over ranks of w * y[slot_pair[row, rank], :], rank order, separate mul/add.
+__global__ __launch_bounds__(256) void unbucket_combine_kernel(const float* __restrict__ y,
+                                                               const int32_t* __restrict__ slot_pair,
+                                                               const float* __restrict__ weights, int ne, int n_used,
+                                                               int weight_before, float* __restrict__ dst) {
+    const size_t row = blockIdx.y;
+    const int i = (blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= ne) return;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int k = 0; k < n_used; k++) {
+        const int pr = slot_pair[row * n_used + k];
+        if (pr < 0) continue;
+        const float w = weight_before ? 1.0f : weights[row * n_used + k];
+        const float* yr = y + (size_t)pr * ne + i;
+        if (i + 3 < ne) {
+            const float4 v = *reinterpret_cast<const float4*>(yr);
+            acc.x = __fadd_rn(acc.x, __fmul_rn(w, v.x));
+            acc.y = __fadd_rn(acc.y, __fmul_rn(w, v.y));
+            acc.z = __fadd_rn(acc.z, __fmul_rn(w, v.z));
+            acc.w = __fadd_rn(acc.w, __fmul_rn(w, v.w));
+        } else {
+            float* a = &acc.x;
+            for (int q = 0; i + q < ne; q++) a[q] = __fadd_rn(a[q], __fmul_rn(w, yr[q]));
+        }
+    }
+    float* o = dst + row * ne + i;
+    if (i + 3 < ne) *reinterpret_cast<float4*>(o) = acc;
+    else {
+        const float* a = &acc.x;
+        for (int q = 0; i + q < ne; q++) o[q] = a[q];
+    }
+}
+
+template <class F>
+void rows_to_f16(hipStream_t s, const float* src, int rows, int n, _Float16* dst, float* scale) {
+    INFR_LAUNCH(rows_to_f16_kernel<F>, dim3(rows), dim3(256), 0, s, src, n, dst, scale);
+}
+
+template <class F, bool DOWN>
+void grouped(hipStream_t s, const GroupedParams& p) {
+    const int bn = DOWN ? 256 : 128;
+    GroupedParams q = p;
+    q.n_tiles_n = (p.N + bn - 1) / bn;
+    const int max_tiles = p.n_pairs / kBM + (p.n_expert < p.n_pairs ? p.n_expert : p.n_pairs);
+    INFR_LAUNCH((grouped_mfma<F, DOWN>), dim3((unsigned)max_tiles * q.n_tiles_n), dim3(256), 0, s, q);
+}
+
+}  // namespace
+
+bool grouped_supported(int dt, int k) {
+    if (k <= 0 || (k % kSlice) != 0) return false;
+    if (dt == INFR_Q4K || dt == INFR_Q6K) return (k % 256) == 0;
+    return dt == INFR_Q8_0;
+}
+
+void launch_rows_to_f16(hipStream_t s, int weight_dt, const float* src, int rows, int n, void* dst, float* scale) {
+    if (rows <= 0) return;
+    _Float16* d = reinterpret_cast<_Float16*>(dst);
+    if (weight_dt == INFR_Q4K) rows_to_f16<MQ4K>(s, src, rows, n, d, scale);
+    else if (weight_dt == INFR_Q6K) rows_to_f16<MQ6K>(s, src, rows, n, d, scale);
+    else rows_to_f16<MQ80>(s, src, rows, n, d, scale);
+}
+
+void launch_bucket(hipStream_t s, const int32_t* ids, int n_pairs, int n_expert, int32_t* offsets, int32_t* pair_src,
+                   int32_t* slot_pair) {
+    const int waves = n_expert + 1;
+    INFR_LAUNCH(bucket_kernel, dim3((waves + 15) / 16), dim3(1024), 0, s, ids, n_pairs, n_expert, offsets, pair_src,
+                slot_pair);
+}
+
+void launch_grouped_gate_up(hipStream_t s, int dt, const GroupedParams& p) {
+    if (dt == INFR_Q4K) grouped<MQ4K, false>(s, p);
+    else if (dt == INFR_Q6K) grouped<MQ6K, false>(s, p);
+    else grouped<MQ80, false>(s, p);
+}
+
+void launch_grouped_down(hipStream_t s, int dt, const GroupedParams& p) {
+    if (dt == INFR_Q4K) grouped<MQ4K, true>(s, p);
+    else if (dt == INFR_Q6K) grouped<MQ6K, true>(s, p);
+    else grouped<MQ80, true>(s, p);
+}
+
+void launch_unbucket_combine(hipStream_t s, const float* y, const int32_t* slot_pair, const float* weights, int rows,
+                             int ne, int n_used, int weight_before, float* dst) {
+    if (rows <= 0) return;
+    INFR_LAUNCH(unbucket_combine_kernel, dim3((ne + 1023) / 1024, rows), dim3(256), 0, s, y, slot_pair, weights, ne, n_used,
+                weight_before, dst);
+}
+
+}  // namespace infr

@@ -73,6 +73,33 @@ void launch_moe_gate_up(hipStream_t s, const MoeGemvParams& p);
 // dst[row] = sum over slots (rank order) of w * (down . h).
 void launch_moe_down_combine(hipStream_t s, const MoeGemvParams& p);
 
+// ---- batched path: bucketing + grouped GEMMs on the matrix cores --------------------------------
+struct GroupedParams {
+    const _Float16* a;        // gate/up: [rows, K] activations; down: [n_pairs, K]; f16, virtual k order
+    const float* a_scale;     // one power-of-two scale per row of a
+    const int32_t* offsets;   // [n_expert + 1] first pair of each expert's bucket
+    const int32_t* pair_src;  // [n_pairs] flat (row * n_used + rank) of the pair at each bucket position
+    const uint8_t* w0; size_t w0_stride;  // gate (or down) expert slices
+    const uint8_t* w1; size_t w1_stride;  // up expert slices (gate/up only)
+    const float* route_w;     // [rows, n_used] routing weights, read when weight_before
+    const float* down_scale;  // [n_expert] or null (down only)
+    float* out;               // [n_pairs, N] f32, bucket order
+    int K, N, n_expert, n_used, n_pairs;
+    int act, has_clamp; float clamp; int weight_before;
+    int n_tiles_n;            // set by the launcher
+};
+// Formats and contraction lengths the grouped kernels take.
+bool grouped_supported(int dt, int k);
+// rows of f32 -> f16 with a per-row power-of-two scale, in the k order weights of `weight_dt` unpack to.
+void launch_rows_to_f16(hipStream_t s, int weight_dt, const float* src, int rows, int n, void* dst, float* scale);
+// offsets / pair_src / slot_pair ([n_pairs], -1 for ids outside [0, n_expert)) from ids [n_pairs].
+void launch_bucket(hipStream_t s, const int32_t* ids, int n_pairs, int n_expert, int32_t* offsets, int32_t* pair_src,
+                   int32_t* slot_pair);
+void launch_grouped_gate_up(hipStream_t s, int dt, const GroupedParams& p);
+void launch_grouped_down(hipStream_t s, int dt, const GroupedParams& p);
+void launch_unbucket_combine(hipStream_t s, const float* y, const int32_t* slot_pair, const float* weights, int rows,
+                             int ne, int n_used, int weight_before, float* dst);
+
 // Standalone decode: out[i] = value of element i (exact reference arithmetic).
 void launch_dequant(hipStream_t s, const uint8_t* src, int dtype, uint64_t numel, float* out);
 

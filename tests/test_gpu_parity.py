@@ -453,3 +453,129 @@ def test_benchmark_config_layer_matches_oracle_at_full_size(be, shape, batch):
         buf.free()
     plan.free()
     lw.free()
+
+
+# ------------------------------------------------------------------ batched path (bucketing + grouped GEMM)
+REL_L2_MFMA = 1e-2   # f16 operands on the matrix cores, f32 accumulation
+
+
+def _check_bucketing(b, ref, E):
+    """Bucket order is an integer contract: experts ascending, rows ascending inside a bucket."""
+    counts = np.diff(b["offsets"])
+    want = np.zeros(E, np.int64)
+    want[ref["bucket_expert"]] = ref["bucket_count"]
+    assert np.array_equal(counts, want)
+    assert np.array_equal(b["offsets"][ref["bucket_expert"]], ref["bucket_p0"])
+    assert np.array_equal(b["pair_row"], ref["pair_row"])
+    assert np.array_equal(b["slot_pair"], ref["slot_pair"])
+
+
+def _run_batched(be, g, ids, data, rows, ne):
+    keep = []
+    bound = [(ids[k], v) for k, v in data.items() if ids.get(k) is not None and v is not None]
+    out = M.run_graph(be, g, bound, ids["dst"], rows * ne, keep=keep)
+    routing = be.moe_routing(keep[0], 0)
+    bucketing = be.moe_bucketing(keep[0], 0)
+    for buf in keep[2]:
+        buf.free()
+    keep[3].free()
+    keep[0].free()
+    return out.reshape(rows, ne), routing, bucketing
+
+
+@pytest.mark.parametrize("rows,ne,E,K,nff,gdt,ddt", [
+    (64, 512, 8, 2, 256, H.Q4K, H.Q6K),
+    (33, 256, 16, 4, 256, H.Q6K, H.Q4K),        # ragged tile, experts without tokens
+    (40, 320, 6, 3, 192, H.Q8_0, H.Q8_0),       # partial feature tiles on both GEMMs
+    (300, 256, 4, 2, 256, H.Q4K, H.Q8_0),       # buckets larger than one 128-token tile
+    (200, 2048, 128, 8, 768, H.Q4K, H.Q6K),     # config-2 layer shape
+    (128, 2048, 128, 8, 768, H.Q8_0, H.Q8_0),   # config-1 layer shape
+])
+def test_batched_moe_ffn_buckets_exactly_and_matches_oracle(be, rows, ne, E, K, nff, gdt, ddt):
+    rng = np.random.default_rng(rows + ne + gdt)
+    x = rng.standard_normal((rows, ne)).astype(np.float32)
+    x[rows // 2] *= 3.0e4      # a row far outside f16 range: the per-row scale must absorb it
+    x[rows // 3] *= 1.0e-6
+    router = (rng.standard_normal((E, ne)) * 0.02).astype(np.float32)
+    gate, up = _realistic(rng, E, nff, ne, gdt), _realistic(rng, E, nff, ne, gdt)
+    down = _realistic(rng, E, ne, nff, ddt)
+    g, ids = moe_graph(rows, ne, E, K, nff, DType(gdt), DType(ddt))
+    out, r, b = _run_batched(be, g, ids, dict(x=x, router=router, gate=gate, up=up, down=down), rows, ne)
+    ref = O.moe_ffn(x, router, gate, up, down, ne=ne, n_expert=E, n_used=K, n_ff_exp=nff, gate_dtype=gdt, down_dtype=ddt)
+    assert np.array_equal(r["idx"], ref["idx"])
+    assert np.array_equal(bits(r["w"]), bits(ref["w"]))
+    _check_bucketing(b, ref, E)
+    # per-row relative error: rows differ by ten orders of magnitude
+    num = np.linalg.norm((out - ref["dst"]).astype(np.float64), axis=1)
+    den = np.linalg.norm(ref["dst"].astype(np.float64), axis=1)
+    assert (den > 0).all()
+    worst = float((num / den).max())
+    assert worst < REL_L2_MFMA, worst
+    assert H.rel_l2(out, ref["dst"]) < REL_L2_MFMA
+
+
+def test_batched_moe_ffn_option_variants_match_oracle(be):
+    ne, E, K, nff, rows = 256, 8, 3, 256, 48
+    rng = np.random.default_rng(23)
+    x = rng.standard_normal((rows, ne)).astype(np.float32)
+    router = rng.standard_normal((E, ne)).astype(np.float32) * 0.05
+    gate, up = _realistic(rng, E, nff, ne, H.Q4K), _realistic(rng, E, nff, ne, H.Q4K)
+    down = _realistic(rng, E, ne, nff, H.Q6K)
+    ds = rng.uniform(0.5, 1.5, E).astype(np.float32)
+    bias = rng.standard_normal(E).astype(np.float32) * 0.1
+    eids = rng.integers(0, E, (rows, K)).astype(np.int32)
+    base = dict(ne=ne, n_expert=E, n_used=K, n_ff_exp=nff, gate_dtype=H.Q4K, down_dtype=H.Q6K)
+    cases = [
+        (dict(weight_before=True), dict(weight_before=True), {}),
+        (dict(swiglu_clamp=0.05), dict(swiglu_clamp=0.05), {}),
+        (dict(with_down_scale=True), dict(down_scale=ds), dict(down_scale=ds)),
+        (dict(gating=M.MoeGating.Sigmoid, norm_w=False, scale=2.5), dict(gating=O.GATE_SIGMOID, norm_w=False, scale=2.5), {}),
+        (dict(with_exp_probs_b=True, gating=M.MoeGating.Sigmoid), dict(exp_probs_b=bias, gating=O.GATE_SIGMOID), dict(exp_probs_b=bias)),
+        (dict(with_expert_ids=True), dict(expert_ids=eids), dict(expert_ids=eids)),   # duplicates inside a row allowed
+        (dict(act=M.Activation.Gelu), dict(act=O.ACT_GELU), {}),
+    ]
+    for gopts, oopts, extra in cases:
+        g, ids = moe_graph(rows, ne, E, K, nff, DType.Q4K, DType.Q6K, **dict(gopts))
+        out, r, b = _run_batched(be, g, ids, dict(x=x, router=router, gate=gate, up=up, down=down, **extra), rows, ne)
+        ref = O.moe_ffn(x, router, gate, up, down, **base, **oopts)
+        assert np.array_equal(r["idx"], ref["idx"]), gopts
+        _check_bucketing(b, ref, E)
+        assert H.rel_l2(out, ref["dst"]) < REL_L2_MFMA, (gopts, H.rel_l2(out, ref["dst"]))
+
+
+def test_small_batches_keep_the_per_token_path(be):
+    g, ids = moe_graph(16, 256, 8, 2, 256, DType.Q4K, DType.Q6K)
+    plan = be.compile(g)
+    with pytest.raises(M.BackendError):
+        be.moe_bucketing(plan, 0)
+    plan.free()
+
+
+@pytest.mark.parametrize("tokens,gdt,ddt", [(512, DType.Q8_0, DType.Q8_0), (512, DType.Q4K, DType.Q6K)])
+def test_prefill_chunk_with_skewed_routing_matches_oracle(be, tokens, gdt, ddt):
+    """Config-4 shape: one config-1 layer, Zipf(1.1) expert popularity injected through the op's own
+    inputs (x[:,0] = 1, router[:,0] = bias), device-generated weights."""
+    s = S.MoeShape("c4", 1, 2048, 128, 8, 768, gdt, ddt)
+    lw = S.LayerWeights(be, s, seed0=91, layer=0, on_device=True)
+    router = be.download(lw.router, dtype=np.float32).reshape(s.n_expert, s.ne).copy()
+    router[:, 0] = S.zipf_bias(s.n_expert, 1.1, 5)
+    be.upload(lw.router, router)
+    x = S.normal(S.stream_seed(92, 0, S.ROLE_X), tokens * s.ne, 1.0).reshape(tokens, s.ne).copy()
+    x[:, 0] = 1.0
+    g, ids = moe_graph(tokens, s.ne, s.n_expert, s.n_used, s.n_ff, gdt, ddt)
+    plan = be.compile(g)
+    xb, yb = be.buffer_from(x, M.BufferUsage.Activations), be.alloc(tokens * s.ne * 4, M.BufferUsage.Readback)
+    bnd = (M.Bindings().bind(ids["x"], xb).bind(ids["router"], lw.router).bind(ids["gate"], lw.gate)
+           .bind(ids["up"], lw.up).bind(ids["down"], lw.down).bind(ids["dst"], yb))
+    be.execute(plan, bnd)
+    got = be.download(yb, tokens * s.ne * 4, np.float32).reshape(tokens, s.ne)
+    r, b = be.moe_routing(plan, 0), be.moe_bucketing(plan, 0)
+    gate, up, down = be.download(lw.gate), be.download(lw.up), be.download(lw.down)
+    ref = O.moe_ffn(x, router, gate, up, down, ne=s.ne, n_expert=s.n_expert, n_used=s.n_used, n_ff_exp=s.n_ff,
+                    gate_dtype=int(gdt), down_dtype=int(ddt))
+    assert np.array_equal(r["idx"], ref["idx"])
+    _check_bucketing(b, ref, s.n_expert)
+    counts = np.diff(b["offsets"])
+    assert counts.max() > 4 * max(1, int(np.median(counts))), "routing is not skewed"
+    assert H.rel_l2(got, ref["dst"]) < REL_L2_MFMA, H.rel_l2(got, ref["dst"])
+    plan.free()
