@@ -27,6 +27,7 @@ import moe4all_amd as M  # noqa: E402
 from moe4all_amd import DType, TensorDesc, synth  # noqa: E402
 
 HBM_PEAK_GBPS = 8000.0
+MFMA_F16_PEAK_TFLOPS = 2500.0   # dense fp16/bf16 matrix-core peak of one MI355X
 SEED0 = 20260101
 N_TOKENS = 8  # distinct activation sets rotated through the steps
 
@@ -73,7 +74,11 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c5"])
+    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c4", "c4k", "c5"],
+                    help="c1/c2/c5: decode stacks (use --batch for multi-stream decode); c4: one config-1 layer "
+                         "(Q8_0), prefill chunk of --tokens with Zipf(1.1) expert popularity; c4k: same with "
+                         "Q4_K gate/up + Q6_K down")
+    ap.add_argument("--tokens", type=int, default=2048, help="prefill chunk size for c4/c4k")
     ap.add_argument("--layers", type=int, default=0, help="override the layer count (0 = the config's)")
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--no-cpu-baseline", action="store_true")
@@ -87,14 +92,24 @@ def main():
               file=sys.stderr)
         sys.exit(2)
 
-    shape = {"c1": synth.CONFIG_1, "c2": synth.CONFIG_2, "c5": synth.CONFIG_5}[args.config]
+    prefill = args.config in ("c4", "c4k")
+    shape = {"c1": synth.CONFIG_1, "c2": synth.CONFIG_2, "c5": synth.CONFIG_5,
+             "c4": synth.MoeShape(f"c4-prefill-{args.tokens}-zipf1.1-q8_0", 1, 2048, 128, 8, 768, DType.Q8_0, DType.Q8_0),
+             "c4k": synth.MoeShape(f"c4-prefill-{args.tokens}-zipf1.1-q4k-q6k", 1, 2048, 128, 8, 768, DType.Q4K,
+                                   DType.Q6K)}[args.config]
     n_layer = args.layers or shape.n_layer
-    batch = args.batch
+    batch = args.tokens if prefill else args.batch
     be = M.Backend(0)
     caps = be.capabilities()
     t_setup = time.time()
     g, layers, ids = build_stack(be, shape, n_layer, batch)
     plan = be.compile(g)
+    if prefill:
+        # skewed expert popularity through the op's own inputs: x[:, 0] = 1, router[e, 0] = ln Zipf(1.1)
+        for lw in layers:
+            router = be.download(lw.router, dtype=np.float32).reshape(shape.n_expert, shape.ne).copy()
+            router[:, 0] = synth.zipf_bias(shape.n_expert, 1.1, SEED0)
+            be.upload(lw.router, router)
     # activations: N_TOKENS independent sets of per-layer N(0,1) rows, resident in HBM
     xbufs = []
     for t in range(N_TOKENS):
@@ -103,6 +118,10 @@ def main():
             xb = be.alloc(batch * shape.ne * 4)
             synth.weights_device(be, xb, DType.F32, synth.stream_seed(SEED0 + 1 + t, l, synth.ROLE_X),
                                  batch * shape.ne, sigma=1.0)
+            if prefill:
+                xh = be.download(xb, dtype=np.float32).reshape(batch, shape.ne).copy()
+                xh[:, 0] = 1.0
+                be.upload(xb, xh)
             row.append(xb)
         xbufs.append(row)
     ybufs = [be.alloc(batch * shape.ne * 4) for _ in range(n_layer)]
@@ -165,14 +184,28 @@ def main():
         }
         # the decode kernel that routes its own token row also reads that row's logits
         alg["moe_route_gate_up"] = alg["moe_gate_up"] + batch * shape.n_expert * 4
+        flops = {  # algorithmic FLOPs per launch of the grouped GEMMs (2 per multiply-add)
+            "moe_grouped_gate_up": 2.0 * pairs * 2 * shape.n_ff * shape.ne,
+            "moe_grouped_down": 2.0 * pairs * shape.ne * shape.n_ff,
+        }
         for name, p in prof.items():
             avg_us = p["total_ms"] * 1e3 / max(p["launches"], 1)
             kernels[name] = {"launches": int(p["launches"]), "avg_us": round(avg_us, 3), "min_us": round(p["min_ms"] * 1e3, 3)}
             if name in alg:
                 kernels[name]["alg_bytes"] = alg[name]
                 kernels[name]["GBps"] = round(alg[name] / (avg_us * 1e-6) / 1e9, 1)
-        dom = max((k for k in kernels if k in alg), key=lambda k: kernels[k]["avg_us"] * kernels[k]["launches"], default=None)
-        if dom:
+            if name in flops:
+                kernels[name]["alg_flops"] = flops[name]
+                kernels[name]["TFLOPs"] = round(flops[name] / (avg_us * 1e-6) / 1e12, 1)
+        total_us = lambda k: kernels[k]["avg_us"] * kernels[k]["launches"]
+        cand = [k for k in kernels if k in flops] or [k for k in kernels if "alg_bytes" in kernels[k]]
+        dom = max(cand, key=total_us, default=None)
+        if dom and dom in flops:
+            ach = flops[dom] / (kernels[dom]["avg_us"] * 1e-6) / 1e12
+            roofline = {"bound": "mfma", "kernel": dom, "achieved": round(ach, 1), "peak": MFMA_F16_PEAK_TFLOPS,
+                        "unit": "TFLOP/s", "frac": round(ach / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None,
+                        "alg_flops_per_launch": flops[dom], "avg_launch_us": kernels[dom]["avg_us"]}
+        elif dom:
             # HBM bytes per launch measured with hardware counters in a separate profiler run of this
             # same command (profiles/), reported only for the workload they were taken on
             traffic = None
@@ -196,8 +229,12 @@ def main():
         gate, up, down = be.download(lw.gate), be.download(lw.up), be.download(lw.down)
         threads = O.hw_threads()
         n_sample, spent, budget_s = 0, 0.0, 12.0
+        cpu_rows = min(batch, 256)   # a prefill chunk is sampled by its first 256 tokens
         while spent < budget_s and n_sample < 4 * n_layer:
             x = synth.normal(synth.stream_seed(SEED0 + 1, n_sample, synth.ROLE_X), batch * shape.ne, 1.0)
+            x = x.reshape(batch, shape.ne)[:cpu_rows].copy()
+            if prefill:
+                x[:, 0] = 1.0
             t1 = time.perf_counter()
             O.moe_ffn(x, router, gate, up, down, ne=shape.ne, n_expert=shape.n_expert, n_used=shape.n_used,
                       n_ff_exp=shape.n_ff, gate_dtype=int(shape.gate_dtype), down_dtype=int(shape.down_dtype),
@@ -205,14 +242,14 @@ def main():
             spent += time.perf_counter() - t1
             n_sample += 1
         per_layer_s = spent / n_sample
-        cpu = {"value": round(batch / (per_layer_s * n_layer), 3), "unit": "tok/s", "cores": threads, "kind": "port",
-               "sample": f"{n_sample} layer-passes of layer 0 (routed experts only) with distinct seeded tokens, "
+        cpu = {"value": round(cpu_rows / (per_layer_s * n_layer), 3), "unit": "tok/s", "cores": threads, "kind": "port",
+               "sample": f"{n_sample} layer-passes of layer 0 (routed experts only, {cpu_rows} token rows each) with distinct seeded tokens, "
                          f"{per_layer_s * 1e3:.2f} ms per layer-pass, f32 reference numerics, "
                          f"scaled to {n_layer} layers",
                "ms_per_layer": round(per_layer_s * 1e3, 3)}
 
     out = {
-        "metric": "MoE decode tok/s", "value": round(tok_s, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
+        "metric": "MoE prefill tok/s" if prefill else "MoE decode tok/s", "value": round(tok_s, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": shape.name if n_layer == shape.n_layer else f"{shape.name}[{n_layer} layers]",

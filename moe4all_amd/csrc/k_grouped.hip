@@ -236,35 +236,77 @@ __global__ __launch_bounds__(256) void rows_to_f16_kernel(const float* __restric
 
 // --------------------------------------------------------------------------------------------
 // One wavefront per expert e in 0..n_expert (the extra one writes the total and marks pairs
-// whose id is out of range).  Every wave scans all pair ids; the scan order is the flat
-// (row, rank) order, so buckets come out rows ascending.
+// whose id is out of range).  The block stages the pair ids in LDS (16-bit, chunks of 16384) and
+// every wave scans all of them; the scan order is the flat (row, rank) order, so buckets come out
+// rows ascending.
+constexpr int kBucketChunk = 16384;
 __global__ __launch_bounds__(1024) void bucket_kernel(const int32_t* __restrict__ ids, int n_pairs, int n_expert,
                                                       int32_t* __restrict__ offsets, int32_t* __restrict__ pair_src,
                                                       int32_t* __restrict__ slot_pair) {
+    __shared__ uint16_t s_ids[kBucketChunk];
     const int lane = threadIdx.x & 63;
     const int e = blockIdx.x * 16 + (threadIdx.x >> 6);
-    if (e > n_expert) return;
-    uint32_t below = 0;
-    for (int i0 = 0; i0 < n_pairs; i0 += 64) {
-        const int i = i0 + lane;
-        const uint32_t id = i < n_pairs ? (uint32_t)ids[i] : 0xFFFFFFFFu;
-        below += (uint32_t)__popcll(__ballot(id < (uint32_t)e));
-        if (e == n_expert && i < n_pairs && id >= (uint32_t)n_expert) slot_pair[i] = -1;
-    }
-    if (lane == 0) offsets[e] = (int32_t)below;
-    if (e == n_expert) return;
-    uint32_t run = below;
-    for (int i0 = 0; i0 < n_pairs; i0 += 64) {
-        const int i = i0 + lane;
-        const bool hit = i < n_pairs && (uint32_t)ids[i] == (uint32_t)e;
-        const unsigned long long mask = __ballot(hit);
-        if (hit) {
-            const uint32_t p = run + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
-            pair_src[p] = i;
-            slot_pair[i] = (int32_t)p;
+    const bool live = e <= n_expert;
+    uint32_t below = 0, run = 0;
+    // pass 0 counts the pairs below e, pass 1 scatters
+    for (int pass = 0; pass < 2; pass++) {
+        if (pass == 1) {
+            if (live && lane == 0) offsets[e] = (int32_t)below;
+            run = below;
         }
-        run += (uint32_t)__popcll(mask);
+        for (int c0 = 0; c0 < n_pairs; c0 += kBucketChunk) {
+            const int cn = min(kBucketChunk, n_pairs - c0);
+            __syncthreads();
+            for (int i = threadIdx.x; i < cn; i += 1024) {
+                const uint32_t id = (uint32_t)ids[c0 + i];
+                s_ids[i] = id < (uint32_t)n_expert ? (uint16_t)id : (uint16_t)0xFFFF;  // n_expert <= 2048
+            }
+            __syncthreads();
+            if (!live) continue;
+            if (pass == 0) {
+#pragma unroll 8
+                for (int i0 = 0; i0 < cn; i0 += 64) {
+                    const int i = i0 + lane;
+                    const uint32_t id = i < cn ? s_ids[i] : 0xFFFFu;
+                    below += (uint32_t)__popcll(__ballot(id < (uint32_t)e));
+                }
+            } else if (e == n_expert) {
+                for (int i = lane; i < cn; i += 64)
+                    if (s_ids[i] == 0xFFFFu) slot_pair[c0 + i] = -1;
+            } else {
+#pragma unroll 4
+                for (int i0 = 0; i0 < cn; i0 += 64) {
+                    const int i = i0 + lane;
+                    const bool hit = i < cn && s_ids[i] == (uint16_t)e;
+                    const unsigned long long mask = __ballot(hit);
+                    if (hit) {
+                        const uint32_t p = run + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
+                        pair_src[p] = c0 + i;
+                        slot_pair[c0 + i] = (int32_t)p;
+                    }
+                    run += (uint32_t)__popcll(mask);
+                }
+            }
+        }
     }
+}
+
+// Activation for the matrix-core path: hardware exp (about 1e-6 relative), since operands were
+// already rounded to f16.  Same formulas as act_fn / gated_act_fn (crates/infr-cpu/src/kernels.rs:6664-6683).
+__device__ __forceinline__ float act_fast(int act, float g) {
+    if (act == INFR_ACT_SILU) return g / (1.0f + __expf(-g));
+    if (act == INFR_ACT_GELU) {
+        const float inner = 0.7978846f * (g + 0.044715f * g * g * g);
+        return 0.5f * g * (1.0f + tanhf(inner));
+    }
+    return 1.0f / (1.0f + __expf(-g));
+}
+__device__ __forceinline__ float gated_act_fast(int act, bool has_clamp, float clamp, float gate, float up) {
+    if (has_clamp) {
+        gate = fminf(gate, clamp);
+        up = fminf(fmaxf(up, -clamp), clamp);
+    }
+    return act_fast(act, gate) * up;
 }
 
 // --------------------------------------------------------------------------------------------
@@ -311,14 +353,12 @@ __global__ __launch_bounds__(256, 2) void grouped_mfma(GroupedParams p) {
     __shared__ uint4 sA[8 * kAStride];
     __shared__ uint4 sB[8 * 256];
     __shared__ float s_scale[kBM];
-    __shared__ uint64_t s_tab[32];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int nt = blockIdx.x % p.n_tiles_n;
     Tile t;
     if (!find_tile(p.offsets, p.n_expert, blockIdx.x / p.n_tiles_n, lane, t)) return;
     constexpr int kBN = DOWN ? 256 : 128;
     const int n0 = nt * kBN;
-    if (tid < 32) s_tab[tid] = kExp2Table[tid];
 
     const size_t row_bytes = (size_t)(p.K / F::kBlockElems) * F::kBlockBytes;
     const int feat = min(n0 + (DOWN ? tid : (tid & 127)), p.N - 1);
@@ -412,7 +452,7 @@ __global__ __launch_bounds__(256, 2) void grouped_mfma(GroupedParams p) {
                     g = __fmul_rn(wp, g);
                     u = __fmul_rn(wp, u);
                 }
-                if (f < p.N) orow[f] = gated_act_fn(p.act, p.has_clamp, p.clamp, g, u, s_tab);
+                if (f < p.N) orow[f] = gated_act_fast(p.act, p.has_clamp, p.clamp, g, u);
             }
         }
     }

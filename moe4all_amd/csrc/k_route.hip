@@ -167,8 +167,103 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const uint8_t* __res
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Logits for a batch (f32 router, ne a multiple of 32).  Block = 512 threads covering 32 experts
+// x 32 token rows: 8 chains x 8 row groups per wave, one wave per group of 4 experts.  A thread
+// keeps a 4 x 4 (expert, row) patch of accumulators for its chain, so each 128-bit LDS read
+// feeds 16 FMAs.  k advances in chunks of 128 elements staged transposed (chain-major) in LDS;
+// the accumulators run through all chunks, so every chain still adds its terms in ascending
+// order, exactly as the scalar reference does.
+constexpr int kLtTile = 32, kLtChunk = 128, kLtStride = kLtChunk / 8 + 4;
+__global__ __launch_bounds__(512) void router_logits_tiled_kernel(const float* __restrict__ router, size_t row_floats,
+                                                                  const float* __restrict__ x, int ne, int n_expert,
+                                                                  int rows, float* __restrict__ logits) {
+    __shared__ float sw[kLtTile * 8 * kLtStride];
+    __shared__ float sx[kLtTile * 8 * kLtStride];
+    const int tid = threadIdx.x, j = tid & 7, rg = (tid >> 3) & 7, eg = tid >> 6;
+    const int e0 = blockIdx.x * kLtTile, r0 = blockIdx.y * kLtTile;
+    float acc[4][4];
+#pragma unroll
+    for (int a = 0; a < 4; a++)
+#pragma unroll
+        for (int b = 0; b < 4; b++) acc[a][b] = 0.0f;
+    // staging role: two float4 of the router tile and two of the activation tile per chunk
+    const float* src[4];
+    bool ok[4];
+    int dst_base[4];
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const int idx = tid + 512 * (q & 1), row = idx >> 5, v = idx & 31;
+        const bool is_x = q >= 2;
+        const int g = (is_x ? r0 : e0) + row;
+        ok[q] = g < (is_x ? rows : n_expert);
+        src[q] = (is_x ? x + (size_t)(ok[q] ? g : 0) * ne : router + (size_t)(ok[q] ? g : 0) * row_floats) + 4 * v;
+        // element 4v+t of the chunk: chain (4v+t)&7 = 4(v&1)+t, step (4v+t)>>3 = v>>1
+        dst_base[q] = (row * 8 + 4 * (v & 1)) * kLtStride + (v >> 1);
+    }
+    float4 st[4];
+    auto fetch = [&](int k0) {
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const int v4 = 4 * ((tid + 512 * (q & 1)) & 31);
+            st[q] = (ok[q] && k0 + v4 < ne) ? *reinterpret_cast<const float4*>(src[q] + k0) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    };
+    fetch(0);
+    for (int k0 = 0; k0 < ne; k0 += kLtChunk) {
+        __syncthreads();
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            float* d = (q >= 2 ? sx : sw) + dst_base[q];
+            d[0] = st[q].x;
+            d[kLtStride] = st[q].y;
+            d[2 * kLtStride] = st[q].z;
+            d[3 * kLtStride] = st[q].w;
+        }
+        __syncthreads();
+        if (k0 + kLtChunk < ne) fetch(k0 + kLtChunk);
+        const int n_c = min(kLtChunk, ne - k0) >> 3;  // a multiple of 4
+        const float* wp = sw + (eg * 4 * 8 + j) * kLtStride;
+        const float* xp = sx + (rg * 4 * 8 + j) * kLtStride;
+        for (int c = 0; c < n_c; c += 4) {
+            float4 wv[4], xv[4];
+#pragma unroll
+            for (int a = 0; a < 4; a++) {
+                wv[a] = *reinterpret_cast<const float4*>(wp + a * 8 * kLtStride + c);
+                xv[a] = *reinterpret_cast<const float4*>(xp + a * 8 * kLtStride + c);
+            }
+#pragma unroll
+            for (int a = 0; a < 4; a++)
+#pragma unroll
+                for (int b = 0; b < 4; b++) {
+                    acc[a][b] = __fmaf_rn(wv[a].x, xv[b].x, acc[a][b]);
+                    acc[a][b] = __fmaf_rn(wv[a].y, xv[b].y, acc[a][b]);
+                    acc[a][b] = __fmaf_rn(wv[a].z, xv[b].z, acc[a][b]);
+                    acc[a][b] = __fmaf_rn(wv[a].w, xv[b].w, acc[a][b]);
+                }
+        }
+    }
+    const int lane = tid & 63;
+#pragma unroll
+    for (int a = 0; a < 4; a++)
+#pragma unroll
+        for (int b = 0; b < 4; b++) {
+            float s = 0.0f;
+#pragma unroll
+            for (int jj = 0; jj < 8; jj++) s = __fadd_rn(s, __shfl(acc[a][b], (lane & ~7) + jj, kWave));
+            const int e = e0 + eg * 4 + a, r = r0 + rg * 4 + b;
+            if (j == 0 && e < n_expert && r < rows) logits[(size_t)r * n_expert + e] = s;
+        }
+}
+
 bool launch_router_logits(hipStream_t s, const uint8_t* router, int rdt, size_t row_bytes, const float* x, int ne,
                           int n_expert, int rows, float* logits) {
+    if (rows >= 16 && rdt == INFR_F32 && (ne & 31) == 0 && (row_bytes & 15) == 0) {
+        dim3 grid((n_expert + kLtTile - 1) / kLtTile, (rows + kLtTile - 1) / kLtTile);
+        INFR_LAUNCH(router_logits_tiled_kernel, grid, dim3(512), 0, s, reinterpret_cast<const float*>(router), row_bytes / 4,
+                    x, ne, n_expert, rows, logits);
+        return true;
+    }
     // Decode (few rows): many small blocks.  Batches: 8 experts x 4 rows per pass.
     int epb = rows <= 2 ? 2 : 8;
     int rpb = rows <= 2 ? rows : 4;
