@@ -347,93 +347,82 @@ __device__ __forceinline__ bool find_tile(const int32_t* __restrict__ offsets, i
 // --------------------------------------------------------------------------------------------
 // 256 threads = 4 waves.  Thread r stages weight row r of the 256-row B tile (gate rows then up
 // rows, or 256 down rows); wave w owns two 32-feature column tiles (gate w / up w, or down
-// 2w / 2w+1) against up to four 32-token row tiles.
-template <class F, bool DOWN>
-__global__ __launch_bounds__(256, 2) void grouped_mfma(GroupedParams p) {
-    __shared__ uint4 sA[8 * kAStride];
-    __shared__ uint4 sB[8 * 256];
-    __shared__ float s_scale[kBM];
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    const int nt = blockIdx.x % p.n_tiles_n;
-    Tile t;
-    if (!find_tile(p.offsets, p.n_expert, blockIdx.x / p.n_tiles_n, lane, t)) return;
-    constexpr int kBN = DOWN ? 256 : 128;
-    const int n0 = nt * kBN;
-
-    const size_t row_bytes = (size_t)(p.K / F::kBlockElems) * F::kBlockBytes;
-    const int feat = min(n0 + (DOWN ? tid : (tid & 127)), p.N - 1);
-    const uint8_t* wrow = ((DOWN || tid < 128) ? p.w0 + (size_t)t.e * p.w0_stride : p.w1 + (size_t)t.e * p.w1_stride) +
-                          (size_t)feat * row_bytes;
+// 2w / 2w+1) against M 32-token row tiles.  M is a template parameter so that the k loop has no
+// branches: all LDS fragment reads of a k-step are issued ahead of its matrix instructions.
+struct GroupedCtx {
+    uint4* sA;
+    uint4* sB;
+    const float* s_scale;
+    const uint8_t* wrow;
     const uint4* asrc[4];
+    int tid, wave, lane, n0;
+    Tile t;
+};
+
+template <class F, bool DOWN, int M>
+__device__ __forceinline__ void grouped_tile(const GroupedParams& p, const GroupedCtx& c) {
+    const int tid = c.tid, wave = c.wave, lane = c.lane;
+    float16v acc0[M], acc1[M];
 #pragma unroll
-    for (int q = 0; q < 4; q++) {
-        const int c = tid + 256 * q, tok = c >> 3, kg = c & 7;
-        const int pr = t.p0 + min(tok, t.cnt - 1);
-        const size_t src_row = DOWN ? (size_t)pr : (size_t)(p.pair_src[pr] / p.n_used);
-        asrc[q] = reinterpret_cast<const uint4*>(p.a + src_row * p.K) + kg;
-    }
-    if (tid < kBM) {
-        const int pr = t.p0 + min(tid, t.cnt - 1);
-        s_scale[tid] = p.a_scale[DOWN ? pr : p.pair_src[pr] / p.n_used];
-    }
-    const int n_msub = (t.cnt + 31) >> 5;
-    float16v acc0[4], acc1[4];
-#pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < M; i++)
 #pragma unroll
         for (int r = 0; r < 16; r++) acc0[i][r] = acc1[i][r] = 0.0f;
 
     const int n_slices = p.K / kSlice;
-    typename F::Raw raw = F::load(wrow, 0);
+    typename F::Raw raw = F::load(c.wrow, 0);
     uint4 araw[4];
 #pragma unroll
-    for (int q = 0; q < 4; q++) araw[q] = asrc[q][0];
+    for (int q = 0; q < 4; q++) araw[q] = c.asrc[q][0];
     const int bt0 = DOWN ? 2 * wave : wave, bt1 = DOWN ? 2 * wave + 1 : 4 + wave;
+    const uint4* fb0 = c.sB + bt0 * 32 + (lane & 31) + (lane >> 5) * 256;
+    const uint4* fb1 = c.sB + bt1 * 32 + (lane & 31) + (lane >> 5) * 256;
+    const uint4* fa = c.sA + (lane & 31) + (lane >> 5) * kAStride;
     for (int s = 0; s < n_slices; s++) {
         {
             uint4 ch[8];
             F::expand(raw, s, ch);
 #pragma unroll
-            for (int g = 0; g < 8; g++) sB[g * 256 + tid] = ch[g];
+            for (int g = 0; g < 8; g++) c.sB[g * 256 + tid] = ch[g];
 #pragma unroll
             for (int q = 0; q < 4; q++) {
-                const int c = tid + 256 * q;
-                sA[(c & 7) * kAStride + (c >> 3)] = araw[q];
+                const int cc = tid + 256 * q;
+                if ((cc >> 3) < 32 * M) c.sA[(cc & 7) * kAStride + (cc >> 3)] = araw[q];
             }
         }
         __syncthreads();
         if (s + 1 < n_slices) {
-            raw = F::load(wrow, s + 1);
+            raw = F::load(c.wrow, s + 1);
 #pragma unroll
-            for (int q = 0; q < 4; q++) araw[q] = asrc[q][(s + 1) * (kSlice / 8)];
+            for (int q = 0; q < 4; q++)
+                if (((tid + 256 * q) >> 3) < 32 * M) araw[q] = c.asrc[q][(s + 1) * (kSlice / 8)];
         }
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) {
-            const int kg = 2 * ks + (lane >> 5);
-            const half8 b0 = __builtin_bit_cast(half8, sB[kg * 256 + bt0 * 32 + (lane & 31)]);
-            const half8 b1 = __builtin_bit_cast(half8, sB[kg * 256 + bt1 * 32 + (lane & 31)]);
+            const half8 b0 = __builtin_bit_cast(half8, fb0[2 * ks * 256]);
+            const half8 b1 = __builtin_bit_cast(half8, fb1[2 * ks * 256]);
+            half8 a[M];
 #pragma unroll
-            for (int mi = 0; mi < 4; mi++) {
-                if (mi < n_msub) {
-                    const half8 a = __builtin_bit_cast(half8, sA[kg * kAStride + mi * 32 + (lane & 31)]);
-                    acc0[mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b0, acc0[mi], 0, 0, 0);
-                    acc1[mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b1, acc1[mi], 0, 0, 0);
-                }
+            for (int mi = 0; mi < M; mi++) a[mi] = __builtin_bit_cast(half8, fa[2 * ks * kAStride + mi * 32]);
+#pragma unroll
+            for (int mi = 0; mi < M; mi++) {
+                acc0[mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mi], b0, acc0[mi], 0, 0, 0);
+                acc1[mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mi], b1, acc1[mi], 0, 0, 0);
             }
         }
         __syncthreads();
     }
 
     // accumulator register r of a 32x32 tile: row 8*(r/4) + 4*(lane/32) + r%4, column lane%32
+    const Tile& t = c.t;
+    const int n0 = c.n0;
     const float ds = (DOWN && p.down_scale) ? p.down_scale[t.e] : 1.0f;
 #pragma unroll
-    for (int mi = 0; mi < 4; mi++) {
-        if (mi >= n_msub) continue;
+    for (int mi = 0; mi < M; mi++) {
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             const int m = 32 * mi + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
             if (m >= t.cnt) continue;
-            const float sc = s_scale[m];
+            const float sc = c.s_scale[m];
             float* orow = p.out + (size_t)(t.p0 + m) * p.N;
             if (DOWN) {
                 const int f0 = n0 + 64 * wave + (lane & 31), f1 = f0 + 32;
@@ -455,6 +444,47 @@ __global__ __launch_bounds__(256, 2) void grouped_mfma(GroupedParams p) {
                 if (f < p.N) orow[f] = gated_act_fast(p.act, p.has_clamp, p.clamp, g, u);
             }
         }
+    }
+}
+
+template <class F, bool DOWN>
+__global__ __launch_bounds__(256, 2) void grouped_mfma(GroupedParams p) {
+    __shared__ uint4 sA[8 * kAStride];
+    __shared__ uint4 sB[8 * 256];
+    __shared__ float s_scale[kBM];
+    GroupedCtx c;
+    c.sA = sA;
+    c.sB = sB;
+    c.s_scale = s_scale;
+    const int tid = c.tid = threadIdx.x;
+    c.wave = tid >> 6;
+    c.lane = tid & 63;
+    const int nt = blockIdx.x % p.n_tiles_n;
+    if (!find_tile(p.offsets, p.n_expert, blockIdx.x / p.n_tiles_n, c.lane, c.t)) return;
+    const Tile& t = c.t;
+    constexpr int kBN = DOWN ? 256 : 128;
+    c.n0 = nt * kBN;
+
+    const size_t row_bytes = (size_t)(p.K / F::kBlockElems) * F::kBlockBytes;
+    const int feat = min(c.n0 + (DOWN ? tid : (tid & 127)), p.N - 1);
+    c.wrow = ((DOWN || tid < 128) ? p.w0 + (size_t)t.e * p.w0_stride : p.w1 + (size_t)t.e * p.w1_stride) +
+             (size_t)feat * row_bytes;
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const int cc = tid + 256 * q, tok = cc >> 3, kg = cc & 7;
+        const int pr = t.p0 + min(tok, t.cnt - 1);
+        const size_t src_row = DOWN ? (size_t)pr : (size_t)(p.pair_src[pr] / p.n_used);
+        c.asrc[q] = reinterpret_cast<const uint4*>(p.a + src_row * p.K) + kg;
+    }
+    if (tid < kBM) {
+        const int pr = t.p0 + min(tid, t.cnt - 1);
+        s_scale[tid] = p.a_scale[DOWN ? pr : p.pair_src[pr] / p.n_used];
+    }
+    switch ((t.cnt + 31) >> 5) {
+        case 1: grouped_tile<F, DOWN, 1>(p, c); break;
+        case 2: grouped_tile<F, DOWN, 2>(p, c); break;
+        case 3: grouped_tile<F, DOWN, 3>(p, c); break;
+        default: grouped_tile<F, DOWN, 4>(p, c); break;
     }
 }
 
