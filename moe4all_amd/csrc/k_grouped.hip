@@ -345,13 +345,22 @@ __device__ __forceinline__ bool find_tile(const int32_t* __restrict__ offsets, i
 }
 
 // --------------------------------------------------------------------------------------------
-// 256 threads = 4 waves.  Thread r stages weight row r of the 256-row B tile (gate rows then up
-// rows, or 256 down rows); wave w owns two 32-feature column tiles (gate w / up w, or down
-// 2w / 2w+1) against M 32-token row tiles.  M is a template parameter so that the k loop has no
-// branches: all LDS fragment reads of a k-step are issued ahead of its matrix instructions.
+// 512 threads = 8 waves, one block per CU, wave-specialised:
+//   waves 4..7 (producers): thread r stages weight row r of the 256-row B tile (gate rows then up
+//       rows, or 256 down rows) and four 16-byte chunks of the activation tile per 64-k slice;
+//       global loads run two slices ahead in registers, the unpacked f16 operands go to the LDS
+//       buffer the consumers are not reading;
+//   waves 0..3 (consumers): wave w owns two 32-feature column tiles (gate w / up w, or down
+//       2w / 2w+1) against M 32-token row tiles and does nothing but fragment reads and matrix
+//       instructions.
+// One barrier per slice; unpacking (VALU) and contraction (MFMA) of neighbouring slices overlap on
+// every SIMD.  M is a template parameter so that the k loop has no branches.
+constexpr int kABuf = 8 * kAStride, kBBuf = 8 * 256;          // 16-byte chunks per LDS buffer
+constexpr size_t kGroupedLds = (size_t)2 * (kABuf + kBBuf) * 16 + kBM * 4;
+
 struct GroupedCtx {
-    uint4* sA;
-    uint4* sB;
+    uint4* sA;   // [2][kABuf]
+    uint4* sB;   // [2][kBBuf]
     const float* s_scale;
     const uint8_t* wrow;
     const uint4* asrc[4];
@@ -359,57 +368,96 @@ struct GroupedCtx {
     Tile t;
 };
 
+template <class F, int M>
+__device__ __forceinline__ void produce(const GroupedParams& p, const GroupedCtx& c) {
+    const int pt = c.tid - 256;
+    const int n_slices = p.K / kSlice;
+    typename F::Raw raw0 = F::load(c.wrow, 0), raw1 = raw0;
+    uint4 ar0[4], ar1[4];
+    bool mine[4];
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        mine[q] = ((pt + 256 * q) >> 3) < 32 * M;
+        ar0[q] = ar1[q] = uint4{0, 0, 0, 0};
+        if (mine[q]) ar0[q] = c.asrc[q][0];
+    }
+    if (n_slices > 1) {
+        raw1 = F::load(c.wrow, 1);
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+            if (mine[q]) ar1[q] = c.asrc[q][kSlice / 8];
+    }
+    // slice s goes to buffer s & 1; `raw`/`ar` hold slice s on entry and slice s + 2 on exit
+    auto stage = [&](int s, typename F::Raw& raw, uint4 (&ar)[4]) {
+        uint4* sB = c.sB + (s & 1) * kBBuf;
+        uint4* sA = c.sA + (s & 1) * kABuf;
+        uint4 ch[8];
+        F::expand(raw, s, ch);
+#pragma unroll
+        for (int g = 0; g < 8; g++) sB[g * 256 + pt] = ch[g];
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const int cc = pt + 256 * q;
+            if (mine[q]) sA[(cc & 7) * kAStride + (cc >> 3)] = ar[q];
+        }
+        if (s + 2 < n_slices) {
+            raw = F::load(c.wrow, s + 2);
+#pragma unroll
+            for (int q = 0; q < 4; q++)
+                if (mine[q]) ar[q] = c.asrc[q][(s + 2) * (kSlice / 8)];
+        }
+    };
+    stage(0, raw0, ar0);
+    __syncthreads();
+    for (int s = 0; s < n_slices; s += 2) {
+        if (s + 1 < n_slices) stage(s + 1, raw1, ar1);
+        __syncthreads();
+        if (s + 1 < n_slices) {
+            if (s + 2 < n_slices) stage(s + 2, raw0, ar0);
+            __syncthreads();
+        }
+    }
+}
+
 template <class F, bool DOWN, int M>
-__device__ __forceinline__ void grouped_tile(const GroupedParams& p, const GroupedCtx& c) {
-    const int tid = c.tid, wave = c.wave, lane = c.lane;
+__device__ __forceinline__ void consume(const GroupedParams& p, const GroupedCtx& c) {
+    const int wave = c.wave, lane = c.lane;
     float16v acc0[M], acc1[M];
 #pragma unroll
     for (int i = 0; i < M; i++)
 #pragma unroll
         for (int r = 0; r < 16; r++) acc0[i][r] = acc1[i][r] = 0.0f;
-
     const int n_slices = p.K / kSlice;
-    typename F::Raw raw = F::load(c.wrow, 0);
-    uint4 araw[4];
-#pragma unroll
-    for (int q = 0; q < 4; q++) araw[q] = c.asrc[q][0];
     const int bt0 = DOWN ? 2 * wave : wave, bt1 = DOWN ? 2 * wave + 1 : 4 + wave;
     const uint4* fb0 = c.sB + bt0 * 32 + (lane & 31) + (lane >> 5) * 256;
     const uint4* fb1 = c.sB + bt1 * 32 + (lane & 31) + (lane >> 5) * 256;
     const uint4* fa = c.sA + (lane & 31) + (lane >> 5) * kAStride;
-    for (int s = 0; s < n_slices; s++) {
-        {
-            uint4 ch[8];
-            F::expand(raw, s, ch);
-#pragma unroll
-            for (int g = 0; g < 8; g++) c.sB[g * 256 + tid] = ch[g];
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-                const int cc = tid + 256 * q;
-                if ((cc >> 3) < 32 * M) c.sA[(cc & 7) * kAStride + (cc >> 3)] = araw[q];
-            }
-        }
-        __syncthreads();
-        if (s + 1 < n_slices) {
-            raw = F::load(c.wrow, s + 1);
-#pragma unroll
-            for (int q = 0; q < 4; q++)
-                if (((tid + 256 * q) >> 3) < 32 * M) araw[q] = c.asrc[q][(s + 1) * (kSlice / 8)];
-        }
+    auto slice = [&](int buf) {
+        const uint4* b0p = fb0 + buf * kBBuf;
+        const uint4* b1p = fb1 + buf * kBBuf;
+        const uint4* ap = fa + buf * kABuf;
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) {
-            const half8 b0 = __builtin_bit_cast(half8, fb0[2 * ks * 256]);
-            const half8 b1 = __builtin_bit_cast(half8, fb1[2 * ks * 256]);
+            const half8 b0 = __builtin_bit_cast(half8, b0p[2 * ks * 256]);
+            const half8 b1 = __builtin_bit_cast(half8, b1p[2 * ks * 256]);
             half8 a[M];
 #pragma unroll
-            for (int mi = 0; mi < M; mi++) a[mi] = __builtin_bit_cast(half8, fa[2 * ks * kAStride + mi * 32]);
+            for (int mi = 0; mi < M; mi++) a[mi] = __builtin_bit_cast(half8, ap[2 * ks * kAStride + mi * 32]);
 #pragma unroll
             for (int mi = 0; mi < M; mi++) {
                 acc0[mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mi], b0, acc0[mi], 0, 0, 0);
                 acc1[mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mi], b1, acc1[mi], 0, 0, 0);
             }
         }
+    };
+    __syncthreads();  // slice 0 staged
+    for (int s = 0; s < n_slices; s += 2) {
+        slice(0);
         __syncthreads();
+        if (s + 1 < n_slices) {
+            slice(1);
+            __syncthreads();
+        }
     }
 
     // accumulator register r of a 32x32 tile: row 8*(r/4) + 4*(lane/32) + r%4, column lane%32
@@ -447,14 +495,19 @@ __device__ __forceinline__ void grouped_tile(const GroupedParams& p, const Group
     }
 }
 
+template <class F, bool DOWN, int M>
+__device__ __forceinline__ void grouped_tile(const GroupedParams& p, const GroupedCtx& c) {
+    if (c.wave >= 4) produce<F, M>(p, c);
+    else consume<F, DOWN, M>(p, c);
+}
+
 template <class F, bool DOWN>
-__global__ __launch_bounds__(256, 2) void grouped_mfma(GroupedParams p) {
-    __shared__ uint4 sA[8 * kAStride];
-    __shared__ uint4 sB[8 * 256];
-    __shared__ float s_scale[kBM];
+__global__ __launch_bounds__(512) void grouped_mfma(GroupedParams p) {
+    extern __shared__ uint4 lds[];
     GroupedCtx c;
-    c.sA = sA;
-    c.sB = sB;
+    c.sA = lds;
+    c.sB = lds + 2 * kABuf;
+    float* s_scale = reinterpret_cast<float*>(lds + 2 * (kABuf + kBBuf));
     c.s_scale = s_scale;
     const int tid = c.tid = threadIdx.x;
     c.wave = tid >> 6;
@@ -464,14 +517,15 @@ __global__ __launch_bounds__(256, 2) void grouped_mfma(GroupedParams p) {
     const Tile& t = c.t;
     constexpr int kBN = DOWN ? 256 : 128;
     c.n0 = nt * kBN;
+    const int pt = tid & 255;  // staging role (used by the producer half)
 
     const size_t row_bytes = (size_t)(p.K / F::kBlockElems) * F::kBlockBytes;
-    const int feat = min(c.n0 + (DOWN ? tid : (tid & 127)), p.N - 1);
-    c.wrow = ((DOWN || tid < 128) ? p.w0 + (size_t)t.e * p.w0_stride : p.w1 + (size_t)t.e * p.w1_stride) +
+    const int feat = min(c.n0 + (DOWN ? pt : (pt & 127)), p.N - 1);
+    c.wrow = ((DOWN || pt < 128) ? p.w0 + (size_t)t.e * p.w0_stride : p.w1 + (size_t)t.e * p.w1_stride) +
              (size_t)feat * row_bytes;
 #pragma unroll
     for (int q = 0; q < 4; q++) {
-        const int cc = tid + 256 * q, tok = cc >> 3, kg = cc & 7;
+        const int cc = pt + 256 * q, tok = cc >> 3, kg = cc & 7;
         const int pr = t.p0 + min(tok, t.cnt - 1);
         const size_t src_row = DOWN ? (size_t)pr : (size_t)(p.pair_src[pr] / p.n_used);
         c.asrc[q] = reinterpret_cast<const uint4*>(p.a + src_row * p.K) + kg;
@@ -532,7 +586,13 @@ void grouped(hipStream_t s, const GroupedParams& p) {
     GroupedParams q = p;
     q.n_tiles_n = (p.N + bn - 1) / bn;
     const int max_tiles = p.n_pairs / kBM + (p.n_expert < p.n_pairs ? p.n_expert : p.n_pairs);
-    INFR_LAUNCH((grouped_mfma<F, DOWN>), dim3((unsigned)max_tiles * q.n_tiles_n), dim3(256), 0, s, q);
+    static bool attr_set = false;  // per instantiation
+    if (!attr_set) {
+        (void)hipFuncSetAttribute((const void*)grouped_mfma<F, DOWN>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  (int)kGroupedLds);
+        attr_set = true;
+    }
+    INFR_LAUNCH((grouped_mfma<F, DOWN>), dim3((unsigned)max_tiles * q.n_tiles_n), dim3(512), kGroupedLds, s, q);
 }
 
 }  // namespace
