@@ -46,19 +46,25 @@ __device__ __forceinline__ half2v splat(float v) {
 __device__ __forceinline__ half2v unbias(uint32_t magic_pair, float bias) { return as_h2(magic_pair) - splat(bias); }
 
 // --------------------------------------------------------------------------------------------
-// Weight formats.  load() fetches the 64 k-elements of virtual slice s of one weight row,
-// expand() turns them into 8 operand chunks of 8 f16 (chunk g = virtual k 8g..8g+7 of the slice).
-// chunk_src() gives, for virtual chunk c of a row, the two real offsets whose float4s feed it
-// and whether the 4 elements of each come out in the order 0,2,1,3.
+// Weight formats.  A 64-k slice of a weight row unpacks to 8 operand chunks of 8 f16; the matrix
+// instruction's lane halves split them: lanes 0..31 (half 0) own chunks 0..3, lanes 32..63 own
+// chunks 4..7, and k-step ks of the slice contracts chunk ks of each half.
+//   load(row, s, h)   the bytes half h needs from virtual slice s of a row
+//   prep(frag, s)     per-slice scale constants
+//   chunk(frag, c, ks) operand chunk 4h + ks as 8 f16
+//   chunk_src()       for virtual chunk c of a row, the two real offsets whose float4s feed it and
+//                     whether the 4 elements of each come out in the order 0,2,1,3
 struct MQ4K {
     static constexpr int kDt = INFR_Q4K, kBlockElems = 256, kBlockBytes = 144;
-    struct Raw {
-        uint4 hdr, qa, qb;
+    struct Frag {
+        uint4 hdr, q;
     };
-    static __device__ __forceinline__ Raw load(const uint8_t* row, int s) {
+    struct Prep {
+        half2v s_lo, n_lo, s_hi, n_hi;
+    };
+    static __device__ __forceinline__ Frag load(const uint8_t* row, int s, int h) {
         const uint8_t* blk = row + (size_t)(s >> 2) * 144;
-        const uint4* q = reinterpret_cast<const uint4*>(blk + 16 + (s & 3) * 32);
-        return Raw{*reinterpret_cast<const uint4*>(blk), q[0], q[1]};
+        return Frag{*reinterpret_cast<const uint4*>(blk), *reinterpret_cast<const uint4*>(blk + 16 + (s & 3) * 32 + 16 * h)};
     }
     static __device__ __forceinline__ uint32_t scale_byte(const uint4& hdr, int i) {  // scales[i], i in 0..11
         const uint32_t w = i < 4 ? hdr.y : (i < 8 ? hdr.z : hdr.w);
@@ -74,25 +80,23 @@ struct MQ4K {
             m = (scale_byte(hdr, j + 4) >> 4) | ((scale_byte(hdr, j) >> 6) << 4);
         }
     }
-    static __device__ __forceinline__ void expand(const Raw& r, int s, uint4 out[8]) {
+    static __device__ __forceinline__ Prep prep(const Frag& f, int s) {
         const int j = s & 3;
-        const float d = f16_bits_to_f32(r.hdr.x & 0xFFFFu), dmin = f16_bits_to_f32(r.hdr.x >> 16);
+        const float d = f16_bits_to_f32(f.hdr.x & 0xFFFFu), dmin = f16_bits_to_f32(f.hdr.x >> 16);
         uint32_t sc0, m0, sc1, m1;
-        scale_min(r.hdr, 2 * j, sc0, m0);
-        scale_min(r.hdr, 2 * j + 1, sc1, m1);
-        const half2v s_lo = splat(d * (float)sc0), n_lo = splat(-(dmin * (float)m0));
-        const half2v s_hi = splat(d * (float)sc1), n_hi = splat(-(dmin * (float)m1));
-        const uint32_t q[8] = {r.qa.x, r.qa.y, r.qa.z, r.qa.w, r.qb.x, r.qb.y, r.qb.z, r.qb.w};
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const uint32_t v = q[i];
-            const half2v a = unbias((v & 0x000F000Fu) | 0x64006400u, 1024.f);
-            const half2v b = unbias(((v >> 8) & 0x000F000Fu) | 0x64006400u, 1024.f);
-            const half2v c = unbias(((v >> 4) & 0x000F000Fu) | 0x64006400u, 1024.f);
-            const half2v e = unbias(((v >> 12) & 0x000F000Fu) | 0x64006400u, 1024.f);
-            out[i] = uint4{as_u32(__builtin_elementwise_fma(a, s_lo, n_lo)), as_u32(__builtin_elementwise_fma(b, s_lo, n_lo)),
-                           as_u32(__builtin_elementwise_fma(c, s_hi, n_hi)), as_u32(__builtin_elementwise_fma(e, s_hi, n_hi))};
-        }
+        scale_min(f.hdr, 2 * j, sc0, m0);
+        scale_min(f.hdr, 2 * j + 1, sc1, m1);
+        return Prep{splat(d * (float)sc0), splat(-(dmin * (float)m0)), splat(d * (float)sc1), splat(-(dmin * (float)m1))};
+    }
+    // byte l of the slice holds element l (low nibble, first 32-group) and 32 + l (high nibble)
+    static __device__ __forceinline__ uint4 chunk(const Frag& f, const Prep& c, int ks) {
+        const uint32_t v = ks == 0 ? f.q.x : ks == 1 ? f.q.y : ks == 2 ? f.q.z : f.q.w;
+        const half2v a = unbias((v & 0x000F000Fu) | 0x64006400u, 1024.f);
+        const half2v b = unbias(((v >> 8) & 0x000F000Fu) | 0x64006400u, 1024.f);
+        const half2v g = unbias(((v >> 4) & 0x000F000Fu) | 0x64006400u, 1024.f);
+        const half2v e = unbias(((v >> 12) & 0x000F000Fu) | 0x64006400u, 1024.f);
+        return uint4{as_u32(__builtin_elementwise_fma(a, c.s_lo, c.n_lo)), as_u32(__builtin_elementwise_fma(b, c.s_lo, c.n_lo)),
+                     as_u32(__builtin_elementwise_fma(g, c.s_hi, c.n_hi)), as_u32(__builtin_elementwise_fma(e, c.s_hi, c.n_hi))};
     }
     static __device__ __forceinline__ void chunk_src(int c, int& lo, int& hi, bool& swz) {
         const int i = c & 7;
@@ -104,42 +108,40 @@ struct MQ4K {
 
 struct MQ6K {
     static constexpr int kDt = INFR_Q6K, kBlockElems = 256, kBlockBytes = 210;
-    struct Raw {
-        uint4 la, lb, ha, hb;
-        uint32_t sc_lo, sc_hi, d;  // two int8 scales each, f16 d
+    struct Frag {
+        uint4 l, hq;
+        uint32_t sc_lo, sc_hi, d;  // one int8 scale each (16 elements = 4 chunks share one), f16 d
     };
-    // virtual slice t of a block: t = 2*half + ab; ab picks ql bytes [32ab, 32ab+32) of the half
-    static __device__ __forceinline__ Raw load(const uint8_t* row, int s) {
+    struct Prep {
+        half2v s_lo, s_hi;
+    };
+    // virtual slice t of a block: t = 2*half128 + ab; ab picks ql bytes [32ab, 32ab+32) of the
+    // 128-element half; their low nibbles are elements [32ab, 32ab+32), their high nibbles +64
+    static __device__ __forceinline__ Frag load(const uint8_t* row, int s, int h) {
         const uint8_t* blk = row + (size_t)(s >> 2) * 210;
         const int hh = (s >> 1) & 1, ab = s & 1;
-        Raw r;
-        r.la = ldu<uint4>(blk + 64 * hh + 32 * ab);
-        r.lb = ldu<uint4>(blk + 64 * hh + 32 * ab + 16);
-        r.ha = ldu<uint4>(blk + 128 + 32 * hh);
-        r.hb = ldu<uint4>(blk + 128 + 32 * hh + 16);
-        r.sc_lo = ldu<uint16_t>(blk + 192 + 8 * hh + 2 * ab);
-        r.sc_hi = ldu<uint16_t>(blk + 192 + 8 * hh + 2 * ab + 4);
-        r.d = ldu<uint16_t>(blk + 208);
-        return r;
+        Frag f;
+        f.l = ldu<uint4>(blk + 64 * hh + 32 * ab + 16 * h);
+        f.hq = ldu<uint4>(blk + 128 + 32 * hh + 16 * h);
+        f.sc_lo = blk[192 + 8 * hh + 2 * ab + h];
+        f.sc_hi = blk[192 + 8 * hh + 2 * ab + 4 + h];
+        f.d = ldu<uint16_t>(blk + 208);
+        return f;
     }
-    static __device__ __forceinline__ void expand(const Raw& r, int s, uint4 out[8]) {
-        const int sh = 2 * (s & 1);  // qh bit pair of this slice: bits sh..sh+1 (low codes), sh+4.. (high codes)
-        const float d = f16_bits_to_f32(r.d);
-        const half2v sl[2] = {splat(d * (float)(int8_t)(r.sc_lo & 0xFF)), splat(d * (float)(int8_t)(r.sc_lo >> 8))};
-        const half2v sh2[2] = {splat(d * (float)(int8_t)(r.sc_hi & 0xFF)), splat(d * (float)(int8_t)(r.sc_hi >> 8))};
-        const uint32_t ql[8] = {r.la.x, r.la.y, r.la.z, r.la.w, r.lb.x, r.lb.y, r.lb.z, r.lb.w};
-        const uint32_t qh[8] = {r.ha.x, r.ha.y, r.ha.z, r.ha.w, r.hb.x, r.hb.y, r.hb.z, r.hb.w};
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            const uint32_t L = ql[i], H = qh[i] >> sh;
-            const uint32_t a = (L & 0x000F000Fu) | ((H & 0x00030003u) << 4) | 0x64006400u;
-            const uint32_t b = ((L >> 8) & 0x000F000Fu) | (((H >> 8) & 0x00030003u) << 4) | 0x64006400u;
-            const uint32_t c = ((L >> 4) & 0x000F000Fu) | (H & 0x00300030u) | 0x64006400u;
-            const uint32_t e = ((L >> 12) & 0x000F000Fu) | ((H >> 8) & 0x00300030u) | 0x64006400u;
-            const half2v s0 = sl[i >> 2], s1 = sh2[i >> 2];
-            out[i] = uint4{as_u32(unbias(a, 1056.f) * s0), as_u32(unbias(b, 1056.f) * s0), as_u32(unbias(c, 1056.f) * s1),
-                           as_u32(unbias(e, 1056.f) * s1)};
-        }
+    static __device__ __forceinline__ Prep prep(const Frag& f, int) {
+        const float d = f16_bits_to_f32(f.d);
+        return Prep{splat(d * (float)(int8_t)f.sc_lo), splat(d * (float)(int8_t)f.sc_hi)};
+    }
+    static __device__ __forceinline__ uint4 chunk(const Frag& f, const Prep& c, int ks, int s) {
+        const int sh = 2 * (s & 1);  // qh bits sh..sh+1 complete the low codes, sh+4.. the high codes
+        const uint32_t L = ks == 0 ? f.l.x : ks == 1 ? f.l.y : ks == 2 ? f.l.z : f.l.w;
+        const uint32_t H = (ks == 0 ? f.hq.x : ks == 1 ? f.hq.y : ks == 2 ? f.hq.z : f.hq.w) >> sh;
+        const uint32_t a = (L & 0x000F000Fu) | ((H & 0x00030003u) << 4) | 0x64006400u;
+        const uint32_t b = ((L >> 8) & 0x000F000Fu) | (((H >> 8) & 0x00030003u) << 4) | 0x64006400u;
+        const uint32_t g = ((L >> 4) & 0x000F000Fu) | (H & 0x00300030u) | 0x64006400u;
+        const uint32_t e = ((L >> 12) & 0x000F000Fu) | ((H >> 8) & 0x00300030u) | 0x64006400u;
+        return uint4{as_u32(unbias(a, 1056.f) * c.s_lo), as_u32(unbias(b, 1056.f) * c.s_lo), as_u32(unbias(g, 1056.f) * c.s_hi),
+                     as_u32(unbias(e, 1056.f) * c.s_hi)};
     }
     static __device__ __forceinline__ void chunk_src(int c, int& lo, int& hi, bool& swz) {
         const int blk = c >> 5, t = (c >> 3) & 3, i = c & 7;
@@ -151,38 +153,28 @@ struct MQ6K {
 
 struct MQ80 {
     static constexpr int kDt = INFR_Q8_0, kBlockElems = 32, kBlockBytes = 34;
-    struct Raw {
-        uint32_t q[16];
-        uint32_t d0, d1;
+    struct Frag {
+        uint4 qa, qb;  // the 32 codes of block h of the slice
+        uint32_t d;
     };
-    static __device__ __forceinline__ Raw load(const uint8_t* row, int s) {
-        const uint8_t* p = row + (size_t)s * 68;
-        Raw r;
-        r.d0 = ldu<uint16_t>(p);
-        r.d1 = ldu<uint16_t>(p + 34);
-#pragma unroll
-        for (int i = 0; i < 8; i++) {
-            r.q[i] = ldu<uint32_t>(p + 2 + 4 * i);
-            r.q[8 + i] = ldu<uint32_t>(p + 36 + 4 * i);
-        }
-        return r;
+    struct Prep {
+        half2v d;
+    };
+    static __device__ __forceinline__ Frag load(const uint8_t* row, int s, int h) {
+        const uint8_t* p = row + (size_t)s * 68 + 34 * h;
+        return Frag{ldu<uint4>(p + 2), ldu<uint4>(p + 18), ldu<uint16_t>(p)};
     }
-    static __device__ __forceinline__ void expand(const Raw& r, int, uint4 out[8]) {
-        const half2v d[2] = {splat(f16_bits_to_f32(r.d0)), splat(f16_bits_to_f32(r.d1))};
-#pragma unroll
-        for (int g = 0; g < 8; g++) {
-            uint32_t o[4];
-#pragma unroll
-            for (int h = 0; h < 2; h++) {
-                const uint32_t v = r.q[2 * g + h];
-                // bytes (b0,b1) and (b2,b3) to the low bytes of the two halves; x ^ 0x80 = x + 128 as unsigned
-                const uint32_t p01 = __builtin_amdgcn_perm(0u, v, 0x0C010C00u) ^ 0x64806480u;
-                const uint32_t p23 = __builtin_amdgcn_perm(0u, v, 0x0C030C02u) ^ 0x64806480u;
-                o[2 * h] = as_u32(unbias(p01, 1152.f) * d[g >> 2]);
-                o[2 * h + 1] = as_u32(unbias(p23, 1152.f) * d[g >> 2]);
-            }
-            out[g] = uint4{o[0], o[1], o[2], o[3]};
-        }
+    static __device__ __forceinline__ Prep prep(const Frag& f, int) { return Prep{splat(f16_bits_to_f32(f.d))}; }
+    static __device__ __forceinline__ uint4 chunk(const Frag& f, const Prep& c, int ks) {
+        const uint32_t v0 = ks == 0 ? f.qa.x : ks == 1 ? f.qa.z : ks == 2 ? f.qb.x : f.qb.z;
+        const uint32_t v1 = ks == 0 ? f.qa.y : ks == 1 ? f.qa.w : ks == 2 ? f.qb.y : f.qb.w;
+        // bytes (b0,b1) and (b2,b3) to the low bytes of the two halves; x ^ 0x80 = x + 128 as unsigned
+        const uint32_t a = __builtin_amdgcn_perm(0u, v0, 0x0C010C00u) ^ 0x64806480u;
+        const uint32_t b = __builtin_amdgcn_perm(0u, v0, 0x0C030C02u) ^ 0x64806480u;
+        const uint32_t g = __builtin_amdgcn_perm(0u, v1, 0x0C010C00u) ^ 0x64806480u;
+        const uint32_t e = __builtin_amdgcn_perm(0u, v1, 0x0C030C02u) ^ 0x64806480u;
+        return uint4{as_u32(unbias(a, 1152.f) * c.d), as_u32(unbias(b, 1152.f) * c.d), as_u32(unbias(g, 1152.f) * c.d),
+                     as_u32(unbias(e, 1152.f) * c.d)};
     }
     static __device__ __forceinline__ void chunk_src(int c, int& lo, int& hi, bool& swz) {
         lo = 8 * c;
@@ -190,6 +182,12 @@ struct MQ80 {
         swz = false;
     }
 };
+
+template <class F>
+__device__ __forceinline__ uint4 fmt_chunk(const typename F::Frag& f, const typename F::Prep& c, int ks, int s) {
+    if constexpr (F::kDt == INFR_Q6K) return F::chunk(f, c, ks, s);
+    else return F::chunk(f, c, ks);
+}
 
 // --------------------------------------------------------------------------------------------
 // One block per row: amax -> power-of-two scale -> f16 in the virtual k order of format F.
@@ -346,33 +344,31 @@ __device__ __forceinline__ bool find_tile(const int32_t* __restrict__ offsets, i
 
 // --------------------------------------------------------------------------------------------
 // 512 threads = 8 waves, one block per CU, wave-specialised:
-//   waves 4..7 (producers): thread r stages weight row r of the 256-row B tile (gate rows then up
-//       rows, or 256 down rows) and four 16-byte chunks of the activation tile per 64-k slice;
-//       global loads run two slices ahead in registers, the unpacked f16 operands go to the LDS
-//       buffer the consumers are not reading;
+//   waves 4..7 (producers) copy the 128-token x 64-k activation tile of each slice from global
+//       memory (two slices ahead, in registers) into the LDS buffer the consumers are not reading;
 //   waves 0..3 (consumers): wave w owns two 32-feature column tiles (gate w / up w, or down
-//       2w / 2w+1) against M 32-token row tiles and does nothing but fragment reads and matrix
-//       instructions.
-// One barrier per slice; unpacking (VALU) and contraction (MFMA) of neighbouring slices overlap on
-// every SIMD.  M is a template parameter so that the k loop has no branches.
-constexpr int kABuf = 8 * kAStride, kBBuf = 8 * 256;          // 16-byte chunks per LDS buffer
-constexpr size_t kGroupedLds = (size_t)2 * (kABuf + kBBuf) * 16 + kBM * 4;
+//       2w / 2w+1) against M 32-token row tiles.  Each lane fetches the quantised bytes of ITS
+//       weight row and k half straight from global memory (two slices ahead) and unpacks them in
+//       registers into exactly the operand fragments it feeds to the matrix instruction, so the
+//       weights never pass through LDS; unpacking (VALU) interleaves with the MFMAs in flight.
+// One barrier per slice.  M is a template parameter so that the k loop has no branches.
+constexpr int kABuf = 8 * kAStride;                            // 16-byte chunks per LDS buffer
+constexpr size_t kGroupedLds = (size_t)2 * kABuf * 16 + kBM * 4;
 
 struct GroupedCtx {
     uint4* sA;   // [2][kABuf]
-    uint4* sB;   // [2][kBBuf]
     const float* s_scale;
-    const uint8_t* wrow;
-    const uint4* asrc[4];
+    const uint8_t* wrow0;   // consumer: weight rows of the lane's two column tiles
+    const uint8_t* wrow1;
+    const uint4* asrc[4];   // producer: the thread's four activation chunks
     int tid, wave, lane, n0;
     Tile t;
 };
 
-template <class F, int M>
+template <int M>
 __device__ __forceinline__ void produce(const GroupedParams& p, const GroupedCtx& c) {
     const int pt = c.tid - 256;
     const int n_slices = p.K / kSlice;
-    typename F::Raw raw0 = F::load(c.wrow, 0), raw1 = raw0;
     uint4 ar0[4], ar1[4];
     bool mine[4];
 #pragma unroll
@@ -382,38 +378,31 @@ __device__ __forceinline__ void produce(const GroupedParams& p, const GroupedCtx
         if (mine[q]) ar0[q] = c.asrc[q][0];
     }
     if (n_slices > 1) {
-        raw1 = F::load(c.wrow, 1);
 #pragma unroll
         for (int q = 0; q < 4; q++)
             if (mine[q]) ar1[q] = c.asrc[q][kSlice / 8];
     }
-    // slice s goes to buffer s & 1; `raw`/`ar` hold slice s on entry and slice s + 2 on exit
-    auto stage = [&](int s, typename F::Raw& raw, uint4 (&ar)[4]) {
-        uint4* sB = c.sB + (s & 1) * kBBuf;
+    // slice s goes to buffer s & 1; `ar` holds slice s on entry and slice s + 2 on exit
+    auto stage = [&](int s, uint4 (&ar)[4]) {
         uint4* sA = c.sA + (s & 1) * kABuf;
-        uint4 ch[8];
-        F::expand(raw, s, ch);
-#pragma unroll
-        for (int g = 0; g < 8; g++) sB[g * 256 + pt] = ch[g];
 #pragma unroll
         for (int q = 0; q < 4; q++) {
             const int cc = pt + 256 * q;
             if (mine[q]) sA[(cc & 7) * kAStride + (cc >> 3)] = ar[q];
         }
         if (s + 2 < n_slices) {
-            raw = F::load(c.wrow, s + 2);
 #pragma unroll
             for (int q = 0; q < 4; q++)
                 if (mine[q]) ar[q] = c.asrc[q][(s + 2) * (kSlice / 8)];
         }
     };
-    stage(0, raw0, ar0);
+    stage(0, ar0);
     __syncthreads();
     for (int s = 0; s < n_slices; s += 2) {
-        if (s + 1 < n_slices) stage(s + 1, raw1, ar1);
+        if (s + 1 < n_slices) stage(s + 1, ar1);
         __syncthreads();
         if (s + 1 < n_slices) {
-            if (s + 2 < n_slices) stage(s + 2, raw0, ar0);
+            if (s + 2 < n_slices) stage(s + 2, ar0);
             __syncthreads();
         }
     }
@@ -421,41 +410,49 @@ __device__ __forceinline__ void produce(const GroupedParams& p, const GroupedCtx
 
 template <class F, bool DOWN, int M>
 __device__ __forceinline__ void consume(const GroupedParams& p, const GroupedCtx& c) {
-    const int wave = c.wave, lane = c.lane;
+    const int wave = c.wave, lane = c.lane, half = lane >> 5;
     float16v acc0[M], acc1[M];
 #pragma unroll
     for (int i = 0; i < M; i++)
 #pragma unroll
         for (int r = 0; r < 16; r++) acc0[i][r] = acc1[i][r] = 0.0f;
     const int n_slices = p.K / kSlice;
-    const int bt0 = DOWN ? 2 * wave : wave, bt1 = DOWN ? 2 * wave + 1 : 4 + wave;
-    const uint4* fb0 = c.sB + bt0 * 32 + (lane & 31) + (lane >> 5) * 256;
-    const uint4* fb1 = c.sB + bt1 * 32 + (lane & 31) + (lane >> 5) * 256;
-    const uint4* fa = c.sA + (lane & 31) + (lane >> 5) * kAStride;
-    auto slice = [&](int buf) {
-        const uint4* b0p = fb0 + buf * kBBuf;
-        const uint4* b1p = fb1 + buf * kBBuf;
-        const uint4* ap = fa + buf * kABuf;
+    const uint4* fa = c.sA + (lane & 31) + 4 * half * kAStride;
+    typename F::Frag e0 = F::load(c.wrow0, 0, half), e1 = F::load(c.wrow1, 0, half);   // even slices
+    typename F::Frag o0 = e0, o1 = e1;                                                  // odd slices
+    if (n_slices > 1) {
+        o0 = F::load(c.wrow0, 1, half);
+        o1 = F::load(c.wrow1, 1, half);
+    }
+    // contracts slice s from LDS buffer s & 1 with the fragments in (f0, f1), then refills them
+    // with slice s + 2
+    auto slice = [&](int s, typename F::Frag& f0, typename F::Frag& f1) {
+        const uint4* ap = fa + (s & 1) * kABuf;
+        const typename F::Prep c0 = F::prep(f0, s), c1 = F::prep(f1, s);
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) {
-            const half8 b0 = __builtin_bit_cast(half8, b0p[2 * ks * 256]);
-            const half8 b1 = __builtin_bit_cast(half8, b1p[2 * ks * 256]);
+            const half8 b0 = __builtin_bit_cast(half8, fmt_chunk<F>(f0, c0, ks, s));
+            const half8 b1 = __builtin_bit_cast(half8, fmt_chunk<F>(f1, c1, ks, s));
             half8 a[M];
 #pragma unroll
-            for (int mi = 0; mi < M; mi++) a[mi] = __builtin_bit_cast(half8, ap[2 * ks * kAStride + mi * 32]);
+            for (int mi = 0; mi < M; mi++) a[mi] = __builtin_bit_cast(half8, ap[ks * kAStride + mi * 32]);
 #pragma unroll
             for (int mi = 0; mi < M; mi++) {
                 acc0[mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mi], b0, acc0[mi], 0, 0, 0);
                 acc1[mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mi], b1, acc1[mi], 0, 0, 0);
             }
         }
+        if (s + 2 < n_slices) {
+            f0 = F::load(c.wrow0, s + 2, half);
+            f1 = F::load(c.wrow1, s + 2, half);
+        }
     };
     __syncthreads();  // slice 0 staged
     for (int s = 0; s < n_slices; s += 2) {
-        slice(0);
+        slice(s, e0, e1);
         __syncthreads();
         if (s + 1 < n_slices) {
-            slice(1);
+            slice(s + 1, o0, o1);
             __syncthreads();
         }
     }
@@ -497,7 +494,7 @@ __device__ __forceinline__ void consume(const GroupedParams& p, const GroupedCtx
 
 template <class F, bool DOWN, int M>
 __device__ __forceinline__ void grouped_tile(const GroupedParams& p, const GroupedCtx& c) {
-    if (c.wave >= 4) produce<F, M>(p, c);
+    if (c.wave >= 4) produce<M>(p, c);
     else consume<F, DOWN, M>(p, c);
 }
 
@@ -506,8 +503,7 @@ __global__ __launch_bounds__(512) void grouped_mfma(GroupedParams p) {
     extern __shared__ uint4 lds[];
     GroupedCtx c;
     c.sA = lds;
-    c.sB = lds + 2 * kABuf;
-    float* s_scale = reinterpret_cast<float*>(lds + 2 * (kABuf + kBBuf));
+    float* s_scale = reinterpret_cast<float*>(lds + 2 * kABuf);
     c.s_scale = s_scale;
     const int tid = c.tid = threadIdx.x;
     c.wave = tid >> 6;
@@ -517,12 +513,22 @@ __global__ __launch_bounds__(512) void grouped_mfma(GroupedParams p) {
     const Tile& t = c.t;
     constexpr int kBN = DOWN ? 256 : 128;
     c.n0 = nt * kBN;
-    const int pt = tid & 255;  // staging role (used by the producer half)
 
+    // consumer role: the lane's weight rows
     const size_t row_bytes = (size_t)(p.K / F::kBlockElems) * F::kBlockBytes;
-    const int feat = min(c.n0 + (DOWN ? pt : (pt & 127)), p.N - 1);
-    c.wrow = ((DOWN || pt < 128) ? p.w0 + (size_t)t.e * p.w0_stride : p.w1 + (size_t)t.e * p.w1_stride) +
-             (size_t)feat * row_bytes;
+    const int cw = c.wave & 3;
+    if (DOWN) {
+        const int f0 = min(c.n0 + 64 * cw + (c.lane & 31), p.N - 1), f1 = min(c.n0 + 64 * cw + 32 + (c.lane & 31), p.N - 1);
+        const uint8_t* base = p.w0 + (size_t)t.e * p.w0_stride;
+        c.wrow0 = base + (size_t)f0 * row_bytes;
+        c.wrow1 = base + (size_t)f1 * row_bytes;
+    } else {
+        const int f = min(c.n0 + 32 * cw + (c.lane & 31), p.N - 1);
+        c.wrow0 = p.w0 + (size_t)t.e * p.w0_stride + (size_t)f * row_bytes;
+        c.wrow1 = p.w1 + (size_t)t.e * p.w1_stride + (size_t)f * row_bytes;
+    }
+    // producer role: the thread's activation chunks
+    const int pt = tid & 255;
 #pragma unroll
     for (int q = 0; q < 4; q++) {
         const int cc = pt + 256 * q, tok = cc >> 3, kg = cc & 7;
