@@ -61,24 +61,24 @@ struct MQ4K {
     };
     struct Prep {
         half2v s_lo, n_lo, s_hi, n_hi;
+        uint32_t magic;
     };
     static __device__ __forceinline__ Frag load(const uint8_t* row, int s, int h) {
         const uint8_t* blk = row + (size_t)(s >> 2) * 144;
         return Frag{*reinterpret_cast<const uint4*>(blk), *reinterpret_cast<const uint4*>(blk + 16 + (s & 3) * 32 + 16 * h)};
     }
-    static __device__ __forceinline__ uint32_t scale_byte(const uint4& hdr, int i) {  // scales[i], i in 0..11
-        const uint32_t w = i < 4 ? hdr.y : (i < 8 ? hdr.z : hdr.w);
-        return (w >> (8 * (i & 3))) & 0xFFu;
+    // scales[i] of the 12 packed bytes, i in 0..11, without branches
+    static __device__ __forceinline__ uint32_t scale_byte(const uint4& hdr, int i) {
+        const uint64_t lo = ((uint64_t)hdr.z << 32) | hdr.y;   // bytes 0..7
+        const uint32_t w = i < 8 ? (uint32_t)(lo >> (8 * (i & 7))) : hdr.w >> (8 * (i & 3));
+        return w & 0xFFu;
     }
     static __device__ __forceinline__ void scale_min(const uint4& hdr, int j, uint32_t& sc, uint32_t& m) {
-        // get_scale_min_k4 (crates/infr-gguf/src/dequant.rs:77-87)
-        if (j < 4) {
-            sc = scale_byte(hdr, j) & 63u;
-            m = scale_byte(hdr, j + 4) & 63u;
-        } else {
-            sc = (scale_byte(hdr, j + 4) & 0x0Fu) | ((scale_byte(hdr, j - 4) >> 6) << 4);
-            m = (scale_byte(hdr, j + 4) >> 4) | ((scale_byte(hdr, j) >> 6) << 4);
-        }
+        // get_scale_min_k4 (crates/infr-gguf/src/dequant.rs:77-87), both arms evaluated and selected
+        const uint32_t a = scale_byte(hdr, j & 3), b = scale_byte(hdr, (j & 3) + 4), c = scale_byte(hdr, (j & 3) + 8);
+        const bool low = j < 4;
+        sc = low ? (a & 63u) : ((c & 0x0Fu) | ((a >> 6) << 4));
+        m = low ? (b & 63u) : ((c >> 4) | ((b >> 6) << 4));
     }
     static __device__ __forceinline__ Prep prep(const Frag& f, int s) {
         const int j = s & 3;
@@ -86,15 +86,18 @@ struct MQ4K {
         uint32_t sc0, m0, sc1, m1;
         scale_min(f.hdr, 2 * j, sc0, m0);
         scale_min(f.hdr, 2 * j + 1, sc1, m1);
-        return Prep{splat(d * (float)sc0), splat(-(dmin * (float)m0)), splat(d * (float)sc1), splat(-(dmin * (float)m1))};
+        uint32_t magic = 0x64006400u;
+        asm volatile("" : "+v"(magic));   // keep it in a vector register (a literal cannot share an instruction with the mask)
+        return Prep{splat(d * (float)sc0), splat(-(dmin * (float)m0)), splat(d * (float)sc1), splat(-(dmin * (float)m1)), magic};
     }
     // byte l of the slice holds element l (low nibble, first 32-group) and 32 + l (high nibble)
     static __device__ __forceinline__ uint4 chunk(const Frag& f, const Prep& c, int ks) {
         const uint32_t v = ks == 0 ? f.q.x : ks == 1 ? f.q.y : ks == 2 ? f.q.z : f.q.w;
-        const half2v a = unbias((v & 0x000F000Fu) | 0x64006400u, 1024.f);
-        const half2v b = unbias(((v >> 8) & 0x000F000Fu) | 0x64006400u, 1024.f);
-        const half2v g = unbias(((v >> 4) & 0x000F000Fu) | 0x64006400u, 1024.f);
-        const half2v e = unbias(((v >> 12) & 0x000F000Fu) | 0x64006400u, 1024.f);
+        const uint32_t magic = c.magic;   // 0x64006400 in a register: one v_and_or_b32 per pair
+        const half2v a = unbias((v & 0x000F000Fu) | magic, 1024.f);
+        const half2v b = unbias(((v >> 8) & 0x000F000Fu) | magic, 1024.f);
+        const half2v g = unbias(((v >> 4) & 0x000F000Fu) | magic, 1024.f);
+        const half2v e = unbias(((v >> 12) & 0x000F000Fu) | magic, 1024.f);
         return uint4{as_u32(__builtin_elementwise_fma(a, c.s_lo, c.n_lo)), as_u32(__builtin_elementwise_fma(b, c.s_lo, c.n_lo)),
                      as_u32(__builtin_elementwise_fma(g, c.s_hi, c.n_hi)), as_u32(__builtin_elementwise_fma(e, c.s_hi, c.n_hi))};
     }
@@ -343,163 +346,156 @@ __device__ __forceinline__ bool find_tile(const int32_t* __restrict__ offsets, i
 }
 
 // --------------------------------------------------------------------------------------------
-// 512 threads = 8 waves, one block per CU, wave-specialised:
-//   waves 4..7 (producers) copy the 128-token x 64-k activation tile of each slice from global
-//       memory (two slices ahead, in registers) into the LDS buffer the consumers are not reading;
-//   waves 0..3 (consumers): wave w owns two 32-feature column tiles (gate w / up w, or down
-//       2w / 2w+1) against M 32-token row tiles.  Each lane fetches the quantised bytes of ITS
-//       weight row and k half straight from global memory (two slices ahead) and unpacks them in
-//       registers into exactly the operand fragments it feeds to the matrix instruction, so the
-//       weights never pass through LDS; unpacking (VALU) interleaves with the MFMAs in flight.
-// One barrier per slice.  M is a template parameter so that the k loop has no branches.
+// 256 threads = 4 waves, one wave per SIMD (so each may use the whole 512-entry register file:
+// the accumulators sit in AccVGPRs, deep prefetch rings in VGPRs).  Per 64-k slice every wave
+//   * contracts the slice: wave w owns two 32-feature column tiles (gate w / up w, or down
+//     2w / 2w+1) against M 32-token row tiles.  Each lane fetches the quantised bytes of ITS
+//     weight row and k half straight from global memory (kWRing slices ahead) and unpacks them in
+//     registers into exactly the operand fragments it feeds to the matrix instruction, so the
+//     weights never pass through LDS; unpacking (VALU) is issued between the MFMAs in flight;
+//   * copies its share of the next slice's 128-token x 64-k activation tile (loaded kARing slices
+//     ahead) into the LDS buffer nobody is reading.
+// One barrier per slice.  Every global load is unconditional (slice indices are clamped) and the
+// steady-state loop is straight-line code, so the wait counters the compiler inserts only wait for
+// the slice that is needed.  M is a template parameter so that the k loop has no branches.
 constexpr int kABuf = 8 * kAStride;                            // 16-byte chunks per LDS buffer
 constexpr size_t kGroupedLds = (size_t)2 * kABuf * 16 + kBM * 4;
+constexpr int kWRing = 4, kARing = 2, kUnroll = 4;             // kUnroll = lcm(kWRing, kARing, 2)
 
 struct GroupedCtx {
     uint4* sA;   // [2][kABuf]
     const float* s_scale;
-    const uint8_t* wrow0;   // consumer: weight rows of the lane's two column tiles
+    const uint8_t* wrow0;   // weight rows of the lane's two column tiles
     const uint8_t* wrow1;
-    const uint4* asrc[4];   // producer: the thread's four activation chunks
+    const uint4* asrc[4];   // the thread's four activation chunks
     int tid, wave, lane, n0;
     Tile t;
 };
 
-template <int M>
-__device__ __forceinline__ void produce(const GroupedParams& p, const GroupedCtx& c) {
-    const int pt = c.tid - 256;
-    const int n_slices = p.K / kSlice;
-    uint4 ar0[4], ar1[4];
-    bool mine[4];
-#pragma unroll
-    for (int q = 0; q < 4; q++) {
-        mine[q] = ((pt + 256 * q) >> 3) < 32 * M;
-        ar0[q] = ar1[q] = uint4{0, 0, 0, 0};
-        if (mine[q]) ar0[q] = c.asrc[q][0];
-    }
-    if (n_slices > 1) {
-#pragma unroll
-        for (int q = 0; q < 4; q++)
-            if (mine[q]) ar1[q] = c.asrc[q][kSlice / 8];
-    }
-    // slice s goes to buffer s & 1; `ar` holds slice s on entry and slice s + 2 on exit
-    auto stage = [&](int s, uint4 (&ar)[4]) {
-        uint4* sA = c.sA + (s & 1) * kABuf;
-#pragma unroll
-        for (int q = 0; q < 4; q++) {
-            const int cc = pt + 256 * q;
-            if (mine[q]) sA[(cc & 7) * kAStride + (cc >> 3)] = ar[q];
-        }
-        if (s + 2 < n_slices) {
-#pragma unroll
-            for (int q = 0; q < 4; q++)
-                if (mine[q]) ar[q] = c.asrc[q][(s + 2) * (kSlice / 8)];
-        }
-    };
-    stage(0, ar0);
-    __syncthreads();
-    for (int s = 0; s < n_slices; s += 2) {
-        if (s + 1 < n_slices) stage(s + 1, ar1);
-        __syncthreads();
-        if (s + 1 < n_slices) {
-            if (s + 2 < n_slices) stage(s + 2, ar0);
-            __syncthreads();
-        }
-    }
-}
-
 template <class F, bool DOWN, int M>
-__device__ __forceinline__ void consume(const GroupedParams& p, const GroupedCtx& c) {
-    const int wave = c.wave, lane = c.lane, half = lane >> 5;
+__device__ __forceinline__ void grouped_tile(const GroupedParams& p, const GroupedCtx& c) {
+    const int tid = c.tid, wave = c.wave, lane = c.lane, half = lane >> 5;
     float16v acc0[M], acc1[M];
 #pragma unroll
     for (int i = 0; i < M; i++)
 #pragma unroll
         for (int r = 0; r < 16; r++) acc0[i][r] = acc1[i][r] = 0.0f;
-    const int n_slices = p.K / kSlice;
+    const int n_slices = p.K / kSlice;   // a multiple of kUnroll (K is a multiple of 256)
+    const int last = n_slices - 1;
     const uint4* fa = c.sA + (lane & 31) + 4 * half * kAStride;
-    typename F::Frag e0 = F::load(c.wrow0, 0, half), e1 = F::load(c.wrow1, 0, half);   // even slices
-    typename F::Frag o0 = e0, o1 = e1;                                                  // odd slices
-    if (n_slices > 1) {
-        o0 = F::load(c.wrow0, 1, half);
-        o1 = F::load(c.wrow1, 1, half);
-    }
-    // contracts slice s from LDS buffer s & 1 with the fragments in (f0, f1), then refills them
-    // with slice s + 2
-    auto slice = [&](int s, typename F::Frag& f0, typename F::Frag& f1) {
+
+    // rings (named variables, so that they stay in registers): weights of slices s..s+3 in
+    // wa/wb/wc/wd by s % 4, activation chunks of slices s+1, s+2 in ae (even slice) / ao (odd)
+    static_assert(kWRing == 4 && kARing == 2 && kUnroll == 4, "the slice loop below is written for these depths");
+    typename F::Frag wa0 = F::load(c.wrow0, 0, half), wa1 = F::load(c.wrow1, 0, half);
+    typename F::Frag wb0 = F::load(c.wrow0, min(1, last), half), wb1 = F::load(c.wrow1, min(1, last), half);
+    typename F::Frag wc0 = F::load(c.wrow0, min(2, last), half), wc1 = F::load(c.wrow1, min(2, last), half);
+    typename F::Frag wd0 = F::load(c.wrow0, min(3, last), half), wd1 = F::load(c.wrow1, min(3, last), half);
+    const uint4 *as0 = c.asrc[0], *as1 = c.asrc[1], *as2 = c.asrc[2], *as3 = c.asrc[3];
+    struct A4 {
+        uint4 q0, q1, q2, q3;
+    };
+    auto load_a = [&](int sl) {
+        const int o = min(sl, last) * (kSlice / 8);
+        return A4{as0[o], as1[o], as2[o], as3[o]};
+    };
+    A4 ae = load_a(0), ao = load_a(1);
+    // (all four chunks are staged whatever M is: rows past the tile's tokens repeat its last token)
+    uint4* const st0 = c.sA + (tid & 7) * kAStride + (tid >> 3);   // chunk q of this thread sits 32 tokens further
+    auto stage = [&](int s, A4& a4) {   // slice s -> buffer s & 1, then refill with slice s + kARing
+        uint4* d = st0 + (s & 1) * kABuf;
+        d[0] = a4.q0;
+        d[32] = a4.q1;
+        d[64] = a4.q2;
+        d[96] = a4.q3;
+        a4 = load_a(s + kARing);
+    };
+    // contracts slice s from LDS buffer s & 1 with the fragments in (f0, f1), stages slice s + 1,
+    // refills the fragments with slice s + kWRing
+    auto slice = [&](int s, typename F::Frag& f0, typename F::Frag& f1, A4& a_next) {
         const uint4* ap = fa + (s & 1) * kABuf;
         const typename F::Prep c0 = F::prep(f0, s), c1 = F::prep(f1, s);
+        // software pipeline over the four k-steps: as soon as the two matrix instructions that
+        // use activation fragment mi are issued, the fragment register is reloaded for step
+        // ks + 1, and the unpacking of step ks + 1's weight chunks is spread between them
+        uint4 b0 = fmt_chunk<F>(f0, c0, 0, s), b1 = fmt_chunk<F>(f1, c1, 0, s);
+        uint4 a[M];
+#pragma unroll
+        for (int mi = 0; mi < M; mi++) a[mi] = ap[mi * 32];
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) {
-            const half8 b0 = __builtin_bit_cast(half8, fmt_chunk<F>(f0, c0, ks, s));
-            const half8 b1 = __builtin_bit_cast(half8, fmt_chunk<F>(f1, c1, ks, s));
-            half8 a[M];
-#pragma unroll
-            for (int mi = 0; mi < M; mi++) a[mi] = __builtin_bit_cast(half8, ap[ks * kAStride + mi * 32]);
+            uint4 nb0 = b0, nb1 = b1;
+            if (ks < 3) {
+                nb0 = fmt_chunk<F>(f0, c0, ks + 1, s);
+                nb1 = fmt_chunk<F>(f1, c1, ks + 1, s);
+            } else {
+                stage(s + 1, a_next);
+                f0 = F::load(c.wrow0, min(s + kWRing, last), half);
+                f1 = F::load(c.wrow1, min(s + kWRing, last), half);
+            }
 #pragma unroll
             for (int mi = 0; mi < M; mi++) {
-                acc0[mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mi], b0, acc0[mi], 0, 0, 0);
-                acc1[mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mi], b1, acc1[mi], 0, 0, 0);
+                acc0[mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, a[mi]), __builtin_bit_cast(half8, b0),
+                                                                  acc0[mi], 0, 0, 0);
+                acc1[mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, a[mi]), __builtin_bit_cast(half8, b1),
+                                                                  acc1[mi], 0, 0, 0);
+                if (ks < 3) a[mi] = ap[(ks + 1) * kAStride + mi * 32];
             }
-        }
-        if (s + 2 < n_slices) {
-            f0 = F::load(c.wrow0, s + 2, half);
-            f1 = F::load(c.wrow1, s + 2, half);
+            b0 = nb0;
+            b1 = nb1;
         }
     };
-    __syncthreads();  // slice 0 staged
-    for (int s = 0; s < n_slices; s += 2) {
-        slice(s, e0, e1);
+    stage(0, ae);
+    __syncthreads();
+    for (int s0 = 0; s0 < n_slices; s0 += kUnroll) {
+        slice(s0, wa0, wa1, ao);
         __syncthreads();
-        if (s + 1 < n_slices) {
-            slice(s + 1, o0, o1);
-            __syncthreads();
-        }
+        slice(s0 + 1, wb0, wb1, ae);
+        __syncthreads();
+        slice(s0 + 2, wc0, wc1, ao);
+        __syncthreads();
+        slice(s0 + 3, wd0, wd1, ae);
+        __syncthreads();
     }
 
     // accumulator register r of a 32x32 tile: row 8*(r/4) + 4*(lane/32) + r%4, column lane%32
     const Tile& t = c.t;
     const int n0 = c.n0;
+    const int fc0 = n0 + (DOWN ? 64 : 32) * wave + (lane & 31);   // the lane's column (second column tile of DOWN: + 32)
+    float* const obase = p.out + (size_t)t.p0 * p.N;
+    const bool plain_silu = !DOWN && p.act == INFR_ACT_SILU && !p.has_clamp && !p.weight_before;
     const float ds = (DOWN && p.down_scale) ? p.down_scale[t.e] : 1.0f;
 #pragma unroll
     for (int mi = 0; mi < M; mi++) {
 #pragma unroll
         for (int r = 0; r < 16; r++) {
             const int m = 32 * mi + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-            if (m >= t.cnt) continue;
             const float sc = c.s_scale[m];
-            float* orow = p.out + (size_t)(t.p0 + m) * p.N;
+            float* orow = obase + (size_t)m * p.N;
             if (DOWN) {
-                const int f0 = n0 + 64 * wave + (lane & 31), f1 = f0 + 32;
-                float y0 = __fmul_rn(acc0[mi][r], sc), y1 = __fmul_rn(acc1[mi][r], sc);
-                if (p.down_scale) {
-                    y0 = __fmul_rn(y0, ds);
-                    y1 = __fmul_rn(y1, ds);
-                }
-                if (f0 < p.N) orow[f0] = y0;
-                if (f1 < p.N) orow[f1] = y1;
+                const float y0 = acc0[mi][r] * sc * ds, y1 = acc1[mi][r] * sc * ds;
+                if (m < t.cnt && fc0 < p.N) orow[fc0] = y0;
+                if (m < t.cnt && fc0 + 32 < p.N) orow[fc0 + 32] = y1;
+            } else if (plain_silu) {
+                // silu(g) * u with the hardware exp and reciprocal
+                const float g = acc0[mi][r] * sc, u = acc1[mi][r] * sc;
+                const float h = g * u * __frcp_rn(1.0f + __expf(-g));
+                if (m < t.cnt && fc0 < p.N) orow[fc0] = h;
             } else {
-                const int f = n0 + 32 * wave + (lane & 31);
-                float g = __fmul_rn(acc0[mi][r], sc), u = __fmul_rn(acc1[mi][r], sc);
-                if (p.weight_before) {
+                float g = acc0[mi][r] * sc, u = acc1[mi][r] * sc;
+                if (p.weight_before && m < t.cnt) {
                     const float wp = p.route_w[p.pair_src[t.p0 + m]];
-                    g = __fmul_rn(wp, g);
-                    u = __fmul_rn(wp, u);
+                    g *= wp;
+                    u *= wp;
                 }
-                if (f < p.N) orow[f] = gated_act_fast(p.act, p.has_clamp, p.clamp, g, u);
+                if (m < t.cnt && fc0 < p.N) orow[fc0] = gated_act_fast(p.act, p.has_clamp, p.clamp, g, u);
             }
         }
     }
 }
 
-template <class F, bool DOWN, int M>
-__device__ __forceinline__ void grouped_tile(const GroupedParams& p, const GroupedCtx& c) {
-    if (c.wave >= 4) produce<M>(p, c);
-    else consume<F, DOWN, M>(p, c);
-}
-
 template <class F, bool DOWN>
-__global__ __launch_bounds__(512) void grouped_mfma(GroupedParams p) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void grouped_mfma(GroupedParams p) {
     extern __shared__ uint4 lds[];
     GroupedCtx c;
     c.sA = lds;
@@ -514,24 +510,22 @@ __global__ __launch_bounds__(512) void grouped_mfma(GroupedParams p) {
     constexpr int kBN = DOWN ? 256 : 128;
     c.n0 = nt * kBN;
 
-    // consumer role: the lane's weight rows
+    // the lane's weight rows
     const size_t row_bytes = (size_t)(p.K / F::kBlockElems) * F::kBlockBytes;
-    const int cw = c.wave & 3;
     if (DOWN) {
-        const int f0 = min(c.n0 + 64 * cw + (c.lane & 31), p.N - 1), f1 = min(c.n0 + 64 * cw + 32 + (c.lane & 31), p.N - 1);
+        const int f0 = min(c.n0 + 64 * c.wave + (c.lane & 31), p.N - 1), f1 = min(c.n0 + 64 * c.wave + 32 + (c.lane & 31), p.N - 1);
         const uint8_t* base = p.w0 + (size_t)t.e * p.w0_stride;
         c.wrow0 = base + (size_t)f0 * row_bytes;
         c.wrow1 = base + (size_t)f1 * row_bytes;
     } else {
-        const int f = min(c.n0 + 32 * cw + (c.lane & 31), p.N - 1);
+        const int f = min(c.n0 + 32 * c.wave + (c.lane & 31), p.N - 1);
         c.wrow0 = p.w0 + (size_t)t.e * p.w0_stride + (size_t)f * row_bytes;
         c.wrow1 = p.w1 + (size_t)t.e * p.w1_stride + (size_t)f * row_bytes;
     }
-    // producer role: the thread's activation chunks
-    const int pt = tid & 255;
+    // the thread's activation chunks
 #pragma unroll
     for (int q = 0; q < 4; q++) {
-        const int cc = pt + 256 * q, tok = cc >> 3, kg = cc & 7;
+        const int cc = tid + 256 * q, tok = cc >> 3, kg = cc & 7;
         const int pr = t.p0 + min(tok, t.cnt - 1);
         const size_t src_row = DOWN ? (size_t)pr : (size_t)(p.pair_src[pr] / p.n_used);
         c.asrc[q] = reinterpret_cast<const uint4*>(p.a + src_row * p.K) + kg;
@@ -598,15 +592,15 @@ void grouped(hipStream_t s, const GroupedParams& p) {
                                   (int)kGroupedLds);
         attr_set = true;
     }
-    INFR_LAUNCH((grouped_mfma<F, DOWN>), dim3((unsigned)max_tiles * q.n_tiles_n), dim3(512), kGroupedLds, s, q);
+    INFR_LAUNCH((grouped_mfma<F, DOWN>), dim3((unsigned)max_tiles * q.n_tiles_n), dim3(256), kGroupedLds, s, q);
 }
 
 }  // namespace
 
 bool grouped_supported(int dt, int k) {
-    if (k <= 0 || (k % kSlice) != 0) return false;
-    if (dt == INFR_Q4K || dt == INFR_Q6K) return (k % 256) == 0;
-    return dt == INFR_Q8_0;
+    // the k loop runs in groups of kUnroll 64-element slices
+    if (k <= 0 || (k % (kSlice * kUnroll)) != 0) return false;
+    return dt == INFR_Q4K || dt == INFR_Q6K || dt == INFR_Q8_0;
 }
 
 void launch_rows_to_f16(hipStream_t s, int weight_dt, const float* src, int rows, int n, void* dst, float* scale) {
