@@ -236,56 +236,105 @@ __global__ __launch_bounds__(256) void rows_to_f16_kernel(const float* __restric
 }
 
 // --------------------------------------------------------------------------------------------
-// One wavefront per expert e in 0..n_expert (the extra one writes the total and marks pairs
-// whose id is out of range).  The block stages the pair ids in LDS (16-bit, chunks of 16384) and
-// every wave scans all of them; the scan order is the flat (row, rank) order, so buckets come out
-// rows ascending.
+// One wavefront (= one block, so the experts spread over the CUs) per expert e in 0..n_expert; the
+// extra one writes the total and marks pairs whose id is out of range.  The wave stages the pair
+// ids in LDS (16-bit, chunks of 16384, sixteen 16-byte loads in flight per lane) and scans them
+// twice: count the pairs below e, then scatter.  The scan order is the flat (row, rank) order, so
+// buckets come out rows ascending.
 constexpr int kBucketChunk = 16384;
-__global__ __launch_bounds__(1024) void bucket_kernel(const int32_t* __restrict__ ids, int n_pairs, int n_expert,
-                                                      int32_t* __restrict__ offsets, int32_t* __restrict__ pair_src,
-                                                      int32_t* __restrict__ slot_pair) {
+__global__ __launch_bounds__(64) void bucket_kernel(const int32_t* __restrict__ ids, int n_pairs, int n_expert,
+                                                    int32_t* __restrict__ offsets, int32_t* __restrict__ pair_src,
+                                                    int32_t* __restrict__ slot_pair) {
     __shared__ uint16_t s_ids[kBucketChunk];
-    const int lane = threadIdx.x & 63;
-    const int e = blockIdx.x * 16 + (threadIdx.x >> 6);
-    const bool live = e <= n_expert;
+    const int lane = threadIdx.x;
+    const uint32_t e = blockIdx.x;
+    auto narrow = [&](int32_t v) { return (uint32_t)v < (uint32_t)n_expert ? (uint32_t)v : 0xFFFFu; };  // n_expert <= 2048
+    auto stage = [&](int c0, int cn) {
+        __syncthreads();  // orders the LDS reads of the previous chunk before these writes
+        // full groups of four ids: sixteen unconditional (index-clamped) 16-byte loads in flight per lane
+        const int full = cn & ~3;
+        for (int b0 = 0; b0 < full; b0 += 64 * 4 * 16) {
+            int4 v[16];
+#pragma unroll
+            for (int j = 0; j < 16; j++) {
+                const int i = min(b0 + (j * 64 + lane) * 4, full - 4);
+                v[j] = *reinterpret_cast<const int4*>(ids + c0 + i);
+            }
+#pragma unroll
+            for (int j = 0; j < 16; j++) {
+                const int i = b0 + (j * 64 + lane) * 4;
+                if (i < full) {
+                    const uint32_t lo = narrow(v[j].x) | (narrow(v[j].y) << 16), hi = narrow(v[j].z) | (narrow(v[j].w) << 16);
+                    *reinterpret_cast<uint2*>(&s_ids[i]) = make_uint2(lo, hi);
+                }
+            }
+        }
+        // the last one to three ids, padded to a group of four with 0xFFFF
+        if (lane < 4 && full < cn) s_ids[full + lane] = full + lane < cn ? (uint16_t)narrow(ids[c0 + full + lane]) : (uint16_t)0xFFFF;
+        __syncthreads();
+    };
     uint32_t below = 0, run = 0;
-    // pass 0 counts the pairs below e, pass 1 scatters
     for (int pass = 0; pass < 2; pass++) {
         if (pass == 1) {
-            if (live && lane == 0) offsets[e] = (int32_t)below;
+#pragma unroll
+            for (int d = 32; d >= 1; d >>= 1) below += __shfl_xor(below, d, 64);
+            if (lane == 0) offsets[e] = (int32_t)below;
             run = below;
         }
         for (int c0 = 0; c0 < n_pairs; c0 += kBucketChunk) {
             const int cn = min(kBucketChunk, n_pairs - c0);
-            __syncthreads();
-            for (int i = threadIdx.x; i < cn; i += 1024) {
-                const uint32_t id = (uint32_t)ids[c0 + i];
-                s_ids[i] = id < (uint32_t)n_expert ? (uint16_t)id : (uint16_t)0xFFFF;  // n_expert <= 2048
-            }
-            __syncthreads();
-            if (!live) continue;
-            if (pass == 0) {
-#pragma unroll 8
-                for (int i0 = 0; i0 < cn; i0 += 64) {
-                    const int i = i0 + lane;
-                    const uint32_t id = i < cn ? s_ids[i] : 0xFFFFu;
-                    below += (uint32_t)__popcll(__ballot(id < (uint32_t)e));
+            if (pass == 0 || n_pairs > kBucketChunk) stage(c0, cn);   // a single chunk stays staged for the second pass
+            // eight ids per lane per step (one 128-bit LDS read); the staging filled the chunk's last
+            // partial group of four with 0xFFFF, the tail of a partial group of eight is masked here
+            const int n8 = (cn + 7) >> 3;
+            auto ids8 = [&](int g, uint32_t (&id)[8]) {
+                const uint4 v = *reinterpret_cast<const uint4*>(&s_ids[8 * g]);
+                const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                for (int c = 0; c < 8; c++) {
+                    id[c] = (w[c >> 1] >> (16 * (c & 1))) & 0xFFFFu;
+                    if (8 * g + c >= ((cn + 3) & ~3)) id[c] = 0xFFFFu;
                 }
-            } else if (e == n_expert) {
+            };
+            if (pass == 0) {
+#pragma unroll 4
+                for (int g = lane; g < n8; g += 64) {
+                    uint32_t id[8];
+                    ids8(g, id);
+#pragma unroll
+                    for (int c = 0; c < 8; c++) below += id[c] < e;
+                }
+            } else if (e == (uint32_t)n_expert) {
                 for (int i = lane; i < cn; i += 64)
                     if (s_ids[i] == 0xFFFFu) slot_pair[c0 + i] = -1;
             } else {
-#pragma unroll 4
-                for (int i0 = 0; i0 < cn; i0 += 64) {
-                    const int i = i0 + lane;
-                    const bool hit = i < cn && s_ids[i] == (uint16_t)e;
-                    const unsigned long long mask = __ballot(hit);
-                    if (hit) {
-                        const uint32_t p = run + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
-                        pair_src[p] = c0 + i;
-                        slot_pair[c0 + i] = (int32_t)p;
+#pragma unroll 2
+                for (int g0 = 0; g0 < n8; g0 += 64) {
+                    const int g = g0 + lane;
+                    uint32_t id[8];
+#pragma unroll
+                    for (int c = 0; c < 8; c++) id[c] = 0xFFFFu;
+                    if (g < n8) ids8(g, id);
+                    uint32_t mine = 0;
+#pragma unroll
+                    for (int c = 0; c < 8; c++) mine += id[c] == e;
+                    // inclusive prefix of the per-lane hit counts (a lane's eight pairs are consecutive)
+                    uint32_t incl = mine;
+#pragma unroll
+                    for (int d = 1; d < 64; d <<= 1) {
+                        const uint32_t o = __shfl_up(incl, d, 64);
+                        if (lane >= d) incl += o;
                     }
-                    run += (uint32_t)__popcll(mask);
+                    uint32_t pos = run + incl - mine;
+#pragma unroll
+                    for (int c = 0; c < 8; c++) {
+                        if (id[c] == e) {
+                            pair_src[pos] = c0 + 8 * g + c;
+                            slot_pair[c0 + 8 * g + c] = (int32_t)pos;
+                            pos++;
+                        }
+                    }
+                    run += __shfl(incl, 63, 64);
                 }
             }
         }
@@ -613,9 +662,7 @@ void launch_rows_to_f16(hipStream_t s, int weight_dt, const float* src, int rows
 
 void launch_bucket(hipStream_t s, const int32_t* ids, int n_pairs, int n_expert, int32_t* offsets, int32_t* pair_src,
                    int32_t* slot_pair) {
-    const int waves = n_expert + 1;
-    INFR_LAUNCH(bucket_kernel, dim3((waves + 15) / 16), dim3(1024), 0, s, ids, n_pairs, n_expert, offsets, pair_src,
-                slot_pair);
+    INFR_LAUNCH(bucket_kernel, dim3(n_expert + 1), dim3(64), 0, s, ids, n_pairs, n_expert, offsets, pair_src, slot_pair);
 }
 
 void launch_grouped_gate_up(hipStream_t s, int dt, const GroupedParams& p) {
