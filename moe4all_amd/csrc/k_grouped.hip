@@ -48,24 +48,31 @@ __device__ __forceinline__ half2v unbias(uint32_t magic_pair, float bias) { retu
 // --------------------------------------------------------------------------------------------
 // Weight formats.  A 64-k slice of a weight row unpacks to 8 operand chunks of 8 f16; the matrix
 // instruction's lane halves split them: lanes 0..31 (half 0) own chunks 0..3, lanes 32..63 own
-// chunks 4..7, and k-step ks of the slice contracts chunk ks of each half.
-//   load(row, s, h)   the bytes half h needs from virtual slice s of a row
-//   prep(frag, s)     per-slice scale constants
-//   chunk(frag, c, ks) operand chunk 4h + ks as 8 f16
-//   chunk_src()       for virtual chunk c of a row, the two real offsets whose float4s feed it and
-//                     whether the 4 elements of each come out in the order 0,2,1,3
+// chunks 4..7, and k-step ks of the slice contracts chunk ks of each half.  Four slices make one
+// 256-element step (a K-quant super-block); what is shared by the four slices is fetched once:
+//   load_blk(row, b, h)     per-256 part (scales, high bits) half h needs of step b
+//   load_q(row, s, h)       the code bytes half h needs of virtual slice s
+//   prep(blk, q, s, h)      per-slice scale constants
+//   chunk(blk, q, c, ks, s) operand chunk 4h + ks as 8 f16
+//   chunk_src()             for virtual chunk c of a row, the two real offsets whose float4s feed
+//                           it and whether the 4 elements of each come out in the order 0,2,1,3
 struct MQ4K {
     static constexpr int kDt = INFR_Q4K, kBlockElems = 256, kBlockBytes = 144;
-    struct Frag {
-        uint4 hdr, q;
+    struct Blk {
+        uint4 hdr;   // d, dmin, 12 packed 6-bit scales / mins
+    };
+    struct Q {
+        uint4 q;
     };
     struct Prep {
         half2v s_lo, n_lo, s_hi, n_hi;
         uint32_t magic;
     };
-    static __device__ __forceinline__ Frag load(const uint8_t* row, int s, int h) {
-        const uint8_t* blk = row + (size_t)(s >> 2) * 144;
-        return Frag{*reinterpret_cast<const uint4*>(blk), *reinterpret_cast<const uint4*>(blk + 16 + (s & 3) * 32 + 16 * h)};
+    static __device__ __forceinline__ Blk load_blk(const uint8_t* row, int b, int) {
+        return Blk{*reinterpret_cast<const uint4*>(row + (size_t)b * 144)};
+    }
+    static __device__ __forceinline__ Q load_q(const uint8_t* row, int s, int h) {
+        return Q{*reinterpret_cast<const uint4*>(row + (size_t)(s >> 2) * 144 + 16 + (s & 3) * 32 + 16 * h)};
     }
     // scales[i] of the 12 packed bytes, i in 0..11, without branches
     static __device__ __forceinline__ uint32_t scale_byte(const uint4& hdr, int i) {
@@ -80,18 +87,18 @@ struct MQ4K {
         sc = low ? (a & 63u) : ((c & 0x0Fu) | ((a >> 6) << 4));
         m = low ? (b & 63u) : ((c >> 4) | ((b >> 6) << 4));
     }
-    static __device__ __forceinline__ Prep prep(const Frag& f, int s) {
+    static __device__ __forceinline__ Prep prep(const Blk& blk, const Q&, int s, int) {
         const int j = s & 3;
-        const float d = f16_bits_to_f32(f.hdr.x & 0xFFFFu), dmin = f16_bits_to_f32(f.hdr.x >> 16);
+        const float d = f16_bits_to_f32(blk.hdr.x & 0xFFFFu), dmin = f16_bits_to_f32(blk.hdr.x >> 16);
         uint32_t sc0, m0, sc1, m1;
-        scale_min(f.hdr, 2 * j, sc0, m0);
-        scale_min(f.hdr, 2 * j + 1, sc1, m1);
+        scale_min(blk.hdr, 2 * j, sc0, m0);
+        scale_min(blk.hdr, 2 * j + 1, sc1, m1);
         uint32_t magic = 0x64006400u;
         asm volatile("" : "+v"(magic));   // keep it in a vector register (a literal cannot share an instruction with the mask)
         return Prep{splat(d * (float)sc0), splat(-(dmin * (float)m0)), splat(d * (float)sc1), splat(-(dmin * (float)m1)), magic};
     }
     // byte l of the slice holds element l (low nibble, first 32-group) and 32 + l (high nibble)
-    static __device__ __forceinline__ uint4 chunk(const Frag& f, const Prep& c, int ks) {
+    static __device__ __forceinline__ uint4 chunk(const Blk&, const Q& f, const Prep& c, int ks, int) {
         const uint32_t v = ks == 0 ? f.q.x : ks == 1 ? f.q.y : ks == 2 ? f.q.z : f.q.w;
         const uint32_t magic = c.magic;   // 0x64006400 in a register: one v_and_or_b32 per pair
         const half2v a = unbias((v & 0x000F000Fu) | magic, 1024.f);
@@ -111,34 +118,42 @@ struct MQ4K {
 
 struct MQ6K {
     static constexpr int kDt = INFR_Q6K, kBlockElems = 256, kBlockBytes = 210;
-    struct Frag {
-        uint4 l, hq;
-        uint32_t sc_lo, sc_hi, d;  // one int8 scale each (16 elements = 4 chunks share one), f16 d
+    // virtual slice t of a block: t = 2*half128 + ab; ab picks ql bytes [32ab, 32ab+32) of the
+    // 128-element half; their low nibbles are elements [32ab, 32ab+32), their high nibbles +64.
+    // The 2-bit tops of both ab of a half share the same qh bytes.
+    struct Blk {
+        uint4 sc;        // 16 int8 scales
+        uint4 hq0, hq1;  // qh bytes [16h, 16h+16) of 128-element half 0 / 1
+        uint32_t d;      // f16
+    };
+    struct Q {
+        uint4 l;
     };
     struct Prep {
         half2v s_lo, s_hi;
     };
-    // virtual slice t of a block: t = 2*half128 + ab; ab picks ql bytes [32ab, 32ab+32) of the
-    // 128-element half; their low nibbles are elements [32ab, 32ab+32), their high nibbles +64
-    static __device__ __forceinline__ Frag load(const uint8_t* row, int s, int h) {
+    static __device__ __forceinline__ Blk load_blk(const uint8_t* row, int b, int h) {
+        const uint8_t* blk = row + (size_t)b * 210;
+        return Blk{ldu<uint4>(blk + 192), ldu<uint4>(blk + 128 + 16 * h), ldu<uint4>(blk + 160 + 16 * h), ldu<uint16_t>(blk + 208)};
+    }
+    static __device__ __forceinline__ Q load_q(const uint8_t* row, int s, int h) {
         const uint8_t* blk = row + (size_t)(s >> 2) * 210;
+        return Q{ldu<uint4>(blk + 64 * ((s >> 1) & 1) + 32 * (s & 1) + 16 * h)};
+    }
+    static __device__ __forceinline__ Prep prep(const Blk& blk, const Q&, int s, int h) {
+        // the lane's four chunks are 16 consecutive elements: one scale for the low codes
+        // (scales[8hh + 2ab + h]) and one for the high codes (+4)
         const int hh = (s >> 1) & 1, ab = s & 1;
-        Frag f;
-        f.l = ldu<uint4>(blk + 64 * hh + 32 * ab + 16 * h);
-        f.hq = ldu<uint4>(blk + 128 + 32 * hh + 16 * h);
-        f.sc_lo = blk[192 + 8 * hh + 2 * ab + h];
-        f.sc_hi = blk[192 + 8 * hh + 2 * ab + 4 + h];
-        f.d = ldu<uint16_t>(blk + 208);
-        return f;
+        const uint32_t w_lo = hh ? blk.sc.z : blk.sc.x, w_hi = hh ? blk.sc.w : blk.sc.y;
+        const int sh = 8 * (2 * ab + h);
+        const float d = f16_bits_to_f32(blk.d);
+        return Prep{splat(d * (float)(int8_t)(w_lo >> sh)), splat(d * (float)(int8_t)(w_hi >> sh))};
     }
-    static __device__ __forceinline__ Prep prep(const Frag& f, int) {
-        const float d = f16_bits_to_f32(f.d);
-        return Prep{splat(d * (float)(int8_t)f.sc_lo), splat(d * (float)(int8_t)f.sc_hi)};
-    }
-    static __device__ __forceinline__ uint4 chunk(const Frag& f, const Prep& c, int ks, int s) {
+    static __device__ __forceinline__ uint4 chunk(const Blk& blk, const Q& f, const Prep& c, int ks, int s) {
         const int sh = 2 * (s & 1);  // qh bits sh..sh+1 complete the low codes, sh+4.. the high codes
+        const uint4& hq = ((s >> 1) & 1) ? blk.hq1 : blk.hq0;
         const uint32_t L = ks == 0 ? f.l.x : ks == 1 ? f.l.y : ks == 2 ? f.l.z : f.l.w;
-        const uint32_t H = (ks == 0 ? f.hq.x : ks == 1 ? f.hq.y : ks == 2 ? f.hq.z : f.hq.w) >> sh;
+        const uint32_t H = (ks == 0 ? hq.x : ks == 1 ? hq.y : ks == 2 ? hq.z : hq.w) >> sh;
         const uint32_t a = (L & 0x000F000Fu) | ((H & 0x00030003u) << 4) | 0x64006400u;
         const uint32_t b = ((L >> 8) & 0x000F000Fu) | (((H >> 8) & 0x00030003u) << 4) | 0x64006400u;
         const uint32_t g = ((L >> 4) & 0x000F000Fu) | (H & 0x00300030u) | 0x64006400u;
@@ -156,19 +171,21 @@ struct MQ6K {
 
 struct MQ80 {
     static constexpr int kDt = INFR_Q8_0, kBlockElems = 32, kBlockBytes = 34;
-    struct Frag {
+    struct Blk {};
+    struct Q {
         uint4 qa, qb;  // the 32 codes of block h of the slice
         uint32_t d;
     };
     struct Prep {
         half2v d;
     };
-    static __device__ __forceinline__ Frag load(const uint8_t* row, int s, int h) {
+    static __device__ __forceinline__ Blk load_blk(const uint8_t*, int, int) { return Blk{}; }
+    static __device__ __forceinline__ Q load_q(const uint8_t* row, int s, int h) {
         const uint8_t* p = row + (size_t)s * 68 + 34 * h;
-        return Frag{ldu<uint4>(p + 2), ldu<uint4>(p + 18), ldu<uint16_t>(p)};
+        return Q{ldu<uint4>(p + 2), ldu<uint4>(p + 18), ldu<uint16_t>(p)};
     }
-    static __device__ __forceinline__ Prep prep(const Frag& f, int) { return Prep{splat(f16_bits_to_f32(f.d))}; }
-    static __device__ __forceinline__ uint4 chunk(const Frag& f, const Prep& c, int ks) {
+    static __device__ __forceinline__ Prep prep(const Blk&, const Q& f, int, int) { return Prep{splat(f16_bits_to_f32(f.d))}; }
+    static __device__ __forceinline__ uint4 chunk(const Blk&, const Q& f, const Prep& c, int ks, int) {
         const uint32_t v0 = ks == 0 ? f.qa.x : ks == 1 ? f.qa.z : ks == 2 ? f.qb.x : f.qb.z;
         const uint32_t v1 = ks == 0 ? f.qa.y : ks == 1 ? f.qa.w : ks == 2 ? f.qb.y : f.qb.w;
         // bytes (b0,b1) and (b2,b3) to the low bytes of the two halves; x ^ 0x80 = x + 128 as unsigned
@@ -185,12 +202,6 @@ struct MQ80 {
         swz = false;
     }
 };
-
-template <class F>
-__device__ __forceinline__ uint4 fmt_chunk(const typename F::Frag& f, const typename F::Prep& c, int ks, int s) {
-    if constexpr (F::kDt == INFR_Q6K) return F::chunk(f, c, ks, s);
-    else return F::chunk(f, c, ks);
-}
 
 // --------------------------------------------------------------------------------------------
 // One block per row: amax -> power-of-two scale -> f16 in the virtual k order of format F.
@@ -433,13 +444,17 @@ __device__ __forceinline__ void grouped_tile(const GroupedParams& p, const Group
     const int last = n_slices - 1;
     const uint4* fa = c.sA + (lane & 31) + 4 * half * kAStride;
 
-    // rings (named variables, so that they stay in registers): weights of slices s..s+3 in
-    // wa/wb/wc/wd by s % 4, activation chunks of slices s+1, s+2 in ae (even slice) / ao (odd)
+    // rings (named variables, so that they stay in registers): code bytes of slices s..s+3 in
+    // qa/qb/qc/qd by s % 4, the per-256 parts of the current and of the next 256-element step,
+    // activation chunks of slices s+1, s+2 in ae (even slice) / ao (odd)
     static_assert(kWRing == 4 && kARing == 2 && kUnroll == 4, "the slice loop below is written for these depths");
-    typename F::Frag wa0 = F::load(c.wrow0, 0, half), wa1 = F::load(c.wrow1, 0, half);
-    typename F::Frag wb0 = F::load(c.wrow0, min(1, last), half), wb1 = F::load(c.wrow1, min(1, last), half);
-    typename F::Frag wc0 = F::load(c.wrow0, min(2, last), half), wc1 = F::load(c.wrow1, min(2, last), half);
-    typename F::Frag wd0 = F::load(c.wrow0, min(3, last), half), wd1 = F::load(c.wrow1, min(3, last), half);
+    const int last_blk = last >> 2;
+    typename F::Blk bc0 = F::load_blk(c.wrow0, 0, half), bc1 = F::load_blk(c.wrow1, 0, half);
+    typename F::Blk bn0 = F::load_blk(c.wrow0, min(1, last_blk), half), bn1 = F::load_blk(c.wrow1, min(1, last_blk), half);
+    typename F::Q qa0 = F::load_q(c.wrow0, 0, half), qa1 = F::load_q(c.wrow1, 0, half);
+    typename F::Q qb0 = F::load_q(c.wrow0, 1, half), qb1 = F::load_q(c.wrow1, 1, half);
+    typename F::Q qc0 = F::load_q(c.wrow0, 2, half), qc1 = F::load_q(c.wrow1, 2, half);
+    typename F::Q qd0 = F::load_q(c.wrow0, 3, half), qd1 = F::load_q(c.wrow1, 3, half);
     const uint4 *as0 = c.asrc[0], *as1 = c.asrc[1], *as2 = c.asrc[2], *as3 = c.asrc[3];
     struct A4 {
         uint4 q0, q1, q2, q3;
@@ -459,15 +474,15 @@ __device__ __forceinline__ void grouped_tile(const GroupedParams& p, const Group
         d[96] = a4.q3;
         a4 = load_a(s + kARing);
     };
-    // contracts slice s from LDS buffer s & 1 with the fragments in (f0, f1), stages slice s + 1,
-    // refills the fragments with slice s + kWRing
-    auto slice = [&](int s, typename F::Frag& f0, typename F::Frag& f1, A4& a_next) {
+    // contracts slice s from LDS buffer s & 1 with the code bytes in (f0, f1), stages slice s + 1,
+    // refills the code bytes with slice s + kWRing
+    auto slice = [&](int s, typename F::Q& f0, typename F::Q& f1, A4& a_next) {
         const uint4* ap = fa + (s & 1) * kABuf;
-        const typename F::Prep c0 = F::prep(f0, s), c1 = F::prep(f1, s);
+        const typename F::Prep c0 = F::prep(bc0, f0, s, half), c1 = F::prep(bc1, f1, s, half);
         // software pipeline over the four k-steps: as soon as the two matrix instructions that
         // use activation fragment mi are issued, the fragment register is reloaded for step
         // ks + 1, and the unpacking of step ks + 1's weight chunks is spread between them
-        uint4 b0 = fmt_chunk<F>(f0, c0, 0, s), b1 = fmt_chunk<F>(f1, c1, 0, s);
+        uint4 b0 = F::chunk(bc0, f0, c0, 0, s), b1 = F::chunk(bc1, f1, c1, 0, s);
         uint4 a[M];
 #pragma unroll
         for (int mi = 0; mi < M; mi++) a[mi] = ap[mi * 32];
@@ -475,12 +490,12 @@ __device__ __forceinline__ void grouped_tile(const GroupedParams& p, const Group
         for (int ks = 0; ks < 4; ks++) {
             uint4 nb0 = b0, nb1 = b1;
             if (ks < 3) {
-                nb0 = fmt_chunk<F>(f0, c0, ks + 1, s);
-                nb1 = fmt_chunk<F>(f1, c1, ks + 1, s);
+                nb0 = F::chunk(bc0, f0, c0, ks + 1, s);
+                nb1 = F::chunk(bc1, f1, c1, ks + 1, s);
             } else {
                 stage(s + 1, a_next);
-                f0 = F::load(c.wrow0, min(s + kWRing, last), half);
-                f1 = F::load(c.wrow1, min(s + kWRing, last), half);
+                f0 = F::load_q(c.wrow0, min(s + kWRing, last), half);
+                f1 = F::load_q(c.wrow1, min(s + kWRing, last), half);
             }
 #pragma unroll
             for (int mi = 0; mi < M; mi++) {
@@ -497,14 +512,18 @@ __device__ __forceinline__ void grouped_tile(const GroupedParams& p, const Group
     stage(0, ae);
     __syncthreads();
     for (int s0 = 0; s0 < n_slices; s0 += kUnroll) {
-        slice(s0, wa0, wa1, ao);
+        slice(s0, qa0, qa1, ao);
         __syncthreads();
-        slice(s0 + 1, wb0, wb1, ae);
+        slice(s0 + 1, qb0, qb1, ae);
         __syncthreads();
-        slice(s0 + 2, wc0, wc1, ao);
+        slice(s0 + 2, qc0, qc1, ao);
         __syncthreads();
-        slice(s0 + 3, wd0, wd1, ae);
+        slice(s0 + 3, qd0, qd1, ae);
         __syncthreads();
+        bc0 = bn0;
+        bc1 = bn1;
+        bn0 = F::load_blk(c.wrow0, min((s0 >> 2) + 2, last_blk), half);
+        bn1 = F::load_blk(c.wrow1, min((s0 >> 2) + 2, last_blk), half);
     }
 
     // accumulator register r of a 32x32 tile: row 8*(r/4) + 4*(lane/32) + r%4, column lane%32
