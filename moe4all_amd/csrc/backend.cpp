@@ -45,6 +45,9 @@ constexpr uint64_t kPlanMagic = 0x494e4652504c414eull;     // "INFRPLAN"
 // Token rows from which Op::MoeFfn buckets tokens by expert and runs grouped GEMMs on the matrix
 // cores (f16 operands, f32 accumulation) instead of one GEMV pass per token row.
 constexpr uint32_t kBatchedMinRows = 32;
+// Token rows from which a decode batch is bucketed by expert so that each selected expert's rows are
+// read from HBM once (same f32-accurate inner product as the per-token kernels).
+constexpr uint32_t kBucketedMinRows = 16;
 
 bool geometry(int dtype, int* elems, int* bytes) {
     switch (dtype) {
@@ -88,7 +91,8 @@ struct MoeScratch {
     float* h = nullptr;       // [rows, n_used, nff] (bucket order on the batched path); shared by all ops of a plan
     int rows = 0;
     // batched path (bucketing + grouped GEMMs); the large buffers are shared by all ops of a plan
-    bool batched = false;
+    bool batched = false;    // >= kBatchedMinRows: grouped GEMMs on the matrix cores
+    bool bucketed = false;   // kBucketedMinRows .. : f32-accurate GEMV per (expert, bucket), weights read once per expert
     int32_t* offsets = nullptr;   // [n_expert + 1]
     int32_t* pair_src = nullptr;  // [rows * n_used]
     int32_t* slot_pair = nullptr; // [rows * n_used]
@@ -544,9 +548,25 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
                               round_up(pairs * m.n_ff_exp * 2, 256) + round_up(pairs * 4, 256) +
                               round_up(pairs * m.ne * 4, 256);
                 }
+                bool bucketed = false;
+                if (!batched && rows >= kBucketedMinRows && m.n_used <= 64) {
+                    infr::MoeGemvParams probe{};
+                    probe.gate_dt = c.dt(m.gate_exps);
+                    probe.up_dt = m.fused_gate_up ? probe.gate_dt : c.dt(m.up_exps);
+                    probe.down_dt = c.dt(m.down_exps);
+                    probe.fused_gate_up = (int)m.fused_gate_up;
+                    probe.ne = (int)m.ne;
+                    probe.nff = (int)m.n_ff_exp;
+                    bucketed = infr::moe_bucketed_supported(probe);
+                }
+                if (bucketed) {
+                    arena += round_up(((size_t)m.n_expert + 2) * 4, 256) + 2 * round_up(pairs * 4 + 4, 256);
+                    shared += round_up(pairs * m.ne * 4, 256);
+                }
                 if (shared > shared_need) shared_need = shared;
                 plan->moe[oi].rows = (int)rows;
                 plan->moe[oi].batched = batched;
+                plan->moe[oi].bucketed = bucketed;
                 break;
             }
             case INFR_OP_LINEAR: {
@@ -641,7 +661,7 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
         s.ids = (int32_t*)p;  p += round_up(rows * m.n_used * 4 + 4, 256);
         s.weights = (float*)p; p += round_up(rows * m.n_used * 4 + 4, 256);
         const size_t pairs = rows * m.n_used;
-        if (s.batched) {
+        if (s.batched || s.bucketed) {
             s.offsets = (int32_t*)p;   p += round_up(((size_t)m.n_expert + 2) * 4, 256);
             s.pair_src = (int32_t*)p;  p += round_up(pairs * 4 + 4, 256);
             s.slot_pair = (int32_t*)p;
@@ -653,6 +673,8 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
             s.xs = (float*)p;    p += round_up(rows * 4, 256);
             s.hh = (_Float16*)p; p += round_up(pairs * m.n_ff_exp * 2, 256);
             s.hs = (float*)p;    p += round_up(pairs * 4, 256);
+            s.y = (float*)p;
+        } else if (s.bucketed) {
             s.y = (float*)p;
         }
     }
@@ -814,6 +836,33 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                     }
                     break;
                 }
+                if (sc.bucketed) {
+                    const int pairs = rows * (int)m.n_used;
+                    {
+                        Timed t(be, "route_topk");
+                        infr::launch_route(s, rp);
+                    }
+                    {
+                        Timed t(be, "moe_bucket");
+                        infr::launch_bucket(s, sc.ids, pairs, (int)m.n_expert, sc.offsets, sc.pair_src, sc.slot_pair);
+                    }
+                    gp.bk_offsets = sc.offsets; gp.bk_pair_src = sc.pair_src; gp.y = sc.y;
+                    {
+                        Timed t(be, "moe_gate_up_bucketed");
+                        infr::launch_moe_gate_up_bucketed(s, gp);
+                    }
+                    gp.x = sc.h;
+                    {
+                        Timed t(be, "moe_down_bucketed");
+                        infr::launch_moe_down_bucketed(s, gp);
+                    }
+                    {
+                        Timed t(be, "moe_unbucket_combine");
+                        infr::launch_unbucket_combine(s, sc.y, sc.slot_pair, sc.weights, rows, (int)m.ne, (int)m.n_used,
+                                                      (int)m.weight_before, gp.dst, 1);
+                    }
+                    break;
+                }
                 gp.route = rp;
                 gp.route_inline = infr::moe_gate_up_routes_inline(gp) ? 1 : 0;
                 if (!gp.route_inline) {
@@ -935,7 +984,7 @@ extern "C" infr_status infr_hip_plan_moe_bucketing(infr_hip_backend* be, const i
         return fail(INFR_ERR_INVALID, "moe_bucketing: op %u is not a MoeFfn", op_index);
     const infr_op_moe_ffn& m = plan->ops[op_index].u.moe_ffn;
     const MoeScratch& sc = plan->moe[op_index];
-    if (!sc.batched)
+    if (!sc.batched && !sc.bucketed)
         return fail(INFR_ERR_INVALID, "moe_bucketing: op %u runs the per-token path (%d rows), which does not bucket", op_index, sc.rows);
     std::lock_guard<std::mutex> lk(be->mu);
     HIP_TRY(hipSetDevice(be->device));

@@ -714,6 +714,217 @@ void launch_moe_down_combine(hipStream_t s, const MoeGemvParams& p) {
     INFR_LAUNCH(moe_down_combine_generic, grid, block, 0, s, p, row_bytes_of(p.down_dt, p.nff));
 }
 
+// ------------------------------------------------------------------------------- bucketed batches
+// Decode batches of several token rows: grid.x = tiles of `ft` features (gate/up) or `ot` output
+// rows (down), grid.y = expert, grid.z = chunk of T tokens of the expert's bucket.  A block stages
+// the activations of its T tokens once (all waves share the cells), then every weight row of its
+// tile is loaded once and dotted with each of them.  Same inner product as the per-token kernels,
+// so the results are the same bits whichever path a batch takes.
+template <class F, int T>
+__device__ __forceinline__ void stage_tokens(const float* const (&rows)[T], int nt, int n, uint32_t* cells,
+                                             size_t cell_words) {
+    const int ncell = (n + 31) / 32;
+    for (int idx = threadIdx.x; idx < T * ncell; idx += 256) {
+        const int tau = idx / ncell, c0 = idx - tau * ncell;
+        if (tau < nt) {
+            const XLoad l = stage_x_load(rows[tau], n, c0);
+            stage_x_convert<F::kGroup, F::kSigned>(l, n, c0, cells + (size_t)tau * cell_words);
+        }
+    }
+    __syncthreads();
+}
+
+template <class F, int U, int T>
+__global__ __launch_bounds__(256) void moe_gate_up_bucketed(MoeGemvParams p, int ft) {
+    extern __shared__ uint32_t dyn_lds[];
+    __shared__ uint64_t s_tab[32];
+    __shared__ float s_g[4][T][64], s_u[4][T][64];
+    const int e = blockIdx.y;
+    const int t0 = p.bk_offsets[e] + blockIdx.z * T, t1 = p.bk_offsets[e + 1];
+    if (t0 >= t1) return;
+    const int nt = min(T, t1 - t0);
+    const int f0 = blockIdx.x * ft;
+    const int fcount = min(ft, p.nff - f0);
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int nblk = p.ne / F::kBlockElems;
+    const size_t row_bytes = (size_t)nblk * F::kBlockBytes;
+    const Place<F> pl(nblk, lane);
+    const size_t cell_words = (size_t)((p.ne + 31) / 32) * kCellDwords;
+    if (threadIdx.x < 32) s_tab[threadIdx.x] = kExp2Table[threadIdx.x];
+    int pair[T];
+    const float* xrows[T];
+#pragma unroll
+    for (int tau = 0; tau < T; tau++) {
+        pair[tau] = p.bk_pair_src[t0 + min(tau, nt - 1)];
+        xrows[tau] = p.x + (size_t)(pair[tau] / p.n_used) * p.ne;
+    }
+    const uint8_t* gbank = p.gate + (size_t)e * p.gate_stride + (size_t)f0 * row_bytes;
+    const uint8_t* ubank = p.up + (size_t)e * p.up_stride + (size_t)f0 * row_bytes;
+    const int per_round = 4 * pl.rw_count;
+    // the first round of weight rows is requested before the activations are staged
+    typename F::Raw graw[U], uraw[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const int f = min((u * 4 + wave) * pl.rw_count + pl.rw, fcount - 1);
+        graw[u] = load_row<F>(pl, gbank + (size_t)f * row_bytes);
+        uraw[u] = load_row<F>(pl, ubank + (size_t)f * row_bytes);
+    }
+    stage_tokens<F, T>(xrows, nt, p.ne, dyn_lds, cell_words);
+    typename F::X x[T];
+#pragma unroll
+    for (int tau = 0; tau < T; tau++) F::fetch_x(x[tau], dyn_lds + (size_t)min(tau, nt - 1) * cell_words, pl.blk, pl.sub);
+    for (int base = 0; base < fcount; base += per_round * U) {
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+#pragma unroll
+            for (int tau = 0; tau < T; tau++) {
+                float gs = row_sum<F>(F::dot(graw[u], pl.sub, x[tau]), pl, nblk);
+                float us = row_sum<F>(F::dot(uraw[u], pl.sub, x[tau]), pl, nblk);
+                if (pl.writer()) {
+                    s_g[wave][tau][u * pl.rw_count + pl.rw] = gs;
+                    s_u[wave][tau][u * pl.rw_count + pl.rw] = us;
+                }
+            }
+        }
+        // next round's rows are in flight while this round's activations are applied
+        if (base + per_round * U < fcount) {
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                const int f = min(base + per_round * U + (u * 4 + wave) * pl.rw_count + pl.rw, fcount - 1);
+                graw[u] = load_row<F>(pl, gbank + (size_t)f * row_bytes);
+                uraw[u] = load_row<F>(pl, ubank + (size_t)f * row_bytes);
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+        if (lane < U * pl.rw_count) {
+            const int u = lane / pl.rw_count, rw = lane - u * pl.rw_count;
+            const int f = base + (u * 4 + wave) * pl.rw_count + rw;
+            if (f < fcount) {
+#pragma unroll
+                for (int tau = 0; tau < T; tau++) {
+                    if (tau >= nt) break;
+                    float gs = s_g[wave][tau][lane], us = s_u[wave][tau][lane];
+                    if (p.weight_before) {
+                        const float wp = p.weights[pair[tau]];
+                        gs = __fmul_rn(wp, gs);
+                        us = __fmul_rn(wp, us);
+                    }
+                    p.h[(size_t)pair[tau] * p.nff + f0 + f] = gated_act_fn(p.act, p.has_clamp, p.clamp, gs, us, s_tab);
+                }
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+}
+
+template <class F, int U, int T>
+__global__ __launch_bounds__(256) void moe_down_bucketed(MoeGemvParams p, int ot) {
+    extern __shared__ uint32_t dyn_lds[];
+    const int e = blockIdx.y;
+    const int t0 = p.bk_offsets[e] + blockIdx.z * T, t1 = p.bk_offsets[e + 1];
+    if (t0 >= t1) return;
+    const int nt = min(T, t1 - t0);
+    const int o0 = blockIdx.x * ot;
+    const int ocount = min(ot, p.ne - o0);
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int nblk = p.nff / F::kBlockElems;
+    const size_t row_bytes = (size_t)nblk * F::kBlockBytes;
+    const Place<F> pl(nblk, lane);
+    const uint8_t* bank = p.down + (size_t)e * p.down_stride + (size_t)o0 * row_bytes;
+    const int per_round = 4 * pl.rw_count;
+    const size_t cell_words = (size_t)((p.nff + 31) / 32) * kCellDwords;
+    const float ds = p.down_scale ? p.down_scale[e] : 1.0f;
+    int pair[T];
+    const float* xrows[T];
+#pragma unroll
+    for (int tau = 0; tau < T; tau++) {
+        pair[tau] = p.bk_pair_src[t0 + min(tau, nt - 1)];
+        xrows[tau] = p.x + (size_t)pair[tau] * p.nff;   // h of the pair
+    }
+    typename F::Raw raw[U];
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const int o = min((u * 4 + wave) * pl.rw_count + pl.rw, ocount - 1);
+        raw[u] = load_row<F>(pl, bank + (size_t)o * row_bytes);
+    }
+    stage_tokens<F, T>(xrows, nt, p.nff, dyn_lds, cell_words);
+    typename F::X x[T];
+#pragma unroll
+    for (int tau = 0; tau < T; tau++) F::fetch_x(x[tau], dyn_lds + (size_t)min(tau, nt - 1) * cell_words, pl.blk, pl.sub);
+    for (int base = 0; base < ocount; base += per_round * U) {
+        float y[U][T];
+#pragma unroll
+        for (int u = 0; u < U; u++)
+#pragma unroll
+            for (int tau = 0; tau < T; tau++) y[u][tau] = row_sum<F>(F::dot(raw[u], pl.sub, x[tau]), pl, nblk);
+        const int base_next = base + per_round * U;
+        typename F::Raw nxt[U];
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int o = min(base_next + (u * 4 + wave) * pl.rw_count + pl.rw, ocount - 1);
+            nxt[u] = load_row<F>(pl, bank + (size_t)o * row_bytes);
+        }
+#pragma unroll
+        for (int u = 0; u < U; u++) {
+            const int o = base + (u * 4 + wave) * pl.rw_count + pl.rw;
+#pragma unroll
+            for (int tau = 0; tau < T; tau++) {
+                float v = y[u][tau];
+                if (p.down_scale) v = __fmul_rn(v, ds);
+                if (o < ocount && tau < nt && pl.writer()) p.y[(size_t)pair[tau] * p.ne + o0 + o] = v;
+            }
+            raw[u] = nxt[u];
+        }
+    }
+}
+
+constexpr int kBucketT = 2;   // tokens a block of the bucketed kernels handles together
+
+template <class F>
+static void gate_up_bucketed(hipStream_t s, const MoeGemvParams& p) {
+    const int rw = 64 / (p.ne / F::kBlockElems * F::kLPB);
+    // about four blocks per CU if every expert had one chunk of tokens
+    int tiles = max(1, 4 * p.n_cu / max(p.n_expert, 1));
+    int ft = ceil_div(p.nff, tiles);
+    ft = ceil_div(ft, 4 * rw) * 4 * rw;
+    dim3 grid(ceil_div(p.nff, ft), p.n_expert, ceil_div(p.rows, kBucketT)), block(256);
+    INFR_LAUNCH((moe_gate_up_bucketed<F, 2, kBucketT>), grid, block, kBucketT * cells_bytes(p.ne), s, p, ft);
+}
+
+template <class F>
+static void down_bucketed(hipStream_t s, const MoeGemvParams& p) {
+    const int rw = 64 / (p.nff / F::kBlockElems * F::kLPB);
+    int tiles = max(1, 4 * p.n_cu / max(p.n_expert, 1));
+    int ot = ceil_div(p.ne, tiles);
+    ot = ceil_div(ot, 4 * rw) * 4 * rw;
+    dim3 grid(ceil_div(p.ne, ot), p.n_expert, ceil_div(p.rows, kBucketT)), block(256);
+    INFR_LAUNCH((moe_down_bucketed<F, 4, kBucketT>), grid, block, kBucketT * cells_bytes(p.nff), s, p, ot);
+}
+
+bool moe_bucketed_supported(const MoeGemvParams& p) {
+    if (p.gate_dt != p.up_dt || p.fused_gate_up) return false;
+    auto ok = [](int dt, int k) {
+        if (kBucketT * cells_bytes(k) > 48 * 1024) return false;   // the staged cells must fit the default LDS window
+        if (dt == INFR_Q4K) return fast_ok<Q4KFmt>(k);
+        if (dt == INFR_Q6K) return fast_ok<Q6KFmt>(k);
+        if (dt == INFR_Q8_0) return fast_ok<Q80Fmt>(k);
+        return false;
+    };
+    return ok(p.gate_dt, p.ne) && ok(p.down_dt, p.nff);
+}
+
+void launch_moe_gate_up_bucketed(hipStream_t s, const MoeGemvParams& p) {
+    if (p.gate_dt == INFR_Q4K) gate_up_bucketed<Q4KFmt>(s, p);
+    else if (p.gate_dt == INFR_Q6K) gate_up_bucketed<Q6KFmt>(s, p);
+    else gate_up_bucketed<Q80Fmt>(s, p);
+}
+
+void launch_moe_down_bucketed(hipStream_t s, const MoeGemvParams& p) {
+    if (p.down_dt == INFR_Q4K) down_bucketed<Q4KFmt>(s, p);
+    else if (p.down_dt == INFR_Q6K) down_bucketed<Q6KFmt>(s, p);
+    else down_bucketed<Q80Fmt>(s, p);
+}
+
 // ------------------------------------------------------------------------------- Op::Linear
 // dst[m, out_f] = x . W^T, the dense neighbour of the expert GEMVs (shared expert).
 template <class F>

@@ -614,14 +614,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 __global__ __launch_bounds__(256) void unbucket_combine_kernel(const float* __restrict__ y,
                                                                const int32_t* __restrict__ slot_pair,
                                                                const float* __restrict__ weights, int ne, int n_used,
-                                                               int weight_before, float* __restrict__ dst) {
+                                                               int weight_before, float* __restrict__ dst, int identity) {
     const size_t row = blockIdx.y;
     const int i = (blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= ne) return;
     float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
     for (int k = 0; k < n_used; k++) {
-        const int pr = slot_pair[row * n_used + k];
+        int pr = slot_pair[row * n_used + k];
         if (pr < 0) continue;
+        if (identity) pr = (int)(row * n_used + k);
         const float w = weight_before ? 1.0f : weights[row * n_used + k];
         const float* yr = y + (size_t)pr * ne + i;
         if (i + 3 < ne) {
@@ -697,10 +698,10 @@ void launch_grouped_down(hipStream_t s, int dt, const GroupedParams& p) {
 }
 
 void launch_unbucket_combine(hipStream_t s, const float* y, const int32_t* slot_pair, const float* weights, int rows,
-                             int ne, int n_used, int weight_before, float* dst) {
+                             int ne, int n_used, int weight_before, float* dst, int identity) {
     if (rows <= 0) return;
     INFR_LAUNCH(unbucket_combine_kernel, dim3((ne + 1023) / 1024, rows), dim3(256), 0, s, y, slot_pair, weights, ne, n_used,
-                weight_before, dst);
+                weight_before, dst, identity);
 }
 
 }  // namespace infr

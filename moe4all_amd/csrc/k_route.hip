@@ -59,7 +59,8 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const uint8_t* __res
     // block, activations included, is issued before the first LDS store, so the block pays the
     // memory latency once.
     const int nv = ne >> 2;
-    const bool one_shot = rdt == INFR_F32 && (ne & 3) == 0 && gridDim.y == 1 && rows <= rpb && EPB * nv <= 8 * 256 &&
+    const int rbase = blockIdx.y * rpb;   // first token row of this block's (only) pass when one_shot
+    const bool one_shot = rdt == INFR_F32 && (ne & 3) == 0 && (int)gridDim.y * rpb >= rows && EPB * nv <= 8 * 256 &&
                           rpb * nv <= 4 * 256;
     if (one_shot) {
         float4 wr[8], xr[4];
@@ -67,7 +68,7 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const uint8_t* __res
         for (int i = 0; i < 4; i++) {
             const int idx = tid + 256 * i, rr = idx / nv, v = idx - rr * nv;
             xr[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (rr < rows) xr[i] = reinterpret_cast<const float4*>(x + (size_t)rr * ne)[v];
+            if (rr < rpb && rbase + rr < rows) xr[i] = reinterpret_cast<const float4*>(x + (size_t)(rbase + rr) * ne)[v];
         }
 #pragma unroll
         for (int i = 0; i < 8; i++) {
@@ -258,15 +259,17 @@ __global__ __launch_bounds__(512) void router_logits_tiled_kernel(const float* _
 
 bool launch_router_logits(hipStream_t s, const uint8_t* router, int rdt, size_t row_bytes, const float* x, int ne,
                           int n_expert, int rows, float* logits) {
-    if (rows >= 16 && rdt == INFR_F32 && (ne & 31) == 0 && (row_bytes & 15) == 0) {
+    if (rows >= 32 && rdt == INFR_F32 && (ne & 31) == 0 && (row_bytes & 15) == 0) {
         dim3 grid((n_expert + kLtTile - 1) / kLtTile, (rows + kLtTile - 1) / kLtTile);
         INFR_LAUNCH(router_logits_tiled_kernel, grid, dim3(512), 0, s, reinterpret_cast<const float*>(router), row_bytes / 4,
                     x, ne, n_expert, rows, logits);
         return true;
     }
-    // Decode (few rows): many small blocks.  Batches: 8 experts x 4 rows per pass.
-    int epb = rows <= 2 ? 2 : 8;
-    int rpb = rows <= 2 ? rows : 4;
+    // Decode and small batches of an f32 router: many small blocks of 2 experts x 2 rows, each
+    // staging its operands with one burst of loads.  Otherwise: 8 experts x 4 rows per pass.
+    const bool small = rows <= 2 || (rows < 32 && rdt == INFR_F32 && (ne & 3) == 0 && ne <= 4096);
+    int epb = small ? 2 : 8;
+    int rpb = small ? ((rows < 2 || ne > 2048) ? 1 : 2) : 4;   // the one-burst staging holds 1024 float4 of activations
     const size_t budget = 140 * 1024;
     const int nc = ne >> 3;
     const size_t estride = (size_t)8 * (((nc + 63) & ~63) + 4);
@@ -278,7 +281,7 @@ bool launch_router_logits(hipStream_t s, const uint8_t* router, int rdt, size_t 
     int gx = (n_expert + epb - 1) / epb;
     int passes = (rows + rpb - 1) / rpb;
     int gy = passes;
-    int cap = (1024 + gx - 1) / gx;
+    int cap = small ? passes : (1024 + gx - 1) / gx;
     if (gy > cap) gy = cap;
     if (gy < 1) gy = 1;
     dim3 grid(gx, gy), block(256);

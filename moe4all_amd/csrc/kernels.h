@@ -65,6 +65,10 @@ struct MoeGemvParams {
     // redundantly; block 0 of a row publishes ids / weights / probs) and no route launch is needed.
     int route_inline;
     RouteParams route;
+    // bucketed decode batches (launch_moe_*_bucketed): pairs grouped by expert
+    const int32_t* bk_offsets;   // [n_expert + 1]
+    const int32_t* bk_pair_src;  // [rows * n_used] flat (row * n_used + rank) in bucket order
+    float* y;                    // [rows * n_used, ne] per-pair down outputs, flat pair order
 };
 // True when launch_moe_gate_up will take the kernel that can route inline.
 bool moe_gate_up_routes_inline(const MoeGemvParams& p);
@@ -97,8 +101,16 @@ void launch_bucket(hipStream_t s, const int32_t* ids, int n_pairs, int n_expert,
                    int32_t* slot_pair);
 void launch_grouped_gate_up(hipStream_t s, int dt, const GroupedParams& p);
 void launch_grouped_down(hipStream_t s, int dt, const GroupedParams& p);
+// identity != 0: y is in flat (row, rank) order and slot_pair only flags invalid pairs (< 0).
 void launch_unbucket_combine(hipStream_t s, const float* y, const int32_t* slot_pair, const float* weights, int rows,
-                             int ne, int n_used, int weight_before, float* dst);
+                             int ne, int n_used, int weight_before, float* dst, int identity = 0);
+
+// Decode batches with weight reuse: one block per (feature tile, expert) walks the expert's bucket,
+// so an expert's rows are read from HBM once however many token rows selected it.  h and y are in
+// flat (row, rank) order; launch_unbucket_combine with slot_pair_is_flags sums them.
+bool moe_bucketed_supported(const MoeGemvParams& p);
+void launch_moe_gate_up_bucketed(hipStream_t s, const MoeGemvParams& p);
+void launch_moe_down_bucketed(hipStream_t s, const MoeGemvParams& p);
 
 // Standalone decode: out[i] = value of element i (exact reference arithmetic).
 void launch_dequant(hipStream_t s, const uint8_t* src, int dtype, uint64_t numel, float* out);

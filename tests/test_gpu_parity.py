@@ -544,8 +544,37 @@ def test_batched_moe_ffn_option_variants_match_oracle(be):
         assert H.rel_l2(out, ref["dst"]) < REL_L2_MFMA, (gopts, H.rel_l2(out, ref["dst"]))
 
 
+@pytest.mark.parametrize("rows,ne,E,K,nff,gdt,ddt", [
+    (16, 512, 8, 2, 256, H.Q4K, H.Q6K),
+    (19, 256, 16, 4, 256, H.Q6K, H.Q4K),       # experts without tokens, odd bucket sizes
+    (31, 2048, 128, 8, 768, H.Q8_0, H.Q8_0),   # the largest batch below the matrix-core path
+])
+def test_bucketed_decode_batches_bucket_exactly_and_keep_f32_accuracy(be, rows, ne, E, K, nff, gdt, ddt):
+    """16..31 token rows: pairs are bucketed by expert and each expert's rows are read once; the inner
+    product is the per-token kernels', so the f32 bar applies."""
+    rng = np.random.default_rng(rows * 3 + ne)
+    x = rng.standard_normal((rows, ne)).astype(np.float32)
+    router = (rng.standard_normal((E, ne)) * 0.02).astype(np.float32)
+    gate, up = _realistic(rng, E, nff, ne, gdt), _realistic(rng, E, nff, ne, gdt)
+    down = _realistic(rng, E, ne, nff, ddt)
+    ds = rng.uniform(0.5, 1.5, E).astype(np.float32)
+    eids = rng.integers(0, E, (rows, K)).astype(np.int32)
+    base = dict(ne=ne, n_expert=E, n_used=K, n_ff_exp=nff, gate_dtype=gdt, down_dtype=ddt)
+    for gopts, oopts, extra in [({}, {}, {}),
+                                (dict(weight_before=True, with_down_scale=True), dict(weight_before=True, down_scale=ds), dict(down_scale=ds)),
+                                (dict(with_expert_ids=True), dict(expert_ids=eids), dict(expert_ids=eids))]:
+        g, ids = moe_graph(rows, ne, E, K, nff, DType(gdt), DType(ddt), **dict(gopts))
+        out, r, b = _run_batched(be, g, ids, dict(x=x, router=router, gate=gate, up=up, down=down, **extra), rows, ne)
+        ref = O.moe_ffn(x, router, gate, up, down, **base, **oopts)
+        assert np.array_equal(r["idx"], ref["idx"])
+        _check_bucketing(b, ref, E)
+        scale = float(np.abs(ref["dst"]).max())
+        assert H.rel_l2(out, ref["dst"]) < REL_L2, (gopts, H.rel_l2(out, ref["dst"]))
+        assert H.max_abs(out, ref["dst"]) < MAX_ABS * max(1.0, scale)
+
+
 def test_small_batches_keep_the_per_token_path(be):
-    g, ids = moe_graph(16, 256, 8, 2, 256, DType.Q4K, DType.Q6K)
+    g, ids = moe_graph(4, 256, 8, 2, 256, DType.Q4K, DType.Q6K)
     plan = be.compile(g)
     with pytest.raises(M.BackendError):
         be.moe_bucketing(plan, 0)
