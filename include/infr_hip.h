@@ -162,11 +162,12 @@ typedef struct infr_hip_capabilities {
 } infr_hip_capabilities;
 
 typedef struct infr_hip_config {
-    /* 0: let execute() replay a captured HIP graph when a plan is re-run with identical
-     *    bindings; 1: always launch kernels directly. */
+    /* Reserved for HIP-graph replay of a plan that is re-run with identical bindings.  This build
+     * always launches its kernels directly on the backend's stream; the field is ignored. */
     uint32_t disable_graph_replay;
-    /* rows above which Op::MoeFfn takes the bucketed grouped-GEMM path instead of the
-     * per-token GEMV path; 0 selects the built-in default. */
+    /* Token rows from which Op::MoeFfn takes the bucketed grouped-GEMM path on the matrix cores
+     * (f16 operands, f32 accumulation) instead of the f32-accurate GEMV paths; 0 selects the
+     * built-in default (32). */
     uint32_t moe_batched_min_rows;
     uint32_t reserved[6];
 } infr_hip_config;

@@ -234,7 +234,8 @@ extern "C" const char* infr_hip_name(const infr_hip_backend* be) { return ok_bac
 extern "C" infr_status infr_hip_capabilities_get(const infr_hip_backend* be, infr_hip_capabilities* out) {
     if (!ok_backend(be) || !out) return fail(INFR_ERR_INVALID, "capabilities: bad handle");
     memset(out, 0, sizeof *out);
-    snprintf(out->name, sizeof out->name, "hip-gfx950 (%s)", be->prop.name);
+    // some driver stacks report an empty marketing name; the architecture string is always there
+    snprintf(out->name, sizeof out->name, "hip-gfx950 (%s)", be->prop.name[0] ? be->prop.name : be->prop.gcnArchName);
     out->f16 = 1; out->bf16 = 1; out->i8 = 1; out->i8_dot = 1;
     out->subgroup_min = 64; out->subgroup_max = 64;
     out->integrated = 0;

@@ -609,3 +609,29 @@ def test_prefill_chunk_with_skewed_routing_matches_oracle(be, tokens, gdt, ddt):
     assert counts.max() > 4 * max(1, int(np.median(counts))), "routing is not skewed"
     assert H.rel_l2(got, ref["dst"]) < REL_L2_MFMA, H.rel_l2(got, ref["dst"])
     plan.free()
+
+
+def test_batched_threshold_is_configurable_and_the_paths_agree():
+    """moe_batched_min_rows moves the switch to the matrix-core path; with it out of reach a 48-row batch
+    runs the bucketed f32-accurate kernels and must meet the f32 bar, with it at 1 even two rows take
+    the grouped GEMMs; both bucket identically."""
+    rows, ne, E, K, nff = 48, 512, 8, 2, 256
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((rows, ne)).astype(np.float32)
+    router = (rng.standard_normal((E, ne)) * 0.02).astype(np.float32)
+    gate, up = _realistic(rng, E, nff, ne, H.Q4K), _realistic(rng, E, nff, ne, H.Q4K)
+    down = _realistic(rng, E, ne, nff, H.Q6K)
+    ref = O.moe_ffn(x, router, gate, up, down, ne=ne, n_expert=E, n_used=K, n_ff_exp=nff, gate_dtype=H.Q4K, down_dtype=H.Q6K)
+    outs = {}
+    for name, min_rows, bar in (("gemv", 1000, REL_L2), ("mfma", 1, REL_L2_MFMA)):
+        be2 = M.Backend(0, moe_batched_min_rows=min_rows)
+        try:
+            g, ids = moe_graph(rows, ne, E, K, nff, DType.Q4K, DType.Q6K)
+            out, r, b = _run_batched(be2, g, ids, dict(x=x, router=router, gate=gate, up=up, down=down), rows, ne)
+            assert np.array_equal(r["idx"], ref["idx"])
+            _check_bucketing(b, ref, E)
+            assert H.rel_l2(out, ref["dst"]) < bar, (name, H.rel_l2(out, ref["dst"]))
+            outs[name] = out
+        finally:
+            be2.close()
+    assert H.rel_l2(outs["mfma"], outs["gemv"]) < REL_L2_MFMA
