@@ -536,27 +536,33 @@ __device__ __forceinline__ void grouped_tile(const GroupedParams& p, const Group
 #pragma unroll
     for (int mi = 0; mi < M; mi++) {
 #pragma unroll
-        for (int r = 0; r < 16; r++) {
-            const int m = 32 * mi + 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-            const float sc = c.s_scale[m];
-            float* orow = obase + (size_t)m * p.N;
-            if (DOWN) {
-                const float y0 = acc0[mi][r] * sc * ds, y1 = acc1[mi][r] * sc * ds;
-                if (m < t.cnt && fc0 < p.N) orow[fc0] = y0;
-                if (m < t.cnt && fc0 + 32 < p.N) orow[fc0 + 32] = y1;
-            } else if (plain_silu) {
-                // silu(g) * u with the hardware exp and reciprocal
-                const float g = acc0[mi][r] * sc, u = acc1[mi][r] * sc;
-                const float h = g * u * __frcp_rn(1.0f + __expf(-g));
-                if (m < t.cnt && fc0 < p.N) orow[fc0] = h;
-            } else {
-                float g = acc0[mi][r] * sc, u = acc1[mi][r] * sc;
-                if (p.weight_before && m < t.cnt) {
-                    const float wp = p.route_w[p.pair_src[t.p0 + m]];
-                    g *= wp;
-                    u *= wp;
+        for (int r4 = 0; r4 < 4; r4++) {
+            const int m0 = 32 * mi + 8 * r4 + 4 * (lane >> 5);   // rows m0 .. m0 + 3
+            const float4 sc4 = *reinterpret_cast<const float4*>(c.s_scale + m0);
+            const float scs[4] = {sc4.x, sc4.y, sc4.z, sc4.w};
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int r = 4 * r4 + i, m = m0 + i;
+                const float sc = scs[i];
+                float* orow = obase + (size_t)m * p.N;
+                if (DOWN) {
+                    const float y0 = acc0[mi][r] * sc * ds, y1 = acc1[mi][r] * sc * ds;
+                    if (m < t.cnt && fc0 < p.N) orow[fc0] = y0;
+                    if (m < t.cnt && fc0 + 32 < p.N) orow[fc0 + 32] = y1;
+                } else if (plain_silu) {
+                    // silu(g) * u with the hardware exp and reciprocal
+                    const float g = acc0[mi][r] * sc, u = acc1[mi][r] * sc;
+                    const float h = g * u * __frcp_rn(1.0f + __expf(-g));
+                    if (m < t.cnt && fc0 < p.N) orow[fc0] = h;
+                } else {
+                    float g = acc0[mi][r] * sc, u = acc1[mi][r] * sc;
+                    if (p.weight_before && m < t.cnt) {
+                        const float wp = p.route_w[p.pair_src[t.p0 + m]];
+                        g *= wp;
+                        u *= wp;
+                    }
+                    if (m < t.cnt && fc0 < p.N) orow[fc0] = gated_act_fast(p.act, p.has_clamp, p.clamp, g, u);
                 }
-                if (m < t.cnt && fc0 < p.N) orow[fc0] = gated_act_fast(p.act, p.has_clamp, p.clamp, g, u);
             }
         }
     }
@@ -572,41 +578,46 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const int tid = c.tid = threadIdx.x;
     c.wave = tid >> 6;
     c.lane = tid & 63;
-    const int nt = blockIdx.x % p.n_tiles_n;
-    if (!find_tile(p.offsets, p.n_expert, blockIdx.x / p.n_tiles_n, c.lane, c.t)) return;
-    const Tile& t = c.t;
-    constexpr int kBN = DOWN ? 256 : 128;
-    c.n0 = nt * kBN;
+    // one tile per block (a persistent loop over tiles was measured: no faster, and the static
+    // assignment balances the ragged tiles worse than the hardware dispatcher does)
+    {
+        const int item = blockIdx.x;
+        const int nt = item % p.n_tiles_n;
+        if (!find_tile(p.offsets, p.n_expert, item / p.n_tiles_n, c.lane, c.t)) return;
+        const Tile& t = c.t;
+        constexpr int kBN = DOWN ? 256 : 128;
+        c.n0 = nt * kBN;
 
-    // the lane's weight rows
-    const size_t row_bytes = (size_t)(p.K / F::kBlockElems) * F::kBlockBytes;
-    if (DOWN) {
-        const int f0 = min(c.n0 + 64 * c.wave + (c.lane & 31), p.N - 1), f1 = min(c.n0 + 64 * c.wave + 32 + (c.lane & 31), p.N - 1);
-        const uint8_t* base = p.w0 + (size_t)t.e * p.w0_stride;
-        c.wrow0 = base + (size_t)f0 * row_bytes;
-        c.wrow1 = base + (size_t)f1 * row_bytes;
-    } else {
-        const int f = min(c.n0 + 32 * c.wave + (c.lane & 31), p.N - 1);
-        c.wrow0 = p.w0 + (size_t)t.e * p.w0_stride + (size_t)f * row_bytes;
-        c.wrow1 = p.w1 + (size_t)t.e * p.w1_stride + (size_t)f * row_bytes;
-    }
-    // the thread's activation chunks
+        // the lane's weight rows
+        const size_t row_bytes = (size_t)(p.K / F::kBlockElems) * F::kBlockBytes;
+        if (DOWN) {
+            const int f0 = min(c.n0 + 64 * c.wave + (c.lane & 31), p.N - 1), f1 = min(c.n0 + 64 * c.wave + 32 + (c.lane & 31), p.N - 1);
+            const uint8_t* base = p.w0 + (size_t)t.e * p.w0_stride;
+            c.wrow0 = base + (size_t)f0 * row_bytes;
+            c.wrow1 = base + (size_t)f1 * row_bytes;
+        } else {
+            const int f = min(c.n0 + 32 * c.wave + (c.lane & 31), p.N - 1);
+            c.wrow0 = p.w0 + (size_t)t.e * p.w0_stride + (size_t)f * row_bytes;
+            c.wrow1 = p.w1 + (size_t)t.e * p.w1_stride + (size_t)f * row_bytes;
+        }
+        // the thread's activation chunks
 #pragma unroll
-    for (int q = 0; q < 4; q++) {
-        const int cc = tid + 256 * q, tok = cc >> 3, kg = cc & 7;
-        const int pr = t.p0 + min(tok, t.cnt - 1);
-        const size_t src_row = DOWN ? (size_t)pr : (size_t)(p.pair_src[pr] / p.n_used);
-        c.asrc[q] = reinterpret_cast<const uint4*>(p.a + src_row * p.K) + kg;
-    }
-    if (tid < kBM) {
-        const int pr = t.p0 + min(tid, t.cnt - 1);
-        s_scale[tid] = p.a_scale[DOWN ? pr : p.pair_src[pr] / p.n_used];
-    }
-    switch ((t.cnt + 31) >> 5) {
-        case 1: grouped_tile<F, DOWN, 1>(p, c); break;
-        case 2: grouped_tile<F, DOWN, 2>(p, c); break;
-        case 3: grouped_tile<F, DOWN, 3>(p, c); break;
-        default: grouped_tile<F, DOWN, 4>(p, c); break;
+        for (int q = 0; q < 4; q++) {
+            const int cc = tid + 256 * q, tok = cc >> 3, kg = cc & 7;
+            const int pr = t.p0 + min(tok, t.cnt - 1);
+            const size_t src_row = DOWN ? (size_t)pr : (size_t)(p.pair_src[pr] / p.n_used);
+            c.asrc[q] = reinterpret_cast<const uint4*>(p.a + src_row * p.K) + kg;
+        }
+        if (tid < kBM) {
+            const int pr = t.p0 + min(tid, t.cnt - 1);
+            s_scale[tid] = p.a_scale[DOWN ? pr : p.pair_src[pr] / p.n_used];
+        }
+        switch ((t.cnt + 31) >> 5) {
+            case 1: grouped_tile<F, DOWN, 1>(p, c); break;
+            case 2: grouped_tile<F, DOWN, 2>(p, c); break;
+            case 3: grouped_tile<F, DOWN, 3>(p, c); break;
+            default: grouped_tile<F, DOWN, 4>(p, c); break;
+        }
     }
 }
 
