@@ -114,6 +114,16 @@ struct infr_hip_plan {
     size_t arena_bytes = 0;
     std::vector<MoeScratch> moe;       // per op (valid for MoeFfn ops)
     int last_moe_op = -1;
+    // Launch fusion of the dense SwiGLU FFN the reference emits beside the routed experts
+    // (crates/infr-llama/src/runner.rs:8116-8174: Linear gate, Linear up, GatedAct, Linear down, Add).
+    // fuse[i]: what op i does at execute time.
+    enum Fuse : uint8_t { kPlain = 0, kSkip, kGateUpAct, kLinearAdd };
+    struct FuseOp {
+        Fuse kind = kPlain;
+        uint32_t a = 0, b = 0;   // kGateUpAct: index of the up Linear and of the GatedAct; kLinearAdd: index of the Add
+    };
+    std::vector<FuseOp> fuse;
+    int32_t* zero_ids = nullptr;       // [max rows of a fused gate/up] expert id 0 for every row
 };
 
 struct infr_hip_backend {
@@ -646,6 +656,81 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
     const size_t shared_off = arena;
     arena += shared_need;
 
+    // ---- launch fusion: Linear + Linear + GatedAct on one input -> one gate/up kernel; Linear + Add
+    // -> one kernel.  A temporary may disappear only if it is an Internal tensor written once and read
+    // once.  The fused kernels run the same inner products and the same rounding sequence, so the
+    // results are the bits the separate ops give.
+    plan->fuse.assign(g->n_ops, infr_hip_plan::FuseOp{});
+    size_t zero_rows = 0;
+    {
+        std::vector<int> reads(plan->tensors.size(), 0), writes(plan->tensors.size(), 0);
+        auto rd = [&](uint32_t t) { if (t != INFR_NO_TENSOR && t < reads.size()) reads[t]++; };
+        auto wr = [&](uint32_t t) { if (t != INFR_NO_TENSOR && t < writes.size()) writes[t]++; };
+        for (uint32_t oi = 0; oi < g->n_ops; oi++) {
+            const infr_op& op = plan->ops[oi];
+            switch (op.kind) {
+                case INFR_OP_MOE_FFN: {
+                    const infr_op_moe_ffn& m = op.u.moe_ffn;
+                    rd(m.x); rd(m.router_x); rd(m.router); rd(m.gate_exps); rd(m.up_exps); rd(m.down_exps);
+                    rd(m.down_scale); rd(m.exp_probs_b); rd(m.expert_ids); wr(m.dst);
+                    break;
+                }
+                case INFR_OP_LINEAR: rd(op.u.linear.x); rd(op.u.linear.weight); wr(op.u.linear.dst); break;
+                case INFR_OP_GATED_ACT: rd(op.u.gated_act.gate); rd(op.u.gated_act.up); wr(op.u.gated_act.dst); break;
+                case INFR_OP_ADD: rd(op.u.add.a); rd(op.u.add.b); wr(op.u.add.dst); break;
+                case INFR_OP_MOE_SHARED_EXPERT_ADD: {
+                    const infr_op_moe_shared_expert_add& a = op.u.moe_shared_expert_add;
+                    rd(a.moe); rd(a.shexp); rd(a.gate); wr(a.dst);
+                    break;
+                }
+                default: break;
+            }
+        }
+        auto temp = [&](uint32_t t) {
+            return plan->tensors[t].kind == INFR_KIND_INTERNAL && reads[t] == 1 && writes[t] == 1;
+        };
+        for (uint32_t oi = 0; oi + 1 < g->n_ops; oi++) {
+            if (plan->fuse[oi].kind != infr_hip_plan::kPlain || plan->ops[oi].kind != INFR_OP_LINEAR) continue;
+            const infr_op_linear& l1 = plan->ops[oi].u.linear;
+            if (l1.m == 0) continue;
+            // Linear, Linear, GatedAct
+            if (oi + 2 < g->n_ops && plan->ops[oi + 1].kind == INFR_OP_LINEAR && plan->ops[oi + 2].kind == INFR_OP_GATED_ACT) {
+                const infr_op_linear& l2 = plan->ops[oi + 1].u.linear;
+                const infr_op_gated_act& ga = plan->ops[oi + 2].u.gated_act;
+                const bool gate_first = ga.gate == l1.dst && ga.up == l2.dst, up_first = ga.gate == l2.dst && ga.up == l1.dst;
+                infr::MoeGemvParams probe{};
+                probe.gate_dt = probe.up_dt = c.dt(l1.weight);
+                probe.ne = (int)l1.in_f;
+                probe.n_used = 1;
+                if ((gate_first || up_first) && l1.x == l2.x && l1.m == l2.m && l1.in_f == l2.in_f && l1.out_f == l2.out_f &&
+                    l1.w_off == 0 && l2.w_off == 0 && l1.dst != l2.dst && c.dt(l1.weight) == c.dt(l2.weight) &&
+                    temp(l1.dst) && temp(l2.dst) && ga.rows == l1.m && ga.nff == l1.out_f && ga.up_off == 0 &&
+                    ga.gate_block_width == 0 && (ga.up_stride == 0 || ga.up_stride == ga.nff) &&
+                    (ga.gate_stride == 0 || ga.gate_stride == ga.nff) && ga.dst != l1.x &&
+                    infr::moe_gate_up_routes_inline(probe)) {
+                    plan->fuse[oi].kind = infr_hip_plan::kGateUpAct;
+                    plan->fuse[oi].a = gate_first ? oi + 1 : oi;       // the up Linear
+                    plan->fuse[oi].b = oi + 2;
+                    plan->fuse[oi + 1].kind = plan->fuse[oi + 2].kind = infr_hip_plan::kSkip;
+                    if (l1.m > zero_rows) zero_rows = l1.m;
+                    continue;
+                }
+            }
+            // Linear, Add
+            if (plan->ops[oi + 1].kind == INFR_OP_ADD && plan->fuse[oi + 1].kind == infr_hip_plan::kPlain) {
+                const infr_op_add& ad = plan->ops[oi + 1].u.add;
+                const bool is_b = ad.b == l1.dst && ad.a != l1.dst, is_a = ad.a == l1.dst && ad.b != l1.dst;
+                if ((is_a || is_b) && temp(l1.dst) && (uint64_t)ad.n == (uint64_t)l1.m * l1.out_f && ad.dst != l1.x) {
+                    plan->fuse[oi].kind = infr_hip_plan::kLinearAdd;
+                    plan->fuse[oi].a = oi + 1;
+                    plan->fuse[oi + 1].kind = infr_hip_plan::kSkip;
+                }
+            }
+        }
+    }
+    const size_t zero_off = arena;
+    arena += round_up(zero_rows * 4 + 4, 256);
+
     std::lock_guard<std::mutex> lk(be->mu);
     hipError_t e = hipSetDevice(be->device);
     if (e == hipSuccess && arena) e = hipMalloc(&plan->arena, arena);
@@ -679,6 +764,7 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
             s.y = (float*)p;
         }
     }
+    plan->zero_ids = (int32_t*)((char*)plan->arena + zero_off);   // stays zero: the arena is zero-filled and nothing writes here
     if (plan->arena) infr::launch_fill_zero(be->stream, plan->arena, arena);
     *out = plan;
     return INFR_OK;
@@ -738,6 +824,44 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
     const int n_cu = be->prop.multiProcessorCount;
     for (size_t oi = 0; oi < plan->ops.size(); oi++) {
         const infr_op& op = plan->ops[oi];
+        const infr_hip_plan::FuseOp fz = plan->fuse[oi];
+        if (fz.kind == infr_hip_plan::kSkip) continue;
+        if (fz.kind == infr_hip_plan::kGateUpAct) {
+            const infr_op_linear& lu = plan->ops[fz.a].u.linear;                       // up
+            const infr_op_linear& lg = plan->ops[fz.a == oi ? oi + 1 : oi].u.linear;   // gate
+            const infr_op_gated_act& ga = plan->ops[fz.b].u.gated_act;
+            if (!(need(lg.x, "Linear.x") && need(lg.weight, "Linear.weight") && need(lu.weight, "Linear.weight") &&
+                  need(ga.dst, "GatedAct.dst")))
+                return INFR_ERR_BACKEND;
+            infr::MoeGemvParams gp{};
+            gp.x = (const float*)ptr[lg.x];
+            gp.ids = plan->zero_ids;
+            gp.weights = (const float*)plan->zero_ids;   // never used: weight_before is off
+            gp.gate = (const uint8_t*)ptr[lg.weight];
+            gp.up = (const uint8_t*)ptr[lu.weight];
+            gp.gate_dt = gp.up_dt = plan->tensors[lg.weight].dtype;
+            gp.rows = (int)lg.m; gp.ne = (int)lg.in_f; gp.nff = (int)lg.out_f; gp.n_used = 1; gp.n_expert = 1;
+            gp.act = ga.act; gp.has_clamp = (int)ga.has_swiglu_clamp; gp.clamp = ga.swiglu_clamp;
+            gp.h = (float*)ptr[ga.dst]; gp.n_cu = n_cu;
+            Timed t(be, "linear_gate_up_act");
+            infr::launch_moe_gate_up(s, gp);
+            continue;
+        }
+        if (fz.kind == infr_hip_plan::kLinearAdd) {
+            const infr_op_linear& l = op.u.linear;
+            const infr_op_add& ad = plan->ops[fz.a].u.add;
+            const uint32_t other = ad.a == l.dst ? ad.b : ad.a;
+            if (!(need(l.x, "Linear.x") && need(l.weight, "Linear.weight") && need(other, "Add.a") && need(ad.dst, "Add.dst")))
+                return INFR_ERR_BACKEND;
+            int we = 1, wb = 4;
+            geometry(plan->tensors[l.weight].dtype, &we, &wb);
+            size_t row_bytes = (size_t)(l.in_f / we) * wb;
+            const uint8_t* w = (const uint8_t*)ptr[l.weight] + (size_t)(l.w_off / l.in_f) * row_bytes;
+            Timed t(be, "linear_add");
+            infr::launch_linear(s, (const float*)ptr[l.x], w, plan->tensors[l.weight].dtype, row_bytes, (int)l.m, (int)l.in_f,
+                                (int)l.out_f, (float*)ptr[ad.dst], n_cu, (const float*)ptr[other]);
+            continue;
+        }
         switch (op.kind) {
             case INFR_OP_MOE_FFN: {
                 const infr_op_moe_ffn& m = op.u.moe_ffn;

@@ -567,7 +567,8 @@ __global__ __launch_bounds__(512) void moe_down_combine_fast(MoeGemvParams p, in
             float wk = p.weight_before ? 1.0f : w[k];
             acc = __fadd_rn(acc, __fmul_rn(wk, ypart[k][threadIdx.x]));
         }
-        p.dst[(size_t)r * p.ne + o0 + threadIdx.x] = acc;
+        const size_t oi = (size_t)r * p.ne + o0 + threadIdx.x;
+        p.dst[oi] = p.addend ? __fadd_rn(p.addend[oi], acc) : acc;
     }
 }
 
@@ -619,7 +620,10 @@ __global__ __launch_bounds__(256) void moe_down_combine_generic(MoeGemvParams p,
         float wk = p.weight_before ? 1.0f : p.weights[(size_t)r * p.n_used + slot];
         acc = __fadd_rn(acc, __fmul_rn(wk, y));
     }
-    if (lane == 0) p.dst[(size_t)r * p.ne + o] = acc;
+    if (lane == 0) {
+        const size_t oi = (size_t)r * p.ne + o;
+        p.dst[oi] = p.addend ? __fadd_rn(p.addend[oi], acc) : acc;
+    }
 }
 
 // ------------------------------------------------------------------------------- dispatch
@@ -702,6 +706,14 @@ static bool try_down(hipStream_t s, const MoeGemvParams& p) {
         default: INFR_LAUNCH((moe_down_combine_fast<F, 8>), grid, block, lds, s, p, ot); break;
     }
     return true;
+}
+
+bool moe_down_is_fast(const MoeGemvParams& p) {
+    if (p.n_used > kMaxUsedFast) return false;
+    if (p.down_dt == INFR_Q4K) return fast_ok<Q4KFmt>(p.nff);
+    if (p.down_dt == INFR_Q6K) return fast_ok<Q6KFmt>(p.nff);
+    if (p.down_dt == INFR_Q8_0) return fast_ok<Q80Fmt>(p.nff);
+    return false;
 }
 
 void launch_moe_down_combine(hipStream_t s, const MoeGemvParams& p) {
@@ -929,7 +941,8 @@ void launch_moe_down_bucketed(hipStream_t s, const MoeGemvParams& p) {
 // dst[m, out_f] = x . W^T, the dense neighbour of the expert GEMVs (shared expert).
 template <class F>
 __global__ __launch_bounds__(256) void linear_fast(const float* __restrict__ xin, const uint8_t* __restrict__ w,
-                                                   int in_f, int out_f, float* __restrict__ dst, int ot) {
+                                                   int in_f, int out_f, float* __restrict__ dst, int ot,
+                                                   const float* __restrict__ addend) {
     extern __shared__ uint32_t dyn_lds[];
     constexpr int U = 4;  // rows a wave keeps in flight
     const int r = blockIdx.y;
@@ -963,14 +976,17 @@ __global__ __launch_bounds__(256) void linear_fast(const float* __restrict__ xin
         for (int u = 0; u < U; u++) {
             const int o = base + (u * 4 + wave) * pl.rw_count + pl.rw;
             float y = row_sum<F>(F::dot(raw[u], pl.sub, x), pl, nblk);
-            if (o < ocount && pl.writer()) dst[(size_t)r * out_f + o0 + o] = y;
+            if (o < ocount && pl.writer()) {
+                const size_t oi = (size_t)r * out_f + o0 + o;
+                dst[oi] = addend ? __fadd_rn(addend[oi], y) : y;
+            }
         }
     }
 }
 
 __global__ __launch_bounds__(256) void linear_generic(const float* __restrict__ x, const uint8_t* __restrict__ w,
                                                       int dt, size_t row_bytes, int in_f, int out_f,
-                                                      float* __restrict__ dst) {
+                                                      float* __restrict__ dst, const float* __restrict__ addend) {
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int o = blockIdx.x * 4 + wave;
     const int r = blockIdx.y;
@@ -980,30 +996,33 @@ __global__ __launch_bounds__(256) void linear_generic(const float* __restrict__ 
     float y = 0.f;
     for (int k = lane; k < in_f; k += kWave) y = fmaf(decode_elem(dt, row, (uint32_t)k), xr[k], y);
     y = wave_sum(y);
-    if (lane == 0) dst[(size_t)r * out_f + o] = y;
+    if (lane == 0) {
+        const size_t oi = (size_t)r * out_f + o;
+        dst[oi] = addend ? __fadd_rn(addend[oi], y) : y;
+    }
 }
 
 template <class F>
 static bool try_linear(hipStream_t s, const float* x, const uint8_t* w, int m, int in_f, int out_f, float* dst,
-                       int n_cu) {
+                       int n_cu, const float* addend) {
     if (!fast_ok<F>(in_f)) return false;
     const int rw = 64 / (in_f / F::kBlockElems * F::kLPB);
     int ot = ceil_div(out_f, n_cu);
     ot = ceil_div(ot, 4 * rw) * 4 * rw;  // whole rounds of the block's 4 waves
     dim3 grid(ceil_div(out_f, ot), m), block(256);
-    INFR_LAUNCH((linear_fast<F>), grid, block, 4 * cells_bytes(in_f), s, x, w, in_f, out_f, dst, ot);
+    INFR_LAUNCH((linear_fast<F>), grid, block, 4 * cells_bytes(in_f), s, x, w, in_f, out_f, dst, ot, addend);
     return true;
 }
 
 void launch_linear(hipStream_t s, const float* x, const uint8_t* w, int dt, size_t row_bytes, int m, int in_f,
-                   int out_f, float* dst, int n_cu) {
+                   int out_f, float* dst, int n_cu, const float* addend) {
     bool done = false;
-    if (dt == INFR_Q4K) done = try_linear<Q4KFmt>(s, x, w, m, in_f, out_f, dst, n_cu);
-    else if (dt == INFR_Q6K) done = try_linear<Q6KFmt>(s, x, w, m, in_f, out_f, dst, n_cu);
-    else if (dt == INFR_Q8_0) done = try_linear<Q80Fmt>(s, x, w, m, in_f, out_f, dst, n_cu);
+    if (dt == INFR_Q4K) done = try_linear<Q4KFmt>(s, x, w, m, in_f, out_f, dst, n_cu, addend);
+    else if (dt == INFR_Q6K) done = try_linear<Q6KFmt>(s, x, w, m, in_f, out_f, dst, n_cu, addend);
+    else if (dt == INFR_Q8_0) done = try_linear<Q80Fmt>(s, x, w, m, in_f, out_f, dst, n_cu, addend);
     if (done) return;
     dim3 grid((out_f + 3) / 4, m), block(256);
-    INFR_LAUNCH(linear_generic, grid, block, 0, s, x, w, dt, row_bytes, in_f, out_f, dst);
+    INFR_LAUNCH(linear_generic, grid, block, 0, s, x, w, dt, row_bytes, in_f, out_f, dst, addend);
 }
 
 }  // namespace infr

@@ -60,6 +60,7 @@ struct MoeGemvParams {
     int fused_gate_up;
     float* h;                 // [rows, n_used, nff]
     float* dst;               // [rows, ne]
+    const float* addend;      // down: optional [rows, ne] added to the combined result (fused residual / MoE sum)
     int n_cu;
     // When set, the gate/up kernel routes each token row itself from route.logits (every block
     // redundantly; block 0 of a row publishes ids / weights / probs) and no route launch is needed.
@@ -70,6 +71,8 @@ struct MoeGemvParams {
     const int32_t* bk_pair_src;  // [rows * n_used] flat (row * n_used + rank) in bucket order
     float* y;                    // [rows * n_used, ne] per-pair down outputs, flat pair order
 };
+// True when launch_moe_down_combine will take the bandwidth-bound kernel.
+bool moe_down_is_fast(const MoeGemvParams& p);
 // True when launch_moe_gate_up will take the kernel that can route inline.
 bool moe_gate_up_routes_inline(const MoeGemvParams& p);
 // h = act(gate.x) * (up.x) for every (row, slot).
@@ -116,8 +119,9 @@ void launch_moe_down_bucketed(hipStream_t s, const MoeGemvParams& p);
 void launch_dequant(hipStream_t s, const uint8_t* src, int dtype, uint64_t numel, float* out);
 
 // dst[m, out_f] = x[m, in_f] . W^T (W rows start at `w`, `row_bytes` apart).
+// With `addend` ([m, out_f]) the result is addend + x . W^T (a following Op::Add folded in).
 void launch_linear(hipStream_t s, const float* x, const uint8_t* w, int dt, size_t row_bytes, int m, int in_f,
-                   int out_f, float* dst, int n_cu);
+                   int out_f, float* dst, int n_cu, const float* addend = nullptr);
 void launch_gated_act(hipStream_t s, const float* gate, const float* up, float* dst, int rows, int nff, int act,
                       int up_off, int up_stride, int gate_stride, int gate_block_width, int has_clamp, float clamp);
 void launch_add(hipStream_t s, const float* a, const float* b, float* dst, uint32_t n);

@@ -380,6 +380,64 @@ def test_shared_expert_branch_matches_oracle(be):
     assert np.array_equal(got2, O.add(x, moe).ravel())
 
 
+@pytest.mark.parametrize("rows,act", [(1, M.Activation.Silu), (5, M.Activation.Gelu)])
+def test_fused_dense_ffn_launches_give_the_bits_of_the_separate_ops(be, rows, act):
+    """Linear+Linear+GatedAct and Linear+Add collapse into one launch each when their temporaries are
+    single-use Internal tensors; declaring the temporaries as Outputs keeps the ops separate.  Both
+    run the same inner products in the same rounding order, so the results must be identical bits."""
+    ne, nff = 1024, 512
+    rng = np.random.default_rng(rows)
+    x = rng.standard_normal((rows, ne)).astype(np.float32)
+    res = rng.standard_normal((rows, ne)).astype(np.float32)
+    wg, wu = _realistic(rng, 1, nff, ne, H.Q4K), _realistic(rng, 1, nff, ne, H.Q4K)
+    wd = _realistic(rng, 1, ne, nff, H.Q6K)
+
+    def run(fusable):
+        g = M.Graph()
+        mk = g.internal if fusable else g.output
+        xi, ri = g.input(TensorDesc([rows, ne], DType.F32)), g.input(TensorDesc([rows, ne], DType.F32))
+        wgt, wut = g.weight(TensorDesc([nff, ne], DType.Q4K)), g.weight(TensorDesc([nff, ne], DType.Q4K))
+        wdt = g.weight(TensorDesc([ne, nff], DType.Q6K))
+        gt, ut = mk(TensorDesc([rows, nff], DType.F32)), mk(TensorDesc([rows, nff], DType.F32))
+        at, st = g.internal(TensorDesc([rows, nff], DType.F32)), mk(TensorDesc([rows, ne], DType.F32))
+        yi = g.output(TensorDesc([rows, ne], DType.F32))
+        g.linear(x=xi, weight=wut, dst=ut, m=rows, in_f=ne, out_f=nff)       # up first: either order fuses
+        g.linear(x=xi, weight=wgt, dst=gt, m=rows, in_f=ne, out_f=nff)
+        g.gated_act(gate=gt, up=ut, dst=at, rows=rows, nff=nff, act=act)
+        g.linear(x=at, weight=wdt, dst=st, m=rows, in_f=nff, out_f=ne)
+        g.add(a=ri, b=st, dst=yi, n=rows * ne)
+        plan = be.compile(g)
+        bufs = [be.buffer_from(v) for v in (x, res, wg, wu, wd)]
+        b = M.Bindings()
+        for tid, buf in zip((xi, ri, wgt, wut, wdt), bufs):
+            b.bind(tid, buf)
+        extra = []
+        if not fusable:
+            for tid, n in ((gt, rows * nff), (ut, rows * nff), (st, rows * ne)):
+                extra.append(be.alloc(n * 4))
+                b.bind(tid, extra[-1])
+        yb = be.alloc(rows * ne * 4)
+        b.bind(yi, yb)
+        be.prof_enable(True)
+        be.execute(plan, b)
+        out = be.download(yb, rows * ne * 4, np.float32)
+        names = set(be.prof_read())
+        be.prof_enable(False)
+        for buf in bufs + extra + [yb]:
+            buf.free()
+        plan.free()
+        return out, names
+
+    fused, fused_names = run(True)
+    plain, plain_names = run(False)
+    assert {"linear_gate_up_act", "linear_add"} <= fused_names
+    assert "gated_act" in plain_names and "add" in plain_names
+    assert np.array_equal(bits(fused), bits(plain))
+    og, ou = O.linear(x, wg, H.Q4K, ne, nff), O.linear(x, wu, H.Q4K, ne, nff)
+    want = O.add(res, O.linear(O.gated_act_rows(og, ou, act=int(act)), wd, H.Q6K, nff, ne))
+    assert H.rel_l2(fused.reshape(rows, ne), want.reshape(rows, ne)) < REL_L2
+
+
 # ------------------------------------------------------------------ synthetic workloads at full size
 from moe4all_amd import synth as S  # noqa: E402
 
