@@ -184,6 +184,14 @@ def main():
         }
         # the decode kernel that routes its own token row also reads that row's logits
         alg["moe_route_gate_up"] = alg["moe_gate_up"] + batch * shape.n_expert * 4
+        if shape.shared_ff:
+            sh_gate_b = M.backend.bytes_for(shape.gate_dtype, shape.shared_ff * shape.ne)
+            sh_down_b = M.backend.bytes_for(shape.down_dtype, shape.ne * shape.shared_ff)
+            # the always-on expert as one more slot of the routed kernels
+            alg["moe_route_gate_up_shared"] = alg["moe_route_gate_up"] + 2 * sh_gate_b + batch * shape.shared_ff * 4
+            alg["moe_down_combine_shared"] = alg["moe_down_combine"] + sh_down_b + batch * shape.shared_ff * 4
+            alg["linear_gate_up_act"] = 2 * sh_gate_b + batch * shape.ne * 4 + batch * shape.shared_ff * 4
+            alg["linear_add"] = sh_down_b + batch * shape.shared_ff * 4 + 2 * batch * shape.ne * 4
         flops = {  # algorithmic FLOPs per launch of the grouped GEMMs (2 per multiply-add)
             "moe_grouped_gate_up": 2.0 * pairs * 2 * shape.n_ff * shape.ne,
             "moe_grouped_down": 2.0 * pairs * shape.ne * shape.n_ff,

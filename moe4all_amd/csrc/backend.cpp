@@ -117,12 +117,14 @@ struct infr_hip_plan {
     // Launch fusion of the dense SwiGLU FFN the reference emits beside the routed experts
     // (crates/infr-llama/src/runner.rs:8116-8174: Linear gate, Linear up, GatedAct, Linear down, Add).
     // fuse[i]: what op i does at execute time.
-    enum Fuse : uint8_t { kPlain = 0, kSkip, kGateUpAct, kLinearAdd };
+    enum Fuse : uint8_t { kPlain = 0, kSkip, kGateUpAct, kLinearAdd, kMoeShared };
     struct FuseOp {
         Fuse kind = kPlain;
-        uint32_t a = 0, b = 0;   // kGateUpAct: index of the up Linear and of the GatedAct; kLinearAdd: index of the Add
+        uint32_t a = 0, b = 0;   // kGateUpAct: index of the up Linear and of the GatedAct; kLinearAdd: index of the Add;
+                                 // kMoeShared: index of the always-on expert's first Linear and of its down Linear
     };
     std::vector<FuseOp> fuse;
+    std::vector<FuseOp> fuse_head;     // kMoeShared: the records of the ops it absorbed, as they were before
     int32_t* zero_ids = nullptr;       // [max rows of a fused gate/up] expert id 0 for every row
 };
 
@@ -547,7 +549,7 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
                 arena += round_up((size_t)rows * m.n_expert * 4 + 4, 256) * 2;
                 arena += round_up((size_t)rows * m.n_used * 4 + 4, 256) * 2;
                 const size_t pairs = (size_t)rows * m.n_used;
-                size_t shared = round_up(pairs * m.n_ff_exp * 4 + 4, 256);
+                size_t shared = round_up((pairs + rows) * m.n_ff_exp * 4 + 4, 256);   // one more slot per row: see kMoeShared
                 const uint32_t min_rows = be->cfg.moe_batched_min_rows ? be->cfg.moe_batched_min_rows : kBatchedMinRows;
                 const bool batched = rows >= min_rows && m.n_used <= 64 && !m.fused_gate_up &&
                                      c.dt(m.gate_exps) == c.dt(m.up_exps) &&
@@ -727,6 +729,47 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
                 }
             }
         }
+        // MoeFfn followed by an always-on ("shared") expert on the same rows whose result is added to
+        // the routed sum: on the per-token path the expert runs as one more slot of the two routed
+        // kernels.  The slot's inner products are the ones the fused Linear kernels run, its weight is
+        // exactly 1 and it is combined last, which is the Add's rounding: the bits do not change.
+        plan->fuse_head = plan->fuse;
+        for (uint32_t oi = 0; oi + 5 < g->n_ops; oi++) {
+            if (plan->ops[oi].kind != INFR_OP_MOE_FFN || plan->fuse[oi + 1].kind != infr_hip_plan::kGateUpAct ||
+                plan->fuse[oi + 4].kind != infr_hip_plan::kLinearAdd)
+                continue;
+            const infr_op_moe_ffn& m = plan->ops[oi].u.moe_ffn;
+            const MoeScratch& sc = plan->moe[oi];
+            const infr_hip_plan::FuseOp fg = plan->fuse[oi + 1];
+            const infr_op_linear& lu = plan->ops[fg.a].u.linear;
+            const infr_op_linear& lg = plan->ops[fg.a == oi + 1 ? oi + 2 : oi + 1].u.linear;
+            const infr_op_gated_act& ga = plan->ops[oi + 3].u.gated_act;
+            const infr_op_linear& ld = plan->ops[oi + 4].u.linear;
+            const infr_op_add& ad = plan->ops[oi + 5].u.add;
+            const uint32_t other = ad.a == ld.dst ? ad.b : ad.a;
+            if (sc.batched || sc.bucketed || sc.rows == 0 || m.fused_gate_up) continue;
+            if (lg.x != m.x || (int)lg.m != sc.rows || lg.in_f != m.ne || lg.out_f != m.n_ff_exp) continue;
+            if (ld.x != ga.dst || !temp(ga.dst) || ld.in_f != m.n_ff_exp || ld.out_f != m.ne || ld.w_off != 0) continue;
+            if (other != m.dst || !temp(m.dst)) continue;
+            if (c.dt(lg.weight) != c.dt(m.gate_exps) || c.dt(lu.weight) != c.dt(m.up_exps) ||
+                c.dt(ld.weight) != c.dt(m.down_exps))
+                continue;
+            if (ga.act != m.act || ga.has_swiglu_clamp != m.has_swiglu_clamp ||
+                (ga.has_swiglu_clamp && ga.swiglu_clamp != m.swiglu_clamp))
+                continue;
+            infr::MoeGemvParams probe{};
+            probe.gate_dt = c.dt(m.gate_exps); probe.up_dt = c.dt(m.up_exps); probe.down_dt = c.dt(m.down_exps);
+            probe.ne = (int)m.ne; probe.nff = (int)m.n_ff_exp; probe.n_used = (int)m.n_used; probe.n_expert = (int)m.n_expert;
+            probe.rows = sc.rows;
+            probe.route.n_expert = (int)m.n_expert; probe.route.n_used = (int)m.n_used;
+            probe.route.n_groups = (int)m.n_expert_groups; probe.route.n_groups_used = (int)m.n_expert_groups_used;
+            probe.sh_gate = probe.sh_up = probe.sh_down = (const uint8_t*)plan;   // any non-null value: shape checks only
+            if (m.n_used >= 63 || !infr::moe_gate_up_routes_inline(probe) || !infr::moe_down_is_fast(probe)) continue;
+            plan->fuse[oi].kind = infr_hip_plan::kMoeShared;
+            plan->fuse[oi].a = oi + 1;
+            plan->fuse[oi].b = oi + 4;
+            for (uint32_t k = oi + 1; k <= oi + 5; k++) plan->fuse[k].kind = infr_hip_plan::kSkip;
+        }
     }
     const size_t zero_off = arena;
     arena += round_up(zero_rows * 4 + 4, 256);
@@ -753,7 +796,7 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
             s.slot_pair = (int32_t*)p;
         }
         p = (char*)plan->arena + shared_off;
-        s.h = (float*)p; p += round_up(pairs * m.n_ff_exp * 4 + 4, 256);
+        s.h = (float*)p; p += round_up((pairs + rows) * m.n_ff_exp * 4 + 4, 256);
         if (s.batched) {
             s.xh = (_Float16*)p; p += round_up(rows * m.ne * 2, 256);
             s.xs = (float*)p;    p += round_up(rows * 4, 256);
@@ -988,6 +1031,20 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                     }
                     break;
                 }
+                if (fz.kind == infr_hip_plan::kMoeShared) {
+                    const infr_hip_plan::FuseOp fg = plan->fuse_head[fz.a];
+                    const infr_op_linear& lu = plan->ops[fg.a].u.linear;
+                    const infr_op_linear& lg = plan->ops[fg.a == fz.a ? fz.a + 1 : fz.a].u.linear;
+                    const infr_op_linear& ld = plan->ops[fz.b].u.linear;
+                    const infr_op_add& ad = plan->ops[fz.b + 1].u.add;
+                    if (!(need(lg.weight, "Linear.weight") && need(lu.weight, "Linear.weight") &&
+                          need(ld.weight, "Linear.weight") && need(ad.dst, "Add.dst")))
+                        return INFR_ERR_BACKEND;
+                    gp.sh_gate = (const uint8_t*)ptr[lg.weight];
+                    gp.sh_up = (const uint8_t*)ptr[lu.weight];
+                    gp.sh_down = (const uint8_t*)ptr[ld.weight];
+                    gp.dst = (float*)ptr[ad.dst];
+                }
                 gp.route = rp;
                 gp.route_inline = infr::moe_gate_up_routes_inline(gp) ? 1 : 0;
                 if (!gp.route_inline) {
@@ -995,12 +1052,12 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                     infr::launch_route(s, rp);
                 }
                 {
-                    Timed t(be, gp.route_inline ? "moe_route_gate_up" : "moe_gate_up");
+                    Timed t(be, gp.sh_gate ? "moe_route_gate_up_shared" : gp.route_inline ? "moe_route_gate_up" : "moe_gate_up");
                     infr::launch_moe_gate_up(s, gp);
                 }
                 gp.x = nullptr;
                 {
-                    Timed t(be, "moe_down_combine");
+                    Timed t(be, gp.sh_down ? "moe_down_combine_shared" : "moe_down_combine");
                     infr::launch_moe_down_combine(s, gp);
                 }
                 break;

@@ -453,10 +453,15 @@ __global__ __launch_bounds__(256) void moe_gate_up_fast(MoeGemvParams p, int ft)
         s_ids[threadIdx.x] = p.ids[(size_t)r * p.n_used + threadIdx.x];
         s_w[threadIdx.x] = p.weights[(size_t)r * p.n_used + threadIdx.x];
     }
+    const int n_slots = p.n_used + (p.sh_gate ? 1 : 0);   // the always-on expert is slot n_used (<= 63 then)
+    if (p.sh_gate && threadIdx.x == 255) {
+        s_ids[p.n_used] = 0;
+        s_w[p.n_used] = 1.0f;
+    }
     __syncthreads();
     TRACE(1, s_ids[0]);
     __builtin_amdgcn_wave_barrier();
-    const int nitems = fcount * p.n_used;
+    const int nitems = fcount * n_slots;
     const int per_round = 4 * pl.rw_count;
     typename F::X x;
     bool have_x = false;
@@ -467,8 +472,11 @@ __global__ __launch_bounds__(256) void moe_gate_up_fast(MoeGemvParams p, int ft)
             const int it = min(base + (u * 4 + wave) * pl.rw_count + pl.rw, nitems - 1);  // past the end: re-read the last
             const int slot = it / fcount, f = f0 + (it - slot * fcount);
             const int e = s_ids[slot];
-            graw[u] = load_row<F>(pl, p.gate + (size_t)e * p.gate_stride + (size_t)f * row_bytes);
-            uraw[u] = load_row<F>(pl, p.up + (size_t)e * p.up_stride + (size_t)f * row_bytes);
+            const bool routed = slot < p.n_used;
+            const uint8_t* gb = routed ? p.gate + (size_t)e * p.gate_stride : p.sh_gate;
+            const uint8_t* ub = routed ? p.up + (size_t)e * p.up_stride : p.sh_up;
+            graw[u] = load_row<F>(pl, gb + (size_t)f * row_bytes);
+            uraw[u] = load_row<F>(pl, ub + (size_t)f * row_bytes);
         }
         if (!have_x) {
             // while the weights are in flight: the wave converts x to fixed point once, together
@@ -497,12 +505,12 @@ __global__ __launch_bounds__(256) void moe_gate_up_fast(MoeGemvParams p, int ft)
             if (it < nitems) {
                 const int slot = it / fcount, f = f0 + (it - slot * fcount);
                 float gs = s_g[wave][lane], us = s_u[wave][lane];
-                if (p.weight_before) {
+                if (p.weight_before && slot < p.n_used) {
                     const float wp = s_w[slot];
                     gs = __fmul_rn(wp, gs);
                     us = __fmul_rn(wp, us);
                 }
-                p.h[((size_t)r * p.n_used + slot) * p.nff + f] = gated_act_fn(p.act, p.has_clamp, p.clamp, gs, us, s_tab);
+                p.h[((size_t)r * n_slots + slot) * p.nff + f] = gated_act_fn(p.act, p.has_clamp, p.clamp, gs, us, s_tab);
             }
         }
         __builtin_amdgcn_wave_barrier();
@@ -534,11 +542,13 @@ __global__ __launch_bounds__(512) void moe_down_combine_fast(MoeGemvParams p, in
     const int32_t* ids = p.ids + (size_t)r * p.n_used;
     uint32_t* cells = dyn_lds + (size_t)wave * ((p.nff + 31) / 32) * kCellDwords;
 
-    for (int slot = wave; slot < p.n_used; slot += nwaves) {
-        const int e = ids[slot];  // first: every weight address below waits on it
-        const float* hrow = p.h + ((size_t)r * p.n_used + slot) * p.nff;
+    const int n_slots = p.n_used + (p.sh_down ? 1 : 0);   // the always-on expert is slot n_used
+    for (int slot = wave; slot < n_slots; slot += nwaves) {
+        const bool routed = slot < p.n_used;
+        const int e = routed ? ids[slot] : 0;  // first: every weight address below waits on it
+        const float* hrow = p.h + ((size_t)r * n_slots + slot) * p.nff;
         const XLoad xl = stage_x_load(hrow, p.nff, lane);
-        const uint8_t* bank = p.down + (size_t)e * p.down_stride + (size_t)o0 * row_bytes;
+        const uint8_t* bank = (routed ? p.down + (size_t)e * p.down_stride : p.sh_down) + (size_t)o0 * row_bytes;
         typename F::Raw raw[S];
 #pragma unroll
         for (int st = 0; st < S; st++) {
@@ -551,20 +561,21 @@ __global__ __launch_bounds__(512) void moe_down_combine_fast(MoeGemvParams p, in
         __builtin_amdgcn_wave_barrier();
         typename F::X x;
         F::fetch_x(x, cells, pl.blk, pl.sub);
-        const float ds = p.down_scale ? p.down_scale[e] : 1.0f;
+        const bool scaled = p.down_scale && routed;
+        const float ds = scaled ? p.down_scale[e] : 1.0f;
 #pragma unroll
         for (int st = 0; st < S; st++) {
             const int o = st * pl.rw_count + pl.rw;
             float y = row_sum<F>(F::dot(raw[st], pl.sub, x), pl, nblk);
-            if (o < ocount && pl.writer()) ypart[slot][o] = p.down_scale ? __fmul_rn(y, ds) : y;
+            if (o < ocount && pl.writer()) ypart[slot][o] = scaled ? __fmul_rn(y, ds) : y;
         }
     }
     __syncthreads();
     if ((int)threadIdx.x < ocount) {
         const float* w = p.weights + (size_t)r * p.n_used;
         float acc = 0.0f;
-        for (int k = 0; k < p.n_used; k++) {
-            float wk = p.weight_before ? 1.0f : w[k];
+        for (int k = 0; k < n_slots; k++) {
+            float wk = (p.weight_before || k >= p.n_used) ? 1.0f : w[k];
             acc = __fadd_rn(acc, __fmul_rn(wk, ypart[k][threadIdx.x]));
         }
         const size_t oi = (size_t)r * p.ne + o0 + threadIdx.x;
@@ -649,7 +660,7 @@ static bool try_gate_up(hipStream_t s, const MoeGemvParams& p) {
     // about one block per compute unit; a block's ft * n_used items go to 4 waves of rw rows each
     int ft = ceil_div(p.nff, p.n_cu);
     if (ft < 1) ft = 1;
-    const int per_wave = ceil_div(ft * p.n_used, 4 * rw);
+    const int per_wave = ceil_div(ft * (p.n_used + (p.sh_gate ? 1 : 0)), 4 * rw);
     dim3 grid(ceil_div(p.nff, ft), p.rows), block(256);
     // U * rw results per wave must fit the 64-entry staging rows
     int u = per_wave < 1 ? 1 : per_wave;
@@ -687,7 +698,8 @@ void launch_moe_gate_up(hipStream_t s, const MoeGemvParams& p) {
 
 template <class F>
 static bool try_down(hipStream_t s, const MoeGemvParams& p) {
-    if (!fast_ok<F>(p.nff) || p.n_used > kMaxUsedFast) return false;
+    const int n_slots = p.n_used + (p.sh_down ? 1 : 0);
+    if (!fast_ok<F>(p.nff) || n_slots > kMaxUsedFast) return false;
     const int rw = 64 / (p.nff / F::kBlockElems * F::kLPB);
     // output rows per block ~ ne / n_cu, as S row groups of rw rows per wave, S in {1,2,4,8}
     const int want = ceil_div(p.ne, p.n_cu);
@@ -696,7 +708,7 @@ static bool try_down(hipStream_t s, const MoeGemvParams& p) {
     while (steps > 1 && steps * rw > kMaxOt) steps >>= 1;
     if (steps * rw > kMaxOt) return false;
     const int ot = steps * rw;
-    const int nwaves = p.n_used < 8 ? p.n_used : 8;
+    const int nwaves = n_slots < 8 ? n_slots : 8;
     dim3 grid(ceil_div(p.ne, ot), p.rows), block(64 * nwaves);
     const size_t lds = nwaves * cells_bytes(p.nff);
     switch (steps) {
@@ -709,7 +721,7 @@ static bool try_down(hipStream_t s, const MoeGemvParams& p) {
 }
 
 bool moe_down_is_fast(const MoeGemvParams& p) {
-    if (p.n_used > kMaxUsedFast) return false;
+    if (p.n_used + (p.sh_down ? 1 : 0) > kMaxUsedFast) return false;
     if (p.down_dt == INFR_Q4K) return fast_ok<Q4KFmt>(p.nff);
     if (p.down_dt == INFR_Q6K) return fast_ok<Q6KFmt>(p.nff);
     if (p.down_dt == INFR_Q8_0) return fast_ok<Q80Fmt>(p.nff);

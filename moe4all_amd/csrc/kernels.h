@@ -61,6 +61,9 @@ struct MoeGemvParams {
     float* h;                 // [rows, n_used, nff]
     float* dst;               // [rows, ne]
     const float* addend;      // down: optional [rows, ne] added to the combined result (fused residual / MoE sum)
+    // optional always-on expert handled as one more slot after the n_used routed ones (same dtypes,
+    // same n_ff, routing weight 1): h then has n_used + 1 slots per row
+    const uint8_t* sh_gate; const uint8_t* sh_up; const uint8_t* sh_down;
     int n_cu;
     // When set, the gate/up kernel routes each token row itself from route.logits (every block
     // redundantly; block 0 of a row publishes ids / weights / probs) and no route launch is needed.

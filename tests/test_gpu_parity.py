@@ -438,6 +438,80 @@ def test_fused_dense_ffn_launches_give_the_bits_of_the_separate_ops(be, rows, ac
     assert H.rel_l2(fused.reshape(rows, ne), want.reshape(rows, ne)) < REL_L2
 
 
+@pytest.mark.parametrize("rows,K,opts", [(1, 4, {}), (3, 8, {"weight_before": True}), (2, 6, {"with_down_scale": True})])
+def test_shared_expert_as_an_extra_slot_gives_the_bits_of_the_separate_ops(be, rows, K, opts):
+    """MoeFfn followed by an ungated shared expert (Linear, Linear, GatedAct, Linear, Add —
+    crates/infr-llama/src/seam/runner.rs:8116-8174) runs as one more slot of the two routed decode
+    kernels when the routed sum is a single-use Internal tensor.  Declaring that tensor an Output
+    keeps MoeFfn and the dense FFN apart; both must give identical bits."""
+    ne, nff, E = 1024, 512, 16
+    rng = np.random.default_rng(100 + rows)
+    x = rng.standard_normal((rows, ne)).astype(np.float32)
+    router = (rng.standard_normal((E, ne)) * 0.1).astype(np.float32)
+    eg, eu = _realistic(rng, E, nff, ne, H.Q4K), _realistic(rng, E, nff, ne, H.Q4K)
+    ed = _realistic(rng, E, ne, nff, H.Q6K)
+    wg, wu = _realistic(rng, 1, nff, ne, H.Q4K), _realistic(rng, 1, nff, ne, H.Q4K)
+    wd = _realistic(rng, 1, ne, nff, H.Q6K)
+    dscale = (0.5 + rng.random(E)).astype(np.float32) if opts.get("with_down_scale") else None
+    mopts = {k: v for k, v in opts.items() if not k.startswith("with_")}
+
+    def run(fusable):
+        g = M.Graph()
+        xi = g.input(TensorDesc([rows, ne], DType.F32))
+        rt = g.weight(TensorDesc([E, ne], DType.F32))
+        egt, eut = g.weight(TensorDesc([E, nff, ne], DType.Q4K)), g.weight(TensorDesc([E, nff, ne], DType.Q4K))
+        edt = g.weight(TensorDesc([E, ne, nff], DType.Q6K))
+        wgt, wut = g.weight(TensorDesc([nff, ne], DType.Q4K)), g.weight(TensorDesc([nff, ne], DType.Q4K))
+        wdt = g.weight(TensorDesc([ne, nff], DType.Q6K))
+        dst = g.weight(TensorDesc([E], DType.F32)) if dscale is not None else None
+        moe = (g.internal if fusable else g.output)(TensorDesc([rows, ne], DType.F32))
+        gt, ut = g.internal(TensorDesc([rows, nff], DType.F32)), g.internal(TensorDesc([rows, nff], DType.F32))
+        at, st = g.internal(TensorDesc([rows, nff], DType.F32)), g.internal(TensorDesc([rows, ne], DType.F32))
+        yi = g.output(TensorDesc([rows, ne], DType.F32))
+        g.moe_ffn(x=xi, router=rt, gate_exps=egt, up_exps=eut, down_exps=edt, dst=moe, ne=ne, n_expert=E, n_used=K,
+                  n_ff_exp=nff, down_scale=dst, **mopts)
+        g.linear(x=xi, weight=wgt, dst=gt, m=rows, in_f=ne, out_f=nff)
+        g.linear(x=xi, weight=wut, dst=ut, m=rows, in_f=ne, out_f=nff)
+        g.gated_act(gate=gt, up=ut, dst=at, rows=rows, nff=nff)
+        g.linear(x=at, weight=wdt, dst=st, m=rows, in_f=nff, out_f=ne)
+        g.add(a=moe, b=st, dst=yi, n=rows * ne)
+        plan = be.compile(g)
+        pairs = [(xi, x), (rt, router), (egt, eg), (eut, eu), (edt, ed), (wgt, wg), (wut, wu), (wdt, wd)]
+        if dscale is not None:
+            pairs.append((dst, dscale))
+        bufs, b = [], M.Bindings()
+        for tid, v in pairs:
+            bufs.append(be.buffer_from(v))
+            b.bind(tid, bufs[-1])
+        if not fusable:
+            bufs.append(be.alloc(rows * ne * 4))
+            b.bind(moe, bufs[-1])
+        yb = be.alloc(rows * ne * 4)
+        b.bind(yi, yb)
+        be.prof_enable(True)
+        be.execute(plan, b)
+        out = be.download(yb, rows * ne * 4, np.float32)
+        names = set(be.prof_read())
+        be.prof_enable(False)
+        routing = be.moe_routing(plan, 0)
+        for buf in bufs + [yb]:
+            buf.free()
+        plan.free()
+        return out, names, routing
+
+    fused, fused_names, r1 = run(True)
+    plain, plain_names, r2 = run(False)
+    assert {"moe_route_gate_up_shared", "moe_down_combine_shared"} <= fused_names and "linear_add" not in fused_names
+    assert {"moe_route_gate_up", "linear_gate_up_act", "linear_add"} <= plain_names
+    assert np.array_equal(r1["idx"], r2["idx"]) and np.array_equal(bits(r1["w"]), bits(r2["w"]))
+    assert np.array_equal(bits(fused), bits(plain))
+    want_moe = O.moe_ffn(x, router, eg, eu, ed, ne=ne, n_expert=E, n_used=K, n_ff_exp=nff, gate_dtype=H.Q4K,
+                         down_dtype=H.Q6K, down_scale=dscale, **mopts)["dst"]
+    og, ou = O.linear(x, wg, H.Q4K, ne, nff), O.linear(x, wu, H.Q4K, ne, nff)
+    want = O.add(want_moe, O.linear(O.gated_act_rows(og, ou), wd, H.Q6K, nff, ne))
+    assert H.rel_l2(fused.reshape(rows, ne), want.reshape(rows, ne)) < REL_L2
+
+
 # ------------------------------------------------------------------ synthetic workloads at full size
 from moe4all_amd import synth as S  # noqa: E402
 
