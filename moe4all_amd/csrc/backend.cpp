@@ -747,7 +747,9 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
             const infr_op_linear& ld = plan->ops[oi + 4].u.linear;
             const infr_op_add& ad = plan->ops[oi + 5].u.add;
             const uint32_t other = ad.a == ld.dst ? ad.b : ad.a;
-            if (sc.batched || sc.bucketed || sc.rows == 0 || m.fused_gate_up) continue;
+            // one token row only: with more rows the launches saved no longer matter and the down kernel
+            // streams best with one wave per routed slot
+            if (sc.batched || sc.bucketed || sc.rows != 1 || m.fused_gate_up) continue;
             if (lg.x != m.x || (int)lg.m != sc.rows || lg.in_f != m.ne || lg.out_f != m.n_ff_exp) continue;
             if (ld.x != ga.dst || !temp(ga.dst) || ld.in_f != m.n_ff_exp || ld.out_f != m.ne || ld.w_off != 0) continue;
             if (other != m.dst || !temp(m.dst)) continue;
@@ -1046,7 +1048,9 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                     gp.dst = (float*)ptr[ad.dst];
                 }
                 gp.route = rp;
-                gp.route_inline = infr::moe_gate_up_routes_inline(gp) ? 1 : 0;
+                // Every block of the gate/up kernel routes its own token row when that is cheaper than a
+                // launch of the routing kernel: the blocks of one compute unit repeat it once per row.
+                gp.route_inline = infr::moe_gate_up_routes_inline(gp) && (rows == 1 || (uint64_t)rows * m.n_expert <= 512) ? 1 : 0;
                 if (!gp.route_inline) {
                     Timed t(be, "route_topk");
                     infr::launch_route(s, rp);

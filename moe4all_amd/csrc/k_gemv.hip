@@ -422,23 +422,88 @@ __device__ __forceinline__ float row_sum(float v, const Place<F>& pl, int nblk) 
 // (slot, f) of its tile; x is identical for every slot of a token.  U = items a wave has in
 // flight per round.  Results wait in LDS and one lane per item applies the gated activation
 // after the round, so the f64 exp and the divide run once per wave, not once per item.
+// One stage of a wave's work: U (gate row, up row) pairs per row lane group, loaded together.
 template <class F, int U>
+struct GuStage { typename F::Raw g[U], u[U]; };
+
+struct GuTile {
+    int r, f0, fcount, nitems, n_slots, wave, lane;
+    size_t row_bytes;
+};
+
+// Issue every load of the stage that starts at item `base`; items past the end re-read the last.
+template <class F, int U>
+__device__ __forceinline__ void gu_issue(GuStage<F, U>& st, const MoeGemvParams& p, const Place<F>& pl, const GuTile& t,
+                                         const int32_t* s_ids, int base) {
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        const int it = min(base + (u * 4 + t.wave) * pl.rw_count + pl.rw, t.nitems - 1);
+        const int slot = it / t.fcount, f = t.f0 + (it - slot * t.fcount);
+        const int e = s_ids[slot];
+        const bool routed = slot < p.n_used;
+        const uint8_t* gb = routed ? p.gate + (size_t)e * p.gate_stride : p.sh_gate;
+        const uint8_t* ub = routed ? p.up + (size_t)e * p.up_stride : p.sh_up;
+        st.g[u] = load_row<F>(pl, gb + (size_t)f * t.row_bytes);
+        st.u[u] = load_row<F>(pl, ub + (size_t)f * t.row_bytes);
+    }
+}
+
+// Dot the stage's rows with x; results wait in LDS and one lane per item applies the gated
+// activation, so the f64 exp and the divide run once per wave, not once per item.
+template <class F, int U>
+__device__ __forceinline__ void gu_finish(const GuStage<F, U>& st, const MoeGemvParams& p, const Place<F>& pl,
+                                          const GuTile& t, const typename F::X& x, int nblk, int base, float (*s_g)[64],
+                                          float (*s_u)[64], const float* s_w, const uint64_t* s_tab) {
+#pragma unroll
+    for (int u = 0; u < U; u++) {
+        float gs = row_sum<F>(F::dot(st.g[u], pl.sub, x), pl, nblk);
+        float us = row_sum<F>(F::dot(st.u[u], pl.sub, x), pl, nblk);
+        if (pl.writer()) {
+            s_g[t.wave][u * pl.rw_count + pl.rw] = gs;
+            s_u[t.wave][u * pl.rw_count + pl.rw] = us;
+        }
+    }
+    __builtin_amdgcn_wave_barrier();
+    if (t.lane < U * pl.rw_count) {
+        const int u = t.lane / pl.rw_count, rw = t.lane - u * pl.rw_count;
+        const int it = base + (u * 4 + t.wave) * pl.rw_count + rw;
+        if (it < t.nitems) {
+            const int slot = it / t.fcount, f = t.f0 + (it - slot * t.fcount);
+            float gs = s_g[t.wave][t.lane], us = s_u[t.wave][t.lane];
+            if (p.weight_before && slot < p.n_used) {
+                const float wp = s_w[slot];
+                gs = __fmul_rn(wp, gs);
+                us = __fmul_rn(wp, us);
+            }
+            p.h[((size_t)t.r * t.n_slots + slot) * p.nff + f] = gated_act_fn(p.act, p.has_clamp, p.clamp, gs, us, s_tab);
+        }
+    }
+    __builtin_amdgcn_wave_barrier();
+}
+
+// PIPE == false: every stage is loaded, then finished (one stage is the common decode case and
+// then all of the block's loads are in flight at once).  PIPE == true, for tiles of three or more
+// stages: two stage buffers, the next stage's loads are issued before the current stage is
+// finished, so a wave always has a stage in flight while it computes.
+template <class F, int U, bool PIPE>
 __global__ __launch_bounds__(256) void moe_gate_up_fast(MoeGemvParams p, int ft) {
     extern __shared__ uint32_t dyn_lds[];
     __shared__ uint64_t s_tab[32];
     __shared__ int32_t s_ids[64];
     __shared__ float s_w[64];
     __shared__ float s_g[4][64], s_u[4][64];
-    const int r = blockIdx.y;
-    const int f0 = blockIdx.x * ft;
-    const int fcount = min(ft, p.nff - f0);
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    GuTile t;
+    t.r = blockIdx.y;
+    t.f0 = blockIdx.x * ft;
+    t.fcount = min(ft, p.nff - t.f0);
+    t.wave = threadIdx.x >> 6;
+    t.lane = threadIdx.x & 63;
+    const int r = t.r, wave = t.wave, lane = t.lane;
     const int nblk = p.ne / F::kBlockElems;
-    const size_t row_bytes = (size_t)nblk * F::kBlockBytes;
+    t.row_bytes = (size_t)nblk * F::kBlockBytes;
     const Place<F> pl(nblk, lane);
     const size_t cell_words = (size_t)((p.ne + 31) / 32) * kCellDwords;
     uint32_t* cells = dyn_lds + (size_t)wave * cell_words;
-    TRACE(0, lane);
     // x is requested first; it does not depend on the routing
     const float* xrow = p.x + (size_t)r * p.ne;
     const XLoad xl = stage_x_load(xrow, p.ne, lane);
@@ -453,68 +518,55 @@ __global__ __launch_bounds__(256) void moe_gate_up_fast(MoeGemvParams p, int ft)
         s_ids[threadIdx.x] = p.ids[(size_t)r * p.n_used + threadIdx.x];
         s_w[threadIdx.x] = p.weights[(size_t)r * p.n_used + threadIdx.x];
     }
-    const int n_slots = p.n_used + (p.sh_gate ? 1 : 0);   // the always-on expert is slot n_used (<= 63 then)
+    t.n_slots = p.n_used + (p.sh_gate ? 1 : 0);   // the always-on expert is slot n_used (<= 63 then)
     if (p.sh_gate && threadIdx.x == 255) {
         s_ids[p.n_used] = 0;
         s_w[p.n_used] = 1.0f;
     }
     __syncthreads();
-    TRACE(1, s_ids[0]);
     __builtin_amdgcn_wave_barrier();
-    const int nitems = fcount * n_slots;
-    const int per_round = 4 * pl.rw_count;
+    t.nitems = t.fcount * t.n_slots;
+    const int step = 4 * pl.rw_count * U;
     typename F::X x;
-    bool have_x = false;
-    for (int base = 0; base < nitems; base += per_round * U) {
-        typename F::Raw graw[U], uraw[U];
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-            const int it = min(base + (u * 4 + wave) * pl.rw_count + pl.rw, nitems - 1);  // past the end: re-read the last
-            const int slot = it / fcount, f = f0 + (it - slot * fcount);
-            const int e = s_ids[slot];
-            const bool routed = slot < p.n_used;
-            const uint8_t* gb = routed ? p.gate + (size_t)e * p.gate_stride : p.sh_gate;
-            const uint8_t* ub = routed ? p.up + (size_t)e * p.up_stride : p.sh_up;
-            graw[u] = load_row<F>(pl, gb + (size_t)f * row_bytes);
-            uraw[u] = load_row<F>(pl, ub + (size_t)f * row_bytes);
-        }
-        if (!have_x) {
-            // while the weights are in flight: the wave converts x to fixed point once, together
-            stage_x_finish<F::kGroup, F::kSigned>(xl, xrow, p.ne, cells, lane);
-            __builtin_amdgcn_wave_barrier();
-            F::fetch_x(x, cells, pl.blk, pl.sub);
-            have_x = true;
-        }
-        TRACE(4, *reinterpret_cast<const uint32_t*>(&x));
-        TRACE(2, *reinterpret_cast<const uint32_t*>(&graw[0]));
-        TRACE(3, *reinterpret_cast<const uint32_t*>(&uraw[U - 1]));
-#pragma unroll
-        for (int u = 0; u < U; u++) {
-            float gs = row_sum<F>(F::dot(graw[u], pl.sub, x), pl, nblk);
-            float us = row_sum<F>(F::dot(uraw[u], pl.sub, x), pl, nblk);
-            if (pl.writer()) {
-                s_g[wave][u * pl.rw_count + pl.rw] = gs;
-                s_u[wave][u * pl.rw_count + pl.rw] = us;
+    if (!PIPE) {
+        bool have_x = false;
+        for (int base = 0; base < t.nitems; base += step) {
+            GuStage<F, U> st;
+            gu_issue<F, U>(st, p, pl, t, s_ids, base);
+            if (!have_x) {
+                // while the weights are in flight: the wave converts x to fixed point once, together
+                stage_x_finish<F::kGroup, F::kSigned>(xl, xrow, p.ne, cells, lane);
+                __builtin_amdgcn_wave_barrier();
+                F::fetch_x(x, cells, pl.blk, pl.sub);
+                have_x = true;
             }
+            gu_finish<F, U>(st, p, pl, t, x, nblk, base, s_g, s_u, s_w, s_tab);
         }
+    } else {
+        GuStage<F, U> sa, sb;
+        gu_issue<F, U>(sa, p, pl, t, s_ids, 0);
+        gu_issue<F, U>(sb, p, pl, t, s_ids, step);
+        stage_x_finish<F::kGroup, F::kSigned>(xl, xrow, p.ne, cells, lane);
         __builtin_amdgcn_wave_barrier();
-        TRACE(5, s_g[wave][0]);
-        if (lane < U * pl.rw_count) {
-            const int u = lane / pl.rw_count, rw = lane - u * pl.rw_count;
-            const int it = base + (u * 4 + wave) * pl.rw_count + rw;
-            if (it < nitems) {
-                const int slot = it / fcount, f = f0 + (it - slot * fcount);
-                float gs = s_g[wave][lane], us = s_u[wave][lane];
-                if (p.weight_before && slot < p.n_used) {
-                    const float wp = s_w[slot];
-                    gs = __fmul_rn(wp, gs);
-                    us = __fmul_rn(wp, us);
-                }
-                p.h[((size_t)r * n_slots + slot) * p.nff + f] = gated_act_fn(p.act, p.has_clamp, p.clamp, gs, us, s_tab);
+        F::fetch_x(x, cells, pl.blk, pl.sub);
+        gu_finish<F, U>(sa, p, pl, t, x, nblk, 0, s_g, s_u, s_w, s_tab);
+        int base = step;   // the stage sb holds
+        for (;;) {
+            if (base + step >= t.nitems) {
+                gu_finish<F, U>(sb, p, pl, t, x, nblk, base, s_g, s_u, s_w, s_tab);
+                break;
             }
+            gu_issue<F, U>(sa, p, pl, t, s_ids, base + step);
+            gu_finish<F, U>(sb, p, pl, t, x, nblk, base, s_g, s_u, s_w, s_tab);
+            base += step;
+            if (base + step >= t.nitems) {
+                gu_finish<F, U>(sa, p, pl, t, x, nblk, base, s_g, s_u, s_w, s_tab);
+                break;
+            }
+            gu_issue<F, U>(sb, p, pl, t, s_ids, base + step);
+            gu_finish<F, U>(sa, p, pl, t, x, nblk, base, s_g, s_u, s_w, s_tab);
+            base += step;
         }
-        __builtin_amdgcn_wave_barrier();
-        TRACE(6, lane);
     }
 }
 
@@ -525,22 +577,56 @@ __global__ __launch_bounds__(256) void moe_gate_up_fast(MoeGemvParams p, int ft)
 // out += w_rank * y_rank as a separate multiply and add
 // (crates/infr-cpu/src/lib.rs:4290-4302).
 constexpr int kMaxUsedFast = 16;
-constexpr int kMaxOt = 64;
+constexpr int kMaxOt = 128;
+
+struct DownTile {
+    int slot, ocount;
+    size_t row_bytes;
+    bool scaled;
+    float ds;
+};
+
+// Issue the loads of the S row groups that start at output row `obase` of the tile; rows past
+// the tile re-read its last row.
+template <class F, int S>
+__device__ __forceinline__ void down_issue(typename F::Raw (&raw)[S], const Place<F>& pl, const DownTile& t,
+                                           const uint8_t* bank, int obase) {
+#pragma unroll
+    for (int st = 0; st < S; st++) {
+        const int o = min(obase + st * pl.rw_count + pl.rw, t.ocount - 1);
+        raw[st] = load_row<F>(pl, bank + (size_t)o * t.row_bytes);
+    }
+}
 
 template <class F, int S>
+__device__ __forceinline__ void down_finish(const typename F::Raw (&raw)[S], const Place<F>& pl, const DownTile& t,
+                                            const typename F::X& x, int nblk, int obase, float (*ypart)[kMaxOt]) {
+#pragma unroll
+    for (int st = 0; st < S; st++) {
+        const int o = obase + st * pl.rw_count + pl.rw;
+        float y = row_sum<F>(F::dot(raw[st], pl.sub, x), pl, nblk);
+        if (o < t.ocount && pl.writer()) ypart[t.slot][o] = t.scaled ? __fmul_rn(y, t.ds) : y;
+    }
+}
+
+// PIPE == false: ot = S row groups, all loaded up front (single-token decode: everything in
+// flight at once).  PIPE == true: the tile is any number of stages of S row groups; a wave keeps
+// the next stage's loads in flight while it finishes the current one.
+template <class F, int S, bool PIPE>
 __global__ __launch_bounds__(512) void moe_down_combine_fast(MoeGemvParams p, int ot) {
     extern __shared__ uint32_t dyn_lds[];
     __shared__ float ypart[kMaxUsedFast][kMaxOt];
     const int r = blockIdx.y;
     const int o0 = blockIdx.x * ot;
-    const int ocount = min(ot, p.ne - o0);
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int nwaves = blockDim.x >> 6;
     const int nblk = p.nff / F::kBlockElems;
-    const size_t row_bytes = (size_t)nblk * F::kBlockBytes;
     const Place<F> pl(nblk, lane);
     const int32_t* ids = p.ids + (size_t)r * p.n_used;
     uint32_t* cells = dyn_lds + (size_t)wave * ((p.nff + 31) / 32) * kCellDwords;
+    DownTile t;
+    t.ocount = min(ot, p.ne - o0);
+    t.row_bytes = (size_t)nblk * F::kBlockBytes;
 
     const int n_slots = p.n_used + (p.sh_down ? 1 : 0);   // the always-on expert is slot n_used
     for (int slot = wave; slot < n_slots; slot += nwaves) {
@@ -548,37 +634,59 @@ __global__ __launch_bounds__(512) void moe_down_combine_fast(MoeGemvParams p, in
         const int e = routed ? ids[slot] : 0;  // first: every weight address below waits on it
         const float* hrow = p.h + ((size_t)r * n_slots + slot) * p.nff;
         const XLoad xl = stage_x_load(hrow, p.nff, lane);
-        const uint8_t* bank = (routed ? p.down + (size_t)e * p.down_stride : p.sh_down) + (size_t)o0 * row_bytes;
-        typename F::Raw raw[S];
-#pragma unroll
-        for (int st = 0; st < S; st++) {
-            const int o = min(st * pl.rw_count + pl.rw, ocount - 1);  // rows past the tile re-read its last row
-            raw[st] = load_row<F>(pl, bank + (size_t)o * row_bytes);
-        }
-        // while the weights are in flight: this slot's h to fixed point, once per wave
-        __builtin_amdgcn_wave_barrier();
-        stage_x_finish<F::kGroup, F::kSigned>(xl, hrow, p.nff, cells, lane);
-        __builtin_amdgcn_wave_barrier();
+        const uint8_t* bank = (routed ? p.down + (size_t)e * p.down_stride : p.sh_down) + (size_t)o0 * t.row_bytes;
+        t.slot = slot;
+        t.scaled = p.down_scale && routed;
+        typename F::Raw ra[S];
+        down_issue<F, S>(ra, pl, t, bank, 0);
         typename F::X x;
-        F::fetch_x(x, cells, pl.blk, pl.sub);
-        const bool scaled = p.down_scale && routed;
-        const float ds = scaled ? p.down_scale[e] : 1.0f;
-#pragma unroll
-        for (int st = 0; st < S; st++) {
-            const int o = st * pl.rw_count + pl.rw;
-            float y = row_sum<F>(F::dot(raw[st], pl.sub, x), pl, nblk);
-            if (o < ocount && pl.writer()) ypart[slot][o] = scaled ? __fmul_rn(y, ds) : y;
+        if (!PIPE) {
+            // while the weights are in flight: this slot's h to fixed point, once per wave
+            __builtin_amdgcn_wave_barrier();
+            stage_x_finish<F::kGroup, F::kSigned>(xl, hrow, p.nff, cells, lane);
+            __builtin_amdgcn_wave_barrier();
+            F::fetch_x(x, cells, pl.blk, pl.sub);
+            t.ds = t.scaled ? p.down_scale[e] : 1.0f;
+            down_finish<F, S>(ra, pl, t, x, nblk, 0, ypart);
+        } else {
+            const int gstep = S * pl.rw_count;
+            typename F::Raw rb[S];
+            down_issue<F, S>(rb, pl, t, bank, gstep);
+            __builtin_amdgcn_wave_barrier();
+            stage_x_finish<F::kGroup, F::kSigned>(xl, hrow, p.nff, cells, lane);
+            __builtin_amdgcn_wave_barrier();
+            F::fetch_x(x, cells, pl.blk, pl.sub);
+            t.ds = t.scaled ? p.down_scale[e] : 1.0f;
+            down_finish<F, S>(ra, pl, t, x, nblk, 0, ypart);
+            int o = gstep;   // the stage rb holds
+            for (;;) {
+                if (o + gstep >= t.ocount) {
+                    down_finish<F, S>(rb, pl, t, x, nblk, o, ypart);
+                    break;
+                }
+                down_issue<F, S>(ra, pl, t, bank, o + gstep);
+                down_finish<F, S>(rb, pl, t, x, nblk, o, ypart);
+                o += gstep;
+                if (o + gstep >= t.ocount) {
+                    down_finish<F, S>(ra, pl, t, x, nblk, o, ypart);
+                    break;
+                }
+                down_issue<F, S>(rb, pl, t, bank, o + gstep);
+                down_finish<F, S>(ra, pl, t, x, nblk, o, ypart);
+                o += gstep;
+            }
+            __builtin_amdgcn_wave_barrier();   // the next slot's h overwrites this wave's cells
         }
     }
     __syncthreads();
-    if ((int)threadIdx.x < ocount) {
+    for (int o = threadIdx.x; o < t.ocount; o += blockDim.x) {
         const float* w = p.weights + (size_t)r * p.n_used;
         float acc = 0.0f;
         for (int k = 0; k < n_slots; k++) {
             float wk = (p.weight_before || k >= p.n_used) ? 1.0f : w[k];
-            acc = __fadd_rn(acc, __fmul_rn(wk, ypart[k][threadIdx.x]));
+            acc = __fadd_rn(acc, __fmul_rn(wk, ypart[k][o]));
         }
-        const size_t oi = (size_t)r * p.ne + o0 + threadIdx.x;
+        const size_t oi = (size_t)r * p.ne + o0 + o;
         p.dst[oi] = p.addend ? __fadd_rn(p.addend[oi], acc) : acc;
     }
 }
@@ -657,21 +765,25 @@ template <class F>
 static bool try_gate_up(hipStream_t s, const MoeGemvParams& p) {
     if (!fast_ok<F>(p.ne) || p.n_used > 64) return false;
     const int rw = 64 / (p.ne / F::kBlockElems * F::kLPB);
-    // about one block per compute unit; a block's ft * n_used items go to 4 waves of rw rows each
+    // about one block per compute unit; a block's ft * n_slots items go to 4 waves of rw rows each
+    const int n_slots = p.n_used + (p.sh_gate ? 1 : 0);
     int ft = ceil_div(p.nff, p.n_cu);
     if (ft < 1) ft = 1;
-    const int per_wave = ceil_div(ft * (p.n_used + (p.sh_gate ? 1 : 0)), 4 * rw);
+    const int per_wave = ceil_div(ft * n_slots, 4 * rw);
+    // tiles of three or more stages stream with the next stage in flight
+    const bool pipe = per_wave > 6 && 3 * rw <= 64;
     dim3 grid(ceil_div(p.nff, ft), p.rows), block(256);
     // U * rw results per wave must fit the 64-entry staging rows
     int u = per_wave < 1 ? 1 : per_wave;
     while (u * rw > 64) u--;
     const size_t lds = 4 * cells_bytes(p.ne) +
                        (p.route_inline ? route_scratch_floats(p.route.n_expert, p.route.n_groups) * sizeof(float) : 0);
-    if (u >= 6) INFR_LAUNCH((moe_gate_up_fast<F, 6>), grid, block, lds, s, p, ft);
-    else if (u == 5 || u == 4) INFR_LAUNCH((moe_gate_up_fast<F, 4>), grid, block, lds, s, p, ft);
-    else if (u == 3) INFR_LAUNCH((moe_gate_up_fast<F, 3>), grid, block, lds, s, p, ft);
-    else if (u == 2) INFR_LAUNCH((moe_gate_up_fast<F, 2>), grid, block, lds, s, p, ft);
-    else INFR_LAUNCH((moe_gate_up_fast<F, 1>), grid, block, lds, s, p, ft);
+    if (pipe) INFR_LAUNCH((moe_gate_up_fast<F, 3, true>), grid, block, lds, s, p, ft);
+    else if (u >= 6) INFR_LAUNCH((moe_gate_up_fast<F, 6, false>), grid, block, lds, s, p, ft);
+    else if (u == 5 || u == 4) INFR_LAUNCH((moe_gate_up_fast<F, 4, false>), grid, block, lds, s, p, ft);
+    else if (u == 3) INFR_LAUNCH((moe_gate_up_fast<F, 3, false>), grid, block, lds, s, p, ft);
+    else if (u == 2) INFR_LAUNCH((moe_gate_up_fast<F, 2, false>), grid, block, lds, s, p, ft);
+    else INFR_LAUNCH((moe_gate_up_fast<F, 1, false>), grid, block, lds, s, p, ft);
     return true;
 }
 
@@ -701,21 +813,41 @@ static bool try_down(hipStream_t s, const MoeGemvParams& p) {
     const int n_slots = p.n_used + (p.sh_down ? 1 : 0);
     if (!fast_ok<F>(p.nff) || n_slots > kMaxUsedFast) return false;
     const int rw = 64 / (p.nff / F::kBlockElems * F::kLPB);
-    // output rows per block ~ ne / n_cu, as S row groups of rw rows per wave, S in {1,2,4,8}
+    // output rows per block ~ rows * ne / n_cu
     const int want = ceil_div(p.ne, p.n_cu);
+    if (p.rows >= 2) {
+        // several token rows: tiles of whole stages of 2 row groups, about one block per compute
+        // unit in total, streamed with the next stage in flight; one wave per slot
+        const int gstep = 2 * rw;
+        // tile height: whole stages; fewest rounds of blocks over the compute units, counting a
+        // block's fixed cost (ids, h staging, combine) as about a dozen rows of streaming
+        int ot = 0;
+        long best = 0;
+        for (int cand = 2 * gstep; cand <= kMaxOt; cand += gstep) {
+            const long blocks = (long)p.rows * ceil_div(p.ne, cand);
+            const long cost = ((blocks + p.n_cu - 1) / p.n_cu) * (cand + 12);
+            if (ot == 0 || cost < best) { ot = cand; best = cost; }
+        }
+        if (ot >= 2 * gstep) {
+            const int nwaves = n_slots < 8 ? n_slots : 8;
+            dim3 grid(ceil_div(p.ne, ot), p.rows), block(64 * nwaves);
+            const size_t lds = nwaves * cells_bytes(p.nff);
+            INFR_LAUNCH((moe_down_combine_fast<F, 2, true>), grid, block, lds, s, p, ot);
+            return true;
+        }
+    }
     int steps = 1;
     while (steps < 8 && steps * rw < want) steps <<= 1;
     while (steps > 1 && steps * rw > kMaxOt) steps >>= 1;
-    if (steps * rw > kMaxOt) return false;
     const int ot = steps * rw;
     const int nwaves = n_slots < 8 ? n_slots : 8;
     dim3 grid(ceil_div(p.ne, ot), p.rows), block(64 * nwaves);
     const size_t lds = nwaves * cells_bytes(p.nff);
     switch (steps) {
-        case 1: INFR_LAUNCH((moe_down_combine_fast<F, 1>), grid, block, lds, s, p, ot); break;
-        case 2: INFR_LAUNCH((moe_down_combine_fast<F, 2>), grid, block, lds, s, p, ot); break;
-        case 4: INFR_LAUNCH((moe_down_combine_fast<F, 4>), grid, block, lds, s, p, ot); break;
-        default: INFR_LAUNCH((moe_down_combine_fast<F, 8>), grid, block, lds, s, p, ot); break;
+        case 1: INFR_LAUNCH((moe_down_combine_fast<F, 1, false>), grid, block, lds, s, p, ot); break;
+        case 2: INFR_LAUNCH((moe_down_combine_fast<F, 2, false>), grid, block, lds, s, p, ot); break;
+        case 4: INFR_LAUNCH((moe_down_combine_fast<F, 4, false>), grid, block, lds, s, p, ot); break;
+        default: INFR_LAUNCH((moe_down_combine_fast<F, 8, false>), grid, block, lds, s, p, ot); break;
     }
     return true;
 }

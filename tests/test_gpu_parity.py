@@ -438,12 +438,14 @@ def test_fused_dense_ffn_launches_give_the_bits_of_the_separate_ops(be, rows, ac
     assert H.rel_l2(fused.reshape(rows, ne), want.reshape(rows, ne)) < REL_L2
 
 
-@pytest.mark.parametrize("rows,K,opts", [(1, 4, {}), (3, 8, {"weight_before": True}), (2, 6, {"with_down_scale": True})])
+@pytest.mark.parametrize("rows,K,opts", [(1, 4, {}), (1, 8, {"weight_before": True}), (1, 6, {"with_down_scale": True}),
+                                         (3, 8, {})])
 def test_shared_expert_as_an_extra_slot_gives_the_bits_of_the_separate_ops(be, rows, K, opts):
     """MoeFfn followed by an ungated shared expert (Linear, Linear, GatedAct, Linear, Add —
     crates/infr-llama/src/seam/runner.rs:8116-8174) runs as one more slot of the two routed decode
-    kernels when the routed sum is a single-use Internal tensor.  Declaring that tensor an Output
-    keeps MoeFfn and the dense FFN apart; both must give identical bits."""
+    kernels when the routed sum is a single-use Internal tensor and there is one token row.
+    Declaring that tensor an Output keeps MoeFfn and the dense FFN apart; both must give identical
+    bits.  With several rows the ops stay apart either way."""
     ne, nff, E = 1024, 512, 16
     rng = np.random.default_rng(100 + rows)
     x = rng.standard_normal((rows, ne)).astype(np.float32)
@@ -501,7 +503,10 @@ def test_shared_expert_as_an_extra_slot_gives_the_bits_of_the_separate_ops(be, r
 
     fused, fused_names, r1 = run(True)
     plain, plain_names, r2 = run(False)
-    assert {"moe_route_gate_up_shared", "moe_down_combine_shared"} <= fused_names and "linear_add" not in fused_names
+    if rows == 1:
+        assert {"moe_route_gate_up_shared", "moe_down_combine_shared"} <= fused_names and "linear_add" not in fused_names
+    else:
+        assert fused_names == plain_names
     assert {"moe_route_gate_up", "linear_gate_up_act", "linear_add"} <= plain_names
     assert np.array_equal(r1["idx"], r2["idx"]) and np.array_equal(bits(r1["w"]), bits(r2["w"]))
     assert np.array_equal(bits(fused), bits(plain))
