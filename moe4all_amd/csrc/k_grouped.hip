@@ -526,44 +526,58 @@ __device__ __forceinline__ void grouped_tile(const GroupedParams& p, const Group
         bn1 = F::load_blk(c.wrow1, min((s0 >> 2) + 2, last_blk), half);
     }
 
-    // accumulator register r of a 32x32 tile: row 8*(r/4) + 4*(lane/32) + r%4, column lane%32
+    // accumulator register r of a 32x32 tile: row 8*(r/4) + 4*(lane/32) + r%4, column lane%32.
+    // The epilogue variant is chosen once, outside the loops; rows below the last 32-row sub-tile
+    // are all inside the tile, so only that sub-tile tests the row count.
     const Tile& t = c.t;
     const int n0 = c.n0;
     const int fc0 = n0 + (DOWN ? 64 : 32) * wave + (lane & 31);   // the lane's column (second column tile of DOWN: + 32)
-    float* const obase = p.out + (size_t)t.p0 * p.N;
-    const bool plain_silu = !DOWN && p.act == INFR_ACT_SILU && !p.has_clamp && !p.weight_before;
-    const float ds = (DOWN && p.down_scale) ? p.down_scale[t.e] : 1.0f;
+    float* const obase = p.out + (size_t)t.p0 * p.N + fc0;
+    const int mrow = 4 * (lane >> 5);
+    auto for_each = [&](auto&& body) {
 #pragma unroll
-    for (int mi = 0; mi < M; mi++) {
+        for (int mi = 0; mi < M; mi++) {
 #pragma unroll
-        for (int r4 = 0; r4 < 4; r4++) {
-            const int m0 = 32 * mi + 8 * r4 + 4 * (lane >> 5);   // rows m0 .. m0 + 3
-            const float4 sc4 = *reinterpret_cast<const float4*>(c.s_scale + m0);
-            const float scs[4] = {sc4.x, sc4.y, sc4.z, sc4.w};
+            for (int r4 = 0; r4 < 4; r4++) {
+                const int m0 = 32 * mi + 8 * r4 + mrow;   // rows m0 .. m0 + 3
+                const float4 sc4 = *reinterpret_cast<const float4*>(c.s_scale + m0);
+                const float scs[4] = {sc4.x, sc4.y, sc4.z, sc4.w};
 #pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const int r = 4 * r4 + i, m = m0 + i;
-                const float sc = scs[i];
-                float* orow = obase + (size_t)m * p.N;
-                if (DOWN) {
-                    const float y0 = acc0[mi][r] * sc * ds, y1 = acc1[mi][r] * sc * ds;
-                    if (m < t.cnt && fc0 < p.N) orow[fc0] = y0;
-                    if (m < t.cnt && fc0 + 32 < p.N) orow[fc0 + 32] = y1;
-                } else if (plain_silu) {
-                    // silu(g) * u with the hardware exp and reciprocal
-                    const float g = acc0[mi][r] * sc, u = acc1[mi][r] * sc;
-                    const float h = g * u * __frcp_rn(1.0f + __expf(-g));
-                    if (m < t.cnt && fc0 < p.N) orow[fc0] = h;
-                } else {
-                    float g = acc0[mi][r] * sc, u = acc1[mi][r] * sc;
-                    if (p.weight_before && m < t.cnt) {
-                        const float wp = p.route_w[p.pair_src[t.p0 + m]];
-                        g *= wp;
-                        u *= wp;
-                    }
-                    if (m < t.cnt && fc0 < p.N) orow[fc0] = gated_act_fast(p.act, p.has_clamp, p.clamp, g, u);
+                for (int i = 0; i < 4; i++) {
+                    const int m = m0 + i;
+                    if (mi < M - 1 || m < t.cnt) body(mi, 4 * r4 + i, m, scs[i], obase + (size_t)m * p.N);
                 }
             }
+        }
+    };
+    if (DOWN) {
+        const float ds = p.down_scale ? p.down_scale[t.e] : 1.0f;
+        const bool ok0 = fc0 < p.N, ok1 = fc0 + 32 < p.N;
+        if (ok1) {
+            for_each([&](int mi, int r, int, float sc, float* o) {
+                o[0] = acc0[mi][r] * sc * ds;
+                o[32] = acc1[mi][r] * sc * ds;
+            });
+        } else if (ok0) {
+            for_each([&](int mi, int r, int, float sc, float* o) { o[0] = acc0[mi][r] * sc * ds; });
+        }
+    } else if (fc0 < p.N) {
+        if (p.act == INFR_ACT_SILU && !p.has_clamp && !p.weight_before) {
+            // silu(g) * u with the hardware exp2 and reciprocal (1 ulp each; the operands were f16)
+            for_each([&](int mi, int r, int, float sc, float* o) {
+                const float g = acc0[mi][r] * sc, u = acc1[mi][r] * sc;
+                o[0] = g * u * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g * -1.4426950408889634f));
+            });
+        } else {
+            for_each([&](int mi, int r, int m, float sc, float* o) {
+                float g = acc0[mi][r] * sc, u = acc1[mi][r] * sc;
+                if (p.weight_before) {
+                    const float wp = p.route_w[p.pair_src[t.p0 + min(m, t.cnt - 1)]];
+                    g *= wp;
+                    u *= wp;
+                }
+                o[0] = gated_act_fast(p.act, p.has_clamp, p.clamp, g, u);
+            });
         }
     }
 }
