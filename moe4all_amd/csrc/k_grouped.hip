@@ -21,6 +21,8 @@
 // exact packed subtract and one packed multiply(-add) with the group's scale.  The order in
 // which codes fall out of a dword is not the element order; since a dot product does not care
 // about the order of its terms, the activation rows are stored in that same ("virtual") order.
+#include <type_traits>
+
 #include "device_common.h"
 #include "kernels.h"
 
@@ -374,8 +376,13 @@ __device__ __forceinline__ float gated_act_fast(int act, bool has_clamp, float c
 struct Tile {
     int e, p0, cnt;
 };
-// Tile number `tile` in the order (expert ascending, 128-row tile ascending).  Uniform per wave.
-__device__ __forceinline__ bool find_tile(const int32_t* __restrict__ offsets, int n_expert, int tile, int lane, Tile& t) {
+// The block's work item: (expert, 128-row tile of its bucket, column tile nt), items ordered by
+// expert, row tile, column tile.  Workgroups go to the chip's 8 XCDs round-robin by workgroup id
+// and every XCD has its own L2, so each XCD takes a contiguous eighth of the items: the column
+// tiles of one row tile, which read the same activation tile, then sit behind the same L2.
+// Uniform per wave; false when the block has nothing to do (the grid is an upper bound).
+__device__ __forceinline__ bool find_item(const int32_t* __restrict__ offsets, int n_expert, int n_tiles_n, int lane,
+                                          Tile& t, int& nt) {
     const int epl = (n_expert + 63) >> 6;
     const int e_lo = lane * epl, e_hi = min(n_expert, e_lo + epl);
     int mine = 0;
@@ -386,6 +393,13 @@ __device__ __forceinline__ bool find_tile(const int32_t* __restrict__ offsets, i
         const int o = __shfl_up(incl, d, 64);
         if (lane >= d) incl += o;
     }
+    const int n_items = __shfl(incl, 63, 64) * n_tiles_n;
+    const int per = (n_items + 7) >> 3;
+    const int k = (int)(blockIdx.x >> 3);
+    const int item = (int)(blockIdx.x & 7) * per + k;
+    if (k >= per || item >= n_items) return false;
+    nt = item % n_tiles_n;
+    const int tile = item / n_tiles_n;
     const unsigned long long past = __ballot(incl > tile);
     if (past == 0) return false;
     const int owner = __ffsll((long long)past) - 1;
@@ -393,16 +407,75 @@ __device__ __forceinline__ bool find_tile(const int32_t* __restrict__ offsets, i
     const int o_lo = owner * epl, o_hi = min(n_expert, o_lo + epl);
     for (int e = o_lo; e < o_hi; e++) {
         const int cnt = offsets[e + 1] - offsets[e];
-        const int nt = (cnt + kBM - 1) / kBM;
-        if (rem < nt) {
+        const int ntile = (cnt + kBM - 1) / kBM;
+        if (rem < ntile) {
             t.e = e;
             t.p0 = offsets[e] + rem * kBM;
             t.cnt = min(kBM, cnt - rem * kBM);
             return true;
         }
-        rem -= nt;
+        rem -= ntile;
     }
     return false;
+}
+
+// Epilogue of a tile whose accumulators are acc0/acc1[M] (column tiles of the wave, M 32-row
+// sub-tiles): SwiGLU of (gate, up) or the scaled down-projection row, stored to p.out.
+template <bool DOWN, int M>
+__device__ __forceinline__ void tile_epilogue(const GroupedParams& p, const Tile& t, int n0, int wave, int lane,
+                                              const float* s_scale, const float16v (&acc0)[M], const float16v (&acc1)[M]) {
+    // accumulator register r of a 32x32 tile: row 8*(r/4) + 4*(lane/32) + r%4, column lane%32.
+    // The epilogue variant is chosen once, outside the loops; rows below the last 32-row sub-tile
+    // are all inside the tile, so only that sub-tile tests the row count.
+    const int fc0 = n0 + (DOWN ? 64 : 32) * wave + (lane & 31);   // the lane's column (second column tile of DOWN: + 32)
+    float* const obase = p.out + (size_t)t.p0 * p.N + fc0;
+    const int mrow = 4 * (lane >> 5);
+    auto for_each = [&](auto&& body) {
+#pragma unroll
+        for (int mi = 0; mi < M; mi++) {
+#pragma unroll
+            for (int r4 = 0; r4 < 4; r4++) {
+                const int m0 = 32 * mi + 8 * r4 + mrow;   // rows m0 .. m0 + 3
+                const float4 sc4 = *reinterpret_cast<const float4*>(s_scale + m0);
+                const float scs[4] = {sc4.x, sc4.y, sc4.z, sc4.w};
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int m = m0 + i;
+                    if (mi < M - 1 || m < t.cnt) body(mi, 4 * r4 + i, m, scs[i], obase + (size_t)m * p.N);
+                }
+            }
+        }
+    };
+    if (DOWN) {
+        const float ds = p.down_scale ? p.down_scale[t.e] : 1.0f;
+        const bool ok0 = fc0 < p.N, ok1 = fc0 + 32 < p.N;
+        if (ok1) {
+            for_each([&](int mi, int r, int, float sc, float* o) {
+                o[0] = acc0[mi][r] * sc * ds;
+                o[32] = acc1[mi][r] * sc * ds;
+            });
+        } else if (ok0) {
+            for_each([&](int mi, int r, int, float sc, float* o) { o[0] = acc0[mi][r] * sc * ds; });
+        }
+    } else if (fc0 < p.N) {
+        if (p.act == INFR_ACT_SILU && !p.has_clamp && !p.weight_before) {
+            // silu(g) * u with the hardware exp2 and reciprocal (1 ulp each; the operands were f16)
+            for_each([&](int mi, int r, int, float sc, float* o) {
+                const float g = acc0[mi][r] * sc, u = acc1[mi][r] * sc;
+                o[0] = g * u * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g * -1.4426950408889634f));
+            });
+        } else {
+            for_each([&](int mi, int r, int m, float sc, float* o) {
+                float g = acc0[mi][r] * sc, u = acc1[mi][r] * sc;
+                if (p.weight_before) {
+                    const float wp = p.route_w[p.pair_src[t.p0 + min(m, t.cnt - 1)]];
+                    g *= wp;
+                    u *= wp;
+                }
+                o[0] = gated_act_fast(p.act, p.has_clamp, p.clamp, g, u);
+            });
+        }
+    }
 }
 
 // --------------------------------------------------------------------------------------------
@@ -526,60 +599,7 @@ __device__ __forceinline__ void grouped_tile(const GroupedParams& p, const Group
         bn1 = F::load_blk(c.wrow1, min((s0 >> 2) + 2, last_blk), half);
     }
 
-    // accumulator register r of a 32x32 tile: row 8*(r/4) + 4*(lane/32) + r%4, column lane%32.
-    // The epilogue variant is chosen once, outside the loops; rows below the last 32-row sub-tile
-    // are all inside the tile, so only that sub-tile tests the row count.
-    const Tile& t = c.t;
-    const int n0 = c.n0;
-    const int fc0 = n0 + (DOWN ? 64 : 32) * wave + (lane & 31);   // the lane's column (second column tile of DOWN: + 32)
-    float* const obase = p.out + (size_t)t.p0 * p.N + fc0;
-    const int mrow = 4 * (lane >> 5);
-    auto for_each = [&](auto&& body) {
-#pragma unroll
-        for (int mi = 0; mi < M; mi++) {
-#pragma unroll
-            for (int r4 = 0; r4 < 4; r4++) {
-                const int m0 = 32 * mi + 8 * r4 + mrow;   // rows m0 .. m0 + 3
-                const float4 sc4 = *reinterpret_cast<const float4*>(c.s_scale + m0);
-                const float scs[4] = {sc4.x, sc4.y, sc4.z, sc4.w};
-#pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const int m = m0 + i;
-                    if (mi < M - 1 || m < t.cnt) body(mi, 4 * r4 + i, m, scs[i], obase + (size_t)m * p.N);
-                }
-            }
-        }
-    };
-    if (DOWN) {
-        const float ds = p.down_scale ? p.down_scale[t.e] : 1.0f;
-        const bool ok0 = fc0 < p.N, ok1 = fc0 + 32 < p.N;
-        if (ok1) {
-            for_each([&](int mi, int r, int, float sc, float* o) {
-                o[0] = acc0[mi][r] * sc * ds;
-                o[32] = acc1[mi][r] * sc * ds;
-            });
-        } else if (ok0) {
-            for_each([&](int mi, int r, int, float sc, float* o) { o[0] = acc0[mi][r] * sc * ds; });
-        }
-    } else if (fc0 < p.N) {
-        if (p.act == INFR_ACT_SILU && !p.has_clamp && !p.weight_before) {
-            // silu(g) * u with the hardware exp2 and reciprocal (1 ulp each; the operands were f16)
-            for_each([&](int mi, int r, int, float sc, float* o) {
-                const float g = acc0[mi][r] * sc, u = acc1[mi][r] * sc;
-                o[0] = g * u * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g * -1.4426950408889634f));
-            });
-        } else {
-            for_each([&](int mi, int r, int m, float sc, float* o) {
-                float g = acc0[mi][r] * sc, u = acc1[mi][r] * sc;
-                if (p.weight_before) {
-                    const float wp = p.route_w[p.pair_src[t.p0 + min(m, t.cnt - 1)]];
-                    g *= wp;
-                    u *= wp;
-                }
-                o[0] = gated_act_fast(p.act, p.has_clamp, p.clamp, g, u);
-            });
-        }
-    }
+    tile_epilogue<DOWN, M>(p, c.t, c.n0, wave, lane, c.s_scale, acc0, acc1);
 }
 
 template <class F, bool DOWN>
@@ -595,9 +615,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     // one tile per block (a persistent loop over tiles was measured: no faster, and the static
     // assignment balances the ragged tiles worse than the hardware dispatcher does)
     {
-        const int item = blockIdx.x;
-        const int nt = item % p.n_tiles_n;
-        if (!find_tile(p.offsets, p.n_expert, item / p.n_tiles_n, c.lane, c.t)) return;
+        int nt;
+        if (!find_item(p.offsets, p.n_expert, p.n_tiles_n, c.lane, c.t, nt)) return;
         const Tile& t = c.t;
         constexpr int kBN = DOWN ? 256 : 128;
         c.n0 = nt * kBN;
@@ -632,6 +651,250 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
             case 3: grouped_tile<F, DOWN, 3>(p, c); break;
             default: grouped_tile<F, DOWN, 4>(p, c); break;
         }
+    }
+}
+
+// --------------------------------------------------------------------------------------------
+// K-quant variant with every k-loop load going straight from global memory into LDS
+// (global_load_lds_dwordx4: lane i of a wave's load deposits its 16 bytes at base + 16 i), so that
+// each load instruction covers whole cache lines and nothing is staged in registers:
+//   * activation stage = the tile's 128 tokens x one 64-k slice (16 KB), token-major, the eight
+//     16-byte chunks of a token rotated by (token & 7) so that the operand reads of 32 consecutive
+//     tokens spread over all banks; every wave loads a quarter of it, kNA stages in the ring;
+//   * weight stage = the parts of the 64 weight rows of ONE wave that a half super-block (128 k,
+//     two slices) needs, row-major (Q4_K: header + 4 code chunks = 80 B per row; Q6_K: 4 low-code
+//     chunks, 2 high-bit chunks, scales, tail = 128 B per row, chunks rotated by the row number);
+//     private to the wave, 3 stages in the ring.
+// The loads are issued from inline assembly, so the compiler neither counts them nor orders LDS
+// reads against them: one explicit "s_waitcnt vmcnt(n); s_barrier" per slice does both.  The issue
+// order is fixed (the same number of loads in every even and in every odd slice), so the number
+// of loads younger than the ones slice s needs is a compile-time constant.
+__device__ __forceinline__ void dma16(const void* gsrc, uint32_t lds_base) {
+    uint32_t keep;
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off\n\ts_mov_b32 m0, %0"
+                 : "=&s"(keep)
+                 : "v"(gsrc), "s"(lds_base)
+                 : "memory");
+}
+template <int N>
+__device__ __forceinline__ void wait_loads_then_barrier() {
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" : : "n"(N) : "memory");
+}
+__device__ __forceinline__ uint32_t lds_address(const void* p) {
+    return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)p;
+}
+
+struct D4K : MQ4K {
+    static constexpr int kNC = 5, kRowStride = 80, kNA = 4;
+    // chunk `64 j + lane` of a weight stage: which staged row, where in the super-block its 16
+    // bytes start for the first half, and how far the second half's lie behind
+    static __device__ __forceinline__ void lane_chunk(int j, int lane, int& row, int& off0, int& hoff) {
+        const int c = 64 * j + lane;
+        row = c / 5;
+        const int part = c - 5 * row;   // 0: header, 1..4: code bytes of the half
+        off0 = 16 * part;
+        hoff = part == 0 ? 0 : 64;
+    }
+    static __device__ __forceinline__ Blk read_blk(const uint8_t* st, int row, int) {
+        return Blk{*reinterpret_cast<const uint4*>(st + row * kRowStride)};
+    }
+    static __device__ __forceinline__ Q read_q(const uint8_t* st, int row, int sl, int h) {
+        return Q{*reinterpret_cast<const uint4*>(st + row * kRowStride + 16 + 32 * sl + 16 * h)};
+    }
+};
+
+struct D6K : MQ6K {
+    static constexpr int kNC = 8, kRowStride = 128, kNA = 3;
+    static __device__ __forceinline__ int pos(int row, int part) { return row * kRowStride + ((part + row) & 7) * 16; }
+    static __device__ __forceinline__ void lane_chunk(int j, int lane, int& row, int& off0, int& hoff) {
+        row = 8 * j + (lane >> 3);
+        const int part = ((lane & 7) - row) & 7;   // 0..3 low codes, 4..5 high bits, 6 scales, 7 tail (d in its last 2 bytes)
+        off0 = part < 4 ? 16 * part : part < 6 ? 128 + 16 * (part - 4) : part == 6 ? 192 : 194;
+        hoff = part < 4 ? 64 : part < 6 ? 32 : 0;
+    }
+    static __device__ __forceinline__ Blk read_blk(const uint8_t* st, int row, int h) {
+        const uint4 hq = *reinterpret_cast<const uint4*>(st + pos(row, 4 + h));
+        return Blk{*reinterpret_cast<const uint4*>(st + pos(row, 6)), hq, hq,
+                   *reinterpret_cast<const uint16_t*>(st + pos(row, 7) + 14)};
+    }
+    static __device__ __forceinline__ Q read_q(const uint8_t* st, int row, int sl, int h) {
+        return Q{*reinterpret_cast<const uint4*>(st + pos(row, 2 * sl + h))};
+    }
+};
+
+constexpr int kNW6 = 3;                    // weight stages per wave
+constexpr int kAStage6 = kBM * 128;        // bytes per activation stage
+template <class D>
+constexpr size_t grouped6_lds() { return (size_t)D::kNA * kAStage6 + (size_t)4 * kNW6 * 64 * D::kRowStride + kBM * 4; }
+
+struct Grouped6Ctx {
+    uint8_t* lds;             // [kNA activation stages][4 waves x kNW6 weight stages][row scales]
+    const float* s_scale;
+    const uint8_t* asrc[4];   // the lane's four activation chunks of slice 0
+    int wave, lane, n0;
+    Tile t;
+};
+
+template <class D, bool DOWN, int M>
+__device__ __forceinline__ void grouped6_tile(const GroupedParams& p, const Grouped6Ctx& c, const uint8_t* const (&wsrc)[D::kNC],
+                                              const int (&whoff)[D::kNC]) {
+    constexpr int NA = D::kNA, NC = D::kNC, NW = kNW6;
+    constexpr int kWStage = 64 * D::kRowStride;
+    const int wave = c.wave, lane = c.lane, half = lane >> 5;
+    float16v acc0[M], acc1[M];
+#pragma unroll
+    for (int i = 0; i < M; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc0[i][r] = acc1[i][r] = 0.0f;
+    const int n_slices = p.K / kSlice, last = n_slices - 1, last_hs = (n_slices >> 1) - 1;
+    const uint32_t lds0 = lds_address(c.lds);
+    const uint32_t uwave = __builtin_amdgcn_readfirstlane(wave);
+    const uint32_t a_dst = lds0 + uwave * 4096;                                   // + stage * kAStage6 + q * 1024
+    const uint32_t w_dst = lds0 + NA * kAStage6 + uwave * (NW * kWStage);         // + stage * kWStage + j * 1024
+    const uint8_t* const w_lds = c.lds + NA * kAStage6 + wave * (NW * kWStage);
+    const uint8_t* const as0 = c.asrc[0];
+    const uint8_t* const as1 = c.asrc[1];
+    const uint8_t* const as2 = c.asrc[2];
+    const uint8_t* const as3 = c.asrc[3];
+    // Loads issued while slice s is contracted, a quarter after each k step so that the four waves
+    // do not queue up at the address unit together: part ks = (on even s the weight chunks
+    // 0..(NC+1)/2-1, on odd s the rest, one per k step) of half-step s/2 + NW - 1, then activation
+    // quarter ks of slice s + NA - 1.  The last load of a slice is its activation quarter 3.
+    constexpr int kWEven = (NC + 1) / 2;
+    auto issue_part = [&](int s, int odd, int ks) {   // odd = s & 1, a constant where this is called
+        const int hs = (s >> 1) + NW - 1;
+        const int j = odd ? kWEven + ks : ks;
+        if (hs >= 0 && j < (odd ? NC : kWEven)) {
+            const int hc = min(hs, last_hs);
+            const uint8_t* src = wsrc[0];
+            int ho = whoff[0];
+#pragma unroll
+            for (int q = 1; q < NC; q++)
+                if (q == j) {
+                    src = wsrc[q];
+                    ho = whoff[q];
+                }
+            dma16(src + (size_t)(hc >> 1) * D::kBlockBytes + ((hc & 1) ? ho : 0), w_dst + (uint32_t)(hs % NW) * kWStage + j * 1024);
+        }
+        const int sa = s + NA - 1;
+        if (sa >= 0) {
+            const uint8_t* src = ks == 0 ? as0 : ks == 1 ? as1 : ks == 2 ? as2 : as3;
+            dma16(src + (size_t)min(sa, last) * 128, a_dst + (uint32_t)(sa % NA) * kAStage6 + ks * 1024);
+        }
+    };
+#pragma unroll
+    for (int s = -2 * (NW - 1); s < 0; s++)
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) issue_part(s, s & 1, ks);
+
+    // operand reads: token 32 mi + (lane & 31), k chunk ks + 4 half, rotated by the token's low bits
+    const int x7 = lane & 7;
+    const int a_lane = (lane & 31) * 128;
+    int a_off[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) a_off[ks] = a_lane + (((ks + 4 * half) ^ x7) * 16);
+    const int row0 = lane & 31, row1 = 32 + (lane & 31);
+
+    // slice s (compile-time position j4 = s & 3 inside its super-block)
+    auto slice = [&](int s, auto j4c) {
+        constexpr int j4 = decltype(j4c)::value;
+        // loads younger than the last one this slice needs (activation quarter 3 of slice s, issued at
+        // the end of slice s - NA + 1): everything issued during the NA - 2 slices since
+        constexpr int kWOdd = NC - kWEven;
+        constexpr int kYoung = NA == 4 ? 8 + NC : 4 + ((j4 & 1) ? kWEven : kWOdd);
+        static_assert(NA == 3 || NA == 4, "the load counts above are written for these ring depths");
+        wait_loads_then_barrier<kYoung>();
+        const uint8_t* ap = c.lds + (s % NA) * kAStage6;
+        const uint8_t* wst = w_lds + ((s >> 1) % NW) * kWStage;
+        const typename D::Blk k0 = D::read_blk(wst, row0, half), k1 = D::read_blk(wst, row1, half);
+        const typename D::Q f0 = D::read_q(wst, row0, j4 & 1, half), f1 = D::read_q(wst, row1, j4 & 1, half);
+        uint4 a[M];
+#pragma unroll
+        for (int mi = 0; mi < M; mi++) a[mi] = *reinterpret_cast<const uint4*>(ap + a_off[0] + mi * 4096);
+        const typename D::Prep c0 = D::prep(k0, f0, j4, half), c1 = D::prep(k1, f1, j4, half);
+        uint4 b0 = D::chunk(k0, f0, c0, 0, j4), b1 = D::chunk(k1, f1, c1, 0, j4);
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) {
+            uint4 nb0 = b0, nb1 = b1;
+            if (ks < 3) {
+                nb0 = D::chunk(k0, f0, c0, ks + 1, j4);
+                nb1 = D::chunk(k1, f1, c1, ks + 1, j4);
+            }
+            issue_part(s, j4 & 1, ks);
+#pragma unroll
+            for (int mi = 0; mi < M; mi++) {
+                acc0[mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, a[mi]), __builtin_bit_cast(half8, b0),
+                                                                  acc0[mi], 0, 0, 0);
+                acc1[mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, a[mi]), __builtin_bit_cast(half8, b1),
+                                                                  acc1[mi], 0, 0, 0);
+                if (ks < 3) a[mi] = *reinterpret_cast<const uint4*>(ap + a_off[ks + 1] + mi * 4096);
+            }
+            b0 = nb0;
+            b1 = nb1;
+        }
+    };
+    for (int s0 = 0; s0 < n_slices; s0 += 4) {
+        slice(s0, std::integral_constant<int, 0>{});
+        slice(s0 + 1, std::integral_constant<int, 1>{});
+        slice(s0 + 2, std::integral_constant<int, 2>{});
+        slice(s0 + 3, std::integral_constant<int, 3>{});
+    }
+    // nothing may still be landing in LDS when the block ends (or another block takes over the CU's LDS)
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    tile_epilogue<DOWN, M>(p, c.t, c.n0, wave, lane, c.s_scale, acc0, acc1);
+}
+
+template <class D, bool DOWN>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void grouped_mfma6(GroupedParams p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds6[];
+    Grouped6Ctx c;
+    c.lds = lds6;
+    float* s_scale = reinterpret_cast<float*>(lds6 + grouped6_lds<D>() - kBM * 4);
+    c.s_scale = s_scale;
+    const int tid = threadIdx.x;
+    c.wave = tid >> 6;
+    c.lane = tid & 63;
+    int nt;
+    if (!find_item(p.offsets, p.n_expert, p.n_tiles_n, c.lane, c.t, nt)) return;
+    const Tile& t = c.t;
+    constexpr int kBN = DOWN ? 256 : 128;
+    c.n0 = nt * kBN;
+    // sources of the lane's chunks of the wave's weight stage (half-step 0)
+    const size_t row_bytes = (size_t)(p.K / D::kBlockElems) * D::kBlockBytes;
+    const uint8_t* wsrc[D::kNC];
+    int whoff[D::kNC];
+#pragma unroll
+    for (int j = 0; j < D::kNC; j++) {
+        int row, off0;
+        D::lane_chunk(j, c.lane, row, off0, whoff[j]);
+        const uint8_t* base;
+        int f;
+        if (DOWN) {
+            base = p.w0 + (size_t)t.e * p.w0_stride;
+            f = c.n0 + 64 * c.wave + row;
+        } else {
+            base = row < 32 ? p.w0 + (size_t)t.e * p.w0_stride : p.w1 + (size_t)t.e * p.w1_stride;
+            f = c.n0 + 32 * c.wave + (row & 31);
+        }
+        wsrc[j] = base + (size_t)min(f, p.N - 1) * row_bytes + off0;
+    }
+    // the lane's activation chunks: token 32 wave + 8 q + lane / 8, chunk (lane & 7) ^ (token & 7)
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const int tok = 32 * c.wave + 8 * q + (c.lane >> 3), kg = (c.lane & 7) ^ ((c.lane >> 3) & 7);
+        const int pr = t.p0 + min(tok, t.cnt - 1);
+        const size_t src_row = DOWN ? (size_t)pr : (size_t)(p.pair_src[pr] / p.n_used);
+        c.asrc[q] = reinterpret_cast<const uint8_t*>(p.a + src_row * p.K) + 16 * kg;
+    }
+    if (tid < kBM) {
+        const int pr = t.p0 + min(tid, t.cnt - 1);
+        s_scale[tid] = p.a_scale[DOWN ? pr : p.pair_src[pr] / p.n_used];
+    }
+    switch ((t.cnt + 31) >> 5) {
+        case 1: grouped6_tile<D, DOWN, 1>(p, c, wsrc, whoff); break;
+        case 2: grouped6_tile<D, DOWN, 2>(p, c, wsrc, whoff); break;
+        case 3: grouped6_tile<D, DOWN, 3>(p, c, wsrc, whoff); break;
+        default: grouped6_tile<D, DOWN, 4>(p, c, wsrc, whoff); break;
     }
 }
 
@@ -674,6 +937,21 @@ void rows_to_f16(hipStream_t s, const float* src, int rows, int n, _Float16* dst
     INFR_LAUNCH(rows_to_f16_kernel<F>, dim3(rows), dim3(256), 0, s, src, n, dst, scale);
 }
 
+template <class D, bool DOWN>
+void grouped6(hipStream_t s, const GroupedParams& p) {
+    const int bn = DOWN ? 256 : 128;
+    GroupedParams q = p;
+    q.n_tiles_n = (p.N + bn - 1) / bn;
+    const int max_tiles = p.n_pairs / kBM + (p.n_expert < p.n_pairs ? p.n_expert : p.n_pairs);
+    static bool attr_set = false;  // per instantiation
+    if (!attr_set) {
+        (void)hipFuncSetAttribute((const void*)grouped_mfma6<D, DOWN>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  (int)grouped6_lds<D>());
+        attr_set = true;
+    }
+    INFR_LAUNCH((grouped_mfma6<D, DOWN>), dim3((unsigned)((max_tiles * q.n_tiles_n + 7) & ~7)), dim3(256), grouped6_lds<D>(), s, q);   // whole rounds of the 8 XCDs
+}
+
 template <class F, bool DOWN>
 void grouped(hipStream_t s, const GroupedParams& p) {
     const int bn = DOWN ? 256 : 128;
@@ -686,7 +964,7 @@ void grouped(hipStream_t s, const GroupedParams& p) {
                                   (int)kGroupedLds);
         attr_set = true;
     }
-    INFR_LAUNCH((grouped_mfma<F, DOWN>), dim3((unsigned)max_tiles * q.n_tiles_n), dim3(256), kGroupedLds, s, q);
+    INFR_LAUNCH((grouped_mfma<F, DOWN>), dim3((unsigned)((max_tiles * q.n_tiles_n + 7) & ~7)), dim3(256), kGroupedLds, s, q);   // whole rounds of the 8 XCDs
 }
 
 }  // namespace
@@ -711,14 +989,14 @@ void launch_bucket(hipStream_t s, const int32_t* ids, int n_pairs, int n_expert,
 }
 
 void launch_grouped_gate_up(hipStream_t s, int dt, const GroupedParams& p) {
-    if (dt == INFR_Q4K) grouped<MQ4K, false>(s, p);
-    else if (dt == INFR_Q6K) grouped<MQ6K, false>(s, p);
+    if (dt == INFR_Q4K) grouped6<D4K, false>(s, p);
+    else if (dt == INFR_Q6K) grouped6<D6K, false>(s, p);
     else grouped<MQ80, false>(s, p);
 }
 
 void launch_grouped_down(hipStream_t s, int dt, const GroupedParams& p) {
-    if (dt == INFR_Q4K) grouped<MQ4K, true>(s, p);
-    else if (dt == INFR_Q6K) grouped<MQ6K, true>(s, p);
+    if (dt == INFR_Q4K) grouped6<D4K, true>(s, p);
+    else if (dt == INFR_Q6K) grouped6<D6K, true>(s, p);
     else grouped<MQ80, true>(s, p);
 }
 
