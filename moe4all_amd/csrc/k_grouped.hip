@@ -9,8 +9,9 @@
 //                         an integer contract and is reproduced exactly).
 //   rows_to_f16_kernel    activation rows -> f16 with one power-of-two scale per row (so any f32
 //                         magnitude fits), laid out in the k order the weight format unpacks to.
-//   grouped_mfma<F,DOWN>  per (expert, 128-token tile, 128/256-feature tile): quantised weight rows
-//                         are unpacked to f16 straight into LDS with packed 16-bit arithmetic, the
+//   grouped_mfma6<D,DOWN> per (expert, 128-token tile, 128/256-feature tile): the raw quantised bytes
+//                         of the tile's weight rows are copied into LDS, every lane unpacks its
+//                         row's codes to f16 in registers with packed 16-bit arithmetic, the
 //                         contraction runs on v_mfma_f32_32x32x16_f16 with f32 accumulation;
 //                         epilogue = SwiGLU (gate/up) or plain scaled store (down).
 //   unbucket_combine      dst[row] = sum over ranks (rank order, separate mul and add,
@@ -36,7 +37,6 @@ namespace {
 
 constexpr int kBM = 128;        // token rows per tile
 constexpr int kSlice = 64;      // k elements per LDS stage
-constexpr int kAStride = 129;   // 16-byte chunks per k-group of the activation tile (+1: bank spread)
 
 __device__ __forceinline__ half2v as_h2(uint32_t v) { return __builtin_bit_cast(half2v, v); }
 __device__ __forceinline__ uint32_t as_u32(half2v v) { return __builtin_bit_cast(uint32_t, v); }
@@ -52,14 +52,14 @@ __device__ __forceinline__ half2v unbias(uint32_t magic_pair, float bias) { retu
 // instruction's lane halves split them: lanes 0..31 (half 0) own chunks 0..3, lanes 32..63 own
 // chunks 4..7, and k-step ks of the slice contracts chunk ks of each half.  Four slices make one
 // 256-element step (a K-quant super-block); what is shared by the four slices is fetched once:
-//   load_blk(row, b, h)     per-256 part (scales, high bits) half h needs of step b
-//   load_q(row, s, h)       the code bytes half h needs of virtual slice s
+//   Blk                     per-256 part (scales, high bits) half h needs of a step
+//   Q                       the code bytes half h needs of virtual slice s
 //   prep(blk, q, s, h)      per-slice scale constants
 //   chunk(blk, q, c, ks, s) operand chunk 4h + ks as 8 f16
 //   chunk_src()             for virtual chunk c of a row, the two real offsets whose float4s feed
 //                           it and whether the 4 elements of each come out in the order 0,2,1,3
 struct MQ4K {
-    static constexpr int kDt = INFR_Q4K, kBlockElems = 256, kBlockBytes = 144;
+    static constexpr int kBlockElems = 256, kBlockBytes = 144;
     struct Blk {
         uint4 hdr;   // d, dmin, 12 packed 6-bit scales / mins
     };
@@ -70,12 +70,6 @@ struct MQ4K {
         half2v s_lo, n_lo, s_hi, n_hi;
         uint32_t magic;
     };
-    static __device__ __forceinline__ Blk load_blk(const uint8_t* row, int b, int) {
-        return Blk{*reinterpret_cast<const uint4*>(row + (size_t)b * 144)};
-    }
-    static __device__ __forceinline__ Q load_q(const uint8_t* row, int s, int h) {
-        return Q{*reinterpret_cast<const uint4*>(row + (size_t)(s >> 2) * 144 + 16 + (s & 3) * 32 + 16 * h)};
-    }
     // scales[i] of the 12 packed bytes, i in 0..11, without branches
     static __device__ __forceinline__ uint32_t scale_byte(const uint4& hdr, int i) {
         const uint64_t lo = ((uint64_t)hdr.z << 32) | hdr.y;   // bytes 0..7
@@ -119,7 +113,7 @@ struct MQ4K {
 };
 
 struct MQ6K {
-    static constexpr int kDt = INFR_Q6K, kBlockElems = 256, kBlockBytes = 210;
+    static constexpr int kBlockElems = 256, kBlockBytes = 210;
     // virtual slice t of a block: t = 2*half128 + ab; ab picks ql bytes [32ab, 32ab+32) of the
     // 128-element half; their low nibbles are elements [32ab, 32ab+32), their high nibbles +64.
     // The 2-bit tops of both ab of a half share the same qh bytes.
@@ -134,14 +128,6 @@ struct MQ6K {
     struct Prep {
         half2v s_lo, s_hi;
     };
-    static __device__ __forceinline__ Blk load_blk(const uint8_t* row, int b, int h) {
-        const uint8_t* blk = row + (size_t)b * 210;
-        return Blk{ldu<uint4>(blk + 192), ldu<uint4>(blk + 128 + 16 * h), ldu<uint4>(blk + 160 + 16 * h), ldu<uint16_t>(blk + 208)};
-    }
-    static __device__ __forceinline__ Q load_q(const uint8_t* row, int s, int h) {
-        const uint8_t* blk = row + (size_t)(s >> 2) * 210;
-        return Q{ldu<uint4>(blk + 64 * ((s >> 1) & 1) + 32 * (s & 1) + 16 * h)};
-    }
     static __device__ __forceinline__ Prep prep(const Blk& blk, const Q&, int s, int h) {
         // the lane's four chunks are 16 consecutive elements: one scale for the low codes
         // (scales[8hh + 2ab + h]) and one for the high codes (+4)
@@ -172,7 +158,7 @@ struct MQ6K {
 };
 
 struct MQ80 {
-    static constexpr int kDt = INFR_Q8_0, kBlockElems = 32, kBlockBytes = 34;
+    static constexpr int kBlockElems = 32, kBlockBytes = 34;
     struct Blk {};
     struct Q {
         uint4 qa, qb;  // the 32 codes of block h of the slice
@@ -181,11 +167,6 @@ struct MQ80 {
     struct Prep {
         half2v d;
     };
-    static __device__ __forceinline__ Blk load_blk(const uint8_t*, int, int) { return Blk{}; }
-    static __device__ __forceinline__ Q load_q(const uint8_t* row, int s, int h) {
-        const uint8_t* p = row + (size_t)s * 68 + 34 * h;
-        return Q{ldu<uint4>(p + 2), ldu<uint4>(p + 18), ldu<uint16_t>(p)};
-    }
     static __device__ __forceinline__ Prep prep(const Blk&, const Q& f, int, int) { return Prep{splat(f16_bits_to_f32(f.d))}; }
     static __device__ __forceinline__ uint4 chunk(const Blk&, const Q& f, const Prep& c, int ks, int) {
         const uint32_t v0 = ks == 0 ? f.qa.x : ks == 1 ? f.qa.z : ks == 2 ? f.qb.x : f.qb.z;
@@ -479,183 +460,12 @@ __device__ __forceinline__ void tile_epilogue(const GroupedParams& p, const Tile
 }
 
 // --------------------------------------------------------------------------------------------
-// 256 threads = 4 waves, one wave per SIMD (so each may use the whole 512-entry register file:
-// the accumulators sit in AccVGPRs, deep prefetch rings in VGPRs).  Per 64-k slice every wave
-//   * contracts the slice: wave w owns two 32-feature column tiles (gate w / up w, or down
-//     2w / 2w+1) against M 32-token row tiles.  Each lane fetches the quantised bytes of ITS
-//     weight row and k half straight from global memory (kWRing slices ahead) and unpacks them in
-//     registers into exactly the operand fragments it feeds to the matrix instruction, so the
-//     weights never pass through LDS; unpacking (VALU) is issued between the MFMAs in flight;
-//   * copies its share of the next slice's 128-token x 64-k activation tile (loaded kARing slices
-//     ahead) into the LDS buffer nobody is reading.
-// One barrier per slice.  Every global load is unconditional (slice indices are clamped) and the
-// steady-state loop is straight-line code, so the wait counters the compiler inserts only wait for
-// the slice that is needed.  M is a template parameter so that the k loop has no branches.
-constexpr int kABuf = 8 * kAStride;                            // 16-byte chunks per LDS buffer
-constexpr size_t kGroupedLds = (size_t)2 * kABuf * 16 + kBM * 4;
-constexpr int kWRing = 4, kARing = 2, kUnroll = 4;             // kUnroll = lcm(kWRing, kARing, 2)
-
-struct GroupedCtx {
-    uint4* sA;   // [2][kABuf]
-    const float* s_scale;
-    const uint8_t* wrow0;   // weight rows of the lane's two column tiles
-    const uint8_t* wrow1;
-    const uint4* asrc[4];   // the thread's four activation chunks
-    int tid, wave, lane, n0;
-    Tile t;
-};
-
-template <class F, bool DOWN, int M>
-__device__ __forceinline__ void grouped_tile(const GroupedParams& p, const GroupedCtx& c) {
-    const int tid = c.tid, wave = c.wave, lane = c.lane, half = lane >> 5;
-    float16v acc0[M], acc1[M];
-#pragma unroll
-    for (int i = 0; i < M; i++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) acc0[i][r] = acc1[i][r] = 0.0f;
-    const int n_slices = p.K / kSlice;   // a multiple of kUnroll (K is a multiple of 256)
-    const int last = n_slices - 1;
-    const uint4* fa = c.sA + (lane & 31) + 4 * half * kAStride;
-
-    // rings (named variables, so that they stay in registers): code bytes of slices s..s+3 in
-    // qa/qb/qc/qd by s % 4, the per-256 parts of the current and of the next 256-element step,
-    // activation chunks of slices s+1, s+2 in ae (even slice) / ao (odd)
-    static_assert(kWRing == 4 && kARing == 2 && kUnroll == 4, "the slice loop below is written for these depths");
-    const int last_blk = last >> 2;
-    typename F::Blk bc0 = F::load_blk(c.wrow0, 0, half), bc1 = F::load_blk(c.wrow1, 0, half);
-    typename F::Blk bn0 = F::load_blk(c.wrow0, min(1, last_blk), half), bn1 = F::load_blk(c.wrow1, min(1, last_blk), half);
-    typename F::Q qa0 = F::load_q(c.wrow0, 0, half), qa1 = F::load_q(c.wrow1, 0, half);
-    typename F::Q qb0 = F::load_q(c.wrow0, 1, half), qb1 = F::load_q(c.wrow1, 1, half);
-    typename F::Q qc0 = F::load_q(c.wrow0, 2, half), qc1 = F::load_q(c.wrow1, 2, half);
-    typename F::Q qd0 = F::load_q(c.wrow0, 3, half), qd1 = F::load_q(c.wrow1, 3, half);
-    const uint4 *as0 = c.asrc[0], *as1 = c.asrc[1], *as2 = c.asrc[2], *as3 = c.asrc[3];
-    struct A4 {
-        uint4 q0, q1, q2, q3;
-    };
-    auto load_a = [&](int sl) {
-        const int o = min(sl, last) * (kSlice / 8);
-        return A4{as0[o], as1[o], as2[o], as3[o]};
-    };
-    A4 ae = load_a(0), ao = load_a(1);
-    // (all four chunks are staged whatever M is: rows past the tile's tokens repeat its last token)
-    uint4* const st0 = c.sA + (tid & 7) * kAStride + (tid >> 3);   // chunk q of this thread sits 32 tokens further
-    auto stage = [&](int s, A4& a4) {   // slice s -> buffer s & 1, then refill with slice s + kARing
-        uint4* d = st0 + (s & 1) * kABuf;
-        d[0] = a4.q0;
-        d[32] = a4.q1;
-        d[64] = a4.q2;
-        d[96] = a4.q3;
-        a4 = load_a(s + kARing);
-    };
-    // contracts slice s from LDS buffer s & 1 with the code bytes in (f0, f1), stages slice s + 1,
-    // refills the code bytes with slice s + kWRing
-    auto slice = [&](int s, typename F::Q& f0, typename F::Q& f1, A4& a_next) {
-        const uint4* ap = fa + (s & 1) * kABuf;
-        const typename F::Prep c0 = F::prep(bc0, f0, s, half), c1 = F::prep(bc1, f1, s, half);
-        // software pipeline over the four k-steps: as soon as the two matrix instructions that
-        // use activation fragment mi are issued, the fragment register is reloaded for step
-        // ks + 1, and the unpacking of step ks + 1's weight chunks is spread between them
-        uint4 b0 = F::chunk(bc0, f0, c0, 0, s), b1 = F::chunk(bc1, f1, c1, 0, s);
-        uint4 a[M];
-#pragma unroll
-        for (int mi = 0; mi < M; mi++) a[mi] = ap[mi * 32];
-#pragma unroll
-        for (int ks = 0; ks < 4; ks++) {
-            uint4 nb0 = b0, nb1 = b1;
-            if (ks < 3) {
-                nb0 = F::chunk(bc0, f0, c0, ks + 1, s);
-                nb1 = F::chunk(bc1, f1, c1, ks + 1, s);
-            } else {
-                stage(s + 1, a_next);
-                f0 = F::load_q(c.wrow0, min(s + kWRing, last), half);
-                f1 = F::load_q(c.wrow1, min(s + kWRing, last), half);
-            }
-#pragma unroll
-            for (int mi = 0; mi < M; mi++) {
-                acc0[mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, a[mi]), __builtin_bit_cast(half8, b0),
-                                                                  acc0[mi], 0, 0, 0);
-                acc1[mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, a[mi]), __builtin_bit_cast(half8, b1),
-                                                                  acc1[mi], 0, 0, 0);
-                if (ks < 3) a[mi] = ap[(ks + 1) * kAStride + mi * 32];
-            }
-            b0 = nb0;
-            b1 = nb1;
-        }
-    };
-    stage(0, ae);
-    __syncthreads();
-    for (int s0 = 0; s0 < n_slices; s0 += kUnroll) {
-        slice(s0, qa0, qa1, ao);
-        __syncthreads();
-        slice(s0 + 1, qb0, qb1, ae);
-        __syncthreads();
-        slice(s0 + 2, qc0, qc1, ao);
-        __syncthreads();
-        slice(s0 + 3, qd0, qd1, ae);
-        __syncthreads();
-        bc0 = bn0;
-        bc1 = bn1;
-        bn0 = F::load_blk(c.wrow0, min((s0 >> 2) + 2, last_blk), half);
-        bn1 = F::load_blk(c.wrow1, min((s0 >> 2) + 2, last_blk), half);
-    }
-
-    tile_epilogue<DOWN, M>(p, c.t, c.n0, wave, lane, c.s_scale, acc0, acc1);
-}
-
-template <class F, bool DOWN>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void grouped_mfma(GroupedParams p) {
-    extern __shared__ uint4 lds[];
-    GroupedCtx c;
-    c.sA = lds;
-    float* s_scale = reinterpret_cast<float*>(lds + 2 * kABuf);
-    c.s_scale = s_scale;
-    const int tid = c.tid = threadIdx.x;
-    c.wave = tid >> 6;
-    c.lane = tid & 63;
-    // one tile per block (a persistent loop over tiles was measured: no faster, and the static
-    // assignment balances the ragged tiles worse than the hardware dispatcher does)
-    {
-        int nt;
-        if (!find_item(p.offsets, p.n_expert, p.n_tiles_n, c.lane, c.t, nt)) return;
-        const Tile& t = c.t;
-        constexpr int kBN = DOWN ? 256 : 128;
-        c.n0 = nt * kBN;
-
-        // the lane's weight rows
-        const size_t row_bytes = (size_t)(p.K / F::kBlockElems) * F::kBlockBytes;
-        if (DOWN) {
-            const int f0 = min(c.n0 + 64 * c.wave + (c.lane & 31), p.N - 1), f1 = min(c.n0 + 64 * c.wave + 32 + (c.lane & 31), p.N - 1);
-            const uint8_t* base = p.w0 + (size_t)t.e * p.w0_stride;
-            c.wrow0 = base + (size_t)f0 * row_bytes;
-            c.wrow1 = base + (size_t)f1 * row_bytes;
-        } else {
-            const int f = min(c.n0 + 32 * c.wave + (c.lane & 31), p.N - 1);
-            c.wrow0 = p.w0 + (size_t)t.e * p.w0_stride + (size_t)f * row_bytes;
-            c.wrow1 = p.w1 + (size_t)t.e * p.w1_stride + (size_t)f * row_bytes;
-        }
-        // the thread's activation chunks
-#pragma unroll
-        for (int q = 0; q < 4; q++) {
-            const int cc = tid + 256 * q, tok = cc >> 3, kg = cc & 7;
-            const int pr = t.p0 + min(tok, t.cnt - 1);
-            const size_t src_row = DOWN ? (size_t)pr : (size_t)(p.pair_src[pr] / p.n_used);
-            c.asrc[q] = reinterpret_cast<const uint4*>(p.a + src_row * p.K) + kg;
-        }
-        if (tid < kBM) {
-            const int pr = t.p0 + min(tid, t.cnt - 1);
-            s_scale[tid] = p.a_scale[DOWN ? pr : p.pair_src[pr] / p.n_used];
-        }
-        switch ((t.cnt + 31) >> 5) {
-            case 1: grouped_tile<F, DOWN, 1>(p, c); break;
-            case 2: grouped_tile<F, DOWN, 2>(p, c); break;
-            case 3: grouped_tile<F, DOWN, 3>(p, c); break;
-            default: grouped_tile<F, DOWN, 4>(p, c); break;
-        }
-    }
-}
-
-// --------------------------------------------------------------------------------------------
-// K-quant variant with every k-loop load going straight from global memory into LDS
+// Grouped GEMM: 256 threads = 4 waves, one wave per SIMD (so each may use the whole 512-entry
+// register file: the 128 accumulators sit in AccVGPRs).  Per 64-k slice every wave contracts the
+// slice for its two 32-feature column tiles (gate w / up w, or down 2w / 2w+1) against M 32-token
+// row tiles; each lane unpacks the quantised bytes of ITS weight row and k half in registers into
+// exactly the operand fragments it feeds to the matrix instruction.  M is a template parameter so
+// that the k loop has no branches.  Every k-loop load goes straight from global memory into LDS
 // (global_load_lds_dwordx4: lane i of a wave's load deposits its 16 bytes at base + 16 i), so that
 // each load instruction covers whole cache lines and nothing is staged in registers:
 //   * activation stage = the tile's 128 tokens x one 64-k slice (16 KB), token-major, the eight
@@ -685,7 +495,7 @@ __device__ __forceinline__ uint32_t lds_address(const void* p) {
 }
 
 struct D4K : MQ4K {
-    static constexpr int kNC = 5, kRowStride = 80, kNA = 4;
+    static constexpr int kNC = 5, kRowStride = 80, kNA = 4, kStepBytes = 144;   // kStepBytes: a row's bytes per 256 k
     // chunk `64 j + lane` of a weight stage: which staged row, where in the super-block its 16
     // bytes start for the first half, and how far the second half's lie behind
     static __device__ __forceinline__ void lane_chunk(int j, int lane, int& row, int& off0, int& hoff) {
@@ -704,7 +514,7 @@ struct D4K : MQ4K {
 };
 
 struct D6K : MQ6K {
-    static constexpr int kNC = 8, kRowStride = 128, kNA = 3;
+    static constexpr int kNC = 8, kRowStride = 128, kNA = 3, kStepBytes = 210;
     static __device__ __forceinline__ int pos(int row, int part) { return row * kRowStride + ((part + row) & 7) * 16; }
     static __device__ __forceinline__ void lane_chunk(int j, int lane, int& row, int& off0, int& hoff) {
         row = 8 * j + (lane >> 3);
@@ -719,6 +529,25 @@ struct D6K : MQ6K {
     }
     static __device__ __forceinline__ Q read_q(const uint8_t* st, int row, int sl, int h) {
         return Q{*reinterpret_cast<const uint4*>(st + pos(row, 2 * sl + h))};
+    }
+};
+
+// Q8_0: a half-step is four 34-byte blocks = 136 bytes of a row: eight chunks for bytes 0..127 and a
+// ninth for bytes 120..135 (the last block's upper 16 codes, so that nothing past the row is read).
+struct D80 : MQ80 {
+    static constexpr int kNC = 9, kRowStride = 144, kNA = 3, kStepBytes = 272;
+    static __device__ __forceinline__ void lane_chunk(int j, int lane, int& row, int& off0, int& hoff) {
+        const int c = 64 * j + lane;
+        row = c / 9;
+        const int part = c - 9 * row;
+        off0 = part < 8 ? 16 * part : 120;
+        hoff = 136;
+    }
+    static __device__ __forceinline__ Blk read_blk(const uint8_t*, int, int) { return Blk{}; }
+    static __device__ __forceinline__ Q read_q(const uint8_t* st, int row, int sl, int h) {
+        const int i = 2 * sl + h;   // block of the half-step
+        const uint8_t* r = st + row * kRowStride;
+        return Q{ldu<uint4>(r + 34 * i + 2), ldu<uint4>(r + (i == 3 ? 128 : 34 * i + 18)), ldu<uint16_t>(r + 34 * i)};
     }
 };
 
@@ -759,23 +588,21 @@ __device__ __forceinline__ void grouped6_tile(const GroupedParams& p, const Grou
     // Loads issued while slice s is contracted, a quarter after each k step so that the four waves
     // do not queue up at the address unit together: part ks = (on even s the weight chunks
     // 0..(NC+1)/2-1, on odd s the rest, one per k step) of half-step s/2 + NW - 1, then activation
-    // quarter ks of slice s + NA - 1.  The last load of a slice is its activation quarter 3.
+    // quarter ks of slice s + NA - 1 (a fifth weight chunk of a slice goes with k step 0).  The last load
+    // of a slice is its activation quarter 3.
     constexpr int kWEven = (NC + 1) / 2;
-    auto issue_part = [&](int s, int odd, int ks) {   // odd = s & 1, a constant where this is called
+    auto issue_w = [&](int s, int j) {
         const int hs = (s >> 1) + NW - 1;
-        const int j = odd ? kWEven + ks : ks;
-        if (hs >= 0 && j < (odd ? NC : kWEven)) {
-            const int hc = min(hs, last_hs);
-            const uint8_t* src = wsrc[0];
-            int ho = whoff[0];
+        if (hs < 0) return;
+        const int hc = min(hs, last_hs);
+        dma16(wsrc[j] + (size_t)(hc >> 1) * D::kStepBytes + ((hc & 1) ? whoff[j] : 0),
+              w_dst + (uint32_t)(hs % NW) * kWStage + j * 1024);
+    };
+    auto issue_part = [&](int s, int odd, int ks) {   // odd = s & 1; odd and ks are constants where this is called
+        const int lo = odd ? kWEven : 0, hi = odd ? NC : kWEven;
 #pragma unroll
-            for (int q = 1; q < NC; q++)
-                if (q == j) {
-                    src = wsrc[q];
-                    ho = whoff[q];
-                }
-            dma16(src + (size_t)(hc >> 1) * D::kBlockBytes + ((hc & 1) ? ho : 0), w_dst + (uint32_t)(hs % NW) * kWStage + j * 1024);
-        }
+        for (int j = 0; j < NC; j++)
+            if (j >= lo && j < hi && ((j - lo) & 3) == ks) issue_w(s, j);
         const int sa = s + NA - 1;
         if (sa >= 0) {
             const uint8_t* src = ks == 0 ? as0 : ks == 1 ? as1 : ks == 2 ? as2 : as3;
@@ -952,26 +779,11 @@ void grouped6(hipStream_t s, const GroupedParams& p) {
     INFR_LAUNCH((grouped_mfma6<D, DOWN>), dim3((unsigned)((max_tiles * q.n_tiles_n + 7) & ~7)), dim3(256), grouped6_lds<D>(), s, q);   // whole rounds of the 8 XCDs
 }
 
-template <class F, bool DOWN>
-void grouped(hipStream_t s, const GroupedParams& p) {
-    const int bn = DOWN ? 256 : 128;
-    GroupedParams q = p;
-    q.n_tiles_n = (p.N + bn - 1) / bn;
-    const int max_tiles = p.n_pairs / kBM + (p.n_expert < p.n_pairs ? p.n_expert : p.n_pairs);
-    static bool attr_set = false;  // per instantiation
-    if (!attr_set) {
-        (void)hipFuncSetAttribute((const void*)grouped_mfma<F, DOWN>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  (int)kGroupedLds);
-        attr_set = true;
-    }
-    INFR_LAUNCH((grouped_mfma<F, DOWN>), dim3((unsigned)((max_tiles * q.n_tiles_n + 7) & ~7)), dim3(256), kGroupedLds, s, q);   // whole rounds of the 8 XCDs
-}
-
 }  // namespace
 
 bool grouped_supported(int dt, int k) {
-    // the k loop runs in groups of kUnroll 64-element slices
-    if (k <= 0 || (k % (kSlice * kUnroll)) != 0) return false;
+    // the k loop runs in groups of four 64-element slices (one K-quant super-block)
+    if (k <= 0 || (k % (kSlice * 4)) != 0) return false;
     return dt == INFR_Q4K || dt == INFR_Q6K || dt == INFR_Q8_0;
 }
 
@@ -991,13 +803,13 @@ void launch_bucket(hipStream_t s, const int32_t* ids, int n_pairs, int n_expert,
 void launch_grouped_gate_up(hipStream_t s, int dt, const GroupedParams& p) {
     if (dt == INFR_Q4K) grouped6<D4K, false>(s, p);
     else if (dt == INFR_Q6K) grouped6<D6K, false>(s, p);
-    else grouped<MQ80, false>(s, p);
+    else grouped6<D80, false>(s, p);
 }
 
 void launch_grouped_down(hipStream_t s, int dt, const GroupedParams& p) {
     if (dt == INFR_Q4K) grouped6<D4K, true>(s, p);
     else if (dt == INFR_Q6K) grouped6<D6K, true>(s, p);
-    else grouped<MQ80, true>(s, p);
+    else grouped6<D80, true>(s, p);
 }
 
 void launch_unbucket_combine(hipStream_t s, const float* y, const int32_t* slot_pair, const float* weights, int rows,
