@@ -889,7 +889,13 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
             gp.act = ga.act; gp.has_clamp = (int)ga.has_swiglu_clamp; gp.clamp = ga.swiglu_clamp;
             gp.h = (float*)ptr[ga.dst]; gp.n_cu = n_cu;
             Timed t(be, "linear_gate_up_act");
-            infr::launch_moe_gate_up(s, gp);
+            if (gp.rows >= 2 && infr::bucketed_rows_supported(gp.gate_dt, gp.ne)) {
+                // several rows: one bucket of the bucketed kernel, two rows share each weight row
+                gp.h = (float*)ptr[ga.dst];
+                infr::launch_moe_gate_up_bucketed(s, gp);
+            } else {
+                infr::launch_moe_gate_up(s, gp);
+            }
             continue;
         }
         if (fz.kind == infr_hip_plan::kLinearAdd) {
@@ -1017,11 +1023,21 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                         infr::launch_bucket(s, sc.ids, pairs, (int)m.n_expert, sc.offsets, sc.pair_src, sc.slot_pair);
                     }
                     gp.bk_offsets = sc.offsets; gp.bk_pair_src = sc.pair_src; gp.y = sc.y;
+                    gp.max_bucket = m.expert_ids == INFR_NO_TENSOR ? rows : pairs;   // given ids may repeat an expert in a row
                     {
                         Timed t(be, "moe_gate_up_bucketed");
                         infr::launch_moe_gate_up_bucketed(s, gp);
                     }
                     gp.x = sc.h;
+                    if (infr::moe_down_is_fast(gp)) {
+                        // h is in flat (row, rank) order, which is what the per-token down kernel reads: it
+                        // streams each pair's expert rows and combines in its epilogue, measured faster
+                        // than the bucketed down kernel + combine up to the batched threshold
+                        gp.x = nullptr;
+                        Timed t(be, "moe_down_combine");
+                        infr::launch_moe_down_combine(s, gp);
+                        break;
+                    }
                     {
                         Timed t(be, "moe_down_bucketed");
                         infr::launch_moe_down_bucketed(s, gp);

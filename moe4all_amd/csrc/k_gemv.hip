@@ -896,7 +896,8 @@ __global__ __launch_bounds__(256) void moe_gate_up_bucketed(MoeGemvParams p, int
     __shared__ uint64_t s_tab[32];
     __shared__ float s_g[4][T][64], s_u[4][T][64];
     const int e = blockIdx.y;
-    const int t0 = p.bk_offsets[e] + blockIdx.z * T, t1 = p.bk_offsets[e + 1];
+    // without tables there is one bucket holding every row in order (a dense layer)
+    const int t0 = (p.bk_offsets ? p.bk_offsets[e] : 0) + blockIdx.z * T, t1 = p.bk_offsets ? p.bk_offsets[e + 1] : p.rows;
     if (t0 >= t1) return;
     const int nt = min(T, t1 - t0);
     const int f0 = blockIdx.x * ft;
@@ -911,7 +912,7 @@ __global__ __launch_bounds__(256) void moe_gate_up_bucketed(MoeGemvParams p, int
     const float* xrows[T];
 #pragma unroll
     for (int tau = 0; tau < T; tau++) {
-        pair[tau] = p.bk_pair_src[t0 + min(tau, nt - 1)];
+        pair[tau] = p.bk_pair_src ? p.bk_pair_src[t0 + min(tau, nt - 1)] : t0 + min(tau, nt - 1);
         xrows[tau] = p.x + (size_t)(pair[tau] / p.n_used) * p.ne;
     }
     const uint8_t* gbank = p.gate + (size_t)e * p.gate_stride + (size_t)f0 * row_bytes;
@@ -977,7 +978,7 @@ template <class F, int U, int T>
 __global__ __launch_bounds__(256) void moe_down_bucketed(MoeGemvParams p, int ot) {
     extern __shared__ uint32_t dyn_lds[];
     const int e = blockIdx.y;
-    const int t0 = p.bk_offsets[e] + blockIdx.z * T, t1 = p.bk_offsets[e + 1];
+    const int t0 = (p.bk_offsets ? p.bk_offsets[e] : 0) + blockIdx.z * T, t1 = p.bk_offsets ? p.bk_offsets[e + 1] : p.rows;
     if (t0 >= t1) return;
     const int nt = min(T, t1 - t0);
     const int o0 = blockIdx.x * ot;
@@ -994,7 +995,7 @@ __global__ __launch_bounds__(256) void moe_down_bucketed(MoeGemvParams p, int ot
     const float* xrows[T];
 #pragma unroll
     for (int tau = 0; tau < T; tau++) {
-        pair[tau] = p.bk_pair_src[t0 + min(tau, nt - 1)];
+        pair[tau] = p.bk_pair_src ? p.bk_pair_src[t0 + min(tau, nt - 1)] : t0 + min(tau, nt - 1);
         xrows[tau] = p.x + (size_t)pair[tau] * p.nff;   // h of the pair
     }
     typename F::Raw raw[U];
@@ -1027,7 +1028,10 @@ __global__ __launch_bounds__(256) void moe_down_bucketed(MoeGemvParams p, int ot
             for (int tau = 0; tau < T; tau++) {
                 float v = y[u][tau];
                 if (p.down_scale) v = __fmul_rn(v, ds);
-                if (o < ocount && tau < nt && pl.writer()) p.y[(size_t)pair[tau] * p.ne + o0 + o] = v;
+                if (o < ocount && tau < nt && pl.writer()) {
+                    const size_t oi = (size_t)pair[tau] * p.ne + o0 + o;
+                    p.y[oi] = p.addend ? __fadd_rn(p.addend[oi], v) : v;
+                }
             }
             raw[u] = nxt[u];
         }
@@ -1039,34 +1043,37 @@ constexpr int kBucketT = 2;   // tokens a block of the bucketed kernels handles 
 template <class F>
 static void gate_up_bucketed(hipStream_t s, const MoeGemvParams& p) {
     const int rw = 64 / (p.ne / F::kBlockElems * F::kLPB);
-    // about four blocks per CU if every expert had one chunk of tokens
-    int tiles = max(1, 4 * p.n_cu / max(p.n_expert, 1));
+    // about four blocks per CU if every expert had one chunk of tokens (dense: the chunks of the one bucket)
+    const int groups = p.bk_offsets ? max(p.n_expert, 1) : ceil_div(p.rows, kBucketT);
+    int tiles = max(1, 4 * p.n_cu / groups);
     int ft = ceil_div(p.nff, tiles);
-    ft = ceil_div(ft, 4 * rw) * 4 * rw;
-    dim3 grid(ceil_div(p.nff, ft), p.n_expert, ceil_div(p.rows, kBucketT)), block(256);
+    ft = ceil_div(ft, 4 * rw * 2) * 4 * rw * 2;   // whole rounds of 4 waves x U = 2 row groups
+    dim3 grid(ceil_div(p.nff, ft), p.n_expert, ceil_div(p.max_bucket ? p.max_bucket : p.rows, kBucketT)), block(256);
     INFR_LAUNCH((moe_gate_up_bucketed<F, 2, kBucketT>), grid, block, kBucketT * cells_bytes(p.ne), s, p, ft);
 }
 
 template <class F>
 static void down_bucketed(hipStream_t s, const MoeGemvParams& p) {
     const int rw = 64 / (p.nff / F::kBlockElems * F::kLPB);
-    int tiles = max(1, 4 * p.n_cu / max(p.n_expert, 1));
+    const int groups = p.bk_offsets ? max(p.n_expert, 1) : ceil_div(p.rows, kBucketT);
+    int tiles = max(1, 4 * p.n_cu / groups);
     int ot = ceil_div(p.ne, tiles);
-    ot = ceil_div(ot, 4 * rw) * 4 * rw;
-    dim3 grid(ceil_div(p.ne, ot), p.n_expert, ceil_div(p.rows, kBucketT)), block(256);
+    ot = ceil_div(ot, 4 * rw * 4) * 4 * rw * 4;   // whole rounds of 4 waves x U = 4 row groups
+    dim3 grid(ceil_div(p.ne, ot), p.n_expert, ceil_div(p.max_bucket ? p.max_bucket : p.rows, kBucketT)), block(256);
     INFR_LAUNCH((moe_down_bucketed<F, 4, kBucketT>), grid, block, kBucketT * cells_bytes(p.nff), s, p, ot);
+}
+
+bool bucketed_rows_supported(int dt, int k) {
+    if (kBucketT * cells_bytes(k) > 48 * 1024) return false;   // the staged cells must fit the default LDS window
+    if (dt == INFR_Q4K) return fast_ok<Q4KFmt>(k);
+    if (dt == INFR_Q6K) return fast_ok<Q6KFmt>(k);
+    if (dt == INFR_Q8_0) return fast_ok<Q80Fmt>(k);
+    return false;
 }
 
 bool moe_bucketed_supported(const MoeGemvParams& p) {
     if (p.gate_dt != p.up_dt || p.fused_gate_up) return false;
-    auto ok = [](int dt, int k) {
-        if (kBucketT * cells_bytes(k) > 48 * 1024) return false;   // the staged cells must fit the default LDS window
-        if (dt == INFR_Q4K) return fast_ok<Q4KFmt>(k);
-        if (dt == INFR_Q6K) return fast_ok<Q6KFmt>(k);
-        if (dt == INFR_Q8_0) return fast_ok<Q80Fmt>(k);
-        return false;
-    };
-    return ok(p.gate_dt, p.ne) && ok(p.down_dt, p.nff);
+    return bucketed_rows_supported(p.gate_dt, p.ne) && bucketed_rows_supported(p.down_dt, p.nff);
 }
 
 void launch_moe_gate_up_bucketed(hipStream_t s, const MoeGemvParams& p) {
@@ -1158,8 +1165,29 @@ static bool try_linear(hipStream_t s, const float* x, const uint8_t* w, int m, i
     return true;
 }
 
+// Several rows: the rows are one bucket of the bucketed down kernel (two rows share each weight row).
+static bool linear_rows(hipStream_t s, const float* x, const uint8_t* w, int dt, int m, int in_f, int out_f, float* dst,
+                        int n_cu, const float* addend) {
+    if (!bucketed_rows_supported(dt, in_f)) return false;
+    MoeGemvParams q{};
+    q.x = x;
+    q.down = w;
+    q.down_dt = dt;
+    q.nff = in_f;
+    q.ne = out_f;
+    q.rows = m;
+    q.n_expert = 1;
+    q.n_used = 1;
+    q.y = dst;
+    q.addend = addend;
+    q.n_cu = n_cu;
+    launch_moe_down_bucketed(s, q);
+    return true;
+}
+
 void launch_linear(hipStream_t s, const float* x, const uint8_t* w, int dt, size_t row_bytes, int m, int in_f,
                    int out_f, float* dst, int n_cu, const float* addend) {
+    if (m >= 2 && linear_rows(s, x, w, dt, m, in_f, out_f, dst, n_cu, addend)) return;
     bool done = false;
     if (dt == INFR_Q4K) done = try_linear<Q4KFmt>(s, x, w, m, in_f, out_f, dst, n_cu, addend);
     else if (dt == INFR_Q6K) done = try_linear<Q6KFmt>(s, x, w, m, in_f, out_f, dst, n_cu, addend);

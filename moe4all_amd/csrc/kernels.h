@@ -64,6 +64,9 @@ struct MoeGemvParams {
     // optional always-on expert handled as one more slot after the n_used routed ones (same dtypes,
     // same n_ff, routing weight 1): h then has n_used + 1 slots per row
     const uint8_t* sh_gate; const uint8_t* sh_up; const uint8_t* sh_down;
+    // bucketed kernels: the most pairs one bucket can hold (0 = rows; rows * n_used when given expert ids
+    // may repeat an expert inside a row)
+    int max_bucket;
     int n_cu;
     // When set, the gate/up kernel routes each token row itself from route.logits (every block
     // redundantly; block 0 of a row publishes ids / weights / probs) and no route launch is needed.
@@ -115,6 +118,9 @@ void launch_unbucket_combine(hipStream_t s, const float* y, const int32_t* slot_
 // so an expert's rows are read from HBM once however many token rows selected it.  h and y are in
 // flat (row, rank) order; launch_unbucket_combine with slot_pair_is_flags sums them.
 bool moe_bucketed_supported(const MoeGemvParams& p);
+// One side of it: rows of k elements in format dt.  Without bucket tables (bk_offsets == nullptr)
+// the bucketed kernels treat all p.rows rows as one bucket in order: a dense layer.
+bool bucketed_rows_supported(int dt, int k);
 void launch_moe_gate_up_bucketed(hipStream_t s, const MoeGemvParams& p);
 void launch_moe_down_bucketed(hipStream_t s, const MoeGemvParams& p);
 

@@ -685,10 +685,12 @@ def test_batched_moe_ffn_option_variants_match_oracle(be):
     (16, 512, 8, 2, 256, H.Q4K, H.Q6K),
     (19, 256, 16, 4, 256, H.Q6K, H.Q4K),       # experts without tokens, odd bucket sizes
     (31, 2048, 128, 8, 768, H.Q8_0, H.Q8_0),   # the largest batch below the matrix-core path
+    (18, 256, 24, 17, 256, H.Q4K, H.Q6K),      # more ranks than the per-token down kernel combines: bucketed down + combine
 ])
 def test_bucketed_decode_batches_bucket_exactly_and_keep_f32_accuracy(be, rows, ne, E, K, nff, gdt, ddt):
-    """16..31 token rows: pairs are bucketed by expert and each expert's rows are read once; the inner
-    product is the per-token kernels', so the f32 bar applies."""
+    """16..31 token rows: pairs are bucketed by expert and the gate/up rows of an expert serve two tokens
+    per read (the down projection streams per pair); the inner product is the per-token kernels', so the
+    f32 bar applies."""
     rng = np.random.default_rng(rows * 3 + ne)
     x = rng.standard_normal((rows, ne)).astype(np.float32)
     router = (rng.standard_normal((E, ne)) * 0.02).astype(np.float32)
