@@ -81,7 +81,9 @@ typedef enum infr_op_kind {
     INFR_OP_LINEAR = 1,                /* Op::Linear              graph.rs:200-212   */
     INFR_OP_GATED_ACT = 2,             /* Op::GatedAct            graph.rs:935-975   */
     INFR_OP_ADD = 3,                   /* Op::Add                                   */
-    INFR_OP_MOE_SHARED_EXPERT_ADD = 4  /* Op::MoeSharedExpertAdd  graph.rs:1449-1463 */
+    INFR_OP_MOE_SHARED_EXPERT_ADD = 4, /* Op::MoeSharedExpertAdd  graph.rs:1449-1463 */
+    INFR_OP_COPY = 5,                  /* Op::Copy                graph.rs:1230-1237 */
+    INFR_OP_COPY_STRIDED = 6           /* Op::CopyStrided         graph.rs:1238-1251 */
 } infr_op_kind;
 
 /* Field-for-field Op::MoeFfn.  Option<TensorId> = INFR_NO_TENSOR; Option<f32> and
@@ -124,6 +126,15 @@ typedef struct infr_op_moe_shared_expert_add {
     uint32_t rows, n;
 } infr_op_moe_shared_expert_add;
 
+/* Op::Copy is the rows = 1 case (strides unused).  Offsets, strides and n count elements of the
+ * tensors' common dtype (F32, I32, U32, F16 or BF16).  src may equal dst: the source window is read
+ * before anything is written, as the CPU backend does (crates/infr-cpu/src/lib.rs:3532-3583). */
+typedef struct infr_op_copy {
+    uint32_t src, src_off, src_stride;
+    uint32_t dst, dst_off, dst_stride;
+    uint32_t rows, n;
+} infr_op_copy;
+
 typedef struct infr_op {
     int32_t kind; /* infr_op_kind */
     union {
@@ -132,6 +143,7 @@ typedef struct infr_op {
         infr_op_gated_act gated_act;
         infr_op_add add;
         infr_op_moe_shared_expert_add moe_shared_expert_add;
+        infr_op_copy copy;
     } u;
 } infr_op;
 

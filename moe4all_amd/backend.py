@@ -123,9 +123,13 @@ class _OpSharedAdd(C.Structure):
     _fields_ = [(n, C.c_uint32) for n in ("moe", "shexp", "gate", "dst", "rows", "n")]
 
 
+class _OpCopy(C.Structure):
+    _fields_ = [(n, C.c_uint32) for n in ("src", "src_off", "src_stride", "dst", "dst_off", "dst_stride", "rows", "n")]
+
+
 class _OpUnion(C.Union):
     _fields_ = [("moe_ffn", _OpMoeFfn), ("linear", _OpLinear), ("gated_act", _OpGatedAct), ("add", _OpAdd),
-                ("moe_shared_expert_add", _OpSharedAdd)]
+                ("moe_shared_expert_add", _OpSharedAdd), ("copy", _OpCopy)]
 
 
 class _Op(C.Structure):
@@ -330,6 +334,21 @@ class Graph:
         op = _Op(kind=4)
         s = op.u.moe_shared_expert_add
         s.moe, s.shexp, s.gate, s.dst, s.rows, s.n = moe, shexp, gate, dst, rows, n
+        self.ops.append(op)
+
+    def copy(self, *, src, src_off, dst, dst_off, n) -> None:
+        """Op::Copy (crates/infr-core/src/graph.rs:1230-1237)."""
+        op = _Op(kind=5)
+        c = op.u.copy
+        c.src, c.src_off, c.dst, c.dst_off, c.rows, c.n = src, src_off, dst, dst_off, 1, n
+        self.ops.append(op)
+
+    def copy_strided(self, *, src, src_off, src_stride, dst, dst_off, dst_stride, rows, n) -> None:
+        """Op::CopyStrided (crates/infr-core/src/graph.rs:1238-1251)."""
+        op = _Op(kind=6)
+        c = op.u.copy
+        c.src, c.src_off, c.src_stride, c.dst, c.dst_off, c.dst_stride, c.rows, c.n = (
+            src, src_off, src_stride, dst, dst_off, dst_stride, rows, n)
         self.ops.append(op)
 
     def push_raw(self, kind: int) -> None:

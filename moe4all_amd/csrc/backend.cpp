@@ -126,6 +126,7 @@ struct infr_hip_plan {
     std::vector<FuseOp> fuse;
     std::vector<FuseOp> fuse_head;     // kMoeShared: the records of the ops it absorbed, as they were before
     int32_t* zero_ids = nullptr;       // [max rows of a fused gate/up] expert id 0 for every row
+    std::vector<size_t> copy_tmp;      // per op: arena offset of the staging window of an aliasing Copy, else 0
 };
 
 struct infr_hip_backend {
@@ -475,6 +476,7 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
     }
     Check c{*plan};
     std::vector<size_t> moe_off(g->n_ops, 0);
+    plan->copy_tmp.assign(g->n_ops, 0);
     size_t shared_need = 0;
     for (uint32_t oi = 0; oi < g->n_ops && c.st == INFR_OK; oi++) {
         const infr_op& op = plan->ops[oi];
@@ -648,6 +650,31 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
                     c.set(INFR_ERR_INVALID, "MoeSharedExpertAdd: rows*n exceeds an operand");
                 break;
             }
+            case INFR_OP_COPY:
+            case INFR_OP_COPY_STRIDED: {
+                const infr_op_copy& cp = op.u.copy;
+                if (!(c.tensor(cp.src, "Copy.src") && c.tensor(cp.dst, "Copy.dst"))) break;
+                c.want_writable(cp.dst, "Copy.dst");
+                const int dt = c.dt(cp.src);
+                if (dt != c.dt(cp.dst)) { c.set(INFR_ERR_INVALID, "Copy: src and dst differ in dtype"); break; }
+                if (!(dt == INFR_F32 || dt == INFR_I32 || dt == INFR_U32 || dt == INFR_F16 || dt == INFR_BF16)) {
+                    c.set(INFR_ERR_UNSUPPORTED, "Copy: only F32/I32/U32/F16/BF16 tensors");
+                    break;
+                }
+                const uint64_t rows = op.kind == INFR_OP_COPY ? 1 : cp.rows;
+                if (rows && cp.n) {
+                    const uint64_t s_end = cp.src_off + (rows - 1) * (uint64_t)cp.src_stride + cp.n;
+                    const uint64_t d_end = cp.dst_off + (rows - 1) * (uint64_t)cp.dst_stride + cp.n;
+                    if (s_end > c.n(cp.src) || d_end > c.n(cp.dst)) { c.set(INFR_ERR_INVALID, "Copy: window outside a tensor"); break; }
+                    if (rows > 65535) { c.set(INFR_ERR_UNSUPPORTED, "Copy: more than 65535 rows"); break; }
+                    if (cp.src == cp.dst) {
+                        // the source window is staged first (the CPU backend clones it, lib.rs:3540-3545)
+                        plan->copy_tmp[oi] = arena;
+                        arena += round_up(rows * cp.n * 4, 256);
+                    }
+                }
+                break;
+            }
             default:
                 c.set(INFR_ERR_UNSUPPORTED, "compile: op kind " + std::to_string(op.kind) +
                                                 " is not on the routed-expert FFN path this backend implements");
@@ -685,6 +712,8 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
                     rd(a.moe); rd(a.shexp); rd(a.gate); wr(a.dst);
                     break;
                 }
+                case INFR_OP_COPY:
+                case INFR_OP_COPY_STRIDED: rd(op.u.copy.src); rd(op.u.copy.dst); wr(op.u.copy.dst); break;   // a partial write keeps the rest
                 default: break;
             }
         }
@@ -1119,6 +1148,25 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                 Timed t(be, "moe_shared_expert_add");
                 infr::launch_moe_shared_expert_add(s, (const float*)ptr[a.moe], (const float*)ptr[a.shexp],
                                                    (const float*)ptr[a.gate], (float*)ptr[a.dst], (int)a.rows, (int)a.n);
+                break;
+            }
+            case INFR_OP_COPY:
+            case INFR_OP_COPY_STRIDED: {
+                const infr_op_copy& cp = op.u.copy;
+                if (!(need(cp.src, "Copy.src") && need(cp.dst, "Copy.dst"))) return INFR_ERR_BACKEND;
+                const uint32_t rows = op.kind == INFR_OP_COPY ? 1 : cp.rows;
+                const int dt = plan->tensors[cp.src].dtype;
+                const int eb = (dt == INFR_F16 || dt == INFR_BF16) ? 2 : 4;
+                const char* src = (const char*)ptr[cp.src] + (size_t)cp.src_off * eb;
+                char* dst = (char*)ptr[cp.dst] + (size_t)cp.dst_off * eb;
+                Timed t(be, "copy");
+                if (cp.src == cp.dst && rows && cp.n) {
+                    char* tmp = (char*)plan->arena + plan->copy_tmp[oi];
+                    infr::launch_copy_rows(s, src, tmp, rows, cp.n, cp.src_stride, cp.n, eb);
+                    infr::launch_copy_rows(s, tmp, dst, rows, cp.n, cp.n, cp.dst_stride, eb);
+                } else {
+                    infr::launch_copy_rows(s, src, dst, rows, cp.n, cp.src_stride, cp.dst_stride, eb);
+                }
                 break;
             }
             default:

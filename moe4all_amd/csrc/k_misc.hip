@@ -72,6 +72,27 @@ void launch_add(hipStream_t s, const float* a, const float* b, float* dst, uint3
     INFR_LAUNCH(add_kernel, dim3(blocks), dim3(256), 0, s, a, b, dst, n);
 }
 
+// Op::Copy / Op::CopyStrided (crates/infr-cpu/src/lib.rs:3532-3583).
+template <class T>
+__global__ __launch_bounds__(256) void copy_rows_kernel(const T* __restrict__ src, T* __restrict__ dst, uint32_t n,
+                                                        uint32_t src_stride, uint32_t dst_stride) {
+    const size_t r = blockIdx.y;
+    for (uint32_t i = blockIdx.x * 256 + threadIdx.x; i < n; i += gridDim.x * 256)
+        dst[r * dst_stride + i] = src[r * src_stride + i];
+}
+void launch_copy_rows(hipStream_t s, const void* src, void* dst, uint32_t rows, uint32_t n, uint32_t src_stride,
+                      uint32_t dst_stride, int elem_bytes) {
+    if (rows == 0 || n == 0) return;
+    uint32_t bx = (n + 255) / 256;
+    if (bx > 1024) bx = 1024;
+    if (elem_bytes == 4)
+        INFR_LAUNCH(copy_rows_kernel<uint32_t>, dim3(bx, rows), dim3(256), 0, s, (const uint32_t*)src, (uint32_t*)dst, n,
+                    src_stride, dst_stride);
+    else
+        INFR_LAUNCH(copy_rows_kernel<uint16_t>, dim3(bx, rows), dim3(256), 0, s, (const uint16_t*)src, (uint16_t*)dst, n,
+                    src_stride, dst_stride);
+}
+
 // Op::MoeSharedExpertAdd (crates/infr-cpu/src/lib.rs:3336-3356):
 // dst = moe + sigmoid(gate[r]) * shexp, multiply and add rounded separately.
 __global__ __launch_bounds__(256) void moe_shared_expert_add_kernel(const float* __restrict__ moe,

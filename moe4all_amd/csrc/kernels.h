@@ -134,6 +134,10 @@ void launch_linear(hipStream_t s, const float* x, const uint8_t* w, int dt, size
 void launch_gated_act(hipStream_t s, const float* gate, const float* up, float* dst, int rows, int nff, int act,
                       int up_off, int up_stride, int gate_stride, int gate_block_width, int has_clamp, float clamp);
 void launch_add(hipStream_t s, const float* a, const float* b, float* dst, uint32_t n);
+// Op::Copy / Op::CopyStrided on elements of `elem_bytes` (2 or 4): row r copies n elements from
+// src + r * src_stride to dst + r * dst_stride (pointers already at the ops' offsets).
+void launch_copy_rows(hipStream_t s, const void* src, void* dst, uint32_t rows, uint32_t n, uint32_t src_stride,
+                      uint32_t dst_stride, int elem_bytes);
 void launch_moe_shared_expert_add(hipStream_t s, const float* moe, const float* shexp, const float* gate, float* dst,
                                   int rows, int n);
 void launch_fill_zero(hipStream_t s, void* p, size_t bytes);

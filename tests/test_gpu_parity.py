@@ -380,6 +380,37 @@ def test_shared_expert_branch_matches_oracle(be):
     assert np.array_equal(got2, O.add(x, moe).ravel())
 
 
+def test_copy_and_copy_strided_follow_the_cpu_semantics(be):
+    """Op::Copy / Op::CopyStrided (crates/infr-cpu/src/lib.rs:3532-3583): windows counted in elements,
+    the rest of dst untouched, and a copy inside one tensor reads its source window before it
+    writes (overlapping windows included)."""
+    rng = np.random.default_rng(5)
+    a = rng.standard_normal(4096).astype(np.float32)
+    g = M.Graph()
+    src = g.input(TensorDesc([4096], DType.F32))
+    dst = g.output(TensorDesc([6, 100], DType.F32))
+    mid = g.internal(TensorDesc([4096], DType.F32))
+    g.copy(src=src, src_off=0, dst=mid, dst_off=0, n=4096)
+    g.copy(src=mid, src_off=10, dst=mid, dst_off=50, n=1000)             # overlapping, forward
+    g.copy_strided(src=mid, src_off=3, src_stride=300, dst=mid, dst_off=7, dst_stride=300, rows=5, n=250)  # overlapping rows
+    g.copy_strided(src=mid, src_off=20, src_stride=64, dst=dst, dst_off=10, dst_stride=100, rows=6, n=37)
+    got = M.run_graph(be, g, [(src, a)], dst, 600).reshape(6, 100)
+    m = a.copy()
+    m[50:1050] = m[10:1010].copy()
+    snap = m.copy()
+    for r in range(5):
+        m[7 + 300 * r:7 + 300 * r + 250] = snap[3 + 300 * r:3 + 300 * r + 250]
+    want = np.zeros((6, 100), np.float32)
+    for r in range(6):
+        want[r, 10:47] = m[20 + 64 * r:20 + 64 * r + 37]
+    assert np.array_equal(bits(got), bits(want))
+    g2 = M.Graph()
+    s2, d2 = g2.input(TensorDesc([8], DType.F32)), g2.output(TensorDesc([8], DType.F32))
+    g2.copy(src=s2, src_off=4, dst=d2, dst_off=0, n=5)   # reads past the source
+    with pytest.raises(M.BackendError):
+        be.compile(g2)
+
+
 @pytest.mark.parametrize("rows,act", [(1, M.Activation.Silu), (5, M.Activation.Gelu)])
 def test_fused_dense_ffn_launches_give_the_bits_of_the_separate_ops(be, rows, act):
     """Linear+Linear+GatedAct and Linear+Add collapse into one launch each when their temporaries are
