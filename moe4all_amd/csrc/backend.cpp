@@ -1030,6 +1030,7 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                     }
                     q.a = sc.hh; q.a_scale = sc.hs; q.w0 = gp.down; q.w0_stride = gp.down_stride; q.w1 = nullptr; q.w1_stride = 0;
                     q.down_scale = gp.down_scale; q.out = sc.y; q.K = (int)m.n_ff_exp; q.N = (int)m.ne;
+                    q.out_f16 = 1;   // y is written and read once: f16 halves that traffic, hs restores the scale
                     {
                         Timed t(be, "moe_grouped_down");
                         infr::launch_grouped_down(s, gp.down_dt, q);
@@ -1037,7 +1038,7 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                     {
                         Timed t(be, "moe_unbucket_combine");
                         infr::launch_unbucket_combine(s, sc.y, sc.slot_pair, sc.weights, rows, (int)m.ne, (int)m.n_used,
-                                                      (int)m.weight_before, gp.dst);
+                                                      (int)m.weight_before, gp.dst, 0, sc.hs);
                     }
                     break;
                 }

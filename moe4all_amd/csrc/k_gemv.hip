@@ -26,23 +26,6 @@
 
 namespace infr {
 
-#ifdef INFR_TRACE
-// Experiment-only stage timestamps (100 MHz wall clock), one record of 8 per wave.
-__device__ unsigned long long g_trace[8 * 8192];
-unsigned long long* trace_ptr() {
-    void* p = nullptr;
-    (void)hipGetSymbolAddress(&p, HIP_SYMBOL(g_trace));
-    return (unsigned long long*)p;
-}
-#define TRACE(slot, dep)                                                               \
-    do {                                                                               \
-        asm volatile("" ::"v"(dep));                                                   \
-        if (lane == 0) g_trace[(size_t)((blockIdx.x * 8 + wave) & 8191) * 8 + (slot)] = wall_clock64(); \
-    } while (0)
-#else
-#define TRACE(slot, dep) do {} while (0)
-#endif
-
 __device__ __forceinline__ int dot4i(uint32_t a, uint32_t b, int c) {
     return __builtin_amdgcn_sdot4((int)a, (int)b, c, false);
 }

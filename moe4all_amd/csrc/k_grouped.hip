@@ -427,7 +427,20 @@ __device__ __forceinline__ void tile_epilogue(const GroupedParams& p, const Tile
             }
         }
     };
-    if (DOWN) {
+    if (DOWN && p.out_f16) {
+        // f16 without the row's power-of-two scale (|acc| stays far inside the f16 range: the
+        // activation rows were normalised below 1); the combine multiplies the scale back in
+        const float ds = p.down_scale ? p.down_scale[t.e] : 1.0f;
+        const bool ok0 = fc0 < p.N, ok1 = fc0 + 32 < p.N;
+        _Float16* const hbase = reinterpret_cast<_Float16*>(p.out) + (size_t)t.p0 * p.N + fc0;
+        if (ok0) {
+            for_each([&](int mi, int r, int m, float, float*) {
+                _Float16* o = hbase + (size_t)m * p.N;
+                o[0] = (_Float16)(acc0[mi][r] * ds);
+                if (ok1) o[32] = (_Float16)(acc1[mi][r] * ds);
+            });
+        }
+    } else if (DOWN) {
         const float ds = p.down_scale ? p.down_scale[t.e] : 1.0f;
         const bool ok0 = fc0 < p.N, ok1 = fc0 + 32 < p.N;
         if (ok1) {
@@ -726,10 +739,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 }
 
 // dst[row, :] = sum over ranks of w * y[slot_pair[row, rank], :], rank order, separate mul/add.
-__global__ __launch_bounds__(256) void unbucket_combine_kernel(const float* __restrict__ y,
-                                                               const int32_t* __restrict__ slot_pair,
+// Y = _Float16: y rows carry no row scale, pair_scale[pair] multiplies it back in.
+template <class Y>
+__global__ __launch_bounds__(256) void unbucket_combine_kernel(const Y* __restrict__ y, const int32_t* __restrict__ slot_pair,
                                                                const float* __restrict__ weights, int ne, int n_used,
-                                                               int weight_before, float* __restrict__ dst, int identity) {
+                                                               int weight_before, float* __restrict__ dst, int identity,
+                                                               const float* __restrict__ pair_scale) {
     const size_t row = blockIdx.y;
     const int i = (blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= ne) return;
@@ -739,17 +754,29 @@ __global__ __launch_bounds__(256) void unbucket_combine_kernel(const float* __re
         if (pr < 0) continue;
         if (identity) pr = (int)(row * n_used + k);
         const float w = weight_before ? 1.0f : weights[row * n_used + k];
-        const float* yr = y + (size_t)pr * ne + i;
+        const float sc = pair_scale ? pair_scale[pr] : 1.0f;
+        const Y* yr = y + (size_t)pr * ne + i;
+        float v[4] = {0.f, 0.f, 0.f, 0.f};
         if (i + 3 < ne) {
-            const float4 v = *reinterpret_cast<const float4*>(yr);
-            acc.x = __fadd_rn(acc.x, __fmul_rn(w, v.x));
-            acc.y = __fadd_rn(acc.y, __fmul_rn(w, v.y));
-            acc.z = __fadd_rn(acc.z, __fmul_rn(w, v.z));
-            acc.w = __fadd_rn(acc.w, __fmul_rn(w, v.w));
+            if (sizeof(Y) == 2) {
+                const uint2 raw = *reinterpret_cast<const uint2*>(yr);
+                const half2v a = as_h2(raw.x), b = as_h2(raw.y);
+                v[0] = (float)a[0]; v[1] = (float)a[1]; v[2] = (float)b[0]; v[3] = (float)b[1];
+            } else {
+                const float4 f = *reinterpret_cast<const float4*>(yr);
+                v[0] = f.x; v[1] = f.y; v[2] = f.z; v[3] = f.w;
+            }
         } else {
-            float* a = &acc.x;
-            for (int q = 0; i + q < ne; q++) a[q] = __fadd_rn(a[q], __fmul_rn(w, yr[q]));
+            for (int q = 0; i + q < ne; q++) v[q] = (float)yr[q];
         }
+        if (pair_scale) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) v[q] *= sc;
+        }
+        acc.x = __fadd_rn(acc.x, __fmul_rn(w, v[0]));
+        acc.y = __fadd_rn(acc.y, __fmul_rn(w, v[1]));
+        acc.z = __fadd_rn(acc.z, __fmul_rn(w, v[2]));
+        acc.w = __fadd_rn(acc.w, __fmul_rn(w, v[3]));
     }
     float* o = dst + row * ne + i;
     if (i + 3 < ne) *reinterpret_cast<float4*>(o) = acc;
@@ -812,11 +839,16 @@ void launch_grouped_down(hipStream_t s, int dt, const GroupedParams& p) {
     else grouped6<D80, true>(s, p);
 }
 
-void launch_unbucket_combine(hipStream_t s, const float* y, const int32_t* slot_pair, const float* weights, int rows,
-                             int ne, int n_used, int weight_before, float* dst, int identity) {
+void launch_unbucket_combine(hipStream_t s, const void* y, const int32_t* slot_pair, const float* weights, int rows,
+                             int ne, int n_used, int weight_before, float* dst, int identity, const float* pair_scale) {
     if (rows <= 0) return;
-    INFR_LAUNCH(unbucket_combine_kernel, dim3((ne + 1023) / 1024, rows), dim3(256), 0, s, y, slot_pair, weights, ne, n_used,
-                weight_before, dst, identity);
+    const dim3 grid((ne + 1023) / 1024, rows), block(256);
+    if (pair_scale)
+        INFR_LAUNCH(unbucket_combine_kernel<_Float16>, grid, block, 0, s, (const _Float16*)y, slot_pair, weights, ne, n_used,
+                    weight_before, dst, identity, pair_scale);
+    else
+        INFR_LAUNCH(unbucket_combine_kernel<float>, grid, block, 0, s, (const float*)y, slot_pair, weights, ne, n_used,
+                    weight_before, dst, identity, pair_scale);
 }
 
 }  // namespace infr

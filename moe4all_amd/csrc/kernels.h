@@ -96,7 +96,8 @@ struct GroupedParams {
     const uint8_t* w1; size_t w1_stride;  // up expert slices (gate/up only)
     const float* route_w;     // [rows, n_used] routing weights, read when weight_before
     const float* down_scale;  // [n_expert] or null (down only)
-    float* out;               // [n_pairs, N] f32, bucket order
+    float* out;               // [n_pairs, N] f32, bucket order (down with out_f16: f16 without the row scale)
+    int out_f16;              // down only: store f16(acc * down_scale); the combine applies the row's a_scale
     int K, N, n_expert, n_used, n_pairs;
     int act, has_clamp; float clamp; int weight_before;
     int n_tiles_n;            // set by the launcher
@@ -111,8 +112,9 @@ void launch_bucket(hipStream_t s, const int32_t* ids, int n_pairs, int n_expert,
 void launch_grouped_gate_up(hipStream_t s, int dt, const GroupedParams& p);
 void launch_grouped_down(hipStream_t s, int dt, const GroupedParams& p);
 // identity != 0: y is in flat (row, rank) order and slot_pair only flags invalid pairs (< 0).
-void launch_unbucket_combine(hipStream_t s, const float* y, const int32_t* slot_pair, const float* weights, int rows,
-                             int ne, int n_used, int weight_before, float* dst, int identity = 0);
+void launch_unbucket_combine(hipStream_t s, const void* y, const int32_t* slot_pair, const float* weights, int rows,
+                             int ne, int n_used, int weight_before, float* dst, int identity = 0,
+                             const float* pair_scale = nullptr);   // pair_scale != null: y is f16, y[pair] * pair_scale[pair]
 
 // Decode batches with weight reuse: one block per (feature tile, expert) walks the expert's bucket,
 // so an expert's rows are read from HBM once however many token rows selected it.  h and y are in
