@@ -100,6 +100,10 @@ typedef struct infr_op_moe_ffn {
     int32_t gating;                /* infr_moe_gating */
     uint32_t norm_w;               /* bool */
     uint32_t weight_before;        /* bool */
+    /* Option<(base, n_local)> (graph.rs:1307-1319): routing stays global over n_expert, the expert
+     * tensors (gate/up/down, down_scale) hold only the shard [ep_base, ep_base + ep_n_local);
+     * selections of other experts become (id 0, weight 0) as in moe_ep_band_remap.comp, so dst is
+     * this rank's partial sum. */
     uint32_t has_ep_band; uint32_t ep_base, ep_n_local;
     uint32_t exp_probs_b;          /* optional */
     uint32_t n_expert_groups, n_expert_groups_used;

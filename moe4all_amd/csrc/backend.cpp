@@ -93,6 +93,7 @@ struct MoeScratch {
     // batched path (bucketing + grouped GEMMs); the large buffers are shared by all ops of a plan
     bool batched = false;    // >= kBatchedMinRows: grouped GEMMs on the matrix cores
     bool bucketed = false;   // kBucketedMinRows .. : f32-accurate GEMV per (expert, bucket), weights read once per expert
+    int32_t* live_ids = nullptr;  // [pairs] ids with the pairs an expert-parallel band dropped set to -1
     int32_t* offsets = nullptr;   // [n_expert + 1]
     int32_t* pair_src = nullptr;  // [rows * n_used]
     int32_t* slot_pair = nullptr; // [rows * n_used]
@@ -496,11 +497,13 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
                     break;
                 }
                 if (m.n_expert > 2048 || m.n_used > 64) { c.set(INFR_ERR_UNSUPPORTED, "MoeFfn: n_expert > 2048 or n_used > 64"); break; }
-                if (m.has_ep_band) {
-                    c.set(INFR_ERR_UNSUPPORTED, "MoeFfn: ep_band (expert-parallel shard) is a multi-device lowering; "
-                                                "this backend runs all experts on one device");
+                // expert-parallel band (graph.rs:1307-1319): global routing, the expert tensors hold only the
+                // shard [ep_base, ep_base + ep_n_local)
+                if (m.has_ep_band && (m.ep_n_local == 0 || (uint64_t)m.ep_base + m.ep_n_local > m.n_expert)) {
+                    c.set(INFR_ERR_INVALID, "MoeFfn: ep_band is not a non-empty range inside [0, n_expert)");
                     break;
                 }
+                const uint64_t n_local = m.has_ep_band ? m.ep_n_local : m.n_expert;
                 // Same refusals as the reference (crates/infr-cpu/src/lib.rs:3613-3629).
                 if (m.has_swiglu_clamp && (m.act == INFR_ACT_SIGMOID || m.weight_before)) {
                     c.set(INFR_ERR_INVALID, "MoeFfn: swiglu_clamp is defined for the gated SiLU/GELU forms with "
@@ -531,14 +534,14 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
                 c.want_numel(m.dst, rows * m.ne, "MoeFfn.dst");
                 c.want_numel(m.router, (uint64_t)m.n_expert * m.ne, "MoeFfn.router");
                 uint64_t gu_rows = m.fused_gate_up ? 2ull * m.n_ff_exp : m.n_ff_exp;
-                c.want_numel(m.gate_exps, (uint64_t)m.n_expert * gu_rows * m.ne, "MoeFfn.gate_exps");
-                if (!m.fused_gate_up) c.want_numel(m.up_exps, (uint64_t)m.n_expert * m.n_ff_exp * m.ne, "MoeFfn.up_exps");
-                c.want_numel(m.down_exps, (uint64_t)m.n_expert * m.ne * m.n_ff_exp, "MoeFfn.down_exps");
+                c.want_numel(m.gate_exps, n_local * gu_rows * m.ne, "MoeFfn.gate_exps");
+                if (!m.fused_gate_up) c.want_numel(m.up_exps, n_local * m.n_ff_exp * m.ne, "MoeFfn.up_exps");
+                c.want_numel(m.down_exps, n_local * m.ne * m.n_ff_exp, "MoeFfn.down_exps");
                 c.want_weight_dtype(m.router, m.ne, "MoeFfn.router");
                 c.want_weight_dtype(m.gate_exps, m.ne, "MoeFfn.gate_exps");
                 if (!m.fused_gate_up) c.want_weight_dtype(m.up_exps, m.ne, "MoeFfn.up_exps");
                 c.want_weight_dtype(m.down_exps, m.n_ff_exp, "MoeFfn.down_exps");
-                if (m.down_scale != INFR_NO_TENSOR) { c.want_f32(m.down_scale, "MoeFfn.down_scale"); c.want_numel(m.down_scale, m.n_expert, "MoeFfn.down_scale"); }
+                if (m.down_scale != INFR_NO_TENSOR) { c.want_f32(m.down_scale, "MoeFfn.down_scale"); c.want_numel(m.down_scale, n_local, "MoeFfn.down_scale"); }
                 if (m.exp_probs_b != INFR_NO_TENSOR) { c.want_f32(m.exp_probs_b, "MoeFfn.exp_probs_b"); c.want_numel(m.exp_probs_b, m.n_expert, "MoeFfn.exp_probs_b"); }
                 if (m.expert_ids != INFR_NO_TENSOR) {
                     if (c.dt(m.expert_ids) != INFR_I32) c.set(INFR_ERR_UNSUPPORTED, "MoeFfn.expert_ids must be I32");
@@ -558,7 +561,7 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
                                      infr::grouped_supported(c.dt(m.gate_exps), (int)m.ne) &&
                                      infr::grouped_supported(c.dt(m.down_exps), (int)m.n_ff_exp);
                 if (batched) {
-                    arena += round_up(((size_t)m.n_expert + 2) * 4, 256) + 2 * round_up(pairs * 4 + 4, 256);
+                    arena += round_up(((size_t)m.n_expert + 2) * 4, 256) + 3 * round_up(pairs * 4 + 4, 256);
                     shared += round_up((size_t)rows * m.ne * 2, 256) + round_up((size_t)rows * 4, 256) +
                               round_up(pairs * m.n_ff_exp * 2, 256) + round_up(pairs * 4, 256) +
                               round_up(pairs * m.ne * 4, 256);
@@ -575,7 +578,7 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
                     bucketed = infr::moe_bucketed_supported(probe);
                 }
                 if (bucketed) {
-                    arena += round_up(((size_t)m.n_expert + 2) * 4, 256) + 2 * round_up(pairs * 4 + 4, 256);
+                    arena += round_up(((size_t)m.n_expert + 2) * 4, 256) + 3 * round_up(pairs * 4 + 4, 256);
                     shared += round_up(pairs * m.ne * 4, 256);
                 }
                 if (shared > shared_need) shared_need = shared;
@@ -824,7 +827,8 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
         if (s.batched || s.bucketed) {
             s.offsets = (int32_t*)p;   p += round_up(((size_t)m.n_expert + 2) * 4, 256);
             s.pair_src = (int32_t*)p;  p += round_up(pairs * 4 + 4, 256);
-            s.slot_pair = (int32_t*)p;
+            s.slot_pair = (int32_t*)p; p += round_up(pairs * 4 + 4, 256);
+            s.live_ids = (int32_t*)p;
         }
         p = (char*)plan->arena + shared_off;
         s.h = (float*)p; p += round_up((pairs + rows) * m.n_ff_exp * 4 + 4, 256);
@@ -964,6 +968,9 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                 rp.exp_probs_b = m.exp_probs_b == INFR_NO_TENSOR ? nullptr : (const float*)ptr[m.exp_probs_b];
                 rp.n_groups = (int)m.n_expert_groups; rp.n_groups_used = (int)m.n_expert_groups_used;
                 rp.expert_ids = m.expert_ids == INFR_NO_TENSOR ? nullptr : (const int32_t*)ptr[m.expert_ids];
+                rp.ep_lo = m.has_ep_band ? (int)m.ep_base : 0;
+                rp.ep_n = m.has_ep_band ? (int)m.ep_n_local : 0;
+                const uint32_t n_local = m.has_ep_band ? m.ep_n_local : m.n_expert;   // experts the weight tensors hold
                 rp.ids = sc.ids; rp.weights = sc.weights; rp.probs = sc.probs;
                 {
                     Timed t(be, "router_logits");
@@ -979,7 +986,7 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                 size_t gbytes = tensor_bytes(plan->tensors[m.gate_exps], plan->numel[m.gate_exps]);
                 size_t dbytes = tensor_bytes(plan->tensors[m.down_exps], plan->numel[m.down_exps]);
                 gp.gate = (const uint8_t*)ptr[m.gate_exps];
-                gp.gate_stride = gbytes / m.n_expert;  // reference: gst = gb.len() / n_expert (lib.rs:3666)
+                gp.gate_stride = gbytes / n_local;  // reference: gst = gb.len() / n_expert (lib.rs:3666)
                 if (m.fused_gate_up) {
                     // gate rows first, up rows second inside each expert slice
                     gp.up = gp.gate + gp.gate_stride / 2;
@@ -988,15 +995,16 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                 } else {
                     size_t ubytes = tensor_bytes(plan->tensors[m.up_exps], plan->numel[m.up_exps]);
                     gp.up = (const uint8_t*)ptr[m.up_exps];
-                    gp.up_stride = ubytes / m.n_expert;
+                    gp.up_stride = ubytes / n_local;
                     gp.up_dt = plan->tensors[m.up_exps].dtype;
                 }
                 gp.down = (const uint8_t*)ptr[m.down_exps];
-                gp.down_stride = dbytes / m.n_expert;
+                gp.down_stride = dbytes / n_local;
                 gp.down_scale = m.down_scale == INFR_NO_TENSOR ? nullptr : (const float*)ptr[m.down_scale];
-                gp.rows = rows; gp.ne = (int)m.ne; gp.nff = (int)m.n_ff_exp; gp.n_used = (int)m.n_used; gp.n_expert = (int)m.n_expert;
+                gp.rows = rows; gp.ne = (int)m.ne; gp.nff = (int)m.n_ff_exp; gp.n_used = (int)m.n_used; gp.n_expert = (int)n_local;
                 gp.act = m.act; gp.has_clamp = (int)m.has_swiglu_clamp; gp.clamp = m.swiglu_clamp;
                 gp.weight_before = (int)m.weight_before; gp.fused_gate_up = (int)m.fused_gate_up;
+                gp.skip_zero_w = (int)m.has_ep_band;
                 gp.h = sc.h; gp.dst = (float*)ptr[m.dst]; gp.n_cu = n_cu;
                 gp.x = (const float*)ptr[m.x];
                 if (sc.batched) {
@@ -1007,7 +1015,12 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                     }
                     {
                         Timed t(be, "moe_bucket");
-                        infr::launch_bucket(s, sc.ids, pairs, (int)m.n_expert, sc.offsets, sc.pair_src, sc.slot_pair);
+                        const int32_t* bucket_ids = sc.ids;
+                        if (m.has_ep_band) {   // pairs of foreign experts (weight 0) are not bucketed at all
+                            infr::launch_mask_dropped_pairs(s, sc.ids, sc.weights, pairs, sc.live_ids);
+                            bucket_ids = sc.live_ids;
+                        }
+                        infr::launch_bucket(s, bucket_ids, pairs, (int)n_local, sc.offsets, sc.pair_src, sc.slot_pair);
                     }
                     {
                         Timed t(be, "rows_to_f16");
@@ -1017,7 +1030,7 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                     q.a = sc.xh; q.a_scale = sc.xs; q.offsets = sc.offsets; q.pair_src = sc.pair_src;
                     q.w0 = gp.gate; q.w0_stride = gp.gate_stride; q.w1 = gp.up; q.w1_stride = gp.up_stride;
                     q.route_w = sc.weights; q.down_scale = nullptr; q.out = sc.h;
-                    q.K = (int)m.ne; q.N = (int)m.n_ff_exp; q.n_expert = (int)m.n_expert; q.n_used = (int)m.n_used;
+                    q.K = (int)m.ne; q.N = (int)m.n_ff_exp; q.n_expert = (int)n_local; q.n_used = (int)m.n_used;
                     q.n_pairs = pairs; q.act = m.act; q.has_clamp = (int)m.has_swiglu_clamp; q.clamp = m.swiglu_clamp;
                     q.weight_before = (int)m.weight_before;
                     {
@@ -1050,7 +1063,12 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                     }
                     {
                         Timed t(be, "moe_bucket");
-                        infr::launch_bucket(s, sc.ids, pairs, (int)m.n_expert, sc.offsets, sc.pair_src, sc.slot_pair);
+                        const int32_t* bucket_ids = sc.ids;
+                        if (m.has_ep_band) {   // pairs of foreign experts (weight 0) are not bucketed at all
+                            infr::launch_mask_dropped_pairs(s, sc.ids, sc.weights, pairs, sc.live_ids);
+                            bucket_ids = sc.live_ids;
+                        }
+                        infr::launch_bucket(s, bucket_ids, pairs, (int)n_local, sc.offsets, sc.pair_src, sc.slot_pair);
                     }
                     gp.bk_offsets = sc.offsets; gp.bk_pair_src = sc.pair_src; gp.y = sc.y;
                     gp.max_bucket = m.expert_ids == INFR_NO_TENSOR ? rows : pairs;   // given ids may repeat an expert in a row

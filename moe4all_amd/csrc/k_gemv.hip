@@ -666,6 +666,7 @@ __global__ __launch_bounds__(512) void moe_down_combine_fast(MoeGemvParams p, in
         const float* w = p.weights + (size_t)r * p.n_used;
         float acc = 0.0f;
         for (int k = 0; k < n_slots; k++) {
+            if (p.skip_zero_w && k < p.n_used && w[k] == 0.0f) continue;
             float wk = (p.weight_before || k >= p.n_used) ? 1.0f : w[k];
             acc = __fadd_rn(acc, __fmul_rn(wk, ypart[k][o]));
         }
@@ -719,6 +720,7 @@ __global__ __launch_bounds__(256) void moe_down_combine_generic(MoeGemvParams p,
         for (int k = lane; k < p.nff; k += kWave) y = fmaf(decode_elem(p.down_dt, row, (uint32_t)k), h[k], y);
         y = wave_sum(y);
         if (p.down_scale) y = __fmul_rn(y, p.down_scale[e]);
+        if (p.skip_zero_w && p.weights[(size_t)r * p.n_used + slot] == 0.0f) continue;
         float wk = p.weight_before ? 1.0f : p.weights[(size_t)r * p.n_used + slot];
         acc = __fadd_rn(acc, __fmul_rn(wk, y));
     }

@@ -72,6 +72,16 @@ void launch_add(hipStream_t s, const float* a, const float* b, float* dst, uint3
     INFR_LAUNCH(add_kernel, dim3(blocks), dim3(256), 0, s, a, b, dst, n);
 }
 
+__global__ __launch_bounds__(256) void mask_dropped_pairs_kernel(const int32_t* __restrict__ ids, const float* __restrict__ w,
+                                                                 int n, int32_t* __restrict__ out) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n) out[i] = w[i] == 0.0f ? -1 : ids[i];
+}
+void launch_mask_dropped_pairs(hipStream_t s, const int32_t* ids, const float* weights, int n_pairs, int32_t* out) {
+    if (n_pairs <= 0) return;
+    INFR_LAUNCH(mask_dropped_pairs_kernel, dim3((n_pairs + 255) / 256), dim3(256), 0, s, ids, weights, n_pairs, out);
+}
+
 // Op::Copy / Op::CopyStrided (crates/infr-cpu/src/lib.rs:3532-3583).
 template <class T>
 __global__ __launch_bounds__(256) void copy_rows_kernel(const T* __restrict__ src, T* __restrict__ dst, uint32_t n,

@@ -39,6 +39,9 @@ struct RouteParams {
     const float* exp_probs_b; // [n_expert] or null
     int n_groups, n_groups_used;
     const int32_t* expert_ids;  // [rows, n_used] or null (hash routing)
+    // expert-parallel band (crates/infr-vulkan/shaders/moe_ep_band_remap.comp): ep_n > 0 keeps the
+    // selections inside [ep_lo, ep_lo + ep_n) as id - ep_lo and turns the others into id 0, weight 0
+    int ep_lo, ep_n;
     int32_t* ids;             // out [rows, n_used] rank order
     float* weights;           // out [rows, n_used]
     float* probs;             // out [rows, n_expert]
@@ -67,6 +70,9 @@ struct MoeGemvParams {
     // bucketed kernels: the most pairs one bucket can hold (0 = rows; rows * n_used when given expert ids
     // may repeat an expert inside a row)
     int max_bucket;
+    // down: ranks whose routing weight is exactly 0 are left out of the combine (pairs an
+    // expert-parallel band dropped: their h rows may never have been written)
+    int skip_zero_w;
     int n_cu;
     // When set, the gate/up kernel routes each token row itself from route.logits (every block
     // redundantly; block 0 of a row publishes ids / weights / probs) and no route launch is needed.
@@ -107,6 +113,8 @@ bool grouped_supported(int dt, int k);
 // rows of f32 -> f16 with a per-row power-of-two scale, in the k order weights of `weight_dt` unpack to.
 void launch_rows_to_f16(hipStream_t s, int weight_dt, const float* src, int rows, int n, void* dst, float* scale);
 // offsets / pair_src / slot_pair ([n_pairs], -1 for ids outside [0, n_expert)) from ids [n_pairs].
+// ids with the pairs of weight exactly 0 replaced by -1 (pairs an expert-parallel band dropped).
+void launch_mask_dropped_pairs(hipStream_t s, const int32_t* ids, const float* weights, int n_pairs, int32_t* out);
 void launch_bucket(hipStream_t s, const int32_t* ids, int n_pairs, int n_expert, int32_t* offsets, int32_t* pair_src,
                    int32_t* slot_pair);
 void launch_grouped_gate_up(hipStream_t s, int dt, const GroupedParams& p);

@@ -169,6 +169,12 @@ __device__ __forceinline__ void route_row(const RouteParams& p, int row, int lan
     } else {
         w = __fmul_rn(pk, p.scale);
     }
+    if (p.ep_n > 0) {
+        // expert-parallel band: ids become indices into the local shard, foreign selections weigh nothing
+        const bool own = my_id >= p.ep_lo && my_id < p.ep_lo + p.ep_n;
+        my_id = own ? my_id - p.ep_lo : 0;
+        w = own ? w : 0.0f;
+    }
     if (mine) {
         if (store_global) {
             ids_out[lane] = my_id;

@@ -326,8 +326,11 @@ def test_compile_refuses_what_the_path_does_not_cover(be):
     g, _ = moe_graph(1, 256, 8, 2, 256, DType.Q5K, DType.Q5K)
     with pytest.raises(M.Unsupported, match="Q5K"):
         be.compile(g)
-    g, _ = moe_graph(1, 256, 8, 2, 256, DType.Q4K, DType.Q4K, ep_band=(0, 4))
-    with pytest.raises(M.Unsupported, match="ep_band"):
+    g, _ = moe_graph(1, 256, 8, 2, 256, DType.Q4K, DType.Q4K, ep_band=(6, 4))   # band past the last expert
+    with pytest.raises(M.BackendError, match="ep_band"):
+        be.compile(g)
+    g, _ = moe_graph(1, 256, 8, 2, 256, DType.Q4K, DType.Q4K, ep_band=(0, 4))   # tensors hold 8 experts, the band says 4
+    with pytest.raises(M.BackendError, match="gate_exps"):
         be.compile(g)
     g, _ = moe_graph(1, 256, 8, 2, 256, DType.Q4K, DType.Q4K, swiglu_clamp=1.0, weight_before=True)
     with pytest.raises(M.BackendError):
@@ -741,6 +744,60 @@ def test_bucketed_decode_batches_bucket_exactly_and_keep_f32_accuracy(be, rows, 
         scale = float(np.abs(ref["dst"]).max())
         assert H.rel_l2(out, ref["dst"]) < REL_L2, (gopts, H.rel_l2(out, ref["dst"]))
         assert H.max_abs(out, ref["dst"]) < MAX_ABS * max(1.0, scale)
+
+
+@pytest.mark.parametrize("rows,opts", [(1, {}), (3, {"weight_before": True}), (20, {}), (20, {"weight_before": True}), (40, {})])
+def test_expert_parallel_bands_sum_to_the_full_layer(be, rows, opts):
+    """ep_band (crates/infr-core/src/graph.rs:1307-1319, crates/infr-vulkan/shaders/moe_ep_band_remap.comp):
+    routing stays global, the expert tensors hold one rank's shard, selections of foreign experts become
+    (id 0, weight 0).  The partial outputs of all ranks must add up to the single-device layer, and the
+    remapped ids / weights must be the shader's."""
+    ne, nff, E, K, W = 512, 256, 16, 4, 2
+    rng = np.random.default_rng(rows)
+    x = rng.standard_normal((rows, ne)).astype(np.float32)
+    router = (rng.standard_normal((E, ne)) * 0.05).astype(np.float32)
+    gate, up = _realistic(rng, E, nff, ne, H.Q4K), _realistic(rng, E, nff, ne, H.Q4K)
+    down = _realistic(rng, E, ne, nff, H.Q6K)
+    ds = rng.uniform(0.5, 1.5, E).astype(np.float32)
+
+    def run(band):
+        n_loc = E if band is None else band[1]
+        lo = 0 if band is None else band[0]
+        g = M.Graph()
+        xi = g.input(TensorDesc([rows, ne], DType.F32))
+        rt = g.weight(TensorDesc([E, ne], DType.F32))
+        gt, ut = g.weight(TensorDesc([n_loc, nff, ne], DType.Q4K)), g.weight(TensorDesc([n_loc, nff, ne], DType.Q4K))
+        dt = g.weight(TensorDesc([n_loc, ne, nff], DType.Q6K))
+        dst = g.weight(TensorDesc([n_loc], DType.F32))
+        yo = g.output(TensorDesc([rows, ne], DType.F32))
+        g.moe_ffn(x=xi, router=rt, gate_exps=gt, up_exps=ut, down_exps=dt, dst=yo, ne=ne, n_expert=E, n_used=K,
+                  n_ff_exp=nff, down_scale=dst, ep_band=band, **opts)
+        shard = lambda raw: raw.reshape(E, -1)[lo:lo + n_loc].reshape(-1)
+        keep = []
+        out = M.run_graph(be, g, [(xi, x), (rt, router), (gt, shard(gate)), (ut, shard(up)), (dt, shard(down)),
+                                  (dst, ds[lo:lo + n_loc].copy())], yo, rows * ne, keep=keep)
+        r = be.moe_routing(keep[0], 0)
+        for buf in keep[2]:
+            buf.free()
+        keep[3].free()
+        keep[0].free()
+        return out.reshape(rows, ne), r
+
+    full, rf = run(None)
+    ref = O.moe_ffn(x, router, gate, up, down, ne=ne, n_expert=E, n_used=K, n_ff_exp=nff, gate_dtype=H.Q4K,
+                    down_dtype=H.Q6K, down_scale=ds, **opts)
+    assert np.array_equal(rf["idx"], ref["idx"])
+    total = np.zeros_like(full)
+    for rank in range(W):
+        lo, n = rank * (E // W), E // W
+        part, rp = run((lo, n))
+        own = (rf["idx"] >= lo) & (rf["idx"] < lo + n)
+        assert np.array_equal(rp["idx"], np.where(own, rf["idx"] - lo, 0))
+        assert np.array_equal(bits(rp["w"]), bits(np.where(own, rf["w"], np.float32(0))))
+        total += part
+    tol = REL_L2_MFMA if rows >= 32 else REL_L2
+    assert H.rel_l2(total, ref["dst"]) < tol
+    assert H.rel_l2(total, full) < 1e-5   # the ranks' sum differs from one device only by reassociation
 
 
 def test_small_batches_keep_the_per_token_path(be):
