@@ -208,21 +208,23 @@ def main():
         total_us = lambda k: kernels[k]["avg_us"] * kernels[k]["launches"]
         cand = [k for k in kernels if k in flops] or [k for k in kernels if "alg_bytes" in kernels[k]]
         dom = max(cand, key=total_us, default=None)
-        if dom and dom in flops:
-            ach = flops[dom] / (kernels[dom]["avg_us"] * 1e-6) / 1e12
-            roofline = {"bound": "mfma", "kernel": dom, "achieved": round(ach, 1), "peak": MFMA_F16_PEAK_TFLOPS,
-                        "unit": "TFLOP/s", "frac": round(ach / MFMA_F16_PEAK_TFLOPS, 4), "traffic": None,
-                        "alg_flops_per_launch": flops[dom], "avg_launch_us": kernels[dom]["avg_us"]}
-        elif dom:
-            # HBM bytes per launch measured with hardware counters in a separate profiler run of this
-            # same command (profiles/), reported only for the workload they were taken on
-            traffic = None
+        # HBM bytes per launch measured with hardware counters in a separate profiler run of this same
+        # command (profiles/), reported only for the workload they were taken on
+        traffic = None
+        if dom:
             try:
                 with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
                     if n_layer == shape.n_layer:
-                        traffic = json.load(f).get(f"{args.config}/batch{batch}", {}).get(dom)
+                        key = f"{args.config}/tokens{batch}" if prefill else f"{args.config}/batch{batch}"
+                        traffic = json.load(f).get(key, {}).get(dom)
             except OSError:
                 pass
+        if dom and dom in flops:
+            ach = flops[dom] / (kernels[dom]["avg_us"] * 1e-6) / 1e12
+            roofline = {"bound": "mfma", "kernel": dom, "achieved": round(ach, 1), "peak": MFMA_F16_PEAK_TFLOPS,
+                        "unit": "TFLOP/s", "frac": round(ach / MFMA_F16_PEAK_TFLOPS, 4), "traffic": traffic,
+                        "alg_flops_per_launch": flops[dom], "avg_launch_us": kernels[dom]["avg_us"]}
+        elif dom:
             ach = alg[dom] / (kernels[dom]["avg_us"] * 1e-6) / 1e9
             roofline = {"bound": "hbm", "kernel": dom, "achieved": round(ach, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                         "frac": round(ach / HBM_PEAK_GBPS, 4), "traffic": traffic,
