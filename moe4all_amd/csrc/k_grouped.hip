@@ -492,12 +492,10 @@ __device__ __forceinline__ void tile_epilogue(const GroupedParams& p, const Tile
 // reads against them: one explicit "s_waitcnt vmcnt(n); s_barrier" per slice does both.  The issue
 // order is fixed (the same number of loads in every even and in every odd slice), so the number
 // of loads younger than the ones slice s needs is a compile-time constant.
+// M0 carries the LDS base of the transfer.  Nothing else in these kernels uses M0 (no other LDS-direct
+// load, no indirect register addressing, no message), so it is not saved around the load.
 __device__ __forceinline__ void dma16(const void* gsrc, uint32_t lds_base) {
-    uint32_t keep;
-    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off\n\ts_mov_b32 m0, %0"
-                 : "=&s"(keep)
-                 : "v"(gsrc), "s"(lds_base)
-                 : "memory");
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(gsrc), "s"(lds_base) : "memory");
 }
 template <int N>
 __device__ __forceinline__ void wait_loads_then_barrier() {
