@@ -660,6 +660,7 @@ def _run_batched(be, g, ids, data, rows, ne):
     (33, 256, 16, 4, 256, H.Q6K, H.Q4K),        # ragged tile, experts without tokens
     (40, 768, 6, 3, 512, H.Q8_0, H.Q8_0),       # three 256-feature down tiles, four 128-feature gate/up tiles
     (300, 256, 4, 2, 256, H.Q4K, H.Q8_0),       # buckets larger than one 128-token tile
+    (700, 512, 3, 2, 256, H.Q4K, H.Q4K),        # buckets of 400-500 pairs: 256-token tiles, then 128-token ones, then a ragged one
     (200, 2048, 128, 8, 768, H.Q4K, H.Q6K),     # config-2 layer shape
     (128, 2048, 128, 8, 768, H.Q8_0, H.Q8_0),   # config-1 layer shape
 ])
