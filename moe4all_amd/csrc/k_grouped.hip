@@ -5,7 +5,7 @@
 // per bucket (crates/infr-cpu/src/moe.rs:142-173).  Here:
 //
 //   bucket_kernel         offsets[e] = number of pairs whose expert id is below e, and the stable
-//                         scatter of the pairs into that order (one wavefront per expert; order is
+//                         scatter of the pairs into that order (one block per expert; order is
 //                         an integer contract and is reproduced exactly).
 //   rows_to_f16_kernel    activation rows -> f16 with one power-of-two scale per row (so any f32
 //                         magnitude fits), laid out in the k order the weight format unpacks to.
@@ -230,33 +230,35 @@ __global__ __launch_bounds__(256) void rows_to_f16_kernel(const float* __restric
 }
 
 // --------------------------------------------------------------------------------------------
-// One wavefront (= one block, so the experts spread over the CUs) per expert e in 0..n_expert; the
-// extra one writes the total and marks pairs whose id is out of range.  The wave stages the pair
-// ids in LDS (16-bit, chunks of 16384, sixteen 16-byte loads in flight per lane) and scans them
-// twice: count the pairs below e, then scatter.  The scan order is the flat (row, rank) order, so
-// buckets come out rows ascending.
+// One block of four wavefronts per expert e in 0..n_expert; the extra one marks pairs whose id is
+// out of range.  The block stages the pair ids in LDS (16-bit, chunks of 16384, sixteen 16-byte
+// loads in flight per thread), counts the pairs below e (= the bucket's offset), and then scatters
+// the pairs equal to e: each wavefront takes a contiguous quarter of the chunk, the quarters' hit
+// counts give every wavefront its base, and inside a quarter a wave-wide prefix keeps the flat
+// (row, rank) order, so buckets come out rows ascending.
 constexpr int kBucketChunk = 16384;
-__global__ __launch_bounds__(64) void bucket_kernel(const int32_t* __restrict__ ids, int n_pairs, int n_expert,
-                                                    int32_t* __restrict__ offsets, int32_t* __restrict__ pair_src,
-                                                    int32_t* __restrict__ slot_pair) {
+__global__ __launch_bounds__(256) void bucket_kernel(const int32_t* __restrict__ ids, int n_pairs, int n_expert,
+                                                     int32_t* __restrict__ offsets, int32_t* __restrict__ pair_src,
+                                                     int32_t* __restrict__ slot_pair) {
     __shared__ uint16_t s_ids[kBucketChunk];
-    const int lane = threadIdx.x;
+    __shared__ uint32_t s_cnt[4];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const uint32_t e = blockIdx.x;
     auto narrow = [&](int32_t v) { return (uint32_t)v < (uint32_t)n_expert ? (uint32_t)v : 0xFFFFu; };  // n_expert <= 2048
     auto stage = [&](int c0, int cn) {
         __syncthreads();  // orders the LDS reads of the previous chunk before these writes
-        // full groups of four ids: sixteen unconditional (index-clamped) 16-byte loads in flight per lane
+        // full groups of four ids: sixteen unconditional (index-clamped) 16-byte loads in flight per thread
         const int full = cn & ~3;
-        for (int b0 = 0; b0 < full; b0 += 64 * 4 * 16) {
+        if (full) {
             int4 v[16];
 #pragma unroll
             for (int j = 0; j < 16; j++) {
-                const int i = min(b0 + (j * 64 + lane) * 4, full - 4);
+                const int i = min((j * 256 + tid) * 4, full - 4);
                 v[j] = *reinterpret_cast<const int4*>(ids + c0 + i);
             }
 #pragma unroll
             for (int j = 0; j < 16; j++) {
-                const int i = b0 + (j * 64 + lane) * 4;
+                const int i = (j * 256 + tid) * 4;
                 if (i < full) {
                     const uint32_t lo = narrow(v[j].x) | (narrow(v[j].y) << 16), hi = narrow(v[j].z) | (narrow(v[j].w) << 16);
                     *reinterpret_cast<uint2*>(&s_ids[i]) = make_uint2(lo, hi);
@@ -264,73 +266,102 @@ __global__ __launch_bounds__(64) void bucket_kernel(const int32_t* __restrict__ 
             }
         }
         // the last one to three ids, padded to a group of four with 0xFFFF
-        if (lane < 4 && full < cn) s_ids[full + lane] = full + lane < cn ? (uint16_t)narrow(ids[c0 + full + lane]) : (uint16_t)0xFFFF;
+        if (tid < 4 && full < cn) s_ids[full + tid] = full + tid < cn ? (uint16_t)narrow(ids[c0 + full + tid]) : (uint16_t)0xFFFF;
         __syncthreads();
     };
-    uint32_t below = 0, run = 0;
-    for (int pass = 0; pass < 2; pass++) {
-        if (pass == 1) {
+    // eight ids of group g (one 128-bit LDS read); the staging filled the chunk's last partial group
+    // of four with 0xFFFF, the tail of a partial group of eight is masked here
+    auto ids8 = [&](int g, int cn, uint32_t (&id)[8]) {
+        const uint4 v = *reinterpret_cast<const uint4*>(&s_ids[8 * g]);
+        const uint32_t w[4] = {v.x, v.y, v.z, v.w};
 #pragma unroll
-            for (int d = 32; d >= 1; d >>= 1) below += __shfl_xor(below, d, 64);
-            if (lane == 0) offsets[e] = (int32_t)below;
-            run = below;
+        for (int c = 0; c < 8; c++) {
+            id[c] = (w[c >> 1] >> (16 * (c & 1))) & 0xFFFFu;
+            if (8 * g + c >= ((cn + 3) & ~3)) id[c] = 0xFFFFu;
         }
-        for (int c0 = 0; c0 < n_pairs; c0 += kBucketChunk) {
-            const int cn = min(kBucketChunk, n_pairs - c0);
-            if (pass == 0 || n_pairs > kBucketChunk) stage(c0, cn);   // a single chunk stays staged for the second pass
-            // eight ids per lane per step (one 128-bit LDS read); the staging filled the chunk's last
-            // partial group of four with 0xFFFF, the tail of a partial group of eight is masked here
-            const int n8 = (cn + 7) >> 3;
-            auto ids8 = [&](int g, uint32_t (&id)[8]) {
-                const uint4 v = *reinterpret_cast<const uint4*>(&s_ids[8 * g]);
-                const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+    };
+    auto wave_total = [&](uint32_t v) {
 #pragma unroll
-                for (int c = 0; c < 8; c++) {
-                    id[c] = (w[c >> 1] >> (16 * (c & 1))) & 0xFFFFu;
-                    if (8 * g + c >= ((cn + 3) & ~3)) id[c] = 0xFFFFu;
-                }
-            };
-            if (pass == 0) {
-#pragma unroll 4
-                for (int g = lane; g < n8; g += 64) {
-                    uint32_t id[8];
-                    ids8(g, id);
-#pragma unroll
-                    for (int c = 0; c < 8; c++) below += id[c] < e;
-                }
-            } else if (e == (uint32_t)n_expert) {
-                for (int i = lane; i < cn; i += 64)
-                    if (s_ids[i] == 0xFFFFu) slot_pair[c0 + i] = -1;
-            } else {
+        for (int d = 32; d >= 1; d >>= 1) v += __shfl_xor(v, d, 64);
+        return v;
+    };
+    const bool single = n_pairs <= kBucketChunk;   // a single chunk stays staged for the second pass
+
+    // ---- pass 0: pairs with an id below e
+    uint32_t below = 0;
+    for (int c0 = 0; c0 < n_pairs; c0 += kBucketChunk) {
+        const int cn = min(kBucketChunk, n_pairs - c0);
+        stage(c0, cn);
+        const int n8 = (cn + 7) >> 3;
 #pragma unroll 2
-                for (int g0 = 0; g0 < n8; g0 += 64) {
-                    const int g = g0 + lane;
-                    uint32_t id[8];
+        for (int g = tid; g < n8; g += 256) {
+            uint32_t id[8];
+            ids8(g, cn, id);
 #pragma unroll
-                    for (int c = 0; c < 8; c++) id[c] = 0xFFFFu;
-                    if (g < n8) ids8(g, id);
-                    uint32_t mine = 0;
+            for (int c = 0; c < 8; c++) below += id[c] < e;
+        }
+    }
+    below = wave_total(below);
+    __syncthreads();   // (s_cnt is free: nothing has used it yet)
+    if (lane == 0) s_cnt[wave] = below;
+    __syncthreads();
+    below = s_cnt[0] + s_cnt[1] + s_cnt[2] + s_cnt[3];
+    if (tid == 0) offsets[e] = (int32_t)below;
+
+    // ---- pass 1: scatter the pairs with id e (the extra block: mark the ids out of range)
+    uint32_t run = below;
+    for (int c0 = 0; c0 < n_pairs; c0 += kBucketChunk) {
+        const int cn = min(kBucketChunk, n_pairs - c0);
+        if (!single) stage(c0, cn);
+        if (e == (uint32_t)n_expert) {
+            for (int i = tid; i < cn; i += 256)
+                if (s_ids[i] == 0xFFFFu) slot_pair[c0 + i] = -1;
+            continue;
+        }
+        const int n8 = (cn + 7) >> 3;
+        const int per_wave = ((n8 + 255) >> 8) << 6;   // whole steps of 64 groups
+        const int g_lo = wave * per_wave, g_hi = min(n8, g_lo + per_wave);
+        // hits of this wavefront's quarter
+        uint32_t hits = 0;
+        for (int g = g_lo + lane; g < g_hi; g += 64) {
+            uint32_t id[8];
+            ids8(g, cn, id);
 #pragma unroll
-                    for (int c = 0; c < 8; c++) mine += id[c] == e;
-                    // inclusive prefix of the per-lane hit counts (a lane's eight pairs are consecutive)
-                    uint32_t incl = mine;
+            for (int c = 0; c < 8; c++) hits += id[c] == e;
+        }
+        hits = wave_total(hits);
+        __syncthreads();   // the previous chunk's readers of s_cnt are done
+        if (lane == 0) s_cnt[wave] = hits;
+        __syncthreads();
+        uint32_t base = run;
+        for (int w = 0; w < wave; w++) base += s_cnt[w];
+        run += s_cnt[0] + s_cnt[1] + s_cnt[2] + s_cnt[3];
+        for (int g0 = g_lo; g0 < g_hi; g0 += 64) {
+            const int g = g0 + lane;
+            uint32_t id[8];
 #pragma unroll
-                    for (int d = 1; d < 64; d <<= 1) {
-                        const uint32_t o = __shfl_up(incl, d, 64);
-                        if (lane >= d) incl += o;
-                    }
-                    uint32_t pos = run + incl - mine;
+            for (int c = 0; c < 8; c++) id[c] = 0xFFFFu;
+            if (g < g_hi) ids8(g, cn, id);
+            uint32_t mine = 0;
 #pragma unroll
-                    for (int c = 0; c < 8; c++) {
-                        if (id[c] == e) {
-                            pair_src[pos] = c0 + 8 * g + c;
-                            slot_pair[c0 + 8 * g + c] = (int32_t)pos;
-                            pos++;
-                        }
-                    }
-                    run += __shfl(incl, 63, 64);
+            for (int c = 0; c < 8; c++) mine += id[c] == e;
+            // inclusive prefix of the per-lane hit counts (a lane's eight pairs are consecutive)
+            uint32_t incl = mine;
+#pragma unroll
+            for (int d = 1; d < 64; d <<= 1) {
+                const uint32_t o = __shfl_up(incl, d, 64);
+                if (lane >= d) incl += o;
+            }
+            uint32_t pos = base + incl - mine;
+#pragma unroll
+            for (int c = 0; c < 8; c++) {
+                if (id[c] == e) {
+                    pair_src[pos] = c0 + 8 * g + c;
+                    slot_pair[c0 + 8 * g + c] = (int32_t)pos;
+                    pos++;
                 }
             }
+            base += __shfl(incl, 63, 64);
         }
     }
 }
@@ -822,7 +853,7 @@ void launch_rows_to_f16(hipStream_t s, int weight_dt, const float* src, int rows
 
 void launch_bucket(hipStream_t s, const int32_t* ids, int n_pairs, int n_expert, int32_t* offsets, int32_t* pair_src,
                    int32_t* slot_pair) {
-    INFR_LAUNCH(bucket_kernel, dim3(n_expert + 1), dim3(64), 0, s, ids, n_pairs, n_expert, offsets, pair_src, slot_pair);
+    INFR_LAUNCH(bucket_kernel, dim3(n_expert + 1), dim3(256), 0, s, ids, n_pairs, n_expert, offsets, pair_src, slot_pair);
 }
 
 void launch_grouped_gate_up(hipStream_t s, int dt, const GroupedParams& p) {
