@@ -721,6 +721,7 @@ def test_batched_moe_ffn_option_variants_match_oracle(be):
     (19, 256, 16, 4, 256, H.Q6K, H.Q4K),       # experts without tokens, odd bucket sizes
     (31, 2048, 128, 8, 768, H.Q8_0, H.Q8_0),   # the largest batch below the matrix-core path
     (18, 256, 24, 17, 256, H.Q4K, H.Q6K),      # more ranks than the per-token down kernel combines: bucketed down + combine
+    (70, 320, 8, 2, 96, H.Q8_0, H.Q8_0),       # ne is no multiple of 256: no matrix-core path, the bucketed GEMV takes any row count
 ])
 def test_bucketed_decode_batches_bucket_exactly_and_keep_f32_accuracy(be, rows, ne, E, K, nff, gdt, ddt):
     """16..31 token rows: pairs are bucketed by expert and the gate/up rows of an expert serve two tokens
