@@ -32,20 +32,27 @@ SEED0 = 20260101
 N_TOKENS = 8  # distinct activation sets rotated through the steps
 
 
-def build_stack(be, shape, n_layer, batch):
-    """One graph with n_layer MoeFfn ops (+ shared-expert ops), weights generated in HBM."""
+def build_stack(be, shape, n_layer, batch, sublayer=False):
+    """One graph with n_layer MoeFfn ops (+ shared-expert ops), weights generated in HBM.  With
+    `sublayer` every layer is the model's whole FFN sublayer: y = x + ffn(rmsnorm(x) * w)."""
     g = M.Graph()
     layers, ids = [], []
     for l in range(n_layer):
         lw = synth.LayerWeights(be, shape, SEED0, l, on_device=True)
         layers.append(lw)
-        x = g.input(TensorDesc([batch, shape.ne], DType.F32))
+        x = x_raw = g.input(TensorDesc([batch, shape.ne], DType.F32))
+        out = g.output(TensorDesc([batch, shape.ne], DType.F32))
+        norm_w = None
+        if sublayer:
+            norm_w = g.weight(TensorDesc([shape.ne], DType.F32))
+            x = g.internal(TensorDesc([batch, shape.ne], DType.F32))
+            g.rms_norm(x=x_raw, weight=norm_w, dst=x, rows=batch, dim=shape.ne, eps=1e-6)
         router = g.weight(TensorDesc([shape.n_expert, shape.ne], DType.F32))
         gate = g.weight(TensorDesc([shape.n_expert, shape.n_ff, shape.ne], shape.gate_dtype))
         up = g.weight(TensorDesc([shape.n_expert, shape.n_ff, shape.ne], shape.gate_dtype))
         down = g.weight(TensorDesc([shape.n_expert, shape.ne, shape.n_ff], shape.down_dtype))
-        dst = g.output(TensorDesc([batch, shape.ne], DType.F32))
-        d = dict(x=x, router=router, gate=gate, up=up, down=down, dst=dst)
+        dst = g.internal(TensorDesc([batch, shape.ne], DType.F32)) if sublayer else out
+        d = dict(x=x_raw, router=router, gate=gate, up=up, down=down, dst=out, norm_w=norm_w)
         if shape.shared_ff:
             moe = g.internal(TensorDesc([batch, shape.ne], DType.F32))
             g.moe_ffn(x=x, router=router, gate_exps=gate, up_exps=up, down_exps=down, dst=moe, ne=shape.ne,
@@ -65,6 +72,8 @@ def build_stack(be, shape, n_layer, batch):
         else:
             g.moe_ffn(x=x, router=router, gate_exps=gate, up_exps=up, down_exps=down, dst=dst, ne=shape.ne,
                       n_expert=shape.n_expert, n_used=shape.n_used, n_ff_exp=shape.n_ff)
+        if sublayer:
+            g.add(a=x_raw, b=dst, dst=out, n=batch * shape.ne)
         ids.append(d)
     return g, layers, ids
 
@@ -81,6 +90,10 @@ def main():
     ap.add_argument("--tokens", type=int, default=2048, help="prefill chunk size for c4/c4k")
     ap.add_argument("--layers", type=int, default=0, help="override the layer count (0 = the config's)")
     ap.add_argument("--batch", type=int, default=1)
+    ap.add_argument("--sublayer", action="store_true",
+                    help="time the model's whole FFN sublayer per layer (RmsNorm -> MoeFfn [+ shared expert] -> "
+                         "residual Add) instead of the MoeFfn op alone; not the headline metric")
+    ap.add_argument("--no-fusion", action="store_true", help="one launch per op (infr_hip_config.disable_op_fusion)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-timing", action="store_true")
     ap.add_argument("--copy-probe-mib", type=int, default=0,
@@ -92,6 +105,8 @@ def main():
               file=sys.stderr)
         sys.exit(2)
 
+    if args.sublayer:
+        args.no_cpu_baseline = True   # the CPU sample times Op::MoeFfn alone
     prefill = args.config in ("c4", "c4k")
     shape = {"c1": synth.CONFIG_1, "c2": synth.CONFIG_2, "c5": synth.CONFIG_5,
              "c4": synth.MoeShape(f"c4-prefill-{args.tokens}-zipf1.1-q8_0", 1, 2048, 128, 8, 768, DType.Q8_0, DType.Q8_0),
@@ -99,10 +114,11 @@ def main():
                                    DType.Q6K)}[args.config]
     n_layer = args.layers or shape.n_layer
     batch = args.tokens if prefill else args.batch
-    be = M.Backend(0)
+    be = M.Backend(0, disable_op_fusion=args.no_fusion)
     caps = be.capabilities()
     t_setup = time.time()
-    g, layers, ids = build_stack(be, shape, n_layer, batch)
+    g, layers, ids = build_stack(be, shape, n_layer, batch, args.sublayer)
+    norm_w = be.buffer_from(np.ones(shape.ne, np.float32)) if args.sublayer else None
     plan = be.compile(g)
     if prefill:
         # skewed expert popularity through the op's own inputs: x[:, 0] = 1, router[e, 0] = ln Zipf(1.1)
@@ -134,6 +150,8 @@ def main():
             b.bind(d["up"], lw.up).bind(d["down"], lw.down).bind(d["dst"], ybufs[l])
             if shape.shared_ff:
                 b.bind(d["sg"], lw.shared[0]).bind(d["su"], lw.shared[1]).bind(d["sd"], lw.shared[2])
+            if norm_w is not None:
+                b.bind(d["norm_w"], norm_w)
         binds.append(b)
     if args.copy_probe_mib:
         n = args.copy_probe_mib << 20
@@ -157,7 +175,7 @@ def main():
     tok_s = batch * args.steps / elapsed
 
     # distinct experts actually selected per layer (batch > 1 shares experts between tokens)
-    r = be.moe_routing(plan, 0)
+    r = be.moe_routing(plan, 1 if args.sublayer else 0)
     distinct = len(set(r["idx"].ravel().tolist()))
     layer_bytes = shape.algorithmic_bytes(batch, distinct if batch > 1 else None)
     layer_gbps = layer_bytes * n_layer / (ms_per_step * 1e-3) / 1e9
@@ -184,6 +202,7 @@ def main():
         }
         # the decode kernel that routes its own token row also reads that row's logits
         alg["moe_route_gate_up"] = alg["moe_gate_up"] + batch * shape.n_expert * 4
+        alg["rms_norm_router_logits"] = alg["router_logits"] + shape.ne * 4 + batch * shape.ne * 4
         if shape.shared_ff:
             sh_gate_b = M.backend.bytes_for(shape.gate_dtype, shape.shared_ff * shape.ne)
             sh_down_b = M.backend.bytes_for(shape.down_dtype, shape.ne * shape.shared_ff)
@@ -214,7 +233,7 @@ def main():
         if dom:
             try:
                 with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
-                    if n_layer == shape.n_layer:
+                    if n_layer == shape.n_layer and not args.sublayer and not args.no_fusion:
                         key = f"{args.config}/tokens{batch}" if prefill else f"{args.config}/batch{batch}"
                         traffic = json.load(f).get(key, {}).get(dom)
             except OSError:
@@ -262,7 +281,8 @@ def main():
         "metric": "MoE prefill tok/s" if prefill else "MoE decode tok/s", "value": round(tok_s, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": shape.name if n_layer == shape.n_layer else f"{shape.name}[{n_layer} layers]",
+        "config": {"workload": (shape.name if n_layer == shape.n_layer else f"{shape.name}[{n_layer} layers]") +
+                               ("+rmsnorm+residual" if args.sublayer else "") + ("/unfused" if args.no_fusion else ""),
                    "layers": n_layer, "hidden": shape.ne, "experts": shape.n_expert, "top_k": shape.n_used,
                    "intermediate": shape.n_ff, "gate_up": shape.gate_dtype.name, "down": shape.down_dtype.name,
                    "shared_intermediate": shape.shared_ff, "batch": batch, "parallelism": "single-gpu",

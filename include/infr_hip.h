@@ -83,7 +83,9 @@ typedef enum infr_op_kind {
     INFR_OP_ADD = 3,                   /* Op::Add                                   */
     INFR_OP_MOE_SHARED_EXPERT_ADD = 4, /* Op::MoeSharedExpertAdd  graph.rs:1449-1463 */
     INFR_OP_COPY = 5,                  /* Op::Copy                graph.rs:1230-1237 */
-    INFR_OP_COPY_STRIDED = 6           /* Op::CopyStrided         graph.rs:1238-1251 */
+    INFR_OP_COPY_STRIDED = 6,          /* Op::CopyStrided         graph.rs:1238-1251 */
+    INFR_OP_RMS_NORM = 7,              /* Op::RmsNorm             graph.rs:160-169   */
+    INFR_OP_RMS_NORM_ADD = 8           /* Op::RmsNormAdd          graph.rs:170-179   */
 } infr_op_kind;
 
 /* Field-for-field Op::MoeFfn.  Option<TensorId> = INFR_NO_TENSOR; Option<f32> and
@@ -139,6 +141,15 @@ typedef struct infr_op_copy {
     uint32_t rows, n;
 } infr_op_copy;
 
+/* Op::RmsNorm: dst = rmsnorm(x) * weight over the last `dim` of each of `rows` rows;
+ * Op::RmsNormAdd: dst += rmsnorm(x) * weight (crates/infr-cpu/src/lib.rs:1046-1093).  x, dst: F32
+ * [rows, dim]; weight: F32 [dim].  dst may be x. */
+typedef struct infr_op_rms_norm {
+    uint32_t x, weight, dst;
+    uint32_t rows, dim;
+    float eps;
+} infr_op_rms_norm;
+
 typedef struct infr_op {
     int32_t kind; /* infr_op_kind */
     union {
@@ -148,6 +159,7 @@ typedef struct infr_op {
         infr_op_add add;
         infr_op_moe_shared_expert_add moe_shared_expert_add;
         infr_op_copy copy;
+        infr_op_rms_norm rms_norm;
     } u;
 } infr_op;
 
@@ -185,7 +197,11 @@ typedef struct infr_hip_config {
      * (f16 operands, f32 accumulation) instead of the f32-accurate GEMV paths; 0 selects the
      * built-in default (32). */
     uint32_t moe_batched_min_rows;
-    uint32_t reserved[6];
+    /* Non-zero: every op of a graph gets its own launch(es); no neighbouring ops are folded into one
+     * kernel.  The escape hatch the reference's backends keep for their rewrites
+     * (crates/infr-core/src/fusion.rs:49-52, `enabled`); results are bit-identical either way. */
+    uint32_t disable_op_fusion;
+    uint32_t reserved[5];
 } infr_hip_config;
 
 /* Construction of the backend object (reference: VulkanBackend::new / CpuBackend::new,

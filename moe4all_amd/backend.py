@@ -127,9 +127,13 @@ class _OpCopy(C.Structure):
     _fields_ = [(n, C.c_uint32) for n in ("src", "src_off", "src_stride", "dst", "dst_off", "dst_stride", "rows", "n")]
 
 
+class _OpRmsNorm(C.Structure):
+    _fields_ = [(n, C.c_uint32) for n in ("x", "weight", "dst", "rows", "dim")] + [("eps", C.c_float)]
+
+
 class _OpUnion(C.Union):
     _fields_ = [("moe_ffn", _OpMoeFfn), ("linear", _OpLinear), ("gated_act", _OpGatedAct), ("add", _OpAdd),
-                ("moe_shared_expert_add", _OpSharedAdd), ("copy", _OpCopy)]
+                ("moe_shared_expert_add", _OpSharedAdd), ("copy", _OpCopy), ("rms_norm", _OpRmsNorm)]
 
 
 class _Op(C.Structure):
@@ -154,7 +158,7 @@ class _Caps(C.Structure):
 
 class _Config(C.Structure):
     _fields_ = [("disable_graph_replay", C.c_uint32), ("moe_batched_min_rows", C.c_uint32),
-                ("reserved", C.c_uint32 * 6)]
+                ("disable_op_fusion", C.c_uint32), ("reserved", C.c_uint32 * 5)]
 
 
 class _ProfEntry(C.Structure):
@@ -351,6 +355,13 @@ class Graph:
             src, src_off, src_stride, dst, dst_off, dst_stride, rows, n)
         self.ops.append(op)
 
+    def rms_norm(self, *, x, weight, dst, rows, dim, eps, add=False) -> None:
+        """Op::RmsNorm (crates/infr-core/src/graph.rs:160-169); add=True is Op::RmsNormAdd (:170-179)."""
+        op = _Op(kind=8 if add else 7)
+        r = op.u.rms_norm
+        r.x, r.weight, r.dst, r.rows, r.dim, r.eps = x, weight, dst, rows, dim, eps
+        self.ops.append(op)
+
     def push_raw(self, kind: int) -> None:
         """Append an op of an arbitrary kind code (used to test the Unsupported path)."""
         self.ops.append(_Op(kind=kind))
@@ -437,10 +448,12 @@ class Bindings:
 class Backend:
     """The gfx950 compute device (crates/infr-core/src/backend.rs:630 `trait Backend`)."""
 
-    def __init__(self, device: int = 0, *, disable_graph_replay: bool = False, moe_batched_min_rows: int = 0):
+    def __init__(self, device: int = 0, *, disable_graph_replay: bool = False, moe_batched_min_rows: int = 0,
+                 disable_op_fusion: bool = False):
         self._h = None
         lib = load_library()
-        cfg = _Config(disable_graph_replay=int(disable_graph_replay), moe_batched_min_rows=moe_batched_min_rows)
+        cfg = _Config(disable_graph_replay=int(disable_graph_replay), moe_batched_min_rows=moe_batched_min_rows,
+                      disable_op_fusion=int(disable_op_fusion))
         h = _V()
         _check(lib.infr_hip_create(device, C.byref(cfg), C.byref(h)))
         self._h = h.value
@@ -589,8 +602,11 @@ def run_graph(be: Backend, g: Graph, bound: Sequence, out: int, out_n: int, keep
         be.upload(buf, raw)
         bufs.append(buf)
         b.bind(tid, buf)
-    ob = be.alloc(out_n * 4, BufferUsage.Readback)
-    b.bind(out, ob)
+    ob = b.get(out)   # an output the caller pre-filled (an op that accumulates, or runs in place)
+    own = ob is None
+    if own:
+        ob = be.alloc(out_n * 4, BufferUsage.Readback)
+        b.bind(out, ob)
     be.execute(plan, b)
     res = be.download(ob, out_n * 4, np.float32).copy()
     if keep is not None:
@@ -598,6 +614,7 @@ def run_graph(be: Backend, g: Graph, bound: Sequence, out: int, out_n: int, keep
     else:
         for buf in bufs:
             buf.free()
-        ob.free()
+        if own:
+            ob.free()
         plan.free()
     return res

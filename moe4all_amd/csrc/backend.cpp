@@ -123,6 +123,8 @@ struct infr_hip_plan {
         Fuse kind = kPlain;
         uint32_t a = 0, b = 0;   // kGateUpAct: index of the up Linear and of the GatedAct; kLinearAdd: index of the Add;
                                  // kMoeShared: index of the always-on expert's first Linear and of its down Linear
+        uint32_t norm = 0;       // MoeFfn: 1 + index of the Op::RmsNorm its logits kernel applies to the token row
+        uint32_t res = 0;        // MoeFfn: 1 + index of the following Op::Add folded into the combine
     };
     std::vector<FuseOp> fuse;
     std::vector<FuseOp> fuse_head;     // kMoeShared: the records of the ops it absorbed, as they were before
@@ -653,6 +655,19 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
                     c.set(INFR_ERR_INVALID, "MoeSharedExpertAdd: rows*n exceeds an operand");
                 break;
             }
+            case INFR_OP_RMS_NORM:
+            case INFR_OP_RMS_NORM_ADD: {
+                const infr_op_rms_norm& nr = op.u.rms_norm;
+                if (!(c.tensor(nr.x, "RmsNorm.x") && c.tensor(nr.weight, "RmsNorm.weight") && c.tensor(nr.dst, "RmsNorm.dst"))) break;
+                c.want_f32(nr.x, "RmsNorm.x"); c.want_f32(nr.weight, "RmsNorm.weight"); c.want_f32(nr.dst, "RmsNorm.dst");
+                c.want_writable(nr.dst, "RmsNorm.dst");
+                if (!nr.dim) { c.set(INFR_ERR_INVALID, "RmsNorm: dim must be positive"); break; }
+                const uint64_t tot = (uint64_t)nr.rows * nr.dim;
+                if (c.n(nr.x) < tot || c.n(nr.dst) < tot || c.n(nr.weight) < nr.dim)
+                    c.set(INFR_ERR_INVALID, "RmsNorm: rows*dim exceeds an operand");
+                if (nr.rows > 0x7fffffffu / nr.dim) c.set(INFR_ERR_UNSUPPORTED, "RmsNorm: more than 2^31 elements");
+                break;
+            }
             case INFR_OP_COPY:
             case INFR_OP_COPY_STRIDED: {
                 const infr_op_copy& cp = op.u.copy;
@@ -693,8 +708,9 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
     // once.  The fused kernels run the same inner products and the same rounding sequence, so the
     // results are the bits the separate ops give.
     plan->fuse.assign(g->n_ops, infr_hip_plan::FuseOp{});
+    plan->fuse_head = plan->fuse;
     size_t zero_rows = 0;
-    {
+    if (!be->cfg.disable_op_fusion) {
         std::vector<int> reads(plan->tensors.size(), 0), writes(plan->tensors.size(), 0);
         auto rd = [&](uint32_t t) { if (t != INFR_NO_TENSOR && t < reads.size()) reads[t]++; };
         auto wr = [&](uint32_t t) { if (t != INFR_NO_TENSOR && t < writes.size()) writes[t]++; };
@@ -717,6 +733,10 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
                 }
                 case INFR_OP_COPY:
                 case INFR_OP_COPY_STRIDED: rd(op.u.copy.src); rd(op.u.copy.dst); wr(op.u.copy.dst); break;   // a partial write keeps the rest
+                case INFR_OP_RMS_NORM: rd(op.u.rms_norm.x); rd(op.u.rms_norm.weight); wr(op.u.rms_norm.dst); break;
+                case INFR_OP_RMS_NORM_ADD:
+                    rd(op.u.rms_norm.x); rd(op.u.rms_norm.weight); rd(op.u.rms_norm.dst); wr(op.u.rms_norm.dst);
+                    break;
                 default: break;
             }
         }
@@ -803,6 +823,37 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
             plan->fuse[oi].a = oi + 1;
             plan->fuse[oi].b = oi + 4;
             for (uint32_t k = oi + 1; k <= oi + 5; k++) plan->fuse[k].kind = infr_hip_plan::kSkip;
+        }
+        // MoeFfn -> Add (the residual; the reference's moe_add rewrite, crates/infr-core/src/fusion.rs:20-24):
+        // every combine kernel ends with "other operand + finished sum", the Add's own rounding.
+        // RmsNorm -> MoeFfn on one token row (fusion.rs:15-19 with moe_ok): the logits kernel normalises the
+        // raw row while staging it and stores the normalised row, which the expert kernels then read.
+        for (uint32_t oi = 0; oi < g->n_ops; oi++) {
+            if (plan->ops[oi].kind != INFR_OP_MOE_FFN) continue;
+            const infr_hip_plan::Fuse kind = plan->fuse[oi].kind;
+            if (kind != infr_hip_plan::kPlain && kind != infr_hip_plan::kMoeShared) continue;
+            const infr_op_moe_ffn& m = plan->ops[oi].u.moe_ffn;
+            const MoeScratch& sc = plan->moe[oi];
+            const uint32_t nx = kind == infr_hip_plan::kMoeShared ? oi + 6 : oi + 1;
+            const uint32_t sum_t = kind == infr_hip_plan::kMoeShared ? plan->ops[oi + 5].u.add.dst : m.dst;
+            if (nx < g->n_ops && plan->ops[nx].kind == INFR_OP_ADD && plan->fuse[nx].kind == infr_hip_plan::kPlain && sc.rows > 0) {
+                const infr_op_add& ad = plan->ops[nx].u.add;
+                const bool one_side = (ad.a == sum_t) != (ad.b == sum_t);
+                if (one_side && temp(sum_t) && (uint64_t)ad.n == (uint64_t)sc.rows * m.ne) {
+                    plan->fuse[oi].res = nx + 1;
+                    plan->fuse[nx].kind = infr_hip_plan::kSkip;
+                }
+            }
+            if (oi > 0 && plan->ops[oi - 1].kind == INFR_OP_RMS_NORM && plan->fuse[oi - 1].kind == infr_hip_plan::kPlain) {
+                const infr_op_rms_norm& nr = plan->ops[oi - 1].u.rms_norm;
+                int re = 1, rb = 4;
+                geometry(c.dt(m.router), &re, &rb);
+                if (nr.rows == 1 && sc.rows == 1 && !sc.batched && !sc.bucketed && nr.dim == m.ne && nr.dst == m.router_x &&
+                    nr.x != nr.dst && infr::router_logits_can_norm(c.dt(m.router), (size_t)(m.ne / re) * rb, (int)m.ne, 1)) {
+                    plan->fuse[oi].norm = oi;   // 1 + (oi - 1)
+                    plan->fuse[oi - 1].kind = infr_hip_plan::kSkip;
+                }
+            }
         }
     }
     const size_t zero_off = arena;
@@ -972,7 +1023,25 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                 rp.ep_n = m.has_ep_band ? (int)m.ep_n_local : 0;
                 const uint32_t n_local = m.has_ep_band ? m.ep_n_local : m.n_expert;   // experts the weight tensors hold
                 rp.ids = sc.ids; rp.weights = sc.weights; rp.probs = sc.probs;
-                {
+                bool normed = false;
+                if (fz.norm) {
+                    const infr_op_rms_norm& nr = plan->ops[fz.norm - 1].u.rms_norm;
+                    if (!(need(nr.x, "RmsNorm.x") && need(nr.weight, "RmsNorm.weight") && need(nr.dst, "RmsNorm.dst")))
+                        return INFR_ERR_BACKEND;
+                    infr::RouterNorm rn;
+                    rn.weight = (const float*)ptr[nr.weight]; rn.eps = nr.eps; rn.xn_out = (float*)ptr[nr.dst];
+                    {
+                        Timed t(be, "rms_norm_router_logits");
+                        normed = infr::launch_router_logits(s, (const uint8_t*)ptr[m.router], plan->tensors[m.router].dtype,
+                                                            router_row_bytes, (const float*)ptr[nr.x], (int)m.ne,
+                                                            (int)m.n_expert, rows, sc.logits, &rn);
+                    }
+                    if (!normed) {   // operands the fold cannot take (alignment): the op on its own
+                        Timed t(be, "rms_norm");
+                        infr::launch_rms_norm(s, (const float*)ptr[nr.x], rn.weight, rn.xn_out, 1, (int)nr.dim, nr.eps, 0);
+                    }
+                }
+                if (!normed) {
                     Timed t(be, "router_logits");
                     if (!infr::launch_router_logits(s, (const uint8_t*)ptr[m.router], plan->tensors[m.router].dtype,
                                                     router_row_bytes, (const float*)ptr[m.router_x], (int)m.ne,
@@ -1007,6 +1076,14 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                 gp.skip_zero_w = (int)m.has_ep_band;
                 gp.h = sc.h; gp.dst = (float*)ptr[m.dst]; gp.n_cu = n_cu;
                 gp.x = (const float*)ptr[m.x];
+                if (fz.res) {
+                    const infr_op_add& ad = plan->ops[fz.res - 1].u.add;
+                    const uint32_t sum_t = fz.kind == infr_hip_plan::kMoeShared ? plan->ops[fz.b + 1].u.add.dst : m.dst;
+                    const uint32_t other = ad.a == sum_t ? ad.b : ad.a;
+                    if (!(need(other, "Add.a") && need(ad.dst, "Add.dst"))) return INFR_ERR_BACKEND;
+                    gp.addend = (const float*)ptr[other];
+                    gp.dst = (float*)ptr[ad.dst];
+                }
                 if (sc.batched) {
                     const int pairs = rows * (int)m.n_used;
                     {
@@ -1051,7 +1128,7 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                     {
                         Timed t(be, "moe_unbucket_combine");
                         infr::launch_unbucket_combine(s, sc.y, sc.slot_pair, sc.weights, rows, (int)m.ne, (int)m.n_used,
-                                                      (int)m.weight_before, gp.dst, 0, sc.hs);
+                                                      (int)m.weight_before, gp.dst, 0, sc.hs, gp.addend);
                     }
                     break;
                 }
@@ -1088,12 +1165,14 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                     }
                     {
                         Timed t(be, "moe_down_bucketed");
-                        infr::launch_moe_down_bucketed(s, gp);
+                        infr::MoeGemvParams gd = gp;
+                        gd.addend = nullptr;   // the kernel writes per-pair rows; the addend joins the combined sum
+                        infr::launch_moe_down_bucketed(s, gd);
                     }
                     {
                         Timed t(be, "moe_unbucket_combine");
                         infr::launch_unbucket_combine(s, sc.y, sc.slot_pair, sc.weights, rows, (int)m.ne, (int)m.n_used,
-                                                      (int)m.weight_before, gp.dst, 1);
+                                                      (int)m.weight_before, gp.dst, 1, nullptr, gp.addend);
                     }
                     break;
                 }
@@ -1104,12 +1183,12 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                     const infr_op_linear& ld = plan->ops[fz.b].u.linear;
                     const infr_op_add& ad = plan->ops[fz.b + 1].u.add;
                     if (!(need(lg.weight, "Linear.weight") && need(lu.weight, "Linear.weight") &&
-                          need(ld.weight, "Linear.weight") && need(ad.dst, "Add.dst")))
+                          need(ld.weight, "Linear.weight") && (fz.res || need(ad.dst, "Add.dst"))))
                         return INFR_ERR_BACKEND;
                     gp.sh_gate = (const uint8_t*)ptr[lg.weight];
                     gp.sh_up = (const uint8_t*)ptr[lu.weight];
                     gp.sh_down = (const uint8_t*)ptr[ld.weight];
-                    gp.dst = (float*)ptr[ad.dst];
+                    if (!fz.res) gp.dst = (float*)ptr[ad.dst];
                 }
                 gp.route = rp;
                 // Every block of the gate/up kernel routes its own token row when that is cheaper than a
@@ -1167,6 +1246,16 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                 Timed t(be, "moe_shared_expert_add");
                 infr::launch_moe_shared_expert_add(s, (const float*)ptr[a.moe], (const float*)ptr[a.shexp],
                                                    (const float*)ptr[a.gate], (float*)ptr[a.dst], (int)a.rows, (int)a.n);
+                break;
+            }
+            case INFR_OP_RMS_NORM:
+            case INFR_OP_RMS_NORM_ADD: {
+                const infr_op_rms_norm& nr = op.u.rms_norm;
+                if (!(need(nr.x, "RmsNorm.x") && need(nr.weight, "RmsNorm.weight") && need(nr.dst, "RmsNorm.dst")))
+                    return INFR_ERR_BACKEND;
+                Timed t(be, "rms_norm");
+                infr::launch_rms_norm(s, (const float*)ptr[nr.x], (const float*)ptr[nr.weight], (float*)ptr[nr.dst],
+                                      (int)nr.rows, (int)nr.dim, nr.eps, op.kind == INFR_OP_RMS_NORM_ADD);
                 break;
             }
             case INFR_OP_COPY:

@@ -221,6 +221,28 @@ __device__ __forceinline__ float wave_sum(float v) {
     v = row16_sum(v);
     return (readlane_f(v, 0) + readlane_f(v, 16)) + (readlane_f(v, 32) + readlane_f(v, 48));
 }
+// Sum over a block of 256 threads, the same bits in every thread; red: 4 floats of LDS.
+__device__ __forceinline__ float block256_sum(float v, float* red) {
+    v = wave_sum(v);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return (red[0] + red[1]) + (red[2] + red[3]);
+}
+// Op::RmsNorm's row scale 1 / sqrt(sum(x^2) / dim + eps) (crates/infr-cpu/src/lib.rs:1062-1063).
+__device__ __forceinline__ float rms_scale(float sumsq, int dim, float eps) {
+    return __fdiv_rn(1.0f, __fsqrt_rn(__fadd_rn(__fdiv_rn(sumsq, (float)dim), eps)));
+}
+// A thread's share of a row's sum of squares when thread t of 256 owns the float4s t, t + 256, ...
+__device__ __forceinline__ float sumsq4(float acc, const float4& f) {
+    acc = __fmaf_rn(f.x, f.x, acc);
+    acc = __fmaf_rn(f.y, f.y, acc);
+    acc = __fmaf_rn(f.z, f.z, acc);
+    return __fmaf_rn(f.w, f.w, acc);
+}
+__device__ __forceinline__ float4 rms_apply4(const float4& x, float s, const float4& w) {
+    return make_float4(__fmul_rn(__fmul_rn(x.x, s), w.x), __fmul_rn(__fmul_rn(x.y, s), w.y),
+                       __fmul_rn(__fmul_rn(x.z, s), w.z), __fmul_rn(__fmul_rn(x.w, s), w.w));
+}
 __device__ __forceinline__ float wave_max(float v) {
     v = fmaxf(v, dpp_f<kDppXor1>(v));
     v = fmaxf(v, dpp_f<kDppXor2>(v));

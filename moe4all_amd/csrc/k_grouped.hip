@@ -772,8 +772,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 template <class Y>
 __global__ __launch_bounds__(256) void unbucket_combine_kernel(const Y* __restrict__ y, const int32_t* __restrict__ slot_pair,
                                                                const float* __restrict__ weights, int ne, int n_used,
-                                                               int weight_before, float* __restrict__ dst, int identity,
-                                                               const float* __restrict__ pair_scale) {
+                                                               int weight_before, float* dst, int identity,
+                                                               const float* __restrict__ pair_scale, const float* addend) {
     const size_t row = blockIdx.y;
     const int i = (blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= ne) return;
@@ -808,6 +808,17 @@ __global__ __launch_bounds__(256) void unbucket_combine_kernel(const Y* __restri
         acc.w = __fadd_rn(acc.w, __fmul_rn(w, v[3]));
     }
     float* o = dst + row * ne + i;
+    if (addend) {   // a following Op::Add folded in: the finished sum is added to the other operand
+        const float* ad = addend + row * ne + i;
+        if (i + 3 < ne) {
+            const float4 f = *reinterpret_cast<const float4*>(ad);
+            acc.x = __fadd_rn(f.x, acc.x); acc.y = __fadd_rn(f.y, acc.y);
+            acc.z = __fadd_rn(f.z, acc.z); acc.w = __fadd_rn(f.w, acc.w);
+        } else {
+            float* a = &acc.x;
+            for (int q = 0; i + q < ne; q++) a[q] = __fadd_rn(ad[q], a[q]);
+        }
+    }
     if (i + 3 < ne) *reinterpret_cast<float4*>(o) = acc;
     else {
         const float* a = &acc.x;
@@ -869,15 +880,16 @@ void launch_grouped_down(hipStream_t s, int dt, const GroupedParams& p) {
 }
 
 void launch_unbucket_combine(hipStream_t s, const void* y, const int32_t* slot_pair, const float* weights, int rows,
-                             int ne, int n_used, int weight_before, float* dst, int identity, const float* pair_scale) {
+                             int ne, int n_used, int weight_before, float* dst, int identity, const float* pair_scale,
+                             const float* addend) {
     if (rows <= 0) return;
     const dim3 grid((ne + 1023) / 1024, rows), block(256);
     if (pair_scale)
         INFR_LAUNCH(unbucket_combine_kernel<_Float16>, grid, block, 0, s, (const _Float16*)y, slot_pair, weights, ne, n_used,
-                    weight_before, dst, identity, pair_scale);
+                    weight_before, dst, identity, pair_scale, addend);
     else
         INFR_LAUNCH(unbucket_combine_kernel<float>, grid, block, 0, s, (const float*)y, slot_pair, weights, ne, n_used,
-                    weight_before, dst, identity, pair_scale);
+                    weight_before, dst, identity, pair_scale, addend);
 }
 
 }  // namespace infr

@@ -72,6 +72,46 @@ void launch_add(hipStream_t s, const float* a, const float* b, float* dst, uint3
     INFR_LAUNCH(add_kernel, dim3(blocks), dim3(256), 0, s, a, b, dst, n);
 }
 
+// Op::RmsNorm / Op::RmsNormAdd (crates/infr-cpu/src/lib.rs:1046-1093), one block per row.  The
+// reference sums the squares left to right; here each thread sums its share and the shares are
+// added in a fixed tree, which moves the result by a few units in the last place.  dst may be x:
+// every thread has read the whole row before the first element is written.
+__global__ __launch_bounds__(256) void rms_norm_kernel(const float* x, const float* __restrict__ w, float* dst, int dim,
+                                                       float eps, int add, int vec) {
+    __shared__ float red[4];
+    const float* xr = x + (size_t)blockIdx.x * dim;
+    float* d = dst + (size_t)blockIdx.x * dim;
+    const int tid = threadIdx.x;
+    float part = 0.0f;
+    if (vec) {
+        for (int v = tid; v < (dim >> 2); v += 256) part = sumsq4(part, reinterpret_cast<const float4*>(xr)[v]);
+    } else {
+        for (int k = tid; k < dim; k += 256) part = __fmaf_rn(xr[k], xr[k], part);
+    }
+    const float s = rms_scale(block256_sum(part, red), dim, eps);
+    if (vec) {
+        for (int v = tid; v < (dim >> 2); v += 256) {
+            float4 t = rms_apply4(reinterpret_cast<const float4*>(xr)[v], s, reinterpret_cast<const float4*>(w)[v]);
+            if (add) {
+                const float4 o = reinterpret_cast<const float4*>(d)[v];
+                t = make_float4(__fadd_rn(o.x, t.x), __fadd_rn(o.y, t.y), __fadd_rn(o.z, t.z), __fadd_rn(o.w, t.w));
+            }
+            reinterpret_cast<float4*>(d)[v] = t;
+        }
+    } else {
+        for (int k = tid; k < dim; k += 256) {
+            const float t = __fmul_rn(__fmul_rn(xr[k], s), w[k]);
+            d[k] = add ? __fadd_rn(d[k], t) : t;
+        }
+    }
+}
+
+void launch_rms_norm(hipStream_t s, const float* x, const float* weight, float* dst, int rows, int dim, float eps, int add) {
+    if (rows <= 0 || dim <= 0) return;
+    const int vec = (dim & 3) == 0 && (((uintptr_t)x | (uintptr_t)weight | (uintptr_t)dst) & 15) == 0;
+    INFR_LAUNCH(rms_norm_kernel, dim3(rows), dim3(256), 0, s, x, weight, dst, dim, eps, add, vec);
+}
+
 __global__ __launch_bounds__(256) void mask_dropped_pairs_kernel(const int32_t* __restrict__ ids, const float* __restrict__ w,
                                                                  int n, int32_t* __restrict__ out) {
     const int i = blockIdx.x * 256 + threadIdx.x;

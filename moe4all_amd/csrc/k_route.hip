@@ -42,8 +42,9 @@ template <int EPB>
 __global__ __launch_bounds__(256) void router_logits_kernel(const uint8_t* __restrict__ router, int rdt,
                                                             size_t row_bytes, const float* __restrict__ x, int ne,
                                                             int n_expert, int rows, int rpb,
-                                                            float* __restrict__ logits) {
+                                                            float* __restrict__ logits, RouterNorm nrm) {
     extern __shared__ float lds[];
+    __shared__ float red[4];
     const int nc = ne >> 3;                 // full chunks of 8
     const int ntail = ne & 7;
     const int jstride = ((nc + 63) & ~63) + 4;
@@ -63,12 +64,20 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const uint8_t* __res
     const bool one_shot = rdt == INFR_F32 && (ne & 3) == 0 && (int)gridDim.y * rpb >= rows && EPB * nv <= 8 * 256 &&
                           rpb * nv <= 4 * 256;
     if (one_shot) {
-        float4 wr[8], xr[4];
+        float4 wr[8], xr[4], nw[4];
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const int idx = tid + 256 * i, rr = idx / nv, v = idx - rr * nv;
             xr[i] = make_float4(0.f, 0.f, 0.f, 0.f);
             if (rr < rpb && rbase + rr < rows) xr[i] = reinterpret_cast<const float4*>(x + (size_t)(rbase + rr) * ne)[v];
+        }
+        if (nrm.weight) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int idx = tid + 256 * i;
+                nw[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (idx < nv) nw[i] = reinterpret_cast<const float4*>(nrm.weight)[idx];
+            }
         }
 #pragma unroll
         for (int i = 0; i < 8; i++) {
@@ -76,6 +85,22 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const uint8_t* __res
             wr[i] = make_float4(0.f, 0.f, 0.f, 0.f);
             if (e < EPB && e0 + e < n_expert)
                 wr[i] = reinterpret_cast<const float4*>(router + (size_t)(e0 + e) * row_bytes)[v];
+        }
+        if (nrm.weight) {
+            // The single token row arrives raw: Op::RmsNorm is applied while it is staged, with the
+            // summation tree of the standalone kernel, and the first block stores the normalised row.
+            float part = 0.0f;
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+                if (tid + 256 * i < nv) part = sumsq4(part, xr[i]);
+            const float sc = rms_scale(block256_sum(part, red), ne, nrm.eps);
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int idx = tid + 256 * i;
+                if (idx >= nv) continue;
+                xr[i] = rms_apply4(xr[i], sc, nw[i]);
+                if (blockIdx.x == 0 && blockIdx.y == 0) reinterpret_cast<float4*>(nrm.xn_out)[idx] = xr[i];
+            }
         }
 #pragma unroll
         for (int i = 0; i < 4; i++) {
@@ -257,8 +282,17 @@ __global__ __launch_bounds__(512) void router_logits_tiled_kernel(const float* _
         }
 }
 
+// The fold needs the one-burst staging of a single row (rows = 1 gives 2 experts x 1 row per block).
+bool router_logits_can_norm(int rdt, size_t row_bytes, int ne, int rows) {
+    return rows == 1 && rdt == INFR_F32 && (ne & 3) == 0 && ne >= 4 && ne <= 4096 && (row_bytes & 15) == 0;
+}
+
 bool launch_router_logits(hipStream_t s, const uint8_t* router, int rdt, size_t row_bytes, const float* x, int ne,
-                          int n_expert, int rows, float* logits) {
+                          int n_expert, int rows, float* logits, const RouterNorm* norm) {
+    const RouterNorm nrm = norm ? *norm : RouterNorm{};
+    if (nrm.weight && (!router_logits_can_norm(rdt, row_bytes, ne, rows) || !nrm.xn_out || nrm.xn_out == x ||
+                       (((uintptr_t)x | (uintptr_t)nrm.weight | (uintptr_t)nrm.xn_out) & 15) != 0))
+        return false;
     if (rows >= 32 && rdt == INFR_F32 && (ne & 31) == 0 && (row_bytes & 15) == 0) {
         dim3 grid((n_expert + kLtTile - 1) / kLtTile, (rows + kLtTile - 1) / kLtTile);
         INFR_LAUNCH(router_logits_tiled_kernel, grid, dim3(512), 0, s, reinterpret_cast<const float*>(router), row_bytes / 4,
@@ -294,7 +328,7 @@ bool launch_router_logits(hipStream_t s, const uint8_t* router, int rdt, size_t 
             attr_set = true;                                                                                       \
         }                                                                                                          \
         INFR_LAUNCH(router_logits_kernel<E>, grid, block, lds, s, router, rdt, row_bytes, x, ne, n_expert,  \
-                           rows, rpb, logits);                                                        \
+                           rows, rpb, logits, nrm);                                                   \
     } while (0)
     switch (epb) {
         case 8: LAUNCH_RL(8); break;

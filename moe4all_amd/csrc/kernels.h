@@ -25,11 +25,19 @@ extern thread_local const LaunchTiming* tl_launch_timing;
         else hipLaunchKernelGGL(kernel, grid, block, lds, stream, __VA_ARGS__);                                  \
     } while (0)
 
+// An Op::RmsNorm of the single token row folded into the logits kernel: x is the raw row, every
+// block normalises it while staging and the first block also stores the normalised row to xn_out.
+struct RouterNorm {
+    const float* weight = nullptr;   // [ne]
+    float eps = 0.0f;
+    float* xn_out = nullptr;         // [ne], not x
+};
+bool router_logits_can_norm(int rdt, size_t row_bytes, int ne, int rows);
 // Router logits with the reference's dot order (8 FMA lanes, lanes summed 0..7).
 // logits[rows, n_expert]; router rows are `row_bytes` apart, decoded as `rdt`.
-// Returns false when the shape does not fit the kernel's LDS budget.
+// Returns false when the shape does not fit the kernel's LDS budget (or the fold of `norm`).
 bool launch_router_logits(hipStream_t s, const uint8_t* router, int rdt, size_t row_bytes, const float* x,
-                          int ne, int n_expert, int rows, float* logits);
+                          int ne, int n_expert, int rows, float* logits, const RouterNorm* norm = nullptr);
 
 struct RouteParams {
     const float* logits;      // [rows, n_expert]
@@ -122,7 +130,8 @@ void launch_grouped_down(hipStream_t s, int dt, const GroupedParams& p);
 // identity != 0: y is in flat (row, rank) order and slot_pair only flags invalid pairs (< 0).
 void launch_unbucket_combine(hipStream_t s, const void* y, const int32_t* slot_pair, const float* weights, int rows,
                              int ne, int n_used, int weight_before, float* dst, int identity = 0,
-                             const float* pair_scale = nullptr);   // pair_scale != null: y is f16, y[pair] * pair_scale[pair]
+                             const float* pair_scale = nullptr,   // != null: y is f16, y[pair] * pair_scale[pair]
+                             const float* addend = nullptr);      // != null: dst = addend + sum ([rows, ne], may be dst)
 
 // Decode batches with weight reuse: one block per (feature tile, expert) walks the expert's bucket,
 // so an expert's rows are read from HBM once however many token rows selected it.  h and y are in
@@ -144,6 +153,8 @@ void launch_linear(hipStream_t s, const float* x, const uint8_t* w, int dt, size
 void launch_gated_act(hipStream_t s, const float* gate, const float* up, float* dst, int rows, int nff, int act,
                       int up_off, int up_stride, int gate_stride, int gate_block_width, int has_clamp, float clamp);
 void launch_add(hipStream_t s, const float* a, const float* b, float* dst, uint32_t n);
+// Op::RmsNorm (add = 0) / Op::RmsNormAdd (add = 1); dst may be x.
+void launch_rms_norm(hipStream_t s, const float* x, const float* weight, float* dst, int rows, int dim, float eps, int add);
 // Op::Copy / Op::CopyStrided on elements of `elem_bytes` (2 or 4): row r copies n elements from
 // src + r * src_stride to dst + r * dst_stride (pointers already at the ops' offsets).
 void launch_copy_rows(hipStream_t s, const void* src, void* dst, uint32_t rows, uint32_t n, uint32_t src_stride,

@@ -98,6 +98,8 @@ def lib() -> C.CDLL:
         L.orc_moe_shared_expert_add.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int, C.c_int,
                                                 C.c_void_p]
         L.orc_moe_shared_expert_add.restype = None
+        L.orc_rms_norm.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_float, C.c_int, C.c_void_p]
+        L.orc_rms_norm.restype = None
         L.orc_hw_threads.restype = C.c_int
         _lib = L
     return _lib
@@ -277,6 +279,16 @@ def moe_shared_expert_add(moe, shexp, gate) -> np.ndarray:
     rows = g.size
     dst = np.empty_like(m)
     lib().orc_moe_shared_expert_add(_p(m), _p(s), _p(g), rows, m.size // rows, _p(dst))
+    return dst
+
+
+def rms_norm(x, weight, eps, add_to=None) -> np.ndarray:
+    """Op::RmsNorm; with add_to, Op::RmsNormAdd applied to a copy of add_to."""
+    x, w = _f32(x), _f32(weight).reshape(-1)
+    dim = w.size
+    rows = x.size // dim
+    dst = np.empty_like(x) if add_to is None else _f32(add_to).copy()
+    lib().orc_rms_norm(_p(x), _p(w), rows, dim, eps, add_to is not None, _p(dst))
     return dst
 
 

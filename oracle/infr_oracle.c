@@ -675,3 +675,25 @@ void orc_moe_shared_expert_add(const float *moe, const float *shexp, const float
         }
     }
 }
+
+/* Op::RmsNorm / Op::RmsNormAdd (crates/infr-cpu/src/lib.rs:1046-1093): per row the squares are
+ * summed left to right in f32 (multiply, then add: rustc never contracts), divided by dim,
+ * s = 1 / sqrt(ss + eps), and each element is (x * s) * w; the Add form accumulates into dst. */
+void orc_rms_norm(const float *x, const float *w, int rows, int dim, float eps, int add, float *dst) {
+    for (int r = 0; r < rows; r++) {
+        const float *xr = x + (size_t)r * dim;
+        float *d = dst + (size_t)r * dim;
+        float ss = 0.0f;
+        for (int i = 0; i < dim; i++) {
+            float sq = xr[i] * xr[i];
+            ss = ss + sq;
+        }
+        ss = ss / (float)dim;
+        float s = 1.0f / sqrtf(ss + eps);
+        for (int i = 0; i < dim; i++) {
+            float t = xr[i] * s;
+            t = t * w[i];
+            d[i] = add ? d[i] + t : t;
+        }
+    }
+}

@@ -117,6 +117,9 @@ void orc_add(const float *a, const float *b, int64_t n, float *dst);
 void orc_moe_shared_expert_add(const float *moe, const float *shexp, const float *gate,
                                int rows, int n, float *dst);
 
+/* Op::RmsNorm (add = 0) and Op::RmsNormAdd (add = 1: dst += ...), crates/infr-cpu/src/lib.rs:1046-1093. */
+void orc_rms_norm(const float *x, const float *w, int rows, int dim, float eps, int add, float *dst);
+
 /* Number of hardware threads the pool would use. */
 int orc_hw_threads(void);
 

@@ -551,6 +551,147 @@ def test_shared_expert_as_an_extra_slot_gives_the_bits_of_the_separate_ops(be, r
     assert H.rel_l2(fused.reshape(rows, ne), want.reshape(rows, ne)) < REL_L2
 
 
+@pytest.mark.parametrize("rows,dim,add,inplace", [(1, 2048, False, False), (5, 100, False, False), (3, 8192, True, False),
+                                                  (2, 4096, False, True), (1, 6, True, False), (0, 64, False, False)])
+def test_rms_norm_and_rms_norm_add_match_the_oracle(be, rows, dim, add, inplace):
+    """Op::RmsNorm / Op::RmsNormAdd (crates/infr-cpu/src/lib.rs:1046-1093): dims with and without
+    a 16-byte row pitch, several passes per thread, in place, and an empty batch."""
+    rng = np.random.default_rng(rows * 131 + dim)
+    x = (rng.standard_normal((rows, dim)) * 3).astype(np.float32)
+    w = (1 + 0.2 * rng.standard_normal(dim)).astype(np.float32)
+    y0 = rng.standard_normal((rows, dim)).astype(np.float32)
+    eps = 1e-6
+    g = M.Graph()
+    wt = g.weight(TensorDesc([dim], DType.F32))
+    if inplace:
+        xi = yi = g.output(TensorDesc([rows, dim], DType.F32))
+    else:
+        xi = g.input(TensorDesc([rows, dim], DType.F32))
+        yi = g.output(TensorDesc([rows, dim], DType.F32))
+    g.rms_norm(x=xi, weight=wt, dst=yi, rows=rows, dim=dim, eps=eps, add=add)
+    bound = [(wt, w), (yi, x if inplace else y0)] + ([] if inplace else [(xi, x)])
+    got = M.run_graph(be, g, bound, yi, rows * dim).reshape(rows, dim)
+    want = O.rms_norm(x, w, eps, add_to=y0 if add else None).reshape(rows, dim)
+    if rows:
+        assert H.max_abs(got, want) < 2e-5 * max(1.0, float(np.abs(want).max()))
+        assert H.rel_l2(got, want) < 1e-6
+
+
+@pytest.mark.parametrize("rows,shared", [(1, False), (1, True), (3, False), (20, False), (40, False)])
+def test_norm_moe_residual_chain_folds_into_the_moe_kernels(be, rows, shared):
+    """RmsNorm -> MoeFfn [-> shared expert -> Add] -> Add(residual), the FFN sublayer the model emits
+    (crates/infr-llama/src/seam/runner.rs:8037-8174).  On one token row the norm rides in the logits
+    kernel (crates/infr-core/src/fusion.rs:15-19) and on every path the residual Add rides in the combine
+    (fusion.rs:20-24); the folded chain must give the bits of the ops run one graph at a time."""
+    ne, nff, E, K = 1024, 512, 16, 4
+    rng = np.random.default_rng(700 + rows)
+    x = (rng.standard_normal((rows, ne)) * 2).astype(np.float32)
+    nw = (1 + 0.1 * rng.standard_normal(ne)).astype(np.float32)
+    router = (rng.standard_normal((E, ne)) * 0.1).astype(np.float32)
+    eg, eu = _realistic(rng, E, nff, ne, H.Q4K), _realistic(rng, E, nff, ne, H.Q4K)
+    ed = _realistic(rng, E, ne, nff, H.Q6K)
+    wg, wu = _realistic(rng, 1, nff, ne, H.Q4K), _realistic(rng, 1, nff, ne, H.Q4K)
+    wd = _realistic(rng, 1, ne, nff, H.Q6K)
+    eps = 1e-6
+
+    def graph(folded, xn_given=None):
+        """folded: the whole chain in one graph with single-use Internal temporaries.  Otherwise the norm
+        has already run (xn_given) and the routed sum is an Output, so nothing folds."""
+        g = M.Graph()
+        xi = g.input(TensorDesc([rows, ne], DType.F32))
+        nwt = g.weight(TensorDesc([ne], DType.F32))
+        rt = g.weight(TensorDesc([E, ne], DType.F32))
+        egt, eut = g.weight(TensorDesc([E, nff, ne], DType.Q4K)), g.weight(TensorDesc([E, nff, ne], DType.Q4K))
+        edt = g.weight(TensorDesc([E, ne, nff], DType.Q6K))
+        pairs = [(xi, x), (rt, router), (egt, eg), (eut, eu), (edt, ed)]
+        if folded:
+            xn = g.internal(TensorDesc([rows, ne], DType.F32))
+            g.rms_norm(x=xi, weight=nwt, dst=xn, rows=rows, dim=ne, eps=eps)
+            pairs.append((nwt, nw))
+        else:
+            xn = g.input(TensorDesc([rows, ne], DType.F32))
+            pairs.append((xn, xn_given))
+        extra_out = []
+        moe = g.internal(TensorDesc([rows, ne], DType.F32)) if folded else g.output(TensorDesc([rows, ne], DType.F32))
+        if not folded:
+            extra_out.append(moe)
+        g.moe_ffn(x=xn, router=rt, gate_exps=egt, up_exps=eut, down_exps=edt, dst=moe, ne=ne, n_expert=E, n_used=K,
+                  n_ff_exp=nff)
+        sub = moe
+        if shared:
+            wgt, wut = g.weight(TensorDesc([nff, ne], DType.Q4K)), g.weight(TensorDesc([nff, ne], DType.Q4K))
+            wdt = g.weight(TensorDesc([ne, nff], DType.Q6K))
+            gt, ut = g.internal(TensorDesc([rows, nff], DType.F32)), g.internal(TensorDesc([rows, nff], DType.F32))
+            at, st = g.internal(TensorDesc([rows, nff], DType.F32)), g.internal(TensorDesc([rows, ne], DType.F32))
+            sub = g.internal(TensorDesc([rows, ne], DType.F32)) if folded else g.output(TensorDesc([rows, ne], DType.F32))
+            if not folded:
+                extra_out.append(sub)
+            g.linear(x=xn, weight=wgt, dst=gt, m=rows, in_f=ne, out_f=nff)
+            g.linear(x=xn, weight=wut, dst=ut, m=rows, in_f=ne, out_f=nff)
+            g.gated_act(gate=gt, up=ut, dst=at, rows=rows, nff=nff)
+            g.linear(x=at, weight=wdt, dst=st, m=rows, in_f=nff, out_f=ne)
+            g.add(a=moe, b=st, dst=sub, n=rows * ne)
+            pairs += [(wgt, wg), (wut, wu), (wdt, wd)]
+        yi = g.output(TensorDesc([rows, ne], DType.F32))
+        g.add(a=xi, b=sub, dst=yi, n=rows * ne)
+        return g, pairs, extra_out, yi
+
+    def run(folded, xn_given=None):
+        g, pairs, extra_out, yi = graph(folded, xn_given)
+        plan = be.compile(g)
+        bufs, b = [], M.Bindings()
+        for tid, v in pairs:
+            bufs.append(be.buffer_from(v))
+            b.bind(tid, bufs[-1])
+        for tid in extra_out + [yi]:
+            bufs.append(be.alloc(rows * ne * 4))
+            b.bind(tid, bufs[-1])
+        be.prof_enable(True)
+        be.execute(plan, b)
+        out = be.download(bufs[-1], rows * ne * 4, np.float32)
+        names = set(be.prof_read())
+        be.prof_enable(False)
+        moe_op = 1 if folded else 0
+        routing = be.moe_routing(plan, moe_op)
+        for buf in bufs:
+            buf.free()
+        plan.free()
+        return out, names, routing
+
+    # the norm on its own
+    g0 = M.Graph()
+    x0, w0 = g0.input(TensorDesc([rows, ne], DType.F32)), g0.weight(TensorDesc([ne], DType.F32))
+    y0 = g0.output(TensorDesc([rows, ne], DType.F32))
+    g0.rms_norm(x=x0, weight=w0, dst=y0, rows=rows, dim=ne, eps=eps)
+    xn_dev = M.run_graph(be, g0, [(x0, x), (w0, nw)], y0, rows * ne).reshape(rows, ne)
+
+    folded, fnames, r1 = run(True)
+    plain, pnames, r2 = run(False, xn_dev)
+    assert "add" not in fnames and "add" in pnames
+    if rows == 1:
+        assert "rms_norm_router_logits" in fnames and "rms_norm" not in fnames and "router_logits" not in fnames
+        if shared:
+            assert {"moe_route_gate_up_shared", "moe_down_combine_shared"} <= fnames and "linear_add" not in fnames
+    else:
+        assert "rms_norm" in fnames and "router_logits" in fnames
+    assert np.array_equal(r1["idx"], r2["idx"]) and np.array_equal(bits(r1["w"]), bits(r2["w"]))
+    assert np.array_equal(bits(folded), bits(plain))
+
+    # against the oracle, routed from the device's normalised rows so that a last-place difference
+    # of the norm cannot flip a near-tie of the selection
+    assert H.rel_l2(xn_dev, O.rms_norm(x, nw, eps).reshape(rows, ne)) < 1e-6
+    want = O.moe_ffn(xn_dev, router, eg, eu, ed, ne=ne, n_expert=E, n_used=K, n_ff_exp=nff, gate_dtype=H.Q4K,
+                     down_dtype=H.Q6K)
+    assert np.array_equal(r1["idx"], want["idx"])
+    sub = want["dst"]
+    if shared:
+        og, ou = O.linear(xn_dev, wg, H.Q4K, ne, nff), O.linear(xn_dev, wu, H.Q4K, ne, nff)
+        sub = O.add(sub, O.linear(O.gated_act_rows(og, ou), wd, H.Q6K, nff, ne))
+    want_y = O.add(x, sub).reshape(rows, ne)
+    tol = 1e-2 if rows >= 32 else REL_L2
+    assert H.rel_l2(folded.reshape(rows, ne) - x, want_y - x) < tol
+
+
 # ------------------------------------------------------------------ synthetic workloads at full size
 from moe4all_amd import synth as S  # noqa: E402
 

@@ -390,3 +390,34 @@ def test_elementwise_neighbours():
     got = O.moe_shared_expert_add(a, b, gate)
     want = a + (1 / (1 + np.exp(-gate.astype(np.float64))))[:, None] * b
     assert np.allclose(got, want, rtol=1e-6, atol=1e-7)
+
+
+def test_rms_norm_closed_forms_and_f64():
+    """Op::RmsNorm (crates/infr-cpu/src/lib.rs:1046-1069).  Pinned by what the definition fixes: a
+    constant row of c with unit weight gives c / sqrt(c^2 + eps) in every column; with eps = 0 the
+    mean square of out / weight is 1; rows do not mix; the weight multiplies per column; and the whole
+    thing agrees with an f64 evaluation.  The Add form accumulates onto dst (lib.rs:1070-1093)."""
+    dim = 96
+    c = np.float32(3.0)
+    out = O.rms_norm(np.full((2, dim), c, np.float32), np.ones(dim, np.float32), 1e-2)
+    assert np.allclose(out, c / np.sqrt(np.float64(c) ** 2 + 1e-2), rtol=2e-7, atol=0)
+    rng = np.random.default_rng(5)
+    x = (rng.standard_normal((4, dim)) * 5).astype(np.float32)
+    w = (1 + 0.3 * rng.standard_normal(dim)).astype(np.float32)
+    out = O.rms_norm(x, w, 0.0)
+    assert np.allclose(np.mean((out.astype(np.float64) / w) ** 2, axis=1), 1.0, rtol=1e-5)
+    x64 = x.astype(np.float64)
+    eps = 1e-5
+    want = x64 / np.sqrt(np.mean(x64 * x64, axis=1, keepdims=True) + eps) * w
+    got = O.rms_norm(x, w, eps)
+    assert H.rel_l2(got, want) < 2e-7
+    # rows are independent: a row alone gives the bits it gives inside the batch
+    assert np.array_equal(O.rms_norm(x[2:3], w, eps).view(np.uint32), got[2:3].view(np.uint32))
+    # a column's weight reaches that column only
+    w2 = w.copy()
+    w2[7] *= 2
+    got2 = O.rms_norm(x, w2, eps)
+    assert np.array_equal(np.delete(got2, 7, axis=1), np.delete(got, 7, axis=1)) and np.allclose(got2[:, 7], 2 * got[:, 7])
+    base = rng.standard_normal((4, dim)).astype(np.float32)
+    assert np.array_equal(O.rms_norm(x, w, eps, add_to=base), base + got)
+    assert O.rms_norm(np.zeros((0, dim), np.float32), w, eps).shape == (0, dim)
