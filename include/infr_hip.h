@@ -34,7 +34,9 @@ typedef enum infr_status {
     INFR_ERR_BACKEND = 1,     /* Error::Backend: HIP failure, bad binding, size mismatch */
     INFR_ERR_UNSUPPORTED = 2, /* Error::Unsupported: op / dtype / option not implemented */
     INFR_ERR_ABORTED = 3,     /* Error::Aborted: shutdown latch set */
-    INFR_ERR_INVALID = 4      /* null / foreign handle, malformed graph */
+    INFR_ERR_INVALID = 4,     /* null / foreign handle, malformed graph */
+    INFR_ERR_LOADER = 5,      /* Error::Loader: malformed or inconsistent weight file */
+    INFR_ERR_IO = 6           /* Error::Io: the file could not be opened or mapped */
 } infr_status;
 
 /* infr_core::DType, same ordinal order (crates/infr-core/src/tensor.rs:7-57). */
