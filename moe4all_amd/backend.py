@@ -79,7 +79,8 @@ class MoeGating(enum.IntEnum):
 
 
 _BLOCK = {DType.F32: (1, 4), DType.I32: (1, 4), DType.U32: (1, 4), DType.F16: (1, 2), DType.Bf16: (1, 2),
-          DType.Q8_0: (32, 34), DType.Q4K: (256, 144), DType.Q6K: (256, 210)}
+          DType.Q8_0: (32, 34), DType.Q4K: (256, 144), DType.Q6K: (256, 210), DType.Q4_0: (32, 18), DType.Q4_1: (32, 20),
+          DType.Q5_0: (32, 22), DType.Q5_1: (32, 24), DType.Q2K: (256, 84), DType.Q3K: (256, 110), DType.Q5K: (256, 176)}
 
 
 def bytes_for(dtype: DType, numel: int) -> int:

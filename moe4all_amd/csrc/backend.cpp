@@ -53,8 +53,15 @@ bool geometry(int dtype, int* elems, int* bytes) {
     switch (dtype) {
         case INFR_F32: case INFR_I32: case INFR_U32: *elems = 1; *bytes = 4; return true;
         case INFR_F16: case INFR_BF16: *elems = 1; *bytes = 2; return true;
+        case INFR_Q4_0: *elems = 32; *bytes = 18; return true;
+        case INFR_Q4_1: *elems = 32; *bytes = 20; return true;
+        case INFR_Q5_0: *elems = 32; *bytes = 22; return true;
+        case INFR_Q5_1: *elems = 32; *bytes = 24; return true;
         case INFR_Q8_0: *elems = 32; *bytes = 34; return true;
+        case INFR_Q2K: *elems = 256; *bytes = 84; return true;
+        case INFR_Q3K: *elems = 256; *bytes = 110; return true;
         case INFR_Q4K: *elems = 256; *bytes = 144; return true;
+        case INFR_Q5K: *elems = 256; *bytes = 176; return true;
         case INFR_Q6K: *elems = 256; *bytes = 210; return true;
         default: return false;
     }
@@ -428,7 +435,7 @@ struct Check {
         int be = 0, bb = 0;
         if (!geometry(dt(id), &be, &bb) || dt(id) == INFR_I32 || dt(id) == INFR_U32) {
             set(INFR_ERR_UNSUPPORTED, std::string(role) + ": weight dtype " + dtype_name(dt(id)) +
-                                          " has no decode on this backend (F32/F16/Bf16/Q8_0/Q4K/Q6K)");
+                                          " has no decode on this backend (F32/F16/Bf16 and the affine quants Q4_0..Q8_0, Q2K..Q6K)");
             return;
         }
         if (in_f % (uint64_t)be != 0)

@@ -105,8 +105,15 @@ __host__ __device__ inline bool block_geometry(int dtype, int* elems, int* bytes
     switch (dtype) {
         case INFR_F32: case INFR_I32: case INFR_U32: *elems = 1; *bytes = 4; return true;
         case INFR_F16: case INFR_BF16: *elems = 1; *bytes = 2; return true;
+        case INFR_Q4_0: *elems = 32; *bytes = 18; return true;
+        case INFR_Q4_1: *elems = 32; *bytes = 20; return true;
+        case INFR_Q5_0: *elems = 32; *bytes = 22; return true;
+        case INFR_Q5_1: *elems = 32; *bytes = 24; return true;
         case INFR_Q8_0: *elems = 32; *bytes = 34; return true;
+        case INFR_Q2K: *elems = 256; *bytes = 84; return true;
+        case INFR_Q3K: *elems = 256; *bytes = 110; return true;
         case INFR_Q4K: *elems = 256; *bytes = 144; return true;
+        case INFR_Q5K: *elems = 256; *bytes = 176; return true;
         case INFR_Q6K: *elems = 256; *bytes = 210; return true;
         default: return false;
     }
@@ -154,6 +161,65 @@ __device__ inline float decode_elem(int dtype, const uint8_t* row, uint32_t k) {
             uint32_t code = hi ? (uint32_t)(v >> 4) : (uint32_t)(v & 0xF);
             float scf = __fmul_rn(d, (float)(int)sc);
             float mn = __fmul_rn(dmin, (float)(-(int)m));
+            return __fadd_rn(__fmul_rn(scf, (float)code), mn);
+        }
+        case INFR_Q4_0: case INFR_Q4_1: case INFR_Q5_0: case INFR_Q5_1: {
+            // 32-element blocks [f16 d][f16 m?][u32 qh?][16 nibble bytes] (dequant.rs:137-209): element j < 16 is
+            // the low nibble of byte j, element j + 16 the high nibble; the fifth bit of element e is bit e of qh
+            const bool has_m = dtype == INFR_Q4_1 || dtype == INFR_Q5_1, five = dtype == INFR_Q5_0 || dtype == INFR_Q5_1;
+            const uint32_t bb = 18u + (has_m ? 2u : 0u) + (five ? 4u : 0u);
+            const uint8_t* blk = row + (size_t)(k >> 5) * bb;
+            const uint32_t e = k & 31u, j = e & 15u;
+            const uint8_t* p = blk + 2 + (has_m ? 2 : 0);
+            uint32_t code = 0;
+            if (five) {
+                code = ((ldu<uint32_t>(p) >> e) & 1u) << 4;
+                p += 4;
+            }
+            code |= e < 16 ? (uint32_t)(p[j] & 0xF) : (uint32_t)(p[j] >> 4);
+            const float d = f16_bits_to_f32(ldu<uint16_t>(blk));
+            const float mn = has_m ? __fmul_rn(f16_bits_to_f32(ldu<uint16_t>(blk + 2)), 1.0f)
+                                   : __fmul_rn(d, five ? -16.0f : -8.0f);
+            return __fadd_rn(__fmul_rn(__fmul_rn(d, 1.0f), (float)code), mn);
+        }
+        case INFR_Q2K: {
+            // [16 scale bytes][64 qs][f16 d][f16 dmin] (dequant.rs:224-250): 16-element group g = w / 16 reads the
+            // 2-bit field at shift 2 * ((g % 8) / 2) of qs[32 * (g / 8) + 16 * (g % 2) + l]
+            const uint8_t* blk = row + (size_t)(k >> 8) * 84u;
+            const uint32_t w = k & 255u, g = w >> 4, l = w & 15u;
+            const uint32_t sc = blk[g];
+            const uint32_t code = ((uint32_t)blk[16 + 32 * (g >> 3) + 16 * (g & 1u) + l] >> (2u * ((g & 7u) >> 1))) & 3u;
+            const float scf = __fmul_rn(f16_bits_to_f32(ldu<uint16_t>(blk + 80)), (float)(sc & 0xFu));
+            const float mn = __fmul_rn(f16_bits_to_f32(ldu<uint16_t>(blk + 82)), (float)(-(int)(sc >> 4)));   // integer negation: -0 does not exist
+            return __fadd_rn(__fmul_rn(scf, (float)code), mn);
+        }
+        case INFR_Q3K: {
+            // [32 hmask][64 qs][12 scale bytes][f16 d] (dequant.rs:251-312).  6-bit scale g: low 4 bits = nibble
+            // (g / 8) of scale byte g % 8, high 2 bits = field (g / 4) of scale byte 8 + g % 4; value - 32.
+            // Code = 2 bits from qs as in Q2_K + bit (g / 2) of hmask[16 * (g % 2) + l] as bit 2; min = -4 * scale.
+            const uint8_t* blk = row + (size_t)(k >> 8) * 110u;
+            const uint32_t w = k & 255u, g = w >> 4, l = w & 15u;
+            const uint32_t lo = ((uint32_t)blk[96 + (g & 7u)] >> (g >= 8u ? 4u : 0u)) & 0xFu;
+            const uint32_t hi = ((uint32_t)blk[104 + (g & 3u)] >> (2u * (g >> 2))) & 3u;
+            const int s = (int)(lo | (hi << 4)) - 32;
+            const uint32_t low2 = ((uint32_t)blk[32 + 32 * (g >> 3) + 16 * (g & 1u) + l] >> (2u * ((g & 7u) >> 1))) & 3u;
+            const uint32_t high = ((uint32_t)blk[16 * (g & 1u) + l] >> (g >> 1)) & 1u;
+            const float d = f16_bits_to_f32(ldu<uint16_t>(blk + 108));
+            const float scf = __fmul_rn(d, (float)s);
+            const float mn = __fmul_rn(d, (float)(-4 * s));
+            return __fadd_rn(__fmul_rn(scf, (float)(low2 | (high << 2))), mn);
+        }
+        case INFR_Q5K: {
+            // Q4_K with 32 bytes of fifth bits after the scales (dequant.rs:336-363): bit (2j + hi) of qh[l]
+            const uint8_t* blk = row + (size_t)(k >> 8) * 176u;
+            const uint32_t w = k & 255u;
+            const uint32_t j = w >> 6, hi = (w >> 5) & 1u, l = w & 31u;
+            uint32_t sc, m;
+            k4((int)(2 * j + hi), blk + 4, sc, m);
+            const uint8_t v = blk[48 + j * 32 + l];
+            const uint32_t code = (hi ? (uint32_t)(v >> 4) : (uint32_t)(v & 0xF)) + ((((uint32_t)blk[16 + l] >> (2 * j + hi)) & 1u) << 4);
+            const float scf = __fmul_rn(f16_bits_to_f32(ldu<uint16_t>(blk)), (float)(int)sc);
+            const float mn = __fmul_rn(f16_bits_to_f32(ldu<uint16_t>(blk + 2)), (float)(-(int)m));
             return __fadd_rn(__fmul_rn(scf, (float)code), mn);
         }
         case INFR_Q6K: {

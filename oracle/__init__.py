@@ -17,7 +17,7 @@ _LIB_PATH = os.path.join(_HERE, "libinfr_oracle.so")
 
 # infr_core::DType ordinals (crates/infr-core/src/tensor.rs:7-57)
 F32, F16, BF16, I32, U32 = 0, 1, 2, 3, 4
-Q8_0, Q4K, Q6K = 9, 12, 14
+Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q2K, Q3K, Q4K, Q5K, Q6K = 5, 6, 7, 8, 9, 10, 11, 12, 13, 14
 ACT_SILU, ACT_GELU, ACT_SIGMOID = 0, 1, 2
 GATE_SOFTMAX, GATE_SIGMOID, GATE_SQRT_SOFTPLUS = 0, 1, 2
 

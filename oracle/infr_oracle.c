@@ -50,8 +50,15 @@ int orc_block_geometry(int dtype, int *block_elems, int *block_bytes) {
     switch (dtype) {
     case ORC_F32: case ORC_I32: case ORC_U32: e = 1; b = 4; break;
     case ORC_F16: case ORC_BF16: e = 1; b = 2; break;
+    case ORC_Q4_0: e = 32; b = 18; break;
+    case ORC_Q4_1: e = 32; b = 20; break;
+    case ORC_Q5_0: e = 32; b = 22; break;
+    case ORC_Q5_1: e = 32; b = 24; break;
     case ORC_Q8_0: e = 32; b = 34; break;
+    case ORC_Q2K: e = 256; b = 84; break;
+    case ORC_Q3K: e = 256; b = 110; break;
     case ORC_Q4K: e = 256; b = 144; break;
+    case ORC_Q5K: e = 256; b = 176; break;
     case ORC_Q6K: e = 256; b = 210; break;
     default: return -1;
     }
@@ -167,6 +174,100 @@ static void factor_q6k(const uint8_t *blk, factored_block *f) {
     }
 }
 
+static uint32_t rd_u32(const uint8_t *p) {
+    return (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16) | ((uint32_t)p[3] << 24);
+}
+
+/* The four legacy 32-element formats (dequant.rs:137-209): `nib` low nibbles are elements 0..15,
+ * high nibbles 16..31; the 5-bit forms take bit j of qh for element j and bit j+16 for j+16
+ * (written there as ((qh >> j) << 4) & 0x10 and (qh >> (j + 12)) & 0x10). */
+static void factor_legacy(const uint8_t *blk, int has_min, int has_high, factored_block *f) {
+    const uint8_t *p = blk + 2;
+    f->dd[0] = rd_u16(blk);
+    if (has_min) { f->dd[1] = rd_u16(p); p += 2; } else f->dd[1] = f->dd[0];
+    uint32_t qh = 0;
+    if (has_high) { qh = rd_u32(p); p += 4; }
+    int16_t m = has_min ? 1 : (has_high ? -16 : -8);
+    f->scm[0] = 1; f->scm[1] = m;
+    f->scm[2] = 1; f->scm[3] = m;
+    for (int j = 0; j < 16; j++) {
+        uint32_t h0 = ((qh >> j) << 4) & 0x10u;
+        uint32_t h1 = (qh >> (j + 12)) & 0x10u;
+        f->codes[j] = (uint8_t)((p[j] & 0x0Fu) | h0);
+        f->codes[j + 16] = (uint8_t)((uint32_t)(p[j] >> 4) | h1);
+    }
+}
+
+/* dequant.rs:224-250: [scales 16][qs 64][d][dmin]; 16-element group g = 8n + 2j + half takes its
+ * codes from qs[32n + 16*half ..][l] >> 2j and its (scale, min) nibbles from scales[g]. */
+static void factor_q2k(const uint8_t *blk, factored_block *f) {
+    const uint8_t *scales = blk, *qs = blk + 16;
+    f->dd[0] = rd_u16(blk + 80);
+    f->dd[1] = rd_u16(blk + 82);
+    int g = 0;
+    for (int n = 0; n < 2; n++)
+        for (int j = 0; j < 4; j++)
+            for (int half = 0; half < 2; half++, g++) {
+                uint8_t sc = scales[g];
+                f->scm[2 * g] = (int16_t)(sc & 0xF);
+                f->scm[2 * g + 1] = (int16_t)(-(int16_t)(sc >> 4));
+                for (int l = 0; l < 16; l++)
+                    f->codes[16 * g + l] = (uint8_t)((qs[32 * n + 16 * half + l] >> (2 * j)) & 3);
+            }
+}
+
+/* dequant.rs:251-312: [hmask 32][qs 64][scales 12][d]; the sixteen 6-bit scales are unpacked
+ * with ggml's kmask shuffle, then each is offset by -32; the code is the 2 low bits from qs plus
+ * bit (4n + j) of hmask[16*half + l] as bit 2; min = -4 * scale. */
+static void factor_q3k(const uint8_t *blk, factored_block *f) {
+    const uint8_t *hmask = blk, *qs = blk + 32, *sr = blk + 96;
+    f->dd[0] = rd_u16(blk + 108);
+    f->dd[1] = f->dd[0];
+    const uint32_t k1 = 0x03030303u, k2 = 0x0f0f0f0fu;
+    uint32_t a0 = rd_u32(sr), a1 = rd_u32(sr + 4), t = rd_u32(sr + 8);
+    uint32_t aux[4];
+    aux[2] = ((a0 >> 4) & k2) | (((t >> 4) & k1) << 4);
+    aux[3] = ((a1 >> 4) & k2) | (((t >> 6) & k1) << 4);
+    aux[0] = (a0 & k2) | ((t & k1) << 4);
+    aux[1] = (a1 & k2) | (((t >> 2) & k1) << 4);
+    int g = 0;
+    for (int n = 0; n < 2; n++)
+        for (int j = 0; j < 4; j++)
+            for (int half = 0; half < 2; half++, g++) {
+                int16_t s = (int16_t)((int16_t)(int8_t)((aux[g / 4] >> ((g % 4) * 8)) & 0xFF) - 32);
+                f->scm[2 * g] = s;
+                f->scm[2 * g + 1] = (int16_t)(-4 * s);
+                uint8_t mbit = (uint8_t)(1u << (4 * n + j));
+                for (int l = 0; l < 16; l++) {
+                    uint8_t low2 = (uint8_t)((qs[32 * n + 16 * half + l] >> (2 * j)) & 3);
+                    uint8_t high = (hmask[16 * half + l] & mbit) ? 1 : 0;
+                    f->codes[16 * g + l] = (uint8_t)(low2 | (high << 2));
+                }
+            }
+}
+
+/* dequant.rs:336-363: Q4_K's layout with 32 bytes of fifth bits between the scales and the
+ * nibbles: bit 2j of qh[l] belongs to the low-nibble element, bit 2j+1 to the high-nibble one. */
+static void factor_q5k(const uint8_t *blk, factored_block *f) {
+    f->dd[0] = rd_u16(blk);
+    f->dd[1] = rd_u16(blk + 2);
+    const uint8_t *scales = blk + 4, *qh = blk + 16, *qs = blk + 48;
+    for (int j = 0; j < 4; j++) {
+        uint32_t sc1, m1, sc2, m2;
+        orc_k4(2 * j, scales, &sc1, &m1);
+        orc_k4(2 * j + 1, scales, &sc2, &m2);
+        for (int q = 0; q < 4; q++) {
+            f->scm[2 * (4 * j + q)] = (int16_t)(q < 2 ? sc1 : sc2);
+            f->scm[2 * (4 * j + q) + 1] = (int16_t)(-(int16_t)(q < 2 ? m1 : m2));
+        }
+        for (int l = 0; l < 32; l++) {
+            uint8_t v = qs[j * 32 + l];
+            f->codes[j * 64 + l] = (uint8_t)((v & 0xF) + (((qh[l] >> (2 * j)) & 1) ? 16 : 0));
+            f->codes[j * 64 + 32 + l] = (uint8_t)((v >> 4) + (((qh[l] >> (2 * j + 1)) & 1) ? 16 : 0));
+        }
+    }
+}
+
 int64_t orc_dequant(int dtype, const uint8_t *bytes, size_t nbytes, float *out) {
     int be, bb;
     if (orc_block_geometry(dtype, &be, &bb) != 0) return -1;
@@ -197,6 +298,13 @@ int64_t orc_dequant(int dtype, const uint8_t *bytes, size_t nbytes, float *out) 
     for (size_t b = 0; b < nblk; b++) {
         const uint8_t *blk = bytes + b * (size_t)bb;
         switch (dtype) {
+        case ORC_Q4_0: factor_legacy(blk, 0, 0, &f); break;
+        case ORC_Q4_1: factor_legacy(blk, 1, 0, &f); break;
+        case ORC_Q5_0: factor_legacy(blk, 0, 1, &f); break;
+        case ORC_Q5_1: factor_legacy(blk, 1, 1, &f); break;
+        case ORC_Q2K: factor_q2k(blk, &f); break;
+        case ORC_Q3K: factor_q3k(blk, &f); break;
+        case ORC_Q5K: factor_q5k(blk, &f); break;
         case ORC_Q8_0: factor_q8_0(blk, &f); break;
         case ORC_Q4K: factor_q4k(blk, &f); break;
         case ORC_Q6K: factor_q6k(blk, &f); break;

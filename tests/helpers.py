@@ -6,8 +6,12 @@ from __future__ import annotations
 import numpy as np
 
 F32, F16, BF16 = 0, 1, 2
-Q8_0, Q4K, Q6K = 9, 12, 14
-BLOCK = {Q8_0: (32, 34), Q4K: (256, 144), Q6K: (256, 210), F32: (1, 4), F16: (1, 2), BF16: (1, 2)}
+Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q2K, Q3K, Q4K, Q5K, Q6K = 5, 6, 7, 8, 9, 10, 11, 12, 13, 14
+BLOCK = {Q8_0: (32, 34), Q4K: (256, 144), Q6K: (256, 210), F32: (1, 4), F16: (1, 2), BF16: (1, 2),
+         Q4_0: (32, 18), Q4_1: (32, 20), Q5_0: (32, 22), Q5_1: (32, 24), Q2K: (256, 84), Q3K: (256, 110), Q5K: (256, 176)}
+# byte offsets of the f16 scale fields inside a block
+F16_SLOTS = {Q4_0: (0,), Q4_1: (0, 2), Q5_0: (0,), Q5_1: (0, 2), Q8_0: (0,), Q2K: (80, 82), Q3K: (108,), Q4K: (0, 2),
+             Q5K: (0, 2), Q6K: (208,)}
 
 
 # ---- generators of the reference's tests ------------------------------------------------
@@ -44,6 +48,11 @@ def synth_weight(dtype: int, n_elem: int, seed: int) -> np.ndarray:
     elif dtype == Q8_0:
         blk = lcg_bytes_blocks(seed, nblk, 34)
         blk[:, 0:2] = f16_bytes(0.01)
+    elif dtype in F16_SLOTS:
+        # the remaining affine formats: LCG payload everywhere, then finite scales of either sign
+        blk = lcg_bytes_blocks(seed, nblk, bb)
+        for k, off in enumerate(F16_SLOTS[dtype]):
+            blk[:, off:off + 2] = f16_bytes(0.02 if k == 0 else -0.07)
     else:
         raise ValueError(dtype)
     return blk.reshape(-1)
@@ -142,6 +151,74 @@ def ggml_dequant(dtype: int, data: np.ndarray) -> np.ndarray:
             y[:, base + l + 32] = d[:, None] * scn[:, is_ + 2] * q2 + d[:, None] * (-32 * scn[:, is_ + 2])
             y[:, base + l + 64] = d[:, None] * scn[:, is_ + 4] * q3 + d[:, None] * (-32 * scn[:, is_ + 4])
             y[:, base + l + 96] = d[:, None] * scn[:, is_ + 6] * q4 + d[:, None] * (-32 * scn[:, is_ + 6])
+        return y.reshape(-1)
+    if dtype in (Q4_0, Q4_1, Q5_0, Q5_1):
+        # ggml dequantize_row_q4_0 / q4_1 / q5_0 / q5_1: x0 = (qs[j] & 0xF | bit j of qh << 4), x1 = (qs[j] >> 4 |
+        # bit j+16 of qh << 4); y[j] = x0, y[j+16] = x1 through d*(x - 8|16) or d*x + m.  Written in the reference's
+        # affine form d*x + (d*-8 | d*-16 | m) so that an exact cancellation is +0.0 as there.
+        five, has_m = dtype in (Q5_0, Q5_1), dtype in (Q4_1, Q5_1)
+        d = _f16(blk[:, 0:2])
+        o = 2
+        m = None
+        if has_m:
+            m = _f16(blk[:, 2:4])
+            o = 4
+        qh = np.zeros(nb, np.int64)
+        if five:
+            qh = blk[:, o:o + 4].copy().view(np.uint32).reshape(-1).astype(np.int64)
+            o += 4
+        qs = blk[:, o:o + 16].astype(np.int64)
+        j = np.arange(16)
+        x0 = (qs & 0xF) | (((qh[:, None] >> j) & 1) << 4)
+        x1 = (qs >> 4) | (((qh[:, None] >> (j + 16)) & 1) << 4)
+        x = np.concatenate([x0, x1], axis=1).astype(np.longdouble)
+        off = m if has_m else d * (-16 if five else -8)
+        return (d[:, None] * x + off[:, None]).reshape(-1)
+    if dtype == Q2K:
+        # ggml dequantize_row_q2_K: 16-element group g takes scales[g] (low nibble scale, high nibble min) and the
+        # 2-bit fields at shift 2*((g % 8) // 2) of qs[32*(g // 8) + 16*(g % 2) ..+16)
+        scales = blk[:, 0:16].astype(np.int64)
+        qs = blk[:, 16:80].astype(np.int64)
+        d, dmin = _f16(blk[:, 80:82]), _f16(blk[:, 82:84])
+        y = np.empty((nb, 256), np.longdouble)
+        for g in range(16):
+            q = (qs[:, 32 * (g // 8) + 16 * (g % 2):][:, :16] >> (2 * ((g % 8) // 2))) & 3
+            y[:, 16 * g:16 * g + 16] = (d * (scales[:, g] & 0xF))[:, None] * q + (dmin * -(scales[:, g] >> 4))[:, None]
+        return y.reshape(-1)
+    if dtype == Q3K:
+        # ggml dequantize_row_q3_K.  The sixteen 6-bit scales: low 4 bits are the nibbles of bytes 0..7 (low nibbles
+        # first), high 2 bits are the 2-bit fields of bytes 8..11; value = (6-bit - 32).  Element = low 2 bits from qs
+        # as in Q2_K, minus 4 unless bit (g // 2) of hmask[16*(g % 2) + l] is set.
+        hm = blk[:, 0:32].astype(np.int64)
+        qs = blk[:, 32:96].astype(np.int64)
+        sr = blk[:, 96:108].astype(np.int64)
+        d = _f16(blk[:, 108:110])
+        y = np.empty((nb, 256), np.longdouble)
+        for g in range(16):
+            lo = (sr[:, g % 8] >> (4 if g >= 8 else 0)) & 0xF
+            hi = (sr[:, 8 + g % 4] >> (2 * (g // 4))) & 3
+            sc = (lo | (hi << 4)) - 32
+            low2 = (qs[:, 32 * (g // 8) + 16 * (g % 2):][:, :16] >> (2 * ((g % 8) // 2))) & 3
+            hbit = (hm[:, 16 * (g % 2):][:, :16] >> (g // 2)) & 1
+            code = low2 + 4 * hbit
+            y[:, 16 * g:16 * g + 16] = (d * sc)[:, None] * code + (d * (-4 * sc))[:, None]
+        return y.reshape(-1)
+    if dtype == Q5K:
+        # ggml dequantize_row_q5_K: Q4_K plus a fifth bit: bit `is` of qh[l] for sub-block `is`
+        d, dmin = _f16(blk[:, 0:2]), _f16(blk[:, 2:4])
+        sc_b = blk[:, 4:16].astype(np.int64)
+        qh = blk[:, 16:48].astype(np.int64)
+        qs = blk[:, 48:176].astype(np.int64)
+        y = np.empty((nb, 256), np.longdouble)
+        for is_ in range(8):
+            if is_ < 4:
+                sc, m = sc_b[:, is_] & 63, sc_b[:, is_ + 4] & 63
+            else:
+                sc = (sc_b[:, is_ + 4] & 0xF) | ((sc_b[:, is_ - 4] >> 6) << 4)
+                m = (sc_b[:, is_ + 4] >> 4) | ((sc_b[:, is_] >> 6) << 4)
+            q = qs[:, (is_ // 2) * 32:(is_ // 2) * 32 + 32]
+            nib = ((q & 0xF) if is_ % 2 == 0 else (q >> 4)) + 16 * ((qh >> is_) & 1)
+            y[:, is_ * 32:(is_ + 1) * 32] = (d * sc)[:, None] * nib - (dmin * m)[:, None]
         return y.reshape(-1)
     raise ValueError(dtype)
 
@@ -242,6 +319,45 @@ def dequant_cases():
     out["q8_0_lcg"] = (Q8_0, synth_weight(Q8_0, 32 * 24, 5))
     out["q4k_lcg"] = (Q4K, synth_weight(Q4K, 256 * 6, 80))
     out["q6k_lcg"] = (Q6K, synth_weight(Q6K, 256 * 6, 90))
+    # the other affine formats: the same (i*29+3)&0xFF pattern (dequant.rs:1206-1230; its f16 fields happen to be
+    # finite for each of them), LCG blocks, and the single blocks of the reference's known-answer tests
+    for name, dt in (("q4_0", Q4_0), ("q4_1", Q4_1), ("q5_0", Q5_0), ("q5_1", Q5_1), ("q2k", Q2K), ("q3k", Q3K), ("q5k", Q5K)):
+        out[f"{name}_all_formats_pattern"] = (dt, pattern(2 * BLOCK[dt][1], 29, 3))
+        out[f"{name}_lcg"] = (dt, synth_weight(dt, BLOCK[dt][0] * 8, 100 + dt))
+    for name, (dt, b, _) in known_answer_blocks().items():
+        out[name] = (dt, b)
+    return out
+
+
+def known_answer_blocks():
+    """The single blocks of the reference's own decoder tests with the values those tests assert
+    (crates/infr-gguf/src/dequant.rs:1619-1846): name -> (dtype, bytes, {element index: value})."""
+    out = {}
+    b = np.zeros(84, np.uint8)          # q2k_single_block: scales 0x23, qs 0x55, d = 1, dmin = 2
+    b[0] = b[1] = 0x23
+    b[16:80] = 0x55
+    b[80:82], b[82:84] = f16_bytes(1.0), f16_bytes(2.0)
+    out["q2k_single_block"] = (Q2K, b, {i: -1.0 for i in range(32)})
+    b = np.zeros(110, np.uint8)         # q3k_single_block: everything 0, d = 1 -> 128 everywhere
+    b[108:110] = f16_bytes(1.0)
+    out["q3k_single_block"] = (Q3K, b, {i: 128.0 for i in range(256)})
+    b = np.full(18, 0x88, np.uint8)     # q4_0_single_block: d = 2, qs[0] = 0x89
+    b[0:2] = f16_bytes(2.0)
+    b[2] = 0x89
+    out["q4_0_single_block"] = (Q4_0, b, {0: 2.0, 16: 0.0, 1: 0.0})
+    b = np.zeros(20, np.uint8)          # q4_1_single_block: d = 1, m = 0.5, qs[0] = 0x30
+    b[0:2], b[2:4] = f16_bytes(1.0), f16_bytes(0.5)
+    b[4] = 0x30
+    out["q4_1_single_block"] = (Q4_1, b, {0: 0.5, 16: 3.5})
+    b = np.zeros(22, np.uint8)          # q5_0_single_block: d = 1, qh bit 0, qs[0] = 0x0F
+    b[0:2] = f16_bytes(1.0)
+    b[2] = 0x01
+    b[6] = 0x0F
+    out["q5_0_single_block"] = (Q5_0, b, {0: 15.0, 16: -16.0})
+    b = np.zeros(24, np.uint8)          # q5_1_single_block: d = 2, m = -1, qs[0] = 0x1F
+    b[0:2], b[2:4] = f16_bytes(2.0), f16_bytes(-1.0)
+    b[8] = 0x1F
+    out["q5_1_single_block"] = (Q5_1, b, {0: 29.0, 16: 1.0})
     return out
 
 

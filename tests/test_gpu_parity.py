@@ -94,7 +94,10 @@ def test_dequant_matches_golden_bits(be):
         assert np.array_equal(bits(got), g[n + ".bits"]), n
 
 
-@pytest.mark.parametrize("dt", [H.Q8_0, H.Q4K, H.Q6K])
+AFFINE = [H.Q4_0, H.Q4_1, H.Q5_0, H.Q5_1, H.Q8_0, H.Q2K, H.Q3K, H.Q4K, H.Q5K, H.Q6K]
+
+
+@pytest.mark.parametrize("dt", AFFINE)
 def test_dequant_matches_oracle_bits_on_a_large_tensor(be, dt):
     e, b = H.BLOCK[dt]
     raw = H.synth_weight(dt, e * 4099, seed=dt)
@@ -106,7 +109,8 @@ def test_dequant_matches_oracle_bits_on_a_large_tensor(be, dt):
 
 @pytest.mark.parametrize("dt,in_f", [(H.Q4K, 2048), (H.Q4K, 4096), (H.Q4K, 256), (H.Q4K, 1024), (H.Q6K, 768),
                                      (H.Q6K, 1536), (H.Q6K, 256), (H.Q6K, 4096), (H.Q8_0, 2048), (H.Q8_0, 768),
-                                     (H.Q8_0, 4096), (H.Q8_0, 96), (H.Q4K, 5120), (H.F16, 100)])
+                                     (H.Q8_0, 4096), (H.Q8_0, 96), (H.Q4K, 5120), (H.F16, 100), (H.Q4_0, 96), (H.Q4_1, 2048),
+                                     (H.Q5_0, 160), (H.Q5_1, 1024), (H.Q2K, 512), (H.Q3K, 768), (H.Q5K, 2048)])
 def test_one_hot_gemv_reads_back_the_decoded_weight(be, dt, in_f):
     """x = e_c makes y[o] = W[o][c]: the in-register unpacking of the GEMV kernels must reproduce
     the reference decode exactly (same trick as crates/infr-vulkan/tests/weight_dequant_parity.rs)."""
@@ -323,8 +327,8 @@ def test_compile_refuses_what_the_path_does_not_cover(be):
     g.push_raw(17)
     with pytest.raises(M.Unsupported):
         be.compile(g)
-    g, _ = moe_graph(1, 256, 8, 2, 256, DType.Q5K, DType.Q5K)
-    with pytest.raises(M.Unsupported, match="Q5K"):
+    g, _ = moe_graph(1, 256, 8, 2, 256, DType.I32, DType.I32)   # an integer table is not a weight format
+    with pytest.raises(M.Unsupported, match="I32"):
         be.compile(g)
     g, _ = moe_graph(1, 256, 8, 2, 256, DType.Q4K, DType.Q4K, ep_band=(6, 4))   # band past the last expert
     with pytest.raises(M.BackendError, match="ep_band"):
@@ -690,6 +694,48 @@ def test_norm_moe_residual_chain_folds_into_the_moe_kernels(be, rows, shared):
     want_y = O.add(x, sub).reshape(rows, ne)
     tol = 1e-2 if rows >= 32 else REL_L2
     assert H.rel_l2(folded.reshape(rows, ne) - x, want_y - x) < tol
+
+
+@pytest.mark.parametrize("m", [1, 3])
+def test_linear_sweep_over_every_affine_weight_format(be, m):
+    """The reference's weight-format sweep for Op::Linear (crates/infr-testkit/src/lib.rs:389-403: every
+    format as a LinearCase at one shape, seeds 0x201 + i) over the formats this backend decodes, at the
+    sweep's 256 x 8 shape and at a decode-sized one; reference-mode tolerance (decode_parity.rs:93-102)."""
+    for i, dt in enumerate(AFFINE):
+        for in_f, out_f in ((256, 8), (2048, 96)):
+            raw = H.synth_weight(dt, out_f * in_f, seed=0x201 + i)
+            x = H.rand_f32(m * in_f, 0x301 + i).reshape(m, in_f)
+            g = M.Graph()
+            xi, wi = g.input(TensorDesc([m, in_f], DType.F32)), g.weight(TensorDesc([out_f, in_f], DType(dt)))
+            yi = g.output(TensorDesc([m, out_f], DType.F32))
+            g.linear(x=xi, weight=wi, dst=yi, m=m, in_f=in_f, out_f=out_f)
+            got = M.run_graph(be, g, [(xi, x), (wi, raw)], yi, m * out_f).reshape(m, out_f)
+            want = O.linear(x, raw, dt, in_f, out_f)
+            assert H.rel_l2(got, want) < 1e-5, (DType(dt).name, in_f)
+
+
+@pytest.mark.parametrize("gdt,ddt,rows", [(H.Q5K, H.Q5K, 1), (H.Q4_0, H.Q5_0, 2), (H.Q2K, H.Q3K, 1), (H.Q4_1, H.Q5_1, 3),
+                                          (H.Q5K, H.Q6K, 40)])
+def test_moe_ffn_with_experts_in_the_other_affine_formats(be, gdt, ddt, rows):
+    """Expert banks in formats without a bandwidth-bound kernel run on the shape-generic kernels, at
+    every batch size (no matrix-core path for them): same routing, same tolerance."""
+    ne, nff, E, K = 512, 256, 8, 3
+    rng = np.random.default_rng(gdt * 17 + ddt)
+    x = rng.standard_normal((rows, ne)).astype(np.float32)
+    router = (rng.standard_normal((E, ne)) * 0.1).astype(np.float32)
+    gate, up = H.synth_weight(gdt, E * nff * ne, 1), H.synth_weight(gdt, E * nff * ne, 2)
+    down = H.synth_weight(ddt, E * ne * nff, 3)
+    g, ids = moe_graph(rows, ne, E, K, nff, DType(gdt), DType(ddt))
+    keep = []
+    got = M.run_graph(be, g, [(ids["x"], x), (ids["router"], router), (ids["gate"], gate), (ids["up"], up),
+                              (ids["down"], down)], ids["dst"], rows * ne, keep=keep).reshape(rows, ne)
+    routing = be.moe_routing(keep[0], 0)
+    want = O.moe_ffn(x, router, gate, up, down, ne=ne, n_expert=E, n_used=K, n_ff_exp=nff, gate_dtype=gdt, down_dtype=ddt)
+    assert np.array_equal(routing["idx"], want["idx"])
+    assert H.rel_l2(got, want["dst"].reshape(rows, ne)) < REL_L2
+    keep[0].free()
+    for buf in keep[2] + [keep[3]]:
+        buf.free()
 
 
 # ------------------------------------------------------------------ synthetic workloads at full size

@@ -20,6 +20,10 @@ def test_block_geometry_matches_ggml_formulas():
     assert O.block_geometry(O.Q8_0) == (32, 2 + 32)
     assert O.block_geometry(O.Q4K) == (256, 2 + 2 + 12 + 128)
     assert O.block_geometry(O.Q6K) == (256, 128 + 64 + 16 + 2)
+    assert O.block_geometry(O.Q4_0) == (32, 2 + 16) and O.block_geometry(O.Q4_1) == (32, 2 + 2 + 16)
+    assert O.block_geometry(O.Q5_0) == (32, 2 + 4 + 16) and O.block_geometry(O.Q5_1) == (32, 2 + 2 + 4 + 16)
+    assert O.block_geometry(O.Q2K) == (256, 16 + 64 + 2 + 2) and O.block_geometry(O.Q3K) == (256, 32 + 64 + 12 + 2)
+    assert O.block_geometry(O.Q5K) == (256, 2 + 2 + 12 + 32 + 128)
     assert O.bytes_for(O.Q4K, 768 * 2048) == 884736
     assert O.bytes_for(O.Q6K, 2048 * 768) == 1290240
     assert O.bytes_for(O.Q8_0, 768 * 2048) == 1671168
@@ -63,7 +67,7 @@ def test_k4_inverts_ggml_scale_packing_exhaustively():
 def test_dequant_matches_golden_fixture_bit_for_bit():
     g = np.load(os.path.join(GOLD, "dequant.npz"))
     names = sorted({k.rsplit(".", 1)[0] for k in g.files})
-    assert len(names) == 8
+    assert len(names) == 8 + 14 + 6
     for n in names:
         got = O.dequant(int(g[n + ".dtype"]), g[n + ".bytes"])
         assert np.array_equal(got.view(np.uint32), g[n + ".bits"]), n
@@ -75,7 +79,16 @@ def test_dequant_fixture_inputs_are_the_reference_test_patterns():
         assert np.array_equal(g[n + ".bytes"], b) and int(g[n + ".dtype"]) == dt
 
 
-@pytest.mark.parametrize("dt,seed", [(O.Q8_0, 1), (O.Q4K, 2), (O.Q6K, 3)])
+def test_dequant_gives_the_values_the_reference_tests_assert():
+    """The single blocks of crates/infr-gguf/src/dequant.rs:1619-1846 and the values asserted there."""
+    for name, (dt, b, want) in H.known_answer_blocks().items():
+        y = O.dequant(dt, b)
+        for i, v in want.items():
+            assert y[i] == np.float32(v), (name, i, y[i], v)
+
+
+@pytest.mark.parametrize("dt,seed", [(O.Q8_0, 1), (O.Q4K, 2), (O.Q6K, 3), (O.Q4_0, 4), (O.Q4_1, 5), (O.Q5_0, 6), (O.Q5_1, 7),
+                                     (O.Q2K, 8), (O.Q3K, 9), (O.Q5K, 10)])
 def test_dequant_matches_independent_decoder_on_random_blocks(dt, seed):
     be, bb = O.block_geometry(dt)
     b = H.synth_weight(dt, be * 64, seed)
