@@ -1,0 +1,278 @@
+// Dense Op::Linear GEMV for every affine GGUF format (Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q2_K, Q3_K,
+// Q4_K, Q5_K, Q6_K) through one common shape: a row is cut into 32-element units; a unit decodes to
+// 32 unsigned byte codes (eight dwords) plus one (scale, min) pair per 16 elements, and
+//     dot(unit, x) = sum_h  sc[h] * sum_{e in half h} code[e] * x[e]  +  mn[h] * sum_{e in half h} x[e].
+// The byte -> float conversion is one instruction per element (the compiler selects the
+// byte-lane convert for (q >> 8b) & 0xFF), the sums of x per 16 elements are computed once per
+// block while the activation row is staged in LDS, and the formats only differ in how the eight
+// dwords and the two pairs are cut out of the block (crates/infr-gguf/src/dequant.rs:137-389).
+//
+// The formats with their own integer-dot kernels (Q4_K, Q6_K, Q8_0) only come here for shapes those
+// kernels do not take.  Work split: a block of four waves stages up to four activation rows, each
+// wave walks output rows two at a time, lanes stride over the units of a row.
+#include "device_common.h"
+#include "kernels.h"
+
+namespace infr {
+
+namespace {
+
+struct Unit {
+    uint32_t q[8];       // element 4k + b of the unit = byte b of q[k]
+    float sc[2], mn[2];  // halves of 16 elements
+};
+
+constexpr uint32_t kLo4 = 0x0F0F0F0Fu, kB0 = 0x01010101u;
+
+// bits 0..3 of t to bit 0 of bytes 0..3 (the four shifted copies of t do not overlap)
+__device__ __forceinline__ uint32_t spread4(uint32_t t) { return ((t & 0xFu) * 0x00204081u) & kB0; }
+
+// Unit u of a row that starts at `row`.
+template <int DT>
+__device__ __forceinline__ void load_unit(const uint8_t* __restrict__ row, int u, Unit& t) {
+    if constexpr (DT == INFR_Q4_0 || DT == INFR_Q4_1 || DT == INFR_Q5_0 || DT == INFR_Q5_1) {
+        constexpr bool has_m = DT == INFR_Q4_1 || DT == INFR_Q5_1, five = DT == INFR_Q5_0 || DT == INFR_Q5_1;
+        constexpr int bb = 18 + (has_m ? 2 : 0) + (five ? 4 : 0);
+        const uint8_t* blk = row + (size_t)u * bb;
+        const uint32_t hdr = has_m ? ldu<uint32_t>(blk) : (uint32_t)ldu<uint16_t>(blk);
+        const uint8_t* p = blk + (has_m ? 4 : 2);
+        uint32_t qh = 0;
+        if constexpr (five) {
+            qh = ldu<uint32_t>(p);
+            p += 4;
+        }
+        const uint4 qs = ldu<uint4>(p);
+        const uint32_t w[4] = {qs.x, qs.y, qs.z, qs.w};
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            t.q[k] = w[k] & kLo4;
+            t.q[4 + k] = (w[k] >> 4) & kLo4;
+            if constexpr (five) {
+                t.q[k] |= spread4(qh >> (4 * k)) << 4;
+                t.q[4 + k] |= spread4(qh >> (16 + 4 * k)) << 4;
+            }
+        }
+        const float d = f16_bits_to_f32(hdr & 0xFFFFu);
+        t.sc[0] = t.sc[1] = d;
+        t.mn[0] = t.mn[1] = has_m ? f16_bits_to_f32(hdr >> 16) : d * (five ? -16.0f : -8.0f);
+    } else if constexpr (DT == INFR_Q8_0) {
+        const uint8_t* blk = row + (size_t)u * 34;
+        const float d = f16_bits_to_f32(ldu<uint16_t>(blk));
+        const uint4 a = ldu<uint4>(blk + 2), b = ldu<uint4>(blk + 18);
+        const uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+        for (int k = 0; k < 8; k++) t.q[k] = w[k] ^ 0x80808080u;   // q + 128 as an unsigned byte
+        t.sc[0] = t.sc[1] = d;
+        t.mn[0] = t.mn[1] = d * -128.0f;
+    } else if constexpr (DT == INFR_Q2K || DT == INFR_Q3K) {
+        // unit s of a block: 16-element groups 2s, 2s+1 = the 2-bit fields at shift 2*(s%4) of qs[32*(s/4) ..+32)
+        constexpr int bb = DT == INFR_Q2K ? 84 : 110;
+        const uint8_t* blk = row + (size_t)(u >> 3) * bb;
+        const int s = u & 7, n = s >> 2, j = s & 3;
+        const uint8_t* qs = blk + (DT == INFR_Q2K ? 16 : 32) + 32 * n;
+        const uint4 a = ldu<uint4>(qs), b = ldu<uint4>(qs + 16);
+        const uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+        for (int k = 0; k < 8; k++) t.q[k] = (w[k] >> (2 * j)) & 0x03030303u;
+        if constexpr (DT == INFR_Q2K) {
+            const uint32_t sb = ldu<uint16_t>(blk + 2 * s);
+            const uint32_t dd = ldu<uint32_t>(blk + 80);
+            const float d = f16_bits_to_f32(dd & 0xFFFFu), dmin = f16_bits_to_f32(dd >> 16);
+            t.sc[0] = d * (float)(sb & 0xFu);
+            t.mn[0] = dmin * (float)(-(int)((sb >> 4) & 0xFu));
+            t.sc[1] = d * (float)((sb >> 8) & 0xFu);
+            t.mn[1] = dmin * (float)(-(int)(sb >> 12));
+        } else {
+            const uint4 ha = ldu<uint4>(blk), hb = ldu<uint4>(blk + 16);
+            const uint32_t hm[8] = {ha.x, ha.y, ha.z, ha.w, hb.x, hb.y, hb.z, hb.w};
+#pragma unroll
+            for (int k = 0; k < 8; k++) t.q[k] |= ((hm[k] >> (4 * n + j)) & kB0) << 2;
+            const float d = f16_bits_to_f32(ldu<uint16_t>(blk + 108));
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const int g = 2 * s + h;   // 6-bit scale g: nibble g/8 of byte g%8, high bits = field g/4 of byte 8 + g%4
+                const uint32_t lo = ((uint32_t)blk[96 + (g & 7)] >> (g >= 8 ? 4 : 0)) & 0xFu;
+                const uint32_t hi = ((uint32_t)blk[104 + (g & 3)] >> (2 * (g >> 2))) & 3u;
+                const float sc = d * (float)((int)(lo | (hi << 4)) - 32);
+                t.sc[h] = sc;
+                t.mn[h] = -4.0f * sc;
+            }
+        }
+    } else if constexpr (DT == INFR_Q4K || DT == INFR_Q5K) {
+        // unit s = sub-block s: nibble s%2 of qs[32*(s/2) ..+32); Q5_K adds bit s of qh[l]
+        constexpr int bb = DT == INFR_Q4K ? 144 : 176;
+        const uint8_t* blk = row + (size_t)(u >> 3) * bb;
+        const int s = u & 7;
+        const uint8_t* qs = blk + (DT == INFR_Q4K ? 16 : 48) + 32 * (s >> 1);
+        const uint4 a = ldu<uint4>(qs), b = ldu<uint4>(qs + 16);
+        const uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+        for (int k = 0; k < 8; k++) t.q[k] = (w[k] >> (4 * (s & 1))) & kLo4;
+        if constexpr (DT == INFR_Q5K) {
+            const uint4 ha = ldu<uint4>(blk + 16), hb = ldu<uint4>(blk + 32);
+            const uint32_t hq[8] = {ha.x, ha.y, ha.z, ha.w, hb.x, hb.y, hb.z, hb.w};
+#pragma unroll
+            for (int k = 0; k < 8; k++) t.q[k] |= ((hq[k] >> s) & kB0) << 4;
+        }
+        uint32_t sc, m;
+        k4(s, blk + 4, sc, m);
+        const uint32_t dd = ldu<uint32_t>(blk);
+        t.sc[0] = t.sc[1] = f16_bits_to_f32(dd & 0xFFFFu) * (float)sc;
+        t.mn[0] = t.mn[1] = f16_bits_to_f32(dd >> 16) * (float)(-(int)m);
+    } else {   // Q6_K: unit s: half s/4, group g = s%4: ql[64*half + 32*(g&1) + l] nibble g/2, qh[32*half + l] field g
+        static_assert(DT == INFR_Q6K, "format without a unit decoder");
+        const uint8_t* blk = row + (size_t)(u >> 3) * 210;
+        const int s = u & 7, half = s >> 2, g = s & 3;
+        const uint8_t* ql = blk + 64 * half + 32 * (g & 1);
+        const uint8_t* qh = blk + 128 + 32 * half;
+        const uint4 a = ldu<uint4>(ql), b = ldu<uint4>(ql + 16), ha = ldu<uint4>(qh), hb = ldu<uint4>(qh + 16);
+        const uint32_t w[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+        const uint32_t hq[8] = {ha.x, ha.y, ha.z, ha.w, hb.x, hb.y, hb.z, hb.w};
+#pragma unroll
+        for (int k = 0; k < 8; k++) t.q[k] = ((w[k] >> (4 * (g >> 1))) & kLo4) | (((hq[k] >> (2 * g)) & 0x03030303u) << 4);
+        const float d = f16_bits_to_f32(ldu<uint16_t>(blk + 208));
+        const uint32_t sb = ldu<uint16_t>(blk + 192 + 8 * half + 2 * g);
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const float sc = d * (float)(int)(int8_t)((sb >> (8 * h)) & 0xFFu);
+            t.sc[h] = sc;
+            t.mn[h] = -32.0f * sc;
+        }
+    }
+}
+
+constexpr int kUnitStride = 36;   // dwords between the x values of consecutive units in LDS: 16 lanes, 64 banks
+constexpr int kRowsPerWave = 2;   // output rows a wave has in flight
+constexpr int kRowsPerBlock = 16; // 4 waves x 2 rows x 2 rounds
+
+// T activation rows per block (grid.y walks chunks of T); dst[r, o] = x[r] . W[o] (+ addend[r, o]).
+template <int DT, int T>
+__global__ __launch_bounds__(256) void linear_units_kernel(const float* __restrict__ x, const uint8_t* __restrict__ w,
+                                                           size_t row_bytes, int m, int in_f, int out_f, float* dst,
+                                                           const float* addend) {
+    extern __shared__ float lds[];
+    const int n_units = in_f >> 5;
+    float* xs = lds;                                   // [T][n_units][kUnitStride]
+    float* xsum = lds + (size_t)T * n_units * kUnitStride;   // [T][2 * n_units]
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int r0 = blockIdx.y * T;
+    // stage: one thread per 16 elements (a half unit), which also gives that half's sum
+    for (int idx = tid; idx < T * 2 * n_units; idx += 256) {
+        const int tr = idx / (2 * n_units), hu = idx - tr * 2 * n_units;
+        float4 v[4];
+        float s = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            v[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (r0 + tr < m) v[k] = reinterpret_cast<const float4*>(x + (size_t)(r0 + tr) * in_f + 16 * hu)[k];
+            s += (v[k].x + v[k].y) + (v[k].z + v[k].w);
+        }
+        float* d = xs + ((size_t)tr * n_units + (hu >> 1)) * kUnitStride + 16 * (hu & 1);
+#pragma unroll
+        for (int k = 0; k < 4; k++) reinterpret_cast<float4*>(d)[k] = v[k];
+        xsum[idx] = s;
+    }
+    __syncthreads();
+    const int row_base = blockIdx.x * kRowsPerBlock;
+    for (int round = 0; round < kRowsPerBlock / (4 * kRowsPerWave); round++) {
+        const int o0 = row_base + (round * 4 + wave) * kRowsPerWave;
+        if (o0 >= out_f) break;
+        float acc[kRowsPerWave][T];
+#pragma unroll
+        for (int a = 0; a < kRowsPerWave; a++)
+#pragma unroll
+            for (int tr = 0; tr < T; tr++) acc[a][tr] = 0.0f;
+        for (int u = lane; u < n_units; u += kWave) {
+            Unit t[kRowsPerWave];
+#pragma unroll
+            for (int a = 0; a < kRowsPerWave; a++) {
+                const int o = o0 + a < out_f ? o0 + a : out_f - 1;   // a clamped duplicate, dropped at the store
+                load_unit<DT>(w + (size_t)o * row_bytes, u, t[a]);
+            }
+#pragma unroll
+            for (int tr = 0; tr < T; tr++) {
+                const float* xu = xs + ((size_t)tr * n_units + u) * kUnitStride;
+                float s[kRowsPerWave][2];
+#pragma unroll
+                for (int a = 0; a < kRowsPerWave; a++) s[a][0] = s[a][1] = 0.0f;
+#pragma unroll
+                for (int k = 0; k < 8; k++) {
+                    const float4 xv = reinterpret_cast<const float4*>(xu)[k];
+#pragma unroll
+                    for (int a = 0; a < kRowsPerWave; a++) {
+                        const uint32_t q = t[a].q[k];
+                        float& sh = s[a][k >> 2];
+                        sh = fmaf((float)(q & 0xFFu), xv.x, sh);
+                        sh = fmaf((float)((q >> 8) & 0xFFu), xv.y, sh);
+                        sh = fmaf((float)((q >> 16) & 0xFFu), xv.z, sh);
+                        sh = fmaf((float)(q >> 24), xv.w, sh);
+                    }
+                }
+                const float2 xsu = *reinterpret_cast<const float2*>(xsum + (size_t)tr * 2 * n_units + 2 * u);
+#pragma unroll
+                for (int a = 0; a < kRowsPerWave; a++)
+                    acc[a][tr] += (t[a].sc[0] * s[a][0] + t[a].mn[0] * xsu.x) + (t[a].sc[1] * s[a][1] + t[a].mn[1] * xsu.y);
+            }
+        }
+#pragma unroll
+        for (int a = 0; a < kRowsPerWave; a++)
+#pragma unroll
+            for (int tr = 0; tr < T; tr++) {
+                const float y = wave_sum(acc[a][tr]);
+                if (lane == 0 && o0 + a < out_f && r0 + tr < m) {
+                    const size_t oi = (size_t)(r0 + tr) * out_f + o0 + a;
+                    dst[oi] = addend ? __fadd_rn(addend[oi], y) : y;
+                }
+            }
+    }
+}
+
+size_t units_lds_bytes(int t, int in_f) { return (size_t)t * (in_f >> 5) * (kUnitStride + 2) * sizeof(float); }
+
+template <int DT, int T>
+void launch_units(hipStream_t s, const float* x, const uint8_t* w, size_t row_bytes, int m, int in_f, int out_f, float* dst,
+                  const float* addend) {
+    const size_t lds = units_lds_bytes(T, in_f);
+    static bool attr_set = false;
+    if (!attr_set) {
+        (void)hipFuncSetAttribute((const void*)linear_units_kernel<DT, T>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        attr_set = true;
+    }
+    dim3 grid((out_f + kRowsPerBlock - 1) / kRowsPerBlock, (m + T - 1) / T), block(256);
+    INFR_LAUNCH((linear_units_kernel<DT, T>), grid, block, lds, s, x, w, row_bytes, m, in_f, out_f, dst, addend);
+}
+
+template <int DT>
+void launch_units_dt(hipStream_t s, const float* x, const uint8_t* w, size_t row_bytes, int m, int in_f, int out_f, float* dst,
+                     const float* addend) {
+    constexpr size_t budget = 144 * 1024;
+    if (m >= 4 && units_lds_bytes(4, in_f) <= budget) launch_units<DT, 4>(s, x, w, row_bytes, m, in_f, out_f, dst, addend);
+    else if (m >= 2 && units_lds_bytes(2, in_f) <= budget) launch_units<DT, 2>(s, x, w, row_bytes, m, in_f, out_f, dst, addend);
+    else launch_units<DT, 1>(s, x, w, row_bytes, m, in_f, out_f, dst, addend);
+}
+
+}  // namespace
+
+bool linear_units_supported(int dt, int in_f, const void* x) {
+    switch (dt) {
+        case INFR_Q4_0: case INFR_Q4_1: case INFR_Q5_0: case INFR_Q5_1: case INFR_Q8_0: break;
+        case INFR_Q2K: case INFR_Q3K: case INFR_Q4K: case INFR_Q5K: case INFR_Q6K:
+            if (in_f % 256) return false;
+            break;
+        default: return false;
+    }
+    return in_f >= 32 && in_f % 32 == 0 && units_lds_bytes(1, in_f) <= 144 * 1024 && ((uintptr_t)x & 15) == 0;
+}
+
+void launch_linear_units(hipStream_t s, const float* x, const uint8_t* w, int dt, size_t row_bytes, int m, int in_f,
+                         int out_f, float* dst, const float* addend) {
+    switch (dt) {
+#define INFR_UNITS(D) case D: launch_units_dt<D>(s, x, w, row_bytes, m, in_f, out_f, dst, addend); break
+        INFR_UNITS(INFR_Q4_0); INFR_UNITS(INFR_Q4_1); INFR_UNITS(INFR_Q5_0); INFR_UNITS(INFR_Q5_1); INFR_UNITS(INFR_Q8_0);
+        INFR_UNITS(INFR_Q2K); INFR_UNITS(INFR_Q3K); INFR_UNITS(INFR_Q4K); INFR_UNITS(INFR_Q5K); INFR_UNITS(INFR_Q6K);
+#undef INFR_UNITS
+        default: break;
+    }
+}
+
+}  // namespace infr

@@ -152,6 +152,10 @@ void launch_linear(hipStream_t s, const float* x, const uint8_t* w, int dt, size
                    int out_f, float* dst, int n_cu, const float* addend = nullptr);
 void launch_gated_act(hipStream_t s, const float* gate, const float* up, float* dst, int rows, int nff, int act,
                       int up_off, int up_stride, int gate_stride, int gate_block_width, int has_clamp, float clamp);
+// GEMV over 32-element units for any affine GGUF format (k_affine.hip); x must be 16-byte aligned.
+bool linear_units_supported(int dt, int in_f, const void* x);
+void launch_linear_units(hipStream_t s, const float* x, const uint8_t* w, int dt, size_t row_bytes, int m, int in_f,
+                         int out_f, float* dst, const float* addend);
 void launch_add(hipStream_t s, const float* a, const float* b, float* dst, uint32_t n);
 // Op::RmsNorm (add = 0) / Op::RmsNormAdd (add = 1); dst may be x.
 void launch_rms_norm(hipStream_t s, const float* x, const float* weight, float* dst, int rows, int dim, float eps, int add);

@@ -696,7 +696,7 @@ def test_norm_moe_residual_chain_folds_into_the_moe_kernels(be, rows, shared):
     assert H.rel_l2(folded.reshape(rows, ne) - x, want_y - x) < tol
 
 
-@pytest.mark.parametrize("m", [1, 3])
+@pytest.mark.parametrize("m", [1, 3, 6])
 def test_linear_sweep_over_every_affine_weight_format(be, m):
     """The reference's weight-format sweep for Op::Linear (crates/infr-testkit/src/lib.rs:389-403: every
     format as a LinearCase at one shape, seeds 0x201 + i) over the formats this backend decodes, at the
