@@ -590,6 +590,7 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
                     arena += round_up(((size_t)m.n_expert + 2) * 4, 256) + 3 * round_up(pairs * 4 + 4, 256);
                     shared += round_up(pairs * m.ne * 4, 256);
                 }
+                if (!batched && !bucketed) shared += round_up(pairs * m.ne * 4, 256);   // per-pair down results of the unit kernels
                 if (shared > shared_need) shared_need = shared;
                 plan->moe[oi].rows = (int)rows;
                 plan->moe[oi].batched = batched;
@@ -896,7 +897,7 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
             s.hh = (_Float16*)p; p += round_up(pairs * m.n_ff_exp * 2, 256);
             s.hs = (float*)p;    p += round_up(pairs * 4, 256);
             s.y = (float*)p;
-        } else if (s.bucketed) {
+        } else {
             s.y = (float*)p;
         }
     }
@@ -1198,6 +1199,7 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                     if (!fz.res) gp.dst = (float*)ptr[ad.dst];
                 }
                 gp.route = rp;
+                gp.y = sc.y;
                 // Every block of the gate/up kernel routes its own token row when that is cheaper than a
                 // launch of the routing kernel: the blocks of one compute unit repeat it once per row.
                 gp.route_inline = infr::moe_gate_up_routes_inline(gp) && (rows == 1 || (uint64_t)rows * m.n_expert <= 512) ? 1 : 0;
@@ -1206,10 +1208,24 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                     infr::launch_route(s, rp);
                 }
                 {
-                    Timed t(be, gp.sh_gate ? "moe_route_gate_up_shared" : gp.route_inline ? "moe_route_gate_up" : "moe_gate_up");
+                    const bool units = !infr::moe_gate_up_routes_inline(gp) && infr::moe_gate_up_units_supported(gp);
+                    Timed t(be, gp.sh_gate ? "moe_route_gate_up_shared" : gp.route_inline ? "moe_route_gate_up"
+                                : units ? "moe_gate_up_units" : "moe_gate_up");
                     infr::launch_moe_gate_up(s, gp);
                 }
                 gp.x = nullptr;
+                if (!gp.sh_down && !infr::moe_down_is_fast(gp) && infr::moe_down_units_supported(gp)) {
+                    // a down bank without an integer-dot kernel: per-pair rows on the unit kernel, then the
+                    // rank-ordered weighted sum
+                    {
+                        Timed t(be, "moe_down_units");
+                        infr::launch_moe_down_units(s, gp);
+                    }
+                    Timed t(be, "moe_unbucket_combine");
+                    infr::launch_unbucket_combine(s, gp.y, nullptr, gp.weights, rows, (int)m.ne, (int)m.n_used,
+                                                  (int)m.weight_before, gp.dst, 1, nullptr, gp.addend, gp.skip_zero_w);
+                    break;
+                }
                 {
                     Timed t(be, gp.sh_down ? "moe_down_combine_shared" : "moe_down_combine");
                     infr::launch_moe_down_combine(s, gp);

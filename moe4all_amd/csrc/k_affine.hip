@@ -227,6 +227,139 @@ __global__ __launch_bounds__(256) void linear_units_kernel(const float* __restri
     }
 }
 
+// Op::MoeFfn's two expert GEMV stages on units, for expert banks in formats without an integer-dot
+// kernel: grid.y = (row, rank) pair; the block stages that pair's activation row (x for gate/up, h for
+// down) and its waves walk the selected expert's rows.  gate/up: h[pair, f] = act(gate . x) * (up . x);
+// down: y[pair, o] = down . h[pair] (* down_scale[e]); the rank-ordered weighted sum is a separate
+// combine launch.  An expert id outside the bank (possible with caller-given ids) yields zeros.
+template <int DT, bool GATE_UP>
+__global__ __launch_bounds__(256) void moe_units_kernel(MoeGemvParams p, size_t row_bytes) {
+    extern __shared__ float lds[];
+    const int in_f = GATE_UP ? p.ne : p.nff, out_f = GATE_UP ? p.nff : p.ne;
+    const int n_units = in_f >> 5;
+    float* xs = lds;
+    float* xsum = lds + (size_t)n_units * kUnitStride;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int pair = blockIdx.y, r = pair / p.n_used;
+    const int e = p.ids[pair];
+    const float* xrow = GATE_UP ? p.x + (size_t)r * p.ne : p.h + (size_t)pair * p.nff;
+    float* out = GATE_UP ? p.h + (size_t)pair * p.nff : p.y + (size_t)pair * p.ne;
+    const int row_base = blockIdx.x * kRowsPerBlock;
+    if (e < 0 || e >= p.n_expert) {
+        for (int o = row_base + tid; o < min(row_base + kRowsPerBlock, out_f); o += 256) out[o] = 0.0f;
+        return;
+    }
+    for (int hu = tid; hu < 2 * n_units; hu += 256) {
+        float4 v[4];
+        float sm = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            v[k] = reinterpret_cast<const float4*>(xrow + 16 * hu)[k];
+            sm += (v[k].x + v[k].y) + (v[k].z + v[k].w);
+        }
+        float* d = xs + (size_t)(hu >> 1) * kUnitStride + 16 * (hu & 1);
+#pragma unroll
+        for (int k = 0; k < 4; k++) reinterpret_cast<float4*>(d)[k] = v[k];
+        xsum[hu] = sm;
+    }
+    __syncthreads();
+    constexpr int M = GATE_UP ? 2 : 1;   // matrices per output row
+    const uint8_t* base[M];
+    base[0] = (GATE_UP ? p.gate + (size_t)e * p.gate_stride : p.down + (size_t)e * p.down_stride);
+    if constexpr (GATE_UP) base[1] = p.up + (size_t)e * p.up_stride;
+    for (int round = 0; round < kRowsPerBlock / (4 * kRowsPerWave); round++) {
+        const int o0 = row_base + (round * 4 + wave) * kRowsPerWave;
+        if (o0 >= out_f) break;
+        float acc[kRowsPerWave][M];
+#pragma unroll
+        for (int a = 0; a < kRowsPerWave; a++)
+#pragma unroll
+            for (int mi = 0; mi < M; mi++) acc[a][mi] = 0.0f;
+        for (int u = lane; u < n_units; u += kWave) {
+            Unit t[kRowsPerWave][M];
+#pragma unroll
+            for (int a = 0; a < kRowsPerWave; a++) {
+                const int o = o0 + a < out_f ? o0 + a : out_f - 1;
+#pragma unroll
+                for (int mi = 0; mi < M; mi++) load_unit<DT>(base[mi] + (size_t)o * row_bytes, u, t[a][mi]);
+            }
+            const float* xu = xs + (size_t)u * kUnitStride;
+            float sh[kRowsPerWave][M][2];
+#pragma unroll
+            for (int a = 0; a < kRowsPerWave; a++)
+#pragma unroll
+                for (int mi = 0; mi < M; mi++) sh[a][mi][0] = sh[a][mi][1] = 0.0f;
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                const float4 xv = reinterpret_cast<const float4*>(xu)[k];
+#pragma unroll
+                for (int a = 0; a < kRowsPerWave; a++)
+#pragma unroll
+                    for (int mi = 0; mi < M; mi++) {
+                        const uint32_t q = t[a][mi].q[k];
+                        float& v = sh[a][mi][k >> 2];
+                        v = fmaf((float)(q & 0xFFu), xv.x, v);
+                        v = fmaf((float)((q >> 8) & 0xFFu), xv.y, v);
+                        v = fmaf((float)((q >> 16) & 0xFFu), xv.z, v);
+                        v = fmaf((float)(q >> 24), xv.w, v);
+                    }
+            }
+            const float2 xsu = *reinterpret_cast<const float2*>(xsum + 2 * u);
+#pragma unroll
+            for (int a = 0; a < kRowsPerWave; a++)
+#pragma unroll
+                for (int mi = 0; mi < M; mi++)
+                    acc[a][mi] += (t[a][mi].sc[0] * sh[a][mi][0] + t[a][mi].mn[0] * xsu.x) +
+                                  (t[a][mi].sc[1] * sh[a][mi][1] + t[a][mi].mn[1] * xsu.y);
+        }
+#pragma unroll
+        for (int a = 0; a < kRowsPerWave; a++) {
+            float v[M];
+#pragma unroll
+            for (int mi = 0; mi < M; mi++) v[mi] = wave_sum(acc[a][mi]);
+            if (lane == 0 && o0 + a < out_f) {
+                if constexpr (GATE_UP) {
+                    if (p.weight_before) {
+                        const float wp = p.weights[pair];
+                        v[0] = __fmul_rn(wp, v[0]);
+                        v[1] = __fmul_rn(wp, v[1]);
+                    }
+                    out[o0 + a] = gated_act_fn(p.act, p.has_clamp, p.clamp, v[0], v[1]);
+                } else {
+                    out[o0 + a] = p.down_scale ? __fmul_rn(v[0], p.down_scale[e]) : v[0];
+                }
+            }
+        }
+    }
+}
+
+template <int DT, bool GATE_UP>
+void launch_moe_units_dt(hipStream_t s, const MoeGemvParams& p) {
+    const int in_f = GATE_UP ? p.ne : p.nff, out_f = GATE_UP ? p.nff : p.ne;
+    int be = 1, bb = 4;
+    block_geometry(DT, &be, &bb);
+    const size_t row_bytes = (size_t)(in_f / be) * bb;
+    static bool attr_set = false;
+    if (!attr_set) {
+        (void)hipFuncSetAttribute((const void*)moe_units_kernel<DT, GATE_UP>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        attr_set = true;
+    }
+    dim3 grid((out_f + kRowsPerBlock - 1) / kRowsPerBlock, p.rows * p.n_used), block(256);
+    INFR_LAUNCH((moe_units_kernel<DT, GATE_UP>), grid, block, (size_t)(in_f >> 5) * (kUnitStride + 2) * sizeof(float), s, p,
+                row_bytes);
+}
+
+template <bool GATE_UP>
+void launch_moe_units_any(hipStream_t s, int dt, const MoeGemvParams& p) {
+    switch (dt) {
+#define INFR_UNITS(D) case D: launch_moe_units_dt<D, GATE_UP>(s, p); break
+        INFR_UNITS(INFR_Q4_0); INFR_UNITS(INFR_Q4_1); INFR_UNITS(INFR_Q5_0); INFR_UNITS(INFR_Q5_1); INFR_UNITS(INFR_Q8_0);
+        INFR_UNITS(INFR_Q2K); INFR_UNITS(INFR_Q3K); INFR_UNITS(INFR_Q4K); INFR_UNITS(INFR_Q5K); INFR_UNITS(INFR_Q6K);
+#undef INFR_UNITS
+        default: break;
+    }
+}
+
 size_t units_lds_bytes(int t, int in_f) { return (size_t)t * (in_f >> 5) * (kUnitStride + 2) * sizeof(float); }
 
 template <int DT, int T>
@@ -263,6 +396,15 @@ bool linear_units_supported(int dt, int in_f, const void* x) {
     }
     return in_f >= 32 && in_f % 32 == 0 && units_lds_bytes(1, in_f) <= 144 * 1024 && ((uintptr_t)x & 15) == 0;
 }
+
+bool moe_gate_up_units_supported(const MoeGemvParams& p) {
+    return p.gate_dt == p.up_dt && p.rows * p.n_used <= 65535 && linear_units_supported(p.gate_dt, p.ne, p.x);
+}
+void launch_moe_gate_up_units(hipStream_t s, const MoeGemvParams& p) { launch_moe_units_any<true>(s, p.gate_dt, p); }
+bool moe_down_units_supported(const MoeGemvParams& p) {
+    return p.y != nullptr && p.rows * p.n_used <= 65535 && linear_units_supported(p.down_dt, p.nff, p.h);
+}
+void launch_moe_down_units(hipStream_t s, const MoeGemvParams& p) { launch_moe_units_any<false>(s, p.down_dt, p); }
 
 void launch_linear_units(hipStream_t s, const float* x, const uint8_t* w, int dt, size_t row_bytes, int m, int in_f,
                          int out_f, float* dst, const float* addend) {

@@ -788,6 +788,10 @@ void launch_moe_gate_up(hipStream_t s, const MoeGemvParams& p) {
         else if (p.gate_dt == INFR_Q8_0) done = try_gate_up<Q80Fmt>(s, p);
         if (done) return;
     }
+    if (!p.sh_gate && moe_gate_up_units_supported(p)) {   // the other affine formats, and shapes the kernels above refuse
+        launch_moe_gate_up_units(s, p);
+        return;
+    }
     dim3 grid((p.nff + 3) / 4, p.rows * p.n_used), block(256);
     INFR_LAUNCH(moe_gate_up_generic, grid, block, 0, s, p, row_bytes_of(p.gate_dt, p.ne),
                        row_bytes_of(p.up_dt, p.ne));

@@ -773,15 +773,17 @@ template <class Y>
 __global__ __launch_bounds__(256) void unbucket_combine_kernel(const Y* __restrict__ y, const int32_t* __restrict__ slot_pair,
                                                                const float* __restrict__ weights, int ne, int n_used,
                                                                int weight_before, float* dst, int identity,
-                                                               const float* __restrict__ pair_scale, const float* addend) {
+                                                               const float* __restrict__ pair_scale, const float* addend,
+                                                               int skip_zero_w) {
     const size_t row = blockIdx.y;
     const int i = (blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= ne) return;
     float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
     for (int k = 0; k < n_used; k++) {
-        int pr = slot_pair[row * n_used + k];
+        int pr = slot_pair ? slot_pair[row * n_used + k] : 0;
         if (pr < 0) continue;
-        if (identity) pr = (int)(row * n_used + k);
+        if (identity || !slot_pair) pr = (int)(row * n_used + k);
+        if (skip_zero_w && weights[row * n_used + k] == 0.0f) continue;
         const float w = weight_before ? 1.0f : weights[row * n_used + k];
         const float sc = pair_scale ? pair_scale[pr] : 1.0f;
         const Y* yr = y + (size_t)pr * ne + i;
@@ -881,15 +883,15 @@ void launch_grouped_down(hipStream_t s, int dt, const GroupedParams& p) {
 
 void launch_unbucket_combine(hipStream_t s, const void* y, const int32_t* slot_pair, const float* weights, int rows,
                              int ne, int n_used, int weight_before, float* dst, int identity, const float* pair_scale,
-                             const float* addend) {
+                             const float* addend, int skip_zero_w) {
     if (rows <= 0) return;
     const dim3 grid((ne + 1023) / 1024, rows), block(256);
     if (pair_scale)
         INFR_LAUNCH(unbucket_combine_kernel<_Float16>, grid, block, 0, s, (const _Float16*)y, slot_pair, weights, ne, n_used,
-                    weight_before, dst, identity, pair_scale, addend);
+                    weight_before, dst, identity, pair_scale, addend, skip_zero_w);
     else
         INFR_LAUNCH(unbucket_combine_kernel<float>, grid, block, 0, s, (const float*)y, slot_pair, weights, ne, n_used,
-                    weight_before, dst, identity, pair_scale, addend);
+                    weight_before, dst, identity, pair_scale, addend, skip_zero_w);
 }
 
 }  // namespace infr

@@ -127,11 +127,13 @@ void launch_bucket(hipStream_t s, const int32_t* ids, int n_pairs, int n_expert,
                    int32_t* slot_pair);
 void launch_grouped_gate_up(hipStream_t s, int dt, const GroupedParams& p);
 void launch_grouped_down(hipStream_t s, int dt, const GroupedParams& p);
-// identity != 0: y is in flat (row, rank) order and slot_pair only flags invalid pairs (< 0).
+// identity != 0: y is in flat (row, rank) order and slot_pair only flags invalid pairs (< 0); a null slot_pair
+// means flat order with every pair valid.  skip_zero_w: pairs of weight 0 are left out (expert-parallel bands).
 void launch_unbucket_combine(hipStream_t s, const void* y, const int32_t* slot_pair, const float* weights, int rows,
                              int ne, int n_used, int weight_before, float* dst, int identity = 0,
                              const float* pair_scale = nullptr,   // != null: y is f16, y[pair] * pair_scale[pair]
-                             const float* addend = nullptr);      // != null: dst = addend + sum ([rows, ne], may be dst)
+                             const float* addend = nullptr,       // != null: dst = addend + sum ([rows, ne], may be dst)
+                             int skip_zero_w = 0);
 
 // Decode batches with weight reuse: one block per (feature tile, expert) walks the expert's bucket,
 // so an expert's rows are read from HBM once however many token rows selected it.  h and y are in
@@ -156,6 +158,12 @@ void launch_gated_act(hipStream_t s, const float* gate, const float* up, float* 
 bool linear_units_supported(int dt, int in_f, const void* x);
 void launch_linear_units(hipStream_t s, const float* x, const uint8_t* w, int dt, size_t row_bytes, int m, int in_f,
                          int out_f, float* dst, const float* addend);
+// Op::MoeFfn's expert stages on the same units, one block column per (row, rank) pair: h[pair] from x (gate/up),
+// y[pair] from h (down; needs p.y).  The weighted sum over ranks is launch_unbucket_combine's.
+bool moe_gate_up_units_supported(const MoeGemvParams& p);
+void launch_moe_gate_up_units(hipStream_t s, const MoeGemvParams& p);
+bool moe_down_units_supported(const MoeGemvParams& p);
+void launch_moe_down_units(hipStream_t s, const MoeGemvParams& p);
 void launch_add(hipStream_t s, const float* a, const float* b, float* dst, uint32_t n);
 // Op::RmsNorm (add = 0) / Op::RmsNormAdd (add = 1); dst may be x.
 void launch_rms_norm(hipStream_t s, const float* x, const float* weight, float* dst, int rows, int dim, float eps, int add);

@@ -715,10 +715,11 @@ def test_linear_sweep_over_every_affine_weight_format(be, m):
 
 
 @pytest.mark.parametrize("gdt,ddt,rows", [(H.Q5K, H.Q5K, 1), (H.Q4_0, H.Q5_0, 2), (H.Q2K, H.Q3K, 1), (H.Q4_1, H.Q5_1, 3),
-                                          (H.Q5K, H.Q6K, 40)])
+                                          (H.Q5K, H.Q6K, 40), (H.Q3K, H.Q2K, 5), (H.Q5_1, H.Q4_0, 1)])
 def test_moe_ffn_with_experts_in_the_other_affine_formats(be, gdt, ddt, rows):
-    """Expert banks in formats without a bandwidth-bound kernel run on the shape-generic kernels, at
-    every batch size (no matrix-core path for them): same routing, same tolerance."""
+    """Expert banks in formats without an integer-dot kernel run on the 32-element-unit kernels, one
+    block column per (row, rank) pair at every batch size (no matrix-core path for them): same
+    routing, same tolerance."""
     ne, nff, E, K = 512, 256, 8, 3
     rng = np.random.default_rng(gdt * 17 + ddt)
     x = rng.standard_normal((rows, ne)).astype(np.float32)
@@ -733,6 +734,12 @@ def test_moe_ffn_with_experts_in_the_other_affine_formats(be, gdt, ddt, rows):
     want = O.moe_ffn(x, router, gate, up, down, ne=ne, n_expert=E, n_used=K, n_ff_exp=nff, gate_dtype=gdt, down_dtype=ddt)
     assert np.array_equal(routing["idx"], want["idx"])
     assert H.rel_l2(got, want["dst"].reshape(rows, ne)) < REL_L2
+    be.prof_enable(True)
+    be.execute(keep[0], keep[1])
+    be.sync()
+    names = set(be.prof_read())
+    be.prof_enable(False)
+    assert "moe_gate_up_units" in names and ("moe_down_units" in names or ddt == H.Q6K)
     keep[0].free()
     for buf in keep[2] + [keep[3]]:
         buf.free()
