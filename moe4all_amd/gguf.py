@@ -199,6 +199,7 @@ class MoeHyper:
     n_used: int
     n_ff_exp: int
     eps: float
+    shexp_ff: int = 0   # {arch}.expert_shared_feed_forward_length (config.rs:1189, :1508); 0 = no shared expert
 
 
 def moe_hyper(g: Gguf) -> MoeHyper:
@@ -214,7 +215,8 @@ def moe_hyper(g: Gguf) -> MoeHyper:
 
     eps = g.meta_f64(f"{arch}.attention.layer_norm_rms_epsilon")
     return MoeHyper(arch, need("block_count"), need("embedding_length"), need("expert_count"), need("expert_used_count"),
-                    need("expert_feed_forward_length"), 1e-6 if eps is None else eps)
+                    need("expert_feed_forward_length"), 1e-6 if eps is None else eps,
+                    g.meta_u64(f"{arch}.expert_shared_feed_forward_length") or 0)
 
 
 class MoeFfnLayer:
@@ -224,26 +226,44 @@ class MoeFfnLayer:
     ffn_gate_exps / ffn_up_exps / ffn_down_exps.weight.  qwen3moe parameterisation
     (config.rs:1270-1272): softmax gating, renormalised weights, scale 1.  GGUF lists a tensor's
     fastest axis first, so ffn_gate_exps [ne, n_ff, n_expert] is the row-major [n_expert, n_ff, ne]
-    bank Op::MoeFfn reads."""
+    bank Op::MoeFfn reads.
+
+    With a shared expert (`expert_shared_feed_forward_length` > 0; runner.rs:2586-2596, :8089-8174) the
+    layer also binds ffn_{gate,up,down}_shexp.weight and emits Linear, Linear, GatedAct, Linear on the same
+    normalised input, combined by Op::MoeSharedExpertAdd when the file carries ffn_gate_inp_shexp.weight
+    (a per-token sigmoid gate, qwen35moe) and by a plain Op::Add otherwise (llama4)."""
 
     ROLES = {"norm": "ffn_norm.weight", "router": "ffn_gate_inp.weight", "gate": "ffn_gate_exps.weight",
              "up": "ffn_up_exps.weight", "down": "ffn_down_exps.weight"}
+    SHARED = {"sh_gate": "ffn_gate_shexp.weight", "sh_up": "ffn_up_shexp.weight", "sh_down": "ffn_down_shexp.weight"}
 
     def __init__(self, be: Backend, g: Gguf, layer: int, rows: int, hyper: Optional[MoeHyper] = None):
         hp = hyper or moe_hyper(g)
         self.be, self.hyper, self.rows, self.layer = be, hp, rows, layer
         self.buffers: Dict[str, Buffer] = {}
         infos = {}
-        for role, suffix in self.ROLES.items():
+        roles = dict(self.ROLES)
+        self.gated = False
+        if hp.shexp_ff:
+            roles.update(self.SHARED)
+            self.gated = g.has(f"blk.{layer}.ffn_gate_inp_shexp.weight")
+            if self.gated:
+                roles["sh_gate_inp"] = "ffn_gate_inp_shexp.weight"
+        for role, suffix in roles.items():
             name = f"blk.{layer}.{suffix}"
             info = g.find(name)
             infos[role] = info
             self.buffers[role], _, _ = g.bind_weight(be, name)
         want = {"norm": (hp.ne,), "router": (hp.ne, hp.n_expert), "gate": (hp.ne, hp.n_ff_exp, hp.n_expert),
                 "up": (hp.ne, hp.n_ff_exp, hp.n_expert), "down": (hp.n_ff_exp, hp.ne, hp.n_expert)}
+        if hp.shexp_ff:
+            want.update({"sh_gate": (hp.ne, hp.shexp_ff), "sh_up": (hp.ne, hp.shexp_ff), "sh_down": (hp.shexp_ff, hp.ne)})
+            if self.gated and infos["sh_gate_inp"].numel != hp.ne:
+                raise LoaderError(f"GGUF: blk.{layer}.ffn_gate_inp_shexp.weight has {infos['sh_gate_inp'].numel} elements, "
+                                  f"the model's hyperparameters need {hp.ne}")
         for role, shape in want.items():
             if infos[role].shape != shape:
-                raise LoaderError(f"GGUF: blk.{layer}.{self.ROLES[role]} has shape {infos[role].shape}, the model's "
+                raise LoaderError(f"GGUF: blk.{layer}.{roles[role]} has shape {infos[role].shape}, the model's "
                                   f"hyperparameters need {shape}")
         gr = Graph()
         self.x = gr.input(TensorDesc([rows, hp.ne], DType.F32))
@@ -258,9 +278,29 @@ class MoeFfnLayer:
         sub = gr.internal(TensorDesc([rows, hp.ne], DType.F32))
         self.y = gr.output(TensorDesc([rows, hp.ne], DType.F32))
         gr.rms_norm(x=self.x, weight=self.t["norm"], dst=self.xn, rows=rows, dim=hp.ne, eps=hp.eps)
+        moe_dst = gr.internal(TensorDesc([rows, hp.ne], DType.F32)) if hp.shexp_ff else sub
         gr.moe_ffn(x=self.xn, router=self.t["router"], gate_exps=self.t["gate"], up_exps=self.t["up"],
-                   down_exps=self.t["down"], dst=sub, ne=hp.ne, n_expert=hp.n_expert, n_used=hp.n_used,
+                   down_exps=self.t["down"], dst=moe_dst, ne=hp.ne, n_expert=hp.n_expert, n_used=hp.n_used,
                    n_ff_exp=hp.n_ff_exp)
+        if hp.shexp_ff:
+            sff = hp.shexp_ff
+            self.t["sh_gate"] = gr.weight(TensorDesc([sff, hp.ne], DType(infos["sh_gate"].dtype)))
+            self.t["sh_up"] = gr.weight(TensorDesc([sff, hp.ne], DType(infos["sh_up"].dtype)))
+            self.t["sh_down"] = gr.weight(TensorDesc([hp.ne, sff], DType(infos["sh_down"].dtype)))
+            gbuf, ubuf = gr.internal(TensorDesc([rows, sff], DType.F32)), gr.internal(TensorDesc([rows, sff], DType.F32))
+            act, d_out = gr.internal(TensorDesc([rows, sff], DType.F32)), gr.internal(TensorDesc([rows, hp.ne], DType.F32))
+            if self.gated:   # the gate logit comes first, as the reference emits it (runner.rs:8104-8114)
+                self.t["sh_gate_inp"] = gr.weight(TensorDesc([1, hp.ne], DType(infos["sh_gate_inp"].dtype)))
+                gate_logit = gr.internal(TensorDesc([rows, 1], DType.F32))
+                gr.linear(x=self.xn, weight=self.t["sh_gate_inp"], dst=gate_logit, m=rows, in_f=hp.ne, out_f=1)
+            gr.linear(x=self.xn, weight=self.t["sh_gate"], dst=gbuf, m=rows, in_f=hp.ne, out_f=sff)
+            gr.linear(x=self.xn, weight=self.t["sh_up"], dst=ubuf, m=rows, in_f=hp.ne, out_f=sff)
+            gr.gated_act(gate=gbuf, up=ubuf, dst=act, rows=rows, nff=sff)
+            gr.linear(x=act, weight=self.t["sh_down"], dst=d_out, m=rows, in_f=sff, out_f=hp.ne)
+            if self.gated:
+                gr.moe_shared_expert_add(moe=moe_dst, shexp=d_out, gate=gate_logit, dst=sub, rows=rows, n=hp.ne)
+            else:
+                gr.add(a=moe_dst, b=d_out, dst=sub, n=rows * hp.ne)
         gr.add(a=self.x, b=sub, dst=self.y, n=rows * hp.ne)
         self.graph = gr
         self.moe_op = 1

@@ -27,8 +27,9 @@ def _bf16(a):
     return (np.ascontiguousarray(a, np.float32).view(np.uint32) >> 16).astype(np.uint16)
 
 
-def _moe_file(path, rng, *, ne, n_ff, E, K, layers, gdt, ddt, shards=1):
-    """A qwen3moe-shaped file: per layer ffn_norm, ffn_gate_inp and the three expert banks."""
+def _moe_file(path, rng, *, ne, n_ff, E, K, layers, gdt, ddt, shards=1, shexp=0, gated=False):
+    """A qwen3moe-shaped file: per layer ffn_norm, ffn_gate_inp and the three expert banks; with `shexp`
+    also the shared expert's three matrices and, if `gated`, its gate vector."""
     per_layer = []
     for l in range(layers):
         w = {
@@ -38,6 +39,12 @@ def _moe_file(path, rng, *, ne, n_ff, E, K, layers, gdt, ddt, shards=1):
             "ffn_up_exps.weight": ((ne, n_ff, E), W.GGML[gdt], H.synth_weight(getattr(H, gdt), E * n_ff * ne, 20 + l)),
             "ffn_down_exps.weight": ((n_ff, ne, E), W.GGML[ddt], H.synth_weight(getattr(H, ddt), E * ne * n_ff, 30 + l)),
         }
+        if shexp:
+            w["ffn_gate_shexp.weight"] = ((ne, shexp), W.GGML[gdt], H.synth_weight(getattr(H, gdt), shexp * ne, 40 + l))
+            w["ffn_up_shexp.weight"] = ((ne, shexp), W.GGML[gdt], H.synth_weight(getattr(H, gdt), shexp * ne, 50 + l))
+            w["ffn_down_shexp.weight"] = ((shexp, ne), W.GGML[ddt], H.synth_weight(getattr(H, ddt), ne * shexp, 60 + l))
+            if gated:
+                w["ffn_gate_inp_shexp.weight"] = ((ne,), 0, (rng.standard_normal(ne) * 0.05).astype(np.float32))
         per_layer.append(w)
     tensors = [(f"blk.{l}.{k}", shape, gt, np.ascontiguousarray(data).view(np.uint8).tobytes())
                for l, w in enumerate(per_layer) for k, (shape, gt, data) in w.items()]
@@ -46,6 +53,8 @@ def _moe_file(path, rng, *, ne, n_ff, E, K, layers, gdt, ddt, shards=1):
             ("qwen3moe.expert_used_count", W.U32, K), ("qwen3moe.expert_feed_forward_length", W.U32, n_ff),
             ("qwen3moe.attention.layer_norm_rms_epsilon", W.F32, 1e-6),
             ("tokenizer.ggml.tokens", W.ARR, (W.STR, ["<s>", "a", "b"]))]
+    if shexp:
+        meta.append(("qwen3moe.expert_shared_feed_forward_length", W.U32, shexp))
     if shards == 1:
         W.write(path, meta, tensors)
         return path, per_layer
@@ -109,6 +118,38 @@ def test_ffn_sublayer_from_a_gguf_file_matches_the_oracle(be, tmp_path, rows, sh
             tol = 1e-2 if rows >= 32 else 1e-3
             assert H.rel_l2(got - x, want["dst"].reshape(rows, ne)) < tol
             assert H.max_abs(got - x, want["dst"].reshape(rows, ne)) < 2e-3 * max(1.0, float(np.abs(want["dst"]).max()))
+
+
+@pytest.mark.parametrize("rows,gated", [(1, False), (1, True), (4, True), (36, False)])
+def test_ffn_sublayer_with_a_shared_expert_from_a_gguf_file(be, tmp_path, rows, gated):
+    """The shared-expert branch as the model emits it (crates/infr-llama/src/seam/runner.rs:8089-8174):
+    summed in plain, or gated by sigmoid(ffn_gate_inp_shexp . x) through Op::MoeSharedExpertAdd."""
+    ne, n_ff, E, K, sff = 512, 256, 8, 2, 512
+    rng = np.random.default_rng(90 + rows)
+    path, per_layer = _moe_file(tmp_path / "sh.gguf", rng, ne=ne, n_ff=n_ff, E=E, K=K, layers=1, gdt="Q4K", ddt="Q6K",
+                                shexp=sff, gated=gated)
+    x = (rng.standard_normal((rows, ne)) * 2).astype(np.float32)
+    with G.Gguf(path) as g:
+        assert G.moe_hyper(g).shexp_ff == sff
+        layer = G.MoeFfnLayer(be, g, 0, rows)
+        assert layer.gated == gated
+        got = layer.forward(x)
+        layer.free()
+    w = per_layer[0]
+    xn = O.rms_norm(x, w["ffn_norm.weight"][2], 1e-6).reshape(rows, ne)
+    moe = O.moe_ffn(xn, w["ffn_gate_inp.weight"][2], w["ffn_gate_exps.weight"][2], w["ffn_up_exps.weight"][2],
+                    w["ffn_down_exps.weight"][2], ne=ne, n_expert=E, n_used=K, n_ff_exp=n_ff, gate_dtype=H.Q4K,
+                    down_dtype=H.Q6K)["dst"].reshape(rows, ne)
+    og = O.linear(xn, w["ffn_gate_shexp.weight"][2], H.Q4K, ne, sff)
+    ou = O.linear(xn, w["ffn_up_shexp.weight"][2], H.Q4K, ne, sff)
+    sh = O.linear(O.gated_act_rows(og, ou), w["ffn_down_shexp.weight"][2], H.Q6K, sff, ne)
+    if gated:
+        logit = O.linear(xn, w["ffn_gate_inp_shexp.weight"][2], H.F32, ne, 1)
+        want = O.moe_shared_expert_add(moe, sh, logit).reshape(rows, ne)
+    else:
+        want = O.add(moe, sh).reshape(rows, ne)
+    tol = 1e-2 if rows >= 32 else 1e-3
+    assert H.rel_l2(got - x, want) < tol
 
 
 def test_a_file_with_the_wrong_shapes_is_refused(be, tmp_path):
