@@ -1058,3 +1058,54 @@ def test_batched_threshold_is_configurable_and_the_paths_agree():
         finally:
             be2.close()
     assert H.rel_l2(outs["mfma"], outs["gemv"]) < REL_L2_MFMA
+
+
+@pytest.mark.parametrize("rows", [1, 5])
+def test_disabling_op_fusion_changes_the_launches_not_the_bits(rows):
+    """infr_hip_config.disable_op_fusion (the reference keeps the same hatch for its rewrites,
+    crates/infr-core/src/fusion.rs:49-52): one launch per op, identical output bits."""
+    ne, nff, E, K = 512, 256, 8, 2
+    rng = np.random.default_rng(31 + rows)
+    x = rng.standard_normal((rows, ne)).astype(np.float32)
+    nw = (1 + 0.1 * rng.standard_normal(ne)).astype(np.float32)
+    router = (rng.standard_normal((E, ne)) * 0.1).astype(np.float32)
+    eg, eu, ed = _realistic(rng, E, nff, ne, H.Q4K), _realistic(rng, E, nff, ne, H.Q4K), _realistic(rng, E, ne, nff, H.Q6K)
+    wg, wu, wd = _realistic(rng, 1, nff, ne, H.Q4K), _realistic(rng, 1, nff, ne, H.Q4K), _realistic(rng, 1, ne, nff, H.Q6K)
+    outs, names = {}, {}
+    for off in (False, True):
+        be2 = M.Backend(0, disable_op_fusion=off)
+        try:
+            g = M.Graph()
+            xi, nwt = g.input(TensorDesc([rows, ne], DType.F32)), g.weight(TensorDesc([ne], DType.F32))
+            rt = g.weight(TensorDesc([E, ne], DType.F32))
+            egt, eut = g.weight(TensorDesc([E, nff, ne], DType.Q4K)), g.weight(TensorDesc([E, nff, ne], DType.Q4K))
+            edt = g.weight(TensorDesc([E, ne, nff], DType.Q6K))
+            wgt, wut = g.weight(TensorDesc([nff, ne], DType.Q4K)), g.weight(TensorDesc([nff, ne], DType.Q4K))
+            wdt = g.weight(TensorDesc([ne, nff], DType.Q6K))
+            t = lambda n: g.internal(TensorDesc([rows, n], DType.F32))  # noqa: E731
+            xn, moe, gt, ut, at, st, sub = t(ne), t(ne), t(nff), t(nff), t(nff), t(ne), t(ne)
+            yi = g.output(TensorDesc([rows, ne], DType.F32))
+            g.rms_norm(x=xi, weight=nwt, dst=xn, rows=rows, dim=ne, eps=1e-6)
+            g.moe_ffn(x=xn, router=rt, gate_exps=egt, up_exps=eut, down_exps=edt, dst=moe, ne=ne, n_expert=E, n_used=K,
+                      n_ff_exp=nff)
+            g.linear(x=xn, weight=wgt, dst=gt, m=rows, in_f=ne, out_f=nff)
+            g.linear(x=xn, weight=wut, dst=ut, m=rows, in_f=ne, out_f=nff)
+            g.gated_act(gate=gt, up=ut, dst=at, rows=rows, nff=nff)
+            g.linear(x=at, weight=wdt, dst=st, m=rows, in_f=nff, out_f=ne)
+            g.add(a=moe, b=st, dst=sub, n=rows * ne)
+            g.add(a=xi, b=sub, dst=yi, n=rows * ne)
+            keep = []
+            be2.prof_enable(True)
+            outs[off] = M.run_graph(be2, g, [(xi, x), (nwt, nw), (rt, router), (egt, eg), (eut, eu), (edt, ed), (wgt, wg),
+                                             (wut, wu), (wdt, wd)], yi, rows * ne, keep=keep)
+            be2.sync()
+            names[off] = set(be2.prof_read())
+        finally:
+            be2.close()
+    assert np.array_equal(bits(outs[False]), bits(outs[True]))
+    assert {"rms_norm", "add", "gated_act", "linear"} <= names[True]
+    assert "gated_act" not in names[False]
+    if rows == 1:
+        assert names[False] == {"rms_norm_router_logits", "moe_route_gate_up_shared", "moe_down_combine_shared"}
+    else:   # several rows: the dense FFN folds into two launches, the residual Add after it stays a launch
+        assert {"linear_gate_up_act", "linear_add", "add"} <= names[False]
