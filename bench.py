@@ -29,7 +29,7 @@ from moe4all_amd import DType, TensorDesc, synth  # noqa: E402
 HBM_PEAK_GBPS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0   # dense fp16/bf16 matrix-core peak of one MI355X
 SEED0 = 20260101
-N_TOKENS = 8  # distinct activation sets rotated through the steps
+N_TOKENS = 16  # distinct activation sets rotated through the steps
 
 
 def build_stack(be, shape, n_layer, batch, sublayer=False):
