@@ -386,6 +386,109 @@ void launch_units_dt(hipStream_t s, const float* x, const uint8_t* w, size_t row
 
 }  // namespace
 
+namespace {
+
+// Op::Linear on unquantised weights (F16, BF16, F32): lanes read 16 bytes of a weight row at a time against
+// the activation row(s) staged in LDS; the same block / wave / row split as the unit kernel.
+template <int DT, int T>
+__global__ __launch_bounds__(256) void linear_float_kernel(const float* __restrict__ x, const uint8_t* __restrict__ w,
+                                                           size_t row_bytes, int m, int in_f, int out_f, float* dst,
+                                                           const float* addend) {
+    extern __shared__ float lds[];
+    constexpr int E = DT == INFR_F32 ? 4 : 8;   // elements per 16-byte load
+    const int n_chunks = in_f / E;
+    const int pitch = in_f + 4;                  // row pitch in LDS
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int r0 = blockIdx.y * T;
+    for (int idx = tid; idx < T * (in_f >> 2); idx += 256) {
+        const int tr = idx / (in_f >> 2), v = idx - tr * (in_f >> 2);
+        float4 f = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (r0 + tr < m) f = reinterpret_cast<const float4*>(x + (size_t)(r0 + tr) * in_f)[v];
+        reinterpret_cast<float4*>(lds + (size_t)tr * pitch)[v] = f;
+    }
+    __syncthreads();
+    const int row_base = blockIdx.x * kRowsPerBlock;
+    for (int round = 0; round < kRowsPerBlock / (4 * kRowsPerWave); round++) {
+        const int o0 = row_base + (round * 4 + wave) * kRowsPerWave;
+        if (o0 >= out_f) break;
+        float acc[kRowsPerWave][T];
+#pragma unroll
+        for (int a = 0; a < kRowsPerWave; a++)
+#pragma unroll
+            for (int tr = 0; tr < T; tr++) acc[a][tr] = 0.0f;
+        for (int c = lane; c < n_chunks; c += kWave) {
+            float wv[kRowsPerWave][E];
+#pragma unroll
+            for (int a = 0; a < kRowsPerWave; a++) {
+                const int o = o0 + a < out_f ? o0 + a : out_f - 1;
+                const uint4 raw = *reinterpret_cast<const uint4*>(w + (size_t)o * row_bytes + 16 * (size_t)c);
+                const uint32_t d[4] = {raw.x, raw.y, raw.z, raw.w};
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    if constexpr (DT == INFR_F32) {
+                        wv[a][k] = __uint_as_float(d[k]);
+                    } else if constexpr (DT == INFR_BF16) {
+                        wv[a][2 * k] = __uint_as_float(d[k] << 16);
+                        wv[a][2 * k + 1] = __uint_as_float(d[k] & 0xFFFF0000u);
+                    } else {
+                        wv[a][2 * k] = f16_bits_to_f32(d[k] & 0xFFFFu);
+                        wv[a][2 * k + 1] = f16_bits_to_f32(d[k] >> 16);
+                    }
+                }
+            }
+#pragma unroll
+            for (int tr = 0; tr < T; tr++) {
+                const float* xr = lds + (size_t)tr * pitch + E * c;
+#pragma unroll
+                for (int q = 0; q < E / 4; q++) {
+                    const float4 xv = reinterpret_cast<const float4*>(xr)[q];
+#pragma unroll
+                    for (int a = 0; a < kRowsPerWave; a++) {
+                        acc[a][tr] = fmaf(wv[a][4 * q], xv.x, acc[a][tr]);
+                        acc[a][tr] = fmaf(wv[a][4 * q + 1], xv.y, acc[a][tr]);
+                        acc[a][tr] = fmaf(wv[a][4 * q + 2], xv.z, acc[a][tr]);
+                        acc[a][tr] = fmaf(wv[a][4 * q + 3], xv.w, acc[a][tr]);
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int a = 0; a < kRowsPerWave; a++)
+#pragma unroll
+            for (int tr = 0; tr < T; tr++) {
+                const float y = wave_sum(acc[a][tr]);
+                if (lane == 0 && o0 + a < out_f && r0 + tr < m) {
+                    const size_t oi = (size_t)(r0 + tr) * out_f + o0 + a;
+                    dst[oi] = addend ? __fadd_rn(addend[oi], y) : y;
+                }
+            }
+    }
+}
+
+template <int DT, int T>
+void launch_float(hipStream_t s, const float* x, const uint8_t* w, size_t row_bytes, int m, int in_f, int out_f, float* dst,
+                  const float* addend) {
+    static bool attr_set = false;
+    if (!attr_set) {
+        (void)hipFuncSetAttribute((const void*)linear_float_kernel<DT, T>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        attr_set = true;
+    }
+    dim3 grid((out_f + kRowsPerBlock - 1) / kRowsPerBlock, (m + T - 1) / T), block(256);
+    INFR_LAUNCH((linear_float_kernel<DT, T>), grid, block, (size_t)T * (in_f + 4) * sizeof(float), s, x, w, row_bytes, m, in_f,
+                out_f, dst, addend);
+}
+
+template <int DT>
+void launch_float_dt(hipStream_t s, const float* x, const uint8_t* w, size_t row_bytes, int m, int in_f, int out_f, float* dst,
+                     const float* addend) {
+    const size_t budget = 144 * 1024, row = (size_t)(in_f + 4) * sizeof(float);
+    if (m >= 4 && 4 * row <= budget) launch_float<DT, 4>(s, x, w, row_bytes, m, in_f, out_f, dst, addend);
+    else if (m >= 2 && 2 * row <= budget) launch_float<DT, 2>(s, x, w, row_bytes, m, in_f, out_f, dst, addend);
+    else launch_float<DT, 1>(s, x, w, row_bytes, m, in_f, out_f, dst, addend);
+}
+
+}  // namespace
+
 bool linear_units_supported(int dt, int in_f, const void* x) {
     switch (dt) {
         case INFR_Q4_0: case INFR_Q4_1: case INFR_Q5_0: case INFR_Q5_1: case INFR_Q8_0: break;
@@ -405,6 +508,20 @@ bool moe_down_units_supported(const MoeGemvParams& p) {
     return p.y != nullptr && p.rows * p.n_used <= 65535 && linear_units_supported(p.down_dt, p.nff, p.h);
 }
 void launch_moe_down_units(hipStream_t s, const MoeGemvParams& p) { launch_moe_units_any<false>(s, p.down_dt, p); }
+
+// 16-byte loads of the weight rows and of x: in_f a multiple of 8, rows and bases 16-byte aligned.
+bool linear_float_supported(int dt, int in_f, size_t row_bytes, const void* x, const void* w) {
+    if (dt != INFR_F32 && dt != INFR_F16 && dt != INFR_BF16) return false;
+    return in_f >= 8 && in_f % 8 == 0 && (row_bytes & 15) == 0 && (((uintptr_t)x | (uintptr_t)w) & 15) == 0 &&
+           (size_t)(in_f + 4) * sizeof(float) <= 144 * 1024;
+}
+
+void launch_linear_float(hipStream_t s, const float* x, const uint8_t* w, int dt, size_t row_bytes, int m, int in_f,
+                         int out_f, float* dst, const float* addend) {
+    if (dt == INFR_F32) launch_float_dt<INFR_F32>(s, x, w, row_bytes, m, in_f, out_f, dst, addend);
+    else if (dt == INFR_F16) launch_float_dt<INFR_F16>(s, x, w, row_bytes, m, in_f, out_f, dst, addend);
+    else launch_float_dt<INFR_BF16>(s, x, w, row_bytes, m, in_f, out_f, dst, addend);
+}
 
 void launch_linear_units(hipStream_t s, const float* x, const uint8_t* w, int dt, size_t row_bytes, int m, int in_f,
                          int out_f, float* dst, const float* addend) {

@@ -1182,6 +1182,10 @@ void launch_linear(hipStream_t s, const float* x, const uint8_t* w, int dt, size
     else if (dt == INFR_Q6K) done = try_linear<Q6KFmt>(s, x, w, m, in_f, out_f, dst, n_cu, addend);
     else if (dt == INFR_Q8_0) done = try_linear<Q80Fmt>(s, x, w, m, in_f, out_f, dst, n_cu, addend);
     if (done) return;
+    if (linear_float_supported(dt, in_f, row_bytes, x, w)) {
+        launch_linear_float(s, x, w, dt, row_bytes, m, in_f, out_f, dst, addend);
+        return;
+    }
     if (linear_units_supported(dt, in_f, x)) {   // every other affine format, and the shapes the kernels above refuse
         launch_linear_units(s, x, w, dt, row_bytes, m, in_f, out_f, dst, addend);
         return;

@@ -158,6 +158,10 @@ void launch_gated_act(hipStream_t s, const float* gate, const float* up, float* 
 bool linear_units_supported(int dt, int in_f, const void* x);
 void launch_linear_units(hipStream_t s, const float* x, const uint8_t* w, int dt, size_t row_bytes, int m, int in_f,
                          int out_f, float* dst, const float* addend);
+// Op::Linear on F32 / F16 / BF16 weights with 16-byte loads (k_affine.hip).
+bool linear_float_supported(int dt, int in_f, size_t row_bytes, const void* x, const void* w);
+void launch_linear_float(hipStream_t s, const float* x, const uint8_t* w, int dt, size_t row_bytes, int m, int in_f,
+                         int out_f, float* dst, const float* addend);
 // Op::MoeFfn's expert stages on the same units, one block column per (row, rank) pair: h[pair] from x (gate/up),
 // y[pair] from h (down; needs p.y).  The weighted sum over ranks is launch_unbucket_combine's.
 bool moe_gate_up_units_supported(const MoeGemvParams& p);

@@ -714,6 +714,24 @@ def test_linear_sweep_over_every_affine_weight_format(be, m):
             assert H.rel_l2(got, want) < 1e-5, (DType(dt).name, in_f)
 
 
+@pytest.mark.parametrize("dt", [H.F32, H.F16, H.BF16])
+@pytest.mark.parametrize("m,in_f,out_f", [(1, 2048, 96), (3, 4096, 37), (6, 264, 8), (1, 100, 5)])
+def test_linear_on_float_weights(be, dt, m, in_f, out_f):
+    """Unquantised weight matrices (norm-adjacent projections, F16 heads): 16-byte loads when the row pitch
+    allows, the element-wise kernel otherwise (in_f = 100: a 200-byte F16 row)."""
+    rng = np.random.default_rng(in_f + m)
+    w32 = (rng.standard_normal(out_f * in_f) * 0.1).astype(np.float32)
+    raw = w32 if dt == H.F32 else w32.astype(np.float16) if dt == H.F16 else (w32.view(np.uint32) >> 16).astype(np.uint16)
+    x = rng.standard_normal((m, in_f)).astype(np.float32)
+    g = M.Graph()
+    xi, wi = g.input(TensorDesc([m, in_f], DType.F32)), g.weight(TensorDesc([out_f, in_f], DType(dt)))
+    yi = g.output(TensorDesc([m, out_f], DType.F32))
+    g.linear(x=xi, weight=wi, dst=yi, m=m, in_f=in_f, out_f=out_f)
+    got = M.run_graph(be, g, [(xi, x), (wi, raw)], yi, m * out_f).reshape(m, out_f)
+    want = O.linear(x, raw, dt, in_f, out_f)
+    assert H.rel_l2(got, want) < 1e-5
+
+
 @pytest.mark.parametrize("gdt,ddt,rows", [(H.Q5K, H.Q5K, 1), (H.Q4_0, H.Q5_0, 2), (H.Q2K, H.Q3K, 1), (H.Q4_1, H.Q5_1, 3),
                                           (H.Q5K, H.Q6K, 40), (H.Q3K, H.Q2K, 5), (H.Q5_1, H.Q4_0, 1)])
 def test_moe_ffn_with_experts_in_the_other_affine_formats(be, gdt, ddt, rows):
