@@ -100,6 +100,7 @@ struct MoeScratch {
     // batched path (bucketing + grouped GEMMs); the large buffers are shared by all ops of a plan
     bool batched = false;    // >= kBatchedMinRows: grouped GEMMs on the matrix cores
     bool bucketed = false;   // kBucketedMinRows .. : f32-accurate GEMV per (expert, bucket), weights read once per expert
+    bool units_batch = false;   // with bucketed: batches of banks in the other affine formats, unit kernels over the buckets
     int32_t* live_ids = nullptr;  // [pairs] ids with the pairs an expert-parallel band dropped set to -1
     int32_t* offsets = nullptr;   // [n_expert + 1]
     int32_t* pair_src = nullptr;  // [rows * n_used]
@@ -586,6 +587,14 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
                     probe.nff = (int)m.n_ff_exp;
                     bucketed = infr::moe_bucketed_supported(probe);
                 }
+                // banks without a matrix-core decoder: from the batched threshold on, the unit kernels walk the
+                // expert buckets (weights fetched once per chunk of tokens)
+                const bool units_batch = !batched && !bucketed && rows >= min_rows && m.n_used <= 64 &&
+                                         infr::moe_units_batch_supported(c.dt(m.gate_exps),
+                                                                         m.fused_gate_up ? c.dt(m.gate_exps) : c.dt(m.up_exps),
+                                                                         c.dt(m.down_exps), (int)m.ne, (int)m.n_ff_exp);
+                if (units_batch) bucketed = true;
+                plan->moe[oi].units_batch = units_batch;
                 if (bucketed) {
                     arena += round_up(((size_t)m.n_expert + 2) * 4, 256) + 3 * round_up(pairs * 4 + 4, 256);
                     shared += round_up(pairs * m.ne * 4, 256);
@@ -1157,6 +1166,22 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                     }
                     gp.bk_offsets = sc.offsets; gp.bk_pair_src = sc.pair_src; gp.y = sc.y;
                     gp.max_bucket = m.expert_ids == INFR_NO_TENSOR ? rows : pairs;   // given ids may repeat an expert in a row
+                    if (sc.units_batch) {
+                        if ((((uintptr_t)gp.x | (uintptr_t)gp.h | (uintptr_t)gp.y) & 15) != 0)
+                            return fail(INFR_ERR_BACKEND, "MoeFfn: activation rows must be 16-byte aligned");
+                        {
+                            Timed t(be, "moe_gate_up_units_bucketed");
+                            infr::launch_moe_gate_up_units_bucketed(s, gp);
+                        }
+                        {
+                            Timed t(be, "moe_down_units_bucketed");
+                            infr::launch_moe_down_units_bucketed(s, gp);
+                        }
+                        Timed t(be, "moe_unbucket_combine");
+                        infr::launch_unbucket_combine(s, sc.y, sc.slot_pair, sc.weights, rows, (int)m.ne, (int)m.n_used,
+                                                      (int)m.weight_before, gp.dst, 0, nullptr, gp.addend);
+                        break;
+                    }
                     {
                         Timed t(be, "moe_gate_up_bucketed");
                         infr::launch_moe_gate_up_bucketed(s, gp);

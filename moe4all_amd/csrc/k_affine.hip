@@ -333,6 +333,192 @@ __global__ __launch_bounds__(256) void moe_units_kernel(MoeGemvParams p, size_t 
     }
 }
 
+// The (expert, chunk) a block works on when an expert's bucket [offsets[e], offsets[e+1]) is cut into
+// chunks of `chunk` tokens and the chunks of all experts are numbered in order.  Every wave computes it
+// for itself (lanes share out the experts, a prefix sum over the lanes finds the owner); false past the
+// last chunk (the grid is an upper bound).
+__device__ __forceinline__ bool find_chunk(const int32_t* __restrict__ offsets, int n_expert, int chunk, int item, int lane,
+                                           int& e_out, int& p0, int& cnt) {
+    const int epl = (n_expert + 63) >> 6;
+    const int e_lo = lane * epl, e_hi = min(n_expert, e_lo + epl);
+    int mine = 0;
+    for (int e = e_lo; e < e_hi; e++) mine += (offsets[e + 1] - offsets[e] + chunk - 1) / chunk;
+    int incl = mine;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const int o = __shfl_up(incl, d, 64);
+        if (lane >= d) incl += o;
+    }
+    const unsigned long long past = __ballot(incl > item);
+    if (past == 0) return false;
+    const int owner = __ffsll((long long)past) - 1;
+    int rem = item - (__shfl(incl, owner, 64) - __shfl(mine, owner, 64));
+    const int o_lo = owner * epl, o_hi = min(n_expert, o_lo + epl);
+    for (int e = o_lo; e < o_hi; e++) {
+        const int n = offsets[e + 1] - offsets[e];
+        const int nc = (n + chunk - 1) / chunk;
+        if (rem < nc) {
+            e_out = e;
+            p0 = offsets[e] + rem * chunk;
+            cnt = min(chunk, n - rem * chunk);
+            return true;
+        }
+        rem -= nc;
+    }
+    return false;
+}
+
+// Batches: the same two stages over expert buckets.  A block takes one 16-row tile of one expert and up
+// to T tokens of that expert's bucket: the tile's units are decoded once and dotted with each token, so an
+// expert's rows are fetched once per T tokens instead of once per pair.  h and y are in bucket order
+// (position t of the bucket tables), as on the matrix-core path; launch_unbucket_combine maps them back.
+template <int DT, bool GATE_UP, int T>
+__global__ __launch_bounds__(256) void moe_units_bucketed_kernel(MoeGemvParams p, size_t row_bytes, int n_tiles) {
+    extern __shared__ float lds[];
+    const int in_f = GATE_UP ? p.ne : p.nff, out_f = GATE_UP ? p.nff : p.ne;
+    const int n_units = in_f >> 5;
+    float* xs = lds;                                           // [T][n_units][kUnitStride]
+    float* xsum = lds + (size_t)T * n_units * kUnitStride;     // [T][2 * n_units]
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int tile = (int)(blockIdx.x % (unsigned)n_tiles), item = (int)(blockIdx.x / (unsigned)n_tiles);
+    int e, p0, nt;
+    if (!find_chunk(p.bk_offsets, p.n_expert, T, item, lane, e, p0, nt)) return;
+    for (int idx = tid; idx < T * 2 * n_units; idx += 256) {
+        const int tr = idx / (2 * n_units), hu = idx - tr * 2 * n_units;
+        const int pos = p0 + min(tr, nt - 1);
+        const float* xrow = GATE_UP ? p.x + (size_t)(p.bk_pair_src[pos] / p.n_used) * p.ne : p.h + (size_t)pos * p.nff;
+        float4 v[4];
+        float sm = 0.0f;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            v[k] = reinterpret_cast<const float4*>(xrow + 16 * hu)[k];
+            sm += (v[k].x + v[k].y) + (v[k].z + v[k].w);
+        }
+        float* d = xs + ((size_t)tr * n_units + (hu >> 1)) * kUnitStride + 16 * (hu & 1);
+#pragma unroll
+        for (int k = 0; k < 4; k++) reinterpret_cast<float4*>(d)[k] = v[k];
+        xsum[idx] = sm;
+    }
+    __syncthreads();
+    constexpr int M = GATE_UP ? 2 : 1;
+    const uint8_t* base[M];
+    base[0] = (GATE_UP ? p.gate + (size_t)e * p.gate_stride : p.down + (size_t)e * p.down_stride);
+    if constexpr (GATE_UP) base[1] = p.up + (size_t)e * p.up_stride;
+    const int row_base = tile * kRowsPerBlock;
+    for (int round = 0; round < kRowsPerBlock / (4 * kRowsPerWave); round++) {
+        const int o0 = row_base + (round * 4 + wave) * kRowsPerWave;
+        if (o0 >= out_f) break;
+        float acc[kRowsPerWave][M][T];
+#pragma unroll
+        for (int a = 0; a < kRowsPerWave; a++)
+#pragma unroll
+            for (int mi = 0; mi < M; mi++)
+#pragma unroll
+                for (int tr = 0; tr < T; tr++) acc[a][mi][tr] = 0.0f;
+        for (int u = lane; u < n_units; u += kWave) {
+            Unit t[kRowsPerWave][M];
+#pragma unroll
+            for (int a = 0; a < kRowsPerWave; a++) {
+                const int o = o0 + a < out_f ? o0 + a : out_f - 1;
+#pragma unroll
+                for (int mi = 0; mi < M; mi++) load_unit<DT>(base[mi] + (size_t)o * row_bytes, u, t[a][mi]);
+            }
+#pragma unroll
+            for (int tr = 0; tr < T; tr++) {
+                const float* xu = xs + ((size_t)tr * n_units + u) * kUnitStride;
+                float sh[kRowsPerWave][M][2];
+#pragma unroll
+                for (int a = 0; a < kRowsPerWave; a++)
+#pragma unroll
+                    for (int mi = 0; mi < M; mi++) sh[a][mi][0] = sh[a][mi][1] = 0.0f;
+#pragma unroll
+                for (int k = 0; k < 8; k++) {
+                    const float4 xv = reinterpret_cast<const float4*>(xu)[k];
+#pragma unroll
+                    for (int a = 0; a < kRowsPerWave; a++)
+#pragma unroll
+                        for (int mi = 0; mi < M; mi++) {
+                            const uint32_t q = t[a][mi].q[k];
+                            float& v = sh[a][mi][k >> 2];
+                            v = fmaf((float)(q & 0xFFu), xv.x, v);
+                            v = fmaf((float)((q >> 8) & 0xFFu), xv.y, v);
+                            v = fmaf((float)((q >> 16) & 0xFFu), xv.z, v);
+                            v = fmaf((float)(q >> 24), xv.w, v);
+                        }
+                }
+                const float2 xsu = *reinterpret_cast<const float2*>(xsum + (size_t)tr * 2 * n_units + 2 * u);
+#pragma unroll
+                for (int a = 0; a < kRowsPerWave; a++)
+#pragma unroll
+                    for (int mi = 0; mi < M; mi++)
+                        acc[a][mi][tr] += (t[a][mi].sc[0] * sh[a][mi][0] + t[a][mi].mn[0] * xsu.x) +
+                                          (t[a][mi].sc[1] * sh[a][mi][1] + t[a][mi].mn[1] * xsu.y);
+            }
+        }
+#pragma unroll
+        for (int a = 0; a < kRowsPerWave; a++)
+#pragma unroll
+            for (int tr = 0; tr < T; tr++) {
+                float v[M];
+#pragma unroll
+                for (int mi = 0; mi < M; mi++) v[mi] = wave_sum(acc[a][mi][tr]);
+                if (lane == 0 && o0 + a < out_f && tr < nt) {
+                    const int pos = p0 + tr;
+                    if constexpr (GATE_UP) {
+                        if (p.weight_before) {
+                            const float wp = p.weights[p.bk_pair_src[pos]];
+                            v[0] = __fmul_rn(wp, v[0]);
+                            v[1] = __fmul_rn(wp, v[1]);
+                        }
+                        p.h[(size_t)pos * p.nff + o0 + a] = gated_act_fn(p.act, p.has_clamp, p.clamp, v[0], v[1]);
+                    } else {
+                        p.y[(size_t)pos * p.ne + o0 + a] = p.down_scale ? __fmul_rn(v[0], p.down_scale[e]) : v[0];
+                    }
+                }
+            }
+    }
+}
+
+template <int DT, bool GATE_UP, int T>
+void launch_moe_units_bucketed_t(hipStream_t s, const MoeGemvParams& p, int n_pairs) {
+    const int in_f = GATE_UP ? p.ne : p.nff, out_f = GATE_UP ? p.nff : p.ne;
+    int be = 1, bb = 4;
+    block_geometry(DT, &be, &bb);
+    const size_t row_bytes = (size_t)(in_f / be) * bb;
+    static bool attr_set = false;
+    if (!attr_set) {
+        (void)hipFuncSetAttribute((const void*)moe_units_bucketed_kernel<DT, GATE_UP, T>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  160 * 1024);
+        attr_set = true;
+    }
+    const int n_tiles = (out_f + kRowsPerBlock - 1) / kRowsPerBlock;
+    // every expert with tokens has at most one ragged chunk: chunks <= pairs / T + min(experts, pairs)
+    const long items = (long)n_pairs / T + (p.n_expert < n_pairs ? p.n_expert : n_pairs);
+    dim3 grid((unsigned)(items * n_tiles)), block(256);
+    INFR_LAUNCH((moe_units_bucketed_kernel<DT, GATE_UP, T>), grid, block, (size_t)T * (in_f >> 5) * (kUnitStride + 2) * sizeof(float),
+                s, p, row_bytes, n_tiles);
+}
+
+template <int DT, bool GATE_UP>
+void launch_moe_units_bucketed_dt(hipStream_t s, const MoeGemvParams& p, int n_pairs) {
+    const int in_f = GATE_UP ? p.ne : p.nff;
+    const size_t per_token = (size_t)(in_f >> 5) * (kUnitStride + 2) * sizeof(float), budget = 80 * 1024;
+    if (8 * per_token <= budget) launch_moe_units_bucketed_t<DT, GATE_UP, 8>(s, p, n_pairs);
+    else if (4 * per_token <= budget) launch_moe_units_bucketed_t<DT, GATE_UP, 4>(s, p, n_pairs);
+    else launch_moe_units_bucketed_t<DT, GATE_UP, 2>(s, p, n_pairs);
+}
+
+template <bool GATE_UP>
+void launch_moe_units_bucketed_any(hipStream_t s, int dt, const MoeGemvParams& p, int n_pairs) {
+    switch (dt) {
+#define INFR_UNITS(D) case D: launch_moe_units_bucketed_dt<D, GATE_UP>(s, p, n_pairs); break
+        INFR_UNITS(INFR_Q4_0); INFR_UNITS(INFR_Q4_1); INFR_UNITS(INFR_Q5_0); INFR_UNITS(INFR_Q5_1); INFR_UNITS(INFR_Q8_0);
+        INFR_UNITS(INFR_Q2K); INFR_UNITS(INFR_Q3K); INFR_UNITS(INFR_Q4K); INFR_UNITS(INFR_Q5K); INFR_UNITS(INFR_Q6K);
+#undef INFR_UNITS
+        default: break;
+    }
+}
+
 template <int DT, bool GATE_UP>
 void launch_moe_units_dt(hipStream_t s, const MoeGemvParams& p) {
     const int in_f = GATE_UP ? p.ne : p.nff, out_f = GATE_UP ? p.nff : p.ne;
@@ -508,6 +694,20 @@ bool moe_down_units_supported(const MoeGemvParams& p) {
     return p.y != nullptr && p.rows * p.n_used <= 65535 && linear_units_supported(p.down_dt, p.nff, p.h);
 }
 void launch_moe_down_units(hipStream_t s, const MoeGemvParams& p) { launch_moe_units_any<false>(s, p.down_dt, p); }
+
+// x and h rows must be 16-byte aligned: ne and nff are multiples of 32 here, the bases are checked by the caller.
+bool moe_units_batch_supported(int gate_dt, int up_dt, int down_dt, int ne, int nff) {
+    const void* aligned = nullptr;
+    return gate_dt == up_dt && linear_units_supported(gate_dt, ne, aligned) && linear_units_supported(down_dt, nff, aligned) &&
+           (size_t)2 * (ne >> 5) * (kUnitStride + 2) * sizeof(float) <= 144 * 1024 &&
+           (size_t)2 * (nff >> 5) * (kUnitStride + 2) * sizeof(float) <= 144 * 1024;
+}
+void launch_moe_gate_up_units_bucketed(hipStream_t s, const MoeGemvParams& p) {
+    launch_moe_units_bucketed_any<true>(s, p.gate_dt, p, p.rows * p.n_used);
+}
+void launch_moe_down_units_bucketed(hipStream_t s, const MoeGemvParams& p) {
+    launch_moe_units_bucketed_any<false>(s, p.down_dt, p, p.rows * p.n_used);
+}
 
 // 16-byte loads of the weight rows and of x: in_f a multiple of 8, rows and bases 16-byte aligned.
 bool linear_float_supported(int dt, int in_f, size_t row_bytes, const void* x, const void* w) {

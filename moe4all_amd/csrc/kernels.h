@@ -168,6 +168,11 @@ bool moe_gate_up_units_supported(const MoeGemvParams& p);
 void launch_moe_gate_up_units(hipStream_t s, const MoeGemvParams& p);
 bool moe_down_units_supported(const MoeGemvParams& p);
 void launch_moe_down_units(hipStream_t s, const MoeGemvParams& p);
+// Batches on the unit kernels: an expert's rows are fetched once per chunk of tokens of its bucket
+// (p.bk_offsets / p.bk_pair_src from launch_bucket); h and y are written in bucket order.
+bool moe_units_batch_supported(int gate_dt, int up_dt, int down_dt, int ne, int nff);
+void launch_moe_gate_up_units_bucketed(hipStream_t s, const MoeGemvParams& p);
+void launch_moe_down_units_bucketed(hipStream_t s, const MoeGemvParams& p);
 void launch_add(hipStream_t s, const float* a, const float* b, float* dst, uint32_t n);
 // Op::RmsNorm (add = 0) / Op::RmsNormAdd (add = 1); dst may be x.
 void launch_rms_norm(hipStream_t s, const float* x, const float* weight, float* dst, int rows, int dim, float eps, int add);
