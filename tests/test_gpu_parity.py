@@ -1056,6 +1056,86 @@ def test_prefill_chunk_with_skewed_routing_matches_oracle(be, tokens, gdt, ddt):
     plan.free()
 
 
+@pytest.mark.parametrize("gdt,ddt", [(DType.Q4K, DType.Q6K), (DType.Q8_0, DType.Q8_0)])
+def test_prefill_rows_do_not_depend_on_their_neighbours(be, gdt, ddt):
+    """Properties that hold at any size, checked at the full 2048-token chunk of the config-4 shape:
+    a token's output row is a function of that row alone, so (1) shuffling the tokens shuffles the output rows
+    bit for bit although every expert bucket and GEMM tile is composed differently, (2) a prefix of the chunk
+    run on its own gives the bits it gives inside the chunk, and (3) a token repeated in the chunk gives
+    the same row each time."""
+    tokens = 2048
+    s = S.MoeShape("c4", 1, 2048, 128, 8, 768, gdt, ddt)
+    lw = S.LayerWeights(be, s, seed0=17, layer=0, on_device=True)
+    router = be.download(lw.router, dtype=np.float32).reshape(s.n_expert, s.ne).copy()
+    router[:, 0] = S.zipf_bias(s.n_expert, 1.1, 9)
+    be.upload(lw.router, router)
+    x = S.normal(S.stream_seed(18, 0, S.ROLE_X), tokens * s.ne, 1.0).reshape(tokens, s.ne).copy()
+    x[:, 0] = 1.0
+    x[1500] = x[3]          # a repeated token
+    x[77] *= 1.0e3          # rows of very different magnitude share tiles
+    x[78] *= 1.0e-4
+
+    def run(xin):
+        n = xin.shape[0]
+        g, ids = moe_graph(n, s.ne, s.n_expert, s.n_used, s.n_ff, gdt, ddt)
+        plan = be.compile(g)
+        xb, yb = be.buffer_from(xin, M.BufferUsage.Activations), be.alloc(n * s.ne * 4, M.BufferUsage.Readback)
+        bnd = (M.Bindings().bind(ids["x"], xb).bind(ids["router"], lw.router).bind(ids["gate"], lw.gate)
+               .bind(ids["up"], lw.up).bind(ids["down"], lw.down).bind(ids["dst"], yb))
+        be.execute(plan, bnd)
+        out = be.download(yb, n * s.ne * 4, np.float32).reshape(n, s.ne).copy()
+        idx = be.moe_routing(plan, 0)["idx"].copy()
+        plan.free()
+        xb.free()
+        yb.free()
+        return out, idx
+
+    full, idx = run(x)
+    assert np.isfinite(full).all()
+    perm = np.random.default_rng(3).permutation(tokens)
+    shuffled, idx_p = run(np.ascontiguousarray(x[perm]))
+    assert np.array_equal(idx_p, idx[perm])
+    assert np.array_equal(bits(shuffled), bits(full[perm]))
+    head, _ = run(np.ascontiguousarray(x[:700]))
+    assert np.array_equal(bits(head), bits(full[:700]))
+    assert np.array_equal(bits(full[1500]), bits(full[3]))
+
+
+@pytest.mark.parametrize("shape_name", ["c2", "c5"])
+def test_decode_rows_give_the_same_bits_in_any_batch(be, shape_name):
+    """At the full layer shapes: a token row alone (routing inside the gate/up kernel), inside a batch of 8
+    (staged per-token kernels, separate routing launch) and inside a batch of 20 (bucketed GEMV, two tokens of
+    an expert share each weight row) runs the same inner products in the same order, so the three outputs
+    agree bit for bit; so do ids and routing weights."""
+    s = S.CONFIG_2 if shape_name == "c2" else S.MoeShape("c5-routed", 1, 4096, 256, 8, 1536, DType.Q4K, DType.Q6K)
+    lw = S.LayerWeights(be, s, seed0=23, layer=0, on_device=True)
+    x = S.normal(S.stream_seed(24, 0, S.ROLE_X), 20 * s.ne, 1.0).reshape(20, s.ne).copy()
+
+    def run(xin):
+        n = xin.shape[0]
+        g, ids = moe_graph(n, s.ne, s.n_expert, s.n_used, s.n_ff, s.gate_dtype, s.down_dtype)
+        plan = be.compile(g)
+        xb, yb = be.buffer_from(xin, M.BufferUsage.Activations), be.alloc(n * s.ne * 4, M.BufferUsage.Readback)
+        bnd = (M.Bindings().bind(ids["x"], xb).bind(ids["router"], lw.router).bind(ids["gate"], lw.gate)
+               .bind(ids["up"], lw.up).bind(ids["down"], lw.down).bind(ids["dst"], yb))
+        be.execute(plan, bnd)
+        out = be.download(yb, n * s.ne * 4, np.float32).reshape(n, s.ne).copy()
+        r = be.moe_routing(plan, 0)
+        plan.free()
+        xb.free()
+        yb.free()
+        return out, r["idx"].copy(), r["w"].copy()
+
+    full, idx, w = run(x)
+    eight, idx8, w8 = run(np.ascontiguousarray(x[:8]))
+    assert np.array_equal(idx8, idx[:8]) and np.array_equal(bits(w8), bits(w[:8]))
+    assert np.array_equal(bits(eight), bits(full[:8]))
+    for r in (0, 7, 19):
+        one, idx1, w1 = run(np.ascontiguousarray(x[r:r + 1]))
+        assert np.array_equal(idx1[0], idx[r]) and np.array_equal(bits(w1[0]), bits(w[r]))
+        assert np.array_equal(bits(one[0]), bits(full[r])), r
+
+
 def test_batched_threshold_is_configurable_and_the_paths_agree():
     """moe_batched_min_rows moves the switch to the matrix-core path; with it out of reach a 48-row batch
     runs the bucketed f32-accurate kernels and must meet the f32 bar, with it at 1 even two rows take
