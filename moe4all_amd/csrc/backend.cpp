@@ -101,6 +101,7 @@ struct MoeScratch {
     bool batched = false;    // >= kBatchedMinRows: grouped GEMMs on the matrix cores
     bool bucketed = false;   // kBucketedMinRows .. : f32-accurate GEMV per (expert, bucket), weights read once per expert
     bool units_batch = false;   // with bucketed: batches of banks in the other affine formats, unit kernels over the buckets
+    bool units_mfma = false;    // with batched: the grouped GEMMs decode through the 32-element units (any affine format)
     int32_t* live_ids = nullptr;  // [pairs] ids with the pairs an expert-parallel band dropped set to -1
     int32_t* offsets = nullptr;   // [n_expert + 1]
     int32_t* pair_src = nullptr;  // [rows * n_used]
@@ -566,10 +567,17 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
                 const size_t pairs = (size_t)rows * m.n_used;
                 size_t shared = round_up((pairs + rows) * m.n_ff_exp * 4 + 4, 256);   // one more slot per row: see kMoeShared
                 const uint32_t min_rows = be->cfg.moe_batched_min_rows ? be->cfg.moe_batched_min_rows : kBatchedMinRows;
-                const bool batched = rows >= min_rows && m.n_used <= 64 && !m.fused_gate_up &&
-                                     c.dt(m.gate_exps) == c.dt(m.up_exps) &&
-                                     infr::grouped_supported(c.dt(m.gate_exps), (int)m.ne) &&
-                                     infr::grouped_supported(c.dt(m.down_exps), (int)m.n_ff_exp);
+                bool batched = rows >= min_rows && m.n_used <= 64 && !m.fused_gate_up &&
+                               c.dt(m.gate_exps) == c.dt(m.up_exps) &&
+                               infr::grouped_supported(c.dt(m.gate_exps), (int)m.ne) &&
+                               infr::grouped_supported(c.dt(m.down_exps), (int)m.n_ff_exp);
+                // a bank in one of the other affine formats: the same path with the unit-decoder GEMM for all three
+                const bool units_mfma = !batched && rows >= min_rows && m.n_used <= 64 &&
+                                        (m.fused_gate_up || c.dt(m.gate_exps) == c.dt(m.up_exps)) &&
+                                        infr::grouped_units_supported(c.dt(m.gate_exps), (int)m.ne) &&
+                                        infr::grouped_units_supported(c.dt(m.down_exps), (int)m.n_ff_exp);
+                if (units_mfma) batched = true;
+                plan->moe[oi].units_mfma = units_mfma;
                 if (batched) {
                     arena += round_up(((size_t)m.n_expert + 2) * 4, 256) + 3 * round_up(pairs * 4 + 4, 256);
                     shared += round_up((size_t)rows * m.ne * 2, 256) + round_up((size_t)rows * 4, 256) +
@@ -1116,9 +1124,11 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                         }
                         infr::launch_bucket(s, bucket_ids, pairs, (int)n_local, sc.offsets, sc.pair_src, sc.slot_pair);
                     }
+                    // the unit-decoder GEMM reads activations in natural k order, which is Q8_0's
+                    const int a_dt_gu = sc.units_mfma ? INFR_Q8_0 : gp.gate_dt, a_dt_dn = sc.units_mfma ? INFR_Q8_0 : gp.down_dt;
                     {
                         Timed t(be, "rows_to_f16");
-                        infr::launch_rows_to_f16(s, gp.gate_dt, gp.x, rows, (int)m.ne, sc.xh, sc.xs);
+                        infr::launch_rows_to_f16(s, a_dt_gu, gp.x, rows, (int)m.ne, sc.xh, sc.xs);
                     }
                     infr::GroupedParams q{};
                     q.a = sc.xh; q.a_scale = sc.xs; q.offsets = sc.offsets; q.pair_src = sc.pair_src;
@@ -1128,19 +1138,21 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                     q.n_pairs = pairs; q.act = m.act; q.has_clamp = (int)m.has_swiglu_clamp; q.clamp = m.swiglu_clamp;
                     q.weight_before = (int)m.weight_before;
                     {
-                        Timed t(be, "moe_grouped_gate_up");
-                        infr::launch_grouped_gate_up(s, gp.gate_dt, q);
+                        Timed t(be, sc.units_mfma ? "moe_grouped_units_gate_up" : "moe_grouped_gate_up");
+                        if (sc.units_mfma) infr::launch_grouped_units_gate_up(s, gp.gate_dt, q);
+                        else infr::launch_grouped_gate_up(s, gp.gate_dt, q);
                     }
                     {
                         Timed t(be, "rows_to_f16");
-                        infr::launch_rows_to_f16(s, gp.down_dt, sc.h, pairs, (int)m.n_ff_exp, sc.hh, sc.hs);
+                        infr::launch_rows_to_f16(s, a_dt_dn, sc.h, pairs, (int)m.n_ff_exp, sc.hh, sc.hs);
                     }
                     q.a = sc.hh; q.a_scale = sc.hs; q.w0 = gp.down; q.w0_stride = gp.down_stride; q.w1 = nullptr; q.w1_stride = 0;
                     q.down_scale = gp.down_scale; q.out = sc.y; q.K = (int)m.n_ff_exp; q.N = (int)m.ne;
                     q.out_f16 = 1;   // y is written and read once: f16 halves that traffic, hs restores the scale
                     {
-                        Timed t(be, "moe_grouped_down");
-                        infr::launch_grouped_down(s, gp.down_dt, q);
+                        Timed t(be, sc.units_mfma ? "moe_grouped_units_down" : "moe_grouped_down");
+                        if (sc.units_mfma) infr::launch_grouped_units_down(s, gp.down_dt, q);
+                        else infr::launch_grouped_down(s, gp.down_dt, q);
                     }
                     {
                         Timed t(be, "moe_unbucket_combine");

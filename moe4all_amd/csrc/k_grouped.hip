@@ -26,6 +26,7 @@
 
 #include "device_common.h"
 #include "kernels.h"
+#include "units.h"
 
 namespace infr {
 
@@ -848,7 +849,172 @@ void grouped6(hipStream_t s, const GroupedParams& p) {
     INFR_LAUNCH((grouped_mfma6<D, DOWN>), dim3((unsigned)((max_tiles * q.n_tiles_n + 7) & ~7)), dim3(256), grouped6_lds<D>(), s, q);   // whole rounds of the 8 XCDs
 }
 
+// --------------------------------------------------------------------------------------------
+// Grouped GEMM for every affine format through the 32-element unit decoder: the matrix-core path of banks
+// that have no byte-exact LDS layout above.  Same tiles (expert, <= 128 tokens, 128 features with gate and
+// up, or 256 features of down), same accumulator layout and epilogue.  Per 64-k slice a lane decodes ONE
+// unit of each of its two weight rows - lanes 0..31 the slice's first 32 k, lanes 32..63 the second - into
+// four 8-element f16 operand fragments (f32 sc * code + mn, rounded once), so no element is decoded
+// twice; k step ks of the slice contracts elements 8 ks .. 8 ks + 7 of both units.  The activation tile
+// (natural k order) goes through registers into a two-stage LDS ring with the chunk rotation of the
+// kernel above; the next slice's units and activation chunks are requested before the current slice is
+// contracted.
+constexpr int kUStage = kBM * 128;   // 128 tokens x 64 halfs
+
+template <int DT, bool DOWN, int M>
+__device__ __forceinline__ void grouped_units_tile(const GroupedParams& p, const Tile& t, int n0, uint8_t* lds, const float* s_scale) {
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, half = lane >> 5;
+    float16v acc0[M], acc1[M];
+#pragma unroll
+    for (int i = 0; i < M; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc0[i][r] = acc1[i][r] = 0.0f;
+    int be = 1, bb = 4;
+    block_geometry(DT, &be, &bb);
+    const size_t row_bytes = (size_t)(p.K / be) * bb;
+    // the lane's two weight rows
+    const uint8_t* w0;
+    const uint8_t* w1;
+    {
+        const int c = lane & 31;
+        if (DOWN) {
+            const uint8_t* base = p.w0 + (size_t)t.e * p.w0_stride;
+            w0 = base + (size_t)min(n0 + 64 * wave + c, p.N - 1) * row_bytes;
+            w1 = base + (size_t)min(n0 + 64 * wave + 32 + c, p.N - 1) * row_bytes;
+        } else {
+            const int f = min(n0 + 32 * wave + c, p.N - 1);
+            w0 = p.w0 + (size_t)t.e * p.w0_stride + (size_t)f * row_bytes;
+            w1 = p.w1 + (size_t)t.e * p.w1_stride + (size_t)f * row_bytes;
+        }
+    }
+    // the lane's four activation chunks of a slice: token 32 wave + 8 q + lane / 8, LDS position lane & 7
+    const uint8_t* asrc[4];
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const int tok = 32 * wave + 8 * q + (lane >> 3), kg = (lane & 7) ^ ((lane >> 3) & 7);
+        const int pr = t.p0 + min(tok, t.cnt - 1);
+        const size_t src_row = DOWN ? (size_t)pr : (size_t)(p.pair_src[pr] / p.n_used);
+        asrc[q] = reinterpret_cast<const uint8_t*>(p.a + src_row * p.K) + 16 * kg;
+    }
+    uint8_t* const a_dst = lds + wave * 4096 + lane * 16;   // + stage * kUStage + q * 1024
+    const int x7 = lane & 7;
+    int a_off[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) a_off[ks] = (lane & 31) * 128 + (((ks + 4 * half) ^ x7) * 16);
+
+    const int n_slices = p.K / kSlice;
+    Unit u0, u1;
+    uint4 areg[4];
+    load_unit<DT>(w0, half, u0);
+    load_unit<DT>(w1, half, u1);
+#pragma unroll
+    for (int q = 0; q < 4; q++) areg[q] = *reinterpret_cast<const uint4*>(asrc[q]);
+#pragma unroll
+    for (int q = 0; q < 4; q++) *reinterpret_cast<uint4*>(a_dst + q * 1024) = areg[q];
+    __syncthreads();
+    // eight codes of a unit (dwords 2 ks, 2 ks + 1) as f16 values
+    auto frag = [](const Unit& u, int ks) {
+        const float sc = u.sc[ks >> 1], mn = u.mn[ks >> 1];
+        const uint32_t a = u.q[2 * ks], b = u.q[2 * ks + 1];
+        half8 h;
+        h[0] = (_Float16)fmaf(sc, (float)(a & 0xFFu), mn);
+        h[1] = (_Float16)fmaf(sc, (float)((a >> 8) & 0xFFu), mn);
+        h[2] = (_Float16)fmaf(sc, (float)((a >> 16) & 0xFFu), mn);
+        h[3] = (_Float16)fmaf(sc, (float)(a >> 24), mn);
+        h[4] = (_Float16)fmaf(sc, (float)(b & 0xFFu), mn);
+        h[5] = (_Float16)fmaf(sc, (float)((b >> 8) & 0xFFu), mn);
+        h[6] = (_Float16)fmaf(sc, (float)((b >> 16) & 0xFFu), mn);
+        h[7] = (_Float16)fmaf(sc, (float)(b >> 24), mn);
+        return h;
+    };
+    for (int s = 0; s < n_slices; s++) {
+        const bool more = s + 1 < n_slices;
+        Unit v0, v1;
+        if (more) {   // requests for the next slice
+            load_unit<DT>(w0, 2 * (s + 1) + half, v0);
+            load_unit<DT>(w1, 2 * (s + 1) + half, v1);
+#pragma unroll
+            for (int q = 0; q < 4; q++) areg[q] = *reinterpret_cast<const uint4*>(asrc[q] + (size_t)(s + 1) * 128);
+        }
+        const uint8_t* ap = lds + (s & 1) * kUStage;
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) {
+            const half8 b0 = frag(u0, ks), b1 = frag(u1, ks);
+#pragma unroll
+            for (int mi = 0; mi < M; mi++) {
+                const half8 a = *reinterpret_cast<const half8*>(ap + a_off[ks] + mi * 4096);
+                acc0[mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b0, acc0[mi], 0, 0, 0);
+                acc1[mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b1, acc1[mi], 0, 0, 0);
+            }
+        }
+        if (more) {
+            uint8_t* d = a_dst + ((s + 1) & 1) * kUStage;
+#pragma unroll
+            for (int q = 0; q < 4; q++) *reinterpret_cast<uint4*>(d + q * 1024) = areg[q];
+            u0 = v0;
+            u1 = v1;
+        }
+        __syncthreads();   // the stage just written is complete; the stage just read may be overwritten
+    }
+    tile_epilogue<DOWN, M>(p, t, n0, wave, lane, s_scale, acc0, acc1);
+}
+
+template <int DT, bool DOWN>
+__global__ __launch_bounds__(256) void grouped_units_mfma(GroupedParams p) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * kUStage];
+    __shared__ __attribute__((aligned(16))) float s_scale[kBM];
+    const int tid = threadIdx.x, lane = tid & 63;
+    Tile t;
+    int nt;
+    if (!find_item(p.offsets, p.n_expert, p.n_tiles_n, lane, t, nt)) return;
+    constexpr int kBN = DOWN ? 256 : 128;
+    if (tid < kBM) {
+        const int pr = t.p0 + min(tid, t.cnt - 1);
+        s_scale[tid] = p.a_scale[DOWN ? pr : p.pair_src[pr] / p.n_used];
+    }
+    switch ((t.cnt + 31) >> 5) {
+        case 1: grouped_units_tile<DT, DOWN, 1>(p, t, nt * kBN, lds, s_scale); break;
+        case 2: grouped_units_tile<DT, DOWN, 2>(p, t, nt * kBN, lds, s_scale); break;
+        case 3: grouped_units_tile<DT, DOWN, 3>(p, t, nt * kBN, lds, s_scale); break;
+        default: grouped_units_tile<DT, DOWN, 4>(p, t, nt * kBN, lds, s_scale); break;
+    }
+}
+
+template <int DT, bool DOWN>
+void grouped_units(hipStream_t s, const GroupedParams& p) {
+    const int bn = DOWN ? 256 : 128;
+    GroupedParams q = p;
+    q.n_tiles_n = (p.N + bn - 1) / bn;
+    const int max_tiles = p.n_pairs / kBM + (p.n_expert < p.n_pairs ? p.n_expert : p.n_pairs);
+    INFR_LAUNCH((grouped_units_mfma<DT, DOWN>), dim3((unsigned)((max_tiles * q.n_tiles_n + 7) & ~7)), dim3(256), 0, s, q);
+}
+
+template <bool DOWN>
+void grouped_units_any(hipStream_t s, int dt, const GroupedParams& p) {
+    switch (dt) {
+#define INFR_UNITS(D) case D: grouped_units<D, DOWN>(s, p); break
+        INFR_UNITS(INFR_Q4_0); INFR_UNITS(INFR_Q4_1); INFR_UNITS(INFR_Q5_0); INFR_UNITS(INFR_Q5_1); INFR_UNITS(INFR_Q8_0);
+        INFR_UNITS(INFR_Q2K); INFR_UNITS(INFR_Q3K); INFR_UNITS(INFR_Q4K); INFR_UNITS(INFR_Q5K); INFR_UNITS(INFR_Q6K);
+#undef INFR_UNITS
+        default: break;
+    }
+}
+
 }  // namespace
+
+// The unit-decoder grouped GEMM: any affine format, contraction length a whole number of 64-k slices
+// (and of the format's blocks).  Its activations come from launch_rows_to_f16 in natural k order (ask it
+// for a format without an LDS layout of its own, e.g. INFR_Q5K).
+bool grouped_units_supported(int dt, int k) {
+    if (k <= 0 || k % kSlice != 0) return false;
+    switch (dt) {
+        case INFR_Q4_0: case INFR_Q4_1: case INFR_Q5_0: case INFR_Q5_1: case INFR_Q8_0: return true;
+        case INFR_Q2K: case INFR_Q3K: case INFR_Q4K: case INFR_Q5K: case INFR_Q6K: return k % 256 == 0;
+        default: return false;
+    }
+}
+void launch_grouped_units_gate_up(hipStream_t s, int dt, const GroupedParams& p) { grouped_units_any<false>(s, dt, p); }
+void launch_grouped_units_down(hipStream_t s, int dt, const GroupedParams& p) { grouped_units_any<true>(s, dt, p); }
 
 bool grouped_supported(int dt, int k) {
     // the k loop runs in groups of four 64-element slices (one K-quant super-block)

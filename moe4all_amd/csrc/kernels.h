@@ -125,6 +125,10 @@ void launch_rows_to_f16(hipStream_t s, int weight_dt, const float* src, int rows
 void launch_mask_dropped_pairs(hipStream_t s, const int32_t* ids, const float* weights, int n_pairs, int32_t* out);
 void launch_bucket(hipStream_t s, const int32_t* ids, int n_pairs, int n_expert, int32_t* offsets, int32_t* pair_src,
                    int32_t* slot_pair);
+// The same GEMMs for any affine format through the 32-element unit decoder; activations (p.a) in natural k order.
+bool grouped_units_supported(int dt, int k);
+void launch_grouped_units_gate_up(hipStream_t s, int dt, const GroupedParams& p);
+void launch_grouped_units_down(hipStream_t s, int dt, const GroupedParams& p);
 void launch_grouped_gate_up(hipStream_t s, int dt, const GroupedParams& p);
 void launch_grouped_down(hipStream_t s, int dt, const GroupedParams& p);
 // identity != 0: y is in flat (row, rank) order and slot_pair only flags invalid pairs (< 0); a null slot_pair

@@ -58,6 +58,20 @@ def synth_weight(dtype: int, n_elem: int, seed: int) -> np.ndarray:
     return blk.reshape(-1)
 
 
+def centred_weight(dtype: int, n_elem: int, seed: int, band: float = 0.02) -> np.ndarray:
+    """synth_weight with the f16 scale fields chosen so that random codes decode to values of mean ~0 and
+    magnitude ~band, like trained weights: the min term of the formats that have one cancels the mean of
+    the scaled codes (Q4_1: m = -7.5 d; Q5_1: -15.5 d; Q2_K: dmin = 1.5 d; Q4_K, Q5_K: dmin = mean code * d)."""
+    blk = synth_weight(dtype, n_elem, seed).reshape(-1, BLOCK[dtype][1])
+    # (d, second scale) per format; code ranges: q4 0..15, q5 0..31, 6-bit sub-scales mean 31.5, 4-bit 7.5
+    d2 = {Q4_0: (band / 4,), Q5_0: (band / 8,), Q8_0: (band / 64,), Q4_1: (band / 4, -7.5 * band / 4),
+          Q5_1: (band / 8, -15.5 * band / 8), Q2K: (band / 8, 1.5 * band / 8), Q3K: (band / 32,),
+          Q4K: (band / 128, 7.5 * band / 128), Q5K: (band / 256, 15.5 * band / 256), Q6K: (band / 1024,)}[dtype]
+    for off, v in zip(F16_SLOTS[dtype], d2):
+        blk[:, off:off + 2] = f16_bytes(v)
+    return blk.reshape(-1)
+
+
 def rand_f32(n: int, seed: int) -> np.ndarray:
     """crates/infr-metal/tests/parity.rs:15-25: 64-bit LCG, top 24 bits -> [-1, 1)."""
     out = np.empty(n, np.float32)

@@ -732,19 +732,25 @@ def test_linear_on_float_weights(be, dt, m, in_f, out_f):
     assert H.rel_l2(got, want) < 1e-5
 
 
-@pytest.mark.parametrize("gdt,ddt,rows", [(H.Q5K, H.Q5K, 1), (H.Q4_0, H.Q5_0, 2), (H.Q2K, H.Q3K, 1), (H.Q4_1, H.Q5_1, 3),
-                                          (H.Q5K, H.Q6K, 40), (H.Q3K, H.Q2K, 5), (H.Q5_1, H.Q4_0, 1), (H.Q4_0, H.Q4_1, 77),
-                                          (H.Q5K, H.Q5K, 300)])
-def test_moe_ffn_with_experts_in_the_other_affine_formats(be, gdt, ddt, rows):
-    """Expert banks in formats without an integer-dot kernel run on the 32-element-unit kernels, one
-    block column per (row, rank) pair at every batch size (no matrix-core path for them): same
-    routing, same tolerance."""
-    ne, nff, E, K = 512, 256, 8, 3
-    rng = np.random.default_rng(gdt * 17 + ddt)
+@pytest.mark.parametrize("gdt,ddt,rows,ne,nff", [
+    (H.Q5K, H.Q5K, 1, 512, 256), (H.Q4_0, H.Q5_0, 2, 512, 256), (H.Q2K, H.Q3K, 1, 512, 256), (H.Q4_1, H.Q5_1, 3, 512, 256),
+    (H.Q3K, H.Q2K, 5, 512, 256), (H.Q5_1, H.Q4_0, 1, 512, 256),
+    (H.Q5K, H.Q6K, 40, 512, 256), (H.Q4_0, H.Q4_1, 77, 512, 256), (H.Q5K, H.Q5K, 300, 512, 256), (H.Q2K, H.Q3K, 130, 256, 512),
+    (H.Q5_0, H.Q5_1, 64, 192, 320), (H.Q8_0, H.Q4_0, 33, 2048, 64),
+    (H.Q4_0, H.Q5_0, 40, 480, 96), (H.Q4_1, H.Q4_1, 70, 96, 32)])
+def test_moe_ffn_with_experts_in_the_other_affine_formats(be, gdt, ddt, rows, ne, nff):
+    """Expert banks in formats without an integer-dot kernel.  Up to 31 rows: the 32-element-unit GEMV kernels,
+    one block column per (row, rank) pair (f32, bar 1e-3).  From 32 rows: bucketing + the unit-decoder grouped
+    GEMM on the matrix cores (f16 operands, bar 1e-2) when both contraction lengths are whole 64-k slices,
+    otherwise the unit GEMV over the expert buckets (f32).  Same routing everywhere."""
+    E, K = 8, 3
+    rng = np.random.default_rng(gdt * 17 + ddt + rows)
     x = rng.standard_normal((rows, ne)).astype(np.float32)
+    if rows > 4:
+        x[rows // 2] *= 2.0e4    # far outside the f16 range: the per-row scale must absorb it
     router = (rng.standard_normal((E, ne)) * 0.1).astype(np.float32)
-    gate, up = H.synth_weight(gdt, E * nff * ne, 1), H.synth_weight(gdt, E * nff * ne, 2)
-    down = H.synth_weight(ddt, E * ne * nff, 3)
+    gate, up = H.centred_weight(gdt, E * nff * ne, 1), H.centred_weight(gdt, E * nff * ne, 2)
+    down = H.centred_weight(ddt, E * ne * nff, 3)
     g, ids = moe_graph(rows, ne, E, K, nff, DType(gdt), DType(ddt))
     keep = []
     got = M.run_graph(be, g, [(ids["x"], x), (ids["router"], router), (ids["gate"], gate), (ids["up"], up),
@@ -752,13 +758,20 @@ def test_moe_ffn_with_experts_in_the_other_affine_formats(be, gdt, ddt, rows):
     routing = be.moe_routing(keep[0], 0)
     want = O.moe_ffn(x, router, gate, up, down, ne=ne, n_expert=E, n_used=K, n_ff_exp=nff, gate_dtype=gdt, down_dtype=ddt)
     assert np.array_equal(routing["idx"], want["idx"])
-    assert H.rel_l2(got, want["dst"].reshape(rows, ne)) < REL_L2
     be.prof_enable(True)
     be.execute(keep[0], keep[1])
     be.sync()
     names = set(be.prof_read())
     be.prof_enable(False)
-    if rows >= 32:   # batches walk the expert buckets
+    mfma = rows >= 32 and ne % 64 == 0 and nff % 64 == 0
+    wd = want["dst"].reshape(rows, ne)
+    for r in range(rows):   # per row: a row scaled by 2e4 must not drown the others
+        assert H.rel_l2(got[r], wd[r]) < (REL_L2_MFMA if mfma else REL_L2), r
+    if mfma:
+        assert {"moe_grouped_units_gate_up", "moe_grouped_units_down", "moe_unbucket_combine"} <= names
+        b = be.moe_bucketing(keep[0], 0)
+        _check_bucketing(b, want, E)
+    elif rows >= 32:   # batches walk the expert buckets on the f32 unit kernels
         assert {"moe_gate_up_units_bucketed", "moe_down_units_bucketed", "moe_unbucket_combine"} <= names
     else:
         assert "moe_gate_up_units" in names and ("moe_down_units" in names or ddt == H.Q6K)
