@@ -48,6 +48,8 @@ constexpr uint32_t kBatchedMinRows = 32;
 // Token rows from which a decode batch is bucketed by expert so that each selected expert's rows are
 // read from HBM once (same f32-accurate inner product as the per-token kernels).
 constexpr uint32_t kBucketedMinRows = 16;
+// Token rows from which a dense Op::Linear runs as one bucket of the grouped GEMMs.
+constexpr uint32_t kLinearBatchedMinRows = 128;
 
 bool geometry(int dtype, int* elems, int* bytes) {
     switch (dtype) {
@@ -123,6 +125,13 @@ struct infr_hip_plan {
     void* arena = nullptr;             // Internal tensors + per-op scratch
     size_t arena_bytes = 0;
     std::vector<MoeScratch> moe;       // per op (valid for MoeFfn ops)
+    // Op::Linear with a batch of rows on the matrix cores: the rows are one bucket of the grouped GEMM.
+    struct LinearBatch {
+        int mode = 0;                  // 0: GEMV kernels; 1: grouped_mfma6 (Q4_K/Q6_K/Q8_0); 2: unit-decoder GEMM
+        size_t offsets_off = 0;        // arena offset of the bucket table {0, m}
+    };
+    std::vector<LinearBatch> lin;      // per op (valid for Linear ops)
+    _Float16* lin_xh = nullptr;        // shared by all ops of a plan: f16 rows, then their scales
     int last_moe_op = -1;
     // Launch fusion of the dense SwiGLU FFN the reference emits beside the routed experts
     // (crates/infr-llama/src/runner.rs:8116-8174: Linear gate, Linear up, GatedAct, Linear down, Add).
@@ -468,6 +477,7 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
     plan->numel.resize(g->n_tensors);
     plan->internal_off.assign(g->n_tensors, (size_t)-1);
     plan->moe.resize(g->n_ops);
+    plan->lin.resize(g->n_ops);
     auto bail = [&](infr_status st, const std::string& m) {
         delete plan;
         return fail(st, "%s", m.c_str());
@@ -627,6 +637,25 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
                 if (c.n(l.weight) % l.in_f != 0 || l.w_off % l.in_f != 0 ||
                     (uint64_t)l.w_off / l.in_f + l.out_f > c.n(l.weight) / l.in_f)
                     c.set(INFR_ERR_INVALID, "Linear: w_off/out_f select rows outside the weight tensor");
+                if (c.st == INFR_OK) {
+                    // a batch of rows (prefill): f16 operands on the matrix cores, as Op::MoeFfn does from the same row count
+                    // (one bucket means ceil(m / 128) x ceil(out_f / 256) tiles in all: below about a tile of rows the
+                    // GEMV kernels, which spread over the output rows, are faster)
+                    const uint32_t min_rows = be->cfg.moe_batched_min_rows ? be->cfg.moe_batched_min_rows : kLinearBatchedMinRows;
+                    const int dt = c.dt(l.weight);
+                    int mode = 0;
+                    if (l.m >= min_rows && l.m <= (1u << 24)) {
+                        if (infr::grouped_supported(dt, (int)l.in_f)) mode = 1;
+                        else if (infr::grouped_units_supported(dt, (int)l.in_f)) mode = 2;
+                    }
+                    plan->lin[oi].mode = mode;
+                    if (mode) {
+                        plan->lin[oi].offsets_off = arena;
+                        arena += 256;
+                        const size_t shared = round_up((size_t)l.m * l.in_f * 2, 256) + round_up((size_t)l.m * 4, 256);
+                        if (shared > shared_need) shared_need = shared;
+                    }
+                }
                 break;
             }
             case INFR_OP_GATED_ACT: {
@@ -772,6 +801,7 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
             if (plan->fuse[oi].kind != infr_hip_plan::kPlain || plan->ops[oi].kind != INFR_OP_LINEAR) continue;
             const infr_op_linear& l1 = plan->ops[oi].u.linear;
             if (l1.m == 0) continue;
+            if (plan->lin[oi].mode) continue;   // a batch on the matrix cores: the epilogues there take no second operand
             // Linear, Linear, GatedAct
             if (oi + 2 < g->n_ops && plan->ops[oi + 1].kind == INFR_OP_LINEAR && plan->ops[oi + 2].kind == INFR_OP_GATED_ACT) {
                 const infr_op_linear& l2 = plan->ops[oi + 1].u.linear;
@@ -920,6 +950,18 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
     }
     plan->zero_ids = (int32_t*)((char*)plan->arena + zero_off);   // stays zero: the arena is zero-filled and nothing writes here
     if (plan->arena) infr::launch_fill_zero(be->stream, plan->arena, arena);
+    for (uint32_t oi = 0; oi < g->n_ops; oi++) {
+        if (plan->ops[oi].kind != INFR_OP_LINEAR || !plan->lin[oi].mode) continue;
+        const infr_op_linear& l = plan->ops[oi].u.linear;
+        plan->lin_xh = (_Float16*)((char*)plan->arena + shared_off);
+        const int32_t table[2] = {0, (int32_t)l.m};
+        e = hipMemcpyAsync((char*)plan->arena + plan->lin[oi].offsets_off, table, sizeof table, hipMemcpyHostToDevice, be->stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(be->stream);   // `table` is on this stack frame
+        if (e != hipSuccess) {
+            hipFree(plan->arena);
+            return bail(INFR_ERR_BACKEND, std::string("compile: bucket table upload failed: ") + hipGetErrorString(e));
+        }
+    }
     *out = plan;
     return INFR_OK;
 }
@@ -1277,6 +1319,26 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                 geometry(plan->tensors[l.weight].dtype, &we, &wb);
                 size_t row_bytes = (size_t)(l.in_f / we) * wb;
                 const uint8_t* w = (const uint8_t*)ptr[l.weight] + (size_t)(l.w_off / l.in_f) * row_bytes;
+                if (plan->lin[oi].mode) {
+                    const int dt = plan->tensors[l.weight].dtype, mode = plan->lin[oi].mode;
+                    _Float16* xh = plan->lin_xh;
+                    float* xs = (float*)((char*)xh + round_up((size_t)l.m * l.in_f * 2, 256));
+                    {
+                        Timed t(be, "rows_to_f16");
+                        // the unit-decoder GEMM reads activations in natural k order, which is Q8_0's
+                        infr::launch_rows_to_f16(s, mode == 2 ? INFR_Q8_0 : dt, (const float*)ptr[l.x], (int)l.m, (int)l.in_f, xh, xs);
+                    }
+                    infr::GroupedParams q{};
+                    q.a = xh; q.a_scale = xs;
+                    q.offsets = (const int32_t*)((const char*)plan->arena + plan->lin[oi].offsets_off);
+                    q.w0 = w; q.w0_stride = 0;
+                    q.out = (float*)ptr[l.dst];
+                    q.K = (int)l.in_f; q.N = (int)l.out_f; q.n_expert = 1; q.n_used = 1; q.n_pairs = (int)l.m;
+                    Timed t(be, mode == 2 ? "linear_grouped_units" : "linear_grouped");
+                    if (mode == 2) infr::launch_grouped_units_down(s, dt, q);
+                    else infr::launch_grouped_down(s, dt, q);
+                    break;
+                }
                 Timed t(be, "linear");
                 infr::launch_linear(s, (const float*)ptr[l.x], w, plan->tensors[l.weight].dtype, row_bytes, (int)l.m,
                                     (int)l.in_f, (int)l.out_f, (float*)ptr[l.dst], n_cu);

@@ -732,6 +732,38 @@ def test_linear_on_float_weights(be, dt, m, in_f, out_f):
     assert H.rel_l2(got, want) < 1e-5
 
 
+@pytest.mark.parametrize("dt,m,in_f,out_f", [(H.Q4K, 140, 512, 100), (H.Q6K, 300, 768, 2048), (H.Q8_0, 129, 2048, 256),
+                                             (H.Q5K, 128, 512, 96), (H.Q4_0, 200, 192, 300), (H.Q3K, 133, 256, 40),
+                                             (H.Q4K, 2048, 4096, 1536), (H.Q4_1, 150, 96, 64), (H.F16, 170, 256, 64),
+                                             (H.Q4K, 100, 512, 64)])
+def test_linear_with_a_batch_of_rows_runs_on_the_matrix_cores(be, dt, m, in_f, out_f):
+    """Op::Linear from 128 rows on (a prefill chunk through a dense projection or the shared expert): the rows
+    are one bucket of the grouped GEMMs, f16 operands with a power-of-two scale per row, bar 1e-2 per row.
+    Shapes the GEMMs do not take (a width that is no whole 64-k slice, unquantised weights) stay on the f32 kernels."""
+    rng = np.random.default_rng(m + in_f)
+    x = rng.standard_normal((m, in_f)).astype(np.float32)
+    x[m // 2] *= 3.0e4
+    x[m // 3] *= 1.0e-5
+    if dt == H.F16:
+        raw = (rng.standard_normal(out_f * in_f) * 0.02).astype(np.float16)
+    else:
+        raw = H.centred_weight(dt, out_f * in_f, 5)
+    g = M.Graph()
+    xi, wi = g.input(TensorDesc([m, in_f], DType.F32)), g.weight(TensorDesc([out_f, in_f], DType(dt)))
+    yi = g.output(TensorDesc([m, out_f], DType.F32))
+    g.linear(x=xi, weight=wi, dst=yi, m=m, in_f=in_f, out_f=out_f)
+    be.prof_enable(True)
+    got = M.run_graph(be, g, [(xi, x), (wi, raw)], yi, m * out_f).reshape(m, out_f)
+    be.sync()
+    names = set(be.prof_read())
+    be.prof_enable(False)
+    want = O.linear(x, raw, dt, in_f, out_f)
+    mfma = dt != H.F16 and in_f % 64 == 0 and m >= 128
+    assert (("linear_grouped" in names or "linear_grouped_units" in names) and "linear" not in names) if mfma else names == {"linear"}
+    for r in range(m):
+        assert H.rel_l2(got[r], want[r]) < (REL_L2_MFMA if mfma else 1e-5), r
+
+
 @pytest.mark.parametrize("gdt,ddt,rows,ne,nff", [
     (H.Q5K, H.Q5K, 1, 512, 256), (H.Q4_0, H.Q5_0, 2, 512, 256), (H.Q2K, H.Q3K, 1, 512, 256), (H.Q4_1, H.Q5_1, 3, 512, 256),
     (H.Q3K, H.Q2K, 5, 512, 256), (H.Q5_1, H.Q4_0, 1, 512, 256),
