@@ -861,6 +861,72 @@ void grouped6(hipStream_t s, const GroupedParams& p) {
 // contracted.
 constexpr int kUStage = kBM * 128;   // 128 tokens x 64 halfs
 
+// The 32 k of one weight row that a lane contracts in a slice, and its four 8-element f16 fragments.
+template <int DT>
+struct WSlice {
+    Unit u;
+    __device__ __forceinline__ void load(const uint8_t* __restrict__ row, int idx) { load_unit<DT>(row, idx, u); }
+    __device__ __forceinline__ half8 frag(int ks) const {
+        const float sc = u.sc[ks >> 1], mn = u.mn[ks >> 1];
+        const uint32_t a = u.q[2 * ks], b = u.q[2 * ks + 1];
+        half8 h;
+        h[0] = (_Float16)fmaf(sc, (float)(a & 0xFFu), mn);
+        h[1] = (_Float16)fmaf(sc, (float)((a >> 8) & 0xFFu), mn);
+        h[2] = (_Float16)fmaf(sc, (float)((a >> 16) & 0xFFu), mn);
+        h[3] = (_Float16)fmaf(sc, (float)(a >> 24), mn);
+        h[4] = (_Float16)fmaf(sc, (float)(b & 0xFFu), mn);
+        h[5] = (_Float16)fmaf(sc, (float)((b >> 8) & 0xFFu), mn);
+        h[6] = (_Float16)fmaf(sc, (float)((b >> 16) & 0xFFu), mn);
+        h[7] = (_Float16)fmaf(sc, (float)(b >> 24), mn);
+        return h;
+    }
+};
+// Unquantised weights: F16 rows are the fragments as they lie in memory; BF16 / F32 are rounded to f16.
+template <>
+struct WSlice<INFR_F16> {
+    uint4 v[4];
+    __device__ __forceinline__ void load(const uint8_t* __restrict__ row, int idx) {
+#pragma unroll
+        for (int k = 0; k < 4; k++) v[k] = ldu<uint4>(row + (size_t)idx * 64 + 16 * k);
+    }
+    __device__ __forceinline__ half8 frag(int ks) const { return __builtin_bit_cast(half8, v[ks]); }
+};
+template <>
+struct WSlice<INFR_BF16> {
+    uint4 v[4];
+    __device__ __forceinline__ void load(const uint8_t* __restrict__ row, int idx) {
+#pragma unroll
+        for (int k = 0; k < 4; k++) v[k] = ldu<uint4>(row + (size_t)idx * 64 + 16 * k);
+    }
+    __device__ __forceinline__ half8 frag(int ks) const {
+        const uint32_t d[4] = {v[ks].x, v[ks].y, v[ks].z, v[ks].w};
+        half8 h;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            h[2 * k] = (_Float16)__uint_as_float(d[k] << 16);
+            h[2 * k + 1] = (_Float16)__uint_as_float(d[k] & 0xFFFF0000u);
+        }
+        return h;
+    }
+};
+template <>
+struct WSlice<INFR_F32> {
+    uint4 v[8];
+    __device__ __forceinline__ void load(const uint8_t* __restrict__ row, int idx) {
+#pragma unroll
+        for (int k = 0; k < 8; k++) v[k] = ldu<uint4>(row + (size_t)idx * 128 + 16 * k);
+    }
+    __device__ __forceinline__ half8 frag(int ks) const {
+        const uint4 a = v[2 * ks], b = v[2 * ks + 1];
+        half8 h;
+        h[0] = (_Float16)__uint_as_float(a.x); h[1] = (_Float16)__uint_as_float(a.y);
+        h[2] = (_Float16)__uint_as_float(a.z); h[3] = (_Float16)__uint_as_float(a.w);
+        h[4] = (_Float16)__uint_as_float(b.x); h[5] = (_Float16)__uint_as_float(b.y);
+        h[6] = (_Float16)__uint_as_float(b.z); h[7] = (_Float16)__uint_as_float(b.w);
+        return h;
+    }
+};
+
 template <int DT, bool DOWN, int M>
 __device__ __forceinline__ void grouped_units_tile(const GroupedParams& p, const Tile& t, int n0, uint8_t* lds, const float* s_scale) {
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, half = lane >> 5;
@@ -903,43 +969,28 @@ __device__ __forceinline__ void grouped_units_tile(const GroupedParams& p, const
     for (int ks = 0; ks < 4; ks++) a_off[ks] = (lane & 31) * 128 + (((ks + 4 * half) ^ x7) * 16);
 
     const int n_slices = p.K / kSlice;
-    Unit u0, u1;
+    WSlice<DT> u0, u1;
     uint4 areg[4];
-    load_unit<DT>(w0, half, u0);
-    load_unit<DT>(w1, half, u1);
+    u0.load(w0, half);
+    u1.load(w1, half);
 #pragma unroll
     for (int q = 0; q < 4; q++) areg[q] = *reinterpret_cast<const uint4*>(asrc[q]);
 #pragma unroll
     for (int q = 0; q < 4; q++) *reinterpret_cast<uint4*>(a_dst + q * 1024) = areg[q];
     __syncthreads();
-    // eight codes of a unit (dwords 2 ks, 2 ks + 1) as f16 values
-    auto frag = [](const Unit& u, int ks) {
-        const float sc = u.sc[ks >> 1], mn = u.mn[ks >> 1];
-        const uint32_t a = u.q[2 * ks], b = u.q[2 * ks + 1];
-        half8 h;
-        h[0] = (_Float16)fmaf(sc, (float)(a & 0xFFu), mn);
-        h[1] = (_Float16)fmaf(sc, (float)((a >> 8) & 0xFFu), mn);
-        h[2] = (_Float16)fmaf(sc, (float)((a >> 16) & 0xFFu), mn);
-        h[3] = (_Float16)fmaf(sc, (float)(a >> 24), mn);
-        h[4] = (_Float16)fmaf(sc, (float)(b & 0xFFu), mn);
-        h[5] = (_Float16)fmaf(sc, (float)((b >> 8) & 0xFFu), mn);
-        h[6] = (_Float16)fmaf(sc, (float)((b >> 16) & 0xFFu), mn);
-        h[7] = (_Float16)fmaf(sc, (float)(b >> 24), mn);
-        return h;
-    };
     for (int s = 0; s < n_slices; s++) {
         const bool more = s + 1 < n_slices;
-        Unit v0, v1;
+        WSlice<DT> v0, v1;
         if (more) {   // requests for the next slice
-            load_unit<DT>(w0, 2 * (s + 1) + half, v0);
-            load_unit<DT>(w1, 2 * (s + 1) + half, v1);
+            v0.load(w0, 2 * (s + 1) + half);
+            v1.load(w1, 2 * (s + 1) + half);
 #pragma unroll
             for (int q = 0; q < 4; q++) areg[q] = *reinterpret_cast<const uint4*>(asrc[q] + (size_t)(s + 1) * 128);
         }
         const uint8_t* ap = lds + (s & 1) * kUStage;
 #pragma unroll
         for (int ks = 0; ks < 4; ks++) {
-            const half8 b0 = frag(u0, ks), b1 = frag(u1, ks);
+            const half8 b0 = u0.frag(ks), b1 = u1.frag(ks);
 #pragma unroll
             for (int mi = 0; mi < M; mi++) {
                 const half8 a = *reinterpret_cast<const half8*>(ap + a_off[ks] + mi * 4096);
@@ -995,6 +1046,7 @@ void grouped_units_any(hipStream_t s, int dt, const GroupedParams& p) {
 #define INFR_UNITS(D) case D: grouped_units<D, DOWN>(s, p); break
         INFR_UNITS(INFR_Q4_0); INFR_UNITS(INFR_Q4_1); INFR_UNITS(INFR_Q5_0); INFR_UNITS(INFR_Q5_1); INFR_UNITS(INFR_Q8_0);
         INFR_UNITS(INFR_Q2K); INFR_UNITS(INFR_Q3K); INFR_UNITS(INFR_Q4K); INFR_UNITS(INFR_Q5K); INFR_UNITS(INFR_Q6K);
+        INFR_UNITS(INFR_F16); INFR_UNITS(INFR_BF16); INFR_UNITS(INFR_F32);
 #undef INFR_UNITS
         default: break;
     }
@@ -1010,6 +1062,7 @@ bool grouped_units_supported(int dt, int k) {
     switch (dt) {
         case INFR_Q4_0: case INFR_Q4_1: case INFR_Q5_0: case INFR_Q5_1: case INFR_Q8_0: return true;
         case INFR_Q2K: case INFR_Q3K: case INFR_Q4K: case INFR_Q5K: case INFR_Q6K: return k % 256 == 0;
+        case INFR_F16: case INFR_BF16: case INFR_F32: return true;   // rounded to f16 (weights beyond 65504 would not fit)
         default: return false;
     }
 }

@@ -735,17 +735,19 @@ def test_linear_on_float_weights(be, dt, m, in_f, out_f):
 @pytest.mark.parametrize("dt,m,in_f,out_f", [(H.Q4K, 140, 512, 100), (H.Q6K, 300, 768, 2048), (H.Q8_0, 129, 2048, 256),
                                              (H.Q5K, 128, 512, 96), (H.Q4_0, 200, 192, 300), (H.Q3K, 133, 256, 40),
                                              (H.Q4K, 2048, 4096, 1536), (H.Q4_1, 150, 96, 64), (H.F16, 170, 256, 64),
+                                             (H.BF16, 130, 320, 100), (H.F32, 260, 128, 300), (H.F16, 140, 100, 64),
                                              (H.Q4K, 100, 512, 64)])
 def test_linear_with_a_batch_of_rows_runs_on_the_matrix_cores(be, dt, m, in_f, out_f):
     """Op::Linear from 128 rows on (a prefill chunk through a dense projection or the shared expert): the rows
     are one bucket of the grouped GEMMs, f16 operands with a power-of-two scale per row, bar 1e-2 per row.
-    Shapes the GEMMs do not take (a width that is no whole 64-k slice, unquantised weights) stay on the f32 kernels."""
+    Unquantised weights are rounded to f16 operands.  Widths that are no whole 64-k slice stay on the f32 kernels."""
     rng = np.random.default_rng(m + in_f)
     x = rng.standard_normal((m, in_f)).astype(np.float32)
     x[m // 2] *= 3.0e4
     x[m // 3] *= 1.0e-5
-    if dt == H.F16:
-        raw = (rng.standard_normal(out_f * in_f) * 0.02).astype(np.float16)
+    if dt in (H.F16, H.BF16, H.F32):
+        w32 = (rng.standard_normal(out_f * in_f) * 0.02).astype(np.float32)
+        raw = w32 if dt == H.F32 else w32.astype(np.float16) if dt == H.F16 else (w32.view(np.uint32) >> 16).astype(np.uint16)
     else:
         raw = H.centred_weight(dt, out_f * in_f, 5)
     g = M.Graph()
@@ -758,7 +760,7 @@ def test_linear_with_a_batch_of_rows_runs_on_the_matrix_cores(be, dt, m, in_f, o
     names = set(be.prof_read())
     be.prof_enable(False)
     want = O.linear(x, raw, dt, in_f, out_f)
-    mfma = dt != H.F16 and in_f % 64 == 0 and m >= 128
+    mfma = in_f % 64 == 0 and m >= 128
     assert (("linear_grouped" in names or "linear_grouped_units" in names) and "linear" not in names) if mfma else names == {"linear"}
     for r in range(m):
         assert H.rel_l2(got[r], want[r]) < (REL_L2_MFMA if mfma else 1e-5), r
