@@ -58,6 +58,7 @@ class _MoeArgs(C.Structure):
         ("n_buckets_out", C.c_void_p), ("bucket_expert_out", C.c_void_p),
         ("bucket_p0_out", C.c_void_p), ("bucket_count_out", C.c_void_p),
         ("pair_row_out", C.c_void_p), ("slot_pair_out", C.c_void_p),
+        ("production", C.c_int),
     ]
 
 
@@ -100,6 +101,10 @@ def lib() -> C.CDLL:
         L.orc_moe_shared_expert_add.restype = None
         L.orc_rms_norm.argtypes = [C.c_void_p, C.c_void_p, C.c_int, C.c_int, C.c_float, C.c_int, C.c_void_p]
         L.orc_rms_norm.restype = None
+        L.orc_quantize_q8.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
+        L.orc_quantize_q8.restype = None
+        L.orc_vec_dot_q8.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]
+        L.orc_vec_dot_q8.restype = C.c_float
         L.orc_hw_threads.restype = C.c_int
         _lib = L
     return _lib
@@ -187,8 +192,11 @@ def moe_ffn(x, router, gate, up, down, *, ne, n_expert, n_used, n_ff_exp,
             router_dtype=F32, gate_dtype=F32, up_dtype=None, down_dtype=None, router_x=None,
             scale=1.0, act=ACT_SILU, gating=GATE_SOFTMAX, norm_w=True, weight_before=False,
             fused_gate_up=False, down_scale=None, swiglu_clamp=None, exp_probs_b=None,
-            n_expert_groups=0, n_expert_groups_used=0, expert_ids=None, n_threads=0):
+            n_expert_groups=0, n_expert_groups_used=0, expert_ids=None, n_threads=0, production=False):
     """Run Op::MoeFfn in reference numerics.  Weights are raw GGUF bytes (any array; viewed as u8).
+
+    production=True: the CPU backend's batch numerics (int8 activations for Q4_K / Q6_K / Q8_0 banks from two
+    rows on) - for the timed CPU baseline only, not a parity reference.
 
     Returns a dict with dst [rows, ne] plus the routing/bucketing captures.
     """
@@ -231,7 +239,7 @@ def moe_ffn(x, router, gate, up, down, *, ne, n_expert, n_used, n_ff_exp,
         idx_out=_p(out["idx"]), w_out=_p(out["w"]), n_buckets_out=_p(out["n_buckets"]),
         bucket_expert_out=_p(out["bucket_expert"]), bucket_p0_out=_p(out["bucket_p0"]),
         bucket_count_out=_p(out["bucket_count"]), pair_row_out=_p(out["pair_row"]),
-        slot_pair_out=_p(out["slot_pair"]),
+        slot_pair_out=_p(out["slot_pair"]), production=int(production),
     )
     rc = lib().orc_moe_ffn(C.byref(a))
     if rc != 0:
@@ -290,6 +298,22 @@ def rms_norm(x, weight, eps, add_to=None) -> np.ndarray:
     dst = np.empty_like(x) if add_to is None else _f32(add_to).copy()
     lib().orc_rms_norm(_p(x), _p(w), rows, dim, eps, add_to is not None, _p(dst))
     return dst
+
+
+def quantize_q8(x):
+    """quantize_q8 of one row (length a multiple of 256): (int8 codes, f32 scale per 256, i32 sums per 32)."""
+    x = _f32(x).reshape(-1)
+    nb = x.size // 256
+    qs, d, bs = np.zeros(nb * 256, np.int8), np.zeros(nb, np.float32), np.zeros(nb * 8, np.int32)
+    lib().orc_quantize_q8(_p(x), x.size, _p(qs), _p(d), _p(bs))
+    return qs, d, bs
+
+
+def vec_dot_q8(dtype, row, q8) -> np.float32:
+    """One quantised weight row against one quantize_q8 activation row (the int8 production dot)."""
+    qs, d, bs = q8
+    r = _u8(row)
+    return np.float32(lib().orc_vec_dot_q8(dtype, _p(r), _p(qs), _p(d), _p(bs), qs.size))
 
 
 def hw_threads() -> int:

@@ -485,6 +485,159 @@ static int gemm_range_raw(const uint8_t *wbytes, size_t wlen, int dt, int in_f, 
     return 0;
 }
 
+/* ------------------------------------------------------------------ production int8 path (timed baseline only) */
+
+/* crates/infr-cpu/src/quant.rs:27-63 */
+void orc_quantize_q8(const float *x, int n, int8_t *qs, float *d, int32_t *bsums) {
+    int nb = n / 256;
+    for (int b = 0; b < nb; b++) {
+        const float *blk = x + (size_t)b * 256;
+        float amax = 0.0f;
+        for (int i = 0; i < 256; i++) { float v = fabsf(blk[i]); if (v > amax) amax = v; }
+        float dd = amax / 127.0f;
+        float id = dd > 0.0f ? 1.0f / dd : 0.0f;
+        d[b] = dd;
+        for (int i = 0; i < 256; i++) {
+            float r = roundf(blk[i] * id);   /* f32::round: half away from zero */
+            if (r < -127.0f) r = -127.0f;
+            if (r > 127.0f) r = 127.0f;
+            qs[(size_t)b * 256 + i] = (int8_t)r;
+        }
+        for (int s8 = 0; s8 < 8; s8++) {
+            int32_t acc = 0;
+            for (int i = 0; i < 32; i++) acc += qs[(size_t)b * 256 + s8 * 32 + i];
+            bsums[b * 8 + s8] = acc;
+        }
+    }
+}
+
+/* kernels.rs:151-184 */
+static float vec_dot_q4k_q8(const uint8_t *row, const int8_t *qs8, const float *d8, const int32_t *bsums, int in_f) {
+    float sumf = 0.0f;
+    for (int b = 0; b < in_f / 256; b++) {
+        const uint8_t *blk = row + (size_t)b * 144;
+        float d = orc_f16_to_f32(rd_u16(blk)), dmin = orc_f16_to_f32(rd_u16(blk + 2));
+        const uint8_t *scales = blk + 4, *qs = blk + 16;
+        const int8_t *q8b = qs8 + (size_t)b * 256;
+        int32_t sd = 0, sm = 0;
+        for (int s8 = 0; s8 < 8; s8++) {
+            uint32_t sc, m;
+            orc_k4(s8, scales, &sc, &m);
+            const uint8_t *qbyte = qs + (s8 / 2) * 32;
+            int32_t iprod = 0;
+            for (int l = 0; l < 32; l++) {
+                int q4 = (s8 & 1) ? (qbyte[l] >> 4) : (qbyte[l] & 0xF);
+                iprod += q4 * (int32_t)q8b[s8 * 32 + l];
+            }
+            sd += (int32_t)sc * iprod;
+            sm += (int32_t)m * bsums[b * 8 + s8];
+        }
+        float t1 = d * (float)sd, t2 = dmin * (float)sm;
+        float t = t1 - t2;
+        sumf = sumf + d8[b] * t;
+    }
+    return sumf;
+}
+
+/* kernels.rs:487-526 */
+static float vec_dot_q6k_q8(const uint8_t *row, const int8_t *qs8, const float *d8, int in_f) {
+    float sumf = 0.0f;
+    for (int b = 0; b < in_f / 256; b++) {
+        const uint8_t *blk = row + (size_t)b * 210;
+        const uint8_t *ql = blk, *qh = blk + 128;
+        const int8_t *scales = (const int8_t *)(blk + 192);
+        float d = orc_f16_to_f32(rd_u16(blk + 208));
+        const int8_t *q8b = qs8 + (size_t)b * 256;
+        int32_t sumi[16] = {0}, bsum[16] = {0};
+        for (int half = 0; half < 2; half++) {
+            int qlo = half * 64, qho = half * 32, sco = half * 8, base = half * 128;
+            for (int l = 0; l < 32; l++) {
+                int is = l / 16;
+                int q[4];
+                q[0] = (ql[qlo + l] & 0xF) | ((qh[qho + l] & 3) << 4);
+                q[1] = (ql[qlo + l + 32] & 0xF) | (((qh[qho + l] >> 2) & 3) << 4);
+                q[2] = (ql[qlo + l] >> 4) | (((qh[qho + l] >> 4) & 3) << 4);
+                q[3] = (ql[qlo + l + 32] >> 4) | (((qh[qho + l] >> 6) & 3) << 4);
+                for (int c = 0; c < 4; c++) {
+                    int sub = sco + is + 2 * c;
+                    int32_t v = q8b[base + l + 32 * c];
+                    sumi[sub] += q[c] * v;
+                    bsum[sub] += v;
+                }
+            }
+        }
+        int32_t isum = 0;
+        for (int sub = 0; sub < 16; sub++) isum += (int32_t)scales[sub] * (sumi[sub] - 32 * bsum[sub]);
+        float dd = d * d8[b];
+        sumf = sumf + dd * (float)isum;
+    }
+    return sumf;
+}
+
+/* kernels.rs:1170-1187 */
+static float vec_dot_q8_0_q8(const uint8_t *row, const int8_t *qs8, const float *d8, int in_f) {
+    float sumf = 0.0f;
+    for (int b = 0; b < in_f / 256; b++) {
+        for (int s8 = 0; s8 < 8; s8++) {
+            const uint8_t *blk = row + (size_t)(b * 8 + s8) * 34;
+            float dw = orc_f16_to_f32(rd_u16(blk));
+            const int8_t *qw = (const int8_t *)(blk + 2);
+            const int8_t *qx = qs8 + (size_t)b * 256 + s8 * 32;
+            int32_t iprod = 0;
+            for (int i = 0; i < 32; i++) iprod += (int32_t)qw[i] * (int32_t)qx[i];
+            float dd = d8[b] * dw;
+            sumf = sumf + dd * (float)iprod;
+        }
+    }
+    return sumf;
+}
+
+float orc_vec_dot_q8(int dtype, const uint8_t *row, const int8_t *qs, const float *d, const int32_t *bsums, int in_f) {
+    switch (dtype) {
+    case ORC_Q4K: return vec_dot_q4k_q8(row, qs, d, bsums, in_f);
+    case ORC_Q6K: return vec_dot_q6k_q8(row, qs, d, in_f);
+    case ORC_Q8_0: return vec_dot_q8_0_q8(row, qs, d, in_f);
+    default: return 0.0f / 0.0f;
+    }
+}
+
+/* expert_acts_kind == Super (crates/infr-cpu/src/moe.rs:42-53; Q5_K has no restatement here) */
+static int acts_super(int production, int rows, int dt, int in_f) {
+    return production && rows >= 2 && (dt == ORC_Q4K || dt == ORC_Q6K || dt == ORC_Q8_0) && in_f % 256 == 0;
+}
+
+/* `rows` activation rows quantised once for a stage (lib.rs:4009-4060: each row a single time) */
+typedef struct { int8_t *qs; float *d; int32_t *bsums; int in_f; } q8_rows;
+
+static q8_rows quantize_rows(const float *x, int rows, int in_f, int nthreads) {
+    q8_rows q;
+    int nb = in_f / 256;
+    q.in_f = in_f;
+    q.qs = (int8_t *)malloc((size_t)rows * in_f + 4);
+    q.d = (float *)malloc(sizeof(float) * (size_t)rows * nb + 4);
+    q.bsums = (int32_t *)malloc(sizeof(int32_t) * (size_t)rows * nb * 8 + 4);
+#pragma omp parallel for schedule(static) num_threads(nthreads)
+    for (int r = 0; r < rows; r++)
+        orc_quantize_q8(x + (size_t)r * in_f, in_f, q.qs + (size_t)r * in_f, q.d + (size_t)r * nb, q.bsums + (size_t)r * nb * 8);
+    return q;
+}
+static void free_rows(q8_rows *q) { free(q->qs); free(q->d); free(q->bsums); }
+
+/* expert_gemm_range, ExpertActs::Super arm (moe.rs:80-115), per-row form: rows [o0,o1) x `count` activations */
+static void gemm_range_q8(const uint8_t *wbytes, size_t wlen, int dt, int out_f, const q8_rows *q, int first, int count,
+                          int o0, int o1, float *out_t) {
+    size_t bpr = wlen / (size_t)out_f;
+    int nb = q->in_f / 256;
+    for (int o = o0; o < o1; o++) {
+        const uint8_t *row = wbytes + (size_t)o * bpr;
+        float *col = out_t + (size_t)(o - o0) * (size_t)count;
+        for (int r = 0; r < count; r++) {
+            size_t a = (size_t)(first + r);
+            col[r] = orc_vec_dot_q8(dt, row, q->qs + a * q->in_f, q->d + a * nb, q->bsums + a * nb * 8, q->in_f);
+        }
+    }
+}
+
 int orc_hw_threads(void) {
 #ifdef _OPENMP
     return omp_get_num_procs();
@@ -628,6 +781,10 @@ int orc_moe_ffn(const orc_moe_ffn_args *a) {
     /* ---- stage B (lib.rs:4087-4141) */
     float *gu_all = (float *)malloc(sizeof(float) * gu_off[n_buckets] + 4);
     float *up_all = a->fused_gate_up ? NULL : (float *)malloc(sizeof(float) * gu_off[n_buckets] + 4);
+    const int g_q8 = acts_super(a->production, rows, a->gate_dtype, ne);
+    const int u_q8 = !a->fused_gate_up && acts_super(a->production, rows, a->up_dtype, ne);
+    q8_rows xq = {0};
+    if (g_q8 || u_q8) xq = quantize_rows(xin_pairs, n_pairs, ne, nthreads);
 #pragma omp parallel num_threads(nthreads)
     {
         float *wf = (float *)malloc(sizeof(float) * (size_t)maxdim);
@@ -635,6 +792,11 @@ int orc_moe_ffn(const orc_moe_ffn_args *a) {
         for (int t = 0; t < ntask_gu; t++) {
             int b = tasks_gu[t].bucket, o0 = tasks_gu[t].o0, o1 = tasks_gu[t].o1;
             int e = b_expert[b], count = b_count[b];
+            if (g_q8) {
+                gemm_range_q8(a->gate + (size_t)e * gst, gst, a->gate_dtype, out_gu, &xq, b_p0[b], count, o0, o1,
+                              gu_all + gu_off[b] + (size_t)o0 * count);
+                continue;
+            }
             if (gemm_range_raw(a->gate + (size_t)e * gst, gst, a->gate_dtype, ne, out_gu,
                                xin_pairs + (size_t)b_p0[b] * ne, count, o0, o1,
                                gu_all + gu_off[b] + (size_t)o0 * count, wf) != 0) {
@@ -647,6 +809,11 @@ int orc_moe_ffn(const orc_moe_ffn_args *a) {
             for (int t = 0; t < ntask_gu; t++) {
                 int b = tasks_gu[t].bucket, o0 = tasks_gu[t].o0, o1 = tasks_gu[t].o1;
                 int e = b_expert[b], count = b_count[b];
+                if (u_q8) {
+                    gemm_range_q8(a->up + (size_t)e * ust, ust, a->up_dtype, nffx, &xq, b_p0[b], count, o0, o1,
+                                  up_all + gu_off[b] + (size_t)o0 * count);
+                    continue;
+                }
                 if (gemm_range_raw(a->up + (size_t)e * ust, ust, a->up_dtype, ne, nffx,
                                    xin_pairs + (size_t)b_p0[b] * ne, count, o0, o1,
                                    up_all + gu_off[b] + (size_t)o0 * count, wf) != 0) {
@@ -673,7 +840,11 @@ int orc_moe_ffn(const orc_moe_ffn_args *a) {
     }
 
     /* ---- stage D (lib.rs:4218-4265) */
+    if (g_q8 || u_q8) free_rows(&xq);
     float *down_all = (float *)malloc(sizeof(float) * d_off[n_buckets] + 4);
+    const int d_q8 = acts_super(a->production, rows, a->down_dtype, nffx);
+    q8_rows hq = {0};
+    if (d_q8 && !rc) hq = quantize_rows(dact, n_pairs, nffx, nthreads);
 #pragma omp parallel num_threads(nthreads)
     {
         float *wf = (float *)malloc(sizeof(float) * (size_t)maxdim);
@@ -681,6 +852,11 @@ int orc_moe_ffn(const orc_moe_ffn_args *a) {
         for (int t = 0; t < ntask_d; t++) {
             int b = tasks_d[t].bucket, o0 = tasks_d[t].o0, o1 = tasks_d[t].o1;
             int e = b_expert[b], count = b_count[b];
+            if (d_q8 && rc == 0) {
+                gemm_range_q8(a->down + (size_t)e * dstr, dstr, a->down_dtype, ne, &hq, b_p0[b], count, o0, o1,
+                              down_all + d_off[b] + (size_t)o0 * count);
+                continue;
+            }
             if (rc == 0 &&
                 gemm_range_raw(a->down + (size_t)e * dstr, dstr, a->down_dtype, nffx, ne,
                                dact + (size_t)b_p0[b] * nffx, count, o0, o1,
@@ -691,6 +867,7 @@ int orc_moe_ffn(const orc_moe_ffn_args *a) {
         }
         free(wf);
     }
+    if (d_q8 && hq.qs) free_rows(&hq);
     float *y_pairs = (float *)malloc(sizeof(float) * (size_t)n_pairs * ne + 4);
     for (int p = 0; p < n_pairs && !rc; p++) {
         int b = pair_bucket[p], i = pair_local[p], count = b_count[b], e = b_expert[b];

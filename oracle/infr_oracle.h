@@ -98,6 +98,12 @@ typedef struct orc_moe_ffn_args {
     int32_t *bucket_count_out; /* [n_expert] */
     int32_t *pair_row_out;     /* [rows*n_used] */
     int32_t *slot_pair_out;    /* [rows, n_used] -> flat pair index */
+    /* 0: reference (f32) numerics, the parity oracle.  1: the CPU backend's production numerics for a
+     * batch (crates/infr-cpu/src/lib.rs:3679 `int8_ok = rows >= 2 && !reference`): banks in Q4_K / Q6_K /
+     * Q8_0 whose row length is a multiple of 256 are dotted against int8 activations
+     * (crates/infr-cpu/src/moe.rs:42-53).  Only the timed CPU baseline uses it: it misses the parity bar by
+     * design (activation rounding of 1/127 per 256-element block). */
+    int production;
 } orc_moe_ffn_args;
 
 /* Op::MoeFfn, reference (f32) numerics (crates/infr-cpu/src/lib.rs:3584-4304).
@@ -119,6 +125,13 @@ void orc_moe_shared_expert_add(const float *moe, const float *shexp, const float
 
 /* Op::RmsNorm (add = 0) and Op::RmsNormAdd (add = 1: dst += ...), crates/infr-cpu/src/lib.rs:1046-1093. */
 void orc_rms_norm(const float *x, const float *w, int rows, int dim, float eps, int add, float *dst);
+
+/* quantize_q8 (crates/infr-cpu/src/quant.rs:27-63): per 256 elements d = amax / 127, q = round half away
+ * from zero of x / d clamped to +-127, bsums = sums of q per 32 elements.  n a multiple of 256. */
+void orc_quantize_q8(const float *x, int n, int8_t *qs, float *d, int32_t *bsums);
+/* vec_dot_q4k / q6k / q8_0, scalar forms (crates/infr-cpu/src/kernels.rs:151-184, :487-526, :1170-1187):
+ * one quantised weight row against one quantize_q8 activation row. */
+float orc_vec_dot_q8(int dtype, const uint8_t *row, const int8_t *qs, const float *d, const int32_t *bsums, int in_f);
 
 /* Number of hardware threads the pool would use. */
 int orc_hw_threads(void);

@@ -434,3 +434,64 @@ def test_rms_norm_closed_forms_and_f64():
     base = rng.standard_normal((4, dim)).astype(np.float32)
     assert np.array_equal(O.rms_norm(x, w, eps, add_to=base), base + got)
     assert O.rms_norm(np.zeros((0, dim), np.float32), w, eps).shape == (0, dim)
+
+
+# ------------------------------------------------------------------ production int8 path (timed baseline only)
+def test_quantize_q8_follows_the_definition():
+    """crates/infr-cpu/src/quant.rs:27-63: d = amax / 127 per 256, round half AWAY from zero, clamp to +-127,
+    sums per 32; an all-zero block gives d = 0 and zero codes."""
+    x = np.zeros(512, np.float32)
+    x[:256] = np.linspace(-2.0, 2.0, 256, dtype=np.float32)
+    x[3] = 2.0 * 0.5 / 127      # exactly half a step: rounds away from zero, to 1 (round-half-even would give 0)
+    x[4] = -2.0 * 2.5 / 127     # -2.5 steps -> -3
+    qs, d, bs = O.quantize_q8(x)
+    assert d[0] == np.float32(2.0) / np.float32(127.0) and d[1] == 0.0
+    assert qs[0] == -127 and qs[255] == 127 and qs[3] == 1 and qs[4] == -3
+    assert not qs[256:].any() and np.abs(qs).max() == 127
+    assert np.array_equal(bs, qs.astype(np.int32).reshape(-1, 32).sum(axis=1))
+    idv = np.float32(1.0) / d[0]
+    want = np.clip(np.sign(x[:256]) * np.floor(np.abs(x[:256] * idv) + np.float32(0.5)), -127, 127)
+    assert np.array_equal(qs[:256], want.astype(np.int8))
+
+
+@pytest.mark.parametrize("dt,in_f,d,dmin", [(O.Q4K, 768, 0.05, 0.015), (O.Q6K, 768, 0.04, None), (O.Q8_0, 512, 0.03, None)])
+def test_int8_dot_matches_the_dequantised_dot(dt, in_f, d, dmin):
+    """The reference's own check of its int8 kernels (crates/infr-cpu/src/kernels.rs:6782-6826): the integer dot
+    equals dot(dequant(weight row), dequant(q8 activations)) to 1e-3 of max(|want|, 1)."""
+    rng = np.random.default_rng(dt)
+    be, bb = O.block_geometry(dt)
+    w = rng.integers(0, 256, in_f // be * bb, dtype=np.uint8).reshape(-1, bb)
+    slots = H.F16_SLOTS[dt]
+    w[:, slots[0]:slots[0] + 2] = H.f16_bytes(d)
+    if dmin is not None:
+        w[:, slots[1]:slots[1] + 2] = H.f16_bytes(dmin)
+    w = w.reshape(-1)
+    x = (rng.standard_normal(in_f) * 1.5).astype(np.float32)
+    q8 = O.quantize_q8(x)
+    xq = (q8[0].astype(np.float32).reshape(-1, 256) * q8[1][:, None]).reshape(-1)
+    want = float(np.dot(H.ggml_dequant(dt, w).astype(np.float64), xq.astype(np.float64)))
+    got = float(O.vec_dot_q8(dt, w, q8))
+    assert abs(got - want) / max(abs(want), 1.0) < 1e-3
+    # and the activation rounding itself is the only other error: 1/254 of the block's amax per element
+    assert np.abs(xq - x).max() <= np.abs(x).max() / 254 * 1.0001
+
+
+@pytest.mark.parametrize("gdt,ddt", [(O.Q4K, O.Q6K), (O.Q8_0, O.Q8_0)])
+def test_production_mode_stays_close_to_reference_mode(gdt, ddt):
+    """Batch numerics of the CPU backend (int8 activations): same routing, outputs within the activation
+    quantisation error of the f32 reference; a single row is not affected (int8_ok needs two rows, lib.rs:3679)."""
+    ne, E, K, nff, rows = 512, 8, 2, 256, 6
+    rng = np.random.default_rng(9)
+    x = rng.standard_normal((rows, ne)).astype(np.float32)
+    router = (rng.standard_normal((E, ne)) * 0.1).astype(np.float32)
+    gate, up = H.centred_weight(gdt, E * nff * ne, 1), H.centred_weight(gdt, E * nff * ne, 2)
+    down = H.centred_weight(ddt, E * ne * nff, 3)
+    kw = dict(ne=ne, n_expert=E, n_used=K, n_ff_exp=nff, gate_dtype=gdt, down_dtype=ddt)
+    ref = O.moe_ffn(x, router, gate, up, down, **kw)
+    prod = O.moe_ffn(x, router, gate, up, down, production=True, **kw)
+    assert np.array_equal(ref["idx"], prod["idx"]) and np.array_equal(ref["w"].view(np.uint32), prod["w"].view(np.uint32))
+    err = H.rel_l2(prod["dst"], ref["dst"])
+    assert 1e-6 < err < 3e-2, err
+    one_ref = O.moe_ffn(x[:1], router, gate, up, down, **kw)
+    one_prod = O.moe_ffn(x[:1], router, gate, up, down, production=True, **kw)
+    assert np.array_equal(one_ref["dst"].view(np.uint32), one_prod["dst"].view(np.uint32))
