@@ -766,6 +766,26 @@ def test_linear_with_a_batch_of_rows_runs_on_the_matrix_cores(be, dt, m, in_f, o
         assert H.rel_l2(got[r], want[r]) < (REL_L2_MFMA if mfma else 1e-5), r
 
 
+def test_batched_linear_reads_a_row_band_of_a_concatenated_weight(be):
+    """w_off selects rows [w_off / in_f, + out_f) of a larger weight tensor (graph.rs:208-211), on the matrix-core
+    form as on the GEMV form: both bands of a 2 x out_f matrix, against the oracle and against each other's rows."""
+    m, in_f, out_f = 150, 512, 96
+    rng = np.random.default_rng(77)
+    x = rng.standard_normal((m, in_f)).astype(np.float32)
+    raw = H.centred_weight(H.Q4K, 2 * out_f * in_f, 8)
+    outs = []
+    for band in (0, 1):
+        g = M.Graph()
+        xi, wi = g.input(TensorDesc([m, in_f], DType.F32)), g.weight(TensorDesc([2 * out_f, in_f], DType.Q4K))
+        yi = g.output(TensorDesc([m, out_f], DType.F32))
+        g.linear(x=xi, weight=wi, dst=yi, m=m, in_f=in_f, out_f=out_f, w_off=band * out_f * in_f)
+        got = M.run_graph(be, g, [(xi, x), (wi, raw)], yi, m * out_f).reshape(m, out_f)
+        want = O.linear(x, raw, H.Q4K, in_f, out_f, w_off=band * out_f * in_f)
+        assert H.rel_l2(got, want) < REL_L2_MFMA
+        outs.append(got)
+    assert not np.array_equal(outs[0], outs[1])
+
+
 @pytest.mark.parametrize("gdt,ddt,rows,ne,nff", [
     (H.Q5K, H.Q5K, 1, 512, 256), (H.Q4_0, H.Q5_0, 2, 512, 256), (H.Q2K, H.Q3K, 1, 512, 256), (H.Q4_1, H.Q5_1, 3, 512, 256),
     (H.Q3K, H.Q2K, 5, 512, 256), (H.Q5_1, H.Q4_0, 1, 512, 256),
