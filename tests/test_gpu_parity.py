@@ -1031,18 +1031,26 @@ def test_bucketed_decode_batches_bucket_exactly_and_keep_f32_accuracy(be, rows, 
         assert H.max_abs(out, ref["dst"]) < MAX_ABS * max(1.0, scale)
 
 
-@pytest.mark.parametrize("rows,opts", [(1, {}), (3, {"weight_before": True}), (20, {}), (20, {"weight_before": True}), (40, {})])
+@pytest.mark.parametrize("rows,opts", [(1, {}), (3, {"weight_before": True}), (20, {}), (20, {"weight_before": True}), (40, {}),
+                                       (1, {"fmt": (H.Q5K, H.Q5_0)}), (20, {"fmt": (H.Q5K, H.Q5_0)}),
+                                       (40, {"fmt": (H.Q5K, H.Q5_0), "weight_before": True})])
 def test_expert_parallel_bands_sum_to_the_full_layer(be, rows, opts):
     """ep_band (crates/infr-core/src/graph.rs:1307-1319, crates/infr-vulkan/shaders/moe_ep_band_remap.comp):
     routing stays global, the expert tensors hold one rank's shard, selections of foreign experts become
     (id 0, weight 0).  The partial outputs of all ranks must add up to the single-device layer, and the
     remapped ids / weights must be the shader's."""
     ne, nff, E, K, W = 512, 256, 16, 4, 2
+    opts = dict(opts)
+    gdt, ddt = opts.pop("fmt", (H.Q4K, H.Q6K))   # the second pair runs on the 32-element-unit kernels
     rng = np.random.default_rng(rows)
     x = rng.standard_normal((rows, ne)).astype(np.float32)
     router = (rng.standard_normal((E, ne)) * 0.05).astype(np.float32)
-    gate, up = _realistic(rng, E, nff, ne, H.Q4K), _realistic(rng, E, nff, ne, H.Q4K)
-    down = _realistic(rng, E, ne, nff, H.Q6K)
+    if gdt == H.Q4K:
+        gate, up = _realistic(rng, E, nff, ne, H.Q4K), _realistic(rng, E, nff, ne, H.Q4K)
+        down = _realistic(rng, E, ne, nff, H.Q6K)
+    else:
+        gate, up = H.centred_weight(gdt, E * nff * ne, 1), H.centred_weight(gdt, E * nff * ne, 2)
+        down = H.centred_weight(ddt, E * ne * nff, 3)
     ds = rng.uniform(0.5, 1.5, E).astype(np.float32)
 
     def run(band):
@@ -1051,8 +1059,8 @@ def test_expert_parallel_bands_sum_to_the_full_layer(be, rows, opts):
         g = M.Graph()
         xi = g.input(TensorDesc([rows, ne], DType.F32))
         rt = g.weight(TensorDesc([E, ne], DType.F32))
-        gt, ut = g.weight(TensorDesc([n_loc, nff, ne], DType.Q4K)), g.weight(TensorDesc([n_loc, nff, ne], DType.Q4K))
-        dt = g.weight(TensorDesc([n_loc, ne, nff], DType.Q6K))
+        gt, ut = g.weight(TensorDesc([n_loc, nff, ne], DType(gdt))), g.weight(TensorDesc([n_loc, nff, ne], DType(gdt)))
+        dt = g.weight(TensorDesc([n_loc, ne, nff], DType(ddt)))
         dst = g.weight(TensorDesc([n_loc], DType.F32))
         yo = g.output(TensorDesc([rows, ne], DType.F32))
         g.moe_ffn(x=xi, router=rt, gate_exps=gt, up_exps=ut, down_exps=dt, dst=yo, ne=ne, n_expert=E, n_used=K,
@@ -1069,8 +1077,8 @@ def test_expert_parallel_bands_sum_to_the_full_layer(be, rows, opts):
         return out.reshape(rows, ne), r
 
     full, rf = run(None)
-    ref = O.moe_ffn(x, router, gate, up, down, ne=ne, n_expert=E, n_used=K, n_ff_exp=nff, gate_dtype=H.Q4K,
-                    down_dtype=H.Q6K, down_scale=ds, **opts)
+    ref = O.moe_ffn(x, router, gate, up, down, ne=ne, n_expert=E, n_used=K, n_ff_exp=nff, gate_dtype=gdt,
+                    down_dtype=ddt, down_scale=ds, **opts)
     assert np.array_equal(rf["idx"], ref["idx"])
     total = np.zeros_like(full)
     for rank in range(W):
