@@ -251,18 +251,26 @@ def test_moe_ffn_matches_oracle(be, rows, ne, E, K, nff, gdt, ddt):
     assert H.max_abs(out, ref["dst"]) < MAX_ABS * max(1.0, scale), (H.max_abs(out, ref["dst"]), scale)
 
 
-def test_moe_ffn_option_variants_match_oracle(be):
+def _bank_weights(rng, E, nff, ne, gdt, ddt):
+    """Q4_K / Q6_K / Q8_0 banks as the other tests make them; any other affine format as centred synthetic blocks."""
+    if gdt in (H.Q4K, H.Q6K, H.Q8_0) and ddt in (H.Q4K, H.Q6K, H.Q8_0):
+        return _realistic(rng, E, nff, ne, gdt), _realistic(rng, E, nff, ne, gdt), _realistic(rng, E, ne, nff, ddt)
+    return (H.centred_weight(gdt, E * nff * ne, 1), H.centred_weight(gdt, E * nff * ne, 2),
+            H.centred_weight(ddt, E * ne * nff, 3))
+
+
+@pytest.mark.parametrize("gdt,ddt", [(H.Q4K, H.Q6K), (H.Q5K, H.Q4_0)])
+def test_moe_ffn_option_variants_match_oracle(be, gdt, ddt):
     ne, E, K, nff, rows = 256, 8, 3, 256, 3
     rng = np.random.default_rng(21)
     x = rng.standard_normal((rows, ne)).astype(np.float32)
     router = rng.standard_normal((E, ne)).astype(np.float32) * 0.05
-    gate, up = _realistic(rng, E, nff, ne, H.Q4K), _realistic(rng, E, nff, ne, H.Q4K)
-    down = _realistic(rng, E, ne, nff, H.Q6K)
+    gate, up, down = _bank_weights(rng, E, nff, ne, gdt, ddt)
     ds = rng.uniform(0.5, 1.5, E).astype(np.float32)
-    base = dict(ne=ne, n_expert=E, n_used=K, n_ff_exp=nff, gate_dtype=H.Q4K, down_dtype=H.Q6K)
+    base = dict(ne=ne, n_expert=E, n_used=K, n_ff_exp=nff, gate_dtype=gdt, down_dtype=ddt)
 
     def check(gopts, oopts, data_extra=None, fused=False):
-        g, ids = moe_graph(rows, ne, E, K, nff, DType.Q4K, DType.Q6K, **gopts)
+        g, ids = moe_graph(rows, ne, E, K, nff, DType(gdt), DType(ddt), **gopts)
         data = dict(x=x, router=router, gate=gate, up=up, down=down)
         ogate, oup = gate, up
         if fused:
@@ -970,17 +978,17 @@ def test_batched_moe_ffn_buckets_exactly_and_matches_oracle(be, rows, ne, E, K, 
     assert H.rel_l2(out, ref["dst"]) < REL_L2_MFMA
 
 
-def test_batched_moe_ffn_option_variants_match_oracle(be):
+@pytest.mark.parametrize("gdt,ddt", [(H.Q4K, H.Q6K), (H.Q5K, H.Q4_0)])
+def test_batched_moe_ffn_option_variants_match_oracle(be, gdt, ddt):
     ne, E, K, nff, rows = 256, 8, 3, 256, 48
     rng = np.random.default_rng(23)
     x = rng.standard_normal((rows, ne)).astype(np.float32)
     router = rng.standard_normal((E, ne)).astype(np.float32) * 0.05
-    gate, up = _realistic(rng, E, nff, ne, H.Q4K), _realistic(rng, E, nff, ne, H.Q4K)
-    down = _realistic(rng, E, ne, nff, H.Q6K)
+    gate, up, down = _bank_weights(rng, E, nff, ne, gdt, ddt)
     ds = rng.uniform(0.5, 1.5, E).astype(np.float32)
     bias = rng.standard_normal(E).astype(np.float32) * 0.1
     eids = rng.integers(0, E, (rows, K)).astype(np.int32)
-    base = dict(ne=ne, n_expert=E, n_used=K, n_ff_exp=nff, gate_dtype=H.Q4K, down_dtype=H.Q6K)
+    base = dict(ne=ne, n_expert=E, n_used=K, n_ff_exp=nff, gate_dtype=gdt, down_dtype=ddt)
     cases = [
         (dict(weight_before=True), dict(weight_before=True), {}),
         (dict(swiglu_clamp=0.05), dict(swiglu_clamp=0.05), {}),
@@ -991,12 +999,20 @@ def test_batched_moe_ffn_option_variants_match_oracle(be):
         (dict(act=M.Activation.Gelu), dict(act=O.ACT_GELU), {}),
     ]
     for gopts, oopts, extra in cases:
-        g, ids = moe_graph(rows, ne, E, K, nff, DType.Q4K, DType.Q6K, **dict(gopts))
+        g, ids = moe_graph(rows, ne, E, K, nff, DType(gdt), DType(ddt), **dict(gopts))
         out, r, b = _run_batched(be, g, ids, dict(x=x, router=router, gate=gate, up=up, down=down, **extra), rows, ne)
         ref = O.moe_ffn(x, router, gate, up, down, **base, **oopts)
         assert np.array_equal(r["idx"], ref["idx"]), gopts
         _check_bucketing(b, ref, E)
         assert H.rel_l2(out, ref["dst"]) < REL_L2_MFMA, (gopts, H.rel_l2(out, ref["dst"]))
+    if gdt != H.Q4K:
+        # gate and up rows of an expert in one tensor: the unit-decoder GEMM takes that layout on the matrix cores too
+        gu = np.concatenate([gate.reshape(E, -1), up.reshape(E, -1)], axis=1).reshape(-1)
+        g, ids = moe_graph(rows, ne, E, K, nff, DType(gdt), DType(ddt), fused_gate_up=True)
+        out, r, b = _run_batched(be, g, ids, dict(x=x, router=router, gate=gu, up=None, down=down), rows, ne)
+        ref = O.moe_ffn(x, router, gu, None, down, **base, fused_gate_up=True)
+        assert np.array_equal(r["idx"], ref["idx"])
+        assert H.rel_l2(out, ref["dst"]) < REL_L2_MFMA
 
 
 @pytest.mark.parametrize("rows,ne,E,K,nff,gdt,ddt", [
