@@ -283,7 +283,10 @@ def main():
     out = {
         "metric": "MoE prefill tok/s" if prefill else "MoE decode tok/s", "value": round(tok_s, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "vs_baseline": None,
+        # decode: exact integer dots on 23-bit fixed-point activations, scales and sums in f32; batched path: f16
+        # operands on the matrix cores with f32 accumulation
+        "dtype": "f16" if batch >= 32 else "f32", "data": "synthetic",
         "config": {"workload": (shape.name if n_layer == shape.n_layer else f"{shape.name}[{n_layer} layers]") +
                                ("+rmsnorm+residual" if args.sublayer else "") + ("/unfused" if args.no_fusion else ""),
                    "layers": n_layer, "hidden": shape.ne, "experts": shape.n_expert, "top_k": shape.n_used,
