@@ -141,6 +141,7 @@ struct infr_hip_plan {
         Fuse kind = kPlain;
         uint32_t a = 0, b = 0;   // kGateUpAct: index of the up Linear and of the GatedAct; kLinearAdd: index of the Add;
                                  // kMoeShared: index of the always-on expert's first Linear and of its down Linear
+        uint32_t gated = 0;      // kMoeShared: 1 + index of the Op::MoeSharedExpertAdd that closes the pattern (0: a plain Op::Add)
         uint32_t norm = 0;       // MoeFfn: 1 + index of the Op::RmsNorm its logits kernel applies to the token row
         uint32_t res = 0;        // MoeFfn: 1 + index of the following Op::Add folded into the combine
     };
@@ -842,18 +843,36 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
         // exactly 1 and it is combined last, which is the Add's rounding: the bits do not change.
         plan->fuse_head = plan->fuse;
         for (uint32_t oi = 0; oi + 5 < g->n_ops; oi++) {
-            if (plan->ops[oi].kind != INFR_OP_MOE_FFN || plan->fuse[oi + 1].kind != infr_hip_plan::kGateUpAct ||
-                plan->fuse[oi + 4].kind != infr_hip_plan::kLinearAdd)
+            if (plan->ops[oi].kind != INFR_OP_MOE_FFN) continue;
+            // the gated form (crates/infr-llama/src/seam/runner.rs:8104-8163): the gate-logit Linear (out_f = 1) comes
+            // first and Op::MoeSharedExpertAdd closes the pattern; that Linear stays a launch of its own
+            const bool gated = oi + 6 < g->n_ops && plan->ops[oi + 1].kind == INFR_OP_LINEAR &&
+                               plan->ops[oi + 1].u.linear.out_f == 1 && plan->fuse[oi + 1].kind == infr_hip_plan::kPlain &&
+                               plan->ops[oi + 6].kind == INFR_OP_MOE_SHARED_EXPERT_ADD;
+            const uint32_t b0 = gated ? oi + 2 : oi + 1;   // first op of the dense FFN
+            if (plan->fuse[b0].kind != infr_hip_plan::kGateUpAct) continue;
+            if (gated ? plan->fuse[b0 + 3].kind != infr_hip_plan::kPlain || plan->ops[b0 + 3].kind != INFR_OP_LINEAR
+                      : plan->fuse[b0 + 3].kind != infr_hip_plan::kLinearAdd)
                 continue;
             const infr_op_moe_ffn& m = plan->ops[oi].u.moe_ffn;
             const MoeScratch& sc = plan->moe[oi];
-            const infr_hip_plan::FuseOp fg = plan->fuse[oi + 1];
+            const infr_hip_plan::FuseOp fg = plan->fuse[b0];
             const infr_op_linear& lu = plan->ops[fg.a].u.linear;
-            const infr_op_linear& lg = plan->ops[fg.a == oi + 1 ? oi + 2 : oi + 1].u.linear;
-            const infr_op_gated_act& ga = plan->ops[oi + 3].u.gated_act;
-            const infr_op_linear& ld = plan->ops[oi + 4].u.linear;
-            const infr_op_add& ad = plan->ops[oi + 5].u.add;
-            const uint32_t other = ad.a == ld.dst ? ad.b : ad.a;
+            const infr_op_linear& lg = plan->ops[fg.a == b0 ? b0 + 1 : b0].u.linear;
+            const infr_op_gated_act& ga = plan->ops[b0 + 2].u.gated_act;
+            const infr_op_linear& ld = plan->ops[b0 + 3].u.linear;
+            uint32_t other;
+            if (gated) {
+                const infr_op_moe_shared_expert_add& sa = plan->ops[oi + 6].u.moe_shared_expert_add;
+                const infr_op_linear& lq = plan->ops[oi + 1].u.linear;
+                if (sa.shexp != ld.dst || !temp(ld.dst) || sa.gate != lq.dst || !temp(lq.dst) || (int)sa.rows != sc.rows ||
+                    sa.n != m.ne || lq.x != m.x || (int)lq.m != sc.rows || lq.in_f != m.ne)
+                    continue;
+                other = sa.moe;
+            } else {
+                const infr_op_add& ad = plan->ops[b0 + 4].u.add;
+                other = ad.a == ld.dst ? ad.b : ad.a;
+            }
             // one token row only: with more rows the launches saved no longer matter and the down kernel
             // streams best with one wave per routed slot
             if (sc.batched || sc.bucketed || sc.rows != 1 || m.fused_gate_up) continue;
@@ -875,9 +894,11 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
             probe.sh_gate = probe.sh_up = probe.sh_down = (const uint8_t*)plan;   // any non-null value: shape checks only
             if (m.n_used >= 63 || !infr::moe_gate_up_routes_inline(probe) || !infr::moe_down_is_fast(probe)) continue;
             plan->fuse[oi].kind = infr_hip_plan::kMoeShared;
-            plan->fuse[oi].a = oi + 1;
-            plan->fuse[oi].b = oi + 4;
-            for (uint32_t k = oi + 1; k <= oi + 5; k++) plan->fuse[k].kind = infr_hip_plan::kSkip;
+            plan->fuse[oi].a = b0;
+            plan->fuse[oi].b = b0 + 3;
+            plan->fuse[oi].gated = gated ? oi + 7 : 0;
+            // (the gate-logit Linear of the gated form is launched by the fused op, ahead of the kernel that reads it)
+            for (uint32_t k = oi + 1; k <= b0 + 4; k++) plan->fuse[k].kind = infr_hip_plan::kSkip;
         }
         // MoeFfn -> Add (the residual; the reference's moe_add rewrite, crates/infr-core/src/fusion.rs:20-24):
         // every combine kernel ends with "other operand + finished sum", the Add's own rounding.
@@ -889,8 +910,11 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
             if (kind != infr_hip_plan::kPlain && kind != infr_hip_plan::kMoeShared) continue;
             const infr_op_moe_ffn& m = plan->ops[oi].u.moe_ffn;
             const MoeScratch& sc = plan->moe[oi];
-            const uint32_t nx = kind == infr_hip_plan::kMoeShared ? oi + 6 : oi + 1;
-            const uint32_t sum_t = kind == infr_hip_plan::kMoeShared ? plan->ops[oi + 5].u.add.dst : m.dst;
+            const uint32_t close = plan->fuse[oi].b + 1;   // kMoeShared: the Add / MoeSharedExpertAdd that ends the pattern
+            const uint32_t nx = kind == infr_hip_plan::kMoeShared ? close + 1 : oi + 1;
+            const uint32_t sum_t = kind != infr_hip_plan::kMoeShared ? m.dst
+                                   : plan->fuse[oi].gated ? plan->ops[close].u.moe_shared_expert_add.dst
+                                                          : plan->ops[close].u.add.dst;
             if (nx < g->n_ops && plan->ops[nx].kind == INFR_OP_ADD && plan->fuse[nx].kind == infr_hip_plan::kPlain && sc.rows > 0) {
                 const infr_op_add& ad = plan->ops[nx].u.add;
                 const bool one_side = (ad.a == sum_t) != (ad.b == sum_t);
@@ -1145,7 +1169,9 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                 gp.x = (const float*)ptr[m.x];
                 if (fz.res) {
                     const infr_op_add& ad = plan->ops[fz.res - 1].u.add;
-                    const uint32_t sum_t = fz.kind == infr_hip_plan::kMoeShared ? plan->ops[fz.b + 1].u.add.dst : m.dst;
+                    const uint32_t sum_t = fz.kind != infr_hip_plan::kMoeShared ? m.dst
+                                           : fz.gated ? plan->ops[fz.b + 1].u.moe_shared_expert_add.dst
+                                                      : plan->ops[fz.b + 1].u.add.dst;
                     const uint32_t other = ad.a == sum_t ? ad.b : ad.a;
                     if (!(need(other, "Add.a") && need(ad.dst, "Add.dst"))) return INFR_ERR_BACKEND;
                     gp.addend = (const float*)ptr[other];
@@ -1268,14 +1294,28 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                     const infr_op_linear& lu = plan->ops[fg.a].u.linear;
                     const infr_op_linear& lg = plan->ops[fg.a == fz.a ? fz.a + 1 : fz.a].u.linear;
                     const infr_op_linear& ld = plan->ops[fz.b].u.linear;
-                    const infr_op_add& ad = plan->ops[fz.b + 1].u.add;
+                    const uint32_t sum_dst = fz.gated ? plan->ops[fz.b + 1].u.moe_shared_expert_add.dst : plan->ops[fz.b + 1].u.add.dst;
                     if (!(need(lg.weight, "Linear.weight") && need(lu.weight, "Linear.weight") &&
-                          need(ld.weight, "Linear.weight") && (fz.res || need(ad.dst, "Add.dst"))))
+                          need(ld.weight, "Linear.weight") && (fz.res || need(sum_dst, "Add.dst"))))
                         return INFR_ERR_BACKEND;
                     gp.sh_gate = (const uint8_t*)ptr[lg.weight];
                     gp.sh_up = (const uint8_t*)ptr[lu.weight];
                     gp.sh_down = (const uint8_t*)ptr[ld.weight];
-                    if (!fz.res) gp.dst = (float*)ptr[ad.dst];
+                    if (!fz.res) gp.dst = (float*)ptr[sum_dst];
+                    if (fz.gated) {
+                        // the row's gate logit (a Linear with one output row), ahead of the kernel that weighs with it
+                        const infr_op_linear& lq = plan->ops[oi + 1].u.linear;
+                        if (!(need(lq.x, "Linear.x") && need(lq.weight, "Linear.weight") && need(lq.dst, "Linear.dst")))
+                            return INFR_ERR_BACKEND;
+                        int we = 1, wb = 4;
+                        geometry(plan->tensors[lq.weight].dtype, &we, &wb);
+                        const size_t rb = (size_t)(lq.in_f / we) * wb;
+                        Timed t(be, "linear");
+                        infr::launch_linear(s, (const float*)ptr[lq.x], (const uint8_t*)ptr[lq.weight] + (size_t)(lq.w_off / lq.in_f) * rb,
+                                            plan->tensors[lq.weight].dtype, rb, (int)lq.m, (int)lq.in_f, (int)lq.out_f,
+                                            (float*)ptr[lq.dst], n_cu);
+                        gp.sh_logit = (const float*)ptr[lq.dst];
+                    }
                 }
                 gp.route = rp;
                 gp.y = sc.y;

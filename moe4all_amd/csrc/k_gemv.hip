@@ -668,6 +668,8 @@ __global__ __launch_bounds__(512) void moe_down_combine_fast(MoeGemvParams p, in
         for (int k = 0; k < n_slots; k++) {
             if (p.skip_zero_w && k < p.n_used && w[k] == 0.0f) continue;
             float wk = (p.weight_before || k >= p.n_used) ? 1.0f : w[k];
+            if (k >= p.n_used && p.sh_logit)   // crates/infr-cpu/src/lib.rs:3336-3356: sigmoid of the row's gate logit
+                wk = __fdiv_rn(1.0f, __fadd_rn(1.0f, expf_libm(-p.sh_logit[r])));
             acc = __fadd_rn(acc, __fmul_rn(wk, ypart[k][o]));
         }
         const size_t oi = (size_t)r * p.ne + o0 + o;

@@ -75,6 +75,9 @@ struct MoeGemvParams {
     // optional always-on expert handled as one more slot after the n_used routed ones (same dtypes,
     // same n_ff, routing weight 1): h then has n_used + 1 slots per row
     const uint8_t* sh_gate; const uint8_t* sh_up; const uint8_t* sh_down;
+    // null: the always-on expert weighs 1 (Op::Add); else [rows] gate logits, its weight is sigmoid(logit)
+    // (Op::MoeSharedExpertAdd)
+    const float* sh_logit;
     // bucketed kernels: the most pairs one bucket can hold (0 = rows; rows * n_used when given expert ids
     // may repeat an expert inside a row)
     int max_bucket;

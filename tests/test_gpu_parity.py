@@ -1253,8 +1253,8 @@ def test_batched_threshold_is_configurable_and_the_paths_agree():
     assert H.rel_l2(outs["mfma"], outs["gemv"]) < REL_L2_MFMA
 
 
-@pytest.mark.parametrize("rows", [1, 5])
-def test_disabling_op_fusion_changes_the_launches_not_the_bits(rows):
+@pytest.mark.parametrize("rows,gated", [(1, False), (5, False), (1, True), (4, True)])
+def test_disabling_op_fusion_changes_the_launches_not_the_bits(rows, gated):
     """infr_hip_config.disable_op_fusion (the reference keeps the same hatch for its rewrites,
     crates/infr-core/src/fusion.rs:49-52): one launch per op, identical output bits."""
     ne, nff, E, K = 512, 256, 8, 2
@@ -1264,6 +1264,7 @@ def test_disabling_op_fusion_changes_the_launches_not_the_bits(rows):
     router = (rng.standard_normal((E, ne)) * 0.1).astype(np.float32)
     eg, eu, ed = _realistic(rng, E, nff, ne, H.Q4K), _realistic(rng, E, nff, ne, H.Q4K), _realistic(rng, E, ne, nff, H.Q6K)
     wg, wu, wd = _realistic(rng, 1, nff, ne, H.Q4K), _realistic(rng, 1, nff, ne, H.Q4K), _realistic(rng, 1, ne, nff, H.Q6K)
+    wq = (rng.standard_normal(ne) * 0.05).astype(np.float32)   # gate vector of the gated shared expert
     outs, names = {}, {}
     for off in (False, True):
         be2 = M.Backend(0, disable_op_fusion=off)
@@ -1281,24 +1282,42 @@ def test_disabling_op_fusion_changes_the_launches_not_the_bits(rows):
             g.rms_norm(x=xi, weight=nwt, dst=xn, rows=rows, dim=ne, eps=1e-6)
             g.moe_ffn(x=xn, router=rt, gate_exps=egt, up_exps=eut, down_exps=edt, dst=moe, ne=ne, n_expert=E, n_used=K,
                       n_ff_exp=nff)
+            extra = []
+            if gated:   # sigmoid(gate . x) weighs the shared expert (crates/infr-llama/src/seam/runner.rs:8104-8163)
+                wqt = g.weight(TensorDesc([1, ne], DType.F32))
+                logit = g.internal(TensorDesc([rows, 1], DType.F32))
+                g.linear(x=xn, weight=wqt, dst=logit, m=rows, in_f=ne, out_f=1)
+                extra.append((wqt, wq))
             g.linear(x=xn, weight=wgt, dst=gt, m=rows, in_f=ne, out_f=nff)
             g.linear(x=xn, weight=wut, dst=ut, m=rows, in_f=ne, out_f=nff)
             g.gated_act(gate=gt, up=ut, dst=at, rows=rows, nff=nff)
             g.linear(x=at, weight=wdt, dst=st, m=rows, in_f=nff, out_f=ne)
-            g.add(a=moe, b=st, dst=sub, n=rows * ne)
+            if gated:
+                g.moe_shared_expert_add(moe=moe, shexp=st, gate=logit, dst=sub, rows=rows, n=ne)
+            else:
+                g.add(a=moe, b=st, dst=sub, n=rows * ne)
             g.add(a=xi, b=sub, dst=yi, n=rows * ne)
             keep = []
             be2.prof_enable(True)
             outs[off] = M.run_graph(be2, g, [(xi, x), (nwt, nw), (rt, router), (egt, eg), (eut, eu), (edt, ed), (wgt, wg),
-                                             (wut, wu), (wdt, wd)], yi, rows * ne, keep=keep)
+                                             (wut, wu), (wdt, wd)] + extra, yi, rows * ne, keep=keep)
             be2.sync()
             names[off] = set(be2.prof_read())
         finally:
             be2.close()
     assert np.array_equal(bits(outs[False]), bits(outs[True]))
     assert {"rms_norm", "add", "gated_act", "linear"} <= names[True]
+    assert ("moe_shared_expert_add" in names[True]) == gated
     assert "gated_act" not in names[False]
-    if rows == 1:
-        assert names[False] == {"rms_norm_router_logits", "moe_route_gate_up_shared", "moe_down_combine_shared"}
+    if rows == 1:   # the gated form keeps one launch for the gate logit
+        assert names[False] == {"rms_norm_router_logits", "moe_route_gate_up_shared", "moe_down_combine_shared"} | ({"linear"} if gated else set())
+    elif gated:
+        assert {"linear_gate_up_act", "linear", "moe_shared_expert_add", "add"} <= names[False]
     else:   # several rows: the dense FFN folds into two launches, the residual Add after it stays a launch
         assert {"linear_gate_up_act", "linear_add", "add"} <= names[False]
+    # and against the oracle
+    xn_o = O.rms_norm(x, nw, 1e-6).reshape(rows, ne)
+    moe_o = O.moe_ffn(xn_o, router, eg, eu, ed, ne=ne, n_expert=E, n_used=K, n_ff_exp=nff, gate_dtype=H.Q4K, down_dtype=H.Q6K)
+    sh_o = O.linear(O.gated_act_rows(O.linear(xn_o, wg, H.Q4K, ne, nff), O.linear(xn_o, wu, H.Q4K, ne, nff)), wd, H.Q6K, nff, ne)
+    sub_o = O.moe_shared_expert_add(moe_o["dst"], sh_o, O.linear(xn_o, wq, H.F32, ne, 1)) if gated else O.add(moe_o["dst"], sh_o)
+    assert H.rel_l2(outs[False].reshape(rows, ne) - x, sub_o.reshape(rows, ne)) < REL_L2
