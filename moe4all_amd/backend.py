@@ -48,6 +48,21 @@ class DType(enum.IntEnum):
     Q4K = 12
     Q5K = 13
     Q6K = 14
+    Iq1S = 15
+    Iq1M = 16
+    Iq2Xxs = 17
+    Iq2Xs = 18
+    Iq2S = 19
+    Iq3Xxs = 20
+    Iq3S = 21
+    Iq4Nl = 22
+    Iq4Xs = 23
+    Tq1_0 = 24
+    Tq2_0 = 25
+    I2S = 26
+    Q2_0 = 27
+    Mxfp4 = 28
+    Nvfp4 = 29
 
 
 class BufferUsage(enum.IntEnum):
@@ -80,7 +95,9 @@ class MoeGating(enum.IntEnum):
 
 _BLOCK = {DType.F32: (1, 4), DType.I32: (1, 4), DType.U32: (1, 4), DType.F16: (1, 2), DType.Bf16: (1, 2),
           DType.Q8_0: (32, 34), DType.Q4K: (256, 144), DType.Q6K: (256, 210), DType.Q4_0: (32, 18), DType.Q4_1: (32, 20),
-          DType.Q5_0: (32, 22), DType.Q5_1: (32, 24), DType.Q2K: (256, 84), DType.Q3K: (256, 110), DType.Q5K: (256, 176)}
+          DType.Q5_0: (32, 22), DType.Q5_1: (32, 24), DType.Q2K: (256, 84), DType.Q3K: (256, 110), DType.Q5K: (256, 176),
+          DType.Iq4Nl: (32, 18), DType.Iq4Xs: (256, 136), DType.Tq1_0: (256, 54), DType.Tq2_0: (256, 66), DType.Q2_0: (64, 18),
+          DType.Mxfp4: (32, 17), DType.Nvfp4: (64, 36)}
 
 
 def bytes_for(dtype: DType, numel: int) -> int:

@@ -115,9 +115,41 @@ __host__ __device__ inline bool block_geometry(int dtype, int* elems, int* bytes
         case INFR_Q4K: *elems = 256; *bytes = 144; return true;
         case INFR_Q5K: *elems = 256; *bytes = 176; return true;
         case INFR_Q6K: *elems = 256; *bytes = 210; return true;
+        case INFR_IQ4_NL: *elems = 32; *bytes = 18; return true;
+        case INFR_IQ4_XS: *elems = 256; *bytes = 136; return true;
+        case INFR_TQ1_0: *elems = 256; *bytes = 54; return true;
+        case INFR_TQ2_0: *elems = 256; *bytes = 66; return true;
+        case INFR_Q2_0: *elems = 64; *bytes = 18; return true;
+        case INFR_MXFP4: *elems = 32; *bytes = 17; return true;
+        case INFR_NVFP4: *elems = 64; *bytes = 36; return true;
         default: return false;
     }
 }
+
+// The 16-entry code books (crates/infr-gguf/src/dequant.rs:407-444) as sixteen signed bytes in two
+// 64-bit halves, entry i = byte i % 8 of half i / 8.
+// IQ4_NL / IQ4_XS: -127 -104 -83 -65 -49 -35 -22 -10 1 13 25 38 53 69 89 113.
+// MXFP4 / NVFP4 (twice the E2M1 value): 0 1 2 3 4 6 8 12 0 -1 -2 -3 -4 -6 -8 -12.
+constexpr uint64_t kIq4nlLo = 0xF6EADDCFBFAD9881ull, kIq4nlHi = 0x7159453526190D01ull;
+constexpr uint64_t kFp4Lo = 0x0C08060403020100ull, kFp4Hi = 0xF4F8FAFCFDFEFF00ull;
+__device__ __forceinline__ int book16(uint64_t lo, uint64_t hi, uint32_t i) {
+    return (int)(int8_t)(((i & 8u) ? hi : lo) >> (8u * (i & 7u)));
+}
+
+// e8m0_to_fp32_half (dequant.rs:415-421): 2^(x - 128), the two smallest as subnormals.
+__device__ __forceinline__ float e8m0_half(uint32_t x) {
+    return __uint_as_float(x < 2u ? 0x00200000u << x : (x - 1u) << 23);
+}
+// ue4m3_to_fp32 (dequant.rs:427-438): unsigned 4-bit exponent (bias 7), 3-bit mantissa, halved;
+// 0x00 and 0x7F decode to zero, bit 7 is not read.
+__device__ __forceinline__ float ue4m3_half(uint32_t x) {
+    if (x == 0u || x == 0x7Fu) return 0.0f;
+    const uint32_t e = (x >> 3) & 0xFu, m = x & 7u;
+    return e == 0u ? (float)m * 0x1p-10f : __uint_as_float(((e + 119u) << 23) | (m << 20));
+}
+
+// Ternary digit n of a TQ1_0 byte (dequant.rs:938-944): 0, 1 or 2.
+__device__ __forceinline__ uint32_t trit(uint32_t q, uint32_t pow3) { return (((q * pow3) & 0xFFu) * 3u) >> 8; }
 
 // get_scale_min_k4 (crates/infr-gguf/src/dequant.rs:77-87).
 __device__ __forceinline__ void k4(int j, const uint8_t* q, uint32_t& sc, uint32_t& m) {
@@ -237,6 +269,62 @@ __device__ inline float decode_elem(int dtype, const uint8_t* row, uint32_t k) {
             float scf = __fmul_rn(d, (float)s);
             float mn = __fmul_rn(d, (float)(-32 * s));
             return __fadd_rn(__fmul_rn(scf, (float)code), mn);
+        }
+        case INFR_IQ4_NL: {
+            // [f16 d][16 nibble bytes] (dequant.rs:499-519): element j < 16 low nibble of byte j, j + 16 the high one
+            const uint8_t* blk = row + (size_t)(k >> 5) * 18u;
+            const uint32_t e = k & 31u, v = blk[2 + (e & 15u)];
+            return __fmul_rn(f16_bits_to_f32(ldu<uint16_t>(blk)), (float)book16(kIq4nlLo, kIq4nlHi, e < 16u ? v & 0xFu : v >> 4));
+        }
+        case INFR_IQ4_XS: {
+            // [f16 d][u16 scales_h][4 scales_l][128 qs] (dequant.rs:521-559): sub-block ib of 32 elements has the
+            // 6-bit scale nibble ib of scales_l | field ib of scales_h << 4, minus 32; codes as in IQ4_NL
+            const uint8_t* blk = row + (size_t)(k >> 8) * 136u;
+            const uint32_t w = k & 255u, ib = w >> 5, e = w & 31u;
+            const uint32_t lo = ((uint32_t)blk[4 + (ib >> 1)] >> (4u * (ib & 1u))) & 0xFu;
+            const uint32_t hi = ((uint32_t)ldu<uint16_t>(blk + 2) >> (2u * ib)) & 3u;
+            const float dl = __fmul_rn(f16_bits_to_f32(ldu<uint16_t>(blk)), (float)((int)(lo | (hi << 4)) - 32));
+            const uint32_t v = blk[8 + 16u * ib + (e & 15u)];
+            return __fmul_rn(dl, (float)book16(kIq4nlLo, kIq4nlHi, e < 16u ? v & 0xFu : v >> 4));
+        }
+        case INFR_TQ1_0: {
+            // [48 qs][4 qh][f16 d] (dequant.rs:926-970): elements 0..159 = digit n of qs[m], n * 32 + m;
+            // 160..239 = digit n of qs[32 + m], n * 16 + m; 240..255 = digit n of qh[j], n * 4 + j
+            const uint8_t* blk = row + (size_t)(k >> 8) * 54u;
+            const uint32_t w = k & 255u;
+            uint32_t byte, n;
+            if (w < 160u) { n = w >> 5; byte = blk[w & 31u]; }
+            else if (w < 240u) { n = (w - 160u) >> 4; byte = blk[32u + (w & 15u)]; }
+            else { n = (w - 240u) >> 2; byte = blk[48u + (w & 3u)]; }
+            const uint32_t p3 = n == 0u ? 1u : n == 1u ? 3u : n == 2u ? 9u : n == 3u ? 27u : 81u;
+            return __fmul_rn((float)((int)trit(byte, p3) - 1), f16_bits_to_f32(ldu<uint16_t>(blk + 52)));
+        }
+        case INFR_TQ2_0: {
+            // [64 qs][f16 d] (dequant.rs:978-1000): element 128 c + 32 l + m = field l of qs[32 c + m]
+            const uint8_t* blk = row + (size_t)(k >> 8) * 66u;
+            const uint32_t w = k & 255u;
+            const uint32_t q = ((uint32_t)blk[32u * (w >> 7) + (w & 31u)] >> (2u * ((w >> 5) & 3u))) & 3u;
+            return __fmul_rn((float)((int)q - 1), f16_bits_to_f32(ldu<uint16_t>(blk + 64)));
+        }
+        case INFR_Q2_0: {
+            // [f16 d][16 qs] (dequant.rs:1007-1022): element j = field j % 4 of qs[j / 4]
+            const uint8_t* blk = row + (size_t)(k >> 6) * 18u;
+            const uint32_t j = k & 63u;
+            const uint32_t q = ((uint32_t)blk[2u + (j >> 2)] >> (2u * (j & 3u))) & 3u;
+            return __fmul_rn((float)((int)q - 1), f16_bits_to_f32(ldu<uint16_t>(blk)));
+        }
+        case INFR_MXFP4: {
+            // [u8 e][16 nibble bytes] (dequant.rs:1029-1045): nibble order of IQ4_NL, scale 2^(e - 128)
+            const uint8_t* blk = row + (size_t)(k >> 5) * 17u;
+            const uint32_t e = k & 31u, v = blk[1 + (e & 15u)];
+            return __fmul_rn((float)book16(kFp4Lo, kFp4Hi, e < 16u ? v & 0xFu : v >> 4), e8m0_half(blk[0]));
+        }
+        case INFR_NVFP4: {
+            // [4 ue4m3 scales][32 qs] (dequant.rs:1053-1073): sub-block s of 16 elements: element j < 8 low
+            // nibble of qs[8 s + j], element j + 8 the high one
+            const uint8_t* blk = row + (size_t)(k >> 6) * 36u;
+            const uint32_t w = k & 63u, s = w >> 4, e = w & 15u, v = blk[4u + 8u * s + (e & 7u)];
+            return __fmul_rn((float)book16(kFp4Lo, kFp4Hi, e < 8u ? v & 0xFu : v >> 4), ue4m3_half(blk[s]));
         }
         default: return 0.0f;
     }

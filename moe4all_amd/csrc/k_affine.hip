@@ -1,11 +1,12 @@
 // Dense Op::Linear GEMV for every affine GGUF format (Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q2_K, Q3_K,
-// Q4_K, Q5_K, Q6_K) through one common shape: a row is cut into 32-element units; a unit decodes to
+// Q4_K, Q5_K, Q6_K) and the scale-times-code formats (IQ4_NL, IQ4_XS, MXFP4, NVFP4, TQ1_0, TQ2_0, Q2_0,
+// their codes shifted to unsigned bytes) through one common shape: a row is cut into 32-element units; a unit decodes to
 // 32 unsigned byte codes (eight dwords) plus one (scale, min) pair per 16 elements, and
 //     dot(unit, x) = sum_h  sc[h] * sum_{e in half h} code[e] * x[e]  +  mn[h] * sum_{e in half h} x[e].
 // The byte -> float conversion is one instruction per element (the compiler selects the
 // byte-lane convert for (q >> 8b) & 0xFF), the sums of x per 16 elements are computed once per
 // block while the activation row is staged in LDS, and the formats only differ in how the eight
-// dwords and the two pairs are cut out of the block (crates/infr-gguf/src/dequant.rs:137-389).
+// dwords and the two pairs are cut out of the block (crates/infr-gguf/src/dequant.rs:137-389, :499-1073).
 //
 // The formats with their own integer-dot kernels (Q4_K, Q6_K, Q8_0) only come here for shapes those
 // kernels do not take.  Work split: a block of four waves stages up to four activation rows, each
@@ -388,9 +389,8 @@ void launch_moe_units_bucketed_dt(hipStream_t s, const MoeGemvParams& p, int n_p
 template <bool GATE_UP>
 void launch_moe_units_bucketed_any(hipStream_t s, int dt, const MoeGemvParams& p, int n_pairs) {
     switch (dt) {
-#define INFR_UNITS(D) case D: launch_moe_units_bucketed_dt<D, GATE_UP>(s, p, n_pairs); break
-        INFR_UNITS(INFR_Q4_0); INFR_UNITS(INFR_Q4_1); INFR_UNITS(INFR_Q5_0); INFR_UNITS(INFR_Q5_1); INFR_UNITS(INFR_Q8_0);
-        INFR_UNITS(INFR_Q2K); INFR_UNITS(INFR_Q3K); INFR_UNITS(INFR_Q4K); INFR_UNITS(INFR_Q5K); INFR_UNITS(INFR_Q6K);
+#define INFR_UNITS(D) case D: launch_moe_units_bucketed_dt<D, GATE_UP>(s, p, n_pairs); break;
+        INFR_FOR_UNIT_FORMATS(INFR_UNITS)
 #undef INFR_UNITS
         default: break;
     }
@@ -415,9 +415,8 @@ void launch_moe_units_dt(hipStream_t s, const MoeGemvParams& p) {
 template <bool GATE_UP>
 void launch_moe_units_any(hipStream_t s, int dt, const MoeGemvParams& p) {
     switch (dt) {
-#define INFR_UNITS(D) case D: launch_moe_units_dt<D, GATE_UP>(s, p); break
-        INFR_UNITS(INFR_Q4_0); INFR_UNITS(INFR_Q4_1); INFR_UNITS(INFR_Q5_0); INFR_UNITS(INFR_Q5_1); INFR_UNITS(INFR_Q8_0);
-        INFR_UNITS(INFR_Q2K); INFR_UNITS(INFR_Q3K); INFR_UNITS(INFR_Q4K); INFR_UNITS(INFR_Q5K); INFR_UNITS(INFR_Q6K);
+#define INFR_UNITS(D) case D: launch_moe_units_dt<D, GATE_UP>(s, p); break;
+        INFR_FOR_UNIT_FORMATS(INFR_UNITS)
 #undef INFR_UNITS
         default: break;
     }
@@ -553,13 +552,8 @@ void launch_float_dt(hipStream_t s, const float* x, const uint8_t* w, size_t row
 }  // namespace
 
 bool linear_units_supported(int dt, int in_f, const void* x) {
-    switch (dt) {
-        case INFR_Q4_0: case INFR_Q4_1: case INFR_Q5_0: case INFR_Q5_1: case INFR_Q8_0: break;
-        case INFR_Q2K: case INFR_Q3K: case INFR_Q4K: case INFR_Q5K: case INFR_Q6K:
-            if (in_f % 256) return false;
-            break;
-        default: return false;
-    }
+    const int block = unit_format_block(dt);
+    if (block == 0 || in_f % block) return false;
     return in_f >= 32 && in_f % 32 == 0 && units_lds_bytes(1, in_f) <= 144 * 1024 && ((uintptr_t)x & 15) == 0;
 }
 
@@ -603,9 +597,8 @@ void launch_linear_float(hipStream_t s, const float* x, const uint8_t* w, int dt
 void launch_linear_units(hipStream_t s, const float* x, const uint8_t* w, int dt, size_t row_bytes, int m, int in_f,
                          int out_f, float* dst, const float* addend) {
     switch (dt) {
-#define INFR_UNITS(D) case D: launch_units_dt<D>(s, x, w, row_bytes, m, in_f, out_f, dst, addend); break
-        INFR_UNITS(INFR_Q4_0); INFR_UNITS(INFR_Q4_1); INFR_UNITS(INFR_Q5_0); INFR_UNITS(INFR_Q5_1); INFR_UNITS(INFR_Q8_0);
-        INFR_UNITS(INFR_Q2K); INFR_UNITS(INFR_Q3K); INFR_UNITS(INFR_Q4K); INFR_UNITS(INFR_Q5K); INFR_UNITS(INFR_Q6K);
+#define INFR_UNITS(D) case D: launch_units_dt<D>(s, x, w, row_bytes, m, in_f, out_f, dst, addend); break;
+        INFR_FOR_UNIT_FORMATS(INFR_UNITS)
 #undef INFR_UNITS
         default: break;
     }

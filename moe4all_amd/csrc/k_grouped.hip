@@ -1043,10 +1043,9 @@ void grouped_units(hipStream_t s, const GroupedParams& p) {
 template <bool DOWN>
 void grouped_units_any(hipStream_t s, int dt, const GroupedParams& p) {
     switch (dt) {
-#define INFR_UNITS(D) case D: grouped_units<D, DOWN>(s, p); break
-        INFR_UNITS(INFR_Q4_0); INFR_UNITS(INFR_Q4_1); INFR_UNITS(INFR_Q5_0); INFR_UNITS(INFR_Q5_1); INFR_UNITS(INFR_Q8_0);
-        INFR_UNITS(INFR_Q2K); INFR_UNITS(INFR_Q3K); INFR_UNITS(INFR_Q4K); INFR_UNITS(INFR_Q5K); INFR_UNITS(INFR_Q6K);
-        INFR_UNITS(INFR_F16); INFR_UNITS(INFR_BF16); INFR_UNITS(INFR_F32);
+#define INFR_UNITS(D) case D: grouped_units<D, DOWN>(s, p); break;
+        INFR_FOR_UNIT_FORMATS(INFR_UNITS)
+        INFR_UNITS(INFR_F16) INFR_UNITS(INFR_BF16) INFR_UNITS(INFR_F32)
 #undef INFR_UNITS
         default: break;
     }
@@ -1059,12 +1058,9 @@ void grouped_units_any(hipStream_t s, int dt, const GroupedParams& p) {
 // for a format without an LDS layout of its own, e.g. INFR_Q5K).
 bool grouped_units_supported(int dt, int k) {
     if (k <= 0 || k % kSlice != 0) return false;
-    switch (dt) {
-        case INFR_Q4_0: case INFR_Q4_1: case INFR_Q5_0: case INFR_Q5_1: case INFR_Q8_0: return true;
-        case INFR_Q2K: case INFR_Q3K: case INFR_Q4K: case INFR_Q5K: case INFR_Q6K: return k % 256 == 0;
-        case INFR_F16: case INFR_BF16: case INFR_F32: return true;   // rounded to f16 (weights beyond 65504 would not fit)
-        default: return false;
-    }
+    if (dt == INFR_F16 || dt == INFR_BF16 || dt == INFR_F32) return true;   // rounded to f16 (weights beyond 65504 would not fit)
+    const int block = unit_format_block(dt);
+    return block != 0 && k % block == 0;
 }
 void launch_grouped_units_gate_up(hipStream_t s, int dt, const GroupedParams& p) { grouped_units_any<false>(s, dt, p); }
 void launch_grouped_units_down(hipStream_t s, int dt, const GroupedParams& p) { grouped_units_any<true>(s, dt, p); }

@@ -18,6 +18,7 @@ _LIB_PATH = os.path.join(_HERE, "libinfr_oracle.so")
 # infr_core::DType ordinals (crates/infr-core/src/tensor.rs:7-57)
 F32, F16, BF16, I32, U32 = 0, 1, 2, 3, 4
 Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q2K, Q3K, Q4K, Q5K, Q6K = 5, 6, 7, 8, 9, 10, 11, 12, 13, 14
+IQ4_NL, IQ4_XS, TQ1_0, TQ2_0, Q2_0, MXFP4, NVFP4 = 22, 23, 24, 25, 27, 28, 29
 ACT_SILU, ACT_GELU, ACT_SIGMOID = 0, 1, 2
 GATE_SOFTMAX, GATE_SIGMOID, GATE_SQRT_SOFTPLUS = 0, 1, 2
 

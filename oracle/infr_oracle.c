@@ -60,6 +60,14 @@ int orc_block_geometry(int dtype, int *block_elems, int *block_bytes) {
     case ORC_Q4K: e = 256; b = 144; break;
     case ORC_Q5K: e = 256; b = 176; break;
     case ORC_Q6K: e = 256; b = 210; break;
+    /* decode_spec.rs:349-363 */
+    case ORC_IQ4_NL: e = 32; b = 18; break;
+    case ORC_IQ4_XS: e = 256; b = 136; break;
+    case ORC_TQ1_0: e = 256; b = 54; break;
+    case ORC_TQ2_0: e = 256; b = 66; break;
+    case ORC_Q2_0: e = 64; b = 18; break;
+    case ORC_MXFP4: e = 32; b = 17; break;
+    case ORC_NVFP4: e = 64; b = 36; break;
     default: return -1;
     }
     if (block_elems) *block_elems = e;
@@ -246,6 +254,110 @@ static void factor_q3k(const uint8_t *blk, factored_block *f) {
             }
 }
 
+/* ------------------------------------------------------------------ scale-times-code formats
+ * dequant_codebook (crates/infr-gguf/src/dequant.rs:493-1073) for the formats whose book fits in
+ * sixteen entries or is arithmetic: one block in, its elements out, value = code * scale with the
+ * reference's operand order. */
+static const int8_t BOOK_IQ4NL[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113}; /* :442-444 */
+static const int8_t BOOK_FP4[16] = {0, 1, 2, 3, 4, 6, 8, 12, 0, -1, -2, -3, -4, -6, -8, -12};                    /* :409 */
+
+/* e8m0_to_fp32_half (dequant.rs:415-421) */
+static float e8m0_half(uint8_t x) {
+    uint32_t bits = x < 2 ? 0x00200000u << x : ((uint32_t)x - 1u) << 23;
+    float f;
+    memcpy(&f, &bits, 4);
+    return f;
+}
+
+/* ue4m3_to_fp32 (dequant.rs:427-438) */
+static float ue4m3_half(uint8_t x) {
+    if (x == 0 || x == 0x7F) return 0.0f;
+    int exp = (x >> 3) & 0xF;
+    float man = (float)(x & 7);
+    float raw = exp == 0 ? man * ldexpf(1.0f, -9) : (1.0f + man / 8.0f) * ldexpf(1.0f, exp - 7);
+    return raw * 0.5f;
+}
+
+static int codebook_block(int dtype, const uint8_t *blk, float *out) {
+    switch (dtype) {
+    case ORC_IQ4_NL: { /* :499-519 */
+        float d = orc_f16_to_f32(rd_u16(blk));
+        for (int j = 0; j < 16; j++) {
+            out[j] = d * (float)BOOK_IQ4NL[blk[2 + j] & 0xF];
+            out[j + 16] = d * (float)BOOK_IQ4NL[blk[2 + j] >> 4];
+        }
+        return 0;
+    }
+    case ORC_IQ4_XS: { /* :521-559 */
+        float d = orc_f16_to_f32(rd_u16(blk));
+        unsigned scales_h = rd_u16(blk + 2);
+        for (int ib = 0; ib < 8; ib++) {
+            int ls = ((blk[4 + ib / 2] >> (4 * (ib % 2))) & 0xF) | (((scales_h >> (2 * ib)) & 3) << 4);
+            float dl = d * (float)(ls - 32);
+            const uint8_t *qs = blk + 8 + 16 * ib;
+            for (int j = 0; j < 16; j++) {
+                out[32 * ib + j] = dl * (float)BOOK_IQ4NL[qs[j] & 0xF];
+                out[32 * ib + j + 16] = dl * (float)BOOK_IQ4NL[qs[j] >> 4];
+            }
+        }
+        return 0;
+    }
+    case ORC_TQ1_0: { /* :926-970: five ternary digits per byte, most significant first after the multiply */
+        static const uint8_t pow3[5] = {1, 3, 9, 27, 81};
+        float d = orc_f16_to_f32(rd_u16(blk + 52));
+        float *o = out;
+        for (int n = 0; n < 5; n++)
+            for (int m = 0; m < 32; m++) {
+                uint8_t q = (uint8_t)(blk[m] * pow3[n]);
+                *o++ = (float)((int)(((unsigned)q * 3u) >> 8) - 1) * d;
+            }
+        for (int n = 0; n < 5; n++)
+            for (int m = 0; m < 16; m++) {
+                uint8_t q = (uint8_t)(blk[32 + m] * pow3[n]);
+                *o++ = (float)((int)(((unsigned)q * 3u) >> 8) - 1) * d;
+            }
+        for (int n = 0; n < 4; n++)
+            for (int j = 0; j < 4; j++) {
+                uint8_t q = (uint8_t)(blk[48 + j] * pow3[n]);
+                *o++ = (float)((int)(((unsigned)q * 3u) >> 8) - 1) * d;
+            }
+        return 0;
+    }
+    case ORC_TQ2_0: { /* :978-1000 */
+        float d = orc_f16_to_f32(rd_u16(blk + 64));
+        float *o = out;
+        for (int chunk = 0; chunk < 2; chunk++)
+            for (int l = 0; l < 4; l++)
+                for (int m = 0; m < 32; m++) *o++ = (float)(((blk[32 * chunk + m] >> (2 * l)) & 3) - 1) * d;
+        return 0;
+    }
+    case ORC_Q2_0: { /* :1007-1022 */
+        float d = orc_f16_to_f32(rd_u16(blk));
+        for (int j = 0; j < 64; j++) out[j] = (float)(((blk[2 + j / 4] >> (2 * (j % 4))) & 3) - 1) * d;
+        return 0;
+    }
+    case ORC_MXFP4: { /* :1029-1045 */
+        float d = e8m0_half(blk[0]);
+        for (int j = 0; j < 16; j++) {
+            out[j] = (float)BOOK_FP4[blk[1 + j] & 0xF] * d;
+            out[j + 16] = (float)BOOK_FP4[blk[1 + j] >> 4] * d;
+        }
+        return 0;
+    }
+    case ORC_NVFP4: { /* :1053-1073 */
+        for (int s = 0; s < 4; s++) {
+            float d = ue4m3_half(blk[s]);
+            for (int j = 0; j < 8; j++) {
+                out[16 * s + j] = (float)BOOK_FP4[blk[4 + 8 * s + j] & 0xF] * d;
+                out[16 * s + j + 8] = (float)BOOK_FP4[blk[4 + 8 * s + j] >> 4] * d;
+            }
+        }
+        return 0;
+    }
+    default: return -1;
+    }
+}
+
 /* dequant.rs:336-363: Q4_K's layout with 32 bytes of fifth bits between the scales and the
  * nibbles: bit 2j of qh[l] belongs to the low-nibble element, bit 2j+1 to the high-nibble one. */
 static void factor_q5k(const uint8_t *blk, factored_block *f) {
@@ -308,7 +420,9 @@ int64_t orc_dequant(int dtype, const uint8_t *bytes, size_t nbytes, float *out) 
         case ORC_Q8_0: factor_q8_0(blk, &f); break;
         case ORC_Q4K: factor_q4k(blk, &f); break;
         case ORC_Q6K: factor_q6k(blk, &f); break;
-        default: return -1;
+        default:
+            if (codebook_block(dtype, blk, out + b * (size_t)be) != 0) return -1;
+            continue;
         }
         expand_block(&f, be, out + b * (size_t)be);
     }

@@ -26,7 +26,8 @@ extern "C" {
 enum orc_dtype {
     ORC_F32 = 0, ORC_F16 = 1, ORC_BF16 = 2, ORC_I32 = 3, ORC_U32 = 4,
     ORC_Q4_0 = 5, ORC_Q4_1 = 6, ORC_Q5_0 = 7, ORC_Q5_1 = 8, ORC_Q8_0 = 9,
-    ORC_Q2K = 10, ORC_Q3K = 11, ORC_Q4K = 12, ORC_Q5K = 13, ORC_Q6K = 14
+    ORC_Q2K = 10, ORC_Q3K = 11, ORC_Q4K = 12, ORC_Q5K = 13, ORC_Q6K = 14,
+    ORC_IQ4_NL = 22, ORC_IQ4_XS = 23, ORC_TQ1_0 = 24, ORC_TQ2_0 = 25, ORC_Q2_0 = 27, ORC_MXFP4 = 28, ORC_NVFP4 = 29
 };
 /* infr_core::graph::Activation (graph.rs:47-54) and MoeGating (graph.rs:73-85). */
 enum orc_activation { ORC_ACT_SILU = 0, ORC_ACT_GELU = 1, ORC_ACT_SIGMOID = 2 };

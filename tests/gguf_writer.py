@@ -7,7 +7,8 @@ U8, I8, U16, I16, U32, I32, F32, BOOL, STR, ARR, U64, I64, F64 = range(13)
 _FMT = {U8: "<B", I8: "<b", U16: "<H", I16: "<h", U32: "<I", I32: "<i", F32: "<f", BOOL: "<B", U64: "<Q", I64: "<q",
         F64: "<d"}
 GGML = {"F32": 0, "F16": 1, "Q4_0": 2, "Q4_1": 3, "Q5_0": 6, "Q5_1": 7, "Q8_0": 8, "Q2K": 10, "Q3K": 11, "Q4K": 12,
-        "Q5K": 13, "Q6K": 14, "I32": 26, "BF16": 30, "I2S": 36}
+        "Q5K": 13, "Q6K": 14, "IQ4_NL": 20, "IQ4_XS": 23, "I32": 26, "BF16": 30, "TQ1_0": 34, "TQ2_0": 35, "I2S": 36,
+        "MXFP4": 39, "NVFP4": 40, "Q2_0": 42}
 
 
 def gstr(s) -> bytes:

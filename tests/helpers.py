@@ -7,11 +7,15 @@ import numpy as np
 
 F32, F16, BF16 = 0, 1, 2
 Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q2K, Q3K, Q4K, Q5K, Q6K = 5, 6, 7, 8, 9, 10, 11, 12, 13, 14
-BLOCK = {Q8_0: (32, 34), Q4K: (256, 144), Q6K: (256, 210), F32: (1, 4), F16: (1, 2), BF16: (1, 2),
+IQ4_NL, IQ4_XS, TQ1_0, TQ2_0, Q2_0, MXFP4, NVFP4 = 22, 23, 24, 25, 27, 28, 29
+SCALE_CODE = (IQ4_NL, IQ4_XS, TQ1_0, TQ2_0, Q2_0, MXFP4, NVFP4)   # value = scale * small signed code
+BLOCK = {IQ4_NL: (32, 18), IQ4_XS: (256, 136), TQ1_0: (256, 54), TQ2_0: (256, 66), Q2_0: (64, 18), MXFP4: (32, 17),
+         NVFP4: (64, 36),
+         Q8_0: (32, 34), Q4K: (256, 144), Q6K: (256, 210), F32: (1, 4), F16: (1, 2), BF16: (1, 2),
          Q4_0: (32, 18), Q4_1: (32, 20), Q5_0: (32, 22), Q5_1: (32, 24), Q2K: (256, 84), Q3K: (256, 110), Q5K: (256, 176)}
 # byte offsets of the f16 scale fields inside a block
 F16_SLOTS = {Q4_0: (0,), Q4_1: (0, 2), Q5_0: (0,), Q5_1: (0, 2), Q8_0: (0,), Q2K: (80, 82), Q3K: (108,), Q4K: (0, 2),
-             Q5K: (0, 2), Q6K: (208,)}
+             Q5K: (0, 2), Q6K: (208,), IQ4_NL: (0,), IQ4_XS: (0,), TQ1_0: (52,), TQ2_0: (64,), Q2_0: (0,)}
 
 
 # ---- generators of the reference's tests ------------------------------------------------
@@ -48,6 +52,14 @@ def synth_weight(dtype: int, n_elem: int, seed: int) -> np.ndarray:
     elif dtype == Q8_0:
         blk = lcg_bytes_blocks(seed, nblk, 34)
         blk[:, 0:2] = f16_bytes(0.01)
+    elif dtype == MXFP4:
+        # LCG nibbles, shared exponents 2^-11 .. 2^-8 (byte 117..120)
+        blk = lcg_bytes_blocks(seed, nblk, bb)
+        blk[:, 0] = 117 + (blk[:, 0] & 3)
+    elif dtype == NVFP4:
+        # LCG nibbles, the four sub-block scales with exponent field 0..3 (subnormal and normal, up to 2^-4)
+        blk = lcg_bytes_blocks(seed, nblk, bb)
+        blk[:, 0:4] &= 0x1F
     elif dtype in F16_SLOTS:
         # the remaining affine formats: LCG payload everywhere, then finite scales of either sign
         blk = lcg_bytes_blocks(seed, nblk, bb)
@@ -63,10 +75,13 @@ def centred_weight(dtype: int, n_elem: int, seed: int, band: float = 0.02) -> np
     magnitude ~band, like trained weights: the min term of the formats that have one cancels the mean of
     the scaled codes (Q4_1: m = -7.5 d; Q5_1: -15.5 d; Q2_K: dmin = 1.5 d; Q4_K, Q5_K: dmin = mean code * d)."""
     blk = synth_weight(dtype, n_elem, seed).reshape(-1, BLOCK[dtype][1])
+    if dtype in (MXFP4, NVFP4):   # symmetric books, scales already of that order
+        return blk.reshape(-1)
     # (d, second scale) per format; code ranges: q4 0..15, q5 0..31, 6-bit sub-scales mean 31.5, 4-bit 7.5
     d2 = {Q4_0: (band / 4,), Q5_0: (band / 8,), Q8_0: (band / 64,), Q4_1: (band / 4, -7.5 * band / 4),
           Q5_1: (band / 8, -15.5 * band / 8), Q2K: (band / 8, 1.5 * band / 8), Q3K: (band / 32,),
-          Q4K: (band / 128, 7.5 * band / 128), Q5K: (band / 256, 15.5 * band / 256), Q6K: (band / 1024,)}[dtype]
+          Q4K: (band / 128, 7.5 * band / 128), Q5K: (band / 256, 15.5 * band / 256), Q6K: (band / 1024,),
+          IQ4_NL: (band / 64,), IQ4_XS: (band / 1024,), TQ1_0: (band,), TQ2_0: (band,), Q2_0: (band,)}[dtype]
     for off, v in zip(F16_SLOTS[dtype], d2):
         blk[:, off:off + 2] = f16_bytes(v)
     return blk.reshape(-1)
@@ -234,7 +249,64 @@ def ggml_dequant(dtype: int, data: np.ndarray) -> np.ndarray:
             nib = ((q & 0xF) if is_ % 2 == 0 else (q >> 4)) + 16 * ((qh >> is_) & 1)
             y[:, is_ * 32:(is_ + 1) * 32] = (d * sc)[:, None] * nib - (dmin * m)[:, None]
         return y.reshape(-1)
+    if dtype in (IQ4_NL, IQ4_XS):
+        # ggml dequantize_row_iq4_nl / iq4_xs: kvalues_iq4nl[nibble] * d (* (ls - 32), ls = 6-bit sub-block scale)
+        kv = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], np.longdouble)
+        d = _f16(blk[:, 0:2])
+        if dtype == IQ4_NL:
+            qs = blk[:, 2:18].astype(np.int64)
+            return (np.concatenate([kv[qs & 0xF], kv[qs >> 4]], axis=1) * d[:, None]).reshape(-1)
+        sh = blk[:, 2:4].copy().view(np.uint16).reshape(-1).astype(np.int64)
+        sl = blk[:, 4:8].astype(np.int64)
+        qs = blk[:, 8:136].astype(np.int64).reshape(nb, 8, 16)
+        ib = np.arange(8)
+        ls = ((sl[:, ib // 2] >> (4 * (ib % 2))) & 0xF) | (((sh[:, None] >> (2 * ib)) & 3) << 4)
+        y = np.concatenate([kv[qs & 0xF], kv[qs >> 4]], axis=2) * (d[:, None] * (ls - 32))[:, :, None]
+        return y.reshape(-1)
+    if dtype in (MXFP4, NVFP4):
+        # the 4-bit codes are E2M1 floats (sign, 2-bit exponent of bias 1, 1-bit mantissa), decoded arithmetically
+        # here; the scale is E8M0 (2^(e - 127)) per 32 elements, or UE4M3 (4-bit exponent of bias 7, 3-bit mantissa,
+        # 0x00 and the NaN code 0x7F giving 0) per 16 elements
+        def e2m1(q):
+            e, m = (q >> 1) & 3, q & 1
+            mag = np.where(e == 0, m * 0.5, (1 + m * 0.5) * np.exp2(e - 1.0))
+            return np.where(q & 8, -mag, mag).astype(np.longdouble) + 0.0   # ggml's integer table has no -0: code 8 is +0
+        if dtype == MXFP4:
+            scale = np.ldexp(np.longdouble(1), blk[:, 0].astype(np.int64) - 127)
+            qs = blk[:, 1:17].astype(np.int64)
+            return (np.concatenate([e2m1(qs & 0xF), e2m1(qs >> 4)], axis=1) * scale[:, None]).reshape(-1)
+        sb = blk[:, 0:4].astype(np.int64)
+        e, m = (sb >> 3) & 0xF, sb & 7
+        scale = np.where(e == 0, np.ldexp(m.astype(np.longdouble), -9), np.ldexp((8 + m).astype(np.longdouble), e - 10))
+        scale = np.where((sb == 0) | (sb == 0x7F), 0, scale)
+        qs = blk[:, 4:36].astype(np.int64).reshape(nb, 4, 8)
+        return (np.concatenate([e2m1(qs & 0xF), e2m1(qs >> 4)], axis=2) * scale[:, :, None]).reshape(-1)
+    if dtype == TQ2_0:
+        # ggml dequantize_row_tq2_0: two runs of 32 bytes, their four 2-bit fields field-major
+        qs = blk[:, 0:64].astype(np.int64).reshape(nb, 2, 1, 32)
+        q = (qs >> (2 * np.arange(4)).reshape(1, 1, 4, 1)) & 3
+        return ((q - 1).reshape(nb, 256) * _f16(blk[:, 64:66])[:, None]).reshape(-1)
+    if dtype == Q2_0:
+        q = (blk[:, 2:18].astype(np.int64)[:, :, None] >> (2 * np.arange(4))) & 3   # fields of a byte are consecutive elements
+        return ((q - 1).reshape(nb, 64) * _f16(blk[:, 0:2])[:, None]).reshape(-1)
+    if dtype == TQ1_0:
+        # ggml dequantize_row_tq1_0: a byte q holds five ternary digits as the fraction q / 256 in base 3, first digit
+        # = floor(3 * frac(q / 256)), digit n = the same of frac(q * 3^n / 256); runs of 32, 16 and 4 bytes, digit-major
+        def digits(b, n):
+            q = b.astype(np.int64)[:, None, :] * (3 ** np.arange(n)).reshape(1, n, 1)
+            return ((q % 256) * 3) // 256
+        y = np.concatenate([digits(blk[:, 0:32], 5).reshape(nb, -1), digits(blk[:, 32:48], 5).reshape(nb, -1),
+                            digits(blk[:, 48:52], 4).reshape(nb, -1)], axis=1)
+        return ((y - 1) * _f16(blk[:, 52:54])[:, None]).reshape(-1)
     raise ValueError(dtype)
+
+
+def tq1_0_pack(trits: np.ndarray) -> np.ndarray:
+    """ggml quantize_row_tq1_0_ref's byte: five digits t0..t4 in {0, 1, 2}, most significant first, stored as
+    ceil(value * 256 / 243) so that multiplying by 3^n brings digit n to the top."""
+    t = np.asarray(trits, np.int64).reshape(-1, 5)
+    v = t @ np.array([81, 27, 9, 3, 1])
+    return ((v * 256 + 242) // 243).astype(np.uint8)
 
 
 # ---- independent f64 model of Op::MoeFfn (shape of moe_ref / moe_v4_ref) -----------------
@@ -338,6 +410,13 @@ def dequant_cases():
     for name, dt in (("q4_0", Q4_0), ("q4_1", Q4_1), ("q5_0", Q5_0), ("q5_1", Q5_1), ("q2k", Q2K), ("q3k", Q3K), ("q5k", Q5K)):
         out[f"{name}_all_formats_pattern"] = (dt, pattern(2 * BLOCK[dt][1], 29, 3))
         out[f"{name}_lcg"] = (dt, synth_weight(dt, BLOCK[dt][0] * 8, 100 + dt))
+    for name, dt in (("iq4_nl", IQ4_NL), ("iq4_xs", IQ4_XS), ("tq1_0", TQ1_0), ("tq2_0", TQ2_0), ("q2_0", Q2_0),
+                     ("mxfp4", MXFP4), ("nvfp4", NVFP4)):
+        b = pattern(2 * BLOCK[dt][1], 29, 3)
+        if dt == MXFP4:   # keep the shared exponents of the pattern inside f32 after the multiply by 12
+            b[0::17] = 64 + (b[0::17] >> 1)
+        out[f"{name}_pattern"] = (dt, b)
+        out[f"{name}_lcg"] = (dt, synth_weight(dt, BLOCK[dt][0] * 8, 100 + dt))
     for name, (dt, b, _) in known_answer_blocks().items():
         out[name] = (dt, b)
     return out
@@ -372,6 +451,28 @@ def known_answer_blocks():
     b[0:2], b[2:4] = f16_bytes(2.0), f16_bytes(-1.0)
     b[8] = 0x1F
     out["q5_1_single_block"] = (Q5_1, b, {0: 29.0, 16: 1.0})
+    # the scale-times-code formats (dequant.rs:1228-1432)
+    b = np.zeros(18, np.uint8)          # iq4nl_single_block: d = 1, qs[0] = 0x80
+    b[0:2] = f16_bytes(1.0)
+    b[2] = 0x80
+    out["iq4nl_single_block"] = (IQ4_NL, b, {0: -127.0, 16: 1.0})
+    b = np.zeros(136, np.uint8)         # iq4xs_single_block: d = 1, everything else 0 -> -32 * -127
+    b[0:2] = f16_bytes(1.0)
+    out["iq4xs_single_block"] = (IQ4_XS, b, {i: 4064.0 for i in range(256)})
+    b = np.zeros(17, np.uint8)          # mxfp4_single_block: e = 128, qs[0] = 0x21
+    b[0], b[1] = 128, 0x21
+    out["mxfp4_single_block"] = (MXFP4, b, {0: 1.0, 16: 2.0, **{i: 0.0 for i in range(1, 16)}})
+    out["nvfp4_single_block"] = (NVFP4, np.zeros(36, np.uint8), {i: 0.0 for i in range(64)})
+    b = np.zeros(54, np.uint8)          # tq1_0_single_block: d = 1
+    b[52:54] = f16_bytes(1.0)
+    out["tq1_0_single_block"] = (TQ1_0, b, {i: -1.0 for i in range(256)})
+    b = np.zeros(66, np.uint8)          # tq2_0_single_block: d = 1
+    b[64:66] = f16_bytes(1.0)
+    out["tq2_0_single_block"] = (TQ2_0, b, {i: -1.0 for i in range(256)})
+    b = np.zeros(18, np.uint8)          # q2_0_single_block: d = 0.5, qs[0] = 0b11100100
+    b[0:2] = f16_bytes(0.5)
+    b[2] = 0b11100100
+    out["q2_0_single_block"] = (Q2_0, b, {0: -0.5, 1: 0.0, 2: 0.5, 3: 1.0, **{i: -0.5 for i in range(4, 64)}})
     return out
 
 

@@ -72,8 +72,10 @@ int main(void) {
 
 def test_dtype_ordinals_follow_the_reference_enum():
     # crates/infr-core/src/tensor.rs:7-57
-    names = ["F32", "F16", "Bf16", "I32", "U32", "Q4_0", "Q4_1", "Q5_0", "Q5_1", "Q8_0", "Q2K", "Q3K", "Q4K", "Q5K", "Q6K"]
-    assert [d.name for d in M.DType] == names and [int(d) for d in M.DType] == list(range(15))
+    names = ["F32", "F16", "Bf16", "I32", "U32", "Q4_0", "Q4_1", "Q5_0", "Q5_1", "Q8_0", "Q2K", "Q3K", "Q4K", "Q5K", "Q6K",
+             "Iq1S", "Iq1M", "Iq2Xxs", "Iq2Xs", "Iq2S", "Iq3Xxs", "Iq3S", "Iq4Nl", "Iq4Xs", "Tq1_0", "Tq2_0", "I2S", "Q2_0",
+             "Mxfp4", "Nvfp4"]
+    assert [d.name for d in M.DType] == names and [int(d) for d in M.DType] == list(range(30))
     assert [int(u) for u in M.BufferUsage] == list(range(6))
     assert [k.name for k in M.TensorKind] == ["Input", "Weight", "Internal", "Output"]
 

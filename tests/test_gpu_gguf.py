@@ -67,7 +67,12 @@ def _moe_file(path, rng, *, ne, n_ff, E, K, layers, gdt, ddt, shards=1, shexp=0,
     return first, per_layer
 
 
-@pytest.mark.parametrize("dt", ["F32", "F16", "BF16", "Q8_0", "Q4K", "Q6K"])
+_DTYPE = {"IQ4_NL": M.DType.Iq4Nl, "IQ4_XS": M.DType.Iq4Xs, "TQ1_0": M.DType.Tq1_0, "TQ2_0": M.DType.Tq2_0,
+          "Q2_0": M.DType.Q2_0, "MXFP4": M.DType.Mxfp4, "NVFP4": M.DType.Nvfp4}
+
+
+@pytest.mark.parametrize("dt", ["F32", "F16", "BF16", "Q8_0", "Q4K", "Q6K", "IQ4_NL", "IQ4_XS", "TQ1_0", "TQ2_0", "Q2_0", "MXFP4",
+                                "NVFP4"])
 def test_bound_weight_decodes_to_the_oracle_values(be, tmp_path, dt):
     """BindWeight (alloc_uninit + upload of the file's bytes) followed by the device decode of the whole
     tensor: bit-identical to the oracle's decode of the same file bytes."""
@@ -80,7 +85,7 @@ def test_bound_weight_decodes_to_the_oracle_values(be, tmp_path, dt):
     elif dt == "BF16":
         data, code = _bf16(rng.standard_normal(n)), M.DType.Bf16
     else:
-        data, code = H.synth_weight(getattr(H, dt), n, 5), getattr(M.DType, dt)
+        data, code = H.synth_weight(getattr(H, dt), n, 5), _DTYPE.get(dt) or getattr(M.DType, dt)
     p = tmp_path / "w.gguf"
     W.write(p, [("general.architecture", W.STR, "x")], [("pad", (3,), 0, b"\0" * 12), ("w", (256, 4), W.GGML[dt], data.tobytes())])
     with G.Gguf(p) as g:
@@ -93,7 +98,8 @@ def test_bound_weight_decodes_to_the_oracle_values(be, tmp_path, dt):
     assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
 
 
-@pytest.mark.parametrize("rows,shards,gdt,ddt", [(1, 1, "Q4K", "Q6K"), (5, 2, "Q8_0", "Q8_0"), (40, 1, "Q4K", "Q6K")])
+@pytest.mark.parametrize("rows,shards,gdt,ddt", [(1, 1, "Q4K", "Q6K"), (5, 2, "Q8_0", "Q8_0"), (40, 1, "Q4K", "Q6K"),
+                                                 (1, 1, "MXFP4", "MXFP4"), (48, 1, "MXFP4", "MXFP4"), (3, 1, "IQ4_XS", "IQ4_NL")])
 def test_ffn_sublayer_from_a_gguf_file_matches_the_oracle(be, tmp_path, rows, shards, gdt, ddt):
     ne, n_ff, E, K, layers = 512, 256, 8, 2, 2
     rng = np.random.default_rng(40 + rows)

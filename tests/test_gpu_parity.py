@@ -95,9 +95,10 @@ def test_dequant_matches_golden_bits(be):
 
 
 AFFINE = [H.Q4_0, H.Q4_1, H.Q5_0, H.Q5_1, H.Q8_0, H.Q2K, H.Q3K, H.Q4K, H.Q5K, H.Q6K]
+DECODED = AFFINE + list(H.SCALE_CODE)   # every block format the device decodes
 
 
-@pytest.mark.parametrize("dt", AFFINE)
+@pytest.mark.parametrize("dt", DECODED)
 def test_dequant_matches_oracle_bits_on_a_large_tensor(be, dt):
     e, b = H.BLOCK[dt]
     raw = H.synth_weight(dt, e * 4099, seed=dt)
@@ -110,7 +111,9 @@ def test_dequant_matches_oracle_bits_on_a_large_tensor(be, dt):
 @pytest.mark.parametrize("dt,in_f", [(H.Q4K, 2048), (H.Q4K, 4096), (H.Q4K, 256), (H.Q4K, 1024), (H.Q6K, 768),
                                      (H.Q6K, 1536), (H.Q6K, 256), (H.Q6K, 4096), (H.Q8_0, 2048), (H.Q8_0, 768),
                                      (H.Q8_0, 4096), (H.Q8_0, 96), (H.Q4K, 5120), (H.F16, 100), (H.Q4_0, 96), (H.Q4_1, 2048),
-                                     (H.Q5_0, 160), (H.Q5_1, 1024), (H.Q2K, 512), (H.Q3K, 768), (H.Q5K, 2048)])
+                                     (H.Q5_0, 160), (H.Q5_1, 1024), (H.Q2K, 512), (H.Q3K, 768), (H.Q5K, 2048),
+                                     (H.IQ4_NL, 96), (H.IQ4_XS, 512), (H.TQ1_0, 256), (H.TQ1_0, 1024), (H.TQ2_0, 768),
+                                     (H.Q2_0, 192), (H.MXFP4, 2880), (H.MXFP4, 160), (H.NVFP4, 320)])
 def test_one_hot_gemv_reads_back_the_decoded_weight(be, dt, in_f):
     """x = e_c makes y[o] = W[o][c]: the in-register unpacking of the GEMV kernels must reproduce
     the reference decode exactly (same trick as crates/infr-vulkan/tests/weight_dequant_parity.rs)."""
@@ -705,11 +708,11 @@ def test_norm_moe_residual_chain_folds_into_the_moe_kernels(be, rows, shared):
 
 
 @pytest.mark.parametrize("m", [1, 3, 6])
-def test_linear_sweep_over_every_affine_weight_format(be, m):
+def test_linear_sweep_over_every_decoded_weight_format(be, m):
     """The reference's weight-format sweep for Op::Linear (crates/infr-testkit/src/lib.rs:389-403: every
     format as a LinearCase at one shape, seeds 0x201 + i) over the formats this backend decodes, at the
     sweep's 256 x 8 shape and at a decode-sized one; reference-mode tolerance (decode_parity.rs:93-102)."""
-    for i, dt in enumerate(AFFINE):
+    for i, dt in enumerate(DECODED):
         for in_f, out_f in ((256, 8), (2048, 96)):
             raw = H.synth_weight(dt, out_f * in_f, seed=0x201 + i)
             x = H.rand_f32(m * in_f, 0x301 + i).reshape(m, in_f)
@@ -744,7 +747,8 @@ def test_linear_on_float_weights(be, dt, m, in_f, out_f):
                                              (H.Q5K, 128, 512, 96), (H.Q4_0, 200, 192, 300), (H.Q3K, 133, 256, 40),
                                              (H.Q4K, 2048, 4096, 1536), (H.Q4_1, 150, 96, 64), (H.F16, 170, 256, 64),
                                              (H.BF16, 130, 320, 100), (H.F32, 260, 128, 300), (H.F16, 140, 100, 64),
-                                             (H.Q4K, 100, 512, 64)])
+                                             (H.Q4K, 100, 512, 64), (H.MXFP4, 160, 2880, 96), (H.IQ4_XS, 130, 512, 64),
+                                             (H.NVFP4, 140, 192, 50), (H.TQ2_0, 128, 256, 40), (H.IQ4_NL, 131, 96, 64)])
 def test_linear_with_a_batch_of_rows_runs_on_the_matrix_cores(be, dt, m, in_f, out_f):
     """Op::Linear from 128 rows on (a prefill chunk through a dense projection or the shared expert): the rows
     are one bucket of the grouped GEMMs, f16 operands with a power-of-two scale per row, bar 1e-2 per row.
@@ -799,7 +803,10 @@ def test_batched_linear_reads_a_row_band_of_a_concatenated_weight(be):
     (H.Q3K, H.Q2K, 5, 512, 256), (H.Q5_1, H.Q4_0, 1, 512, 256),
     (H.Q5K, H.Q6K, 40, 512, 256), (H.Q4_0, H.Q4_1, 77, 512, 256), (H.Q5K, H.Q5K, 300, 512, 256), (H.Q2K, H.Q3K, 130, 256, 512),
     (H.Q5_0, H.Q5_1, 64, 192, 320), (H.Q8_0, H.Q4_0, 33, 2048, 64),
-    (H.Q4_0, H.Q5_0, 40, 480, 96), (H.Q4_1, H.Q4_1, 70, 96, 32)])
+    (H.Q4_0, H.Q5_0, 40, 480, 96), (H.Q4_1, H.Q4_1, 70, 96, 32),
+    (H.MXFP4, H.MXFP4, 1, 512, 256), (H.MXFP4, H.MXFP4, 64, 512, 256), (H.IQ4_XS, H.IQ4_NL, 3, 512, 256),
+    (H.IQ4_NL, H.IQ4_XS, 40, 512, 256), (H.NVFP4, H.Q2_0, 2, 512, 256), (H.TQ2_0, H.TQ1_0, 5, 512, 256),
+    (H.TQ1_0, H.TQ2_0, 50, 256, 256), (H.Q2_0, H.NVFP4, 35, 192, 320), (H.MXFP4, H.IQ4_NL, 40, 480, 96)])
 def test_moe_ffn_with_experts_in_the_other_affine_formats(be, gdt, ddt, rows, ne, nff):
     """Expert banks in formats without an integer-dot kernel.  Up to 31 rows: the 32-element-unit GEMV kernels,
     one block column per (row, rank) pair (f32, bar 1e-3).  From 32 rows: bucketing + the unit-decoder grouped
@@ -837,6 +844,35 @@ def test_moe_ffn_with_experts_in_the_other_affine_formats(be, gdt, ddt, rows, ne
         assert {"moe_gate_up_units_bucketed", "moe_down_units_bucketed", "moe_unbucket_combine"} <= names
     else:
         assert "moe_gate_up_units" in names and ("moe_down_units" in names or ddt == H.Q6K)
+    keep[0].free()
+    for buf in keep[2] + [keep[3]]:
+        buf.free()
+
+
+@pytest.mark.parametrize("rows,grouped", [(32, False), (33, True)])
+def test_sparse_batches_of_unit_formats_stay_on_the_per_pair_gemv(be, rows, grouped):
+    """A batch that selects each expert about twice or less (rows * n_used <= 2 * n_expert) fills no tile of the
+    grouped GEMM: banks in the unit formats then run the per-pair GEMV (f32, bar 1e-3) whatever the row count."""
+    ne, nff, E, K = 256, 256, 32, 2
+    rng = np.random.default_rng(rows)
+    x = rng.standard_normal((rows, ne)).astype(np.float32)
+    router = (rng.standard_normal((E, ne)) * 0.1).astype(np.float32)
+    gate, up = H.centred_weight(H.MXFP4, E * nff * ne, 1), H.centred_weight(H.MXFP4, E * nff * ne, 2)
+    down = H.centred_weight(H.IQ4_XS, E * ne * nff, 3)
+    g, ids = moe_graph(rows, ne, E, K, nff, DType.Mxfp4, DType.Iq4Xs)
+    keep = []
+    be.prof_enable(True)
+    got = M.run_graph(be, g, [(ids["x"], x), (ids["router"], router), (ids["gate"], gate), (ids["up"], up),
+                              (ids["down"], down)], ids["dst"], rows * ne, keep=keep).reshape(rows, ne)
+    be.sync()
+    names = set(be.prof_read())
+    be.prof_enable(False)
+    want = O.moe_ffn(x, router, gate, up, down, ne=ne, n_expert=E, n_used=K, n_ff_exp=nff, gate_dtype=H.MXFP4, down_dtype=H.IQ4_XS)
+    assert np.array_equal(be.moe_routing(keep[0], 0)["idx"], want["idx"])
+    assert ("moe_grouped_units_gate_up" in names) == grouped and ("moe_gate_up_units" in names) == (not grouped)
+    wd = want["dst"].reshape(rows, ne)
+    for r in range(rows):
+        assert H.rel_l2(got[r], wd[r]) < (REL_L2_MFMA if grouped else REL_L2), r
     keep[0].free()
     for buf in keep[2] + [keep[3]]:
         buf.free()

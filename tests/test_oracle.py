@@ -67,7 +67,7 @@ def test_k4_inverts_ggml_scale_packing_exhaustively():
 def test_dequant_matches_golden_fixture_bit_for_bit():
     g = np.load(os.path.join(GOLD, "dequant.npz"))
     names = sorted({k.rsplit(".", 1)[0] for k in g.files})
-    assert len(names) == 8 + 14 + 6
+    assert len(names) == 8 + 14 + 6 + 14 + 7
     for n in names:
         got = O.dequant(int(g[n + ".dtype"]), g[n + ".bytes"])
         assert np.array_equal(got.view(np.uint32), g[n + ".bits"]), n
@@ -88,12 +88,51 @@ def test_dequant_gives_the_values_the_reference_tests_assert():
 
 
 @pytest.mark.parametrize("dt,seed", [(O.Q8_0, 1), (O.Q4K, 2), (O.Q6K, 3), (O.Q4_0, 4), (O.Q4_1, 5), (O.Q5_0, 6), (O.Q5_1, 7),
-                                     (O.Q2K, 8), (O.Q3K, 9), (O.Q5K, 10)])
+                                     (O.Q2K, 8), (O.Q3K, 9), (O.Q5K, 10), (O.IQ4_NL, 11), (O.IQ4_XS, 12), (O.TQ1_0, 13),
+                                     (O.TQ2_0, 14), (O.Q2_0, 15), (O.MXFP4, 16), (O.NVFP4, 17)])
 def test_dequant_matches_independent_decoder_on_random_blocks(dt, seed):
     be, bb = O.block_geometry(dt)
     b = H.synth_weight(dt, be * 64, seed)
     want = H.ggml_dequant(dt, b).astype(np.float32)
     assert np.array_equal(O.dequant(dt, b).view(np.uint32), want.view(np.uint32))
+
+
+def test_fp4_scales_match_their_arithmetic_definition_for_every_byte():
+    """E8M0 (MXFP4) and UE4M3 (NVFP4) scale bytes 0..255 against 2^(e - 127) and (8 + m) 2^(e - 10); element 0 carries
+    the code 1 (E2M1 0.5), element 16 / 8 the code 2 (E2M1 1.0)."""
+    b = np.zeros((256, 17), np.uint8)
+    b[:, 0], b[:, 1] = np.arange(256), 0x21
+    y = O.dequant(O.MXFP4, b.reshape(-1)).reshape(256, 32)
+    with np.errstate(over="ignore"):   # byte 255 (NaN in the E8M0 definition) decodes to 2^127, the code 2 overflows on it
+        assert np.array_equal(y[:, 16], np.ldexp(np.float32(1), np.arange(256) - 127))
+    assert np.array_equal(y[:255, 0], y[:255, 16] / 2) and y[255, 0] == np.float32(2.0) ** 127
+    assert np.array_equal(y, H.ggml_dequant(H.MXFP4, b.reshape(-1)).astype(np.float32).reshape(256, 32))
+    b = np.zeros((256, 36), np.uint8)
+    b[:, 0], b[:, 4] = np.arange(256), 0x21
+    y = O.dequant(O.NVFP4, b.reshape(-1)).reshape(256, 64)
+    x = np.arange(256)
+    want = np.where((x >> 3) & 15, (8 + (x & 7)) * np.exp2(((x >> 3) & 15) - 10.0), (x & 7) * 2.0 ** -9)
+    want[[0, 0x7F]] = 0
+    assert np.array_equal(y[:, 8], want.astype(np.float32)) and not y[:, 16:].any()
+    assert np.array_equal(y, H.ggml_dequant(H.NVFP4, b.reshape(-1)).astype(np.float32).reshape(256, 64))
+
+
+def test_tq1_0_decodes_what_the_published_packing_stores():
+    """All 243 five-digit ternary numbers packed as ggml's quantiser packs them (ceil(v * 256 / 243)) come back
+    digit by digit, in the three byte runs of a block (32, 16 and 4 bytes; the last holds four digits per byte)."""
+    import itertools
+    trits = np.array(list(itertools.product(range(3), repeat=5)))
+    packed = H.tq1_0_pack(trits)
+    for start in range(0, 243, 16):
+        chunk, t = packed[start:start + 16], trits[start:start + 16]
+        n = len(chunk)
+        blk = np.zeros(54, np.uint8)
+        blk[52:54] = H.f16_bytes(2.0)
+        blk[:n], blk[32:32 + n], blk[48:48 + min(n, 4)] = chunk, chunk, chunk[:4]
+        y = O.dequant(O.TQ1_0, blk) / 2 + 1
+        assert np.array_equal(y[:160].reshape(5, 32)[:, :n].T, t)
+        assert np.array_equal(y[160:240].reshape(5, 16)[:, :n].T, t)
+        assert np.array_equal(y[240:].reshape(4, 4)[:, :min(n, 4)].T, t[:4, :4])
 
 
 def test_dequant_hand_computed_values():
