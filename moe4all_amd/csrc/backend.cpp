@@ -300,7 +300,7 @@ static infr_status alloc_impl(infr_hip_backend* be, size_t bytes, int32_t usage,
     if (usage < INFR_USAGE_WEIGHTS || usage > INFR_USAGE_HOST_WEIGHTS)
         return fail(INFR_ERR_INVALID, "alloc: unknown buffer usage %d", usage);
     size_t len = bytes < 4 ? 4 : bytes;  // reference: vec![0u8; bytes.max(4)]
-    size_t cap = round_up(len, 256);
+    size_t cap = round_up(len + 16, 256);  // 16 bytes of slack: kernels that fetch weight rows in 16-byte chunks may run past the last row's end
     std::lock_guard<std::mutex> lk(be->mu);
     HIP_TRY(hipSetDevice(be->device));
     void* p = nullptr;

@@ -970,13 +970,17 @@ __device__ __forceinline__ void grouped_units_tile(const GroupedParams& p, const
 
     const int n_slices = p.K / kSlice;
     WSlice<DT> u0, u1;
-    uint4 areg[4];
+    uint4 ar0, ar1, ar2, ar3;   // named, not an array: the array form ends up in scratch memory
     u0.load(w0, half);
     u1.load(w1, half);
-#pragma unroll
-    for (int q = 0; q < 4; q++) areg[q] = *reinterpret_cast<const uint4*>(asrc[q]);
-#pragma unroll
-    for (int q = 0; q < 4; q++) *reinterpret_cast<uint4*>(a_dst + q * 1024) = areg[q];
+    ar0 = *reinterpret_cast<const uint4*>(asrc[0]);
+    ar1 = *reinterpret_cast<const uint4*>(asrc[1]);
+    ar2 = *reinterpret_cast<const uint4*>(asrc[2]);
+    ar3 = *reinterpret_cast<const uint4*>(asrc[3]);
+    *reinterpret_cast<uint4*>(a_dst) = ar0;
+    *reinterpret_cast<uint4*>(a_dst + 1024) = ar1;
+    *reinterpret_cast<uint4*>(a_dst + 2048) = ar2;
+    *reinterpret_cast<uint4*>(a_dst + 3072) = ar3;
     __syncthreads();
     for (int s = 0; s < n_slices; s++) {
         const bool more = s + 1 < n_slices;
@@ -984,8 +988,11 @@ __device__ __forceinline__ void grouped_units_tile(const GroupedParams& p, const
         if (more) {   // requests for the next slice
             v0.load(w0, 2 * (s + 1) + half);
             v1.load(w1, 2 * (s + 1) + half);
-#pragma unroll
-            for (int q = 0; q < 4; q++) areg[q] = *reinterpret_cast<const uint4*>(asrc[q] + (size_t)(s + 1) * 128);
+            const size_t ao = (size_t)(s + 1) * 128;
+            ar0 = *reinterpret_cast<const uint4*>(asrc[0] + ao);
+            ar1 = *reinterpret_cast<const uint4*>(asrc[1] + ao);
+            ar2 = *reinterpret_cast<const uint4*>(asrc[2] + ao);
+            ar3 = *reinterpret_cast<const uint4*>(asrc[3] + ao);
         }
         const uint8_t* ap = lds + (s & 1) * kUStage;
 #pragma unroll
@@ -1000,12 +1007,160 @@ __device__ __forceinline__ void grouped_units_tile(const GroupedParams& p, const
         }
         if (more) {
             uint8_t* d = a_dst + ((s + 1) & 1) * kUStage;
-#pragma unroll
-            for (int q = 0; q < 4; q++) *reinterpret_cast<uint4*>(d + q * 1024) = areg[q];
+            *reinterpret_cast<uint4*>(d) = ar0;
+            *reinterpret_cast<uint4*>(d + 1024) = ar1;
+            *reinterpret_cast<uint4*>(d + 2048) = ar2;
+            *reinterpret_cast<uint4*>(d + 3072) = ar3;
             u0 = v0;
             u1 = v1;
         }
         __syncthreads();   // the stage just written is complete; the stage just read may be overwritten
+    }
+    tile_epilogue<DOWN, M>(p, t, n0, wave, lane, s_scale, acc0, acc1);
+}
+
+// Weight rows through LDS.  A lane that reads its own row's unit straight from memory makes every load
+// instruction of the wave touch 64 rows, one or two cache lines each: the address unit of the CU, not the
+// matrix pipe, then sets the pace (measured: 93 line look-ups per load instruction, 73 % of the kernel's
+// cycles).  Here each wave copies the next 256 k of its 64 rows (the window: a whole number of blocks, WB
+// bytes per row) into a region of its own with consecutive lanes on consecutive 16-byte chunks of a row, and
+// the units are cut out of LDS.  Row pitch 16 * odd: sixteen lanes reading the same offset of sixteen rows
+// fall on distinct banks.  Windows alternate between two stages; window g + 1 is requested at the first
+// slice of window g and written after its third, one barrier before its first unit is read.
+template <int DT>
+struct StagedW {
+    static constexpr int kBlock = DT == INFR_Q4_0 || DT == INFR_Q4_1 || DT == INFR_Q5_0 || DT == INFR_Q5_1 || DT == INFR_Q8_0 ||
+                                          DT == INFR_IQ4_NL || DT == INFR_MXFP4 ? 32
+                                  : DT == INFR_Q2_0 || DT == INFR_NVFP4 ? 64 : 256;
+    static constexpr int kBlockBytes = DT == INFR_Q4_0 ? 18 : DT == INFR_Q4_1 ? 20 : DT == INFR_Q5_0 ? 22 : DT == INFR_Q5_1 ? 24
+                                       : DT == INFR_Q8_0 ? 34 : DT == INFR_Q2K ? 84 : DT == INFR_Q3K ? 110 : DT == INFR_Q4K ? 144
+                                       : DT == INFR_Q5K ? 176 : DT == INFR_Q6K ? 210 : DT == INFR_IQ4_NL ? 18 : DT == INFR_IQ4_XS ? 136
+                                       : DT == INFR_TQ1_0 ? 54 : DT == INFR_TQ2_0 ? 66 : DT == INFR_Q2_0 ? 18 : DT == INFR_MXFP4 ? 17
+                                       : DT == INFR_NVFP4 ? 36 : 0;
+    static constexpr int kWB = kBlockBytes * (256 / kBlock);   // bytes of one row in a window of 256 k
+    static constexpr int kChunks = (kWB + 15) / 16;
+    static constexpr int kPitch = 16 * (kChunks | 1);
+    // every block format except Q8_0 (272-byte windows: two stages of four waves would not fit beside the
+    // activation ring); unquantised rows are read in whole cache lines as they are
+    static constexpr bool kOn = kBlockBytes != 0 && DT != INFR_Q8_0;
+    static constexpr size_t kLds = kOn ? (size_t)4 * 2 * 64 * kPitch : 0;
+};
+
+template <int DT, bool DOWN, int M>
+__device__ __forceinline__ void grouped_units_tile_staged(const GroupedParams& p, const Tile& t, int n0, uint8_t* lds,
+                                                          const float* s_scale, uint8_t* wlds) {
+    using W = StagedW<DT>;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, half = lane >> 5;
+    float16v acc0[M], acc1[M];
+#pragma unroll
+    for (int i = 0; i < M; i++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc0[i][r] = acc1[i][r] = 0.0f;
+    const int row_bytes = (p.K / W::kBlock) * W::kBlockBytes;
+    // chunk i of the lane: row (64 i + lane) / kChunks of the wave's 64, 16-byte chunk (64 i + lane) % kChunks
+    const uint8_t* csrc[W::kChunks];
+    int cdst[W::kChunks], coff[W::kChunks];
+#pragma unroll
+    for (int i = 0; i < W::kChunks; i++) {
+        const int idx = 64 * i + lane, r = idx / W::kChunks, ch = idx - r * W::kChunks;
+        const uint8_t* row;
+        if (DOWN) row = p.w0 + (size_t)t.e * p.w0_stride + (size_t)min(n0 + 64 * wave + r, p.N - 1) * row_bytes;
+        else row = (r < 32 ? p.w0 + (size_t)t.e * p.w0_stride : p.w1 + (size_t)t.e * p.w1_stride) +
+                   (size_t)min(n0 + 32 * wave + (r & 31), p.N - 1) * row_bytes;
+        csrc[i] = row + 16 * ch;
+        coff[i] = 16 * ch;
+        cdst[i] = r * W::kPitch + 16 * ch;
+    }
+    uint8_t* const wbase = wlds + wave * (2 * 64 * W::kPitch);
+    const uint8_t* const u0row = wbase + (lane & 31) * W::kPitch;
+    const uint8_t* const u1row = u0row + 32 * W::kPitch;
+    const uint8_t* asrc[4];
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        const int tok = 32 * wave + 8 * q + (lane >> 3), kg = (lane & 7) ^ ((lane >> 3) & 7);
+        const int pr = t.p0 + min(tok, t.cnt - 1);
+        const size_t src_row = DOWN ? (size_t)pr : (size_t)(p.pair_src[pr] / p.n_used);
+        asrc[q] = reinterpret_cast<const uint8_t*>(p.a + src_row * p.K) + 16 * kg;
+    }
+    uint8_t* const a_dst = lds + wave * 4096 + lane * 16;
+    const int x7 = lane & 7;
+    int a_off[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ks++) a_off[ks] = (lane & 31) * 128 + (((ks + 4 * half) ^ x7) * 16);
+
+    const int n_slices = p.K / kSlice, n_win = (n_slices + 3) >> 2;
+    uint4 wreg[W::kChunks];
+    uint4 ar0, ar1, ar2, ar3;   // named, not an array: the array form ends up in scratch memory
+    // a chunk that starts past the row's end (last window of a row that is no whole number of windows) is not read;
+    // one that starts inside may run up to 15 bytes past it, which every buffer of the backend has room for
+    auto request = [&](int g) {
+        const int valid = row_bytes - g * W::kWB;
+        const size_t o = (size_t)g * W::kWB;
+        if (valid >= W::kWB) {   // uniform: only a row's last window can be short
+#pragma unroll
+            for (int i = 0; i < W::kChunks; i++) wreg[i] = ldu<uint4>(csrc[i] + o);
+        } else {
+#pragma unroll
+            for (int i = 0; i < W::kChunks; i++) wreg[i] = ldu<uint4>(csrc[i] + o - (coff[i] < valid ? 0 : coff[i]));
+        }
+    };
+    auto deposit = [&](int g) {
+        uint8_t* d = wbase + (g & 1) * (64 * W::kPitch);
+#pragma unroll
+        for (int i = 0; i < W::kChunks; i++)
+            *reinterpret_cast<uint4*>(d + cdst[i]) = wreg[i];
+    };
+    request(0);
+    ar0 = *reinterpret_cast<const uint4*>(asrc[0]);
+    ar1 = *reinterpret_cast<const uint4*>(asrc[1]);
+    ar2 = *reinterpret_cast<const uint4*>(asrc[2]);
+    ar3 = *reinterpret_cast<const uint4*>(asrc[3]);
+    deposit(0);
+    *reinterpret_cast<uint4*>(a_dst) = ar0;
+    *reinterpret_cast<uint4*>(a_dst + 1024) = ar1;
+    *reinterpret_cast<uint4*>(a_dst + 2048) = ar2;
+    *reinterpret_cast<uint4*>(a_dst + 3072) = ar3;
+    __syncthreads();
+    WSlice<DT> u0, u1;
+    u0.load(u0row, half);
+    u1.load(u1row, half);
+    for (int s = 0; s < n_slices; s++) {
+        const bool more = s + 1 < n_slices;
+        const int g = s >> 2, j = s & 3;
+        WSlice<DT> v0, v1;
+        if (j == 0 && g + 1 < n_win) request(g + 1);
+        if (more) {
+            const int so = (((s + 1) >> 2) & 1) * (64 * W::kPitch), ui = 2 * ((s + 1) & 3) + half;
+            v0.load(u0row + so, ui);
+            v1.load(u1row + so, ui);
+            const size_t ao = (size_t)(s + 1) * 128;
+            ar0 = *reinterpret_cast<const uint4*>(asrc[0] + ao);
+            ar1 = *reinterpret_cast<const uint4*>(asrc[1] + ao);
+            ar2 = *reinterpret_cast<const uint4*>(asrc[2] + ao);
+            ar3 = *reinterpret_cast<const uint4*>(asrc[3] + ao);
+        }
+        const uint8_t* ap = lds + (s & 1) * kUStage;
+#pragma unroll
+        for (int ks = 0; ks < 4; ks++) {
+            const half8 b0 = u0.frag(ks), b1 = u1.frag(ks);
+#pragma unroll
+            for (int mi = 0; mi < M; mi++) {
+                const half8 a = *reinterpret_cast<const half8*>(ap + a_off[ks] + mi * 4096);
+                acc0[mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b0, acc0[mi], 0, 0, 0);
+                acc1[mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b1, acc1[mi], 0, 0, 0);
+            }
+        }
+        if (more) {
+            uint8_t* d = a_dst + ((s + 1) & 1) * kUStage;
+            *reinterpret_cast<uint4*>(d) = ar0;
+            *reinterpret_cast<uint4*>(d + 1024) = ar1;
+            *reinterpret_cast<uint4*>(d + 2048) = ar2;
+            *reinterpret_cast<uint4*>(d + 3072) = ar3;
+            u0 = v0;
+            u1 = v1;
+        }
+        if (j == 2 && g + 1 < n_win) deposit(g + 1);
+        __syncthreads();
     }
     tile_epilogue<DOWN, M>(p, t, n0, wave, lane, s_scale, acc0, acc1);
 }
@@ -1023,11 +1178,21 @@ __global__ __launch_bounds__(256) void grouped_units_mfma(GroupedParams p) {
         const int pr = t.p0 + min(tid, t.cnt - 1);
         s_scale[tid] = p.a_scale[DOWN ? pr : p.pair_src[pr] / p.n_used];
     }
-    switch ((t.cnt + 31) >> 5) {
-        case 1: grouped_units_tile<DT, DOWN, 1>(p, t, nt * kBN, lds, s_scale); break;
-        case 2: grouped_units_tile<DT, DOWN, 2>(p, t, nt * kBN, lds, s_scale); break;
-        case 3: grouped_units_tile<DT, DOWN, 3>(p, t, nt * kBN, lds, s_scale); break;
-        default: grouped_units_tile<DT, DOWN, 4>(p, t, nt * kBN, lds, s_scale); break;
+    if constexpr (StagedW<DT>::kOn) {
+        extern __shared__ __attribute__((aligned(16))) uint8_t wlds[];
+        switch ((t.cnt + 31) >> 5) {
+            case 1: grouped_units_tile_staged<DT, DOWN, 1>(p, t, nt * kBN, lds, s_scale, wlds); break;
+            case 2: grouped_units_tile_staged<DT, DOWN, 2>(p, t, nt * kBN, lds, s_scale, wlds); break;
+            case 3: grouped_units_tile_staged<DT, DOWN, 3>(p, t, nt * kBN, lds, s_scale, wlds); break;
+            default: grouped_units_tile_staged<DT, DOWN, 4>(p, t, nt * kBN, lds, s_scale, wlds); break;
+        }
+    } else {
+        switch ((t.cnt + 31) >> 5) {
+            case 1: grouped_units_tile<DT, DOWN, 1>(p, t, nt * kBN, lds, s_scale); break;
+            case 2: grouped_units_tile<DT, DOWN, 2>(p, t, nt * kBN, lds, s_scale); break;
+            case 3: grouped_units_tile<DT, DOWN, 3>(p, t, nt * kBN, lds, s_scale); break;
+            default: grouped_units_tile<DT, DOWN, 4>(p, t, nt * kBN, lds, s_scale); break;
+        }
     }
 }
 
@@ -1037,7 +1202,14 @@ void grouped_units(hipStream_t s, const GroupedParams& p) {
     GroupedParams q = p;
     q.n_tiles_n = (p.N + bn - 1) / bn;
     const int max_tiles = p.n_pairs / kBM + (p.n_expert < p.n_pairs ? p.n_expert : p.n_pairs);
-    INFR_LAUNCH((grouped_units_mfma<DT, DOWN>), dim3((unsigned)((max_tiles * q.n_tiles_n + 7) & ~7)), dim3(256), 0, s, q);
+    static bool attr_set = false;
+    if (!attr_set && StagedW<DT>::kLds) {
+        (void)hipFuncSetAttribute((const void*)grouped_units_mfma<DT, DOWN>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  (int)StagedW<DT>::kLds);
+        attr_set = true;
+    }
+    INFR_LAUNCH((grouped_units_mfma<DT, DOWN>), dim3((unsigned)((max_tiles * q.n_tiles_n + 7) & ~7)), dim3(256), StagedW<DT>::kLds,
+                s, q);
 }
 
 template <bool DOWN>
