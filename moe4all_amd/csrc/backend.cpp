@@ -591,10 +591,11 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
                                infr::grouped_supported(c.dt(m.gate_exps), (int)m.ne) &&
                                infr::grouped_supported(c.dt(m.down_exps), (int)m.n_ff_exp);
                 // a bank in one of the other affine formats: the same path with the unit-decoder GEMM for all three
-                // ... unless the batch selects each expert about twice or less: then no bucket fills a corner of a
-                // 128-token tile, and the per-pair unit GEMV, which streams an expert's rows at full width, is faster
-                // (2880 x 2880 MXFP4 banks, 128 experts, top-4: 32 rows 0.66 ms against 1.30 ms, 64 rows 1.32 against 1.96)
-                const bool sparse_batch = pairs <= 2 * (size_t)n_local && be->cfg.moe_batched_min_rows == 0;
+                // ... unless the batch selects each expert one and a half times or less: then no bucket fills a corner
+                // of a 128-token tile, and the per-pair unit GEMV, which streams an expert's rows at full width, is
+                // faster (2880 x 2880 MXFP4 banks, 128 experts, top-4: 32 rows 0.66 ms, 64 rows 1.04 ms, against the
+                // 1.2 ms that one tile pass over every expert costs)
+                const bool sparse_batch = 2 * pairs <= 3 * (size_t)n_local && be->cfg.moe_batched_min_rows == 0;
                 const bool units_mfma = !batched && rows >= min_rows && m.n_used <= 64 && !sparse_batch &&
                                         (m.fused_gate_up || c.dt(m.gate_exps) == c.dt(m.up_exps)) &&
                                         infr::grouped_units_supported(c.dt(m.gate_exps), (int)m.ne) &&

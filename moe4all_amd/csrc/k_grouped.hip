@@ -1005,6 +1005,13 @@ __device__ __forceinline__ void grouped_units_tile(const GroupedParams& p, const
                 acc1[mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b1, acc1[mi], 0, 0, 0);
             }
         }
+        // One wave per SIMD: the decode of the next fragments has to issue between this wave's own matrix
+        // instructions, or the two pipes take turns.  Ask the scheduler for one MFMA, then a share of the VALU work.
+#pragma unroll
+        for (int i = 0; i < 8 * M; i++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 256 / (8 * M), 0);
+        }
         if (more) {
             uint8_t* d = a_dst + ((s + 1) & 1) * kUStage;
             *reinterpret_cast<uint4*>(d) = ar0;
@@ -1149,6 +1156,13 @@ __device__ __forceinline__ void grouped_units_tile_staged(const GroupedParams& p
                 acc0[mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b0, acc0[mi], 0, 0, 0);
                 acc1[mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b1, acc1[mi], 0, 0, 0);
             }
+        }
+        // One wave per SIMD: the decode of the next fragments has to issue between this wave's own matrix
+        // instructions, or the two pipes take turns.  Ask the scheduler for one MFMA, then a share of the VALU work.
+#pragma unroll
+        for (int i = 0; i < 8 * M; i++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, 256 / (8 * M), 0);
         }
         if (more) {
             uint8_t* d = a_dst + ((s + 1) & 1) * kUStage;

@@ -44,7 +44,7 @@ __device__ __forceinline__ uint32_t spread4(uint32_t t) { return ((t & 0xFu) * 0
 __device__ __forceinline__ uint32_t book4(uint32_t w, uint32_t t0, uint32_t t1, uint32_t t2, uint32_t t3) {
     const uint32_t sel = w & 0x07070707u;
     const uint32_t lo = __builtin_amdgcn_perm(t1, t0, sel), hi = __builtin_amdgcn_perm(t3, t2, sel);
-    const uint32_t m = ((w >> 3) & kB0) * 0xFFu;
+    const uint32_t b3 = (w >> 3) & kB0, m = (b3 << 8) - b3;   // 0xFF in the bytes whose nibble has bit 3 set
     return lo ^ ((lo ^ hi) & m);
 }
 // IQ4_NL book + 127 and twice-E2M1 book + 12 as unsigned bytes.

@@ -849,11 +849,12 @@ def test_moe_ffn_with_experts_in_the_other_affine_formats(be, gdt, ddt, rows, ne
         buf.free()
 
 
-@pytest.mark.parametrize("rows,grouped", [(32, False), (33, True)])
+@pytest.mark.parametrize("rows,grouped", [(48, False), (49, True)])
 def test_sparse_batches_of_unit_formats_stay_on_the_per_pair_gemv(be, rows, grouped):
-    """A batch that selects each expert about twice or less (rows * n_used <= 2 * n_expert) fills no tile of the
-    grouped GEMM: banks in the unit formats then run the per-pair GEMV (f32, bar 1e-3) whatever the row count."""
-    ne, nff, E, K = 256, 256, 32, 2
+    """A batch that selects each expert one and a half times or less (2 * rows * n_used <= 3 * n_expert) fills no
+    tile of the grouped GEMM: banks in the unit formats then run the per-pair GEMV (f32, bar 1e-3) whatever the
+    row count."""
+    ne, nff, E, K = 256, 256, 64, 2
     rng = np.random.default_rng(rows)
     x = rng.standard_normal((rows, ne)).astype(np.float32)
     router = (rng.standard_normal((E, ne)) * 0.1).astype(np.float32)
