@@ -1334,15 +1334,17 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                 gp.y = sc.y;
                 // Every block of the gate/up kernel routes its own token row when that is cheaper than a
                 // launch of the routing kernel: the blocks of one compute unit repeat it once per row.
-                gp.route_inline = infr::moe_gate_up_routes_inline(gp) && (rows == 1 || (uint64_t)rows * m.n_expert <= 512) ? 1 : 0;
+                const bool fast_gu = infr::moe_gate_up_routes_inline(gp);
+                const bool units = !fast_gu && !gp.sh_gate && infr::moe_gate_up_units_supported(gp);
+                gp.route_inline = (fast_gu || (units && infr::moe_gate_up_units_routes_inline(gp))) &&
+                                          (rows == 1 || (uint64_t)rows * m.n_expert <= 512) ? 1 : 0;
                 if (!gp.route_inline) {
                     Timed t(be, "route_topk");
                     infr::launch_route(s, rp);
                 }
                 {
-                    const bool units = !infr::moe_gate_up_routes_inline(gp) && infr::moe_gate_up_units_supported(gp);
-                    Timed t(be, gp.sh_gate ? "moe_route_gate_up_shared" : gp.route_inline ? "moe_route_gate_up"
-                                : units ? "moe_gate_up_units" : "moe_gate_up");
+                    Timed t(be, gp.sh_gate ? "moe_route_gate_up_shared" : units ? (gp.route_inline ? "moe_route_gate_up_units" : "moe_gate_up_units")
+                                : gp.route_inline ? "moe_route_gate_up" : "moe_gate_up");
                     infr::launch_moe_gate_up(s, gp);
                 }
                 gp.x = nullptr;

@@ -13,6 +13,7 @@
 // wave walks output rows two at a time, lanes stride over the units of a row.
 #include "device_common.h"
 #include "kernels.h"
+#include "route.h"
 #include "units.h"
 
 namespace infr {
@@ -119,13 +120,30 @@ __global__ __launch_bounds__(256) void moe_units_kernel(MoeGemvParams p, size_t 
     float* xsum = lds + (size_t)n_units * kUnitStride;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const int pair = blockIdx.y, r = pair / p.n_used;
-    const int e = p.ids[pair];
     const float* xrow = GATE_UP ? p.x + (size_t)r * p.ne : p.h + (size_t)pair * p.nff;
     float* out = GATE_UP ? p.h + (size_t)pair * p.nff : p.y + (size_t)pair * p.ne;
     const int row_base = blockIdx.x * kRowsPerBlock;
-    if (e < 0 || e >= p.n_expert) {
-        for (int o = row_base + tid; o < min(row_base + kRowsPerBlock, out_f); o += 256) out[o] = 0.0f;
-        return;
+    // gate/up with routing folded in: the block routes its token row itself (one wave, the same routine as the
+    // routing kernel) while the activation row is on its way; block column 0 of a row's first pair stores the result
+    const bool routes = GATE_UP && p.route_inline;
+    __shared__ uint64_t s_tab[32];
+    __shared__ int32_t s_ids[64];
+    __shared__ float s_w[64];
+    int e = 0;
+    if (!routes) {
+        e = p.ids[pair];
+        if (e < 0 || e >= p.n_expert) {
+            for (int o = row_base + tid; o < min(row_base + kRowsPerBlock, out_f); o += 256) out[o] = 0.0f;
+            return;
+        }
+    } else if (wave == 3) {
+        // the last wave has the smallest share of the activation row to stage (none up to 3072 elements): it
+        // routes while the others stage
+        if (lane < 32) s_tab[lane] = kExp2Table[lane];
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        const int slot0 = pair - r * p.n_used;
+        route_row_any(p.route, r, lane, xsum + 2 * n_units, s_tab, s_ids, s_w, blockIdx.x == 0 && slot0 == 0);
     }
     for (int hu = tid; hu < 2 * n_units; hu += 256) {
         float4 v[4];
@@ -141,6 +159,20 @@ __global__ __launch_bounds__(256) void moe_units_kernel(MoeGemvParams p, size_t 
         xsum[hu] = sm;
     }
     __syncthreads();
+    float w_before = 1.0f;
+    if constexpr (GATE_UP) {
+        if (routes) {
+            const int slot = pair - r * p.n_used;
+            e = s_ids[slot];
+            w_before = s_w[slot];
+            if (e < 0 || e >= p.n_expert) {
+                for (int o = row_base + tid; o < min(row_base + kRowsPerBlock, out_f); o += 256) out[o] = 0.0f;
+                return;
+            }
+        } else if (p.weight_before) {
+            w_before = p.weights[pair];
+        }
+    }
     constexpr int M = GATE_UP ? 2 : 1;   // matrices per output row
     const uint8_t* base[M];
     base[0] = (GATE_UP ? p.gate + (size_t)e * p.gate_stride : p.down + (size_t)e * p.down_stride);
@@ -198,9 +230,8 @@ __global__ __launch_bounds__(256) void moe_units_kernel(MoeGemvParams p, size_t 
             if (lane == 0 && o0 + a < out_f) {
                 if constexpr (GATE_UP) {
                     if (p.weight_before) {
-                        const float wp = p.weights[pair];
-                        v[0] = __fmul_rn(wp, v[0]);
-                        v[1] = __fmul_rn(wp, v[1]);
+                        v[0] = __fmul_rn(w_before, v[0]);
+                        v[1] = __fmul_rn(w_before, v[1]);
                     }
                     out[o0 + a] = gated_act_fn(p.act, p.has_clamp, p.clamp, v[0], v[1]);
                 } else {
@@ -404,12 +435,13 @@ void launch_moe_units_dt(hipStream_t s, const MoeGemvParams& p) {
     const size_t row_bytes = (size_t)(in_f / be) * bb;
     static bool attr_set = false;
     if (!attr_set) {
-        (void)hipFuncSetAttribute((const void*)moe_units_kernel<DT, GATE_UP>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        (void)hipFuncSetAttribute((const void*)moe_units_kernel<DT, GATE_UP>, hipFuncAttributeMaxDynamicSharedMemorySize, 158 * 1024);
         attr_set = true;
     }
     dim3 grid((out_f + kRowsPerBlock - 1) / kRowsPerBlock, p.rows * p.n_used), block(256);
-    INFR_LAUNCH((moe_units_kernel<DT, GATE_UP>), grid, block, (size_t)(in_f >> 5) * (kUnitStride + 2) * sizeof(float), s, p,
-                row_bytes);
+    const size_t route_lds = GATE_UP && p.route_inline ? route_scratch_floats(p.route.n_expert, p.route.n_groups) * sizeof(float) : 0;
+    INFR_LAUNCH((moe_units_kernel<DT, GATE_UP>), grid, block, (size_t)(in_f >> 5) * (kUnitStride + 2) * sizeof(float) + route_lds,
+                s, p, row_bytes);
 }
 
 template <bool GATE_UP>
@@ -561,6 +593,9 @@ bool moe_gate_up_units_supported(const MoeGemvParams& p) {
     return p.gate_dt == p.up_dt && p.rows * p.n_used <= 65535 && linear_units_supported(p.gate_dt, p.ne, p.x);
 }
 void launch_moe_gate_up_units(hipStream_t s, const MoeGemvParams& p) { launch_moe_units_any<true>(s, p.gate_dt, p); }
+// The unit gate/up kernel can route a token row inside each of its blocks (p.route_inline) for as many slots as its
+// LDS tables hold.
+bool moe_gate_up_units_routes_inline(const MoeGemvParams& p) { return moe_gate_up_units_supported(p) && p.n_used <= 64; }
 bool moe_down_units_supported(const MoeGemvParams& p) {
     return p.y != nullptr && p.rows * p.n_used <= 65535 && linear_units_supported(p.down_dt, p.nff, p.h);
 }

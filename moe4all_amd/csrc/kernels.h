@@ -173,6 +173,7 @@ void launch_linear_float(hipStream_t s, const float* x, const uint8_t* w, int dt
 // y[pair] from h (down; needs p.y).  The weighted sum over ranks is launch_unbucket_combine's.
 bool moe_gate_up_units_supported(const MoeGemvParams& p);
 void launch_moe_gate_up_units(hipStream_t s, const MoeGemvParams& p);
+bool moe_gate_up_units_routes_inline(const MoeGemvParams& p);
 bool moe_down_units_supported(const MoeGemvParams& p);
 void launch_moe_down_units(hipStream_t s, const MoeGemvParams& p);
 // Batches on the unit kernels: an expert's rows are fetched once per chunk of tokens of its bucket

@@ -843,7 +843,9 @@ def test_moe_ffn_with_experts_in_the_other_affine_formats(be, gdt, ddt, rows, ne
     elif rows >= 32:   # batches walk the expert buckets on the f32 unit kernels
         assert {"moe_gate_up_units_bucketed", "moe_down_units_bucketed", "moe_unbucket_combine"} <= names
     else:
-        assert "moe_gate_up_units" in names and ("moe_down_units" in names or ddt == H.Q6K)
+        # routing rides in the gate/up kernel while rows * n_expert <= 512 (as on the integer-dot kernels)
+        assert ("moe_route_gate_up_units" if rows * E <= 512 else "moe_gate_up_units") in names
+        assert ("route_topk" in names) == (rows * E > 512) and ("moe_down_units" in names or ddt == H.Q6K)
     keep[0].free()
     for buf in keep[2] + [keep[3]]:
         buf.free()
