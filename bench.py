@@ -83,10 +83,11 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c4", "c4k", "c5"],
+    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c4", "c4k", "c5", "mxfp4"],
                     help="c1/c2/c5: decode stacks (use --batch for multi-stream decode); c4: one config-1 layer "
                          "(Q8_0), prefill chunk of --tokens with Zipf(1.1) expert popularity; c4k: same with "
-                         "Q4_K gate/up + Q6_K down")
+                         "Q4_K gate/up + Q6_K down; mxfp4: a decode stack of the gpt-oss-120b expert shape with MXFP4 banks "
+                         "(the 32-element-unit kernels; use --batch >= 32 for the unit-decoder grouped GEMM)")
     ap.add_argument("--tokens", type=int, default=2048, help="prefill chunk size for c4/c4k")
     ap.add_argument("--layers", type=int, default=0, help="override the layer count (0 = the config's)")
     ap.add_argument("--batch", type=int, default=1)
@@ -108,7 +109,7 @@ def main():
     if args.sublayer:
         args.no_cpu_baseline = True   # the CPU sample times Op::MoeFfn alone
     prefill = args.config in ("c4", "c4k")
-    shape = {"c1": synth.CONFIG_1, "c2": synth.CONFIG_2, "c5": synth.CONFIG_5,
+    shape = {"c1": synth.CONFIG_1, "c2": synth.CONFIG_2, "c5": synth.CONFIG_5, "mxfp4": synth.CONFIG_MXFP4,
              "c4": synth.MoeShape(f"c4-prefill-{args.tokens}-zipf1.1-q8_0", 1, 2048, 128, 8, 768, DType.Q8_0, DType.Q8_0),
              "c4k": synth.MoeShape(f"c4-prefill-{args.tokens}-zipf1.1-q4k-q6k", 1, 2048, 128, 8, 768, DType.Q4K,
                                    DType.Q6K)}[args.config]
@@ -131,9 +132,9 @@ def main():
     for t in range(N_TOKENS):
         row = []
         for l in range(n_layer):
-            xb = be.alloc(batch * shape.ne * 4)
-            synth.weights_device(be, xb, DType.F32, synth.stream_seed(SEED0 + 1 + t, l, synth.ROLE_X),
-                                 batch * shape.ne, sigma=1.0)
+            n_x = -(-batch * shape.ne // 256) * 256   # the generator writes whole 256-element groups
+            xb = be.alloc(n_x * 4)
+            synth.weights_device(be, xb, DType.F32, synth.stream_seed(SEED0 + 1 + t, l, synth.ROLE_X), n_x, sigma=1.0)
             if prefill:
                 xh = be.download(xb, dtype=np.float32).reshape(batch, shape.ne).copy()
                 xh[:, 0] = 1.0
@@ -202,6 +203,11 @@ def main():
         }
         # the decode kernel that routes its own token row also reads that row's logits
         alg["moe_route_gate_up"] = alg["moe_gate_up"] + batch * shape.n_expert * 4
+        # banks on the 32-element-unit kernels: per-pair down results, then the rank-ordered sum as its own launch
+        alg["moe_gate_up_units"], alg["moe_route_gate_up_units"] = alg["moe_gate_up"], alg["moe_route_gate_up"]
+        alg["moe_down_units"] = n_sel * down_b + pairs * shape.n_ff * 4 + pairs * shape.ne * 4
+        if not prefill and batch < 32:
+            alg["moe_unbucket_combine"] = pairs * shape.ne * 4 + batch * shape.ne * 4
         alg["rms_norm_router_logits"] = alg["router_logits"] + shape.ne * 4 + batch * shape.ne * 4
         if shape.shared_ff:
             sh_gate_b = M.backend.bytes_for(shape.gate_dtype, shape.shared_ff * shape.ne)
@@ -215,6 +221,7 @@ def main():
             "moe_grouped_gate_up": 2.0 * pairs * 2 * shape.n_ff * shape.ne,
             "moe_grouped_down": 2.0 * pairs * shape.ne * shape.n_ff,
         }
+        flops["moe_grouped_units_gate_up"], flops["moe_grouped_units_down"] = flops["moe_grouped_gate_up"], flops["moe_grouped_down"]
         for name, p in prof.items():
             avg_us = p["total_ms"] * 1e3 / max(p["launches"], 1)
             kernels[name] = {"launches": int(p["launches"]), "avg_us": round(avg_us, 3), "min_us": round(p["min_ms"] * 1e3, 3)}
@@ -259,6 +266,8 @@ def main():
         threads = O.hw_threads()
         n_sample, spent, budget_s = 0, 0.0, 12.0
         cpu_rows = min(batch, 256)   # a prefill chunk is sampled by its first 256 tokens
+        # the int8 batch numerics exist for the formats with an integer dot on the CPU (Q8_0, Q4_K, Q6_K)
+        production = cpu_rows >= 2 and {shape.gate_dtype, shape.down_dtype} <= {DType.Q8_0, DType.Q4K, DType.Q6K}
         while spent < budget_s and n_sample < 4 * n_layer:
             x = synth.normal(synth.stream_seed(SEED0 + 1, n_sample, synth.ROLE_X), batch * shape.ne, 1.0)
             x = x.reshape(batch, shape.ne)[:cpu_rows].copy()
@@ -269,14 +278,14 @@ def main():
             # (crates/infr-cpu/src/lib.rs:3679); a single row runs the f32 dequantise-and-dot path either way
             O.moe_ffn(x, router, gate, up, down, ne=shape.ne, n_expert=shape.n_expert, n_used=shape.n_used,
                       n_ff_exp=shape.n_ff, gate_dtype=int(shape.gate_dtype), down_dtype=int(shape.down_dtype),
-                      n_threads=threads, production=cpu_rows >= 2)
+                      n_threads=threads, production=production)
             spent += time.perf_counter() - t1
             n_sample += 1
         per_layer_s = spent / n_sample
         cpu = {"value": round(cpu_rows / (per_layer_s * n_layer), 3), "unit": "tok/s", "cores": threads, "kind": "port",
                "sample": f"{n_sample} layer-passes of layer 0 (routed experts only, {cpu_rows} token rows each) with distinct seeded tokens, "
                          f"{per_layer_s * 1e3:.2f} ms per layer-pass, "
-                         f"{'production numerics (int8 activations, scalar integer dots)' if cpu_rows >= 2 else 'f32 numerics (dequantise a row, f32 dot)'}, "
+                         f"{'production numerics (int8 activations, scalar integer dots)' if production else 'f32 numerics (dequantise a row, f32 dot)'}, "
                          f"scaled to {n_layer} layers",
                "ms_per_layer": round(per_layer_s * 1e3, 3)}
 

@@ -5,7 +5,7 @@
  * inputs with test-local helpers (crates/infr-testkit/src/lib.rs:49-123,
  * crates/infr-metal/tests/parity.rs:271-287) and its models read real GGUF files.  These
  * entry points produce N(0, sigma) tensors from a counter-based generator and quantise them
- * to Q8_0 / Q4_K / Q6_K, on the host or directly into a device buffer, with identical bytes.
+ * to Q8_0 / Q4_K / Q6_K / MXFP4, on the host or directly into a device buffer, with identical bytes.
  */
 #ifndef INFR_SYNTH_H
 #define INFR_SYNTH_H
@@ -18,7 +18,7 @@ extern "C" {
 
 /* out[i] = element (offset + i) of the N(0, sigma) stream `seed`, i < n.  Host only. */
 int infr_synth_normal_host(uint64_t seed, uint64_t offset, uint64_t n, double sigma, float *out);
-/* Quantise n f32 values (n a whole number of blocks) to `dtype` (Q8_0, Q4K, Q6K) on the host.
+/* Quantise n f32 values (n a whole number of blocks) to `dtype` (Q8_0, Q4K, Q6K, MXFP4) on the host.
  * Returns the number of bytes written or -1. */
 int64_t infr_synth_quantize_host(int32_t dtype, const float *src, uint64_t n, void *dst);
 /* dst = dtype-quantised elements [offset, offset + numel) of the N(0, sigma) stream `seed`

@@ -435,8 +435,40 @@ SYN_HD inline void quantize_block_q6_K(const float* x, uint8_t* y /*210 B*/) {
     }
 }
 
+// ---- MXFP4: shared exponent e = floor(log2(amax)) - 2 + 127 (E8M0, so that the largest magnitude lands in
+// [4, 8) of the E2M1 range 0 .. 6), each element the nearest entry of the twice-E2M1 book times 2^(e - 128)
+// (first entry on a tie), low nibbles = elements 0..15, high nibbles = 16..31: ggml's quantize_row_mxfp4_ref.
+SYN_HD inline void quantize_block_mxfp4(const float* x, uint8_t* out /*17 B*/) {
+    const int book[16] = {0, 1, 2, 3, 4, 6, 8, 12, 0, -1, -2, -3, -4, -6, -8, -12};
+    float amax = 0.f;
+    for (int i = 0; i < 32; i++) { float a = fabs_(x[i]); if (a > amax) amax = a; }
+    uint32_t bits;
+    memcpy(&bits, &amax, 4);
+    // floor(log2(amax)) from the exponent field (a subnormal amax counts as the smallest normal)
+    const int eb = amax > 0.f ? imax((int)((bits >> 23) & 0xFF), 1) - 2 : 0;
+    const uint8_t e = (uint8_t)imax(eb, 0);
+    const uint32_t dbits = e < 2 ? 0x00200000u << e : ((uint32_t)e - 1u) << 23;   // 2^(e - 128)
+    float d;
+    memcpy(&d, &dbits, 4);
+    out[0] = e;
+    for (int j = 0; j < 16; j++) {
+        uint8_t nib[2];
+        for (int h = 0; h < 2; h++) {
+            const float v = x[j + 16 * h];
+            int best = 0;
+            float berr = fabs_((float)book[0] * d - v);
+            for (int i = 1; i < 16; i++) {
+                const float err = fabs_((float)book[i] * d - v);
+                if (err < berr) { berr = err; best = i; }
+            }
+            nib[h] = (uint8_t)best;
+        }
+        out[1 + j] = (uint8_t)(nib[0] | (nib[1] << 4));
+    }
+}
+
 // Quantise 256 consecutive elements starting at element index e0 of the N(0,sigma) tensor
-// `seed` into `out` (Q8_0: 8 blocks = 272 B, Q4_K: 144 B, Q6_K: 210 B).
+// `seed` into `out` (Q8_0: 8 blocks = 272 B, Q4_K: 144 B, Q6_K: 210 B, MXFP4: 8 blocks = 136 B).
 SYN_HD inline void synth_superblock(int dtype, uint64_t seed, uint64_t e0, double sigma, uint8_t* out) {
     float x[256];
     for (int k = 0; k < 128; k++) {
@@ -449,6 +481,8 @@ SYN_HD inline void synth_superblock(int dtype, uint64_t seed, uint64_t e0, doubl
         for (int b = 0; b < 8; b++) quantize_block_q8_0(x + 32 * b, out + 34 * b);
     } else if (dtype == 12) {
         quantize_block_q4_K(x, out);
+    } else if (dtype == 28) {
+        for (int b = 0; b < 8; b++) quantize_block_mxfp4(x + 32 * b, out + 17 * b);
     } else {
         quantize_block_q6_K(x, out);
     }

@@ -12,7 +12,7 @@
 namespace {
 
 SYN_HD inline size_t superblock_bytes(int dtype) {
-    return dtype == INFR_Q8_0 ? 8 * 34 : dtype == INFR_Q4K ? 144 : dtype == INFR_Q6K ? 210 : 256 * 4;
+    return dtype == INFR_Q8_0 ? 8 * 34 : dtype == INFR_Q4K ? 144 : dtype == INFR_Q6K ? 210 : dtype == INFR_MXFP4 ? 8 * 17 : 256 * 4;
 }
 
 __global__ __launch_bounds__(64) void synth_weights_kernel(uint8_t* dst, int dtype, uint64_t seed, uint64_t offset,
@@ -50,7 +50,9 @@ void host_range(int dtype, uint64_t seed, uint64_t offset, uint64_t sb0, uint64_
     }
 }
 
-bool dtype_ok(int dtype) { return dtype == INFR_F32 || dtype == INFR_Q8_0 || dtype == INFR_Q4K || dtype == INFR_Q6K; }
+bool dtype_ok(int dtype) {
+    return dtype == INFR_F32 || dtype == INFR_Q8_0 || dtype == INFR_Q4K || dtype == INFR_Q6K || dtype == INFR_MXFP4;
+}
 
 }  // namespace
 
@@ -66,6 +68,11 @@ extern "C" int64_t infr_synth_quantize_host(int32_t dtype, const float* src, uin
         if (n % 32) return -1;
         for (uint64_t b = 0; b < n / 32; b++) synth::quantize_block_q8_0(src + 32 * b, o + 34 * b);
         return (int64_t)(n / 32 * 34);
+    }
+    if (dtype == INFR_MXFP4) {
+        if (n % 32) return -1;
+        for (uint64_t b = 0; b < n / 32; b++) synth::quantize_block_mxfp4(src + 32 * b, o + 17 * b);
+        return (int64_t)(n / 32 * 17);
     }
     if (n % 256) return -1;
     if (dtype == INFR_Q4K) {
@@ -104,7 +111,7 @@ extern "C" infr_status infr_hip_internal_fail(infr_status st, const char* msg);
 extern "C" infr_status infr_synth_weights_device(infr_hip_backend* be, infr_hip_buffer* buf, size_t byte_offset,
                                                  int32_t dtype, uint64_t seed, uint64_t offset, uint64_t numel,
                                                  double sigma) {
-    if (!dtype_ok(dtype)) return infr_hip_internal_fail(INFR_ERR_UNSUPPORTED, "synth: dtype must be F32, Q8_0, Q4K or Q6K");
+    if (!dtype_ok(dtype)) return infr_hip_internal_fail(INFR_ERR_UNSUPPORTED, "synth: dtype must be F32, Q8_0, Q4K, Q6K or Mxfp4");
     if (numel % 256 || offset % 256)
         return infr_hip_internal_fail(INFR_ERR_INVALID, "synth: offset and numel must be multiples of 256");
     const uint64_t n_super = numel / 256;

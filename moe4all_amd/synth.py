@@ -120,6 +120,9 @@ class MoeShape:
 CONFIG_1 = MoeShape("c1-single-layer-q8_0", 1, 2048, 128, 8, 768, DType.Q8_0, DType.Q8_0)
 CONFIG_2 = MoeShape("c2-qwen3-30b-a3b-q4k-q6k-48L", 48, 2048, 128, 8, 768, DType.Q4K, DType.Q6K)
 CONFIG_5 = MoeShape("c5-large-moe-256e-shared-q4k-q6k-40L", 40, 4096, 256, 8, 1536, DType.Q4K, DType.Q6K, shared_ff=1536)
+# the routed-expert shape of gpt-oss-120b (hidden and intermediate 2880, 128 experts, top-4, 36 layers) with its MXFP4
+# expert banks as they lie in a GGUF file: 60.9 GB resident
+CONFIG_MXFP4 = MoeShape("gptoss-120b-shape-mxfp4-36L", 36, 2880, 128, 4, 2880, DType.Mxfp4, DType.Mxfp4)
 
 
 class LayerWeights:

@@ -885,7 +885,7 @@ def test_sparse_batches_of_unit_formats_stay_on_the_per_pair_gemv(be, rows, grou
 from moe4all_amd import synth as S  # noqa: E402
 
 
-@pytest.mark.parametrize("dt", [DType.F32, DType.Q8_0, DType.Q4K, DType.Q6K])
+@pytest.mark.parametrize("dt", [DType.F32, DType.Q8_0, DType.Q4K, DType.Q6K, DType.Mxfp4])
 def test_device_generator_writes_the_host_generator_bytes(be, dt):
     numel = 256 * 1000
     seed = S.stream_seed(42, 7, int(dt))
@@ -898,7 +898,8 @@ def test_device_generator_writes_the_host_generator_bytes(be, dt):
 
 
 @pytest.mark.parametrize("shape,batch", [(S.CONFIG_1, 1), (S.CONFIG_2, 1), (S.CONFIG_1, 4), (S.CONFIG_1, 16),
-                                         (S.CONFIG_2, 8), (S.CONFIG_5, 1), (S.CONFIG_5, 8)])
+                                         (S.CONFIG_2, 8), (S.CONFIG_5, 1), (S.CONFIG_5, 8), (S.CONFIG_MXFP4, 1),
+                                         (S.CONFIG_MXFP4, 8)])
 def test_benchmark_config_layer_matches_oracle_at_full_size(be, shape, batch):
     """One full-size layer of each benchmark configuration: N(0,0.02) weights quantised on the
     device, N(0,1) activations; the oracle runs on the downloaded bytes."""

@@ -71,6 +71,31 @@ def test_quantise_then_oracle_decode_reconstructs_the_weights(dt, rel_rmse):
     assert (np.abs(back - w).reshape(-1, 256) <= step * amax * 1.01 + 1e-9).all()
 
 
+def test_mxfp4_quantiser_picks_the_nearest_code_under_the_shared_exponent():
+    """ggml's quantize_row_mxfp4_ref: shared exponent floor(log2(amax)) - 2, so that amax lands in [4, 8) code units
+    of the E2M1 range 0 .. 6; every element the nearest representable value.  Checked against a brute-force
+    nearest-value search under the same exponent and against the error bound of the format."""
+    w = S.normal(77, 32 * 500, 0.02)
+    q = S.quantize(DType.Mxfp4, w).reshape(-1, 17)
+    amax = np.abs(w.reshape(-1, 32)).max(axis=1)
+    want_e = np.floor(np.log2(amax)).astype(np.int64) - 2 + 127
+    assert np.array_equal(q[:, 0].astype(np.int64), want_e)
+    back = O.dequant(O.MXFP4, q.reshape(-1)).reshape(-1, 32)
+    unit = np.ldexp(1.0, want_e - 127)[:, None]                       # value of E2M1 1.0 in this block
+    grid = np.array([0, .5, 1, 1.5, 2, 3, 4, 6])
+    grid = np.concatenate([-grid[::-1], grid])
+    best = np.abs(w.reshape(-1, 32)[:, :, None] / unit[:, :, None] - grid).min(axis=2) * unit
+    assert np.allclose(np.abs(back - w.reshape(-1, 32)), best, rtol=0, atol=1e-9)
+    # magnitudes up to 6 units are at most half a step (<= 1 unit) away; amax in (6, 8) units clips to 6
+    assert (np.abs(back - w.reshape(-1, 32)) <= 2.0 * unit + 1e-9).all()
+    err = np.sqrt(np.mean((back.ravel() - w) ** 2)) / np.sqrt(np.mean(w ** 2))
+    assert 0.03 < err < 0.16, err
+    assert not O.dequant(O.MXFP4, S.quantize(DType.Mxfp4, np.zeros(64, np.float32))).any()
+    seed = S.stream_seed(2, 1, S.ROLE_UP)
+    a = S.weights_host(DType.Mxfp4, seed, 256 * 24, n_threads=3)
+    assert np.array_equal(a, S.quantize(DType.Mxfp4, S.normal(seed, 256 * 24, 0.02)))
+
+
 def test_quantisers_accept_degenerate_blocks():
     z = np.zeros(256, np.float32)
     for dt in (DType.Q8_0, DType.Q4K, DType.Q6K):
