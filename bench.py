@@ -206,6 +206,7 @@ def main():
         # banks on the 32-element-unit kernels: per-pair down results, then the rank-ordered sum as its own launch
         alg["moe_gate_up_units"], alg["moe_route_gate_up_units"] = alg["moe_gate_up"], alg["moe_route_gate_up"]
         alg["moe_down_units"] = n_sel * down_b + pairs * shape.n_ff * 4 + pairs * shape.ne * 4
+        alg["moe_down_combine_units"] = alg["moe_down_combine"]
         if not prefill and batch < 32:
             alg["moe_unbucket_combine"] = pairs * shape.ne * 4 + batch * shape.ne * 4
         alg["rms_norm_router_logits"] = alg["router_logits"] + shape.ne * 4 + batch * shape.ne * 4

@@ -1349,8 +1349,15 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                 }
                 gp.x = nullptr;
                 if (!gp.sh_down && !infr::moe_down_is_fast(gp) && infr::moe_down_units_supported(gp)) {
-                    // a down bank without an integer-dot kernel: per-pair rows on the unit kernel, then the
-                    // rank-ordered weighted sum
+                    // a down bank without an integer-dot kernel: the unit kernel over all slots of a row with the
+                    // rank-ordered weighted sum at its end, or per-pair rows and the sum as a launch of its own
+                    // (one or two token rows: from four rows on the per-pair grid spreads better; C2 shape, MXFP4:
+                    // 1 row 11.2 -> 6.9 us, 4 rows 22.6 -> 23.6, 8 rows 36.6 -> 45.4)
+                    if (rows <= 2 && infr::moe_down_combine_units_supported(gp)) {
+                        Timed t(be, "moe_down_combine_units");
+                        infr::launch_moe_down_combine_units(s, gp);
+                        break;
+                    }
                     {
                         Timed t(be, "moe_down_units");
                         infr::launch_moe_down_units(s, gp);

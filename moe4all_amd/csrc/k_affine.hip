@@ -113,6 +113,9 @@ __global__ __launch_bounds__(256) void linear_units_kernel(const float* __restri
 // combine launch.  An expert id outside the bank (possible with caller-given ids) yields zeros.
 template <int DT, bool GATE_UP>
 __global__ __launch_bounds__(256) void moe_units_kernel(MoeGemvParams p, size_t row_bytes) {
+    // output rows a wave has in flight: two rows of two matrices for gate/up (two rounds per 16-row tile), four
+    // rows for down (one round; measured 11.5 -> 10.0 us on 2880 x 2880 MXFP4 banks, four rows of gate/up are slower)
+    constexpr int kRW = GATE_UP ? 2 : 4;
     extern __shared__ float lds[];
     const int in_f = GATE_UP ? p.ne : p.nff, out_f = GATE_UP ? p.nff : p.ne;
     const int n_units = in_f >> 5;
@@ -177,33 +180,33 @@ __global__ __launch_bounds__(256) void moe_units_kernel(MoeGemvParams p, size_t 
     const uint8_t* base[M];
     base[0] = (GATE_UP ? p.gate + (size_t)e * p.gate_stride : p.down + (size_t)e * p.down_stride);
     if constexpr (GATE_UP) base[1] = p.up + (size_t)e * p.up_stride;
-    for (int round = 0; round < kRowsPerBlock / (4 * kRowsPerWave); round++) {
-        const int o0 = row_base + (round * 4 + wave) * kRowsPerWave;
+    for (int round = 0; round < kRowsPerBlock / (4 * kRW); round++) {
+        const int o0 = row_base + (round * 4 + wave) * kRW;
         if (o0 >= out_f) break;
-        float acc[kRowsPerWave][M];
+        float acc[kRW][M];
 #pragma unroll
-        for (int a = 0; a < kRowsPerWave; a++)
+        for (int a = 0; a < kRW; a++)
 #pragma unroll
             for (int mi = 0; mi < M; mi++) acc[a][mi] = 0.0f;
         for (int u = lane; u < n_units; u += kWave) {
-            Unit t[kRowsPerWave][M];
+            Unit t[kRW][M];
 #pragma unroll
-            for (int a = 0; a < kRowsPerWave; a++) {
+            for (int a = 0; a < kRW; a++) {
                 const int o = o0 + a < out_f ? o0 + a : out_f - 1;
 #pragma unroll
                 for (int mi = 0; mi < M; mi++) load_unit<DT>(base[mi] + (size_t)o * row_bytes, u, t[a][mi]);
             }
             const float* xu = xs + (size_t)u * kUnitStride;
-            float sh[kRowsPerWave][M][2];
+            float sh[kRW][M][2];
 #pragma unroll
-            for (int a = 0; a < kRowsPerWave; a++)
+            for (int a = 0; a < kRW; a++)
 #pragma unroll
                 for (int mi = 0; mi < M; mi++) sh[a][mi][0] = sh[a][mi][1] = 0.0f;
 #pragma unroll
             for (int k = 0; k < 8; k++) {
                 const float4 xv = reinterpret_cast<const float4*>(xu)[k];
 #pragma unroll
-                for (int a = 0; a < kRowsPerWave; a++)
+                for (int a = 0; a < kRW; a++)
 #pragma unroll
                     for (int mi = 0; mi < M; mi++) {
                         const uint32_t q = t[a][mi].q[k];
@@ -216,14 +219,14 @@ __global__ __launch_bounds__(256) void moe_units_kernel(MoeGemvParams p, size_t 
             }
             const float2 xsu = *reinterpret_cast<const float2*>(xsum + 2 * u);
 #pragma unroll
-            for (int a = 0; a < kRowsPerWave; a++)
+            for (int a = 0; a < kRW; a++)
 #pragma unroll
                 for (int mi = 0; mi < M; mi++)
                     acc[a][mi] += (t[a][mi].sc[0] * sh[a][mi][0] + t[a][mi].mn[0] * xsu.x) +
                                   (t[a][mi].sc[1] * sh[a][mi][1] + t[a][mi].mn[1] * xsu.y);
         }
 #pragma unroll
-        for (int a = 0; a < kRowsPerWave; a++) {
+        for (int a = 0; a < kRW; a++) {
             float v[M];
 #pragma unroll
             for (int mi = 0; mi < M; mi++) v[mi] = wave_sum(acc[a][mi]);
@@ -427,6 +430,132 @@ void launch_moe_units_bucketed_any(hipStream_t s, int dt, const MoeGemvParams& p
     }
 }
 
+// Decode: the down stage and the rank-ordered weighted sum of a token row in one launch.  grid.x = tiles of 16
+// output elements, grid.y = token row; sixteen waves share out the (slot, four-row group) items of the tile, each
+// dot computed exactly as moe_units_kernel<DT, false> computes it (same lane-to-unit map, same sums), so the
+// result has the bits of that kernel followed by the combine kernel.  The row's n_used activation rows h are
+// staged once per block.
+constexpr int kDcRows = 4;
+template <int DT, int kDcTile>
+__global__ __launch_bounds__(1024) void moe_down_combine_units_kernel(MoeGemvParams p, size_t row_bytes) {
+    extern __shared__ float lds[];
+    const int n_units = p.nff >> 5, K = p.n_used;
+    float* xs = lds;                                              // [K][n_units][kUnitStride]
+    float* xsum = xs + (size_t)K * n_units * kUnitStride;         // [K][2 * n_units]
+    float* ys = xsum + (size_t)K * 2 * n_units;                   // [K][kDcTile]
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int r = blockIdx.y, row_base = blockIdx.x * kDcTile;
+    for (int idx = tid; idx < K * 2 * n_units; idx += 1024) {
+        const int k = idx / (2 * n_units), hu = idx - k * 2 * n_units;
+        const float* xrow = p.h + ((size_t)r * K + k) * p.nff;
+        float4 v[4];
+        float sm = 0.0f;
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            v[q] = reinterpret_cast<const float4*>(xrow + 16 * hu)[q];
+            sm += (v[q].x + v[q].y) + (v[q].z + v[q].w);
+        }
+        float* d = xs + ((size_t)k * n_units + (hu >> 1)) * kUnitStride + 16 * (hu & 1);
+#pragma unroll
+        for (int q = 0; q < 4; q++) reinterpret_cast<float4*>(d)[q] = v[q];
+        xsum[idx] = sm;
+    }
+    __syncthreads();
+    constexpr int kGroups = kDcTile / kDcRows;
+    for (int it = wave; it < K * kGroups; it += 16) {
+        const int k = it / kGroups, o0 = row_base + (it - k * kGroups) * kDcRows;
+        if (o0 >= p.ne) continue;
+        const int e = p.ids[(size_t)r * K + k];
+        float v[kDcRows];
+#pragma unroll
+        for (int a = 0; a < kDcRows; a++) v[a] = 0.0f;
+        if (e >= 0 && e < p.n_expert) {   // an id outside the bank contributes zeros, as in the separate kernels
+            const uint8_t* base = p.down + (size_t)e * p.down_stride;
+            const float* xk = xs + (size_t)k * n_units * kUnitStride;
+            const float* sk = xsum + (size_t)k * 2 * n_units;
+            float acc[kDcRows];
+#pragma unroll
+            for (int a = 0; a < kDcRows; a++) acc[a] = 0.0f;
+            for (int u = lane; u < n_units; u += kWave) {
+                Unit t[kDcRows];
+#pragma unroll
+                for (int a = 0; a < kDcRows; a++) {
+                    const int o = o0 + a < p.ne ? o0 + a : p.ne - 1;
+                    load_unit<DT>(base + (size_t)o * row_bytes, u, t[a]);
+                }
+                const float* xu = xk + (size_t)u * kUnitStride;
+                float sh[kDcRows][2];
+#pragma unroll
+                for (int a = 0; a < kDcRows; a++) sh[a][0] = sh[a][1] = 0.0f;
+#pragma unroll
+                for (int q = 0; q < 8; q++) {
+                    const float4 xv = reinterpret_cast<const float4*>(xu)[q];
+#pragma unroll
+                    for (int a = 0; a < kDcRows; a++) {
+                        const uint32_t c = t[a].q[q];
+                        float& w = sh[a][q >> 2];
+                        w = fmaf((float)(c & 0xFFu), xv.x, w);
+                        w = fmaf((float)((c >> 8) & 0xFFu), xv.y, w);
+                        w = fmaf((float)((c >> 16) & 0xFFu), xv.z, w);
+                        w = fmaf((float)(c >> 24), xv.w, w);
+                    }
+                }
+                const float2 xsu = *reinterpret_cast<const float2*>(sk + 2 * u);
+#pragma unroll
+                for (int a = 0; a < kDcRows; a++)
+                    acc[a] += (t[a].sc[0] * sh[a][0] + t[a].mn[0] * xsu.x) + (t[a].sc[1] * sh[a][1] + t[a].mn[1] * xsu.y);
+            }
+#pragma unroll
+            for (int a = 0; a < kDcRows; a++) {
+                v[a] = wave_sum(acc[a]);
+                if (p.down_scale) v[a] = __fmul_rn(v[a], p.down_scale[e]);
+            }
+        }
+        if (lane == 0) {
+#pragma unroll
+            for (int a = 0; a < kDcRows; a++) ys[k * kDcTile + (o0 - row_base) + a] = v[a];
+        }
+    }
+    __syncthreads();
+    if (tid < kDcTile && row_base + tid < p.ne) {
+        float acc = 0.0f;
+        for (int k = 0; k < K; k++) {   // rank order, separate multiply and add (crates/infr-cpu/src/lib.rs:4290-4302)
+            const float w = p.weights[(size_t)r * K + k];
+            if (p.skip_zero_w && w == 0.0f) continue;
+            acc = __fadd_rn(acc, __fmul_rn(p.weight_before ? 1.0f : w, ys[k * kDcTile + tid]));
+        }
+        const size_t oi = (size_t)r * p.ne + row_base + tid;
+        p.dst[oi] = p.addend ? __fadd_rn(p.addend[oi], acc) : acc;
+    }
+}
+
+// Output elements per block: as many as give every one of the sixteen waves one (slot, four-row group) item.
+int down_combine_units_tile(int n_used) { return n_used <= 4 ? 16 : n_used <= 8 ? 8 : 4; }
+size_t down_combine_units_lds(const MoeGemvParams& p) {
+    return ((size_t)p.n_used * (p.nff >> 5) * (kUnitStride + 2) + (size_t)p.n_used * 16) * sizeof(float);
+}
+
+template <int DT, int TILE>
+void launch_moe_down_combine_units_t(hipStream_t s, const MoeGemvParams& p) {
+    int be = 1, bb = 4;
+    block_geometry(DT, &be, &bb);
+    static bool attr_set = false;
+    if (!attr_set) {
+        (void)hipFuncSetAttribute((const void*)moe_down_combine_units_kernel<DT, TILE>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  158 * 1024);
+        attr_set = true;
+    }
+    dim3 grid((p.ne + TILE - 1) / TILE, p.rows), block(1024);
+    INFR_LAUNCH((moe_down_combine_units_kernel<DT, TILE>), grid, block, down_combine_units_lds(p), s, p, (size_t)(p.nff / be) * bb);
+}
+template <int DT>
+void launch_moe_down_combine_units_dt(hipStream_t s, const MoeGemvParams& p) {
+    const int tile = down_combine_units_tile(p.n_used);
+    if (tile == 16) launch_moe_down_combine_units_t<DT, 16>(s, p);
+    else if (tile == 8) launch_moe_down_combine_units_t<DT, 8>(s, p);
+    else launch_moe_down_combine_units_t<DT, 4>(s, p);
+}
+
 template <int DT, bool GATE_UP>
 void launch_moe_units_dt(hipStream_t s, const MoeGemvParams& p) {
     const int in_f = GATE_UP ? p.ne : p.nff, out_f = GATE_UP ? p.nff : p.ne;
@@ -600,6 +729,19 @@ bool moe_down_units_supported(const MoeGemvParams& p) {
     return p.y != nullptr && p.rows * p.n_used <= 65535 && linear_units_supported(p.down_dt, p.nff, p.h);
 }
 void launch_moe_down_units(hipStream_t s, const MoeGemvParams& p) { launch_moe_units_any<false>(s, p.down_dt, p); }
+// The fused form needs the row's n_used activation rows side by side in LDS.
+bool moe_down_combine_units_supported(const MoeGemvParams& p) {
+    return p.rows * p.n_used <= 65535 && p.n_used <= 16 && linear_units_supported(p.down_dt, p.nff, p.h) &&
+           down_combine_units_lds(p) <= 144 * 1024;
+}
+void launch_moe_down_combine_units(hipStream_t s, const MoeGemvParams& p) {
+    switch (p.down_dt) {
+#define INFR_UNITS(D) case D: launch_moe_down_combine_units_dt<D>(s, p); break;
+        INFR_FOR_UNIT_FORMATS(INFR_UNITS)
+#undef INFR_UNITS
+        default: break;
+    }
+}
 
 // x and h rows must be 16-byte aligned: ne and nff are multiples of 32 here, the bases are checked by the caller.
 bool moe_units_batch_supported(int gate_dt, int up_dt, int down_dt, int ne, int nff) {

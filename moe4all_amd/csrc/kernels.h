@@ -176,6 +176,8 @@ void launch_moe_gate_up_units(hipStream_t s, const MoeGemvParams& p);
 bool moe_gate_up_units_routes_inline(const MoeGemvParams& p);
 bool moe_down_units_supported(const MoeGemvParams& p);
 void launch_moe_down_units(hipStream_t s, const MoeGemvParams& p);
+bool moe_down_combine_units_supported(const MoeGemvParams& p);
+void launch_moe_down_combine_units(hipStream_t s, const MoeGemvParams& p);
 // Batches on the unit kernels: an expert's rows are fetched once per chunk of tokens of its bucket
 // (p.bk_offsets / p.bk_pair_src from launch_bucket); h and y are written in bucket order.
 bool moe_units_batch_supported(int gate_dt, int up_dt, int down_dt, int ne, int nff);

@@ -262,9 +262,10 @@ def _bank_weights(rng, E, nff, ne, gdt, ddt):
             H.centred_weight(ddt, E * ne * nff, 3))
 
 
+@pytest.mark.parametrize("rows", [3, 1])   # one row: the unit formats' down stage and combine are one launch
 @pytest.mark.parametrize("gdt,ddt", [(H.Q4K, H.Q6K), (H.Q5K, H.Q4_0)])
-def test_moe_ffn_option_variants_match_oracle(be, gdt, ddt):
-    ne, E, K, nff, rows = 256, 8, 3, 256, 3
+def test_moe_ffn_option_variants_match_oracle(be, gdt, ddt, rows):
+    ne, E, K, nff = 256, 8, 3, 256
     rng = np.random.default_rng(21)
     x = rng.standard_normal((rows, ne)).astype(np.float32)
     router = rng.standard_normal((E, ne)).astype(np.float32) * 0.05
@@ -845,7 +846,7 @@ def test_moe_ffn_with_experts_in_the_other_affine_formats(be, gdt, ddt, rows, ne
     else:
         # routing rides in the gate/up kernel while rows * n_expert <= 512 (as on the integer-dot kernels)
         assert ("moe_route_gate_up_units" if rows * E <= 512 else "moe_gate_up_units") in names
-        assert ("route_topk" in names) == (rows * E > 512) and ("moe_down_units" in names or ddt == H.Q6K)
+        assert ("route_topk" in names) == (rows * E > 512) and (("moe_down_combine_units" if rows <= 2 else "moe_down_units") in names or ddt == H.Q6K)
     keep[0].free()
     for buf in keep[2] + [keep[3]]:
         buf.free()
