@@ -829,6 +829,52 @@ __global__ __launch_bounds__(256) void unbucket_combine_kernel(const Y* __restri
     }
 }
 
+// The same sum for f16 pair rows whose length is a multiple of 8: eight elements (16 bytes) per lane and slot, all
+// slots of the row requested before the first is used.  Same operations per element as the kernel above.
+template <int K>
+__global__ __launch_bounds__(256) void unbucket_combine_h8_kernel(const _Float16* __restrict__ y, const int32_t* __restrict__ slot_pair,
+                                                                  const float* __restrict__ weights, int ne, int weight_before,
+                                                                  float* dst, int identity, const float* __restrict__ pair_scale,
+                                                                  const float* addend, int skip_zero_w) {
+    const size_t row = blockIdx.y;
+    const int i = (blockIdx.x * 256 + threadIdx.x) * 8;
+    if (i >= ne) return;
+    uint4 raw[K];
+    float w[K], sc[K];
+    bool live[K];
+#pragma unroll
+    for (int k = 0; k < K; k++) {
+        int pr = slot_pair ? slot_pair[row * K + k] : 0;
+        const float wk = weights[row * K + k];
+        live[k] = pr >= 0 && !(skip_zero_w && wk == 0.0f);
+        if (identity || !slot_pair) pr = (int)(row * K + k);
+        w[k] = weight_before ? 1.0f : wk;
+        sc[k] = live[k] ? pair_scale[pr] : 0.0f;
+        raw[k] = live[k] ? *reinterpret_cast<const uint4*>(y + (size_t)pr * ne + i) : make_uint4(0, 0, 0, 0);
+    }
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int k = 0; k < K; k++) {
+        if (!live[k]) continue;
+        const uint32_t d[4] = {raw[k].x, raw[k].y, raw[k].z, raw[k].w};
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const half2v h = as_h2(d[q]);
+            acc[2 * q] = __fadd_rn(acc[2 * q], __fmul_rn(w[k], (float)h[0] * sc[k]));
+            acc[2 * q + 1] = __fadd_rn(acc[2 * q + 1], __fmul_rn(w[k], (float)h[1] * sc[k]));
+        }
+    }
+    float* o = dst + row * ne + i;
+    if (addend) {
+        const float4 a0 = *reinterpret_cast<const float4*>(addend + row * ne + i), a1 = *reinterpret_cast<const float4*>(addend + row * ne + i + 4);
+        const float ad[8] = {a0.x, a0.y, a0.z, a0.w, a1.x, a1.y, a1.z, a1.w};
+#pragma unroll
+        for (int q = 0; q < 8; q++) acc[q] = __fadd_rn(ad[q], acc[q]);
+    }
+    *reinterpret_cast<float4*>(o) = make_float4(acc[0], acc[1], acc[2], acc[3]);
+    *reinterpret_cast<float4*>(o + 4) = make_float4(acc[4], acc[5], acc[6], acc[7]);
+}
+
 template <class F>
 void rows_to_f16(hipStream_t s, const float* src, int rows, int n, _Float16* dst, float* scale) {
     INFR_LAUNCH(rows_to_f16_kernel<F>, dim3(rows), dim3(256), 0, s, src, n, dst, scale);
@@ -1287,6 +1333,19 @@ void launch_unbucket_combine(hipStream_t s, const void* y, const int32_t* slot_p
                              const float* addend, int skip_zero_w) {
     if (rows <= 0) return;
     const dim3 grid((ne + 1023) / 1024, rows), block(256);
+    if (pair_scale && ne % 8 == 0 && (((uintptr_t)y | (uintptr_t)dst | (uintptr_t)addend) & 15) == 0 &&
+        (n_used == 8 || n_used == 4 || n_used == 6 || n_used == 2)) {
+        const dim3 g8((ne + 2047) / 2048, rows);
+#define INFR_H8(KK)                                                                                                       \
+    INFR_LAUNCH(unbucket_combine_h8_kernel<KK>, g8, block, 0, s, (const _Float16*)y, slot_pair, weights, ne, weight_before, \
+                dst, identity, pair_scale, addend, skip_zero_w)
+        if (n_used == 8) INFR_H8(8);
+        else if (n_used == 6) INFR_H8(6);
+        else if (n_used == 4) INFR_H8(4);
+        else INFR_H8(2);
+#undef INFR_H8
+        return;
+    }
     if (pair_scale)
         INFR_LAUNCH(unbucket_combine_kernel<_Float16>, grid, block, 0, s, (const _Float16*)y, slot_pair, weights, ne, n_used,
                     weight_before, dst, identity, pair_scale, addend, skip_zero_w);
