@@ -200,38 +200,46 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const uint8_t* __res
 // feeds 16 FMAs.  k advances in chunks of 128 elements staged transposed (chain-major) in LDS;
 // the accumulators run through all chunks, so every chain still adds its terms in ascending
 // order, exactly as the scalar reference does.
-constexpr int kLtTile = 32, kLtChunk = 128, kLtStride = kLtChunk / 8 + 4;
-__global__ __launch_bounds__(512) void router_logits_tiled_kernel(const float* __restrict__ router, size_t row_floats,
-                                                                  const float* __restrict__ x, int ne, int n_expert,
-                                                                  int rows, float* __restrict__ logits) {
+constexpr int kLtChunk = 128, kLtStride = kLtChunk / 8 + 4;
+// kLtTile experts x kLtTile rows per block, (kLtTile / 4)^2 * 8 threads: 32 (512 threads) for large batches, 16
+// (128 threads) when 32-wide tiles would leave compute units without a block.
+template <int kLtTile>
+__global__ __launch_bounds__(kLtTile * kLtTile / 2) void router_logits_tiled_kernel(const float* __restrict__ router,
+                                                                                      size_t row_floats,
+                                                                                      const float* __restrict__ x, int ne,
+                                                                                      int n_expert, int rows,
+                                                                                      float* __restrict__ logits) {
+    constexpr int NT = kLtTile * kLtTile / 2;    // threads
+    constexpr int G = kLtTile / 4;               // 4-row (4-expert) groups per tile side
+    constexpr int NQ = kLtTile * 32 / NT;        // float4 per thread, operand and chunk
     __shared__ float sw[kLtTile * 8 * kLtStride];
     __shared__ float sx[kLtTile * 8 * kLtStride];
-    const int tid = threadIdx.x, j = tid & 7, rg = (tid >> 3) & 7, eg = tid >> 6;
+    const int tid = threadIdx.x, j = tid & 7, rg = (tid >> 3) % G, eg = tid / (8 * G);
     const int e0 = blockIdx.x * kLtTile, r0 = blockIdx.y * kLtTile;
     float acc[4][4];
 #pragma unroll
     for (int a = 0; a < 4; a++)
 #pragma unroll
         for (int b = 0; b < 4; b++) acc[a][b] = 0.0f;
-    // staging role: two float4 of the router tile and two of the activation tile per chunk
-    const float* src[4];
-    bool ok[4];
-    int dst_base[4];
+    // staging role: NQ float4 of the router tile and NQ of the activation tile per chunk
+    const float* src[2 * NQ];
+    bool ok[2 * NQ];
+    int dst_base[2 * NQ];
 #pragma unroll
-    for (int q = 0; q < 4; q++) {
-        const int idx = tid + 512 * (q & 1), row = idx >> 5, v = idx & 31;
-        const bool is_x = q >= 2;
+    for (int q = 0; q < 2 * NQ; q++) {
+        const int idx = tid + NT * (q % NQ), row = idx >> 5, v = idx & 31;
+        const bool is_x = q >= NQ;
         const int g = (is_x ? r0 : e0) + row;
         ok[q] = g < (is_x ? rows : n_expert);
         src[q] = (is_x ? x + (size_t)(ok[q] ? g : 0) * ne : router + (size_t)(ok[q] ? g : 0) * row_floats) + 4 * v;
         // element 4v+t of the chunk: chain (4v+t)&7 = 4(v&1)+t, step (4v+t)>>3 = v>>1
         dst_base[q] = (row * 8 + 4 * (v & 1)) * kLtStride + (v >> 1);
     }
-    float4 st[4];
+    float4 st[2 * NQ];
     auto fetch = [&](int k0) {
 #pragma unroll
-        for (int q = 0; q < 4; q++) {
-            const int v4 = 4 * ((tid + 512 * (q & 1)) & 31);
+        for (int q = 0; q < 2 * NQ; q++) {
+            const int v4 = 4 * ((tid + NT * (q % NQ)) & 31);
             st[q] = (ok[q] && k0 + v4 < ne) ? *reinterpret_cast<const float4*>(src[q] + k0) : make_float4(0.f, 0.f, 0.f, 0.f);
         }
     };
@@ -239,8 +247,8 @@ __global__ __launch_bounds__(512) void router_logits_tiled_kernel(const float* _
     for (int k0 = 0; k0 < ne; k0 += kLtChunk) {
         __syncthreads();
 #pragma unroll
-        for (int q = 0; q < 4; q++) {
-            float* d = (q >= 2 ? sx : sw) + dst_base[q];
+        for (int q = 0; q < 2 * NQ; q++) {
+            float* d = (q >= NQ ? sx : sw) + dst_base[q];
             d[0] = st[q].x;
             d[kLtStride] = st[q].y;
             d[2 * kLtStride] = st[q].z;
@@ -294,9 +302,16 @@ bool launch_router_logits(hipStream_t s, const uint8_t* router, int rdt, size_t 
                        (((uintptr_t)x | (uintptr_t)nrm.weight | (uintptr_t)nrm.xn_out) & 15) != 0))
         return false;
     if (rows >= 32 && rdt == INFR_F32 && (ne & 31) == 0 && (row_bytes & 15) == 0) {
-        dim3 grid((n_expert + kLtTile - 1) / kLtTile, (rows + kLtTile - 1) / kLtTile);
-        INFR_LAUNCH(router_logits_tiled_kernel, grid, dim3(512), 0, s, reinterpret_cast<const float*>(router), row_bytes / 4,
-                    x, ne, n_expert, rows, logits);
+        // 32 x 32 tiles when they give every compute unit a block, 16 x 16 otherwise
+        if ((size_t)((n_expert + 31) / 32) * ((rows + 31) / 32) >= 256) {
+            dim3 grid((n_expert + 31) / 32, (rows + 31) / 32);
+            INFR_LAUNCH(router_logits_tiled_kernel<32>, grid, dim3(512), 0, s, reinterpret_cast<const float*>(router),
+                        row_bytes / 4, x, ne, n_expert, rows, logits);
+        } else {
+            dim3 grid((n_expert + 15) / 16, (rows + 15) / 16);
+            INFR_LAUNCH(router_logits_tiled_kernel<16>, grid, dim3(128), 0, s, reinterpret_cast<const float*>(router),
+                        row_bytes / 4, x, ne, n_expert, rows, logits);
+        }
         return true;
     }
     // Decode and small batches of an f32 router: many small blocks of 2 experts x 2 rows, each
