@@ -201,26 +201,27 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const uint8_t* __res
 // the accumulators run through all chunks, so every chain still adds its terms in ascending
 // order, exactly as the scalar reference does.
 constexpr int kLtChunk = 128, kLtStride = kLtChunk / 8 + 4;
-// kLtTile experts x kLtTile rows per block, (kLtTile / 4)^2 * 8 threads: 32 (512 threads) for large batches, 16
-// (128 threads) when 32-wide tiles would leave compute units without a block.
-template <int kLtTile>
-__global__ __launch_bounds__(kLtTile * kLtTile / 2) void router_logits_tiled_kernel(const float* __restrict__ router,
+// kLtTile experts x kLtTile rows per block, a P x P patch per thread: 32 / 4 (512 threads) for large batches; 16 / 2
+// (512 threads, a quarter of the chain work per thread) when 32-wide tiles would leave compute units without a block:
+// a block's time is its chunks' latency chain, which the smaller patch shortens.
+template <int kLtTile, int P>
+__global__ __launch_bounds__((kLtTile / P) * (kLtTile / P) * 8) void router_logits_tiled_kernel(const float* __restrict__ router,
                                                                                       size_t row_floats,
                                                                                       const float* __restrict__ x, int ne,
                                                                                       int n_expert, int rows,
                                                                                       float* __restrict__ logits) {
-    constexpr int NT = kLtTile * kLtTile / 2;    // threads
-    constexpr int G = kLtTile / 4;               // 4-row (4-expert) groups per tile side
+    constexpr int G = kLtTile / P;               // P-row (P-expert) groups per tile side
+    constexpr int NT = G * G * 8;                // threads: a P x P patch of (expert, row) pairs for each of 8 chains
     constexpr int NQ = kLtTile * 32 / NT;        // float4 per thread, operand and chunk
     __shared__ float sw[kLtTile * 8 * kLtStride];
     __shared__ float sx[kLtTile * 8 * kLtStride];
     const int tid = threadIdx.x, j = tid & 7, rg = (tid >> 3) % G, eg = tid / (8 * G);
     const int e0 = blockIdx.x * kLtTile, r0 = blockIdx.y * kLtTile;
-    float acc[4][4];
+    float acc[P][P];
 #pragma unroll
-    for (int a = 0; a < 4; a++)
+    for (int a = 0; a < P; a++)
 #pragma unroll
-        for (int b = 0; b < 4; b++) acc[a][b] = 0.0f;
+        for (int b = 0; b < P; b++) acc[a][b] = 0.0f;
     // staging role: NQ float4 of the router tile and NQ of the activation tile per chunk
     const float* src[2 * NQ];
     bool ok[2 * NQ];
@@ -257,19 +258,19 @@ __global__ __launch_bounds__(kLtTile * kLtTile / 2) void router_logits_tiled_ker
         __syncthreads();
         if (k0 + kLtChunk < ne) fetch(k0 + kLtChunk);
         const int n_c = min(kLtChunk, ne - k0) >> 3;  // a multiple of 4
-        const float* wp = sw + (eg * 4 * 8 + j) * kLtStride;
-        const float* xp = sx + (rg * 4 * 8 + j) * kLtStride;
+        const float* wp = sw + (eg * P * 8 + j) * kLtStride;
+        const float* xp = sx + (rg * P * 8 + j) * kLtStride;
         for (int c = 0; c < n_c; c += 4) {
-            float4 wv[4], xv[4];
+            float4 wv[P], xv[P];
 #pragma unroll
-            for (int a = 0; a < 4; a++) {
+            for (int a = 0; a < P; a++) {
                 wv[a] = *reinterpret_cast<const float4*>(wp + a * 8 * kLtStride + c);
                 xv[a] = *reinterpret_cast<const float4*>(xp + a * 8 * kLtStride + c);
             }
 #pragma unroll
-            for (int a = 0; a < 4; a++)
+            for (int a = 0; a < P; a++)
 #pragma unroll
-                for (int b = 0; b < 4; b++) {
+                for (int b = 0; b < P; b++) {
                     acc[a][b] = __fmaf_rn(wv[a].x, xv[b].x, acc[a][b]);
                     acc[a][b] = __fmaf_rn(wv[a].y, xv[b].y, acc[a][b]);
                     acc[a][b] = __fmaf_rn(wv[a].z, xv[b].z, acc[a][b]);
@@ -279,13 +280,13 @@ __global__ __launch_bounds__(kLtTile * kLtTile / 2) void router_logits_tiled_ker
     }
     const int lane = tid & 63;
 #pragma unroll
-    for (int a = 0; a < 4; a++)
+    for (int a = 0; a < P; a++)
 #pragma unroll
-        for (int b = 0; b < 4; b++) {
+        for (int b = 0; b < P; b++) {
             float s = 0.0f;
 #pragma unroll
             for (int jj = 0; jj < 8; jj++) s = __fadd_rn(s, __shfl(acc[a][b], (lane & ~7) + jj, kWave));
-            const int e = e0 + eg * 4 + a, r = r0 + rg * 4 + b;
+            const int e = e0 + eg * P + a, r = r0 + rg * P + b;
             if (j == 0 && e < n_expert && r < rows) logits[(size_t)r * n_expert + e] = s;
         }
 }
@@ -305,11 +306,11 @@ bool launch_router_logits(hipStream_t s, const uint8_t* router, int rdt, size_t 
         // 32 x 32 tiles when they give every compute unit a block, 16 x 16 otherwise
         if ((size_t)((n_expert + 31) / 32) * ((rows + 31) / 32) >= 256) {
             dim3 grid((n_expert + 31) / 32, (rows + 31) / 32);
-            INFR_LAUNCH(router_logits_tiled_kernel<32>, grid, dim3(512), 0, s, reinterpret_cast<const float*>(router),
+            INFR_LAUNCH((router_logits_tiled_kernel<32, 4>), grid, dim3(512), 0, s, reinterpret_cast<const float*>(router),
                         row_bytes / 4, x, ne, n_expert, rows, logits);
         } else {
             dim3 grid((n_expert + 15) / 16, (rows + 15) / 16);
-            INFR_LAUNCH(router_logits_tiled_kernel<16>, grid, dim3(128), 0, s, reinterpret_cast<const float*>(router),
+            INFR_LAUNCH((router_logits_tiled_kernel<16, 2>), grid, dim3(512), 0, s, reinterpret_cast<const float*>(router),
                         row_bytes / 4, x, ne, n_expert, rows, logits);
         }
         return true;
