@@ -807,7 +807,8 @@ def test_batched_linear_reads_a_row_band_of_a_concatenated_weight(be):
     (H.Q4_0, H.Q5_0, 40, 480, 96), (H.Q4_1, H.Q4_1, 70, 96, 32),
     (H.MXFP4, H.MXFP4, 1, 512, 256), (H.MXFP4, H.MXFP4, 64, 512, 256), (H.IQ4_XS, H.IQ4_NL, 3, 512, 256),
     (H.IQ4_NL, H.IQ4_XS, 40, 512, 256), (H.NVFP4, H.Q2_0, 2, 512, 256), (H.TQ2_0, H.TQ1_0, 5, 512, 256),
-    (H.TQ1_0, H.TQ2_0, 50, 256, 256), (H.Q2_0, H.NVFP4, 35, 192, 320), (H.MXFP4, H.IQ4_NL, 40, 480, 96)])
+    (H.TQ1_0, H.TQ2_0, 50, 256, 256), (H.Q2_0, H.NVFP4, 35, 192, 320), (H.MXFP4, H.IQ4_NL, 40, 480, 96),
+    (H.Q4K, H.Q5K, 48, 512, 256), (H.Q8_0, H.Q5K, 40, 512, 256), (H.Q6K, H.Q4_1, 36, 256, 256)])
 def test_moe_ffn_with_experts_in_the_other_affine_formats(be, gdt, ddt, rows, ne, nff):
     """Expert banks in formats without an integer-dot kernel.  Up to 31 rows: the 32-element-unit GEMV kernels,
     one block column per (row, rank) pair (f32, bar 1e-3).  From 32 rows: bucketing + the unit-decoder grouped
