@@ -112,7 +112,7 @@ __global__ __launch_bounds__(256) void linear_units_kernel(const float* __restri
 // down: y[pair, o] = down . h[pair] (* down_scale[e]); the rank-ordered weighted sum is a separate
 // combine launch.  An expert id outside the bank (possible with caller-given ids) yields zeros.
 template <int DT, bool GATE_UP>
-__global__ __launch_bounds__(256) void moe_units_kernel(MoeGemvParams p, size_t row_bytes) {
+__global__ __launch_bounds__(256) void moe_units_kernel(MoeGemvParams p, size_t row_bytes, int kRB) {
     // output rows a wave has in flight: two rows of two matrices for gate/up (two rounds per 16-row tile), four
     // rows for down (one round; measured 11.5 -> 10.0 us on 2880 x 2880 MXFP4 banks, four rows of gate/up are slower)
     constexpr int kRW = GATE_UP ? 2 : 4;
@@ -125,7 +125,7 @@ __global__ __launch_bounds__(256) void moe_units_kernel(MoeGemvParams p, size_t 
     const int pair = blockIdx.y, r = pair / p.n_used;
     const float* xrow = GATE_UP ? p.x + (size_t)r * p.ne : p.h + (size_t)pair * p.nff;
     float* out = GATE_UP ? p.h + (size_t)pair * p.nff : p.y + (size_t)pair * p.ne;
-    const int row_base = blockIdx.x * kRowsPerBlock;
+    const int row_base = blockIdx.x * kRB;
     // gate/up with routing folded in: the block routes its token row itself (one wave, the same routine as the
     // routing kernel) while the activation row is on its way; block column 0 of a row's first pair stores the result
     const bool routes = GATE_UP && p.route_inline;
@@ -136,7 +136,7 @@ __global__ __launch_bounds__(256) void moe_units_kernel(MoeGemvParams p, size_t 
     if (!routes) {
         e = p.ids[pair];
         if (e < 0 || e >= p.n_expert) {
-            for (int o = row_base + tid; o < min(row_base + kRowsPerBlock, out_f); o += 256) out[o] = 0.0f;
+            for (int o = row_base + tid; o < min(row_base + kRB, out_f); o += 256) out[o] = 0.0f;
             return;
         }
     } else if (wave == 3) {
@@ -169,7 +169,7 @@ __global__ __launch_bounds__(256) void moe_units_kernel(MoeGemvParams p, size_t 
             e = s_ids[slot];
             w_before = s_w[slot];
             if (e < 0 || e >= p.n_expert) {
-                for (int o = row_base + tid; o < min(row_base + kRowsPerBlock, out_f); o += 256) out[o] = 0.0f;
+                for (int o = row_base + tid; o < min(row_base + kRB, out_f); o += 256) out[o] = 0.0f;
                 return;
             }
         } else if (p.weight_before) {
@@ -180,7 +180,7 @@ __global__ __launch_bounds__(256) void moe_units_kernel(MoeGemvParams p, size_t 
     const uint8_t* base[M];
     base[0] = (GATE_UP ? p.gate + (size_t)e * p.gate_stride : p.down + (size_t)e * p.down_stride);
     if constexpr (GATE_UP) base[1] = p.up + (size_t)e * p.up_stride;
-    for (int round = 0; round < kRowsPerBlock / (4 * kRW); round++) {
+    for (int round = 0; round < kRB / (4 * kRW); round++) {
         const int o0 = row_base + (round * 4 + wave) * kRW;
         if (o0 >= out_f) break;
         float acc[kRW][M];
@@ -567,10 +567,14 @@ void launch_moe_units_dt(hipStream_t s, const MoeGemvParams& p) {
         (void)hipFuncSetAttribute((const void*)moe_units_kernel<DT, GATE_UP>, hipFuncAttributeMaxDynamicSharedMemorySize, 158 * 1024);
         attr_set = true;
     }
-    dim3 grid((out_f + kRowsPerBlock - 1) / kRowsPerBlock, p.rows * p.n_used), block(256);
+    // output rows of a block (kRB in the kernel): 16, or 8 for gate/up when that still leaves the compute units short
+    // of two blocks each (one round per block instead of two serial ones; C2 shape, one row: 11.5 -> 10.1 us)
+    const int blocks16 = ((out_f + kRowsPerBlock - 1) / kRowsPerBlock) * p.rows * p.n_used;
+    const int rb = GATE_UP && blocks16 < 512 ? 8 : kRowsPerBlock;
+    dim3 grid((out_f + rb - 1) / rb, p.rows * p.n_used), block(256);
     const size_t route_lds = GATE_UP && p.route_inline ? route_scratch_floats(p.route.n_expert, p.route.n_groups) * sizeof(float) : 0;
     INFR_LAUNCH((moe_units_kernel<DT, GATE_UP>), grid, block, (size_t)(in_f >> 5) * (kUnitStride + 2) * sizeof(float) + route_lds,
-                s, p, row_bytes);
+                s, p, row_bytes, rb);
 }
 
 template <bool GATE_UP>
