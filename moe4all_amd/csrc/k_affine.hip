@@ -28,7 +28,7 @@ constexpr int kRowsPerBlock = 16; // 4 waves x 2 rows x 2 rounds
 template <int DT, int T>
 __global__ __launch_bounds__(256) void linear_units_kernel(const float* __restrict__ x, const uint8_t* __restrict__ w,
                                                            size_t row_bytes, int m, int in_f, int out_f, float* dst,
-                                                           const float* addend) {
+                                                           const float* addend, int rows_per_block) {
     extern __shared__ float lds[];
     const int n_units = in_f >> 5;
     float* xs = lds;                                   // [T][n_units][kUnitStride]
@@ -52,8 +52,8 @@ __global__ __launch_bounds__(256) void linear_units_kernel(const float* __restri
         xsum[idx] = s;
     }
     __syncthreads();
-    const int row_base = blockIdx.x * kRowsPerBlock;
-    for (int round = 0; round < kRowsPerBlock / (4 * kRowsPerWave); round++) {
+    const int row_base = blockIdx.x * rows_per_block;
+    for (int round = 0; round < rows_per_block / (4 * kRowsPerWave); round++) {
         const int o0 = row_base + (round * 4 + wave) * kRowsPerWave;
         if (o0 >= out_f) break;
         float acc[kRowsPerWave][T];
@@ -598,8 +598,11 @@ void launch_units(hipStream_t s, const float* x, const uint8_t* w, size_t row_by
         (void)hipFuncSetAttribute((const void*)linear_units_kernel<DT, T>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         attr_set = true;
     }
-    dim3 grid((out_f + kRowsPerBlock - 1) / kRowsPerBlock, (m + T - 1) / T), block(256);
-    INFR_LAUNCH((linear_units_kernel<DT, T>), grid, block, lds, s, x, w, row_bytes, m, in_f, out_f, dst, addend);
+    // 16 output rows per block, or 8 (one round instead of two serial ones) while the grid would be small
+    const int gy = (m + T - 1) / T;
+    const int rb = ((out_f + kRowsPerBlock - 1) / kRowsPerBlock) * gy < 512 ? 8 : kRowsPerBlock;
+    dim3 grid((out_f + rb - 1) / rb, gy), block(256);
+    INFR_LAUNCH((linear_units_kernel<DT, T>), grid, block, lds, s, x, w, row_bytes, m, in_f, out_f, dst, addend, rb);
 }
 
 template <int DT>
