@@ -207,7 +207,12 @@ typedef struct infr_hip_config {
      * kernel.  The escape hatch the reference's backends keep for their rewrites
      * (crates/infr-core/src/fusion.rs:49-52, `enabled`); results are bit-identical either way. */
     uint32_t disable_op_fusion;
-    uint32_t reserved[5];
+    /* Non-zero: the single-token gate/up kernel computes the reference's routing before it requests any
+     * expert row.  0 (default): it starts from the top n_used experts by logit, checks that pick against
+     * the exact routing while the rows are in flight and runs again on a mismatch.  Same bits either
+     * way; the switch exists to compare the two. */
+    uint32_t moe_route_exact_first;
+    uint32_t reserved[4];
 } infr_hip_config;
 
 /* Construction of the backend object (reference: VulkanBackend::new / CpuBackend::new,

@@ -1342,6 +1342,7 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                     Timed t(be, "route_topk");
                     infr::launch_route(s, rp);
                 }
+                gp.route_exact_first = be->cfg.moe_route_exact_first ? 1 : 0;
                 {
                     Timed t(be, gp.sh_gate ? "moe_route_gate_up_shared" : units ? (gp.route_inline ? "moe_route_gate_up_units" : "moe_gate_up_units")
                                 : gp.route_inline ? "moe_route_gate_up" : "moe_gate_up");

@@ -23,382 +23,9 @@
 #include "device_common.h"
 #include "kernels.h"
 #include "route.h"
+#include "gemv_fmt.h"
 
 namespace infr {
-
-__device__ __forceinline__ int dot4i(uint32_t a, uint32_t b, int c) {
-    return __builtin_amdgcn_sdot4((int)a, (int)b, c, false);
-}
-
-// ---- activation staging -------------------------------------------------------------------
-// A wavefront converts the activation vector once, cooperatively, into LDS "cells" of 32
-// elements (28 dwords: byte planes A, B, C of the fixed-point values, then scales and sums),
-// and each lane then fetches the cells of its own K slice.  Element 4k+q of a group sits in
-// byte q of dword k of each plane, the order in which byte-parallel unpacking yields codes.
-//   G == 32: [A 8][B 8][C 8][scale][sum][pad 2]            one group of 32
-//   G == 16: [A0 4][B0 4][C0 4][A1 4][B1 4][C1 4][k0][s0][k1][s1]   two groups of 16
-// SIGNED digits (X = 65536*A + 256*B + C with every digit in [-128,127]) serve signed weight
-// codes; otherwise B and C are the plain unsigned bytes of X's two's complement (A signed),
-// which costs no arithmetic to extract and pairs with the unsigned dot for non-negative codes.
-constexpr int kCellDwords = 28;
-
-__device__ __forceinline__ uint32_t perm(uint32_t hi, uint32_t lo, uint32_t sel) {
-    return __builtin_amdgcn_perm(hi, lo, sel);
-}
-
-// Byte `B` of four dwords -> one dword (x0's byte in byte 0).
-template <int B>
-__device__ __forceinline__ uint32_t gather_byte(uint32_t x0, uint32_t x1, uint32_t x2, uint32_t x3) {
-    // v_perm_b32 selects bytes from {hi,lo}: selector values 0-3 = lo bytes, 4-7 = hi bytes
-    const uint32_t lo = perm(x1, x0, (uint32_t)(B | ((4 + B) << 8)));          // [x0.B, x1.B, -, -]
-    const uint32_t hi = perm(x3, x2, (uint32_t)(B | ((4 + B) << 8)));          // [x2.B, x3.B, -, -]
-    return perm(hi, lo, 0x05040100u);                                          // [lo.0, lo.1, hi.0, hi.1]
-}
-
-template <int N, bool SIGNED>
-__device__ __forceinline__ void quant_to_cell(const float* x, uint32_t* a, uint32_t* b, uint32_t* c, uint32_t* ks) {
-    float amax = 0.f;
-#pragma unroll
-    for (int i = 0; i < N; i++) amax = fmaxf(amax, fabsf(x[i]));
-    const uint32_t eb = (__float_as_uint(amax) >> 23) & 0xFFu;  // amax in [2^(eb-127), 2^(eb-126))
-    const bool live = eb >= 22u && eb < 255u;
-    const float inv = live ? __uint_as_float((274u - eb) << 23) : 0.f;  // 2^(20 - E): |x| * inv < 2^21
-    const float scale = live ? __uint_as_float((eb - 20u) << 23) : 0.f; // 2^(E - 20)
-    int sx = 0;
-#pragma unroll
-    for (int k = 0; k < N / 4; k++) {
-        int X[4];
-#pragma unroll
-        for (int q = 0; q < 4; q++) {
-            X[q] = __float2int_rn(x[4 * k + q] * inv);  // exact scaling, |X| <= 2^21
-            sx += X[q];
-        }
-        if (SIGNED) {
-            uint32_t aw = 0, bw = 0, cw = 0;
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-                const int C = (int)(int8_t)(X[q] & 0xFF);
-                const int R = (X[q] - C) >> 8;
-                const int B = (int)(int8_t)(R & 0xFF);
-                const int A = (R - B) >> 8;
-                aw |= (uint32_t)(A & 0xFF) << (8 * q);
-                bw |= (uint32_t)(B & 0xFF) << (8 * q);
-                cw |= (uint32_t)(C & 0xFF) << (8 * q);
-            }
-            a[k] = aw; b[k] = bw; c[k] = cw;
-        } else {
-            a[k] = gather_byte<2>((uint32_t)X[0], (uint32_t)X[1], (uint32_t)X[2], (uint32_t)X[3]);
-            b[k] = gather_byte<1>((uint32_t)X[0], (uint32_t)X[1], (uint32_t)X[2], (uint32_t)X[3]);
-            c[k] = gather_byte<0>((uint32_t)X[0], (uint32_t)X[1], (uint32_t)X[2], (uint32_t)X[3]);
-        }
-    }
-    ks[0] = __float_as_uint(scale);
-    ks[1] = __float_as_uint((float)sx * scale);  // sum(x~); |sx| <= 2^26 rounds at 2^-24 like any f32 sum
-}
-
-// Lane L of the wave converts elements [32L, 32L+32) of x[0..n) (n <= 2048 per pass).  The
-// global loads are split from the conversion so a kernel can request x early and convert it
-// while later loads are in flight.
-struct XLoad { float t[32]; };
-__device__ __forceinline__ XLoad stage_x_load(const float* __restrict__ x, int n, int c0) {
-    XLoad l;
-    const float4* src = reinterpret_cast<const float4*>(x + (size_t)(c0 * 32 < n ? c0 : 0) * 32);
-#pragma unroll
-    for (int k = 0; k < 8; k++) {
-        float4 v = src[k];
-        l.t[4 * k] = v.x; l.t[4 * k + 1] = v.y; l.t[4 * k + 2] = v.z; l.t[4 * k + 3] = v.w;
-    }
-    return l;
-}
-template <int G, bool SIGNED>
-__device__ __forceinline__ void stage_x_convert(const XLoad& l, int n, int c0, uint32_t* cells) {
-    if (c0 * 32 >= n) return;
-    uint32_t cell[kCellDwords];
-    if (G == 32) {
-        quant_to_cell<32, SIGNED>(l.t, cell, cell + 8, cell + 16, cell + 24);
-        cell[26] = cell[27] = 0;
-    } else {
-        quant_to_cell<16, SIGNED>(l.t, cell, cell + 4, cell + 8, cell + 24);
-        quant_to_cell<16, SIGNED>(l.t + 16, cell + 12, cell + 16, cell + 20, cell + 26);
-    }
-    uint4* dst = reinterpret_cast<uint4*>(cells + (size_t)c0 * kCellDwords);
-#pragma unroll
-    for (int k = 0; k < 7; k++) dst[k] = make_uint4(cell[4 * k], cell[4 * k + 1], cell[4 * k + 2], cell[4 * k + 3]);
-}
-// Whole vector, any n: first pass from an early load, further passes loaded here.
-template <int G, bool SIGNED>
-__device__ __forceinline__ void stage_x_finish(const XLoad& first, const float* __restrict__ x, int n, uint32_t* cells,
-                                               int lane) {
-    stage_x_convert<G, SIGNED>(first, n, lane, cells);
-    for (int c0 = lane + kWave; c0 * 32 < n; c0 += kWave) {
-        XLoad l = stage_x_load(x, n, c0);
-        stage_x_convert<G, SIGNED>(l, n, c0, cells);
-    }
-}
-
-__device__ __forceinline__ void fetch_dwords(uint32_t* dst, const uint32_t* src, int n4) {
-    const uint4* s4 = reinterpret_cast<const uint4*>(src);
-    for (int k = 0; k < n4; k++) {
-        uint4 v = s4[k];
-        dst[4 * k] = v.x; dst[4 * k + 1] = v.y; dst[4 * k + 2] = v.z; dst[4 * k + 3] = v.w;
-    }
-}
-
-__device__ __forceinline__ int udot4i(uint32_t a, uint32_t b, int c) {
-    return (int)__builtin_amdgcn_udot4(a, b, (uint32_t)c, false);
-}
-
-// sum(q * X) from the three exact byte-plane sums, rounded once or twice at 2^-24.
-__device__ __forceinline__ float join3(int sa, int sb, int sc) {
-    return fmaf((float)sa, 65536.0f, fmaf((float)sb, 256.0f, (float)sc));
-}
-
-__device__ __forceinline__ void load16(float* dst, const float* src) {
-    const float4* s = reinterpret_cast<const float4*>(src);
-#pragma unroll
-    for (int k = 0; k < 4; k++) {
-        float4 v = s[k];
-        dst[4 * k + 0] = v.x; dst[4 * k + 1] = v.y; dst[4 * k + 2] = v.z; dst[4 * k + 3] = v.w;
-    }
-}
-
-// ------------------------------------------------------------------------------- Q4_K
-// 144 B: [f16 d][f16 dmin][12 B 6-bit scales/mins][128 B nibbles].  4 lanes per block; lane j
-// owns nibble bytes [32j, 32j+32): low nibbles are elements j*64+t (sub-block 2j), high
-// nibbles j*64+32+t (sub-block 2j+1), t < 32.
-struct Q4KFmt {
-    static constexpr int kBlockBytes = 144, kBlockElems = 256, kLPB = 4;
-    static constexpr int kGroup = 32;
-    static constexpr bool kSigned = false;
-    struct X { uint32_t alo[8], blo[8], clo[8], ahi[8], bhi[8], chi[8]; float klo, khi, slo, shi; };
-    struct Raw { uint4 hdr, qa, qb; };
-    // lane j of block blk: cells 8*blk + 2j (low nibbles) and + 1 (high nibbles)
-    static __device__ __forceinline__ void fetch_x(X& x, const uint32_t* cells, int blk, int j) {
-        const uint32_t* lo = cells + (size_t)(8 * blk + 2 * j) * kCellDwords;
-        const uint32_t* hi = lo + kCellDwords;
-        uint32_t t[28];
-#pragma unroll
-        for (int k = 0; k < 7; k++) {
-            uint4 v = reinterpret_cast<const uint4*>(lo)[k];
-            t[4 * k] = v.x; t[4 * k + 1] = v.y; t[4 * k + 2] = v.z; t[4 * k + 3] = v.w;
-        }
-#pragma unroll
-        for (int k = 0; k < 8; k++) { x.alo[k] = t[k]; x.blo[k] = t[8 + k]; x.clo[k] = t[16 + k]; }
-        x.klo = __uint_as_float(t[24]); x.slo = __uint_as_float(t[25]);
-#pragma unroll
-        for (int k = 0; k < 7; k++) {
-            uint4 v = reinterpret_cast<const uint4*>(hi)[k];
-            t[4 * k] = v.x; t[4 * k + 1] = v.y; t[4 * k + 2] = v.z; t[4 * k + 3] = v.w;
-        }
-#pragma unroll
-        for (int k = 0; k < 8; k++) { x.ahi[k] = t[k]; x.bhi[k] = t[8 + k]; x.chi[k] = t[16 + k]; }
-        x.khi = __uint_as_float(t[24]); x.shi = __uint_as_float(t[25]);
-    }
-    static __device__ __forceinline__ Raw load(const uint8_t* blk, int j) {
-        Raw r;
-        r.hdr = *reinterpret_cast<const uint4*>(blk);
-        r.qa = *reinterpret_cast<const uint4*>(blk + 16 + 32 * j);
-        r.qb = *reinterpret_cast<const uint4*>(blk + 32 + 32 * j);
-        return r;
-    }
-    static __device__ __forceinline__ float dot(const Raw& r, int j, const X& x) {
-        const float d = f16_bits_to_f32(r.hdr.x & 0xFFFFu);
-        const float dmin = f16_bits_to_f32(r.hdr.x >> 16);
-        // 6-bit (scale, min) of sub-blocks 2j and 2j+1, as adjacent bytes (get_scale_min_k4)
-        const uint32_t sh = (uint32_t)(j & 1) * 16u;
-        const uint32_t y = r.hdr.y >> sh, z = r.hdr.z >> sh, w = r.hdr.w >> sh;
-        uint32_t sc, m;
-        if (j < 2) {
-            sc = y & 0x3F3Fu;
-            m = z & 0x3F3Fu;
-        } else {
-            sc = (w & 0x0F0Fu) | ((y >> 2) & 0x3030u);
-            m = ((w >> 4) & 0x0F0Fu) | ((z >> 2) & 0x3030u);
-        }
-        const uint32_t q[8] = {r.qa.x, r.qa.y, r.qa.z, r.qa.w, r.qb.x, r.qb.y, r.qb.z, r.qb.w};
-        int la = 0, lb = 0, lc = 0, ha = 0, hb = 0, hc = 0;
-#pragma unroll
-        for (int k = 0; k < 8; k++) {
-            const uint32_t lo = q[k] & 0x0F0F0F0Fu, hi = (q[k] >> 4) & 0x0F0F0F0Fu;
-            la = dot4i(lo, x.alo[k], la);   // A signed; B, C plain unsigned bytes; codes are 0..15
-            lb = udot4i(lo, x.blo[k], lb);
-            lc = udot4i(lo, x.clo[k], lc);
-            ha = dot4i(hi, x.ahi[k], ha);
-            hb = udot4i(hi, x.bhi[k], hb);
-            hc = udot4i(hi, x.chi[k], hc);
-        }
-        const float flo = join3(la, lb, lc) * x.klo;
-        const float fhi = join3(ha, hb, hc) * x.khi;
-        const float s0 = d * (float)(sc & 0xFFu), s1 = d * (float)(sc >> 8);
-        const float m0 = dmin * (float)(m & 0xFFu), m1 = dmin * (float)(m >> 8);
-        return (s0 * flo - m0 * x.slo) + (s1 * fhi - m1 * x.shi);
-    }
-};
-
-// ------------------------------------------------------------------------------- Q6_K
-// 210 B: [128 B ql][64 B qh][16 x i8 scales][f16 d].  4 lanes per block; lane i owns, in half
-// h = i/2 at l0 = 16*(i&1), the bytes ql[h*64+l0 ..+16), ql[h*64+32+l0 ..+16) and
-// qh[h*32+l0 ..+16): 64 elements in four 16-element scale groups g = 0..3 at
-// h*128 + g*32 + l0 (scale byte h*8 + 2g + (i&1)).  Blocks are only 2-byte aligned.
-struct Q6KFmt {
-    static constexpr int kBlockBytes = 210, kBlockElems = 256, kLPB = 4;
-    static constexpr int kGroup = 16;
-    static constexpr bool kSigned = false;
-    struct X { uint32_t a[4][4], b[4][4], c[4][4]; float k[4], s32[4]; };
-    struct Raw { uint4 qla, qlb, qh; uint2 sc; uint32_t d; };
-    // lane i of block blk: 16-groups 16*blk + 8h + 2g + (i&1), g = 0..3; a cell holds two
-    static __device__ __forceinline__ void fetch_x(X& x, const uint32_t* cells, int blk, int i) {
-        const int h = i >> 1, odd = i & 1;
-#pragma unroll
-        for (int g = 0; g < 4; g++) {
-            const int t = 16 * blk + 8 * h + 2 * g + odd;
-            const uint32_t* cell = cells + (size_t)(t >> 1) * kCellDwords;
-            const uint32_t* pl = cell + (t & 1) * 12;
-#pragma unroll
-            for (int q = 0; q < 3; q++) {
-                uint4 v = reinterpret_cast<const uint4*>(pl)[q];
-                uint32_t* dst = q == 0 ? x.a[g] : q == 1 ? x.b[g] : x.c[g];
-                dst[0] = v.x; dst[1] = v.y; dst[2] = v.z; dst[3] = v.w;
-            }
-            const uint2 ks = *reinterpret_cast<const uint2*>(cell + 24 + 2 * (t & 1));
-            x.k[g] = __uint_as_float(ks.x);
-            x.s32[g] = 32.0f * __uint_as_float(ks.y);
-        }
-    }
-    static __device__ __forceinline__ Raw load(const uint8_t* blk, int i) {
-        const int h = i >> 1, l0 = (i & 1) * 16;
-        Raw r;
-        r.qla = ldu<uint4>(blk + h * 64 + l0);
-        r.qlb = ldu<uint4>(blk + h * 64 + 32 + l0);
-        r.qh = ldu<uint4>(blk + 128 + h * 32 + l0);
-        r.sc = ldu<uint2>(blk + 192 + h * 8);
-        r.d = ldu<uint16_t>(blk + 208);
-        return r;
-    }
-    static __device__ __forceinline__ float dot(const Raw& r, int i, const X& x) {
-        const uint32_t a[4] = {r.qla.x, r.qla.y, r.qla.z, r.qla.w};
-        const uint32_t b[4] = {r.qlb.x, r.qlb.y, r.qlb.z, r.qlb.w};
-        const uint32_t hq[4] = {r.qh.x, r.qh.y, r.qh.z, r.qh.w};
-        int sa[4] = {0, 0, 0, 0}, sb[4] = {0, 0, 0, 0}, sc[4] = {0, 0, 0, 0};
-#pragma unroll
-        for (int k = 0; k < 4; k++) {
-            uint32_t q[4];
-            q[0] = (a[k] & 0x0F0F0F0Fu) | ((hq[k] << 4) & 0x30303030u);
-            q[1] = (b[k] & 0x0F0F0F0Fu) | ((hq[k] << 2) & 0x30303030u);
-            q[2] = ((a[k] >> 4) & 0x0F0F0F0Fu) | (hq[k] & 0x30303030u);
-            q[3] = ((b[k] >> 4) & 0x0F0F0F0Fu) | ((hq[k] >> 2) & 0x30303030u);
-#pragma unroll
-            for (int g = 0; g < 4; g++) {
-                sa[g] = dot4i(q[g], x.a[g][k], sa[g]);   // codes are 0..63
-                sb[g] = udot4i(q[g], x.b[g][k], sb[g]);
-                sc[g] = udot4i(q[g], x.c[g][k], sc[g]);
-            }
-        }
-        const float d = f16_bits_to_f32(r.d);
-        const uint32_t sx = (i & 1) ? (r.sc.x >> 8) : r.sc.x;
-        const uint32_t sy = (i & 1) ? (r.sc.y >> 8) : r.sc.y;
-        const float s[4] = {(float)(int)(int8_t)(sx & 0xFFu), (float)(int)(int8_t)((sx >> 16) & 0xFFu),
-                            (float)(int)(int8_t)(sy & 0xFFu), (float)(int)(int8_t)((sy >> 16) & 0xFFu)};
-        float acc = 0.f;
-#pragma unroll
-        for (int g = 0; g < 4; g++) {
-            const float f = join3(sa[g], sb[g], sc[g]) * x.k[g];  // sum(q*x~)
-            acc += (d * s[g]) * (f - x.s32[g]);                    // d*s*sum((q-32)*x~)
-        }
-        return acc;
-    }
-};
-
-// ------------------------------------------------------------------------------- Q8_0
-// 34 B: [f16 d][32 x i8].  One lane per block; the signed codes contract directly.
-struct Q80Fmt {
-    static constexpr int kBlockBytes = 34, kBlockElems = 32, kLPB = 1;
-    static constexpr int kGroup = 32;
-    static constexpr bool kSigned = true;  // signed weight codes need signed digits throughout
-    struct X { uint32_t a[8], b[8], c[8]; float k; };
-    struct Raw { uint4 a, b; uint32_t d; };
-    static __device__ __forceinline__ void fetch_x(X& x, const uint32_t* cells, int blk, int) {
-        const uint32_t* cell = cells + (size_t)blk * kCellDwords;
-        uint32_t t[28];
-#pragma unroll
-        for (int k = 0; k < 7; k++) {
-            uint4 v = reinterpret_cast<const uint4*>(cell)[k];
-            t[4 * k] = v.x; t[4 * k + 1] = v.y; t[4 * k + 2] = v.z; t[4 * k + 3] = v.w;
-        }
-#pragma unroll
-        for (int k = 0; k < 8; k++) { x.a[k] = t[k]; x.b[k] = t[8 + k]; x.c[k] = t[16 + k]; }
-        x.k = __uint_as_float(t[24]);
-    }
-    static __device__ __forceinline__ Raw load(const uint8_t* blk, int) {
-        Raw r;
-        r.d = ldu<uint16_t>(blk);
-        r.a = ldu<uint4>(blk + 2);
-        r.b = ldu<uint4>(blk + 18);
-        return r;
-    }
-    static __device__ __forceinline__ float dot(const Raw& r, int, const X& x) {
-        const uint32_t q[8] = {r.a.x, r.a.y, r.a.z, r.a.w, r.b.x, r.b.y, r.b.z, r.b.w};
-        int sa = 0, sb = 0, sc = 0;
-#pragma unroll
-        for (int k = 0; k < 8; k++) {
-            sa = dot4i(q[k], x.a[k], sa);
-            sb = dot4i(q[k], x.b[k], sb);
-            sc = dot4i(q[k], x.c[k], sc);
-        }
-        const float f = join3(sa, sb, sc) * x.k;
-        return f16_bits_to_f32(r.d) * f;
-    }
-};
-
-// Lane placement of a wavefront over weight rows of nblk blocks: lanes_per_row = nblk*LPB
-// (<= 64), rows_per_wave = 64 / lanes_per_row.  Left-over lanes of the wave are pointed at the
-// last row and flagged off: they load and compute like everyone else, so the code stays
-// branch-free and every load of a round is issued back to back; their result is dropped.
-template <class F>
-struct Place {
-    int lpr, rw_count, rw, pos;  // lanes per row, rows per wave, my row (clamped), my lane in the row
-    bool row_on;
-    int blk, sub;                // my block in the row and my lane inside the block
-    int wpos;                    // lane-in-row where the row's sum lands
-    __device__ __forceinline__ Place(int nblk, int lane) {
-        lpr = nblk * F::kLPB;
-        rw_count = kWave / lpr;
-        const int rw_raw = lane / lpr;
-        pos = lane - rw_raw * lpr;
-        row_on = rw_raw < rw_count;
-        rw = row_on ? rw_raw : rw_count - 1;
-        blk = pos / F::kLPB;
-        sub = pos - blk * F::kLPB;
-        wpos = (lpr == 64 || lpr == 32 || lpr == 16) ? lpr - 1 : 0;
-    }
-    __device__ __forceinline__ bool writer() const { return row_on && pos == wpos; }
-};
-
-// LDS bytes one wave needs to stage an activation vector of n elements.
-static inline size_t cells_bytes(int n) { return (size_t)((n + 31) / 32) * kCellDwords * sizeof(uint32_t); }
-template <class F>
-__device__ __forceinline__ typename F::Raw load_row(const Place<F>& pl, const uint8_t* row) {
-    return F::load(row + (size_t)pl.blk * F::kBlockBytes, pl.sub);
-}
-
-// Sum of v over the lanes of each weight row; valid in the row's writer lane.
-template <class F>
-__device__ __forceinline__ float row_sum(float v, const Place<F>& pl, int nblk) {
-    if (pl.lpr >= 16 && (pl.lpr & (pl.lpr - 1)) == 0) {
-        v = row16_sum(v);                                            // every lane: sum of its 16
-        if (pl.lpr >= 32) v += dpp_rows_f<0x142, 0xA>(v);            // rows 1,3 += lane 15 of rows 0,2
-        if (pl.lpr == 64) v += dpp_rows_f<0x143, 0xC>(v);            // rows 2,3 += lane 31
-        return v;
-    }
-    // lanes of one block first (rows start at multiples of kLPB lanes, so DPP groups line up) ...
-    if (F::kLPB == 4) v = quad_sum(v);
-    // ... then the row's blocks, by doubling; the total lands in the row's first lane
-    for (int ob = 1; ob < nblk; ob <<= 1) {
-        float t = __shfl_down(v, ob * F::kLPB, kWave);
-        if (pl.blk + ob < nblk) v += t;
-    }
-    return v;
-}
 
 // ------------------------------------------------------------------------------- gate/up
 // grid.x = tiles of `ft` features, grid.y = token row.  A block's 4 waves share the items
@@ -468,88 +95,122 @@ __device__ __forceinline__ void gu_finish(const GuStage<F, U>& st, const MoeGemv
 // then all of the block's loads are in flight at once).  PIPE == true, for tiles of three or more
 // stages: two stage buffers, the next stage's loads are issued before the current stage is
 // finished, so a wave always has a stage in flight while it computes.
-template <class F, int U, bool PIPE>
-__global__ __launch_bounds__(256) void moe_gate_up_fast(MoeGemvParams p, int ft) {
+// When the kernel routes its token row itself (p.route_inline) the block has a fifth wavefront that does
+// nothing else.  spec != 0: it publishes the top n_used by logit at once, so the four workers can request
+// their expert rows, and runs the reference's routing while those bytes are in flight; the pick is checked
+// against the exact probabilities and, if any rank differs, the workers run again with the exact ids
+// (gate_up_router in route.h).  The expert ids are all this kernel needs of the routing; the routing weights
+// are first used by the down kernel (and here with weight_before, which therefore routes exactly first).
+// ROUTER instances have the five wavefronts (two of them share a SIMD and its registers, so they keep fewer
+// rows in flight per wave); the others are the plain four-wave kernel for ids that are given.
+constexpr int kGuRouterWave = 4;
+template <class F, int U, bool PIPE, bool ROUTER>
+__global__ __launch_bounds__(ROUTER ? 320 : 256) void moe_gate_up_fast(MoeGemvParams p, int ft, int spec) {
     extern __shared__ uint32_t dyn_lds[];
     __shared__ uint64_t s_tab[32];
-    __shared__ int32_t s_ids[64];
+    __shared__ int32_t s_ids[64], s_early[64];
     __shared__ float s_w[64];
+    __shared__ int s_redo;
     __shared__ float s_g[4][64], s_u[4][64];
     GuTile t;
     t.r = blockIdx.y;
     t.f0 = blockIdx.x * ft;
     t.fcount = min(ft, p.nff - t.f0);
-    t.wave = threadIdx.x >> 6;
+    t.wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     t.lane = threadIdx.x & 63;
     const int r = t.r, wave = t.wave, lane = t.lane;
     const int nblk = p.ne / F::kBlockElems;
     t.row_bytes = (size_t)nblk * F::kBlockBytes;
     const Place<F> pl(nblk, lane);
     const size_t cell_words = (size_t)((p.ne + 31) / 32) * kCellDwords;
-    uint32_t* cells = dyn_lds + (size_t)wave * cell_words;
-    // x is requested first; it does not depend on the routing
-    const float* xrow = p.x + (size_t)r * p.ne;
-    const XLoad xl = stage_x_load(xrow, p.ne, lane);
-    if (threadIdx.x < 32) s_tab[threadIdx.x] = kExp2Table[threadIdx.x];
-    if (p.route_inline) {
-        // every block routes its token row itself (one wave, redundantly across blocks)
-        __syncthreads();
-        if (wave == 0)
-            route_row_any(p.route, r, lane, reinterpret_cast<float*>(dyn_lds + 4 * cell_words), s_tab, s_ids, s_w,
-                          blockIdx.x == 0);
-    } else if ((int)threadIdx.x < p.n_used) {  // n_used <= 64
-        s_ids[threadIdx.x] = p.ids[(size_t)r * p.n_used + threadIdx.x];
-        s_w[threadIdx.x] = p.weights[(size_t)r * p.n_used + threadIdx.x];
-    }
+    uint32_t* cells = dyn_lds + (size_t)min(wave, 3) * cell_words;
     t.n_slots = p.n_used + (p.sh_gate ? 1 : 0);   // the always-on expert is slot n_used (<= 63 then)
-    if (p.sh_gate && threadIdx.x == 255) {
-        s_ids[p.n_used] = 0;
-        s_w[p.n_used] = 1.0f;
+    const float* xrow = p.x + (size_t)r * p.ne;
+    XLoad xl;
+    if (ROUTER && wave == kGuRouterWave) {
+        float* lds_prob = reinterpret_cast<float*>(dyn_lds + 4 * cell_words);
+        const int n = p.route.n_expert, n_pad = n <= 128 ? 128 : 256;
+        if (n <= 128) gate_up_router<2>(p.route, r, lane, spec != 0, lds_prob, lds_prob + n_pad, s_tab, s_ids, s_early, s_w, &s_redo, blockIdx.x == 0);
+        else if (n <= 256) gate_up_router<4>(p.route, r, lane, spec != 0, lds_prob, lds_prob + n_pad, s_tab, s_ids, s_early, s_w, &s_redo, blockIdx.x == 0);
+        else {
+            if (lane < 32) s_tab[lane] = kExp2Table[lane];
+            __builtin_amdgcn_wave_barrier();
+            route_row_large(p.route, r, lane, lds_prob, s_tab, s_ids, s_w, blockIdx.x == 0);
+            __builtin_amdgcn_wave_barrier();
+            if (lane < p.n_used) s_early[lane] = s_ids[lane];
+            __syncthreads();   // (1)
+        }
+    } else {
+        // x is requested first; it does not depend on the routing
+        xl = stage_x_load(xrow, p.ne, lane);
+        if (!ROUTER) {
+            if (threadIdx.x < 32) s_tab[threadIdx.x] = kExp2Table[threadIdx.x];
+            if ((int)threadIdx.x < p.n_used) {  // n_used <= 64
+                s_ids[threadIdx.x] = s_early[threadIdx.x] = p.ids[(size_t)r * p.n_used + threadIdx.x];
+                s_w[threadIdx.x] = p.weights[(size_t)r * p.n_used + threadIdx.x];
+            }
+        }
+        if (p.sh_gate && threadIdx.x == 255) {
+            s_ids[p.n_used] = s_early[p.n_used] = 0;
+            s_w[p.n_used] = 1.0f;
+        }
+        if (threadIdx.x == 0) s_redo = 0;
+        __syncthreads();   // (1) the ids to start from are in LDS
     }
-    __syncthreads();
-    __builtin_amdgcn_wave_barrier();
     t.nitems = t.fcount * t.n_slots;
     const int step = 4 * pl.rw_count * U;
     typename F::X x;
-    if (!PIPE) {
-        bool have_x = false;
-        for (int base = 0; base < t.nitems; base += step) {
-            GuStage<F, U> st;
-            gu_issue<F, U>(st, p, pl, t, s_ids, base);
-            if (!have_x) {
-                // while the weights are in flight: the wave converts x to fixed point once, together
-                stage_x_finish<F::kGroup, F::kSigned>(xl, xrow, p.ne, cells, lane);
-                __builtin_amdgcn_wave_barrier();
-                F::fetch_x(x, cells, pl.blk, pl.sub);
-                have_x = true;
+    bool have_x = false;
+#pragma nounroll
+    for (int attempt = 0; attempt < 2; attempt++) {
+        const int32_t* ids = attempt == 0 ? s_early : s_ids;
+        if (!ROUTER || wave != kGuRouterWave) {
+            if (!PIPE) {
+                for (int base = 0; base < t.nitems; base += step) {
+                    GuStage<F, U> st;
+                    gu_issue<F, U>(st, p, pl, t, ids, base);
+                    if (!have_x) {
+                        // while the weights are in flight: the wave converts x to fixed point once, together
+                        stage_x_finish<F::kGroup, F::kSigned>(xl, xrow, p.ne, cells, lane);
+                        __builtin_amdgcn_wave_barrier();
+                        F::fetch_x(x, cells, pl.blk, pl.sub);
+                        have_x = true;
+                    }
+                    gu_finish<F, U>(st, p, pl, t, x, nblk, base, s_g, s_u, s_w, s_tab);
+                }
+            } else {
+                GuStage<F, U> sa, sb;
+                gu_issue<F, U>(sa, p, pl, t, ids, 0);
+                gu_issue<F, U>(sb, p, pl, t, ids, step);
+                if (!have_x) {
+                    stage_x_finish<F::kGroup, F::kSigned>(xl, xrow, p.ne, cells, lane);
+                    __builtin_amdgcn_wave_barrier();
+                    F::fetch_x(x, cells, pl.blk, pl.sub);
+                    have_x = true;
+                }
+                gu_finish<F, U>(sa, p, pl, t, x, nblk, 0, s_g, s_u, s_w, s_tab);
+                int base = step;   // the stage sb holds
+                for (;;) {
+                    if (base + step >= t.nitems) {
+                        gu_finish<F, U>(sb, p, pl, t, x, nblk, base, s_g, s_u, s_w, s_tab);
+                        break;
+                    }
+                    gu_issue<F, U>(sa, p, pl, t, ids, base + step);
+                    gu_finish<F, U>(sb, p, pl, t, x, nblk, base, s_g, s_u, s_w, s_tab);
+                    base += step;
+                    if (base + step >= t.nitems) {
+                        gu_finish<F, U>(sa, p, pl, t, x, nblk, base, s_g, s_u, s_w, s_tab);
+                        break;
+                    }
+                    gu_issue<F, U>(sb, p, pl, t, ids, base + step);
+                    gu_finish<F, U>(sa, p, pl, t, x, nblk, base, s_g, s_u, s_w, s_tab);
+                    base += step;
+                }
             }
-            gu_finish<F, U>(st, p, pl, t, x, nblk, base, s_g, s_u, s_w, s_tab);
         }
-    } else {
-        GuStage<F, U> sa, sb;
-        gu_issue<F, U>(sa, p, pl, t, s_ids, 0);
-        gu_issue<F, U>(sb, p, pl, t, s_ids, step);
-        stage_x_finish<F::kGroup, F::kSigned>(xl, xrow, p.ne, cells, lane);
-        __builtin_amdgcn_wave_barrier();
-        F::fetch_x(x, cells, pl.blk, pl.sub);
-        gu_finish<F, U>(sa, p, pl, t, x, nblk, 0, s_g, s_u, s_w, s_tab);
-        int base = step;   // the stage sb holds
-        for (;;) {
-            if (base + step >= t.nitems) {
-                gu_finish<F, U>(sb, p, pl, t, x, nblk, base, s_g, s_u, s_w, s_tab);
-                break;
-            }
-            gu_issue<F, U>(sa, p, pl, t, s_ids, base + step);
-            gu_finish<F, U>(sb, p, pl, t, x, nblk, base, s_g, s_u, s_w, s_tab);
-            base += step;
-            if (base + step >= t.nitems) {
-                gu_finish<F, U>(sa, p, pl, t, x, nblk, base, s_g, s_u, s_w, s_tab);
-                break;
-            }
-            gu_issue<F, U>(sb, p, pl, t, s_ids, base + step);
-            gu_finish<F, U>(sa, p, pl, t, x, nblk, base, s_g, s_u, s_w, s_tab);
-            base += step;
-        }
+        if (!spec || attempt == 1) break;   // spec is uniform over the grid
+        __syncthreads();   // (2) the exact routing is in LDS
+        if (!s_redo) break;
     }
 }
 
@@ -759,18 +420,35 @@ static bool try_gate_up(hipStream_t s, const MoeGemvParams& p) {
     const int per_wave = ceil_div(ft * n_slots, 4 * rw);
     // tiles of three or more stages stream with the next stage in flight
     const bool pipe = per_wave > 6 && 3 * rw <= 64;
-    dim3 grid(ceil_div(p.nff, ft), p.rows), block(256);
+    dim3 grid(ceil_div(p.nff, ft), p.rows);
     // U * rw results per wave must fit the 64-entry staging rows
     int u = per_wave < 1 ? 1 : per_wave;
     while (u * rw > 64) u--;
+    const int n_pad = p.route.n_expert <= 128 ? 128 : 256;
     const size_t lds = 4 * cells_bytes(p.ne) +
-                       (p.route_inline ? route_scratch_floats(p.route.n_expert, p.route.n_groups) * sizeof(float) : 0);
-    if (pipe) INFR_LAUNCH((moe_gate_up_fast<F, 3, true>), grid, block, lds, s, p, ft);
-    else if (u >= 6) INFR_LAUNCH((moe_gate_up_fast<F, 6, false>), grid, block, lds, s, p, ft);
-    else if (u == 5 || u == 4) INFR_LAUNCH((moe_gate_up_fast<F, 4, false>), grid, block, lds, s, p, ft);
-    else if (u == 3) INFR_LAUNCH((moe_gate_up_fast<F, 3, false>), grid, block, lds, s, p, ft);
-    else if (u == 2) INFR_LAUNCH((moe_gate_up_fast<F, 2, false>), grid, block, lds, s, p, ft);
-    else INFR_LAUNCH((moe_gate_up_fast<F, 1, false>), grid, block, lds, s, p, ft);
+                       (p.route_inline ? (route_scratch_floats(p.route.n_expert, p.route.n_groups) + n_pad) * sizeof(float) : 0);
+    // the top-k by logit is the selection of any monotone gating without a bias, groups, given ids or a band; the
+    // routing weights are not known before the exact routing, so weight_before routes exactly first
+    const int spec = p.route_inline && !p.route_exact_first && p.route.n_expert <= 256 && !p.route.exp_probs_b &&
+                     !(p.route.n_groups > 1 && p.route.n_groups_used > 0) && !p.route.expert_ids && p.route.ep_n == 0 &&
+                     !p.weight_before;
+    if (p.route_inline) {
+        // five wavefronts: at most four row pairs in flight per wave (two stages of two when streaming)
+        const dim3 block(320);
+        if (pipe || u > 4) INFR_LAUNCH((moe_gate_up_fast<F, 2, true, true>), grid, block, lds, s, p, ft, spec);
+        else if (u == 4) INFR_LAUNCH((moe_gate_up_fast<F, 4, false, true>), grid, block, lds, s, p, ft, spec);
+        else if (u == 3) INFR_LAUNCH((moe_gate_up_fast<F, 3, false, true>), grid, block, lds, s, p, ft, spec);
+        else if (u == 2) INFR_LAUNCH((moe_gate_up_fast<F, 2, false, true>), grid, block, lds, s, p, ft, spec);
+        else INFR_LAUNCH((moe_gate_up_fast<F, 1, false, true>), grid, block, lds, s, p, ft, spec);
+        return true;
+    }
+    const dim3 block(256);
+    if (pipe) INFR_LAUNCH((moe_gate_up_fast<F, 3, true, false>), grid, block, lds, s, p, ft, 0);
+    else if (u >= 6) INFR_LAUNCH((moe_gate_up_fast<F, 6, false, false>), grid, block, lds, s, p, ft, 0);
+    else if (u == 5 || u == 4) INFR_LAUNCH((moe_gate_up_fast<F, 4, false, false>), grid, block, lds, s, p, ft, 0);
+    else if (u == 3) INFR_LAUNCH((moe_gate_up_fast<F, 3, false, false>), grid, block, lds, s, p, ft, 0);
+    else if (u == 2) INFR_LAUNCH((moe_gate_up_fast<F, 2, false, false>), grid, block, lds, s, p, ft, 0);
+    else INFR_LAUNCH((moe_gate_up_fast<F, 1, false, false>), grid, block, lds, s, p, ft, 0);
     return true;
 }
 

@@ -88,6 +88,9 @@ struct MoeGemvParams {
     // When set, the gate/up kernel routes each token row itself from route.logits (every block
     // redundantly; block 0 of a row publishes ids / weights / probs) and no route launch is needed.
     int route_inline;
+    // route_inline only: 1 = route exactly before any expert row is requested; 0 = the kernel may start from the
+    // top n_used by logit and check that pick against the exact routing while the rows are in flight
+    int route_exact_first;
     RouteParams route;
     // bucketed decode batches (launch_moe_*_bucketed): pairs grouped by expert
     const int32_t* bk_offsets;   // [n_expert + 1]
