@@ -287,6 +287,30 @@ infr_status infr_hip_plan_moe_bucketing(infr_hip_backend *be, const infr_hip_pla
  * `numel` elements of `src` interpreted as `dtype`. */
 infr_status infr_hip_dequant(infr_hip_backend *be, const infr_hip_buffer *src, int32_t dtype, uint64_t numel, infr_hip_buffer *dst);
 
+/* One Op::MoeFfn WITHOUT ANY ALLOCATION.  This entry point has no counterpart in the reference; it is for callers
+ * that cannot allocate device memory: code under HIP-graph capture, tight serving loops, harnesses that forbid it.
+ * It is infr_hip_compile + infr_hip_execute of a graph holding one MoeFfn in the plain qwen3moe parameterisation
+ * (softmax gating, renormalised weights, scale 1, SiLU, no option tensors, f32 router; 1 to 15 token rows), except
+ * that the routing results and the rows between the two expert stages live in a static device array of
+ * INFR_HIP_STATIC_SCRATCH_BYTES per GPU instead of a plan's arena; the output is the bits infr_hip_execute writes.
+ * Shapes that need more scratch return INFR_ERR_UNSUPPORTED (needed bytes = 2 * rows * n_expert * 4 +
+ * 2 * rows * n_used * 4 + rows * n_used * (n_ff_exp + ne) * 4, each term rounded up to 256).  Every call on a GPU
+ * uses that GPU's one array: calls that overlap in time on one GPU (two backends, two threads) race; a call reads
+ * only what it has written itself, so nothing needs clearing between calls.  Enqueues on the backend's stream like
+ * infr_hip_execute; no profiling events are recorded for it. */
+#define INFR_HIP_STATIC_SCRATCH_BYTES (1u << 20)
+typedef struct infr_hip_moe_ffn_static_args {
+    const infr_hip_buffer *x;          /* [rows, ne] f32 */
+    const infr_hip_buffer *router;     /* [n_expert, ne] f32 */
+    const infr_hip_buffer *gate_exps;  /* [n_expert, n_ff_exp, ne] */
+    const infr_hip_buffer *up_exps;    /* [n_expert, n_ff_exp, ne] */
+    const infr_hip_buffer *down_exps;  /* [n_expert, ne, n_ff_exp] */
+    infr_hip_buffer *dst;              /* [rows, ne] f32 */
+    int32_t gate_dtype, up_dtype, down_dtype;   /* infr_dtype of the three banks */
+    uint32_t rows, ne, n_expert, n_used, n_ff_exp;
+} infr_hip_moe_ffn_static_args;
+infr_status infr_hip_moe_ffn_static(infr_hip_backend *be, const infr_hip_moe_ffn_static_args *a);
+
 #ifdef __cplusplus
 }
 #endif

@@ -179,6 +179,17 @@ class _Config(C.Structure):
                 ("disable_op_fusion", C.c_uint32), ("moe_route_exact_first", C.c_uint32), ("reserved", C.c_uint32 * 4)]
 
 
+class _MoeFfnStaticArgs(C.Structure):
+    _fields_ = [("x", C.c_void_p), ("router", C.c_void_p), ("gate_exps", C.c_void_p), ("up_exps", C.c_void_p),
+                ("down_exps", C.c_void_p), ("dst", C.c_void_p),
+                ("gate_dtype", C.c_int32), ("up_dtype", C.c_int32), ("down_dtype", C.c_int32),
+                ("rows", C.c_uint32), ("ne", C.c_uint32), ("n_expert", C.c_uint32), ("n_used", C.c_uint32),
+                ("n_ff_exp", C.c_uint32)]
+
+
+STATIC_SCRATCH_BYTES = 1 << 20   # INFR_HIP_STATIC_SCRATCH_BYTES
+
+
 class _ProfEntry(C.Structure):
     _fields_ = [("kernel", C.c_char * 64), ("launches", C.c_uint64), ("total_ms", C.c_double),
                 ("min_ms", C.c_double), ("max_ms", C.c_double)]
@@ -211,6 +222,7 @@ _SIGNATURES = {
     "infr_hip_plan_moe_routing": ([_V, _V, C.c_uint32, _V, _V, _V, _V], C.c_int),
     "infr_hip_plan_moe_bucketing": ([_V, _V, C.c_uint32, _V, _V, _V], C.c_int),
     "infr_hip_dequant": ([_V, _V, C.c_int32, C.c_uint64, _V], C.c_int),
+    "infr_hip_moe_ffn_static": ([_V, C.POINTER(_MoeFfnStaticArgs)], C.c_int),
 }
 
 _lib: Optional[C.CDLL] = None
@@ -597,6 +609,15 @@ class Backend:
         _check(self._lib.infr_hip_plan_moe_bucketing(self._h, plan._h, op_index, offsets.ctypes.data_as(_V),
                                                      src.ctypes.data_as(_V), slot.ctypes.data_as(_V)))
         return {"offsets": offsets, "pair_row": src // m.n_used, "pair_rank": src % m.n_used, "slot_pair": slot}
+
+    def moe_ffn_static(self, *, x: Buffer, router: Buffer, gate_exps: Buffer, up_exps: Buffer, down_exps: Buffer,
+                       dst: Buffer, gate_dtype: DType, down_dtype: DType, rows: int, ne: int, n_expert: int, n_used: int,
+                       n_ff_exp: int, up_dtype: Optional[DType] = None) -> None:
+        """infr_hip_moe_ffn_static: one plain Op::MoeFfn on the caller's buffers; allocates nothing."""
+        a = _MoeFfnStaticArgs(x=x._h, router=router._h, gate_exps=gate_exps._h, up_exps=up_exps._h, down_exps=down_exps._h,
+                              dst=dst._h, gate_dtype=int(gate_dtype), up_dtype=int(gate_dtype if up_dtype is None else up_dtype),
+                              down_dtype=int(down_dtype), rows=rows, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=n_ff_exp)
+        _check(self._lib.infr_hip_moe_ffn_static(self._h, C.byref(a)))
 
     def dequant(self, src: Buffer, dtype: DType, numel: int) -> np.ndarray:
         dst = self.alloc(numel * 4, BufferUsage.Readback)

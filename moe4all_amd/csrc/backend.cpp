@@ -39,6 +39,15 @@ infr_status fail(infr_status st, const char* fmt, ...) {
         if (e_ != hipSuccess) return fail(INFR_ERR_BACKEND, "hip: %s failed: %s", #expr, hipGetErrorString(e_)); \
     } while (0)
 
+// Scratch of infr_hip_moe_ffn_static, the entry point that allocates nothing: routing results and the activation rows
+// between the two expert stages live in this file-scope device array.  Every GPU holds its own copy at its own
+// address until the process ends; host code never passes the array's name to a kernel (the name is only a host-side
+// stand-in): infr_hip_create asks for the current device's address once and all uses go through that pointer.
+static __device__ __align__(256) unsigned char scratch[INFR_HIP_STATIC_SCRATCH_BYTES];
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mu;
+void* g_scratch_ptr[kMaxDevices] = {};   // per device ordinal, filled by infr_hip_create with that device current
+
 constexpr uint64_t kBackendMagic = 0x494e465242454e44ull;  // "INFRBEND"
 constexpr uint64_t kBufferMagic = 0x494e465242554646ull;   // "INFRBUFF"
 constexpr uint64_t kPlanMagic = 0x494e4652504c414eull;     // "INFRPLAN"
@@ -171,6 +180,7 @@ struct infr_hip_backend {
     struct Pending { std::string name; hipEvent_t a, b; };
     std::vector<Pending> pending;
     std::vector<hipEvent_t> event_pool;
+    void* static_scratch = nullptr;   // this device's copy of the file-scope scratch array (infr_hip_moe_ffn_static)
 };
 
 namespace {
@@ -185,8 +195,8 @@ struct Timed {
     infr_hip_backend* be;
     const char* name;
     infr::LaunchTiming lt{nullptr, nullptr};
-    Timed(infr_hip_backend* be_, const char* n) : be(be_), name(n) {
-        if (!be->prof_on.load(std::memory_order_relaxed)) return;
+    Timed(infr_hip_backend* be_, const char* n) : be(be_), name(n) {   // be_ == nullptr: never timed (no event is created)
+        if (!be || !be->prof_on.load(std::memory_order_relaxed)) return;
         auto get = [&]() {
             hipEvent_t e = nullptr;
             if (!be->event_pool.empty()) { e = be->event_pool.back(); be->event_pool.pop_back(); }
@@ -218,6 +228,51 @@ void drain_prof(infr_hip_backend* be) {
         be->event_pool.push_back(p.b);
     }
     be->pending.clear();
+}
+
+// The per-token path of Op::MoeFfn (1 to 15 token rows) once logits are in rp.logits and gp / rp are filled in:
+// routing (inside the gate/up kernel where that is cheaper than a launch), gate/up with the gated activation,
+// down with the rank-ordered combine.  timed == false: no profiling events (nothing is created or allocated).
+void moe_per_token(infr_hip_backend* be, hipStream_t s, infr::MoeGemvParams& gp, const infr::RouteParams& rp, int rows,
+                   uint32_t n_expert_total, bool timed) {
+    infr_hip_backend* tb = timed ? be : nullptr;
+    // Every block of the gate/up kernel routes its own token row when that is cheaper than a
+    // launch of the routing kernel: the blocks of one compute unit repeat it once per row.
+    const bool fast_gu = infr::moe_gate_up_routes_inline(gp);
+    const bool units = !fast_gu && !gp.sh_gate && infr::moe_gate_up_units_supported(gp);
+    gp.route_inline = (fast_gu || (units && infr::moe_gate_up_units_routes_inline(gp))) &&
+                              (rows == 1 || (uint64_t)rows * n_expert_total <= 512) ? 1 : 0;
+    if (!gp.route_inline) {
+        Timed t(tb, "route_topk");
+        infr::launch_route(s, rp);
+    }
+    {
+        Timed t(tb, gp.sh_gate ? "moe_route_gate_up_shared" : units ? (gp.route_inline ? "moe_route_gate_up_units" : "moe_gate_up_units")
+                    : gp.route_inline ? "moe_route_gate_up" : "moe_gate_up");
+        infr::launch_moe_gate_up(s, gp);
+    }
+    gp.x = nullptr;
+    if (!gp.sh_down && !infr::moe_down_is_fast(gp) && infr::moe_down_units_supported(gp)) {
+        // a down bank without an integer-dot kernel: the unit kernel over all slots of a row with the
+        // rank-ordered weighted sum at its end, or per-pair rows and the sum as a launch of its own
+        // (one or two token rows: from four rows on the per-pair grid spreads better; C2 shape, MXFP4:
+        // 1 row 11.2 -> 6.9 us, 4 rows 22.6 -> 23.6, 8 rows 36.6 -> 45.4)
+        if (rows <= 2 && infr::moe_down_combine_units_supported(gp)) {
+            Timed t(tb, "moe_down_combine_units");
+            infr::launch_moe_down_combine_units(s, gp);
+            return;
+        }
+        {
+            Timed t(tb, "moe_down_units");
+            infr::launch_moe_down_units(s, gp);
+        }
+        Timed t(tb, "moe_unbucket_combine");
+        infr::launch_unbucket_combine(s, gp.y, nullptr, gp.weights, rows, gp.ne, gp.n_used, gp.weight_before, gp.dst, 1,
+                                      nullptr, gp.addend, gp.skip_zero_w);
+        return;
+    }
+    Timed t(tb, gp.sh_down ? "moe_down_combine_shared" : "moe_down_combine");
+    infr::launch_moe_down_combine(s, gp);
 }
 
 size_t round_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
@@ -256,6 +311,21 @@ extern "C" infr_status infr_hip_create(int device_ordinal, const infr_hip_config
     if (e != hipSuccess) {
         delete be;
         return fail(INFR_ERR_BACKEND, "hip: hipStreamCreate failed: %s", hipGetErrorString(e));
+    }
+    if (device_ordinal < kMaxDevices) {
+        // this device's address of the static scratch array, once per device, with the device current
+        std::lock_guard<std::mutex> lk(g_scratch_mu);
+        if (!g_scratch_ptr[device_ordinal]) {
+            void* ptr = nullptr;
+            e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+            if (e != hipSuccess || !ptr) {
+                (void)hipStreamDestroy(be->stream);
+                delete be;
+                return fail(INFR_ERR_BACKEND, "hip: hipGetSymbolAddress(scratch) failed: %s", hipGetErrorString(e));
+            }
+            g_scratch_ptr[device_ordinal] = ptr;
+        }
+        be->static_scratch = g_scratch_ptr[device_ordinal];
     }
     *out = be;
     return INFR_OK;
@@ -1332,46 +1402,8 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                 }
                 gp.route = rp;
                 gp.y = sc.y;
-                // Every block of the gate/up kernel routes its own token row when that is cheaper than a
-                // launch of the routing kernel: the blocks of one compute unit repeat it once per row.
-                const bool fast_gu = infr::moe_gate_up_routes_inline(gp);
-                const bool units = !fast_gu && !gp.sh_gate && infr::moe_gate_up_units_supported(gp);
-                gp.route_inline = (fast_gu || (units && infr::moe_gate_up_units_routes_inline(gp))) &&
-                                          (rows == 1 || (uint64_t)rows * m.n_expert <= 512) ? 1 : 0;
-                if (!gp.route_inline) {
-                    Timed t(be, "route_topk");
-                    infr::launch_route(s, rp);
-                }
                 gp.route_exact_first = be->cfg.moe_route_exact_first ? 1 : 0;
-                {
-                    Timed t(be, gp.sh_gate ? "moe_route_gate_up_shared" : units ? (gp.route_inline ? "moe_route_gate_up_units" : "moe_gate_up_units")
-                                : gp.route_inline ? "moe_route_gate_up" : "moe_gate_up");
-                    infr::launch_moe_gate_up(s, gp);
-                }
-                gp.x = nullptr;
-                if (!gp.sh_down && !infr::moe_down_is_fast(gp) && infr::moe_down_units_supported(gp)) {
-                    // a down bank without an integer-dot kernel: the unit kernel over all slots of a row with the
-                    // rank-ordered weighted sum at its end, or per-pair rows and the sum as a launch of its own
-                    // (one or two token rows: from four rows on the per-pair grid spreads better; C2 shape, MXFP4:
-                    // 1 row 11.2 -> 6.9 us, 4 rows 22.6 -> 23.6, 8 rows 36.6 -> 45.4)
-                    if (rows <= 2 && infr::moe_down_combine_units_supported(gp)) {
-                        Timed t(be, "moe_down_combine_units");
-                        infr::launch_moe_down_combine_units(s, gp);
-                        break;
-                    }
-                    {
-                        Timed t(be, "moe_down_units");
-                        infr::launch_moe_down_units(s, gp);
-                    }
-                    Timed t(be, "moe_unbucket_combine");
-                    infr::launch_unbucket_combine(s, gp.y, nullptr, gp.weights, rows, (int)m.ne, (int)m.n_used,
-                                                  (int)m.weight_before, gp.dst, 1, nullptr, gp.addend, gp.skip_zero_w);
-                    break;
-                }
-                {
-                    Timed t(be, gp.sh_down ? "moe_down_combine_shared" : "moe_down_combine");
-                    infr::launch_moe_down_combine(s, gp);
-                }
+                moe_per_token(be, s, gp, rp, rows, m.n_expert, true);
                 break;
             }
             case INFR_OP_LINEAR: {
@@ -1468,6 +1500,83 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
     }
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(INFR_ERR_BACKEND, "execute: kernel launch failed: %s", hipGetErrorString(e));
+    return INFR_OK;
+}
+
+// ============================================================================ entry point without allocation
+extern "C" infr_status infr_hip_moe_ffn_static(infr_hip_backend* be, const infr_hip_moe_ffn_static_args* a) {
+    if (!ok_backend(be) || !a) return fail(INFR_ERR_INVALID, "moe_ffn_static: bad handle");
+    if (!be->static_scratch) return fail(INFR_ERR_BACKEND, "moe_ffn_static: device %d has no static scratch", be->device);
+    const infr_hip_buffer* bufs[6] = {a->x, a->router, a->gate_exps, a->up_exps, a->down_exps, a->dst};
+    static const char* const names[6] = {"x", "router", "gate_exps", "up_exps", "down_exps", "dst"};
+    for (int i = 0; i < 6; i++) {
+        if (!ok_buffer(bufs[i])) return fail(INFR_ERR_INVALID, "moe_ffn_static: %s is not a buffer", names[i]);
+        if (bufs[i]->be != be) return fail(INFR_ERR_INVALID, "moe_ffn_static: %s belongs to another backend", names[i]);
+    }
+    if (a->rows == 0) return INFR_OK;
+    if (a->ne == 0 || a->n_expert == 0 || a->n_used == 0 || a->n_ff_exp == 0 || a->n_used > a->n_expert)
+        return fail(INFR_ERR_INVALID, "moe_ffn_static: ne/n_expert/n_used/n_ff_exp must be positive and n_used <= n_expert");
+    if (a->rows >= kBucketedMinRows || a->n_expert > 2048 || a->n_used > 64)
+        return fail(INFR_ERR_UNSUPPORTED, "moe_ffn_static: %u token rows / %u experts / top-%u: the entry point takes 1..%u rows, "
+                    "up to 2048 experts, top-64", a->rows, a->n_expert, a->n_used, kBucketedMinRows - 1);
+    // operand extents against the shapes
+    const int dts[3] = {a->gate_dtype, a->up_dtype, a->down_dtype};
+    const uint32_t kdims[3] = {a->ne, a->ne, a->n_ff_exp};
+    size_t wbytes[3];
+    for (int i = 0; i < 3; i++) {
+        int el = 1, by = 4;
+        if (!geometry(dts[i], &el, &by) || dts[i] == INFR_I32 || dts[i] == INFR_U32)
+            return fail(INFR_ERR_UNSUPPORTED, "moe_ffn_static: %s has no decodable weight dtype (%d)", names[2 + i], dts[i]);
+        if (kdims[i] % (uint32_t)el != 0)
+            return fail(INFR_ERR_INVALID, "moe_ffn_static: %s rows of %u elements are not whole %s blocks", names[2 + i], kdims[i], dtype_name(dts[i]));
+        wbytes[i] = (size_t)a->n_expert * a->n_ff_exp * a->ne / (size_t)el * (size_t)by;
+        if (bufs[2 + i]->len < wbytes[i])
+            return fail(INFR_ERR_INVALID, "moe_ffn_static: %s holds %zu bytes, the shapes need %zu", names[2 + i], bufs[2 + i]->len, wbytes[i]);
+    }
+    const size_t act_bytes = (size_t)a->rows * a->ne * 4, router_bytes = (size_t)a->n_expert * a->ne * 4;
+    if (a->x->len < act_bytes || a->dst->len < act_bytes || a->router->len < router_bytes)
+        return fail(INFR_ERR_INVALID, "moe_ffn_static: x / dst / router hold fewer bytes than [rows, ne] / [n_expert, ne] f32");
+    // scratch layout: logits, probs [rows, n_expert]; ids, weights [rows, n_used]; h [rows, n_used, n_ff_exp]; y [rows, n_used, ne]
+    const size_t pairs = (size_t)a->rows * a->n_used;
+    const size_t sz_l = round_up((size_t)a->rows * a->n_expert * 4, 256), sz_p = round_up(pairs * 4, 256);
+    const size_t sz_h = round_up(pairs * a->n_ff_exp * 4, 256), sz_y = round_up(pairs * a->ne * 4, 256);
+    const size_t need = 2 * sz_l + 2 * sz_p + sz_h + sz_y;
+    if (need > INFR_HIP_STATIC_SCRATCH_BYTES)
+        return fail(INFR_ERR_UNSUPPORTED, "moe_ffn_static: these shapes need %zu bytes of scratch, the static scratch holds %u",
+                    need, (unsigned)INFR_HIP_STATIC_SCRATCH_BYTES);
+    std::lock_guard<std::mutex> lk(be->mu);
+    HIP_TRY(hipSetDevice(be->device));
+    char* sp = static_cast<char*>(be->static_scratch);   // the device address, never the array's name
+    float* logits = reinterpret_cast<float*>(sp);
+    float* probs = reinterpret_cast<float*>(sp + sz_l);
+    int32_t* ids = reinterpret_cast<int32_t*>(sp + 2 * sz_l);
+    float* weights = reinterpret_cast<float*>(sp + 2 * sz_l + sz_p);
+    float* h = reinterpret_cast<float*>(sp + 2 * sz_l + 2 * sz_p);
+    float* y = reinterpret_cast<float*>(sp + 2 * sz_l + 2 * sz_p + sz_h);
+    hipStream_t s = be->stream;
+    const int rows = (int)a->rows;
+    if (!infr::launch_router_logits(s, (const uint8_t*)a->router->dptr, INFR_F32, (size_t)a->ne * 4, (const float*)a->x->dptr,
+                                    (int)a->ne, (int)a->n_expert, rows, logits))
+        return fail(INFR_ERR_UNSUPPORTED, "moe_ffn_static: ne=%u does not fit the router kernel's LDS budget", a->ne);
+    infr::RouteParams rp{};
+    rp.logits = logits; rp.n_expert = (int)a->n_expert; rp.n_used = (int)a->n_used; rp.rows = rows;
+    rp.gating = INFR_GATING_SOFTMAX; rp.norm_w = 1; rp.scale = 1.0f;
+    rp.ids = ids; rp.weights = weights; rp.probs = probs;
+    infr::MoeGemvParams gp{};
+    gp.ids = ids; gp.weights = weights;
+    gp.gate_dt = a->gate_dtype; gp.up_dt = a->up_dtype; gp.down_dt = a->down_dtype;
+    gp.gate = (const uint8_t*)a->gate_exps->dptr; gp.gate_stride = wbytes[0] / a->n_expert;
+    gp.up = (const uint8_t*)a->up_exps->dptr; gp.up_stride = wbytes[1] / a->n_expert;
+    gp.down = (const uint8_t*)a->down_exps->dptr; gp.down_stride = wbytes[2] / a->n_expert;
+    gp.rows = rows; gp.ne = (int)a->ne; gp.nff = (int)a->n_ff_exp; gp.n_used = (int)a->n_used; gp.n_expert = (int)a->n_expert;
+    gp.act = INFR_ACT_SILU;
+    gp.h = h; gp.y = y; gp.dst = (float*)a->dst->dptr; gp.x = (const float*)a->x->dptr;
+    gp.n_cu = be->prop.multiProcessorCount;
+    gp.route = rp;
+    gp.route_exact_first = be->cfg.moe_route_exact_first ? 1 : 0;
+    moe_per_token(be, s, gp, rp, rows, a->n_expert, false);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(INFR_ERR_BACKEND, "moe_ffn_static: kernel launch failed: %s", hipGetErrorString(e));
     return INFR_OK;
 }
 
