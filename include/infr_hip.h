@@ -33,7 +33,7 @@ typedef enum infr_status {
     INFR_OK = 0,
     INFR_ERR_BACKEND = 1,     /* Error::Backend: HIP failure, bad binding, size mismatch */
     INFR_ERR_UNSUPPORTED = 2, /* Error::Unsupported: op / dtype / option not implemented */
-    INFR_ERR_ABORTED = 3,     /* Error::Aborted: shutdown latch set */
+    INFR_ERR_ABORTED = 3,     /* Error::Aborted: shutdown latch set (reserved: this library has no latch and never returns it) */
     INFR_ERR_INVALID = 4,     /* null / foreign handle, malformed graph */
     INFR_ERR_LOADER = 5,      /* Error::Loader: malformed or inconsistent weight file */
     INFR_ERR_IO = 6           /* Error::Io: the file could not be opened or mapped */
@@ -217,7 +217,10 @@ typedef struct infr_hip_config {
 
 /* Construction of the backend object (reference: VulkanBackend::new / CpuBackend::new,
  * crates/infr-cpu/src/lib.rs:868).  cfg may be NULL.  Fails with INFR_ERR_BACKEND when no
- * gfx950 device is visible: there is no CPU fallback. */
+ * gfx950 device is visible: there is no CPU fallback.
+ * infr_hip_destroy drains and closes the backend's stream; buffers and plans made by it may be freed
+ * afterwards in any order (each keeps the backend object alive until it is freed, as the reference's buffers
+ * keep their device alive), every other call on the destroyed handle or with such a buffer is refused. */
 infr_status infr_hip_create(int device_ordinal, const infr_hip_config *cfg, infr_hip_backend **out);
 void infr_hip_destroy(infr_hip_backend *be);
 

@@ -431,8 +431,7 @@ class Buffer:
 
     def __del__(self):
         try:
-            if self._h and self._be._h:
-                self.free()
+            self.free()   # safe after Backend.close(): a buffer keeps its backend object alive until it is freed
         except Exception:
             pass
 
@@ -448,8 +447,7 @@ class Plan:
 
     def __del__(self):
         try:
-            if self._h and self._be._h:
-                self.free()
+            self.free()   # safe after Backend.close(), as for buffers
         except Exception:
             pass
 

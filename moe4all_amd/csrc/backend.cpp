@@ -12,7 +12,10 @@
 #include <cstdio>
 #include <cstring>
 #include <map>
+#include <memory>
 #include <mutex>
+#include <new>
+#include <stdexcept>
 #include <string>
 #include <vector>
 
@@ -31,6 +34,24 @@ infr_status fail(infr_status st, const char* fmt, ...) {
     va_end(ap);
     g_last_error = buf;
     return st;
+}
+
+// No exception crosses the C ABI: every entry point that can allocate host memory or touch a container is a
+// function-try-block whose handler lands here (called inside a catch clause; rethrows to classify).
+infr_status guard_fail(const char* what) noexcept {
+    try {
+        try {
+            throw;
+        } catch (const std::bad_alloc&) {
+            return fail(INFR_ERR_BACKEND, "%s: out of host memory", what);
+        } catch (const std::exception& e) {
+            return fail(INFR_ERR_BACKEND, "%s: %s", what, e.what());
+        } catch (...) {
+            return fail(INFR_ERR_BACKEND, "%s: unknown exception", what);
+        }
+    } catch (...) {
+        return INFR_ERR_BACKEND;   // not even the message could be stored
+    }
 }
 
 #define HIP_TRY(expr)                                                                                        \
@@ -166,6 +187,10 @@ struct infr_hip_plan {
     std::vector<FuseOp> fuse_head;     // kMoeShared: the records of the ops it absorbed, as they were before
     int32_t* zero_ids = nullptr;       // [max rows of a fused gate/up] expert id 0 for every row
     std::vector<size_t> copy_tmp;      // per op: arena offset of the staging window of an aliasing Copy, else 0
+    ~infr_hip_plan() {
+        magic = 0;
+        if (arena) (void)hipFree(arena);   // the caller has made the plan's device current and drained its stream
+    }
 };
 
 struct infr_hip_backend {
@@ -181,11 +206,22 @@ struct infr_hip_backend {
     std::vector<Pending> pending;
     std::vector<hipEvent_t> event_pool;
     void* static_scratch = nullptr;   // this device's copy of the file-scope scratch array (infr_hip_moe_ffn_static)
+    // The object outlives infr_hip_destroy while buffers or plans still point at it (the reference's buffers keep their
+    // device alive the same way): destroy drains and closes the stream and drops the creator's reference, the last
+    // buffer / plan freed afterwards deletes the object.
+    std::atomic<int> refs{1};
+    std::atomic<int> closed{0};
 };
 
 namespace {
 
-bool ok_backend(const infr_hip_backend* be) { return be && be->magic == kBackendMagic; }
+bool ok_backend(const infr_hip_backend* be) { return be && be->magic == kBackendMagic && !be->closed.load(); }
+void release_backend(infr_hip_backend* be) {
+    if (be && be->magic == kBackendMagic && be->refs.fetch_sub(1) == 1) {
+        be->magic = 0;
+        delete be;
+    }
+}
 bool ok_buffer(const infr_hip_buffer* b) { return b && b->magic == kBufferMagic; }
 bool ok_plan(const infr_hip_plan* p) { return p && p->magic == kPlanMagic; }
 
@@ -275,6 +311,37 @@ void moe_per_token(infr_hip_backend* be, hipStream_t s, infr::MoeGemvParams& gp,
     infr::launch_moe_down_combine(s, gp);
 }
 
+// Every tensor id an op names (INFR_NO_TENSOR for absent options), for the walk that checks the bindings of a whole
+// plan before its first launch.
+int op_tensors(const infr_op& op, uint32_t (&ids)[12], const char** role) {
+    int n = 0;
+    switch (op.kind) {
+        case INFR_OP_MOE_FFN: {
+            const infr_op_moe_ffn& m = op.u.moe_ffn;
+            *role = "MoeFfn";
+            ids[n++] = m.x; ids[n++] = m.router_x; ids[n++] = m.router; ids[n++] = m.gate_exps;
+            if (!m.fused_gate_up) ids[n++] = m.up_exps;
+            ids[n++] = m.down_exps; ids[n++] = m.dst; ids[n++] = m.down_scale; ids[n++] = m.exp_probs_b; ids[n++] = m.expert_ids;
+            break;
+        }
+        case INFR_OP_LINEAR: *role = "Linear"; ids[n++] = op.u.linear.x; ids[n++] = op.u.linear.weight; ids[n++] = op.u.linear.dst; break;
+        case INFR_OP_GATED_ACT: *role = "GatedAct"; ids[n++] = op.u.gated_act.gate; ids[n++] = op.u.gated_act.up; ids[n++] = op.u.gated_act.dst; break;
+        case INFR_OP_ADD: *role = "Add"; ids[n++] = op.u.add.a; ids[n++] = op.u.add.b; ids[n++] = op.u.add.dst; break;
+        case INFR_OP_MOE_SHARED_EXPERT_ADD: {
+            const infr_op_moe_shared_expert_add& a = op.u.moe_shared_expert_add;
+            *role = "MoeSharedExpertAdd";
+            ids[n++] = a.moe; ids[n++] = a.shexp; ids[n++] = a.gate; ids[n++] = a.dst;
+            break;
+        }
+        case INFR_OP_COPY:
+        case INFR_OP_COPY_STRIDED: *role = "Copy"; ids[n++] = op.u.copy.src; ids[n++] = op.u.copy.dst; break;
+        case INFR_OP_RMS_NORM:
+        case INFR_OP_RMS_NORM_ADD: *role = "RmsNorm"; ids[n++] = op.u.rms_norm.x; ids[n++] = op.u.rms_norm.weight; ids[n++] = op.u.rms_norm.dst; break;
+        default: *role = "op"; break;
+    }
+    return n;
+}
+
 size_t round_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
 }  // namespace
@@ -282,7 +349,7 @@ size_t round_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 // ============================================================================ lifecycle
 extern "C" const char* infr_hip_last_error(void) { return g_last_error.c_str(); }
 
-extern "C" infr_status infr_hip_create(int device_ordinal, const infr_hip_config* cfg, infr_hip_backend** out) {
+extern "C" infr_status infr_hip_create(int device_ordinal, const infr_hip_config* cfg, infr_hip_backend** out) try {
     if (!out) return fail(INFR_ERR_INVALID, "infr_hip_create: out is null");
     *out = nullptr;
     int n = 0;
@@ -329,22 +396,29 @@ extern "C" infr_status infr_hip_create(int device_ordinal, const infr_hip_config
     }
     *out = be;
     return INFR_OK;
-}
+} catch (...) { return guard_fail("infr_hip_create"); }
 
-extern "C" void infr_hip_destroy(infr_hip_backend* be) {
+extern "C" void infr_hip_destroy(infr_hip_backend* be) try {
     if (!ok_backend(be)) return;
-    (void)hipSetDevice(be->device);
-    (void)hipStreamSynchronize(be->stream);
-    for (auto& p : be->pending) { (void)hipEventDestroy(p.a); (void)hipEventDestroy(p.b); }
-    for (auto e : be->event_pool) (void)hipEventDestroy(e);
-    (void)hipStreamDestroy(be->stream);
-    be->magic = 0;
-    delete be;
+    {
+        std::lock_guard<std::mutex> lk(be->mu);
+        (void)hipSetDevice(be->device);
+        (void)hipStreamSynchronize(be->stream);
+        for (auto& p : be->pending) { (void)hipEventDestroy(p.a); (void)hipEventDestroy(p.b); }
+        for (auto e : be->event_pool) (void)hipEventDestroy(e);
+        be->pending.clear();
+        be->event_pool.clear();
+        (void)hipStreamDestroy(be->stream);
+        be->stream = nullptr;
+        be->closed.store(1);   // every later call on this handle is refused; buffers and plans can still be freed
+    }
+    release_backend(be);
+} catch (...) {
 }
 
 extern "C" const char* infr_hip_name(const infr_hip_backend* be) { return ok_backend(be) ? "hip-gfx950" : ""; }
 
-extern "C" infr_status infr_hip_capabilities_get(const infr_hip_backend* be, infr_hip_capabilities* out) {
+extern "C" infr_status infr_hip_capabilities_get(const infr_hip_backend* be, infr_hip_capabilities* out) try {
     if (!ok_backend(be) || !out) return fail(INFR_ERR_INVALID, "capabilities: bad handle");
     memset(out, 0, sizeof *out);
     // some driver stacks report an empty marketing name; the architecture string is always there
@@ -361,7 +435,7 @@ extern "C" infr_status infr_hip_capabilities_get(const infr_hip_backend* be, inf
     out->graph_input_inplace = 1;
     out->device_memory_bytes = (uint64_t)be->prop.totalGlobalMem;
     return INFR_OK;
-}
+} catch (...) { return guard_fail("infr_hip_capabilities_get"); }
 
 // ============================================================================ memory
 static infr_status alloc_impl(infr_hip_backend* be, size_t bytes, int32_t usage, bool zero, infr_hip_buffer** out) {
@@ -378,33 +452,40 @@ static infr_status alloc_impl(infr_hip_backend* be, size_t bytes, int32_t usage,
     if (e != hipSuccess)
         return fail(INFR_ERR_BACKEND, "alloc: hipMalloc(%zu) failed: %s", cap, hipGetErrorString(e));
     if (zero) infr::launch_fill_zero(be->stream, p, cap);
-    auto* b = new infr_hip_buffer();
+    infr_hip_buffer* b = new (std::nothrow) infr_hip_buffer();
+    if (!b) {
+        (void)hipFree(p);
+        return fail(INFR_ERR_BACKEND, "alloc: out of host memory");
+    }
     b->be = be; b->dptr = p; b->len = len; b->cap = cap; b->usage = usage;
+    be->refs.fetch_add(1);   // the buffer keeps its backend alive
     *out = b;
     return INFR_OK;
 }
 
-extern "C" infr_status infr_hip_alloc(infr_hip_backend* be, size_t bytes, int32_t usage, infr_hip_buffer** out) {
+extern "C" infr_status infr_hip_alloc(infr_hip_backend* be, size_t bytes, int32_t usage, infr_hip_buffer** out) try {
     return alloc_impl(be, bytes, usage, true, out);
-}
-extern "C" infr_status infr_hip_alloc_uninit(infr_hip_backend* be, size_t bytes, int32_t usage, infr_hip_buffer** out) {
+} catch (...) { return guard_fail("infr_hip_alloc"); }
+extern "C" infr_status infr_hip_alloc_uninit(infr_hip_backend* be, size_t bytes, int32_t usage, infr_hip_buffer** out) try {
     return alloc_impl(be, bytes, usage, false, out);
-}
+} catch (...) { return guard_fail("infr_hip_alloc_uninit"); }
 extern "C" size_t infr_hip_buffer_len(const infr_hip_buffer* buf) { return ok_buffer(buf) ? buf->len : 0; }
 extern "C" uint64_t infr_hip_buffer_device_addr(const infr_hip_buffer* buf) {
     return ok_buffer(buf) ? (uint64_t)(uintptr_t)buf->dptr : 0;
 }
-extern "C" void infr_hip_buffer_free(infr_hip_buffer* buf) {
+extern "C" void infr_hip_buffer_free(infr_hip_buffer* buf) try {
     if (!ok_buffer(buf)) return;
-    infr_hip_backend* be = buf->be;
-    if (ok_backend(be)) {
+    infr_hip_backend* be = buf->be;   // alive: the buffer holds a reference
+    {
         std::lock_guard<std::mutex> lk(be->mu);
         (void)hipSetDevice(be->device);
-        (void)hipStreamSynchronize(be->stream);  // work that still reads it must drain first
+        if (!be->closed.load()) (void)hipStreamSynchronize(be->stream);  // work that still reads it must drain first
         (void)hipFree(buf->dptr);
     }
     buf->magic = 0;
     delete buf;
+    release_backend(be);
+} catch (...) {
 }
 
 static infr_status check_owned(infr_hip_backend* be, const infr_hip_buffer* b, const char* what) {
@@ -415,7 +496,7 @@ static infr_status check_owned(infr_hip_backend* be, const infr_hip_buffer* b, c
 }
 
 extern "C" infr_status infr_hip_upload_range(infr_hip_backend* be, infr_hip_buffer* dst, size_t offset,
-                                             const void* src, size_t n) {
+                                             const void* src, size_t n) try {
     if (infr_status st = check_owned(be, dst, "upload")) return st;
     if (n && !src) return fail(INFR_ERR_INVALID, "upload: src is null");
     if (offset > dst->len || n > dst->len - offset)
@@ -426,12 +507,12 @@ extern "C" infr_status infr_hip_upload_range(infr_hip_backend* be, infr_hip_buff
     HIP_TRY(hipMemcpyAsync((char*)dst->dptr + offset, src, n, hipMemcpyHostToDevice, be->stream));
     HIP_TRY(hipStreamSynchronize(be->stream));  // src may be freed by the caller on return
     return INFR_OK;
-}
-extern "C" infr_status infr_hip_upload(infr_hip_backend* be, infr_hip_buffer* dst, const void* src, size_t n) {
+} catch (...) { return guard_fail("infr_hip_upload_range"); }
+extern "C" infr_status infr_hip_upload(infr_hip_backend* be, infr_hip_buffer* dst, const void* src, size_t n) try {
     return infr_hip_upload_range(be, dst, 0, src, n);
-}
+} catch (...) { return guard_fail("infr_hip_upload"); }
 extern "C" infr_status infr_hip_download_range(infr_hip_backend* be, const infr_hip_buffer* src, size_t offset,
-                                               void* dst, size_t n) {
+                                               void* dst, size_t n) try {
     if (infr_status st = check_owned(be, src, "download")) return st;
     if (n && !dst) return fail(INFR_ERR_INVALID, "download: dst is null");
     if (offset > src->len || n > src->len - offset)
@@ -442,12 +523,12 @@ extern "C" infr_status infr_hip_download_range(infr_hip_backend* be, const infr_
     if (n) HIP_TRY(hipMemcpyAsync(dst, (const char*)src->dptr + offset, n, hipMemcpyDeviceToHost, be->stream));
     HIP_TRY(hipStreamSynchronize(be->stream));
     return INFR_OK;
-}
-extern "C" infr_status infr_hip_download(infr_hip_backend* be, const infr_hip_buffer* src, void* dst, size_t n) {
+} catch (...) { return guard_fail("infr_hip_download_range"); }
+extern "C" infr_status infr_hip_download(infr_hip_backend* be, const infr_hip_buffer* src, void* dst, size_t n) try {
     return infr_hip_download_range(be, src, 0, dst, n);
-}
+} catch (...) { return guard_fail("infr_hip_download"); }
 extern "C" infr_status infr_hip_copy_buffer(infr_hip_backend* be, const infr_hip_buffer* src, infr_hip_buffer* dst,
-                                            size_t n) {
+                                            size_t n) try {
     if (infr_status st = check_owned(be, src, "copy_buffer")) return st;
     if (infr_status st = check_owned(be, dst, "copy_buffer")) return st;
     if (n > src->len || n > dst->len)
@@ -457,25 +538,25 @@ extern "C" infr_status infr_hip_copy_buffer(infr_hip_backend* be, const infr_hip
     HIP_TRY(hipSetDevice(be->device));
     HIP_TRY(hipMemcpyAsync(dst->dptr, src->dptr, n, hipMemcpyDeviceToDevice, be->stream));
     return INFR_OK;
-}
+} catch (...) { return guard_fail("infr_hip_copy_buffer"); }
 
-extern "C" infr_status infr_hip_sync(infr_hip_backend* be) {
+extern "C" infr_status infr_hip_sync(infr_hip_backend* be) try {
     if (!ok_backend(be)) return fail(INFR_ERR_INVALID, "sync: bad handle");
     std::lock_guard<std::mutex> lk(be->mu);
     HIP_TRY(hipSetDevice(be->device));
     HIP_TRY(hipStreamSynchronize(be->stream));
     HIP_TRY(hipGetLastError());
     return INFR_OK;
-}
+} catch (...) { return guard_fail("infr_hip_sync"); }
 
 // ---- shared with sibling translation units of this library (not part of the public ABI)
-extern "C" infr_status infr_hip_internal_fail(infr_status st, const char* msg) { return fail(st, "%s", msg); }
+extern "C" infr_status infr_hip_internal_fail(infr_status st, const char* msg) try { return fail(st, "%s", msg); } catch (...) { return guard_fail("infr_hip_internal_fail"); }
 
 // Validates [byte_offset, byte_offset+bytes) of buf, makes the device current and returns the
 // device pointer and the backend's stream WITH the submission lock held; the caller enqueues
 // its work and then calls infr_hip_internal_unlock.  On error the lock is not held.
 extern "C" infr_status infr_hip_internal_buffer_span(infr_hip_backend* be, infr_hip_buffer* buf, size_t byte_offset,
-                                                     size_t bytes, void** dptr, hipStream_t* stream) {
+                                                     size_t bytes, void** dptr, hipStream_t* stream) try {
     if (infr_status st = check_owned(be, buf, "buffer_span")) return st;
     if (byte_offset > buf->len || bytes > buf->len - byte_offset)
         return fail(INFR_ERR_BACKEND, "byte range %zu..%zu exceeds buffer size %zu", byte_offset, byte_offset + bytes,
@@ -489,7 +570,7 @@ extern "C" infr_status infr_hip_internal_buffer_span(infr_hip_backend* be, infr_
     *dptr = (char*)buf->dptr + byte_offset;
     *stream = be->stream;
     return INFR_OK;
-}
+} catch (...) { return guard_fail("infr_hip_internal_buffer_span"); }
 extern "C" void infr_hip_internal_unlock(infr_hip_backend* be) { be->mu.unlock(); }
 
 // ============================================================================ compile
@@ -525,7 +606,8 @@ struct Check {
         int be = 0, bb = 0;
         if (!geometry(dt(id), &be, &bb) || dt(id) == INFR_I32 || dt(id) == INFR_U32) {
             set(INFR_ERR_UNSUPPORTED, std::string(role) + ": weight dtype " + dtype_name(dt(id)) +
-                                          " has no decode on this backend (F32/F16/Bf16 and the affine quants Q4_0..Q8_0, Q2K..Q6K)");
+                                          " has no decode on this backend (decoded: F32/F16/Bf16, Q4_0 Q4_1 Q5_0 Q5_1 Q8_0, Q2K..Q6K, "
+                                          "IQ4_NL IQ4_XS MXFP4 NVFP4 TQ1_0 TQ2_0 Q2_0 and the grid i-quants)");
             return;
         }
         if (in_f % (uint64_t)be != 0)
@@ -545,11 +627,12 @@ size_t tensor_bytes(const infr_tensor_decl& t, uint64_t numel) {
 
 }  // namespace
 
-extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* g, infr_hip_plan** out) {
+extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* g, infr_hip_plan** out) try {
     if (!ok_backend(be) || !g || !out) return fail(INFR_ERR_INVALID, "compile: bad handle");
     *out = nullptr;
     if ((g->n_tensors && !g->tensors) || (g->n_ops && !g->ops)) return fail(INFR_ERR_INVALID, "compile: null arrays");
-    auto plan = new infr_hip_plan();
+    std::unique_ptr<infr_hip_plan> holder(new infr_hip_plan());   // freed on every early return and on an exception
+    infr_hip_plan* plan = holder.get();
     plan->be = be;
     plan->tensors.assign(g->tensors, g->tensors + g->n_tensors);
     plan->ops.assign(g->ops, g->ops + g->n_ops);
@@ -558,7 +641,7 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
     plan->moe.resize(g->n_ops);
     plan->lin.resize(g->n_ops);
     auto bail = [&](infr_status st, const std::string& m) {
-        delete plan;
+        holder.reset();
         return fail(st, "%s", m.c_str());
     };
     size_t arena = 0;
@@ -703,6 +786,22 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
                 }
                 if (!batched && !bucketed) shared += round_up(pairs * m.ne * 4, 256);   // per-pair down results of the unit kernels
                 if (shared > shared_need) shared_need = shared;
+                if (!batched && !bucketed && rows * m.n_used > 65535) {
+                    // the per-token kernels put the token rows (the generic ones rows * n_used) on the grid's y axis
+                    c.set(INFR_ERR_UNSUPPORTED, "MoeFfn: " + std::to_string(rows) + " token rows on expert banks without a "
+                          "batched kernel (" + dtype_name(c.dt(m.gate_exps)) + " / " + dtype_name(c.dt(m.down_exps)) +
+                          ") exceed the per-token path's grid (rows * n_used <= 65535)");
+                    break;
+                }
+                {
+                    // the logits kernel's staging must fit the LDS: refused here, not in the middle of execute
+                    int re = 1, rb = 4;
+                    geometry(c.dt(m.router), &re, &rb);
+                    if (!infr::router_logits_fits(c.dt(m.router), (size_t)(m.ne / re) * rb, (int)m.ne, (int)rows)) {
+                        c.set(INFR_ERR_UNSUPPORTED, "MoeFfn: ne=" + std::to_string(m.ne) + " does not fit the router kernel's LDS budget");
+                        break;
+                    }
+                }
                 plan->moe[oi].rows = (int)rows;
                 plan->moe[oi].batched = batched;
                 plan->moe[oi].bucketed = bucketed;
@@ -1064,31 +1163,30 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
         const int32_t table[2] = {0, (int32_t)l.m};
         e = hipMemcpyAsync((char*)plan->arena + plan->lin[oi].offsets_off, table, sizeof table, hipMemcpyHostToDevice, be->stream);
         if (e == hipSuccess) e = hipStreamSynchronize(be->stream);   // `table` is on this stack frame
-        if (e != hipSuccess) {
-            hipFree(plan->arena);
+        if (e != hipSuccess)
             return bail(INFR_ERR_BACKEND, std::string("compile: bucket table upload failed: ") + hipGetErrorString(e));
-        }
     }
-    *out = plan;
+    be->refs.fetch_add(1);   // the plan keeps its backend alive
+    *out = holder.release();
     return INFR_OK;
-}
+} catch (...) { return guard_fail("infr_hip_compile"); }
 
-extern "C" void infr_hip_plan_free(infr_hip_plan* plan) {
+extern "C" void infr_hip_plan_free(infr_hip_plan* plan) try {
     if (!ok_plan(plan)) return;
-    infr_hip_backend* be = plan->be;
-    if (ok_backend(be)) {
+    infr_hip_backend* be = plan->be;   // alive: the plan holds a reference
+    {
         std::lock_guard<std::mutex> lk(be->mu);
         (void)hipSetDevice(be->device);
-        (void)hipStreamSynchronize(be->stream);
-        if (plan->arena) (void)hipFree(plan->arena);
+        if (!be->closed.load()) (void)hipStreamSynchronize(be->stream);
+        delete plan;   // frees the arena
     }
-    plan->magic = 0;
-    delete plan;
+    release_backend(be);
+} catch (...) {
 }
 
 // ============================================================================ execute
 extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* plan, const infr_binding* bindings,
-                                        uint32_t n_bindings) {
+                                        uint32_t n_bindings) try {
     if (!ok_backend(be)) return fail(INFR_ERR_INVALID, "execute: backend handle is not a hip backend");
     if (!ok_plan(plan) || plan->be != be) return fail(INFR_ERR_BACKEND, "hip backend: incompatible plan");
     if (n_bindings && !bindings) return fail(INFR_ERR_INVALID, "execute: bindings is null");
@@ -1121,6 +1219,14 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
         }
         return true;
     };
+    // every tensor of every op is resolved before the first launch: a plan either runs whole or not at all
+    for (size_t oi = 0; oi < plan->ops.size(); oi++) {
+        uint32_t ids[12];
+        const char* role = "op";
+        const int n_ids = op_tensors(plan->ops[oi], ids, &role);
+        for (int k = 0; k < n_ids; k++)
+            if (!need(ids[k], role)) return INFR_ERR_BACKEND;
+    }
     std::lock_guard<std::mutex> lk(be->mu);
     HIP_TRY(hipSetDevice(be->device));
     hipStream_t s = be->stream;
@@ -1501,10 +1607,10 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(INFR_ERR_BACKEND, "execute: kernel launch failed: %s", hipGetErrorString(e));
     return INFR_OK;
-}
+} catch (...) { return guard_fail("infr_hip_execute"); }
 
 // ============================================================================ entry point without allocation
-extern "C" infr_status infr_hip_moe_ffn_static(infr_hip_backend* be, const infr_hip_moe_ffn_static_args* a) {
+extern "C" infr_status infr_hip_moe_ffn_static(infr_hip_backend* be, const infr_hip_moe_ffn_static_args* a) try {
     if (!ok_backend(be) || !a) return fail(INFR_ERR_INVALID, "moe_ffn_static: bad handle");
     if (!be->static_scratch) return fail(INFR_ERR_BACKEND, "moe_ffn_static: device %d has no static scratch", be->device);
     const infr_hip_buffer* bufs[6] = {a->x, a->router, a->gate_exps, a->up_exps, a->down_exps, a->dst};
@@ -1578,17 +1684,17 @@ extern "C" infr_status infr_hip_moe_ffn_static(infr_hip_backend* be, const infr_
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(INFR_ERR_BACKEND, "moe_ffn_static: kernel launch failed: %s", hipGetErrorString(e));
     return INFR_OK;
-}
+} catch (...) { return guard_fail("infr_hip_moe_ffn_static"); }
 
 // ============================================================================ taps
-extern "C" infr_status infr_hip_prof_enable(infr_hip_backend* be, int on) {
+extern "C" infr_status infr_hip_prof_enable(infr_hip_backend* be, int on) try {
     if (!ok_backend(be)) return fail(INFR_ERR_INVALID, "prof: bad handle");
     std::lock_guard<std::mutex> lk(be->mu);
     be->prof_on.store(on ? 1 : 0);
     return INFR_OK;
-}
+} catch (...) { return guard_fail("infr_hip_prof_enable"); }
 
-extern "C" infr_status infr_hip_prof_read(infr_hip_backend* be, infr_hip_prof_entry* out, uint32_t cap, uint32_t* n_out) {
+extern "C" infr_status infr_hip_prof_read(infr_hip_backend* be, infr_hip_prof_entry* out, uint32_t cap, uint32_t* n_out) try {
     if (!ok_backend(be) || !n_out) return fail(INFR_ERR_INVALID, "prof: bad handle");
     std::lock_guard<std::mutex> lk(be->mu);
     HIP_TRY(hipSetDevice(be->device));
@@ -1608,10 +1714,10 @@ extern "C" infr_status infr_hip_prof_read(infr_hip_backend* be, infr_hip_prof_en
     *n_out = n;
     if (out) be->prof.clear();
     return INFR_OK;
-}
+} catch (...) { return guard_fail("infr_hip_prof_read"); }
 
 extern "C" infr_status infr_hip_plan_moe_routing(infr_hip_backend* be, const infr_hip_plan* plan, uint32_t op_index,
-                                                 int32_t* ids, float* weights, float* logits, float* probs) {
+                                                 int32_t* ids, float* weights, float* logits, float* probs) try {
     if (!ok_backend(be) || !ok_plan(plan) || plan->be != be) return fail(INFR_ERR_INVALID, "moe_routing: bad handle");
     if (op_index >= plan->ops.size() || plan->ops[op_index].kind != INFR_OP_MOE_FFN)
         return fail(INFR_ERR_INVALID, "moe_routing: op %u is not a MoeFfn", op_index);
@@ -1627,10 +1733,10 @@ extern "C" infr_status infr_hip_plan_moe_routing(infr_hip_backend* be, const inf
     if (logits) HIP_TRY(hipMemcpy(logits, sc.logits, rows * m.n_expert * 4, hipMemcpyDeviceToHost));
     if (probs) HIP_TRY(hipMemcpy(probs, sc.probs, rows * m.n_expert * 4, hipMemcpyDeviceToHost));
     return INFR_OK;
-}
+} catch (...) { return guard_fail("infr_hip_plan_moe_routing"); }
 
 extern "C" infr_status infr_hip_plan_moe_bucketing(infr_hip_backend* be, const infr_hip_plan* plan, uint32_t op_index,
-                                                   int32_t* offsets, int32_t* pair_src, int32_t* slot_pair) {
+                                                   int32_t* offsets, int32_t* pair_src, int32_t* slot_pair) try {
     if (!ok_backend(be) || !ok_plan(plan) || plan->be != be) return fail(INFR_ERR_INVALID, "moe_bucketing: bad handle");
     if (op_index >= plan->ops.size() || plan->ops[op_index].kind != INFR_OP_MOE_FFN)
         return fail(INFR_ERR_INVALID, "moe_bucketing: op %u is not a MoeFfn", op_index);
@@ -1646,10 +1752,10 @@ extern "C" infr_status infr_hip_plan_moe_bucketing(infr_hip_backend* be, const i
     if (pair_src) HIP_TRY(hipMemcpy(pair_src, sc.pair_src, pairs * 4, hipMemcpyDeviceToHost));
     if (slot_pair) HIP_TRY(hipMemcpy(slot_pair, sc.slot_pair, pairs * 4, hipMemcpyDeviceToHost));
     return INFR_OK;
-}
+} catch (...) { return guard_fail("infr_hip_plan_moe_bucketing"); }
 
 extern "C" infr_status infr_hip_dequant(infr_hip_backend* be, const infr_hip_buffer* src, int32_t dtype, uint64_t numel,
-                                        infr_hip_buffer* dst) {
+                                        infr_hip_buffer* dst) try {
     if (infr_status st = check_owned(be, src, "dequant")) return st;
     if (infr_status st = check_owned(be, dst, "dequant")) return st;
     int e = 1, b = 4;
@@ -1663,4 +1769,4 @@ extern "C" infr_status infr_hip_dequant(infr_hip_backend* be, const infr_hip_buf
     Timed t(be, "dequant");
     infr::launch_dequant(be->stream, (const uint8_t*)src->dptr, dtype, numel, (float*)dst->dptr);
     return INFR_OK;
-}
+} catch (...) { return guard_fail("infr_hip_dequant"); }

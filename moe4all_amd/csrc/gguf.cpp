@@ -15,6 +15,8 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <new>
+#include <stdexcept>
 #include <string>
 #include <string_view>
 #include <unordered_map>
@@ -35,6 +37,23 @@ infr_status fail(infr_status st, const char* fmt, ...) {
     va_end(ap);
     g_err = buf;
     return st;
+}
+
+// No exception crosses the C ABI: the entry points are function-try-blocks whose handler lands here.
+infr_status guard_fail(const char* what) noexcept {
+    try {
+        try {
+            throw;
+        } catch (const std::bad_alloc&) {
+            return fail(INFR_ERR_BACKEND, "%s: out of host memory", what);
+        } catch (const std::exception& e) {
+            return fail(INFR_ERR_BACKEND, "%s: %s", what, e.what());
+        } catch (...) {
+            return fail(INFR_ERR_BACKEND, "%s: unknown exception", what);
+        }
+    } catch (...) {
+        return INFR_ERR_BACKEND;
+    }
 }
 
 constexpr uint32_t kMagic = 0x46554747u;       // "GGUF"
@@ -374,7 +393,7 @@ void fill(const Tensor& t, infr_gguf_tensor* out) {
 
 extern "C" const char* infr_gguf_last_error(void) { return g_err.c_str(); }
 
-extern "C" infr_status infr_gguf_open(const char* path, infr_gguf** out) {
+extern "C" infr_status infr_gguf_open(const char* path, infr_gguf** out) try {
     if (!path || !out) return fail(INFR_ERR_INVALID, "gguf open: null argument");
     *out = nullptr;
     std::string why;
@@ -447,29 +466,29 @@ extern "C" infr_status infr_gguf_open(const char* path, infr_gguf** out) {
     }
     *out = g;
     return INFR_OK;
-}
+} catch (...) { return guard_fail("infr_gguf_open"); }
 
 extern "C" void infr_gguf_close(infr_gguf* g) { delete g; }
 
 extern "C" uint64_t infr_gguf_tensor_count(const infr_gguf* g) { return g ? g->tensors.size() : 0; }
 extern "C" uint32_t infr_gguf_shard_count(const infr_gguf* g) { return g ? (uint32_t)g->shards.size() : 0; }
 
-extern "C" infr_status infr_gguf_tensor_at(const infr_gguf* g, uint64_t index, infr_gguf_tensor* out) {
+extern "C" infr_status infr_gguf_tensor_at(const infr_gguf* g, uint64_t index, infr_gguf_tensor* out) try {
     if (!g || !out) return fail(INFR_ERR_INVALID, "gguf: null argument");
     if (index >= g->tensors.size()) return fail(INFR_ERR_INVALID, "gguf: tensor index %llu out of range", (unsigned long long)index);
     fill(g->tensors[(size_t)index], out);
     return INFR_OK;
-}
+} catch (...) { return guard_fail("infr_gguf_tensor_at"); }
 
-extern "C" infr_status infr_gguf_tensor_find(const infr_gguf* g, const char* name, infr_gguf_tensor* out) {
+extern "C" infr_status infr_gguf_tensor_find(const infr_gguf* g, const char* name, infr_gguf_tensor* out) try {
     if (!g || !name || !out) return fail(INFR_ERR_INVALID, "gguf: null argument");
     auto it = g->by_name.find(name);
     if (it == g->by_name.end()) return fail(INFR_ERR_LOADER, "tensor not found: '%s'", name);
     fill(g->tensors[it->second], out);
     return INFR_OK;
-}
+} catch (...) { return guard_fail("infr_gguf_tensor_find"); }
 
-extern "C" infr_status infr_gguf_tensor_bytes(const infr_gguf* g, const char* name, const void** data, uint64_t* nbytes) {
+extern "C" infr_status infr_gguf_tensor_bytes(const infr_gguf* g, const char* name, const void** data, uint64_t* nbytes) try {
     if (!g || !name || !data) return fail(INFR_ERR_INVALID, "gguf: null argument");
     auto it = g->by_name.find(name);
     if (it == g->by_name.end()) return fail(INFR_ERR_LOADER, "tensor not found: '%s'", name);
@@ -486,56 +505,56 @@ extern "C" infr_status infr_gguf_tensor_bytes(const infr_gguf* g, const char* na
     *data = static_cast<const uint8_t*>(sh.map) + off;
     if (nbytes) *nbytes = t.nbytes;
     return INFR_OK;
-}
+} catch (...) { return guard_fail("infr_gguf_tensor_bytes"); }
 
-extern "C" infr_status infr_gguf_meta_u64(const infr_gguf* g, const char* key, uint64_t* out) {
+extern "C" infr_status infr_gguf_meta_u64(const infr_gguf* g, const char* key, uint64_t* out) try {
     if (!g || !key || !out) return fail(INFR_ERR_INVALID, "gguf: null argument");
     if (!meta_u64(g->meta(), key, out)) return fail(INFR_ERR_INVALID, "gguf: no unsigned metadata value '%s'", key);
     return INFR_OK;
-}
-extern "C" infr_status infr_gguf_meta_i64(const infr_gguf* g, const char* key, int64_t* out) {
+} catch (...) { return guard_fail("infr_gguf_meta_u64"); }
+extern "C" infr_status infr_gguf_meta_i64(const infr_gguf* g, const char* key, int64_t* out) try {
     if (!g || !key || !out) return fail(INFR_ERR_INVALID, "gguf: null argument");
     auto it = g->meta().find(key);
     if (it != g->meta().end() && it->second.kind == Meta::I64) { *out = it->second.i; return INFR_OK; }
     if (it != g->meta().end() && it->second.kind == Meta::U64 && it->second.u <= (uint64_t)INT64_MAX) { *out = (int64_t)it->second.u; return INFR_OK; }
     return fail(INFR_ERR_INVALID, "gguf: no integer metadata value '%s'", key);
-}
-extern "C" infr_status infr_gguf_meta_f64(const infr_gguf* g, const char* key, double* out) {
+} catch (...) { return guard_fail("infr_gguf_meta_i64"); }
+extern "C" infr_status infr_gguf_meta_f64(const infr_gguf* g, const char* key, double* out) try {
     const Meta* m = find_meta(g, key, Meta::F64, "a float");
     if (!m || !out) return INFR_ERR_INVALID;
     *out = m->f;
     return INFR_OK;
-}
-extern "C" infr_status infr_gguf_meta_bool(const infr_gguf* g, const char* key, int32_t* out) {
+} catch (...) { return guard_fail("infr_gguf_meta_f64"); }
+extern "C" infr_status infr_gguf_meta_bool(const infr_gguf* g, const char* key, int32_t* out) try {
     const Meta* m = find_meta(g, key, Meta::BOOL, "a bool");
     if (!m || !out) return INFR_ERR_INVALID;
     *out = (int32_t)m->u;
     return INFR_OK;
-}
-extern "C" infr_status infr_gguf_meta_str(const infr_gguf* g, const char* key, const char** data, uint64_t* len) {
+} catch (...) { return guard_fail("infr_gguf_meta_bool"); }
+extern "C" infr_status infr_gguf_meta_str(const infr_gguf* g, const char* key, const char** data, uint64_t* len) try {
     const Meta* m = find_meta(g, key, Meta::STR, "a string");
     if (!m || !data || !len) return INFR_ERR_INVALID;
     *data = m->s.data();
     *len = m->s.size();
     return INFR_OK;
-}
-extern "C" infr_status infr_gguf_meta_array_len(const infr_gguf* g, const char* key, uint64_t* out) {
+} catch (...) { return guard_fail("infr_gguf_meta_str"); }
+extern "C" infr_status infr_gguf_meta_array_len(const infr_gguf* g, const char* key, uint64_t* out) try {
     const Meta* m = find_meta(g, key, Meta::ARR, "an array");
     if (!m || !out) return INFR_ERR_INVALID;
     *out = m->u;
     return INFR_OK;
-}
+} catch (...) { return guard_fail("infr_gguf_meta_array_len"); }
 
-extern "C" infr_status infr_gguf_block_layout(int32_t dtype, uint32_t* block_elems, uint32_t* block_bytes) {
+extern "C" infr_status infr_gguf_block_layout(int32_t dtype, uint32_t* block_elems, uint32_t* block_bytes) try {
     uint32_t e, b;
     if (!block_layout(dtype, &e, &b)) return fail(INFR_ERR_UNSUPPORTED, "gguf: dtype %d has no block layout", dtype);
     if (block_elems) *block_elems = e;
     if (block_bytes) *block_bytes = b;
     return INFR_OK;
-}
+} catch (...) { return guard_fail("infr_gguf_block_layout"); }
 
 extern "C" infr_status infr_gguf_bind_weight(const infr_gguf* g, const char* name, infr_hip_backend* be,
-                                             infr_hip_buffer** out, int32_t* dtype, uint64_t* numel) {
+                                             infr_hip_buffer** out, int32_t* dtype, uint64_t* numel) try {
     if (!out) return fail(INFR_ERR_INVALID, "gguf bind: null argument");
     *out = nullptr;
     infr_gguf_tensor t;
@@ -554,4 +573,4 @@ extern "C" infr_status infr_gguf_bind_weight(const infr_gguf* g, const char* nam
     if (dtype) *dtype = t.dtype;
     if (numel) *numel = t.numel;
     return INFR_OK;
-}
+} catch (...) { return guard_fail("infr_gguf_bind_weight"); }

@@ -291,6 +291,32 @@ __global__ __launch_bounds__((kLtTile / P) * (kLtTile / P) * 8) void router_logi
         }
 }
 
+// Experts and token rows per block of router_logits_kernel for a shape, or false when even one of each does
+// not fit the LDS budget.
+constexpr size_t kRouterLdsBudget = 140 * 1024;
+static bool router_logits_tile(int rdt, int ne, int rows, int* epb_out, int* rpb_out) {
+    // Decode and small batches of an f32 router: many small blocks of 2 experts x 2 rows, each
+    // staging its operands with one burst of loads.  Otherwise: 8 experts x 4 rows per pass.
+    const bool small = rows <= 2 || (rows < 32 && rdt == INFR_F32 && (ne & 3) == 0 && ne <= 4096);
+    int epb = small ? 2 : 8;
+    int rpb = small ? ((rows < 2 || ne > 2048) ? 1 : 2) : 4;   // the one-burst staging holds 1024 float4 of activations
+    const int nc = ne >> 3;
+    const size_t estride = (size_t)8 * (((nc + 63) & ~63) + 4);
+    auto lds_bytes = [&](int e, int r) { return ((size_t)(e + r) * (estride + 8)) * sizeof(float); };
+    while (lds_bytes(epb, rpb) > kRouterLdsBudget && rpb > 1) rpb >>= 1;
+    while (lds_bytes(epb, rpb) > kRouterLdsBudget && epb > 1) epb >>= 1;
+    if (lds_bytes(epb, rpb) > kRouterLdsBudget) return false;
+    *epb_out = epb;
+    *rpb_out = rpb;
+    return true;
+}
+
+bool router_logits_fits(int rdt, size_t row_bytes, int ne, int rows) {
+    if (rows >= 32 && rdt == INFR_F32 && (ne & 31) == 0 && (row_bytes & 15) == 0) return true;   // the tiled kernel
+    int epb, rpb;
+    return router_logits_tile(rdt, ne, rows, &epb, &rpb);
+}
+
 // The fold needs the one-burst staging of a single row (rows = 1 gives 2 experts x 1 row per block).
 bool router_logits_can_norm(int rdt, size_t row_bytes, int ne, int rows) {
     return rows == 1 && rdt == INFR_F32 && (ne & 3) == 0 && ne >= 4 && ne <= 4096 && (row_bytes & 15) == 0;
@@ -315,18 +341,13 @@ bool launch_router_logits(hipStream_t s, const uint8_t* router, int rdt, size_t 
         }
         return true;
     }
-    // Decode and small batches of an f32 router: many small blocks of 2 experts x 2 rows, each
-    // staging its operands with one burst of loads.  Otherwise: 8 experts x 4 rows per pass.
+    int epb = 0, rpb = 0;
+    if (!router_logits_tile(rdt, ne, rows, &epb, &rpb)) return false;
     const bool small = rows <= 2 || (rows < 32 && rdt == INFR_F32 && (ne & 3) == 0 && ne <= 4096);
-    int epb = small ? 2 : 8;
-    int rpb = small ? ((rows < 2 || ne > 2048) ? 1 : 2) : 4;   // the one-burst staging holds 1024 float4 of activations
-    const size_t budget = 140 * 1024;
+    const size_t budget = kRouterLdsBudget;
     const int nc = ne >> 3;
     const size_t estride = (size_t)8 * (((nc + 63) & ~63) + 4);
     auto lds_bytes = [&](int e, int r) { return ((size_t)(e + r) * (estride + 8)) * sizeof(float); };
-    while (lds_bytes(epb, rpb) > budget && rpb > 1) rpb >>= 1;
-    while (lds_bytes(epb, rpb) > budget && epb > 1) epb >>= 1;
-    if (lds_bytes(epb, rpb) > budget) return false;
     size_t lds = lds_bytes(epb, rpb);
     int gx = (n_expert + epb - 1) / epb;
     int passes = (rows + rpb - 1) / rpb;

@@ -33,6 +33,8 @@ struct RouterNorm {
     float* xn_out = nullptr;         // [ne], not x
 };
 bool router_logits_can_norm(int rdt, size_t row_bytes, int ne, int rows);
+// False when launch_router_logits would refuse the shape (its staging does not fit the LDS): asked at compile time.
+bool router_logits_fits(int rdt, size_t row_bytes, int ne, int rows);
 // Router logits with the reference's dot order (8 FMA lanes, lanes summed 0..7).
 // logits[rows, n_expert]; router rows are `row_bytes` apart, decoded as `rdt`.
 // Returns false when the shape does not fit the kernel's LDS budget (or the fold of `norm`).

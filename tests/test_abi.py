@@ -107,3 +107,15 @@ def test_null_and_foreign_handles_are_errors():
     lib.infr_hip_buffer_free(None)
     lib.infr_hip_plan_free(None)
     lib.infr_hip_destroy(None)
+
+
+def test_every_status_returning_entry_point_catches_exceptions():
+    """No exception may cross the C ABI (the header promises it): every extern "C" function that returns a status is a
+    function-try-block in the sources, and the void ones that free objects swallow what their bodies throw."""
+    for name in ("backend.cpp", "gguf.cpp"):
+        src = open(os.path.join(ROOT, "moe4all_amd", "csrc", name)).read()
+        heads = re.findall(r'^extern "C" infr_status (\w+)\((?:[^;{]|\n)*?\)\s*(try)?\s*\{', src, flags=re.M)
+        assert len(heads) >= 10
+        missing = [n for n, t in heads if not t]
+        assert not missing, f"{name}: {missing} can let an exception escape"
+        assert src.count("catch (...) { return guard_fail(") >= len(heads)

@@ -3,6 +3,7 @@ seeded inputs and against the committed golden fixtures.
 
 Bars: bit-exact for decoded weights, router logits, probabilities, expert ids and routing
 weights; layer outputs within max-abs 2e-3 and relative L2 1e-3 (f32 accumulation)."""
+import ctypes as C
 import os
 
 import numpy as np
@@ -12,6 +13,7 @@ import helpers as H
 import moe4all_amd as M
 import oracle as O
 from moe4all_amd import DType, TensorDesc
+from moe4all_amd import backend as B
 
 pytestmark = pytest.mark.gpu
 GOLD = os.path.join(os.path.dirname(__file__), "golden")
@@ -292,6 +294,34 @@ def test_moe_ffn_option_variants_match_oracle(be, gdt, ddt, rows):
     check(dict(with_down_scale=True, scale=1.7), dict(down_scale=ds, scale=1.7), dict(down_scale=ds))
     check(dict(swiglu_clamp=0.05, act=M.Activation.Gelu), dict(swiglu_clamp=0.05, act=O.ACT_GELU))
     check(dict(fused_gate_up=True), dict(fused_gate_up=True), fused=True)
+
+
+def test_buffers_and_plans_may_outlive_their_backend():
+    """infr_hip_destroy first, frees afterwards: the reference's buffers keep their device alive, so this order is legal.
+    Every other call with the destroyed handle is refused with a status."""
+    be2 = M.Backend(0)
+    buf = be2.alloc(4096)
+    g, ids = moe_graph(1, 256, 4, 2, 256, DType.Q4K, DType.Q4K)
+    plan = be2.compile(g)
+    handle = be2._h
+    be2.close()
+    lib = M.load_library()
+    out = C.c_void_p()
+    assert lib.infr_hip_alloc(handle, 16, 1, C.byref(out)) != 0 and b"bad handle" in lib.infr_hip_last_error()
+    assert lib.infr_hip_upload(handle, buf._h, (C.c_char * 4)(), 4) != 0
+    plan.free()
+    buf.free()
+
+
+def test_no_exception_crosses_the_abi(be):
+    """A graph whose op count cannot be allocated: std::bad_alloc inside infr_hip_compile comes back as a status."""
+    gr = B._Graph()
+    op = B._Op(kind=3)
+    gr.ops, gr.n_ops = C.pointer(op), 0xFFFFFFFF
+    out = C.c_void_p()
+    st = M.load_library().infr_hip_compile(be._h, C.byref(gr), C.byref(out))
+    assert st == 1 and not out.value, st
+    assert b"infr_hip_compile" in M.load_library().infr_hip_last_error()
 
 
 def test_execute_is_repeatable_and_rebinding_works(be):
