@@ -1,14 +1,19 @@
 #!/usr/bin/env python3
-"""Decode benchmark of the routed-expert MoE FFN path on one MI355X.
+"""Benchmark of the routed-expert MoE FFN path on one MI355X.
 
-A step is one decode token through every MoE layer of the workload (one execute of a graph
-with one Op::MoeFfn per layer, each with its own HBM-resident weights and its own N(0,1)
-activation row).  Default workload: the Qwen3-30B-A3B-shaped stack (48 layers, hidden 2048,
-128 experts, top-8, intermediate 768, Q4_K gate/up + Q6_K down), synthetic seeded weights.
+A step is one pass of a workload's batch through every MoE layer of the workload: one execute of a graph with
+one Op::MoeFfn per layer (plus the shared-expert ops where the shape has one), each layer with its own
+HBM-resident weights and its own N(0,1) activation rows.  Headline workload: the Qwen3-30B-A3B-shaped stack
+(48 layers, hidden 2048, 128 experts, top-8, intermediate 768, Q4_K gate/up + Q6_K down), decode batch 1,
+synthetic seeded weights.
 
-Prints ONE JSON line: whole-job decode tok/s, the roofline of the dominant kernel measured
-live with HIP events on the backend's stream, and a CPU baseline (the oracle, a C restatement
-of the reference's CPU path, timed on this host's cores on a bounded sample).
+Prints ONE JSON line: whole-job decode tok/s of the headline workload, the roofline of its dominant kernel
+measured live with HIP events attached to each dispatch on the backend's stream, the time a chain of dependent
+plain reads of the same sizes takes on this device (what a kernel chain of this shape cannot go below), and a
+CPU baseline (the oracle, a scalar C restatement of the reference's CPU path, timed on this host's cores on a
+bounded sample).  With no --config the same line carries a "configs" array with the other benchmark
+configurations (single Q8_0 layer, multi-stream decode, prefill chunks, the large shape with a shared expert),
+each measured the same way on fewer steps.
 """
 from __future__ import annotations
 
@@ -30,16 +35,44 @@ HBM_PEAK_GBPS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0   # dense fp16/bf16 matrix-core peak of one MI355X
 SEED0 = 20260101
 N_TOKENS = 16  # distinct activation sets rotated through the steps
+TRAFFIC_FILE = os.path.join("profiles", "hbm_traffic.json")
 
 
-def build_stack(be, shape, n_layer, batch, sublayer=False):
-    """One graph with n_layer MoeFfn ops (+ shared-expert ops), weights generated in HBM.  With
-    `sublayer` every layer is the model's whole FFN sublayer: y = x + ffn(rmsnorm(x) * w)."""
+def shape_of(config, tokens):
+    return {"c1": synth.CONFIG_1, "c2": synth.CONFIG_2, "c5": synth.CONFIG_5, "mxfp4": synth.CONFIG_MXFP4,
+            "c4": synth.MoeShape(f"c4-prefill-{tokens}-zipf1.1-q8_0", 1, 2048, 128, 8, 768, DType.Q8_0, DType.Q8_0),
+            "c4k": synth.MoeShape(f"c4-prefill-{tokens}-zipf1.1-q4k-q6k", 1, 2048, 128, 8, 768, DType.Q4K, DType.Q6K)}[config]
+
+
+class Stack:
+    """The resident weights of a workload's layers, generated in HBM, shared by every batch size measured on them."""
+
+    def __init__(self, be, shape, n_layer, prefill):
+        self.be, self.shape, self.n_layer, self.prefill = be, shape, n_layer, prefill
+        t0 = time.time()
+        self.layers = [synth.LayerWeights(be, shape, SEED0, l, on_device=True) for l in range(n_layer)]
+        if prefill:
+            # skewed expert popularity through the op's own inputs: x[:, 0] = 1, router[e, 0] = ln Zipf(1.1)
+            for lw in self.layers:
+                router = be.download(lw.router, dtype=np.float32).reshape(shape.n_expert, shape.ne).copy()
+                router[:, 0] = synth.zipf_bias(shape.n_expert, 1.1, SEED0)
+                be.upload(lw.router, router)
+        be.sync()
+        self.setup_s = time.time() - t0
+
+    def free(self):
+        for lw in self.layers:
+            lw.free()
+        self.layers = []
+
+
+def build_graph(stack, batch, sublayer=False):
+    """One graph with n_layer MoeFfn ops (+ shared-expert ops).  With `sublayer` every layer is the model's whole FFN
+    sublayer: y = x + ffn(rmsnorm(x) * w)."""
+    shape = stack.shape
     g = M.Graph()
-    layers, ids = [], []
-    for l in range(n_layer):
-        lw = synth.LayerWeights(be, shape, SEED0, l, on_device=True)
-        layers.append(lw)
+    ids = []
+    for _ in range(stack.n_layer):
         x = x_raw = g.input(TensorDesc([batch, shape.ne], DType.F32))
         out = g.output(TensorDesc([batch, shape.ne], DType.F32))
         norm_w = None
@@ -75,58 +108,53 @@ def build_stack(be, shape, n_layer, batch, sublayer=False):
         if sublayer:
             g.add(a=x_raw, b=dst, dst=out, n=batch * shape.ne)
         ids.append(d)
-    return g, layers, ids
+    return g, ids
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
-    ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--config", default="c2", choices=["c1", "c2", "c4", "c4k", "c5", "mxfp4"],
-                    help="c1/c2/c5: decode stacks (use --batch for multi-stream decode); c4: one config-1 layer "
-                         "(Q8_0), prefill chunk of --tokens with Zipf(1.1) expert popularity; c4k: same with "
-                         "Q4_K gate/up + Q6_K down; mxfp4: a decode stack of the gpt-oss-120b expert shape with MXFP4 banks "
-                         "(the 32-element-unit kernels; use --batch >= 32 for the unit-decoder grouped GEMM)")
-    ap.add_argument("--tokens", type=int, default=2048, help="prefill chunk size for c4/c4k")
-    ap.add_argument("--layers", type=int, default=0, help="override the layer count (0 = the config's)")
-    ap.add_argument("--batch", type=int, default=1)
-    ap.add_argument("--sublayer", action="store_true",
-                    help="time the model's whole FFN sublayer per layer (RmsNorm -> MoeFfn [+ shared expert] -> "
-                         "residual Add) instead of the MoeFfn op alone; not the headline metric")
-    ap.add_argument("--no-fusion", action="store_true", help="one launch per op (infr_hip_config.disable_op_fusion)")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--no-kernel-timing", action="store_true")
-    ap.add_argument("--copy-probe-mib", type=int, default=0,
-                    help="also run one plain device-to-device copy of this many MiB (a known-size kernel that "
-                         "calibrates hardware byte counters in a profiler run)")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py: this build runs on ONE GPU; --gpus must be 1 (no multi-GPU path exists in this tree)",
-              file=sys.stderr)
-        sys.exit(2)
+def algorithmic_tables(shape, batch, distinct, prefill):
+    """Algorithmic HBM bytes and FLOPs per launch of each kernel name the backend's profiler reports."""
+    gate_b = M.backend.bytes_for(shape.gate_dtype, shape.n_ff * shape.ne)
+    down_b = M.backend.bytes_for(shape.down_dtype, shape.ne * shape.n_ff)
+    n_sel = distinct if batch > 1 else shape.n_used
+    pairs = batch * shape.n_used
+    alg = {
+        "router_logits": shape.router_bytes() + batch * shape.ne * 4 + batch * shape.n_expert * 4,
+        "moe_gate_up": n_sel * 2 * gate_b + batch * shape.ne * 4 + pairs * shape.n_ff * 4,
+        "moe_down_combine": n_sel * down_b + pairs * shape.n_ff * 4 + batch * shape.ne * 4,
+    }
+    # the decode kernel that routes its own token row also reads that row's logits
+    alg["moe_route_gate_up"] = alg["moe_gate_up"] + batch * shape.n_expert * 4
+    # banks on the 32-element-unit kernels: per-pair down results, then the rank-ordered sum as its own launch
+    alg["moe_gate_up_units"], alg["moe_route_gate_up_units"] = alg["moe_gate_up"], alg["moe_route_gate_up"]
+    alg["moe_down_units"] = n_sel * down_b + pairs * shape.n_ff * 4 + pairs * shape.ne * 4
+    alg["moe_down_combine_units"] = alg["moe_down_combine"]
+    alg["moe_gate_up_bucketed"] = alg["moe_gate_up"]
+    if not prefill and batch < 32:
+        alg["moe_unbucket_combine"] = pairs * shape.ne * 4 + batch * shape.ne * 4
+    alg["rms_norm_router_logits"] = alg["router_logits"] + shape.ne * 4 + batch * shape.ne * 4
+    if shape.shared_ff:
+        sh_gate_b = M.backend.bytes_for(shape.gate_dtype, shape.shared_ff * shape.ne)
+        sh_down_b = M.backend.bytes_for(shape.down_dtype, shape.ne * shape.shared_ff)
+        # the always-on expert as one more slot of the routed kernels
+        alg["moe_route_gate_up_shared"] = alg["moe_route_gate_up"] + 2 * sh_gate_b + batch * shape.shared_ff * 4
+        alg["moe_down_combine_shared"] = alg["moe_down_combine"] + sh_down_b + batch * shape.shared_ff * 4
+        alg["linear_gate_up_act"] = 2 * sh_gate_b + batch * shape.ne * 4 + batch * shape.shared_ff * 4
+        alg["linear_add"] = sh_down_b + batch * shape.shared_ff * 4 + 2 * batch * shape.ne * 4
+    flops = {  # 2 per multiply-add
+        "moe_grouped_gate_up": 2.0 * pairs * 2 * shape.n_ff * shape.ne,
+        "moe_grouped_down": 2.0 * pairs * shape.ne * shape.n_ff,
+    }
+    flops["moe_grouped_units_gate_up"], flops["moe_grouped_units_down"] = flops["moe_grouped_gate_up"], flops["moe_grouped_down"]
+    return alg, flops
 
-    if args.sublayer:
-        args.no_cpu_baseline = True   # the CPU sample times Op::MoeFfn alone
-    prefill = args.config in ("c4", "c4k")
-    shape = {"c1": synth.CONFIG_1, "c2": synth.CONFIG_2, "c5": synth.CONFIG_5, "mxfp4": synth.CONFIG_MXFP4,
-             "c4": synth.MoeShape(f"c4-prefill-{args.tokens}-zipf1.1-q8_0", 1, 2048, 128, 8, 768, DType.Q8_0, DType.Q8_0),
-             "c4k": synth.MoeShape(f"c4-prefill-{args.tokens}-zipf1.1-q4k-q6k", 1, 2048, 128, 8, 768, DType.Q4K,
-                                   DType.Q6K)}[args.config]
-    n_layer = args.layers or shape.n_layer
-    batch = args.tokens if prefill else args.batch
-    be = M.Backend(0, disable_op_fusion=args.no_fusion)
-    caps = be.capabilities()
-    t_setup = time.time()
-    g, layers, ids = build_stack(be, shape, n_layer, batch, args.sublayer)
-    norm_w = be.buffer_from(np.ones(shape.ne, np.float32)) if args.sublayer else None
+
+def measure(be, stack, config, batch, steps, warmup, *, sublayer=False, kernel_timing=True, cpu_budget_s=12.0, floor=True,
+            no_fusion=False):
+    """One workload on resident weights: the timed steps, per-kernel durations, the dependent-read floor, the CPU baseline."""
+    shape, n_layer, prefill = stack.shape, stack.n_layer, stack.prefill
+    g, ids = build_graph(stack, batch, sublayer)
+    norm_w = be.buffer_from(np.ones(shape.ne, np.float32)) if sublayer else None
     plan = be.compile(g)
-    if prefill:
-        # skewed expert popularity through the op's own inputs: x[:, 0] = 1, router[e, 0] = ln Zipf(1.1)
-        for lw in layers:
-            router = be.download(lw.router, dtype=np.float32).reshape(shape.n_expert, shape.ne).copy()
-            router[:, 0] = synth.zipf_bias(shape.n_expert, 1.1, SEED0)
-            be.upload(lw.router, router)
     # activations: N_TOKENS independent sets of per-layer N(0,1) rows, resident in HBM
     xbufs = []
     for t in range(N_TOKENS):
@@ -146,7 +174,7 @@ def main():
     for t in range(N_TOKENS):
         b = M.Bindings()
         for l in range(n_layer):
-            d, lw = ids[l], layers[l]
+            d, lw = ids[l], stack.layers[l]
             b.bind(d["x"], xbufs[t][l]).bind(d["router"], lw.router).bind(d["gate"], lw.gate)
             b.bind(d["up"], lw.up).bind(d["down"], lw.down).bind(d["dst"], ybufs[l])
             if shape.shared_ff:
@@ -154,75 +182,45 @@ def main():
             if norm_w is not None:
                 b.bind(d["norm_w"], norm_w)
         binds.append(b)
-    if args.copy_probe_mib:
-        n = args.copy_probe_mib << 20
-        src, dst = be.alloc(n), be.alloc(n)
-        be.copy_buffer(src, dst, n)
-        be.sync()
-        src.free()
-        dst.free()
     be.sync()
-    setup_s = time.time() - t_setup
 
-    for i in range(args.warmup):
+    for i in range(warmup):
         be.execute(plan, binds[i % N_TOKENS])
     be.sync()
     t0 = time.perf_counter()
-    for i in range(args.steps):
+    for i in range(steps):
         be.execute(plan, binds[i % N_TOKENS])
     be.sync()
     elapsed = time.perf_counter() - t0
-    ms_per_step = elapsed * 1e3 / args.steps
-    tok_s = batch * args.steps / elapsed
+    ms_per_step = elapsed * 1e3 / steps
+    tok_s = batch * steps / elapsed
+    # spread: the same steps again in ten groups, each bracketed by a sync
+    groups = max(1, min(10, steps))
+    per_group = max(1, steps // groups)
+    group_ms = []
+    for gi in range(groups):
+        t1 = time.perf_counter()
+        for i in range(per_group):
+            be.execute(plan, binds[(gi * per_group + i) % N_TOKENS])
+        be.sync()
+        group_ms.append((time.perf_counter() - t1) * 1e3 / per_group)
 
     # distinct experts actually selected per layer (batch > 1 shares experts between tokens)
-    r = be.moe_routing(plan, 1 if args.sublayer else 0)
+    r = be.moe_routing(plan, 1 if sublayer else 0)
     distinct = len(set(r["idx"].ravel().tolist()))
     layer_bytes = shape.algorithmic_bytes(batch, distinct if batch > 1 else None)
     layer_gbps = layer_bytes * n_layer / (ms_per_step * 1e-3) / 1e9
 
-    # ---- per-kernel durations, HIP events on the backend's own stream, separate pass
-    roofline = None
-    kernels = {}
-    if not args.no_kernel_timing:
+    # ---- per-kernel durations: HIP events attached to each kernel's own dispatch on the backend's stream, separate pass
+    roofline, kernels = None, {}
+    alg, flops = algorithmic_tables(shape, batch, distinct, prefill)
+    if kernel_timing:
         be.prof_enable(True)
-        ksteps = max(1, min(args.steps, 50))
-        for i in range(ksteps):
+        for i in range(max(1, min(steps, 50))):
             be.execute(plan, binds[i % N_TOKENS])
         be.sync()
         prof = be.prof_read()
         be.prof_enable(False)
-        gate_b = M.backend.bytes_for(shape.gate_dtype, shape.n_ff * shape.ne)
-        down_b = M.backend.bytes_for(shape.down_dtype, shape.ne * shape.n_ff)
-        n_sel = distinct if batch > 1 else shape.n_used
-        pairs = batch * shape.n_used
-        alg = {  # algorithmic HBM bytes per launch
-            "router_logits": shape.router_bytes() + batch * shape.ne * 4 + batch * shape.n_expert * 4,
-            "moe_gate_up": n_sel * 2 * gate_b + batch * shape.ne * 4 + pairs * shape.n_ff * 4,
-            "moe_down_combine": n_sel * down_b + pairs * shape.n_ff * 4 + batch * shape.ne * 4,
-        }
-        # the decode kernel that routes its own token row also reads that row's logits
-        alg["moe_route_gate_up"] = alg["moe_gate_up"] + batch * shape.n_expert * 4
-        # banks on the 32-element-unit kernels: per-pair down results, then the rank-ordered sum as its own launch
-        alg["moe_gate_up_units"], alg["moe_route_gate_up_units"] = alg["moe_gate_up"], alg["moe_route_gate_up"]
-        alg["moe_down_units"] = n_sel * down_b + pairs * shape.n_ff * 4 + pairs * shape.ne * 4
-        alg["moe_down_combine_units"] = alg["moe_down_combine"]
-        if not prefill and batch < 32:
-            alg["moe_unbucket_combine"] = pairs * shape.ne * 4 + batch * shape.ne * 4
-        alg["rms_norm_router_logits"] = alg["router_logits"] + shape.ne * 4 + batch * shape.ne * 4
-        if shape.shared_ff:
-            sh_gate_b = M.backend.bytes_for(shape.gate_dtype, shape.shared_ff * shape.ne)
-            sh_down_b = M.backend.bytes_for(shape.down_dtype, shape.ne * shape.shared_ff)
-            # the always-on expert as one more slot of the routed kernels
-            alg["moe_route_gate_up_shared"] = alg["moe_route_gate_up"] + 2 * sh_gate_b + batch * shape.shared_ff * 4
-            alg["moe_down_combine_shared"] = alg["moe_down_combine"] + sh_down_b + batch * shape.shared_ff * 4
-            alg["linear_gate_up_act"] = 2 * sh_gate_b + batch * shape.ne * 4 + batch * shape.shared_ff * 4
-            alg["linear_add"] = sh_down_b + batch * shape.shared_ff * 4 + 2 * batch * shape.ne * 4
-        flops = {  # algorithmic FLOPs per launch of the grouped GEMMs (2 per multiply-add)
-            "moe_grouped_gate_up": 2.0 * pairs * 2 * shape.n_ff * shape.ne,
-            "moe_grouped_down": 2.0 * pairs * shape.ne * shape.n_ff,
-        }
-        flops["moe_grouped_units_gate_up"], flops["moe_grouped_units_down"] = flops["moe_grouped_gate_up"], flops["moe_grouped_down"]
         for name, p in prof.items():
             avg_us = p["total_ms"] * 1e3 / max(p["launches"], 1)
             kernels[name] = {"launches": int(p["launches"]), "avg_us": round(avg_us, 3), "min_us": round(p["min_ms"] * 1e3, 3)}
@@ -235,41 +233,66 @@ def main():
         total_us = lambda k: kernels[k]["avg_us"] * kernels[k]["launches"]
         cand = [k for k in kernels if k in flops] or [k for k in kernels if "alg_bytes" in kernels[k]]
         dom = max(cand, key=total_us, default=None)
-        # HBM bytes per launch measured with hardware counters in a separate profiler run of this same
-        # command (profiles/), reported only for the workload they were taken on
-        traffic = None
+        # HBM bytes per launch from hardware counters: taken in separate profiler runs of this same command and kept in
+        # profiles/ (the counters cannot be read from inside this process); reported only for the workload they cover
+        traffic, traffic_source = None, None
         if dom:
             try:
-                with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
-                    if n_layer == shape.n_layer and not args.sublayer and not args.no_fusion:
-                        key = f"{args.config}/tokens{batch}" if prefill else f"{args.config}/batch{batch}"
+                with open(os.path.join(ROOT, TRAFFIC_FILE)) as f:
+                    if n_layer == shape.n_layer and not sublayer and not no_fusion:
+                        key = f"{config}/tokens{batch}" if prefill else f"{config}/batch{batch}"
                         traffic = json.load(f).get(key, {}).get(dom)
+                        traffic_source = TRAFFIC_FILE if traffic is not None else None
             except OSError:
                 pass
         if dom and dom in flops:
             ach = flops[dom] / (kernels[dom]["avg_us"] * 1e-6) / 1e12
             roofline = {"bound": "mfma", "kernel": dom, "achieved": round(ach, 1), "peak": MFMA_F16_PEAK_TFLOPS,
                         "unit": "TFLOP/s", "frac": round(ach / MFMA_F16_PEAK_TFLOPS, 4), "traffic": traffic,
+                        "traffic_source": traffic_source,
                         "alg_flops_per_launch": flops[dom], "avg_launch_us": kernels[dom]["avg_us"]}
         elif dom:
             ach = alg[dom] / (kernels[dom]["avg_us"] * 1e-6) / 1e9
             roofline = {"bound": "hbm", "kernel": dom, "achieved": round(ach, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                        "frac": round(ach / HBM_PEAK_GBPS, 4), "traffic": traffic,
+                        "frac": round(ach / HBM_PEAK_GBPS, 4), "traffic": traffic, "traffic_source": traffic_source,
                         "alg_bytes_per_launch": alg[dom], "avg_launch_us": kernels[dom]["avg_us"]}
+
+    # ---- what a chain of dependent kernels of these sizes cannot go below: plain reads, no arithmetic, the window of
+    # each stage chosen by a word the stage before wrote (decode workloads; stage sizes = the kernels' algorithmic bytes)
+    floor_out = None
+    if floor and kernels and not prefill and roofline and roofline["bound"] == "hbm":
+        chain = [k for k in kernels if "alg_bytes" in kernels[k]]
+        order = {"router_logits": 0, "rms_norm_router_logits": 0, "route_topk": 1}
+        chain.sort(key=lambda k: (order.get(k, 2 if "gate_up" in k else 3), k))
+        sizes = [max(1024, int(kernels[k]["alg_bytes"])) for k in chain]
+        pool = be.alloc_uninit(2 << 30)
+        try:
+            pr = be.probe_dependent_reads(pool, sizes, 200)
+        finally:
+            pool.free()
+        floor_out = {"kernels": chain, "stage_bytes": sizes, "stage_us": [round(v, 3) for v in pr["stage_us"]],
+                     "chain_us": round(pr["chain_us"], 3),
+                     "achievable_frac_of_hbm_peak": round(sum(sizes) / (pr["chain_us"] * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4),
+                     "note": "dependent kernels that only read these byte counts (all loads of a block in flight at once)"}
+        dom = roofline["kernel"]
+        if dom in chain:
+            st = pr["stage_us"][chain.index(dom)]
+            roofline["floor_launch_us"] = round(st, 3)
+            roofline["achievable_frac"] = round(kernels[dom]["alg_bytes"] / (st * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)
 
     # ---- CPU baseline: the oracle on this host's cores, layer 0's weights, a bounded sample
     cpu = None
-    if not args.no_cpu_baseline:
+    if cpu_budget_s > 0:
         import oracle as O
-        lw = layers[0]
+        lw = stack.layers[0]
         router = be.download(lw.router, dtype=np.float32)
         gate, up, down = be.download(lw.gate), be.download(lw.up), be.download(lw.down)
         threads = O.hw_threads()
-        n_sample, spent, budget_s = 0, 0.0, 12.0
+        n_sample, spent = 0, 0.0
         cpu_rows = min(batch, 256)   # a prefill chunk is sampled by its first 256 tokens
         # the int8 batch numerics exist for the formats with an integer dot on the CPU (Q8_0, Q4_K, Q6_K)
         production = cpu_rows >= 2 and {shape.gate_dtype, shape.down_dtype} <= {DType.Q8_0, DType.Q4K, DType.Q6K}
-        while spent < budget_s and n_sample < 4 * n_layer:
+        while spent < cpu_budget_s and n_sample < 4 * max(n_layer, 12):
             x = synth.normal(synth.stream_seed(SEED0 + 1, n_sample, synth.ROLE_X), batch * shape.ne, 1.0)
             x = x.reshape(batch, shape.ne)[:cpu_rows].copy()
             if prefill:
@@ -284,21 +307,25 @@ def main():
             n_sample += 1
         per_layer_s = spent / n_sample
         cpu = {"value": round(cpu_rows / (per_layer_s * n_layer), 3), "unit": "tok/s", "cores": threads, "kind": "port",
-               "sample": f"{n_sample} layer-passes of layer 0 (routed experts only, {cpu_rows} token rows each) with distinct seeded tokens, "
+               "sample": f"scalar, auto-vectorised C restatement of the reference's CPU path (not its hand-written AVX2 / AVX-512 / "
+                         f"VNNI tiers: a floor for what the reference's CPU backend would do); {n_sample} layer-passes of layer 0 "
+                         f"(routed experts only, {cpu_rows} token rows each) with distinct seeded tokens, "
                          f"{per_layer_s * 1e3:.2f} ms per layer-pass, "
                          f"{'production numerics (int8 activations, scalar integer dots)' if production else 'f32 numerics (dequantise a row, f32 dot)'}, "
                          f"scaled to {n_layer} layers",
                "ms_per_layer": round(per_layer_s * 1e3, 3)}
 
     out = {
-        "metric": "MoE prefill tok/s" if prefill else "MoE decode tok/s", "value": round(tok_s, 2), "unit": "tok/s", "n_gpus": 1, "steps": args.steps,
-        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None,
+        "metric": "MoE prefill tok/s" if prefill else "MoE decode tok/s", "value": round(tok_s, 2), "unit": "tok/s", "n_gpus": 1,
+        "steps": steps, "warmup": warmup, "ms_per_step": round(ms_per_step, 4),
+        "ms_per_step_min": round(min(group_ms), 4), "ms_per_step_max": round(max(group_ms), 4),
+        "spread": f"min / max over {groups} groups of {per_group} steps run after the timed region, a sync after each group",
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         # decode: exact integer dots on 23-bit fixed-point activations, scales and sums in f32; batched path: f16
         # operands on the matrix cores with f32 accumulation
         "dtype": "f16" if batch >= 32 else "f32", "data": "synthetic",
         "config": {"workload": (shape.name if n_layer == shape.n_layer else f"{shape.name}[{n_layer} layers]") +
-                               ("+rmsnorm+residual" if args.sublayer else "") + ("/unfused" if args.no_fusion else ""),
+                               ("+rmsnorm+residual" if sublayer else "") + ("/unfused" if no_fusion else ""),
                    "layers": n_layer, "hidden": shape.ne, "experts": shape.n_expert, "top_k": shape.n_used,
                    "intermediate": shape.n_ff, "gate_up": shape.gate_dtype.name, "down": shape.down_dtype.name,
                    "shared_intermediate": shape.shared_ff, "batch": batch, "parallelism": "single-gpu",
@@ -306,9 +333,104 @@ def main():
         "layer": {"us_per_layer": round(ms_per_step * 1e3 / n_layer, 3), "alg_bytes_per_layer": layer_bytes,
                   "achieved_GBps": round(layer_gbps, 1), "frac_of_hbm_peak": round(layer_gbps / HBM_PEAK_GBPS, 4),
                   "distinct_experts_layer0": distinct},
-        "roofline": roofline, "kernels": kernels, "cpu_baseline": cpu,
-        "device": caps["name"], "compute_units": caps["compute_units"], "setup_s": round(setup_s, 1),
+        "roofline": roofline, "floor": floor_out, "kernels": kernels, "cpu_baseline": cpu,
     }
+    plan.free()
+    for row in xbufs:
+        for xb in row:
+            xb.free()
+    for yb in ybufs:
+        yb.free()
+    if norm_w is not None:
+        norm_w.free()
+    return out
+
+
+# the other benchmark configurations, measured after the headline when no --config is given:
+# (config, layers (0 = the shape's), batches or chunk sizes)
+OTHER_WORKLOADS = (("c1", 0, (1, 4, 16)), ("c4", 0, (512, 2048)), ("c4k", 0, (512, 2048)), ("c5", 0, (1, 8)))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--config", default=None, choices=["c1", "c2", "c4", "c4k", "c5", "mxfp4"],
+                    help="one workload only.  c1/c2/c5: decode stacks (use --batch for multi-stream decode); c4: one config-1 layer "
+                         "(Q8_0), prefill chunk of --tokens with Zipf(1.1) expert popularity; c4k: same with "
+                         "Q4_K gate/up + Q6_K down; mxfp4: a decode stack of the gpt-oss-120b expert shape with MXFP4 banks "
+                         "(the 32-element-unit kernels; use --batch >= 32 for the unit-decoder grouped GEMM).  Default: c2 as the "
+                         "headline plus every other benchmark configuration in a \"configs\" array")
+    ap.add_argument("--headline-only", action="store_true", help="with no --config: skip the \"configs\" array")
+    ap.add_argument("--tokens", type=int, default=2048, help="prefill chunk size for c4/c4k")
+    ap.add_argument("--layers", type=int, default=0, help="override the layer count (0 = the config's)")
+    ap.add_argument("--batch", type=int, default=1)
+    ap.add_argument("--sublayer", action="store_true",
+                    help="time the model's whole FFN sublayer per layer (RmsNorm -> MoeFfn [+ shared expert] -> "
+                         "residual Add) instead of the MoeFfn op alone; not the headline metric")
+    ap.add_argument("--no-fusion", action="store_true", help="one launch per op (infr_hip_config.disable_op_fusion)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-kernel-timing", action="store_true")
+    ap.add_argument("--no-floor", action="store_true", help="skip the dependent-read probe")
+    ap.add_argument("--copy-probe-mib", type=int, default=0,
+                    help="also run one plain device-to-device copy of this many MiB (a known-size kernel that "
+                         "calibrates hardware byte counters in a profiler run)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; --gpus must be 1 (no multi-GPU path exists in this tree)",
+              file=sys.stderr)
+        sys.exit(2)
+
+    headline_cfg = args.config or "c2"
+    prefill = headline_cfg in ("c4", "c4k")
+    shape = shape_of(headline_cfg, args.tokens)
+    n_layer = args.layers or shape.n_layer
+    batch = args.tokens if prefill else args.batch
+    be = M.Backend(0, disable_op_fusion=args.no_fusion)
+    caps = be.capabilities()
+    stack = Stack(be, shape, n_layer, prefill)
+    if args.copy_probe_mib:
+        n = args.copy_probe_mib << 20
+        src, dst = be.alloc(n), be.alloc(n)
+        be.copy_buffer(src, dst, n)
+        be.sync()
+        src.free()
+        dst.free()
+    out = measure(be, stack, headline_cfg, batch, args.steps, args.warmup, sublayer=args.sublayer,
+                  kernel_timing=not args.no_kernel_timing,
+                  cpu_budget_s=0.0 if (args.no_cpu_baseline or args.sublayer) else 12.0,   # the CPU sample times Op::MoeFfn alone
+                  floor=not args.no_floor, no_fusion=args.no_fusion)
+    out["device"], out["compute_units"], out["setup_s"] = caps["name"], caps["compute_units"], round(stack.setup_s, 1)
+    stack.free()
+
+    if args.config is None and not args.headline_only:
+        configs = []
+        for cfg, layers, sizes in OTHER_WORKLOADS:
+            pf = cfg in ("c4", "c4k")
+            stacks = {}
+            for size in sizes:
+                sh = shape_of(cfg, size)
+                key = 0 if not pf else size    # a prefill shape's name carries its chunk size; the weights are the same
+                if key not in stacks:
+                    if pf and stacks:
+                        st = next(iter(stacks.values()))
+                        st.shape = sh
+                        stacks[key] = st
+                    else:
+                        stacks[key] = Stack(be, sh, layers or sh.n_layer, pf)
+                st = stacks[key]
+                steps = max(5, min(args.steps, 40 if st.n_layer > 1 else 100))
+                res = measure(be, st, cfg, size, steps, min(args.warmup, 5), cpu_budget_s=0.0 if args.no_cpu_baseline else 2.5,
+                              kernel_timing=not args.no_kernel_timing, floor=not args.no_floor)
+                res["setup_s"] = round(st.setup_s, 1)
+                for k in ("n_gpus", "higher_is_better", "scaling", "vs_baseline", "data"):
+                    res.pop(k, None)
+                configs.append(res)
+            for st in {id(v): v for v in stacks.values()}.values():
+                st.free()
+        out["configs"] = configs
+    be.close()
     print(json.dumps(out))
 
 

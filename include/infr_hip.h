@@ -207,12 +207,7 @@ typedef struct infr_hip_config {
      * kernel.  The escape hatch the reference's backends keep for their rewrites
      * (crates/infr-core/src/fusion.rs:49-52, `enabled`); results are bit-identical either way. */
     uint32_t disable_op_fusion;
-    /* Non-zero: the single-token gate/up kernel computes the reference's routing before it requests any
-     * expert row.  0 (default): it starts from the top n_used experts by logit, checks that pick against
-     * the exact routing while the rows are in flight and runs again on a mismatch.  Same bits either
-     * way; the switch exists to compare the two. */
-    uint32_t moe_route_exact_first;
-    uint32_t reserved[4];
+    uint32_t reserved[5];
 } infr_hip_config;
 
 /* Construction of the backend object (reference: VulkanBackend::new / CpuBackend::new,
@@ -289,6 +284,15 @@ infr_status infr_hip_plan_moe_bucketing(infr_hip_backend *be, const infr_hip_pla
  * crates/infr-gguf/src/dequant.rs:11-55): dst f32 buffer receives the decoded prefix of
  * `numel` elements of `src` interpreted as `dtype`. */
 infr_status infr_hip_dequant(infr_hip_backend *be, const infr_hip_buffer *src, int32_t dtype, uint64_t numel, infr_hip_buffer *dst);
+
+/* Measurement aid, no counterpart in the reference: the time a chain of DEPENDENT kernels of given sizes cannot go below
+ * on this device.  Stage k is one kernel that reads stage_bytes[k] bytes of `pool` (a window whose position depends on
+ * a word the previous stage wrote; windows rotate through the pool, so make it larger than the caches) with every load
+ * of a block in flight at once and no arithmetic.  us_per_stage[k]: stage k alone, launched back to back `iters`
+ * times; us_per_chain: the stages in order, `iters` times.  Either pointer may be NULL.  Each stage needs 1 KB up to a
+ * quarter of the pool.  Allocates a control word and two events for the duration of the call. */
+infr_status infr_hip_probe_dependent_reads(infr_hip_backend *be, const infr_hip_buffer *pool, const uint64_t *stage_bytes,
+                                           uint32_t n_stages, uint32_t iters, double *us_per_stage, double *us_per_chain);
 
 /* One Op::MoeFfn WITHOUT ANY ALLOCATION.  This entry point has no counterpart in the reference; it is for callers
  * that cannot allocate device memory: code under HIP-graph capture, tight serving loops, harnesses that forbid it.

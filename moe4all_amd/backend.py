@@ -176,7 +176,7 @@ class _Caps(C.Structure):
 
 class _Config(C.Structure):
     _fields_ = [("disable_graph_replay", C.c_uint32), ("moe_batched_min_rows", C.c_uint32),
-                ("disable_op_fusion", C.c_uint32), ("moe_route_exact_first", C.c_uint32), ("reserved", C.c_uint32 * 4)]
+                ("disable_op_fusion", C.c_uint32), ("reserved", C.c_uint32 * 5)]
 
 
 class _MoeFfnStaticArgs(C.Structure):
@@ -223,6 +223,8 @@ _SIGNATURES = {
     "infr_hip_plan_moe_bucketing": ([_V, _V, C.c_uint32, _V, _V, _V], C.c_int),
     "infr_hip_dequant": ([_V, _V, C.c_int32, C.c_uint64, _V], C.c_int),
     "infr_hip_moe_ffn_static": ([_V, C.POINTER(_MoeFfnStaticArgs)], C.c_int),
+    "infr_hip_probe_dependent_reads": ([_V, _V, C.POINTER(C.c_uint64), C.c_uint32, C.c_uint32, C.POINTER(C.c_double),
+                                        C.POINTER(C.c_double)], C.c_int),
 }
 
 _lib: Optional[C.CDLL] = None
@@ -477,11 +479,11 @@ class Backend:
     """The gfx950 compute device (crates/infr-core/src/backend.rs:630 `trait Backend`)."""
 
     def __init__(self, device: int = 0, *, disable_graph_replay: bool = False, moe_batched_min_rows: int = 0,
-                 disable_op_fusion: bool = False, moe_route_exact_first: bool = False):
+                 disable_op_fusion: bool = False):
         self._h = None
         lib = load_library()
         cfg = _Config(disable_graph_replay=int(disable_graph_replay), moe_batched_min_rows=moe_batched_min_rows,
-                      disable_op_fusion=int(disable_op_fusion), moe_route_exact_first=int(moe_route_exact_first))
+                      disable_op_fusion=int(disable_op_fusion))
         h = _V()
         _check(lib.infr_hip_create(device, C.byref(cfg), C.byref(h)))
         self._h = h.value
@@ -616,6 +618,15 @@ class Backend:
                               dst=dst._h, gate_dtype=int(gate_dtype), up_dtype=int(gate_dtype if up_dtype is None else up_dtype),
                               down_dtype=int(down_dtype), rows=rows, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=n_ff_exp)
         _check(self._lib.infr_hip_moe_ffn_static(self._h, C.byref(a)))
+
+    def probe_dependent_reads(self, pool: Buffer, stage_bytes: Sequence[int], iters: int = 200) -> dict:
+        """infr_hip_probe_dependent_reads: microseconds of each stage alone and of the whole chain."""
+        n = len(stage_bytes)
+        sizes = (C.c_uint64 * n)(*[int(b) for b in stage_bytes])
+        per = (C.c_double * n)()
+        chain = C.c_double()
+        _check(self._lib.infr_hip_probe_dependent_reads(self._h, pool._h, sizes, n, iters, per, C.byref(chain)))
+        return {"stage_us": [float(v) for v in per], "chain_us": float(chain.value)}
 
     def dequant(self, src: Buffer, dtype: DType, numel: int) -> np.ndarray:
         dst = self.alloc(numel * 4, BufferUsage.Readback)

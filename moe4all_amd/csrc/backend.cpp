@@ -1508,7 +1508,6 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                 }
                 gp.route = rp;
                 gp.y = sc.y;
-                gp.route_exact_first = be->cfg.moe_route_exact_first ? 1 : 0;
                 moe_per_token(be, s, gp, rp, rows, m.n_expert, true);
                 break;
             }
@@ -1679,12 +1678,58 @@ extern "C" infr_status infr_hip_moe_ffn_static(infr_hip_backend* be, const infr_
     gp.h = h; gp.y = y; gp.dst = (float*)a->dst->dptr; gp.x = (const float*)a->x->dptr;
     gp.n_cu = be->prop.multiProcessorCount;
     gp.route = rp;
-    gp.route_exact_first = be->cfg.moe_route_exact_first ? 1 : 0;
     moe_per_token(be, s, gp, rp, rows, a->n_expert, false);
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return fail(INFR_ERR_BACKEND, "moe_ffn_static: kernel launch failed: %s", hipGetErrorString(e));
     return INFR_OK;
 } catch (...) { return guard_fail("infr_hip_moe_ffn_static"); }
+
+// ============================================================================ measurement aid
+extern "C" infr_status infr_hip_probe_dependent_reads(infr_hip_backend* be, const infr_hip_buffer* pool,
+                                                      const uint64_t* stage_bytes, uint32_t n_stages, uint32_t iters,
+                                                      double* us_per_stage, double* us_per_chain) try {
+    if (check_owned(be, pool, "probe") != INFR_OK) return INFR_ERR_INVALID;
+    if (!stage_bytes || n_stages == 0 || n_stages > 16 || iters == 0 || iters > 100000)
+        return fail(INFR_ERR_INVALID, "probe: 1..16 stages and 1..100000 iterations");
+    for (uint32_t i = 0; i < n_stages; i++)
+        if (stage_bytes[i] < 1024 || stage_bytes[i] * 4 > pool->len)
+            return fail(INFR_ERR_INVALID, "probe: stage %u of %llu bytes needs 1 KB .. a quarter of the pool (%zu bytes)", i,
+                        (unsigned long long)stage_bytes[i], pool->len);
+    std::lock_guard<std::mutex> lk(be->mu);
+    HIP_TRY(hipSetDevice(be->device));
+    uint32_t* ctl = nullptr;
+    HIP_TRY(hipMalloc(&ctl, 256));
+    hipEvent_t a = nullptr, b = nullptr;
+    hipError_t e = hipEventCreate(&a);
+    if (e == hipSuccess) e = hipEventCreate(&b);
+    hipStream_t s = be->stream;
+    const int n_cu = be->prop.multiProcessorCount;
+    infr::launch_fill_zero(s, ctl, 256);
+    uint32_t salt = 1;
+    auto timed = [&](uint32_t first, uint32_t count, double* out) {
+        for (uint32_t w = 0; w < 3 && e == hipSuccess; w++)   // warm-up
+            for (uint32_t k = first; k < first + count; k++)
+                infr::launch_probe_dependent_read(s, (const uint8_t*)pool->dptr, pool->len, stage_bytes[k], ctl, salt++, n_cu);
+        if (e == hipSuccess) e = hipEventRecord(a, s);
+        for (uint32_t it = 0; it < iters && e == hipSuccess; it++)
+            for (uint32_t k = first; k < first + count; k++)
+                infr::launch_probe_dependent_read(s, (const uint8_t*)pool->dptr, pool->len, stage_bytes[k], ctl, salt++, n_cu);
+        if (e == hipSuccess) e = hipEventRecord(b, s);
+        if (e == hipSuccess) e = hipEventSynchronize(b);
+        float ms = 0.0f;
+        if (e == hipSuccess) e = hipEventElapsedTime(&ms, a, b);
+        if (out) *out = (double)ms * 1e3 / iters;
+    };
+    for (uint32_t k = 0; k < n_stages; k++) timed(k, 1, us_per_stage ? us_per_stage + k : nullptr);
+    timed(0, n_stages, us_per_chain);
+    if (e == hipSuccess) e = hipGetLastError();
+    if (a) (void)hipEventDestroy(a);
+    if (b) (void)hipEventDestroy(b);
+    (void)hipStreamSynchronize(s);
+    (void)hipFree(ctl);
+    if (e != hipSuccess) return fail(INFR_ERR_BACKEND, "probe: %s", hipGetErrorString(e));
+    return INFR_OK;
+} catch (...) { return guard_fail("infr_hip_probe_dependent_reads"); }
 
 // ============================================================================ taps
 extern "C" infr_status infr_hip_prof_enable(infr_hip_backend* be, int on) try {

@@ -95,122 +95,88 @@ __device__ __forceinline__ void gu_finish(const GuStage<F, U>& st, const MoeGemv
 // then all of the block's loads are in flight at once).  PIPE == true, for tiles of three or more
 // stages: two stage buffers, the next stage's loads are issued before the current stage is
 // finished, so a wave always has a stage in flight while it computes.
-// When the kernel routes its token row itself (p.route_inline) the block has a fifth wavefront that does
-// nothing else.  spec != 0: it publishes the top n_used by logit at once, so the four workers can request
-// their expert rows, and runs the reference's routing while those bytes are in flight; the pick is checked
-// against the exact probabilities and, if any rank differs, the workers run again with the exact ids
-// (gate_up_router in route.h).  The expert ids are all this kernel needs of the routing; the routing weights
-// are first used by the down kernel (and here with weight_before, which therefore routes exactly first).
-// ROUTER instances have the five wavefronts (two of them share a SIMD and its registers, so they keep fewer
-// rows in flight per wave); the others are the plain four-wave kernel for ids that are given.
-constexpr int kGuRouterWave = 4;
-template <class F, int U, bool PIPE, bool ROUTER>
-__global__ __launch_bounds__(ROUTER ? 320 : 256) void moe_gate_up_fast(MoeGemvParams p, int ft, int spec) {
+template <class F, int U, bool PIPE>
+__global__ __launch_bounds__(256) void moe_gate_up_fast(MoeGemvParams p, int ft) {
     extern __shared__ uint32_t dyn_lds[];
     __shared__ uint64_t s_tab[32];
-    __shared__ int32_t s_ids[64], s_early[64];
+    __shared__ int32_t s_ids[64];
     __shared__ float s_w[64];
-    __shared__ int s_redo;
     __shared__ float s_g[4][64], s_u[4][64];
     GuTile t;
     t.r = blockIdx.y;
     t.f0 = blockIdx.x * ft;
     t.fcount = min(ft, p.nff - t.f0);
-    t.wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    t.wave = threadIdx.x >> 6;
     t.lane = threadIdx.x & 63;
     const int r = t.r, wave = t.wave, lane = t.lane;
     const int nblk = p.ne / F::kBlockElems;
     t.row_bytes = (size_t)nblk * F::kBlockBytes;
     const Place<F> pl(nblk, lane);
     const size_t cell_words = (size_t)((p.ne + 31) / 32) * kCellDwords;
-    uint32_t* cells = dyn_lds + (size_t)min(wave, 3) * cell_words;
-    t.n_slots = p.n_used + (p.sh_gate ? 1 : 0);   // the always-on expert is slot n_used (<= 63 then)
+    uint32_t* cells = dyn_lds + (size_t)wave * cell_words;
+    // x is requested first; it does not depend on the routing
     const float* xrow = p.x + (size_t)r * p.ne;
-    XLoad xl;
-    if (ROUTER && wave == kGuRouterWave) {
-        float* lds_prob = reinterpret_cast<float*>(dyn_lds + 4 * cell_words);
-        const int n = p.route.n_expert, n_pad = n <= 128 ? 128 : 256;
-        if (n <= 128) gate_up_router<2>(p.route, r, lane, spec != 0, lds_prob, lds_prob + n_pad, s_tab, s_ids, s_early, s_w, &s_redo, blockIdx.x == 0);
-        else if (n <= 256) gate_up_router<4>(p.route, r, lane, spec != 0, lds_prob, lds_prob + n_pad, s_tab, s_ids, s_early, s_w, &s_redo, blockIdx.x == 0);
-        else {
-            if (lane < 32) s_tab[lane] = kExp2Table[lane];
-            __builtin_amdgcn_wave_barrier();
-            route_row_large(p.route, r, lane, lds_prob, s_tab, s_ids, s_w, blockIdx.x == 0);
-            __builtin_amdgcn_wave_barrier();
-            if (lane < p.n_used) s_early[lane] = s_ids[lane];
-            __syncthreads();   // (1)
-        }
-    } else {
-        // x is requested first; it does not depend on the routing
-        xl = stage_x_load(xrow, p.ne, lane);
-        if (!ROUTER) {
-            if (threadIdx.x < 32) s_tab[threadIdx.x] = kExp2Table[threadIdx.x];
-            if ((int)threadIdx.x < p.n_used) {  // n_used <= 64
-                s_ids[threadIdx.x] = s_early[threadIdx.x] = p.ids[(size_t)r * p.n_used + threadIdx.x];
-                s_w[threadIdx.x] = p.weights[(size_t)r * p.n_used + threadIdx.x];
-            }
-        }
-        if (p.sh_gate && threadIdx.x == 255) {
-            s_ids[p.n_used] = s_early[p.n_used] = 0;
-            s_w[p.n_used] = 1.0f;
-        }
-        if (threadIdx.x == 0) s_redo = 0;
-        __syncthreads();   // (1) the ids to start from are in LDS
+    const XLoad xl = stage_x_load(xrow, p.ne, lane);
+    if (threadIdx.x < 32) s_tab[threadIdx.x] = kExp2Table[threadIdx.x];
+    if (p.route_inline) {
+        // every block routes its token row itself (one wave, redundantly across blocks)
+        __syncthreads();
+        if (wave == 0)
+            route_row_any(p.route, r, lane, reinterpret_cast<float*>(dyn_lds + 4 * cell_words), s_tab, s_ids, s_w,
+                          blockIdx.x == 0);
+    } else if ((int)threadIdx.x < p.n_used) {  // n_used <= 64
+        s_ids[threadIdx.x] = p.ids[(size_t)r * p.n_used + threadIdx.x];
+        s_w[threadIdx.x] = p.weights[(size_t)r * p.n_used + threadIdx.x];
     }
+    t.n_slots = p.n_used + (p.sh_gate ? 1 : 0);   // the always-on expert is slot n_used (<= 63 then)
+    if (p.sh_gate && threadIdx.x == 255) {
+        s_ids[p.n_used] = 0;
+        s_w[p.n_used] = 1.0f;
+    }
+    __syncthreads();
+    __builtin_amdgcn_wave_barrier();
     t.nitems = t.fcount * t.n_slots;
     const int step = 4 * pl.rw_count * U;
     typename F::X x;
-    bool have_x = false;
-#pragma nounroll
-    for (int attempt = 0; attempt < 2; attempt++) {
-        const int32_t* ids = attempt == 0 ? s_early : s_ids;
-        if (!ROUTER || wave != kGuRouterWave) {
-            if (!PIPE) {
-                for (int base = 0; base < t.nitems; base += step) {
-                    GuStage<F, U> st;
-                    gu_issue<F, U>(st, p, pl, t, ids, base);
-                    if (!have_x) {
-                        // while the weights are in flight: the wave converts x to fixed point once, together
-                        stage_x_finish<F::kGroup, F::kSigned>(xl, xrow, p.ne, cells, lane);
-                        __builtin_amdgcn_wave_barrier();
-                        F::fetch_x(x, cells, pl.blk, pl.sub);
-                        have_x = true;
-                    }
-                    gu_finish<F, U>(st, p, pl, t, x, nblk, base, s_g, s_u, s_w, s_tab);
-                }
-            } else {
-                GuStage<F, U> sa, sb;
-                gu_issue<F, U>(sa, p, pl, t, ids, 0);
-                gu_issue<F, U>(sb, p, pl, t, ids, step);
-                if (!have_x) {
-                    stage_x_finish<F::kGroup, F::kSigned>(xl, xrow, p.ne, cells, lane);
-                    __builtin_amdgcn_wave_barrier();
-                    F::fetch_x(x, cells, pl.blk, pl.sub);
-                    have_x = true;
-                }
-                gu_finish<F, U>(sa, p, pl, t, x, nblk, 0, s_g, s_u, s_w, s_tab);
-                int base = step;   // the stage sb holds
-                for (;;) {
-                    if (base + step >= t.nitems) {
-                        gu_finish<F, U>(sb, p, pl, t, x, nblk, base, s_g, s_u, s_w, s_tab);
-                        break;
-                    }
-                    gu_issue<F, U>(sa, p, pl, t, ids, base + step);
-                    gu_finish<F, U>(sb, p, pl, t, x, nblk, base, s_g, s_u, s_w, s_tab);
-                    base += step;
-                    if (base + step >= t.nitems) {
-                        gu_finish<F, U>(sa, p, pl, t, x, nblk, base, s_g, s_u, s_w, s_tab);
-                        break;
-                    }
-                    gu_issue<F, U>(sb, p, pl, t, ids, base + step);
-                    gu_finish<F, U>(sa, p, pl, t, x, nblk, base, s_g, s_u, s_w, s_tab);
-                    base += step;
-                }
+    if (!PIPE) {
+        bool have_x = false;
+        for (int base = 0; base < t.nitems; base += step) {
+            GuStage<F, U> st;
+            gu_issue<F, U>(st, p, pl, t, s_ids, base);
+            if (!have_x) {
+                // while the weights are in flight: the wave converts x to fixed point once, together
+                stage_x_finish<F::kGroup, F::kSigned>(xl, xrow, p.ne, cells, lane);
+                __builtin_amdgcn_wave_barrier();
+                F::fetch_x(x, cells, pl.blk, pl.sub);
+                have_x = true;
             }
+            gu_finish<F, U>(st, p, pl, t, x, nblk, base, s_g, s_u, s_w, s_tab);
         }
-        if (!spec || attempt == 1) break;   // spec is uniform over the grid
-        __syncthreads();   // (2) the exact routing is in LDS
-        if (!s_redo) break;
+    } else {
+        GuStage<F, U> sa, sb;
+        gu_issue<F, U>(sa, p, pl, t, s_ids, 0);
+        gu_issue<F, U>(sb, p, pl, t, s_ids, step);
+        stage_x_finish<F::kGroup, F::kSigned>(xl, xrow, p.ne, cells, lane);
+        __builtin_amdgcn_wave_barrier();
+        F::fetch_x(x, cells, pl.blk, pl.sub);
+        gu_finish<F, U>(sa, p, pl, t, x, nblk, 0, s_g, s_u, s_w, s_tab);
+        int base = step;   // the stage sb holds
+        for (;;) {
+            if (base + step >= t.nitems) {
+                gu_finish<F, U>(sb, p, pl, t, x, nblk, base, s_g, s_u, s_w, s_tab);
+                break;
+            }
+            gu_issue<F, U>(sa, p, pl, t, s_ids, base + step);
+            gu_finish<F, U>(sb, p, pl, t, x, nblk, base, s_g, s_u, s_w, s_tab);
+            base += step;
+            if (base + step >= t.nitems) {
+                gu_finish<F, U>(sa, p, pl, t, x, nblk, base, s_g, s_u, s_w, s_tab);
+                break;
+            }
+            gu_issue<F, U>(sb, p, pl, t, s_ids, base + step);
+            gu_finish<F, U>(sa, p, pl, t, x, nblk, base, s_g, s_u, s_w, s_tab);
+            base += step;
+        }
     }
 }
 
@@ -420,35 +386,18 @@ static bool try_gate_up(hipStream_t s, const MoeGemvParams& p) {
     const int per_wave = ceil_div(ft * n_slots, 4 * rw);
     // tiles of three or more stages stream with the next stage in flight
     const bool pipe = per_wave > 6 && 3 * rw <= 64;
-    dim3 grid(ceil_div(p.nff, ft), p.rows);
+    dim3 grid(ceil_div(p.nff, ft), p.rows), block(256);
     // U * rw results per wave must fit the 64-entry staging rows
     int u = per_wave < 1 ? 1 : per_wave;
     while (u * rw > 64) u--;
-    const int n_pad = p.route.n_expert <= 128 ? 128 : 256;
     const size_t lds = 4 * cells_bytes(p.ne) +
-                       (p.route_inline ? (route_scratch_floats(p.route.n_expert, p.route.n_groups) + n_pad) * sizeof(float) : 0);
-    // the top-k by logit is the selection of any monotone gating without a bias, groups, given ids or a band; the
-    // routing weights are not known before the exact routing, so weight_before routes exactly first
-    const int spec = p.route_inline && !p.route_exact_first && p.route.n_expert <= 256 && !p.route.exp_probs_b &&
-                     !(p.route.n_groups > 1 && p.route.n_groups_used > 0) && !p.route.expert_ids && p.route.ep_n == 0 &&
-                     !p.weight_before;
-    if (p.route_inline) {
-        // five wavefronts: at most four row pairs in flight per wave (two stages of two when streaming)
-        const dim3 block(320);
-        if (pipe || u > 4) INFR_LAUNCH((moe_gate_up_fast<F, 2, true, true>), grid, block, lds, s, p, ft, spec);
-        else if (u == 4) INFR_LAUNCH((moe_gate_up_fast<F, 4, false, true>), grid, block, lds, s, p, ft, spec);
-        else if (u == 3) INFR_LAUNCH((moe_gate_up_fast<F, 3, false, true>), grid, block, lds, s, p, ft, spec);
-        else if (u == 2) INFR_LAUNCH((moe_gate_up_fast<F, 2, false, true>), grid, block, lds, s, p, ft, spec);
-        else INFR_LAUNCH((moe_gate_up_fast<F, 1, false, true>), grid, block, lds, s, p, ft, spec);
-        return true;
-    }
-    const dim3 block(256);
-    if (pipe) INFR_LAUNCH((moe_gate_up_fast<F, 3, true, false>), grid, block, lds, s, p, ft, 0);
-    else if (u >= 6) INFR_LAUNCH((moe_gate_up_fast<F, 6, false, false>), grid, block, lds, s, p, ft, 0);
-    else if (u == 5 || u == 4) INFR_LAUNCH((moe_gate_up_fast<F, 4, false, false>), grid, block, lds, s, p, ft, 0);
-    else if (u == 3) INFR_LAUNCH((moe_gate_up_fast<F, 3, false, false>), grid, block, lds, s, p, ft, 0);
-    else if (u == 2) INFR_LAUNCH((moe_gate_up_fast<F, 2, false, false>), grid, block, lds, s, p, ft, 0);
-    else INFR_LAUNCH((moe_gate_up_fast<F, 1, false, false>), grid, block, lds, s, p, ft, 0);
+                       (p.route_inline ? route_scratch_floats(p.route.n_expert, p.route.n_groups) * sizeof(float) : 0);
+    if (pipe) INFR_LAUNCH((moe_gate_up_fast<F, 3, true>), grid, block, lds, s, p, ft);
+    else if (u >= 6) INFR_LAUNCH((moe_gate_up_fast<F, 6, false>), grid, block, lds, s, p, ft);
+    else if (u == 5 || u == 4) INFR_LAUNCH((moe_gate_up_fast<F, 4, false>), grid, block, lds, s, p, ft);
+    else if (u == 3) INFR_LAUNCH((moe_gate_up_fast<F, 3, false>), grid, block, lds, s, p, ft);
+    else if (u == 2) INFR_LAUNCH((moe_gate_up_fast<F, 2, false>), grid, block, lds, s, p, ft);
+    else INFR_LAUNCH((moe_gate_up_fast<F, 1, false>), grid, block, lds, s, p, ft);
     return true;
 }
 

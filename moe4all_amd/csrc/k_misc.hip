@@ -178,4 +178,49 @@ void launch_fill_zero(hipStream_t s, void* p, size_t bytes) {
     INFR_LAUNCH(fill_zero_kernel, dim3((uint32_t)blocks), dim3(256), 0, s, (uint32_t*)p, words);
 }
 
+// ------------------------------------------------------------------------------------------------
+// Measurement aid: one stage of a chain of DEPENDENT reads.  The stage reads `bytes` of `pool`, spread over the
+// grid, from a window whose position depends on the word the previous stage left in ctl[0], does no arithmetic on
+// what it reads, and leaves a new word for the next stage.  Timed back to back it gives the time a kernel of this
+// size cannot go below on this device, whatever it computes: dispatch of a dependent kernel, one round trip for the
+// control word, one burst of loads (straight into LDS, 16 bytes per lane, every load of a block in flight at once).
+__global__ __launch_bounds__(256) void probe_dependent_read_kernel(const uint8_t* __restrict__ pool, uint64_t pool_bytes,
+                                                                   uint64_t bytes, uint32_t* ctl, uint32_t salt) {
+    extern __shared__ uint32_t probe_lds[];
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const uint32_t word = ctl[0];                                   // the dependence on the previous stage
+    const uint64_t windows = pool_bytes / bytes;
+    const uint8_t* win = pool + (uint64_t)((word * 2654435761u + salt) % (uint32_t)windows) * bytes;
+    const uint64_t per_block = (bytes / gridDim.x) & ~(uint64_t)1023;   // whole 1 KB copies
+    const uint8_t* mine = win + (uint64_t)blockIdx.x * per_block;
+    const uint32_t base = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)probe_lds;
+    const int n_copies = (int)(per_block >> 10);
+    int issued = 0;
+    for (int i = wave; i < n_copies; i += 4) {
+        const uint32_t lds_at = __builtin_amdgcn_readfirstlane(base + (uint32_t)(i % 128) * 1024u);
+        asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(mine + (size_t)i * 1024 + lane * 16), "s"(lds_at) : "memory");
+        if (++issued == 32) {   // the LDS window holds 128 copies: four waves x 32
+            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+            issued = 0;
+        }
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    const uint32_t seen = probe_lds[threadIdx.x];
+    if (blockIdx.x == 0 && threadIdx.x == 0) ctl[0] = word + 1u + (seen == 0x9E3779B9u ? 1u : 0u);
+}
+
+void launch_probe_dependent_read(hipStream_t s, const uint8_t* pool, uint64_t pool_bytes, uint64_t bytes, uint32_t* ctl,
+                                 uint32_t salt, int n_cu) {
+    static bool attr_set = false;
+    if (!attr_set) {
+        (void)hipFuncSetAttribute((const void*)probe_dependent_read_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
+        attr_set = true;
+    }
+    uint64_t blocks = bytes >> 10;   // at least one 1 KB copy per block
+    if (blocks > (uint64_t)n_cu) blocks = (uint64_t)n_cu;
+    if (blocks < 1) blocks = 1;
+    INFR_LAUNCH(probe_dependent_read_kernel, dim3((uint32_t)blocks), dim3(256), 128 * 1024, s, pool, pool_bytes, bytes, ctl, salt);
+}
+
 }  // namespace infr

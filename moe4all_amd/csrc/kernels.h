@@ -90,9 +90,6 @@ struct MoeGemvParams {
     // When set, the gate/up kernel routes each token row itself from route.logits (every block
     // redundantly; block 0 of a row publishes ids / weights / probs) and no route launch is needed.
     int route_inline;
-    // route_inline only: 1 = route exactly before any expert row is requested; 0 = the kernel may start from the
-    // top n_used by logit and check that pick against the exact routing while the rows are in flight
-    int route_exact_first;
     RouteParams route;
     // bucketed decode batches (launch_moe_*_bucketed): pairs grouped by expert
     const int32_t* bk_offsets;   // [n_expert + 1]
@@ -198,5 +195,8 @@ void launch_copy_rows(hipStream_t s, const void* src, void* dst, uint32_t rows, 
 void launch_moe_shared_expert_add(hipStream_t s, const float* moe, const float* shexp, const float* gate, float* dst,
                                   int rows, int n);
 void launch_fill_zero(hipStream_t s, void* p, size_t bytes);
+// One stage of a chain of dependent reads (measurement aid): `bytes` of `pool` from a window chosen by ctl[0].
+void launch_probe_dependent_read(hipStream_t s, const uint8_t* pool, uint64_t pool_bytes, uint64_t bytes, uint32_t* ctl,
+                                 uint32_t salt, int n_cu);
 
 }  // namespace infr

@@ -202,166 +202,6 @@ __device__ __forceinline__ void route_row_any(const RouteParams& p, int row, int
     else route_row<32>(p, row, lane, lds, tab, lds_ids, lds_w, store_global);
 }
 
-// The routing wavefront of the single-token gate/up kernel: everything up to and including the block's barrier (1).
-//
-// spec: the top n_used by (logit descending, id ascending) are picked on a key that keeps the upper bits of the
-// order-preserving integer image of the logit and carries the inverted id in the bits below (one wave-wide max per
-// rank finds value and position together) and published as s_early before barrier (1), so the workers start their
-// copies at once.  Behind the barrier the probabilities are computed in the reference's operation order
-// (crates/infr-cpu/src/lib.rs:3746-3774) and the pick is CHECKED against them: consecutive ranks in the order
-// (probability descending, id ascending) of the reference's stable sort (lib.rs:3847-3850), every other expert
-// behind the last rank in that order.  The order is total, so a pick that passes is the reference's selection rank
-// by rank and the routing weights follow (lib.rs:3856-3861).  A pick that fails (logits that agree in every kept
-// bit, distinct logits whose probabilities round to the same float, NaN) is replaced by the full routine's
-// selection, and s_redo tells the workers to run again if any rank differs.
-// !spec (selection bias, expert groups, given ids, an expert-parallel band: the logits' order does not decide): the
-// full routine runs before barrier (1).
-template <int NS>
-__device__ __forceinline__ void gate_up_router(const RouteParams& p, int row, int lane, bool spec, float* lds_prob,
-                                               float* scratch, uint64_t* s_tab, int32_t* s_ids, int32_t* s_early,
-                                               float* s_w, int* s_redo, bool store_global) {
-    const int n = p.n_expert;
-    const float ninf = -__builtin_huge_valf();
-    if (lane < 32) s_tab[lane] = kExp2Table[lane];
-    float pr[NS];
-    uint32_t taken = 0;   // bit s: this lane's candidate s was picked
-    int id = 0;           // lane k < n_used: the rank-k pick
-    if (spec) {
-        const float* lg = p.logits + (size_t)row * n;
-        const uint32_t mask = (1u << (32 - __builtin_clz((uint32_t)(n > 1 ? n - 1 : 1)))) - 1u;
-        uint32_t key[NS];
-#pragma unroll
-        for (int s = 0; s < NS; s++) {
-            const int i = s * kWave + lane;
-            pr[s] = i < n ? lg[i] : ninf;
-            key[s] = i < n ? ((order_key(pr[s]) & ~mask) | (mask - (uint32_t)i)) : 0u;
-        }
-        for (int k = 0; k < p.n_used; k++) {
-            uint32_t m = key[0];
-#pragma unroll
-            for (int s = 1; s < NS; s++) m = max(m, key[s]);
-            const uint32_t best = wave_max_u32(m);
-#pragma unroll
-            for (int s = 0; s < NS; s++)
-                if (key[s] == best && best != 0u) { key[s] = 0u; taken |= 1u << s; }
-            if (lane == k) id = min((int)(mask - (best & mask)), n - 1);
-        }
-        if (lane < p.n_used) s_early[lane] = id;
-    }
-    bool need_full = !spec;
-#pragma nounroll
-    for (int phase = 0; phase < 2; phase++) {
-        if (phase == 1 && spec) {
-            // ---- probabilities (lib.rs:3746-3774)
-            if (p.gating == INFR_GATING_SOFTMAX) {
-                float m = ninf;
-#pragma unroll
-                for (int s = 0; s < NS; s++) m = fmaxf(m, pr[s]);
-                m = wave_max(m);
-#pragma unroll
-                for (int s = 0; s < NS; s++) {
-                    const int i = s * kWave + lane;
-                    pr[s] = i < n ? expf_libm(__fsub_rn(pr[s], m), s_tab) : 0.0f;
-                    if (i < n) lds_prob[i] = pr[s];
-                }
-                __builtin_amdgcn_wave_barrier();
-                // psum = p[0] + p[1] + ... strictly left to right; every lane runs the same chain on broadcast reads
-                float psum = 0.0f;
-                int i = 0;
-                for (; i + 4 <= n; i += 4) {
-                    const float4 v = *reinterpret_cast<const float4*>(lds_prob + i);
-                    psum = __fadd_rn(__fadd_rn(__fadd_rn(__fadd_rn(psum, v.x), v.y), v.z), v.w);
-                }
-                for (; i < n; i++) psum = __fadd_rn(psum, lds_prob[i]);
-                __builtin_amdgcn_wave_barrier();
-#pragma unroll
-                for (int s = 0; s < NS; s++) pr[s] = __fdiv_rn(pr[s], psum);
-            } else if (p.gating == INFR_GATING_SIGMOID) {
-#pragma unroll
-                for (int s = 0; s < NS; s++) pr[s] = __fdiv_rn(1.0f, __fadd_rn(1.0f, expf_libm(-pr[s], s_tab)));
-            } else {
-#pragma unroll
-                for (int s = 0; s < NS; s++) {
-                    const float v = pr[s];
-                    const float sp = v > 20.0f ? v : logf(__fadd_rn(1.0f, expf_libm(v, s_tab)));
-                    pr[s] = __fsqrt_rn(sp);
-                }
-            }
-#pragma unroll
-            for (int s = 0; s < NS; s++) {
-                const int i = s * kWave + lane;
-                if (i < n) lds_prob[i] = pr[s];
-            }
-            __builtin_amdgcn_wave_barrier();
-            // ---- the pick against the probabilities: lane k < n_used holds rank k
-            const bool mine = lane < p.n_used;
-            const float pk = mine ? lds_prob[id] : 0.0f;
-            const int id_next = __shfl_down(id, 1, kWave);
-            const float pk_next = __shfl_down(pk, 1, kWave);
-            bool ok = true;
-            if (lane + 1 < p.n_used) ok = pk > pk_next || (pk == pk_next && id < id_next);
-            const float p_last = readlane_f(pk, p.n_used - 1);
-            const int id_last = __builtin_amdgcn_readlane(id, p.n_used - 1);
-#pragma unroll
-            for (int s = 0; s < NS; s++) {
-                const int i = s * kWave + lane;
-                if (i < n && !(taken & (1u << s))) ok = ok && (pr[s] < p_last || (pr[s] == p_last && i > id_last));
-            }
-            if (mine) ok = ok && pk == pk;   // a NaN probability is the reference's panic: leave it to the full routine
-            if (__all(ok)) {
-                // ---- routing weights (lib.rs:3856-3861)
-                float w;
-                if (p.norm_w) {
-                    float wsum = 0.0f;
-                    for (int k = 0; k < p.n_used; k++) wsum = __fadd_rn(wsum, readlane_f(pk, k));
-                    wsum = fmaxf(wsum, 1e-20f);
-                    w = __fmul_rn(__fdiv_rn(pk, wsum), p.scale);
-                } else {
-                    w = __fmul_rn(pk, p.scale);
-                }
-                if (mine) {
-                    s_ids[lane] = id;
-                    s_w[lane] = w;
-                    if (store_global) {
-                        p.ids[(size_t)row * p.n_used + lane] = id;
-                        p.weights[(size_t)row * p.n_used + lane] = w;
-                    }
-                }
-                if (p.probs && store_global) {
-#pragma unroll
-                    for (int s = 0; s < NS; s++) {
-                        const int i = s * kWave + lane;
-                        if (i < n) p.probs[(size_t)row * n + i] = pr[s];
-                    }
-                }
-            } else {
-                need_full = true;
-            }
-        }
-        if (need_full) {
-            __builtin_amdgcn_wave_barrier();
-            route_row<NS>(p, row, lane, scratch, s_tab, s_ids, s_w, store_global);
-            __builtin_amdgcn_wave_barrier();
-            if (phase == 0) {
-                if (lane < p.n_used) s_early[lane] = s_ids[lane];
-            } else {
-                bool differs = false;
-                if (lane < p.n_used) differs = s_ids[lane] != s_early[lane];
-                if (__any(differs) && lane == 0) *s_redo = 1;
-            }
-            need_full = false;
-        }
-        if (phase == 0) __syncthreads();   // (1)
-    }
-}
-
-// Rows of more than 256 experts.
-__device__ __forceinline__ void route_row_large(const RouteParams& p, int row, int lane, float* lds, const uint64_t* tab,
-                                                int32_t* lds_ids, float* lds_w, bool store_global) {
-    if (p.n_expert <= 512) route_row<8>(p, row, lane, lds, tab, lds_ids, lds_w, store_global);
-    else route_row<32>(p, row, lane, lds, tab, lds_ids, lds_w, store_global);
-}
-
 // LDS floats route_row_any needs behind the 64-float exp table.
 __host__ __device__ inline size_t route_scratch_floats(int n_expert, int n_groups) {
     return (size_t)2 * n_expert + (size_t)(n_groups > 0 ? n_groups : 0);
