@@ -44,12 +44,15 @@ typedef enum infr_dtype {
     INFR_F32 = 0, INFR_F16 = 1, INFR_BF16 = 2, INFR_I32 = 3, INFR_U32 = 4,
     INFR_Q4_0 = 5, INFR_Q4_1 = 6, INFR_Q5_0 = 7, INFR_Q5_1 = 8, INFR_Q8_0 = 9,
     INFR_Q2K = 10, INFR_Q3K = 11, INFR_Q4K = 12, INFR_Q5K = 13, INFR_Q6K = 14,
-    /* small-table codebook, ternary and fp4 formats, decoded on the device like the affine ones
-     * (crates/infr-gguf/src/dequant.rs:499-559, :926-1073) */
+    /* lattice-codebook i-quants (crates/infr-gguf/src/dequant.rs:565-916) */
+    INFR_IQ1_S = 15, INFR_IQ1_M = 16, INFR_IQ2_XXS = 17, INFR_IQ2_XS = 18, INFR_IQ2_S = 19, INFR_IQ3_XXS = 20,
+    INFR_IQ3_S = 21,
+    /* small-table codebook, ternary and fp4 formats (dequant.rs:499-559, :926-1073) */
     INFR_IQ4_NL = 22, INFR_IQ4_XS = 23, INFR_TQ1_0 = 24, INFR_TQ2_0 = 25,
     INFR_Q2_0 = 27, INFR_MXFP4 = 28, INFR_NVFP4 = 29
-    /* the other ordinals from 15 on (grid i-quants Iq1S..Iq3S = 15..21, I2S = 26, turbo) are accepted
-     * in declarations and rejected with INFR_ERR_UNSUPPORTED by any op that would decode them */
+    /* every format above is decoded on the device.  The remaining ordinals (I2S = 26, whose scale lives outside the
+     * tensor bytes, and the turbo formats from 30 on) are accepted in declarations and rejected with
+     * INFR_ERR_UNSUPPORTED by any op that would decode them */
 } infr_dtype;
 
 /* infr_core::backend::BufferUsage (backend.rs:384-406). */

@@ -97,7 +97,9 @@ _BLOCK = {DType.F32: (1, 4), DType.I32: (1, 4), DType.U32: (1, 4), DType.F16: (1
           DType.Q8_0: (32, 34), DType.Q4K: (256, 144), DType.Q6K: (256, 210), DType.Q4_0: (32, 18), DType.Q4_1: (32, 20),
           DType.Q5_0: (32, 22), DType.Q5_1: (32, 24), DType.Q2K: (256, 84), DType.Q3K: (256, 110), DType.Q5K: (256, 176),
           DType.Iq4Nl: (32, 18), DType.Iq4Xs: (256, 136), DType.Tq1_0: (256, 54), DType.Tq2_0: (256, 66), DType.Q2_0: (64, 18),
-          DType.Mxfp4: (32, 17), DType.Nvfp4: (64, 36)}
+          DType.Mxfp4: (32, 17), DType.Nvfp4: (64, 36),
+          DType.Iq1S: (256, 50), DType.Iq1M: (256, 56), DType.Iq2Xxs: (256, 66), DType.Iq2Xs: (256, 74), DType.Iq2S: (256, 82),
+          DType.Iq3Xxs: (256, 98), DType.Iq3S: (256, 110)}
 
 
 def bytes_for(dtype: DType, numel: int) -> int:

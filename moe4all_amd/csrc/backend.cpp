@@ -102,6 +102,13 @@ bool geometry(int dtype, int* elems, int* bytes) {
         case INFR_Q2_0: *elems = 64; *bytes = 18; return true;
         case INFR_MXFP4: *elems = 32; *bytes = 17; return true;
         case INFR_NVFP4: *elems = 64; *bytes = 36; return true;
+        case INFR_IQ1_S: *elems = 256; *bytes = 50; return true;
+        case INFR_IQ1_M: *elems = 256; *bytes = 56; return true;
+        case INFR_IQ2_XXS: *elems = 256; *bytes = 66; return true;
+        case INFR_IQ2_XS: *elems = 256; *bytes = 74; return true;
+        case INFR_IQ2_S: *elems = 256; *bytes = 82; return true;
+        case INFR_IQ3_XXS: *elems = 256; *bytes = 98; return true;
+        case INFR_IQ3_S: *elems = 256; *bytes = 110; return true;
         default: return false;
     }
 }

@@ -6,6 +6,7 @@
 #include <stdint.h>
 
 #include "../../include/infr_hip.h"
+#include "iquant.h"
 
 namespace infr {
 
@@ -122,6 +123,14 @@ __host__ __device__ inline bool block_geometry(int dtype, int* elems, int* bytes
         case INFR_Q2_0: *elems = 64; *bytes = 18; return true;
         case INFR_MXFP4: *elems = 32; *bytes = 17; return true;
         case INFR_NVFP4: *elems = 64; *bytes = 36; return true;
+        // decode_spec.rs:334-347
+        case INFR_IQ1_S: *elems = 256; *bytes = 50; return true;
+        case INFR_IQ1_M: *elems = 256; *bytes = 56; return true;
+        case INFR_IQ2_XXS: *elems = 256; *bytes = 66; return true;
+        case INFR_IQ2_XS: *elems = 256; *bytes = 74; return true;
+        case INFR_IQ2_S: *elems = 256; *bytes = 82; return true;
+        case INFR_IQ3_XXS: *elems = 256; *bytes = 98; return true;
+        case INFR_IQ3_S: *elems = 256; *bytes = 110; return true;
         default: return false;
     }
 }
@@ -326,6 +335,13 @@ __device__ inline float decode_elem(int dtype, const uint8_t* row, uint32_t k) {
             const uint32_t w = k & 63u, s = w >> 4, e = w & 15u, v = blk[4u + 8u * s + (e & 7u)];
             return __fmul_rn((float)book16(kFp4Lo, kFp4Hi, e < 8u ? v & 0xFu : v >> 4), ue4m3_half(blk[s]));
         }
+        case INFR_IQ1_S: return decode_iq1s(row, k);
+        case INFR_IQ1_M: return decode_iq1m(row, k);
+        case INFR_IQ2_XXS: return decode_iq2xxs(row, k);
+        case INFR_IQ2_XS: return decode_iq2xs(row, k);
+        case INFR_IQ2_S: return decode_iq2s(row, k);
+        case INFR_IQ3_XXS: return decode_iq3xxs(row, k);
+        case INFR_IQ3_S: return decode_iq3s(row, k);
         default: return 0.0f;
     }
 }

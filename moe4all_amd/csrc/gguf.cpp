@@ -63,7 +63,8 @@ constexpr uint32_t kMaxDims = 4;
 constexpr int kMaxArrayDepth = 64;
 constexpr size_t kMaxShardDigits = 5;
 
-// infr_dtype ordinals beyond the ones infr_hip.h names (crates/infr-core/src/tensor.rs:25-50)
+// infr_dtype ordinals from 15 on under the loader's own names; I2S is known to the loader only
+// (crates/infr-core/src/tensor.rs:25-50)
 enum : int32_t {
     DT_IQ1S = 15, DT_IQ1M, DT_IQ2XXS, DT_IQ2XS, DT_IQ2S, DT_IQ3XXS, DT_IQ3S, DT_IQ4NL, DT_IQ4XS,
     DT_TQ1_0, DT_TQ2_0, DT_I2S, DT_Q2_0, DT_MXFP4, DT_NVFP4

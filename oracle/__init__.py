@@ -18,6 +18,7 @@ _LIB_PATH = os.path.join(_HERE, "libinfr_oracle.so")
 # infr_core::DType ordinals (crates/infr-core/src/tensor.rs:7-57)
 F32, F16, BF16, I32, U32 = 0, 1, 2, 3, 4
 Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q2K, Q3K, Q4K, Q5K, Q6K = 5, 6, 7, 8, 9, 10, 11, 12, 13, 14
+IQ1_S, IQ1_M, IQ2_XXS, IQ2_XS, IQ2_S, IQ3_XXS, IQ3_S = 15, 16, 17, 18, 19, 20, 21
 IQ4_NL, IQ4_XS, TQ1_0, TQ2_0, Q2_0, MXFP4, NVFP4 = 22, 23, 24, 25, 27, 28, 29
 ACT_SILU, ACT_GELU, ACT_SIGMOID = 0, 1, 2
 GATE_SOFTMAX, GATE_SIGMOID, GATE_SQRT_SOFTPLUS = 0, 1, 2
@@ -27,8 +28,9 @@ def build(force: bool = False) -> str:
     """Compile the oracle with the committed Makefile (gcc only, no GPU code)."""
     src = os.path.join(_HERE, "infr_oracle.c")
     hdr = os.path.join(_HERE, "infr_oracle.h")
+    grids = os.path.join(_HERE, "..", "moe4all_amd", "csrc", "iquant_grids.h")
     stale = (not os.path.exists(_LIB_PATH)
-             or os.path.getmtime(_LIB_PATH) < max(os.path.getmtime(src), os.path.getmtime(hdr)))
+             or os.path.getmtime(_LIB_PATH) < max(os.path.getmtime(f) for f in (src, hdr, grids)))
     if force or stale:
         subprocess.check_call(["make", "-C", _HERE, "-B", "libinfr_oracle.so"],
                               stdout=subprocess.DEVNULL)
@@ -107,6 +109,9 @@ def lib() -> C.CDLL:
         L.orc_vec_dot_q8.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int]
         L.orc_vec_dot_q8.restype = C.c_float
         L.orc_hw_threads.restype = C.c_int
+        L.orc_grid_entry.argtypes = [C.c_int, C.c_int, C.c_void_p]
+        L.orc_ksigns.argtypes = [C.c_int]
+        L.orc_ksigns.restype = C.c_uint8
         _lib = L
     return _lib
 
@@ -147,6 +152,26 @@ def k4(j: int, scales) -> tuple:
     sc, m = C.c_uint32(), C.c_uint32()
     lib().orc_k4(j, _p(s), C.byref(sc), C.byref(m))
     return sc.value, m.value
+
+
+GRID_NAMES = ("iq2xxs", "iq2xs", "iq2s", "iq3xxs", "iq3s", "iq1s")
+GRID_SIZES = (256, 512, 1024, 256, 512, 2048)
+
+
+def grid(which: int) -> np.ndarray:
+    """Lattice codebook `which` (index into GRID_NAMES) as [entries, 8 or 4] int8, one signed byte per element as in
+    crates/infr-core/src/iquant_grids.rs."""
+    buf = np.zeros(8, np.int8)
+    rows = []
+    for e in range(GRID_SIZES[which]):
+        n = lib().orc_grid_entry(which, e, _p(buf))
+        rows.append(buf[:n].copy())
+    assert lib().orc_grid_entry(which, GRID_SIZES[which], _p(buf)) == -1
+    return np.stack(rows)
+
+
+def ksigns() -> np.ndarray:
+    return np.array([lib().orc_ksigns(i) for i in range(128)], np.uint8)
 
 
 def dequant(dtype: int, data) -> np.ndarray:

@@ -68,6 +68,14 @@ int orc_block_geometry(int dtype, int *block_elems, int *block_bytes) {
     case ORC_Q2_0: e = 64; b = 18; break;
     case ORC_MXFP4: e = 32; b = 17; break;
     case ORC_NVFP4: e = 64; b = 36; break;
+    /* decode_spec.rs:334-347 */
+    case ORC_IQ1_S: e = 256; b = 50; break;
+    case ORC_IQ1_M: e = 256; b = 56; break;
+    case ORC_IQ2_XXS: e = 256; b = 66; break;
+    case ORC_IQ2_XS: e = 256; b = 74; break;
+    case ORC_IQ2_S: e = 256; b = 82; break;
+    case ORC_IQ3_XXS: e = 256; b = 98; break;
+    case ORC_IQ3_S: e = 256; b = 110; break;
     default: return -1;
     }
     if (block_elems) *block_elems = e;
@@ -358,6 +366,173 @@ static int codebook_block(int dtype, const uint8_t *blk, float *out) {
     }
 }
 
+/* ------------------------------------------------------------------ grid i-quants */
+
+/* The lattice codebooks (crates/infr-core/src/iquant_grids.rs) in the packed form the device library
+ * uses: 2 or 3 bits per element into a small alphabet.  grid_entry() widens entry e back to the
+ * reference's representation, one signed byte per element. */
+#include "../moe4all_amd/csrc/iquant_grids.h"
+
+enum { GRID_IQ2XXS, GRID_IQ2XS, GRID_IQ2S, GRID_IQ3XXS, GRID_IQ3S, GRID_IQ1S };
+static const int8_t ALPHA_IQ2[3] = {8, 25, 43}, ALPHA_IQ3XXS[8] = {4, 12, 20, 28, 36, 44, 52, 62},
+                    ALPHA_IQ3S[8] = {1, 3, 5, 7, 9, 11, 13, 15}, ALPHA_IQ1[3] = {0, 1, -1};
+
+int orc_grid_entry(int grid, int e, int8_t *out) {
+    const uint16_t *t;
+    const int8_t *alpha;
+    int n, bits, size;
+    switch (grid) {
+    case GRID_IQ2XXS: t = kIq2xxsGrid; size = 256; alpha = ALPHA_IQ2; n = 8; bits = 2; break;
+    case GRID_IQ2XS: t = kIq2xsGrid; size = 512; alpha = ALPHA_IQ2; n = 8; bits = 2; break;
+    case GRID_IQ2S: t = kIq2sGrid; size = 1024; alpha = ALPHA_IQ2; n = 8; bits = 2; break;
+    case GRID_IQ3XXS: t = kIq3xxsGrid; size = 256; alpha = ALPHA_IQ3XXS; n = 4; bits = 3; break;
+    case GRID_IQ3S: t = kIq3sGrid; size = 512; alpha = ALPHA_IQ3S; n = 4; bits = 3; break;
+    case GRID_IQ1S: t = kIq1sGrid; size = 2048; alpha = ALPHA_IQ1; n = 8; bits = 2; break;
+    default: return -1;
+    }
+    if (e < 0 || e >= size) return -1;
+    for (int j = 0; j < n; j++) out[j] = alpha[(t[e] >> (bits * j)) & ((1 << bits) - 1)];
+    return n;
+}
+
+/* KSIGNS_IQ2XS[i]: i with bit 7 set so that the number of one bits is even. */
+uint8_t orc_ksigns(int i) { return (uint8_t)(i | ((__builtin_popcount((unsigned)i) & 1) << 7)); }
+
+/* apply_signs (dequant.rs:477-488): out[j] = db * grid[j] * (bit sign_off + j of signs ? -1 : 1) */
+static void apply_signs(float *out, const int8_t *grid, uint8_t signs, int sign_off, int n, float db) {
+    for (int j = 0; j < n; j++) out[j] = db * (float)grid[j] * ((signs >> (sign_off + j)) & 1 ? -1.0f : 1.0f);
+}
+
+#define IQ1S_DELTA 0.125f /* dequant.rs:405 */
+
+static int iquant_block(int dtype, const uint8_t *blk, float *out) {
+    int8_t g[8], g2[8];
+    switch (dtype) {
+    case ORC_IQ2_XXS: { /* :565-596 */
+        float d = orc_f16_to_f32(rd_u16(blk));
+        const uint8_t *qs = blk + 2;
+        for (int ib32 = 0; ib32 < 8; ib32++) {
+            uint32_t aux0 = rd_u32(qs + 8 * ib32), aux1 = rd_u32(qs + 8 * ib32 + 4);
+            float db = d * (0.5f + (float)(aux1 >> 28)) * 0.25f;
+            for (int l = 0; l < 4; l++) {
+                orc_grid_entry(GRID_IQ2XXS, (aux0 >> (8 * l)) & 0xFF, g);
+                apply_signs(out, g, orc_ksigns((aux1 >> (7 * l)) & 127), 0, 8, db);
+                out += 8;
+            }
+        }
+        return 0;
+    }
+    case ORC_IQ2_XS: { /* :605-636 */
+        float d = orc_f16_to_f32(rd_u16(blk));
+        const uint8_t *qs = blk + 2, *scales = blk + 66;
+        for (int ib32 = 0; ib32 < 8; ib32++) {
+            float db0 = d * (0.5f + (float)(scales[ib32] & 0xF)) * 0.25f;
+            float db1 = d * (0.5f + (float)(scales[ib32] >> 4)) * 0.25f;
+            for (int l = 0; l < 4; l++) {
+                unsigned q = rd_u16(qs + 2 * (4 * ib32 + l));
+                orc_grid_entry(GRID_IQ2XS, q & 511, g);
+                apply_signs(out, g, orc_ksigns(q >> 9), 0, 8, l < 2 ? db0 : db1);
+                out += 8;
+            }
+        }
+        return 0;
+    }
+    case ORC_IQ2_S: { /* :642-676 */
+        float d = orc_f16_to_f32(rd_u16(blk));
+        const uint8_t *qs = blk + 2, *qh = blk + 66, *scales = blk + 74;
+        for (int ib32 = 0; ib32 < 8; ib32++) {
+            float db0 = d * (0.5f + (float)(scales[ib32] & 0xF)) * 0.25f;
+            float db1 = d * (0.5f + (float)(scales[ib32] >> 4)) * 0.25f;
+            for (int l = 0; l < 4; l++) {
+                int idx = qs[4 * ib32 + l] | (((unsigned)qh[ib32] << (8 - 2 * l)) & 0x300);
+                orc_grid_entry(GRID_IQ2S, idx, g);
+                apply_signs(out, g, qs[32 + 4 * ib32 + l], 0, 8, l < 2 ? db0 : db1);
+                out += 8;
+            }
+        }
+        return 0;
+    }
+    case ORC_IQ3_XXS: { /* :685-714 */
+        float d = orc_f16_to_f32(rd_u16(blk));
+        const uint8_t *qs = blk + 2, *sas = blk + 66;
+        for (int ib32 = 0; ib32 < 8; ib32++) {
+            uint32_t aux = rd_u32(sas + 4 * ib32);
+            float db = d * (0.5f + (float)(aux >> 28)) * 0.5f;
+            for (int l = 0; l < 4; l++) {
+                uint8_t signs = orc_ksigns((aux >> (7 * l)) & 127);
+                orc_grid_entry(GRID_IQ3XXS, qs[2 * l], g);
+                orc_grid_entry(GRID_IQ3XXS, qs[2 * l + 1], g2);
+                apply_signs(out, g, signs, 0, 4, db);
+                apply_signs(out + 4, g2, signs, 4, 4, db);
+                out += 8;
+            }
+            qs += 8;
+        }
+        return 0;
+    }
+    case ORC_IQ3_S: { /* :724-781: the reference walks pairs of sub-blocks; sub-block ib takes nibble ib % 2 of scales[ib / 2] */
+        float d = orc_f16_to_f32(rd_u16(blk));
+        const uint8_t *qs = blk + 2, *qh = blk + 66, *signs = blk + 74, *scales = blk + 106;
+        for (int ib32 = 0; ib32 < 8; ib32++) {
+            int nib = ib32 % 2 ? scales[ib32 / 2] >> 4 : scales[ib32 / 2] & 0xF;
+            float db = d * (1.0f + 2.0f * (float)nib);
+            for (int l = 0; l < 4; l++) {
+                int i1 = qs[2 * l] | (((unsigned)qh[ib32] << (8 - 2 * l)) & 256);
+                int i2 = qs[2 * l + 1] | (((unsigned)qh[ib32] << (7 - 2 * l)) & 256);
+                orc_grid_entry(GRID_IQ3S, i1, g);
+                orc_grid_entry(GRID_IQ3S, i2, g2);
+                apply_signs(out, g, signs[l], 0, 4, db);
+                apply_signs(out + 4, g2, signs[l], 4, 4, db);
+                out += 8;
+            }
+            qs += 8;
+            signs += 4;
+        }
+        return 0;
+    }
+    case ORC_IQ1_S: { /* :789-824 */
+        float d = orc_f16_to_f32(rd_u16(blk));
+        const uint8_t *qs = blk + 2, *qh_raw = blk + 34;
+        for (int ib = 0; ib < 8; ib++) {
+            unsigned qh = rd_u16(qh_raw + 2 * ib);
+            float dl = d * (2.0f * (float)((qh >> 12) & 7) + 1.0f);
+            float delta = qh & 0x8000 ? -IQ1S_DELTA : IQ1S_DELTA;
+            for (int l = 0; l < 4; l++) {
+                orc_grid_entry(GRID_IQ1S, qs[l] | (((qh >> (3 * l)) & 7) << 8), g);
+                for (int j = 0; j < 8; j++) out[j] = dl * ((float)g[j] + delta);
+                out += 8;
+            }
+            qs += 4;
+        }
+        return 0;
+    }
+    case ORC_IQ1_M: { /* :838-916 */
+        const uint8_t *qs = blk, *qh = blk + 32;
+        unsigned sc[4];
+        for (int i = 0; i < 4; i++) sc[i] = rd_u16(blk + 48 + 2 * i);
+        uint16_t d_bits = (uint16_t)((sc[0] >> 12) | ((sc[1] >> 8) & 0x00F0) | ((sc[2] >> 4) & 0x0F00) | (sc[3] & 0xF000));
+        float d = orc_f16_to_f32(d_bits);
+        for (int ib = 0; ib < 8; ib++) {
+            float dl1 = d * (2.0f * (float)((sc[ib / 2] >> (6 * (ib % 2))) & 7) + 1.0f);
+            float dl2 = d * (2.0f * (float)((sc[ib / 2] >> (6 * (ib % 2) + 3)) & 7) + 1.0f);
+            int idx[4] = {qs[0] | (((unsigned)qh[0] << 8) & 0x700), qs[1] | (((unsigned)qh[0] << 4) & 0x700),
+                          qs[2] | (((unsigned)qh[1] << 8) & 0x700), qs[3] | (((unsigned)qh[1] << 4) & 0x700)};
+            float delta[4] = {qh[0] & 0x08 ? -IQ1S_DELTA : IQ1S_DELTA, qh[0] & 0x80 ? -IQ1S_DELTA : IQ1S_DELTA,
+                              qh[1] & 0x08 ? -IQ1S_DELTA : IQ1S_DELTA, qh[1] & 0x80 ? -IQ1S_DELTA : IQ1S_DELTA};
+            for (int l = 0; l < 4; l++) {
+                orc_grid_entry(GRID_IQ1S, idx[l], g);
+                for (int j = 0; j < 8; j++) out[j] = (l < 2 ? dl1 : dl2) * ((float)g[j] + delta[l]);
+                out += 8;
+            }
+            qs += 4;
+            qh += 2;
+        }
+        return 0;
+    }
+    default: return -1;
+    }
+}
+
 /* dequant.rs:336-363: Q4_K's layout with 32 bytes of fifth bits between the scales and the
  * nibbles: bit 2j of qh[l] belongs to the low-nibble element, bit 2j+1 to the high-nibble one. */
 static void factor_q5k(const uint8_t *blk, factored_block *f) {
@@ -421,7 +596,7 @@ int64_t orc_dequant(int dtype, const uint8_t *bytes, size_t nbytes, float *out) 
         case ORC_Q4K: factor_q4k(blk, &f); break;
         case ORC_Q6K: factor_q6k(blk, &f); break;
         default:
-            if (codebook_block(dtype, blk, out + b * (size_t)be) != 0) return -1;
+            if (codebook_block(dtype, blk, out + b * (size_t)be) != 0 && iquant_block(dtype, blk, out + b * (size_t)be) != 0) return -1;
             continue;
         }
         expand_block(&f, be, out + b * (size_t)be);

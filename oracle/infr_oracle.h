@@ -27,6 +27,7 @@ enum orc_dtype {
     ORC_F32 = 0, ORC_F16 = 1, ORC_BF16 = 2, ORC_I32 = 3, ORC_U32 = 4,
     ORC_Q4_0 = 5, ORC_Q4_1 = 6, ORC_Q5_0 = 7, ORC_Q5_1 = 8, ORC_Q8_0 = 9,
     ORC_Q2K = 10, ORC_Q3K = 11, ORC_Q4K = 12, ORC_Q5K = 13, ORC_Q6K = 14,
+    ORC_IQ1_S = 15, ORC_IQ1_M = 16, ORC_IQ2_XXS = 17, ORC_IQ2_XS = 18, ORC_IQ2_S = 19, ORC_IQ3_XXS = 20, ORC_IQ3_S = 21,
     ORC_IQ4_NL = 22, ORC_IQ4_XS = 23, ORC_TQ1_0 = 24, ORC_TQ2_0 = 25, ORC_Q2_0 = 27, ORC_MXFP4 = 28, ORC_NVFP4 = 29
 };
 /* infr_core::graph::Activation (graph.rs:47-54) and MoeGating (graph.rs:73-85). */
@@ -36,6 +37,11 @@ enum orc_gating { ORC_GATE_SOFTMAX = 0, ORC_GATE_SIGMOID = 1, ORC_GATE_SQRT_SOFT
 /* Block geometry (crates/infr-core/src/decode_spec.rs:320,327,331).  Returns 0, or -1 for a
  * dtype this oracle does not decode.  Float dtypes report 1 element per "block". */
 int orc_block_geometry(int dtype, int *block_elems, int *block_bytes);
+/* Entry e of lattice codebook `grid` (0 IQ2_XXS, 1 IQ2_XS, 2 IQ2_S, 3 IQ3_XXS, 4 IQ3_S, 5 IQ1_S) as signed bytes, in the
+ * representation of crates/infr-core/src/iquant_grids.rs; returns the entry's length (8 or 4), -1 out of range. */
+int orc_grid_entry(int grid, int e, int8_t *out);
+/* KSIGNS_IQ2XS[i] of the same file, i in 0..127. */
+uint8_t orc_ksigns(int i);
 /* Bytes of `numel` elements of `dtype` (numel must be a whole number of blocks); -1 on error. */
 int64_t orc_bytes_for(int dtype, int64_t numel);
 

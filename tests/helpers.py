@@ -7,15 +7,20 @@ import numpy as np
 
 F32, F16, BF16 = 0, 1, 2
 Q4_0, Q4_1, Q5_0, Q5_1, Q8_0, Q2K, Q3K, Q4K, Q5K, Q6K = 5, 6, 7, 8, 9, 10, 11, 12, 13, 14
+IQ1_S, IQ1_M, IQ2_XXS, IQ2_XS, IQ2_S, IQ3_XXS, IQ3_S = 15, 16, 17, 18, 19, 20, 21
 IQ4_NL, IQ4_XS, TQ1_0, TQ2_0, Q2_0, MXFP4, NVFP4 = 22, 23, 24, 25, 27, 28, 29
+GRID_IQUANTS = (IQ1_S, IQ1_M, IQ2_XXS, IQ2_XS, IQ2_S, IQ3_XXS, IQ3_S)   # groups of 8 elements drawn from a lattice codebook
 SCALE_CODE = (IQ4_NL, IQ4_XS, TQ1_0, TQ2_0, Q2_0, MXFP4, NVFP4)   # value = scale * small signed code
 BLOCK = {IQ4_NL: (32, 18), IQ4_XS: (256, 136), TQ1_0: (256, 54), TQ2_0: (256, 66), Q2_0: (64, 18), MXFP4: (32, 17),
          NVFP4: (64, 36),
+         IQ1_S: (256, 50), IQ1_M: (256, 56), IQ2_XXS: (256, 66), IQ2_XS: (256, 74), IQ2_S: (256, 82), IQ3_XXS: (256, 98),
+         IQ3_S: (256, 110),
          Q8_0: (32, 34), Q4K: (256, 144), Q6K: (256, 210), F32: (1, 4), F16: (1, 2), BF16: (1, 2),
          Q4_0: (32, 18), Q4_1: (32, 20), Q5_0: (32, 22), Q5_1: (32, 24), Q2K: (256, 84), Q3K: (256, 110), Q5K: (256, 176)}
 # byte offsets of the f16 scale fields inside a block
 F16_SLOTS = {Q4_0: (0,), Q4_1: (0, 2), Q5_0: (0,), Q5_1: (0, 2), Q8_0: (0,), Q2K: (80, 82), Q3K: (108,), Q4K: (0, 2),
-             Q5K: (0, 2), Q6K: (208,), IQ4_NL: (0,), IQ4_XS: (0,), TQ1_0: (52,), TQ2_0: (64,), Q2_0: (0,)}
+             Q5K: (0, 2), Q6K: (208,), IQ4_NL: (0,), IQ4_XS: (0,), TQ1_0: (52,), TQ2_0: (64,), Q2_0: (0,),
+             IQ1_S: (0,), IQ2_XXS: (0,), IQ2_XS: (0,), IQ2_S: (0,), IQ3_XXS: (0,), IQ3_S: (0,)}
 
 
 # ---- generators of the reference's tests ------------------------------------------------
@@ -32,6 +37,14 @@ def lcg_bytes_blocks(seed: int, nblk: int, nbytes: int) -> np.ndarray:
 
 def f16_bytes(v: float) -> np.ndarray:
     return np.array([v], np.float16).view(np.uint8)
+
+
+def iq1m_set_d(blk: np.ndarray, v: float) -> None:
+    """IQ1_M has no d field: the f16 is cut into four nibbles that sit on top of the four u16 scale words
+    (the inverse of the extraction at crates/infr-gguf/src/dequant.rs:854-856)."""
+    bits = int(np.array([v], np.float16).view(np.uint16)[0])
+    for i in range(4):
+        blk[:, 48 + 2 * i + 1] = (blk[:, 48 + 2 * i + 1] & 0x0F) | (((bits >> (4 * i)) & 0xF) << 4)
 
 
 def synth_weight(dtype: int, n_elem: int, seed: int) -> np.ndarray:
@@ -60,6 +73,9 @@ def synth_weight(dtype: int, n_elem: int, seed: int) -> np.ndarray:
         # LCG nibbles, the four sub-block scales with exponent field 0..3 (subnormal and normal, up to 2^-4)
         blk = lcg_bytes_blocks(seed, nblk, bb)
         blk[:, 0:4] &= 0x1F
+    elif dtype == IQ1_M:
+        blk = lcg_bytes_blocks(seed, nblk, bb)
+        iq1m_set_d(blk, 0.03)   # the d the reference's own IQ1_M test writes (crates/infr-core/src/decode_spec.rs:554)
     elif dtype in F16_SLOTS:
         # the remaining affine formats: LCG payload everywhere, then finite scales of either sign
         blk = lcg_bytes_blocks(seed, nblk, bb)
@@ -77,11 +93,17 @@ def centred_weight(dtype: int, n_elem: int, seed: int, band: float = 0.02) -> np
     blk = synth_weight(dtype, n_elem, seed).reshape(-1, BLOCK[dtype][1])
     if dtype in (MXFP4, NVFP4):   # symmetric books, scales already of that order
         return blk.reshape(-1)
+    if dtype == IQ1_M:            # ternary grid times an odd multiplier of mean 8
+        iq1m_set_d(blk, band / 8)
+        return blk.reshape(-1)
     # (d, second scale) per format; code ranges: q4 0..15, q5 0..31, 6-bit sub-scales mean 31.5, 4-bit 7.5
     d2 = {Q4_0: (band / 4,), Q5_0: (band / 8,), Q8_0: (band / 64,), Q4_1: (band / 4, -7.5 * band / 4),
           Q5_1: (band / 8, -15.5 * band / 8), Q2K: (band / 8, 1.5 * band / 8), Q3K: (band / 32,),
           Q4K: (band / 128, 7.5 * band / 128), Q5K: (band / 256, 15.5 * band / 256), Q6K: (band / 1024,),
-          IQ4_NL: (band / 64,), IQ4_XS: (band / 1024,), TQ1_0: (band,), TQ2_0: (band,), Q2_0: (band,)}[dtype]
+          IQ4_NL: (band / 64,), IQ4_XS: (band / 1024,), TQ1_0: (band,), TQ2_0: (band,), Q2_0: (band,),
+          # signed lattice magnitudes (~25, ~30, ~8, ~1) times a sub-block multiplier of mean 2, 4, 16, 8
+          IQ2_XXS: (band / 64,), IQ2_XS: (band / 64,), IQ2_S: (band / 64,), IQ3_XXS: (band / 128,), IQ3_S: (band / 128,),
+          IQ1_S: (band / 8,)}[dtype]
     for off, v in zip(F16_SLOTS[dtype], d2):
         blk[:, off:off + 2] = f16_bytes(v)
     return blk.reshape(-1)
@@ -298,6 +320,129 @@ def ggml_dequant(dtype: int, data: np.ndarray) -> np.ndarray:
         y = np.concatenate([digits(blk[:, 0:32], 5).reshape(nb, -1), digits(blk[:, 32:48], 5).reshape(nb, -1),
                             digits(blk[:, 48:52], 4).reshape(nb, -1)], axis=1)
         return ((y - 1) * _f16(blk[:, 52:54])[:, None]).reshape(-1)
+    if dtype in GRID_IQUANTS:
+        return _ggml_dequant_iquant(dtype, blk)
+    raise ValueError(dtype)
+
+
+# ---- lattice codebooks of the grid i-quants -------------------------------------------------
+_GRID_ALPHABET = {"kIq2xxsGrid": (8, 25, 43), "kIq2xsGrid": (8, 25, 43), "kIq2sGrid": (8, 25, 43),
+                  "kIq3xxsGrid": (4, 12, 20, 28, 36, 44, 52, 62), "kIq3sGrid": (1, 3, 5, 7, 9, 11, 13, 15),
+                  "kIq1sGrid": (0, 1, -1)}
+_GRIDS: dict = {}
+
+
+def iquant_grid(name: str) -> np.ndarray:
+    """Codebook `name` of moe4all_amd/csrc/iquant_grids.h widened to [entries, 8 or 4] int64 (a second reader of the
+    packed table, separate from the C one the oracle and the device use)."""
+    if not _GRIDS:
+        import os
+        import re
+        path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "..", "moe4all_amd", "csrc", "iquant_grids.h")
+        for m in re.finditer(r"uint16_t (\w+)\[(\d+)\] = \{(.*?)\};", open(path).read(), re.S):
+            vals = np.array([int(v, 16) for v in re.findall(r"0x[0-9a-f]+", m.group(3))], np.int64)
+            assert len(vals) == int(m.group(2))
+            alpha = np.array(_GRID_ALPHABET[m.group(1)], np.int64)
+            bits, n = (2, 8) if len(alpha) == 3 else (3, 4)
+            digits = (vals[:, None] >> (bits * np.arange(n))) & ((1 << bits) - 1)
+            assert digits.max() < len(alpha)
+            _GRIDS[m.group(1)] = alpha[digits]
+    return _GRIDS[name]
+
+
+def ksigns() -> np.ndarray:
+    """ggml's ksigns_iq2xs: entry i = i with bit 7 completing an even number of one bits."""
+    i = np.arange(128, dtype=np.int64)
+    par = np.zeros(128, np.int64)
+    for b in range(7):
+        par ^= (i >> b) & 1
+    return i | (par << 7)
+
+
+def _signs(byte: np.ndarray) -> np.ndarray:
+    """[...] sign bytes -> [..., 8] factors: bit j set means element j is negated (ggml's kmask_iq2xs[j] = 1 << j)."""
+    return 1 - 2 * ((byte[..., None] >> np.arange(8)) & 1)
+
+
+def _ggml_dequant_iquant(dtype: int, blk: np.ndarray) -> np.ndarray:
+    """ggml's dequantize_row_iq2_xxs / iq2_xs / iq2_s / iq3_xxs / iq3_s / iq1_s / iq1_m, vectorised over blocks:
+    [blocks, 8 sub-blocks of 32, 4 groups, 8 elements]."""
+    nb = blk.shape[0]
+    L = np.longdouble
+    u8 = blk.astype(np.int64)
+
+    def u16(a):   # [..., 2k] bytes -> [..., k] little-endian words
+        return a[..., 0::2] | (a[..., 1::2] << 8)
+
+    def u32(a):
+        return a[..., 0::4] | (a[..., 1::4] << 8) | (a[..., 2::4] << 16) | (a[..., 3::4] << 24)
+
+    l4 = np.arange(4)
+    if dtype == IQ2_XXS:
+        d = _f16(blk[:, 0:2])
+        q = u8[:, 2:66].reshape(nb, 8, 8)
+        aux1 = u32(q[:, :, 4:8])[:, :, 0]                                  # [nb, 8]
+        db = d[:, None] * (L(0.5) + (aux1 >> 28)) * L(0.25)
+        g = iquant_grid("kIq2xxsGrid")[q[:, :, 0:4]]                       # [nb, 8, 4, 8]
+        sg = _signs(ksigns()[(aux1[:, :, None] >> (7 * l4)) & 127])
+        return (db[:, :, None, None] * g * sg).reshape(-1)
+    if dtype in (IQ2_XS, IQ2_S):
+        d = _f16(blk[:, 0:2])
+        if dtype == IQ2_XS:
+            q = u16(u8[:, 2:66]).reshape(nb, 8, 4)
+            g = iquant_grid("kIq2xsGrid")[q & 511]
+            sg = _signs(ksigns()[q >> 9])
+            sc = u8[:, 66:74]
+        else:
+            qs = u8[:, 2:34].reshape(nb, 8, 4)
+            qh = u8[:, 66:74]
+            idx = qs | ((qh[:, :, None] << (8 - 2 * l4)) & 0x300)
+            g = iquant_grid("kIq2sGrid")[idx]
+            sg = _signs(u8[:, 34:66].reshape(nb, 8, 4))
+            sc = u8[:, 74:82]
+        db = d[:, None, None] * (L(0.5) + np.stack([sc & 0xF, sc & 0xF, sc >> 4, sc >> 4], axis=2)) * L(0.25)   # [nb, 8, 4]
+        return (db[:, :, :, None] * g * sg).reshape(-1)
+    if dtype == IQ3_XXS:
+        d = _f16(blk[:, 0:2])
+        q = u8[:, 2:66].reshape(nb, 8, 4, 2)
+        aux = u32(u8[:, 66:98])                                            # [nb, 8]
+        db = d[:, None] * (L(0.5) + (aux >> 28)) * L(0.5)
+        g = iquant_grid("kIq3xxsGrid")[q].reshape(nb, 8, 4, 8)             # the two 4-element entries side by side
+        sg = _signs(ksigns()[(aux[:, :, None] >> (7 * l4)) & 127])
+        return (db[:, :, None, None] * g * sg).reshape(-1)
+    if dtype == IQ3_S:
+        d = _f16(blk[:, 0:2])
+        q = u8[:, 2:66].reshape(nb, 8, 4, 2)
+        qh = u8[:, 66:74]
+        hi = np.stack([(qh[:, :, None] << (8 - 2 * l4)) & 256, (qh[:, :, None] << (7 - 2 * l4)) & 256], axis=3)
+        g = iquant_grid("kIq3sGrid")[q | hi].reshape(nb, 8, 4, 8)
+        sg = _signs(u8[:, 74:106].reshape(nb, 8, 4))
+        sc = u8[:, 106:110]
+        nib = np.stack([sc & 0xF, sc >> 4], axis=2).reshape(nb, 8)
+        db = d[:, None] * (1 + 2 * nib)
+        return (db[:, :, None, None] * g * sg).reshape(-1)
+    if dtype == IQ1_S:
+        d = _f16(blk[:, 0:2])
+        qs = u8[:, 2:34].reshape(nb, 8, 4)
+        qh = u16(u8[:, 34:50])                                             # [nb, 8]
+        dl = d[:, None] * (2 * ((qh >> 12) & 7) + 1)
+        delta = np.where(qh & 0x8000, L(-0.125), L(0.125))
+        g = iquant_grid("kIq1sGrid")[qs | (((qh[:, :, None] >> (3 * l4)) & 7) << 8)]
+        return (dl[:, :, None, None] * (g + delta[:, :, None, None])).reshape(-1)
+    if dtype == IQ1_M:
+        sc = u16(u8[:, 48:56])                                             # [nb, 4]
+        dbits = (sc[:, 0] >> 12) | ((sc[:, 1] >> 8) & 0x00F0) | ((sc[:, 2] >> 4) & 0x0F00) | (sc[:, 3] & 0xF000)
+        d = dbits.astype(np.uint16).view(np.float16).astype(L)
+        ib = np.arange(8)
+        s3 = np.stack([(sc[:, ib // 2] >> (6 * (ib % 2))) & 7, (sc[:, ib // 2] >> (6 * (ib % 2) + 3)) & 7], axis=2)   # [nb, 8, 2]
+        dl = (d[:, None, None] * (2 * s3 + 1))[:, :, [0, 0, 1, 1]]          # [nb, 8, 4]
+        qs = u8[:, 0:32].reshape(nb, 8, 4)
+        qh = u8[:, 32:48].reshape(nb, 8, 2)[:, :, [0, 0, 1, 1]]
+        odd = (l4 & 1).astype(bool)
+        idx = qs | np.where(odd, (qh << 4) & 0x700, (qh << 8) & 0x700)
+        delta = np.where(qh & np.where(odd, 0x80, 0x08), L(-0.125), L(0.125))
+        g = iquant_grid("kIq1sGrid")[idx]
+        return (dl[:, :, :, None] * (g + delta[:, :, :, None])).reshape(-1)
     raise ValueError(dtype)
 
 
@@ -417,6 +562,15 @@ def dequant_cases():
             b[0::17] = 64 + (b[0::17] >> 1)
         out[f"{name}_pattern"] = (dt, b)
         out[f"{name}_lcg"] = (dt, synth_weight(dt, BLOCK[dt][0] * 8, 100 + dt))
+    # the grid i-quants: the (i*29+3)&0xFF pattern over two blocks (IQ1_M: with the d nibbles of its own test) and
+    # LCG blocks, which reach every codebook with arbitrary indices, sign bytes and multipliers
+    for name, dt in (("iq1_s", IQ1_S), ("iq1_m", IQ1_M), ("iq2_xxs", IQ2_XXS), ("iq2_xs", IQ2_XS), ("iq2_s", IQ2_S),
+                     ("iq3_xxs", IQ3_XXS), ("iq3_s", IQ3_S)):
+        b = pattern(2 * BLOCK[dt][1], 29, 3)
+        if dt == IQ1_M:
+            iq1m_set_d(b.reshape(2, -1), 0.03)
+        out[f"{name}_pattern"] = (dt, b)
+        out[f"{name}_lcg"] = (dt, synth_weight(dt, 256 * 8, 100 + dt))
     for name, (dt, b, _) in known_answer_blocks().items():
         out[name] = (dt, b)
     return out
@@ -473,6 +627,14 @@ def known_answer_blocks():
     b[0:2] = f16_bytes(0.5)
     b[2] = 0b11100100
     out["q2_0_single_block"] = (Q2_0, b, {0: -0.5, 1: 0.0, 2: 0.5, 3: 1.0, **{i: -0.5 for i in range(4, 64)}})
+    # the grid i-quants (dequant.rs:1290-1308, :1355-1363, :1495-1617): all-zero payload, d = 1 -> entry 0 of the codebook,
+    # no sign set, smallest multiplier
+    for name, dt, v in (("iq2xxs", IQ2_XXS, 1.0), ("iq2xs", IQ2_XS, 1.0), ("iq2s", IQ2_S, 1.0), ("iq3xxs", IQ3_XXS, 1.0),
+                        ("iq3s", IQ3_S, 1.0), ("iq1s", IQ1_S, -0.875)):
+        b = np.zeros(BLOCK[dt][1], np.uint8)
+        b[0:2] = f16_bytes(1.0)
+        out[f"{name}_single_block"] = (dt, b, {i: v for i in range(256)})
+    out["iq1m_single_block"] = (IQ1_M, np.zeros(56, np.uint8), {i: 0.0 for i in range(256)})
     return out
 
 

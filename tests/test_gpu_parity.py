@@ -97,7 +97,7 @@ def test_dequant_matches_golden_bits(be):
 
 
 AFFINE = [H.Q4_0, H.Q4_1, H.Q5_0, H.Q5_1, H.Q8_0, H.Q2K, H.Q3K, H.Q4K, H.Q5K, H.Q6K]
-DECODED = AFFINE + list(H.SCALE_CODE)   # every block format the device decodes
+DECODED = AFFINE + list(H.SCALE_CODE) + list(H.GRID_IQUANTS)   # every block format the device decodes
 
 
 @pytest.mark.parametrize("dt", DECODED)
@@ -115,7 +115,9 @@ def test_dequant_matches_oracle_bits_on_a_large_tensor(be, dt):
                                      (H.Q8_0, 4096), (H.Q8_0, 96), (H.Q4K, 5120), (H.F16, 100), (H.Q4_0, 96), (H.Q4_1, 2048),
                                      (H.Q5_0, 160), (H.Q5_1, 1024), (H.Q2K, 512), (H.Q3K, 768), (H.Q5K, 2048),
                                      (H.IQ4_NL, 96), (H.IQ4_XS, 512), (H.TQ1_0, 256), (H.TQ1_0, 1024), (H.TQ2_0, 768),
-                                     (H.Q2_0, 192), (H.MXFP4, 2880), (H.MXFP4, 160), (H.NVFP4, 320)])
+                                     (H.Q2_0, 192), (H.MXFP4, 2880), (H.MXFP4, 160), (H.NVFP4, 320), (H.IQ1_S, 512),
+                                     (H.IQ1_M, 256), (H.IQ2_XXS, 768), (H.IQ2_XS, 256), (H.IQ2_S, 1024), (H.IQ3_XXS, 512),
+                                     (H.IQ3_S, 2048)])
 def test_one_hot_gemv_reads_back_the_decoded_weight(be, dt, in_f):
     """x = e_c makes y[o] = W[o][c]: the in-register unpacking of the GEMV kernels must reproduce
     the reference decode exactly (same trick as crates/infr-vulkan/tests/weight_dequant_parity.rs)."""
@@ -262,6 +264,26 @@ def _bank_weights(rng, E, nff, ne, gdt, ddt):
         return _realistic(rng, E, nff, ne, gdt), _realistic(rng, E, nff, ne, gdt), _realistic(rng, E, ne, nff, ddt)
     return (H.centred_weight(gdt, E * nff * ne, 1), H.centred_weight(gdt, E * nff * ne, 2),
             H.centred_weight(ddt, E * ne * nff, 3))
+
+
+@pytest.mark.parametrize("rows", [1, 5, 40])
+@pytest.mark.parametrize("gdt,ddt", [(H.IQ2_XXS, H.IQ3_S), (H.IQ1_M, H.IQ2_S), (H.IQ3_XXS, H.IQ2_XS), (H.IQ1_S, H.IQ4_XS)])
+def test_moe_ffn_with_grid_iquant_experts_matches_oracle(be, gdt, ddt, rows):
+    """Expert banks in the lattice-codebook formats (the 1- to 3-bit quantisations MoE checkpoints ship in), one token,
+    a decode batch and a prefill-sized chunk."""
+    ne, E, K, nff = 512, 8, 3, 256
+    rng = np.random.default_rng(rows + gdt)
+    x = rng.standard_normal((rows, ne)).astype(np.float32)
+    router = rng.standard_normal((E, ne)).astype(np.float32) * 0.05
+    gate, up, down = _bank_weights(rng, E, nff, ne, gdt, ddt)
+    g, ids = moe_graph(rows, ne, E, K, nff, DType(gdt), DType(ddt))
+    out, r = run_moe(be, g, ids, dict(x=x, router=router, gate=gate, up=up, down=down), rows, ne)
+    ref = O.moe_ffn(x, router, gate, up, down, ne=ne, n_expert=E, n_used=K, n_ff_exp=nff, gate_dtype=gdt, down_dtype=ddt)
+    assert np.array_equal(r["idx"], ref["idx"])
+    assert float(np.abs(ref["dst"]).max()) > 1e-4, "degenerate case"
+    tol = REL_L2_MFMA if rows >= 32 else REL_L2
+    for row in range(rows):
+        assert H.rel_l2(out.reshape(rows, ne)[row], ref["dst"].reshape(rows, ne)[row]) < tol, row
 
 
 @pytest.mark.parametrize("rows", [3, 1])   # one row: the unit formats' down stage and combine are one launch

@@ -24,6 +24,11 @@ def test_block_geometry_matches_ggml_formulas():
     assert O.block_geometry(O.Q5_0) == (32, 2 + 4 + 16) and O.block_geometry(O.Q5_1) == (32, 2 + 2 + 4 + 16)
     assert O.block_geometry(O.Q2K) == (256, 16 + 64 + 2 + 2) and O.block_geometry(O.Q3K) == (256, 32 + 64 + 12 + 2)
     assert O.block_geometry(O.Q5K) == (256, 2 + 2 + 12 + 32 + 128)
+    # decode_spec.rs:468-474, QK_K = 256
+    assert O.block_geometry(O.IQ1_S) == (256, 2 + 256 // 8 + 256 // 32 * 2) and O.block_geometry(O.IQ1_M) == (256, 256 // 8 + 256 // 16 + 256 // 32)
+    assert O.block_geometry(O.IQ2_XXS) == (256, 2 + 256 // 8 * 2) and O.block_geometry(O.IQ2_XS) == (256, 2 + 256 // 8 * 2 + 256 // 32)
+    assert O.block_geometry(O.IQ2_S) == (256, 2 + 256 // 4 + 256 // 16) and O.block_geometry(O.IQ3_XXS) == (256, 2 + 3 * (256 // 8))
+    assert O.block_geometry(O.IQ3_S) == (256, 2 + 13 * (256 // 32) + 256 // 64)
     assert O.bytes_for(O.Q4K, 768 * 2048) == 884736
     assert O.bytes_for(O.Q6K, 2048 * 768) == 1290240
     assert O.bytes_for(O.Q8_0, 768 * 2048) == 1671168
@@ -67,7 +72,7 @@ def test_k4_inverts_ggml_scale_packing_exhaustively():
 def test_dequant_matches_golden_fixture_bit_for_bit():
     g = np.load(os.path.join(GOLD, "dequant.npz"))
     names = sorted({k.rsplit(".", 1)[0] for k in g.files})
-    assert len(names) == 8 + 14 + 6 + 14 + 7
+    assert len(names) == 8 + 14 + 6 + 14 + 7 + 14 + 7
     for n in names:
         got = O.dequant(int(g[n + ".dtype"]), g[n + ".bytes"])
         assert np.array_equal(got.view(np.uint32), g[n + ".bits"]), n
@@ -89,12 +94,127 @@ def test_dequant_gives_the_values_the_reference_tests_assert():
 
 @pytest.mark.parametrize("dt,seed", [(O.Q8_0, 1), (O.Q4K, 2), (O.Q6K, 3), (O.Q4_0, 4), (O.Q4_1, 5), (O.Q5_0, 6), (O.Q5_1, 7),
                                      (O.Q2K, 8), (O.Q3K, 9), (O.Q5K, 10), (O.IQ4_NL, 11), (O.IQ4_XS, 12), (O.TQ1_0, 13),
-                                     (O.TQ2_0, 14), (O.Q2_0, 15), (O.MXFP4, 16), (O.NVFP4, 17)])
+                                     (O.TQ2_0, 14), (O.Q2_0, 15), (O.MXFP4, 16), (O.NVFP4, 17), (O.IQ1_S, 18), (O.IQ1_M, 19),
+                                     (O.IQ2_XXS, 20), (O.IQ2_XS, 21), (O.IQ2_S, 22), (O.IQ3_XXS, 23), (O.IQ3_S, 24)])
 def test_dequant_matches_independent_decoder_on_random_blocks(dt, seed):
     be, bb = O.block_geometry(dt)
     b = H.synth_weight(dt, be * 64, seed)
     want = H.ggml_dequant(dt, b).astype(np.float32)
     assert np.array_equal(O.dequant(dt, b).view(np.uint32), want.view(np.uint32))
+
+
+def test_iquant_codebooks_are_the_reference_tables():
+    """The packed codebooks, widened to one signed byte per element by the C reader (oracle, device) and by the separate
+    Python reader, hash to the digests taken from crates/infr-core/src/iquant_grids.rs when the tables were packed
+    (tests/golden/iquant_grids.json); the sign table is the parity rule, the mask table 1 << j."""
+    import hashlib
+    import json
+    dig = json.load(open(os.path.join(GOLD, "iquant_grids.json")))
+    names = ("kIq2xxsGrid", "kIq2xsGrid", "kIq2sGrid", "kIq3xxsGrid", "kIq3sGrid", "kIq1sGrid")
+    for which, name in enumerate(names):
+        g = O.grid(which)
+        assert g.shape == (dig[name]["entries"], dig[name]["entry_bytes"]) == (O.GRID_SIZES[which], 8 if which in (0, 1, 2, 5) else 4)
+        assert np.array_equal(g, H.iquant_grid(name)), name
+        assert hashlib.sha256(g.astype(np.int8).tobytes()).hexdigest() == dig[name]["sha256"], name
+    assert hashlib.sha256(bytes(O.ksigns())).hexdigest() == dig["KSIGNS_IQ2XS"]["sha256"]
+    assert np.array_equal(O.ksigns(), H.ksigns())
+    assert hashlib.sha256(bytes(1 << j for j in range(8))).hexdigest() == dig["KMASK_IQ2XS"]["sha256"]
+
+
+def test_iquant_codebooks_have_the_structure_ggml_documents():
+    """IQ2 and IQ3 codebooks are sorted lists of distinct lattice points (read as little-endian integers); every IQ2 point
+    has odd coordinates of the form (8, 25, 43) ~ (1, 3, 5) * 8.5, every IQ3_S coordinate is odd, IQ1 is ternary."""
+    for which in range(5):
+        g = O.grid(which).astype(np.int64)
+        as_int = (g << (8 * np.arange(g.shape[1]))).sum(axis=1)
+        assert (np.diff(as_int) > 0).all(), which
+    assert set(np.unique(O.grid(0))) == set(np.unique(O.grid(1))) == set(np.unique(O.grid(2))) == {8, 25, 43}
+    assert set(np.unique(O.grid(3))) == {4, 12, 20, 28, 36, 44, 52, 62}
+    assert set(np.unique(O.grid(4))) == set(range(1, 16, 2))
+    g1 = O.grid(5)
+    assert set(np.unique(g1)) == {-1, 0, 1} and len({tuple(r) for r in g1}) == 2048
+    assert (g1[0] == -1).all()     # the entry the reference's IQ1_S test decodes (dequant.rs:1286)
+    assert (O.grid(0)[0] == 8).all() and (O.grid(3)[0] == 4).all() and (O.grid(4)[0] == 1).all()   # :1490, :1575, :1598
+
+
+def test_iquant_fields_land_where_the_published_layout_puts_them():
+    """One block per format built field by field (not from random bytes): a chosen codebook index, sign pattern and
+    multiplier for one group must come out at that group's eight positions and nowhere else."""
+    def base(dt):
+        b = np.zeros(H.BLOCK[dt][1], np.uint8)
+        if dt == H.IQ1_M:
+            H.iq1m_set_d(b.reshape(1, -1), 1.0)
+        else:
+            b[0:2] = H.f16_bytes(1.0)
+        return b
+    zero = {dt: O.dequant(dt, base(dt)) for dt in H.GRID_IQUANTS}
+    ks = H.ksigns()
+    # IQ2_XXS: sub-block 3, group 2 -> index 0xA7, sign index 0x55, multiplier 9
+    b = base(H.IQ2_XXS)
+    aux0, aux1 = 0xA7 << 16, (0x55 << 14) | (9 << 28)
+    b[2 + 24:2 + 32] = np.frombuffer(np.array([aux0, aux1], "<u4").tobytes(), np.uint8)
+    y = O.dequant(H.IQ2_XXS, b)
+    g = H.iquant_grid("kIq2xxsGrid")
+    sg = 1 - 2 * ((int(ks[0x55]) >> np.arange(8)) & 1)
+    assert np.array_equal(y[96 + 16:96 + 24], (np.float32(9.5 * 0.25) * g[0xA7] * sg).astype(np.float32))
+    assert np.array_equal(y[96:96 + 16], np.full(16, 9.5 * 0.25 * 8, np.float32))        # same multiplier, entry 0
+    assert np.array_equal(np.delete(y, np.arange(96, 128)), np.delete(zero[H.IQ2_XXS], np.arange(96, 128)))
+    # IQ2_XS: sub-block 5, group 3 -> 9-bit index 0x1B3, sign index 0x2A; high nibble of scale byte 5 = 6
+    b = base(H.IQ2_XS)
+    b[2 + 2 * 23:2 + 2 * 24] = np.frombuffer(np.array([0x1B3 | (0x2A << 9)], "<u2").tobytes(), np.uint8)
+    b[66 + 5] = 6 << 4
+    y = O.dequant(H.IQ2_XS, b)
+    sg = 1 - 2 * ((int(ks[0x2A]) >> np.arange(8)) & 1)
+    assert np.array_equal(y[160 + 24:160 + 32], (np.float32(6.5 * 0.25) * H.iquant_grid("kIq2xsGrid")[0x1B3] * sg).astype(np.float32))
+    assert np.array_equal(y[160:160 + 16], zero[H.IQ2_XS][:16])                            # low nibble untouched
+    # IQ2_S: sub-block 1, group 2 -> index 0x2C5 (high bits 2 from qh), sign byte 0x81, low nibble of scale 1 = 3 (not used
+    # by group 2), high nibble 12
+    b = base(H.IQ2_S)
+    b[2 + 4 + 2] = 0xC5
+    b[66 + 1] = 2 << 4
+    b[34 + 4 + 2] = 0x81
+    b[74 + 1] = 3 | (12 << 4)
+    y = O.dequant(H.IQ2_S, b)
+    sg = np.array([-1, 1, 1, 1, 1, 1, 1, -1])
+    assert np.array_equal(y[32 + 16:32 + 24], (np.float32(12.5 * 0.25) * H.iquant_grid("kIq2sGrid")[0x2C5] * sg).astype(np.float32))
+    assert np.array_equal(y[32:32 + 16], np.full(16, 3.5 * 0.25 * 8, np.float32))
+    # IQ3_XXS: sub-block 6, group 1 -> entries 0x9E then 0x31, sign index 0x13, multiplier 4
+    b = base(H.IQ3_XXS)
+    b[2 + 48 + 2], b[2 + 48 + 3] = 0x9E, 0x31
+    b[66 + 24:66 + 28] = np.frombuffer(np.array([(0x13 << 7) | (4 << 28)], "<u4").tobytes(), np.uint8)
+    y = O.dequant(H.IQ3_XXS, b)
+    g = H.iquant_grid("kIq3xxsGrid")
+    sg = 1 - 2 * ((int(ks[0x13]) >> np.arange(8)) & 1)
+    assert np.array_equal(y[192 + 8:192 + 16], (np.float32(4.5 * 0.5) * np.concatenate([g[0x9E], g[0x31]]) * sg).astype(np.float32))
+    # IQ3_S: sub-block 3 (odd: high nibble of scale byte 1), group 2 -> entries 0x1F0 and 0x0F0: ninth bits are bits 4, 5 of qh
+    b = base(H.IQ3_S)
+    b[2 + 24 + 4], b[2 + 24 + 5] = 0xF0, 0xF0
+    b[66 + 3] = 1 << 4
+    b[74 + 12 + 2] = 0x0F
+    b[106 + 1] = 7 << 4
+    y = O.dequant(H.IQ3_S, b)
+    g = H.iquant_grid("kIq3sGrid")
+    assert np.array_equal(y[96 + 16:96 + 24], (np.float32(15.0) * np.concatenate([-g[0x1F0], g[0x0F0]])).astype(np.float32))
+    assert np.array_equal(y[64:96], zero[H.IQ3_S][64:96])                                   # sub-block 2 keeps the low nibble (0)
+    # IQ1_S: sub-block 4, group 3 -> index 0x5A | 6 << 8, multiplier 2 * 5 + 1, negative shift
+    b = base(H.IQ1_S)
+    b[2 + 16 + 3] = 0x5A
+    b[34 + 8:34 + 10] = np.frombuffer(np.array([(6 << 9) | (5 << 12) | 0x8000], "<u2").tobytes(), np.uint8)
+    y = O.dequant(H.IQ1_S, b)
+    g = H.iquant_grid("kIq1sGrid")
+    assert np.array_equal(y[128 + 24:128 + 32], (np.float32(11.0) * (g[0x65A] - 0.125)).astype(np.float32))
+    assert np.array_equal(y[128:128 + 24], np.full(24, 11.0 * (-1 - 0.125), np.float32))
+    # IQ1_M: sub-block 5 (second six bits of scale word 2), group 1 (high nibble of qh[10]) and group 2 (low nibble of qh[11])
+    b = base(H.IQ1_M)
+    b[20 + 1], b[20 + 2] = 0x33, 0x44
+    b[32 + 10], b[32 + 11] = (0x8 | 5) << 4, 3
+    w = int(np.frombuffer(b[52:54].tobytes(), "<u2")[0]) | (2 << 6) | (6 << 9)
+    b[52:54] = np.frombuffer(np.array([w], "<u2").tobytes(), np.uint8)
+    y = O.dequant(H.IQ1_M, b)
+    assert np.array_equal(y[160 + 8:160 + 16], (np.float32(5.0) * (g[0x533] - 0.125)).astype(np.float32))
+    assert np.array_equal(y[160 + 16:160 + 24], (np.float32(13.0) * (g[0x344] + 0.125)).astype(np.float32))
+    assert np.array_equal(y[160:160 + 8], np.full(8, 5.0 * (-1 + 0.125), np.float32))
+    assert np.array_equal(np.delete(y, np.arange(160, 192)), np.delete(zero[H.IQ1_M], np.arange(160, 192)))
 
 
 def test_fp4_scales_match_their_arithmetic_definition_for_every_byte():
