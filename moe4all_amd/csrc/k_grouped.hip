@@ -1089,7 +1089,8 @@ struct StagedW {
                                        : DT == INFR_Q8_0 ? 34 : DT == INFR_Q2K ? 84 : DT == INFR_Q3K ? 110 : DT == INFR_Q4K ? 144
                                        : DT == INFR_Q5K ? 176 : DT == INFR_Q6K ? 210 : DT == INFR_IQ4_NL ? 18 : DT == INFR_IQ4_XS ? 136
                                        : DT == INFR_TQ1_0 ? 54 : DT == INFR_TQ2_0 ? 66 : DT == INFR_Q2_0 ? 18 : DT == INFR_MXFP4 ? 17
-                                       : DT == INFR_NVFP4 ? 36 : 0;
+                                       : DT == INFR_NVFP4 ? 36 : DT == INFR_IQ1_S ? 50 : DT == INFR_IQ1_M ? 56 : DT == INFR_IQ2_XXS ? 66
+                                       : DT == INFR_IQ2_XS ? 74 : DT == INFR_IQ2_S ? 82 : DT == INFR_IQ3_XXS ? 98 : DT == INFR_IQ3_S ? 110 : 0;
     static constexpr int kWB = kBlockBytes * (256 / kBlock);   // bytes of one row in a window of 256 k
     static constexpr int kChunks = (kWB + 15) / 16;
     static constexpr int kPitch = 16 * (kChunks | 1);

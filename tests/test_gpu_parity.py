@@ -277,7 +277,15 @@ def test_moe_ffn_with_grid_iquant_experts_matches_oracle(be, gdt, ddt, rows):
     router = rng.standard_normal((E, ne)).astype(np.float32) * 0.05
     gate, up, down = _bank_weights(rng, E, nff, ne, gdt, ddt)
     g, ids = moe_graph(rows, ne, E, K, nff, DType(gdt), DType(ddt))
+    be.prof_enable(True)
     out, r = run_moe(be, g, ids, dict(x=x, router=router, gate=gate, up=up, down=down), rows, ne)
+    be.sync()
+    names = set(be.prof_read())
+    be.prof_enable(False)
+    # the 32-element unit decoders, not the element-wise kernels: GEMV forms for decode, matrix cores for the chunk
+    want_names = {"moe_grouped_units_gate_up", "moe_grouped_units_down"} if rows >= 32 else \
+        {"moe_route_gate_up_units", "moe_down_combine_units"} if rows == 1 else {"moe_route_gate_up_units", "moe_down_units"}
+    assert want_names <= names, names
     ref = O.moe_ffn(x, router, gate, up, down, ne=ne, n_expert=E, n_used=K, n_ff_exp=nff, gate_dtype=gdt, down_dtype=ddt)
     assert np.array_equal(r["idx"], ref["idx"])
     assert float(np.abs(ref["dst"]).max()) > 1e-4, "degenerate case"
@@ -801,7 +809,10 @@ def test_linear_on_float_weights(be, dt, m, in_f, out_f):
                                              (H.Q4K, 2048, 4096, 1536), (H.Q4_1, 150, 96, 64), (H.F16, 170, 256, 64),
                                              (H.BF16, 130, 320, 100), (H.F32, 260, 128, 300), (H.F16, 140, 100, 64),
                                              (H.Q4K, 100, 512, 64), (H.MXFP4, 160, 2880, 96), (H.IQ4_XS, 130, 512, 64),
-                                             (H.NVFP4, 140, 192, 50), (H.TQ2_0, 128, 256, 40), (H.IQ4_NL, 131, 96, 64)])
+                                             (H.NVFP4, 140, 192, 50), (H.TQ2_0, 128, 256, 40), (H.IQ4_NL, 131, 96, 64),
+                                             (H.IQ2_XXS, 130, 512, 64), (H.IQ2_XS, 129, 256, 40), (H.IQ2_S, 140, 768, 50),
+                                             (H.IQ3_XXS, 128, 256, 96), (H.IQ3_S, 150, 512, 33), (H.IQ1_S, 131, 256, 64),
+                                             (H.IQ1_M, 160, 1024, 48)])
 def test_linear_with_a_batch_of_rows_runs_on_the_matrix_cores(be, dt, m, in_f, out_f):
     """Op::Linear from 128 rows on (a prefill chunk through a dense projection or the shared expert): the rows
     are one bucket of the grouped GEMMs, f16 operands with a power-of-two scale per row, bar 1e-2 per row.
