@@ -255,7 +255,7 @@ def test_moe_ffn_matches_oracle(be, rows, ne, E, K, nff, gdt, ddt):
     scale = float(np.abs(ref["dst"]).max())
     assert scale > 1e-4, "degenerate case"
     assert H.rel_l2(out, ref["dst"]) < REL_L2, H.rel_l2(out, ref["dst"])
-    assert H.max_abs(out, ref["dst"]) < MAX_ABS * max(1.0, scale), (H.max_abs(out, ref["dst"]), scale)
+    assert H.max_abs(out, ref["dst"]) < MAX_ABS, (H.max_abs(out, ref["dst"]), scale)
 
 
 def _bank_weights(rng, E, nff, ne, gdt, ddt):
@@ -1149,7 +1149,7 @@ def test_bucketed_decode_batches_bucket_exactly_and_keep_f32_accuracy(be, rows, 
         _check_bucketing(b, ref, E)
         scale = float(np.abs(ref["dst"]).max())
         assert H.rel_l2(out, ref["dst"]) < REL_L2, (gopts, H.rel_l2(out, ref["dst"]))
-        assert H.max_abs(out, ref["dst"]) < MAX_ABS * max(1.0, scale)
+        assert H.max_abs(out, ref["dst"]) < MAX_ABS, (gopts, H.max_abs(out, ref["dst"]), scale)
 
 
 @pytest.mark.parametrize("rows,opts", [(1, {}), (3, {"weight_before": True}), (20, {}), (20, {"weight_before": True}), (40, {}),
@@ -1281,13 +1281,30 @@ def test_prefill_rows_do_not_depend_on_their_neighbours(be, gdt, ddt):
         be.execute(plan, bnd)
         out = be.download(yb, n * s.ne * 4, np.float32).reshape(n, s.ne).copy()
         idx = be.moe_routing(plan, 0)["idx"].copy()
+        buckets.append(be.moe_bucketing(plan, 0))
         plan.free()
         xb.free()
         yb.free()
         return out, idx
 
+    buckets = []
     full, idx = run(x)
     assert np.isfinite(full).all()
+    # the whole chunk against the oracle: ids and the bucket order of all 2048 tokens bit for bit (they depend on the
+    # router alone, so the oracle runs with one-feature dummy experts), and the output rows of a sample of 96 tokens
+    # (the oracle on x[sample] alone: rows are independent, which the rest of this test shows for the device)
+    dummy = np.zeros(s.n_expert * s.ne, np.float32)
+    rt = O.moe_ffn(x, router, dummy, dummy, dummy, ne=s.ne, n_expert=s.n_expert, n_used=s.n_used, n_ff_exp=1)
+    assert np.array_equal(idx, rt["idx"])
+    _check_bucketing(buckets[0], rt, s.n_expert)
+    sample = np.unique(np.concatenate([[0, 3, 77, 78, 1500, tokens - 1], np.random.default_rng(5).choice(tokens, 90, replace=False)]))
+    assert len(sample) >= 64
+    gate, up, down = be.download(lw.gate), be.download(lw.up), be.download(lw.down)
+    ref = O.moe_ffn(x[sample], router, gate, up, down, ne=s.ne, n_expert=s.n_expert, n_used=s.n_used, n_ff_exp=s.n_ff,
+                    gate_dtype=int(gdt), down_dtype=int(ddt))
+    assert np.array_equal(ref["idx"], idx[sample])
+    for i, t in enumerate(sample):
+        assert H.rel_l2(full[t], ref["dst"][i]) < REL_L2_MFMA, (int(t), H.rel_l2(full[t], ref["dst"][i]))
     perm = np.random.default_rng(3).permutation(tokens)
     shuffled, idx_p = run(np.ascontiguousarray(x[perm]))
     assert np.array_equal(idx_p, idx[perm])
