@@ -132,6 +132,9 @@ def algorithmic_tables(shape, batch, distinct, prefill):
     if not prefill and batch < 32:
         alg["moe_unbucket_combine"] = pairs * shape.ne * 4 + batch * shape.ne * 4
     alg["rms_norm_router_logits"] = alg["router_logits"] + shape.ne * 4 + batch * shape.ne * 4
+    # the whole single-token op as one launch: the three stages' bytes, each counted once (h and the logits stay on chip
+    # or in L2: the hand-over records are not algorithmic traffic)
+    alg["moe_layer"] = (shape.router_bytes() + shape.ne * 4 + shape.n_used * (2 * gate_b + down_b) + shape.ne * 4)
     if shape.shared_ff:
         sh_gate_b = M.backend.bytes_for(shape.gate_dtype, shape.shared_ff * shape.ne)
         sh_down_b = M.backend.bytes_for(shape.down_dtype, shape.ne * shape.shared_ff)
@@ -370,6 +373,8 @@ def main():
                     help="time the model's whole FFN sublayer per layer (RmsNorm -> MoeFfn [+ shared expert] -> "
                          "residual Add) instead of the MoeFfn op alone; not the headline metric")
     ap.add_argument("--no-fusion", action="store_true", help="one launch per op (infr_hip_config.disable_op_fusion)")
+    ap.add_argument("--three-launch", action="store_true",
+                    help="single-token MoeFfn as three launches (infr_hip_config.disable_single_launch_moe), for comparison")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-timing", action="store_true")
     ap.add_argument("--no-floor", action="store_true", help="skip the dependent-read probe")
@@ -387,7 +392,7 @@ def main():
     shape = shape_of(headline_cfg, args.tokens)
     n_layer = args.layers or shape.n_layer
     batch = args.tokens if prefill else args.batch
-    be = M.Backend(0, disable_op_fusion=args.no_fusion)
+    be = M.Backend(0, disable_op_fusion=args.no_fusion, disable_single_launch_moe=args.three_launch)
     caps = be.capabilities()
     stack = Stack(be, shape, n_layer, prefill)
     if args.copy_probe_mib:

@@ -210,7 +210,15 @@ typedef struct infr_hip_config {
      * kernel.  The escape hatch the reference's backends keep for their rewrites
      * (crates/infr-core/src/fusion.rs:49-52, `enabled`); results are bit-identical either way. */
     uint32_t disable_op_fusion;
-    uint32_t reserved[5];
+    /* Non-zero: a single-token Op::MoeFfn always runs as three launches (logits, routing + gate/up, down + sum).
+     * By default shapes that fit (8 experts per token, Q4_K / Q6_K or Q8_0 banks, hidden size up to 2048, a device
+     * with 256 compute units) run as ONE launch whose stages hand over inside the kernel; results are bit-identical. */
+    uint32_t disable_single_launch_moe;
+    /* Polls a workgroup of the single-launch kernel spends on one of its hand-overs before it gives up (the error
+     * then surfaces at the next infr_hip_sync / download and the backend falls back to three launches for good).
+     * 0 selects the built-in default (32768, some tens of milliseconds); 1 gives up after the first poll. */
+    uint32_t single_launch_spin_limit;
+    uint32_t reserved[3];
 } infr_hip_config;
 
 /* Construction of the backend object (reference: VulkanBackend::new / CpuBackend::new,

@@ -178,7 +178,8 @@ class _Caps(C.Structure):
 
 class _Config(C.Structure):
     _fields_ = [("disable_graph_replay", C.c_uint32), ("moe_batched_min_rows", C.c_uint32),
-                ("disable_op_fusion", C.c_uint32), ("reserved", C.c_uint32 * 5)]
+                ("disable_op_fusion", C.c_uint32), ("disable_single_launch_moe", C.c_uint32),
+                ("single_launch_spin_limit", C.c_uint32), ("reserved", C.c_uint32 * 3)]
 
 
 class _MoeFfnStaticArgs(C.Structure):
@@ -481,11 +482,13 @@ class Backend:
     """The gfx950 compute device (crates/infr-core/src/backend.rs:630 `trait Backend`)."""
 
     def __init__(self, device: int = 0, *, disable_graph_replay: bool = False, moe_batched_min_rows: int = 0,
-                 disable_op_fusion: bool = False):
+                 disable_op_fusion: bool = False, disable_single_launch_moe: bool = False,
+                 single_launch_spin_limit: int = 0):
         self._h = None
         lib = load_library()
         cfg = _Config(disable_graph_replay=int(disable_graph_replay), moe_batched_min_rows=moe_batched_min_rows,
-                      disable_op_fusion=int(disable_op_fusion))
+                      disable_op_fusion=int(disable_op_fusion), disable_single_launch_moe=int(disable_single_launch_moe),
+                      single_launch_spin_limit=single_launch_spin_limit)
         h = _V()
         _check(lib.infr_hip_create(device, C.byref(cfg), C.byref(h)))
         self._h = h.value

@@ -158,6 +158,7 @@ struct MoeScratch {
     _Float16* hh = nullptr;       // [rows * n_used, nff]
     float* hs = nullptr;          // [rows * n_used]
     float* y = nullptr;           // [rows * n_used, ne]
+    bool single_launch = false;   // one token row, shape taken by the single-launch kernel (k_layer.hip)
 };
 
 struct infr_hip_plan {
@@ -177,6 +178,7 @@ struct infr_hip_plan {
     };
     std::vector<LinearBatch> lin;      // per op (valid for Linear ops)
     _Float16* lin_xh = nullptr;        // shared by all ops of a plan: f16 rows, then their scales
+    char* layer_ws = nullptr;          // workspace of the single-launch MoeFfn kernel, shared by all ops of the plan
     int last_moe_op = -1;
     // Launch fusion of the dense SwiGLU FFN the reference emits beside the routed experts
     // (crates/infr-llama/src/runner.rs:8116-8174: Linear gate, Linear up, GatedAct, Linear down, Add).
@@ -213,6 +215,11 @@ struct infr_hip_backend {
     std::vector<Pending> pending;
     std::vector<hipEvent_t> event_pool;
     void* static_scratch = nullptr;   // this device's copy of the file-scope scratch array (infr_hip_moe_ffn_static)
+    // Single-launch Op::MoeFfn (k_layer.hip): a word in pinned host memory the kernel raises when one of its bounded
+    // waits runs out; read after every stream synchronisation.  Once raised the backend keeps to the three-launch path.
+    uint32_t* fault_host = nullptr;
+    uint32_t* fault_dev = nullptr;
+    std::atomic<int> single_launch_off{0};
     // The object outlives infr_hip_destroy while buffers or plans still point at it (the reference's buffers keep their
     // device alive the same way): destroy drains and closes the stream and drops the creator's reference, the last
     // buffer / plan freed afterwards deletes the object.
@@ -231,6 +238,17 @@ void release_backend(infr_hip_backend* be) {
 }
 bool ok_buffer(const infr_hip_buffer* b) { return b && b->magic == kBufferMagic; }
 bool ok_plan(const infr_hip_plan* p) { return p && p->magic == kPlanMagic; }
+
+// After a stream synchronisation: did a single-launch MoeFfn kernel give up a bounded wait?  The results of that
+// execute are not valid; the error is reported once and later executes use the three-launch path.
+infr_status check_fault(infr_hip_backend* be) {
+    if (!be->fault_host || !*(volatile uint32_t*)be->fault_host) return INFR_OK;
+    *(volatile uint32_t*)be->fault_host = 0;
+    be->single_launch_off.store(1);
+    return fail(INFR_ERR_BACKEND,
+                "MoeFfn: the single-launch kernel timed out waiting for a peer workgroup (is the device shared or partitioned?); "
+                "the results since the last synchronisation are invalid, this backend now uses the three-launch path");
+}
 
 // Times one kernel launch when profiling is on: the events ride on the kernel's own dispatch
 // (begin / end of execution), see INFR_LAUNCH.
@@ -401,6 +419,23 @@ extern "C" infr_status infr_hip_create(int device_ordinal, const infr_hip_config
         }
         be->static_scratch = g_scratch_ptr[device_ordinal];
     }
+    {
+        void* host = nullptr;
+        void* dev = nullptr;
+        e = hipHostMalloc(&host, 64, hipHostMallocMapped);
+        if (e == hipSuccess) {
+            memset(host, 0, 64);
+            e = hipHostGetDevicePointer(&dev, host, 0);
+        }
+        if (e != hipSuccess) {
+            if (host) (void)hipHostFree(host);
+            (void)hipStreamDestroy(be->stream);
+            delete be;
+            return fail(INFR_ERR_BACKEND, "hip: pinned fault word: %s", hipGetErrorString(e));
+        }
+        be->fault_host = (uint32_t*)host;
+        be->fault_dev = (uint32_t*)dev;
+    }
     *out = be;
     return INFR_OK;
 } catch (...) { return guard_fail("infr_hip_create"); }
@@ -417,6 +452,8 @@ extern "C" void infr_hip_destroy(infr_hip_backend* be) try {
         be->event_pool.clear();
         (void)hipStreamDestroy(be->stream);
         be->stream = nullptr;
+        if (be->fault_host) (void)hipHostFree(be->fault_host);
+        be->fault_host = be->fault_dev = nullptr;
         be->closed.store(1);   // every later call on this handle is refused; buffers and plans can still be freed
     }
     release_backend(be);
@@ -529,7 +566,7 @@ extern "C" infr_status infr_hip_download_range(infr_hip_backend* be, const infr_
     HIP_TRY(hipSetDevice(be->device));
     if (n) HIP_TRY(hipMemcpyAsync(dst, (const char*)src->dptr + offset, n, hipMemcpyDeviceToHost, be->stream));
     HIP_TRY(hipStreamSynchronize(be->stream));
-    return INFR_OK;
+    return check_fault(be);
 } catch (...) { return guard_fail("infr_hip_download_range"); }
 extern "C" infr_status infr_hip_download(infr_hip_backend* be, const infr_hip_buffer* src, void* dst, size_t n) try {
     return infr_hip_download_range(be, src, 0, dst, n);
@@ -553,7 +590,7 @@ extern "C" infr_status infr_hip_sync(infr_hip_backend* be) try {
     HIP_TRY(hipSetDevice(be->device));
     HIP_TRY(hipStreamSynchronize(be->stream));
     HIP_TRY(hipGetLastError());
-    return INFR_OK;
+    return check_fault(be);
 } catch (...) { return guard_fail("infr_hip_sync"); }
 
 // ---- shared with sibling translation units of this library (not part of the public ABI)
@@ -1124,6 +1161,37 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
             }
         }
     }
+    // One token row through a MoeFfn that stands alone (no always-on expert folded in): the whole op as one launch
+    // when the shape fits that kernel.  An RmsNorm folded into the logits kernel is unfolded again: it costs one
+    // small launch, the single launch saves two large ones.
+    size_t layer_ws = 0;
+    if (!be->cfg.disable_single_launch_moe && be->prop.multiProcessorCount >= 256) {
+        for (uint32_t oi = 0; oi < g->n_ops; oi++) {
+            if (plan->ops[oi].kind != INFR_OP_MOE_FFN || plan->fuse[oi].kind != infr_hip_plan::kPlain) continue;
+            const infr_op_moe_ffn& m = plan->ops[oi].u.moe_ffn;
+            MoeScratch& sc = plan->moe[oi];
+            if (sc.rows != 1 || sc.batched || sc.bucketed || c.dt(m.router) != INFR_F32) continue;
+            infr::MoeLayerParams probe{};
+            probe.g.rows = 1; probe.g.ne = (int)m.ne; probe.g.nff = (int)m.n_ff_exp; probe.g.n_used = (int)m.n_used;
+            probe.g.n_expert = (int)(m.has_ep_band ? m.ep_n_local : m.n_expert);
+            probe.g.gate_dt = c.dt(m.gate_exps);
+            probe.g.up_dt = m.fused_gate_up ? probe.g.gate_dt : c.dt(m.up_exps);
+            probe.g.down_dt = c.dt(m.down_exps);
+            probe.g.n_cu = be->prop.multiProcessorCount;
+            probe.g.route.n_expert = (int)m.n_expert; probe.g.route.n_used = (int)m.n_used;
+            probe.g.route.n_groups = (int)m.n_expert_groups;
+            probe.router_row_floats = m.ne;
+            if (!infr::moe_layer_fused_supported(probe)) continue;
+            sc.single_launch = true;
+            layer_ws = std::max(layer_ws, infr::moe_layer_workspace_bytes((int)m.ne, (int)m.n_ff_exp, (int)m.n_expert));
+            if (plan->fuse[oi].norm) {
+                plan->fuse[plan->fuse[oi].norm - 1].kind = infr_hip_plan::kPlain;
+                plan->fuse[oi].norm = 0;
+            }
+        }
+    }
+    const size_t layer_ws_off = arena;
+    arena += round_up(layer_ws, 256);
     const size_t zero_off = arena;
     arena += round_up(zero_rows * 4 + 4, 256);
 
@@ -1161,6 +1229,7 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
             s.y = (float*)p;
         }
     }
+    plan->layer_ws = layer_ws ? (char*)plan->arena + layer_ws_off : nullptr;
     plan->zero_ids = (int32_t*)((char*)plan->arena + zero_off);   // stays zero: the arena is zero-filled and nothing writes here
     if (plan->arena) infr::launch_fill_zero(be->stream, plan->arena, arena);
     for (uint32_t oi = 0; oi < g->n_ops; oi++) {
@@ -1310,31 +1379,6 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                 rp.ep_n = m.has_ep_band ? (int)m.ep_n_local : 0;
                 const uint32_t n_local = m.has_ep_band ? m.ep_n_local : m.n_expert;   // experts the weight tensors hold
                 rp.ids = sc.ids; rp.weights = sc.weights; rp.probs = sc.probs;
-                bool normed = false;
-                if (fz.norm) {
-                    const infr_op_rms_norm& nr = plan->ops[fz.norm - 1].u.rms_norm;
-                    if (!(need(nr.x, "RmsNorm.x") && need(nr.weight, "RmsNorm.weight") && need(nr.dst, "RmsNorm.dst")))
-                        return INFR_ERR_BACKEND;
-                    infr::RouterNorm rn;
-                    rn.weight = (const float*)ptr[nr.weight]; rn.eps = nr.eps; rn.xn_out = (float*)ptr[nr.dst];
-                    {
-                        Timed t(be, "rms_norm_router_logits");
-                        normed = infr::launch_router_logits(s, (const uint8_t*)ptr[m.router], plan->tensors[m.router].dtype,
-                                                            router_row_bytes, (const float*)ptr[nr.x], (int)m.ne,
-                                                            (int)m.n_expert, rows, sc.logits, &rn);
-                    }
-                    if (!normed) {   // operands the fold cannot take (alignment): the op on its own
-                        Timed t(be, "rms_norm");
-                        infr::launch_rms_norm(s, (const float*)ptr[nr.x], rn.weight, rn.xn_out, 1, (int)nr.dim, nr.eps, 0);
-                    }
-                }
-                if (!normed) {
-                    Timed t(be, "router_logits");
-                    if (!infr::launch_router_logits(s, (const uint8_t*)ptr[m.router], plan->tensors[m.router].dtype,
-                                                    router_row_bytes, (const float*)ptr[m.router_x], (int)m.ne,
-                                                    (int)m.n_expert, rows, sc.logits))
-                        return fail(INFR_ERR_UNSUPPORTED, "MoeFfn: ne=%u does not fit the router kernel's LDS budget", m.ne);
-                }
                 infr::MoeGemvParams gp{};
                 gp.ids = sc.ids; gp.weights = sc.weights;
                 gp.gate_dt = plan->tensors[m.gate_exps].dtype;
@@ -1372,6 +1416,50 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                     if (!(need(other, "Add.a") && need(ad.dst, "Add.dst"))) return INFR_ERR_BACKEND;
                     gp.addend = (const float*)ptr[other];
                     gp.dst = (float*)ptr[ad.dst];
+                }
+                if (sc.single_launch && plan->layer_ws && !be->single_launch_off.load(std::memory_order_relaxed)) {
+                    infr::MoeLayerParams lp{};
+                    lp.g = gp;
+                    lp.g.route = rp;
+                    lp.router = (const float*)ptr[m.router];
+                    lp.router_row_floats = router_row_bytes / 4;
+                    lp.router_x = (const float*)ptr[m.router_x];
+                    lp.logits_out = sc.logits;
+                    char* ws = plan->layer_ws;
+                    lp.seq = (uint32_t*)ws;
+                    lp.cnt = (uint32_t*)(ws + 16);
+                    lp.xl = (uint64_t*)(ws + 256);
+                    lp.xh = lp.xl + (size_t)8 * m.n_expert;
+                    lp.ypart = lp.xh + (size_t)8 * m.n_ff_exp;
+                    lp.fault = be->fault_dev;
+                    lp.spin_limit = be->cfg.single_launch_spin_limit ? (int)be->cfg.single_launch_spin_limit - 1 : 1 << 15;
+                    Timed t(be, "moe_layer");
+                    if (infr::launch_moe_layer_fused(s, lp)) break;   // false: operands the kernel cannot take (alignment)
+                }
+                bool normed = false;
+                if (fz.norm) {
+                    const infr_op_rms_norm& nr = plan->ops[fz.norm - 1].u.rms_norm;
+                    if (!(need(nr.x, "RmsNorm.x") && need(nr.weight, "RmsNorm.weight") && need(nr.dst, "RmsNorm.dst")))
+                        return INFR_ERR_BACKEND;
+                    infr::RouterNorm rn;
+                    rn.weight = (const float*)ptr[nr.weight]; rn.eps = nr.eps; rn.xn_out = (float*)ptr[nr.dst];
+                    {
+                        Timed t(be, "rms_norm_router_logits");
+                        normed = infr::launch_router_logits(s, (const uint8_t*)ptr[m.router], plan->tensors[m.router].dtype,
+                                                            router_row_bytes, (const float*)ptr[nr.x], (int)m.ne,
+                                                            (int)m.n_expert, rows, sc.logits, &rn);
+                    }
+                    if (!normed) {   // operands the fold cannot take (alignment): the op on its own
+                        Timed t(be, "rms_norm");
+                        infr::launch_rms_norm(s, (const float*)ptr[nr.x], rn.weight, rn.xn_out, 1, (int)nr.dim, nr.eps, 0);
+                    }
+                }
+                if (!normed) {
+                    Timed t(be, "router_logits");
+                    if (!infr::launch_router_logits(s, (const uint8_t*)ptr[m.router], plan->tensors[m.router].dtype,
+                                                    router_row_bytes, (const float*)ptr[m.router_x], (int)m.ne,
+                                                    (int)m.n_expert, rows, sc.logits))
+                        return fail(INFR_ERR_UNSUPPORTED, "MoeFfn: ne=%u does not fit the router kernel's LDS budget", m.ne);
                 }
                 if (sc.batched) {
                     const int pairs = rows * (int)m.n_used;

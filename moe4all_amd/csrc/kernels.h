@@ -105,6 +105,28 @@ void launch_moe_gate_up(hipStream_t s, const MoeGemvParams& p);
 // dst[row] = sum over slots (rank order) of w * (down . h).
 void launch_moe_down_combine(hipStream_t s, const MoeGemvParams& p);
 
+// Single-token Op::MoeFfn in one launch (k_layer.hip): logits, routing, gate/up, down and the weighted sum, the
+// stages handing over inside the kernel.  g: as for the two-launch path (g.route filled, rows == 1); the workspace
+// (moe_layer_workspace_bytes, zeroed once) holds the hand-over records, the per-rank partial results and the
+// launch sequence number; *fault (host-visible) is raised when a bounded wait runs out.
+struct MoeLayerParams {
+    MoeGemvParams g;
+    const float* router;        // [n_expert, ne] f32
+    size_t router_row_floats;
+    const float* router_x;      // [ne]
+    float* logits_out;          // [n_expert] or null: the logits, for the plan's routing capture
+    uint32_t* seq;              // workspace + 0
+    uint32_t* cnt;              // workspace + 16: 32 slice counters, then the finished-slice counter
+    uint64_t* xl;               // [8][n_expert] logit records
+    uint64_t* xh;               // [8][nff] activation records
+    uint64_t* ypart;            // [8][ne] partial-result records
+    uint32_t* fault;
+    int spin_limit;
+};
+size_t moe_layer_workspace_bytes(int ne, int nff, int n_expert);
+bool moe_layer_fused_supported(const MoeLayerParams& q);
+bool launch_moe_layer_fused(hipStream_t s, const MoeLayerParams& q);
+
 // ---- batched path: bucketing + grouped GEMMs on the matrix cores --------------------------------
 struct GroupedParams {
     const _Float16* a;        // gate/up: [rows, K] activations; down: [n_pairs, K]; f16, virtual k order

@@ -43,19 +43,27 @@ __device__ __forceinline__ void route_row(const RouteParams& p, int row, int lan
         m = wave_max(m);
 #pragma unroll
         for (int s = 0; s < NS; s++) pr[s] = (s * kWave + lane < n) ? expf_libm(__fsub_rn(pr[s], m), tab) : 0.0f;
-        // psum = p[0] + p[1] + ... strictly left to right: element s*64+l sits in lane l, slot s
-        // (constant lane numbers: the chain is one readlane + one add per element)
+        // psum = p[0] + p[1] + ... strictly left to right (lib.rs:3752-3755).  The terms go through LDS and every
+        // lane adds all of them in order (same-address reads are broadcasts): one dependent add per term, where a
+        // chain over lanes would pay a cross-lane read per term as well.
+#pragma unroll
+        for (int s = 0; s < NS; s++)
+            if (s * kWave + lane < n) prob[s * kWave + lane] = pr[s];
+        __builtin_amdgcn_wave_barrier();
         float psum = 0.0f;
+        {
+            int i = 0;
+#pragma unroll 2
+            for (; i + 8 <= n; i += 8) {
+                float t[8];
 #pragma unroll
-        for (int s = 0; s < NS; s++) {
-            const int cnt = n - s * kWave;
-            if (cnt >= kWave) {
+                for (int k = 0; k < 8; k++) t[k] = prob[i + k];
 #pragma unroll
-                for (int l = 0; l < kWave; l++) psum = __fadd_rn(psum, readlane_f(pr[s], l));
-            } else {
-                for (int l = 0; l < cnt; l++) psum = __fadd_rn(psum, readlane_f(pr[s], l));
+                for (int k = 0; k < 8; k++) psum = __fadd_rn(psum, t[k]);
             }
+            for (; i < n; i++) psum = __fadd_rn(psum, prob[i]);
         }
+        __builtin_amdgcn_wave_barrier();   // prob is rewritten with the final probabilities below
 #pragma unroll
         for (int s = 0; s < NS; s++) pr[s] = __fdiv_rn(pr[s], psum);
     } else if (p.gating == INFR_GATING_SIGMOID) {
@@ -142,16 +150,27 @@ __device__ __forceinline__ void route_row(const RouteParams& p, int row, int lan
 #pragma unroll
         for (int s = 0; s < NS; s++)
             if (s * kWave + lane >= n) taken |= 1u << s;
+        uint32_t keys[NS];
+#pragma unroll
+        for (int s = 0; s < NS; s++) keys[s] = order_key(sl[s]);
         for (int k = 0; k < p.n_used; k++) {
             uint32_t bk = 0, bi = 0xFFFFFFFFu;
 #pragma unroll
             for (int s = 0; s < NS; s++) {
                 if (taken & (1u << s)) continue;
-                uint32_t key = order_key(sl[s]);
-                if (bi == 0xFFFFFFFFu || key > bk) { bk = key; bi = (uint32_t)(s * kWave + lane); }
+                if (bi == 0xFFFFFFFFu || keys[s] > bk) { bk = keys[s]; bi = (uint32_t)(s * kWave + lane); }
             }
-            uint32_t kmax = wave_max_u32(bi == 0xFFFFFFFFu ? 0u : bk);
-            uint32_t win = wave_min_u32((bi != 0xFFFFFFFFu && bk == kmax) ? bi : 0xFFFFFFFFu);
+            // the winner: largest key, then smallest id = smallest slot s, then smallest lane.  One reduction for the
+            // key; the id comes from ballots of the lanes that hold the key, slot by slot.
+            const bool has = bi != 0xFFFFFFFFu;
+            const uint32_t kmax = wave_max_u32(has ? bk : 0u);
+            const bool match = has && bk == kmax;
+            uint32_t win = 0xFFFFFFFFu;
+#pragma unroll
+            for (int s = 0; s < NS; s++) {
+                const uint64_t mk = __ballot(match && (int)(bi >> 6) == s);
+                if (win == 0xFFFFFFFFu && mk) win = (uint32_t)(s * kWave) + (uint32_t)__builtin_ctzll(mk);
+            }
             if (win == 0xFFFFFFFFu) win = 0;
             if ((int)(win & 63u) == lane) taken |= 1u << (win >> 6);
             if (lane == k) my_id = (int)win;
