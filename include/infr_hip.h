@@ -118,7 +118,9 @@ typedef struct infr_op_moe_ffn {
     uint32_t has_ep_band; uint32_t ep_base, ep_n_local;
     uint32_t exp_probs_b;          /* optional */
     uint32_t n_expert_groups, n_expert_groups_used;
-    uint32_t expert_ids;           /* optional */
+    uint32_t expert_ids;           /* optional: I32 [rows, n_used], the selection in table order (hash routing,
+                                    * crates/infr-cpu/src/lib.rs:3776-3793); an id outside [0, n_expert) is clamped into
+                                    * the range before use (the reference indexes with it unchecked and would panic) */
 } infr_op_moe_ffn;
 
 typedef struct infr_op_linear {
