@@ -22,170 +22,11 @@
 // exact packed subtract and one packed multiply(-add) with the group's scale.  The order in
 // which codes fall out of a dword is not the element order; since a dot product does not care
 // about the order of its terms, the activation rows are stored in that same ("virtual") order.
-#include <type_traits>
-
-#include "device_common.h"
-#include "kernels.h"
-#include "units.h"
+#include "grouped_common.h"
 
 namespace infr {
 
-typedef _Float16 half8 __attribute__((ext_vector_type(8)));
-typedef _Float16 half2v __attribute__((ext_vector_type(2)));
-typedef float float16v __attribute__((ext_vector_type(16)));
-
 namespace {
-
-constexpr int kBM = 128;        // token rows per tile
-constexpr int kSlice = 64;      // k elements per LDS stage
-
-__device__ __forceinline__ half2v as_h2(uint32_t v) { return __builtin_bit_cast(half2v, v); }
-__device__ __forceinline__ uint32_t as_u32(half2v v) { return __builtin_bit_cast(uint32_t, v); }
-__device__ __forceinline__ half2v splat(float v) {
-    _Float16 h = (_Float16)v;
-    return half2v{h, h};
-}
-// (1024 + code pair) -> code pair - bias, exact
-__device__ __forceinline__ half2v unbias(uint32_t magic_pair, float bias) { return as_h2(magic_pair) - splat(bias); }
-
-// --------------------------------------------------------------------------------------------
-// Weight formats.  A 64-k slice of a weight row unpacks to 8 operand chunks of 8 f16; the matrix
-// instruction's lane halves split them: lanes 0..31 (half 0) own chunks 0..3, lanes 32..63 own
-// chunks 4..7, and k-step ks of the slice contracts chunk ks of each half.  Four slices make one
-// 256-element step (a K-quant super-block); what is shared by the four slices is fetched once:
-//   Blk                     per-256 part (scales, high bits) half h needs of a step
-//   Q                       the code bytes half h needs of virtual slice s
-//   prep(blk, q, s, h)      per-slice scale constants
-//   chunk(blk, q, c, ks, s) operand chunk 4h + ks as 8 f16
-//   chunk_src()             for virtual chunk c of a row, the two real offsets whose float4s feed
-//                           it and whether the 4 elements of each come out in the order 0,2,1,3
-struct MQ4K {
-    static constexpr int kBlockElems = 256, kBlockBytes = 144;
-    struct Blk {
-        uint4 hdr;   // d, dmin, 12 packed 6-bit scales / mins
-    };
-    struct Q {
-        uint4 q;
-    };
-    struct Prep {
-        half2v s_lo, n_lo, s_hi, n_hi;
-        uint32_t magic;
-    };
-    // scales[i] of the 12 packed bytes, i in 0..11, without branches
-    static __device__ __forceinline__ uint32_t scale_byte(const uint4& hdr, int i) {
-        const uint64_t lo = ((uint64_t)hdr.z << 32) | hdr.y;   // bytes 0..7
-        const uint32_t w = i < 8 ? (uint32_t)(lo >> (8 * (i & 7))) : hdr.w >> (8 * (i & 3));
-        return w & 0xFFu;
-    }
-    static __device__ __forceinline__ void scale_min(const uint4& hdr, int j, uint32_t& sc, uint32_t& m) {
-        // get_scale_min_k4 (crates/infr-gguf/src/dequant.rs:77-87), both arms evaluated and selected
-        const uint32_t a = scale_byte(hdr, j & 3), b = scale_byte(hdr, (j & 3) + 4), c = scale_byte(hdr, (j & 3) + 8);
-        const bool low = j < 4;
-        sc = low ? (a & 63u) : ((c & 0x0Fu) | ((a >> 6) << 4));
-        m = low ? (b & 63u) : ((c >> 4) | ((b >> 6) << 4));
-    }
-    static __device__ __forceinline__ Prep prep(const Blk& blk, const Q&, int s, int) {
-        const int j = s & 3;
-        const float d = f16_bits_to_f32(blk.hdr.x & 0xFFFFu), dmin = f16_bits_to_f32(blk.hdr.x >> 16);
-        uint32_t sc0, m0, sc1, m1;
-        scale_min(blk.hdr, 2 * j, sc0, m0);
-        scale_min(blk.hdr, 2 * j + 1, sc1, m1);
-        uint32_t magic = 0x64006400u;
-        asm volatile("" : "+v"(magic));   // keep it in a vector register (a literal cannot share an instruction with the mask)
-        return Prep{splat(d * (float)sc0), splat(-(dmin * (float)m0)), splat(d * (float)sc1), splat(-(dmin * (float)m1)), magic};
-    }
-    // byte l of the slice holds element l (low nibble, first 32-group) and 32 + l (high nibble)
-    static __device__ __forceinline__ uint4 chunk(const Blk&, const Q& f, const Prep& c, int ks, int) {
-        const uint32_t v = ks == 0 ? f.q.x : ks == 1 ? f.q.y : ks == 2 ? f.q.z : f.q.w;
-        const uint32_t magic = c.magic;   // 0x64006400 in a register: one v_and_or_b32 per pair
-        const half2v a = unbias((v & 0x000F000Fu) | magic, 1024.f);
-        const half2v b = unbias(((v >> 8) & 0x000F000Fu) | magic, 1024.f);
-        const half2v g = unbias(((v >> 4) & 0x000F000Fu) | magic, 1024.f);
-        const half2v e = unbias(((v >> 12) & 0x000F000Fu) | magic, 1024.f);
-        return uint4{as_u32(__builtin_elementwise_fma(a, c.s_lo, c.n_lo)), as_u32(__builtin_elementwise_fma(b, c.s_lo, c.n_lo)),
-                     as_u32(__builtin_elementwise_fma(g, c.s_hi, c.n_hi)), as_u32(__builtin_elementwise_fma(e, c.s_hi, c.n_hi))};
-    }
-    static __device__ __forceinline__ void chunk_src(int c, int& lo, int& hi, bool& swz) {
-        const int i = c & 7;
-        lo = (c >> 3) * 64 + 4 * i;
-        hi = lo + 32;
-        swz = true;
-    }
-};
-
-struct MQ6K {
-    static constexpr int kBlockElems = 256, kBlockBytes = 210;
-    // virtual slice t of a block: t = 2*half128 + ab; ab picks ql bytes [32ab, 32ab+32) of the
-    // 128-element half; their low nibbles are elements [32ab, 32ab+32), their high nibbles +64.
-    // The 2-bit tops of both ab of a half share the same qh bytes.
-    struct Blk {
-        uint4 sc;        // 16 int8 scales
-        uint4 hq0, hq1;  // qh bytes [16h, 16h+16) of 128-element half 0 / 1
-        uint32_t d;      // f16
-    };
-    struct Q {
-        uint4 l;
-    };
-    struct Prep {
-        half2v s_lo, s_hi;
-    };
-    static __device__ __forceinline__ Prep prep(const Blk& blk, const Q&, int s, int h) {
-        // the lane's four chunks are 16 consecutive elements: one scale for the low codes
-        // (scales[8hh + 2ab + h]) and one for the high codes (+4)
-        const int hh = (s >> 1) & 1, ab = s & 1;
-        const uint32_t w_lo = hh ? blk.sc.z : blk.sc.x, w_hi = hh ? blk.sc.w : blk.sc.y;
-        const int sh = 8 * (2 * ab + h);
-        const float d = f16_bits_to_f32(blk.d);
-        return Prep{splat(d * (float)(int8_t)(w_lo >> sh)), splat(d * (float)(int8_t)(w_hi >> sh))};
-    }
-    static __device__ __forceinline__ uint4 chunk(const Blk& blk, const Q& f, const Prep& c, int ks, int s) {
-        const int sh = 2 * (s & 1);  // qh bits sh..sh+1 complete the low codes, sh+4.. the high codes
-        const uint4& hq = ((s >> 1) & 1) ? blk.hq1 : blk.hq0;
-        const uint32_t L = ks == 0 ? f.l.x : ks == 1 ? f.l.y : ks == 2 ? f.l.z : f.l.w;
-        const uint32_t H = (ks == 0 ? hq.x : ks == 1 ? hq.y : ks == 2 ? hq.z : hq.w) >> sh;
-        const uint32_t a = (L & 0x000F000Fu) | ((H & 0x00030003u) << 4) | 0x64006400u;
-        const uint32_t b = ((L >> 8) & 0x000F000Fu) | (((H >> 8) & 0x00030003u) << 4) | 0x64006400u;
-        const uint32_t g = ((L >> 4) & 0x000F000Fu) | (H & 0x00300030u) | 0x64006400u;
-        const uint32_t e = ((L >> 12) & 0x000F000Fu) | ((H >> 8) & 0x00300030u) | 0x64006400u;
-        return uint4{as_u32(unbias(a, 1056.f) * c.s_lo), as_u32(unbias(b, 1056.f) * c.s_lo), as_u32(unbias(g, 1056.f) * c.s_hi),
-                     as_u32(unbias(e, 1056.f) * c.s_hi)};
-    }
-    static __device__ __forceinline__ void chunk_src(int c, int& lo, int& hi, bool& swz) {
-        const int blk = c >> 5, t = (c >> 3) & 3, i = c & 7;
-        lo = blk * 256 + 128 * (t >> 1) + 32 * (t & 1) + 4 * i;
-        hi = lo + 64;
-        swz = true;
-    }
-};
-
-struct MQ80 {
-    static constexpr int kBlockElems = 32, kBlockBytes = 34;
-    struct Blk {};
-    struct Q {
-        uint4 qa, qb;  // the 32 codes of block h of the slice
-        uint32_t d;
-    };
-    struct Prep {
-        half2v d;
-    };
-    static __device__ __forceinline__ Prep prep(const Blk&, const Q& f, int, int) { return Prep{splat(f16_bits_to_f32(f.d))}; }
-    static __device__ __forceinline__ uint4 chunk(const Blk&, const Q& f, const Prep& c, int ks, int) {
-        const uint32_t v0 = ks == 0 ? f.qa.x : ks == 1 ? f.qa.z : ks == 2 ? f.qb.x : f.qb.z;
-        const uint32_t v1 = ks == 0 ? f.qa.y : ks == 1 ? f.qa.w : ks == 2 ? f.qb.y : f.qb.w;
-        // bytes (b0,b1) and (b2,b3) to the low bytes of the two halves; x ^ 0x80 = x + 128 as unsigned
-        const uint32_t a = __builtin_amdgcn_perm(0u, v0, 0x0C010C00u) ^ 0x64806480u;
-        const uint32_t b = __builtin_amdgcn_perm(0u, v0, 0x0C030C02u) ^ 0x64806480u;
-        const uint32_t g = __builtin_amdgcn_perm(0u, v1, 0x0C010C00u) ^ 0x64806480u;
-        const uint32_t e = __builtin_amdgcn_perm(0u, v1, 0x0C030C02u) ^ 0x64806480u;
-        return uint4{as_u32(unbias(a, 1152.f) * c.d), as_u32(unbias(b, 1152.f) * c.d), as_u32(unbias(g, 1152.f) * c.d),
-                     as_u32(unbias(e, 1152.f) * c.d)};
-    }
-    static __device__ __forceinline__ void chunk_src(int c, int& lo, int& hi, bool& swz) {
-        lo = 8 * c;
-        hi = lo + 4;
-        swz = false;
-    }
-};
 
 // --------------------------------------------------------------------------------------------
 // One block per row: amax -> power-of-two scale -> f16 in the virtual k order of format F.
@@ -367,165 +208,32 @@ __global__ __launch_bounds__(256) void bucket_kernel(const int32_t* __restrict__
     }
 }
 
-// Activation for the matrix-core path: hardware exp (about 1e-6 relative), since operands were
-// already rounded to f16.  Same formulas as act_fn / gated_act_fn (crates/infr-cpu/src/kernels.rs:6664-6683).
-__device__ __forceinline__ float act_fast(int act, float g) {
-    if (act == INFR_ACT_SILU) return g / (1.0f + __expf(-g));
-    if (act == INFR_ACT_GELU) {
-        const float inner = 0.7978846f * (g + 0.044715f * g * g * g);
-        return 0.5f * g * (1.0f + tanhf(inner));
-    }
-    return 1.0f / (1.0f + __expf(-g));
-}
-__device__ __forceinline__ float gated_act_fast(int act, bool has_clamp, float clamp, float gate, float up) {
-    if (has_clamp) {
-        gate = fminf(gate, clamp);
-        up = fminf(fmaxf(up, -clamp), clamp);
-    }
-    return act_fast(act, gate) * up;
-}
-
 // --------------------------------------------------------------------------------------------
-struct Tile {
-    int e, p0, cnt;
-};
-// The block's work item: (expert, 128-row tile of its bucket, column tile nt), items ordered by
-// expert, row tile, column tile.  Workgroups go to the chip's 8 XCDs round-robin by workgroup id
-// and every XCD has its own L2, so each XCD takes a contiguous eighth of the items: the column
-// tiles of one row tile, which read the same activation tile, then sit behind the same L2.
-// Uniform per wave; false when the block has nothing to do (the grid is an upper bound).
-__device__ __forceinline__ bool find_item(const int32_t* __restrict__ offsets, int n_expert, int n_tiles_n, int lane,
-                                          Tile& t, int& nt) {
-    const int epl = (n_expert + 63) >> 6;
-    const int e_lo = lane * epl, e_hi = min(n_expert, e_lo + epl);
-    int mine = 0;
-    for (int e = e_lo; e < e_hi; e++) mine += (offsets[e + 1] - offsets[e] + kBM - 1) / kBM;
-    int incl = mine;
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-        const int o = __shfl_up(incl, d, 64);
-        if (lane >= d) incl += o;
-    }
-    const int n_items = __shfl(incl, 63, 64) * n_tiles_n;
-    const int per = (n_items + 7) >> 3;
-    const int k = (int)(blockIdx.x >> 3);
-    const int item = (int)(blockIdx.x & 7) * per + k;
-    if (k >= per || item >= n_items) return false;
-    nt = item % n_tiles_n;
-    const int tile = item / n_tiles_n;
-    const unsigned long long past = __ballot(incl > tile);
-    if (past == 0) return false;
-    const int owner = __ffsll((long long)past) - 1;
-    int rem = tile - (__shfl(incl, owner, 64) - __shfl(mine, owner, 64));
-    const int o_lo = owner * epl, o_hi = min(n_expert, o_lo + epl);
-    for (int e = o_lo; e < o_hi; e++) {
-        const int cnt = offsets[e + 1] - offsets[e];
-        const int ntile = (cnt + kBM - 1) / kBM;
-        if (rem < ntile) {
-            t.e = e;
-            t.p0 = offsets[e] + rem * kBM;
-            t.cnt = min(kBM, cnt - rem * kBM);
-            return true;
-        }
-        rem -= ntile;
-    }
-    return false;
-}
-
-// Epilogue of a tile whose accumulators are acc0/acc1[M] (column tiles of the wave, M 32-row
-// sub-tiles): SwiGLU of (gate, up) or the scaled down-projection row, stored to p.out.
-template <bool DOWN, int M>
-__device__ __forceinline__ void tile_epilogue(const GroupedParams& p, const Tile& t, int n0, int wave, int lane,
-                                              const float* s_scale, const float16v (&acc0)[M], const float16v (&acc1)[M]) {
-    // accumulator register r of a 32x32 tile: row 8*(r/4) + 4*(lane/32) + r%4, column lane%32.
-    // The epilogue variant is chosen once, outside the loops; rows below the last 32-row sub-tile
-    // are all inside the tile, so only that sub-tile tests the row count.
-    const int fc0 = n0 + (DOWN ? 64 : 32) * wave + (lane & 31);   // the lane's column (second column tile of DOWN: + 32)
-    float* const obase = p.out + (size_t)t.p0 * p.N + fc0;
-    const int mrow = 4 * (lane >> 5);
-    auto for_each = [&](auto&& body) {
-#pragma unroll
-        for (int mi = 0; mi < M; mi++) {
-#pragma unroll
-            for (int r4 = 0; r4 < 4; r4++) {
-                const int m0 = 32 * mi + 8 * r4 + mrow;   // rows m0 .. m0 + 3
-                const float4 sc4 = *reinterpret_cast<const float4*>(s_scale + m0);
-                const float scs[4] = {sc4.x, sc4.y, sc4.z, sc4.w};
-#pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const int m = m0 + i;
-                    if (mi < M - 1 || m < t.cnt) body(mi, 4 * r4 + i, m, scs[i], obase + (size_t)m * p.N);
-                }
-            }
-        }
-    };
-    if (DOWN && p.out_f16) {
-        // f16 without the row's power-of-two scale (|acc| stays far inside the f16 range: the
-        // activation rows were normalised below 1); the combine multiplies the scale back in
-        const float ds = p.down_scale ? p.down_scale[t.e] : 1.0f;
-        const bool ok0 = fc0 < p.N, ok1 = fc0 + 32 < p.N;
-        _Float16* const hbase = reinterpret_cast<_Float16*>(p.out) + (size_t)t.p0 * p.N + fc0;
-        if (ok0) {
-            for_each([&](int mi, int r, int m, float, float*) {
-                _Float16* o = hbase + (size_t)m * p.N;
-                o[0] = (_Float16)(acc0[mi][r] * ds);
-                if (ok1) o[32] = (_Float16)(acc1[mi][r] * ds);
-            });
-        }
-    } else if (DOWN) {
-        const float ds = p.down_scale ? p.down_scale[t.e] : 1.0f;
-        const bool ok0 = fc0 < p.N, ok1 = fc0 + 32 < p.N;
-        if (ok1) {
-            for_each([&](int mi, int r, int, float sc, float* o) {
-                o[0] = acc0[mi][r] * sc * ds;
-                o[32] = acc1[mi][r] * sc * ds;
-            });
-        } else if (ok0) {
-            for_each([&](int mi, int r, int, float sc, float* o) { o[0] = acc0[mi][r] * sc * ds; });
-        }
-    } else if (fc0 < p.N) {
-        if (p.act == INFR_ACT_SILU && !p.has_clamp && !p.weight_before) {
-            // silu(g) * u with the hardware exp2 and reciprocal (1 ulp each; the operands were f16)
-            for_each([&](int mi, int r, int, float sc, float* o) {
-                const float g = acc0[mi][r] * sc, u = acc1[mi][r] * sc;
-                o[0] = g * u * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(g * -1.4426950408889634f));
-            });
-        } else {
-            for_each([&](int mi, int r, int m, float sc, float* o) {
-                float g = acc0[mi][r] * sc, u = acc1[mi][r] * sc;
-                if (p.weight_before) {
-                    const float wp = p.route_w[p.pair_src[t.p0 + min(m, t.cnt - 1)]];
-                    g *= wp;
-                    u *= wp;
-                }
-                o[0] = gated_act_fast(p.act, p.has_clamp, p.clamp, g, u);
-            });
-        }
-    }
-}
-
-// --------------------------------------------------------------------------------------------
-// Grouped GEMM: 256 threads = 4 waves, one wave per SIMD (so each may use the whole 512-entry
-// register file: the 128 accumulators sit in AccVGPRs).  Per 64-k slice every wave contracts the
-// slice for its two 32-feature column tiles (gate w / up w, or down 2w / 2w+1) against M 32-token
-// row tiles; each lane unpacks the quantised bytes of ITS weight row and k half in registers into
-// exactly the operand fragments it feeds to the matrix instruction.  M is a template parameter so
-// that the k loop has no branches.  Every k-loop load goes straight from global memory into LDS
+// Grouped GEMM: 512 threads = 8 waves, two per SIMD (256 registers each, 128 of them accumulators).  Waves p and
+// p + 4 form a pair that owns two 32-feature column tiles (gate p / up p, or down 2p / 2p+1) against M 32-token row
+// tiles; of every 64-k slice the first wave of the pair contracts k steps 0 and 1, the second k steps 2 and 3, each
+// into accumulators of its own, and the two sets are added through LDS after the k loop.  A lane unpacks the quantised
+// bytes of ITS weight row and k half in registers into exactly the operand fragments it feeds to the matrix instruction.
+// M is a template parameter so that the k loop has no branches.  Every k-loop load goes straight from global memory
+// into LDS
 // (global_load_lds_dwordx4: lane i of a wave's load deposits its 16 bytes at base + 16 i), so that
 // each load instruction covers whole cache lines and nothing is staged in registers:
 //   * activation stage = the tile's 128 tokens x one 64-k slice (16 KB), token-major, the eight
-//     16-byte chunks of a token rotated by (token & 7) so that the operand reads of 32 consecutive
-//     tokens spread over all banks; every wave loads a quarter of it, kNA stages in the ring;
-//   * weight stage = the parts of the 64 weight rows of ONE wave that a half super-block (128 k,
+//     16-byte chunks of a token rotated by rot7(token) so that the operand reads of 32 consecutive
+//     tokens spread over all banks; every pair loads a quarter of it, kNA stages in the ring;
+//   * weight stage = the parts of the 64 weight rows of ONE pair that a half super-block (128 k,
 //     two slices) needs, row-major (Q4_K: header + 4 code chunks = 80 B per row; Q6_K: 4 low-code
 //     chunks, 2 high-bit chunks, scales, tail = 128 B per row, chunks rotated by the row number);
-//     private to the wave, 3 stages in the ring.
+//     private to the pair, 3 stages in the ring.
 // The loads are issued from inline assembly, so the compiler neither counts them nor orders LDS
 // reads against them: one explicit "s_waitcnt vmcnt(n); s_barrier" per slice does both.  The issue
 // order is fixed (the same number of loads in every even and in every odd slice), so the number
 // of loads younger than the ones slice s needs is a compile-time constant.
 // M0 carries the LDS base of the transfer.  Nothing else in these kernels uses M0 (no other LDS-direct
 // load, no indirect register addressing, no message), so it is not saved around the load.
+#ifndef INFR_ABLATE
+#define INFR_ABLATE 0
+#endif
 __device__ __forceinline__ void dma16(const void* gsrc, uint32_t lds_base) {
     asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(gsrc), "s"(lds_base) : "memory");
 }
@@ -539,6 +247,7 @@ __device__ __forceinline__ uint32_t lds_address(const void* p) {
 
 struct D4K : MQ4K {
     static constexpr int kNC = 5, kRowStride = 80, kNA = 4, kStepBytes = 144;   // kStepBytes: a row's bytes per 256 k
+    static constexpr bool kApart = true;   // a slice is contracted one barrier after it is unpacked (needs a fourth activation stage)
     // chunk `64 j + lane` of a weight stage: which staged row, where in the super-block its 16
     // bytes start for the first half, and how far the second half's lie behind
     static __device__ __forceinline__ void lane_chunk(int j, int lane, int& row, int& off0, int& hoff) {
@@ -557,11 +266,12 @@ struct D4K : MQ4K {
 };
 
 struct D6K : MQ6K {
-    static constexpr int kNC = 8, kRowStride = 128, kNA = 3, kStepBytes = 210;
-    static __device__ __forceinline__ int pos(int row, int part) { return row * kRowStride + ((part + row) & 7) * 16; }
+    static constexpr int kNC = 8, kRowStride = 128, kNA = 4, kStepBytes = 210;
+    static constexpr bool kApart = true;
+    static __device__ __forceinline__ int pos(int row, int part) { return row * kRowStride + ((part + rot7(row)) & 7) * 16; }
     static __device__ __forceinline__ void lane_chunk(int j, int lane, int& row, int& off0, int& hoff) {
         row = 8 * j + (lane >> 3);
-        const int part = ((lane & 7) - row) & 7;   // 0..3 low codes, 4..5 high bits, 6 scales, 7 tail (d in its last 2 bytes)
+        const int part = ((lane & 7) - rot7(row)) & 7;   // 0..3 low codes, 4..5 high bits, 6 scales, 7 tail (d in its last 2 bytes)
         off0 = part < 4 ? 16 * part : part < 6 ? 128 + 16 * (part - 4) : part == 6 ? 192 : 194;
         hoff = part < 4 ? 64 : part < 6 ? 32 : 0;
     }
@@ -579,6 +289,7 @@ struct D6K : MQ6K {
 // ninth for bytes 120..135 (the last block's upper 16 codes, so that nothing past the row is read).
 struct D80 : MQ80 {
     static constexpr int kNC = 9, kRowStride = 144, kNA = 3, kStepBytes = 272;
+    static constexpr bool kApart = false;   // 108 KB of weight stages leave room for three activation stages only
     static __device__ __forceinline__ void lane_chunk(int j, int lane, int& row, int& off0, int& hoff) {
         const int c = 64 * j + lane;
         row = c / 9;
@@ -597,22 +308,70 @@ struct D80 : MQ80 {
 constexpr int kNW6 = 3;                    // weight stages per wave
 constexpr int kAStage6 = kBM * 128;        // bytes per activation stage
 template <class D>
-constexpr size_t grouped6_lds() { return (size_t)D::kNA * kAStage6 + (size_t)4 * kNW6 * 64 * D::kRowStride + kBM * 4; }
+constexpr size_t grouped6_lds() { return (size_t)D::kNA * kAStage6 + (size_t)4 * kNW6 * 64 * D::kRowStride; }   // Q6_K: all 160 KB
+constexpr int kScaleAt6 = 8 * 8192;       // after the k loop: the pairs' hand-over area, then the tile's row scales
+
+// Time stamps of every workgroup for a measurement build (-DINFR_GROUPED_TRACE with a buffer in GroupedParams::trace);
+// compiled out otherwise.
+#ifdef INFR_GROUPED_TRACE
+#define GROUPED_STAMP(i)                                                                                \
+    do {                                                                                                \
+        if (threadIdx.x == 0 && p.trace) p.trace[(size_t)blockIdx.x * 32 + (i)] = wall_clock64();        \
+    } while (0)
+#define GROUPED_NOTE(i, v)                                                                              \
+    do {                                                                                                \
+        if (threadIdx.x == 0 && p.trace) p.trace[(size_t)blockIdx.x * 32 + (i)] = (v);                  \
+    } while (0)
+#else
+#define GROUPED_STAMP(i) do { } while (0)
+#define GROUPED_NOTE(i, v) do { } while (0)
+#endif
+
+// measurement builds: INFR_ABLATE bit 0 = weight loads re-read half-step 0, bit 1 = activation loads re-read slice 0,
+// bit 2 = no unpacking (raw bytes as fragments), bit 3 = one vector instruction in place of each matrix instruction,
+// bit 4 = no k-loop loads at all.  Results are wrong in every case; only the time is of interest.
+template <class D>
+__device__ __forceinline__ uint4 chunk_of(const typename D::Blk& k, const typename D::Q& f, const typename D::Prep& c, int ks, int j4) {
+    if (INFR_ABLATE & 4) {
+        uint4 r = *reinterpret_cast<const uint4*>(&f);
+        r.x += ks;
+        return r;
+    }
+    return D::chunk(k, f, c, ks, j4);
+}
+__device__ __forceinline__ float16v mma(const uint4& a, const uint4& b, float16v acc) {
+    if (INFR_ABLATE & 8) {
+        acc[0] += __uint_as_float((a.x ^ b.x) & 0x3FFFFFFFu);
+        acc[1] += __uint_as_float((a.w ^ b.w) & 0x3FFFFFFFu);
+        return acc;
+    }
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, a), __builtin_bit_cast(half8, b), acc, 0, 0, 0);
+}
 
 struct Grouped6Ctx {
-    uint8_t* lds;             // [kNA activation stages][4 waves x kNW6 weight stages][row scales]
-    const float* s_scale;
-    const uint8_t* asrc[4];   // the lane's four activation chunks of slice 0
-    int wave, lane, n0;
+    uint8_t* lds;             // [kNA activation stages][4 pairs x kNW6 weight stages]
+    const uint8_t* asrc[4];   // the lane's activation chunks of slice 0: quarters 0..3 of the pair's 32 tokens
+    int pair, lane, n0;
     Tile t;
 };
 
-template <class D, bool DOWN, int M>
+// KH = which wave of the pair: it contracts k steps 2 KH and 2 KH + 1 of every slice and stores the accumulator
+// registers 8 KH .. 8 KH + 7 of every tile.  The pair's loads are all issued by its first wave: a load instruction holds
+// up the wave that issues it until the address unit has taken it (with rows of 80 to 144 bytes a wave-load touches 20
+// to 30 cache lines), and the first wave, being the older one on its SIMD, is served first and has time to spare before
+// every barrier.
+template <class D, bool DOWN, int M, int KH>
 __device__ __forceinline__ void grouped6_tile(const GroupedParams& p, const Grouped6Ctx& c, const uint8_t* const (&wsrc)[D::kNC],
                                               const int (&whoff)[D::kNC]) {
     constexpr int NA = D::kNA, NC = D::kNC, NW = kNW6;
+    // kApart: a wave unpacks slice s after barrier s and contracts it only after barrier s + 1, next to the unpacking of
+    // slice s + 1, so that its matrix and vector instructions are independent and can be interleaved one to seven, and
+    // the first k step's activation fragments are read from LDS a slice before they are used.  Activation stage s is
+    // then still read after barrier s + 1, so loads run one slice less ahead (kAhead) and never target it.
+    constexpr bool kLate = D::kApart;
+    constexpr int kAhead = kLate ? NA - 2 : NA - 1;
     constexpr int kWStage = 64 * D::kRowStride;
-    const int wave = c.wave, lane = c.lane, half = lane >> 5;
+    const int pair = c.pair, lane = c.lane, half = lane >> 5;
     float16v acc0[M], acc1[M];
 #pragma unroll
     for (int i = 0; i < M; i++)
@@ -620,87 +379,130 @@ __device__ __forceinline__ void grouped6_tile(const GroupedParams& p, const Grou
         for (int r = 0; r < 16; r++) acc0[i][r] = acc1[i][r] = 0.0f;
     const int n_slices = p.K / kSlice, last = n_slices - 1, last_hs = (n_slices >> 1) - 1;
     const uint32_t lds0 = lds_address(c.lds);
-    const uint32_t uwave = __builtin_amdgcn_readfirstlane(wave);
-    const uint32_t a_dst = lds0 + uwave * 4096;                                   // + stage * kAStage6 + q * 1024
-    const uint32_t w_dst = lds0 + NA * kAStage6 + uwave * (NW * kWStage);         // + stage * kWStage + j * 1024
-    const uint8_t* const w_lds = c.lds + NA * kAStage6 + wave * (NW * kWStage);
-    const uint8_t* const as0 = c.asrc[0];
-    const uint8_t* const as1 = c.asrc[1];
-    const uint8_t* const as2 = c.asrc[2];
-    const uint8_t* const as3 = c.asrc[3];
-    // Loads issued while slice s is contracted, a quarter after each k step so that the four waves
-    // do not queue up at the address unit together: part ks = (on even s the weight chunks
-    // 0..(NC+1)/2-1, on odd s the rest, one per k step) of half-step s/2 + NW - 1, then activation
-    // quarter ks of slice s + NA - 1 (a fifth weight chunk of a slice goes with k step 0).  The last load
-    // of a slice is its activation quarter 3.
+    const uint32_t upair = __builtin_amdgcn_readfirstlane(pair);
+    const uint32_t a_dst = lds0 + upair * 4096;                                   // + stage * kAStage6 + q * 1024
+    const uint32_t w_dst = lds0 + NA * kAStage6 + upair * (NW * kWStage);         // + stage * kWStage + j * 1024
+    const uint8_t* const w_lds = c.lds + NA * kAStage6 + pair * (NW * kWStage);
+    // Loads the first wave issues while slice s is contracted, in two parts i = 0, 1: of the weight chunks of half-step
+    // s/2 + NW - 1 that belong to the slice's parity (even s: chunks 0..(NC+1)/2-1, odd s: the rest) every second one,
+    // then the activation quarters 2 i and 2 i + 1 of slice s + kAhead.  The last load of a slice is an activation quarter.
     constexpr int kWEven = (NC + 1) / 2;
-    auto issue_w = [&](int s, int j) {
-        const int hs = (s >> 1) + NW - 1;
-        if (hs < 0) return;
-        const int hc = min(hs, last_hs);
-        dma16(wsrc[j] + (size_t)(hc >> 1) * D::kStepBytes + ((hc & 1) ? whoff[j] : 0),
-              w_dst + (uint32_t)(hs % NW) * kWStage + j * 1024);
-    };
-    auto issue_part = [&](int s, int odd, int ks) {   // odd = s & 1; odd and ks are constants where this is called
+    auto issue_part = [&](int s, int odd, int i) {   // odd = s & 1; odd and i are constants where this is called
+        if (KH == 1 || (INFR_ABLATE & 16)) return;
         const int lo = odd ? kWEven : 0, hi = odd ? NC : kWEven;
+        const int hs = (s >> 1) + NW - 1, hc = min(hs, last_hs);
 #pragma unroll
         for (int j = 0; j < NC; j++)
-            if (j >= lo && j < hi && ((j - lo) & 3) == ks) issue_w(s, j);
-        const int sa = s + NA - 1;
+            if (j >= lo && j < hi && ((j - lo) & 1) == i && hs >= 0)
+                dma16(wsrc[j] + ((INFR_ABLATE & 1) ? (size_t)0 : (size_t)(hc >> 1) * D::kStepBytes + ((hc & 1) ? whoff[j] : 0)),
+                      w_dst + (uint32_t)(hs % NW) * kWStage + j * 1024);
+        const int sa = s + kAhead;
         if (sa >= 0) {
-            const uint8_t* src = ks == 0 ? as0 : ks == 1 ? as1 : ks == 2 ? as2 : as3;
-            dma16(src + (size_t)min(sa, last) * 128, a_dst + (uint32_t)(sa % NA) * kAStage6 + ks * 1024);
+            const size_t ao = (INFR_ABLATE & 2) ? (size_t)0 : (size_t)min(sa, last) * 128;
+            dma16(c.asrc[2 * i] + ao, a_dst + (uint32_t)(sa % NA) * kAStage6 + (2 * i) * 1024);
+            dma16(c.asrc[2 * i + 1] + ao, a_dst + (uint32_t)(sa % NA) * kAStage6 + (2 * i + 1) * 1024);
         }
     };
 #pragma unroll
     for (int s = -2 * (NW - 1); s < 0; s++)
 #pragma unroll
-        for (int ks = 0; ks < 4; ks++) issue_part(s, s & 1, ks);
+        for (int i = 0; i < 2; i++) issue_part(s, s & 1, i);
 
-    // operand reads: token 32 mi + (lane & 31), k chunk ks + 4 half, rotated by the token's low bits
-    const int x7 = lane & 7;
+    // operand reads: token 32 mi + (lane & 31), k chunk ks + 4 half, rotated by the token's number
+    const int x7 = rot7(lane & 31);
     const int a_lane = (lane & 31) * 128;
-    int a_off[4];
+    int a_off[2];
 #pragma unroll
-    for (int ks = 0; ks < 4; ks++) a_off[ks] = a_lane + (((ks + 4 * half) ^ x7) * 16);
+    for (int i = 0; i < 2; i++) a_off[i] = a_lane + (((2 * KH + i + 4 * half) ^ x7) * 16);
     const int row0 = lane & 31, row1 = 32 + (lane & 31);
 
+#ifdef INFR_GROUPED_TRACE
+    long long wait_loads = 0, wait_barrier = 0;
+    const long long loop_in = clock64();
+#endif
+    // kLate: the wave's two k steps of the previous slice: first-step fragments a0 (read a slice earlier), second-step
+    // fragments from the activation stage at ap
+    auto contract = [&](const uint8_t* ap, const uint4 (&a0)[M], const uint4 (&b)[4]) {
+        uint4 a1[M];
+#pragma unroll
+        for (int mi = 0; mi < M; mi++) a1[mi] = *reinterpret_cast<const uint4*>(ap + a_off[1] + mi * 4096);
+#pragma unroll
+        for (int mi = 0; mi < M; mi++) {
+            acc0[mi] = mma(a0[mi], b[0], acc0[mi]);
+            acc1[mi] = mma(a0[mi], b[1], acc1[mi]);
+        }
+#pragma unroll
+        for (int mi = 0; mi < M; mi++) {
+            acc0[mi] = mma(a1[mi], b[2], acc0[mi]);
+            acc1[mi] = mma(a1[mi], b[3], acc1[mi]);
+        }
+    };
+    uint4 afirst[M] = {};   // kLate: the first k step's activation fragments of the previous slice
+    uint4 held[4] = {};     // kLate: the unpacked weight fragments of the previous slice (k step 2 KH: rows 0, 1; 2 KH + 1: rows 0, 1)
     // slice s (compile-time position j4 = s & 3 inside its super-block)
     auto slice = [&](int s, auto j4c) {
         constexpr int j4 = decltype(j4c)::value;
-        // loads younger than the last one this slice needs (activation quarter 3 of slice s, issued at
-        // the end of slice s - NA + 1): everything issued during the NA - 2 slices since
+        // loads of the first wave younger than the last one this slice needs (an activation quarter of slice s, issued
+        // at the end of slice s - kAhead): everything it issued during the kAhead - 1 slices since
         constexpr int kWOdd = NC - kWEven;
-        constexpr int kYoung = NA == 4 ? 8 + NC : 4 + ((j4 & 1) ? kWEven : kWOdd);
-        static_assert(NA == 3 || NA == 4, "the load counts above are written for these ring depths");
+        constexpr int kYoung = KH == 1 ? 0 : kAhead == 3 ? 8 + NC : 4 + ((j4 & 1) ? kWEven : kWOdd);
+        static_assert(kAhead == 2 || kAhead == 3, "the load counts above are written for these distances");
+#ifdef INFR_GROUPED_TRACE
+        const long long w_in = clock64();
+        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" : : "n"(kYoung) : "memory");
+        const long long w_mid = clock64();
+        asm volatile("s_barrier" ::: "memory");
+        wait_loads += w_mid - w_in;
+        wait_barrier += clock64() - w_mid;
+#else
         wait_loads_then_barrier<kYoung>();
+#endif
         const uint8_t* ap = c.lds + (s % NA) * kAStage6;
         const uint8_t* wst = w_lds + ((s >> 1) % NW) * kWStage;
+        if (kLate) {
+            // all of the slice's loads first: what follows is one region for the instruction scheduler
+            issue_part(s, j4 & 1, 0);
+            issue_part(s, j4 & 1, 1);
+            if (s > 0) contract(c.lds + ((s - 1) % NA) * kAStage6, afirst, held);
+        }
         const typename D::Blk k0 = D::read_blk(wst, row0, half), k1 = D::read_blk(wst, row1, half);
         const typename D::Q f0 = D::read_q(wst, row0, j4 & 1, half), f1 = D::read_q(wst, row1, j4 & 1, half);
-        uint4 a[M];
-#pragma unroll
-        for (int mi = 0; mi < M; mi++) a[mi] = *reinterpret_cast<const uint4*>(ap + a_off[0] + mi * 4096);
         const typename D::Prep c0 = D::prep(k0, f0, j4, half), c1 = D::prep(k1, f1, j4, half);
-        uint4 b0 = D::chunk(k0, f0, c0, 0, j4), b1 = D::chunk(k1, f1, c1, 0, j4);
+        if (kLate) {
+            held[0] = chunk_of<D>(k0, f0, c0, 2 * KH, j4);
+            held[1] = chunk_of<D>(k1, f1, c1, 2 * KH, j4);
+            held[2] = chunk_of<D>(k0, f0, c0, 2 * KH + 1, j4);
+            held[3] = chunk_of<D>(k1, f1, c1, 2 * KH + 1, j4);
 #pragma unroll
-        for (int ks = 0; ks < 4; ks++) {
-            uint4 nb0 = b0, nb1 = b1;
-            if (ks < 3) {
-                nb0 = D::chunk(k0, f0, c0, ks + 1, j4);
-                nb1 = D::chunk(k1, f1, c1, ks + 1, j4);
-            }
-            issue_part(s, j4 & 1, ks);
+            for (int mi = 0; mi < M; mi++) afirst[mi] = *reinterpret_cast<const uint4*>(ap + a_off[0] + mi * 4096);
+            // one matrix instruction, then a share of the vector work
 #pragma unroll
-            for (int mi = 0; mi < M; mi++) {
-                acc0[mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, a[mi]), __builtin_bit_cast(half8, b0),
-                                                                  acc0[mi], 0, 0, 0);
-                acc1[mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8, a[mi]), __builtin_bit_cast(half8, b1),
-                                                                  acc1[mi], 0, 0, 0);
-                if (ks < 3) a[mi] = *reinterpret_cast<const uint4*>(ap + a_off[ks + 1] + mi * 4096);
+            for (int i = 0; i < 4 * M; i++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, (112 + 4 * M - 1) / (4 * M), 0);
             }
-            b0 = nb0;
-            b1 = nb1;
+        } else {
+            uint4 a[M];
+#pragma unroll
+            for (int mi = 0; mi < M; mi++) a[mi] = *reinterpret_cast<const uint4*>(ap + a_off[0] + mi * 4096);
+            uint4 b0 = chunk_of<D>(k0, f0, c0, 2 * KH, j4), b1 = chunk_of<D>(k1, f1, c1, 2 * KH, j4);
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                uint4 nb0 = b0, nb1 = b1;
+                if (i < 1) {
+                    nb0 = chunk_of<D>(k0, f0, c0, 2 * KH + 1, j4);
+                    nb1 = chunk_of<D>(k1, f1, c1, 2 * KH + 1, j4);
+                }
+                issue_part(s, j4 & 1, i);
+#pragma unroll
+                for (int mi = 0; mi < M; mi++) {
+                    acc0[mi] = mma(a[mi], b0, acc0[mi]);
+                    acc1[mi] = mma(a[mi], b1, acc1[mi]);
+                    if (i < 1) a[mi] = *reinterpret_cast<const uint4*>(ap + a_off[1] + mi * 4096);
+                }
+                b0 = nb0;
+                b1 = nb1;
+            }
         }
     };
     for (int s0 = 0; s0 < n_slices; s0 += 4) {
@@ -709,27 +511,84 @@ __device__ __forceinline__ void grouped6_tile(const GroupedParams& p, const Grou
         slice(s0 + 2, std::integral_constant<int, 2>{});
         slice(s0 + 3, std::integral_constant<int, 3>{});
     }
-    // nothing may still be landing in LDS when the block ends (or another block takes over the CU's LDS)
+    if (kLate) contract(c.lds + (last % NA) * kAStage6, afirst, held);
+    // nothing may still be landing in LDS when the rings are reused below or the block ends
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    tile_epilogue<DOWN, M>(p, c.t, c.n0, wave, lane, c.s_scale, acc0, acc1);
+    GROUPED_STAMP(3);
+#ifdef INFR_GROUPED_TRACE
+    GROUPED_NOTE(8, wait_loads);
+    GROUPED_NOTE(9, wait_barrier);
+    GROUPED_NOTE(10, clock64() - loop_in);
+    if (lane == 0 && p.trace) {
+        p.trace[(size_t)blockIdx.x * 32 + 16 + pair + 4 * KH] = wait_loads;
+        p.trace[(size_t)blockIdx.x * 32 + 24 + pair + 4 * KH] = wait_barrier;
+    }
+#endif
+
+    // The pair's two partial sums: each wave hands over the accumulator registers the other one stores (this wave keeps
+    // registers 8 KH .. 8 KH + 7 of every tile) through the ring memory, two row tiles per round, 8 KB per wave.
+    float* const s_scale = reinterpret_cast<float*>(c.lds + kScaleAt6);
+    uint8_t* const mine = c.lds + (size_t)(pair + 4 * KH) * 8192 + lane * 16;
+    const uint8_t* const theirs = c.lds + (size_t)(pair + 4 * (1 - KH)) * 8192 + lane * 16;
+#pragma unroll
+    for (int g = 0; g < (M + 1) / 2; g++) {
+        __syncthreads();   // the rings (first round) or the previous round's hand-over have been read by everyone
+        if (g == 0 && KH == 0 && lane < 32) {   // the tile's row scales for the epilogue
+            const int pr = c.t.p0 + min(32 * pair + lane, c.t.cnt - 1);
+            s_scale[32 * pair + lane] = p.a_scale[DOWN ? pr : p.pair_src[pr] / p.n_used];
+        }
+#pragma unroll
+        for (int q = 0; q < 2; q++) {
+            const int mi = 2 * g + q;
+            if (mi < M) {
+                constexpr int o = 8 * (1 - KH);
+                *reinterpret_cast<float4*>(mine + (4 * q + 0) * 1024) = make_float4(acc0[mi][o], acc0[mi][o + 1], acc0[mi][o + 2], acc0[mi][o + 3]);
+                *reinterpret_cast<float4*>(mine + (4 * q + 1) * 1024) = make_float4(acc0[mi][o + 4], acc0[mi][o + 5], acc0[mi][o + 6], acc0[mi][o + 7]);
+                *reinterpret_cast<float4*>(mine + (4 * q + 2) * 1024) = make_float4(acc1[mi][o], acc1[mi][o + 1], acc1[mi][o + 2], acc1[mi][o + 3]);
+                *reinterpret_cast<float4*>(mine + (4 * q + 3) * 1024) = make_float4(acc1[mi][o + 4], acc1[mi][o + 5], acc1[mi][o + 6], acc1[mi][o + 7]);
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int q = 0; q < 2; q++) {
+            const int mi = 2 * g + q;
+            if (mi < M) {
+                constexpr int o = 8 * KH;
+                const float4 v0 = *reinterpret_cast<const float4*>(theirs + (4 * q + 0) * 1024), v1 = *reinterpret_cast<const float4*>(theirs + (4 * q + 1) * 1024);
+                const float4 v2 = *reinterpret_cast<const float4*>(theirs + (4 * q + 2) * 1024), v3 = *reinterpret_cast<const float4*>(theirs + (4 * q + 3) * 1024);
+                // first wave's part + second wave's part, whichever of the two this is
+                const float t0[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w}, t1[8] = {v2.x, v2.y, v2.z, v2.w, v3.x, v3.y, v3.z, v3.w};
+#pragma unroll
+                for (int r = 0; r < 8; r++) {
+                    acc0[mi][o + r] = KH ? t0[r] + acc0[mi][o + r] : acc0[mi][o + r] + t0[r];
+                    acc1[mi][o + r] = KH ? t1[r] + acc1[mi][o + r] : acc1[mi][o + r] + t1[r];
+                }
+            }
+        }
+    }
+    GROUPED_STAMP(4);
+    tile_epilogue<DOWN, M, 2 * KH, 2 * KH + 2>(p, c.t, c.n0, pair, lane, s_scale, acc0, acc1);
+    GROUPED_STAMP(5);
 }
 
 template <class D, bool DOWN>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void grouped_mfma6(GroupedParams p) {
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void grouped_mfma6(GroupedParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds6[];
     Grouped6Ctx c;
     c.lds = lds6;
-    float* s_scale = reinterpret_cast<float*>(lds6 + grouped6_lds<D>() - kBM * 4);
-    c.s_scale = s_scale;
     const int tid = threadIdx.x;
-    c.wave = tid >> 6;
+    const int kh = tid >> 8;
+    c.pair = (tid >> 6) & 3;
     c.lane = tid & 63;
     int nt;
+    GROUPED_STAMP(0);
     if (!find_item(p.offsets, p.n_expert, p.n_tiles_n, c.lane, c.t, nt)) return;
     const Tile& t = c.t;
+    GROUPED_STAMP(1);
+    GROUPED_NOTE(7, (long long)t.cnt);
     constexpr int kBN = DOWN ? 256 : 128;
     c.n0 = nt * kBN;
-    // sources of the lane's chunks of the wave's weight stage (half-step 0)
+    // sources of the lane's chunks of the pair's weight stage (half-step 0)
     const size_t row_bytes = (size_t)(p.K / D::kBlockElems) * D::kBlockBytes;
     const uint8_t* wsrc[D::kNC];
     int whoff[D::kNC];
@@ -741,31 +600,31 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         int f;
         if (DOWN) {
             base = p.w0 + (size_t)t.e * p.w0_stride;
-            f = c.n0 + 64 * c.wave + row;
+            f = c.n0 + 64 * c.pair + row;
         } else {
             base = row < 32 ? p.w0 + (size_t)t.e * p.w0_stride : p.w1 + (size_t)t.e * p.w1_stride;
-            f = c.n0 + 32 * c.wave + (row & 31);
+            f = c.n0 + 32 * c.pair + (row & 31);
         }
         wsrc[j] = base + (size_t)min(f, p.N - 1) * row_bytes + off0;
     }
-    // the lane's activation chunks: token 32 wave + 8 q + lane / 8, chunk (lane & 7) ^ (token & 7)
+    // the lane's activation chunks: token 32 pair + 8 q + lane / 8, chunk (lane & 7) ^ rot7(token)
 #pragma unroll
     for (int q = 0; q < 4; q++) {
-        const int tok = 32 * c.wave + 8 * q + (c.lane >> 3), kg = (c.lane & 7) ^ ((c.lane >> 3) & 7);
+        const int tok = 32 * c.pair + 8 * q + (c.lane >> 3), kg = (c.lane & 7) ^ rot7(tok);
         const int pr = t.p0 + min(tok, t.cnt - 1);
         const size_t src_row = DOWN ? (size_t)pr : (size_t)(p.pair_src[pr] / p.n_used);
         c.asrc[q] = reinterpret_cast<const uint8_t*>(p.a + src_row * p.K) + 16 * kg;
     }
-    if (tid < kBM) {
-        const int pr = t.p0 + min(tid, t.cnt - 1);
-        s_scale[tid] = p.a_scale[DOWN ? pr : p.pair_src[pr] / p.n_used];
-    }
-    switch ((t.cnt + 31) >> 5) {
-        case 1: grouped6_tile<D, DOWN, 1>(p, c, wsrc, whoff); break;
-        case 2: grouped6_tile<D, DOWN, 2>(p, c, wsrc, whoff); break;
-        case 3: grouped6_tile<D, DOWN, 3>(p, c, wsrc, whoff); break;
-        default: grouped6_tile<D, DOWN, 4>(p, c, wsrc, whoff); break;
-    }
+    const int m = (t.cnt + 31) >> 5;
+    GROUPED_STAMP(2);
+#define INFR_TILE(MM)                                                     \
+    if (kh) grouped6_tile<D, DOWN, MM, 1>(p, c, wsrc, whoff);             \
+    else grouped6_tile<D, DOWN, MM, 0>(p, c, wsrc, whoff)
+    if (m == 1) { INFR_TILE(1); }
+    else if (m == 2) { INFR_TILE(2); }
+    else if (m == 3) { INFR_TILE(3); }
+    else { INFR_TILE(4); }
+#undef INFR_TILE
 }
 
 // dst[row, :] = sum over ranks of w * y[slot_pair[row, rank], :], rank order, separate mul/add.
@@ -892,411 +751,10 @@ void grouped6(hipStream_t s, const GroupedParams& p) {
                                   (int)grouped6_lds<D>());
         attr_set = true;
     }
-    INFR_LAUNCH((grouped_mfma6<D, DOWN>), dim3((unsigned)((max_tiles * q.n_tiles_n + 7) & ~7)), dim3(256), grouped6_lds<D>(), s, q);   // whole rounds of the 8 XCDs
-}
-
-// --------------------------------------------------------------------------------------------
-// Grouped GEMM for every affine format through the 32-element unit decoder: the matrix-core path of banks
-// that have no byte-exact LDS layout above.  Same tiles (expert, <= 128 tokens, 128 features with gate and
-// up, or 256 features of down), same accumulator layout and epilogue.  Per 64-k slice a lane decodes ONE
-// unit of each of its two weight rows - lanes 0..31 the slice's first 32 k, lanes 32..63 the second - into
-// four 8-element f16 operand fragments (f32 sc * code + mn, rounded once), so no element is decoded
-// twice; k step ks of the slice contracts elements 8 ks .. 8 ks + 7 of both units.  The activation tile
-// (natural k order) goes through registers into a two-stage LDS ring with the chunk rotation of the
-// kernel above; the next slice's units and activation chunks are requested before the current slice is
-// contracted.
-constexpr int kUStage = kBM * 128;   // 128 tokens x 64 halfs
-
-// The 32 k of one weight row that a lane contracts in a slice, and its four 8-element f16 fragments.
-template <int DT>
-struct WSlice {
-    Unit u;
-    __device__ __forceinline__ void load(const uint8_t* __restrict__ row, int idx) { load_unit<DT>(row, idx, u); }
-    __device__ __forceinline__ half8 frag(int ks) const {
-        const float sc = u.sc[ks >> 1], mn = u.mn[ks >> 1];
-        const uint32_t a = u.q[2 * ks], b = u.q[2 * ks + 1];
-        half8 h;
-        h[0] = (_Float16)fmaf(sc, (float)(a & 0xFFu), mn);
-        h[1] = (_Float16)fmaf(sc, (float)((a >> 8) & 0xFFu), mn);
-        h[2] = (_Float16)fmaf(sc, (float)((a >> 16) & 0xFFu), mn);
-        h[3] = (_Float16)fmaf(sc, (float)(a >> 24), mn);
-        h[4] = (_Float16)fmaf(sc, (float)(b & 0xFFu), mn);
-        h[5] = (_Float16)fmaf(sc, (float)((b >> 8) & 0xFFu), mn);
-        h[6] = (_Float16)fmaf(sc, (float)((b >> 16) & 0xFFu), mn);
-        h[7] = (_Float16)fmaf(sc, (float)(b >> 24), mn);
-        return h;
-    }
-};
-// Unquantised weights: F16 rows are the fragments as they lie in memory; BF16 / F32 are rounded to f16.
-template <>
-struct WSlice<INFR_F16> {
-    uint4 v[4];
-    __device__ __forceinline__ void load(const uint8_t* __restrict__ row, int idx) {
-#pragma unroll
-        for (int k = 0; k < 4; k++) v[k] = ldu<uint4>(row + (size_t)idx * 64 + 16 * k);
-    }
-    __device__ __forceinline__ half8 frag(int ks) const { return __builtin_bit_cast(half8, v[ks]); }
-};
-template <>
-struct WSlice<INFR_BF16> {
-    uint4 v[4];
-    __device__ __forceinline__ void load(const uint8_t* __restrict__ row, int idx) {
-#pragma unroll
-        for (int k = 0; k < 4; k++) v[k] = ldu<uint4>(row + (size_t)idx * 64 + 16 * k);
-    }
-    __device__ __forceinline__ half8 frag(int ks) const {
-        const uint32_t d[4] = {v[ks].x, v[ks].y, v[ks].z, v[ks].w};
-        half8 h;
-#pragma unroll
-        for (int k = 0; k < 4; k++) {
-            h[2 * k] = (_Float16)__uint_as_float(d[k] << 16);
-            h[2 * k + 1] = (_Float16)__uint_as_float(d[k] & 0xFFFF0000u);
-        }
-        return h;
-    }
-};
-template <>
-struct WSlice<INFR_F32> {
-    uint4 v[8];
-    __device__ __forceinline__ void load(const uint8_t* __restrict__ row, int idx) {
-#pragma unroll
-        for (int k = 0; k < 8; k++) v[k] = ldu<uint4>(row + (size_t)idx * 128 + 16 * k);
-    }
-    __device__ __forceinline__ half8 frag(int ks) const {
-        const uint4 a = v[2 * ks], b = v[2 * ks + 1];
-        half8 h;
-        h[0] = (_Float16)__uint_as_float(a.x); h[1] = (_Float16)__uint_as_float(a.y);
-        h[2] = (_Float16)__uint_as_float(a.z); h[3] = (_Float16)__uint_as_float(a.w);
-        h[4] = (_Float16)__uint_as_float(b.x); h[5] = (_Float16)__uint_as_float(b.y);
-        h[6] = (_Float16)__uint_as_float(b.z); h[7] = (_Float16)__uint_as_float(b.w);
-        return h;
-    }
-};
-
-template <int DT, bool DOWN, int M>
-__device__ __forceinline__ void grouped_units_tile(const GroupedParams& p, const Tile& t, int n0, uint8_t* lds, const float* s_scale) {
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, half = lane >> 5;
-    float16v acc0[M], acc1[M];
-#pragma unroll
-    for (int i = 0; i < M; i++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) acc0[i][r] = acc1[i][r] = 0.0f;
-    int be = 1, bb = 4;
-    block_geometry(DT, &be, &bb);
-    const size_t row_bytes = (size_t)(p.K / be) * bb;
-    // the lane's two weight rows
-    const uint8_t* w0;
-    const uint8_t* w1;
-    {
-        const int c = lane & 31;
-        if (DOWN) {
-            const uint8_t* base = p.w0 + (size_t)t.e * p.w0_stride;
-            w0 = base + (size_t)min(n0 + 64 * wave + c, p.N - 1) * row_bytes;
-            w1 = base + (size_t)min(n0 + 64 * wave + 32 + c, p.N - 1) * row_bytes;
-        } else {
-            const int f = min(n0 + 32 * wave + c, p.N - 1);
-            w0 = p.w0 + (size_t)t.e * p.w0_stride + (size_t)f * row_bytes;
-            w1 = p.w1 + (size_t)t.e * p.w1_stride + (size_t)f * row_bytes;
-        }
-    }
-    // the lane's four activation chunks of a slice: token 32 wave + 8 q + lane / 8, LDS position lane & 7
-    const uint8_t* asrc[4];
-#pragma unroll
-    for (int q = 0; q < 4; q++) {
-        const int tok = 32 * wave + 8 * q + (lane >> 3), kg = (lane & 7) ^ ((lane >> 3) & 7);
-        const int pr = t.p0 + min(tok, t.cnt - 1);
-        const size_t src_row = DOWN ? (size_t)pr : (size_t)(p.pair_src[pr] / p.n_used);
-        asrc[q] = reinterpret_cast<const uint8_t*>(p.a + src_row * p.K) + 16 * kg;
-    }
-    uint8_t* const a_dst = lds + wave * 4096 + lane * 16;   // + stage * kUStage + q * 1024
-    const int x7 = lane & 7;
-    int a_off[4];
-#pragma unroll
-    for (int ks = 0; ks < 4; ks++) a_off[ks] = (lane & 31) * 128 + (((ks + 4 * half) ^ x7) * 16);
-
-    const int n_slices = p.K / kSlice;
-    WSlice<DT> u0, u1;
-    uint4 ar0, ar1, ar2, ar3;   // named, not an array: the array form ends up in scratch memory
-    u0.load(w0, half);
-    u1.load(w1, half);
-    ar0 = *reinterpret_cast<const uint4*>(asrc[0]);
-    ar1 = *reinterpret_cast<const uint4*>(asrc[1]);
-    ar2 = *reinterpret_cast<const uint4*>(asrc[2]);
-    ar3 = *reinterpret_cast<const uint4*>(asrc[3]);
-    *reinterpret_cast<uint4*>(a_dst) = ar0;
-    *reinterpret_cast<uint4*>(a_dst + 1024) = ar1;
-    *reinterpret_cast<uint4*>(a_dst + 2048) = ar2;
-    *reinterpret_cast<uint4*>(a_dst + 3072) = ar3;
-    __syncthreads();
-    for (int s = 0; s < n_slices; s++) {
-        const bool more = s + 1 < n_slices;
-        WSlice<DT> v0, v1;
-        if (more) {   // requests for the next slice
-            v0.load(w0, 2 * (s + 1) + half);
-            v1.load(w1, 2 * (s + 1) + half);
-            const size_t ao = (size_t)(s + 1) * 128;
-            ar0 = *reinterpret_cast<const uint4*>(asrc[0] + ao);
-            ar1 = *reinterpret_cast<const uint4*>(asrc[1] + ao);
-            ar2 = *reinterpret_cast<const uint4*>(asrc[2] + ao);
-            ar3 = *reinterpret_cast<const uint4*>(asrc[3] + ao);
-        }
-        const uint8_t* ap = lds + (s & 1) * kUStage;
-#pragma unroll
-        for (int ks = 0; ks < 4; ks++) {
-            const half8 b0 = u0.frag(ks), b1 = u1.frag(ks);
-#pragma unroll
-            for (int mi = 0; mi < M; mi++) {
-                const half8 a = *reinterpret_cast<const half8*>(ap + a_off[ks] + mi * 4096);
-                acc0[mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b0, acc0[mi], 0, 0, 0);
-                acc1[mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b1, acc1[mi], 0, 0, 0);
-            }
-        }
-        // One wave per SIMD: the decode of the next fragments has to issue between this wave's own matrix
-        // instructions, or the two pipes take turns.  Ask the scheduler for one MFMA, then a share of the VALU work.
-#pragma unroll
-        for (int i = 0; i < 8 * M; i++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x002, 256 / (8 * M), 0);
-        }
-        if (more) {
-            uint8_t* d = a_dst + ((s + 1) & 1) * kUStage;
-            *reinterpret_cast<uint4*>(d) = ar0;
-            *reinterpret_cast<uint4*>(d + 1024) = ar1;
-            *reinterpret_cast<uint4*>(d + 2048) = ar2;
-            *reinterpret_cast<uint4*>(d + 3072) = ar3;
-            u0 = v0;
-            u1 = v1;
-        }
-        __syncthreads();   // the stage just written is complete; the stage just read may be overwritten
-    }
-    tile_epilogue<DOWN, M>(p, t, n0, wave, lane, s_scale, acc0, acc1);
-}
-
-// Weight rows through LDS.  A lane that reads its own row's unit straight from memory makes every load
-// instruction of the wave touch 64 rows, one or two cache lines each: the address unit of the CU, not the
-// matrix pipe, then sets the pace (measured: 93 line look-ups per load instruction, 73 % of the kernel's
-// cycles).  Here each wave copies the next 256 k of its 64 rows (the window: a whole number of blocks, WB
-// bytes per row) into a region of its own with consecutive lanes on consecutive 16-byte chunks of a row, and
-// the units are cut out of LDS.  Row pitch 16 * odd: sixteen lanes reading the same offset of sixteen rows
-// fall on distinct banks.  Windows alternate between two stages; window g + 1 is requested at the first
-// slice of window g and written after its third, one barrier before its first unit is read.
-template <int DT>
-struct StagedW {
-    static constexpr int kBlock = DT == INFR_Q4_0 || DT == INFR_Q4_1 || DT == INFR_Q5_0 || DT == INFR_Q5_1 || DT == INFR_Q8_0 ||
-                                          DT == INFR_IQ4_NL || DT == INFR_MXFP4 ? 32
-                                  : DT == INFR_Q2_0 || DT == INFR_NVFP4 ? 64 : 256;
-    static constexpr int kBlockBytes = DT == INFR_Q4_0 ? 18 : DT == INFR_Q4_1 ? 20 : DT == INFR_Q5_0 ? 22 : DT == INFR_Q5_1 ? 24
-                                       : DT == INFR_Q8_0 ? 34 : DT == INFR_Q2K ? 84 : DT == INFR_Q3K ? 110 : DT == INFR_Q4K ? 144
-                                       : DT == INFR_Q5K ? 176 : DT == INFR_Q6K ? 210 : DT == INFR_IQ4_NL ? 18 : DT == INFR_IQ4_XS ? 136
-                                       : DT == INFR_TQ1_0 ? 54 : DT == INFR_TQ2_0 ? 66 : DT == INFR_Q2_0 ? 18 : DT == INFR_MXFP4 ? 17
-                                       : DT == INFR_NVFP4 ? 36 : DT == INFR_IQ1_S ? 50 : DT == INFR_IQ1_M ? 56 : DT == INFR_IQ2_XXS ? 66
-                                       : DT == INFR_IQ2_XS ? 74 : DT == INFR_IQ2_S ? 82 : DT == INFR_IQ3_XXS ? 98 : DT == INFR_IQ3_S ? 110 : 0;
-    static constexpr int kWB = kBlockBytes * (256 / kBlock);   // bytes of one row in a window of 256 k
-    static constexpr int kChunks = (kWB + 15) / 16;
-    static constexpr int kPitch = 16 * (kChunks | 1);
-    // every block format except Q8_0 (272-byte windows: two stages of four waves would not fit beside the
-    // activation ring); unquantised rows are read in whole cache lines as they are
-    static constexpr bool kOn = kBlockBytes != 0 && DT != INFR_Q8_0;
-    static constexpr size_t kLds = kOn ? (size_t)4 * 2 * 64 * kPitch : 0;
-};
-
-template <int DT, bool DOWN, int M>
-__device__ __forceinline__ void grouped_units_tile_staged(const GroupedParams& p, const Tile& t, int n0, uint8_t* lds,
-                                                          const float* s_scale, uint8_t* wlds) {
-    using W = StagedW<DT>;
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, half = lane >> 5;
-    float16v acc0[M], acc1[M];
-#pragma unroll
-    for (int i = 0; i < M; i++)
-#pragma unroll
-        for (int r = 0; r < 16; r++) acc0[i][r] = acc1[i][r] = 0.0f;
-    const int row_bytes = (p.K / W::kBlock) * W::kBlockBytes;
-    // chunk i of the lane: row (64 i + lane) / kChunks of the wave's 64, 16-byte chunk (64 i + lane) % kChunks
-    const uint8_t* csrc[W::kChunks];
-    int cdst[W::kChunks], coff[W::kChunks];
-#pragma unroll
-    for (int i = 0; i < W::kChunks; i++) {
-        const int idx = 64 * i + lane, r = idx / W::kChunks, ch = idx - r * W::kChunks;
-        const uint8_t* row;
-        if (DOWN) row = p.w0 + (size_t)t.e * p.w0_stride + (size_t)min(n0 + 64 * wave + r, p.N - 1) * row_bytes;
-        else row = (r < 32 ? p.w0 + (size_t)t.e * p.w0_stride : p.w1 + (size_t)t.e * p.w1_stride) +
-                   (size_t)min(n0 + 32 * wave + (r & 31), p.N - 1) * row_bytes;
-        csrc[i] = row + 16 * ch;
-        coff[i] = 16 * ch;
-        cdst[i] = r * W::kPitch + 16 * ch;
-    }
-    uint8_t* const wbase = wlds + wave * (2 * 64 * W::kPitch);
-    const uint8_t* const u0row = wbase + (lane & 31) * W::kPitch;
-    const uint8_t* const u1row = u0row + 32 * W::kPitch;
-    const uint8_t* asrc[4];
-#pragma unroll
-    for (int q = 0; q < 4; q++) {
-        const int tok = 32 * wave + 8 * q + (lane >> 3), kg = (lane & 7) ^ ((lane >> 3) & 7);
-        const int pr = t.p0 + min(tok, t.cnt - 1);
-        const size_t src_row = DOWN ? (size_t)pr : (size_t)(p.pair_src[pr] / p.n_used);
-        asrc[q] = reinterpret_cast<const uint8_t*>(p.a + src_row * p.K) + 16 * kg;
-    }
-    uint8_t* const a_dst = lds + wave * 4096 + lane * 16;
-    const int x7 = lane & 7;
-    int a_off[4];
-#pragma unroll
-    for (int ks = 0; ks < 4; ks++) a_off[ks] = (lane & 31) * 128 + (((ks + 4 * half) ^ x7) * 16);
-
-    const int n_slices = p.K / kSlice, n_win = (n_slices + 3) >> 2;
-    uint4 wreg[W::kChunks];
-    uint4 ar0, ar1, ar2, ar3;   // named, not an array: the array form ends up in scratch memory
-    // a chunk that starts past the row's end (last window of a row that is no whole number of windows) is not read;
-    // one that starts inside may run up to 15 bytes past it, which every buffer of the backend has room for
-    auto request = [&](int g) {
-        const int valid = row_bytes - g * W::kWB;
-        const size_t o = (size_t)g * W::kWB;
-        if (valid >= W::kWB) {   // uniform: only a row's last window can be short
-#pragma unroll
-            for (int i = 0; i < W::kChunks; i++) wreg[i] = ldu<uint4>(csrc[i] + o);
-        } else {
-#pragma unroll
-            for (int i = 0; i < W::kChunks; i++) wreg[i] = ldu<uint4>(csrc[i] + o - (coff[i] < valid ? 0 : coff[i]));
-        }
-    };
-    auto deposit = [&](int g) {
-        uint8_t* d = wbase + (g & 1) * (64 * W::kPitch);
-#pragma unroll
-        for (int i = 0; i < W::kChunks; i++)
-            *reinterpret_cast<uint4*>(d + cdst[i]) = wreg[i];
-    };
-    request(0);
-    ar0 = *reinterpret_cast<const uint4*>(asrc[0]);
-    ar1 = *reinterpret_cast<const uint4*>(asrc[1]);
-    ar2 = *reinterpret_cast<const uint4*>(asrc[2]);
-    ar3 = *reinterpret_cast<const uint4*>(asrc[3]);
-    deposit(0);
-    *reinterpret_cast<uint4*>(a_dst) = ar0;
-    *reinterpret_cast<uint4*>(a_dst + 1024) = ar1;
-    *reinterpret_cast<uint4*>(a_dst + 2048) = ar2;
-    *reinterpret_cast<uint4*>(a_dst + 3072) = ar3;
-    __syncthreads();
-    WSlice<DT> u0, u1;
-    u0.load(u0row, half);
-    u1.load(u1row, half);
-    for (int s = 0; s < n_slices; s++) {
-        const bool more = s + 1 < n_slices;
-        const int g = s >> 2, j = s & 3;
-        WSlice<DT> v0, v1;
-        if (j == 0 && g + 1 < n_win) request(g + 1);
-        if (more) {
-            const int so = (((s + 1) >> 2) & 1) * (64 * W::kPitch), ui = 2 * ((s + 1) & 3) + half;
-            v0.load(u0row + so, ui);
-            v1.load(u1row + so, ui);
-            const size_t ao = (size_t)(s + 1) * 128;
-            ar0 = *reinterpret_cast<const uint4*>(asrc[0] + ao);
-            ar1 = *reinterpret_cast<const uint4*>(asrc[1] + ao);
-            ar2 = *reinterpret_cast<const uint4*>(asrc[2] + ao);
-            ar3 = *reinterpret_cast<const uint4*>(asrc[3] + ao);
-        }
-        const uint8_t* ap = lds + (s & 1) * kUStage;
-#pragma unroll
-        for (int ks = 0; ks < 4; ks++) {
-            const half8 b0 = u0.frag(ks), b1 = u1.frag(ks);
-#pragma unroll
-            for (int mi = 0; mi < M; mi++) {
-                const half8 a = *reinterpret_cast<const half8*>(ap + a_off[ks] + mi * 4096);
-                acc0[mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b0, acc0[mi], 0, 0, 0);
-                acc1[mi] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b1, acc1[mi], 0, 0, 0);
-            }
-        }
-        // One wave per SIMD: the decode of the next fragments has to issue between this wave's own matrix
-        // instructions, or the two pipes take turns.  Ask the scheduler for one MFMA, then a share of the VALU work.
-#pragma unroll
-        for (int i = 0; i < 8 * M; i++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x002, 256 / (8 * M), 0);
-        }
-        if (more) {
-            uint8_t* d = a_dst + ((s + 1) & 1) * kUStage;
-            *reinterpret_cast<uint4*>(d) = ar0;
-            *reinterpret_cast<uint4*>(d + 1024) = ar1;
-            *reinterpret_cast<uint4*>(d + 2048) = ar2;
-            *reinterpret_cast<uint4*>(d + 3072) = ar3;
-            u0 = v0;
-            u1 = v1;
-        }
-        if (j == 2 && g + 1 < n_win) deposit(g + 1);
-        __syncthreads();
-    }
-    tile_epilogue<DOWN, M>(p, t, n0, wave, lane, s_scale, acc0, acc1);
-}
-
-template <int DT, bool DOWN>
-__global__ __launch_bounds__(256) void grouped_units_mfma(GroupedParams p) {
-    __shared__ __attribute__((aligned(16))) uint8_t lds[2 * kUStage];
-    __shared__ __attribute__((aligned(16))) float s_scale[kBM];
-    const int tid = threadIdx.x, lane = tid & 63;
-    Tile t;
-    int nt;
-    if (!find_item(p.offsets, p.n_expert, p.n_tiles_n, lane, t, nt)) return;
-    constexpr int kBN = DOWN ? 256 : 128;
-    if (tid < kBM) {
-        const int pr = t.p0 + min(tid, t.cnt - 1);
-        s_scale[tid] = p.a_scale[DOWN ? pr : p.pair_src[pr] / p.n_used];
-    }
-    if constexpr (StagedW<DT>::kOn) {
-        extern __shared__ __attribute__((aligned(16))) uint8_t wlds[];
-        switch ((t.cnt + 31) >> 5) {
-            case 1: grouped_units_tile_staged<DT, DOWN, 1>(p, t, nt * kBN, lds, s_scale, wlds); break;
-            case 2: grouped_units_tile_staged<DT, DOWN, 2>(p, t, nt * kBN, lds, s_scale, wlds); break;
-            case 3: grouped_units_tile_staged<DT, DOWN, 3>(p, t, nt * kBN, lds, s_scale, wlds); break;
-            default: grouped_units_tile_staged<DT, DOWN, 4>(p, t, nt * kBN, lds, s_scale, wlds); break;
-        }
-    } else {
-        switch ((t.cnt + 31) >> 5) {
-            case 1: grouped_units_tile<DT, DOWN, 1>(p, t, nt * kBN, lds, s_scale); break;
-            case 2: grouped_units_tile<DT, DOWN, 2>(p, t, nt * kBN, lds, s_scale); break;
-            case 3: grouped_units_tile<DT, DOWN, 3>(p, t, nt * kBN, lds, s_scale); break;
-            default: grouped_units_tile<DT, DOWN, 4>(p, t, nt * kBN, lds, s_scale); break;
-        }
-    }
-}
-
-template <int DT, bool DOWN>
-void grouped_units(hipStream_t s, const GroupedParams& p) {
-    const int bn = DOWN ? 256 : 128;
-    GroupedParams q = p;
-    q.n_tiles_n = (p.N + bn - 1) / bn;
-    const int max_tiles = p.n_pairs / kBM + (p.n_expert < p.n_pairs ? p.n_expert : p.n_pairs);
-    static bool attr_set = false;
-    if (!attr_set && StagedW<DT>::kLds) {
-        (void)hipFuncSetAttribute((const void*)grouped_units_mfma<DT, DOWN>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  (int)StagedW<DT>::kLds);
-        attr_set = true;
-    }
-    INFR_LAUNCH((grouped_units_mfma<DT, DOWN>), dim3((unsigned)((max_tiles * q.n_tiles_n + 7) & ~7)), dim3(256), StagedW<DT>::kLds,
-                s, q);
-}
-
-template <bool DOWN>
-void grouped_units_any(hipStream_t s, int dt, const GroupedParams& p) {
-    switch (dt) {
-#define INFR_UNITS(D) case D: grouped_units<D, DOWN>(s, p); break;
-        INFR_FOR_UNIT_FORMATS(INFR_UNITS)
-        INFR_UNITS(INFR_F16) INFR_UNITS(INFR_BF16) INFR_UNITS(INFR_F32)
-#undef INFR_UNITS
-        default: break;
-    }
+    INFR_LAUNCH((grouped_mfma6<D, DOWN>), dim3((unsigned)((max_tiles * q.n_tiles_n + 7) & ~7)), dim3(512), grouped6_lds<D>(), s, q);   // whole rounds of the 8 XCDs
 }
 
 }  // namespace
-
-// The unit-decoder grouped GEMM: any affine format, contraction length a whole number of 64-k slices
-// (and of the format's blocks).  Its activations come from launch_rows_to_f16 in natural k order (ask it
-// for a format without an LDS layout of its own, e.g. INFR_Q5K).
-bool grouped_units_supported(int dt, int k) {
-    if (k <= 0 || k % kSlice != 0) return false;
-    if (dt == INFR_F16 || dt == INFR_BF16 || dt == INFR_F32) return true;   // rounded to f16 (weights beyond 65504 would not fit)
-    const int block = unit_format_block(dt);
-    return block != 0 && k % block == 0;
-}
-void launch_grouped_units_gate_up(hipStream_t s, int dt, const GroupedParams& p) { grouped_units_any<false>(s, dt, p); }
-void launch_grouped_units_down(hipStream_t s, int dt, const GroupedParams& p) { grouped_units_any<true>(s, dt, p); }
 
 bool grouped_supported(int dt, int k) {
     // the k loop runs in groups of four 64-element slices (one K-quant super-block)

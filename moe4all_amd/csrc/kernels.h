@@ -142,6 +142,9 @@ struct GroupedParams {
     int K, N, n_expert, n_used, n_pairs;
     int act, has_clamp; float clamp; int weight_before;
     int n_tiles_n;            // set by the launcher
+#ifdef INFR_GROUPED_TRACE
+    long long* trace;         // measurement builds only: 32 slots per workgroup
+#endif
 };
 // Formats and contraction lengths the grouped kernels take.
 bool grouped_supported(int dt, int k);
