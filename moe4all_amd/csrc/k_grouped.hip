@@ -329,7 +329,8 @@ constexpr int kScaleAt6 = 8 * 8192;       // after the k loop: the pairs' hand-o
 
 // measurement builds: INFR_ABLATE bit 0 = weight loads re-read half-step 0, bit 1 = activation loads re-read slice 0,
 // bit 2 = no unpacking (raw bytes as fragments), bit 3 = one vector instruction in place of each matrix instruction,
-// bit 4 = no k-loop loads at all.  Results are wrong in every case; only the time is of interest.
+// bit 4 = no k-loop loads at all, bit 5 = no weight loads, bit 6 = no activation loads.  Results are wrong in every
+// case; only the time is of interest.
 template <class D>
 __device__ __forceinline__ uint4 chunk_of(const typename D::Blk& k, const typename D::Q& f, const typename D::Prep& c, int ks, int j4) {
     if (INFR_ABLATE & 4) {
@@ -393,11 +394,11 @@ __device__ __forceinline__ void grouped6_tile(const GroupedParams& p, const Grou
         const int hs = (s >> 1) + NW - 1, hc = min(hs, last_hs);
 #pragma unroll
         for (int j = 0; j < NC; j++)
-            if (j >= lo && j < hi && ((j - lo) & 1) == i && hs >= 0)
+            if (j >= lo && j < hi && ((j - lo) & 1) == i && hs >= 0 && !(INFR_ABLATE & 32))
                 dma16(wsrc[j] + ((INFR_ABLATE & 1) ? (size_t)0 : (size_t)(hc >> 1) * D::kStepBytes + ((hc & 1) ? whoff[j] : 0)),
                       w_dst + (uint32_t)(hs % NW) * kWStage + j * 1024);
         const int sa = s + kAhead;
-        if (sa >= 0) {
+        if (sa >= 0 && !(INFR_ABLATE & 64)) {
             const size_t ao = (INFR_ABLATE & 2) ? (size_t)0 : (size_t)min(sa, last) * 128;
             dma16(c.asrc[2 * i] + ao, a_dst + (uint32_t)(sa % NA) * kAStage6 + (2 * i) * 1024);
             dma16(c.asrc[2 * i + 1] + ao, a_dst + (uint32_t)(sa % NA) * kAStage6 + (2 * i + 1) * 1024);
@@ -417,7 +418,7 @@ __device__ __forceinline__ void grouped6_tile(const GroupedParams& p, const Grou
     const int row0 = lane & 31, row1 = 32 + (lane & 31);
 
 #ifdef INFR_GROUPED_TRACE
-    long long wait_loads = 0, wait_barrier = 0;
+    long long wait_loads = 0, wait_barrier = 0, issue_time = 0;
     const long long loop_in = clock64();
 #endif
     // kLate: the wave's two k steps of the previous slice: first-step fragments a0 (read a slice earlier), second-step
@@ -461,8 +462,14 @@ __device__ __forceinline__ void grouped6_tile(const GroupedParams& p, const Grou
         const uint8_t* wst = w_lds + ((s >> 1) % NW) * kWStage;
         if (kLate) {
             // all of the slice's loads first: what follows is one region for the instruction scheduler
+#ifdef INFR_GROUPED_TRACE
+            const long long i_in = clock64();
+#endif
             issue_part(s, j4 & 1, 0);
             issue_part(s, j4 & 1, 1);
+#ifdef INFR_GROUPED_TRACE
+            issue_time += clock64() - i_in;
+#endif
             if (s > 0) contract(c.lds + ((s - 1) % NA) * kAStage6, afirst, held);
         }
         const typename D::Blk k0 = D::read_blk(wst, row0, half), k1 = D::read_blk(wst, row1, half);
@@ -519,6 +526,7 @@ __device__ __forceinline__ void grouped6_tile(const GroupedParams& p, const Grou
     GROUPED_NOTE(8, wait_loads);
     GROUPED_NOTE(9, wait_barrier);
     GROUPED_NOTE(10, clock64() - loop_in);
+    GROUPED_NOTE(11, issue_time);
     if (lane == 0 && p.trace) {
         p.trace[(size_t)blockIdx.x * 32 + 16 + pair + 4 * KH] = wait_loads;
         p.trace[(size_t)blockIdx.x * 32 + 24 + pair + 4 * KH] = wait_barrier;

@@ -20,11 +20,11 @@ static void report(const char* name, const std::vector<long long>& t, int blocks
   printf("%s: first start to last end %.1f us\n", name, (t1 - t0) * 0.01);
   printf("  rows of a tile | items | look-up | set-up | k loop | pair sum | epilogue | whole item   (median us; k loop also min / max)\n");
   for (int m = 1; m <= 4; m++) {
-    std::vector<double> v[6], wl, wb;
+    std::vector<double> v[6], wl, wb, wi;
     for (int b = 0; b < blocks; b++) {
       const long long* r = &t[b * 32];
       if (!r[5] || (r[7] + 31) / 32 != m) continue;
-      if (r[10]) { wl.push_back(100.0 * r[8] / r[10]); wb.push_back(100.0 * r[9] / r[10]); }
+      if (r[10]) { wl.push_back(100.0 * r[8] / r[10]); wb.push_back(100.0 * r[9] / r[10]); wi.push_back(100.0 * r[11] / r[10]); }
       for (int i = 0; i < 5; i++) v[i].push_back((r[i + 1] - r[i]) * 0.01);
       v[5].push_back((r[5] - r[0]) * 0.01);
     }
@@ -44,7 +44,8 @@ static void report(const char* name, const std::vector<long long>& t, int blocks
       }
       printf("\n");
     }
-    if (!wl.empty()) printf("                    of the k loop (first wave): %.0f %% waiting for its loads, %.0f %% at the barrier (medians)\n", med(wl), med(wb));
+    std::sort(wi.begin(), wi.end());
+    if (!wl.empty()) printf("                    of the k loop (first wave): %.0f %% waiting for its loads, %.0f %% at the barrier, %.0f %% issuing loads (medians)\n", med(wl), med(wb), med(wi));
   }
   double busy = 0; int items = 0;
   for (int b = 0; b < blocks; b++) if (t[b * 32 + 5]) { busy += (t[b * 32 + 5] - t[b * 32]) * 0.01; items++; }
