@@ -245,28 +245,31 @@ __device__ __forceinline__ uint32_t lds_address(const void* p) {
     return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void*)p;
 }
 
+// Q4_K: a weight stage holds the whole 144-byte blocks of one 256-k step (four slices), nine 16-byte chunks per row in
+// memory order: a wave-load then reads runs of 144 contiguous bytes (34 cycles of the address path against 59 for a
+// header and 64 code bytes per row and half-step).  Row pitch 144 = 36 banks: sixteen rows, sixteen distinct bank groups.
 struct D4K : MQ4K {
-    static constexpr int kNC = 5, kRowStride = 80, kNA = 4, kStepBytes = 144;   // kStepBytes: a row's bytes per 256 k
+    static constexpr int kNC = 9, kRowStride = 144, kNA = 4, kStepBytes = 144;   // kStepBytes: a row's bytes per 256 k
+    static constexpr int kStageSlices = 4, kNW = 2;   // slices per weight stage, stages in the ring
     static constexpr bool kApart = true;   // a slice is contracted one barrier after it is unpacked (needs a fourth activation stage)
-    // chunk `64 j + lane` of a weight stage: which staged row, where in the super-block its 16
-    // bytes start for the first half, and how far the second half's lie behind
+    // chunk `64 j + lane` of a weight stage: which staged row and where in the super-block its 16 bytes start
     static __device__ __forceinline__ void lane_chunk(int j, int lane, int& row, int& off0, int& hoff) {
         const int c = 64 * j + lane;
-        row = c / 5;
-        const int part = c - 5 * row;   // 0: header, 1..4: code bytes of the half
-        off0 = 16 * part;
-        hoff = part == 0 ? 0 : 64;
+        row = c / 9;
+        off0 = 16 * (c - 9 * row);
+        hoff = 0;
     }
     static __device__ __forceinline__ Blk read_blk(const uint8_t* st, int row, int) {
         return Blk{*reinterpret_cast<const uint4*>(st + row * kRowStride)};
     }
-    static __device__ __forceinline__ Q read_q(const uint8_t* st, int row, int sl, int h) {
+    static __device__ __forceinline__ Q read_q(const uint8_t* st, int row, int sl, int h) {   // sl: slice of the stage
         return Q{*reinterpret_cast<const uint4*>(st + row * kRowStride + 16 + 32 * sl + 16 * h)};
     }
 };
 
 struct D6K : MQ6K {
     static constexpr int kNC = 8, kRowStride = 128, kNA = 4, kStepBytes = 210;
+    static constexpr int kStageSlices = 2, kNW = 3;
     static constexpr bool kApart = true;
     static __device__ __forceinline__ int pos(int row, int part) { return row * kRowStride + ((part + rot7(row)) & 7) * 16; }
     static __device__ __forceinline__ void lane_chunk(int j, int lane, int& row, int& off0, int& hoff) {
@@ -289,6 +292,7 @@ struct D6K : MQ6K {
 // ninth for bytes 120..135 (the last block's upper 16 codes, so that nothing past the row is read).
 struct D80 : MQ80 {
     static constexpr int kNC = 9, kRowStride = 144, kNA = 3, kStepBytes = 272;
+    static constexpr int kStageSlices = 2, kNW = 3;
     static constexpr bool kApart = false;   // 108 KB of weight stages leave room for three activation stages only
     static __device__ __forceinline__ void lane_chunk(int j, int lane, int& row, int& off0, int& hoff) {
         const int c = 64 * j + lane;
@@ -305,10 +309,9 @@ struct D80 : MQ80 {
     }
 };
 
-constexpr int kNW6 = 3;                    // weight stages per wave
 constexpr int kAStage6 = kBM * 128;        // bytes per activation stage
 template <class D>
-constexpr size_t grouped6_lds() { return (size_t)D::kNA * kAStage6 + (size_t)4 * kNW6 * 64 * D::kRowStride; }   // Q6_K: all 160 KB
+constexpr size_t grouped6_lds() { return (size_t)D::kNA * kAStage6 + (size_t)4 * D::kNW * 64 * D::kRowStride; }   // Q6_K: all 160 KB
 constexpr int kScaleAt6 = 8 * 8192;       // after the k loop: the pairs' hand-over area, then the tile's row scales
 
 // Time stamps of every workgroup for a measurement build (-DINFR_GROUPED_TRACE with a buffer in GroupedParams::trace);
@@ -350,7 +353,7 @@ __device__ __forceinline__ float16v mma(const uint4& a, const uint4& b, float16v
 }
 
 struct Grouped6Ctx {
-    uint8_t* lds;             // [kNA activation stages][4 pairs x kNW6 weight stages]
+    uint8_t* lds;             // [kNA activation stages][4 pairs x kNW weight stages]
     const uint8_t* asrc[4];   // the lane's activation chunks of slice 0: quarters 0..3 of the pair's 32 tokens
     int pair, lane, n0;
     Tile t;
@@ -364,7 +367,8 @@ struct Grouped6Ctx {
 template <class D, bool DOWN, int M, int KH>
 __device__ __forceinline__ void grouped6_tile(const GroupedParams& p, const Grouped6Ctx& c, const uint8_t* const (&wsrc)[D::kNC],
                                               const int (&whoff)[D::kNC]) {
-    constexpr int NA = D::kNA, NC = D::kNC, NW = kNW6;
+    constexpr int NA = D::kNA, NC = D::kNC, NW = D::kNW;
+    constexpr bool kWhole = D::kStageSlices == 4;   // a weight stage is a whole 256-k step
     // kApart: a wave unpacks slice s after barrier s and contracts it only after barrier s + 1, next to the unpacking of
     // slice s + 1, so that its matrix and vector instructions are independent and can be interleaved one to seven, and
     // the first k step's activation fragments are read from LDS a slice before they are used.  Activation stage s is
@@ -384,19 +388,31 @@ __device__ __forceinline__ void grouped6_tile(const GroupedParams& p, const Grou
     const uint32_t a_dst = lds0 + upair * 4096;                                   // + stage * kAStage6 + q * 1024
     const uint32_t w_dst = lds0 + NA * kAStage6 + upair * (NW * kWStage);         // + stage * kWStage + j * 1024
     const uint8_t* const w_lds = c.lds + NA * kAStage6 + pair * (NW * kWStage);
-    // Loads the first wave issues while slice s is contracted, in two parts i = 0, 1: of the weight chunks of half-step
-    // s/2 + NW - 1 that belong to the slice's parity (even s: chunks 0..(NC+1)/2-1, odd s: the rest) every second one,
-    // then the activation quarters 2 i and 2 i + 1 of slice s + kAhead.  The last load of a slice is an activation quarter.
+    // Loads the first wave issues while slice s is contracted, in two parts i = 0, 1.  Weight chunks: with half-step
+    // stages, of half-step s/2 + NW - 1 the chunks that belong to the slice's parity (even s: chunks 0..(NC+1)/2-1, odd
+    // s: the rest), every second one per part; with whole-step stages, during the first three slices of a step three
+    // chunks each of the NEXT step (so the last of them is two slices old when that step begins, as kAhead assumes, and
+    // the stage they go to was last read before this step's first barrier).  Then the activation quarters 2 i and
+    // 2 i + 1 of slice s + kAhead.  The last load of a slice is an activation quarter.
     constexpr int kWEven = (NC + 1) / 2;
-    auto issue_part = [&](int s, int odd, int i) {   // odd = s & 1; odd and i are constants where this is called
+    const int last_step = (n_slices >> 2) - 1;
+    auto issue_part = [&](int s, int j4, int i) {   // j4 = s & 3; j4 and i are constants where this is called
         if (KH == 1 || (INFR_ABLATE & 16)) return;
-        const int lo = odd ? kWEven : 0, hi = odd ? NC : kWEven;
-        const int hs = (s >> 1) + NW - 1, hc = min(hs, last_hs);
+        if (kWhole) {
+            const int t = (s >> 2) + 1, tc = min(t, last_step);
 #pragma unroll
-        for (int j = 0; j < NC; j++)
-            if (j >= lo && j < hi && ((j - lo) & 1) == i && hs >= 0 && !(INFR_ABLATE & 32))
-                dma16(wsrc[j] + ((INFR_ABLATE & 1) ? (size_t)0 : (size_t)(hc >> 1) * D::kStepBytes + ((hc & 1) ? whoff[j] : 0)),
-                      w_dst + (uint32_t)(hs % NW) * kWStage + j * 1024);
+            for (int j = 0; j < NC; j++)
+                if (j4 < 3 && j / 3 == j4 && ((j % 3) & 1) == i && !(INFR_ABLATE & 32))
+                    dma16(wsrc[j] + ((INFR_ABLATE & 1) ? (size_t)0 : (size_t)tc * D::kStepBytes), w_dst + (uint32_t)(t % NW) * kWStage + j * 1024);
+        } else {
+            const int odd = j4 & 1, lo = odd ? kWEven : 0, hi = odd ? NC : kWEven;
+            const int hs = (s >> 1) + NW - 1, hc = min(hs, last_hs);
+#pragma unroll
+            for (int j = 0; j < NC; j++)
+                if (j >= lo && j < hi && ((j - lo) & 1) == i && hs >= 0 && !(INFR_ABLATE & 32))
+                    dma16(wsrc[j] + ((INFR_ABLATE & 1) ? (size_t)0 : (size_t)(hc >> 1) * D::kStepBytes + ((hc & 1) ? whoff[j] : 0)),
+                          w_dst + (uint32_t)(hs % NW) * kWStage + j * 1024);
+        }
         const int sa = s + kAhead;
         if (sa >= 0 && !(INFR_ABLATE & 64)) {
             const size_t ao = (INFR_ABLATE & 2) ? (size_t)0 : (size_t)min(sa, last) * 128;
@@ -405,9 +421,9 @@ __device__ __forceinline__ void grouped6_tile(const GroupedParams& p, const Grou
         }
     };
 #pragma unroll
-    for (int s = -2 * (NW - 1); s < 0; s++)
+    for (int s = -4; s < 0; s++)
 #pragma unroll
-        for (int i = 0; i < 2; i++) issue_part(s, s & 1, i);
+        for (int i = 0; i < 2; i++) issue_part(s, s & 3, i);
 
     // operand reads: token 32 mi + (lane & 31), k chunk ks + 4 half, rotated by the token's number
     const int x7 = rot7(lane & 31);
@@ -446,8 +462,8 @@ __device__ __forceinline__ void grouped6_tile(const GroupedParams& p, const Grou
         // loads of the first wave younger than the last one this slice needs (an activation quarter of slice s, issued
         // at the end of slice s - kAhead): everything it issued during the kAhead - 1 slices since
         constexpr int kWOdd = NC - kWEven;
-        constexpr int kYoung = KH == 1 ? 0 : kAhead == 3 ? 8 + NC : 4 + ((j4 & 1) ? kWEven : kWOdd);
-        static_assert(kAhead == 2 || kAhead == 3, "the load counts above are written for these distances");
+        constexpr int kYoung = KH == 1 ? 0 : kWhole ? (j4 == 0 ? 4 : 7) : kAhead == 3 ? 8 + NC : 4 + ((j4 & 1) ? kWEven : kWOdd);
+        static_assert(kAhead == 2 || (kAhead == 3 && !kWhole), "the load counts above are written for these distances");
 #ifdef INFR_GROUPED_TRACE
         const long long w_in = clock64();
         asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" : : "n"(kYoung) : "memory");
@@ -459,21 +475,21 @@ __device__ __forceinline__ void grouped6_tile(const GroupedParams& p, const Grou
         wait_loads_then_barrier<kYoung>();
 #endif
         const uint8_t* ap = c.lds + (s % NA) * kAStage6;
-        const uint8_t* wst = w_lds + ((s >> 1) % NW) * kWStage;
+        const uint8_t* wst = w_lds + (kWhole ? (s >> 2) % NW : (s >> 1) % NW) * kWStage;
         if (kLate) {
             // all of the slice's loads first: what follows is one region for the instruction scheduler
 #ifdef INFR_GROUPED_TRACE
             const long long i_in = clock64();
 #endif
-            issue_part(s, j4 & 1, 0);
-            issue_part(s, j4 & 1, 1);
+            issue_part(s, j4, 0);
+            issue_part(s, j4, 1);
 #ifdef INFR_GROUPED_TRACE
             issue_time += clock64() - i_in;
 #endif
             if (s > 0) contract(c.lds + ((s - 1) % NA) * kAStage6, afirst, held);
         }
         const typename D::Blk k0 = D::read_blk(wst, row0, half), k1 = D::read_blk(wst, row1, half);
-        const typename D::Q f0 = D::read_q(wst, row0, j4 & 1, half), f1 = D::read_q(wst, row1, j4 & 1, half);
+        const typename D::Q f0 = D::read_q(wst, row0, j4 % D::kStageSlices, half), f1 = D::read_q(wst, row1, j4 % D::kStageSlices, half);
         const typename D::Prep c0 = D::prep(k0, f0, j4, half), c1 = D::prep(k1, f1, j4, half);
         if (kLate) {
             held[0] = chunk_of<D>(k0, f0, c0, 2 * KH, j4);
@@ -500,7 +516,7 @@ __device__ __forceinline__ void grouped6_tile(const GroupedParams& p, const Grou
                     nb0 = chunk_of<D>(k0, f0, c0, 2 * KH + 1, j4);
                     nb1 = chunk_of<D>(k1, f1, c1, 2 * KH + 1, j4);
                 }
-                issue_part(s, j4 & 1, i);
+                issue_part(s, j4, i);
 #pragma unroll
                 for (int mi = 0; mi < M; mi++) {
                     acc0[mi] = mma(a[mi], b0, acc0[mi]);
