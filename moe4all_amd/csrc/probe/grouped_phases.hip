@@ -50,6 +50,14 @@ static void report(const char* name, const std::vector<long long>& t, int blocks
   double busy = 0; int items = 0;
   for (int b = 0; b < blocks; b++) if (t[b * 32 + 5]) { busy += (t[b * 32 + 5] - t[b * 32]) * 0.01; items++; }
   printf("  %d items, sum of item times / 256 CUs = %.1f us\n", items, busy / 256);
+  // per XCD (workgroup b runs on XCD b & 7): its items' time over its 32 CUs, and when its last item ends
+  printf("  per XCD, sum of item times / 32 CUs | last end:");
+  for (int x = 0; x < 8; x++) {
+    double bx = 0; long long e = 0;
+    for (int b = x; b < blocks; b += 8) if (t[b * 32 + 5]) { bx += (t[b * 32 + 5] - t[b * 32]) * 0.01; e = std::max(e, t[b * 32 + 5]); }
+    printf("  %.0f | %.0f", bx / 32, (e - t0) * 0.01);
+  }
+  printf("\n");
 }
 
 int main(int argc, char** argv) {
