@@ -403,7 +403,11 @@ __device__ __forceinline__ void grouped6_tile(const GroupedParams& p, const Grou
 #pragma unroll
             for (int j = 0; j < NC; j++)
                 if (j4 < 3 && j / 3 == j4 && ((j % 3) & 1) == i && !(INFR_ABLATE & 32))
+#ifdef INFR_W_CONTIG
+                    dma16(wsrc[j] + (size_t)tc * D::kStepBytes * p.N, w_dst + (uint32_t)(t % NW) * kWStage + j * 1024);
+#else
                     dma16(wsrc[j] + ((INFR_ABLATE & 1) ? (size_t)0 : (size_t)tc * D::kStepBytes), w_dst + (uint32_t)(t % NW) * kWStage + j * 1024);
+#endif
         } else {
             const int odd = j4 & 1, lo = odd ? kWEven : 0, hi = odd ? NC : kWEven;
             const int hs = (s >> 1) + NW - 1, hc = min(hs, last_hs);
@@ -629,7 +633,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             base = row < 32 ? p.w0 + (size_t)t.e * p.w0_stride : p.w1 + (size_t)t.e * p.w1_stride;
             f = c.n0 + 32 * c.pair + (row & 31);
         }
+#ifdef INFR_W_CONTIG   // measurement builds: banks laid out [step][row][block] (timing only, the data is not re-laid)
+        wsrc[j] = base + (size_t)min(f, p.N - 1) * D::kStepBytes + off0;
+#else
         wsrc[j] = base + (size_t)min(f, p.N - 1) * row_bytes + off0;
+#endif
     }
     // the lane's activation chunks: token 32 pair + 8 q + lane / 8, chunk (lane & 7) ^ rot7(token)
 #pragma unroll
