@@ -197,7 +197,9 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const uint8_t* __res
 // Logits for a batch (f32 router, ne a multiple of 32).  Block = 512 threads covering 32 experts
 // x 32 token rows: 8 chains x 8 row groups per wave, one wave per group of 4 experts.  A thread
 // keeps a 4 x 4 (expert, row) patch of accumulators for its chain, so each 128-bit LDS read
-// feeds 16 FMAs.  k advances in chunks of 128 elements staged transposed (chain-major) in LDS;
+// feeds 16 FMAs.  The patch's rows are G apart (rows b * G + rg): the sixteen lanes the LDS serves together then read
+// sixteen consecutive 80-byte rows, which fall on distinct banks (rows 32 apart are 2560 bytes = a whole number of
+// bank rounds apart and collided).  k advances in chunks of 128 elements staged transposed (chain-major) in LDS;
 // the accumulators run through all chunks, so every chain still adds its terms in ascending
 // order, exactly as the scalar reference does.
 constexpr int kLtChunk = 128, kLtStride = kLtChunk / 8 + 4;
@@ -259,13 +261,13 @@ __global__ __launch_bounds__((kLtTile / P) * (kLtTile / P) * 8) void router_logi
         if (k0 + kLtChunk < ne) fetch(k0 + kLtChunk);
         const int n_c = min(kLtChunk, ne - k0) >> 3;  // a multiple of 4
         const float* wp = sw + (eg * P * 8 + j) * kLtStride;
-        const float* xp = sx + (rg * P * 8 + j) * kLtStride;
+        const float* xp = sx + (rg * 8 + j) * kLtStride;   // the thread's rows: b * G + rg
         for (int c = 0; c < n_c; c += 4) {
             float4 wv[P], xv[P];
 #pragma unroll
             for (int a = 0; a < P; a++) {
                 wv[a] = *reinterpret_cast<const float4*>(wp + a * 8 * kLtStride + c);
-                xv[a] = *reinterpret_cast<const float4*>(xp + a * 8 * kLtStride + c);
+                xv[a] = *reinterpret_cast<const float4*>(xp + a * G * 8 * kLtStride + c);
             }
 #pragma unroll
             for (int a = 0; a < P; a++)
@@ -286,7 +288,7 @@ __global__ __launch_bounds__((kLtTile / P) * (kLtTile / P) * 8) void router_logi
             float s = 0.0f;
 #pragma unroll
             for (int jj = 0; jj < 8; jj++) s = __fadd_rn(s, __shfl(acc[a][b], (lane & ~7) + jj, kWave));
-            const int e = e0 + eg * P + a, r = r0 + rg * P + b;
+            const int e = e0 + eg * P + a, r = r0 + b * G + rg;
             if (j == 0 && e < n_expert && r < rows) logits[(size_t)r * n_expert + e] = s;
         }
 }
