@@ -283,6 +283,31 @@ def measure(be, stack, config, batch, steps, warmup, *, sublayer=False, kernel_t
             roofline["floor_launch_us"] = round(st, 3)
             roofline["achievable_frac"] = round(kernels[dom]["alg_bytes"] / (st * 1e-6) / 1e9 / HBM_PEAK_GBPS, 4)
 
+    # ---- prefill: what the dominant GEMM's data movement alone takes.  The same launches with the kernels' measurement
+    # variant (loads, LDS reads and barriers as built; no unpacking, no matrix instructions; output meaningless)
+    if floor and kernels and prefill and roofline and roofline["bound"] == "mfma":
+        be.probe_grouped_loads_only(True)
+        try:
+            be.prof_enable(True)
+            for i in range(max(1, min(steps, 30))):
+                be.execute(plan, binds[i % N_TOKENS])
+            be.sync()
+            prof = be.prof_read()
+            be.prof_enable(False)
+        finally:
+            be.probe_grouped_loads_only(False)
+        lo = {k: p["total_ms"] * 1e3 / max(p["launches"], 1) for k, p in prof.items() if k in flops}
+        if lo:
+            dom = roofline["kernel"]
+            floor_out = {"kernels": sorted(lo), "launch_us": [round(lo[k], 3) for k in sorted(lo)],
+                         "note": "the same grouped GEMM launches moving their data (global -> LDS loads, LDS reads, barriers) "
+                                 "without unpacking weights or issuing matrix instructions"}
+            if dom in lo:
+                roofline["floor_launch_us"] = round(lo[dom], 3)
+                roofline["frac_of_data_movement_floor"] = round(lo[dom] / kernels[dom]["avg_us"], 4)
+        be.execute(plan, binds[0])   # leave real results behind
+        be.sync()
+
     # ---- CPU baseline: the oracle on this host's cores, layer 0's weights, a bounded sample
     cpu = None
     if cpu_budget_s > 0:

@@ -276,6 +276,11 @@ typedef struct infr_hip_prof_entry {
 } infr_hip_prof_entry;
 infr_status infr_hip_prof_enable(infr_hip_backend *be, int on);
 infr_status infr_hip_prof_read(infr_hip_backend *be, infr_hip_prof_entry *out, uint32_t cap, uint32_t *n_out);
+/* Measurement only (no counterpart in the reference).  on != 0: from now on the grouped GEMMs of the batched
+ * Op::MoeFfn / Op::Linear paths (Q4_K / Q6_K / Q8_0 weights) run their loads, LDS reads and barriers but neither
+ * unpack weights nor issue matrix instructions, so their launch time is what the kernels' data movement alone takes.
+ * Everything such launches write is meaningless; switch it off again before using results. */
+infr_status infr_hip_probe_grouped_loads_only(infr_hip_backend *be, int on);
 
 /* Debug taps used by the parity tests: Op::MoeFfn's routing decision and bucketing of the
  * LAST executed MoeFfn op of `plan` (the reference exposes the same facts through

@@ -221,6 +221,7 @@ _SIGNATURES = {
     "infr_hip_sync": ([_V], C.c_int),
     "infr_hip_last_error": ([], C.c_char_p),
     "infr_hip_prof_enable": ([_V, C.c_int], C.c_int),
+    "infr_hip_probe_grouped_loads_only": ([_V, C.c_int], C.c_int),
     "infr_hip_prof_read": ([_V, C.POINTER(_ProfEntry), C.c_uint32, C.POINTER(C.c_uint32)], C.c_int),
     "infr_hip_plan_moe_routing": ([_V, _V, C.c_uint32, _V, _V, _V, _V], C.c_int),
     "infr_hip_plan_moe_bucketing": ([_V, _V, C.c_uint32, _V, _V, _V], C.c_int),
@@ -580,6 +581,10 @@ class Backend:
     # ---- taps
     def prof_enable(self, on: bool = True) -> None:
         _check(self._lib.infr_hip_prof_enable(self._h, int(on)))
+
+    def probe_grouped_loads_only(self, on: bool = True) -> None:
+        """Measurement only: the batched path's grouped GEMMs move their data but skip unpacking and matrix work."""
+        _check(self._lib.infr_hip_probe_grouped_loads_only(self._h, int(on)))
 
     def prof_read(self) -> dict:
         n = C.c_uint32()

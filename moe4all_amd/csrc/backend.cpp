@@ -210,6 +210,7 @@ struct infr_hip_backend {
     infr_hip_config cfg{};
     std::mutex mu;  // serialises stream submission and profiling state
     std::atomic<int> prof_on{0};
+    std::atomic<bool> probe_grouped_loads_only{false};   // measurement: see infr_hip_probe_grouped_loads_only
     std::map<std::string, ProfSlot> prof;
     struct Pending { std::string name; hipEvent_t a, b; };
     std::vector<Pending> pending;
@@ -1483,6 +1484,7 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                         infr::launch_rows_to_f16(s, a_dt_gu, gp.x, rows, (int)m.ne, sc.xh, sc.xs);
                     }
                     infr::GroupedParams q{};
+                    q.loads_only = be->probe_grouped_loads_only.load() ? 1 : 0;
                     q.a = sc.xh; q.a_scale = sc.xs; q.offsets = sc.offsets; q.pair_src = sc.pair_src;
                     q.w0 = gp.gate; q.w0_stride = gp.gate_stride; q.w1 = gp.up; q.w1_stride = gp.up_stride;
                     q.route_w = sc.weights; q.down_scale = nullptr; q.out = sc.h;
@@ -1624,6 +1626,7 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                         infr::launch_rows_to_f16(s, mode == 2 ? INFR_Q8_0 : dt, (const float*)ptr[l.x], (int)l.m, (int)l.in_f, xh, xs);
                     }
                     infr::GroupedParams q{};
+                    q.loads_only = be->probe_grouped_loads_only.load() ? 1 : 0;
                     q.a = xh; q.a_scale = xs;
                     q.offsets = (const int32_t*)((const char*)plan->arena + plan->lin[oi].offsets_off);
                     q.w0 = w; q.w0_stride = 0;
@@ -1827,6 +1830,12 @@ extern "C" infr_status infr_hip_probe_dependent_reads(infr_hip_backend* be, cons
 } catch (...) { return guard_fail("infr_hip_probe_dependent_reads"); }
 
 // ============================================================================ taps
+extern "C" infr_status infr_hip_probe_grouped_loads_only(infr_hip_backend* be, int on) try {
+    if (!ok_backend(be)) return fail(INFR_ERR_INVALID, "probe: bad handle");
+    be->probe_grouped_loads_only.store(on != 0);
+    return INFR_OK;
+} catch (...) { return guard_fail("infr_hip_probe_grouped_loads_only"); }
+
 extern "C" infr_status infr_hip_prof_enable(infr_hip_backend* be, int on) try {
     if (!ok_backend(be)) return fail(INFR_ERR_INVALID, "prof: bad handle");
     std::lock_guard<std::mutex> lk(be->mu);

@@ -330,21 +330,23 @@ constexpr int kScaleAt6 = 8 * 8192;       // after the k loop: the pairs' hand-o
 #define GROUPED_NOTE(i, v) do { } while (0)
 #endif
 
-// measurement builds: INFR_ABLATE bit 0 = weight loads re-read half-step 0, bit 1 = activation loads re-read slice 0,
+// measurement variants (template parameter ABL; -DINFR_ABLATE=<bits> makes one the default of a probe build):
+// bit 0 = weight loads re-read half-step 0, bit 1 = activation loads re-read slice 0,
 // bit 2 = no unpacking (raw bytes as fragments), bit 3 = one vector instruction in place of each matrix instruction,
 // bit 4 = no k-loop loads at all, bit 5 = no weight loads, bit 6 = no activation loads.  Results are wrong in every
 // case; only the time is of interest.
-template <class D>
+template <class D, int ABL>
 __device__ __forceinline__ uint4 chunk_of(const typename D::Blk& k, const typename D::Q& f, const typename D::Prep& c, int ks, int j4) {
-    if (INFR_ABLATE & 4) {
+    if (ABL & 4) {
         uint4 r = *reinterpret_cast<const uint4*>(&f);
         r.x += ks;
         return r;
     }
     return D::chunk(k, f, c, ks, j4);
 }
+template <int ABL>
 __device__ __forceinline__ float16v mma(const uint4& a, const uint4& b, float16v acc) {
-    if (INFR_ABLATE & 8) {
+    if (ABL & 8) {
         acc[0] += __uint_as_float((a.x ^ b.x) & 0x3FFFFFFFu);
         acc[1] += __uint_as_float((a.w ^ b.w) & 0x3FFFFFFFu);
         return acc;
@@ -364,7 +366,7 @@ struct Grouped6Ctx {
 // up the wave that issues it until the address unit has taken it (with rows of 80 to 144 bytes a wave-load touches 20
 // to 30 cache lines), and the first wave, being the older one on its SIMD, is served first and has time to spare before
 // every barrier.
-template <class D, bool DOWN, int M, int KH>
+template <class D, bool DOWN, int M, int KH, int ABL>
 __device__ __forceinline__ void grouped6_tile(const GroupedParams& p, const Grouped6Ctx& c, const uint8_t* const (&wsrc)[D::kNC],
                                               const int (&whoff)[D::kNC]) {
     constexpr int NA = D::kNA, NC = D::kNC, NW = D::kNW;
@@ -397,29 +399,29 @@ __device__ __forceinline__ void grouped6_tile(const GroupedParams& p, const Grou
     constexpr int kWEven = (NC + 1) / 2;
     const int last_step = (n_slices >> 2) - 1;
     auto issue_part = [&](int s, int j4, int i) {   // j4 = s & 3; j4 and i are constants where this is called
-        if (KH == 1 || (INFR_ABLATE & 16)) return;
+        if (KH == 1 || (ABL & 16)) return;
         if (kWhole) {
             const int t = (s >> 2) + 1, tc = min(t, last_step);
 #pragma unroll
             for (int j = 0; j < NC; j++)
-                if (j4 < 3 && j / 3 == j4 && ((j % 3) & 1) == i && !(INFR_ABLATE & 32))
+                if (j4 < 3 && j / 3 == j4 && ((j % 3) & 1) == i && !(ABL & 32))
 #ifdef INFR_W_CONTIG
                     dma16(wsrc[j] + (size_t)tc * D::kStepBytes * p.N, w_dst + (uint32_t)(t % NW) * kWStage + j * 1024);
 #else
-                    dma16(wsrc[j] + ((INFR_ABLATE & 1) ? (size_t)0 : (size_t)tc * D::kStepBytes), w_dst + (uint32_t)(t % NW) * kWStage + j * 1024);
+                    dma16(wsrc[j] + ((ABL & 1) ? (size_t)0 : (size_t)tc * D::kStepBytes), w_dst + (uint32_t)(t % NW) * kWStage + j * 1024);
 #endif
         } else {
             const int odd = j4 & 1, lo = odd ? kWEven : 0, hi = odd ? NC : kWEven;
             const int hs = (s >> 1) + NW - 1, hc = min(hs, last_hs);
 #pragma unroll
             for (int j = 0; j < NC; j++)
-                if (j >= lo && j < hi && ((j - lo) & 1) == i && hs >= 0 && !(INFR_ABLATE & 32))
-                    dma16(wsrc[j] + ((INFR_ABLATE & 1) ? (size_t)0 : (size_t)(hc >> 1) * D::kStepBytes + ((hc & 1) ? whoff[j] : 0)),
+                if (j >= lo && j < hi && ((j - lo) & 1) == i && hs >= 0 && !(ABL & 32))
+                    dma16(wsrc[j] + ((ABL & 1) ? (size_t)0 : (size_t)(hc >> 1) * D::kStepBytes + ((hc & 1) ? whoff[j] : 0)),
                           w_dst + (uint32_t)(hs % NW) * kWStage + j * 1024);
         }
         const int sa = s + kAhead;
-        if (sa >= 0 && !(INFR_ABLATE & 64)) {
-            const size_t ao = (INFR_ABLATE & 2) ? (size_t)0 : (size_t)min(sa, last) * 128;
+        if (sa >= 0 && !(ABL & 64)) {
+            const size_t ao = (ABL & 2) ? (size_t)0 : (size_t)min(sa, last) * 128;
             dma16(c.asrc[2 * i] + ao, a_dst + (uint32_t)(sa % NA) * kAStage6 + (2 * i) * 1024);
             dma16(c.asrc[2 * i + 1] + ao, a_dst + (uint32_t)(sa % NA) * kAStage6 + (2 * i + 1) * 1024);
         }
@@ -449,13 +451,13 @@ __device__ __forceinline__ void grouped6_tile(const GroupedParams& p, const Grou
         for (int mi = 0; mi < M; mi++) a1[mi] = *reinterpret_cast<const uint4*>(ap + a_off[1] + mi * 4096);
 #pragma unroll
         for (int mi = 0; mi < M; mi++) {
-            acc0[mi] = mma(a0[mi], b[0], acc0[mi]);
-            acc1[mi] = mma(a0[mi], b[1], acc1[mi]);
+            acc0[mi] = mma<ABL>(a0[mi], b[0], acc0[mi]);
+            acc1[mi] = mma<ABL>(a0[mi], b[1], acc1[mi]);
         }
 #pragma unroll
         for (int mi = 0; mi < M; mi++) {
-            acc0[mi] = mma(a1[mi], b[2], acc0[mi]);
-            acc1[mi] = mma(a1[mi], b[3], acc1[mi]);
+            acc0[mi] = mma<ABL>(a1[mi], b[2], acc0[mi]);
+            acc1[mi] = mma<ABL>(a1[mi], b[3], acc1[mi]);
         }
     };
     uint4 afirst[M] = {};   // kLate: the first k step's activation fragments of the previous slice
@@ -496,10 +498,10 @@ __device__ __forceinline__ void grouped6_tile(const GroupedParams& p, const Grou
         const typename D::Q f0 = D::read_q(wst, row0, j4 % D::kStageSlices, half), f1 = D::read_q(wst, row1, j4 % D::kStageSlices, half);
         const typename D::Prep c0 = D::prep(k0, f0, j4, half), c1 = D::prep(k1, f1, j4, half);
         if (kLate) {
-            held[0] = chunk_of<D>(k0, f0, c0, 2 * KH, j4);
-            held[1] = chunk_of<D>(k1, f1, c1, 2 * KH, j4);
-            held[2] = chunk_of<D>(k0, f0, c0, 2 * KH + 1, j4);
-            held[3] = chunk_of<D>(k1, f1, c1, 2 * KH + 1, j4);
+            held[0] = chunk_of<D, ABL>(k0, f0, c0, 2 * KH, j4);
+            held[1] = chunk_of<D, ABL>(k1, f1, c1, 2 * KH, j4);
+            held[2] = chunk_of<D, ABL>(k0, f0, c0, 2 * KH + 1, j4);
+            held[3] = chunk_of<D, ABL>(k1, f1, c1, 2 * KH + 1, j4);
 #pragma unroll
             for (int mi = 0; mi < M; mi++) afirst[mi] = *reinterpret_cast<const uint4*>(ap + a_off[0] + mi * 4096);
             // one matrix instruction, then a share of the vector work
@@ -512,19 +514,19 @@ __device__ __forceinline__ void grouped6_tile(const GroupedParams& p, const Grou
             uint4 a[M];
 #pragma unroll
             for (int mi = 0; mi < M; mi++) a[mi] = *reinterpret_cast<const uint4*>(ap + a_off[0] + mi * 4096);
-            uint4 b0 = chunk_of<D>(k0, f0, c0, 2 * KH, j4), b1 = chunk_of<D>(k1, f1, c1, 2 * KH, j4);
+            uint4 b0 = chunk_of<D, ABL>(k0, f0, c0, 2 * KH, j4), b1 = chunk_of<D, ABL>(k1, f1, c1, 2 * KH, j4);
 #pragma unroll
             for (int i = 0; i < 2; i++) {
                 uint4 nb0 = b0, nb1 = b1;
                 if (i < 1) {
-                    nb0 = chunk_of<D>(k0, f0, c0, 2 * KH + 1, j4);
-                    nb1 = chunk_of<D>(k1, f1, c1, 2 * KH + 1, j4);
+                    nb0 = chunk_of<D, ABL>(k0, f0, c0, 2 * KH + 1, j4);
+                    nb1 = chunk_of<D, ABL>(k1, f1, c1, 2 * KH + 1, j4);
                 }
                 issue_part(s, j4, i);
 #pragma unroll
                 for (int mi = 0; mi < M; mi++) {
-                    acc0[mi] = mma(a[mi], b0, acc0[mi]);
-                    acc1[mi] = mma(a[mi], b1, acc1[mi]);
+                    acc0[mi] = mma<ABL>(a[mi], b0, acc0[mi]);
+                    acc1[mi] = mma<ABL>(a[mi], b1, acc1[mi]);
                     if (i < 1) a[mi] = *reinterpret_cast<const uint4*>(ap + a_off[1] + mi * 4096);
                 }
                 b0 = nb0;
@@ -599,7 +601,8 @@ __device__ __forceinline__ void grouped6_tile(const GroupedParams& p, const Grou
     GROUPED_STAMP(5);
 }
 
-template <class D, bool DOWN>
+// ABL: measurement variants (see chunk_of); 0 in the product path
+template <class D, bool DOWN, int ABL = INFR_ABLATE>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void grouped_mfma6(GroupedParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds6[];
     Grouped6Ctx c;
@@ -650,8 +653,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const int m = (t.cnt + 31) >> 5;
     GROUPED_STAMP(2);
 #define INFR_TILE(MM)                                                     \
-    if (kh) grouped6_tile<D, DOWN, MM, 1>(p, c, wsrc, whoff);             \
-    else grouped6_tile<D, DOWN, MM, 0>(p, c, wsrc, whoff)
+    if (kh) grouped6_tile<D, DOWN, MM, 1, ABL>(p, c, wsrc, whoff);        \
+    else grouped6_tile<D, DOWN, MM, 0, ABL>(p, c, wsrc, whoff)
     if (m == 1) { INFR_TILE(1); }
     else if (m == 2) { INFR_TILE(2); }
     else if (m == 3) { INFR_TILE(3); }
@@ -777,13 +780,18 @@ void grouped6(hipStream_t s, const GroupedParams& p) {
     GroupedParams q = p;
     q.n_tiles_n = (p.N + bn - 1) / bn;
     const int max_tiles = p.n_pairs / kBM + (p.n_expert < p.n_pairs ? p.n_expert : p.n_pairs);
+    const dim3 grid((unsigned)((max_tiles * q.n_tiles_n + 7) & ~7));   // whole rounds of the 8 XCDs
     static bool attr_set = false;  // per instantiation
     if (!attr_set) {
         (void)hipFuncSetAttribute((const void*)grouped_mfma6<D, DOWN>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                   (int)grouped6_lds<D>());
+        (void)hipFuncSetAttribute((const void*)grouped_mfma6<D, DOWN, 12>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                  (int)grouped6_lds<D>());
         attr_set = true;
     }
-    INFR_LAUNCH((grouped_mfma6<D, DOWN>), dim3((unsigned)((max_tiles * q.n_tiles_n + 7) & ~7)), dim3(512), grouped6_lds<D>(), s, q);   // whole rounds of the 8 XCDs
+    // loads_only: the measurement variant without unpacking and matrix instructions (its output is meaningless)
+    if (p.loads_only) INFR_LAUNCH((grouped_mfma6<D, DOWN, 12>), grid, dim3(512), grouped6_lds<D>(), s, q);
+    else INFR_LAUNCH((grouped_mfma6<D, DOWN>), grid, dim3(512), grouped6_lds<D>(), s, q);
 }
 
 }  // namespace

@@ -142,6 +142,7 @@ struct GroupedParams {
     int K, N, n_expert, n_used, n_pairs;
     int act, has_clamp; float clamp; int weight_before;
     int n_tiles_n;            // set by the launcher
+    int loads_only;           // measurement: run the GEMM's loads, LDS reads and barriers without unpacking or matrix work
 #ifdef INFR_GROUPED_TRACE
     long long* trace;         // measurement builds only: 32 slots per workgroup
 #endif

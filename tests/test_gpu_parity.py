@@ -1507,3 +1507,38 @@ def test_disabling_op_fusion_changes_the_launches_not_the_bits(rows, gated):
     sh_o = O.linear(O.gated_act_rows(O.linear(xn_o, wg, H.Q4K, ne, nff), O.linear(xn_o, wu, H.Q4K, ne, nff)), wd, H.Q6K, nff, ne)
     sub_o = O.moe_shared_expert_add(moe_o["dst"], sh_o, O.linear(xn_o, wq, H.F32, ne, 1)) if gated else O.add(moe_o["dst"], sh_o)
     assert H.rel_l2(outs[False].reshape(rows, ne) - x, sub_o.reshape(rows, ne)) < REL_L2
+
+
+@pytest.mark.gpu
+def test_loads_only_probe_moves_data_without_results_and_switches_off_cleanly():
+    """infr_hip_probe_grouped_loads_only: the measurement variant of the grouped GEMMs runs (same launches, same
+    kernels' names), what it writes is not the layer's output, and after switching it off the backend gives the
+    bits it gave before."""
+    rows, ne, E, K, nff = 96, 512, 8, 2, 256
+    rng = np.random.default_rng(17)
+    x = rng.standard_normal((rows, ne)).astype(np.float32)
+    router = (rng.standard_normal((E, ne)) * 0.02).astype(np.float32)
+    gate, up = _realistic(rng, E, nff, ne, H.Q4K), _realistic(rng, E, nff, ne, H.Q4K)
+    down = _realistic(rng, E, ne, nff, H.Q6K)
+    be2 = M.Backend(0)
+    try:
+        data = dict(x=x, router=router, gate=gate, up=up, down=down)
+        g, ids = moe_graph(rows, ne, E, K, nff, DType.Q4K, DType.Q6K)
+        before, _, _ = _run_batched(be2, g, ids, data, rows, ne)
+        be2.probe_grouped_loads_only(True)
+        be2.prof_enable(True)
+        g2, ids2 = moe_graph(rows, ne, E, K, nff, DType.Q4K, DType.Q6K)
+        probed, r, _ = _run_batched(be2, g2, ids2, data, rows, ne)
+        names = set(be2.prof_read())
+        be2.prof_enable(False)
+        be2.probe_grouped_loads_only(False)
+        assert {"moe_grouped_gate_up", "moe_grouped_down"} <= names
+        assert not np.array_equal(probed, before)          # no matrix work was done
+        g3, ids3 = moe_graph(rows, ne, E, K, nff, DType.Q4K, DType.Q6K)
+        after, _, _ = _run_batched(be2, g3, ids3, data, rows, ne)
+        assert np.array_equal(after.view(np.uint32), before.view(np.uint32))
+    finally:
+        be2.close()
+
+
+
