@@ -396,8 +396,10 @@ __device__ __forceinline__ void grouped6_tile(const GroupedParams& p, const Grou
     // chunks each of the NEXT step (so the last of them is two slices old when that step begins, as kAhead assumes, and
     // the stage they go to was last read before this step's first barrier).  Then the activation quarters 2 i and
     // 2 i + 1 of slice s + kAhead.  The last load of a slice is an activation quarter.
+    // A pair whose 32 tokens lie beyond the tile's rows (pair >= M) loads no activations: nothing reads them.
     constexpr int kWEven = (NC + 1) / 2;
     const int last_step = (n_slices >> 2) - 1;
+    const bool loads_a = pair < M;
     auto issue_part = [&](int s, int j4, int i) {   // j4 = s & 3; j4 and i are constants where this is called
         if (KH == 1 || (ABL & 16)) return;
         if (kWhole) {
@@ -420,7 +422,7 @@ __device__ __forceinline__ void grouped6_tile(const GroupedParams& p, const Grou
                           w_dst + (uint32_t)(hs % NW) * kWStage + j * 1024);
         }
         const int sa = s + kAhead;
-        if (sa >= 0 && !(ABL & 64)) {
+        if (sa >= 0 && loads_a && !(ABL & 64)) {
             const size_t ao = (ABL & 2) ? (size_t)0 : (size_t)min(sa, last) * 128;
             dma16(c.asrc[2 * i] + ao, a_dst + (uint32_t)(sa % NA) * kAStage6 + (2 * i) * 1024);
             dma16(c.asrc[2 * i + 1] + ao, a_dst + (uint32_t)(sa % NA) * kAStage6 + (2 * i + 1) * 1024);
@@ -468,17 +470,20 @@ __device__ __forceinline__ void grouped6_tile(const GroupedParams& p, const Grou
         // loads of the first wave younger than the last one this slice needs (an activation quarter of slice s, issued
         // at the end of slice s - kAhead): everything it issued during the kAhead - 1 slices since
         constexpr int kWOdd = NC - kWEven;
-        constexpr int kYoung = KH == 1 ? 0 : kWhole ? (j4 == 0 ? 4 : 7) : kAhead == 3 ? 8 + NC : 4 + ((j4 & 1) ? kWEven : kWOdd);
+        constexpr int kYoungW = kWhole ? (j4 == 0 ? 0 : 3) : kAhead == 3 ? NC : ((j4 & 1) ? kWEven : kWOdd);   // weight loads among them
+        constexpr int kYoung = KH == 1 ? 0 : kYoungW + 4 * (kAhead - 1);
         static_assert(kAhead == 2 || (kAhead == 3 && !kWhole), "the load counts above are written for these distances");
 #ifdef INFR_GROUPED_TRACE
         const long long w_in = clock64();
-        asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" : : "n"(kYoung) : "memory");
+        if (loads_a) asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" : : "n"(kYoung) : "memory");
+        else asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" : : "n"(KH == 1 ? 0 : kYoungW) : "memory");
         const long long w_mid = clock64();
         asm volatile("s_barrier" ::: "memory");
         wait_loads += w_mid - w_in;
         wait_barrier += clock64() - w_mid;
 #else
-        wait_loads_then_barrier<kYoung>();
+        if (loads_a) wait_loads_then_barrier<kYoung>();
+        else wait_loads_then_barrier<(KH == 1 ? 0 : kYoungW)>();
 #endif
         const uint8_t* ap = c.lds + (s % NA) * kAStage6;
         const uint8_t* wst = w_lds + (kWhole ? (s >> 2) % NW : (s >> 1) % NW) * kWStage;
