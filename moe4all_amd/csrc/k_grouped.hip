@@ -312,7 +312,7 @@ struct D80 : MQ80 {
 constexpr int kAStage6 = kBM * 128;        // bytes per activation stage
 template <class D>
 constexpr size_t grouped6_lds() { return (size_t)D::kNA * kAStage6 + (size_t)4 * D::kNW * 64 * D::kRowStride; }   // Q6_K: all 160 KB
-constexpr int kScaleAt6 = 8 * 8192;       // after the k loop: the pairs' hand-over area, then the tile's row scales
+constexpr int kScaleAt6 = 8 * 16384;      // after the k loop: the pairs' hand-over area (16 KB per wave), then the tile's row scales
 
 // Time stamps of every workgroup for a measurement build (-DINFR_GROUPED_TRACE with a buffer in GroupedParams::trace);
 // compiled out otherwise.
@@ -561,44 +561,36 @@ __device__ __forceinline__ void grouped6_tile(const GroupedParams& p, const Grou
 #endif
 
     // The pair's two partial sums: each wave hands over the accumulator registers the other one stores (this wave keeps
-    // registers 8 KH .. 8 KH + 7 of every tile) through the ring memory, two row tiles per round, 8 KB per wave.
+    // registers 8 KH .. 8 KH + 7 of every tile) through the ring memory, 4 KB per row tile and wave, in one round.
+    static_assert(grouped6_lds<D>() >= kScaleAt6 + kBM * 4, "hand-over area and row scales fit the rings");
     float* const s_scale = reinterpret_cast<float*>(c.lds + kScaleAt6);
-    uint8_t* const mine = c.lds + (size_t)(pair + 4 * KH) * 8192 + lane * 16;
-    const uint8_t* const theirs = c.lds + (size_t)(pair + 4 * (1 - KH)) * 8192 + lane * 16;
+    uint8_t* const mine = c.lds + (size_t)(pair + 4 * KH) * 16384 + lane * 16;
+    const uint8_t* const theirs = c.lds + (size_t)(pair + 4 * (1 - KH)) * 16384 + lane * 16;
+    __syncthreads();   // the rings have been read by everyone
+    if (KH == 0 && lane < 32) {   // the tile's row scales for the epilogue
+        const int pr = c.t.p0 + min(32 * pair + lane, c.t.cnt - 1);
+        s_scale[32 * pair + lane] = p.a_scale[DOWN ? pr : p.pair_src[pr] / p.n_used];
+    }
 #pragma unroll
-    for (int g = 0; g < (M + 1) / 2; g++) {
-        __syncthreads();   // the rings (first round) or the previous round's hand-over have been read by everyone
-        if (g == 0 && KH == 0 && lane < 32) {   // the tile's row scales for the epilogue
-            const int pr = c.t.p0 + min(32 * pair + lane, c.t.cnt - 1);
-            s_scale[32 * pair + lane] = p.a_scale[DOWN ? pr : p.pair_src[pr] / p.n_used];
-        }
+    for (int mi = 0; mi < M; mi++) {
+        constexpr int o = 8 * (1 - KH);
+        *reinterpret_cast<float4*>(mine + (4 * mi + 0) * 1024) = make_float4(acc0[mi][o], acc0[mi][o + 1], acc0[mi][o + 2], acc0[mi][o + 3]);
+        *reinterpret_cast<float4*>(mine + (4 * mi + 1) * 1024) = make_float4(acc0[mi][o + 4], acc0[mi][o + 5], acc0[mi][o + 6], acc0[mi][o + 7]);
+        *reinterpret_cast<float4*>(mine + (4 * mi + 2) * 1024) = make_float4(acc1[mi][o], acc1[mi][o + 1], acc1[mi][o + 2], acc1[mi][o + 3]);
+        *reinterpret_cast<float4*>(mine + (4 * mi + 3) * 1024) = make_float4(acc1[mi][o + 4], acc1[mi][o + 5], acc1[mi][o + 6], acc1[mi][o + 7]);
+    }
+    __syncthreads();
 #pragma unroll
-        for (int q = 0; q < 2; q++) {
-            const int mi = 2 * g + q;
-            if (mi < M) {
-                constexpr int o = 8 * (1 - KH);
-                *reinterpret_cast<float4*>(mine + (4 * q + 0) * 1024) = make_float4(acc0[mi][o], acc0[mi][o + 1], acc0[mi][o + 2], acc0[mi][o + 3]);
-                *reinterpret_cast<float4*>(mine + (4 * q + 1) * 1024) = make_float4(acc0[mi][o + 4], acc0[mi][o + 5], acc0[mi][o + 6], acc0[mi][o + 7]);
-                *reinterpret_cast<float4*>(mine + (4 * q + 2) * 1024) = make_float4(acc1[mi][o], acc1[mi][o + 1], acc1[mi][o + 2], acc1[mi][o + 3]);
-                *reinterpret_cast<float4*>(mine + (4 * q + 3) * 1024) = make_float4(acc1[mi][o + 4], acc1[mi][o + 5], acc1[mi][o + 6], acc1[mi][o + 7]);
-            }
-        }
-        __syncthreads();
+    for (int mi = 0; mi < M; mi++) {
+        constexpr int o = 8 * KH;
+        const float4 v0 = *reinterpret_cast<const float4*>(theirs + (4 * mi + 0) * 1024), v1 = *reinterpret_cast<const float4*>(theirs + (4 * mi + 1) * 1024);
+        const float4 v2 = *reinterpret_cast<const float4*>(theirs + (4 * mi + 2) * 1024), v3 = *reinterpret_cast<const float4*>(theirs + (4 * mi + 3) * 1024);
+        // first wave's part + second wave's part, whichever of the two this is
+        const float t0[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w}, t1[8] = {v2.x, v2.y, v2.z, v2.w, v3.x, v3.y, v3.z, v3.w};
 #pragma unroll
-        for (int q = 0; q < 2; q++) {
-            const int mi = 2 * g + q;
-            if (mi < M) {
-                constexpr int o = 8 * KH;
-                const float4 v0 = *reinterpret_cast<const float4*>(theirs + (4 * q + 0) * 1024), v1 = *reinterpret_cast<const float4*>(theirs + (4 * q + 1) * 1024);
-                const float4 v2 = *reinterpret_cast<const float4*>(theirs + (4 * q + 2) * 1024), v3 = *reinterpret_cast<const float4*>(theirs + (4 * q + 3) * 1024);
-                // first wave's part + second wave's part, whichever of the two this is
-                const float t0[8] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w}, t1[8] = {v2.x, v2.y, v2.z, v2.w, v3.x, v3.y, v3.z, v3.w};
-#pragma unroll
-                for (int r = 0; r < 8; r++) {
-                    acc0[mi][o + r] = KH ? t0[r] + acc0[mi][o + r] : acc0[mi][o + r] + t0[r];
-                    acc1[mi][o + r] = KH ? t1[r] + acc1[mi][o + r] : acc1[mi][o + r] + t1[r];
-                }
-            }
+        for (int r = 0; r < 8; r++) {
+            acc0[mi][o + r] = KH ? t0[r] + acc0[mi][o + r] : acc0[mi][o + r] + t0[r];
+            acc1[mi][o + r] = KH ? t1[r] + acc1[mi][o + r] : acc1[mi][o + r] + t1[r];
         }
     }
     GROUPED_STAMP(4);
