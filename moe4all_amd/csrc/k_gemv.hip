@@ -22,10 +22,29 @@
 // reference as closely as a reordered f32 summation does.
 #include "device_common.h"
 #include "kernels.h"
+#ifdef INFR_GEMV_TRACE
+// the routing's own time stamps go to slots 8..15 of the block's record
+namespace infr { __device__ long long* g_route_trace; }
+#define ROUTE_STAMP(i)                                                                                                 \
+    do {                                                                                                               \
+        if (lane == 0 && infr::g_route_trace) infr::g_route_trace[((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 16 + 8 + (i)] = wall_clock64(); \
+    } while (0)
+#endif
 #include "route.h"
 #include "gemv_fmt.h"
 
 namespace infr {
+
+// Time stamps of every block for a measurement build (-DINFR_GEMV_TRACE with a buffer in p.y, which these kernels do
+// not use otherwise); compiled out in the library.
+#ifdef INFR_GEMV_TRACE
+#define GEMV_STAMP(i)                                                                                                  \
+    do {                                                                                                               \
+        if (threadIdx.x == 0 && p.y) reinterpret_cast<long long*>(p.y)[((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 16 + (i)] = wall_clock64(); \
+    } while (0)
+#else
+#define GEMV_STAMP(i) do { } while (0)
+#endif
 
 // ------------------------------------------------------------------------------- gate/up
 // grid.x = tiles of `ft` features, grid.y = token row.  A block's 4 waves share the items
@@ -97,7 +116,7 @@ __device__ __forceinline__ void gu_finish(const GuStage<F, U>& st, const MoeGemv
 // finished, so a wave always has a stage in flight while it computes.
 template <class F, int U, bool PIPE>
 __global__ __launch_bounds__(256) void moe_gate_up_fast(MoeGemvParams p, int ft) {
-    extern __shared__ uint32_t dyn_lds[];
+    extern __shared__ __attribute__((aligned(16))) uint32_t dyn_lds[];
     __shared__ uint64_t s_tab[32];
     __shared__ int32_t s_ids[64];
     __shared__ float s_w[64];
@@ -114,6 +133,7 @@ __global__ __launch_bounds__(256) void moe_gate_up_fast(MoeGemvParams p, int ft)
     const Place<F> pl(nblk, lane);
     const size_t cell_words = (size_t)((p.ne + 31) / 32) * kCellDwords;
     uint32_t* cells = dyn_lds + (size_t)wave * cell_words;
+    GEMV_STAMP(0);
     // x is requested first; it does not depend on the routing
     const float* xrow = p.x + (size_t)r * p.ne;
     const XLoad xl = stage_x_load(xrow, p.ne, lane);
@@ -135,6 +155,7 @@ __global__ __launch_bounds__(256) void moe_gate_up_fast(MoeGemvParams p, int ft)
     }
     __syncthreads();
     __builtin_amdgcn_wave_barrier();
+    GEMV_STAMP(1);
     t.nitems = t.fcount * t.n_slots;
     const int step = 4 * pl.rw_count * U;
     typename F::X x;
@@ -149,17 +170,24 @@ __global__ __launch_bounds__(256) void moe_gate_up_fast(MoeGemvParams p, int ft)
                 __builtin_amdgcn_wave_barrier();
                 F::fetch_x(x, cells, pl.blk, pl.sub);
                 have_x = true;
+                GEMV_STAMP(2);
             }
             gu_finish<F, U>(st, p, pl, t, x, nblk, base, s_g, s_u, s_w, s_tab);
+            if (base == 0) GEMV_STAMP(3);
         }
     } else {
         GuStage<F, U> sa, sb;
         gu_issue<F, U>(sa, p, pl, t, s_ids, 0);
+        GEMV_STAMP(5);
         gu_issue<F, U>(sb, p, pl, t, s_ids, step);
+        GEMV_STAMP(6);
         stage_x_finish<F::kGroup, F::kSigned>(xl, xrow, p.ne, cells, lane);
         __builtin_amdgcn_wave_barrier();
+        GEMV_STAMP(7);
         F::fetch_x(x, cells, pl.blk, pl.sub);
+        GEMV_STAMP(2);
         gu_finish<F, U>(sa, p, pl, t, x, nblk, 0, s_g, s_u, s_w, s_tab);
+        GEMV_STAMP(3);
         int base = step;   // the stage sb holds
         for (;;) {
             if (base + step >= t.nitems) {
@@ -178,6 +206,154 @@ __global__ __launch_bounds__(256) void moe_gate_up_fast(MoeGemvParams p, int ft)
             base += step;
         }
     }
+    GEMV_STAMP(4);
+}
+
+// ------------------------------------------------------------------------------- gate/up, streamed
+// The same tiles as moe_gate_up_fast, for tiles of several items per wave.  Three things differ.  The routing wave
+// and the conversion of x run side by side: wave 0 routes (or fetches the ids) while waves 1..3 turn x into one set of
+// fixed-point cells for the whole block.  A wave keeps D items (a gate row and an up row each) in flight as a ring:
+// it finishes the oldest item and requests the item D places ahead into the registers that just became free, so its
+// dot products and its loads alternate item by item and the four waves drift apart instead of all waiting for memory
+// and then all computing.  Results wait in LDS until the wave has finished a chunk of its items, then one lane per
+// item applies the gated activation.
+template <class F, int D, int NW>
+__global__ __launch_bounds__(64 * NW, NW <= 8 ? 4 : 3) void moe_gate_up_stream(MoeGemvParams p, int ft) {
+    extern __shared__ __attribute__((aligned(16))) uint32_t dyn_lds[];
+    __shared__ uint64_t s_tab[32];
+    __shared__ int32_t s_ids[64];
+    __shared__ float s_w[64];
+    __shared__ float s_g[NW][64], s_u[NW][64];
+    __shared__ RouteDuo s_duo;
+    const int r = blockIdx.y;
+    const int f0 = blockIdx.x * ft;
+    const int fcount = min(ft, p.nff - f0);
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int nblk = p.ne / F::kBlockElems;
+    const size_t row_bytes = (size_t)nblk * F::kBlockBytes;
+    const Place<F> pl(nblk, lane);
+    const int ncell = (p.ne + 31) / 32;
+    uint32_t* cells = dyn_lds;
+    GEMV_STAMP(0);
+    const float* xrow = p.x + (size_t)r * p.ne;
+    float* route_lds = reinterpret_cast<float*>(dyn_lds + (size_t)ncell * kCellDwords);
+    // plain softmax routing runs on waves 0 and 1 (sum and selection side by side), anything else on wave 0
+    const int duo_ns = !(p.route_inline && route_duo_ok(p.route)) ? 0 : p.route.n_expert <= 128 ? 2 : p.route.n_expert <= 256 ? 4 : 8;
+    const int first_conv = duo_ns ? 2 : 1;   // the waves from here on turn x into cells
+    float pr[8];
+    if (wave < first_conv) {
+        if (duo_ns == 2) route_duo_first<2>(p.route, r, wave, lane, route_lds, s_tab, &s_duo, reinterpret_cast<float(&)[2]>(pr));
+        else if (duo_ns == 4) route_duo_first<4>(p.route, r, wave, lane, route_lds, s_tab, &s_duo, reinterpret_cast<float(&)[4]>(pr));
+        else if (duo_ns == 8) route_duo_first<8>(p.route, r, wave, lane, route_lds, s_tab, &s_duo, pr);
+        else if (p.route_inline) {
+            route_row_any(p.route, r, lane, route_lds, s_tab, s_ids, s_w, blockIdx.x == 0, s_tab);
+        } else {
+            if (lane < p.n_used) {   // n_used <= 64
+                s_ids[lane] = p.ids[(size_t)r * p.n_used + lane];
+                s_w[lane] = p.weights[(size_t)r * p.n_used + lane];
+            }
+            if (lane < 32) s_tab[lane] = kExp2Table[lane];
+        }
+    } else {
+        for (int c0 = (int)threadIdx.x - 64 * first_conv; c0 < ncell; c0 += 64 * (NW - first_conv)) {
+            const XLoad l = stage_x_load(xrow, p.ne, c0);
+            stage_x_convert<F::kGroup, F::kSigned>(l, p.ne, c0, cells);
+        }
+    }
+    const int n_slots = p.n_used + (p.sh_gate ? 1 : 0);   // the always-on expert is slot n_used (<= 63 then)
+    if (p.sh_gate && threadIdx.x == 64 * NW - 1) {
+        s_ids[p.n_used] = 0;
+        s_w[p.n_used] = 1.0f;
+    }
+    __syncthreads();
+    if (duo_ns) {
+        if (wave == 0) {
+            const bool store = blockIdx.x == 0;
+            bool done;
+            if (duo_ns == 2) done = route_duo_second<2>(p.route, r, lane, &s_duo, reinterpret_cast<float(&)[2]>(pr), s_ids, s_w, store);
+            else if (duo_ns == 4) done = route_duo_second<4>(p.route, r, lane, &s_duo, reinterpret_cast<float(&)[4]>(pr), s_ids, s_w, store);
+            else done = route_duo_second<8>(p.route, r, lane, &s_duo, pr, s_ids, s_w, store);
+            if (!done) route_row_any(p.route, r, lane, route_lds, s_tab, s_ids, s_w, store);
+        }
+        __syncthreads();
+    }
+    GEMV_STAMP(1);
+    typename F::X x;
+    F::fetch_x(x, cells, pl.blk, pl.sub);
+    const int nitems = fcount * n_slots;
+    const int per_step = NW * pl.rw_count;   // items the block's waves take per ring step
+    const int n_mine = nitems > wave * pl.rw_count ? (nitems - wave * pl.rw_count + per_step - 1) / per_step : 0;
+    const float inv_fcount = 1.0f / (float)fcount;
+    // item j of this wave's rows: (slot, feature), exact for the few thousand items a tile can hold
+    auto issue = [&](GuStage<F, 1>& st, int j) {
+        const int it = min((j * NW + wave) * pl.rw_count + pl.rw, nitems - 1);
+        const int slot = (int)(((float)it + 0.5f) * inv_fcount), f = f0 + (it - slot * fcount);
+        const int e = s_ids[slot];
+        const bool routed = slot < p.n_used;
+        const uint8_t* gb = routed ? p.gate + (size_t)e * p.gate_stride : p.sh_gate;
+        const uint8_t* ub = routed ? p.up + (size_t)e * p.up_stride : p.sh_up;
+        st.g[0] = load_row<F>(pl, gb + (size_t)f * row_bytes);
+        st.u[0] = load_row<F>(pl, ub + (size_t)f * row_bytes);
+    };
+    const int chunk = 64 / pl.rw_count;   // items of a wave whose results fit its staging row
+    for (int c0 = 0; c0 < n_mine; c0 += chunk) {
+        const int cn = min(chunk, n_mine - c0);
+        GuStage<F, 1> ring[D];
+        auto finish = [&](const GuStage<F, 1>& st, int j) {
+            const float gs = row_sum<F>(F::dot(st.g[0], pl.sub, x), pl, nblk);
+            const float us = row_sum<F>(F::dot(st.u[0], pl.sub, x), pl, nblk);
+            if (pl.writer()) {
+                s_g[wave][j * pl.rw_count + pl.rw] = gs;
+                s_u[wave][j * pl.rw_count + pl.rw] = us;
+            }
+        };
+#pragma unroll
+        for (int d = 0; d < D; d++)
+            if (d < cn) issue(ring[d], c0 + d);
+        if (c0 == 0) GEMV_STAMP(2);
+        // steady state: every step finishes its ring entry and refills it, no branch in between, so the waits count
+        // exactly the loads that are younger than the entry
+        const int refills = cn - D;   // steps that still have an item to request
+        int j0 = 0;
+        for (; j0 + D <= refills; j0 += D) {
+#pragma unroll
+            for (int d = 0; d < D; d++) {
+                finish(ring[d], j0 + d);
+                issue(ring[d], c0 + j0 + d + D);
+            }
+            if (c0 == 0 && j0 == 0) GEMV_STAMP(3);
+        }
+        // the last refills, then the entries still in flight
+#pragma unroll
+        for (int d = 0; d < D; d++) {
+            if (j0 + d >= cn) break;
+            finish(ring[d], j0 + d);
+            if (j0 + d < refills) issue(ring[d], c0 + j0 + d + D);
+        }
+        j0 += D;
+#pragma unroll
+        for (int d = 0; d < D; d++) {
+            if (j0 + d >= cn) break;
+            finish(ring[d], j0 + d);
+        }
+        __builtin_amdgcn_wave_barrier();
+        if (lane < cn * pl.rw_count) {
+            const int j = lane / pl.rw_count, rw = lane - j * pl.rw_count;
+            const int it = ((c0 + j) * NW + wave) * pl.rw_count + rw;
+            if (it < nitems) {
+                const int slot = (int)(((float)it + 0.5f) * inv_fcount), f = f0 + (it - slot * fcount);
+                float gs = s_g[wave][lane], us = s_u[wave][lane];
+                if (p.weight_before && slot < p.n_used) {
+                    const float wp = s_w[slot];
+                    gs = __fmul_rn(wp, gs);
+                    us = __fmul_rn(wp, us);
+                }
+                p.h[((size_t)r * n_slots + slot) * p.nff + f] = gated_act_fn(p.act, p.has_clamp, p.clamp, gs, us, s_tab);
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+    GEMV_STAMP(4);
 }
 
 // ------------------------------------------------------------------------------- down
@@ -224,7 +400,7 @@ __device__ __forceinline__ void down_finish(const typename F::Raw (&raw)[S], con
 // the next stage's loads in flight while it finishes the current one.
 template <class F, int S, bool PIPE>
 __global__ __launch_bounds__(512) void moe_down_combine_fast(MoeGemvParams p, int ot) {
-    extern __shared__ uint32_t dyn_lds[];
+    extern __shared__ __attribute__((aligned(16))) uint32_t dyn_lds[];
     __shared__ float ypart[kMaxUsedFast][kMaxOt];
     const int r = blockIdx.y;
     const int o0 = blockIdx.x * ot;
@@ -237,6 +413,7 @@ __global__ __launch_bounds__(512) void moe_down_combine_fast(MoeGemvParams p, in
     DownTile t;
     t.ocount = min(ot, p.ne - o0);
     t.row_bytes = (size_t)nblk * F::kBlockBytes;
+    GEMV_STAMP(0);
 
     const int n_slots = p.n_used + (p.sh_down ? 1 : 0);   // the always-on expert is slot n_used
     for (int slot = wave; slot < n_slots; slot += nwaves) {
@@ -249,6 +426,7 @@ __global__ __launch_bounds__(512) void moe_down_combine_fast(MoeGemvParams p, in
         t.scaled = p.down_scale && routed;
         typename F::Raw ra[S];
         down_issue<F, S>(ra, pl, t, bank, 0);
+        if (slot == wave) GEMV_STAMP(1);
         typename F::X x;
         if (!PIPE) {
             // while the weights are in flight: this slot's h to fixed point, once per wave
@@ -256,8 +434,10 @@ __global__ __launch_bounds__(512) void moe_down_combine_fast(MoeGemvParams p, in
             stage_x_finish<F::kGroup, F::kSigned>(xl, hrow, p.nff, cells, lane);
             __builtin_amdgcn_wave_barrier();
             F::fetch_x(x, cells, pl.blk, pl.sub);
+            if (slot == wave) GEMV_STAMP(2);
             t.ds = t.scaled ? p.down_scale[e] : 1.0f;
             down_finish<F, S>(ra, pl, t, x, nblk, 0, ypart);
+            if (slot == wave) GEMV_STAMP(3);
         } else {
             const int gstep = S * pl.rw_count;
             typename F::Raw rb[S];
@@ -288,7 +468,9 @@ __global__ __launch_bounds__(512) void moe_down_combine_fast(MoeGemvParams p, in
             __builtin_amdgcn_wave_barrier();   // the next slot's h overwrites this wave's cells
         }
     }
+    GEMV_STAMP(4);
     __syncthreads();
+    GEMV_STAMP(5);
     for (int o = threadIdx.x; o < t.ocount; o += blockDim.x) {
         const float* w = p.weights + (size_t)r * p.n_used;
         float acc = 0.0f;
@@ -302,6 +484,135 @@ __global__ __launch_bounds__(512) void moe_down_combine_fast(MoeGemvParams p, in
         const size_t oi = (size_t)r * p.ne + o0 + o;
         p.dst[oi] = p.addend ? __fadd_rn(p.addend[oi], acc) : acc;
     }
+    GEMV_STAMP(6);
+}
+
+// ------------------------------------------------------------------------------- down, streamed
+// The same tiles as moe_down_combine_fast with the work cut differently: a tile's units (slot, group of rows a wave
+// covers at once) are dealt to the block's 8 waves in equal contiguous runs, so nine slots keep eight waves equally
+// busy, and a wave keeps D units in flight as a ring (finish the oldest, request the unit D places ahead into the
+// registers that became free).  h of every slot is turned into fixed-point cells once, by the whole block; a wave
+// fetches a slot's cells when its run crosses into that slot.
+template <class F, int D, int NW>
+__global__ __launch_bounds__(64 * NW) void moe_down_combine_stream(MoeGemvParams p, int ot) {
+    extern __shared__ __attribute__((aligned(16))) uint32_t dyn_lds[];
+    __shared__ float ypart[kMaxUsedFast][kMaxOt];
+    __shared__ int32_t s_ids[kMaxUsedFast];
+    __shared__ float s_w[kMaxUsedFast], s_ds[kMaxUsedFast];
+    __shared__ int s_skip[kMaxUsedFast];
+    const int r = blockIdx.y;
+    const int o0 = blockIdx.x * ot;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int nblk = p.nff / F::kBlockElems;
+    const Place<F> pl(nblk, lane);
+    const size_t row_bytes = (size_t)nblk * F::kBlockBytes;
+    const int ocount = min(ot, p.ne - o0);
+    const int n_slots = p.n_used + (p.sh_down ? 1 : 0);   // the always-on expert is slot n_used
+    const int ncell = (p.nff + 31) / 32;
+    const size_t cell_words = (size_t)ncell * kCellDwords;
+    GEMV_STAMP(0);
+    // ids and routing weights first: every weight address waits on the ids
+    if ((int)threadIdx.x < n_slots) {
+        const int k = threadIdx.x;
+        const bool routed = k < p.n_used;
+        const int e = routed ? p.ids[(size_t)r * p.n_used + k] : 0;
+        const float w = routed ? p.weights[(size_t)r * p.n_used + k] : 1.0f;
+        float wk = (p.weight_before || !routed) ? 1.0f : w;
+        if (!routed && p.sh_logit)   // crates/infr-cpu/src/lib.rs:3336-3356: sigmoid of the row's gate logit
+            wk = __fdiv_rn(1.0f, __fadd_rn(1.0f, expf_libm(-p.sh_logit[r])));
+        s_ids[k] = e;
+        s_w[k] = wk;
+        s_skip[k] = p.skip_zero_w && routed && w == 0.0f;
+        s_ds[k] = (p.down_scale && routed) ? p.down_scale[e] : 1.0f;
+    }
+    // h of every slot, requested before the weights so that its conversion does not wait behind them
+    const int total_cells = n_slots * ncell;
+    const int my_cell = threadIdx.x;   // further cells of this thread follow in the loop below
+    const int slot0 = my_cell / ncell;
+    const float* hbase = p.h + (size_t)r * n_slots * p.nff;
+    XLoad hl;
+    if (my_cell < total_cells) hl = stage_x_load(hbase + (size_t)slot0 * p.nff, p.nff, my_cell - slot0 * ncell);
+    __syncthreads();
+    const int G = (ocount + pl.rw_count - 1) / pl.rw_count;   // units per slot
+    const int n_units = n_slots * G;
+    const int upw = (n_units + NW - 1) / NW;
+    const int ub = wave * upw;
+    const int cn = max(0, min(upw, n_units - ub));
+    const float inv_G = 1.0f / (float)G;
+    auto issue = [&](typename F::Raw& raw, int j) {
+        const int u = ub + j;
+        const int slot = (int)(((float)u + 0.5f) * inv_G), rg = u - slot * G;
+        const int o = min(rg * pl.rw_count + pl.rw, ocount - 1);
+        const uint8_t* bank = slot < p.n_used ? p.down + (size_t)s_ids[slot] * p.down_stride : p.sh_down;
+        raw = load_row<F>(pl, bank + (size_t)(o0 + o) * row_bytes);
+    };
+    typename F::Raw ring[D];
+#pragma unroll
+    for (int d = 0; d < D; d++)
+        if (d < cn) issue(ring[d], d);
+    GEMV_STAMP(1);
+    // h to fixed point, once per block
+    if (my_cell < total_cells)
+        stage_x_convert<F::kGroup, F::kSigned>(hl, p.nff, my_cell - slot0 * ncell, dyn_lds + slot0 * cell_words);
+    for (int c = my_cell + (int)blockDim.x; c < total_cells; c += blockDim.x) {
+        const int sl = c / ncell;
+        const XLoad l = stage_x_load(hbase + (size_t)sl * p.nff, p.nff, c - sl * ncell);
+        stage_x_convert<F::kGroup, F::kSigned>(l, p.nff, c - sl * ncell, dyn_lds + sl * cell_words);
+    }
+    __syncthreads();
+    GEMV_STAMP(2);
+    typename F::X x;
+    int cur_slot = -1;
+    float ds = 1.0f;
+    auto finish = [&](const typename F::Raw& raw, int j) {
+        const int u = ub + j;
+        const int slot = (int)(((float)u + 0.5f) * inv_G), rg = u - slot * G;
+        if (slot != cur_slot) {   // the same for the whole wave
+            F::fetch_x(x, dyn_lds + slot * cell_words, pl.blk, pl.sub);
+            ds = s_ds[slot];
+            cur_slot = slot;
+        }
+        const int o = rg * pl.rw_count + pl.rw;
+        const float y = row_sum<F>(F::dot(raw, pl.sub, x), pl, nblk);
+        if (o < ocount && pl.writer()) ypart[slot][o] = (p.down_scale && slot < p.n_used) ? __fmul_rn(y, ds) : y;
+    };
+    const int refills = cn - D;
+    int j0 = 0;
+    for (; j0 + D <= refills; j0 += D) {
+#pragma unroll
+        for (int d = 0; d < D; d++) {
+            finish(ring[d], j0 + d);
+            issue(ring[d], j0 + d + D);
+        }
+    }
+#pragma unroll
+    for (int d = 0; d < D; d++) {
+        if (j0 + d >= cn) break;
+        finish(ring[d], j0 + d);
+        if (j0 + d < refills) issue(ring[d], j0 + d + D);
+    }
+    j0 += D;
+#pragma unroll
+    for (int d = 0; d < D; d++) {
+        if (j0 + d >= cn) break;
+        finish(ring[d], j0 + d);
+    }
+#ifdef INFR_GEMV_TRACE
+    if (lane == 0 && p.y) reinterpret_cast<long long*>(p.y)[((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 16 + 8 + (wave & 7)] = wall_clock64();
+#endif
+    GEMV_STAMP(4);
+    __syncthreads();
+    GEMV_STAMP(5);
+    for (int o = threadIdx.x; o < ocount; o += blockDim.x) {
+        float acc = 0.0f;
+        for (int k = 0; k < n_slots; k++) {
+            if (s_skip[k]) continue;
+            acc = __fadd_rn(acc, __fmul_rn(s_w[k], ypart[k][o]));
+        }
+        const size_t oi = (size_t)r * p.ne + o0 + o;
+        p.dst[oi] = p.addend ? __fadd_rn(p.addend[oi], acc) : acc;
+    }
+    GEMV_STAMP(6);
 }
 
 // ------------------------------------------------------------------------------- generic
@@ -381,7 +692,9 @@ static bool try_gate_up(hipStream_t s, const MoeGemvParams& p) {
     const int rw = 64 / (p.ne / F::kBlockElems * F::kLPB);
     // about one block per compute unit; a block's ft * n_slots items go to 4 waves of rw rows each
     const int n_slots = p.n_used + (p.sh_gate ? 1 : 0);
-    int ft = ceil_div(p.nff, p.n_cu);
+    // about one block per compute unit for a single token row; with several rows about two, resident together, so
+    // that a compute unit pays a block's start (routing, x) once while it streams
+    int ft = p.rows >= 2 ? ceil_div(p.nff * p.rows, 2 * p.n_cu) : ceil_div(p.nff, p.n_cu);
     if (ft < 1) ft = 1;
     const int per_wave = ceil_div(ft * n_slots, 4 * rw);
     // tiles of three or more stages stream with the next stage in flight
@@ -392,6 +705,16 @@ static bool try_gate_up(hipStream_t s, const MoeGemvParams& p) {
     while (u * rw > 64) u--;
     const size_t lds = 4 * cells_bytes(p.ne) +
                        (p.route_inline ? route_scratch_floats(p.route.n_expert, p.route.n_groups) * sizeof(float) : 0);
+    if (per_wave >= 3) {
+        // several items per wave: streamed, one set of cells for the block
+        const size_t lds_s = cells_bytes(p.ne) +
+                             (p.route_inline ? route_scratch_floats(p.route.n_expert, p.route.n_groups) * sizeof(float) : 0);
+        // one token row: twelve waves, each with one item in flight, cover the memory latency between them; with
+        // several rows two blocks of eight waves share a compute unit
+        if (p.rows == 1) INFR_LAUNCH((moe_gate_up_stream<F, 1, 12>), grid, dim3(768), lds_s, s, p, ft);
+        else INFR_LAUNCH((moe_gate_up_stream<F, 1, 8>), grid, dim3(512), lds_s, s, p, ft);
+        return true;
+    }
     if (pipe) INFR_LAUNCH((moe_gate_up_fast<F, 3, true>), grid, block, lds, s, p, ft);
     else if (u >= 6) INFR_LAUNCH((moe_gate_up_fast<F, 6, false>), grid, block, lds, s, p, ft);
     else if (u == 5 || u == 4) INFR_LAUNCH((moe_gate_up_fast<F, 4, false>), grid, block, lds, s, p, ft);
@@ -446,6 +769,11 @@ static bool try_down(hipStream_t s, const MoeGemvParams& p) {
             const long cost = ((blocks + p.n_cu - 1) / p.n_cu) * (cand + 12);
             if (ot == 0 || cost < best) { ot = cand; best = cost; }
         }
+        if (ot >= 2 * gstep && n_slots * cells_bytes(p.nff) <= 64 * 1024) {
+            dim3 grid(ceil_div(p.ne, ot), p.rows), block(1024);
+            INFR_LAUNCH((moe_down_combine_stream<F, 1, 16>), grid, block, n_slots * cells_bytes(p.nff), s, p, ot);
+            return true;
+        }
         if (ot >= 2 * gstep) {
             const int nwaves = n_slots < 8 ? n_slots : 8;
             dim3 grid(ceil_div(p.ne, ot), p.rows), block(64 * nwaves);
@@ -458,6 +786,13 @@ static bool try_down(hipStream_t s, const MoeGemvParams& p) {
     while (steps < 8 && steps * rw < want) steps <<= 1;
     while (steps > 1 && steps * rw > kMaxOt) steps >>= 1;
     const int ot = steps * rw;
+    const size_t lds_s = n_slots * cells_bytes(p.nff);
+    if (n_slots * steps >= 16 && lds_s <= 64 * 1024) {
+        // two or more units per wave: dealt evenly to eight waves and streamed
+        dim3 grid(ceil_div(p.ne, ot), p.rows), block(1024);
+        INFR_LAUNCH((moe_down_combine_stream<F, 1, 16>), grid, block, lds_s, s, p, ot);
+        return true;
+    }
     const int nwaves = n_slots < 8 ? n_slots : 8;
     dim3 grid(ceil_div(p.ne, ot), p.rows), block(64 * nwaves);
     const size_t lds = nwaves * cells_bytes(p.nff);
@@ -510,7 +845,7 @@ __device__ __forceinline__ void stage_tokens(const float* const (&rows)[T], int 
 
 template <class F, int U, int T>
 __global__ __launch_bounds__(256) void moe_gate_up_bucketed(MoeGemvParams p, int ft) {
-    extern __shared__ uint32_t dyn_lds[];
+    extern __shared__ __attribute__((aligned(16))) uint32_t dyn_lds[];
     __shared__ uint64_t s_tab[32];
     __shared__ float s_g[4][T][64], s_u[4][T][64];
     const int e = blockIdx.y;
@@ -594,7 +929,7 @@ __global__ __launch_bounds__(256) void moe_gate_up_bucketed(MoeGemvParams p, int
 
 template <class F, int U, int T>
 __global__ __launch_bounds__(256) void moe_down_bucketed(MoeGemvParams p, int ot) {
-    extern __shared__ uint32_t dyn_lds[];
+    extern __shared__ __attribute__((aligned(16))) uint32_t dyn_lds[];
     const int e = blockIdx.y;
     const int t0 = (p.bk_offsets ? p.bk_offsets[e] : 0) + blockIdx.z * T, t1 = p.bk_offsets ? p.bk_offsets[e + 1] : p.rows;
     if (t0 >= t1) return;
@@ -712,7 +1047,7 @@ template <class F>
 __global__ __launch_bounds__(256) void linear_fast(const float* __restrict__ xin, const uint8_t* __restrict__ w,
                                                    int in_f, int out_f, float* __restrict__ dst, int ot,
                                                    const float* __restrict__ addend) {
-    extern __shared__ uint32_t dyn_lds[];
+    extern __shared__ __attribute__((aligned(16))) uint32_t dyn_lds[];
     constexpr int U = 4;  // rows a wave keeps in flight
     const int r = blockIdx.y;
     const int o0 = blockIdx.x * ot;

@@ -82,7 +82,7 @@ __device__ __forceinline__ bool gather_records(const uint64_t* rec, uint32_t tag
 // has in flight; EPB: router rows per block (n_expert / 32); NH: nff / 64.
 template <class FG, class FD, int U, int S, int EPB, int NH>
 __global__ __launch_bounds__(256) void moe_layer_fused(MoeLayerParams q) {
-    extern __shared__ uint32_t dyn_lds[];
+    extern __shared__ __attribute__((aligned(16))) uint32_t dyn_lds[];
     __shared__ uint64_t s_tab[32];
     __shared__ int32_t s_ids[64];
     __shared__ float s_w[64];

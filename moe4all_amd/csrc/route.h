@@ -7,6 +7,11 @@
 #include "device_common.h"
 #include "kernels.h"
 
+// Time stamps for a measurement build; the includer may define the macro, the library compiles it out.
+#ifndef ROUTE_STAMP
+#define ROUTE_STAMP(i) do { } while (0)
+#endif
+
 namespace infr {
 
 // ---------------------------------------------------------------------------------------------
@@ -18,10 +23,11 @@ __device__ __forceinline__ uint32_t order_key(float v) {
 }
 
 // Results go to global memory (p.ids / p.weights / p.probs) when store_global is set, and to
-// lds_ids / lds_w when those are non-null.
+// lds_ids / lds_w when those are non-null.  stage_tab (the LDS array `tab` points at, writable): the wave fills the
+// exp table itself right after it has requested its logits, so the two memory latencies overlap.
 template <int NS>
 __device__ __forceinline__ void route_row(const RouteParams& p, int row, int lane, float* lds, const uint64_t* tab,
-                                          int32_t* lds_ids, float* lds_w, bool store_global) {
+                                          int32_t* lds_ids, float* lds_w, bool store_global, uint64_t* stage_tab) {
     const int n = p.n_expert;
     float* prob = lds;
     float* sel = lds + n;
@@ -35,12 +41,17 @@ __device__ __forceinline__ void route_row(const RouteParams& p, int row, int lan
         int i = s * kWave + lane;
         pr[s] = i < n ? lg[i] : ninf;
     }
+    if (stage_tab) {
+        if (lane < 32) stage_tab[lane] = kExp2Table[lane];
+        __builtin_amdgcn_wave_barrier();
+    }
     // ---- gating (lib.rs:3746-3774)
     if (p.gating == INFR_GATING_SOFTMAX) {
         float m = ninf;
 #pragma unroll
         for (int s = 0; s < NS; s++) m = fmaxf(m, pr[s]);
         m = wave_max(m);
+        ROUTE_STAMP(1);
 #pragma unroll
         for (int s = 0; s < NS; s++) pr[s] = (s * kWave + lane < n) ? expf_libm(__fsub_rn(pr[s], m), tab) : 0.0f;
         // psum = p[0] + p[1] + ... strictly left to right (lib.rs:3752-3755).  The terms go through LDS and every
@@ -50,19 +61,34 @@ __device__ __forceinline__ void route_row(const RouteParams& p, int row, int lan
         for (int s = 0; s < NS; s++)
             if (s * kWave + lane < n) prob[s * kWave + lane] = pr[s];
         __builtin_amdgcn_wave_barrier();
+        ROUTE_STAMP(2);
         float psum = 0.0f;
         {
+            // the terms come in batches of 32 (eight 128-bit broadcast reads), the next batch requested before the
+            // current one is added, so the chain of dependent adds never waits for LDS
             int i = 0;
-#pragma unroll 2
-            for (; i + 8 <= n; i += 8) {
-                float t[8];
+            if (n >= 32 && (reinterpret_cast<uintptr_t>(prob) & 15) == 0) {
+                float4 cur[8], nxt[8];
 #pragma unroll
-                for (int k = 0; k < 8; k++) t[k] = prob[i + k];
+                for (int k = 0; k < 8; k++) cur[k] = reinterpret_cast<const float4*>(prob)[k];
+                for (; i + 32 <= n; i += 32) {
+                    const int ni = i + 64 <= n ? i + 32 : i;   // past the end: re-read, unused
 #pragma unroll
-                for (int k = 0; k < 8; k++) psum = __fadd_rn(psum, t[k]);
+                    for (int k = 0; k < 8; k++) nxt[k] = reinterpret_cast<const float4*>(prob + ni)[k];
+#pragma unroll
+                    for (int k = 0; k < 8; k++) {
+                        psum = __fadd_rn(psum, cur[k].x);
+                        psum = __fadd_rn(psum, cur[k].y);
+                        psum = __fadd_rn(psum, cur[k].z);
+                        psum = __fadd_rn(psum, cur[k].w);
+                    }
+#pragma unroll
+                    for (int k = 0; k < 8; k++) cur[k] = nxt[k];
+                }
             }
             for (; i < n; i++) psum = __fadd_rn(psum, prob[i]);
         }
+        ROUTE_STAMP(3);
         __builtin_amdgcn_wave_barrier();   // prob is rewritten with the final probabilities below
 #pragma unroll
         for (int s = 0; s < NS; s++) pr[s] = __fdiv_rn(pr[s], psum);
@@ -84,6 +110,7 @@ __device__ __forceinline__ void route_row(const RouteParams& p, int row, int lan
     }
     __builtin_amdgcn_wave_barrier();
 
+    ROUTE_STAMP(4);
     int32_t* ids_out = p.ids + (size_t)row * p.n_used;
     float* w_out = p.weights + (size_t)row * p.n_used;
     int my_id = 0;  // lane k < n_used holds the rank-k expert
@@ -166,16 +193,24 @@ __device__ __forceinline__ void route_row(const RouteParams& p, int row, int lan
             const uint32_t kmax = wave_max_u32(has ? bk : 0u);
             const bool match = has && bk == kmax;
             uint32_t win = 0xFFFFFFFFu;
+            const uint64_t holders = __ballot(match);
+            if (__builtin_popcountll(holders) == 1) {
+                // one lane holds the largest key: its candidate is the winner
+                win = (uint32_t)__builtin_amdgcn_readlane((int)bi, __builtin_ctzll(holders));
+            } else {
+                // several lanes hold it: smallest slot first, then smallest lane
 #pragma unroll
-            for (int s = 0; s < NS; s++) {
-                const uint64_t mk = __ballot(match && (int)(bi >> 6) == s);
-                if (win == 0xFFFFFFFFu && mk) win = (uint32_t)(s * kWave) + (uint32_t)__builtin_ctzll(mk);
+                for (int s = 0; s < NS; s++) {
+                    const uint64_t mk = __ballot(match && (int)(bi >> 6) == s);
+                    if (win == 0xFFFFFFFFu && mk) win = (uint32_t)(s * kWave) + (uint32_t)__builtin_ctzll(mk);
+                }
             }
             if (win == 0xFFFFFFFFu) win = 0;
             if ((int)(win & 63u) == lane) taken |= 1u << (win >> 6);
             if (lane == k) my_id = (int)win;
         }
     }
+    ROUTE_STAMP(5);
     // ---- routing weights (lib.rs:3856-3861): lane k owns rank k
     const bool mine = lane < p.n_used;
     float pk = mine ? prob[my_id] : 0.0f;
@@ -202,6 +237,7 @@ __device__ __forceinline__ void route_row(const RouteParams& p, int row, int lan
         if (lds_ids) lds_ids[lane] = my_id;
         if (lds_w) lds_w[lane] = w;
     }
+    ROUTE_STAMP(6);
     if (p.probs && store_global) {
 #pragma unroll
         for (int s = 0; s < NS; s++) {
@@ -213,12 +249,167 @@ __device__ __forceinline__ void route_row(const RouteParams& p, int row, int lan
 
 __device__ __forceinline__ void route_row_any(const RouteParams& p, int row, int lane, float* lds, const uint64_t* tab,
                                               int32_t* lds_ids = nullptr, float* lds_w = nullptr,
-                                              bool store_global = true) {
+                                              bool store_global = true, uint64_t* stage_tab = nullptr) {
     const int n = p.n_expert;
-    if (n <= 128) route_row<2>(p, row, lane, lds, tab, lds_ids, lds_w, store_global);
-    else if (n <= 256) route_row<4>(p, row, lane, lds, tab, lds_ids, lds_w, store_global);
-    else if (n <= 512) route_row<8>(p, row, lane, lds, tab, lds_ids, lds_w, store_global);
-    else route_row<32>(p, row, lane, lds, tab, lds_ids, lds_w, store_global);
+    if (n <= 128) route_row<2>(p, row, lane, lds, tab, lds_ids, lds_w, store_global, stage_tab);
+    else if (n <= 256) route_row<4>(p, row, lane, lds, tab, lds_ids, lds_w, store_global, stage_tab);
+    else if (n <= 512) route_row<8>(p, row, lane, lds, tab, lds_ids, lds_w, store_global, stage_tab);
+    else route_row<32>(p, row, lane, lds, tab, lds_ids, lds_w, store_global, stage_tab);
+}
+
+// ---------------------------------------------------------------------------------------------
+// Plain softmax routing of one token row on two wavefronts of a block.  The serial parts of the routing are the
+// left-to-right sum of the exponentials and the selection rounds; wave 0 runs the sum while wave 1 selects the
+// n_used + 1 largest exponentials, (value descending, id ascending).  A probability is fl(exp / sum), a non-decreasing
+// function of the exponential, so when the candidates' probabilities are strictly decreasing the first n_used are the
+// reference's selection in its order (crates/infr-cpu/src/lib.rs:3847-3850); when two of them collide after the
+// division (exponentials an ulp apart) or anything is not a number, wave 0 runs the complete routine instead.
+// Calling sequence, the same for every thread of the block: route_duo_first on waves 0 and 1, __syncthreads(),
+// route_duo_second on wave 0, __syncthreads().
+struct RouteDuo {
+    float psum;
+    int32_t cand[16];
+    float cand_e[16];
+};
+__host__ __device__ inline bool route_duo_ok(const RouteParams& p) {
+    return p.gating == INFR_GATING_SOFTMAX && !p.exp_probs_b && !p.expert_ids && !(p.n_groups > 1 && p.n_groups_used > 0) &&
+           p.n_used <= 15 && p.n_expert <= 512 && p.n_expert > p.n_used;
+}
+template <int NS>
+__device__ __forceinline__ void route_duo_first(const RouteParams& p, int row, int wave, int lane, float* lds,
+                                                uint64_t* tab, RouteDuo* duo, float (&pr)[NS]) {
+    const int n = p.n_expert;
+    const float* lg = p.logits + (size_t)row * n;
+    const float ninf = -__builtin_huge_valf();
+#pragma unroll
+    for (int s = 0; s < NS; s++) {
+        const int i = s * kWave + lane;
+        pr[s] = i < n ? lg[i] : ninf;
+    }
+    if (lane < 32) tab[lane] = kExp2Table[lane];   // both waves write the same values
+    __builtin_amdgcn_wave_barrier();
+    float m = ninf;
+#pragma unroll
+    for (int s = 0; s < NS; s++) m = fmaxf(m, pr[s]);
+    m = wave_max(m);
+    ROUTE_STAMP(1);
+#pragma unroll
+    for (int s = 0; s < NS; s++) pr[s] = (s * kWave + lane < n) ? expf_libm(__fsub_rn(pr[s], m), tab) : 0.0f;
+    if (wave == 0) {
+        float* ex = lds;
+#pragma unroll
+        for (int s = 0; s < NS; s++)
+            if (s * kWave + lane < n) ex[s * kWave + lane] = pr[s];
+        __builtin_amdgcn_wave_barrier();
+        ROUTE_STAMP(2);
+        float psum = 0.0f;
+        int i = 0;
+        if (n >= 32 && (reinterpret_cast<uintptr_t>(ex) & 15) == 0) {
+            float4 cur[8], nxt[8];
+#pragma unroll
+            for (int k = 0; k < 8; k++) cur[k] = reinterpret_cast<const float4*>(ex)[k];
+            for (; i + 32 <= n; i += 32) {
+                const int ni = i + 64 <= n ? i + 32 : i;   // past the end: re-read, unused
+#pragma unroll
+                for (int k = 0; k < 8; k++) nxt[k] = reinterpret_cast<const float4*>(ex + ni)[k];
+#pragma unroll
+                for (int k = 0; k < 8; k++) {
+                    psum = __fadd_rn(psum, cur[k].x);
+                    psum = __fadd_rn(psum, cur[k].y);
+                    psum = __fadd_rn(psum, cur[k].z);
+                    psum = __fadd_rn(psum, cur[k].w);
+                }
+#pragma unroll
+                for (int k = 0; k < 8; k++) cur[k] = nxt[k];
+            }
+        }
+        for (; i < n; i++) psum = __fadd_rn(psum, ex[i]);
+        if (lane == 0) duo->psum = psum;
+        ROUTE_STAMP(3);
+    } else {
+        uint32_t keys[NS], taken = 0;
+#pragma unroll
+        for (int s = 0; s < NS; s++) {
+            keys[s] = order_key(pr[s]);
+            if (s * kWave + lane >= n) taken |= 1u << s;
+        }
+        for (int k = 0; k <= p.n_used; k++) {
+            uint32_t bk = 0, bi = 0xFFFFFFFFu;
+            float be = 0.0f;
+#pragma unroll
+            for (int s = 0; s < NS; s++) {
+                if (taken & (1u << s)) continue;
+                if (bi == 0xFFFFFFFFu || keys[s] > bk) { bk = keys[s]; bi = (uint32_t)(s * kWave + lane); be = pr[s]; }
+            }
+            const bool has = bi != 0xFFFFFFFFu;
+            const uint32_t kmax = wave_max_u32(has ? bk : 0u);
+            const bool match = has && bk == kmax;
+            uint32_t win = 0xFFFFFFFFu;
+            const uint64_t holders = __ballot(match);
+            if (__builtin_popcountll(holders) == 1) {
+                win = (uint32_t)__builtin_amdgcn_readlane((int)bi, __builtin_ctzll(holders));
+            } else {
+#pragma unroll
+                for (int s = 0; s < NS; s++) {
+                    const uint64_t mk = __ballot(match && (int)(bi >> 6) == s);
+                    if (win == 0xFFFFFFFFu && mk) win = (uint32_t)(s * kWave) + (uint32_t)__builtin_ctzll(mk);
+                }
+            }
+            if (win == 0xFFFFFFFFu) win = 0;
+            if ((int)(win & 63u) == lane && match && bi == win) {   // this lane's best is the winner
+                taken |= 1u << (win >> 6);
+                duo->cand[k] = (int32_t)win;
+                duo->cand_e[k] = be;
+            }
+        }
+    }
+}
+// Wave 0 after the block barrier.  False: the candidates collide (or something is not a number) and the caller runs
+// route_row_any.
+template <int NS>
+__device__ __forceinline__ bool route_duo_second(const RouteParams& p, int row, int lane, const RouteDuo* duo,
+                                                 const float (&pr)[NS], int32_t* lds_ids, float* lds_w, bool store_global) {
+    const int n = p.n_expert;
+    const float psum = duo->psum;
+    const float pc = lane <= p.n_used ? __fdiv_rn(duo->cand_e[lane], psum) : 0.0f;
+    const float nxt = __shfl_down(pc, 1, kWave);
+    if (!__all(lane >= p.n_used || pc > nxt)) return false;
+    ROUTE_STAMP(5);
+    // routing weights (lib.rs:3856-3861): lane k owns rank k
+    const bool mine = lane < p.n_used;
+    int my_id = mine ? duo->cand[lane] : 0;
+    const float pk = mine ? pc : 0.0f;
+    float w;
+    if (p.norm_w) {
+        float wsum = 0.0f;
+        for (int k = 0; k < p.n_used; k++) wsum = __fadd_rn(wsum, readlane_f(pk, k));
+        wsum = fmaxf(wsum, 1e-20f);
+        w = __fmul_rn(__fdiv_rn(pk, wsum), p.scale);
+    } else {
+        w = __fmul_rn(pk, p.scale);
+    }
+    if (p.ep_n > 0) {
+        const bool own = my_id >= p.ep_lo && my_id < p.ep_lo + p.ep_n;
+        my_id = own ? my_id - p.ep_lo : 0;
+        w = own ? w : 0.0f;
+    }
+    if (mine) {
+        if (store_global) {
+            p.ids[(size_t)row * p.n_used + lane] = my_id;
+            p.weights[(size_t)row * p.n_used + lane] = w;
+        }
+        if (lds_ids) lds_ids[lane] = my_id;
+        if (lds_w) lds_w[lane] = w;
+    }
+    ROUTE_STAMP(6);
+    if (p.probs && store_global) {
+#pragma unroll
+        for (int s = 0; s < NS; s++) {
+            const int i = s * kWave + lane;
+            if (i < n) p.probs[(size_t)row * n + i] = __fdiv_rn(pr[s], psum);
+        }
+    }
+    return true;
 }
 
 // LDS floats route_row_any needs behind the 64-float exp table.

@@ -549,14 +549,18 @@ def test_fused_dense_ffn_launches_give_the_bits_of_the_separate_ops(be, rows, ac
 
 
 @pytest.mark.parametrize("rows,K,opts", [(1, 4, {}), (1, 8, {"weight_before": True}), (1, 6, {"with_down_scale": True}),
-                                         (3, 8, {})])
+                                         (3, 8, {}),
+                                         # tiles of several weight rows per wavefront: the streamed decode kernels
+                                         (1, 4, {"with_dims": (2048, 2048)}),
+                                         (1, 8, {"weight_before": True, "with_dims": (2048, 2048)}),
+                                         (1, 6, {"with_down_scale": True, "with_dims": (2048, 1536)})])
 def test_shared_expert_as_an_extra_slot_gives_the_bits_of_the_separate_ops(be, rows, K, opts):
     """MoeFfn followed by an ungated shared expert (Linear, Linear, GatedAct, Linear, Add —
     crates/infr-llama/src/seam/runner.rs:8116-8174) runs as one more slot of the two routed decode
     kernels when the routed sum is a single-use Internal tensor and there is one token row.
     Declaring that tensor an Output keeps MoeFfn and the dense FFN apart; both must give identical
     bits.  With several rows the ops stay apart either way."""
-    ne, nff, E = 1024, 512, 16
+    (ne, nff), E = opts.get("with_dims", (1024, 512)), 16
     rng = np.random.default_rng(100 + rows)
     x = rng.standard_normal((rows, ne)).astype(np.float32)
     router = (rng.standard_normal((E, ne)) * 0.1).astype(np.float32)
