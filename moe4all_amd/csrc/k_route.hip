@@ -13,6 +13,21 @@
 #include "kernels.h"
 #include "route.h"
 
+// Time stamps of every block for a measurement build; compiled out in the library.
+#ifdef INFR_GEMV_TRACE
+namespace infr { __device__ long long* g_logits_trace; }
+#define LOGITS_STAMP(i)                                                                                                \
+    do {                                                                                                               \
+        if (threadIdx.x == 0 && infr::g_logits_trace) {                                                                \
+            long long* rec_ = infr::g_logits_trace + ((size_t)blockIdx.y * gridDim.x + blockIdx.x) * 16;               \
+            rec_[i] = wall_clock64();                                                                                  \
+            rec_[8 + (i)] = clock64();   /* the shader clock beside the 100 MHz wall clock */                          \
+        }                                                                                                              \
+    } while (0)
+#else
+#define LOGITS_STAMP(i) do { } while (0)
+#endif
+
 namespace infr {
 
 // One wavefront per token row (n_used <= 64, n_expert <= 2048).
@@ -59,6 +74,7 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const uint8_t* __res
     // Decode-sized launch (one pass over <= 2 token rows, f32 router): every global load of the
     // block, activations included, is issued before the first LDS store, so the block pays the
     // memory latency once.
+    LOGITS_STAMP(0);
     const int nv = ne >> 2;
     const int rbase = blockIdx.y * rpb;   // first token row of this block's (only) pass when one_shot
     const bool one_shot = rdt == INFR_F32 && (ne & 3) == 0 && (int)gridDim.y * rpb >= rows && EPB * nv <= 8 * 256 &&
@@ -93,7 +109,9 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const uint8_t* __res
 #pragma unroll
             for (int i = 0; i < 4; i++)
                 if (tid + 256 * i < nv) part = sumsq4(part, xr[i]);
+            LOGITS_STAMP(1);
             const float sc = rms_scale(block256_sum(part, red), ne, nrm.eps);
+            LOGITS_STAMP(2);
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 const int idx = tid + 256 * i;
@@ -149,6 +167,7 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const uint8_t* __res
             else wt[e * 8 + j] = v;
         }
     }
+    LOGITS_STAMP(3);
     const int rsub = tid / (EPB * 8);
     const int e = (tid >> 3) % EPB;
     const int j = tid & 7;
@@ -166,6 +185,7 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const uint8_t* __res
             }
         }
         __syncthreads();
+        LOGITS_STAMP(4);
         float acc = 0.0f;
         const bool live = rsub < rpb;
         const float* wp = w + e * estride + j * jstride;
@@ -183,6 +203,7 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const uint8_t* __res
             }
             for (; c < nc; c++) acc = __fmaf_rn(wp[c], xp[c], acc);
         }
+        LOGITS_STAMP(5);
         float s = 0.0f;
 #pragma unroll
         for (int jj = 0; jj < 8; jj++) s = __fadd_rn(s, __shfl(acc, (lane & ~7) + jj, kWave));
@@ -190,6 +211,7 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const uint8_t* __res
             for (int t = 0; t < ntail; t++) s = __fmaf_rn(wt[e * 8 + t], xt[rsub * 8 + t], s);
             if (r0 + rsub < rows && e0 + e < n_expert) logits[(size_t)(r0 + rsub) * n_expert + e0 + e] = s;
         }
+        LOGITS_STAMP(6);
     }
 }
 
@@ -345,6 +367,8 @@ bool launch_router_logits(hipStream_t s, const uint8_t* router, int rdt, size_t 
     }
     int epb = 0, rpb = 0;
     if (!router_logits_tile(rdt, ne, rows, &epb, &rpb)) return false;
+    // one token row and no more experts than compute units: a block per expert halves what a block stages
+    if (rows == 1 && epb == 2 && n_expert <= 256) epb = 1;
     const bool small = rows <= 2 || (rows < 32 && rdt == INFR_F32 && (ne & 3) == 0 && ne <= 4096);
     const size_t budget = kRouterLdsBudget;
     const int nc = ne >> 3;

@@ -4,6 +4,7 @@
 // make -C moe4all_amd/csrc probes; ./moe4all_amd/csrc/probe/gemv_phases [c5|c2|c1] [rows]
 #define INFR_GEMV_TRACE 1
 #include "../k_gemv.hip"
+#include "../k_route.hip"
 #include <algorithm>
 #include <cstdio>
 #include <cstdlib>
@@ -18,7 +19,6 @@ bool linear_float_supported(int, int, size_t, const void*, const void*) { return
 void launch_linear_float(hipStream_t, const float*, const uint8_t*, int, size_t, int, int, int, float*, const float*) {}
 bool moe_gate_up_units_supported(const MoeGemvParams&) { return false; }
 void launch_moe_gate_up_units(hipStream_t, const MoeGemvParams&) {}
-void launch_route(hipStream_t, const RouteParams&) {}
 }
 #define CK(x) do{hipError_t e_=(x); if(e_!=hipSuccess){printf("ERR %s: %s\n",#x,hipGetErrorString(e_)); exit(1);} }while(0)
 
@@ -83,6 +83,27 @@ int main(int argc, char** argv) {
          p.route_inline ? "inside the gate/up kernel" : "as a launch of its own");
   if (!p.route_inline) infr::launch_route(s, p.route);
   hipEvent_t a, b; CK(hipEventCreate(&a)); CK(hipEventCreate(&b));
+  {   // the logits kernel on a router of its own (f32 [E, ne]), the token row normalised on the way as in the layer
+    float *router, *nw, *xn; CK(hipMalloc(&router, (size_t)E * ne * 4)); CK(hipMalloc(&nw, ne * 4)); CK(hipMalloc(&xn, (size_t)rows * ne * 4));
+    { std::vector<float> v((size_t)E * ne); unsigned r = 7; for (auto& q : v) { r = r * 1664525u + 1013904223u; q = ((r >> 8) / 16777216.0f - 0.5f) * 0.05f; }
+      CK(hipMemcpy(router, v.data(), v.size() * 4, hipMemcpyHostToDevice)); std::vector<float> o(ne, 1.0f); CK(hipMemcpy(nw, o.data(), ne * 4, hipMemcpyHostToDevice)); }
+    infr::RouterNorm nrm{}; if (rows == 1) { nrm.weight = nw; nrm.xn_out = xn; nrm.eps = 1e-6f; }
+    float* lg; CK(hipMalloc(&lg, (size_t)rows * E * 4));
+    auto launch = [&]() { infr::launch_router_logits(s, reinterpret_cast<const uint8_t*>(router), INFR_F32, (size_t)ne * 4, x, ne, E, rows, lg, rows == 1 ? &nrm : nullptr); };
+    for (int i = 0; i < 5; i++) launch();
+    CK(hipStreamSynchronize(s));
+    CK(hipEventRecord(a, s)); for (int i = 0; i < 50; i++) launch(); CK(hipEventRecord(b, s)); CK(hipStreamSynchronize(s));
+    float ms; CK(hipEventElapsedTime(&ms, a, b));
+    printf("router logits: %.2f us per launch without time stamps (the same router every launch: it stays in the caches)\n", ms * 1000 / 50);
+    CK(hipMemcpyToSymbol(HIP_SYMBOL(infr::g_logits_trace), &trace, sizeof(trace)));
+    CK(hipMemsetAsync(trace, 0, (size_t)max_blocks * 128, s)); launch(); CK(hipStreamSynchronize(s));
+    std::vector<long long> t((size_t)max_blocks * 16); CK(hipMemcpy(t.data(), trace, t.size() * 8, hipMemcpyDeviceToHost));
+    int blocks = 0; for (int i = 0; i < max_blocks; i++) if (t[i * 16]) blocks = i + 1;
+    report("router logits", t, blocks, {0, 1, 2, 3, 4, 5, 6}, "0 start | 1 operands here, squares summed per thread | 2 norm scale known | 3 operands in LDS | 4 after the barrier | 5 chains done | 6 logits stored");
+    { std::vector<double> f; for (int bk = 0; bk < blocks; bk++) if (t[bk * 16 + 6] > t[bk * 16]) f.push_back((double)(t[bk * 16 + 14] - t[bk * 16 + 8]) / (double)(t[bk * 16 + 6] - t[bk * 16]) * 0.1);
+      std::sort(f.begin(), f.end()); if (!f.empty()) printf("  shader clock over the kernel (clock64 ticks per wall-clock tick): median %.2f GHz\n", f[f.size() / 2]); }
+    long long* none = nullptr; CK(hipMemcpyToSymbol(HIP_SYMBOL(infr::g_logits_trace), &none, sizeof(none)));
+  }
   float gu_ms = 0;
   for (int which = 0; which < 2; which++) {
     int turn = 0;

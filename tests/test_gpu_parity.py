@@ -1379,7 +1379,8 @@ def test_batched_threshold_is_configurable_and_the_paths_agree():
     assert H.rel_l2(outs["mfma"], outs["gemv"]) < REL_L2_MFMA
 
 
-def test_routing_of_logits_a_few_dozen_ulp_apart_is_the_stable_sort_of_the_probabilities(be):
+@pytest.mark.parametrize("three_launch,tie", [(False, False), (True, False), (True, True)])
+def test_routing_of_logits_a_few_dozen_ulp_apart_is_the_stable_sort_of_the_probabilities(be, three_launch, tie):
     """Logits 40 ulp apart: inside the selection the higher logit ranks first although its id is higher, and at the
     selection's edge it decides which expert is in.  A selection on truncated or rounded keys would get both wrong;
     the contract is the reference's stable descending sort of the probabilities (crates/infr-cpu/src/lib.rs:3847-3850)."""
@@ -1398,13 +1399,23 @@ def test_routing_of_logits_a_few_dozen_ulp_apart_is_the_stable_sort_of_the_proba
     col[9] = up_ulps(2.75, 40)          # 9 before 5
     col[20] = 1.25
     col[30] = up_ulps(1.25, 40)         # 30 is rank 8 and 20 is out
+    want = [3, 9, 5, 17, 40, 41, 60, 30]
+    if tie:                             # two equal logits at the selection's edge: the smaller id is in, the other out
+        col[60] = col[70] = 1.25
+        want = [3, 9, 5, 17, 40, 41, 30, 20]
     router[:, 0] = col
+    if three_launch:                    # routing inside the gate/up kernel (sum and selection on two wavefronts)
+        be = M.Backend(0, disable_single_launch_moe=True)
     gate, up = _realistic(rng, E, nff, ne, H.Q4K), _realistic(rng, E, nff, ne, H.Q4K)
     down = _realistic(rng, E, ne, nff, H.Q6K)
     g, ids = moe_graph(1, ne, E, K, nff, DType.Q4K, DType.Q6K)
-    out, r = run_moe(be, g, ids, dict(x=x, router=router, gate=gate, up=up, down=down), 1, ne)
+    try:
+        out, r = run_moe(be, g, ids, dict(x=x, router=router, gate=gate, up=up, down=down), 1, ne)
+    finally:
+        if three_launch:
+            be.close()
     ref = O.moe_ffn(x, router, gate, up, down, ne=ne, n_expert=E, n_used=K, n_ff_exp=nff, gate_dtype=H.Q4K, down_dtype=H.Q6K)
-    assert ref["idx"][0].tolist() == [3, 9, 5, 17, 40, 41, 60, 30]
+    assert ref["idx"][0].tolist() == want
     assert np.array_equal(r["idx"], ref["idx"]) and np.array_equal(bits(r["w"]), bits(ref["w"]))
     assert H.rel_l2(out, ref["dst"]) < REL_L2 and H.max_abs(out, ref["dst"]) < MAX_ABS
 
