@@ -110,11 +110,9 @@ __device__ __forceinline__ void gu_finish(const GuStage<F, U>& st, const MoeGemv
     __builtin_amdgcn_wave_barrier();
 }
 
-// PIPE == false: every stage is loaded, then finished (one stage is the common decode case and
-// then all of the block's loads are in flight at once).  PIPE == true, for tiles of three or more
-// stages: two stage buffers, the next stage's loads are issued before the current stage is
-// finished, so a wave always has a stage in flight while it computes.
-template <class F, int U, bool PIPE>
+// Tiles of at most two items per wave (larger tiles go to moe_gate_up_stream): every load of the block is in flight at
+// once, then the items are finished.
+template <class F, int U>
 __global__ __launch_bounds__(256) void moe_gate_up_fast(MoeGemvParams p, int ft) {
     extern __shared__ __attribute__((aligned(16))) uint32_t dyn_lds[];
     __shared__ uint64_t s_tab[32];
@@ -159,52 +157,20 @@ __global__ __launch_bounds__(256) void moe_gate_up_fast(MoeGemvParams p, int ft)
     t.nitems = t.fcount * t.n_slots;
     const int step = 4 * pl.rw_count * U;
     typename F::X x;
-    if (!PIPE) {
-        bool have_x = false;
-        for (int base = 0; base < t.nitems; base += step) {
-            GuStage<F, U> st;
-            gu_issue<F, U>(st, p, pl, t, s_ids, base);
-            if (!have_x) {
-                // while the weights are in flight: the wave converts x to fixed point once, together
-                stage_x_finish<F::kGroup, F::kSigned>(xl, xrow, p.ne, cells, lane);
-                __builtin_amdgcn_wave_barrier();
-                F::fetch_x(x, cells, pl.blk, pl.sub);
-                have_x = true;
-                GEMV_STAMP(2);
-            }
-            gu_finish<F, U>(st, p, pl, t, x, nblk, base, s_g, s_u, s_w, s_tab);
-            if (base == 0) GEMV_STAMP(3);
+    bool have_x = false;
+    for (int base = 0; base < t.nitems; base += step) {
+        GuStage<F, U> st;
+        gu_issue<F, U>(st, p, pl, t, s_ids, base);
+        if (!have_x) {
+            // while the weights are in flight: the wave converts x to fixed point once, together
+            stage_x_finish<F::kGroup, F::kSigned>(xl, xrow, p.ne, cells, lane);
+            __builtin_amdgcn_wave_barrier();
+            F::fetch_x(x, cells, pl.blk, pl.sub);
+            have_x = true;
+            GEMV_STAMP(2);
         }
-    } else {
-        GuStage<F, U> sa, sb;
-        gu_issue<F, U>(sa, p, pl, t, s_ids, 0);
-        GEMV_STAMP(5);
-        gu_issue<F, U>(sb, p, pl, t, s_ids, step);
-        GEMV_STAMP(6);
-        stage_x_finish<F::kGroup, F::kSigned>(xl, xrow, p.ne, cells, lane);
-        __builtin_amdgcn_wave_barrier();
-        GEMV_STAMP(7);
-        F::fetch_x(x, cells, pl.blk, pl.sub);
-        GEMV_STAMP(2);
-        gu_finish<F, U>(sa, p, pl, t, x, nblk, 0, s_g, s_u, s_w, s_tab);
-        GEMV_STAMP(3);
-        int base = step;   // the stage sb holds
-        for (;;) {
-            if (base + step >= t.nitems) {
-                gu_finish<F, U>(sb, p, pl, t, x, nblk, base, s_g, s_u, s_w, s_tab);
-                break;
-            }
-            gu_issue<F, U>(sa, p, pl, t, s_ids, base + step);
-            gu_finish<F, U>(sb, p, pl, t, x, nblk, base, s_g, s_u, s_w, s_tab);
-            base += step;
-            if (base + step >= t.nitems) {
-                gu_finish<F, U>(sa, p, pl, t, x, nblk, base, s_g, s_u, s_w, s_tab);
-                break;
-            }
-            gu_issue<F, U>(sb, p, pl, t, s_ids, base + step);
-            gu_finish<F, U>(sa, p, pl, t, x, nblk, base, s_g, s_u, s_w, s_tab);
-            base += step;
-        }
+        gu_finish<F, U>(st, p, pl, t, x, nblk, base, s_g, s_u, s_w, s_tab);
+        if (base == 0) GEMV_STAMP(3);
     }
     GEMV_STAMP(4);
 }
@@ -489,7 +455,7 @@ __global__ __launch_bounds__(512) void moe_down_combine_fast(MoeGemvParams p, in
 
 // ------------------------------------------------------------------------------- down, streamed
 // The same tiles as moe_down_combine_fast with the work cut differently: a tile's units (slot, group of rows a wave
-// covers at once) are dealt to the block's 8 waves in equal contiguous runs, so nine slots keep eight waves equally
+// covers at once) are dealt to the block's NW waves in equal contiguous runs, so nine slots keep every wave equally
 // busy, and a wave keeps D units in flight as a ring (finish the oldest, request the unit D places ahead into the
 // registers that became free).  h of every slot is turned into fixed-point cells once, by the whole block; a wave
 // fetches a slot's cells when its run crosses into that slot.
@@ -697,12 +663,7 @@ static bool try_gate_up(hipStream_t s, const MoeGemvParams& p) {
     int ft = p.rows >= 2 ? ceil_div(p.nff * p.rows, 2 * p.n_cu) : ceil_div(p.nff, p.n_cu);
     if (ft < 1) ft = 1;
     const int per_wave = ceil_div(ft * n_slots, 4 * rw);
-    // tiles of three or more stages stream with the next stage in flight
-    const bool pipe = per_wave > 6 && 3 * rw <= 64;
     dim3 grid(ceil_div(p.nff, ft), p.rows), block(256);
-    // U * rw results per wave must fit the 64-entry staging rows
-    int u = per_wave < 1 ? 1 : per_wave;
-    while (u * rw > 64) u--;
     const size_t lds = 4 * cells_bytes(p.ne) +
                        (p.route_inline ? route_scratch_floats(p.route.n_expert, p.route.n_groups) * sizeof(float) : 0);
     if (per_wave >= 3) {
@@ -715,12 +676,9 @@ static bool try_gate_up(hipStream_t s, const MoeGemvParams& p) {
         else INFR_LAUNCH((moe_gate_up_stream<F, 1, 8>), grid, dim3(512), lds_s, s, p, ft);
         return true;
     }
-    if (pipe) INFR_LAUNCH((moe_gate_up_fast<F, 3, true>), grid, block, lds, s, p, ft);
-    else if (u >= 6) INFR_LAUNCH((moe_gate_up_fast<F, 6, false>), grid, block, lds, s, p, ft);
-    else if (u == 5 || u == 4) INFR_LAUNCH((moe_gate_up_fast<F, 4, false>), grid, block, lds, s, p, ft);
-    else if (u == 3) INFR_LAUNCH((moe_gate_up_fast<F, 3, false>), grid, block, lds, s, p, ft);
-    else if (u == 2) INFR_LAUNCH((moe_gate_up_fast<F, 2, false>), grid, block, lds, s, p, ft);
-    else INFR_LAUNCH((moe_gate_up_fast<F, 1, false>), grid, block, lds, s, p, ft);
+    if (per_wave == 2 && 2 * rw <= 64)   // U * rw results per wave must fit the 64-entry staging rows
+        INFR_LAUNCH((moe_gate_up_fast<F, 2>), grid, block, lds, s, p, ft);
+    else INFR_LAUNCH((moe_gate_up_fast<F, 1>), grid, block, lds, s, p, ft);
     return true;
 }
 
@@ -788,7 +746,7 @@ static bool try_down(hipStream_t s, const MoeGemvParams& p) {
     const int ot = steps * rw;
     const size_t lds_s = n_slots * cells_bytes(p.nff);
     if (n_slots * steps >= 16 && lds_s <= 64 * 1024) {
-        // two or more units per wave: dealt evenly to eight waves and streamed
+        // two or more units per slot-wave: dealt evenly to sixteen waves and streamed
         dim3 grid(ceil_div(p.ne, ot), p.rows), block(1024);
         INFR_LAUNCH((moe_down_combine_stream<F, 1, 16>), grid, block, lds_s, s, p, ot);
         return true;

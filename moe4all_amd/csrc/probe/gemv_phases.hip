@@ -1,6 +1,8 @@
-// Measurement aid for the decode kernels of k_gemv.hip (routing + gate/up, down + weighted sum): builds them with their
-// time stamps switched on, runs one token row (or a few) of a layer shape on random banks and prints, per phase boundary,
-// the minimum / median / maximum over the workgroups of the time since the first workgroup started.
+// Measurement aid for the three launches of the per-token MoeFfn path (router logits of k_route.hip; routing + gate/up
+// and down + weighted sum of k_gemv.hip): builds them with their time stamps switched on, runs one token row (or a few)
+// of a layer shape on random banks and prints, per phase boundary, the minimum / median / maximum over the workgroups of
+// the time since the first workgroup started.  The expert kernels cycle through eight sets of logits that select
+// disjoint experts, so their weights come from HBM as they do in a model with many layers.
 // make -C moe4all_amd/csrc probes; ./moe4all_amd/csrc/probe/gemv_phases [c5|c2|c1] [rows]
 #define INFR_GEMV_TRACE 1
 #include "../k_gemv.hip"
@@ -127,8 +129,8 @@ int main(int argc, char** argv) {
     CK(hipMemsetAsync(trace, 0, (size_t)max_blocks * 128, s)); launch(); CK(hipStreamSynchronize(s));
     std::vector<long long> t((size_t)max_blocks * 16); CK(hipMemcpy(t.data(), trace, t.size() * 8, hipMemcpyDeviceToHost));
     int blocks = 0; for (int i = 0; i < max_blocks; i++) if (t[i * 16]) blocks = i + 1;
-    if (which) report("down + sum", t, blocks, {0, 1, 2, 3, 4, 5, 6, 8, 9, 10, 11, 12, 13, 14, 15}, "0 start | 1 weight rows requested | 2 h as cells | 3 rows done | 4 before the block barrier | 5 after it | 6 sums stored | 8..15: waves 0..7 done with their rows");
-    else report("routing + gate/up", t, blocks, {0, 9, 10, 11, 12, 13, 14, 1, 5, 6, 7, 2, 3, 4}, "0 start | 9 logits here, largest known | 10 exps in LDS | 11 sum | 12 probabilities | 13 top-k | 14 weights | 1 routed | 5 first stage requested | 6 second stage requested | 7 x as cells | 2 x in registers | 3 first stage done | 4 end");
+    if (which) report("down + sum", t, blocks, {0, 1, 2, 4, 5, 6, 8, 9, 10, 11, 12, 13, 14, 15}, "0 start | 1 ids here, first units requested | 2 h of every slot as cells (block barrier) | 4 wave 0 done with its units | 5 after the block barrier | 6 sums stored | 8..15: a wave of each residue class mod 8 done with its units");
+    else report("routing + gate/up", t, blocks, {0, 9, 10, 11, 13, 14, 1, 2, 3, 4}, "0 start | 9 logits here, largest known | 10 exponentials in LDS | 11 their sum (wave 0; wave 1 selects meanwhile) | 13 candidates checked | 14 weights | 1 routed, x as cells (block barrier) | 2 x in registers, first items requested | 3 first round of the ring done | 4 end");
   }
   return 0;
 }
