@@ -828,45 +828,66 @@ __global__ __launch_bounds__(256) void moe_gate_up_bucketed(MoeGemvParams p, int
     }
     const uint8_t* gbank = p.gate + (size_t)e * p.gate_stride + (size_t)f0 * row_bytes;
     const uint8_t* ubank = p.up + (size_t)e * p.up_stride + (size_t)f0 * row_bytes;
-    const int per_round = 4 * pl.rw_count;
-    // the first round of weight rows is requested before the activations are staged
+    const int per_round = 4 * pl.rw_count;   // features the block's four waves take per round
+    const int n_rounds = (fcount + per_round - 1) / per_round;
+    // A wave keeps U rounds (a gate row and an up row per row lane group) in flight as a ring: it finishes the oldest
+    // round against its T tokens and requests the round U places ahead into the registers that became free, so loads
+    // and dots alternate round by round.  The first rounds are requested before the activations are staged.
     typename F::Raw graw[U], uraw[U];
-#pragma unroll
-    for (int u = 0; u < U; u++) {
-        const int f = min((u * 4 + wave) * pl.rw_count + pl.rw, fcount - 1);
+    auto issue = [&](int u, int k) {
+        const int f = min((k * 4 + wave) * pl.rw_count + pl.rw, fcount - 1);
         graw[u] = load_row<F>(pl, gbank + (size_t)f * row_bytes);
         uraw[u] = load_row<F>(pl, ubank + (size_t)f * row_bytes);
-    }
+    };
+#pragma unroll
+    for (int u = 0; u < U; u++)
+        if (u < n_rounds) issue(u, u);
     stage_tokens<F, T>(xrows, nt, p.ne, dyn_lds, cell_words);
     typename F::X x[T];
 #pragma unroll
     for (int tau = 0; tau < T; tau++) F::fetch_x(x[tau], dyn_lds + (size_t)min(tau, nt - 1) * cell_words, pl.blk, pl.sub);
-    for (int base = 0; base < fcount; base += per_round * U) {
-#pragma unroll
-        for (int u = 0; u < U; u++) {
+    const int chunk = 64 / pl.rw_count;   // rounds whose results fit a wave's staging row; the ring restarts per chunk
+    for (int c0 = 0; c0 < n_rounds; c0 += chunk) {
+        const int cn = min(chunk, n_rounds - c0);
+        auto finish = [&](int u, int j) {
 #pragma unroll
             for (int tau = 0; tau < T; tau++) {
-                float gs = row_sum<F>(F::dot(graw[u], pl.sub, x[tau]), pl, nblk);
-                float us = row_sum<F>(F::dot(uraw[u], pl.sub, x[tau]), pl, nblk);
+                if (tau >= nt) break;   // a short chunk of the bucket: no dots for tokens it does not have
+                const float gs = row_sum<F>(F::dot(graw[u], pl.sub, x[tau]), pl, nblk);
+                const float us = row_sum<F>(F::dot(uraw[u], pl.sub, x[tau]), pl, nblk);
                 if (pl.writer()) {
-                    s_g[wave][tau][u * pl.rw_count + pl.rw] = gs;
-                    s_u[wave][tau][u * pl.rw_count + pl.rw] = us;
+                    s_g[wave][tau][j * pl.rw_count + pl.rw] = gs;
+                    s_u[wave][tau][j * pl.rw_count + pl.rw] = us;
                 }
             }
+        };
+        if (c0 > 0) {
+#pragma unroll
+            for (int u = 0; u < U; u++)
+                if (u < cn) issue(u, c0 + u);
         }
-        // next round's rows are in flight while this round's activations are applied
-        if (base + per_round * U < fcount) {
+        // steady state: no branch between a round's dots and its refill, so the waits count exactly the younger loads
+        const int refills = cn - U;   // steps of this chunk that still have a round to request
+        int j0 = 0;
+        for (; j0 + U <= refills; j0 += U) {
 #pragma unroll
             for (int u = 0; u < U; u++) {
-                const int f = min(base + per_round * U + (u * 4 + wave) * pl.rw_count + pl.rw, fcount - 1);
-                graw[u] = load_row<F>(pl, gbank + (size_t)f * row_bytes);
-                uraw[u] = load_row<F>(pl, ubank + (size_t)f * row_bytes);
+                finish(u, j0 + u);
+                issue(u, c0 + j0 + u + U);
+            }
+        }
+        for (; j0 < cn; j0 += U) {
+#pragma unroll
+            for (int u = 0; u < U; u++) {
+                if (j0 + u >= cn) break;
+                finish(u, j0 + u);
+                if (j0 + u < refills) issue(u, c0 + j0 + u + U);
             }
         }
         __builtin_amdgcn_wave_barrier();
-        if (lane < U * pl.rw_count) {
-            const int u = lane / pl.rw_count, rw = lane - u * pl.rw_count;
-            const int f = base + (u * 4 + wave) * pl.rw_count + rw;
+        if (lane < cn * pl.rw_count) {
+            const int j = lane / pl.rw_count, rw = lane - j * pl.rw_count;
+            const int f = ((c0 + j) * 4 + wave) * pl.rw_count + rw;
             if (f < fcount) {
 #pragma unroll
                 for (int tau = 0; tau < T; tau++) {
