@@ -1100,9 +1100,9 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
                 const infr_op_add& ad = plan->ops[b0 + 4].u.add;
                 other = ad.a == ld.dst ? ad.b : ad.a;
             }
-            // one token row only: with more rows the launches saved no longer matter and the down kernel
-            // streams best with one wave per routed slot
-            if (sc.batched || sc.bucketed || sc.rows != 1 || m.fused_gate_up) continue;
+            // the per-token kernels only (1 to 15 token rows): every row's blocks read the always-on expert's rows
+            // again, from the L2 after the first
+            if (sc.batched || sc.bucketed || m.fused_gate_up) continue;
             if (lg.x != m.x || (int)lg.m != sc.rows || lg.in_f != m.ne || lg.out_f != m.n_ff_exp) continue;
             if (ld.x != ga.dst || !temp(ga.dst) || ld.in_f != m.n_ff_exp || ld.out_f != m.ne || ld.w_off != 0) continue;
             if (other != m.dst || !temp(m.dst)) continue;
