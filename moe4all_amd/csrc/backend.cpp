@@ -8,6 +8,7 @@
 #include <hip/hip_runtime.h>
 
 #include <atomic>
+#include <cmath>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -78,6 +79,8 @@ constexpr uint32_t kBatchedMinRows = 32;
 // Token rows from which a decode batch is bucketed by expert so that each selected expert's rows are
 // read from HBM once (same f32-accurate inner product as the per-token kernels).
 constexpr uint32_t kBucketedMinRows = 16;
+// ... and only when the expected number of distinct experts of the batch is below this share of its pairs.
+constexpr double kBucketedMaxDistinctRatio = 0.62;
 // Token rows from which a dense Op::Linear runs as one bucket of the grouped GEMMs.
 constexpr uint32_t kLinearBatchedMinRows = 128;
 
@@ -292,18 +295,19 @@ void drain_prof(infr_hip_backend* be) {
     be->pending.clear();
 }
 
-// The per-token path of Op::MoeFfn (1 to 15 token rows) once logits are in rp.logits and gp / rp are filled in:
+// The per-token path of Op::MoeFfn (1 to 31 token rows; the bucketed path takes batches of 16 or more whose pairs fall on few distinct experts) once logits are in rp.logits and gp / rp are filled in:
 // routing (inside the gate/up kernel where that is cheaper than a launch), gate/up with the gated activation,
 // down with the rank-ordered combine.  timed == false: no profiling events (nothing is created or allocated).
 void moe_per_token(infr_hip_backend* be, hipStream_t s, infr::MoeGemvParams& gp, const infr::RouteParams& rp, int rows,
                    uint32_t n_expert_total, bool timed) {
     infr_hip_backend* tb = timed ? be : nullptr;
-    // Every block of the gate/up kernel routes its own token row when that is cheaper than a
-    // launch of the routing kernel: the blocks of one compute unit repeat it once per row.
+    // Every block of the gate/up kernel routes its own token row: two of its waves do, while the others turn the row
+    // into fixed-point cells, which measured 1 to 3 % faster than a launch of the routing kernel at every batch of the
+    // per-token path.  The unit-format kernel routes on its only four waves and keeps the older rule.
     const bool fast_gu = infr::moe_gate_up_routes_inline(gp);
     const bool units = !fast_gu && !gp.sh_gate && infr::moe_gate_up_units_supported(gp);
-    gp.route_inline = (fast_gu || (units && infr::moe_gate_up_units_routes_inline(gp))) &&
-                              (rows == 1 || (uint64_t)rows * n_expert_total <= 512) ? 1 : 0;
+    gp.route_inline = (fast_gu || (units && infr::moe_gate_up_units_routes_inline(gp) &&
+                                   (rows == 1 || (uint64_t)rows * n_expert_total <= 512))) ? 1 : 0;
     if (!gp.route_inline) {
         Timed t(tb, "route_topk");
         infr::launch_route(s, rp);
@@ -807,7 +811,14 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
                               round_up(pairs * m.ne * 4, 256);
                 }
                 bool bucketed = false;
-                if (!batched && rows >= kBucketedMinRows && m.n_used <= 64) {
+                // Bucketing pays when the batch's pairs fall on few enough distinct experts: with uniform routing
+                // E * (1 - (1 - K/E)^rows) of them are expected, and the bucketed kernels move a byte about 0.6 times as
+                // fast as the per-token kernels do (128 experts, top-8, 16 rows: 3.2 against 4.9 TB/s), so they win below
+                // that ratio of distinct experts to pairs (128 experts, top-8: from 18 rows on; 256 experts, top-8: not
+                // before the matrix-core path takes over; measured on both sides of the threshold).
+                const double expect_distinct = (double)m.n_expert * (1.0 - std::pow(1.0 - (double)m.n_used / (double)m.n_expert, (double)rows));
+                const bool few_distinct = expect_distinct < kBucketedMaxDistinctRatio * (double)rows * (double)m.n_used;
+                if (!batched && rows >= kBucketedMinRows && few_distinct && m.n_used <= 64) {
                     infr::MoeGemvParams probe{};
                     probe.gate_dt = c.dt(m.gate_exps);
                     probe.up_dt = m.fused_gate_up ? probe.gate_dt : c.dt(m.up_exps);
@@ -1100,7 +1111,7 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
                 const infr_op_add& ad = plan->ops[b0 + 4].u.add;
                 other = ad.a == ld.dst ? ad.b : ad.a;
             }
-            // the per-token kernels only (1 to 15 token rows): every row's blocks read the always-on expert's rows
+            // the per-token kernels only: every row's blocks read the always-on expert's rows
             // again, from the L2 after the first
             if (sc.batched || sc.bucketed || m.fused_gate_up) continue;
             if (lg.x != m.x || (int)lg.m != sc.rows || lg.in_f != m.ne || lg.out_f != m.n_ff_exp) continue;

@@ -660,7 +660,7 @@ static bool try_gate_up(hipStream_t s, const MoeGemvParams& p) {
     const int n_slots = p.n_used + (p.sh_gate ? 1 : 0);
     // about one block per compute unit for a single token row; with several rows about two, resident together, so
     // that a compute unit pays a block's start (routing, x) once while it streams
-    int ft = p.rows >= 2 ? ceil_div(p.nff * p.rows, 2 * p.n_cu) : ceil_div(p.nff, p.n_cu);
+    int ft = p.rows >= 2 ? ceil_div(p.nff, max(1, 2 * p.n_cu / p.rows)) : ceil_div(p.nff, p.n_cu);
     if (ft < 1) ft = 1;
     const int per_wave = ceil_div(ft * n_slots, 4 * rw);
     dim3 grid(ceil_div(p.nff, ft), p.rows), block(256);
