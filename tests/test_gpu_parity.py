@@ -553,14 +553,17 @@ def test_fused_dense_ffn_launches_give_the_bits_of_the_separate_ops(be, rows, ac
                                          # tiles of several weight rows per wavefront: the streamed decode kernels
                                          (1, 4, {"with_dims": (2048, 2048)}),
                                          (1, 8, {"weight_before": True, "with_dims": (2048, 2048)}),
-                                         (1, 6, {"with_down_scale": True, "with_dims": (2048, 1536)})])
+                                         (1, 6, {"with_down_scale": True, "with_dims": (2048, 1536)}),
+                                         # a decode batch past 16 rows that stays on the per-token kernels (its pairs
+                                         # are expected on too many distinct experts for bucketing to pay)
+                                         (20, 2, {"with_experts": 64})])
 def test_shared_expert_as_an_extra_slot_gives_the_bits_of_the_separate_ops(be, rows, K, opts):
     """MoeFfn followed by an ungated shared expert (Linear, Linear, GatedAct, Linear, Add —
     crates/infr-llama/src/seam/runner.rs:8116-8174) runs as one more slot of the two routed decode
     kernels when the routed sum is a single-use Internal tensor, for one token row and for the few rows of a decode
     batch on the per-token kernels.  Declaring that tensor an Output keeps MoeFfn and the dense FFN apart; both must
     give identical bits."""
-    (ne, nff), E = opts.get("with_dims", (1024, 512)), 16
+    (ne, nff), E = opts.get("with_dims", (1024, 512)), opts.get("with_experts", 16)
     rng = np.random.default_rng(100 + rows)
     x = rng.standard_normal((rows, ne)).astype(np.float32)
     router = (rng.standard_normal((E, ne)) * 0.1).astype(np.float32)
