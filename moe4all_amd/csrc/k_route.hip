@@ -120,28 +120,30 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const uint8_t* __res
                 if (blockIdx.x == 0 && blockIdx.y == 0) reinterpret_cast<float4*>(nrm.xn_out)[idx] = xr[i];
             }
         }
+        // element 4v + t of a row: chain (4v + t) & 7 = 4 (v & 1) + t, step (4v + t) >> 3 = v >> 1: the four
+        // elements of a 128-bit load go to four chains at one step, or all four to the tail
 #pragma unroll
         for (int i = 0; i < 4; i++) {
             const int idx = tid + 256 * i, rr = idx / nv, v = idx - rr * nv;
             if (rr >= rpb) continue;
-            const float fv[4] = {xr[i].x, xr[i].y, xr[i].z, xr[i].w};
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-                int k = 4 * v + q, c = k >> 3, j = k & 7;
-                if (c < nc) xs[rr * estride + j * jstride + c] = fv[q];
-                else xt[rr * 8 + j] = fv[q];
+            if ((v >> 1) < nc) {
+                float* d = xs + rr * estride + 4 * (v & 1) * jstride + (v >> 1);
+                d[0] = xr[i].x; d[jstride] = xr[i].y; d[2 * jstride] = xr[i].z; d[3 * jstride] = xr[i].w;
+            } else {
+                float* d = xt + rr * 8;
+                d[0] = xr[i].x; d[1] = xr[i].y; d[2] = xr[i].z; d[3] = xr[i].w;
             }
         }
 #pragma unroll
         for (int i = 0; i < 8; i++) {
             const int idx = tid + 256 * i, e = idx / nv, v = idx - e * nv;
             if (e >= EPB) continue;
-            const float fv[4] = {wr[i].x, wr[i].y, wr[i].z, wr[i].w};
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-                int k = 4 * v + q, c = k >> 3, j = k & 7;
-                if (c < nc) w[e * estride + j * jstride + c] = fv[q];
-                else wt[e * 8 + j] = fv[q];
+            if ((v >> 1) < nc) {
+                float* d = w + e * estride + 4 * (v & 1) * jstride + (v >> 1);
+                d[0] = wr[i].x; d[jstride] = wr[i].y; d[2 * jstride] = wr[i].z; d[3 * jstride] = wr[i].w;
+            } else {
+                float* d = wt + e * 8;
+                d[0] = wr[i].x; d[1] = wr[i].y; d[2] = wr[i].z; d[3] = wr[i].w;
             }
         }
     } else if (rdt == INFR_F32 && (ne & 3) == 0) {
