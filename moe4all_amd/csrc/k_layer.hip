@@ -275,10 +275,17 @@ __global__ __launch_bounds__(256) void moe_layer_fused(MoeLayerParams q) {
                     const uint32_t kmax = wave_max_u32(has ? bk : 0u);
                     const bool match = has && bk == kmax;
                     uint32_t win = 0xFFFFFFFFu;
+                    const uint64_t holders = __ballot(match);
+                    if (__builtin_popcountll(holders) == 1) {
+                        // one lane holds the largest key: its candidate is the winner
+                        win = (uint32_t)__builtin_amdgcn_readlane((int)bi, __builtin_ctzll(holders));
+                    } else {
+                        // several lanes hold it: smallest slot first, then smallest lane
 #pragma unroll
-                    for (int t = 0; t < NS; t++) {
-                        const uint64_t mk = __ballot(match && (int)(bi >> 6) == t);
-                        if (win == 0xFFFFFFFFu && mk) win = (uint32_t)(t * kWave) + (uint32_t)__builtin_ctzll(mk);
+                        for (int t = 0; t < NS; t++) {
+                            const uint64_t mk = __ballot(match && (int)(bi >> 6) == t);
+                            if (win == 0xFFFFFFFFu && mk) win = (uint32_t)(t * kWave) + (uint32_t)__builtin_ctzll(mk);
+                        }
                     }
                     if (win == 0xFFFFFFFFu) win = 0;
                     if ((int)(win & 63u) == lane) {
