@@ -327,39 +327,52 @@ __device__ __forceinline__ void route_duo_first(const RouteParams& p, int row, i
         if (lane == 0) duo->psum = psum;
         ROUTE_STAMP(3);
     } else {
-        uint32_t keys[NS], taken = 0;
+        // Every lane first sorts its own NS candidates, (key descending, id ascending: adjacent exchanges on a strict
+        // compare keep equal keys in id order), so a round only looks at the lane's head: one reduction for the
+        // largest key, one ballot for who holds it, and the winner's list moves up by one.  An exponential is not
+        // negative, so a live key has its top bit set and 0 marks an empty place.
+        uint32_t key[NS], id[NS];
 #pragma unroll
         for (int s = 0; s < NS; s++) {
-            keys[s] = order_key(pr[s]);
-            if (s * kWave + lane >= n) taken |= 1u << s;
+            id[s] = (uint32_t)(s * kWave + lane);
+            key[s] = (s * kWave + lane < n) ? order_key(pr[s]) : 0u;
+        }
+#pragma unroll
+        for (int a = 0; a + 1 < NS; a++) {
+#pragma unroll
+            for (int b = 0; b + 1 < NS - a; b++) {
+                const bool swap = key[b + 1] > key[b];
+                const uint32_t hk = swap ? key[b + 1] : key[b], lk = swap ? key[b] : key[b + 1];
+                const uint32_t hi = swap ? id[b + 1] : id[b], li = swap ? id[b] : id[b + 1];
+                key[b] = hk; key[b + 1] = lk;
+                id[b] = hi; id[b + 1] = li;
+            }
         }
         for (int k = 0; k <= p.n_used; k++) {
-            uint32_t bk = 0, bi = 0xFFFFFFFFu;
-            float be = 0.0f;
-#pragma unroll
-            for (int s = 0; s < NS; s++) {
-                if (taken & (1u << s)) continue;
-                if (bi == 0xFFFFFFFFu || keys[s] > bk) { bk = keys[s]; bi = (uint32_t)(s * kWave + lane); be = pr[s]; }
-            }
-            const bool has = bi != 0xFFFFFFFFu;
-            const uint32_t kmax = wave_max_u32(has ? bk : 0u);
-            const bool match = has && bk == kmax;
-            uint32_t win = 0xFFFFFFFFu;
+            const uint32_t kmax = wave_max_u32(key[0]);
+            const bool match = key[0] == kmax && kmax != 0u;
             const uint64_t holders = __ballot(match);
+            uint32_t win;
             if (__builtin_popcountll(holders) == 1) {
-                win = (uint32_t)__builtin_amdgcn_readlane((int)bi, __builtin_ctzll(holders));
+                win = (uint32_t)__builtin_amdgcn_readlane((int)id[0], __builtin_ctzll(holders));
             } else {
-#pragma unroll
-                for (int s = 0; s < NS; s++) {
-                    const uint64_t mk = __ballot(match && (int)(bi >> 6) == s);
-                    if (win == 0xFFFFFFFFu && mk) win = (uint32_t)(s * kWave) + (uint32_t)__builtin_ctzll(mk);
-                }
+                // several lanes hold the largest key: the smallest id among their heads (a lane's own equal keys
+                // are already in id order)
+                win = wave_min_u32(match ? id[0] : 0xFFFFFFFFu);
             }
-            if (win == 0xFFFFFFFFu) win = 0;
-            if ((int)(win & 63u) == lane && match && bi == win) {   // this lane's best is the winner
-                taken |= 1u << (win >> 6);
+            if (holders == 0 && lane == 0) {   // nothing comparable left (keys of negative NaNs): the check fails
+                duo->cand[k] = 0;
+                duo->cand_e[k] = __uint_as_float(0x7FC00000u);
+            }
+            if (match && id[0] == win) {
                 duo->cand[k] = (int32_t)win;
-                duo->cand_e[k] = be;
+                duo->cand_e[k] = __uint_as_float(key[0] & 0x7FFFFFFFu);   // the exponential back from its key
+#pragma unroll
+                for (int s = 0; s + 1 < NS; s++) {
+                    key[s] = key[s + 1];
+                    id[s] = id[s + 1];
+                }
+                key[NS - 1] = 0u;
             }
         }
     }
