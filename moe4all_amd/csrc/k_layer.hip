@@ -250,48 +250,75 @@ __global__ __launch_bounds__(256) void moe_layer_fused(MoeLayerParams q) {
                 for (int t = 0; t < NS; t++) ex[t * kWave + lane] = pr[t];
                 __builtin_amdgcn_wave_barrier();
                 float psum = 0.0f;
-#pragma unroll 2
-                for (int i = 0; i < n_expert; i += 8) {   // n_expert is a multiple of 64
-                    float t8[8];
+                {
+                    // the terms come in batches of 32 (eight 128-bit broadcast reads), the next batch requested
+                    // before the current one is added, so the chain of dependent adds never waits for LDS
+                    // (n_expert is a multiple of 64, ex is 16-byte aligned)
+                    float4 cur[8], nxt[8];
 #pragma unroll
-                    for (int k = 0; k < 8; k++) t8[k] = ex[i + k];
+                    for (int k = 0; k < 8; k++) cur[k] = reinterpret_cast<const float4*>(ex)[k];
+                    for (int i = 0; i < n_expert; i += 32) {
+                        const int ni = i + 64 <= n_expert ? i + 32 : i;   // past the end: re-read, unused
 #pragma unroll
-                    for (int k = 0; k < 8; k++) psum = __fadd_rn(psum, t8[k]);
+                        for (int k = 0; k < 8; k++) nxt[k] = reinterpret_cast<const float4*>(ex + ni)[k];
+#pragma unroll
+                        for (int k = 0; k < 8; k++) {
+                            psum = __fadd_rn(psum, cur[k].x);
+                            psum = __fadd_rn(psum, cur[k].y);
+                            psum = __fadd_rn(psum, cur[k].z);
+                            psum = __fadd_rn(psum, cur[k].w);
+                        }
+#pragma unroll
+                        for (int k = 0; k < 8; k++) cur[k] = nxt[k];
+                    }
                 }
                 if (lane == 0) s_psum = psum;
             } else {
-                uint32_t keys[NS], taken = 0;
+                // every lane first sorts its own NS candidates, (key descending, id ascending), so a round only looks
+                // at the lane's head: one reduction for the largest key, one ballot for who holds it, and the winner's
+                // list moves up by one.  An exponential is not negative, so a live key has its top bit set and 0
+                // marks an empty place.
+                uint32_t key[NS], id[NS];
 #pragma unroll
-                for (int t = 0; t < NS; t++) keys[t] = order_key(pr[t]);
+                for (int t = 0; t < NS; t++) {
+                    id[t] = (uint32_t)(t * kWave + lane);
+                    key[t] = order_key(pr[t]);
+                }
+#pragma unroll
+                for (int a = 0; a + 1 < NS; a++) {
+#pragma unroll
+                    for (int b = 0; b + 1 < NS - a; b++) {
+                        const bool swap = key[b + 1] > key[b];   // strict, adjacent: equal keys stay in id order
+                        const uint32_t hk = swap ? key[b + 1] : key[b], lk = swap ? key[b] : key[b + 1];
+                        const uint32_t hi = swap ? id[b + 1] : id[b], li = swap ? id[b] : id[b + 1];
+                        key[b] = hk; key[b + 1] = lk;
+                        id[b] = hi; id[b + 1] = li;
+                    }
+                }
                 for (int k = 0; k < 9; k++) {
-                    uint32_t bk = 0, bi = 0xFFFFFFFFu;
-                    float be = 0.0f;
-#pragma unroll
-                    for (int t = 0; t < NS; t++) {
-                        if (taken & (1u << t)) continue;
-                        if (bi == 0xFFFFFFFFu || keys[t] > bk) { bk = keys[t]; bi = (uint32_t)(t * kWave + lane); be = pr[t]; }
-                    }
-                    const bool has = bi != 0xFFFFFFFFu;
-                    const uint32_t kmax = wave_max_u32(has ? bk : 0u);
-                    const bool match = has && bk == kmax;
-                    uint32_t win = 0xFFFFFFFFu;
+                    const uint32_t kmax = wave_max_u32(key[0]);
+                    const bool match = key[0] == kmax && kmax != 0u;
                     const uint64_t holders = __ballot(match);
+                    uint32_t win;
                     if (__builtin_popcountll(holders) == 1) {
-                        // one lane holds the largest key: its candidate is the winner
-                        win = (uint32_t)__builtin_amdgcn_readlane((int)bi, __builtin_ctzll(holders));
+                        win = (uint32_t)__builtin_amdgcn_readlane((int)id[0], __builtin_ctzll(holders));
                     } else {
-                        // several lanes hold it: smallest slot first, then smallest lane
-#pragma unroll
-                        for (int t = 0; t < NS; t++) {
-                            const uint64_t mk = __ballot(match && (int)(bi >> 6) == t);
-                            if (win == 0xFFFFFFFFu && mk) win = (uint32_t)(t * kWave) + (uint32_t)__builtin_ctzll(mk);
-                        }
+                        // several lanes hold the largest key: the smallest id among their heads
+                        win = wave_min_u32(match ? id[0] : 0xFFFFFFFFu);
                     }
-                    if (win == 0xFFFFFFFFu) win = 0;
-                    if ((int)(win & 63u) == lane) {
-                        taken |= 1u << (win >> 6);
+                    if (holders == 0 && lane == 0) {   // nothing comparable left (keys of negative NaNs): the check fails
+                        s_cand[k] = 0;
+                        s_cand_e[k] = __uint_as_float(0x7FC00000u);
+                    }
+                    if (match && id[0] == win) {
                         s_cand[k] = (int32_t)win;
-                        s_cand_e[k] = be;   // this lane's best is the winner
+                        s_cand_e[k] = __uint_as_float(key[0] & 0x7FFFFFFFu);   // the exponential back from its key
+#pragma unroll
+                        for (int t = 0; t + 1 < NS; t++) {
+                            key[t] = key[t + 1];
+                            id[t] = id[t + 1];
+                        }
+                        key[NS - 1] = 0u;
                     }
                 }
             }
