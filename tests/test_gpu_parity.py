@@ -237,6 +237,7 @@ def _realistic(rng, E, rows_out, cols, dt):
     (4, 2048, 128, 8, 768, H.Q8_0, H.Q8_0),    # config 3, batch 4
     (16, 2048, 128, 8, 768, H.Q4K, H.Q6K),     # config 3 shape with the K-quant mix
     (1, 4096, 256, 8, 1536, H.Q4K, H.Q6K),     # one layer of config 5
+    (1, 512, 384, 15, 1280, H.Q4K, H.Q6K),     # 8 candidates per lane and 16 selection rounds in the two-wave routing; 8 rows per wave
     (3, 256, 8, 3, 256, H.Q6K, H.Q4K),         # small, several weight rows per wavefront
     (2, 512, 8, 2, 1024, H.Q8_0, H.Q4K),
     (2, 96, 6, 2, 64, H.Q8_0, H.Q8_0),         # shape-generic kernels (96 is not a multiple of 256)
