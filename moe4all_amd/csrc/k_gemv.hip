@@ -176,13 +176,15 @@ __global__ __launch_bounds__(256) void moe_gate_up_fast(MoeGemvParams p, int ft)
 }
 
 // ------------------------------------------------------------------------------- gate/up, streamed
-// The same tiles as moe_gate_up_fast, for tiles of several items per wave.  Three things differ.  The routing wave
-// and the conversion of x run side by side: wave 0 routes (or fetches the ids) while waves 1..3 turn x into one set of
-// fixed-point cells for the whole block.  A wave keeps D items (a gate row and an up row each) in flight as a ring:
-// it finishes the oldest item and requests the item D places ahead into the registers that just became free, so its
-// dot products and its loads alternate item by item and the four waves drift apart instead of all waiting for memory
-// and then all computing.  Results wait in LDS until the wave has finished a chunk of its items, then one lane per
-// item applies the gated activation.
+// The same tiles as moe_gate_up_fast, for tiles of several items per wave, on NW waves (8 to 12).  Three things differ.
+// The routing and the conversion of x run side by side: waves 0 and 1 route (plain softmax: the sum on one, the
+// selection on the other; anything else on wave 0 alone; or wave 0 fetches the ids) while the remaining waves turn x
+// into one set of fixed-point cells for the whole block.  A wave keeps D items (a gate row and an up row each) in
+// flight as a ring: it finishes the oldest item and requests the item D places ahead into the registers that just
+// became free, so its dot products and its loads alternate item by item and the waves drift apart instead of all
+// waiting for memory and then all computing; many waves with a shallow ring measured faster than few with a deep one.
+// Results wait in LDS until the wave has finished a chunk of its items, then one lane per item applies the gated
+// activation.  The second launch bound (waves per SIMD) keeps two 8-wave blocks resident on a compute unit.
 template <class F, int D, int NW>
 __global__ __launch_bounds__(64 * NW, NW <= 8 ? 4 : 3) void moe_gate_up_stream(MoeGemvParams p, int ft) {
     extern __shared__ __attribute__((aligned(16))) uint32_t dyn_lds[];
