@@ -503,9 +503,11 @@ __global__ __launch_bounds__(64 * NW) void moe_down_combine_stream(MoeGemvParams
     __syncthreads();
     const int G = (ocount + pl.rw_count - 1) / pl.rw_count;   // units per slot
     const int n_units = n_slots * G;
-    const int upw = (n_units + NW - 1) / NW;
-    const int ub = wave * upw;
-    const int cn = max(0, min(upw, n_units - ub));
+    // equal contiguous runs, the remainder one unit each to the first waves (72 units on 16 waves: 5 for eight waves and
+    // 4 for eight, so every SIMD's four waves carry 18, not 20 on two SIMDs and 15 on another)
+    const int base_units = n_units / NW, rem_units = n_units - base_units * NW;
+    const int ub = wave * base_units + min(wave, rem_units);
+    const int cn = base_units + (wave < rem_units ? 1 : 0);
     const float inv_G = 1.0f / (float)G;
     auto issue = [&](typename F::Raw& raw, int j) {
         const int u = ub + j;
