@@ -246,8 +246,7 @@ __global__ __launch_bounds__(64 * NW, NW <= 8 ? 4 : 3) void moe_gate_up_stream(M
         __syncthreads();
     }
     GEMV_STAMP(1);
-    typename F::X x;
-    F::fetch_x(x, cells, pl.blk, pl.sub);
+    typename F::X x;   // fetched once the first items are requested
     const int nitems = fcount * n_slots;
     const int per_step = NW * pl.rw_count;   // items the block's waves take per ring step
     const int n_mine = nitems > wave * pl.rw_count ? (nitems - wave * pl.rw_count + per_step - 1) / per_step : 0;
@@ -278,7 +277,10 @@ __global__ __launch_bounds__(64 * NW, NW <= 8 ? 4 : 3) void moe_gate_up_stream(M
 #pragma unroll
         for (int d = 0; d < D; d++)
             if (d < cn) issue(ring[d], c0 + d);
-        if (c0 == 0) GEMV_STAMP(2);
+        if (c0 == 0) {
+            F::fetch_x(x, cells, pl.blk, pl.sub);
+            GEMV_STAMP(2);
+        }
         // steady state: every step finishes its ring entry and refills it, no branch in between, so the waits count
         // exactly the loads that are younger than the entry
         const int refills = cn - D;   // steps that still have an item to request
