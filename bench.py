@@ -7,13 +7,14 @@ HBM-resident weights and its own N(0,1) activation rows.  Headline workload: the
 (48 layers, hidden 2048, 128 experts, top-8, intermediate 768, Q4_K gate/up + Q6_K down), decode batch 1,
 synthetic seeded weights.
 
-Prints ONE JSON line: whole-job decode tok/s of the headline workload, the roofline of its dominant kernel
-measured live with HIP events attached to each dispatch on the backend's stream, the time a chain of dependent
-plain reads of the same sizes takes on this device (what a kernel chain of this shape cannot go below), and a
-CPU baseline (the oracle, a scalar C restatement of the reference's CPU path, timed on this host's cores on a
-bounded sample).  With no --config the same line carries a "configs" array with the other benchmark
-configurations (single Q8_0 layer, multi-stream decode, prefill chunks, the large shape with a shared expert),
-each measured the same way on fewer steps.
+The LAST line of stdout is the headline as one compact JSON object (under 2,000 bytes): whole-job decode tok/s of
+the headline workload, the roofline of its dominant kernel measured live with HIP events attached to each dispatch
+on the backend's stream, the time a chain of dependent plain reads of the same sizes takes on this device (what a
+kernel chain of this shape cannot go below), and a CPU baseline (the oracle, a scalar C restatement of the
+reference's CPU path, timed on this host's cores on a bounded sample).  With no --config every other benchmark
+configuration (single Q8_0 layer, multi-stream decode, prefill chunks, the large shape with a shared expert) is
+measured the same way and printed as a compact JSON line of its own BEFORE the headline; the per-kernel tables and
+floors of every workload go to the file named by --detail (default gpurun_out/bench_configs.json).
 """
 from __future__ import annotations
 
@@ -335,11 +336,9 @@ def measure(be, stack, config, batch, steps, warmup, *, sublayer=False, kernel_t
             n_sample += 1
         per_layer_s = spent / n_sample
         cpu = {"value": round(cpu_rows / (per_layer_s * n_layer), 3), "unit": "tok/s", "cores": threads, "kind": "port",
-               "sample": f"scalar, auto-vectorised C restatement of the reference's CPU path (not its hand-written AVX2 / AVX-512 / "
-                         f"VNNI tiers: a floor for what the reference's CPU backend would do); {n_sample} layer-passes of layer 0 "
-                         f"(routed experts only, {cpu_rows} token rows each) with distinct seeded tokens, "
-                         f"{per_layer_s * 1e3:.2f} ms per layer-pass, "
-                         f"{'production numerics (int8 activations, scalar integer dots)' if production else 'f32 numerics (dequantise a row, f32 dot)'}, "
+               "sample": f"scalar auto-vectorised C restatement of the reference's CPU path, not its AVX2/AVX-512/VNNI tiers; "
+                         f"{n_sample} passes of layer 0 (routed experts, {cpu_rows} token rows), {per_layer_s * 1e3:.2f} ms each, "
+                         f"{'int8-activation production numerics' if production else 'f32 dequantise-and-dot numerics'}, "
                          f"scaled to {n_layer} layers",
                "ms_per_layer": round(per_layer_s * 1e3, 3)}
 
@@ -349,9 +348,9 @@ def measure(be, stack, config, batch, steps, warmup, *, sublayer=False, kernel_t
         "ms_per_step_min": round(min(group_ms), 4), "ms_per_step_max": round(max(group_ms), 4),
         "spread": f"min / max over {groups} groups of {per_group} steps run after the timed region, a sync after each group",
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        # decode: exact integer dots on 23-bit fixed-point activations, scales and sums in f32; batched path: f16
-        # operands on the matrix cores with f32 accumulation
-        "dtype": "f16" if batch >= 32 else "f32", "data": "synthetic",
+        # decode: exact integer dots (v_dot4 on byte planes) on 23-bit fixed-point activations, scales and sums in f32;
+        # batched path: f16 operands on the matrix cores with f32 accumulation
+        "dtype": "f16-mfma/f32-acc" if batch >= 32 else "i8dot-23bit-act/f32-acc", "data": "synthetic",
         "config": {"workload": (shape.name if n_layer == shape.n_layer else f"{shape.name}[{n_layer} layers]") +
                                ("+rmsnorm+residual" if sublayer else "") + ("/unfused" if no_fusion else ""),
                    "layers": n_layer, "hidden": shape.ne, "experts": shape.n_expert, "top_k": shape.n_used,
@@ -377,6 +376,34 @@ def measure(be, stack, config, batch, steps, warmup, *, sublayer=False, kernel_t
 # the other benchmark configurations, measured after the headline when no --config is given:
 # (config, layers (0 = the shape's), batches or chunk sizes)
 OTHER_WORKLOADS = (("c1", 0, (1, 4, 16)), ("c4", 0, (512, 2048)), ("c4k", 0, (512, 2048)), ("c5", 0, (1, 8)))
+LINE_LIMIT = 1900   # bytes; the harness that records this run keeps only the tail of stdout
+
+
+def compact(res, headline):
+    """The one-line form of a result: the contract's keys, the roofline and the CPU baseline, no per-kernel tables."""
+    keep = ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "ms_per_step_min", "ms_per_step_max",
+            "higher_is_better", "scaling", "vs_baseline", "dtype", "data")
+    out = {k: res[k] for k in keep if k in res}
+    c = res["config"]
+    out["config"] = {k: c[k] for k in ("workload", "layers", "hidden", "experts", "top_k", "intermediate", "gate_up", "down",
+                                       "shared_intermediate", "batch", "parallelism")}
+    out["layer"] = {k: res["layer"][k] for k in ("us_per_layer", "alg_bytes_per_layer", "frac_of_hbm_peak")}
+    out["roofline"] = res["roofline"]
+    cpu = res.get("cpu_baseline")
+    if cpu:
+        cpu = dict(cpu)
+        if not headline:
+            cpu["sample"] = cpu["sample"].split(";")[1].strip() if ";" in cpu["sample"] else cpu["sample"]
+        out["cpu_baseline"] = cpu
+    if headline:
+        for k in ("device", "compute_units", "detail"):
+            if k in res:
+                out[k] = res[k]
+    line = json.dumps(out, separators=(",", ":"))
+    if len(line) > LINE_LIMIT and cpu:      # never let prose push the line past what the recorder keeps
+        cpu["sample"] = cpu["sample"][:max(40, len(cpu["sample"]) - (len(line) - LINE_LIMIT))]
+        line = json.dumps(out, separators=(",", ":"))
+    return line
 
 
 def main():
@@ -389,8 +416,10 @@ def main():
                          "(Q8_0), prefill chunk of --tokens with Zipf(1.1) expert popularity; c4k: same with "
                          "Q4_K gate/up + Q6_K down; mxfp4: a decode stack of the gpt-oss-120b expert shape with MXFP4 banks "
                          "(the 32-element-unit kernels; use --batch >= 32 for the unit-decoder grouped GEMM).  Default: c2 as the "
-                         "headline plus every other benchmark configuration in a \"configs\" array")
-    ap.add_argument("--headline-only", action="store_true", help="with no --config: skip the \"configs\" array")
+                         "headline (last line) after one line per other benchmark configuration")
+    ap.add_argument("--headline-only", action="store_true", help="with no --config: measure the headline workload only")
+    ap.add_argument("--detail", default=os.path.join(ROOT, "gpurun_out", "bench_configs.json"),
+                    help="file that receives the full results (per-kernel tables, floors) of every workload; '' = none")
     ap.add_argument("--tokens", type=int, default=2048, help="prefill chunk size for c4/c4k")
     ap.add_argument("--layers", type=int, default=0, help="override the layer count (0 = the config's)")
     ap.add_argument("--batch", type=int, default=1)
@@ -434,8 +463,8 @@ def main():
     out["device"], out["compute_units"], out["setup_s"] = caps["name"], caps["compute_units"], round(stack.setup_s, 1)
     stack.free()
 
+    detail = {"headline": out, "configs": []}
     if args.config is None and not args.headline_only:
-        configs = []
         for cfg, layers, sizes in OTHER_WORKLOADS:
             pf = cfg in ("c4", "c4k")
             stacks = {}
@@ -450,18 +479,27 @@ def main():
                     else:
                         stacks[key] = Stack(be, sh, layers or sh.n_layer, pf)
                 st = stacks[key]
-                steps = max(5, min(args.steps, 40 if st.n_layer > 1 else 100))
-                res = measure(be, st, cfg, size, steps, min(args.warmup, 5), cpu_budget_s=0.0 if args.no_cpu_baseline else 2.5,
+                # a one-layer workload of well under a millisecond needs many steps for a stable mean
+                steps = max(5, min(args.steps, 40)) if st.n_layer > 1 else max(args.steps, 200)
+                res = measure(be, st, cfg, size, steps, max(min(args.warmup, 5), 5 if st.n_layer == 1 else 0),
+                              cpu_budget_s=0.0 if args.no_cpu_baseline else 2.5,
                               kernel_timing=not args.no_kernel_timing, floor=not args.no_floor)
                 res["setup_s"] = round(st.setup_s, 1)
-                for k in ("n_gpus", "higher_is_better", "scaling", "vs_baseline", "data"):
-                    res.pop(k, None)
-                configs.append(res)
+                detail["configs"].append(res)
+                print(compact(res, headline=False), flush=True)
             for st in {id(v): v for v in stacks.values()}.values():
                 st.free()
-        out["configs"] = configs
     be.close()
-    print(json.dumps(out))
+    # per-kernel tables, floors and spreads of every workload: to a file, not to stdout
+    if args.detail:
+        try:
+            os.makedirs(os.path.dirname(os.path.abspath(args.detail)), exist_ok=True)
+            with open(args.detail, "w") as f:
+                json.dump(detail, f, indent=1)
+            out["detail"] = os.path.relpath(args.detail, ROOT) if os.path.abspath(args.detail).startswith(ROOT) else args.detail
+        except OSError as e:
+            print(f"bench.py: could not write {args.detail}: {e}", file=sys.stderr)
+    print(compact(out, headline=True), flush=True)
 
 
 if __name__ == "__main__":

@@ -265,23 +265,6 @@ infr_status infr_hip_sync(infr_hip_backend *be);
 /* Thread-local message of the last failing call on this thread ("" if none). */
 const char *infr_hip_last_error(void);
 
-/* Per-kernel timing, the counterpart of the reference's per-op profiler seam
- * (crates/infr-core/src/prof.rs:54-120, enabled by `prof.ops`): while enabled every kernel
- * launch is bracketed by HIP events on the backend's stream.  Reading drains and resets. */
-typedef struct infr_hip_prof_entry {
-    char kernel[64];
-    uint64_t launches;
-    double total_ms;
-    double min_ms, max_ms;
-} infr_hip_prof_entry;
-infr_status infr_hip_prof_enable(infr_hip_backend *be, int on);
-infr_status infr_hip_prof_read(infr_hip_backend *be, infr_hip_prof_entry *out, uint32_t cap, uint32_t *n_out);
-/* Measurement only (no counterpart in the reference).  on != 0: from now on the grouped GEMMs of the batched
- * Op::MoeFfn / Op::Linear paths (Q4_K / Q6_K / Q8_0 weights) run their loads, LDS reads and barriers but neither
- * unpack weights nor issue matrix instructions, so their launch time is what the kernels' data movement alone takes.
- * Everything such launches write is meaningless; switch it off again before using results. */
-infr_status infr_hip_probe_grouped_loads_only(infr_hip_backend *be, int on);
-
 /* Debug taps used by the parity tests: Op::MoeFfn's routing decision and bucketing of the
  * LAST executed MoeFfn op of `plan` (the reference exposes the same facts through
  * `debug.moe_counts`, crates/infr-cpu/src/lib.rs:3919-3980).  ids/weights are
@@ -302,15 +285,6 @@ infr_status infr_hip_plan_moe_bucketing(infr_hip_backend *be, const infr_hip_pla
  * crates/infr-gguf/src/dequant.rs:11-55): dst f32 buffer receives the decoded prefix of
  * `numel` elements of `src` interpreted as `dtype`. */
 infr_status infr_hip_dequant(infr_hip_backend *be, const infr_hip_buffer *src, int32_t dtype, uint64_t numel, infr_hip_buffer *dst);
-
-/* Measurement aid, no counterpart in the reference: the time a chain of DEPENDENT kernels of given sizes cannot go below
- * on this device.  Stage k is one kernel that reads stage_bytes[k] bytes of `pool` (a window whose position depends on
- * a word the previous stage wrote; windows rotate through the pool, so make it larger than the caches) with every load
- * of a block in flight at once and no arithmetic.  us_per_stage[k]: stage k alone, launched back to back `iters`
- * times; us_per_chain: the stages in order, `iters` times.  Either pointer may be NULL.  Each stage needs 1 KB up to a
- * quarter of the pool.  Allocates a control word and two events for the duration of the call. */
-infr_status infr_hip_probe_dependent_reads(infr_hip_backend *be, const infr_hip_buffer *pool, const uint64_t *stage_bytes,
-                                           uint32_t n_stages, uint32_t iters, double *us_per_stage, double *us_per_chain);
 
 /* One Op::MoeFfn WITHOUT ANY ALLOCATION.  This entry point has no counterpart in the reference; it is for callers
  * that cannot allocate device memory: code under HIP-graph capture, tight serving loops, harnesses that forbid it.

@@ -21,6 +21,7 @@
 #include <vector>
 
 #include "../../include/infr_hip.h"
+#include "../../include/infr_hip_probe.h"
 #include "kernels.h"
 
 namespace {

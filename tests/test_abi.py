@@ -13,6 +13,7 @@ from moe4all_amd import backend as B
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 HEADER = os.path.join(ROOT, "include", "infr_hip.h")
+PROBE_HEADER = os.path.join(ROOT, "include", "infr_hip_probe.h")
 SYNTH_HEADER = os.path.join(ROOT, "include", "infr_synth.h")
 
 
@@ -34,10 +35,12 @@ def test_header_declares_the_backend_trait_surface():
 
 def test_library_exports_every_declared_symbol():
     lib = M.load_library()
-    for s in declared_symbols():
-        assert hasattr(lib, s), f"{s} declared in include/infr_hip.h but not exported"
-    # and the Python mirror binds exactly the declared set
-    assert sorted(B._SIGNATURES) == declared_symbols()
+    boundary, probes = declared_symbols(), declared_symbols(PROBE_HEADER)
+    for s in boundary + probes:
+        assert hasattr(lib, s), f"{s} declared in include/ but not exported"
+    # the boundary header holds no measurement call, and the Python mirror binds exactly the declared set
+    assert not [s for s in boundary if "_probe_" in s or "_prof_" in s]
+    assert sorted(B._SIGNATURES) == sorted(set(boundary + probes))
     synth = declared_symbols(SYNTH_HEADER, "infr_synth_")
     assert len(synth) == 4
     for s in synth:
@@ -50,7 +53,7 @@ def test_struct_layouts_match_the_header(tmp_path):
     prog.write_text(r'''
 #include <stdio.h>
 #include <stddef.h>
-#include "infr_hip.h"
+#include "infr_hip_probe.h"
 int main(void) {
   printf("%zu %zu %zu %zu %zu %zu %zu %zu %zu\n", sizeof(infr_tensor_decl), sizeof(infr_op_moe_ffn), sizeof(infr_op),
          sizeof(infr_graph), sizeof(infr_binding), sizeof(infr_hip_capabilities), sizeof(infr_hip_config),
