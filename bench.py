@@ -136,10 +136,12 @@ def algorithmic_tables(shape, batch, distinct, prefill):
     # the whole single-token op as one launch: the three stages' bytes, each counted once (h and the logits stay on chip
     # or in L2: the hand-over records are not algorithmic traffic)
     alg["moe_layer"] = (shape.router_bytes() + shape.ne * 4 + shape.n_used * (2 * gate_b + down_b) + shape.ne * 4)
+    alg["moe_layer_inorder"] = alg["moe_layer"]
     if shape.shared_ff:
         sh_gate_b = M.backend.bytes_for(shape.gate_dtype, shape.shared_ff * shape.ne)
         sh_down_b = M.backend.bytes_for(shape.down_dtype, shape.ne * shape.shared_ff)
         # the always-on expert as one more slot of the routed kernels
+        alg["moe_layer_shared"] = alg["moe_layer"] + 2 * sh_gate_b + sh_down_b
         alg["moe_route_gate_up_shared"] = alg["moe_route_gate_up"] + 2 * sh_gate_b + batch * shape.shared_ff * 4
         alg["moe_down_combine_shared"] = alg["moe_down_combine"] + sh_down_b + batch * shape.shared_ff * 4
         alg["linear_gate_up_act"] = 2 * sh_gate_b + batch * shape.ne * 4 + batch * shape.shared_ff * 4
@@ -429,6 +431,12 @@ def main():
     ap.add_argument("--no-fusion", action="store_true", help="one launch per op (infr_hip_config.disable_op_fusion)")
     ap.add_argument("--three-launch", action="store_true",
                     help="single-token MoeFfn as three launches (infr_hip_config.disable_single_launch_moe), for comparison")
+    ap.add_argument("--in-order", action="store_true",
+                    help="single-token MoeFfn on the single-launch kernel that runs its stages in order "
+                         "(infr_hip_config.disable_single_launch_guess), for comparison")
+    ap.add_argument("--logits", type=int, default=0, choices=[0, 1, 2],
+                    help="single-launch kernel: 1 = every router logit once for the grid, 2 = once per group of workgroups "
+                         "(infr_hip_config.single_launch_logits), 0 = the built-in choice")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-kernel-timing", action="store_true")
     ap.add_argument("--no-floor", action="store_true", help="skip the dependent-read probe")
@@ -446,7 +454,8 @@ def main():
     shape = shape_of(headline_cfg, args.tokens)
     n_layer = args.layers or shape.n_layer
     batch = args.tokens if prefill else args.batch
-    be = M.Backend(0, disable_op_fusion=args.no_fusion, disable_single_launch_moe=args.three_launch)
+    be = M.Backend(0, disable_op_fusion=args.no_fusion, disable_single_launch_moe=args.three_launch,
+                   disable_single_launch_guess=args.in_order, single_launch_logits=args.logits)
     caps = be.capabilities()
     stack = Stack(be, shape, n_layer, prefill)
     if args.copy_probe_mib:

@@ -213,14 +213,23 @@ typedef struct infr_hip_config {
      * (crates/infr-core/src/fusion.rs:49-52, `enabled`); results are bit-identical either way. */
     uint32_t disable_op_fusion;
     /* Non-zero: a single-token Op::MoeFfn always runs as three launches (logits, routing + gate/up, down + sum).
-     * By default shapes that fit (8 experts per token, Q4_K / Q6_K or Q8_0 banks, hidden size up to 2048, a device
+     * By default shapes that fit (8 experts per token, Q4_K / Q6_K or Q8_0 banks, hidden size 2048 or 4096, a device
      * with 256 compute units) run as ONE launch whose stages hand over inside the kernel; results are bit-identical. */
     uint32_t disable_single_launch_moe;
     /* Polls a workgroup of the single-launch kernel spends on one of its hand-overs before it gives up (the error
      * then surfaces at the next infr_hip_sync / download and the backend falls back to three launches for good).
      * 0 selects the built-in default (32768, some tens of milliseconds); 1 gives up after the first poll. */
     uint32_t single_launch_spin_limit;
-    uint32_t reserved[3];
+    /* Single-launch kernel, router logits: 0 = built-in choice per shape, 1 = every logit is computed by one
+     * workgroup and handed to all (the router is read once), 2 = every group of 32 workgroups computes all logits
+     * for itself (the router is read 8 times, the hand-over stays inside a group).  Same bits either way. */
+    uint32_t single_launch_logits;
+    /* Tests only.  The single-launch kernel requests expert rows for a guessed selection before the exact routing is
+     * known; n > 0 makes every guess leave out the n most likely experts, so the path that loads a missed expert late
+     * runs on every launch.  Results are unaffected. */
+    uint32_t single_launch_guess_skew;
+    /* Non-zero: keep the single-launch kernel whose stages run in order (no guess) for every shape it takes. */
+    uint32_t disable_single_launch_guess;
 } infr_hip_config;
 
 /* Construction of the backend object (reference: VulkanBackend::new / CpuBackend::new,

@@ -40,6 +40,11 @@ infr_status infr_hip_probe_grouped_loads_only(infr_hip_backend *be, int on);
 infr_status infr_hip_probe_dependent_reads(infr_hip_backend *be, const infr_hip_buffer *pool, const uint64_t *stage_bytes,
                                            uint32_t n_stages, uint32_t iters, double *us_per_stage, double *us_per_chain);
 
+/* Measurement / tests, no counterpart in the reference.  The single-launch Op::MoeFfn kernel requests expert rows for a
+ * guessed selection and loads an expert late when the exact routing names one the guess missed; *out receives the
+ * number of such late experts over all launches of this backend so far (waits for the backend's stream). */
+infr_status infr_hip_probe_late_experts(infr_hip_backend *be, uint64_t *out);
+
 #ifdef __cplusplus
 }
 #endif

@@ -179,7 +179,8 @@ class _Caps(C.Structure):
 class _Config(C.Structure):
     _fields_ = [("disable_graph_replay", C.c_uint32), ("moe_batched_min_rows", C.c_uint32),
                 ("disable_op_fusion", C.c_uint32), ("disable_single_launch_moe", C.c_uint32),
-                ("single_launch_spin_limit", C.c_uint32), ("reserved", C.c_uint32 * 3)]
+                ("single_launch_spin_limit", C.c_uint32), ("single_launch_logits", C.c_uint32),
+                ("single_launch_guess_skew", C.c_uint32), ("disable_single_launch_guess", C.c_uint32)]
 
 
 class _MoeFfnStaticArgs(C.Structure):
@@ -227,6 +228,7 @@ _SIGNATURES = {
     "infr_hip_plan_moe_bucketing": ([_V, _V, C.c_uint32, _V, _V, _V], C.c_int),
     "infr_hip_dequant": ([_V, _V, C.c_int32, C.c_uint64, _V], C.c_int),
     "infr_hip_moe_ffn_static": ([_V, C.POINTER(_MoeFfnStaticArgs)], C.c_int),
+    "infr_hip_probe_late_experts": ([_V, C.POINTER(C.c_uint64)], C.c_int),
     "infr_hip_probe_dependent_reads": ([_V, _V, C.POINTER(C.c_uint64), C.c_uint32, C.c_uint32, C.POINTER(C.c_double),
                                         C.POINTER(C.c_double)], C.c_int),
 }
@@ -484,12 +486,15 @@ class Backend:
 
     def __init__(self, device: int = 0, *, disable_graph_replay: bool = False, moe_batched_min_rows: int = 0,
                  disable_op_fusion: bool = False, disable_single_launch_moe: bool = False,
-                 single_launch_spin_limit: int = 0):
+                 single_launch_spin_limit: int = 0, single_launch_logits: int = 0, single_launch_guess_skew: int = 0,
+                 disable_single_launch_guess: bool = False):
         self._h = None
         lib = load_library()
         cfg = _Config(disable_graph_replay=int(disable_graph_replay), moe_batched_min_rows=moe_batched_min_rows,
                       disable_op_fusion=int(disable_op_fusion), disable_single_launch_moe=int(disable_single_launch_moe),
-                      single_launch_spin_limit=single_launch_spin_limit)
+                      single_launch_spin_limit=single_launch_spin_limit, single_launch_logits=single_launch_logits,
+                      single_launch_guess_skew=single_launch_guess_skew,
+                      disable_single_launch_guess=int(disable_single_launch_guess))
         h = _V()
         _check(lib.infr_hip_create(device, C.byref(cfg), C.byref(h)))
         self._h = h.value
@@ -628,6 +633,12 @@ class Backend:
                               dst=dst._h, gate_dtype=int(gate_dtype), up_dtype=int(gate_dtype if up_dtype is None else up_dtype),
                               down_dtype=int(down_dtype), rows=rows, ne=ne, n_expert=n_expert, n_used=n_used, n_ff_exp=n_ff_exp)
         _check(self._lib.infr_hip_moe_ffn_static(self._h, C.byref(a)))
+
+    def late_experts(self) -> int:
+        """infr_hip_probe_late_experts: experts the single-launch kernel's guess missed and loaded late, so far."""
+        n = C.c_uint64()
+        _check(self._lib.infr_hip_probe_late_experts(self._h, C.byref(n)))
+        return int(n.value)
 
     def probe_dependent_reads(self, pool: Buffer, stage_bytes: Sequence[int], iters: int = 200) -> dict:
         """infr_hip_probe_dependent_reads: microseconds of each stage alone and of the whole chain."""

@@ -162,7 +162,7 @@ struct MoeScratch {
     _Float16* hh = nullptr;       // [rows * n_used, nff]
     float* hs = nullptr;          // [rows * n_used]
     float* y = nullptr;           // [rows * n_used, ne]
-    bool single_launch = false;   // one token row, shape taken by the single-launch kernel (k_layer.hip)
+    int single_launch = 0;        // one token row as one launch: 1 = stages in order (k_layer.hip), 2 = guessed selection (k_layer_stream.hip)
 };
 
 struct infr_hip_plan {
@@ -182,7 +182,8 @@ struct infr_hip_plan {
     };
     std::vector<LinearBatch> lin;      // per op (valid for Linear ops)
     _Float16* lin_xh = nullptr;        // shared by all ops of a plan: f16 rows, then their scales
-    char* layer_ws = nullptr;          // workspace of the single-launch MoeFfn kernel, shared by all ops of the plan
+    char* layer_ws = nullptr;          // workspace of the in-order single-launch MoeFfn kernel, shared by all ops of the plan
+    char* stream_ws = nullptr;         // the same for the kernel that guesses the selection (its records are tagged differently)
     int last_moe_op = -1;
     // Launch fusion of the dense SwiGLU FFN the reference emits beside the routed experts
     // (crates/infr-llama/src/runner.rs:8116-8174: Linear gate, Linear up, GatedAct, Linear down, Add).
@@ -294,6 +295,14 @@ void drain_prof(infr_hip_backend* be) {
         be->event_pool.push_back(p.b);
     }
     be->pending.clear();
+}
+
+// Single-launch kernel with a guessed selection: is every router logit computed once for the whole grid (and handed
+// over across the XCDs), or by every group of 32 workgroups for itself (eight reads of the router)?
+int moe_logits_once(const infr_hip_backend* be, const infr_op_moe_ffn& m) {
+    if (be->cfg.single_launch_logits == 1) return 1;
+    if (be->cfg.single_launch_logits == 2) return 0;
+    return m.n_expert > 128 || m.ne > 2048 ? 1 : 0;
 }
 
 // The per-token path of Op::MoeFfn (1 to 31 token rows; the bucketed path takes batches of 16 or more whose pairs fall on few distinct experts) once logits are in rp.logits and gp / rp are filled in:
@@ -1174,13 +1183,15 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
             }
         }
     }
-    // One token row through a MoeFfn that stands alone (no always-on expert folded in): the whole op as one launch
-    // when the shape fits that kernel.  An RmsNorm folded into the logits kernel is unfolded again: it costs one
-    // small launch, the single launch saves two large ones.
-    size_t layer_ws = 0;
+    // One token row through a MoeFfn: the whole op (with an always-on expert folded in, if there is one) as one launch
+    // when the shape fits one of the two single-launch kernels.  An RmsNorm folded into the logits kernel is unfolded
+    // again: it costs one small launch, the single launch saves two large ones.
+    size_t layer_ws = 0, stream_ws = 0;
     if (!be->cfg.disable_single_launch_moe && be->prop.multiProcessorCount >= 256) {
         for (uint32_t oi = 0; oi < g->n_ops; oi++) {
-            if (plan->ops[oi].kind != INFR_OP_MOE_FFN || plan->fuse[oi].kind != infr_hip_plan::kPlain) continue;
+            if (plan->ops[oi].kind != INFR_OP_MOE_FFN) continue;
+            const infr_hip_plan::Fuse kind = plan->fuse[oi].kind;
+            if (kind != infr_hip_plan::kPlain && kind != infr_hip_plan::kMoeShared) continue;
             const infr_op_moe_ffn& m = plan->ops[oi].u.moe_ffn;
             MoeScratch& sc = plan->moe[oi];
             if (sc.rows != 1 || sc.batched || sc.bucketed || c.dt(m.router) != INFR_F32) continue;
@@ -1191,18 +1202,34 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
             probe.g.up_dt = m.fused_gate_up ? probe.g.gate_dt : c.dt(m.up_exps);
             probe.g.down_dt = c.dt(m.down_exps);
             probe.g.n_cu = be->prop.multiProcessorCount;
+            probe.g.weight_before = (int)m.weight_before;
+            probe.g.skip_zero_w = (int)m.has_ep_band;
             probe.g.route.n_expert = (int)m.n_expert; probe.g.route.n_used = (int)m.n_used;
-            probe.g.route.n_groups = (int)m.n_expert_groups;
+            probe.g.route.n_groups = (int)m.n_expert_groups; probe.g.route.n_groups_used = (int)m.n_expert_groups_used;
+            probe.g.route.gating = m.gating;
+            probe.g.route.exp_probs_b = m.exp_probs_b == INFR_NO_TENSOR ? nullptr : (const float*)plan;   // non-null: given
+            probe.g.route.expert_ids = m.expert_ids == INFR_NO_TENSOR ? nullptr : (const int32_t*)plan;
+            probe.g.route.ep_n = m.has_ep_band ? (int)m.ep_n_local : 0;
             probe.router_row_floats = m.ne;
-            if (!infr::moe_layer_fused_supported(probe)) continue;
-            sc.single_launch = true;
-            layer_ws = std::max(layer_ws, infr::moe_layer_workspace_bytes((int)m.ne, (int)m.n_ff_exp, (int)m.n_expert));
+            probe.logits_once = moe_logits_once(be, m);
+            if (kind == infr_hip_plan::kMoeShared) probe.g.sh_gate = probe.g.sh_up = probe.g.sh_down = (const uint8_t*)plan;
+            if (!be->cfg.disable_single_launch_guess && infr::moe_layer_stream_supported(probe)) {
+                sc.single_launch = 2;
+                stream_ws = std::max(stream_ws, infr::moe_layer_stream_workspace_bytes((int)m.ne, (int)m.n_ff_exp, (int)m.n_expert));
+            } else if (kind == infr_hip_plan::kPlain && infr::moe_layer_fused_supported(probe)) {
+                sc.single_launch = 1;
+                layer_ws = std::max(layer_ws, infr::moe_layer_workspace_bytes((int)m.ne, (int)m.n_ff_exp, (int)m.n_expert));
+            } else {
+                continue;
+            }
             if (plan->fuse[oi].norm) {
                 plan->fuse[plan->fuse[oi].norm - 1].kind = infr_hip_plan::kPlain;
                 plan->fuse[oi].norm = 0;
             }
         }
     }
+    const size_t stream_ws_off = arena;
+    arena += round_up(stream_ws, 256);
     const size_t layer_ws_off = arena;
     arena += round_up(layer_ws, 256);
     const size_t zero_off = arena;
@@ -1243,6 +1270,7 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
         }
     }
     plan->layer_ws = layer_ws ? (char*)plan->arena + layer_ws_off : nullptr;
+    plan->stream_ws = stream_ws ? (char*)plan->arena + stream_ws_off : nullptr;
     plan->zero_ids = (int32_t*)((char*)plan->arena + zero_off);   // stays zero: the arena is zero-filled and nothing writes here
     if (plan->arena) infr::launch_fill_zero(be->stream, plan->arena, arena);
     for (uint32_t oi = 0; oi < g->n_ops; oi++) {
@@ -1430,7 +1458,40 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                     gp.addend = (const float*)ptr[other];
                     gp.dst = (float*)ptr[ad.dst];
                 }
-                if (sc.single_launch && plan->layer_ws && !be->single_launch_off.load(std::memory_order_relaxed)) {
+                if (fz.kind == infr_hip_plan::kMoeShared && !sc.batched && !sc.bucketed) {
+                    const infr_hip_plan::FuseOp fg = plan->fuse_head[fz.a];
+                    const infr_op_linear& lu = plan->ops[fg.a].u.linear;
+                    const infr_op_linear& lg = plan->ops[fg.a == fz.a ? fz.a + 1 : fz.a].u.linear;
+                    const infr_op_linear& ld = plan->ops[fz.b].u.linear;
+                    const uint32_t sum_dst = fz.gated ? plan->ops[fz.b + 1].u.moe_shared_expert_add.dst : plan->ops[fz.b + 1].u.add.dst;
+                    if (!(need(lg.weight, "Linear.weight") && need(lu.weight, "Linear.weight") &&
+                          need(ld.weight, "Linear.weight") && (fz.res || need(sum_dst, "Add.dst"))))
+                        return INFR_ERR_BACKEND;
+                    gp.sh_gate = (const uint8_t*)ptr[lg.weight];
+                    gp.sh_up = (const uint8_t*)ptr[lu.weight];
+                    gp.sh_down = (const uint8_t*)ptr[ld.weight];
+                    if (!fz.res) gp.dst = (float*)ptr[sum_dst];
+                    if (fz.gated) {
+                        // the row's gate logit (a Linear with one output row) is launched ahead of the kernel that weighs
+                        // with it, but behind whatever produces the row it reads (an RmsNorm folded into the logits kernel)
+                        const infr_op_linear& lq = plan->ops[oi + 1].u.linear;
+                        if (!(need(lq.x, "Linear.x") && need(lq.weight, "Linear.weight") && need(lq.dst, "Linear.dst")))
+                            return INFR_ERR_BACKEND;
+                        gp.sh_logit = (const float*)ptr[lq.dst];
+                    }
+                }
+                auto launch_gate_logit = [&]() {
+                    if (!gp.sh_logit) return;
+                    const infr_op_linear& lq = plan->ops[oi + 1].u.linear;
+                    int we = 1, wb = 4;
+                    geometry(plan->tensors[lq.weight].dtype, &we, &wb);
+                    const size_t rb = (size_t)(lq.in_f / we) * wb;
+                    Timed t(be, "linear");
+                    infr::launch_linear(s, (const float*)ptr[lq.x], (const uint8_t*)ptr[lq.weight] + (size_t)(lq.w_off / lq.in_f) * rb,
+                                        plan->tensors[lq.weight].dtype, rb, (int)lq.m, (int)lq.in_f, (int)lq.out_f,
+                                        (float*)ptr[lq.dst], n_cu);
+                };
+                if (sc.single_launch && !be->single_launch_off.load(std::memory_order_relaxed)) {
                     infr::MoeLayerParams lp{};
                     lp.g = gp;
                     lp.g.route = rp;
@@ -1438,16 +1499,41 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                     lp.router_row_floats = router_row_bytes / 4;
                     lp.router_x = (const float*)ptr[m.router_x];
                     lp.logits_out = sc.logits;
-                    char* ws = plan->layer_ws;
-                    lp.seq = (uint32_t*)ws;
-                    lp.cnt = (uint32_t*)(ws + 16);
-                    lp.xl = (uint64_t*)(ws + 256);
-                    lp.xh = lp.xl + (size_t)8 * m.n_expert;
-                    lp.ypart = lp.xh + (size_t)8 * m.n_ff_exp;
                     lp.fault = be->fault_dev;
                     lp.spin_limit = be->cfg.single_launch_spin_limit ? (int)be->cfg.single_launch_spin_limit - 1 : 1 << 15;
-                    Timed t(be, "moe_layer");
-                    if (infr::launch_moe_layer_fused(s, lp)) break;   // false: operands the kernel cannot take (alignment)
+                    if (sc.single_launch == 2 && plan->stream_ws) {
+                        char* ws = plan->stream_ws;
+                        lp.seq = (uint32_t*)ws;
+                        lp.cnt = (uint32_t*)(ws + 4);
+                        lp.xa = (uint64_t*)(ws + 256);
+                        lp.xl = lp.xa + (size_t)8 * m.n_expert;
+                        lp.xh = lp.xl + (size_t)8 * m.n_expert;
+                        lp.xs = lp.xh + (size_t)8 * m.n_ff_exp;
+                        lp.ypart = lp.xs + (size_t)m.n_ff_exp;
+                        lp.late = be->fault_dev + 1;
+                        lp.logits_once = moe_logits_once(be, m);
+                        lp.guess_skew = (int)be->cfg.single_launch_guess_skew;
+                        if (infr::moe_layer_stream_supported(lp) &&
+                            (((uintptr_t)lp.router | (uintptr_t)lp.router_x | (uintptr_t)gp.x) & 15) == 0 && (lp.router_row_floats & 3) == 0) {
+                            launch_gate_logit();   // no norm is folded on this path: the row it reads is there
+                            Timed t(be, gp.sh_gate ? "moe_layer_shared" : "moe_layer");
+                            if (infr::launch_moe_layer_stream(s, lp)) break;
+                            return fail(INFR_ERR_BACKEND, "MoeFfn: the single-launch kernel refused a shape it had accepted");
+                        }
+                    } else if (sc.single_launch == 1 && plan->layer_ws) {
+                        char* ws = plan->layer_ws;
+                        lp.seq = (uint32_t*)ws;
+                        lp.cnt = (uint32_t*)(ws + 16);
+                        lp.xl = (uint64_t*)(ws + 256);
+                        lp.xh = lp.xl + (size_t)8 * m.n_expert;
+                        lp.ypart = lp.xh + (size_t)8 * m.n_ff_exp;
+                        // asked first, so that no timing events are queued for a launch that does not happen
+                        if ((((uintptr_t)lp.router | (uintptr_t)lp.router_x | (uintptr_t)gp.x) & 15) == 0 && (lp.router_row_floats & 3) == 0) {
+                            Timed t(be, "moe_layer_inorder");
+                            if (infr::launch_moe_layer_fused(s, lp)) break;
+                            return fail(INFR_ERR_BACKEND, "MoeFfn: the single-launch kernel refused a shape it had accepted");
+                        }
+                    }
                 }
                 bool normed = false;
                 if (fz.norm) {
@@ -1587,36 +1673,9 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                     }
                     break;
                 }
-                if (fz.kind == infr_hip_plan::kMoeShared) {
-                    const infr_hip_plan::FuseOp fg = plan->fuse_head[fz.a];
-                    const infr_op_linear& lu = plan->ops[fg.a].u.linear;
-                    const infr_op_linear& lg = plan->ops[fg.a == fz.a ? fz.a + 1 : fz.a].u.linear;
-                    const infr_op_linear& ld = plan->ops[fz.b].u.linear;
-                    const uint32_t sum_dst = fz.gated ? plan->ops[fz.b + 1].u.moe_shared_expert_add.dst : plan->ops[fz.b + 1].u.add.dst;
-                    if (!(need(lg.weight, "Linear.weight") && need(lu.weight, "Linear.weight") &&
-                          need(ld.weight, "Linear.weight") && (fz.res || need(sum_dst, "Add.dst"))))
-                        return INFR_ERR_BACKEND;
-                    gp.sh_gate = (const uint8_t*)ptr[lg.weight];
-                    gp.sh_up = (const uint8_t*)ptr[lu.weight];
-                    gp.sh_down = (const uint8_t*)ptr[ld.weight];
-                    if (!fz.res) gp.dst = (float*)ptr[sum_dst];
-                    if (fz.gated) {
-                        // the row's gate logit (a Linear with one output row), ahead of the kernel that weighs with it
-                        const infr_op_linear& lq = plan->ops[oi + 1].u.linear;
-                        if (!(need(lq.x, "Linear.x") && need(lq.weight, "Linear.weight") && need(lq.dst, "Linear.dst")))
-                            return INFR_ERR_BACKEND;
-                        int we = 1, wb = 4;
-                        geometry(plan->tensors[lq.weight].dtype, &we, &wb);
-                        const size_t rb = (size_t)(lq.in_f / we) * wb;
-                        Timed t(be, "linear");
-                        infr::launch_linear(s, (const float*)ptr[lq.x], (const uint8_t*)ptr[lq.weight] + (size_t)(lq.w_off / lq.in_f) * rb,
-                                            plan->tensors[lq.weight].dtype, rb, (int)lq.m, (int)lq.in_f, (int)lq.out_f,
-                                            (float*)ptr[lq.dst], n_cu);
-                        gp.sh_logit = (const float*)ptr[lq.dst];
-                    }
-                }
                 gp.route = rp;
                 gp.y = sc.y;
+                launch_gate_logit();
                 moe_per_token(be, s, gp, rp, rows, m.n_expert, true);
                 break;
             }
@@ -1842,6 +1901,15 @@ extern "C" infr_status infr_hip_probe_dependent_reads(infr_hip_backend* be, cons
 } catch (...) { return guard_fail("infr_hip_probe_dependent_reads"); }
 
 // ============================================================================ taps
+extern "C" infr_status infr_hip_probe_late_experts(infr_hip_backend* be, uint64_t* out) try {
+    if (!ok_backend(be) || !out) return fail(INFR_ERR_INVALID, "probe: bad handle");
+    std::lock_guard<std::mutex> lk(be->mu);
+    HIP_TRY(hipSetDevice(be->device));
+    HIP_TRY(hipStreamSynchronize(be->stream));
+    *out = be->fault_host ? ((volatile uint32_t*)be->fault_host)[1] : 0;
+    return INFR_OK;
+} catch (...) { return guard_fail("infr_hip_probe_late_experts"); }
+
 extern "C" infr_status infr_hip_probe_grouped_loads_only(infr_hip_backend* be, int on) try {
     if (!ok_backend(be)) return fail(INFR_ERR_INVALID, "probe: bad handle");
     be->probe_grouped_loads_only.store(on != 0);

@@ -1,0 +1,734 @@
+// Single-token Op::MoeFfn as ONE launch in which the expert weights are requested before the routing is known.
+//
+// What the reference fixes for this op is the routing (ids in rank order, routing weights, bit for bit:
+// crates/infr-cpu/src/lib.rs:3684-3716 for the logits' summation order, :3746-3861 for gating, selection and
+// renormalisation) and the rank order of the final sum (:4290-4302).  The expert stages need much less: the SET of
+// selected experts.  This kernel therefore computes every router logit twice.  A fast estimate (each thread multiplies
+// the eight elements it loaded, a tree adds them up) gives a guess of the selected set a few hundred nanoseconds
+// after the operands have arrived, and the expert rows of the guessed set are requested at once.  The exact logits
+// (eight 256- or 512-step chains of dependent multiply-adds per logit), the exact routing routine and the check of the
+// guess run on one wavefront beside the stream of weights.  Only the exact results are published, decide the ranks and
+// weigh the sum.  When the guess misses an expert of the exact set (logits that differ by less than the estimate's
+// rounding), the workgroups that hold an expert outside the set compute the missing one late; a record's tag carries
+// the expert it belongs to, so a consumer can never take the product of a wrong guess for the one it waits for.
+//
+// Work split.  256 workgroups of 8 wavefronts in 8 groups of 32 (group = blockIdx & 7; consecutive workgroups go to
+// consecutive XCDs, so a group shares an L2).  Group g computes one expert of the set: workgroup m of the group the
+// features [m * nff / 32, +nff / 32) of gate and up, then the output rows [m * ne / 32, +ne / 32) of down.  An
+// always-on expert folded into the op is spread over all 256 workgroups (features [b * nff / 256, ..), rows
+// [b * ne / 256, ..)); it needs no routing, so its rows are the first bytes requested.  Wavefront 0 is the router
+// (exact chains, exact routing, check of the guess), wavefronts 1..7 stream weights: each keeps a ring of items
+// (a gate row and an up row, or a group of down rows) in flight, finishes the oldest and requests the one D places
+// ahead.  The first down rows are requested before the group's activations have been handed over.
+//
+// Hand-over between workgroups: 64-bit records {value bits, tag} written and polled with agent-scope relaxed atomics,
+// no fence anywhere; the tag is the launch's sequence number (kept in device memory, advanced by the workgroup that
+// leaves last) and, for the activations, the expert id.  Every wait is bounded: after `spin_limit` polls a workgroup
+// raises the host-visible fault word and skips to the end; its peers run into their own limits, so the grid drains.
+// Inside a workgroup the wavefronts hand over through LDS flags; a flag is always set, also on the failure path.
+//
+// The inner products, the activation, the routing routine and the order of the final sum are those of the
+// three-launch kernels (k_gemv.hip): same bits.
+#include "device_common.h"
+#include "kernels.h"
+#include "route.h"
+#include "gemv_fmt.h"
+
+#include <type_traits>
+
+namespace infr {
+
+namespace {
+
+// Time stamps of every workgroup for a measurement build (-DINFR_LAYER_TRACE with a buffer in g.y); compiled out otherwise.
+#ifdef INFR_LAYER_TRACE
+#define STAMP(i)                                                                                                   \
+    do {                                                                                                           \
+        if ((threadIdx.x & 63) == 0 && q.g.y) reinterpret_cast<long long*>(q.g.y)[blockIdx.x * 32 + (i)] = wall_clock64(); \
+    } while (0)
+#else
+#define STAMP(i) do { } while (0)
+#endif
+
+constexpr int kGroups = 8, kPerGroup = 32, kBlocks = kGroups * kPerGroup;
+constexpr int kThreads = 512, kWaves = 8, kSW = 7;   // wavefronts 1..7 stream
+constexpr uint32_t kCodePlain = 0x1FFu;              // tag code of records that belong to no expert
+
+__device__ __forceinline__ uint64_t rec_load(const uint64_t* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void rec_store(uint64_t* p, float v, uint32_t tag) {
+    __hip_atomic_store(p, (uint64_t)__float_as_uint(v) | ((uint64_t)tag << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Wave-wide: gathers rec[0 .. n) (n a multiple of 64, n <= 64 N) into out[] once all carry `tag`.  Every poll issues
+// all of a lane's loads before it looks at any of them, so a poll costs one memory round trip.  False: spin limit.
+template <int N>
+__device__ __forceinline__ bool gather_records(const uint64_t* rec, int n, uint32_t tag, float* out, int lane, int spin_limit) {
+    uint64_t r[N];
+    const int ns = n >> 6;
+    for (int spin = 0;; spin++) {
+#pragma unroll
+        for (int s = 0; s < N; s++) r[s] = s < ns ? rec_load(rec + s * kWave + lane) : ((uint64_t)tag << 32);
+        bool ok = true;
+#pragma unroll
+        for (int s = 0; s < N; s++) ok = ok && (uint32_t)(r[s] >> 32) == tag;
+        if (__all(ok)) break;
+        if (spin >= spin_limit) return false;
+    }
+#pragma unroll
+    for (int s = 0; s < N; s++)
+        if (s < ns) out[s * kWave + lane] = __uint_as_float((uint32_t)r[s]);
+    return true;
+}
+
+// Hand-over between the wavefronts of a workgroup through a word of LDS.  A wavefront's LDS operations complete in
+// order, so data written before the flag is visible to whoever has read the flag.
+__device__ __forceinline__ void lds_flag_set(volatile int* f, int v) {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    *f = v;
+}
+__device__ __forceinline__ int lds_flag_wait(volatile int* f) {
+    int v;
+    while ((v = __builtin_amdgcn_readfirstlane(*f)) == 0) __builtin_amdgcn_s_sleep(1);
+    asm volatile("" ::: "memory");
+    return v;
+}
+
+// Wave-wide maximum as a scalar: DPP steps inside the rows of 16 lanes, then row_bcast:15 into rows 1 and 3 and
+// row_bcast:31 into rows 2 and 3, after which the last lane holds the maximum.
+__device__ __forceinline__ uint32_t wave_max_scalar(uint32_t v) {
+    v = max(v, dpp_u<kDppXor1>(v));
+    v = max(v, dpp_u<kDppXor2>(v));
+    v = max(v, dpp_u<kDppHalfMirror>(v));
+    v = max(v, dpp_u<kDppMirror>(v));
+    v = max(v, (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, 0x142, 0xA, 0xF, false));
+    v = max(v, (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, 0x143, 0xC, 0xF, false));
+    return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
+}
+
+// The guess: the n_sel indices with the largest estimates, into out[] (any fixed rule will do: every workgroup runs
+// this on the same values, and a wrong guess only costs time).  Keys are made unique by putting 255 - index into the
+// low byte of the order-preserving key (n <= 256), so a round is one wave-wide maximum whose low byte names the
+// winner: estimates that agree in all but their last 8 mantissa bits are ranked by index, like exact ties.  Every lane
+// keeps its NS keys sorted, so a round only looks at heads.  skew > 0 (tests only) leaves the `skew` largest out, so
+// the guess is wrong on purpose.
+template <int NS>
+__device__ __forceinline__ void guess_set(const float* vals, int n_sel, int skew, int lane, int32_t* out) {
+    uint32_t key[NS];
+#pragma unroll
+    for (int s = 0; s < NS; s++) {
+        const int i = s * kWave + lane;
+        key[s] = (order_key(vals[i]) & ~0xFFu) | (uint32_t)(255 - i);
+    }
+    auto order = [&](int a, int b) {
+        const uint32_t hi = max(key[a], key[b]), lo = min(key[a], key[b]);
+        key[a] = hi;
+        key[b] = lo;
+    };
+    if (NS == 2) order(0, 1);
+    if (NS == 4) { order(0, 1); order(2, 3); order(0, 2); order(1, 3); order(1, 2); }
+    static_assert(NS == 1 || NS == 2 || NS == 4, "sorting network");
+    for (int k = 0; k < n_sel + skew; k++) {
+        const uint32_t mx = wave_max_scalar(key[0]);
+        if (k >= skew && lane == 0) out[k - skew] = 255 - (int)(mx & 0xFFu);
+        const bool win = key[0] == mx;
+#pragma unroll
+        for (int s = 0; s + 1 < NS; s++) key[s] = win ? key[s + 1] : key[s];
+        key[NS - 1] = win ? 0u : key[NS - 1];
+    }
+}
+
+// A ring of D items in flight: `issue(slot, j)` requests item j into ring slot `slot`, `finish(slot, j)` consumes it.
+// The first D items have been requested by the caller (ring_prime); items past `cn` are never finished.
+template <int D, class Issue>
+__device__ __forceinline__ void ring_prime(Issue issue) {
+#pragma unroll
+    for (int d = 0; d < D; d++) issue(d, d);
+}
+template <int D, class Issue, class Finish>
+__device__ __forceinline__ void ring_drain(int cn, Issue issue, Finish finish) {
+    const int refills = cn - D;   // steps that still have an item to request
+    int j0 = 0;
+    for (; j0 + D <= refills; j0 += D) {
+#pragma unroll
+        for (int d = 0; d < D; d++) {
+            finish(d, j0 + d);
+            issue(d, j0 + d + D);
+        }
+    }
+#pragma unroll
+    for (int d = 0; d < D; d++) {
+        if (j0 + d >= cn) break;
+        finish(d, j0 + d);
+        if (j0 + d < refills) issue(d, j0 + d + D);
+    }
+    j0 += D;
+#pragma unroll
+    for (int d = 0; d < D; d++) {
+        if (j0 + d >= cn) break;
+        finish(d, j0 + d);
+    }
+}
+
+__device__ __forceinline__ float dot8(const float4& a0, const float4& a1, const float4& b0, const float4& b1) {
+    float s = a0.x * b0.x;
+    s = fmaf(a0.y, b0.y, s);
+    s = fmaf(a0.z, b0.z, s);
+    s = fmaf(a0.w, b0.w, s);
+    s = fmaf(a1.x, b1.x, s);
+    s = fmaf(a1.y, b1.y, s);
+    s = fmaf(a1.z, b1.z, s);
+    return fmaf(a1.w, b1.w, s);
+}
+
+}  // namespace
+
+// FG / FD: formats of the gate/up and down banks; DG / DD: ring depths (items in flight per streaming wavefront);
+// EPT: router rows a thread holds while staging (rows per workgroup / (512 / (ne / 8))); NSP: n_expert / 64.
+template <class FG, class FD, int DG, int DD, int EPT, int NSP>
+__global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
+    extern __shared__ __attribute__((aligned(16))) uint32_t dyn_lds[];
+    __shared__ uint64_t s_tab[32];
+    __shared__ int32_t s_ids[64];
+    __shared__ float s_w[64];
+    __shared__ float s_g[kWaves][64], s_u[kWaves][64];
+    __shared__ float s_part[kWaves][8];
+    __shared__ int32_t s_spec[kGroups], s_final[kGroups], s_gor[kGroups];
+    __shared__ float s_ysh[64];
+    __shared__ int s_f_spec, s_f_route, s_f_h, s_f_hs, s_fault, s_cells_done;
+    __shared__ uint32_t s_seq;
+    const MoeGemvParams& p = q.g;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int b = blockIdx.x, g = b & (kGroups - 1), m = b >> 3;
+    const int ne = p.ne, nff = p.nff, n_expert = p.route.n_expert;
+    const bool shared = p.sh_gate != nullptr;
+
+    // who computes which router logits: every group all of them (epb = n_expert / 32 rows per workgroup, published to
+    // the group), or every logit once for the grid (epb rows per workgroup while they last, published to everyone)
+    const int epb = q.epb;
+    const int area = q.logits_once ? 0 : g;
+    const int row0 = (q.logits_once ? b : m) * epb;
+    const bool has_rows = row0 < n_expert;
+
+    // LDS: [cells of x][chain operands, transposed][estimates][logits][routing scratch][h][cells of h][h, cells: always-on]
+    const int oct_n = ne >> 3;                 // octets of a row: 256 or 512
+    const int jstride = oct_n + 4;
+    const int hsel = tid / oct_n, o = tid - hsel * oct_n;   // replica (0 or 1 when ne = 2048) and octet of this thread
+    const int H = kThreads / oct_n;
+    uint32_t* cells = dyn_lds;
+    float* wst = reinterpret_cast<float*>(cells + (size_t)(ne >> 5) * kCellDwords);
+    float* xst = wst + (size_t)epb * 8 * jstride;
+    float* s_alog = xst + 8 * jstride;
+    float* s_logits = s_alog + n_expert;
+    float* route_scratch = s_logits + n_expert;
+    float* s_h = route_scratch + ((route_scratch_floats(n_expert, p.route.n_groups) + 3) & ~(size_t)3);
+    uint32_t* hcells = reinterpret_cast<uint32_t*>(s_h + nff);
+    float* s_hs = reinterpret_cast<float*>(hcells + (size_t)(nff >> 5) * kCellDwords);
+    uint32_t* hscells = reinterpret_cast<uint32_t*>(s_hs + nff);
+
+    if (tid < 32) s_tab[tid] = kExp2Table[tid];
+    if (tid == 0) {
+        s_f_spec = s_f_route = s_f_h = s_f_hs = s_fault = s_cells_done = 0;
+        s_seq = __hip_atomic_load(q.seq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;   // one load per workgroup
+    }
+    if (wave == 0) STAMP(0);
+
+    // ---- A: operands.  Thread (replica hsel, octet o) holds elements [8 o, 8 o + 8) of the routing row, of the token
+    // row and of the router rows hsel, hsel + H, ...  The token row becomes fixed-point cells later, by the threads
+    // of the last replica (with two replicas that keeps the router's and the guessing wavefront out of it).
+    const bool converts = hsel == H - 1;
+    float4 cx0, cx1;
+    {
+        const float4* rx4 = reinterpret_cast<const float4*>(q.router_x);
+        const float4 rx0 = rx4[2 * o], rx1 = rx4[2 * o + 1];
+        const float4* px4 = reinterpret_cast<const float4*>(p.x);
+        cx0 = px4[2 * o];
+        cx1 = px4[2 * o + 1];
+        float4 w0[EPT], w1[EPT];
+#pragma unroll
+        for (int i = 0; i < EPT; i++) {
+            const int el = hsel + H * i;
+            const bool on = has_rows && el < epb;
+            const float4* row = reinterpret_cast<const float4*>(q.router + (size_t)(on ? row0 + el : 0) * q.router_row_floats);
+            w0[i] = row[2 * o];
+            w1[i] = row[2 * o + 1];
+        }
+        // the estimate's share of this thread, summed over the wavefront
+#pragma unroll
+        for (int i = 0; i < EPT; i++) {
+            const float part = wave_sum(dot8(w0[i], w1[i], rx0, rx1));
+            if (lane == 0) s_part[wave][i] = part;
+        }
+        // chain operands: element 8 o + t belongs to chain t, position o
+        if (hsel == 0) {
+            const float xv[8] = {rx0.x, rx0.y, rx0.z, rx0.w, rx1.x, rx1.y, rx1.z, rx1.w};
+#pragma unroll
+            for (int t = 0; t < 8; t++) xst[t * jstride + o] = xv[t];
+        }
+#pragma unroll
+        for (int i = 0; i < EPT; i++) {
+            const int el = hsel + H * i;
+            if (el < epb) {
+                const float wv[8] = {w0[i].x, w0[i].y, w0[i].z, w0[i].w, w1[i].x, w1[i].y, w1[i].z, w1[i].w};
+#pragma unroll
+                for (int t = 0; t < 8; t++) wst[(el * 8 + t) * jstride + o] = wv[t];
+            }
+        }
+    }
+    __syncthreads();
+    const uint32_t seq_tag = (s_seq & 0x7FFFFFu) << 9;
+    if (wave == 0) STAMP(1);
+    const uint32_t tag = seq_tag | kCodePlain;
+    const int waves_per_replica = oct_n >> 6;
+    if (wave == 1 && has_rows && lane < epb) {
+        // the estimate of logit row0 + lane: the shares of the wavefronts that held that row, in a fixed order
+        const int hs = lane % H, i = lane / H;
+        float a = 0.0f;
+        for (int w = hs * waves_per_replica; w < (hs + 1) * waves_per_replica; w++) a += s_part[w][i];
+        rec_store(q.xa + (size_t)area * n_expert + row0 + lane, a, tag);
+    }
+    // the token row as fixed-point cells, one set for the workgroup; the guessing wavefront takes its share after the guess
+    const int n_conv_waves = oct_n >> 6;
+    auto convert_share = [&]() {
+        if (!converts) return;   // whole wavefronts
+        octet_to_cell<FG::kGroup, FG::kSigned>(cx0, cx1, o, cells);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if (lane == 0) __hip_atomic_fetch_add(&s_cells_done, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    };
+    auto wait_cells = [&]() {
+        while (__builtin_amdgcn_readfirstlane(*(volatile int*)&s_cells_done) < n_conv_waves) __builtin_amdgcn_s_sleep(1);
+        asm volatile("" ::: "memory");
+    };
+    if (wave != 1) convert_share();
+    if (wave == 0) STAMP(2);
+
+    const int spin_limit = q.spin_limit;
+    if (wave == 0) {
+        // ================================================================ the router: exact logits, exact routing
+        bool ok = true;
+        {
+            const int e = lane >> 3, j = lane & 7;
+            const bool live = has_rows && e < epb;
+            float acc = 0.0f;
+            if (live) {
+                // the reference's order: 8 chains over i = j (mod 8), summed 0..7 (crates/infr-cpu/src/kernels.rs:6568-6583)
+                const float4* wp = reinterpret_cast<const float4*>(wst + (e * 8 + j) * jstride);
+                const float4* xp = reinterpret_cast<const float4*>(xst + j * jstride);
+                const int n4 = oct_n >> 2;   // a multiple of 8
+#pragma unroll 1
+                for (int c = 0; c < n4; c += 8) {
+                    float4 a[8], bb[8];
+#pragma unroll
+                    for (int k = 0; k < 8; k++) { a[k] = wp[c + k]; bb[k] = xp[c + k]; }
+#pragma unroll
+                    for (int k = 0; k < 8; k++) {
+                        acc = __fmaf_rn(a[k].x, bb[k].x, acc);
+                        acc = __fmaf_rn(a[k].y, bb[k].y, acc);
+                        acc = __fmaf_rn(a[k].z, bb[k].z, acc);
+                        acc = __fmaf_rn(a[k].w, bb[k].w, acc);
+                    }
+                }
+            }
+            float s = 0.0f;
+#pragma unroll
+            for (int jj = 0; jj < 8; jj++) s = __fadd_rn(s, __shfl(acc, (lane & ~7) + jj, kWave));
+            if (live && j == 0) {
+                rec_store(q.xl + (size_t)area * n_expert + row0 + e, s, tag);
+                if ((q.logits_once || g == 0) && q.logits_out) q.logits_out[row0 + e] = s;
+            }
+        }
+        STAMP(16);
+        ok = gather_records<NSP>(q.xl + (size_t)area * n_expert, n_expert, tag, s_logits, lane, spin_limit);
+        STAMP(17);
+        if (ok) {
+            __builtin_amdgcn_wave_barrier();
+            RouteParams rp = p.route;
+            rp.logits = s_logits;
+            route_row_any(rp, 0, lane, route_scratch, s_tab, s_ids, s_w, b == 0);
+            STAMP(18);
+            __builtin_amdgcn_wave_barrier();
+            // which group holds which rank; groups whose guess is outside the exact set take the missed experts
+            const int guess_state = lds_flag_wait(&s_f_spec);
+            if (guess_state != 1) ok = false;
+            if (ok) {
+                // lane k < 8 owns rank k: the group whose guess is that expert; ranks the guess missed take the groups
+                // whose guess is outside the exact set, both in ascending order
+                const bool rank = lane < kGroups;
+                const int id = rank ? s_ids[lane] : -1;
+                int gk = -1;
+#pragma unroll
+                for (int gg = 0; gg < kGroups; gg++)
+                    if (s_spec[gg] == id) gk = gg;
+                uint32_t used = 0;
+#pragma unroll
+                for (int gg = 0; gg < kGroups; gg++) used |= (__ballot(rank && gk == gg) ? 1u : 0u) << gg;
+                const uint32_t missed = (uint32_t)__ballot(rank && gk < 0) & 0xFFu;
+                if (rank && gk < 0) {
+                    const int j = __builtin_popcount(missed & ((1u << lane) - 1u));
+                    int seen = 0;
+#pragma unroll
+                    for (int gg = 0; gg < kGroups; gg++) {
+                        const bool free_g = !((used >> gg) & 1u);
+                        if (free_g && seen == j) gk = gg;
+                        seen += free_g ? 1 : 0;
+                    }
+                }
+                if (rank) {
+                    s_gor[lane] = gk;
+                    s_final[gk] = id;
+                }
+                if (b == 0 && missed && lane == 0 && q.late)
+                    __hip_atomic_fetch_add(q.late, (uint32_t)__builtin_popcount(missed), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            }
+        }
+        if (!ok && lane == 0) {
+            s_fault = 1;
+            __hip_atomic_store(q.fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+        }
+        lds_flag_set(&s_f_route, ok ? 1 : 2);
+        STAMP(19);
+    } else {
+        // ================================================================ the streaming wavefronts
+        const int sw = wave - 1;
+        const int nblk_g = ne / FG::kBlockElems, nblk_d = nff / FD::kBlockElems;
+        const size_t rb_g = (size_t)nblk_g * FG::kBlockBytes, rb_d = (size_t)nblk_d * FD::kBlockBytes;
+        const Place<FG> pg(nblk_g, lane);
+        const Place<FD> pd(nblk_d, lane);
+        struct GuItem { typename FG::Raw g, u; };
+        bool alive = true;
+
+        // the always-on expert's gate/up share of this workgroup: at most one item per wavefront, requested first
+        const int sfpb = nff / kBlocks, sf0 = b * sfpb;
+        const int n_si = shared ? (sfpb + pg.rw_count - 1) / pg.rw_count : 0;
+        const bool my_si = sw < n_si;
+        GuItem sh_item;
+        if (my_si && wave != 1) {
+            const int f = sf0 + min(sw * pg.rw_count + pg.rw, sfpb - 1);
+            sh_item.g = load_row<FG>(pg, p.sh_gate + (size_t)f * rb_g);
+            sh_item.u = load_row<FG>(pg, p.sh_up + (size_t)f * rb_g);
+        }
+        if (wave == 1) {
+            // the guess of the selected set, from the estimates
+            bool ok = gather_records<NSP>(q.xa + (size_t)area * n_expert, n_expert, tag, s_alog, lane, spin_limit);
+            STAMP(3);
+            if (ok) {
+                __builtin_amdgcn_wave_barrier();
+                guess_set<NSP>(s_alog, kGroups, q.guess_skew, lane, s_spec);
+            } else if (lane == 0) {
+                s_fault = 1;
+                __hip_atomic_store(q.fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            }
+            lds_flag_set(&s_f_spec, ok ? 1 : 2);
+            STAMP(4);
+            alive = ok;
+            convert_share();
+            if (my_si) {
+                const int f = sf0 + min(sw * pg.rw_count + pg.rw, sfpb - 1);
+                sh_item.g = load_row<FG>(pg, p.sh_gate + (size_t)f * rb_g);
+                sh_item.u = load_row<FG>(pg, p.sh_up + (size_t)f * rb_g);
+            }
+        } else {
+            alive = lds_flag_wait(&s_f_spec) == 1;
+        }
+
+        // gate/up items of this wavefront: item j covers features (j * kSW + sw) * rw_count + rw of the workgroup's slice
+        const int fpb = nff / kPerGroup, f0 = m * fpb;
+        const int n_gi = (fpb + pg.rw_count - 1) / pg.rw_count;
+        const int my_gi = n_gi > sw ? (n_gi - sw + kSW - 1) / kSW : 0;
+        // down items: item j covers output rows (j * kSW + sw) * rw_count + rw of the workgroup's slice; behind them the
+        // always-on expert's rows [b * ne / 256, ..) of this workgroup
+        const int R = ne / kPerGroup;
+        const int n_di = (R + pd.rw_count - 1) / pd.rw_count;
+        const int my_di = n_di > sw ? (n_di - sw + kSW - 1) / kSW : 0;
+        const int SR = ne / kBlocks;
+        const int n_sdi = shared ? (SR + pd.rw_count - 1) / pd.rw_count : 0;
+        const int my_sdi = n_sdi > sw ? (n_sdi - sw + kSW - 1) / kSW : 0;
+
+        typename FD::Raw dring[DD];
+        int e_cur = alive ? s_spec[g] : 0;
+        const uint8_t* dbank = nullptr;
+        auto dn_issue = [&](int slot, int j) {
+            const bool routed = j < my_di || !shared;   // items past the end re-read a last row
+            const int jj = routed ? j : j - my_di;
+            const int lim = routed ? R : SR;
+            const int orow = min((jj * kSW + sw) * pd.rw_count + pd.rw, lim - 1);
+            const uint8_t* base = routed ? dbank + (size_t)(m * R + orow) * rb_d : p.sh_down + (size_t)(b * SR + orow) * rb_d;
+            dring[slot] = load_row<FD>(pd, base);
+        };
+        if (alive) {
+            for (int attempt = 0;; attempt++) {
+                const uint8_t* gb = p.gate + (size_t)e_cur * p.gate_stride + (size_t)f0 * rb_g;
+                const uint8_t* ub = p.up + (size_t)e_cur * p.up_stride + (size_t)f0 * rb_g;
+                dbank = p.down + (size_t)e_cur * p.down_stride;
+                GuItem gring[DG];
+                typename FG::X x;   // fetched again on a second pass: not kept alive across the hand-over
+                auto gu_issue = [&](int slot, int j) {
+                    const int f = min((j * kSW + sw) * pg.rw_count + pg.rw, fpb - 1);
+                    gring[slot].g = load_row<FG>(pg, gb + (size_t)f * rb_g);
+                    gring[slot].u = load_row<FG>(pg, ub + (size_t)f * rb_g);
+                };
+                auto gu_finish = [&](int slot, int j) {
+                    const float gs = row_sum<FG>(FG::dot(gring[slot].g, pg.sub, x), pg, nblk_g);
+                    const float us = row_sum<FG>(FG::dot(gring[slot].u, pg.sub, x), pg, nblk_g);
+                    if (pg.writer()) {
+                        s_g[wave][j * pg.rw_count + pg.rw] = gs;
+                        s_u[wave][j * pg.rw_count + pg.rw] = us;
+                    }
+                };
+                ring_prime<DG>(gu_issue);
+                if (q.early_down) ring_prime<DD>(dn_issue);
+                if (wave == 3) STAMP(5);
+                if (wave == 1) STAMP(20);
+                if (attempt == 0) wait_cells();
+                FG::fetch_x(x, cells, pg.blk, pg.sub);
+                if (attempt == 0 && my_si) {
+                    // the always-on expert's item, requested before the guess was known
+                    const float gs = row_sum<FG>(FG::dot(sh_item.g, pg.sub, x), pg, nblk_g);
+                    const float us = row_sum<FG>(FG::dot(sh_item.u, pg.sub, x), pg, nblk_g);
+                    const int fi = sw * pg.rw_count + pg.rw;
+                    if (pg.writer() && fi < sfpb)
+                        rec_store(q.xs + sf0 + fi, gated_act_fn(p.act, p.has_clamp, p.clamp, gs, us, s_tab), tag);
+                }
+                ring_drain<DG>(my_gi, gu_issue, gu_finish);
+                if (wave == 3) STAMP(6);
+                if (!q.early_down) ring_prime<DD>(dn_issue);
+                __builtin_amdgcn_wave_barrier();
+                if (lane < my_gi * pg.rw_count) {
+                    const int j = lane / pg.rw_count, rw = lane - j * pg.rw_count;
+                    const int fi = (j * kSW + sw) * pg.rw_count + rw;
+                    if (fi < fpb)
+                        rec_store(q.xh + (size_t)g * nff + f0 + fi,
+                                  gated_act_fn(p.act, p.has_clamp, p.clamp, s_g[wave][lane], s_u[wave][lane], s_tab),
+                                  seq_tag | (uint32_t)e_cur);
+                }
+                __builtin_amdgcn_wave_barrier();
+                if (wave == 3) STAMP(7);
+                if (wave == 1) STAMP(21);
+                if (wave == 7) STAMP(22);
+                if (lds_flag_wait(&s_f_route) != 1) {
+                    alive = false;
+                    break;
+                }
+                if (wave == 3) STAMP(8);
+                const int e_fin = s_final[g];
+                if (e_fin == e_cur) break;
+                e_cur = e_fin;   // the guess missed this group's expert: once more with the right one
+            }
+        }
+        // ---- hand-over of the group's activations: wavefront 1 gathers and converts, the others wait for its flag;
+        // wavefront 2 gathers the always-on expert's meanwhile
+        if (wave == 1) {
+            bool ok = alive;
+            if (ok) ok = gather_records<24>(q.xh + (size_t)g * nff, nff, seq_tag | (uint32_t)e_cur, s_h, lane, spin_limit);
+            STAMP(9);
+            if (ok) {
+                __builtin_amdgcn_wave_barrier();
+                for (int oct = lane; oct * 8 < nff; oct += kWave) {
+                    const float4 lo = *reinterpret_cast<const float4*>(s_h + 8 * oct), hi = *reinterpret_cast<const float4*>(s_h + 8 * oct + 4);
+                    octet_to_cell<FD::kGroup, FD::kSigned>(lo, hi, oct, hcells);
+                }
+            } else if (alive && lane == 0) {
+                s_fault = 1;
+                __hip_atomic_store(q.fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            }
+            lds_flag_set(&s_f_h, ok ? 1 : 2);
+            STAMP(10);
+            alive = ok;
+        } else if (wave == 2 && shared) {
+            bool ok = alive;
+            if (ok) ok = gather_records<24>(q.xs, nff, tag, s_hs, lane, spin_limit);
+            if (ok) {
+                __builtin_amdgcn_wave_barrier();
+                for (int oct = lane; oct * 8 < nff; oct += kWave) {
+                    const float4 lo = *reinterpret_cast<const float4*>(s_hs + 8 * oct), hi = *reinterpret_cast<const float4*>(s_hs + 8 * oct + 4);
+                    octet_to_cell<FD::kGroup, FD::kSigned>(lo, hi, oct, hscells);
+                }
+            } else if (alive && lane == 0) {
+                s_fault = 1;
+                __hip_atomic_store(q.fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            }
+            lds_flag_set(&s_f_hs, ok ? 1 : 2);
+            alive = ok;
+        }
+        if (wave != 1 && lds_flag_wait(&s_f_h) != 1) alive = false;
+        if (alive) {
+            // ---- down: rows of the group's expert, then of the always-on expert
+            typename FD::X xd;
+            FD::fetch_x(xd, hcells, pd.blk, pd.sub);
+            const bool scaled = p.down_scale != nullptr;
+            const float ds = scaled ? p.down_scale[e_cur] : 1.0f;
+            uint64_t* part = q.ypart + (size_t)g * ne + (size_t)m * R;
+            bool on_shared = false;
+            auto dn_finish = [&](int slot, int j) {
+                const bool routed = j < my_di;
+                if (!routed && !on_shared) {   // the same for the whole wavefront
+                    on_shared = true;
+                    if (wave != 2 && lds_flag_wait(&s_f_hs) != 1) alive = false;
+                    FD::fetch_x(xd, hscells, pd.blk, pd.sub);
+                }
+                const int jj = routed ? j : j - my_di;
+                const int orow = (jj * kSW + sw) * pd.rw_count + pd.rw;
+                const float y = row_sum<FD>(FD::dot(dring[slot], pd.sub, xd), pd, nblk_d);
+                if (pd.writer()) {
+                    if (routed) {
+                        if (orow < R) rec_store(part + orow, scaled ? __fmul_rn(y, ds) : y, tag);
+                    } else if (orow < SR) {
+                        s_ysh[orow] = y;
+                    }
+                }
+            };
+            ring_drain<DD>(my_di + my_sdi, dn_issue, dn_finish);
+            if (wave == 3) STAMP(11);
+        }
+    }
+    __syncthreads();
+    if (wave == 0) STAMP(12);
+    // ---- the rank-ordered sum: workgroup (g, m) owns rows [m R + g R / 8, + R / 8) of the output, which are also the
+    // rows of the always-on expert it has just computed.  out = sum over ranks of w_rank * y_rank as a separate
+    // multiply and add (crates/infr-cpu/src/lib.rs:4290-4302), then the always-on expert, then the residual operand.
+    if (!s_fault) {
+        const int R = ne / kPerGroup, SR = R / kGroups;
+        if (tid < SR) {
+            const size_t oi = (size_t)m * R + (size_t)g * SR + tid;
+            uint64_t yk[kGroups];
+            bool ok = false;
+            for (int spin = 0; !ok && spin <= spin_limit; spin++) {
+#pragma unroll
+                for (int k = 0; k < kGroups; k++) yk[k] = rec_load(q.ypart + (size_t)s_gor[k] * ne + oi);   // rank order
+                ok = true;
+#pragma unroll
+                for (int k = 0; k < kGroups; k++) ok = ok && (uint32_t)(yk[k] >> 32) == tag;
+            }
+            if (!ok) __hip_atomic_store(q.fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            float acc = 0.0f;
+#pragma unroll
+            for (int k = 0; k < kGroups; k++) acc = __fadd_rn(acc, __fmul_rn(s_w[k], __uint_as_float((uint32_t)yk[k])));
+            if (shared) {
+                float ws = 1.0f;
+                if (p.sh_logit)   // crates/infr-cpu/src/lib.rs:3336-3356: sigmoid of the row's gate logit
+                    ws = __fdiv_rn(1.0f, __fadd_rn(1.0f, expf_libm(-p.sh_logit[0], s_tab)));
+                acc = __fadd_rn(acc, __fmul_rn(ws, s_ysh[tid]));
+            }
+            p.dst[oi] = p.addend ? __fadd_rn(p.addend[oi], acc) : acc;
+        }
+    }
+    if (wave == 0) STAMP(13);
+    // the workgroup that leaves last advances the sequence number, whatever happened
+    if (tid == 0) {
+        const uint32_t old = __hip_atomic_fetch_add(q.cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if ((old & (kBlocks - 1)) == kBlocks - 1) __hip_atomic_store(q.seq, s_seq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------
+size_t moe_layer_stream_workspace_bytes(int ne, int nff, int n_expert) {
+    // [seq, done counter][pad to 256][estimates 8 * n_expert][logits 8 * n_expert][h 8 * nff][h always-on nff][partials 8 * ne]
+    return 256 + ((size_t)2 * kGroups * n_expert + (size_t)kGroups * nff + (size_t)nff + (size_t)kGroups * ne) * 8;
+}
+
+namespace {
+
+struct StreamShape {
+    int dg, dd, ept, nsp, epb, once, early_down;
+    size_t lds;
+};
+
+template <class FG, class FD>
+bool stream_shape(const MoeLayerParams& q, StreamShape* out) {
+    const MoeGemvParams& p = q.g;
+    const int ne = p.ne, nff = p.nff, n_expert = p.route.n_expert;
+    const bool shared = p.sh_gate != nullptr;
+    if (ne != 2048 && ne != 4096) return false;                      // 256 or 512 octets on 512 threads
+    if (ne % FG::kBlockElems || nff % FD::kBlockElems || nff % 256 || nff > 1536) return false;
+    const int lpr_g = ne / FG::kBlockElems * FG::kLPB, lpr_d = nff / FD::kBlockElems * FD::kLPB;
+    if (lpr_g > 64 || lpr_d > 64) return false;
+    if (n_expert % 64 || n_expert > 256 || n_expert < 64) return false;
+    const int rwc_g = 64 / lpr_g, rwc_d = 64 / lpr_d;
+    const int fpb = nff / kPerGroup, R = ne / kPerGroup;
+    const int n_gi = (fpb + rwc_g - 1) / rwc_g, n_di = (R + rwc_d - 1) / rwc_d;
+    const int my_gi = (n_gi + kSW - 1) / kSW, my_di = (n_di + kSW - 1) / kSW;
+    if (my_gi * rwc_g > 64) return false;                            // a wavefront's results wait in one 64-float row
+    if (shared) {
+        const int n_si = (nff / kBlocks + rwc_g - 1) / rwc_g;
+        if (n_si > kSW || ne / kBlocks > 64) return false;
+    }
+    // every logit once for the grid when a group's copy of the router would be a large share of the layer's bytes
+    out->once = q.logits_once;
+    out->epb = out->once ? (n_expert + kBlocks - 1) / kBlocks : n_expert / kPerGroup;
+    const int H = kThreads / (ne / 8);
+    out->ept = (out->epb + H - 1) / H;
+    out->nsp = n_expert / 64;
+    // everything in flight at once when a wavefront has few items, rings otherwise
+    out->dg = my_gi <= 2 ? 2 : my_gi <= 4 && std::is_same<FG, Q80Fmt>::value ? 4 : 2;
+    out->early_down = my_gi <= out->dg ? 1 : 0;
+    // down rows requested behind the last gate/up rows ride out the hand-over of the activations: a deep ring
+    out->dd = my_di <= 2 ? 2 : my_di <= 5 && std::is_same<FD, Q80Fmt>::value ? 5 : 3;
+    const int jstride = ne / 8 + 4;
+    const size_t floats = (size_t)(out->epb + 1) * 8 * jstride + 2 * (size_t)n_expert +
+                          ((route_scratch_floats(n_expert, p.route.n_groups) + 3) & ~(size_t)3) + 2 * (size_t)nff;
+    out->lds = cells_bytes(ne) + floats * 4 + 2 * cells_bytes(nff);
+    return out->lds <= 150 * 1024;
+}
+
+template <class FG, class FD, int DG, int DD, int EPT, int NSP>
+bool launch_stream(hipStream_t s, const MoeLayerParams& q, size_t lds) {
+    static bool attr_ok[16] = {};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return false;
+    if (!attr_ok[dev]) {
+        if (hipFuncSetAttribute((const void*)moe_layer_stream<FG, FD, DG, DD, EPT, NSP>,
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024) != hipSuccess)
+            return false;
+        attr_ok[dev] = true;
+    }
+    INFR_LAUNCH((moe_layer_stream<FG, FD, DG, DD, EPT, NSP>), dim3(kBlocks), dim3(kThreads), lds, s, q);
+    return true;
+}
+
+template <class FG, class FD>
+bool dispatch_stream(hipStream_t s, MoeLayerParams q, bool launch) {
+    StreamShape sh;
+    if (!stream_shape<FG, FD>(q, &sh)) return false;
+    q.epb = sh.epb;
+    q.early_down = sh.early_down;
+#define INFR_STREAM(DGv, DDv, EPTv, NSPv)                                                        \
+    if (sh.dg == DGv && sh.dd == DDv && sh.ept == EPTv && sh.nsp == NSPv)                           \
+        return launch ? launch_stream<FG, FD, DGv, DDv, EPTv, NSPv>(s, q, sh.lds) : true;
+    if constexpr (std::is_same<FG, Q4KFmt>::value) {
+        INFR_STREAM(2, 2, 2, 2)   // ne 2048, nff 768, 128 experts, a copy of the router per group
+        INFR_STREAM(2, 2, 1, 2)   // ... every logit once
+        INFR_STREAM(2, 2, 1, 4)   // ... 256 experts
+        INFR_STREAM(2, 3, 1, 4)   // ne 4096, nff 1536, 256 experts, every logit once
+    } else {
+        INFR_STREAM(4, 5, 2, 2)   // Q8_0: ne 2048, nff 768, 128 experts
+        INFR_STREAM(4, 5, 1, 2)
+        INFR_STREAM(4, 5, 1, 4)
+    }
+#undef INFR_STREAM
+    return false;
+}
+
+bool stream_any(hipStream_t s, const MoeLayerParams& q, bool launch) {
+    const MoeGemvParams& p = q.g;
+    const RouteParams& r = p.route;
+    if (p.rows != 1 || p.n_used != kGroups || p.n_cu < kBlocks || p.gate_dt != p.up_dt) return false;
+    if ((p.sh_gate != nullptr) != (p.sh_down != nullptr) || (p.sh_gate != nullptr) != (p.sh_up != nullptr)) return false;
+    // the guess ranks the experts by their logits: gatings that are monotone in the logit, no bias, no groups, no given
+    // ids; options that need the routing weights before the gate/up stage or remap ids stay on the in-order kernels
+    if ((r.gating != INFR_GATING_SOFTMAX && r.gating != INFR_GATING_SIGMOID) || r.exp_probs_b || r.expert_ids ||
+        (r.n_groups > 1 && r.n_groups_used > 0) || r.ep_n > 0 || p.weight_before || p.skip_zero_w)
+        return false;
+    if (launch && ((((uintptr_t)q.router | (uintptr_t)q.router_x | (uintptr_t)p.x) & 15) != 0 || (q.router_row_floats & 3) != 0))
+        return false;
+    if (p.gate_dt == INFR_Q4K && p.down_dt == INFR_Q6K) return dispatch_stream<Q4KFmt, Q6KFmt>(s, q, launch);
+    if (p.gate_dt == INFR_Q8_0 && p.down_dt == INFR_Q8_0) return dispatch_stream<Q80Fmt, Q80Fmt>(s, q, launch);
+    return false;
+}
+
+}  // namespace
+
+bool moe_layer_stream_supported(const MoeLayerParams& q) { return stream_any(nullptr, q, false); }
+bool launch_moe_layer_stream(hipStream_t s, const MoeLayerParams& q) { return stream_any(s, q, true); }
+
+}  // namespace infr

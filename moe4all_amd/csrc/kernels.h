@@ -105,10 +105,14 @@ void launch_moe_gate_up(hipStream_t s, const MoeGemvParams& p);
 // dst[row] = sum over slots (rank order) of w * (down . h).
 void launch_moe_down_combine(hipStream_t s, const MoeGemvParams& p);
 
-// Single-token Op::MoeFfn in one launch (k_layer.hip): logits, routing, gate/up, down and the weighted sum, the
-// stages handing over inside the kernel.  g: as for the two-launch path (g.route filled, rows == 1); the workspace
-// (moe_layer_workspace_bytes, zeroed once) holds the hand-over records, the per-rank partial results and the
-// launch sequence number; *fault (host-visible) is raised when a bounded wait runs out.
+// Single-token Op::MoeFfn in one launch: logits, routing, gate/up, down and the weighted sum, the stages handing over
+// inside the kernel.  g: as for the two-launch path (g.route filled, rows == 1); the workspace (zeroed once) holds the
+// hand-over records, the per-rank partial results and the launch sequence number; *fault (host-visible) is raised when
+// a bounded wait runs out.  Two kernels take these parameters:
+//   moe_layer_stream (k_layer_stream.hip): requests the expert rows of a GUESSED selection (from fast estimates of the
+//     logits) while the exact logits and the exact routing are computed beside the stream; plain gatings only, an
+//     always-on expert may ride along (g.sh_*);
+//   moe_layer_fused (k_layer.hip): the stages in order; every routing option.
 struct MoeLayerParams {
     MoeGemvParams g;
     const float* router;        // [n_expert, ne] f32
@@ -116,16 +120,27 @@ struct MoeLayerParams {
     const float* router_x;      // [ne]
     float* logits_out;          // [n_expert] or null: the logits, for the plan's routing capture
     uint32_t* seq;              // workspace + 0
-    uint32_t* cnt;              // workspace + 16: 32 slice counters, then the finished-slice counter
+    uint32_t* cnt;              // in-order kernel: workspace + 16, 32 slice counters then the finished-slice counter;
+                                // streaming kernel: workspace + 4, one counter of finished workgroups
     uint64_t* xl;               // [8][n_expert] logit records
     uint64_t* xh;               // [8][nff] activation records
     uint64_t* ypart;            // [8][ne] partial-result records
     uint32_t* fault;
     int spin_limit;
+    // streaming kernel only
+    uint64_t* xa;               // [8][n_expert] records of the logits' estimates
+    uint64_t* xs;               // [nff] activation records of the always-on expert
+    uint32_t* late;             // host-visible: experts a guess missed, summed over launches (or null)
+    int logits_once;            // every logit computed by one workgroup for the whole grid, not once per group
+    int guess_skew;             // tests: the guess leaves out this many of the largest estimates
+    int epb, early_down;        // set by the launcher
 };
 size_t moe_layer_workspace_bytes(int ne, int nff, int n_expert);
 bool moe_layer_fused_supported(const MoeLayerParams& q);
 bool launch_moe_layer_fused(hipStream_t s, const MoeLayerParams& q);
+size_t moe_layer_stream_workspace_bytes(int ne, int nff, int n_expert);
+bool moe_layer_stream_supported(const MoeLayerParams& q);
+bool launch_moe_layer_stream(hipStream_t s, const MoeLayerParams& q);
 
 // ---- batched path: bucketing + grouped GEMMs on the matrix cores --------------------------------
 struct GroupedParams {
