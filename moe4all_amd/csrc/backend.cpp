@@ -1503,16 +1503,15 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                     lp.spin_limit = be->cfg.single_launch_spin_limit ? (int)be->cfg.single_launch_spin_limit - 1 : 1 << 15;
                     if (sc.single_launch == 2 && plan->stream_ws) {
                         char* ws = plan->stream_ws;
-                        lp.seq = (uint32_t*)ws;
-                        lp.cnt = (uint32_t*)(ws + 4);
-                        lp.xa = (uint64_t*)(ws + 256);
+                        lp.cnt = (uint32_t*)ws;
+                        lp.xa = (uint64_t*)(ws + 1024);
                         lp.xl = lp.xa + (size_t)8 * m.n_expert;
                         lp.xh = lp.xl + (size_t)8 * m.n_expert;
                         lp.xs = lp.xh + (size_t)8 * m.n_ff_exp;
                         lp.ypart = lp.xs + (size_t)m.n_ff_exp;
                         lp.late = be->fault_dev + 1;
                         lp.logits_once = moe_logits_once(be, m);
-                        lp.guess_skew = (int)be->cfg.single_launch_guess_skew;
+                        lp.guess_skew = (int)std::min<uint32_t>(be->cfg.single_launch_guess_skew, 8u);
                         if (infr::moe_layer_stream_supported(lp) &&
                             (((uintptr_t)lp.router | (uintptr_t)lp.router_x | (uintptr_t)gp.x) & 15) == 0 && (lp.router_row_floats & 3) == 0) {
                             launch_gate_logit();   // no norm is folded on this path: the row it reads is there

@@ -60,9 +60,21 @@ __device__ __forceinline__ uint64_t rec_load(const uint64_t* p) {
 __device__ __forceinline__ void rec_store(uint64_t* p, float v, uint32_t tag) {
     __hip_atomic_store(p, (uint64_t)__float_as_uint(v) | ((uint64_t)tag << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+// A record for readers on the writer's own XCD only: a plain store, which stops in that XCD's L2, where the polling
+// loads (which pass the L1 but not the L2) find it: about a fifth less latency than a write-through store, and the
+// polls of a group no longer travel the fabric.  `local` false: for everyone, as above.
+__device__ __forceinline__ void rec_store_xcd(uint64_t* p, float v, uint32_t tag, bool local) {
+    if (!local) {
+        rec_store(p, v, tag);
+        return;
+    }
+    const uint64_t r = (uint64_t)__float_as_uint(v) | ((uint64_t)tag << 32);
+    asm volatile("global_store_dwordx2 %0, %1, off" ::"v"(p), "v"(r) : "memory");
+}
 
 // Wave-wide: gathers rec[0 .. n) (n a multiple of 64, n <= 64 N) into out[] once all carry `tag`.  Every poll issues
-// all of a lane's loads before it looks at any of them, so a poll costs one memory round trip.  False: spin limit.
+// all of a lane's loads before it looks at any of them, so a poll costs one round trip (two polls in flight half a
+// round trip apart were measured slower: the polls of 256 workgroups share one path).  False: spin limit.
 template <int N>
 __device__ __forceinline__ bool gather_records(const uint64_t* rec, int n, uint32_t tag, float* out, int lane, int spin_limit) {
     uint64_t r[N];
@@ -95,26 +107,17 @@ __device__ __forceinline__ int lds_flag_wait(volatile int* f) {
     return v;
 }
 
-// Wave-wide maximum as a scalar: DPP steps inside the rows of 16 lanes, then row_bcast:15 into rows 1 and 3 and
-// row_bcast:31 into rows 2 and 3, after which the last lane holds the maximum.
-__device__ __forceinline__ uint32_t wave_max_scalar(uint32_t v) {
-    v = max(v, dpp_u<kDppXor1>(v));
-    v = max(v, dpp_u<kDppXor2>(v));
-    v = max(v, dpp_u<kDppHalfMirror>(v));
-    v = max(v, dpp_u<kDppMirror>(v));
-    v = max(v, (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, 0x142, 0xA, 0xF, false));
-    v = max(v, (uint32_t)__builtin_amdgcn_update_dpp((int)v, (int)v, 0x143, 0xC, 0xF, false));
-    return (uint32_t)__builtin_amdgcn_readlane((int)v, 63);
-}
-
 // The guess: the n_sel indices with the largest estimates, into out[] (any fixed rule will do: every workgroup runs
 // this on the same values, and a wrong guess only costs time).  Keys are made unique by putting 255 - index into the
-// low byte of the order-preserving key (n <= 256), so a round is one wave-wide maximum whose low byte names the
-// winner: estimates that agree in all but their last 8 mantissa bits are ranked by index, like exact ties.  Every lane
-// keeps its NS keys sorted, so a round only looks at heads.  skew > 0 (tests only) leaves the `skew` largest out, so
-// the guess is wrong on purpose.
+// low byte of the order-preserving key (n <= 256): estimates that agree in all but their last 8 mantissa bits are
+// ranked by index, like exact ties.  Ranks come from counting, which has no serial chain: every lane sorts its NS keys
+// and counts the lanes whose largest key beats its own; a member of the top K overall lies in one of the K lanes with
+// the largest heads, so those lanes' K * NS keys (<= 64) are ranked among themselves the same way and the ranks
+// [skew, skew + n_sel) are the guess.  skew > 0 (tests only, <= 8) leaves the `skew` largest out, so the guess is wrong
+// on purpose.  scratch: 128 words of LDS.
 template <int NS>
-__device__ __forceinline__ void guess_set(const float* vals, int n_sel, int skew, int lane, int32_t* out) {
+__device__ __forceinline__ void guess_set(const float* vals, int n_sel, int skew, int lane, int32_t* out, uint32_t* scratch) {
+    static_assert(NS == 1 || NS == 2 || NS == 4, "sorting network");
     uint32_t key[NS];
 #pragma unroll
     for (int s = 0; s < NS; s++) {
@@ -128,15 +131,33 @@ __device__ __forceinline__ void guess_set(const float* vals, int n_sel, int skew
     };
     if (NS == 2) order(0, 1);
     if (NS == 4) { order(0, 1); order(2, 3); order(0, 2); order(1, 3); order(1, 2); }
-    static_assert(NS == 1 || NS == 2 || NS == 4, "sorting network");
-    for (int k = 0; k < n_sel + skew; k++) {
-        const uint32_t mx = wave_max_scalar(key[0]);
-        if (k >= skew && lane == 0) out[k - skew] = 255 - (int)(mx & 0xFFu);
-        const bool win = key[0] == mx;
+    uint32_t* heads = scratch;
+    uint32_t* cand = scratch + kWave;
+    heads[lane] = key[0];
+    cand[lane] = 0u;
+    __builtin_amdgcn_wave_barrier();
+    auto beaten_by = [&](const uint32_t* list, int n4, uint32_t mine) {
+        int r0 = 0, r1 = 0, r2 = 0, r3 = 0;
+        for (int c = 0; c < n4; c++) {
+            const uint4 v = reinterpret_cast<const uint4*>(list)[c];   // the same address in every lane: a broadcast
+            r0 += v.x > mine ? 1 : 0;
+            r1 += v.y > mine ? 1 : 0;
+            r2 += v.z > mine ? 1 : 0;
+            r3 += v.w > mine ? 1 : 0;
+        }
+        return (r0 + r1) + (r2 + r3);
+    };
+    const int K = n_sel + skew;   // <= 16
+    const int r = beaten_by(heads, kWave / 4, key[0]);
+    if (r < K) {
 #pragma unroll
-        for (int s = 0; s + 1 < NS; s++) key[s] = win ? key[s + 1] : key[s];
-        key[NS - 1] = win ? 0u : key[NS - 1];
+        for (int s = 0; s < NS; s++) cand[r * NS + s] = key[s];
     }
+    __builtin_amdgcn_wave_barrier();
+    const int nc = K * NS;
+    const uint32_t mine = cand[lane];   // 0 past the candidates
+    const int r2 = beaten_by(cand, (nc + 3) >> 2, mine);
+    if (lane < nc && r2 >= skew && r2 < K) out[r2 - skew] = 255 - (int)(mine & 0xFFu);
 }
 
 // A ring of D items in flight: `issue(slot, j)` requests item j into ring slot `slot`, `finish(slot, j)` consumes it.
@@ -196,7 +217,8 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
     __shared__ float s_part[kWaves][8];
     __shared__ int32_t s_spec[kGroups], s_final[kGroups], s_gor[kGroups];
     __shared__ float s_ysh[64];
-    __shared__ int s_f_spec, s_f_route, s_f_h, s_f_hs, s_fault, s_cells_done;
+    __shared__ uint32_t s_guess[2 * kWave];
+    __shared__ int s_f_spec, s_f_route, s_f_hs, s_fault, s_cells_done, s_h_done, s_done;
     __shared__ uint32_t s_seq;
     const MoeGemvParams& p = q.g;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -207,6 +229,7 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
     // who computes which router logits: every group all of them (epb = n_expert / 32 rows per workgroup, published to
     // the group), or every logit once for the grid (epb rows per workgroup while they last, published to everyone)
     const int epb = q.epb;
+    const bool group_local = !q.logits_once;   // logit records stay inside the group's XCD
     const int area = q.logits_once ? 0 : g;
     const int row0 = (q.logits_once ? b : m) * epb;
     const bool has_rows = row0 < n_expert;
@@ -229,10 +252,16 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
 
     if (tid < 32) s_tab[tid] = kExp2Table[tid];
     if (tid == 0) {
-        s_f_spec = s_f_route = s_f_h = s_f_hs = s_fault = s_cells_done = 0;
-        s_seq = __hip_atomic_load(q.seq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1u;   // one load per workgroup
+        s_f_spec = s_f_route = s_f_hs = s_fault = s_cells_done = s_h_done = s_done = 0;
+        // the launch's number: every workgroup keeps its own count of the launches it has run (a counter shared by all
+        // would serialise 256 atomics, at the start or, worse, at the end of the kernel), read here and written back
+        // with a plain store at the end; launches on a workspace never overlap, so all 256 counts agree
+        s_seq = q.cnt[b] + 1u;
     }
     if (wave == 0) STAMP(0);
+    // (Records written for the own group only stop in the XCD's L2.  Workgroups are dealt to the XCDs in turn by their
+    // index, starting from an XCD that changes from launch to launch, so a group sits on one XCD; were it ever split, a
+    // record would simply not be seen, the wait would run out and the launch be reported: a record is one 64-bit unit.)
 
     // ---- A: operands.  Thread (replica hsel, octet o) holds elements [8 o, 8 o + 8) of the routing row, of the token
     // row and of the router rows hsel, hsel + H, ...  The token row becomes fixed-point cells later, by the threads
@@ -286,7 +315,7 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
         const int hs = lane % H, i = lane / H;
         float a = 0.0f;
         for (int w = hs * waves_per_replica; w < (hs + 1) * waves_per_replica; w++) a += s_part[w][i];
-        rec_store(q.xa + (size_t)area * n_expert + row0 + lane, a, tag);
+        rec_store_xcd(q.xa + (size_t)area * n_expert + row0 + lane, a, tag, group_local);
     }
     // the token row as fixed-point cells, one set for the workgroup; the guessing wavefront takes its share after the guess
     const int n_conv_waves = oct_n >> 6;
@@ -334,7 +363,7 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
 #pragma unroll
             for (int jj = 0; jj < 8; jj++) s = __fadd_rn(s, __shfl(acc, (lane & ~7) + jj, kWave));
             if (live && j == 0) {
-                rec_store(q.xl + (size_t)area * n_expert + row0 + e, s, tag);
+                rec_store_xcd(q.xl + (size_t)area * n_expert + row0 + e, s, tag, group_local);
                 if ((q.logits_once || g == 0) && q.logits_out) q.logits_out[row0 + e] = s;
             }
         }
@@ -398,23 +427,39 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
         struct GuItem { typename FG::Raw g, u; };
         bool alive = true;
 
-        // the always-on expert's gate/up share of this workgroup: at most one item per wavefront, requested first
+        // gate/up items of this wavefront: item j covers features (j * kSW + sw) * rw_count + rw of the workgroup's slice.
+        // With an always-on expert the first kSW-or-fewer wavefronts take one item of its share [b * nff / 256, ..) as
+        // their ring's first entry: it needs no routing, so it is requested before the guess is known.
+        const int fpb = nff / kPerGroup, f0 = m * fpb;
+        const int n_gi = (fpb + pg.rw_count - 1) / pg.rw_count;
+        const int my_gi = n_gi > sw ? (n_gi - sw + kSW - 1) / kSW : 0;
         const int sfpb = nff / kBlocks, sf0 = b * sfpb;
         const int n_si = shared ? (sfpb + pg.rw_count - 1) / pg.rw_count : 0;
-        const bool my_si = sw < n_si;
-        GuItem sh_item;
-        if (my_si && wave != 1) {
+        const int sh_n = sw < n_si ? 1 : 0;
+        // down items: item j covers output rows (j * kSW + sw) * rw_count + rw of the workgroup's slice; behind them the
+        // always-on expert's rows [b * ne / 256, ..), dealt to the wavefronts starting with those that got fewer above
+        const int R = ne / kPerGroup;
+        const int n_di = (R + pd.rw_count - 1) / pd.rw_count;
+        const int my_di = n_di > sw ? (n_di - sw + kSW - 1) / kSW : 0;
+        const int SR = ne / kBlocks;
+        const int n_sdi = shared ? (SR + pd.rw_count - 1) / pd.rw_count : 0;
+        const int ssw = (sw + kSW - n_di % kSW) % kSW;
+        const int my_sdi = n_sdi > ssw ? (n_sdi - ssw + kSW - 1) / kSW : 0;
+
+        GuItem gring[DG];
+        auto sh_issue = [&]() {
             const int f = sf0 + min(sw * pg.rw_count + pg.rw, sfpb - 1);
-            sh_item.g = load_row<FG>(pg, p.sh_gate + (size_t)f * rb_g);
-            sh_item.u = load_row<FG>(pg, p.sh_up + (size_t)f * rb_g);
-        }
+            gring[0].g = load_row<FG>(pg, p.sh_gate + (size_t)f * rb_g);
+            gring[0].u = load_row<FG>(pg, p.sh_up + (size_t)f * rb_g);
+        };
+        if (sh_n && wave != 1) sh_issue();
         if (wave == 1) {
             // the guess of the selected set, from the estimates
             bool ok = gather_records<NSP>(q.xa + (size_t)area * n_expert, n_expert, tag, s_alog, lane, spin_limit);
             STAMP(3);
             if (ok) {
                 __builtin_amdgcn_wave_barrier();
-                guess_set<NSP>(s_alog, kGroups, q.guess_skew, lane, s_spec);
+                guess_set<NSP>(s_alog, kGroups, q.guess_skew, lane, s_spec, s_guess);
             } else if (lane == 0) {
                 s_fault = 1;
                 __hip_atomic_store(q.fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
@@ -423,36 +468,19 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
             STAMP(4);
             alive = ok;
             convert_share();
-            if (my_si) {
-                const int f = sf0 + min(sw * pg.rw_count + pg.rw, sfpb - 1);
-                sh_item.g = load_row<FG>(pg, p.sh_gate + (size_t)f * rb_g);
-                sh_item.u = load_row<FG>(pg, p.sh_up + (size_t)f * rb_g);
-            }
+            if (sh_n) sh_issue();
         } else {
             alive = lds_flag_wait(&s_f_spec) == 1;
         }
 
-        // gate/up items of this wavefront: item j covers features (j * kSW + sw) * rw_count + rw of the workgroup's slice
-        const int fpb = nff / kPerGroup, f0 = m * fpb;
-        const int n_gi = (fpb + pg.rw_count - 1) / pg.rw_count;
-        const int my_gi = n_gi > sw ? (n_gi - sw + kSW - 1) / kSW : 0;
-        // down items: item j covers output rows (j * kSW + sw) * rw_count + rw of the workgroup's slice; behind them the
-        // always-on expert's rows [b * ne / 256, ..) of this workgroup
-        const int R = ne / kPerGroup;
-        const int n_di = (R + pd.rw_count - 1) / pd.rw_count;
-        const int my_di = n_di > sw ? (n_di - sw + kSW - 1) / kSW : 0;
-        const int SR = ne / kBlocks;
-        const int n_sdi = shared ? (SR + pd.rw_count - 1) / pd.rw_count : 0;
-        const int my_sdi = n_sdi > sw ? (n_sdi - sw + kSW - 1) / kSW : 0;
-
         typename FD::Raw dring[DD];
-        int e_cur = alive ? s_spec[g] : 0;
+        int e_cur = alive ? __builtin_amdgcn_readfirstlane(s_spec[g]) : 0;
         const uint8_t* dbank = nullptr;
         auto dn_issue = [&](int slot, int j) {
             const bool routed = j < my_di || !shared;   // items past the end re-read a last row
             const int jj = routed ? j : j - my_di;
             const int lim = routed ? R : SR;
-            const int orow = min((jj * kSW + sw) * pd.rw_count + pd.rw, lim - 1);
+            const int orow = min((jj * kSW + (routed ? sw : ssw)) * pd.rw_count + pd.rw, lim - 1);
             const uint8_t* base = routed ? dbank + (size_t)(m * R + orow) * rb_d : p.sh_down + (size_t)(b * SR + orow) * rb_d;
             dring[slot] = load_row<FD>(pd, base);
         };
@@ -461,36 +489,34 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
                 const uint8_t* gb = p.gate + (size_t)e_cur * p.gate_stride + (size_t)f0 * rb_g;
                 const uint8_t* ub = p.up + (size_t)e_cur * p.up_stride + (size_t)f0 * rb_g;
                 dbank = p.down + (size_t)e_cur * p.down_stride;
-                GuItem gring[DG];
+                const int sh = attempt == 0 ? sh_n : 0;   // ring entries ahead of the expert's items
                 typename FG::X x;   // fetched again on a second pass: not kept alive across the hand-over
                 auto gu_issue = [&](int slot, int j) {
-                    const int f = min((j * kSW + sw) * pg.rw_count + pg.rw, fpb - 1);
+                    const int f = min(((j - sh) * kSW + sw) * pg.rw_count + pg.rw, fpb - 1);
                     gring[slot].g = load_row<FG>(pg, gb + (size_t)f * rb_g);
                     gring[slot].u = load_row<FG>(pg, ub + (size_t)f * rb_g);
                 };
                 auto gu_finish = [&](int slot, int j) {
                     const float gs = row_sum<FG>(FG::dot(gring[slot].g, pg.sub, x), pg, nblk_g);
                     const float us = row_sum<FG>(FG::dot(gring[slot].u, pg.sub, x), pg, nblk_g);
-                    if (pg.writer()) {
-                        s_g[wave][j * pg.rw_count + pg.rw] = gs;
-                        s_u[wave][j * pg.rw_count + pg.rw] = us;
+                    if (j < sh) {   // the always-on expert's item: its activation goes to every workgroup
+                        const int fi = sw * pg.rw_count + pg.rw;
+                        if (pg.writer() && fi < sfpb)
+                            rec_store(q.xs + sf0 + fi, gated_act_fn(p.act, p.has_clamp, p.clamp, gs, us, s_tab), tag);
+                    } else if (pg.writer()) {
+                        s_g[wave][(j - sh) * pg.rw_count + pg.rw] = gs;
+                        s_u[wave][(j - sh) * pg.rw_count + pg.rw] = us;
                     }
                 };
-                ring_prime<DG>(gu_issue);
+#pragma unroll
+                for (int d = 0; d < DG; d++)
+                    if (d >= sh) gu_issue(d, d);
                 if (q.early_down) ring_prime<DD>(dn_issue);
                 if (wave == 3) STAMP(5);
                 if (wave == 1) STAMP(20);
                 if (attempt == 0) wait_cells();
                 FG::fetch_x(x, cells, pg.blk, pg.sub);
-                if (attempt == 0 && my_si) {
-                    // the always-on expert's item, requested before the guess was known
-                    const float gs = row_sum<FG>(FG::dot(sh_item.g, pg.sub, x), pg, nblk_g);
-                    const float us = row_sum<FG>(FG::dot(sh_item.u, pg.sub, x), pg, nblk_g);
-                    const int fi = sw * pg.rw_count + pg.rw;
-                    if (pg.writer() && fi < sfpb)
-                        rec_store(q.xs + sf0 + fi, gated_act_fn(p.act, p.has_clamp, p.clamp, gs, us, s_tab), tag);
-                }
-                ring_drain<DG>(my_gi, gu_issue, gu_finish);
+                ring_drain<DG>(sh + my_gi, gu_issue, gu_finish);
                 if (wave == 3) STAMP(6);
                 if (!q.early_down) ring_prime<DD>(dn_issue);
                 __builtin_amdgcn_wave_barrier();
@@ -498,9 +524,9 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
                     const int j = lane / pg.rw_count, rw = lane - j * pg.rw_count;
                     const int fi = (j * kSW + sw) * pg.rw_count + rw;
                     if (fi < fpb)
-                        rec_store(q.xh + (size_t)g * nff + f0 + fi,
-                                  gated_act_fn(p.act, p.has_clamp, p.clamp, s_g[wave][lane], s_u[wave][lane], s_tab),
-                                  seq_tag | (uint32_t)e_cur);
+                        rec_store_xcd(q.xh + (size_t)g * nff + f0 + fi,
+                                      gated_act_fn(p.act, p.has_clamp, p.clamp, s_g[wave][lane], s_u[wave][lane], s_tab),
+                                      seq_tag | (uint32_t)e_cur, true);
                 }
                 __builtin_amdgcn_wave_barrier();
                 if (wave == 3) STAMP(7);
@@ -511,20 +537,22 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
                     break;
                 }
                 if (wave == 3) STAMP(8);
-                const int e_fin = s_final[g];
+                const int e_fin = __builtin_amdgcn_readfirstlane(s_final[g]);
                 if (e_fin == e_cur) break;
                 e_cur = e_fin;   // the guess missed this group's expert: once more with the right one
             }
         }
-        // ---- hand-over of the group's activations: wavefront 1 gathers and converts, the others wait for its flag;
-        // wavefront 2 gathers the always-on expert's meanwhile
-        if (wave == 1) {
+        // ---- hand-over of the group's activations: six wavefronts gather a sixth each and turn it into cells; the
+        // seventh gathers the always-on expert's meanwhile (written long ago by all 256 workgroups)
+        const int chunk = nff / 6;   // records per gathering wavefront: a multiple of 64
+        if (sw < 6) {
             bool ok = alive;
-            if (ok) ok = gather_records<24>(q.xh + (size_t)g * nff, nff, seq_tag | (uint32_t)e_cur, s_h, lane, spin_limit);
-            STAMP(9);
+            if (ok) ok = gather_records<4>(q.xh + (size_t)g * nff + sw * chunk, chunk, seq_tag | (uint32_t)e_cur, s_h + sw * chunk, lane, spin_limit);
+            if (wave == 1) STAMP(9);
             if (ok) {
                 __builtin_amdgcn_wave_barrier();
-                for (int oct = lane; oct * 8 < nff; oct += kWave) {
+                if (lane * 8 < chunk) {   // whole groups of four lanes
+                    const int oct = sw * (chunk >> 3) + lane;
                     const float4 lo = *reinterpret_cast<const float4*>(s_h + 8 * oct), hi = *reinterpret_cast<const float4*>(s_h + 8 * oct + 4);
                     octet_to_cell<FD::kGroup, FD::kSigned>(lo, hi, oct, hcells);
                 }
@@ -532,10 +560,10 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
                 s_fault = 1;
                 __hip_atomic_store(q.fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
             }
-            lds_flag_set(&s_f_h, ok ? 1 : 2);
-            STAMP(10);
-            alive = ok;
-        } else if (wave == 2 && shared) {
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            if (lane == 0) __hip_atomic_fetch_add(&s_h_done, ok ? 1 : 0x101, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            if (wave == 1) STAMP(10);
+        } else if (shared) {
             bool ok = alive;
             if (ok) ok = gather_records<24>(q.xs, nff, tag, s_hs, lane, spin_limit);
             if (ok) {
@@ -549,9 +577,14 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
                 __hip_atomic_store(q.fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
             }
             lds_flag_set(&s_f_hs, ok ? 1 : 2);
-            alive = ok;
+            alive = alive && ok;
         }
-        if (wave != 1 && lds_flag_wait(&s_f_h) != 1) alive = false;
+        {
+            int v;
+            while (((v = __builtin_amdgcn_readfirstlane(*(volatile int*)&s_h_done)) & 0xFF) < 6) __builtin_amdgcn_s_sleep(1);
+            asm volatile("" ::: "memory");
+            if (v >> 8) alive = false;
+        }
         if (alive) {
             // ---- down: rows of the group's expert, then of the always-on expert
             typename FD::X xd;
@@ -564,11 +597,11 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
                 const bool routed = j < my_di;
                 if (!routed && !on_shared) {   // the same for the whole wavefront
                     on_shared = true;
-                    if (wave != 2 && lds_flag_wait(&s_f_hs) != 1) alive = false;
+                    if (sw != 6 && lds_flag_wait(&s_f_hs) != 1) alive = false;
                     FD::fetch_x(xd, hscells, pd.blk, pd.sub);
                 }
                 const int jj = routed ? j : j - my_di;
-                const int orow = (jj * kSW + sw) * pd.rw_count + pd.rw;
+                const int orow = (jj * kSW + (routed ? sw : ssw)) * pd.rw_count + pd.rw;
                 const float y = row_sum<FD>(FD::dot(dring[slot], pd.sub, xd), pd, nblk_d);
                 if (pd.writer()) {
                     if (routed) {
@@ -581,26 +614,42 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
             ring_drain<DD>(my_di + my_sdi, dn_issue, dn_finish);
             if (wave == 3) STAMP(11);
         }
+        // this wavefront's rows of the always-on expert are in LDS: tell the summing wavefront
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        if (lane == 0) __hip_atomic_fetch_add(&s_done, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
-    __syncthreads();
-    if (wave == 0) STAMP(12);
-    // ---- the rank-ordered sum: workgroup (g, m) owns rows [m R + g R / 8, + R / 8) of the output, which are also the
-    // rows of the always-on expert it has just computed.  out = sum over ranks of w_rank * y_rank as a separate
-    // multiply and add (crates/infr-cpu/src/lib.rs:4290-4302), then the always-on expert, then the residual operand.
-    if (!s_fault) {
+    if (wave == 0) {
+        // ---- the rank-ordered sum, by the router's wavefront: workgroup (g, m) owns rows [m R + g R / 8, + R / 8) of
+        // the output, which are also the rows of the always-on expert it has just computed.  out = sum over ranks of
+        // w_rank * y_rank as a separate multiply and add (crates/infr-cpu/src/lib.rs:4290-4302), then the always-on
+        // expert, then the residual operand.  The partial results are polled while the streaming wavefronts still work.
         const int R = ne / kPerGroup, SR = R / kGroups;
-        if (tid < SR) {
-            const size_t oi = (size_t)m * R + (size_t)g * SR + tid;
-            uint64_t yk[kGroups];
-            bool ok = false;
-            for (int spin = 0; !ok && spin <= spin_limit; spin++) {
+        const bool mine = lane < SR;
+        const size_t oi = (size_t)m * R + (size_t)g * SR + (mine ? lane : 0);
+        uint64_t yk[kGroups];
+        bool ok = *(volatile int*)&s_f_route == 1;
+        if (ok) {
+            for (int spin = 0;; spin++) {
 #pragma unroll
                 for (int k = 0; k < kGroups; k++) yk[k] = rec_load(q.ypart + (size_t)s_gor[k] * ne + oi);   // rank order
-                ok = true;
+                bool got = true;
 #pragma unroll
-                for (int k = 0; k < kGroups; k++) ok = ok && (uint32_t)(yk[k] >> 32) == tag;
+                for (int k = 0; k < kGroups; k++) got = got && (uint32_t)(yk[k] >> 32) == tag;
+                if (__all(got || !mine)) break;
+                if (spin >= spin_limit) {
+                    ok = false;
+                    break;
+                }
             }
-            if (!ok) __hip_atomic_store(q.fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            if (!ok && lane == 0) {
+                s_fault = 1;
+                __hip_atomic_store(q.fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            }
+        }
+        STAMP(12);
+        while (__builtin_amdgcn_readfirstlane(*(volatile int*)&s_done) < kSW) __builtin_amdgcn_s_sleep(1);
+        asm volatile("" ::: "memory");
+        if (ok && mine && !*(volatile int*)&s_fault) {
             float acc = 0.0f;
 #pragma unroll
             for (int k = 0; k < kGroups; k++) acc = __fadd_rn(acc, __fmul_rn(s_w[k], __uint_as_float((uint32_t)yk[k])));
@@ -608,23 +657,19 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
                 float ws = 1.0f;
                 if (p.sh_logit)   // crates/infr-cpu/src/lib.rs:3336-3356: sigmoid of the row's gate logit
                     ws = __fdiv_rn(1.0f, __fadd_rn(1.0f, expf_libm(-p.sh_logit[0], s_tab)));
-                acc = __fadd_rn(acc, __fmul_rn(ws, s_ysh[tid]));
+                acc = __fadd_rn(acc, __fmul_rn(ws, s_ysh[lane]));
             }
             p.dst[oi] = p.addend ? __fadd_rn(p.addend[oi], acc) : acc;
         }
-    }
-    if (wave == 0) STAMP(13);
-    // the workgroup that leaves last advances the sequence number, whatever happened
-    if (tid == 0) {
-        const uint32_t old = __hip_atomic_fetch_add(q.cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if ((old & (kBlocks - 1)) == kBlocks - 1) __hip_atomic_store(q.seq, s_seq, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        STAMP(13);
+        if (lane == 0) q.cnt[b] = s_seq;
     }
 }
 
 // ---------------------------------------------------------------------------------------------
 size_t moe_layer_stream_workspace_bytes(int ne, int nff, int n_expert) {
-    // [seq, done counter][pad to 256][estimates 8 * n_expert][logits 8 * n_expert][h 8 * nff][h always-on nff][partials 8 * ne]
-    return 256 + ((size_t)2 * kGroups * n_expert + (size_t)kGroups * nff + (size_t)nff + (size_t)kGroups * ne) * 8;
+    // [launch count of each workgroup: 1 KB][estimates 8 * n_expert][logits 8 * n_expert][h 8 * nff][h always-on nff][partials 8 * ne]
+    return 1024 + ((size_t)2 * kGroups * n_expert + (size_t)kGroups * nff + (size_t)nff + (size_t)kGroups * ne) * 8;
 }
 
 namespace {
@@ -640,7 +685,7 @@ bool stream_shape(const MoeLayerParams& q, StreamShape* out) {
     const int ne = p.ne, nff = p.nff, n_expert = p.route.n_expert;
     const bool shared = p.sh_gate != nullptr;
     if (ne != 2048 && ne != 4096) return false;                      // 256 or 512 octets on 512 threads
-    if (ne % FG::kBlockElems || nff % FD::kBlockElems || nff % 256 || nff > 1536) return false;
+    if (ne % FG::kBlockElems || nff % FD::kBlockElems || nff % 256 || nff % 384 || nff > 1536) return false;   // six gathering wavefronts
     const int lpr_g = ne / FG::kBlockElems * FG::kLPB, lpr_d = nff / FD::kBlockElems * FD::kLPB;
     if (lpr_g > 64 || lpr_d > 64) return false;
     if (n_expert % 64 || n_expert > 256 || n_expert < 64) return false;
@@ -663,7 +708,7 @@ bool stream_shape(const MoeLayerParams& q, StreamShape* out) {
     out->dg = my_gi <= 2 ? 2 : my_gi <= 4 && std::is_same<FG, Q80Fmt>::value ? 4 : 2;
     out->early_down = my_gi <= out->dg ? 1 : 0;
     // down rows requested behind the last gate/up rows ride out the hand-over of the activations: a deep ring
-    out->dd = my_di <= 2 ? 2 : my_di <= 5 && std::is_same<FD, Q80Fmt>::value ? 5 : 3;
+    out->dd = my_di <= 2 ? 2 : my_di <= 5 && std::is_same<FD, Q80Fmt>::value ? 5 : out->early_down ? 3 : 4;
     const int jstride = ne / 8 + 4;
     const size_t floats = (size_t)(out->epb + 1) * 8 * jstride + 2 * (size_t)n_expert +
                           ((route_scratch_floats(n_expert, p.route.n_groups) + 3) & ~(size_t)3) + 2 * (size_t)nff;
@@ -699,7 +744,7 @@ bool dispatch_stream(hipStream_t s, MoeLayerParams q, bool launch) {
         INFR_STREAM(2, 2, 2, 2)   // ne 2048, nff 768, 128 experts, a copy of the router per group
         INFR_STREAM(2, 2, 1, 2)   // ... every logit once
         INFR_STREAM(2, 2, 1, 4)   // ... 256 experts
-        INFR_STREAM(2, 3, 1, 4)   // ne 4096, nff 1536, 256 experts, every logit once
+        INFR_STREAM(2, 4, 1, 4)   // ne 4096, nff 1536, 256 experts, every logit once
     } else {
         INFR_STREAM(4, 5, 2, 2)   // Q8_0: ne 2048, nff 768, 128 experts
         INFR_STREAM(4, 5, 1, 2)

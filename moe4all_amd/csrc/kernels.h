@@ -121,7 +121,7 @@ struct MoeLayerParams {
     float* logits_out;          // [n_expert] or null: the logits, for the plan's routing capture
     uint32_t* seq;              // workspace + 0
     uint32_t* cnt;              // in-order kernel: workspace + 16, 32 slice counters then the finished-slice counter;
-                                // streaming kernel: workspace + 4, one counter of finished workgroups
+                                // streaming kernel: workspace + 0, the launch count of each of its 256 workgroups
     uint64_t* xl;               // [8][n_expert] logit records
     uint64_t* xh;               // [8][nff] activation records
     uint64_t* ypart;            // [8][ne] partial-result records
