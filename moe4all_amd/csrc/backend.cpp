@@ -302,7 +302,8 @@ void drain_prof(infr_hip_backend* be) {
 int moe_logits_once(const infr_hip_backend* be, const infr_op_moe_ffn& m) {
     if (be->cfg.single_launch_logits == 1) return 1;
     if (be->cfg.single_launch_logits == 2) return 0;
-    return m.n_expert > 128 || m.ne > 2048 ? 1 : 0;
+    (void)m;
+    return 1;   // measured equal or faster on every shape the kernel takes, and the router is read once
 }
 
 // The per-token path of Op::MoeFfn (1 to 31 token rows; the bucketed path takes batches of 16 or more whose pairs fall on few distinct experts) once logits are in rp.logits and gp / rp are filled in:

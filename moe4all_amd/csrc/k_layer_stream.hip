@@ -518,7 +518,6 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
                 FG::fetch_x(x, cells, pg.blk, pg.sub);
                 ring_drain<DG>(sh + my_gi, gu_issue, gu_finish);
                 if (wave == 3) STAMP(6);
-                if (!q.early_down) ring_prime<DD>(dn_issue);
                 __builtin_amdgcn_wave_barrier();
                 if (lane < my_gi * pg.rw_count) {
                     const int j = lane / pg.rw_count, rw = lane - j * pg.rw_count;
@@ -563,6 +562,8 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
             if (lane == 0) __hip_atomic_fetch_add(&s_h_done, ok ? 1 : 0x101, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
             if (wave == 1) STAMP(10);
+            // the first down rows, requested behind the polls: a poll issued behind them would not return before them
+            if (!q.early_down && alive) ring_prime<DD>(dn_issue);
         } else if (shared) {
             bool ok = alive;
             if (ok) ok = gather_records<24>(q.xs, nff, tag, s_hs, lane, spin_limit);
@@ -578,6 +579,9 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
             }
             lds_flag_set(&s_f_hs, ok ? 1 : 2);
             alive = alive && ok;
+            if (!q.early_down && alive) ring_prime<DD>(dn_issue);
+        } else if (!q.early_down && alive) {
+            ring_prime<DD>(dn_issue);
         }
         {
             int v;
