@@ -374,12 +374,20 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
             __builtin_amdgcn_wave_barrier();
             RouteParams rp = p.route;
             rp.logits = s_logits;
-            route_row_any(rp, 0, lane, route_scratch, s_tab, s_ids, s_w, b == 0);
+            // the guess is the candidate for the selection: when the exact probabilities confirm it, the selection
+            // rounds are not needed; else (a missed expert, a tie at the boundary, another gating) the complete routine
+            const int guess_state = lds_flag_wait(&s_f_spec);
+            if (guess_state != 1) ok = false;
+            bool routed = false;
+            if (ok && route_duo_ok(rp) && rp.n_expert == 64 * NSP)
+                routed = route_softmax_checked<NSP>(rp, 0, lane, s_spec, route_scratch, s_tab, s_ids, s_w, b == 0);
+            if (!routed) {
+                __builtin_amdgcn_wave_barrier();
+                route_row_any(rp, 0, lane, route_scratch, s_tab, s_ids, s_w, b == 0);
+            }
             STAMP(18);
             __builtin_amdgcn_wave_barrier();
             // which group holds which rank; groups whose guess is outside the exact set take the missed experts
-            const int guess_state = lds_flag_wait(&s_f_spec);
-            if (guess_state != 1) ok = false;
             if (ok) {
                 // lane k < 8 owns rank k: the group whose guess is that expert; ranks the guess missed take the groups
                 // whose guess is outside the exact set, both in ascending order

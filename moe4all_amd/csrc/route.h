@@ -425,6 +425,133 @@ __device__ __forceinline__ bool route_duo_second(const RouteParams& p, int row, 
     return true;
 }
 
+// ---------------------------------------------------------------------------------------------
+// Plain softmax routing of one token row by one wavefront when a CANDIDATE for the selected set is known (the
+// single-launch kernel has guessed it from estimates of the logits).  The probabilities are computed as always
+// (crates/infr-cpu/src/lib.rs:3747-3756: exp(l - max), the left-to-right sum, one division each); then, instead of
+// n_used selection rounds, one test: if every candidate's probability is strictly above every other expert's, the
+// candidates ARE the reference's selection (lib.rs:3847-3850 sorts by probability descending, ties to the lower id,
+// and no tie crosses the boundary), and their ranks follow from comparing the n_used candidates with each other under
+// that same order.  Otherwise (a wrong candidate set, a tie across the boundary, anything not a number) the function
+// returns false and the caller runs the complete routine.  Needs n_expert == 64 * NS and n_used <= 16.
+// cand: n_used distinct ids in LDS; lds: 2 * n_expert floats, 16-byte aligned.
+template <int NS>
+__device__ __forceinline__ bool route_softmax_checked(const RouteParams& p, int row, int lane, const int32_t* cand, float* lds,
+                                                      const uint64_t* tab, int32_t* lds_ids, float* lds_w, bool store_global) {
+    const int n = p.n_expert;
+    const float* lg = p.logits + (size_t)row * n;
+    float* ex = lds;          // [n] exponentials, then probabilities
+    float pr[NS];
+#pragma unroll
+    for (int s = 0; s < NS; s++) pr[s] = lg[s * kWave + lane];
+    float m = pr[0];
+#pragma unroll
+    for (int s = 1; s < NS; s++) m = fmaxf(m, pr[s]);
+    m = wave_max(m);
+#pragma unroll
+    for (int s = 0; s < NS; s++) {
+        pr[s] = expf_libm(__fsub_rn(pr[s], m), tab);
+        ex[s * kWave + lane] = pr[s];
+    }
+    // which of this lane's experts are candidates (beside the sum's dependent adds, which leave issue slots free)
+    uint32_t member = 0;
+    for (int k = 0; k < p.n_used; k++) {
+        const int c = cand[k];
+#pragma unroll
+        for (int s = 0; s < NS; s++) member |= (c == s * kWave + lane ? 1u : 0u) << s;
+    }
+    __builtin_amdgcn_wave_barrier();
+    float psum = 0.0f;
+    {
+        float4 cur[8], nxt[8];
+#pragma unroll
+        for (int k = 0; k < 8; k++) cur[k] = reinterpret_cast<const float4*>(ex)[k];
+        for (int i = 0; i < n; i += 32) {
+            const int ni = i + 64 <= n ? i + 32 : i;   // past the end: re-read, unused
+#pragma unroll
+            for (int k = 0; k < 8; k++) nxt[k] = reinterpret_cast<const float4*>(ex + ni)[k];
+#pragma unroll
+            for (int k = 0; k < 8; k++) {
+                psum = __fadd_rn(psum, cur[k].x);
+                psum = __fadd_rn(psum, cur[k].y);
+                psum = __fadd_rn(psum, cur[k].z);
+                psum = __fadd_rn(psum, cur[k].w);
+            }
+#pragma unroll
+            for (int k = 0; k < 8; k++) cur[k] = nxt[k];
+        }
+    }
+    __builtin_amdgcn_wave_barrier();
+    // probabilities; the smallest among the candidates against the largest among the rest
+    uint32_t lo_in = 0xFFFFFFFFu, hi_out = 0u;
+#pragma unroll
+    for (int s = 0; s < NS; s++) {
+        pr[s] = __fdiv_rn(pr[s], psum);
+        ex[s * kWave + lane] = pr[s];
+        const uint32_t key = order_key(pr[s]);
+        const bool in = (member >> s) & 1u;
+        lo_in = in ? min(lo_in, key) : lo_in;
+        hi_out = in ? hi_out : max(hi_out, key);
+    }
+    lo_in = wave_min_u32(lo_in);
+    hi_out = wave_max_u32(hi_out);
+    uint32_t cnt = 0;
+#pragma unroll
+    for (int s = 0; s < NS; s++) cnt += (uint32_t)__builtin_popcountll(__ballot((member >> s) & 1u));
+    // a NaN among the probabilities has a key above every number's: it fails one side or the other
+    const bool clean = psum == psum && lo_in > hi_out && lo_in < order_key(__builtin_huge_valf()) + 1u && (int)cnt == p.n_used;
+    if (!clean) return false;
+    __builtin_amdgcn_wave_barrier();
+    // lane k < n_used: candidate k, its rank among the candidates (probability descending, id ascending)
+    const bool own = lane < p.n_used;
+    const int my_cand = own ? cand[lane] : 0;
+    const float my_p = own ? ex[my_cand] : 0.0f;
+    int rank = 0;
+    for (int k = 0; k < p.n_used; k++) {
+        const float pk = readlane_f(my_p, k);
+        const int ik = __builtin_amdgcn_readlane(my_cand, k);
+        rank += (pk > my_p || (pk == my_p && ik < my_cand)) ? 1 : 0;
+    }
+    // into rank order through LDS (the exponentials' copy is no longer needed: probabilities live in ex[], this is ex + n)
+    float* by_rank_p = lds + n;
+    int32_t* by_rank_id = reinterpret_cast<int32_t*>(lds + n + 16);
+    if (own) {
+        by_rank_p[rank] = my_p;
+        by_rank_id[rank] = my_cand;
+    }
+    __builtin_amdgcn_wave_barrier();
+    int my_id = own ? by_rank_id[lane] : 0;
+    const float pk = own ? by_rank_p[lane] : 0.0f;
+    // routing weights (lib.rs:3856-3861): lane k owns rank k
+    float w;
+    if (p.norm_w) {
+        float wsum = 0.0f;
+        for (int k = 0; k < p.n_used; k++) wsum = __fadd_rn(wsum, readlane_f(pk, k));
+        wsum = fmaxf(wsum, 1e-20f);
+        w = __fmul_rn(__fdiv_rn(pk, wsum), p.scale);
+    } else {
+        w = __fmul_rn(pk, p.scale);
+    }
+    if (p.ep_n > 0) {
+        const bool in_band = my_id >= p.ep_lo && my_id < p.ep_lo + p.ep_n;
+        my_id = in_band ? my_id - p.ep_lo : 0;
+        w = in_band ? w : 0.0f;
+    }
+    if (own) {
+        if (store_global) {
+            p.ids[(size_t)row * p.n_used + lane] = my_id;
+            p.weights[(size_t)row * p.n_used + lane] = w;
+        }
+        if (lds_ids) lds_ids[lane] = my_id;
+        if (lds_w) lds_w[lane] = w;
+    }
+    if (p.probs && store_global) {
+#pragma unroll
+        for (int s = 0; s < NS; s++) p.probs[(size_t)row * n + s * kWave + lane] = pr[s];
+    }
+    return true;
+}
+
 // LDS floats route_row_any needs behind the 64-float exp table.
 __host__ __device__ inline size_t route_scratch_floats(int n_expert, int n_groups) {
     return (size_t)2 * n_expert + (size_t)(n_groups > 0 ? n_groups : 0);
