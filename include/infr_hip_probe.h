@@ -45,6 +45,11 @@ infr_status infr_hip_probe_dependent_reads(infr_hip_backend *be, const infr_hip_
  * number of such late experts over all launches of this backend so far (waits for the backend's stream). */
 infr_status infr_hip_probe_late_experts(infr_hip_backend *be, uint64_t *out);
 
+/* Tests, no counterpart in the reference.  *out receives how many calls into the allocating part of the HIP runtime
+ * (device memory, host memory, events) this library has made in this process so far, over all backends: a caller
+ * that must not allocate reads it before and after the calls it wants to vouch for. */
+infr_status infr_hip_probe_alloc_calls(uint64_t *out);
+
 #ifdef __cplusplus
 }
 #endif

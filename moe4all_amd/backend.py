@@ -229,6 +229,7 @@ _SIGNATURES = {
     "infr_hip_dequant": ([_V, _V, C.c_int32, C.c_uint64, _V], C.c_int),
     "infr_hip_moe_ffn_static": ([_V, C.POINTER(_MoeFfnStaticArgs)], C.c_int),
     "infr_hip_probe_late_experts": ([_V, C.POINTER(C.c_uint64)], C.c_int),
+    "infr_hip_probe_alloc_calls": ([C.POINTER(C.c_uint64)], C.c_int),
     "infr_hip_probe_dependent_reads": ([_V, _V, C.POINTER(C.c_uint64), C.c_uint32, C.c_uint32, C.POINTER(C.c_double),
                                         C.POINTER(C.c_double)], C.c_int),
 }
@@ -638,6 +639,12 @@ class Backend:
         """infr_hip_probe_late_experts: experts the single-launch kernel's guess missed and loaded late, so far."""
         n = C.c_uint64()
         _check(self._lib.infr_hip_probe_late_experts(self._h, C.byref(n)))
+        return int(n.value)
+
+    def alloc_calls(self) -> int:
+        """infr_hip_probe_alloc_calls: allocating runtime calls this library has made in this process so far."""
+        n = C.c_uint64()
+        _check(self._lib.infr_hip_probe_alloc_calls(C.byref(n)))
         return int(n.value)
 
     def probe_dependent_reads(self, pool: Buffer, stage_bytes: Sequence[int], iters: int = 200) -> dict:

@@ -69,6 +69,9 @@ infr_status guard_fail(const char* what) noexcept {
 static __device__ __align__(256) unsigned char scratch[INFR_HIP_STATIC_SCRATCH_BYTES];
 constexpr int kMaxDevices = 64;
 std::mutex g_scratch_mu;
+// Calls into the allocating part of the runtime made by this library (device and host memory, events), process-wide:
+// what the test of the entry point that allocates nothing reads before and after its calls.
+std::atomic<uint64_t> g_alloc_calls{0};
 void* g_scratch_ptr[kMaxDevices] = {};   // per device ordinal, filled by infr_hip_create with that device current
 
 constexpr uint64_t kBackendMagic = 0x494e465242454e44ull;  // "INFRBEND"
@@ -225,7 +228,8 @@ struct infr_hip_backend {
     // waits runs out; read after every stream synchronisation.  Once raised the backend keeps to the three-launch path.
     uint32_t* fault_host = nullptr;
     uint32_t* fault_dev = nullptr;
-    std::atomic<int> single_launch_off{0};
+    std::atomic<int> single_launch_off{0};   // MoeFfn ops that still take three launches after a single-launch kernel gave up
+    std::atomic<int> inorder_off{0};         // the in-order single-launch kernel stays off after it gave up (its sequence word did not advance)
     // The object outlives infr_hip_destroy while buffers or plans still point at it (the reference's buffers keep their
     // device alive the same way): destroy drains and closes the stream and drops the creator's reference, the last
     // buffer / plan freed afterwards deletes the object.
@@ -246,14 +250,18 @@ bool ok_buffer(const infr_hip_buffer* b) { return b && b->magic == kBufferMagic;
 bool ok_plan(const infr_hip_plan* p) { return p && p->magic == kPlanMagic; }
 
 // After a stream synchronisation: did a single-launch MoeFfn kernel give up a bounded wait?  The results of that
-// execute are not valid; the error is reported once and later executes use the three-launch path.
+// execute are not valid; the error is reported once and the next kSingleLaunchPause MoeFfn ops take three launches
+// (whatever shared the device has that long to finish) before the single-launch kernel is tried again.
+constexpr int kSingleLaunchPause = 256;
 infr_status check_fault(infr_hip_backend* be) {
     if (!be->fault_host || !*(volatile uint32_t*)be->fault_host) return INFR_OK;
     *(volatile uint32_t*)be->fault_host = 0;
-    be->single_launch_off.store(1);
+    be->single_launch_off.store(kSingleLaunchPause);
+    be->inorder_off.store(1);
     return fail(INFR_ERR_BACKEND,
                 "MoeFfn: the single-launch kernel timed out waiting for a peer workgroup (is the device shared or partitioned?); "
-                "the results since the last synchronisation are invalid, this backend now uses the three-launch path");
+                "the results since the last synchronisation are invalid: run those executes again (the next %d MoeFfn ops take the three-launch path)",
+                kSingleLaunchPause);
 }
 
 // Times one kernel launch when profiling is on: the events ride on the kernel's own dispatch
@@ -267,7 +275,7 @@ struct Timed {
         auto get = [&]() {
             hipEvent_t e = nullptr;
             if (!be->event_pool.empty()) { e = be->event_pool.back(); be->event_pool.pop_back(); }
-            else if (hipEventCreate(&e) != hipSuccess) e = nullptr;
+            else { g_alloc_calls++; if (hipEventCreate(&e) != hipSuccess) e = nullptr; }
             return e;
         };
         lt.start = get();
@@ -438,6 +446,7 @@ extern "C" infr_status infr_hip_create(int device_ordinal, const infr_hip_config
     {
         void* host = nullptr;
         void* dev = nullptr;
+        g_alloc_calls++;
         e = hipHostMalloc(&host, 64, hipHostMallocMapped);
         if (e == hipSuccess) {
             memset(host, 0, 64);
@@ -508,6 +517,7 @@ static infr_status alloc_impl(infr_hip_backend* be, size_t bytes, int32_t usage,
     std::lock_guard<std::mutex> lk(be->mu);
     HIP_TRY(hipSetDevice(be->device));
     void* p = nullptr;
+    g_alloc_calls++;
     hipError_t e = hipMalloc(&p, cap);
     if (e != hipSuccess)
         return fail(INFR_ERR_BACKEND, "alloc: hipMalloc(%zu) failed: %s", cap, hipGetErrorString(e));
@@ -1238,7 +1248,7 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
 
     std::lock_guard<std::mutex> lk(be->mu);
     hipError_t e = hipSetDevice(be->device);
-    if (e == hipSuccess && arena) e = hipMalloc(&plan->arena, arena);
+    if (e == hipSuccess && arena) { g_alloc_calls++; e = hipMalloc(&plan->arena, arena); }
     if (e != hipSuccess) return bail(INFR_ERR_BACKEND, std::string("compile: scratch hipMalloc failed: ") + hipGetErrorString(e));
     plan->arena_bytes = arena;
     for (uint32_t oi = 0; oi < g->n_ops; oi++) {
@@ -1492,7 +1502,13 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                                         plan->tensors[lq.weight].dtype, rb, (int)lq.m, (int)lq.in_f, (int)lq.out_f,
                                         (float*)ptr[lq.dst], n_cu);
                 };
-                if (sc.single_launch && !be->single_launch_off.load(std::memory_order_relaxed)) {
+                bool single = sc.single_launch != 0;
+                if (single && sc.single_launch == 1 && be->inorder_off.load(std::memory_order_relaxed)) single = false;
+                if (single && be->single_launch_off.load(std::memory_order_relaxed) > 0) {
+                    be->single_launch_off.fetch_sub(1, std::memory_order_relaxed);
+                    single = false;
+                }
+                if (single) {
                     infr::MoeLayerParams lp{};
                     lp.g = gp;
                     lp.g.route = rp;
@@ -1793,6 +1809,14 @@ extern "C" infr_status infr_hip_moe_ffn_static(infr_hip_backend* be, const infr_
     if (a->rows >= kBucketedMinRows || a->n_expert > 2048 || a->n_used > 64)
         return fail(INFR_ERR_UNSUPPORTED, "moe_ffn_static: %u token rows / %u experts / top-%u: the entry point takes 1..%u rows, "
                     "up to 2048 experts, top-64", a->rows, a->n_expert, a->n_used, kBucketedMinRows - 1);
+    // scratch layout: logits, probs [rows, n_expert]; ids, weights [rows, n_used]; h [rows, n_used, n_ff_exp]; y [rows, n_used, ne]
+    const size_t pairs = (size_t)a->rows * a->n_used;
+    const size_t sz_l = round_up((size_t)a->rows * a->n_expert * 4, 256), sz_p = round_up(pairs * 4, 256);
+    const size_t sz_h = round_up(pairs * a->n_ff_exp * 4, 256), sz_y = round_up(pairs * a->ne * 4, 256);
+    const size_t need = 2 * sz_l + 2 * sz_p + sz_h + sz_y;
+    if (need > INFR_HIP_STATIC_SCRATCH_BYTES)
+        return fail(INFR_ERR_UNSUPPORTED, "moe_ffn_static: these shapes need %zu bytes of scratch, the static scratch holds %u",
+                    need, (unsigned)INFR_HIP_STATIC_SCRATCH_BYTES);
     // operand extents against the shapes
     const int dts[3] = {a->gate_dtype, a->up_dtype, a->down_dtype};
     const uint32_t kdims[3] = {a->ne, a->ne, a->n_ff_exp};
@@ -1810,14 +1834,6 @@ extern "C" infr_status infr_hip_moe_ffn_static(infr_hip_backend* be, const infr_
     const size_t act_bytes = (size_t)a->rows * a->ne * 4, router_bytes = (size_t)a->n_expert * a->ne * 4;
     if (a->x->len < act_bytes || a->dst->len < act_bytes || a->router->len < router_bytes)
         return fail(INFR_ERR_INVALID, "moe_ffn_static: x / dst / router hold fewer bytes than [rows, ne] / [n_expert, ne] f32");
-    // scratch layout: logits, probs [rows, n_expert]; ids, weights [rows, n_used]; h [rows, n_used, n_ff_exp]; y [rows, n_used, ne]
-    const size_t pairs = (size_t)a->rows * a->n_used;
-    const size_t sz_l = round_up((size_t)a->rows * a->n_expert * 4, 256), sz_p = round_up(pairs * 4, 256);
-    const size_t sz_h = round_up(pairs * a->n_ff_exp * 4, 256), sz_y = round_up(pairs * a->ne * 4, 256);
-    const size_t need = 2 * sz_l + 2 * sz_p + sz_h + sz_y;
-    if (need > INFR_HIP_STATIC_SCRATCH_BYTES)
-        return fail(INFR_ERR_UNSUPPORTED, "moe_ffn_static: these shapes need %zu bytes of scratch, the static scratch holds %u",
-                    need, (unsigned)INFR_HIP_STATIC_SCRATCH_BYTES);
     std::lock_guard<std::mutex> lk(be->mu);
     HIP_TRY(hipSetDevice(be->device));
     char* sp = static_cast<char*>(be->static_scratch);   // the device address, never the array's name
@@ -1867,6 +1883,7 @@ extern "C" infr_status infr_hip_probe_dependent_reads(infr_hip_backend* be, cons
     std::lock_guard<std::mutex> lk(be->mu);
     HIP_TRY(hipSetDevice(be->device));
     uint32_t* ctl = nullptr;
+    g_alloc_calls += 3;
     HIP_TRY(hipMalloc(&ctl, 256));
     hipEvent_t a = nullptr, b = nullptr;
     hipError_t e = hipEventCreate(&a);
@@ -1909,6 +1926,12 @@ extern "C" infr_status infr_hip_probe_late_experts(infr_hip_backend* be, uint64_
     *out = be->fault_host ? ((volatile uint32_t*)be->fault_host)[1] : 0;
     return INFR_OK;
 } catch (...) { return guard_fail("infr_hip_probe_late_experts"); }
+
+extern "C" infr_status infr_hip_probe_alloc_calls(uint64_t* out) try {
+    if (!out) return fail(INFR_ERR_INVALID, "probe: out is null");
+    *out = g_alloc_calls.load();
+    return INFR_OK;
+} catch (...) { return guard_fail("infr_hip_probe_alloc_calls"); }
 
 extern "C" infr_status infr_hip_probe_grouped_loads_only(infr_hip_backend* be, int on) try {
     if (!ok_backend(be)) return fail(INFR_ERR_INVALID, "probe: bad handle");
@@ -1955,6 +1978,7 @@ extern "C" infr_status infr_hip_plan_moe_routing(infr_hip_backend* be, const inf
     std::lock_guard<std::mutex> lk(be->mu);
     HIP_TRY(hipSetDevice(be->device));
     HIP_TRY(hipStreamSynchronize(be->stream));
+    if (infr_status st = check_fault(be)) return st;
     size_t rows = (size_t)sc.rows;
     if (rows == 0) return INFR_OK;
     if (ids) HIP_TRY(hipMemcpy(ids, sc.ids, rows * m.n_used * 4, hipMemcpyDeviceToHost));
@@ -1976,6 +2000,7 @@ extern "C" infr_status infr_hip_plan_moe_bucketing(infr_hip_backend* be, const i
     std::lock_guard<std::mutex> lk(be->mu);
     HIP_TRY(hipSetDevice(be->device));
     HIP_TRY(hipStreamSynchronize(be->stream));
+    if (infr_status st = check_fault(be)) return st;
     const size_t pairs = (size_t)sc.rows * m.n_used;
     if (offsets) HIP_TRY(hipMemcpy(offsets, sc.offsets, ((size_t)m.n_expert + 1) * 4, hipMemcpyDeviceToHost));
     if (pair_src) HIP_TRY(hipMemcpy(pair_src, sc.pair_src, pairs * 4, hipMemcpyDeviceToHost));

@@ -397,12 +397,7 @@ void launch_moe_units_bucketed_t(hipStream_t s, const MoeGemvParams& p, int n_pa
     int be = 1, bb = 4;
     block_geometry(DT, &be, &bb);
     const size_t row_bytes = (size_t)(in_f / be) * bb;
-    static bool attr_set = false;
-    if (!attr_set) {
-        (void)hipFuncSetAttribute((const void*)moe_units_bucketed_kernel<DT, GATE_UP, T>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  160 * 1024);
-        attr_set = true;
-    }
+    INFR_LDS_LIMIT((moe_units_bucketed_kernel<DT, GATE_UP, T>), 160 * 1024);
     const int n_tiles = (out_f + kRowsPerBlock - 1) / kRowsPerBlock;
     // every expert with tokens has at most one ragged chunk: chunks <= pairs / T + min(experts, pairs)
     const long items = (long)n_pairs / T + (p.n_expert < n_pairs ? p.n_expert : n_pairs);
@@ -539,12 +534,7 @@ template <int DT, int TILE>
 void launch_moe_down_combine_units_t(hipStream_t s, const MoeGemvParams& p) {
     int be = 1, bb = 4;
     block_geometry(DT, &be, &bb);
-    static bool attr_set = false;
-    if (!attr_set) {
-        (void)hipFuncSetAttribute((const void*)moe_down_combine_units_kernel<DT, TILE>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  158 * 1024);
-        attr_set = true;
-    }
+    INFR_LDS_LIMIT((moe_down_combine_units_kernel<DT, TILE>), 158 * 1024);
     dim3 grid((p.ne + TILE - 1) / TILE, p.rows), block(1024);
     INFR_LAUNCH((moe_down_combine_units_kernel<DT, TILE>), grid, block, down_combine_units_lds(p), s, p, (size_t)(p.nff / be) * bb);
 }
@@ -562,11 +552,7 @@ void launch_moe_units_dt(hipStream_t s, const MoeGemvParams& p) {
     int be = 1, bb = 4;
     block_geometry(DT, &be, &bb);
     const size_t row_bytes = (size_t)(in_f / be) * bb;
-    static bool attr_set = false;
-    if (!attr_set) {
-        (void)hipFuncSetAttribute((const void*)moe_units_kernel<DT, GATE_UP>, hipFuncAttributeMaxDynamicSharedMemorySize, 158 * 1024);
-        attr_set = true;
-    }
+    INFR_LDS_LIMIT((moe_units_kernel<DT, GATE_UP>), 158 * 1024);
     // output rows of a block (kRB in the kernel): 16, or 8 for gate/up when that still leaves the compute units short
     // of two blocks each (one round per block instead of two serial ones; C2 shape, one row: 11.5 -> 10.1 us)
     const int blocks16 = ((out_f + kRowsPerBlock - 1) / kRowsPerBlock) * p.rows * p.n_used;
@@ -593,11 +579,7 @@ template <int DT, int T>
 void launch_units(hipStream_t s, const float* x, const uint8_t* w, size_t row_bytes, int m, int in_f, int out_f, float* dst,
                   const float* addend) {
     const size_t lds = units_lds_bytes(T, in_f);
-    static bool attr_set = false;
-    if (!attr_set) {
-        (void)hipFuncSetAttribute((const void*)linear_units_kernel<DT, T>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        attr_set = true;
-    }
+    INFR_LDS_LIMIT((linear_units_kernel<DT, T>), 160 * 1024);
     // 16 output rows per block, or 8 (one round instead of two serial ones) while the grid would be small
     const int gy = (m + T - 1) / T;
     const int rb = ((out_f + kRowsPerBlock - 1) / kRowsPerBlock) * gy < 512 ? 8 : kRowsPerBlock;
@@ -698,11 +680,7 @@ __global__ __launch_bounds__(256) void linear_float_kernel(const float* __restri
 template <int DT, int T>
 void launch_float(hipStream_t s, const float* x, const uint8_t* w, size_t row_bytes, int m, int in_f, int out_f, float* dst,
                   const float* addend) {
-    static bool attr_set = false;
-    if (!attr_set) {
-        (void)hipFuncSetAttribute((const void*)linear_float_kernel<DT, T>, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        attr_set = true;
-    }
+    INFR_LDS_LIMIT((linear_float_kernel<DT, T>), 160 * 1024);
     dim3 grid((out_f + kRowsPerBlock - 1) / kRowsPerBlock, (m + T - 1) / T), block(256);
     INFR_LAUNCH((linear_float_kernel<DT, T>), grid, block, (size_t)T * (in_f + 4) * sizeof(float), s, x, w, row_bytes, m, in_f,
                 out_f, dst, addend);

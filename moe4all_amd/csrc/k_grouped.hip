@@ -229,8 +229,10 @@ __global__ __launch_bounds__(256) void bucket_kernel(const int32_t* __restrict__
 // reads against them: one explicit "s_waitcnt vmcnt(n); s_barrier" per slice does both.  The issue
 // order is fixed (the same number of loads in every even and in every odd slice), so the number
 // of loads younger than the ones slice s needs is a compile-time constant.
-// M0 carries the LDS base of the transfer.  Nothing else in these kernels uses M0 (no other LDS-direct
-// load, no indirect register addressing, no message), so it is not saved around the load.
+// M0 carries the LDS base of the transfer.  The statement writes M0 immediately before its only use, and nothing
+// else in these kernels uses M0 (no other LDS-direct load, no indirect register addressing, no message), so no
+// value of the compiler's can be live in it across the statement.  M0 cannot be named as a clobber: the compiler
+// reserves the register and warns that it does not honour such a clobber.
 #ifndef INFR_ABLATE
 #define INFR_ABLATE 0
 #endif
@@ -778,14 +780,8 @@ void grouped6(hipStream_t s, const GroupedParams& p) {
     q.n_tiles_n = (p.N + bn - 1) / bn;
     const int max_tiles = p.n_pairs / kBM + (p.n_expert < p.n_pairs ? p.n_expert : p.n_pairs);
     const dim3 grid((unsigned)((max_tiles * q.n_tiles_n + 7) & ~7));   // whole rounds of the 8 XCDs
-    static bool attr_set = false;  // per instantiation
-    if (!attr_set) {
-        (void)hipFuncSetAttribute((const void*)grouped_mfma6<D, DOWN>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  (int)grouped6_lds<D>());
-        (void)hipFuncSetAttribute((const void*)grouped_mfma6<D, DOWN, 12>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  (int)grouped6_lds<D>());
-        attr_set = true;
-    }
+    INFR_LDS_LIMIT((grouped_mfma6<D, DOWN>), (int)grouped6_lds<D>());
+    INFR_LDS_LIMIT((grouped_mfma6<D, DOWN, 12>), (int)grouped6_lds<D>());
     // loads_only: the measurement variant without unpacking and matrix instructions (its output is meaningless)
     if (p.loads_only) INFR_LAUNCH((grouped_mfma6<D, DOWN, 12>), grid, dim3(512), grouped6_lds<D>(), s, q);
     else INFR_LAUNCH((grouped_mfma6<D, DOWN>), grid, dim3(512), grouped6_lds<D>(), s, q);

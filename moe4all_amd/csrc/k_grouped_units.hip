@@ -376,12 +376,7 @@ void grouped_units(hipStream_t s, const GroupedParams& p) {
     GroupedParams q = p;
     q.n_tiles_n = (p.N + bn - 1) / bn;
     const int max_tiles = p.n_pairs / kBM + (p.n_expert < p.n_pairs ? p.n_expert : p.n_pairs);
-    static bool attr_set = false;
-    if (!attr_set && StagedW<DT>::kLds) {
-        (void)hipFuncSetAttribute((const void*)grouped_units_mfma<DT, DOWN>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                  (int)StagedW<DT>::kLds);
-        attr_set = true;
-    }
+    if (StagedW<DT>::kLds) INFR_LDS_LIMIT((grouped_units_mfma<DT, DOWN>), (int)StagedW<DT>::kLds);
     INFR_LAUNCH((grouped_units_mfma<DT, DOWN>), dim3((unsigned)((max_tiles * q.n_tiles_n + 7) & ~7)), dim3(256), StagedW<DT>::kLds,
                 s, q);
 }

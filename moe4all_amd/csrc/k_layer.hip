@@ -544,11 +544,7 @@ bool layer_shape(const MoeLayerParams& q, LayerShape* out) {
 
 template <class FG, class FD, int U, int S, int EPB, int NH>
 void launch_layer(hipStream_t s, const MoeLayerParams& q, size_t lds) {
-    static bool attr_set = false;
-    if (!attr_set) {
-        (void)hipFuncSetAttribute((const void*)moe_layer_fused<FG, FD, U, S, EPB, NH>, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
-        attr_set = true;
-    }
+    INFR_LDS_LIMIT((moe_layer_fused<FG, FD, U, S, EPB, NH>), 150 * 1024);
     INFR_LAUNCH((moe_layer_fused<FG, FD, U, S, EPB, NH>), dim3(kLayerBlocks), dim3(256), lds, s, q);
 }
 

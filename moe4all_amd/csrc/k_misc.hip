@@ -198,6 +198,7 @@ __global__ __launch_bounds__(256) void probe_dependent_read_kernel(const uint8_t
     int issued = 0;
     for (int i = wave; i < n_copies; i += 4) {
         const uint32_t lds_at = __builtin_amdgcn_readfirstlane(base + (uint32_t)(i % 128) * 1024u);
+        // M0 is written right before its only use; it cannot be listed as a clobber (the compiler reserves it)
         asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(mine + (size_t)i * 1024 + lane * 16), "s"(lds_at) : "memory");
         if (++issued == 32) {   // the LDS window holds 128 copies: four waves x 32
             asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -212,11 +213,7 @@ __global__ __launch_bounds__(256) void probe_dependent_read_kernel(const uint8_t
 
 void launch_probe_dependent_read(hipStream_t s, const uint8_t* pool, uint64_t pool_bytes, uint64_t bytes, uint32_t* ctl,
                                  uint32_t salt, int n_cu) {
-    static bool attr_set = false;
-    if (!attr_set) {
-        (void)hipFuncSetAttribute((const void*)probe_dependent_read_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
-        attr_set = true;
-    }
+    INFR_LDS_LIMIT((probe_dependent_read_kernel), 128 * 1024);
     uint64_t blocks = bytes >> 10;   // at least one 1 KB copy per block
     if (blocks > (uint64_t)n_cu) blocks = (uint64_t)n_cu;
     if (blocks < 1) blocks = 1;

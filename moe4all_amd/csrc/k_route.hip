@@ -386,12 +386,7 @@ bool launch_router_logits(hipStream_t s, const uint8_t* router, int rdt, size_t 
     dim3 grid(gx, gy), block(256);
 #define LAUNCH_RL(E)                                                                                               \
     do {                                                                                                           \
-        static bool attr_set = false;                                                                              \
-        if (!attr_set) {                                                                                           \
-            (void)hipFuncSetAttribute((const void*)router_logits_kernel<E>,                                         \
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)budget);                   \
-            attr_set = true;                                                                                       \
-        }                                                                                                          \
+        INFR_LDS_LIMIT((router_logits_kernel<E>), (int)budget); \
         INFR_LAUNCH(router_logits_kernel<E>, grid, block, lds, s, router, rdt, row_bytes, x, ne, n_expert,  \
                            rows, rpb, logits, nrm);                                                   \
     } while (0)

@@ -8,6 +8,8 @@
 
 #include <hip/hip_ext.h>
 
+#include <atomic>
+
 namespace infr {
 
 // Per-kernel timing.  While a thread has tl_launch_timing set, every launch it makes through
@@ -23,6 +25,22 @@ extern thread_local const LaunchTiming* tl_launch_timing;
         const ::infr::LaunchTiming* lt_ = ::infr::tl_launch_timing;                                              \
         if (lt_) hipExtLaunchKernelGGL(kernel, grid, block, lds, stream, lt_->start, lt_->stop, 0, __VA_ARGS__); \
         else hipLaunchKernelGGL(kernel, grid, block, lds, stream, __VA_ARGS__);                                  \
+    } while (0)
+
+// Raises a kernel's limit of dynamic LDS once per device and kernel (`done`: one bit per device ordinal).  When the
+// runtime refuses, the bit stays clear and the launch that follows fails with the runtime's own error, which the
+// entry point that made the launch reports.
+inline void lds_limit(const void* kernel, int bytes, std::atomic<uint32_t>& done) {
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 32) return;
+    if (done.load(std::memory_order_relaxed) >> dev & 1u) return;
+    if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) == hipSuccess)
+        done.fetch_or(1u << dev, std::memory_order_relaxed);
+}
+#define INFR_LDS_LIMIT(kernel, bytes)                                       \
+    do {                                                                    \
+        static std::atomic<uint32_t> lds_limit_done_{0};                    \
+        ::infr::lds_limit((const void*)kernel, (bytes), lds_limit_done_);   \
     } while (0)
 
 // An Op::RmsNorm of the single token row folded into the logits kernel: x is the raw row, every
