@@ -75,6 +75,39 @@ __device__ __forceinline__ void rec_store_xcd(uint64_t* p, float v, uint32_t tag
 // Wave-wide: gathers rec[0 .. n) (n a multiple of 64, n <= 64 N) into out[] once all carry `tag`.  Every poll issues
 // all of a lane's loads before it looks at any of them, so a poll costs one round trip (two polls in flight half a
 // round trip apart were measured slower: the polls of 256 workgroups share one path).  False: spin limit.
+// Outcome of gather_activations below.
+enum : int { kGathered = 0, kGatherTimeout = 1, kGatherSuperseded = 2 };
+// gather_records for the activations of a group, whose records carry the expert they were computed for: a record of
+// this launch with ANOTHER expert's code means that its writer has seen the exact routing name a different expert for
+// the group and has started over; the records wanted here will not come, and this workgroup is about to see the same
+// routing.  kGatherSuperseded then, with out[] unspecified.  first_pass false: the group is on its second and last pass,
+// and a record with another code is one of the first pass that its writer has not replaced yet.
+template <int N>
+__device__ __forceinline__ int gather_activations(const uint64_t* rec, int n, uint32_t tag, float* out, int lane, int spin_limit,
+                                                  bool first_pass) {
+    uint64_t r[N];
+    const int ns = n >> 6;
+    int state = kGathered;
+    for (int spin = 0;; spin++) {
+#pragma unroll
+        for (int s = 0; s < N; s++) r[s] = s < ns ? rec_load(rec + s * kWave + lane) : ((uint64_t)tag << 32);
+        bool ok = true, other = false;
+#pragma unroll
+        for (int s = 0; s < N; s++) {
+            const uint32_t t = (uint32_t)(r[s] >> 32);
+            ok = ok && t == tag;
+            other = other || (t != tag && (t >> 9) == (tag >> 9));
+        }
+        if (__all(ok)) break;
+        if (first_pass && __any(other)) { state = kGatherSuperseded; break; }
+        if (spin >= spin_limit) return kGatherTimeout;
+    }
+#pragma unroll
+    for (int s = 0; s < N; s++)
+        if (s < ns) out[s * kWave + lane] = __uint_as_float((uint32_t)r[s]);
+    return state;
+}
+
 template <int N>
 __device__ __forceinline__ bool gather_records(const uint64_t* rec, int n, uint32_t tag, float* out, int lane, int spin_limit) {
     uint64_t r[N];
@@ -455,7 +488,7 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
         const int my_sdi = n_sdi > ssw ? (n_sdi - ssw + kSW - 1) / kSW : 0;
 
         GuItem gring[DG];
-        auto sh_issue = [&]() {
+        auto sh_issue = [&]() __attribute__((always_inline)) {
             const int f = sf0 + min(sw * pg.rw_count + pg.rw, sfpb - 1);
             gring[0].g = load_row<FG>(pg, p.sh_gate + (size_t)f * rb_g);
             gring[0].u = load_row<FG>(pg, p.sh_up + (size_t)f * rb_g);
@@ -484,7 +517,7 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
         typename FD::Raw dring[DD];
         int e_cur = alive ? __builtin_amdgcn_readfirstlane(s_spec[g]) : 0;
         const uint8_t* dbank = nullptr;
-        auto dn_issue = [&](int slot, int j) {
+        auto dn_issue = [&](int slot, int j) __attribute__((always_inline)) {
             const bool routed = j < my_di || !shared;   // items past the end re-read a last row
             const int jj = routed ? j : j - my_di;
             const int lim = routed ? R : SR;
@@ -492,19 +525,27 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
             const uint8_t* base = routed ? dbank + (size_t)(m * R + orow) * rb_d : p.sh_down + (size_t)(b * SR + orow) * rb_d;
             dring[slot] = load_row<FD>(pd, base);
         };
-        if (alive) {
-            for (int attempt = 0;; attempt++) {
-                const uint8_t* gb = p.gate + (size_t)e_cur * p.gate_stride + (size_t)f0 * rb_g;
-                const uint8_t* ub = p.up + (size_t)e_cur * p.up_stride + (size_t)f0 * rb_g;
-                dbank = p.down + (size_t)e_cur * p.down_stride;
-                const int sh = attempt == 0 ? sh_n : 0;   // ring entries ahead of the expert's items
+        // One pass per expert this group works on: the guessed one, and once more if the exact routing names another.
+        // A pass does not wait for the routing: the group's activations carry the expert they were computed for, so
+        // the members of a group meet on the guess, and the down rows' results carry it too, so nobody consumes a
+        // result of an expert the routing did not select.  The routing is looked at after the pass (and, without
+        // waiting, before the down stage, which is skipped when it is already known to be for nothing).
+        const int chunk = nff / 6;   // records per gathering wavefront: a multiple of 64
+        // (two straight-line copies of the pass instead of a loop: a loop's invariant addresses would stay in registers
+        // across the whole pass and spill)
+        auto run_pass = [&](const int attempt) __attribute__((always_inline)) -> bool {   // true: once more, with e_cur renewed
+            const uint8_t* gb = p.gate + (size_t)e_cur * p.gate_stride + (size_t)f0 * rb_g;
+            const uint8_t* ub = p.up + (size_t)e_cur * p.up_stride + (size_t)f0 * rb_g;
+            dbank = p.down + (size_t)e_cur * p.down_stride;
+            const int sh = attempt == 0 ? sh_n : 0;   // ring entries ahead of the expert's items
+            {
                 typename FG::X x;   // fetched again on a second pass: not kept alive across the hand-over
-                auto gu_issue = [&](int slot, int j) {
+                auto gu_issue = [&](int slot, int j) __attribute__((always_inline)) {
                     const int f = min(((j - sh) * kSW + sw) * pg.rw_count + pg.rw, fpb - 1);
                     gring[slot].g = load_row<FG>(pg, gb + (size_t)f * rb_g);
                     gring[slot].u = load_row<FG>(pg, ub + (size_t)f * rb_g);
                 };
-                auto gu_finish = [&](int slot, int j) {
+                auto gu_finish = [&](int slot, int j) __attribute__((always_inline)) {
                     const float gs = row_sum<FG>(FG::dot(gring[slot].g, pg.sub, x), pg, nblk_g);
                     const float us = row_sum<FG>(FG::dot(gring[slot].u, pg.sub, x), pg, nblk_g);
                     if (j < sh) {   // the always-on expert's item: its activation goes to every workgroup
@@ -525,107 +566,116 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
                 if (attempt == 0) wait_cells();
                 FG::fetch_x(x, cells, pg.blk, pg.sub);
                 ring_drain<DG>(sh + my_gi, gu_issue, gu_finish);
-                if (wave == 3) STAMP(6);
-                __builtin_amdgcn_wave_barrier();
-                if (lane < my_gi * pg.rw_count) {
-                    const int j = lane / pg.rw_count, rw = lane - j * pg.rw_count;
-                    const int fi = (j * kSW + sw) * pg.rw_count + rw;
-                    if (fi < fpb)
-                        rec_store_xcd(q.xh + (size_t)g * nff + f0 + fi,
-                                      gated_act_fn(p.act, p.has_clamp, p.clamp, s_g[wave][lane], s_u[wave][lane], s_tab),
-                                      seq_tag | (uint32_t)e_cur, true);
-                }
-                __builtin_amdgcn_wave_barrier();
-                if (wave == 3) STAMP(7);
-                if (wave == 1) STAMP(21);
-                if (wave == 7) STAMP(22);
-                if (lds_flag_wait(&s_f_route) != 1) {
-                    alive = false;
-                    break;
-                }
-                if (wave == 3) STAMP(8);
-                const int e_fin = __builtin_amdgcn_readfirstlane(s_final[g]);
-                if (e_fin == e_cur) break;
-                e_cur = e_fin;   // the guess missed this group's expert: once more with the right one
             }
-        }
-        // ---- hand-over of the group's activations: six wavefronts gather a sixth each and turn it into cells; the
-        // seventh gathers the always-on expert's meanwhile (written long ago by all 256 workgroups)
-        const int chunk = nff / 6;   // records per gathering wavefront: a multiple of 64
-        if (sw < 6) {
-            bool ok = alive;
-            if (ok) ok = gather_records<4>(q.xh + (size_t)g * nff + sw * chunk, chunk, seq_tag | (uint32_t)e_cur, s_h + sw * chunk, lane, spin_limit);
-            if (wave == 1) STAMP(9);
-            if (ok) {
-                __builtin_amdgcn_wave_barrier();
-                if (lane * 8 < chunk) {   // whole groups of four lanes
-                    const int oct = sw * (chunk >> 3) + lane;
-                    const float4 lo = *reinterpret_cast<const float4*>(s_h + 8 * oct), hi = *reinterpret_cast<const float4*>(s_h + 8 * oct + 4);
-                    octet_to_cell<FD::kGroup, FD::kSigned>(lo, hi, oct, hcells);
-                }
-            } else if (alive && lane == 0) {
-                s_fault = 1;
-                __hip_atomic_store(q.fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            if (wave == 3) STAMP(6);
+            __builtin_amdgcn_wave_barrier();
+            if (lane < my_gi * pg.rw_count) {
+                const int j = lane / pg.rw_count, rw = lane - j * pg.rw_count;
+                const int fi = (j * kSW + sw) * pg.rw_count + rw;
+                if (fi < fpb)
+                    rec_store_xcd(q.xh + (size_t)g * nff + f0 + fi,
+                                  gated_act_fn(p.act, p.has_clamp, p.clamp, s_g[wave][lane], s_u[wave][lane], s_tab),
+                                  seq_tag | (uint32_t)e_cur, true);
             }
-            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-            if (lane == 0) __hip_atomic_fetch_add(&s_h_done, ok ? 1 : 0x101, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-            if (wave == 1) STAMP(10);
+            __builtin_amdgcn_wave_barrier();
+            if (wave == 3) STAMP(7);
+            if (wave == 1) STAMP(21);
+            if (wave == 7) STAMP(22);
+            // ---- hand-over of the group's activations: six wavefronts gather a sixth each and turn it into cells; the
+            // seventh gathers the always-on expert's meanwhile (written long ago by all 256 workgroups)
+            bool superseded = false;
+            if (sw < 6) {
+                const int st = gather_activations<4>(q.xh + (size_t)g * nff + sw * chunk, chunk, seq_tag | (uint32_t)e_cur,
+                                                     s_h + sw * chunk, lane, spin_limit, attempt == 0);
+                if (wave == 1) STAMP(9);
+                superseded = st == kGatherSuperseded;
+                if (st == kGathered) {
+                    __builtin_amdgcn_wave_barrier();
+                    if (lane * 8 < chunk) {   // whole groups of four lanes
+                        const int oct = sw * (chunk >> 3) + lane;
+                        const float4 lo = *reinterpret_cast<const float4*>(s_h + 8 * oct), hi = *reinterpret_cast<const float4*>(s_h + 8 * oct + 4);
+                        octet_to_cell<FD::kGroup, FD::kSigned>(lo, hi, oct, hcells);
+                    }
+                } else if (st == kGatherTimeout && lane == 0) {
+                    s_fault = 1;
+                    __hip_atomic_store(q.fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                if (lane == 0)
+                    __hip_atomic_fetch_add(&s_h_done, st == kGatherTimeout ? 0x101 : 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+                if (wave == 1) STAMP(10);
+            } else if (shared && attempt == 0) {
+                bool ok = gather_records<24>(q.xs, nff, tag, s_hs, lane, spin_limit);
+                if (ok) {
+                    __builtin_amdgcn_wave_barrier();
+                    for (int oct = lane; oct * 8 < nff; oct += kWave) {
+                        const float4 lo = *reinterpret_cast<const float4*>(s_hs + 8 * oct), hi = *reinterpret_cast<const float4*>(s_hs + 8 * oct + 4);
+                        octet_to_cell<FD::kGroup, FD::kSigned>(lo, hi, oct, hscells);
+                    }
+                } else if (lane == 0) {
+                    s_fault = 1;
+                    __hip_atomic_store(q.fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                }
+                lds_flag_set(&s_f_hs, ok ? 1 : 2);
+                alive = ok;
+            }
             // the first down rows, requested behind the polls: a poll issued behind them would not return before them
             if (!q.early_down && alive) ring_prime<DD>(dn_issue);
-        } else if (shared) {
-            bool ok = alive;
-            if (ok) ok = gather_records<24>(q.xs, nff, tag, s_hs, lane, spin_limit);
-            if (ok) {
-                __builtin_amdgcn_wave_barrier();
-                for (int oct = lane; oct * 8 < nff; oct += kWave) {
-                    const float4 lo = *reinterpret_cast<const float4*>(s_hs + 8 * oct), hi = *reinterpret_cast<const float4*>(s_hs + 8 * oct + 4);
-                    octet_to_cell<FD::kGroup, FD::kSigned>(lo, hi, oct, hscells);
-                }
-            } else if (alive && lane == 0) {
-                s_fault = 1;
-                __hip_atomic_store(q.fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            {
+                int v;
+                while ((((v = __builtin_amdgcn_readfirstlane(*(volatile int*)&s_h_done)) & 0xFF) < 6 * (attempt + 1)) && !(v >> 8))
+                    __builtin_amdgcn_s_sleep(1);
+                asm volatile("" ::: "memory");
+                if (v >> 8) alive = false;
             }
-            lds_flag_set(&s_f_hs, ok ? 1 : 2);
-            alive = alive && ok;
-            if (!q.early_down && alive) ring_prime<DD>(dn_issue);
-        } else if (!q.early_down && alive) {
-            ring_prime<DD>(dn_issue);
-        }
-        {
-            int v;
-            while (((v = __builtin_amdgcn_readfirstlane(*(volatile int*)&s_h_done)) & 0xFF) < 6) __builtin_amdgcn_s_sleep(1);
+            // is this pass already known to be for another expert than the routing's?  (the same answer in every
+            // wavefront is not needed: the down stage has no hand-over between wavefronts)
+            int routed = __builtin_amdgcn_readfirstlane(*(volatile int*)&s_f_route);
             asm volatile("" ::: "memory");
-            if (v >> 8) alive = false;
-        }
-        if (alive) {
-            // ---- down: rows of the group's expert, then of the always-on expert
-            typename FD::X xd;
-            FD::fetch_x(xd, hcells, pd.blk, pd.sub);
-            const bool scaled = p.down_scale != nullptr;
-            const float ds = scaled ? p.down_scale[e_cur] : 1.0f;
-            uint64_t* part = q.ypart + (size_t)g * ne + (size_t)m * R;
-            bool on_shared = false;
-            auto dn_finish = [&](int slot, int j) {
-                const bool routed = j < my_di;
-                if (!routed && !on_shared) {   // the same for the whole wavefront
-                    on_shared = true;
-                    if (sw != 6 && lds_flag_wait(&s_f_hs) != 1) alive = false;
-                    FD::fetch_x(xd, hscells, pd.blk, pd.sub);
-                }
-                const int jj = routed ? j : j - my_di;
-                const int orow = (jj * kSW + (routed ? sw : ssw)) * pd.rw_count + pd.rw;
-                const float y = row_sum<FD>(FD::dot(dring[slot], pd.sub, xd), pd, nblk_d);
-                if (pd.writer()) {
-                    if (routed) {
-                        if (orow < R) rec_store(part + orow, scaled ? __fmul_rn(y, ds) : y, tag);
-                    } else if (orow < SR) {
-                        s_ysh[orow] = y;
+            const bool in_vain = superseded || routed == 2 || (routed == 1 && __builtin_amdgcn_readfirstlane(s_final[g]) != e_cur);
+            if (alive && !in_vain) {
+                // ---- down: rows of the group's expert, then of the always-on expert
+                typename FD::X xd;
+                FD::fetch_x(xd, hcells, pd.blk, pd.sub);
+                const bool scaled = p.down_scale != nullptr;
+                const float ds = scaled ? p.down_scale[e_cur] : 1.0f;
+                uint64_t* part = q.ypart + (size_t)g * ne + (size_t)m * R;
+                const uint32_t ytag = seq_tag | (uint32_t)e_cur;
+                bool on_shared = false;
+                auto dn_finish = [&](int slot, int j) __attribute__((always_inline)) {
+                    const bool own = j < my_di;
+                    if (!own && !on_shared) {   // the same for the whole wavefront
+                        on_shared = true;
+                        if (sw != 6 && lds_flag_wait(&s_f_hs) != 1) alive = false;
+                        FD::fetch_x(xd, hscells, pd.blk, pd.sub);
                     }
-                }
-            };
-            ring_drain<DD>(my_di + my_sdi, dn_issue, dn_finish);
-            if (wave == 3) STAMP(11);
-        }
+                    const int jj = own ? j : j - my_di;
+                    const int orow = (jj * kSW + (own ? sw : ssw)) * pd.rw_count + pd.rw;
+                    const float y = row_sum<FD>(FD::dot(dring[slot], pd.sub, xd), pd, nblk_d);
+                    if (pd.writer()) {
+                        if (own) {
+                            if (orow < R) rec_store(part + orow, scaled ? __fmul_rn(y, ds) : y, ytag);
+                        } else if (orow < SR) {
+                            s_ysh[orow] = y;
+                        }
+                    }
+                };
+                ring_drain<DD>(my_di + my_sdi, dn_issue, dn_finish);
+                if (wave == 3) STAMP(11);
+            }
+            if (!alive) return false;
+            routed = lds_flag_wait(&s_f_route);
+            if (wave == 3) STAMP(8);
+            if (routed != 1) {
+                alive = false;
+                return false;
+            }
+            const int e_fin = __builtin_amdgcn_readfirstlane(s_final[g]);
+            if (e_fin == e_cur) return false;
+            e_cur = e_fin;   // the guess missed this group's expert: once more with the right one
+            return true;
+        };
+        if (alive && run_pass(0)) run_pass(1);
         // this wavefront's rows of the always-on expert are in LDS: tell the summing wavefront
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         if (lane == 0) __hip_atomic_fetch_add(&s_done, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
@@ -646,7 +696,7 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
                 for (int k = 0; k < kGroups; k++) yk[k] = rec_load(q.ypart + (size_t)s_gor[k] * ne + oi);   // rank order
                 bool got = true;
 #pragma unroll
-                for (int k = 0; k < kGroups; k++) got = got && (uint32_t)(yk[k] >> 32) == tag;
+                for (int k = 0; k < kGroups; k++) got = got && (uint32_t)(yk[k] >> 32) == (seq_tag | (uint32_t)s_ids[k]);
                 if (__all(got || !mine)) break;
                 if (spin >= spin_limit) {
                     ok = false;
