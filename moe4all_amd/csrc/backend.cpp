@@ -1205,9 +1205,9 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
             if (kind != infr_hip_plan::kPlain && kind != infr_hip_plan::kMoeShared) continue;
             const infr_op_moe_ffn& m = plan->ops[oi].u.moe_ffn;
             MoeScratch& sc = plan->moe[oi];
-            if (sc.rows != 1 || sc.batched || sc.bucketed || c.dt(m.router) != INFR_F32) continue;
+            if ((sc.rows != 1 && sc.rows != 2 && sc.rows != 4) || sc.batched || sc.bucketed || c.dt(m.router) != INFR_F32) continue;
             infr::MoeLayerParams probe{};
-            probe.g.rows = 1; probe.g.ne = (int)m.ne; probe.g.nff = (int)m.n_ff_exp; probe.g.n_used = (int)m.n_used;
+            probe.g.rows = sc.rows; probe.g.ne = (int)m.ne; probe.g.nff = (int)m.n_ff_exp; probe.g.n_used = (int)m.n_used;
             probe.g.n_expert = (int)(m.has_ep_band ? m.ep_n_local : m.n_expert);
             probe.g.gate_dt = c.dt(m.gate_exps);
             probe.g.up_dt = m.fused_gate_up ? probe.g.gate_dt : c.dt(m.up_exps);
@@ -1226,7 +1226,7 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
             if (kind == infr_hip_plan::kMoeShared) probe.g.sh_gate = probe.g.sh_up = probe.g.sh_down = (const uint8_t*)plan;
             if (!be->cfg.disable_single_launch_guess && infr::moe_layer_stream_supported(probe)) {
                 sc.single_launch = 2;
-                stream_ws = std::max(stream_ws, infr::moe_layer_stream_workspace_bytes((int)m.ne, (int)m.n_ff_exp, (int)m.n_expert));
+                stream_ws = std::max(stream_ws, infr::moe_layer_stream_workspace_bytes((int)m.ne, (int)m.n_ff_exp, (int)m.n_expert, sc.rows));
             } else if (kind == infr_hip_plan::kPlain && infr::moe_layer_fused_supported(probe)) {
                 sc.single_launch = 1;
                 layer_ws = std::max(layer_ws, infr::moe_layer_workspace_bytes((int)m.ne, (int)m.n_ff_exp, (int)m.n_expert));
@@ -1522,10 +1522,11 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                         char* ws = plan->stream_ws;
                         lp.cnt = (uint32_t*)ws;
                         lp.xa = (uint64_t*)(ws + 1024);
-                        lp.xl = lp.xa + (size_t)8 * m.n_expert;
-                        lp.xh = lp.xl + (size_t)8 * m.n_expert;
-                        lp.xs = lp.xh + (size_t)8 * m.n_ff_exp;
-                        lp.ypart = lp.xs + (size_t)m.n_ff_exp;
+                        const size_t nr = (size_t)rows;   // every region holds one part per token row
+                        lp.xl = lp.xa + nr * 8 * m.n_expert;
+                        lp.xh = lp.xl + nr * 8 * m.n_expert;
+                        lp.xs = lp.xh + nr * 8 * m.n_ff_exp;
+                        lp.ypart = lp.xs + nr * m.n_ff_exp;
                         lp.late = be->fault_dev + 1;
                         lp.logits_once = moe_logits_once(be, m);
                         lp.guess_skew = (int)std::min<uint32_t>(be->cfg.single_launch_guess_skew, 8u);

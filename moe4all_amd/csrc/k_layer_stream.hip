@@ -255,16 +255,42 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
     __shared__ uint32_t s_seq;
     const MoeGemvParams& p = q.g;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    const int b = blockIdx.x, g = b & (kGroups - 1), m = b >> 3;
     const int ne = p.ne, nff = p.nff, n_expert = p.route.n_expert;
     const bool shared = p.sh_gate != nullptr;
+    // One, two or four token rows per launch: a row takes 8 / rows of the XCDs (workgroups are dealt to the XCDs in turn,
+    // so workgroup b sits on XCD b & 7 up to a rotation), its eight groups of mpg = 32 / rows members each lie on one XCD
+    // as before, and everything below happens per row among the row's 256 / rows workgroups.
+    const int b = blockIdx.x;
+    const int n_rows = p.rows, xpr = kGroups / n_rows, mpg = kPerGroup / n_rows, bpr = kBlocks / n_rows;
+    const int xcd = b & 7, jx = b >> 3;
+    const int trow = xcd / xpr;                            // this workgroup's token row
+    const int g = (xcd - trow * xpr) * n_rows + jx / mpg;  // its group: the rank slot it works on
+    const int m = jx % mpg;                                // its place in the group
+    const int os = m * kGroups + g;                        // its place among the row's workgroups: output rows, always-on share
+    {   // this row's operands and results
+        MoeGemvParams& pw = q.g;
+        pw.x += (size_t)trow * ne;
+        pw.dst += (size_t)trow * ne;
+        if (pw.addend) pw.addend += (size_t)trow * ne;
+        if (pw.sh_logit) pw.sh_logit += trow;
+        pw.route.ids += (size_t)trow * pw.route.n_used;
+        pw.route.weights += (size_t)trow * pw.route.n_used;
+        if (pw.route.probs) pw.route.probs += (size_t)trow * n_expert;
+        q.router_x += (size_t)trow * ne;
+        if (q.logits_out) q.logits_out += (size_t)trow * n_expert;
+        q.xa += (size_t)trow * kGroups * n_expert;
+        q.xl += (size_t)trow * kGroups * n_expert;
+        q.xh += (size_t)trow * kGroups * nff;
+        q.xs += (size_t)trow * nff;
+        q.ypart += (size_t)trow * kGroups * ne;
+    }
 
     // who computes which router logits: every group all of them (epb = n_expert / 32 rows per workgroup, published to
     // the group), or every logit once for the grid (epb rows per workgroup while they last, published to everyone)
     const int epb = q.epb;
     const bool group_local = !q.logits_once;   // logit records stay inside the group's XCD
     const int area = q.logits_once ? 0 : g;
-    const int row0 = (q.logits_once ? b : m) * epb;
+    const int row0 = (q.logits_once ? os : m) * epb;
     const bool has_rows = row0 < n_expert;
 
     // LDS: [cells of x][chain operands, transposed][estimates][logits][routing scratch][h][cells of h][h, cells: always-on]
@@ -413,10 +439,10 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
             if (guess_state != 1) ok = false;
             bool routed = false;
             if (ok && route_duo_ok(rp) && rp.n_expert == 64 * NSP)
-                routed = route_softmax_checked<NSP>(rp, 0, lane, s_spec, route_scratch, s_tab, s_ids, s_w, b == 0);
+                routed = route_softmax_checked<NSP>(rp, 0, lane, s_spec, route_scratch, s_tab, s_ids, s_w, os == 0);
             if (!routed) {
                 __builtin_amdgcn_wave_barrier();
-                route_row_any(rp, 0, lane, route_scratch, s_tab, s_ids, s_w, b == 0);
+                route_row_any(rp, 0, lane, route_scratch, s_tab, s_ids, s_w, os == 0);
             }
             STAMP(18);
             __builtin_amdgcn_wave_barrier();
@@ -448,7 +474,7 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
                     s_gor[lane] = gk;
                     s_final[gk] = id;
                 }
-                if (b == 0 && missed && lane == 0 && q.late)
+                if (os == 0 && missed && lane == 0 && q.late)
                     __hip_atomic_fetch_add(q.late, (uint32_t)__builtin_popcount(missed), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
             }
         }
@@ -471,18 +497,18 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
         // gate/up items of this wavefront: item j covers features (j * kSW + sw) * rw_count + rw of the workgroup's slice.
         // With an always-on expert the first kSW-or-fewer wavefronts take one item of its share [b * nff / 256, ..) as
         // their ring's first entry: it needs no routing, so it is requested before the guess is known.
-        const int fpb = nff / kPerGroup, f0 = m * fpb;
+        const int fpb = nff / mpg, f0 = m * fpb;
         const int n_gi = (fpb + pg.rw_count - 1) / pg.rw_count;
         const int my_gi = n_gi > sw ? (n_gi - sw + kSW - 1) / kSW : 0;
-        const int sfpb = nff / kBlocks, sf0 = b * sfpb;
+        const int sfpb = nff / bpr, sf0 = os * sfpb;
         const int n_si = shared ? (sfpb + pg.rw_count - 1) / pg.rw_count : 0;
         const int sh_n = sw < n_si ? 1 : 0;
         // down items: item j covers output rows (j * kSW + sw) * rw_count + rw of the workgroup's slice; behind them the
         // always-on expert's rows [b * ne / 256, ..), dealt to the wavefronts starting with those that got fewer above
-        const int R = ne / kPerGroup;
+        const int R = ne / mpg;
         const int n_di = (R + pd.rw_count - 1) / pd.rw_count;
         const int my_di = n_di > sw ? (n_di - sw + kSW - 1) / kSW : 0;
-        const int SR = ne / kBlocks;
+        const int SR = ne / bpr;
         const int n_sdi = shared ? (SR + pd.rw_count - 1) / pd.rw_count : 0;
         const int ssw = (sw + kSW - n_di % kSW) % kSW;
         const int my_sdi = n_sdi > ssw ? (n_sdi - ssw + kSW - 1) / kSW : 0;
@@ -522,7 +548,7 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
             const int jj = routed ? j : j - my_di;
             const int lim = routed ? R : SR;
             const int orow = min((jj * kSW + (routed ? sw : ssw)) * pd.rw_count + pd.rw, lim - 1);
-            const uint8_t* base = routed ? dbank + (size_t)(m * R + orow) * rb_d : p.sh_down + (size_t)(b * SR + orow) * rb_d;
+            const uint8_t* base = routed ? dbank + (size_t)(m * R + orow) * rb_d : p.sh_down + (size_t)(os * SR + orow) * rb_d;
             dring[slot] = load_row<FD>(pd, base);
         };
         // One pass per expert this group works on: the guessed one, and once more if the exact routing names another.
@@ -685,7 +711,7 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
         // the output, which are also the rows of the always-on expert it has just computed.  out = sum over ranks of
         // w_rank * y_rank as a separate multiply and add (crates/infr-cpu/src/lib.rs:4290-4302), then the always-on
         // expert, then the residual operand.  The partial results are polled while the streaming wavefronts still work.
-        const int R = ne / kPerGroup, SR = R / kGroups;
+        const int R = ne / mpg, SR = R / kGroups;
         const bool mine = lane < SR;
         const size_t oi = (size_t)m * R + (size_t)g * SR + (mine ? lane : 0);
         uint64_t yk[kGroups];
@@ -718,7 +744,7 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
             if (shared) {
                 float ws = 1.0f;
                 if (p.sh_logit)   // crates/infr-cpu/src/lib.rs:3336-3356: sigmoid of the row's gate logit
-                    ws = __fdiv_rn(1.0f, __fadd_rn(1.0f, expf_libm(-p.sh_logit[0], s_tab)));
+                    ws = __fdiv_rn(1.0f, __fadd_rn(1.0f, expf_libm(-p.sh_logit[0], s_tab)));   // this row's: the pointer was advanced
                 acc = __fadd_rn(acc, __fmul_rn(ws, s_ysh[lane]));
             }
             p.dst[oi] = p.addend ? __fadd_rn(p.addend[oi], acc) : acc;
@@ -729,9 +755,10 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
 }
 
 // ---------------------------------------------------------------------------------------------
-size_t moe_layer_stream_workspace_bytes(int ne, int nff, int n_expert) {
-    // [launch count of each workgroup: 1 KB][estimates 8 * n_expert][logits 8 * n_expert][h 8 * nff][h always-on nff][partials 8 * ne]
-    return 1024 + ((size_t)2 * kGroups * n_expert + (size_t)kGroups * nff + (size_t)nff + (size_t)kGroups * ne) * 8;
+size_t moe_layer_stream_workspace_bytes(int ne, int nff, int n_expert, int rows) {
+    // [launch count of each workgroup: 1 KB], then for each of the regions one part per token row:
+    // [estimates 8 * n_expert][logits 8 * n_expert][h 8 * nff][h always-on nff][partials 8 * ne]
+    return 1024 + (size_t)rows * ((size_t)2 * kGroups * n_expert + (size_t)kGroups * nff + (size_t)nff + (size_t)kGroups * ne) * 8;
 }
 
 namespace {
@@ -752,17 +779,26 @@ bool stream_shape(const MoeLayerParams& q, StreamShape* out) {
     if (lpr_g > 64 || lpr_d > 64) return false;
     if (n_expert % 64 || n_expert > 256 || n_expert < 64) return false;
     const int rwc_g = 64 / lpr_g, rwc_d = 64 / lpr_d;
-    const int fpb = nff / kPerGroup, R = ne / kPerGroup;
+    const int rows = p.rows;
+    if (rows != 1 && rows != 2 && rows != 4) return false;             // whole XCDs per token row
+    // four rows of Q8_0 banks are no faster here than on the per-token kernels (52.7 against 53.2 us at 128 experts), which
+    // run sixteen wavefronts per compute unit over their long streams; two rows are (33.6 against 36.6 us)
+    if (rows == 4 && std::is_same<FG, Q80Fmt>::value) return false;
+    const int mpg = kPerGroup / rows, bpr = kBlocks / rows;
+    if (nff % mpg || ne % bpr) return false;
+    const int fpb = nff / mpg, R = ne / mpg;
     const int n_gi = (fpb + rwc_g - 1) / rwc_g, n_di = (R + rwc_d - 1) / rwc_d;
     const int my_gi = (n_gi + kSW - 1) / kSW, my_di = (n_di + kSW - 1) / kSW;
     if (my_gi * rwc_g > 64) return false;                            // a wavefront's results wait in one 64-float row
     if (shared) {
-        const int n_si = (nff / kBlocks + rwc_g - 1) / rwc_g;
-        if (n_si > kSW || ne / kBlocks > 64) return false;
+        if (nff % bpr) return false;
+        const int n_si = (nff / bpr + rwc_g - 1) / rwc_g;
+        if (n_si > kSW) return false;
     }
     // every logit once for the grid when a group's copy of the router would be a large share of the layer's bytes
     out->once = q.logits_once;
-    out->epb = out->once ? (n_expert + kBlocks - 1) / kBlocks : n_expert / kPerGroup;
+    if (ne / bpr > 64) return false;                                  // a workgroup's output rows: one per lane of the summing wavefront
+    out->epb = out->once ? (n_expert + bpr - 1) / bpr : n_expert / mpg;
     const int H = kThreads / (ne / 8);
     out->ept = (out->epb + H - 1) / H;
     out->nsp = n_expert / 64;
@@ -806,11 +842,13 @@ bool dispatch_stream(hipStream_t s, MoeLayerParams q, bool launch) {
         INFR_STREAM(2, 2, 2, 2)   // ne 2048, nff 768, 128 experts, a copy of the router per group
         INFR_STREAM(2, 2, 1, 2)   // ... every logit once
         INFR_STREAM(2, 2, 1, 4)   // ... 256 experts
+        INFR_STREAM(2, 4, 1, 2)   // ne 2048, nff 768, 128 experts, two or four token rows
         INFR_STREAM(2, 4, 1, 4)   // ne 4096, nff 1536, 256 experts, every logit once
     } else {
         INFR_STREAM(4, 5, 2, 2)   // Q8_0: ne 2048, nff 768, 128 experts
         INFR_STREAM(4, 5, 1, 2)
         INFR_STREAM(4, 5, 1, 4)
+        INFR_STREAM(2, 4, 1, 2)   // two or four token rows
     }
 #undef INFR_STREAM
     return false;
@@ -819,7 +857,7 @@ bool dispatch_stream(hipStream_t s, MoeLayerParams q, bool launch) {
 bool stream_any(hipStream_t s, const MoeLayerParams& q, bool launch) {
     const MoeGemvParams& p = q.g;
     const RouteParams& r = p.route;
-    if (p.rows != 1 || p.n_used != kGroups || p.n_cu < kBlocks || p.gate_dt != p.up_dt) return false;
+    if (p.n_used != kGroups || p.n_cu < kBlocks || p.gate_dt != p.up_dt) return false;
     if ((p.sh_gate != nullptr) != (p.sh_down != nullptr) || (p.sh_gate != nullptr) != (p.sh_up != nullptr)) return false;
     // the guess ranks the experts by their logits: gatings that are monotone in the logit, no bias, no groups, no given
     // ids; options that need the routing weights before the gate/up stage or remap ids stay on the in-order kernels

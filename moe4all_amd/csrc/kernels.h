@@ -156,7 +156,7 @@ struct MoeLayerParams {
 size_t moe_layer_workspace_bytes(int ne, int nff, int n_expert);
 bool moe_layer_fused_supported(const MoeLayerParams& q);
 bool launch_moe_layer_fused(hipStream_t s, const MoeLayerParams& q);
-size_t moe_layer_stream_workspace_bytes(int ne, int nff, int n_expert);
+size_t moe_layer_stream_workspace_bytes(int ne, int nff, int n_expert, int rows);
 bool moe_layer_stream_supported(const MoeLayerParams& q);
 bool launch_moe_layer_stream(hipStream_t s, const MoeLayerParams& q);
 

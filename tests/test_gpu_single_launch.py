@@ -209,8 +209,8 @@ def test_a_wait_that_runs_out_is_reported_and_the_backend_falls_back(be3, kernel
 
 
 def test_shapes_the_kernel_does_not_take_stay_on_three_launches(be):
-    """Six experts per token, or a hidden size above 2048: compile keeps the three-launch path."""
-    for ne, E, K, nff in ((2048, 128, 6, 768), (4096, 128, 8, 768)):
+    """Six experts per token, or an intermediate size that is no multiple of 384: compile keeps the three-launch path."""
+    for ne, E, K, nff in ((2048, 128, 6, 768), (4096, 128, 8, 1024)):
         rng = np.random.default_rng(ne + K)
         x = rng.standard_normal((1, ne)).astype(np.float32)
         router = (rng.standard_normal((E, ne)) * 0.02).astype(np.float32)
@@ -219,6 +219,18 @@ def test_shapes_the_kernel_does_not_take_stay_on_three_launches(be):
         out, r = _run(be, g, ids, dict(x=x, router=router, gate=gate, up=up, down=down), ne, "moe_route_gate_up")
         ref = O.moe_ffn(x, router, gate, up, down, ne=ne, n_expert=E, n_used=K, n_ff_exp=nff, gate_dtype=H.Q4K, down_dtype=H.Q6K)
         assert np.array_equal(r["idx"], ref["idx"]) and H.rel_l2(out, ref["dst"]) < 1e-3
+
+
+def test_hidden_size_4096_with_the_small_intermediate_size(be, be3):
+    """ne = 4096 with n_ff = 768: a shape between the two benchmark shapes."""
+    ne, E, K, nff = 4096, 128, 8, 768
+    data = _plain_case(4096, ne=ne, nff=nff)
+    g, ids = moe_graph(1, ne, E, K, nff, DType.Q4K, DType.Q6K)
+    one, r1 = _run(be, g, ids, data, ne, GUESS)
+    g, ids = moe_graph(1, ne, E, K, nff, DType.Q4K, DType.Q6K)
+    three, r3 = _run(be3, g, ids, data, ne, "moe_route_gate_up")
+    assert np.array_equal(r1["idx"], r3["idx"]) and np.array_equal(bits(r1["w"]), bits(r3["w"]))
+    assert np.array_equal(bits(one), bits(three))
 
 
 def _plain_case(seed, E=128, gdt=H.Q4K, ddt=H.Q6K, ne=2048, nff=768):
@@ -250,6 +262,53 @@ def test_an_expert_the_guess_missed_is_loaded_late_and_changes_nothing(be3, skew
         assert b.late_experts() - before == 3 * skew
     finally:
         b.close()
+
+
+@pytest.mark.parametrize("rows,gdt,ddt,skew", [(2, H.Q4K, H.Q6K, 0), (4, H.Q4K, H.Q6K, 0), (2, H.Q8_0, H.Q8_0, 0),
+                                               (4, H.Q4K, H.Q6K, 2), (2, H.Q8_0, H.Q8_0, 8)])
+def test_two_and_four_token_rows_in_one_launch_give_the_bits_of_three_launches(be3, rows, gdt, ddt, skew):
+    """Two or four token rows: every row takes 8 / rows of the XCDs and runs the single-token scheme among its own
+    workgroups (its own logits, guess, routing, hand-overs and output rows).  Ids, weights, logits and output bits per row
+    are those of the three-launch path, also when every row's guess misses `skew` experts, and a row's bits do not depend
+    on its neighbours (row 0 alone gives the same)."""
+    ne, E, K, nff = 2048, 128, 8, 768
+    rng = np.random.default_rng(1000 + rows + gdt + skew)
+    x = rng.standard_normal((rows, ne)).astype(np.float32)
+    x[rows - 1] *= 30.0                                    # rows of different magnitude: nothing is shared between rows
+    router = (rng.standard_normal((E, ne)) * 0.02).astype(np.float32)
+    gate, up, down = _banks(rng, E, nff, ne, gdt, ddt)
+    data = dict(x=x, router=router, gate=gate, up=up, down=down)
+    b = M.Backend(0, single_launch_guess_skew=skew)
+    try:
+        before = b.late_experts()
+        for rep in range(2):   # twice on the same shape: records of the launch before are never taken
+            g, ids = moe_graph(rows, ne, E, K, nff, DType(gdt), DType(ddt))
+            one, r1 = _run(b, g, ids, data, rows * ne, GUESS)
+            g, ids = moe_graph(rows, ne, E, K, nff, DType(gdt), DType(ddt))
+            three, r3 = _run(be3, g, ids, data, rows * ne, "moe_route_gate_up")
+            assert np.array_equal(r1["idx"], r3["idx"]) and np.array_equal(bits(r1["w"]), bits(r3["w"]))
+            assert np.array_equal(bits(r1["logits"]), bits(r3["logits"])) and np.array_equal(bits(r1["probs"]), bits(r3["probs"]))
+            assert np.array_equal(bits(one), bits(three))
+        assert b.late_experts() - before == 2 * rows * skew
+        g, ids = moe_graph(1, ne, E, K, nff, DType(gdt), DType(ddt))
+        alone, _ = _run(b, g, ids, dict(data, x=x[:1]), ne, GUESS)
+        assert np.array_equal(bits(alone.reshape(-1)), bits(one.reshape(rows, ne)[0]))
+        ref = O.moe_ffn(x, router, gate, up, down, ne=ne, n_expert=E, n_used=K, n_ff_exp=nff, gate_dtype=gdt, down_dtype=ddt)
+        assert np.array_equal(r1["idx"], ref["idx"])
+        assert H.rel_l2(one.reshape(rows, ne), ref["dst"]) < 1e-3
+    finally:
+        b.close()
+
+
+def test_three_token_rows_stay_on_three_launches(be):
+    """A row count that does not divide the eight XCDs keeps the per-token kernels."""
+    ne, E, K, nff = 2048, 128, 8, 768
+    rng = np.random.default_rng(3)
+    x = rng.standard_normal((3, ne)).astype(np.float32)
+    router = (rng.standard_normal((E, ne)) * 0.02).astype(np.float32)
+    gate, up, down = _banks(rng, E, nff, ne, H.Q4K, H.Q6K)
+    g, ids = moe_graph(3, ne, E, K, nff, DType.Q4K, DType.Q6K)
+    _run(be, g, ids, dict(x=x, router=router, gate=gate, up=up, down=down), 3 * ne, "moe_route_gate_up")
 
 
 def test_a_good_guess_loads_nothing_late(be):
