@@ -368,33 +368,33 @@ def test_near_tied_logits_at_the_edge_of_the_selection(be, be3):
 _SHARED_CASES = {}
 
 
-def _shared_graph(ne, E, K, nff, gated):
+def _shared_graph(ne, E, K, nff, gated, rows=1):
     g = M.Graph()
     T = M.TensorDesc
-    x = g.input(T([1, ne], DType.F32))
+    x = g.input(T([rows, ne], DType.F32))
     router = g.weight(T([E, ne], DType.F32))
     gate, up = g.weight(T([E, nff, ne], DType.Q4K)), g.weight(T([E, nff, ne], DType.Q4K))
     down = g.weight(T([E, ne, nff], DType.Q6K))
     sg, su, sd = g.weight(T([nff, ne], DType.Q4K)), g.weight(T([nff, ne], DType.Q4K)), g.weight(T([ne, nff], DType.Q6K))
-    moe = g.internal(T([1, ne], DType.F32))
-    tg, tu, ta = (g.internal(T([1, nff], DType.F32)) for _ in range(3))
-    ts = g.internal(T([1, ne], DType.F32))
-    dst = g.output(T([1, ne], DType.F32))
+    moe = g.internal(T([rows, ne], DType.F32))
+    tg, tu, ta = (g.internal(T([rows, nff], DType.F32)) for _ in range(3))
+    ts = g.internal(T([rows, ne], DType.F32))
+    dst = g.output(T([rows, ne], DType.F32))
     ids = dict(x=x, router=router, gate=gate, up=up, down=down, sg=sg, su=su, sd=sd, dst=dst)
     g.moe_ffn(x=x, router=router, gate_exps=gate, up_exps=up, down_exps=down, dst=moe, ne=ne, n_expert=E, n_used=K, n_ff_exp=nff)
     if gated:
         wq = g.weight(T([1, ne], DType.F32))
-        tq = g.internal(T([1, 1], DType.F32))
-        g.linear(x=x, weight=wq, dst=tq, m=1, in_f=ne, out_f=1)
+        tq = g.internal(T([rows, 1], DType.F32))
+        g.linear(x=x, weight=wq, dst=tq, m=rows, in_f=ne, out_f=1)
         ids["wq"] = wq
-    g.linear(x=x, weight=sg, dst=tg, m=1, in_f=ne, out_f=nff)
-    g.linear(x=x, weight=su, dst=tu, m=1, in_f=ne, out_f=nff)
-    g.gated_act(gate=tg, up=tu, dst=ta, rows=1, nff=nff)
-    g.linear(x=ta, weight=sd, dst=ts, m=1, in_f=nff, out_f=ne)
+    g.linear(x=x, weight=sg, dst=tg, m=rows, in_f=ne, out_f=nff)
+    g.linear(x=x, weight=su, dst=tu, m=rows, in_f=ne, out_f=nff)
+    g.gated_act(gate=tg, up=tu, dst=ta, rows=rows, nff=nff)
+    g.linear(x=ta, weight=sd, dst=ts, m=rows, in_f=nff, out_f=ne)
     if gated:
-        g.moe_shared_expert_add(moe=moe, shexp=ts, gate=tq, dst=dst, rows=1, n=ne)
+        g.moe_shared_expert_add(moe=moe, shexp=ts, gate=tq, dst=dst, rows=rows, n=ne)
     else:
-        g.add(a=moe, b=ts, dst=dst, n=ne)
+        g.add(a=moe, b=ts, dst=dst, n=rows * ne)
     return g, ids
 
 
@@ -436,3 +436,23 @@ def test_single_launch_with_the_always_on_expert_folded_in(be3, ne, E, nff, gate
                        n_used=1, n_ff_exp=nff, gate_dtype=H.Q4K, down_dtype=H.Q6K)
         want = ref["dst"] + sh["dst"]
         assert H.rel_l2(one, want) < 1e-3 and H.max_abs(one, want) < 2e-3
+
+
+@pytest.mark.parametrize("gated", [False, True])
+def test_two_token_rows_with_the_always_on_expert_folded_in(be, be3, gated):
+    """Two rows of the small shape with an always-on expert: each row's share of that expert is spread over the row's 128
+    workgroups.  Same bits as the three-launch path, row by row."""
+    rows, ne, E, K, nff = 2, 2048, 128, 8, 768
+    rng = np.random.default_rng(50 + gated)
+    data = dict(x=rng.standard_normal((rows, ne)).astype(np.float32), router=(rng.standard_normal((E, ne)) * 0.02).astype(np.float32))
+    data["gate"], data["up"], data["down"] = _banks(rng, E, nff, ne, H.Q4K, H.Q6K)
+    data["sg"], data["su"], data["sd"] = (a.reshape(-1) for a in _banks(rng, 1, nff, ne, H.Q4K, H.Q6K))
+    if gated:
+        data["wq"] = (rng.standard_normal((1, ne)) * 0.02).astype(np.float32)
+    g, ids = _shared_graph(ne, E, K, nff, gated, rows)
+    one, r1 = _run(be, g, ids, data, rows * ne, "moe_layer_shared")
+    g, ids = _shared_graph(ne, E, K, nff, gated, rows)
+    three, r3 = _run(be3, g, ids, data, rows * ne, "moe_route_gate_up_shared")
+    assert np.array_equal(r1["idx"], r3["idx"]) and np.array_equal(bits(r1["w"]), bits(r3["w"]))
+    assert np.array_equal(bits(one), bits(three))
+    assert np.abs(one.reshape(rows, ne)[1]).max() > 1e-5
