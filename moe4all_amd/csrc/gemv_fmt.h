@@ -407,26 +407,38 @@ struct Q80Fmt {
     }
 };
 
-// Lane placement of a wavefront over weight rows of nblk blocks: lanes_per_row = nblk*LPB
-// (<= 64), rows_per_wave = 64 / lanes_per_row.  Left-over lanes of the wave are pointed at the
-// last row and flagged off: they load and compute like everyone else, so the code stays
-// branch-free and every load of a round is issued back to back; their result is dropped.
+// Lane placement of a wavefront over weight rows of nblk blocks: a row holds lpr = nblk * LPB lanes (<= 64) and
+// occupies `slot` lanes: lpr itself, or the next power of two when that leaves as many rows per wavefront (24 -> 32:
+// two rows either way).  rows_per_wave = 64 / slot.  With a power-of-two slot the row's sum takes the DPP path of
+// row_sum instead of cross-lane reads through the LDS.  Padding lanes of a slot and left-over lanes of the wave are
+// pointed at the row's last block / the last row and flagged off: they load and compute like everyone else, so the
+// code stays branch-free and every load of a round is issued back to back; their result is dropped.
 template <class F>
 struct Place {
-    int lpr, rw_count, rw, pos;  // lanes per row, rows per wave, my row (clamped), my lane in the row
-    bool row_on;
-    int blk, sub;                // my block in the row and my lane inside the block
-    int wpos;                    // lane-in-row where the row's sum lands
+    int lpr, slot, rw_count, rw, pos;  // lanes of a row, lanes a row occupies, rows per wave, my row (clamped), my lane in the slot
+    bool row_on, lane_on;              // my row exists; my lane holds a block of it
+    int blk, sub;                      // my block in the row and my lane inside the block
+    int wpos;                          // lane-in-slot where the row's sum lands
     __device__ __forceinline__ Place(int nblk, int lane) {
         lpr = nblk * F::kLPB;
-        rw_count = kWave / lpr;
-        const int rw_raw = lane / lpr;
-        pos = lane - rw_raw * lpr;
+        slot = lpr;
+        // (one-lane-per-block formats only: measured 4 % faster on 24-block Q8_0 rows, whose sum otherwise takes five
+        // cross-lane reads per 32 elements of a lane, and 4 % slower on the 24 lanes of a six-block Q6_K row)
+        if (F::kLPB == 1 && (lpr & (lpr - 1))) {
+            int p2 = 16;
+            while (p2 < lpr) p2 <<= 1;
+            if (kWave / p2 == kWave / lpr) slot = p2;
+        }
+        rw_count = kWave / slot;
+        const int rw_raw = lane / slot;
+        pos = lane - rw_raw * slot;
         row_on = rw_raw < rw_count;
+        lane_on = pos < lpr;
         rw = row_on ? rw_raw : rw_count - 1;
-        blk = pos / F::kLPB;
-        sub = pos - blk * F::kLPB;
-        wpos = (lpr == 64 || lpr == 32 || lpr == 16) ? lpr - 1 : 0;
+        const int bpos = lane_on ? pos : lpr - 1;
+        blk = bpos / F::kLPB;
+        sub = bpos - blk * F::kLPB;
+        wpos = (slot == 64 || slot == 32 || slot == 16) ? slot - 1 : 0;
     }
     __device__ __forceinline__ bool writer() const { return row_on && pos == wpos; }
 };
@@ -441,10 +453,14 @@ __device__ __forceinline__ typename F::Raw load_row(const Place<F>& pl, const ui
 // Sum of v over the lanes of each weight row; valid in the row's writer lane.
 template <class F>
 __device__ __forceinline__ float row_sum(float v, const Place<F>& pl, int nblk) {
-    if (pl.lpr >= 16 && (pl.lpr & (pl.lpr - 1)) == 0) {
+    if (pl.slot >= 16 && (pl.slot & (pl.slot - 1)) == 0) {
+        // Padding lanes add -0.0, the identity of the addition (x + -0.0 == x for every x, -0.0 included).  The DPP tree
+        // then adds the same pairs as the doubling loop below, some with their operands swapped, and the sums of
+        // padding-only subtrees where the loop adds nothing: the same bits.
+        if (pl.slot != pl.lpr && !pl.lane_on) v = -0.0f;
         v = row16_sum(v);                                            // every lane: sum of its 16
-        if (pl.lpr >= 32) v += dpp_rows_f<0x142, 0xA>(v);            // rows 1,3 += lane 15 of rows 0,2
-        if (pl.lpr == 64) v += dpp_rows_f<0x143, 0xC>(v);            // rows 2,3 += lane 31
+        if (pl.slot >= 32) v += dpp_rows_f<0x142, 0xA>(v);           // rows 1,3 += lane 15 of rows 0,2
+        if (pl.slot == 64) v += dpp_rows_f<0x143, 0xC>(v);           // rows 2,3 += lane 31
         return v;
     }
     // lanes of one block first (rows start at multiples of kLPB lanes, so DPP groups line up) ...

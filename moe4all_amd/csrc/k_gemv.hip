@@ -123,7 +123,7 @@ __global__ __launch_bounds__(256) void moe_gate_up_fast(MoeGemvParams p, int ft)
     t.r = blockIdx.y;
     t.f0 = blockIdx.x * ft;
     t.fcount = min(ft, p.nff - t.f0);
-    t.wave = threadIdx.x >> 6;
+    t.wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     t.lane = threadIdx.x & 63;
     const int r = t.r, wave = t.wave, lane = t.lane;
     const int nblk = p.ne / F::kBlockElems;
@@ -196,7 +196,7 @@ __global__ __launch_bounds__(64 * NW, NW <= 8 ? 4 : 3) void moe_gate_up_stream(M
     const int r = blockIdx.y;
     const int f0 = blockIdx.x * ft;
     const int fcount = min(ft, p.nff - f0);
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // uniform: scalar registers
     const int nblk = p.ne / F::kBlockElems;
     const size_t row_bytes = (size_t)nblk * F::kBlockBytes;
     const Place<F> pl(nblk, lane);
@@ -252,10 +252,16 @@ __global__ __launch_bounds__(64 * NW, NW <= 8 ? 4 : 3) void moe_gate_up_stream(M
     const int n_mine = nitems > wave * pl.rw_count ? (nitems - wave * pl.rw_count + per_step - 1) / per_step : 0;
     const float inv_fcount = 1.0f / (float)fcount;
     // item j of this wave's rows: (slot, feature), exact for the few thousand items a tile can hold
+    // (rows of 64 lanes: one item per wave and step, so slot, expert and row address are the same in every lane and are
+    // kept in scalar registers; the loads then take a scalar base and the lane's block offset)
+    const bool one_row = pl.rw_count == 1;
     auto issue = [&](GuStage<F, 1>& st, int j) {
         const int it = min((j * NW + wave) * pl.rw_count + pl.rw, nitems - 1);
-        const int slot = (int)(((float)it + 0.5f) * inv_fcount), f = f0 + (it - slot * fcount);
-        const int e = s_ids[slot];
+        int slot = (int)(((float)it + 0.5f) * inv_fcount);
+        if (one_row) slot = __builtin_amdgcn_readfirstlane(slot);
+        const int f = f0 + ((one_row ? __builtin_amdgcn_readfirstlane(it) : it) - slot * fcount);
+        int e = s_ids[slot];
+        if (one_row) e = __builtin_amdgcn_readfirstlane(e);
         const bool routed = slot < p.n_used;
         const uint8_t* gb = routed ? p.gate + (size_t)e * p.gate_stride : p.sh_gate;
         const uint8_t* ub = routed ? p.up + (size_t)e * p.up_stride : p.sh_up;
@@ -374,7 +380,7 @@ __global__ __launch_bounds__(512) void moe_down_combine_fast(MoeGemvParams p, in
     __shared__ float ypart[kMaxUsedFast][kMaxOt];
     const int r = blockIdx.y;
     const int o0 = blockIdx.x * ot;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // uniform: scalar registers
     const int nwaves = blockDim.x >> 6;
     const int nblk = p.nff / F::kBlockElems;
     const Place<F> pl(nblk, lane);
@@ -472,7 +478,7 @@ __global__ __launch_bounds__(64 * NW) void moe_down_combine_stream(MoeGemvParams
     __shared__ int s_skip[kMaxUsedFast];
     const int r = blockIdx.y;
     const int o0 = blockIdx.x * ot;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // uniform: scalar registers
     const int nblk = p.nff / F::kBlockElems;
     const Place<F> pl(nblk, lane);
     const size_t row_bytes = (size_t)nblk * F::kBlockBytes;
@@ -510,13 +516,24 @@ __global__ __launch_bounds__(64 * NW) void moe_down_combine_stream(MoeGemvParams
     const int base_units = n_units / NW, rem_units = n_units - base_units * NW;
     const int ub = wave * base_units + min(wave, rem_units);
     const int cn = base_units + (wave < rem_units ? 1 : 0);
-    const float inv_G = 1.0f / (float)G;
-    auto issue = [&](typename F::Raw& raw, int j) {
-        const int u = ub + j;
-        const int slot = (int)(((float)u + 0.5f) * inv_G), rg = u - slot * G;
-        const int o = min(rg * pl.rw_count + pl.rw, ocount - 1);
-        const uint8_t* bank = slot < p.n_used ? p.down + (size_t)s_ids[slot] * p.down_stride : p.sh_down;
-        raw = load_row<F>(pl, bank + (size_t)(o0 + o) * row_bytes);
+    // Units are taken in order, once by the requests and once by the dots: two cursors (slot, row group) that step
+    // through the run, in scalar registers (the wave's index is uniform), instead of a division per unit.
+    const int slot_first = __builtin_amdgcn_readfirstlane((int)(((float)ub + 0.5f) * (1.0f / (float)G)));
+    int i_slot = slot_first, i_rg = ub - slot_first * G;   // cursor of the requests
+    const uint8_t* i_bank = nullptr;
+    int i_bank_slot = -1;
+    auto issue = [&](typename F::Raw& raw, int) {
+        if (i_slot != i_bank_slot) {   // the same for the whole wave
+            const int e = __builtin_amdgcn_readfirstlane(s_ids[i_slot < n_slots ? i_slot : 0]);
+            i_bank = i_slot < p.n_used ? p.down + (size_t)e * p.down_stride : p.sh_down;
+            i_bank_slot = i_slot;
+        }
+        const int o = min(i_rg * pl.rw_count + pl.rw, ocount - 1);
+        raw = load_row<F>(pl, i_bank + (size_t)(o0 + o) * row_bytes);
+        if (++i_rg == G) {
+            i_rg = 0;
+            i_slot++;
+        }
     };
     typename F::Raw ring[D];
 #pragma unroll
@@ -536,9 +553,9 @@ __global__ __launch_bounds__(64 * NW) void moe_down_combine_stream(MoeGemvParams
     typename F::X x;
     int cur_slot = -1;
     float ds = 1.0f;
-    auto finish = [&](const typename F::Raw& raw, int j) {
-        const int u = ub + j;
-        const int slot = (int)(((float)u + 0.5f) * inv_G), rg = u - slot * G;
+    int f_slot = slot_first, f_rg = ub - slot_first * G;   // cursor of the dots
+    auto finish = [&](const typename F::Raw& raw, int) {
+        const int slot = f_slot, rg = f_rg;
         if (slot != cur_slot) {   // the same for the whole wave
             F::fetch_x(x, dyn_lds + slot * cell_words, pl.blk, pl.sub);
             ds = s_ds[slot];
@@ -547,6 +564,10 @@ __global__ __launch_bounds__(64 * NW) void moe_down_combine_stream(MoeGemvParams
         const int o = rg * pl.rw_count + pl.rw;
         const float y = row_sum<F>(F::dot(raw, pl.sub, x), pl, nblk);
         if (o < ocount && pl.writer()) ypart[slot][o] = (p.down_scale && slot < p.n_used) ? __fmul_rn(y, ds) : y;
+        if (++f_rg == G) {
+            f_rg = 0;
+            f_slot++;
+        }
     };
     const int refills = cn - D;
     int j0 = 0;
@@ -591,7 +612,7 @@ __global__ __launch_bounds__(64 * NW) void moe_down_combine_stream(MoeGemvParams
 // Any dtype decode_elem understands and any shape: one wave per output, lanes stride over K,
 // plain f32.
 __global__ __launch_bounds__(256) void moe_gate_up_generic(MoeGemvParams p, size_t g_row_bytes, size_t u_row_bytes) {
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // uniform: scalar registers
     const int f = blockIdx.x * 4 + wave;
     const int pair = blockIdx.y;
     if (f >= p.nff) return;
@@ -619,7 +640,7 @@ __global__ __launch_bounds__(256) void moe_gate_up_generic(MoeGemvParams p, size
 }
 
 __global__ __launch_bounds__(256) void moe_down_combine_generic(MoeGemvParams p, size_t row_bytes) {
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // uniform: scalar registers
     const int o = blockIdx.x * 4 + wave;
     const int r = blockIdx.y;
     if (o >= p.ne) return;
@@ -819,7 +840,7 @@ __global__ __launch_bounds__(256) void moe_gate_up_bucketed(MoeGemvParams p, int
     const int nt = min(T, t1 - t0);
     const int f0 = blockIdx.x * ft;
     const int fcount = min(ft, p.nff - f0);
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // uniform: scalar registers
     const int nblk = p.ne / F::kBlockElems;
     const size_t row_bytes = (size_t)nblk * F::kBlockBytes;
     const Place<F> pl(nblk, lane);
@@ -921,7 +942,7 @@ __global__ __launch_bounds__(256) void moe_down_bucketed(MoeGemvParams p, int ot
     const int nt = min(T, t1 - t0);
     const int o0 = blockIdx.x * ot;
     const int ocount = min(ot, p.ne - o0);
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // uniform: scalar registers
     const int nblk = p.nff / F::kBlockElems;
     const size_t row_bytes = (size_t)nblk * F::kBlockBytes;
     const Place<F> pl(nblk, lane);
@@ -1039,7 +1060,7 @@ __global__ __launch_bounds__(256) void linear_fast(const float* __restrict__ xin
     const int r = blockIdx.y;
     const int o0 = blockIdx.x * ot;
     const int ocount = min(ot, out_f - o0);
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // uniform: scalar registers
     const int nblk = in_f / F::kBlockElems;
     const size_t row_bytes = (size_t)nblk * F::kBlockBytes;
     const Place<F> pl(nblk, lane);
@@ -1078,7 +1099,7 @@ __global__ __launch_bounds__(256) void linear_fast(const float* __restrict__ xin
 __global__ __launch_bounds__(256) void linear_generic(const float* __restrict__ x, const uint8_t* __restrict__ w,
                                                       int dt, size_t row_bytes, int in_f, int out_f,
                                                       float* __restrict__ dst, const float* __restrict__ addend) {
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // uniform: scalar registers
     const int o = blockIdx.x * 4 + wave;
     const int r = blockIdx.y;
     if (o >= out_f) return;

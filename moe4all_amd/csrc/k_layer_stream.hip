@@ -254,7 +254,7 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
     __shared__ int s_f_spec, s_f_route, s_f_hs, s_fault, s_cells_done, s_h_done, s_done;
     __shared__ uint32_t s_seq;
     const MoeGemvParams& p = q.g;
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;   // wave: uniform, scalar registers
     const int ne = p.ne, nff = p.nff, n_expert = p.route.n_expert;
     const bool shared = p.sh_gate != nullptr;
     // One, two or four token rows per launch: a row takes 8 / rows of the XCDs (workgroups are dealt to the XCDs in turn,
