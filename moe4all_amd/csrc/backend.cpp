@@ -8,6 +8,7 @@
 #include <hip/hip_runtime.h>
 
 #include <atomic>
+#include <climits>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
@@ -229,6 +230,7 @@ struct infr_hip_backend {
     uint32_t* fault_host = nullptr;
     uint32_t* fault_dev = nullptr;
     std::atomic<int> single_launch_off{0};   // MoeFfn ops that still take three launches after a single-launch kernel gave up
+    std::atomic<int> single_launch_faults{0};   // launches that gave up so far
     std::atomic<int> inorder_off{0};         // the in-order single-launch kernel stays off after it gave up (its sequence word did not advance)
     // The object outlives infr_hip_destroy while buffers or plans still point at it (the reference's buffers keep their
     // device alive the same way): destroy drains and closes the stream and drops the creator's reference, the last
@@ -256,7 +258,10 @@ constexpr int kSingleLaunchPause = 256;
 infr_status check_fault(infr_hip_backend* be) {
     if (!be->fault_host || !*(volatile uint32_t*)be->fault_host) return INFR_OK;
     *(volatile uint32_t*)be->fault_host = 0;
-    be->single_launch_off.store(kSingleLaunchPause);
+    // a device on which the hand-overs keep failing (partitioned, or workgroups dealt to the XCDs in another way) must
+    // not pay a timed-out launch and an error every few hundred ops: the third time is for good
+    const int faults = be->single_launch_faults.fetch_add(1) + 1;
+    be->single_launch_off.store(faults >= 3 ? INT_MAX : kSingleLaunchPause);
     be->inorder_off.store(1);
     return fail(INFR_ERR_BACKEND,
                 "MoeFfn: the single-launch kernel timed out waiting for a peer workgroup (is the device shared or partitioned?); "
@@ -1504,9 +1509,12 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                 };
                 bool single = sc.single_launch != 0;
                 if (single && sc.single_launch == 1 && be->inorder_off.load(std::memory_order_relaxed)) single = false;
-                if (single && be->single_launch_off.load(std::memory_order_relaxed) > 0) {
-                    be->single_launch_off.fetch_sub(1, std::memory_order_relaxed);
-                    single = false;
+                if (single) {
+                    const int off = be->single_launch_off.load(std::memory_order_relaxed);
+                    if (off > 0) {
+                        if (off != INT_MAX) be->single_launch_off.fetch_sub(1, std::memory_order_relaxed);
+                        single = false;
+                    }
                 }
                 if (single) {
                     infr::MoeLayerParams lp{};
