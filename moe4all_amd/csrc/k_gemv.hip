@@ -185,7 +185,9 @@ __global__ __launch_bounds__(256) void moe_gate_up_fast(MoeGemvParams p, int ft)
 // waiting for memory and then all computing; many waves with a shallow ring measured faster than few with a deep one.
 // Results wait in LDS until the wave has finished a chunk of its items, then one lane per item applies the gated
 // activation.  The second launch bound (waves per SIMD) keeps two 8-wave blocks resident on a compute unit.
-template <class F, int D, int NW>
+// NBLK: blocks per weight row when known at compile time (the benchmark shapes), 0 for any: the lane placement and the
+// index arithmetic around the dots then fold.
+template <class F, int D, int NW, int NBLK = 0>
 __global__ __launch_bounds__(64 * NW, NW <= 8 ? 4 : 3) void moe_gate_up_stream(MoeGemvParams p, int ft) {
     extern __shared__ __attribute__((aligned(16))) uint32_t dyn_lds[];
     __shared__ uint64_t s_tab[32];
@@ -197,7 +199,7 @@ __global__ __launch_bounds__(64 * NW, NW <= 8 ? 4 : 3) void moe_gate_up_stream(M
     const int f0 = blockIdx.x * ft;
     const int fcount = min(ft, p.nff - f0);
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // uniform: scalar registers
-    const int nblk = p.ne / F::kBlockElems;
+    const int nblk = NBLK ? NBLK : p.ne / F::kBlockElems;
     const size_t row_bytes = (size_t)nblk * F::kBlockBytes;
     const Place<F> pl(nblk, lane);
     const int ncell = (p.ne + 31) / 32;
@@ -469,7 +471,7 @@ __global__ __launch_bounds__(512) void moe_down_combine_fast(MoeGemvParams p, in
 // busy, and a wave keeps D units in flight as a ring (finish the oldest, request the unit D places ahead into the
 // registers that became free).  h of every slot is turned into fixed-point cells once, by the whole block; a wave
 // fetches a slot's cells when its run crosses into that slot.
-template <class F, int D, int NW>
+template <class F, int D, int NW, int NBLK = 0>
 __global__ __launch_bounds__(64 * NW) void moe_down_combine_stream(MoeGemvParams p, int ot) {
     extern __shared__ __attribute__((aligned(16))) uint32_t dyn_lds[];
     __shared__ float ypart[kMaxUsedFast][kMaxOt];
@@ -479,7 +481,7 @@ __global__ __launch_bounds__(64 * NW) void moe_down_combine_stream(MoeGemvParams
     const int r = blockIdx.y;
     const int o0 = blockIdx.x * ot;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // uniform: scalar registers
-    const int nblk = p.nff / F::kBlockElems;
+    const int nblk = NBLK ? NBLK : p.nff / F::kBlockElems;
     const Place<F> pl(nblk, lane);
     const size_t row_bytes = (size_t)nblk * F::kBlockBytes;
     const int ocount = min(ot, p.ne - o0);
@@ -699,7 +701,12 @@ static bool try_gate_up(hipStream_t s, const MoeGemvParams& p) {
                              (p.route_inline ? route_scratch_floats(p.route.n_expert, p.route.n_groups) * sizeof(float) : 0);
         // one token row: twelve waves, each with one item in flight, cover the memory latency between them; with
         // several rows two blocks of eight waves share a compute unit
+        // the benchmark shapes' rows (2048 or 4096 elements) with their block count as a constant
+        constexpr int kNb0 = 2048 / F::kBlockElems, kNb1 = 4096 / F::kBlockElems;
+        const int nblk = p.ne / F::kBlockElems;
         if (p.rows == 1) INFR_LAUNCH((moe_gate_up_stream<F, 1, 12>), grid, dim3(768), lds_s, s, p, ft);
+        else if (nblk == kNb0) INFR_LAUNCH((moe_gate_up_stream<F, 1, 8, kNb0>), grid, dim3(512), lds_s, s, p, ft);
+        else if (nblk == kNb1 && kNb1 * F::kLPB <= 64) INFR_LAUNCH((moe_gate_up_stream<F, 1, 8, (kNb1 * F::kLPB <= 64 ? kNb1 : 0)>), grid, dim3(512), lds_s, s, p, ft);
         else INFR_LAUNCH((moe_gate_up_stream<F, 1, 8>), grid, dim3(512), lds_s, s, p, ft);
         return true;
     }
@@ -756,7 +763,12 @@ static bool try_down(hipStream_t s, const MoeGemvParams& p) {
         }
         if (ot >= 2 * gstep && n_slots * cells_bytes(p.nff) <= 64 * 1024) {
             dim3 grid(ceil_div(p.ne, ot), p.rows), block(1024);
-            INFR_LAUNCH((moe_down_combine_stream<F, 1, 16>), grid, block, n_slots * cells_bytes(p.nff), s, p, ot);
+            // the benchmark shapes' rows (768 or 1536 elements) with their block count as a constant
+            constexpr int kNb0 = 768 / F::kBlockElems, kNb1 = 1536 / F::kBlockElems;
+            const int nblk = p.nff / F::kBlockElems;
+            if (nblk == kNb0) INFR_LAUNCH((moe_down_combine_stream<F, 1, 16, kNb0>), grid, block, n_slots * cells_bytes(p.nff), s, p, ot);
+            else if (nblk == kNb1) INFR_LAUNCH((moe_down_combine_stream<F, 1, 16, kNb1>), grid, block, n_slots * cells_bytes(p.nff), s, p, ot);
+            else INFR_LAUNCH((moe_down_combine_stream<F, 1, 16>), grid, block, n_slots * cells_bytes(p.nff), s, p, ot);
             return true;
         }
         if (ot >= 2 * gstep) {
