@@ -53,7 +53,10 @@ void launch_route(hipStream_t s, const RouteParams& p) {
 // chain j of a row holds elements j, j+8, j+16, ... contiguously, so a chain thread streams
 // its operands with 128-bit LDS reads.  Strides are padded so the 16 lanes of a read phase
 // (2 experts x 8 chains) hit disjoint banks.
-template <int EPB>
+// XQ: 128-bit loads of activations a thread holds in the one-burst staging (4: up to 1024 per block; 16: four rows of
+// 4096 elements, for small batches of a wide model, whose blocks would otherwise take one token row each and read the
+// router rows once per token row).
+template <int EPB, int XQ = 4>
 __global__ __launch_bounds__(256) void router_logits_kernel(const uint8_t* __restrict__ router, int rdt,
                                                             size_t row_bytes, const float* __restrict__ x, int ne,
                                                             int n_expert, int rows, int rpb,
@@ -78,11 +81,11 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const uint8_t* __res
     const int nv = ne >> 2;
     const int rbase = blockIdx.y * rpb;   // first token row of this block's (only) pass when one_shot
     const bool one_shot = rdt == INFR_F32 && (ne & 3) == 0 && (int)gridDim.y * rpb >= rows && EPB * nv <= 8 * 256 &&
-                          rpb * nv <= 4 * 256;
+                          rpb * nv <= XQ * 256;
     if (one_shot) {
-        float4 wr[8], xr[4], nw[4];
+        float4 wr[8], xr[XQ], nw[4];
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
+        for (int i = 0; i < XQ; i++) {
             const int idx = tid + 256 * i, rr = idx / nv, v = idx - rr * nv;
             xr[i] = make_float4(0.f, 0.f, 0.f, 0.f);
             if (rr < rpb && rbase + rr < rows) xr[i] = reinterpret_cast<const float4*>(x + (size_t)(rbase + rr) * ne)[v];
@@ -123,7 +126,7 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const uint8_t* __res
         // element 4v + t of a row: chain (4v + t) & 7 = 4 (v & 1) + t, step (4v + t) >> 3 = v >> 1: the four
         // elements of a 128-bit load go to four chains at one step, or all four to the tail
 #pragma unroll
-        for (int i = 0; i < 4; i++) {
+        for (int i = 0; i < XQ; i++) {
             const int idx = tid + 256 * i, rr = idx / nv, v = idx - rr * nv;
             if (rr >= rpb) continue;
             if ((v >> 1) < nc) {
@@ -325,7 +328,8 @@ static bool router_logits_tile(int rdt, int ne, int rows, int* epb_out, int* rpb
     // staging its operands with one burst of loads.  Otherwise: 8 experts x 4 rows per pass.
     const bool small = rows <= 2 || (rows < 32 && rdt == INFR_F32 && (ne & 3) == 0 && ne <= 4096);
     int epb = small ? 2 : 8;
-    int rpb = small ? ((rows < 2 || ne > 2048) ? 1 : 2) : 4;   // the one-burst staging holds 1024 float4 of activations
+    // the one-burst staging holds 1024 128-bit loads of activations, or 4096 in its wide form (up to four rows of 4096)
+    int rpb = small ? (rows < 2 ? 1 : ne > 2048 ? (rows < 4 ? 2 : 4) : 2) : 4;
     const int nc = ne >> 3;
     const size_t estride = (size_t)8 * (((nc + 63) & ~63) + 4);
     auto lds_bytes = [&](int e, int r) { return ((size_t)(e + r) * (estride + 8)) * sizeof(float); };
@@ -390,6 +394,15 @@ bool launch_router_logits(hipStream_t s, const uint8_t* router, int rdt, size_t 
         INFR_LAUNCH(router_logits_kernel<E>, grid, block, lds, s, router, rdt, row_bytes, x, ne, n_expert,  \
                            rows, rpb, logits, nrm);                                                   \
     } while (0)
+    if (small && rpb * (ne >> 2) > 4 * 256 && epb <= 2) {   // the wide one-burst staging
+        INFR_LDS_LIMIT((router_logits_kernel<2, 16>), (int)budget);
+        if (epb == 2) INFR_LAUNCH((router_logits_kernel<2, 16>), grid, block, lds, s, router, rdt, row_bytes, x, ne, n_expert, rows, rpb, logits, nrm);
+        else {
+            INFR_LDS_LIMIT((router_logits_kernel<1, 16>), (int)budget);
+            INFR_LAUNCH((router_logits_kernel<1, 16>), grid, block, lds, s, router, rdt, row_bytes, x, ne, n_expert, rows, rpb, logits, nrm);
+        }
+        return true;
+    }
     switch (epb) {
         case 8: LAUNCH_RL(8); break;
         case 4: LAUNCH_RL(4); break;
