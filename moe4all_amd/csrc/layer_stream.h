@@ -411,6 +411,8 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
             __builtin_amdgcn_wave_barrier();
             RouteParams rp = p.route;
             rp.logits = s_logits;
+            rp.n_expert = n_expert;   // compile-time here: the routing code's loops and index arithmetic fold
+            rp.n_used = kGroups;
             // the guess is the candidate for the selection: when the exact probabilities confirm it, the selection
             // rounds are not needed; else (a missed expert, a tie at the boundary, another gating) the complete routine
             const int guess_state = lds_flag_wait(&s_f_spec);
