@@ -54,9 +54,6 @@ bool stream_shape(const MoeLayerParams& q, StreamShape* out) {
     const int rwc_g = 64 / lpr_g, rwc_d = 64 / lpr_d;
     const int rows = p.rows;
     if (rows != 1 && rows != 2 && rows != 4) return false;             // whole XCDs per token row
-    // four rows of Q8_0 banks are no faster here than on the per-token kernels (52.7 against 53.2 us at 128 experts), which
-    // run sixteen wavefronts per compute unit over their long streams; two rows are (33.6 against 36.6 us)
-    if (rows == 4 && std::is_same<FG, Q80Fmt>::value) return false;
     const int mpg = kPerGroup / rows, bpr = kBlocks / rows;
     if (nff % mpg || ne % bpr) return false;
     const int fpb = nff / mpg, R = ne / mpg;

@@ -21,6 +21,7 @@ bool launch_stream_fixed(hipStream_t s, const MoeLayerParams& q, const StreamSha
     } else if (p.gate_dt == INFR_Q8_0 && p.down_dt == INFR_Q8_0) {
         INFR_STREAM_AT(Q80Fmt, Q80Fmt, 4, 5, 1, 2, 2048, 768, 1)
         INFR_STREAM_AT(Q80Fmt, Q80Fmt, 2, 4, 1, 2, 2048, 768, 2)
+        INFR_STREAM_AT(Q80Fmt, Q80Fmt, 2, 4, 1, 2, 2048, 768, 4)
     }
 #undef INFR_STREAM_AT
     *taken = false;
