@@ -1210,7 +1210,7 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
             if (kind != infr_hip_plan::kPlain && kind != infr_hip_plan::kMoeShared) continue;
             const infr_op_moe_ffn& m = plan->ops[oi].u.moe_ffn;
             MoeScratch& sc = plan->moe[oi];
-            if ((sc.rows != 1 && sc.rows != 2 && sc.rows != 4) || sc.batched || sc.bucketed || c.dt(m.router) != INFR_F32) continue;
+            if ((sc.rows != 1 && sc.rows != 2 && sc.rows != 4 && sc.rows != 8) || sc.batched || sc.bucketed || c.dt(m.router) != INFR_F32) continue;
             infr::MoeLayerParams probe{};
             probe.g.rows = sc.rows; probe.g.ne = (int)m.ne; probe.g.nff = (int)m.n_ff_exp; probe.g.n_used = (int)m.n_used;
             probe.g.n_expert = (int)(m.has_ep_band ? m.ep_n_local : m.n_expert);

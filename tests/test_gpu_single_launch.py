@@ -265,9 +265,9 @@ def test_an_expert_the_guess_missed_is_loaded_late_and_changes_nothing(be3, skew
 
 
 @pytest.mark.parametrize("rows,gdt,ddt,skew", [(2, H.Q4K, H.Q6K, 0), (4, H.Q4K, H.Q6K, 0), (2, H.Q8_0, H.Q8_0, 0), (4, H.Q8_0, H.Q8_0, 0),
-                                               (4, H.Q4K, H.Q6K, 2), (2, H.Q8_0, H.Q8_0, 8)])
+                                               (4, H.Q4K, H.Q6K, 2), (2, H.Q8_0, H.Q8_0, 8), (8, H.Q4K, H.Q6K, 0), (8, H.Q4K, H.Q6K, 1)])
 def test_two_and_four_token_rows_in_one_launch_give_the_bits_of_three_launches(be3, rows, gdt, ddt, skew):
-    """Two or four token rows: every row takes 8 / rows of the XCDs and runs the single-token scheme among its own
+    """Two, four or eight token rows: every row takes 8 / rows of the XCDs and runs the single-token scheme among its own
     workgroups (its own logits, guess, routing, hand-overs and output rows).  Ids, weights, logits and output bits per row
     are those of the three-launch path, also when every row's guess misses `skew` experts, and a row's bits do not depend
     on its neighbours (row 0 alone gives the same)."""
