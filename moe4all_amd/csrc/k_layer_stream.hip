@@ -65,8 +65,6 @@ bool stream_shape(const MoeLayerParams& q, StreamShape* out) {
     if (my_gi * rwc_g > 64) return false;                            // a wavefront's results wait in one 64-float row
     if (shared) {
         if (nff % bpr) return false;
-        const int n_si = (nff / bpr + rwc_g - 1) / rwc_g;
-        if (n_si > kSW) return false;
     }
     // every logit once for the grid when a group's copy of the router would be a large share of the layer's bytes
     out->once = q.logits_once;

@@ -19,6 +19,8 @@ bool launch_stream_fixed(hipStream_t s, const MoeLayerParams& q, const StreamSha
         INFR_STREAM_AT(Q4KFmt, Q6KFmt, 2, 4, 1, 2, 2048, 768, 4)
         INFR_STREAM_AT(Q4KFmt, Q6KFmt, 2, 4, 2, 2, 2048, 768, 8)
         INFR_STREAM_AT(Q4KFmt, Q6KFmt, 2, 4, 1, 4, 4096, 1536, 1)   // 256 experts, with or without the always-on expert
+        INFR_STREAM_AT(Q4KFmt, Q6KFmt, 2, 4, 2, 4, 4096, 1536, 2)
+        INFR_STREAM_AT(Q4KFmt, Q6KFmt, 2, 4, 4, 4, 4096, 1536, 4)
     } else if (p.gate_dt == INFR_Q8_0 && p.down_dt == INFR_Q8_0) {
         INFR_STREAM_AT(Q80Fmt, Q80Fmt, 4, 5, 1, 2, 2048, 768, 1)
         INFR_STREAM_AT(Q80Fmt, Q80Fmt, 2, 4, 1, 2, 2048, 768, 2)

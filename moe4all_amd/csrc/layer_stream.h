@@ -475,14 +475,14 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
         bool alive = true;
 
         // gate/up items of this wavefront: item j covers features (j * kSW + sw) * rw_count + rw of the workgroup's slice.
-        // With an always-on expert the first kSW-or-fewer wavefronts take one item of its share [b * nff / 256, ..) as
-        // their ring's first entry: it needs no routing, so it is requested before the guess is known.
+        // With an always-on expert the wavefronts take the items of its share [os * nff / bpr, ..), dealt like the expert's,
+        // as their ring's first entries: they need no routing, so the first of them are requested before the guess is known.
         const int fpb = nff / mpg, f0 = m * fpb;
         const int n_gi = (fpb + pg.rw_count - 1) / pg.rw_count;
         const int my_gi = n_gi > sw ? (n_gi - sw + kSW - 1) / kSW : 0;
         const int sfpb = nff / bpr, sf0 = os * sfpb;
         const int n_si = shared ? (sfpb + pg.rw_count - 1) / pg.rw_count : 0;
-        const int sh_n = sw < n_si ? 1 : 0;
+        const int sh_n = n_si > sw ? (n_si - sw + kSW - 1) / kSW : 0;
         // down items: item j covers output rows (j * kSW + sw) * rw_count + rw of the workgroup's slice; behind them the
         // always-on expert's rows [b * ne / 256, ..), dealt to the wavefronts starting with those that got fewer above
         const int R = ne / mpg;
@@ -494,10 +494,15 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
         const int my_sdi = n_sdi > ssw ? (n_sdi - ssw + kSW - 1) / kSW : 0;
 
         GuItem gring[DG];
-        auto sh_issue = [&]() __attribute__((always_inline)) {
-            const int f = sf0 + min(sw * pg.rw_count + pg.rw, sfpb - 1);
-            gring[0].g = load_row<FG>(pg, p.sh_gate + (size_t)f * rb_g);
-            gring[0].u = load_row<FG>(pg, p.sh_up + (size_t)f * rb_g);
+        auto sh_load = [&](GuItem& it, int j) __attribute__((always_inline)) {   // item j of this wavefront's share
+            const int f = sf0 + min((j * kSW + sw) * pg.rw_count + pg.rw, sfpb - 1);
+            it.g = load_row<FG>(pg, p.sh_gate + (size_t)f * rb_g);
+            it.u = load_row<FG>(pg, p.sh_up + (size_t)f * rb_g);
+        };
+        auto sh_issue = [&]() __attribute__((always_inline)) {   // those of the first ring fill
+#pragma unroll
+            for (int d = 0; d < DG; d++)
+                if (d < sh_n) sh_load(gring[d], d);
         };
         if (sh_n && wave != 1) sh_issue();
         if (wave == 1) {
@@ -547,6 +552,10 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
             {
                 typename FG::X x;   // fetched again on a second pass: not kept alive across the hand-over
                 auto gu_issue = [&](int slot, int j) __attribute__((always_inline)) {
+                    if (j < sh) {   // more items of the always-on expert than the first ring fill held
+                        sh_load(gring[slot], j);
+                        return;
+                    }
                     const int f = min(((j - sh) * kSW + sw) * pg.rw_count + pg.rw, fpb - 1);
                     gring[slot].g = load_row<FG>(pg, gb + (size_t)f * rb_g);
                     gring[slot].u = load_row<FG>(pg, ub + (size_t)f * rb_g);
@@ -555,7 +564,7 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
                     const float gs = row_sum<FG>(FG::dot(gring[slot].g, pg.sub, x), pg, nblk_g);
                     const float us = row_sum<FG>(FG::dot(gring[slot].u, pg.sub, x), pg, nblk_g);
                     if (j < sh) {   // the always-on expert's item: its activation goes to every workgroup
-                        const int fi = sw * pg.rw_count + pg.rw;
+                        const int fi = (j * kSW + sw) * pg.rw_count + pg.rw;
                         if (pg.writer() && fi < sfpb)
                             rec_store(q.xs + sf0 + fi, gated_act_fn(p.act, p.has_clamp, p.clamp, gs, us, s_tab), tag);
                     } else if (pg.writer()) {

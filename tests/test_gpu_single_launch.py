@@ -398,9 +398,10 @@ def _shared_graph(ne, E, K, nff, gated, rows=1):
     return g, ids
 
 
-@pytest.mark.parametrize("ne,E,nff,gated,skew", [(4096, 256, 1536, False, 0), (4096, 256, 1536, True, 0),
-                                                 (4096, 256, 1536, False, 2), (2048, 128, 768, False, 0)])
-def test_single_launch_with_the_always_on_expert_folded_in(be3, ne, E, nff, gated, skew):
+@pytest.mark.parametrize("ne,E,nff,gated,skew,rows", [(4096, 256, 1536, False, 0, 1), (4096, 256, 1536, True, 0, 1),
+                                                      (4096, 256, 1536, False, 2, 1), (4096, 256, 1536, False, 0, 2),
+                                                      (4096, 256, 1536, True, 1, 4), (2048, 128, 768, False, 0, 1)])
+def test_single_launch_with_the_always_on_expert_folded_in(be3, ne, E, nff, gated, skew, rows):
     """The large shape's layer (256 experts, hidden 4096, an always-on expert beside the routed ones) as ONE launch: the
     always-on expert's rows are spread over all workgroups and requested first.  Same bits as the three-launch path,
     within the parity bar of the oracle."""
@@ -416,16 +417,18 @@ def test_single_launch_with_the_always_on_expert_folded_in(be3, ne, E, nff, gate
     data = dict(_SHARED_CASES[(ne, E, nff)])
     if not gated:
         del data["wq"]
+    if rows > 1:   # more token rows: each takes 8 / rows of the XCDs, the always-on expert's share per workgroup grows
+        data["x"] = np.random.default_rng(rows).standard_normal((rows, ne)).astype(np.float32)
     b = M.Backend(0, single_launch_guess_skew=skew)
     try:
-        g, ids = _shared_graph(ne, E, K, nff, gated)
-        one, r1 = _run(b, g, ids, data, ne, "moe_layer_shared")
-        g, ids = _shared_graph(ne, E, K, nff, gated)
-        three, r3 = _run(be3, g, ids, data, ne, "moe_route_gate_up_shared")
+        g, ids = _shared_graph(ne, E, K, nff, gated, rows)
+        one, r1 = _run(b, g, ids, data, rows * ne, "moe_layer_shared")
+        g, ids = _shared_graph(ne, E, K, nff, gated, rows)
+        three, r3 = _run(be3, g, ids, data, rows * ne, "moe_route_gate_up_shared")
         assert np.array_equal(r1["idx"], r3["idx"]) and np.array_equal(bits(r1["w"]), bits(r3["w"]))
         assert np.array_equal(bits(r1["logits"]), bits(r3["logits"]))
         assert np.array_equal(bits(one), bits(three))
-        assert b.late_experts() == skew
+        assert b.late_experts() == skew * rows
     finally:
         b.close()
     ref = O.moe_ffn(data["x"], data["router"], data["gate"], data["up"], data["down"], ne=ne, n_expert=E, n_used=K,
@@ -435,7 +438,7 @@ def test_single_launch_with_the_always_on_expert_folded_in(be3, ne, E, nff, gate
         sh = O.moe_ffn(data["x"], np.zeros((1, ne), np.float32), data["sg"], data["su"], data["sd"], ne=ne, n_expert=1,
                        n_used=1, n_ff_exp=nff, gate_dtype=H.Q4K, down_dtype=H.Q6K)
         want = ref["dst"] + sh["dst"]
-        assert H.rel_l2(one, want) < 1e-3 and H.max_abs(one, want) < 2e-3
+        assert H.rel_l2(one.reshape(want.shape), want) < 1e-3 and H.max_abs(one.reshape(want.shape), want) < 2e-3
 
 
 @pytest.mark.parametrize("gated", [False, True])
