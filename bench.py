@@ -202,7 +202,7 @@ def measure(be, stack, config, batch, steps, warmup, *, sublayer=False, kernel_t
     tok_s = batch * steps / elapsed
     # spread: the same steps again in ten groups, each bracketed by a sync
     groups = max(1, min(10, steps))
-    per_group = max(1, steps // groups)
+    per_group = max(10, steps // groups)   # long enough that a group's sync and first dispatch do not show in its mean
     group_ms = []
     for gi in range(groups):
         t1 = time.perf_counter()
