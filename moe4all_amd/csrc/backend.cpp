@@ -1238,7 +1238,17 @@ extern "C" infr_status infr_hip_compile(infr_hip_backend* be, const infr_graph* 
             } else {
                 continue;
             }
-            if (plan->fuse[oi].norm) {
+            // An RmsNorm folded into the logits kernel stays folded for the streaming kernel, which normalises the row
+            // itself (and for the three launches it falls back to); the in-order kernel has no such fold, and the gated
+            // always-on expert's gate-logit launch reads the normalised row before the layer's launch: both take the norm
+            // as an op of its own.
+            bool keep_norm = false;
+            if (plan->fuse[oi].norm && sc.single_launch == 2 && !plan->fuse[oi].gated) {
+                const infr_op_rms_norm& nr = plan->ops[plan->fuse[oi].norm - 1].u.rms_norm;
+                probe.norm_w = (const float*)plan;   // non-null: asked for
+                keep_norm = sc.rows == 1 && m.x == nr.dst && infr::moe_layer_stream_supported(probe);
+            }
+            if (plan->fuse[oi].norm && !keep_norm) {
                 plan->fuse[plan->fuse[oi].norm - 1].kind = infr_hip_plan::kPlain;
                 plan->fuse[oi].norm = 0;
             }
@@ -1538,9 +1548,21 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                         lp.late = be->fault_dev + 1;
                         lp.logits_once = moe_logits_once(be, m);
                         lp.guess_skew = (int)std::min<uint32_t>(be->cfg.single_launch_guess_skew, 8u);
-                        if (infr::moe_layer_stream_supported(lp) &&
+                        bool norm_ok = true;
+                        if (fz.norm) {   // the token row's RmsNorm, folded: the kernel normalises the raw row
+                            const infr_op_rms_norm& nr = plan->ops[fz.norm - 1].u.rms_norm;
+                            if (!(need(nr.x, "RmsNorm.x") && need(nr.weight, "RmsNorm.weight") && need(nr.dst, "RmsNorm.dst")))
+                                return INFR_ERR_BACKEND;
+                            lp.norm_x = (const float*)ptr[nr.x];
+                            lp.norm_w = (const float*)ptr[nr.weight];
+                            lp.norm_out = (float*)ptr[nr.dst];
+                            lp.norm_eps = nr.eps;
+                            lp.norm_for_x = m.x == nr.dst ? 1 : 0;
+                            norm_ok = nr.x != nr.dst && m.x == nr.dst && rows == 1 && (((uintptr_t)lp.norm_x | (uintptr_t)lp.norm_w | (uintptr_t)lp.norm_out) & 15) == 0;
+                        }
+                        if (norm_ok && infr::moe_layer_stream_supported(lp) &&
                             (((uintptr_t)lp.router | (uintptr_t)lp.router_x | (uintptr_t)gp.x) & 15) == 0 && (lp.router_row_floats & 3) == 0) {
-                            launch_gate_logit();   // no norm is folded on this path: the row it reads is there
+                            launch_gate_logit();   // (a gated always-on expert keeps its norm as an op: the row this reads is there)
                             Timed t(be, gp.sh_gate ? "moe_layer_shared" : "moe_layer");
                             if (infr::launch_moe_layer_stream(s, lp)) break;
                             return fail(INFR_ERR_BACKEND, "MoeFfn: the single-launch kernel refused a shape it had accepted");

@@ -99,6 +99,7 @@ bool dispatch_stream(hipStream_t s, MoeLayerParams q, bool launch) {
         const bool done = launch_stream_fixed(s, q, sh, launch, &taken);
         if (taken) return done;
     }
+    if (q.norm_w) return false;   // the fold of the token row's RmsNorm exists for the fixed shapes only
     if constexpr (std::is_same<FG, Q4KFmt>::value) {
         INFR_STREAM(2, 2, 2, 2)   // ne 2048, nff 768, 128 experts, a copy of the router per group
         INFR_STREAM(2, 2, 1, 2)   // ... every logit once

@@ -152,6 +152,13 @@ struct MoeLayerParams {
     int logits_once;            // every logit computed by one workgroup for the whole grid, not once per group
     int guess_skew;             // tests: the guess leaves out this many of the largest estimates
     int epb, early_down;        // set by the launcher
+    // an Op::RmsNorm of the single token row folded in (null norm_w: none): router_x is then ignored, the routing row is
+    // rmsnorm(norm_x) * norm_w, stored to norm_out by one workgroup; norm_for_x: g.x is that row too (and is not read)
+    const float* norm_x = nullptr;
+    const float* norm_w = nullptr;
+    float* norm_out = nullptr;
+    float norm_eps = 0.0f;
+    int norm_for_x = 0;
 };
 size_t moe_layer_workspace_bytes(int ne, int nff, int n_expert);
 bool moe_layer_fused_supported(const MoeLayerParams& q);

@@ -218,7 +218,9 @@ __device__ __forceinline__ float dot8(const float4& a0, const float4& a1, const 
 // NE, NFF, ROWS: hidden size, intermediate size and token rows when they are known at compile time (the benchmark
 // shapes), 0 for any shape.  With constants the lane placement, the item counts and every index division below fold;
 // with run-time values they are integer arithmetic on the critical path of a kernel that one wavefront paces.
-template <class FG, class FD, int DG, int DD, int EPT, int NSP, int NE = 0, int NFF = 0, int ROWS = 0>
+// NORM: 1 with an Op::RmsNorm of the token row folded in (its own instantiations: the branches of a run-time switch cost
+// the plain kernel a microsecond and a half of its operand staging).
+template <class FG, class FD, int DG, int DD, int EPT, int NSP, int NE = 0, int NFF = 0, int ROWS = 0, int NORM = 0>
 __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
     extern __shared__ __attribute__((aligned(16))) uint32_t dyn_lds[];
     __shared__ uint64_t s_tab[32];
@@ -228,8 +230,9 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
     __shared__ float s_part[kWaves][8];
     __shared__ int32_t s_spec[kGroups], s_final[kGroups], s_gor[kGroups];
     __shared__ float s_ysh[64];
+    __shared__ float s_red[4];
     __shared__ uint32_t s_guess[2 * kWave];
-    __shared__ int s_f_spec, s_f_route, s_f_hs, s_fault, s_cells_done, s_h_done, s_done;
+    __shared__ int s_f_spec, s_f_route, s_f_hs, s_fault, s_cells_done, s_h_done, s_done, s_xn_done;
     __shared__ uint32_t s_seq;
     const MoeGemvParams& p = q.g;
     const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;   // wave: uniform, scalar registers
@@ -289,7 +292,7 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
 
     if (tid < 32) s_tab[tid] = kExp2Table[tid];
     if (tid == 0) {
-        s_f_spec = s_f_route = s_f_hs = s_fault = s_cells_done = s_h_done = s_done = 0;
+        s_f_spec = s_f_route = s_f_hs = s_fault = s_cells_done = s_h_done = s_done = s_xn_done = 0;
         // the launch's number: every workgroup keeps its own count of the launches it has run (a counter shared by all
         // would serialise 256 atomics, at the start or, worse, at the end of the kernel), read here and written back
         // with a plain store at the end; launches on a workspace never overlap, so all 256 counts agree
@@ -304,13 +307,22 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
     // row and of the router rows hsel, hsel + H, ...  The token row becomes fixed-point cells later, by the threads
     // of the last replica (with two replicas that keeps the router's and the guessing wavefront out of it).
     const bool converts = hsel == H - 1;
-    float4 cx0, cx1;
+    constexpr bool normed = NORM != 0;   // one token row only; the token row is then the normalised row (the host checks)
+    float4 cx0, cx1, nw0, nw1;
     {
-        const float4* rx4 = reinterpret_cast<const float4*>(q.router_x);
-        const float4 rx0 = rx4[2 * o], rx1 = rx4[2 * o + 1];
-        const float4* px4 = reinterpret_cast<const float4*>(p.x);
-        cx0 = px4[2 * o];
-        cx1 = px4[2 * o + 1];
+        const float4* rx4 = reinterpret_cast<const float4*>(normed ? q.norm_x : q.router_x);
+        float4 rx0 = rx4[2 * o], rx1 = rx4[2 * o + 1];
+        if (normed) {   // the routing row and the token row are one row, raw so far
+            cx0 = rx0;
+            cx1 = rx1;
+            const float4* nw4 = reinterpret_cast<const float4*>(q.norm_w);
+            nw0 = nw4[2 * o];
+            nw1 = nw4[2 * o + 1];
+        } else {
+            const float4* px4 = reinterpret_cast<const float4*>(p.x);
+            cx0 = px4[2 * o];
+            cx1 = px4[2 * o + 1];
+        }
         float4 w0[EPT], w1[EPT];
 #pragma unroll
         for (int i = 0; i < EPT; i++) {
@@ -320,6 +332,21 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
             w0[i] = row[2 * o];
             w1[i] = row[2 * o + 1];
         }
+        if (normed) {
+            // An Op::RmsNorm of the single token row folded in: the row arrives raw and every workgroup normalises it.
+            // The sum of squares runs exactly as in the standalone kernel - 256 threads, thread t over the 128-bit pieces
+            // t, t + 256, ..., the same tree over the threads - so the scale has the same bits; it takes its own loads of
+            // the row (the pieces this thread holds for the dots are two neighbours).  The scale is applied behind the
+            // barrier below.  The estimates do not wait for it: a positive factor common to all of them does not change
+            // their order, so they are taken from x * w without the scale.
+            float part = 0.0f;
+            if (tid < 256)
+                for (int v = tid; v < (ne >> 2); v += 256) part = sumsq4(part, rx4[v]);
+            part = wave_sum(part);
+            if (lane == 0 && wave < 4) s_red[wave] = part;
+            rx0 = make_float4(rx0.x * nw0.x, rx0.y * nw0.y, rx0.z * nw0.z, rx0.w * nw0.w);
+            rx1 = make_float4(rx1.x * nw1.x, rx1.y * nw1.y, rx1.z * nw1.z, rx1.w * nw1.w);
+        }
         // the estimate's share of this thread, summed over the wavefront
 #pragma unroll
         for (int i = 0; i < EPT; i++) {
@@ -327,7 +354,7 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
             if (lane == 0) s_part[wave][i] = part;
         }
         // chain operands: element 8 o + t belongs to chain t, position o
-        if (hsel == 0) {
+        if (hsel == 0 && !normed) {
             const float xv[8] = {rx0.x, rx0.y, rx0.z, rx0.w, rx1.x, rx1.y, rx1.z, rx1.w};
 #pragma unroll
             for (int t = 0; t < 8; t++) xst[t * jstride + o] = xv[t];
@@ -366,6 +393,24 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
         while (__builtin_amdgcn_readfirstlane(*(volatile int*)&s_cells_done) < n_conv_waves) __builtin_amdgcn_s_sleep(1);
         asm volatile("" ::: "memory");
     };
+    if (normed) {
+        // the scale, the same bits in every thread; the normalised row for the cells, for the exact chains (the router's
+        // wavefront waits for the wavefronts that stage it) and, from one workgroup, for the RmsNorm's dst
+        const float sc = rms_scale((s_red[0] + s_red[1]) + (s_red[2] + s_red[3]), ne, q.norm_eps);
+        cx0 = rms_apply4(cx0, sc, nw0);
+        cx1 = rms_apply4(cx1, sc, nw1);
+        if (hsel == 0) {
+            const float xv[8] = {cx0.x, cx0.y, cx0.z, cx0.w, cx1.x, cx1.y, cx1.z, cx1.w};
+#pragma unroll
+            for (int t = 0; t < 8; t++) xst[t * jstride + o] = xv[t];
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            if (lane == 0) __hip_atomic_fetch_add(&s_xn_done, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            if (os == 0 && q.norm_out) {
+                reinterpret_cast<float4*>(q.norm_out)[2 * o] = cx0;
+                reinterpret_cast<float4*>(q.norm_out)[2 * o + 1] = cx1;
+            }
+        }
+    }
     if (wave != 1) convert_share();
     if (wave == 0) STAMP(2);
 
@@ -377,6 +422,10 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
             const int e = lane >> 3, j = lane & 7;
             const bool live = has_rows && e < epb;
             float acc = 0.0f;
+            if (normed) {   // the normalised row is staged behind the barrier, by oct_n / 64 wavefronts
+                while (__builtin_amdgcn_readfirstlane(*(volatile int*)&s_xn_done) < waves_per_replica) __builtin_amdgcn_s_sleep(1);
+                asm volatile("" ::: "memory");
+            }
             if (live) {
                 // the reference's order: 8 chains over i = j (mod 8), summed 0..7 (crates/infr-cpu/src/kernels.rs:6568-6583)
                 const float4* wp = reinterpret_cast<const float4*>(wst + (e * 8 + j) * jstride);
@@ -751,18 +800,18 @@ struct StreamShape {
 
 namespace {
 
-template <class FG, class FD, int DG, int DD, int EPT, int NSP, int NE = 0, int NFF = 0, int ROWS = 0>
+template <class FG, class FD, int DG, int DD, int EPT, int NSP, int NE = 0, int NFF = 0, int ROWS = 0, int NORM = 0>
 bool launch_stream(hipStream_t s, const MoeLayerParams& q, size_t lds) {
     static bool attr_ok[16] = {};
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return false;
     if (!attr_ok[dev]) {
-        if (hipFuncSetAttribute((const void*)moe_layer_stream<FG, FD, DG, DD, EPT, NSP, NE, NFF, ROWS>,
+        if (hipFuncSetAttribute((const void*)moe_layer_stream<FG, FD, DG, DD, EPT, NSP, NE, NFF, ROWS, NORM>,
                                 hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024) != hipSuccess)
             return false;
         attr_ok[dev] = true;
     }
-    INFR_LAUNCH((moe_layer_stream<FG, FD, DG, DD, EPT, NSP, NE, NFF, ROWS>), dim3(kBlocks), dim3(kThreads), lds, s, q);
+    INFR_LAUNCH((moe_layer_stream<FG, FD, DG, DD, EPT, NSP, NE, NFF, ROWS, NORM>), dim3(kBlocks), dim3(kThreads), lds, s, q);
     return true;
 }
 

@@ -459,3 +459,70 @@ def test_two_token_rows_with_the_always_on_expert_folded_in(be, be3, gated):
     assert np.array_equal(r1["idx"], r3["idx"]) and np.array_equal(bits(r1["w"]), bits(r3["w"]))
     assert np.array_equal(bits(one), bits(three))
     assert np.abs(one.reshape(rows, ne)[1]).max() > 1e-5
+
+
+@pytest.mark.parametrize("shared", [False, True])
+def test_single_launch_with_the_rms_norm_and_the_residual_folded_in(be, shared):
+    """The model's whole FFN sublayer for one token, y = x + ffn(rmsnorm(x) * w), as ONE launch: every workgroup
+    normalises the raw row itself (the sum of squares in the standalone kernel's order, so the same bits) and one of them
+    stores the normalised row where the RmsNorm's dst is.  Same bits as one launch per op, and the normalised row is there."""
+    ne, E, K, nff, eps = 2048, 128, 8, 768, 1e-6
+    rng = np.random.default_rng(90 + shared)
+    x = (rng.standard_normal((1, ne)) * 3.0).astype(np.float32)
+    nw = rng.uniform(0.5, 1.5, ne).astype(np.float32)
+    router = (rng.standard_normal((E, ne)) * 0.02).astype(np.float32)
+    gate, up, down = _banks(rng, E, nff, ne, H.Q4K, H.Q6K)
+    sg, su, sd = (a.reshape(-1) for a in _banks(rng, 1, nff, ne, H.Q4K, H.Q6K))
+    outs, norms, names = {}, {}, {}
+    for off in (False, True):
+        b = be if not off else M.Backend(0, disable_op_fusion=True, disable_single_launch_moe=True)
+        try:
+            g = M.Graph()
+            T = M.TensorDesc
+            xi, nwt = g.input(T([1, ne], DType.F32)), g.weight(T([ne], DType.F32))
+            rt = g.weight(T([E, ne], DType.F32))
+            gt, ut = g.weight(T([E, nff, ne], DType.Q4K)), g.weight(T([E, nff, ne], DType.Q4K))
+            dt = g.weight(T([E, ne, nff], DType.Q6K))
+            xn = g.output(T([1, ne], DType.F32))      # declared an output: the normalised row has to be materialised
+            moe = g.internal(T([1, ne], DType.F32))
+            yi = g.output(T([1, ne], DType.F32))
+            g.rms_norm(x=xi, weight=nwt, dst=xn, rows=1, dim=ne, eps=eps)
+            g.moe_ffn(x=xn, router=rt, gate_exps=gt, up_exps=ut, down_exps=dt, dst=moe, ne=ne, n_expert=E, n_used=K, n_ff_exp=nff)
+            bound = [(xi, x), (nwt, nw), (rt, router), (gt, gate), (ut, up), (dt, down)]
+            sub = moe
+            if shared:
+                wg, wu, wd = g.weight(T([nff, ne], DType.Q4K)), g.weight(T([nff, ne], DType.Q4K)), g.weight(T([ne, nff], DType.Q6K))
+                tg, tu, ta = (g.internal(T([1, nff], DType.F32)) for _ in range(3))
+                ts, sub = g.internal(T([1, ne], DType.F32)), g.internal(T([1, ne], DType.F32))
+                g.linear(x=xn, weight=wg, dst=tg, m=1, in_f=ne, out_f=nff)
+                g.linear(x=xn, weight=wu, dst=tu, m=1, in_f=ne, out_f=nff)
+                g.gated_act(gate=tg, up=tu, dst=ta, rows=1, nff=nff)
+                g.linear(x=ta, weight=wd, dst=ts, m=1, in_f=nff, out_f=ne)
+                g.add(a=moe, b=ts, dst=sub, n=ne)
+                bound += [(wg, sg), (wu, su), (wd, sd)]
+            g.add(a=xi, b=sub, dst=yi, n=ne)
+            plan = b.compile(g)
+            bufs, bind = [], M.Bindings()
+            for tid, v in bound:
+                bufs.append(b.buffer_from(v))
+                bind.bind(tid, bufs[-1])
+            o_xn, o_y = b.alloc(ne * 4), b.alloc(ne * 4)
+            bind.bind(xn, o_xn)
+            bind.bind(yi, o_y)
+            b.prof_enable(True)
+            b.execute(plan, bind)
+            outs[off] = b.download(o_y, ne * 4, np.float32).copy()
+            norms[off] = b.download(o_xn, ne * 4, np.float32).copy()
+            names[off] = set(b.prof_read())
+            b.prof_enable(False)
+            for buf in bufs + [o_xn, o_y]:
+                buf.free()
+            plan.free()
+        finally:
+            if off:
+                b.close()
+    assert names[False] == {"moe_layer_shared" if shared else "moe_layer"}, names[False]
+    assert "rms_norm" in names[True] and "add" in names[True]
+    assert np.array_equal(bits(norms[False]), bits(norms[True]))
+    assert np.array_equal(bits(outs[False]), bits(outs[True]))
+    assert H.rel_l2(norms[False].reshape(1, ne), O.rms_norm(x, nw, eps).reshape(1, ne)) < 1e-5
