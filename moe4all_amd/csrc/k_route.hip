@@ -221,18 +221,18 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const uint8_t* __res
 }
 
 // ---------------------------------------------------------------------------------------------
-// Logits for a batch (f32 router, ne a multiple of 32).  Block = 512 threads covering 32 experts
-// x 32 token rows: 8 chains x 8 row groups per wave, one wave per group of 4 experts.  A thread
-// keeps a 4 x 4 (expert, row) patch of accumulators for its chain, so each 128-bit LDS read
-// feeds 16 FMAs.  The patch's rows are G apart (rows b * G + rg): the sixteen lanes the LDS serves together then read
+// Logits for a batch on the vector ALUs (f32 router, ne a multiple of 32; batches too small to give the matrix-core
+// kernel below a workgroup per compute unit).  Block = 512 threads covering kLtTile experts x kLtTile token rows: 8
+// chains x G row groups x G expert groups.  A thread keeps a P x P (expert, row) patch of accumulators for its chain,
+// so each 128-bit LDS read feeds 4 P FMAs.  The patch's rows are G apart (rows b * G + rg): the sixteen lanes the LDS serves together then read
 // sixteen consecutive 80-byte rows, which fall on distinct banks (rows 32 apart are 2560 bytes = a whole number of
 // bank rounds apart and collided).  k advances in chunks of 128 elements staged transposed (chain-major) in LDS;
 // the accumulators run through all chunks, so every chain still adds its terms in ascending
 // order, exactly as the scalar reference does.
 constexpr int kLtChunk = 128, kLtStride = kLtChunk / 8 + 4;
-// kLtTile experts x kLtTile rows per block, a P x P patch per thread: 32 / 4 (512 threads) for large batches; 16 / 2
-// (512 threads, a quarter of the chain work per thread) when 32-wide tiles would leave compute units without a block:
-// a block's time is its chunks' latency chain, which the smaller patch shortens.
+// kLtTile experts x kLtTile rows per block, a P x P patch per thread.  Instantiated as 16 / 2 (512 threads): a block's
+// time is its chunks' latency chain, which a small patch keeps short (32 / 4 was the kernel for large batches before
+// the matrix-core kernel: 28 us against 18 us for 2048 rows x 128 experts x 2048).
 template <int kLtTile, int P>
 __global__ __launch_bounds__((kLtTile / P) * (kLtTile / P) * 8) void router_logits_tiled_kernel(const float* __restrict__ router,
                                                                                       size_t row_floats,
@@ -320,6 +320,188 @@ __global__ __launch_bounds__((kLtTile / P) * (kLtTile / P) * 8) void router_logi
         }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Logits for a batch on the matrix cores.  v_mfma_f32_16x16x1_4b_f32 computes D_b[i][j] = A_b[i] * B_b[j] + C_b[i][j]
+// for four independent 16 x 16 blocks b: with one k per instruction every element is ONE fused multiply-add, so a
+// chain of them over k = 8 s + c, s ascending, is the reference's chain c term by term (the same bits as __fmaf_rn;
+// the parity tests compare them with the scalar restatement bit for bit).  A block b holds one chain, so two
+// instructions per step cover the eight chains of a 16 (token) x 16 (expert) tile, and the two accumulator sets are
+// independent, which keeps the pipe busy from one wavefront.
+// Workgroup = 32 tokens x 32 experts = 8 wavefronts, two per SIMD: wavefronts 0-3 contract (each a 16 x 16 tile),
+// wavefronts 4-7 only move data, so that no load, LDS store or address arithmetic sits between two matrix
+// instructions of a contracting wavefront (one wavefront doing both ran at half the rate).  Operands are staged per
+// 128-k chunk transposed in LDS as [chain][row][step] (row stride 20 floats, chain stride = 8 mod 16: the 128-bit
+// reads and the 32-bit stores are free of bank conflicts), double-buffered, one barrier per chunk.  A contracting
+// wavefront passes the barrier in the MIDDLE of a chunk's matrix instructions and reads the next chunk's first half
+// behind it, beside the second half of its instructions, so neither the barrier nor the LDS latency empties the pipe.
+// The moving wavefronts load four chunks ahead in registers.
+// Lane l supplies A = x[token l % 16][chain l / 16], B = w[expert l % 16][chain l / 16]; it receives, in register
+// 4 b + i, the element (token 4 (l / 16) + i, expert l % 16) of chain b, so the sum over the chains is lane-local.
+// Workgroups that share a token tile (one per 32 experts) are given indices 8 apart: they run on one XCD and the
+// tile's activations come through one L2.
+constexpr int kLmChunk = 128, kLmRow = kLmChunk / 8 + 4, kLmTile = 32;
+constexpr int kLmChain = kLmTile * kLmRow + 8;                         // floats of one chain
+constexpr int kLmOperand = 8 * kLmChain;                               // floats of one operand's chunk
+constexpr size_t kLmLdsBytes = (size_t)4 * kLmOperand * sizeof(float);   // two operands, two buffers
+typedef float lm_acc_t __attribute__((ext_vector_type(16)));
+struct LmHalf { float4 w[2][2], x[2][2]; };   // operands of half a chunk: [four steps][accumulator set]
+__global__ __launch_bounds__(512) void router_logits_mfma_kernel(const float* __restrict__ router, size_t row_floats,
+                                                                 const float* __restrict__ x, int ne, int n_expert,
+                                                                 int rows, float* __restrict__ logits) {
+    extern __shared__ float lm_lds[];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int neb = (n_expert + kLmTile - 1) / kLmTile, bq = blockIdx.x >> 3;
+    const int e0 = (bq % neb) * kLmTile, r0 = ((bq / neb) * 8 + (blockIdx.x & 7)) * kLmTile;
+    if (r0 >= rows) return;
+    const int nfast = (ne / kLmChunk) & ~3;   // whole chunks that run through the pipelines below, four per trip
+    if (wave >= 4) {
+        // ---- the moving wavefronts: four 128-bit loads of each operand per thread and chunk; load q covers row
+        // srow + 8 (q & 3), floats 4 v .. 4 v + 3 of the chunk.  Rows past the end repeat the last one (their results
+        // are never stored), and so do loads past the end of a row (those steps are never contracted).
+        const int srow = (wave - 4) + 4 * ((tid >> 5) & 1), v = tid & 31;
+        const float* src[8];
+#pragma unroll
+        for (int q = 0; q < 8; q++) {
+            const bool is_x = q >= 4;
+            const int g = min((is_x ? r0 : e0) + srow + 8 * (q & 3), (is_x ? rows : n_expert) - 1);
+            src[q] = is_x ? x + (size_t)g * ne : router + (size_t)g * row_floats;
+        }
+        // element 4 v + t of the chunk: chain 4 (v & 1) + t, step v >> 1
+        const int dst0 = 4 * (v & 1) * kLmChain + srow * kLmRow + (v >> 1);
+        auto fetch = [&](float4 (&st)[8], int k0) __attribute__((always_inline)) {
+            const int k = min(k0 + 4 * v, ne - 4);
+#pragma unroll
+            for (int q = 0; q < 8; q++) st[q] = *reinterpret_cast<const float4*>(src[q] + k);
+        };
+        auto deposit = [&](const float4 (&st)[8], int buf) __attribute__((always_inline)) {
+#pragma unroll
+            for (int q = 0; q < 8; q++) {
+                float* d = lm_lds + (2 * buf + (q >= 4 ? 1 : 0)) * kLmOperand + dst0 + 8 * (q & 3) * kLmRow;
+                d[0] = st[q].x;
+                d[kLmChain] = st[q].y;
+                d[2 * kLmChain] = st[q].z;
+                d[3 * kLmChain] = st[q].w;
+            }
+        };
+        if (nfast > 0) {
+            // chunk c is loaded into register set c % 4 and deposited into LDS buffer c % 2 while chunk c - 1 is contracted
+            // (one basic block per trip, its order pinned: the compiler otherwise sinks the loads to their deposits)
+            float4 s0[8], s1[8], s2[8], s3[8];
+            auto step = [&](int c, float4 (&s_free)[8], const float4 (&s_next)[8], int buf) __attribute__((always_inline)) {
+                fetch(s_free, min(c + 4, nfast - 1) * kLmChunk);
+                __builtin_amdgcn_sched_barrier(0);
+                deposit(s_next, buf ^ 1);   // past the last chunk: a repeat of it that nobody contracts
+                __builtin_amdgcn_sched_barrier(0);
+                __syncthreads();
+                __builtin_amdgcn_sched_barrier(0);
+            };
+            fetch(s0, 0);
+            fetch(s1, kLmChunk);
+            fetch(s2, 2 * kLmChunk);
+            fetch(s3, 3 * kLmChunk);
+            deposit(s0, 0);
+            __syncthreads();
+            for (int c = 0; c < nfast; c += 4) {
+                step(c, s0, s1, 0);
+                step(c + 1, s1, s2, 1);
+                step(c + 2, s2, s3, 0);
+                step(c + 3, s3, s0, 1);
+            }
+        }
+        for (int k0 = nfast * kLmChunk; k0 < ne; k0 += kLmChunk) {   // up to three whole chunks and a shorter one
+            float4 st[8];
+            fetch(st, k0);
+            __syncthreads();
+            deposit(st, 0);
+            __syncthreads();
+        }
+        return;
+    }
+    // ---- the contracting wavefronts
+    const int tw = wave & 1, ew = wave >> 1;   // the wavefront's 16 x 16 tile of the workgroup's 32 x 32
+    // the lane's operands of accumulator set s: chain 4 s + lane / 16, row lane % 16 of the wavefront's tile
+    const int wo = (lane >> 4) * kLmChain + (16 * ew + (lane & 15)) * kLmRow;
+    const int xo = (lane >> 4) * kLmChain + (16 * tw + (lane & 15)) * kLmRow + kLmOperand;
+    auto read_half = [&](LmHalf& o, int buf, int half) __attribute__((always_inline)) {
+        const float* base = lm_lds + 2 * buf * kLmOperand + 8 * half;
+#pragma unroll
+        for (int c = 0; c < 2; c++)
+#pragma unroll
+            for (int s = 0; s < 2; s++) {
+                o.w[c][s] = *reinterpret_cast<const float4*>(base + wo + 4 * s * kLmChain + 4 * c);
+                o.x[c][s] = *reinterpret_cast<const float4*>(base + xo + 4 * s * kLmChain + 4 * c);
+            }
+    };
+    lm_acc_t acc[2];
+#pragma unroll
+    for (int s = 0; s < 2; s++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) acc[s][i] = 0.0f;
+    auto contract4 = [&](const LmHalf& o, int c) __attribute__((always_inline)) {   // four steps of both sets
+#pragma unroll
+        for (int s = 0; s < 2; s++) acc[s] = __builtin_amdgcn_mfma_f32_16x16x1f32(o.x[c][s].x, o.w[c][s].x, acc[s], 0, 0, 0);
+#pragma unroll
+        for (int s = 0; s < 2; s++) acc[s] = __builtin_amdgcn_mfma_f32_16x16x1f32(o.x[c][s].y, o.w[c][s].y, acc[s], 0, 0, 0);
+#pragma unroll
+        for (int s = 0; s < 2; s++) acc[s] = __builtin_amdgcn_mfma_f32_16x16x1f32(o.x[c][s].z, o.w[c][s].z, acc[s], 0, 0, 0);
+#pragma unroll
+        for (int s = 0; s < 2; s++) acc[s] = __builtin_amdgcn_mfma_f32_16x16x1f32(o.x[c][s].w, o.w[c][s].w, acc[s], 0, 0, 0);
+    };
+    if (nfast > 0) {
+        // chunk c is read from LDS buffer c % 2 half a chunk at a time: its first half beside the second half of chunk
+        // c - 1's matrix instructions, its second half beside its own first half
+        LmHalf h1, h2;
+        __syncthreads();
+        read_half(h1, 0, 0);
+        for (int c = 0; c < nfast; c++) {
+            const int buf = c & 1;
+            contract4(h1, 0);
+            contract4(h1, 1);
+            read_half(h2, buf, 1);
+#pragma unroll
+            for (int i = 0; i < 8; i++) {   // one matrix instruction, one LDS read
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            __syncthreads();
+            __builtin_amdgcn_sched_barrier(0);
+            contract4(h2, 0);
+            contract4(h2, 1);
+            read_half(h1, buf ^ 1, 0);
+#pragma unroll
+            for (int i = 0; i < 8; i++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    }
+    for (int k0 = nfast * kLmChunk; k0 < ne; k0 += kLmChunk) {   // up to three whole chunks and a shorter one, unpipelined
+        __syncthreads();
+        __syncthreads();
+        const int steps = min(kLmChunk, ne - k0) >> 3;   // 4, 8, 12 or 16 (ne is a multiple of 32)
+        LmHalf o;
+        read_half(o, 0, 0);
+        contract4(o, 0);
+        if (steps > 4) contract4(o, 1);
+        if (steps > 8) {
+            read_half(o, 0, 1);
+            contract4(o, 0);
+            if (steps > 12) contract4(o, 1);
+        }
+    }
+    const int e = e0 + 16 * ew + (lane & 15);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        float s = 0.0f;
+#pragma unroll
+        for (int c = 0; c < 8; c++) s = __fadd_rn(s, acc[c >> 2][4 * (c & 3) + i]);
+        const int r = r0 + 16 * tw + 4 * (lane >> 4) + i;
+        if (e < n_expert && r < rows) logits[(size_t)r * n_expert + e] = s;
+    }
+}
+
 // Experts and token rows per block of router_logits_kernel for a shape, or false when even one of each does
 // not fit the LDS budget.
 constexpr size_t kRouterLdsBudget = 140 * 1024;
@@ -359,10 +541,13 @@ bool launch_router_logits(hipStream_t s, const uint8_t* router, int rdt, size_t 
                        (((uintptr_t)x | (uintptr_t)nrm.weight | (uintptr_t)nrm.xn_out) & 15) != 0))
         return false;
     if (rows >= 32 && rdt == INFR_F32 && (ne & 31) == 0 && (row_bytes & 15) == 0) {
-        // 32 x 32 tiles when they give every compute unit a block, 16 x 16 otherwise
-        if ((size_t)((n_expert + 31) / 32) * ((rows + 31) / 32) >= 256) {
-            dim3 grid((n_expert + 31) / 32, (rows + 31) / 32);
-            INFR_LAUNCH((router_logits_tiled_kernel<32, 4>), grid, dim3(512), 0, s, reinterpret_cast<const float*>(router),
+        // the matrix-core kernel when its 32 x 32 tiles give every compute unit a workgroup, 16 x 16 tiles on the
+        // vector ALUs otherwise (a workgroup's time does not shrink with the batch: it is its chain length)
+        const int neb = (n_expert + kLmTile - 1) / kLmTile, ntb = (rows + kLmTile - 1) / kLmTile;
+        if ((size_t)neb * ntb >= 256) {
+            dim3 grid((unsigned)(neb * ((ntb + 7) / 8) * 8));
+            INFR_LDS_LIMIT(router_logits_mfma_kernel, (int)kLmLdsBytes);
+            INFR_LAUNCH(router_logits_mfma_kernel, grid, dim3(512), kLmLdsBytes, s, reinterpret_cast<const float*>(router),
                         row_bytes / 4, x, ne, n_expert, rows, logits);
         } else {
             dim3 grid((n_expert + 15) / 16, (rows + 15) / 16);

@@ -150,7 +150,8 @@ def test_one_hot_gemv_reads_back_the_decoded_weight(be, dt, in_f):
                                              (33, 256, 64, 6, H.F32), (3, 100, 10, 3, H.F32),
                                              (1, 4096, 256, 8, H.F32), (5, 512, 16, 4, H.Q8_0),
                                              (2, 256, 8, 2, H.F16), (70, 2048, 100, 8, H.F32),
-                                             (16, 160, 40, 4, H.F32), (1030, 512, 256, 8, H.F32), (500, 288, 128, 4, H.F32)])
+                                             (16, 160, 40, 4, H.F32), (1030, 512, 256, 8, H.F32), (500, 288, 128, 4, H.F32),
+                                             (2050, 288, 100, 4, H.F32), (1024, 640, 256, 8, H.F32)])
 def test_router_logits_probs_ids_weights_bit_exact(be, rows, ne, E, K, rdt):
     rng = np.random.default_rng(rows * 7 + ne)
     x = rng.standard_normal((rows, ne)).astype(np.float32)
