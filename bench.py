@@ -14,7 +14,7 @@ kernel chain of this shape cannot go below), and a CPU baseline (the oracle, a s
 reference's CPU path, timed on this host's cores on a bounded sample).  With no --config every other benchmark
 configuration (single Q8_0 layer, multi-stream decode, prefill chunks, the large shape with a shared expert) is
 measured the same way and printed as a compact JSON line of its own BEFORE the headline; the per-kernel tables and
-floors of every workload go to the file named by --detail (default gpurun_out/bench_configs.json).
+floors of every workload go to the file named by --detail (see its default below).
 """
 from __future__ import annotations
 

@@ -169,6 +169,23 @@ def test_router_logits_probs_ids_weights_bit_exact(be, rows, ne, E, K, rdt):
     assert not out.any()
 
 
+@pytest.mark.parametrize("rows", [1, 64, 2048])
+def test_router_logits_keep_subnormal_terms(be, rows):
+    """Products and sums around 1e-39 are subnormal f32 numbers: the logits kernels of every batch size (per-row chains,
+    tiled vector kernel, matrix-core kernel) must keep them as the CPU's fused multiply-add does."""
+    ne, E, K, nff = 256, 128, 8, 32
+    rng = np.random.default_rng(5)
+    x = (rng.standard_normal((rows, ne)) * 1e-22).astype(np.float32)
+    rf = (rng.standard_normal((E, ne)) * 1e-18).astype(np.float32)
+    z = np.zeros(E * nff * ne, np.float32)
+    g, ids = moe_graph(rows, ne, E, K, nff, DType.F32, DType.F32)
+    _, r = run_moe(be, g, ids, dict(x=x, router=rf, gate=z, up=z, down=z), rows, ne)
+    ref = O.moe_ffn(x, rf, z, z, z, ne=ne, n_expert=E, n_used=K, n_ff_exp=nff)
+    assert np.abs(ref["logits"]).max() < 1.1754944e-38 and ref["logits"].any()
+    assert np.array_equal(bits(r["logits"]), bits(ref["logits"]))
+    assert np.array_equal(r["idx"], ref["idx"])
+
+
 def test_routing_variants_bit_exact_ids(be):
     ne, E, K, nff, rows = 64, 16, 4, 32, 6
     rng = np.random.default_rng(11)
