@@ -232,7 +232,7 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
     __shared__ float s_ysh[64];
     __shared__ float s_red[4];
     __shared__ uint32_t s_guess[2 * kWave];
-    __shared__ int s_f_spec, s_f_route, s_f_hs, s_fault, s_cells_done, s_h_done, s_done, s_xn_done;
+    __shared__ int s_f_spec, s_f_route, s_fault, s_cells_done, s_h_done, s_xn_done;
     __shared__ uint32_t s_seq;
     const MoeGemvParams& p = q.g;
     const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;   // wave: uniform, scalar registers
@@ -292,7 +292,7 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
 
     if (tid < 32) s_tab[tid] = kExp2Table[tid];
     if (tid == 0) {
-        s_f_spec = s_f_route = s_f_hs = s_fault = s_cells_done = s_h_done = s_done = s_xn_done = 0;
+        s_f_spec = s_f_route = s_fault = s_cells_done = s_h_done = s_xn_done = 0;
         // the launch's number: every workgroup keeps its own count of the launches it has run (a counter shared by all
         // would serialise 256 atomics, at the start or, worse, at the end of the kernel), read here and written back
         // with a plain store at the end; launches on a workspace never overlap, so all 256 counts agree
@@ -532,15 +532,11 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
         const int sfpb = nff / bpr, sf0 = os * sfpb;
         const int n_si = shared ? (sfpb + pg.rw_count - 1) / pg.rw_count : 0;
         const int sh_n = n_si > sw ? (n_si - sw + kSW - 1) / kSW : 0;
-        // down items: item j covers output rows (j * kSW + sw) * rw_count + rw of the workgroup's slice; behind them the
-        // always-on expert's rows [b * ne / 256, ..), dealt to the wavefronts starting with those that got fewer above
+        // down items: item j covers output rows (j * kSW + sw) * rw_count + rw of the workgroup's slice (the always-on
+        // expert's down rows are the router's wavefront's: it has nothing else to do while the activations change hands)
         const int R = ne / mpg;
         const int n_di = (R + pd.rw_count - 1) / pd.rw_count;
         const int my_di = n_di > sw ? (n_di - sw + kSW - 1) / kSW : 0;
-        const int SR = ne / bpr;
-        const int n_sdi = shared ? (SR + pd.rw_count - 1) / pd.rw_count : 0;
-        const int ssw = (sw + kSW - n_di % kSW) % kSW;
-        const int my_sdi = n_sdi > ssw ? (n_sdi - ssw + kSW - 1) / kSW : 0;
 
         GuItem gring[DG];
         auto sh_load = [&](GuItem& it, int j) __attribute__((always_inline)) {   // item j of this wavefront's share
@@ -577,13 +573,9 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
         typename FD::Raw dring[DD];
         int e_cur = alive ? __builtin_amdgcn_readfirstlane(s_spec[g]) : 0;
         const uint8_t* dbank = nullptr;
-        auto dn_issue = [&](int slot, int j) __attribute__((always_inline)) {
-            const bool routed = j < my_di || !shared;   // items past the end re-read a last row
-            const int jj = routed ? j : j - my_di;
-            const int lim = routed ? R : SR;
-            const int orow = min((jj * kSW + (routed ? sw : ssw)) * pd.rw_count + pd.rw, lim - 1);
-            const uint8_t* base = routed ? dbank + (size_t)(m * R + orow) * rb_d : p.sh_down + (size_t)(os * SR + orow) * rb_d;
-            dring[slot] = load_row<FD>(pd, base);
+        auto dn_issue = [&](int slot, int j) __attribute__((always_inline)) {   // items past the end re-read the last row
+            const int orow = min((j * kSW + sw) * pd.rw_count + pd.rw, R - 1);
+            dring[slot] = load_row<FD>(pd, dbank + (size_t)(m * R + orow) * rb_d);
         };
         // One pass per expert this group works on: the guessed one, and once more if the exact routing names another.
         // A pass does not wait for the routing: the group's activations carry the expert they were computed for, so
@@ -645,8 +637,7 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
             if (wave == 3) STAMP(7);
             if (wave == 1) STAMP(21);
             if (wave == 7) STAMP(22);
-            // ---- hand-over of the group's activations: six wavefronts gather a sixth each and turn it into cells; the
-            // seventh gathers the always-on expert's meanwhile (written long ago by all 256 workgroups)
+            // ---- hand-over of the group's activations: six wavefronts gather a sixth each and turn it into cells
             bool superseded = false;
             if (sw < 6) {
                 const int st = gather_activations<4>(q.xh + (size_t)g * nff + sw * chunk, chunk, seq_tag | (uint32_t)e_cur,
@@ -668,20 +659,6 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
                 if (lane == 0)
                     __hip_atomic_fetch_add(&s_h_done, st == kGatherTimeout ? 0x101 : 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
                 if (wave == 1) STAMP(10);
-            } else if (shared && attempt == 0) {
-                bool ok = gather_records<24>(q.xs, nff, tag, s_hs, lane, spin_limit);
-                if (ok) {
-                    __builtin_amdgcn_wave_barrier();
-                    for (int oct = lane; oct * 8 < nff; oct += kWave) {
-                        const float4 lo = *reinterpret_cast<const float4*>(s_hs + 8 * oct), hi = *reinterpret_cast<const float4*>(s_hs + 8 * oct + 4);
-                        octet_to_cell<FD::kGroup, FD::kSigned>(lo, hi, oct, hscells);
-                    }
-                } else if (lane == 0) {
-                    s_fault = 1;
-                    __hip_atomic_store(q.fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
-                }
-                lds_flag_set(&s_f_hs, ok ? 1 : 2);
-                alive = ok;
             }
             // the first down rows, requested behind the polls: a poll issued behind them would not return before them
             if (!q.early_down && alive) ring_prime<DD>(dn_issue);
@@ -698,33 +675,19 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
             asm volatile("" ::: "memory");
             const bool in_vain = superseded || routed == 2 || (routed == 1 && __builtin_amdgcn_readfirstlane(s_final[g]) != e_cur);
             if (alive && !in_vain) {
-                // ---- down: rows of the group's expert, then of the always-on expert
+                // ---- down: rows of the group's expert
                 typename FD::X xd;
                 FD::fetch_x(xd, hcells, pd.blk, pd.sub);
                 const bool scaled = p.down_scale != nullptr;
                 const float ds = scaled ? p.down_scale[e_cur] : 1.0f;
                 uint64_t* part = q.ypart + (size_t)g * ne + (size_t)m * R;
                 const uint32_t ytag = seq_tag | (uint32_t)e_cur;
-                bool on_shared = false;
                 auto dn_finish = [&](int slot, int j) __attribute__((always_inline)) {
-                    const bool own = j < my_di;
-                    if (!own && !on_shared) {   // the same for the whole wavefront
-                        on_shared = true;
-                        if (sw != 6 && lds_flag_wait(&s_f_hs) != 1) alive = false;
-                        FD::fetch_x(xd, hscells, pd.blk, pd.sub);
-                    }
-                    const int jj = own ? j : j - my_di;
-                    const int orow = (jj * kSW + (own ? sw : ssw)) * pd.rw_count + pd.rw;
+                    const int orow = (j * kSW + sw) * pd.rw_count + pd.rw;
                     const float y = row_sum<FD>(FD::dot(dring[slot], pd.sub, xd), pd, nblk_d);
-                    if (pd.writer()) {
-                        if (own) {
-                            if (orow < R) rec_store(part + orow, scaled ? __fmul_rn(y, ds) : y, ytag);
-                        } else if (orow < SR) {
-                            s_ysh[orow] = y;
-                        }
-                    }
+                    if (pd.writer() && orow < R) rec_store(part + orow, scaled ? __fmul_rn(y, ds) : y, ytag);
                 };
-                ring_drain<DD>(my_di + my_sdi, dn_issue, dn_finish);
+                ring_drain<DD>(my_di, dn_issue, dn_finish);
                 if (wave == 3) STAMP(11);
             }
             if (!alive) return false;
@@ -740,9 +703,6 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
             return true;
         };
         if (alive && run_pass(0)) run_pass(1);
-        // this wavefront's rows of the always-on expert are in LDS: tell the summing wavefront
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        if (lane == 0) __hip_atomic_fetch_add(&s_done, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     }
     if (wave == 0) {
         // ---- the rank-ordered sum, by the router's wavefront: workgroup (g, m) owns rows [m R + g R / 8, + R / 8) of
@@ -750,6 +710,45 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
         // w_rank * y_rank as a separate multiply and add (crates/infr-cpu/src/lib.rs:4290-4302), then the always-on
         // expert, then the residual operand.  The partial results are polled while the streaming wavefronts still work.
         const int R = ne / mpg, SR = R / kGroups;
+        if (shared) {
+            // ---- the always-on expert's down rows of this workgroup, [os * SR, + SR), while the streaming wavefronts wait
+            // for their group's activations: nothing else is in flight then.  Its activations were written long ago by all
+            // the workgroups of the row.
+            bool got = gather_records<24>(q.xs, nff, tag, s_hs, lane, spin_limit);
+            if (got) {
+                __builtin_amdgcn_wave_barrier();
+                for (int oct = lane; oct * 8 < nff; oct += kWave) {
+                    const float4 lo = *reinterpret_cast<const float4*>(s_hs + 8 * oct), hi = *reinterpret_cast<const float4*>(s_hs + 8 * oct + 4);
+                    octet_to_cell<FD::kGroup, FD::kSigned>(lo, hi, oct, hscells);
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                __builtin_amdgcn_wave_barrier();
+                const int nblk_d = nff / FD::kBlockElems;
+                const size_t rb_d = (size_t)nblk_d * FD::kBlockBytes;
+                const Place<FD> pd(nblk_d, lane);
+                typename FD::X xd;
+                FD::fetch_x(xd, hscells, pd.blk, pd.sub);
+                const uint8_t* rows0 = p.sh_down + (size_t)os * SR * rb_d;
+                const int n_sdi = (SR + pd.rw_count - 1) / pd.rw_count;
+                typename FD::Raw ring[4];
+                for (int j0 = 0; j0 < n_sdi; j0 += 4) {
+#pragma unroll
+                    for (int d = 0; d < 4; d++)
+                        ring[d] = load_row<FD>(pd, rows0 + (size_t)min((j0 + d) * pd.rw_count + pd.rw, SR - 1) * rb_d);
+#pragma unroll
+                    for (int d = 0; d < 4; d++) {
+                        const int orow = (j0 + d) * pd.rw_count + pd.rw;
+                        const float y = row_sum<FD>(FD::dot(ring[d], pd.sub, xd), pd, nblk_d);
+                        if (pd.writer() && orow < SR) s_ysh[orow] = y;
+                    }
+                }
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+                __builtin_amdgcn_wave_barrier();
+            } else if (lane == 0) {
+                s_fault = 1;
+                __hip_atomic_store(q.fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            }
+        }
         const bool mine = lane < SR;
         const size_t oi = (size_t)m * R + (size_t)g * SR + (mine ? lane : 0);
         uint64_t yk[kGroups];
@@ -773,8 +772,6 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
             }
         }
         STAMP(12);
-        while (__builtin_amdgcn_readfirstlane(*(volatile int*)&s_done) < kSW) __builtin_amdgcn_s_sleep(1);
-        asm volatile("" ::: "memory");
         if (ok && mine && !*(volatile int*)&s_fault) {
             float acc = 0.0f;
 #pragma unroll
