@@ -61,7 +61,7 @@ bool stream_shape(const MoeLayerParams& q, StreamShape* out) {
     if (nff % mpg || ne % bpr) return false;
     const int fpb = nff / mpg, R = ne / mpg;
     const int n_gi = (fpb + rwc_g - 1) / rwc_g, n_di = (R + rwc_d - 1) / rwc_d;
-    const int my_gi = (n_gi + kSW - 1) / kSW, my_di = (n_di + kSW - 1) / kSW;
+    const int my_gi = (n_gi + kSW - 1) / kSW, my_di = (n_di - router_wave_down_items(n_di) + kSW - 1) / kSW;
     if (my_gi * rwc_g > 64) return false;                            // a wavefront's results wait in one 64-float row
     if (shared) {
         if (nff % bpr) return false;

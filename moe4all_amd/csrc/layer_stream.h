@@ -213,6 +213,11 @@ __device__ __forceinline__ float dot8(const float4& a0, const float4& a1, const 
 
 }  // namespace
 
+// Down items (groups of output rows a wavefront covers at once) of a workgroup that the router's wavefront takes, the
+// last ones of the n_di: an eighth when that leaves the seven streaming wavefronts equal shares.  It knows the exact
+// routing first and has nothing to do while the others stream.
+__host__ __device__ constexpr int router_wave_down_items(int n_di) { return n_di % 8 == 0 ? n_di / 8 : 0; }
+
 // FG / FD: formats of the gate/up and down banks; DG / DD: ring depths (items in flight per streaming wavefront);
 // EPT: router rows a thread holds while staging (rows per workgroup / (512 / (ne / 8))); NSP: n_expert / 64.
 // NE, NFF, ROWS: hidden size, intermediate size and token rows when they are known at compile time (the benchmark
@@ -536,7 +541,8 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
         // expert's down rows are the router's wavefront's: it has nothing else to do while the activations change hands)
         const int R = ne / mpg;
         const int n_di = (R + pd.rw_count - 1) / pd.rw_count;
-        const int my_di = n_di > sw ? (n_di - sw + kSW - 1) / kSW : 0;
+        const int n_ds = n_di - router_wave_down_items(n_di);   // the streaming wavefronts' items: the first n_ds
+        const int my_di = n_ds > sw ? (n_ds - sw + kSW - 1) / kSW : 0;
 
         GuItem gring[DG];
         auto sh_load = [&](GuItem& it, int j) __attribute__((always_inline)) {   // item j of this wavefront's share
@@ -710,6 +716,11 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
         // w_rank * y_rank as a separate multiply and add (crates/infr-cpu/src/lib.rs:4290-4302), then the always-on
         // expert, then the residual operand.  The partial results are polled while the streaming wavefronts still work.
         const int R = ne / mpg, SR = R / kGroups;
+        const int nblk_d = nff / FD::kBlockElems;
+        const size_t rb_d = (size_t)nblk_d * FD::kBlockBytes;
+        const Place<FD> pd(nblk_d, lane);
+        typename FD::X xd;
+        typename FD::Raw ring[DD];
         if (shared) {
             // ---- the always-on expert's down rows of this workgroup, [os * SR, + SR), while the streaming wavefronts wait
             // for their group's activations: nothing else is in flight then.  Its activations were written long ago by all
@@ -723,30 +734,57 @@ __global__ __launch_bounds__(kThreads) void moe_layer_stream(MoeLayerParams q) {
                 }
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
                 __builtin_amdgcn_wave_barrier();
-                const int nblk_d = nff / FD::kBlockElems;
-                const size_t rb_d = (size_t)nblk_d * FD::kBlockBytes;
-                const Place<FD> pd(nblk_d, lane);
-                typename FD::X xd;
                 FD::fetch_x(xd, hscells, pd.blk, pd.sub);
                 const uint8_t* rows0 = p.sh_down + (size_t)os * SR * rb_d;
                 const int n_sdi = (SR + pd.rw_count - 1) / pd.rw_count;
-                typename FD::Raw ring[4];
-                for (int j0 = 0; j0 < n_sdi; j0 += 4) {
-#pragma unroll
-                    for (int d = 0; d < 4; d++)
-                        ring[d] = load_row<FD>(pd, rows0 + (size_t)min((j0 + d) * pd.rw_count + pd.rw, SR - 1) * rb_d);
-#pragma unroll
-                    for (int d = 0; d < 4; d++) {
-                        const int orow = (j0 + d) * pd.rw_count + pd.rw;
-                        const float y = row_sum<FD>(FD::dot(ring[d], pd.sub, xd), pd, nblk_d);
-                        if (pd.writer() && orow < SR) s_ysh[orow] = y;
-                    }
-                }
+                auto sd_issue = [&](int slot, int j) __attribute__((always_inline)) {
+                    ring[slot] = load_row<FD>(pd, rows0 + (size_t)min(j * pd.rw_count + pd.rw, SR - 1) * rb_d);
+                };
+                auto sd_finish = [&](int slot, int j) __attribute__((always_inline)) {
+                    const int orow = j * pd.rw_count + pd.rw;
+                    const float y = row_sum<FD>(FD::dot(ring[slot], pd.sub, xd), pd, nblk_d);
+                    if (pd.writer() && orow < SR) s_ysh[orow] = y;
+                };
+                ring_prime<DD>(sd_issue);
+                ring_drain<DD>(n_sdi, sd_issue, sd_finish);
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
                 __builtin_amdgcn_wave_barrier();
             } else if (lane == 0) {
                 s_fault = 1;
                 __hip_atomic_store(q.fault, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            }
+        }
+        const int n_di = (R + pd.rw_count - 1) / pd.rw_count, n_w0 = router_wave_down_items(n_di);
+        if (n_w0 > 0 && *(volatile int*)&s_f_route == 1) {
+            // ---- this wavefront's share of the down rows of the group's expert: the one the exact routing names, so
+            // its rows are requested at once and contracted when the pass that gathers that expert's activations is
+            // through (the first if the guess was right, the second otherwise)
+            const int e_fin = __builtin_amdgcn_readfirstlane(s_final[g]);
+            const int through = 6 * (__builtin_amdgcn_readfirstlane(s_spec[g]) == e_fin ? 1 : 2);
+            const uint8_t* rows0 = p.down + (size_t)e_fin * p.down_stride + (size_t)m * R * rb_d;
+            const int i0 = n_di - n_w0;
+            auto wd_issue = [&](int slot, int j) __attribute__((always_inline)) {
+                ring[slot] = load_row<FD>(pd, rows0 + (size_t)min((i0 + j) * pd.rw_count + pd.rw, R - 1) * rb_d);
+            };
+            ring_prime<DD>(wd_issue);
+            int v;
+            bool lost = false;   // a streaming wavefront that gave up has raised the fault: the count will not come
+            while ((((v = __builtin_amdgcn_readfirstlane(*(volatile int*)&s_h_done)) & 0xFF) < through) && !(v >> 8) &&
+                   !(lost = __builtin_amdgcn_readfirstlane(*(volatile int*)&s_fault) != 0))
+                __builtin_amdgcn_s_sleep(1);
+            asm volatile("" ::: "memory");
+            if (!(v >> 8) && !lost) {
+                FD::fetch_x(xd, hcells, pd.blk, pd.sub);
+                const bool scaled = p.down_scale != nullptr;
+                const float ds = scaled ? p.down_scale[e_fin] : 1.0f;
+                uint64_t* part = q.ypart + (size_t)g * ne + (size_t)m * R;
+                const uint32_t ytag = seq_tag | (uint32_t)e_fin;
+                auto wd_finish = [&](int slot, int j) __attribute__((always_inline)) {
+                    const int orow = (i0 + j) * pd.rw_count + pd.rw;
+                    const float y = row_sum<FD>(FD::dot(ring[slot], pd.sub, xd), pd, nblk_d);
+                    if (pd.writer() && orow < R) rec_store(part + orow, scaled ? __fmul_rn(y, ds) : y, ytag);
+                };
+                ring_drain<DD>(n_w0, wd_issue, wd_finish);
             }
         }
         const bool mine = lane < SR;
