@@ -329,9 +329,8 @@ __global__ __launch_bounds__((kLtTile / P) * (kLtTile / P) * 8) void router_logi
 // independent, which keeps the pipe busy from one wavefront.
 // Workgroup = 32 tokens x 32 experts = 8 wavefronts, two per SIMD: wavefronts 0-3 contract (each a 16 x 16 tile),
 // wavefronts 4-7 only move data, so that no load, LDS store or address arithmetic sits between two matrix
-// instructions of a contracting wavefront (one wavefront doing both ran at half the rate).  Operands are staged per
-// 128-k chunk transposed in LDS as [chain][row][step] (row stride 20 floats, chain stride = 8 mod 16: the 128-bit
-// reads and the 32-bit stores are free of bank conflicts), double-buffered, one barrier per chunk.  A contracting
+// instructions of a contracting wavefront.  Operands are staged per 128-k chunk transposed in LDS (layout below: reads
+// and stores free of bank conflicts), double-buffered, one barrier per chunk.  A contracting
 // wavefront passes the barrier in the MIDDLE of a chunk's matrix instructions and reads the next chunk's first half
 // behind it, beside the second half of its instructions, so neither the barrier nor the LDS latency empties the pipe.
 // The moving wavefronts load four chunks ahead in registers.
@@ -339,10 +338,13 @@ __global__ __launch_bounds__((kLtTile / P) * (kLtTile / P) * 8) void router_logi
 // 4 b + i, the element (token 4 (l / 16) + i, expert l % 16) of chain b, so the sum over the chains is lane-local.
 // Workgroups that share a token tile (one per 32 experts) are given indices 8 apart: they run on one XCD and the
 // tile's activations come through one L2.
-constexpr int kLmChunk = 128, kLmRow = kLmChunk / 8 + 4, kLmTile = 32;
-constexpr int kLmChain = kLmTile * kLmRow + 8;                         // floats of one chain
-constexpr int kLmOperand = 8 * kLmChain;                               // floats of one operand's chunk
-constexpr size_t kLmLdsBytes = (size_t)4 * kLmOperand * sizeof(float);   // two operands, two buffers
+constexpr int kLmChunk = 128, kLmTile = 32;
+// LDS layout of a chunk: 1 KB blocks [operand][16-row tile][accumulator set][four steps], inside a block
+// [chain of the set][row][step]: a contracting wavefront's 128-bit read of a block and a moving wavefront's 32-bit store
+// into it are both 64 consecutive lanes on consecutive addresses.
+constexpr int kLmBlock = 256;                                          // floats of a block
+constexpr int kLmBuffer = 2 * 2 * 2 * 4 * kLmBlock;                    // floats of one chunk of both operands
+constexpr size_t kLmLdsBytes = (size_t)2 * kLmBuffer * sizeof(float);   // two buffers
 typedef float lm_acc_t __attribute__((ext_vector_type(16)));
 struct LmHalf { float4 w[2][2], x[2][2]; };   // operands of half a chunk: [four steps][accumulator set]
 __global__ __launch_bounds__(512) void router_logits_mfma_kernel(const float* __restrict__ router, size_t row_floats,
@@ -355,32 +357,29 @@ __global__ __launch_bounds__(512) void router_logits_mfma_kernel(const float* __
     if (r0 >= rows) return;
     const int nfast = (ne / kLmChunk) & ~3;   // whole chunks that run through the pipelines below, four per trip
     if (wave >= 4) {
-        // ---- the moving wavefronts: four 128-bit loads of each operand per thread and chunk; load q covers row
-        // srow + 8 (q & 3), floats 4 v .. 4 v + 3 of the chunk.  Rows past the end repeat the last one (their results
-        // are never stored), and so do loads past the end of a row (those steps are never contracted).
-        const int srow = (wave - 4) + 4 * ((tid >> 5) & 1), v = tid & 31;
-        const float* src[8];
-#pragma unroll
-        for (int q = 0; q < 8; q++) {
-            const bool is_x = q >= 4;
-            const int g = min((is_x ? r0 : e0) + srow + 8 * (q & 3), (is_x ? rows : n_expert) - 1);
-            src[q] = is_x ? x + (size_t)g * ne : router + (size_t)g * row_floats;
-        }
-        // element 4 v + t of the chunk: chain 4 (v & 1) + t, step v >> 1
-        const int dst0 = 4 * (v & 1) * kLmChain + srow * kLmRow + (v >> 1);
+        // ---- the moving wavefronts: wavefronts 4, 5 move the router's two 16-row tiles, 6, 7 the activations'.  Lane
+        // (row, step) = (lane / 4, lane % 4) of a wavefront loads, for q = 4 s + c, the four chains of accumulator set s
+        // at step 4 c + step of its row: chunk elements 32 c + 8 step + 4 s .. + 3, a 128-bit load; component t of it
+        // goes to block (tile, s, c), place 64 t + lane.  Rows past the end repeat the last one (their results are never
+        // stored), and so do loads past the end of a row (those steps are never contracted).
+        const int pw = wave - 4, is_x = pw >> 1, tile = pw & 1;
+        const int grow = min((is_x ? r0 : e0) + 16 * tile + (lane >> 2), (is_x ? rows : n_expert) - 1);
+        const float* src = is_x ? x + (size_t)grow * ne : router + (size_t)grow * row_floats;
+        const int koff = 8 * (lane & 3);
+        const int dst0 = (is_x * 2 + tile) * 8 * kLmBlock + lane;
         auto fetch = [&](float4 (&st)[8], int k0) __attribute__((always_inline)) {
-            const int k = min(k0 + 4 * v, ne - 4);
 #pragma unroll
-            for (int q = 0; q < 8; q++) st[q] = *reinterpret_cast<const float4*>(src[q] + k);
+            for (int q = 0; q < 8; q++)
+                st[q] = *reinterpret_cast<const float4*>(src + min(k0 + 32 * (q & 3) + koff + 4 * (q >> 2), ne - 4));
         };
         auto deposit = [&](const float4 (&st)[8], int buf) __attribute__((always_inline)) {
 #pragma unroll
             for (int q = 0; q < 8; q++) {
-                float* d = lm_lds + (2 * buf + (q >= 4 ? 1 : 0)) * kLmOperand + dst0 + 8 * (q & 3) * kLmRow;
+                float* d = lm_lds + buf * kLmBuffer + dst0 + q * kLmBlock;   // block (tile, s, c): q = 4 s + c
                 d[0] = st[q].x;
-                d[kLmChain] = st[q].y;
-                d[2 * kLmChain] = st[q].z;
-                d[3 * kLmChain] = st[q].w;
+                d[64] = st[q].y;
+                d[128] = st[q].z;
+                d[192] = st[q].w;
             }
         };
         if (nfast > 0) {
@@ -420,16 +419,16 @@ __global__ __launch_bounds__(512) void router_logits_mfma_kernel(const float* __
     // ---- the contracting wavefronts
     const int tw = wave & 1, ew = wave >> 1;   // the wavefront's 16 x 16 tile of the workgroup's 32 x 32
     // the lane's operands of accumulator set s: chain 4 s + lane / 16, row lane % 16 of the wavefront's tile
-    const int wo = (lane >> 4) * kLmChain + (16 * ew + (lane & 15)) * kLmRow;
-    const int xo = (lane >> 4) * kLmChain + (16 * tw + (lane & 15)) * kLmRow + kLmOperand;
+    const int wo = (0 * 2 + ew) * 8 * kLmBlock + 4 * lane;
+    const int xo = (1 * 2 + tw) * 8 * kLmBlock + 4 * lane;
     auto read_half = [&](LmHalf& o, int buf, int half) __attribute__((always_inline)) {
-        const float* base = lm_lds + 2 * buf * kLmOperand + 8 * half;
+        const float* base = lm_lds + buf * kLmBuffer + 2 * half * kLmBlock;
 #pragma unroll
         for (int c = 0; c < 2; c++)
 #pragma unroll
             for (int s = 0; s < 2; s++) {
-                o.w[c][s] = *reinterpret_cast<const float4*>(base + wo + 4 * s * kLmChain + 4 * c);
-                o.x[c][s] = *reinterpret_cast<const float4*>(base + xo + 4 * s * kLmChain + 4 * c);
+                o.w[c][s] = *reinterpret_cast<const float4*>(base + wo + (4 * s + c) * kLmBlock);
+                o.x[c][s] = *reinterpret_cast<const float4*>(base + xo + (4 * s + c) * kLmBlock);
             }
     };
     lm_acc_t acc[2];
