@@ -372,6 +372,12 @@ __global__ __launch_bounds__(512) void router_logits_mfma_kernel(const float* __
             for (int q = 0; q < 8; q++)
                 st[q] = *reinterpret_cast<const float4*>(src + min(k0 + 32 * (q & 3) + koff + 4 * (q >> 2), ne - 4));
         };
+        // whole chunks need no clamp: one address per lane and chunk, the eight loads at constant offsets from it
+        auto fetch_whole = [&](float4 (&st)[8], int k0) __attribute__((always_inline)) {
+            const float* at = src + koff + k0;
+#pragma unroll
+            for (int q = 0; q < 8; q++) st[q] = *reinterpret_cast<const float4*>(at + 32 * (q & 3) + 4 * (q >> 2));
+        };
         auto deposit = [&](const float4 (&st)[8], int buf) __attribute__((always_inline)) {
 #pragma unroll
             for (int q = 0; q < 8; q++) {
@@ -387,17 +393,18 @@ __global__ __launch_bounds__(512) void router_logits_mfma_kernel(const float* __
             // (one basic block per trip, its order pinned: the compiler otherwise sinks the loads to their deposits)
             float4 s0[8], s1[8], s2[8], s3[8];
             auto step = [&](int c, float4 (&s_free)[8], const float4 (&s_next)[8], int buf) __attribute__((always_inline)) {
-                fetch(s_free, min(c + 4, nfast - 1) * kLmChunk);
+                fetch_whole(s_free, min(c + 4, nfast - 1) * kLmChunk);
                 __builtin_amdgcn_sched_barrier(0);
                 deposit(s_next, buf ^ 1);   // past the last chunk: a repeat of it that nobody contracts
                 __builtin_amdgcn_sched_barrier(0);
                 __syncthreads();
                 __builtin_amdgcn_sched_barrier(0);
             };
-            fetch(s0, 0);
-            fetch(s1, kLmChunk);
-            fetch(s2, 2 * kLmChunk);
-            fetch(s3, 3 * kLmChunk);
+            __builtin_amdgcn_s_setprio(3);   // requests ahead of the contracting wavefronts' instructions: 17.4 -> 16.9 us
+            fetch_whole(s0, 0);
+            fetch_whole(s1, kLmChunk);
+            fetch_whole(s2, 2 * kLmChunk);
+            fetch_whole(s3, 3 * kLmChunk);
             deposit(s0, 0);
             __syncthreads();
             for (int c = 0; c < nfast; c += 4) {
