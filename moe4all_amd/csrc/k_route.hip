@@ -221,152 +221,62 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const uint8_t* __res
 }
 
 // ---------------------------------------------------------------------------------------------
-// Logits for a batch on the vector ALUs (f32 router, ne a multiple of 32; batches too small to give the matrix-core
-// kernel below a workgroup per compute unit).  Block = 512 threads covering kLtTile experts x kLtTile token rows: 8
-// chains x G row groups x G expert groups.  A thread keeps a P x P (expert, row) patch of accumulators for its chain,
-// so each 128-bit LDS read feeds 4 P FMAs.  The patch's rows are G apart (rows b * G + rg): the sixteen lanes the LDS serves together then read
-// sixteen consecutive 80-byte rows, which fall on distinct banks (rows 32 apart are 2560 bytes = a whole number of
-// bank rounds apart and collided).  k advances in chunks of 128 elements staged transposed (chain-major) in LDS;
-// the accumulators run through all chunks, so every chain still adds its terms in ascending
-// order, exactly as the scalar reference does.
-constexpr int kLtChunk = 128, kLtStride = kLtChunk / 8 + 4;
-// kLtTile experts x kLtTile rows per block, a P x P patch per thread.  Instantiated as 16 / 2 (512 threads): a block's
-// time is its chunks' latency chain, which a small patch keeps short (32 / 4 was the kernel for large batches before
-// the matrix-core kernel: 28 us against 18 us for 2048 rows x 128 experts x 2048).
-template <int kLtTile, int P>
-__global__ __launch_bounds__((kLtTile / P) * (kLtTile / P) * 8) void router_logits_tiled_kernel(const float* __restrict__ router,
-                                                                                      size_t row_floats,
-                                                                                      const float* __restrict__ x, int ne,
-                                                                                      int n_expert, int rows,
-                                                                                      float* __restrict__ logits) {
-    constexpr int G = kLtTile / P;               // P-row (P-expert) groups per tile side
-    constexpr int NT = G * G * 8;                // threads: a P x P patch of (expert, row) pairs for each of 8 chains
-    constexpr int NQ = kLtTile * 32 / NT;        // float4 per thread, operand and chunk
-    __shared__ float sw[kLtTile * 8 * kLtStride];
-    __shared__ float sx[kLtTile * 8 * kLtStride];
-    const int tid = threadIdx.x, j = tid & 7, rg = (tid >> 3) % G, eg = tid / (8 * G);
-    const int e0 = blockIdx.x * kLtTile, r0 = blockIdx.y * kLtTile;
-    float acc[P][P];
-#pragma unroll
-    for (int a = 0; a < P; a++)
-#pragma unroll
-        for (int b = 0; b < P; b++) acc[a][b] = 0.0f;
-    // staging role: NQ float4 of the router tile and NQ of the activation tile per chunk
-    const float* src[2 * NQ];
-    bool ok[2 * NQ];
-    int dst_base[2 * NQ];
-#pragma unroll
-    for (int q = 0; q < 2 * NQ; q++) {
-        const int idx = tid + NT * (q % NQ), row = idx >> 5, v = idx & 31;
-        const bool is_x = q >= NQ;
-        const int g = (is_x ? r0 : e0) + row;
-        ok[q] = g < (is_x ? rows : n_expert);
-        src[q] = (is_x ? x + (size_t)(ok[q] ? g : 0) * ne : router + (size_t)(ok[q] ? g : 0) * row_floats) + 4 * v;
-        // element 4v+t of the chunk: chain (4v+t)&7 = 4(v&1)+t, step (4v+t)>>3 = v>>1
-        dst_base[q] = (row * 8 + 4 * (v & 1)) * kLtStride + (v >> 1);
-    }
-    float4 st[2 * NQ];
-    auto fetch = [&](int k0) {
-#pragma unroll
-        for (int q = 0; q < 2 * NQ; q++) {
-            const int v4 = 4 * ((tid + NT * (q % NQ)) & 31);
-            st[q] = (ok[q] && k0 + v4 < ne) ? *reinterpret_cast<const float4*>(src[q] + k0) : make_float4(0.f, 0.f, 0.f, 0.f);
-        }
-    };
-    fetch(0);
-    for (int k0 = 0; k0 < ne; k0 += kLtChunk) {
-        __syncthreads();
-#pragma unroll
-        for (int q = 0; q < 2 * NQ; q++) {
-            float* d = (q >= NQ ? sx : sw) + dst_base[q];
-            d[0] = st[q].x;
-            d[kLtStride] = st[q].y;
-            d[2 * kLtStride] = st[q].z;
-            d[3 * kLtStride] = st[q].w;
-        }
-        __syncthreads();
-        if (k0 + kLtChunk < ne) fetch(k0 + kLtChunk);
-        const int n_c = min(kLtChunk, ne - k0) >> 3;  // a multiple of 4
-        const float* wp = sw + (eg * P * 8 + j) * kLtStride;
-        const float* xp = sx + (rg * 8 + j) * kLtStride;   // the thread's rows: b * G + rg
-        for (int c = 0; c < n_c; c += 4) {
-            float4 wv[P], xv[P];
-#pragma unroll
-            for (int a = 0; a < P; a++) {
-                wv[a] = *reinterpret_cast<const float4*>(wp + a * 8 * kLtStride + c);
-                xv[a] = *reinterpret_cast<const float4*>(xp + a * G * 8 * kLtStride + c);
-            }
-#pragma unroll
-            for (int a = 0; a < P; a++)
-#pragma unroll
-                for (int b = 0; b < P; b++) {
-                    acc[a][b] = __fmaf_rn(wv[a].x, xv[b].x, acc[a][b]);
-                    acc[a][b] = __fmaf_rn(wv[a].y, xv[b].y, acc[a][b]);
-                    acc[a][b] = __fmaf_rn(wv[a].z, xv[b].z, acc[a][b]);
-                    acc[a][b] = __fmaf_rn(wv[a].w, xv[b].w, acc[a][b]);
-                }
-        }
-    }
-    const int lane = tid & 63;
-#pragma unroll
-    for (int a = 0; a < P; a++)
-#pragma unroll
-        for (int b = 0; b < P; b++) {
-            float s = 0.0f;
-#pragma unroll
-            for (int jj = 0; jj < 8; jj++) s = __fadd_rn(s, __shfl(acc[a][b], (lane & ~7) + jj, kWave));
-            const int e = e0 + eg * P + a, r = r0 + b * G + rg;
-            if (j == 0 && e < n_expert && r < rows) logits[(size_t)r * n_expert + e] = s;
-        }
-}
-
-// ---------------------------------------------------------------------------------------------
 // Logits for a batch on the matrix cores.  v_mfma_f32_16x16x1_4b_f32 computes D_b[i][j] = A_b[i] * B_b[j] + C_b[i][j]
 // for four independent 16 x 16 blocks b: with one k per instruction every element is ONE fused multiply-add, so a
 // chain of them over k = 8 s + c, s ascending, is the reference's chain c term by term (the same bits as __fmaf_rn;
 // the parity tests compare them with the scalar restatement bit for bit).  A block b holds one chain, so two
 // instructions per step cover the eight chains of a 16 (token) x 16 (expert) tile, and the two accumulator sets are
 // independent, which keeps the pipe busy from one wavefront.
-// Workgroup = 32 tokens x 32 experts = 8 wavefronts, two per SIMD: wavefronts 0-3 contract (each a 16 x 16 tile),
-// wavefronts 4-7 only move data, so that no load, LDS store or address arithmetic sits between two matrix
-// instructions of a contracting wavefront.  Operands are staged per 128-k chunk transposed in LDS (layout below: reads
+// Workgroup (the 2 x 2 form) = 32 tokens x 32 experts = 8 wavefronts, two per SIMD: wavefronts 0-3 contract (each a
+// 16 x 16 tile), wavefronts 4-7 only move data, so that no load, LDS store or address arithmetic sits between two
+// matrix instructions of a contracting wavefront.  Operands are staged per 128-k chunk transposed in LDS (layout below: reads
 // and stores free of bank conflicts), double-buffered, one barrier per chunk.  A contracting
 // wavefront passes the barrier in the MIDDLE of a chunk's matrix instructions and reads the next chunk's first half
 // behind it, beside the second half of its instructions, so neither the barrier nor the LDS latency empties the pipe.
 // The moving wavefronts load four chunks ahead in registers.
 // Lane l supplies A = x[token l % 16][chain l / 16], B = w[expert l % 16][chain l / 16]; it receives, in register
 // 4 b + i, the element (token 4 (l / 16) + i, expert l % 16) of chain b, so the sum over the chains is lane-local.
-// Workgroups that share a token tile (one per 32 experts) are given indices 8 apart: they run on one XCD and the
+// Workgroups that share a token tile (one per expert tile) are given indices 8 apart: they run on one XCD and the
 // tile's activations come through one L2.
-constexpr int kLmChunk = 128, kLmTile = 32;
-// LDS layout of a chunk: 1 KB blocks [operand][16-row tile][accumulator set][four steps], inside a block
+// (The vector-ALU kernel this replaced, 16 x 16 tiles with a 2 x 2 patch of chain accumulators per thread, took 13-14 us
+// for 32 to 512 rows x 128 experts x 2048 where the 1 x 1 form takes 10, and 28-30 us for 2048 rows where the 2 x 2
+// form takes 17.)
+constexpr int kLmChunk = 128;
+// LDS layout of a chunk: 1 KB blocks [16-row tile: the router's, then the activations'][accumulator set][four steps], inside a block
 // [chain of the set][row][step]: a contracting wavefront's 128-bit read of a block and a moving wavefront's 32-bit store
 // into it are both 64 consecutive lanes on consecutive addresses.
 constexpr int kLmBlock = 256;                                          // floats of a block
-constexpr int kLmBuffer = 2 * 2 * 2 * 4 * kLmBlock;                    // floats of one chunk of both operands
-constexpr size_t kLmLdsBytes = (size_t)2 * kLmBuffer * sizeof(float);   // two buffers
+template <int TW, int EW>
+constexpr int lm_buffer() { return (TW + EW) * 8 * kLmBlock; }          // floats of one chunk of both operands
+template <int TW, int EW>
+constexpr size_t lm_lds_bytes() { return (size_t)2 * lm_buffer<TW, EW>() * sizeof(float); }   // two buffers
 typedef float lm_acc_t __attribute__((ext_vector_type(16)));
 struct LmHalf { float4 w[2][2], x[2][2]; };   // operands of half a chunk: [four steps][accumulator set]
-__global__ __launch_bounds__(512) void router_logits_mfma_kernel(const float* __restrict__ router, size_t row_floats,
-                                                                 const float* __restrict__ x, int ne, int n_expert,
-                                                                 int rows, float* __restrict__ logits) {
+// TW x EW: the workgroup's 16 x 16 tiles along the tokens and along the experts, one contracting wavefront each, and
+// one moving wavefront per 16 rows of either operand: 2 x 2 (eight wavefronts) for batches that give every compute unit
+// such a workgroup, 1 x 1 (three wavefronts) for smaller ones.
+template <int TW, int EW>
+__global__ __launch_bounds__(64 * (TW * EW + TW + EW)) void router_logits_mfma_kernel(const float* __restrict__ router, size_t row_floats,
+                                                                                        const float* __restrict__ x, int ne, int n_expert,
+                                                                                        int rows, float* __restrict__ logits) {
     extern __shared__ float lm_lds[];
+    constexpr int kLmBuffer = lm_buffer<TW, EW>(), NC = TW * EW;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int neb = (n_expert + kLmTile - 1) / kLmTile, bq = blockIdx.x >> 3;
-    const int e0 = (bq % neb) * kLmTile, r0 = ((bq / neb) * 8 + (blockIdx.x & 7)) * kLmTile;
+    const int neb = (n_expert + 16 * EW - 1) / (16 * EW), bq = blockIdx.x >> 3;
+    const int e0 = (bq % neb) * 16 * EW, r0 = ((bq / neb) * 8 + (blockIdx.x & 7)) * 16 * TW;
     if (r0 >= rows) return;
     const int nfast = (ne / kLmChunk) & ~3;   // whole chunks that run through the pipelines below, four per trip
-    if (wave >= 4) {
-        // ---- the moving wavefronts: wavefronts 4, 5 move the router's two 16-row tiles, 6, 7 the activations'.  Lane
+    if (wave >= NC) {
+        // ---- the moving wavefronts: the first EW of them move the router's 16-row tiles, the others the activations'.  Lane
         // (row, step) = (lane / 4, lane % 4) of a wavefront loads, for q = 4 s + c, the four chains of accumulator set s
         // at step 4 c + step of its row: chunk elements 32 c + 8 step + 4 s .. + 3, a 128-bit load; component t of it
         // goes to block (tile, s, c), place 64 t + lane.  Rows past the end repeat the last one (their results are never
         // stored), and so do loads past the end of a row (those steps are never contracted).
-        const int pw = wave - 4, is_x = pw >> 1, tile = pw & 1;
+        const int pw = wave - NC, is_x = pw >= EW ? 1 : 0, tile = is_x ? pw - EW : pw;
         const int grow = min((is_x ? r0 : e0) + 16 * tile + (lane >> 2), (is_x ? rows : n_expert) - 1);
         const float* src = is_x ? x + (size_t)grow * ne : router + (size_t)grow * row_floats;
         const int koff = 8 * (lane & 3);
-        const int dst0 = (is_x * 2 + tile) * 8 * kLmBlock + lane;
+        const int dst0 = pw * 8 * kLmBlock + lane;
         auto fetch = [&](float4 (&st)[8], int k0) __attribute__((always_inline)) {
 #pragma unroll
             for (int q = 0; q < 8; q++)
@@ -424,10 +334,10 @@ __global__ __launch_bounds__(512) void router_logits_mfma_kernel(const float* __
         return;
     }
     // ---- the contracting wavefronts
-    const int tw = wave & 1, ew = wave >> 1;   // the wavefront's 16 x 16 tile of the workgroup's 32 x 32
+    const int tw = wave % TW, ew = wave / TW;   // the wavefront's 16 x 16 tile of the workgroup's
     // the lane's operands of accumulator set s: chain 4 s + lane / 16, row lane % 16 of the wavefront's tile
-    const int wo = (0 * 2 + ew) * 8 * kLmBlock + 4 * lane;
-    const int xo = (1 * 2 + tw) * 8 * kLmBlock + 4 * lane;
+    const int wo = ew * 8 * kLmBlock + 4 * lane;
+    const int xo = (EW + tw) * 8 * kLmBlock + 4 * lane;
     auto read_half = [&](LmHalf& o, int buf, int half) __attribute__((always_inline)) {
         const float* base = lm_lds + buf * kLmBuffer + 2 * half * kLmBlock;
 #pragma unroll
@@ -530,7 +440,7 @@ static bool router_logits_tile(int rdt, int ne, int rows, int* epb_out, int* rpb
 }
 
 bool router_logits_fits(int rdt, size_t row_bytes, int ne, int rows) {
-    if (rows >= 32 && rdt == INFR_F32 && (ne & 31) == 0 && (row_bytes & 15) == 0) return true;   // the tiled kernel
+    if (rows >= 32 && rdt == INFR_F32 && (ne & 31) == 0 && (row_bytes & 15) == 0) return true;   // the matrix-core kernel
     int epb, rpb;
     return router_logits_tile(rdt, ne, rows, &epb, &rpb);
 }
@@ -547,18 +457,19 @@ bool launch_router_logits(hipStream_t s, const uint8_t* router, int rdt, size_t 
                        (((uintptr_t)x | (uintptr_t)nrm.weight | (uintptr_t)nrm.xn_out) & 15) != 0))
         return false;
     if (rows >= 32 && rdt == INFR_F32 && (ne & 31) == 0 && (row_bytes & 15) == 0) {
-        // the matrix-core kernel when its 32 x 32 tiles give every compute unit a workgroup, 16 x 16 tiles on the
-        // vector ALUs otherwise (a workgroup's time does not shrink with the batch: it is its chain length)
-        const int neb = (n_expert + kLmTile - 1) / kLmTile, ntb = (rows + kLmTile - 1) / kLmTile;
+        // 32 x 32 tiles when they give every compute unit a workgroup, 16 x 16 otherwise (a workgroup's time does not
+        // shrink with the batch: it is its chain length)
+        const int neb = (n_expert + 31) / 32, ntb = (rows + 31) / 32;
         if ((size_t)neb * ntb >= 256) {
             dim3 grid((unsigned)(neb * ((ntb + 7) / 8) * 8));
-            INFR_LDS_LIMIT(router_logits_mfma_kernel, (int)kLmLdsBytes);
-            INFR_LAUNCH(router_logits_mfma_kernel, grid, dim3(512), kLmLdsBytes, s, reinterpret_cast<const float*>(router),
-                        row_bytes / 4, x, ne, n_expert, rows, logits);
+            INFR_LDS_LIMIT((router_logits_mfma_kernel<2, 2>), (int)(lm_lds_bytes<2, 2>()));
+            INFR_LAUNCH((router_logits_mfma_kernel<2, 2>), grid, dim3(512), (lm_lds_bytes<2, 2>()), s,
+                        reinterpret_cast<const float*>(router), row_bytes / 4, x, ne, n_expert, rows, logits);
         } else {
-            dim3 grid((n_expert + 15) / 16, (rows + 15) / 16);
-            INFR_LAUNCH((router_logits_tiled_kernel<16, 2>), grid, dim3(512), 0, s, reinterpret_cast<const float*>(router),
-                        row_bytes / 4, x, ne, n_expert, rows, logits);
+            const int neb1 = (n_expert + 15) / 16, ntb1 = (rows + 15) / 16;
+            dim3 grid((unsigned)(neb1 * ((ntb1 + 7) / 8) * 8));
+            INFR_LAUNCH((router_logits_mfma_kernel<1, 1>), grid, dim3(192), (lm_lds_bytes<1, 1>()), s,
+                        reinterpret_cast<const float*>(router), row_bytes / 4, x, ne, n_expert, rows, logits);
         }
         return true;
     }
