@@ -251,16 +251,20 @@ constexpr int lm_buffer() { return (TW + EW) * 8 * kLmBlock; }          // float
 template <int TW, int EW>
 constexpr size_t lm_lds_bytes() { return (size_t)2 * lm_buffer<TW, EW>() * sizeof(float); }   // two buffers
 typedef float lm_acc_t __attribute__((ext_vector_type(16)));
-struct LmHalf { float4 w[2][2], x[2][2]; };   // operands of half a chunk: [four steps][accumulator set]
+template <int NS>
+struct LmHalf { float4 w[2][NS], x[2][NS]; };   // operands of half a chunk: [four steps][accumulator set]
 // TW x EW: the workgroup's 16 x 16 tiles along the tokens and along the experts, one contracting wavefront each, and
 // one moving wavefront per 16 rows of either operand: 2 x 2 (eight wavefronts) for batches that give every compute unit
-// such a workgroup, 1 x 1 (three wavefronts) for smaller ones.
-template <int TW, int EW>
-__global__ __launch_bounds__(64 * (TW * EW + TW + EW)) void router_logits_mfma_kernel(const float* __restrict__ router, size_t row_floats,
+// such a workgroup, 1 x 1 for smaller ones.  SPLIT: two contracting wavefronts per tile, one accumulator set (four chains)
+// each; a small batch's time is the chain of dependent matrix instructions, 256 steps at hidden size 2048, and two
+// instructions per step on one wavefront take twice as long as one on each of two.  The second wavefront hands its
+// four chain sums over through LDS at the end; the order of the sum over the chains stays 0..7.
+template <int TW, int EW, int SPLIT>
+__global__ __launch_bounds__(64 * (TW * EW * (SPLIT ? 2 : 1) + TW + EW)) void router_logits_mfma_kernel(const float* __restrict__ router, size_t row_floats,
                                                                                         const float* __restrict__ x, int ne, int n_expert,
                                                                                         int rows, float* __restrict__ logits) {
     extern __shared__ float lm_lds[];
-    constexpr int kLmBuffer = lm_buffer<TW, EW>(), NC = TW * EW;
+    constexpr int kLmBuffer = lm_buffer<TW, EW>(), NT = TW * EW, NC = NT * (SPLIT ? 2 : 1), NS = SPLIT ? 1 : 2;
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int neb = (n_expert + 16 * EW - 1) / (16 * EW), bq = blockIdx.x >> 3;
     const int e0 = (bq % neb) * 16 * EW, r0 = ((bq / neb) * 8 + (blockIdx.x & 7)) * 16 * TW;
@@ -334,39 +338,40 @@ __global__ __launch_bounds__(64 * (TW * EW + TW + EW)) void router_logits_mfma_k
         return;
     }
     // ---- the contracting wavefronts
-    const int tw = wave % TW, ew = wave / TW;   // the wavefront's 16 x 16 tile of the workgroup's
+    const int cw = wave % NT, set0 = wave / NT;   // (set0: the accumulator set of a wavefront that has one)
+    const int tw = cw % TW, ew = cw / TW;   // the wavefront's 16 x 16 tile of the workgroup's
     // the lane's operands of accumulator set s: chain 4 s + lane / 16, row lane % 16 of the wavefront's tile
     const int wo = ew * 8 * kLmBlock + 4 * lane;
     const int xo = (EW + tw) * 8 * kLmBlock + 4 * lane;
-    auto read_half = [&](LmHalf& o, int buf, int half) __attribute__((always_inline)) {
+    auto read_half = [&](LmHalf<NS>& o, int buf, int half) __attribute__((always_inline)) {
         const float* base = lm_lds + buf * kLmBuffer + 2 * half * kLmBlock;
 #pragma unroll
         for (int c = 0; c < 2; c++)
 #pragma unroll
-            for (int s = 0; s < 2; s++) {
-                o.w[c][s] = *reinterpret_cast<const float4*>(base + wo + (4 * s + c) * kLmBlock);
-                o.x[c][s] = *reinterpret_cast<const float4*>(base + xo + (4 * s + c) * kLmBlock);
+            for (int s = 0; s < NS; s++) {
+                o.w[c][s] = *reinterpret_cast<const float4*>(base + wo + (4 * (set0 + s) + c) * kLmBlock);
+                o.x[c][s] = *reinterpret_cast<const float4*>(base + xo + (4 * (set0 + s) + c) * kLmBlock);
             }
     };
-    lm_acc_t acc[2];
+    lm_acc_t acc[NS];
 #pragma unroll
-    for (int s = 0; s < 2; s++)
+    for (int s = 0; s < NS; s++)
 #pragma unroll
         for (int i = 0; i < 16; i++) acc[s][i] = 0.0f;
-    auto contract4 = [&](const LmHalf& o, int c) __attribute__((always_inline)) {   // four steps of both sets
+    auto contract4 = [&](const LmHalf<NS>& o, int c) __attribute__((always_inline)) {   // four steps of the wavefront's sets
 #pragma unroll
-        for (int s = 0; s < 2; s++) acc[s] = __builtin_amdgcn_mfma_f32_16x16x1f32(o.x[c][s].x, o.w[c][s].x, acc[s], 0, 0, 0);
+        for (int s = 0; s < NS; s++) acc[s] = __builtin_amdgcn_mfma_f32_16x16x1f32(o.x[c][s].x, o.w[c][s].x, acc[s], 0, 0, 0);
 #pragma unroll
-        for (int s = 0; s < 2; s++) acc[s] = __builtin_amdgcn_mfma_f32_16x16x1f32(o.x[c][s].y, o.w[c][s].y, acc[s], 0, 0, 0);
+        for (int s = 0; s < NS; s++) acc[s] = __builtin_amdgcn_mfma_f32_16x16x1f32(o.x[c][s].y, o.w[c][s].y, acc[s], 0, 0, 0);
 #pragma unroll
-        for (int s = 0; s < 2; s++) acc[s] = __builtin_amdgcn_mfma_f32_16x16x1f32(o.x[c][s].z, o.w[c][s].z, acc[s], 0, 0, 0);
+        for (int s = 0; s < NS; s++) acc[s] = __builtin_amdgcn_mfma_f32_16x16x1f32(o.x[c][s].z, o.w[c][s].z, acc[s], 0, 0, 0);
 #pragma unroll
-        for (int s = 0; s < 2; s++) acc[s] = __builtin_amdgcn_mfma_f32_16x16x1f32(o.x[c][s].w, o.w[c][s].w, acc[s], 0, 0, 0);
+        for (int s = 0; s < NS; s++) acc[s] = __builtin_amdgcn_mfma_f32_16x16x1f32(o.x[c][s].w, o.w[c][s].w, acc[s], 0, 0, 0);
     };
     if (nfast > 0) {
         // chunk c is read from LDS buffer c % 2 half a chunk at a time: its first half beside the second half of chunk
         // c - 1's matrix instructions, its second half beside its own first half
-        LmHalf h1, h2;
+        LmHalf<NS> h1, h2;
         __syncthreads();
         read_half(h1, 0, 0);
         for (int c = 0; c < nfast; c++) {
@@ -397,7 +402,7 @@ __global__ __launch_bounds__(64 * (TW * EW + TW + EW)) void router_logits_mfma_k
         __syncthreads();
         __syncthreads();
         const int steps = min(kLmChunk, ne - k0) >> 3;   // 4, 8, 12 or 16 (ne is a multiple of 32)
-        LmHalf o;
+        LmHalf<NS> o;
         read_half(o, 0, 0);
         contract4(o, 0);
         if (steps > 4) contract4(o, 1);
@@ -407,12 +412,26 @@ __global__ __launch_bounds__(64 * (TW * EW + TW + EW)) void router_logits_mfma_k
             if (steps > 12) contract4(o, 1);
         }
     }
+    if (SPLIT) {   // chains 4..7 to the tile's first wavefront (the moving wavefronts are through: the buffers are free)
+        __syncthreads();
+        if (set0 == 1) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) lm_lds[(cw * 16 + i) * 64 + lane] = acc[0][i];
+        }
+        __syncthreads();
+        if (set0 == 1) return;
+    }
     const int e = e0 + 16 * ew + (lane & 15);
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         float s = 0.0f;
 #pragma unroll
-        for (int c = 0; c < 8; c++) s = __fadd_rn(s, acc[c >> 2][4 * (c & 3) + i]);
+        for (int c = 0; c < 8; c++) {
+            float a;
+            if (SPLIT) a = c < 4 ? acc[0][4 * c + i] : lm_lds[(cw * 16 + 4 * (c & 3) + i) * 64 + lane];
+            else a = acc[NS - 1 < (c >> 2) ? 0 : (c >> 2)][4 * (c & 3) + i];
+            s = __fadd_rn(s, a);
+        }
         const int r = r0 + 16 * tw + 4 * (lane >> 4) + i;
         if (e < n_expert && r < rows) logits[(size_t)r * n_expert + e] = s;
     }
@@ -457,18 +476,19 @@ bool launch_router_logits(hipStream_t s, const uint8_t* router, int rdt, size_t 
                        (((uintptr_t)x | (uintptr_t)nrm.weight | (uintptr_t)nrm.xn_out) & 15) != 0))
         return false;
     if (rows >= 32 && rdt == INFR_F32 && (ne & 31) == 0 && (row_bytes & 15) == 0) {
-        // 32 x 32 tiles when they give every compute unit a workgroup, 16 x 16 otherwise (a workgroup's time does not
-        // shrink with the batch: it is its chain length)
+        // 32 x 32 tiles when they give every compute unit a workgroup; 16 x 16 with split chains otherwise (a workgroup's
+        // time does not shrink with the batch: it is its chain length; for the large form splitting changed nothing, 16.0
+        // against 16.1 us)
         const int neb = (n_expert + 31) / 32, ntb = (rows + 31) / 32;
         if ((size_t)neb * ntb >= 256) {
             dim3 grid((unsigned)(neb * ((ntb + 7) / 8) * 8));
-            INFR_LDS_LIMIT((router_logits_mfma_kernel<2, 2>), (int)(lm_lds_bytes<2, 2>()));
-            INFR_LAUNCH((router_logits_mfma_kernel<2, 2>), grid, dim3(512), (lm_lds_bytes<2, 2>()), s,
+            INFR_LDS_LIMIT((router_logits_mfma_kernel<2, 2, 0>), (int)(lm_lds_bytes<2, 2>()));
+            INFR_LAUNCH((router_logits_mfma_kernel<2, 2, 0>), grid, dim3(512), (lm_lds_bytes<2, 2>()), s,
                         reinterpret_cast<const float*>(router), row_bytes / 4, x, ne, n_expert, rows, logits);
         } else {
             const int neb1 = (n_expert + 15) / 16, ntb1 = (rows + 15) / 16;
             dim3 grid((unsigned)(neb1 * ((ntb1 + 7) / 8) * 8));
-            INFR_LAUNCH((router_logits_mfma_kernel<1, 1>), grid, dim3(192), (lm_lds_bytes<1, 1>()), s,
+            INFR_LAUNCH((router_logits_mfma_kernel<1, 1, 1>), grid, dim3(256), (lm_lds_bytes<1, 1>()), s,
                         reinterpret_cast<const float*>(router), row_bytes / 4, x, ne, n_expert, rows, logits);
         }
         return true;
