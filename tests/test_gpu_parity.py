@@ -171,8 +171,8 @@ def test_router_logits_probs_ids_weights_bit_exact(be, rows, ne, E, K, rdt):
 
 @pytest.mark.parametrize("rows", [1, 64, 2048])
 def test_router_logits_keep_subnormal_terms(be, rows):
-    """Products and sums around 1e-39 are subnormal f32 numbers: the logits kernels of every batch size (per-row chains,
-    tiled vector kernel, matrix-core kernel) must keep them as the CPU's fused multiply-add does."""
+    """Products and sums around 1e-39 are subnormal f32 numbers: the logits kernels of every batch size (per-row chains
+    on the vector ALUs, the two forms of the matrix-core kernel) must keep them as the CPU's fused multiply-add does."""
     ne, E, K, nff = 256, 128, 8, 32
     rng = np.random.default_rng(5)
     x = (rng.standard_normal((rows, ne)) * 1e-22).astype(np.float32)
