@@ -1609,9 +1609,11 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                 }
                 if (sc.batched) {
                     const int pairs = rows * (int)m.n_used;
-                    {
+                    // the unit-decoder GEMM reads activations in natural k order, which is Q8_0's
+                    const int a_dt_gu = sc.units_mfma ? INFR_Q8_0 : gp.gate_dt, a_dt_dn = sc.units_mfma ? INFR_Q8_0 : gp.down_dt;
+                    {   // routing, and in the same launch the token rows as f16 for the gate/up GEMM
                         Timed t(be, "route_topk");
-                        infr::launch_route(s, rp);
+                        infr::launch_route_rows_to_f16(s, rp, a_dt_gu, gp.x, (int)m.ne, sc.xh, sc.xs);
                     }
                     {
                         Timed t(be, "moe_bucket");
@@ -1621,12 +1623,6 @@ extern "C" infr_status infr_hip_execute(infr_hip_backend* be, infr_hip_plan* pla
                             bucket_ids = sc.live_ids;
                         }
                         infr::launch_bucket(s, bucket_ids, pairs, (int)n_local, sc.offsets, sc.pair_src, sc.slot_pair);
-                    }
-                    // the unit-decoder GEMM reads activations in natural k order, which is Q8_0's
-                    const int a_dt_gu = sc.units_mfma ? INFR_Q8_0 : gp.gate_dt, a_dt_dn = sc.units_mfma ? INFR_Q8_0 : gp.down_dt;
-                    {
-                        Timed t(be, "rows_to_f16");
-                        infr::launch_rows_to_f16(s, a_dt_gu, gp.x, rows, (int)m.ne, sc.xh, sc.xs);
                     }
                     infr::GroupedParams q{};
                     q.loads_only = be->probe_grouped_loads_only.load() ? 1 : 0;

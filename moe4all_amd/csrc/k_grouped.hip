@@ -8,7 +8,8 @@
 //                         scatter of the pairs into that order (one block per expert; order is
 //                         an integer contract and is reproduced exactly).
 //   rows_to_f16_kernel    activation rows -> f16 with one power-of-two scale per row (so any f32
-//                         magnitude fits), laid out in the k order the weight format unpacks to.
+//                         magnitude fits), laid out in the k order the weight format unpacks to
+//                         (route_rows_to_f16_kernel: the same for the token rows, with the row's routing).
 //   grouped_mfma6<D,DOWN> per (expert, 128-token tile, 128/256-feature tile): the raw quantised bytes
 //                         of the tile's weight rows are copied into LDS, every lane unpacks its
 //                         row's codes to f16 in registers with packed 16-bit arithmetic, the
@@ -23,6 +24,7 @@
 // which codes fall out of a dword is not the element order; since a dot product does not care
 // about the order of its terms, the activation rows are stored in that same ("virtual") order.
 #include "grouped_common.h"
+#include "route.h"
 
 namespace infr {
 
@@ -31,10 +33,8 @@ namespace {
 // --------------------------------------------------------------------------------------------
 // One block per row: amax -> power-of-two scale -> f16 in the virtual k order of format F.
 template <class F>
-__global__ __launch_bounds__(256) void rows_to_f16_kernel(const float* __restrict__ src, int n,
-                                                          _Float16* __restrict__ dst, float* __restrict__ scale) {
-    __shared__ float s_max[4];
-    const size_t row = blockIdx.x;
+__device__ __forceinline__ void row_to_f16(const float* __restrict__ src, int n, _Float16* __restrict__ dst,
+                                           float* __restrict__ scale, size_t row, float* s_max) {
     const float* x = src + row * n;
     float m = 0.0f;
     for (int k = threadIdx.x * 4; k < n; k += 1024) {
@@ -69,6 +69,27 @@ __global__ __launch_bounds__(256) void rows_to_f16_kernel(const float* __restric
         }
         out[c] = uint4{as_u32(h0), as_u32(h1), as_u32(h2), as_u32(h3)};
     }
+}
+
+template <class F>
+__global__ __launch_bounds__(256) void rows_to_f16_kernel(const float* __restrict__ src, int n,
+                                                          _Float16* __restrict__ dst, float* __restrict__ scale) {
+    __shared__ float s_max[4];
+    row_to_f16<F>(src, n, dst, scale, blockIdx.x, s_max);
+}
+
+// The routing of token row b (route_kernel's work, on the block's first wavefront) behind the f16 conversion of the same
+// row for the gate/up GEMM: both are per row and both precede the bucketing, and a launch of either alone is mostly its
+// dispatch (32 to 2048 rows: 5.0-7.8 us and 3.9-4.7 us as two launches).
+template <class F>
+__global__ __launch_bounds__(256) void route_rows_to_f16_kernel(RouteParams rp, const float* __restrict__ src, int n,
+                                                                _Float16* __restrict__ dst, float* __restrict__ scale) {
+    extern __shared__ float lds[];
+    __shared__ float s_max[4];
+    uint64_t* tab = reinterpret_cast<uint64_t*>(lds);
+    if (threadIdx.x < 32) tab[threadIdx.x] = kExp2Table[threadIdx.x];
+    row_to_f16<F>(src, n, dst, scale, blockIdx.x, s_max);   // (its barrier also publishes the table)
+    if (threadIdx.x < 64) route_row_any(rp, blockIdx.x, threadIdx.x, lds + 64, tab);
 }
 
 // --------------------------------------------------------------------------------------------
@@ -793,6 +814,15 @@ bool grouped_supported(int dt, int k) {
     // the k loop runs in groups of four 64-element slices (one K-quant super-block)
     if (k <= 0 || (k % (kSlice * 4)) != 0) return false;
     return dt == INFR_Q4K || dt == INFR_Q6K || dt == INFR_Q8_0;
+}
+
+void launch_route_rows_to_f16(hipStream_t s, const RouteParams& rp, int weight_dt, const float* src, int n, void* dst, float* scale) {
+    if (rp.rows <= 0) return;
+    _Float16* d = reinterpret_cast<_Float16*>(dst);
+    const size_t lds = (64 + route_scratch_floats(rp.n_expert, rp.n_groups)) * sizeof(float);
+    if (weight_dt == INFR_Q4K) INFR_LAUNCH(route_rows_to_f16_kernel<MQ4K>, dim3(rp.rows), dim3(256), lds, s, rp, src, n, d, scale);
+    else if (weight_dt == INFR_Q6K) INFR_LAUNCH(route_rows_to_f16_kernel<MQ6K>, dim3(rp.rows), dim3(256), lds, s, rp, src, n, d, scale);
+    else INFR_LAUNCH(route_rows_to_f16_kernel<MQ80>, dim3(rp.rows), dim3(256), lds, s, rp, src, n, d, scale);
 }
 
 void launch_rows_to_f16(hipStream_t s, int weight_dt, const float* src, int rows, int n, void* dst, float* scale) {

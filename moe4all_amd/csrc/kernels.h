@@ -191,6 +191,8 @@ struct GroupedParams {
 bool grouped_supported(int dt, int k);
 // rows of f32 -> f16 with a per-row power-of-two scale, in the k order weights of `weight_dt` unpack to.
 void launch_rows_to_f16(hipStream_t s, int weight_dt, const float* src, int rows, int n, void* dst, float* scale);
+// route_kernel and the conversion of the same rows in one launch (rp.rows rows of n floats)
+void launch_route_rows_to_f16(hipStream_t s, const RouteParams& rp, int weight_dt, const float* src, int n, void* dst, float* scale);
 // offsets / pair_src / slot_pair ([n_pairs], -1 for ids outside [0, n_expert)) from ids [n_pairs].
 // ids with the pairs of weight exactly 0 replaced by -1 (pairs an expert-parallel band dropped).
 void launch_mask_dropped_pairs(hipStream_t s, const int32_t* ids, const float* weights, int n_pairs, int32_t* out);
